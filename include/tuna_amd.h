@@ -1,0 +1,139 @@
+/*
+ * tuna_amd - C ABI of the MI355X (gfx950) FP16-activation x 4-bit-codebook-weight GEMM.
+ *
+ * This is the drop-in boundary: plain pointers and sizes, no torch types.  Every
+ * device pointer is caller-owned memory on the current HIP device; `stream` is a
+ * hipStream_t passed as void* (NULL = the default stream).  All entry points are
+ * stream-ordered and never synchronise the host with the device, unless stated.
+ *
+ * Naming follows the reference: m = weight rows (output features), n = activation
+ * rows (tokens), k = reduction length.
+ *
+ * Tensor layouts (identical to the reference's, extension.cpp:26-49):
+ *   q       uint8  [m/8, k/8, 32]  one 32-byte record per 8x8 weight block; byte b of
+ *                                  block (mb, kb) holds row mb*8 + b/4, column
+ *                                  kb*8 + 2*(b%4) in its high nibble and column
+ *                                  kb*8 + 2*(b%4) + 1 in its low nibble
+ *                                  (test.py:58-65, kernel.cu:3221-3228)
+ *   x       fp16   [n, k]          row-major (test.py:76)
+ *   code    fp32   [16]            codebook (kernel.cu:3014)
+ *   absmax  fp32   [m]             one scale per weight row (kernel.cu:3015)
+ *   out     fp16   [n, m]          row-major (kernel.cu:2872, 2957-2959)
+ */
+#ifndef TUNA_AMD_H
+#define TUNA_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TUNA_AMD_VERSION 100 /* major*10000 + minor*100 + patch */
+
+/* Status codes.  The reference returns void and silently does nothing for
+ * shapes outside its table (kernel.cu:3018-3156); here every call reports. */
+enum {
+    TUNA_OK = 0,
+    TUNA_ERR_INVALID_ARG = 1, /* null pointer, misaligned pointer, bad size          */
+    TUNA_ERR_UNSUPPORTED = 2, /* shape or config the kernels cannot run              */
+    TUNA_ERR_HIP = 3,         /* a HIP runtime call failed (see tuna_last_error)     */
+    TUNA_ERR_NO_DEVICE = 4,   /* no usable gfx950 device                             */
+    TUNA_ERR_WORKSPACE = 5    /* split-K workspace could not be provided             */
+};
+
+/* Decode rounding of a 4-bit code into an fp16 weight.
+ * TUNA_DECODE_GEMM    : fp16(code) * fp16(absmax) as an fp16 multiply - what the
+ *                       reference GEMM feeds its tensor cores (kernel.cu:2178-2192
+ *                       with the fp16 staging of kernel.cu:2770, 2800).
+ * TUNA_DECODE_DEQUANT : fp16(code * absmax) with the product in fp32 - what the
+ *                       reference dequant op writes (kernel.cu:3222-3228).        */
+enum { TUNA_DECODE_GEMM = 1, TUNA_DECODE_DEQUANT = 2 };
+
+/* Tile configuration of one GEMM launch: the CDNA4 counterpart of the reference's
+ * KernelConfig (configs.cu:12-54).  A workgroup is waves_m x waves_k wave64s; a wave
+ * owns rows_per_wave weight rows and walks k in steps of 32; the workgroup owns
+ * rows_per_wave*waves_m rows and a 1/split_k share of k.                          */
+typedef struct tuna_gemm_config {
+    int32_t rows_per_wave; /* 64, 128 or 256: 128-bit loads per lane per k-step x 64 */
+    int32_t waves_m;       /* waves along the weight rows                             */
+    int32_t waves_k;       /* waves along k inside the workgroup (reduced in LDS)     */
+    int32_t split_k;       /* workgroups along k (reduced through the workspace)      */
+    int32_t prefetch;      /* 2, 4 or 8: k-steps of packed weights in flight per wave */
+    int32_t x_chunk;       /* k elements of x staged in LDS at a time (multiple of 32*waves_k*prefetch) */
+    int32_t token_tiles;   /* 1, 2 or 4: 16-token MFMA tiles per pass over the weights */
+    int32_t xcd_swizzle;   /* 1: remap workgroup ids so neighbours share an XCD       */
+} tuna_gemm_config;
+
+int tuna_version(void);
+const char *tuna_status_string(int status);
+/* Message of the last failing call on this host thread ("" if none). */
+const char *tuna_last_error(void);
+
+/* out[n, m] = x[n, k] . decode(q, code, absmax)[m, k]^T, fp32 accumulate, fp16 output.
+ * Replaces  void wrapper(void *q, void *x, void *c, void *s, void *o, int m, int n,
+ * int k, cudaStream_t)  (kernel.cu:3009, declared extension.cpp:22); same argument
+ * order.  `out` is overwritten (it need not be zeroed, unlike kernel.cu:2739-2745).
+ * Uses TUNA_DECODE_GEMM and the built-in shape->config table (any m % 8 == 0,
+ * k % 8 == 0, n >= 1 is accepted; shapes outside the table get a derived config). */
+int tuna_matmul(const void *q, const void *x, const void *code, const void *absmax,
+                void *out, int m, int n, int k, void *stream);
+
+/* Same, with an explicit config (NULL = table lookup) and decode mode. */
+int tuna_matmul_ex(const void *q, const void *x, const void *code, const void *absmax,
+                   void *out, int m, int n, int k, const tuna_gemm_config *cfg,
+                   int decode_mode, void *stream);
+
+/* out[m, k] fp16 row-major = decode(q, code, absmax), TUNA_DECODE_DEQUANT rounding.
+ * Replaces  void dequantize_wrapper(void *q, void *a, void *c, void *o, const int m,
+ * const int k, cudaStream_t)  (kernel.cu:3243, declared extension.cpp:24). */
+int tuna_dequant(const void *q, const void *absmax, const void *code, void *out,
+                 int m, int k, void *stream);
+
+/* Same with the decode rounding selectable (TUNA_DECODE_GEMM gives the image of the
+ * weights the GEMM multiplies with). */
+int tuna_dequant_ex(const void *q, const void *absmax, const void *code, void *out,
+                    int m, int k, int decode_mode, void *stream);
+
+/* Shape -> config.  Replaces the if-chain of kernel.cu:3018-3156 over the constants of
+ * configs.cu:56-3331 by a table lookup on (m, n-bucket, k) with a derived fallback.
+ * Runs on the host only (no device needed).  Returns 1 in *from_table when the shape
+ * hit a tuned entry. */
+int tuna_select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_table);
+/* TUNA_OK if `cfg` can run shape (m, n, k); otherwise an error and tuna_last_error(). */
+int tuna_validate_config(int m, int n, int k, const tuna_gemm_config *cfg);
+/* Dynamic LDS bytes and workspace bytes a launch of `cfg` needs. */
+int tuna_config_footprint(int m, int n, int k, const tuna_gemm_config *cfg,
+                          size_t *lds_bytes, size_t *workspace_bytes);
+/* Enumerate the built-in table: entry i -> its shape key and config. */
+int tuna_config_table_size(void);
+int tuna_config_table_entry(int i, int *m, int *n_lo, int *n_hi, int *k, tuna_gemm_config *cfg);
+
+/* Timing helper for the bench and the tuner: enqueues `warmup` untimed and `iters`
+ * timed GEMMs on `stream`, launch i using weight set (i mod n_sets) of q_list /
+ * absmax_list (rotating over distinct weights defeats the L2 / MALL caches), and
+ * returns the elapsed milliseconds of the timed launches measured with HIP events
+ * recorded on `stream`.  use_graph != 0 captures one rotation into a HIP graph and
+ * replays it.  This call synchronises the host with `stream`. */
+int tuna_time_matmul(const void *const *q_list, const void *const *absmax_list, int n_sets,
+                     const void *x, const void *code, void *out, int m, int n, int k,
+                     const tuna_gemm_config *cfg, int decode_mode, int warmup, int iters,
+                     int use_graph, void *stream, float *elapsed_ms);
+/* Same protocol for the dequant kernel. */
+int tuna_time_dequant(const void *const *q_list, const void *const *absmax_list, int n_sets,
+                      const void *code, void *out, int m, int k, int warmup, int iters,
+                      void *stream, float *elapsed_ms);
+/* Plain device-to-device copy kernel of `bytes` bytes (16-byte multiples), timed the
+ * same way: the known-traffic yardstick the HBM counters are scaled against. */
+int tuna_time_copy(const void *src, void *dst, size_t bytes, int warmup, int iters,
+                   void *stream, float *elapsed_ms);
+
+/* Releases the library-owned split-K workspaces of the current device (synchronises
+ * the device first). */
+int tuna_release_workspaces(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TUNA_AMD_H */

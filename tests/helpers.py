@@ -1,0 +1,73 @@
+"""Shared helpers of the parity tests (oracle side on numpy, product side on torch)."""
+import numpy as np
+
+from oracle import oracle as O
+from tuna_amd.synth import make_inputs_np
+
+# GEMM tolerance of the north star: max relative error 1e-2 (fp16 output, fp32
+# accumulate, any split-K order).  "Relative" is |y - y_ref| / max(|y_ref|, FLOOR * max|y_ref|):
+# outputs are sums of ~k zero-mean terms, so a few land arbitrarily close to zero, where a
+# pure ratio is meaningless; below FLOOR (0.1 % of the largest output) the error is measured
+# against that floor instead.
+REL_TOL = 1e-2
+REL_FLOOR = 1e-3
+
+
+def rel_err(y, y_ref):
+    """Max relative error as defined above; y, y_ref are float64 arrays of one shape."""
+    y = np.asarray(y, np.float64)
+    y_ref = np.asarray(y_ref, np.float64)
+    scale = np.abs(y_ref).max() if y_ref.size else 0.0
+    den = np.maximum(np.abs(y_ref), REL_FLOOR * scale)
+    den[den == 0] = 1.0
+    return float((np.abs(y - y_ref) / den).max()) if y.size else 0.0
+
+
+def f16_bits_to_f64(bits):
+    return np.asarray(bits, np.uint16).view(np.float16).astype(np.float64)
+
+
+def ulp_diff_f16(a_bits, b_bits):
+    """Max distance in fp16 ulps between two bit-pattern arrays (finite values)."""
+    def key(b):
+        b = np.asarray(b, np.uint16).astype(np.int32)
+        return np.where(b & 0x8000, -(b & 0x7fff), b & 0x7fff)
+    return int(np.abs(key(a_bits) - key(b_bits)).max()) if np.size(a_bits) else 0
+
+
+def to_dev(*arrays, device="cuda"):
+    import torch
+
+    return tuple(torch.from_numpy(np.ascontiguousarray(a)).to(device) for a in arrays)
+
+
+def run_gemm(q, x, code, absmax, m, n, k, config=None, decode_mode=1, prefill=None):
+    """Product GEMM through the Python op (-> C ABI -> HIP); returns fp16 bits [n, m]."""
+    import torch
+
+    from tuna_amd import ops
+
+    dq, dx, dc, da = to_dev(q, x, code, absmax)
+    if prefill is None:
+        out = torch.zeros((n, m), dtype=torch.float16, device="cuda")
+    else:
+        out = torch.full((n, m), prefill, dtype=torch.float16, device="cuda")
+    ops.matmul(dx, dq, da, dc, out, m, n, k, config=config, decode_mode=decode_mode)
+    torch.cuda.synchronize()
+    return out.cpu().numpy().view(np.uint16)
+
+
+def run_dequant(q, code, absmax, m, k, decode_mode=2):
+    import torch
+
+    from tuna_amd import ops
+
+    dq, dc, da = to_dev(q, code, absmax)
+    out = torch.full((m, k), float("nan"), dtype=torch.float16, device="cuda")
+    ops.dequant(dq, da, dc, out, m, k, decode_mode=decode_mode)
+    torch.cuda.synchronize()
+    return out.cpu().numpy().view(np.uint16)
+
+
+__all__ = ["O", "make_inputs_np", "rel_err", "REL_TOL", "f16_bits_to_f64", "ulp_diff_f16", "to_dev", "run_gemm",
+           "run_dequant"]

@@ -1,0 +1,116 @@
+"""ctypes binding of tuna_amd/libtuna_amd.so (the C ABI declared in include/tuna_amd.h).
+
+The library is built in-tree by ``make -C tuna_amd/csrc`` (see build()).  There is no
+fallback implementation: if the shared object is missing or does not load, every op
+raises.
+"""
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtuna_amd.so")
+CSRC = os.path.join(_HERE, "csrc")
+
+OK = 0
+ERR_INVALID_ARG = 1
+ERR_UNSUPPORTED = 2
+ERR_HIP = 3
+ERR_NO_DEVICE = 4
+ERR_WORKSPACE = 5
+
+DECODE_GEMM = 1
+DECODE_DEQUANT = 2
+
+
+class GemmConfig(ctypes.Structure):
+    """Mirror of ``tuna_gemm_config`` (include/tuna_amd.h)."""
+
+    _fields_ = [
+        ("rows_per_wave", ctypes.c_int32),
+        ("waves_m", ctypes.c_int32),
+        ("waves_k", ctypes.c_int32),
+        ("split_k", ctypes.c_int32),
+        ("prefetch", ctypes.c_int32),
+        ("x_chunk", ctypes.c_int32),
+        ("token_tiles", ctypes.c_int32),
+        ("xcd_swizzle", ctypes.c_int32),
+    ]
+
+    FIELDS = tuple(f for f, _ in _fields_)
+
+    def to_dict(self):
+        return {f: int(getattr(self, f)) for f in self.FIELDS}
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(**{f: int(d[f]) for f in cls.FIELDS})
+
+
+# name -> (restype, argtypes); also the list of symbols the header declares
+_vp, _i, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+_cfgp = ctypes.POINTER(GemmConfig)
+_ip = ctypes.POINTER(ctypes.c_int)
+_fp = ctypes.POINTER(ctypes.c_float)
+_vpp = ctypes.POINTER(ctypes.c_void_p)
+SIGNATURES = {
+    "tuna_version": (_i, []),
+    "tuna_status_string": (ctypes.c_char_p, [_i]),
+    "tuna_last_error": (ctypes.c_char_p, []),
+    "tuna_matmul": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "tuna_matmul_ex": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _vp]),
+    "tuna_dequant": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "tuna_dequant_ex": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "tuna_select_config": (_i, [_i, _i, _i, _cfgp, _ip]),
+    "tuna_validate_config": (_i, [_i, _i, _i, _cfgp]),
+    "tuna_config_footprint": (_i, [_i, _i, _i, _cfgp, ctypes.POINTER(_sz), ctypes.POINTER(_sz)]),
+    "tuna_config_table_size": (_i, []),
+    "tuna_config_table_entry": (_i, [_i, _ip, _ip, _ip, _ip, _cfgp]),
+    "tuna_time_matmul": (_i, [_vpp, _vpp, _i, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _i, _i, _i, _vp, _fp]),
+    "tuna_time_dequant": (_i, [_vpp, _vpp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _fp]),
+    "tuna_time_copy": (_i, [_vp, _vp, _sz, _i, _i, _vp, _fp]),
+    "tuna_release_workspaces": (_i, []),
+}
+
+
+def build(force: bool = True) -> str:
+    """Compile the HIP sources for gfx950 into libtuna_amd.so (hipcc, in-tree)."""
+    if force:
+        subprocess.run(["make", "-C", CSRC, "clean"], check=True, capture_output=True)
+    r = subprocess.run(["make", "-C", CSRC, "-j8"], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building libtuna_amd.so failed:\n" + r.stdout[-4000:] + r.stderr[-4000:])
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises if it is not built (no fallback path exists)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+                "or `make -C tuna_amd/csrc`; tuna_amd has no non-HIP fallback")
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(L, name)  # AttributeError if the library lacks a declared symbol
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+class TunaError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"tuna_amd status {status}: {message}")
+        self.status = status
+
+
+def check(status: int) -> None:
+    if status != OK:
+        L = lib()
+        msg = L.tuna_last_error().decode() or L.tuna_status_string(status).decode()
+        raise TunaError(status, msg)

@@ -1,0 +1,498 @@
+// Host side of the C ABI: argument checking, shape -> config, launch planning, the
+// library-owned split-K workspace, and the HIP-event timing helpers.
+//
+// Replaces the reference's host dispatcher (kernel.cu:2962-3156: requiredSmem,
+// LAUNCH_KERNEL_IF_CONDITION and the 122-arm if-chain in wrapper) and
+// dequantize_wrapper (kernel.cu:3243-3253).
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "tuna_internal.h"
+
+namespace tuna {
+
+static thread_local std::string g_error;
+
+static int fail(int code, const char *fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_error = buf;
+    return code;
+}
+
+static int hip_fail(hipError_t e, const char *what)
+{
+    return fail(TUNA_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+static inline int round_up(int a, int b) { return ceil_div(a, b) * b; }
+
+// ---------------------------------------------------------------------------------------
+// config validation and launch planning
+// ---------------------------------------------------------------------------------------
+
+static int check_shape(int m, int n, int k)
+{
+    if (m <= 0 || n <= 0 || k <= 0) return fail(TUNA_ERR_INVALID_ARG, "m, n, k must be positive (m=%d n=%d k=%d)", m, n, k);
+    if ((m & 7) || (k & 7))
+        return fail(TUNA_ERR_INVALID_ARG, "m and k must be multiples of 8, the packed block size (m=%d k=%d)", m, k);
+    return TUNA_OK;
+}
+
+static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode, GemmPlan *plan)
+{
+    int rc = check_shape(m, n, k);
+    if (rc) return rc;
+    if (decode != TUNA_DECODE_GEMM && decode != TUNA_DECODE_DEQUANT)
+        return fail(TUNA_ERR_INVALID_ARG, "decode_mode %d is neither TUNA_DECODE_GEMM nor TUNA_DECODE_DEQUANT", decode);
+    if (c.rows_per_wave != 64 && c.rows_per_wave != 128 && c.rows_per_wave != 256)
+        return fail(TUNA_ERR_UNSUPPORTED, "rows_per_wave=%d (64, 128 or 256)", c.rows_per_wave);
+    if (c.prefetch != 2 && c.prefetch != 4 && c.prefetch != 8)
+        return fail(TUNA_ERR_UNSUPPORTED, "prefetch=%d (2, 4 or 8)", c.prefetch);
+    if (c.token_tiles != 1 && c.token_tiles != 2 && c.token_tiles != 4)
+        return fail(TUNA_ERR_UNSUPPORTED, "token_tiles=%d (1, 2 or 4)", c.token_tiles);
+    if (c.waves_m < 1 || c.waves_k < 1 || c.waves_m * c.waves_k * 64 > kMaxThreads)
+        return fail(TUNA_ERR_UNSUPPORTED, "waves_m=%d x waves_k=%d must give 1..16 waves", c.waves_m, c.waves_k);
+    const int steps_total = ceil_div(k, kStepK);
+    if (c.split_k < 1 || c.split_k > steps_total)
+        return fail(TUNA_ERR_UNSUPPORTED, "split_k=%d must be in 1..%d for k=%d", c.split_k, steps_total, k);
+    if (c.x_chunk <= 0 || c.x_chunk % (kStepK * c.waves_k * c.prefetch) != 0)
+        return fail(TUNA_ERR_UNSUPPORTED, "x_chunk=%d must be a positive multiple of 32*waves_k*prefetch=%d", c.x_chunk,
+                    kStepK * c.waves_k * c.prefetch);
+    const int rw = c.rows_per_wave / kRowsPerLoad;
+    const int threads = c.waves_m * c.waves_k * 64;
+    if (!gemm_variant_exists(rw, c.prefetch, c.token_tiles, decode, threads))
+        return fail(TUNA_ERR_UNSUPPORTED,
+                    "no kernel variant for rows_per_wave=%d prefetch=%d token_tiles=%d decode=%d threads=%d", c.rows_per_wave,
+                    c.prefetch, c.token_tiles, decode, threads);
+
+    const int nacc = rw * 4 * c.token_tiles;
+    const int lut = decode == TUNA_DECODE_GEMM ? kLutBytes : 64;
+    const size_t main_lds = (size_t)lut + (size_t)c.token_tiles * 16 * ((size_t)c.x_chunk * 2 + 16);
+    const size_t red_lds = (size_t)(c.waves_k - 1) * c.waves_m * nacc * 1024;
+    const size_t lds = (main_lds > red_lds ? main_lds : red_lds) + 16;
+    if (lds > (size_t)kLdsLimit)
+        return fail(TUNA_ERR_UNSUPPORTED, "config needs %zu bytes of LDS, the CU has %d", lds, kLdsLimit);
+
+    const int rows_wg = c.rows_per_wave * c.waves_m;
+    const int row_tiles = ceil_div(m, rows_wg);
+    const int tok_chunks = ceil_div(n, 16 * c.token_tiles);
+    if (tok_chunks > 65535) return fail(TUNA_ERR_UNSUPPORTED, "n=%d needs %d token chunks (max 65535)", n, tok_chunks);
+    if ((long long)row_tiles * c.split_k > 0x7fffffffLL) return fail(TUNA_ERR_UNSUPPORTED, "grid too large");
+
+    GemmPlan &p = *plan;
+    memset(&p, 0, sizeof(p));
+    p.rw = rw;
+    p.prefetch = c.prefetch;
+    p.token_tiles = c.token_tiles;
+    p.decode = decode;
+    p.threads = threads;
+    p.lds_bytes = lds;
+    p.grid = dim3((unsigned)(row_tiles * c.split_k), (unsigned)tok_chunks, 1);
+    p.ws_bytes = c.split_k > 1 ? (size_t)tok_chunks * row_tiles * c.split_k * c.waves_m * nacc * 1024 : 0;
+    p.n_counters = c.split_k > 1 ? (size_t)tok_chunks * row_tiles : 0;
+    GemmArgs &a = p.args;
+    a.m = m;
+    a.n = n;
+    a.k = k;
+    a.waves_m = c.waves_m;
+    a.waves_k = c.waves_k;
+    a.split_k = c.split_k;
+    a.steps_total = steps_total;
+    a.steps_per_split = ceil_div(steps_total, c.split_k);
+    a.chunk_steps = c.x_chunk / kStepK;
+    a.row_tiles = row_tiles;
+    a.xcd_swizzle = c.xcd_swizzle ? 1 : 0;
+    a.lds_bytes = (int)lds;
+    return TUNA_OK;
+}
+
+// A config for shapes the tuned table does not cover: 8-wave workgroups, enough
+// workgroups along k to occupy the 256 CUs, x staged 1024 k at a time.
+static tuna_gemm_config derive_config(int m, int n, int k)
+{
+    tuna_gemm_config c;
+    c.token_tiles = n <= 16 ? 1 : (n <= 32 ? 2 : 4);
+    c.rows_per_wave = (m >= 16384 && c.token_tiles == 1) ? 128 : 64;
+    c.waves_m = 2;
+    c.waves_k = 4;
+    c.prefetch = 4;
+    c.xcd_swizzle = 0;
+    const int steps = ceil_div(k, kStepK);
+    const int row_tiles = ceil_div(m, c.rows_per_wave * c.waves_m);
+    const int group = c.waves_k * c.prefetch;  // k-steps one workgroup consumes per ring turn
+    int split = (512 + row_tiles / 2) / row_tiles;
+    const int max_split = steps / group > 0 ? steps / group : 1;
+    if (split > max_split) split = max_split;
+    if (split < 1) split = 1;
+    c.split_k = split;
+    const int sps = ceil_div(steps, split);
+    int chunk_steps = round_up(sps, group);
+    const int cap = round_up(32 / c.token_tiles, group);  // keeps table + x within the 160 KB of LDS
+    if (chunk_steps > cap) chunk_steps = cap;
+    c.x_chunk = chunk_steps * kStepK;
+    return c;
+}
+
+static int select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_table)
+{
+    for (int i = 0; i < kConfigTableSize; ++i) {
+        const TableEntry &e = kConfigTable[i];
+        if (e.m == m && e.k == k && n >= e.n_lo && n <= e.n_hi) {
+            *cfg = e.cfg;
+            if (from_table) *from_table = 1;
+            return TUNA_OK;
+        }
+    }
+    *cfg = derive_config(m, n, k);
+    if (from_table) *from_table = 0;
+    return TUNA_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// split-K workspace: owned by the library, one per (device, stream), grown on demand
+// ---------------------------------------------------------------------------------------
+
+struct Workspace {
+    float *ws = nullptr;
+    size_t ws_bytes = 0;
+    unsigned *counters = nullptr;
+    size_t n_counters = 0;
+};
+
+static std::mutex g_ws_mutex;
+static std::map<std::pair<int, hipStream_t>, Workspace> g_workspaces;
+
+static int get_workspace(hipStream_t stream, size_t ws_bytes, size_t n_counters, Workspace *out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    Workspace &w = g_workspaces[std::make_pair(dev, stream)];
+    if (w.ws_bytes < ws_bytes || w.n_counters < n_counters) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+            return fail(TUNA_ERR_WORKSPACE,
+                        "split-K workspace must grow (%zu bytes) while the stream is capturing; run the shape once before capture",
+                        ws_bytes);
+        // hipFree waits for the device, so kernels still using the old buffers are done.
+        if (w.ws_bytes < ws_bytes) {
+            size_t want = ws_bytes < (size_t)(8u << 20) ? (size_t)(8u << 20) : ws_bytes;
+            if (w.ws) (void)hipFree(w.ws);
+            w.ws = nullptr;
+            w.ws_bytes = 0;
+            e = hipMalloc(reinterpret_cast<void **>(&w.ws), want);
+            if (e != hipSuccess) return fail(TUNA_ERR_WORKSPACE, "hipMalloc(%zu) for the split-K workspace: %s", want, hipGetErrorString(e));
+            w.ws_bytes = want;
+        }
+        if (w.n_counters < n_counters) {
+            size_t want = n_counters < 16384 ? 16384 : n_counters;
+            if (w.counters) (void)hipFree(w.counters);
+            w.counters = nullptr;
+            w.n_counters = 0;
+            e = hipMalloc(reinterpret_cast<void **>(&w.counters), want * sizeof(unsigned));
+            if (e != hipSuccess) return fail(TUNA_ERR_WORKSPACE, "hipMalloc for the split-K counters: %s", hipGetErrorString(e));
+            e = hipMemset(w.counters, 0, want * sizeof(unsigned));  // kernels leave them at zero afterwards
+            if (e != hipSuccess) return hip_fail(e, "hipMemset(counters)");
+            e = hipDeviceSynchronize();
+            if (e != hipSuccess) return hip_fail(e, "hipDeviceSynchronize");
+            w.n_counters = want;
+        }
+    }
+    *out = w;
+    return TUNA_OK;
+}
+
+static void drop_workspace(hipStream_t stream)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return;
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    auto it = g_workspaces.find(std::make_pair(dev, stream));
+    if (it == g_workspaces.end()) return;
+    if (it->second.ws) (void)hipFree(it->second.ws);
+    if (it->second.counters) (void)hipFree(it->second.counters);
+    g_workspaces.erase(it);
+}
+
+static int check_ptr(const void *p, const char *name, size_t align)
+{
+    if (!p) return fail(TUNA_ERR_INVALID_ARG, "%s is null", name);
+    if (reinterpret_cast<uintptr_t>(p) % align) return fail(TUNA_ERR_INVALID_ARG, "%s must be %zu-byte aligned", name, align);
+    return TUNA_OK;
+}
+
+static int matmul_impl(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n, int k,
+                       const tuna_gemm_config *cfg, int decode, hipStream_t stream)
+{
+    int rc;
+    if ((rc = check_shape(m, n, k))) return rc;
+    if ((rc = check_ptr(q, "q", 16)) || (rc = check_ptr(x, "x", 16)) || (rc = check_ptr(code, "code", 4)) ||
+        (rc = check_ptr(absmax, "absmax", 4)) || (rc = check_ptr(out, "out", 16)))
+        return rc;
+    tuna_gemm_config c;
+    if (cfg) c = *cfg;
+    else {
+        select_config(m, n, k, &c, nullptr);
+        if (decode != TUNA_DECODE_GEMM) {  // the dequant-rounding variants exist for one tile shape only
+            c.rows_per_wave = 64;
+            c.prefetch = 2;
+            c.x_chunk = round_up(c.x_chunk, kStepK * c.waves_k * c.prefetch);
+        }
+    }
+    GemmPlan plan;
+    if ((rc = plan_gemm(m, n, k, c, decode, &plan))) return rc;
+    plan.args.q = static_cast<const uint8_t *>(q);
+    plan.args.x = x;
+    plan.args.code = static_cast<const float *>(code);
+    plan.args.absmax = static_cast<const float *>(absmax);
+    plan.args.out = out;
+    if (plan.ws_bytes) {
+        Workspace w;
+        if ((rc = get_workspace(stream, plan.ws_bytes, plan.n_counters, &w))) return rc;
+        plan.args.ws = w.ws;
+        plan.args.counters = w.counters;
+    }
+    hipError_t e = launch_gemm(plan, stream);
+    if (e != hipSuccess) return hip_fail(e, "gemm launch");
+    return TUNA_OK;
+}
+
+static int dequant_impl(const void *q, const void *absmax, const void *code, void *out, int m, int k, int decode,
+                        hipStream_t stream)
+{
+    int rc;
+    if ((rc = check_shape(m, 1, k))) return rc;
+    if (decode != TUNA_DECODE_GEMM && decode != TUNA_DECODE_DEQUANT)
+        return fail(TUNA_ERR_INVALID_ARG, "decode_mode %d is neither TUNA_DECODE_GEMM nor TUNA_DECODE_DEQUANT", decode);
+    if ((rc = check_ptr(q, "q", 16)) || (rc = check_ptr(absmax, "absmax", 4)) || (rc = check_ptr(code, "code", 4)) ||
+        (rc = check_ptr(out, "out", 16)))
+        return rc;
+    hipError_t e = launch_dequant(static_cast<const uint8_t *>(q), static_cast<const float *>(absmax),
+                                  static_cast<const float *>(code), out, m, k, decode, stream);
+    if (e != hipSuccess) return hip_fail(e, "dequant launch");
+    return TUNA_OK;
+}
+
+// Times `iters` enqueues of `launch(i)` with HIP events on `stream`.
+template <typename F>
+static int time_loop(F launch, int n_sets, int warmup, int iters, int use_graph, hipStream_t stream, float *elapsed_ms)
+{
+    if (iters <= 0 || warmup < 0 || n_sets <= 0 || !elapsed_ms) return fail(TUNA_ERR_INVALID_ARG, "bad timing arguments");
+    int rc;
+    hipError_t e;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    if ((e = hipEventCreate(&t0)) != hipSuccess) return hip_fail(e, "hipEventCreate");
+    if ((e = hipEventCreate(&t1)) != hipSuccess) {
+        (void)hipEventDestroy(t0);
+        return hip_fail(e, "hipEventCreate");
+    }
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    hipStream_t cap_stream = nullptr;
+    rc = TUNA_OK;
+    do {
+        for (int i = 0; i < warmup && !rc; ++i) rc = launch(i % n_sets, stream);
+        if (rc) break;
+        if (use_graph) {
+            // one rotation over the weight sets per graph launch; capture on a private
+            // stream so that the caller's stream (possibly the default one) is untouched
+            if ((e = hipStreamCreateWithFlags(&cap_stream, hipStreamNonBlocking)) != hipSuccess) { rc = hip_fail(e, "hipStreamCreate"); break; }
+            if ((e = hipStreamSynchronize(stream)) != hipSuccess) { rc = hip_fail(e, "hipStreamSynchronize"); break; }
+            for (int i = 0; i < n_sets && !rc; ++i) rc = launch(i, cap_stream);  // workspace for cap_stream grows here, before capture
+            if (rc) break;
+            if ((e = hipStreamSynchronize(cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipStreamSynchronize"); break; }
+            if ((e = hipStreamBeginCapture(cap_stream, hipStreamCaptureModeThreadLocal)) != hipSuccess) { rc = hip_fail(e, "hipStreamBeginCapture"); break; }
+            for (int i = 0; i < n_sets && !rc; ++i) rc = launch(i, cap_stream);
+            e = hipStreamEndCapture(cap_stream, &graph);
+            if (rc) break;
+            if (e != hipSuccess) { rc = hip_fail(e, "hipStreamEndCapture"); break; }
+            if ((e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0)) != hipSuccess) { rc = hip_fail(e, "hipGraphInstantiate"); break; }
+            const int reps = (iters + n_sets - 1) / n_sets;
+            if ((e = hipGraphLaunch(exec, cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipGraphLaunch"); break; }
+            if ((e = hipEventRecord(t0, cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipEventRecord"); break; }
+            for (int r = 0; r < reps; ++r)
+                if ((e = hipGraphLaunch(exec, cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipGraphLaunch"); break; }
+            if (rc) break;
+            if ((e = hipEventRecord(t1, cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipEventRecord"); break; }
+            if ((e = hipEventSynchronize(t1)) != hipSuccess) { rc = hip_fail(e, "hipEventSynchronize"); break; }
+            float ms = 0.f;
+            if ((e = hipEventElapsedTime(&ms, t0, t1)) != hipSuccess) { rc = hip_fail(e, "hipEventElapsedTime"); break; }
+            *elapsed_ms = ms * (float)iters / (float)(reps * n_sets);  // scaled to exactly `iters` launches
+        } else {
+            if ((e = hipEventRecord(t0, stream)) != hipSuccess) { rc = hip_fail(e, "hipEventRecord"); break; }
+            for (int i = 0; i < iters && !rc; ++i) rc = launch((warmup + i) % n_sets, stream);
+            if (rc) break;
+            if ((e = hipEventRecord(t1, stream)) != hipSuccess) { rc = hip_fail(e, "hipEventRecord"); break; }
+            if ((e = hipEventSynchronize(t1)) != hipSuccess) { rc = hip_fail(e, "hipEventSynchronize"); break; }
+            if ((e = hipEventElapsedTime(elapsed_ms, t0, t1)) != hipSuccess) { rc = hip_fail(e, "hipEventElapsedTime"); break; }
+        }
+    } while (0);
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    if (cap_stream) {
+        (void)hipStreamSynchronize(cap_stream);
+        drop_workspace(cap_stream);
+        (void)hipStreamDestroy(cap_stream);
+    }
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    return rc;
+}
+
+}  // namespace tuna
+
+using namespace tuna;
+
+extern "C" {
+
+#define TUNA_EXPORT __attribute__((visibility("default")))
+
+TUNA_EXPORT int tuna_version(void) { return TUNA_AMD_VERSION; }
+
+TUNA_EXPORT const char *tuna_status_string(int status)
+{
+    switch (status) {
+    case TUNA_OK: return "ok";
+    case TUNA_ERR_INVALID_ARG: return "invalid argument";
+    case TUNA_ERR_UNSUPPORTED: return "unsupported shape or config";
+    case TUNA_ERR_HIP: return "HIP runtime error";
+    case TUNA_ERR_NO_DEVICE: return "no usable device";
+    case TUNA_ERR_WORKSPACE: return "split-K workspace unavailable";
+    default: return "unknown status";
+    }
+}
+
+TUNA_EXPORT const char *tuna_last_error(void) { return g_error.c_str(); }
+
+TUNA_EXPORT int tuna_matmul(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n,
+                            int k, void *stream)
+{
+    return matmul_impl(q, x, code, absmax, out, m, n, k, nullptr, TUNA_DECODE_GEMM, static_cast<hipStream_t>(stream));
+}
+
+TUNA_EXPORT int tuna_matmul_ex(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n,
+                               int k, const tuna_gemm_config *cfg, int decode_mode, void *stream)
+{
+    return matmul_impl(q, x, code, absmax, out, m, n, k, cfg, decode_mode, static_cast<hipStream_t>(stream));
+}
+
+TUNA_EXPORT int tuna_dequant(const void *q, const void *absmax, const void *code, void *out, int m, int k, void *stream)
+{
+    return dequant_impl(q, absmax, code, out, m, k, TUNA_DECODE_DEQUANT, static_cast<hipStream_t>(stream));
+}
+
+TUNA_EXPORT int tuna_dequant_ex(const void *q, const void *absmax, const void *code, void *out, int m, int k,
+                                int decode_mode, void *stream)
+{
+    return dequant_impl(q, absmax, code, out, m, k, decode_mode, static_cast<hipStream_t>(stream));
+}
+
+TUNA_EXPORT int tuna_select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_table)
+{
+    if (!cfg) return fail(TUNA_ERR_INVALID_ARG, "cfg is null");
+    int rc = check_shape(m, n, k);
+    if (rc) return rc;
+    return select_config(m, n, k, cfg, from_table);
+}
+
+TUNA_EXPORT int tuna_validate_config(int m, int n, int k, const tuna_gemm_config *cfg)
+{
+    if (!cfg) return fail(TUNA_ERR_INVALID_ARG, "cfg is null");
+    GemmPlan plan;
+    return plan_gemm(m, n, k, *cfg, TUNA_DECODE_GEMM, &plan);
+}
+
+TUNA_EXPORT int tuna_config_footprint(int m, int n, int k, const tuna_gemm_config *cfg, size_t *lds_bytes,
+                                      size_t *workspace_bytes)
+{
+    if (!cfg) return fail(TUNA_ERR_INVALID_ARG, "cfg is null");
+    GemmPlan plan;
+    int rc = plan_gemm(m, n, k, *cfg, TUNA_DECODE_GEMM, &plan);
+    if (rc) return rc;
+    if (lds_bytes) *lds_bytes = plan.lds_bytes;
+    if (workspace_bytes) *workspace_bytes = plan.ws_bytes;
+    return TUNA_OK;
+}
+
+TUNA_EXPORT int tuna_config_table_size(void) { return kConfigTableSize; }
+
+TUNA_EXPORT int tuna_config_table_entry(int i, int *m, int *n_lo, int *n_hi, int *k, tuna_gemm_config *cfg)
+{
+    if (i < 0 || i >= kConfigTableSize) return fail(TUNA_ERR_INVALID_ARG, "table index %d out of range", i);
+    const TableEntry &e = kConfigTable[i];
+    if (m) *m = e.m;
+    if (n_lo) *n_lo = e.n_lo;
+    if (n_hi) *n_hi = e.n_hi;
+    if (k) *k = e.k;
+    if (cfg) *cfg = e.cfg;
+    return TUNA_OK;
+}
+
+TUNA_EXPORT int tuna_time_matmul(const void *const *q_list, const void *const *absmax_list, int n_sets, const void *x,
+                                 const void *code, void *out, int m, int n, int k, const tuna_gemm_config *cfg,
+                                 int decode_mode, int warmup, int iters, int use_graph, void *stream, float *elapsed_ms)
+{
+    if (!q_list || !absmax_list) return fail(TUNA_ERR_INVALID_ARG, "q_list / absmax_list is null");
+    auto launch = [&](int set, hipStream_t s) {
+        return matmul_impl(q_list[set], x, code, absmax_list[set], out, m, n, k, cfg, decode_mode, s);
+    };
+    return time_loop(launch, n_sets, warmup, iters, use_graph, static_cast<hipStream_t>(stream), elapsed_ms);
+}
+
+TUNA_EXPORT int tuna_time_dequant(const void *const *q_list, const void *const *absmax_list, int n_sets, const void *code,
+                                  void *out, int m, int k, int warmup, int iters, void *stream, float *elapsed_ms)
+{
+    if (!q_list || !absmax_list) return fail(TUNA_ERR_INVALID_ARG, "q_list / absmax_list is null");
+    auto launch = [&](int set, hipStream_t s) {
+        return dequant_impl(q_list[set], absmax_list[set], code, out, m, k, TUNA_DECODE_DEQUANT, s);
+    };
+    return time_loop(launch, n_sets, warmup, iters, 0, static_cast<hipStream_t>(stream), elapsed_ms);
+}
+
+TUNA_EXPORT int tuna_time_copy(const void *src, void *dst, size_t bytes, int warmup, int iters, void *stream,
+                               float *elapsed_ms)
+{
+    int rc;
+    if ((rc = check_ptr(src, "src", 16)) || (rc = check_ptr(dst, "dst", 16))) return rc;
+    if (bytes == 0 || bytes % 16) return fail(TUNA_ERR_INVALID_ARG, "bytes must be a positive multiple of 16");
+    auto launch = [&](int, hipStream_t s) {
+        hipError_t e = launch_copy(src, dst, bytes, s);
+        return e == hipSuccess ? (int)TUNA_OK : hip_fail(e, "copy launch");
+    };
+    return time_loop(launch, 1, warmup, iters, 0, static_cast<hipStream_t>(stream), elapsed_ms);
+}
+
+TUNA_EXPORT int tuna_release_workspaces(void)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    e = hipDeviceSynchronize();
+    if (e != hipSuccess) return hip_fail(e, "hipDeviceSynchronize");
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    for (auto it = g_workspaces.begin(); it != g_workspaces.end();) {
+        if (it->first.first == dev) {
+            if (it->second.ws) (void)hipFree(it->second.ws);
+            if (it->second.counters) (void)hipFree(it->second.counters);
+            it = g_workspaces.erase(it);
+        } else {
+            ++it;
+        }
+    }
+    return TUNA_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,116 @@
+// Packed 4-bit weights -> fp16 [m, k] row-major, for gfx950.
+//
+// Replaces dequantize_4bit / dequantize_wrapper (kernel.cu:3158-3253).  The op is a
+// pure stream (k*m/2 bytes in, 2*k*m bytes out), so the design is about HBM
+// transactions only:
+//   * a wave reads 1 KB of one block row with one global_load_dwordx4 per lane
+//     (lane l: block column kb0 + l/2, rows 4*(l%2) .. +3), nontemporal;
+//   * a dword is one weight row x 8 consecutive k, i.e. 16 bytes of output; lanes of
+//     equal parity write 512 contiguous bytes per output row, nontemporal.  No LDS
+//     transpose is needed (the reference needs one because its lanes own single bytes,
+//     kernel.cu:3218-3240);
+//   * decode: 16-entry fp32 (or fp16) table in LDS - all lanes hit 16 dwords in 16
+//     distinct banks, equal addresses broadcast, so it is conflict free - then
+//     fp32 multiply + round (TUNA_DECODE_DEQUANT, kernel.cu:3222-3228) or an fp16
+//     multiply (TUNA_DECODE_GEMM, kernel.cu:2178-2192).
+#include "tuna_internal.h"
+
+namespace tuna {
+
+typedef _Float16 f16;
+typedef f16 f16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kDqUnroll = 4;  // 1 KB chunks per wave
+
+template <int DEC>
+__global__ __launch_bounds__(256) void dequant_kernel(const uint8_t *__restrict__ q,
+                                                      const float *__restrict__ absmax,
+                                                      const float *__restrict__ code,
+                                                      f16 *__restrict__ out, int m, int k)
+{
+    __shared__ float cf[16];
+    __shared__ f16 ch[16];
+    const int tid = threadIdx.x;
+    if (tid < 16) {
+        cf[tid] = code[tid];
+        ch[tid] = (f16)code[tid];
+    }
+    __syncthreads();
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int kb_total = k >> 3;
+    const int mb = blockIdx.y * 4 + wave;
+    if (mb >= (m >> 3)) return;
+    const int half = lane & 1;
+    const int kb_lane = blockIdx.x * (32 * kDqUnroll) + (lane >> 1);
+
+    float s32[4];
+    f16 s16[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        s32[j] = absmax[mb * 8 + half * 4 + j];
+        s16[j] = (f16)s32[j];
+    }
+    const uint8_t *src = q + ((size_t)mb * kb_total) * 32 + half * 16;
+    u32x4 w[kDqUnroll];
+#pragma unroll
+    for (int u = 0; u < kDqUnroll; ++u) {
+        const int kb = kb_lane + u * 32;
+        if (kb < kb_total) w[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + (size_t)kb * 32));
+    }
+#pragma unroll
+    for (int u = 0; u < kDqUnroll; ++u) {
+        const int kb = kb_lane + u * 32;
+        if (kb >= kb_total) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t d = w[u][j];
+            f16x8 r;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                // column e of the row sits at bit 8*(e/2) + 4*(1 - e%2)  (test.py:58-65)
+                const uint32_t nib = (d >> (8 * (e >> 1) + 4 * (1 - (e & 1)))) & 15u;
+                if constexpr (DEC == TUNA_DECODE_DEQUANT) r[e] = (f16)(cf[nib] * s32[j]);
+                else r[e] = ch[nib] * s16[j];
+            }
+            f16 *dst = out + (size_t)(mb * 8 + half * 4 + j) * k + (size_t)kb * 8;
+            __builtin_nontemporal_store(r, reinterpret_cast<f16x8 *>(dst));
+        }
+    }
+}
+
+hipError_t launch_dequant(const uint8_t *q, const float *absmax, const float *code, void *out,
+                          int m, int k, int decode, hipStream_t stream)
+{
+    const int kb_total = k >> 3;
+    dim3 grid((kb_total + 32 * kDqUnroll - 1) / (32 * kDqUnroll), ((m >> 3) + 3) / 4, 1);
+    if (decode == TUNA_DECODE_DEQUANT)
+        hipLaunchKernelGGL(dequant_kernel<TUNA_DECODE_DEQUANT>, grid, dim3(256), 0, stream, q, absmax, code,
+                           reinterpret_cast<f16 *>(out), m, k);
+    else
+        hipLaunchKernelGGL(dequant_kernel<TUNA_DECODE_GEMM>, grid, dim3(256), 0, stream, q, absmax, code,
+                           reinterpret_cast<f16 *>(out), m, k);
+    return hipGetLastError();
+}
+
+// Plain copy: the known-traffic yardstick for the HBM counters.
+__global__ __launch_bounds__(256) void copy_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst, size_t n16)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
+hipError_t launch_copy(const void *src, void *dst, size_t bytes, hipStream_t stream)
+{
+    const size_t n16 = bytes / 16;
+    size_t blocks = (n16 + 255) / 256;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    if (blocks == 0) blocks = 1;
+    hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
+                       reinterpret_cast<const u32x4 *>(src), reinterpret_cast<u32x4 *>(dst), n16);
+    return hipGetLastError();
+}
+
+}  // namespace tuna

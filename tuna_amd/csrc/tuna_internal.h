@@ -1,0 +1,67 @@
+// Internal declarations shared by the host API and the gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/tuna_amd.h"
+
+namespace tuna {
+
+// LDS byte-pair lookup table: 256 rows (one per packed byte value) x 64 copies
+// (one per lane) of a half2 {code[byte >> 4], code[byte & 15]}.  Row stride is 256
+// bytes so a lane's address is (byte << 8) | (lane << 2): every lane of a wave reads
+// its own bank column, whatever the data.
+constexpr int kLutBytes = 256 * 64 * 4;
+constexpr int kLdsLimit = 160 * 1024;
+constexpr int kStepK = 32;          // k per MFMA step (v_mfma_f32_16x16x32_f16)
+constexpr int kRowsPerLoad = 64;    // weight rows covered by one 128-bit load per lane
+constexpr int kMaxThreads = 1024;
+
+// Everything a GEMM launch needs, filled by the host from a tuna_gemm_config.
+struct GemmArgs {
+    const uint8_t *q;
+    const void *x;
+    const float *code;
+    const float *absmax;
+    void *out;
+    float *ws;           // split-K partial sums (library owned), may be null if split_k == 1
+    unsigned *counters;  // one arrival counter per (token chunk, row tile), zero between launches
+    int m, n, k;
+    int waves_m, waves_k, split_k;
+    int steps_total;      // ceil(k / 32)
+    int steps_per_split;  // k-steps owned by one workgroup
+    int chunk_steps;      // k-steps of x staged in LDS at a time
+    int row_tiles;        // workgroups along m
+    int xcd_swizzle;
+    int lds_bytes;        // dynamic LDS size of the launch (last 16 bytes: arrival ticket)
+};
+
+struct GemmPlan {
+    GemmArgs args;
+    dim3 grid;
+    int threads;
+    int rw, prefetch, token_tiles, decode;
+    size_t lds_bytes;
+    size_t ws_bytes;
+    size_t n_counters;
+};
+
+// gemm_kernel.hip
+hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream);
+bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads);
+
+// dequant_kernel.hip
+hipError_t launch_dequant(const uint8_t *q, const float *absmax, const float *code, void *out,
+                          int m, int k, int decode, hipStream_t stream);
+hipError_t launch_copy(const void *src, void *dst, size_t bytes, hipStream_t stream);
+
+// config_table.cpp
+struct TableEntry {
+    int m, n_lo, n_hi, k;
+    tuna_gemm_config cfg;
+};
+extern const TableEntry kConfigTable[];
+extern const int kConfigTableSize;
+
+}  // namespace tuna

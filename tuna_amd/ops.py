@@ -1,0 +1,169 @@
+"""The two ops of the reference's extension, on PyTorch-ROCm tensors.
+
+Mirror of extension.cpp:26-55: ``matmul(x, q, s, c, o, m, n, k)`` and
+``dequant(q, absmax, codebook, o, m, k)``, both returning None and writing into the
+caller's ``o`` on the current stream of the tensors' device.  Unlike the reference,
+which performs no checks at all (extension.cpp:26-38), wrong dtypes, shapes, devices
+or non-contiguous tensors raise instead of invoking undefined behaviour, and shapes
+outside the tuned table run on a derived config instead of silently doing nothing
+(kernel.cu:3018-3156).
+
+PyTorch is only the carrier of device memory and streams here; the work happens in
+libtuna_amd.so behind the C ABI of include/tuna_amd.h.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import GemmConfig, TunaError  # noqa: F401  (re-exported)
+
+
+def _require(t: torch.Tensor, name: str, dtype: torch.dtype, numel: int) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if t.device.type != "cuda":
+        raise ValueError(f"{name} must live on a HIP device (got {t.device})")
+    if t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype} (got {t.dtype})")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if t.numel() != numel:
+        raise ValueError(f"{name} has {t.numel()} elements, expected {numel}")
+
+
+def _stream(dev: torch.device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def matmul(x, q, s, c, o, m: int, n: int, k: int, config: GemmConfig = None,
+           decode_mode: int = _lib.DECODE_GEMM) -> None:
+    """o[n, m] = x[n, k] @ decode(q, c, s)[m, k]^T  (extension.cpp:26-38).
+
+    x fp16 [n, k]; q uint8 [m/8, k/8, 32]; s fp32 [m] (absmax per weight row);
+    c fp32 [16] (codebook); o fp16 [n, m], overwritten.
+    """
+    m, n, k = int(m), int(n), int(k)
+    if m <= 0 or n <= 0 or k <= 0 or m % 8 or k % 8:
+        raise ValueError(f"m and k must be positive multiples of 8 and n positive (m={m}, n={n}, k={k})")
+    _require(x, "x", torch.float16, n * k)
+    _require(q, "q", torch.uint8, m * k // 2)
+    _require(s, "s", torch.float32, m)
+    _require(c, "c", torch.float32, 16)
+    _require(o, "o", torch.float16, n * m)
+    for name, t in (("q", q), ("s", s), ("c", c), ("o", o)):
+        if t.device != x.device:
+            raise ValueError(f"{name} is on {t.device}, x on {x.device}")
+    L = _lib.lib()
+    with torch.cuda.device(x.device):
+        if config is None and decode_mode == _lib.DECODE_GEMM:
+            rc = L.tuna_matmul(q.data_ptr(), x.data_ptr(), c.data_ptr(), s.data_ptr(), o.data_ptr(), m, n, k,
+                               _stream(x.device))
+        else:
+            rc = L.tuna_matmul_ex(q.data_ptr(), x.data_ptr(), c.data_ptr(), s.data_ptr(), o.data_ptr(), m, n, k,
+                                  ctypes.byref(config) if config is not None else None, int(decode_mode),
+                                  _stream(x.device))
+    _lib.check(rc)
+
+
+def dequant(q, absmax, codebook, o, m: int, k: int, decode_mode: int = _lib.DECODE_DEQUANT) -> None:
+    """o[m, k] = decode(q, codebook, absmax) as fp16  (extension.cpp:40-49)."""
+    m, k = int(m), int(k)
+    if m <= 0 or k <= 0 or m % 8 or k % 8:
+        raise ValueError(f"m and k must be positive multiples of 8 (m={m}, k={k})")
+    _require(q, "q", torch.uint8, m * k // 2)
+    _require(absmax, "absmax", torch.float32, m)
+    _require(codebook, "codebook", torch.float32, 16)
+    _require(o, "o", torch.float16, m * k)
+    for name, t in (("absmax", absmax), ("codebook", codebook), ("o", o)):
+        if t.device != q.device:
+            raise ValueError(f"{name} is on {t.device}, q on {q.device}")
+    L = _lib.lib()
+    with torch.cuda.device(q.device):
+        if decode_mode == _lib.DECODE_DEQUANT:
+            rc = L.tuna_dequant(q.data_ptr(), absmax.data_ptr(), codebook.data_ptr(), o.data_ptr(), m, k,
+                                _stream(q.device))
+        else:
+            rc = L.tuna_dequant_ex(q.data_ptr(), absmax.data_ptr(), codebook.data_ptr(), o.data_ptr(), m, k,
+                                   int(decode_mode), _stream(q.device))
+    _lib.check(rc)
+
+
+def select_config(m: int, n: int, k: int):
+    """(GemmConfig, from_table) the library would use for shape (m, n, k).  Host only."""
+    cfg = GemmConfig()
+    hit = ctypes.c_int(0)
+    _lib.check(_lib.lib().tuna_select_config(int(m), int(n), int(k), ctypes.byref(cfg), ctypes.byref(hit)))
+    return cfg, bool(hit.value)
+
+
+def validate_config(m: int, n: int, k: int, cfg: GemmConfig) -> None:
+    """Raises TunaError unless `cfg` can run shape (m, n, k).  Host only."""
+    _lib.check(_lib.lib().tuna_validate_config(int(m), int(n), int(k), ctypes.byref(cfg)))
+
+
+def config_footprint(m: int, n: int, k: int, cfg: GemmConfig):
+    """(dynamic LDS bytes, split-K workspace bytes) of a launch.  Host only."""
+    lds, ws = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    _lib.check(_lib.lib().tuna_config_footprint(int(m), int(n), int(k), ctypes.byref(cfg), ctypes.byref(lds),
+                                                ctypes.byref(ws)))
+    return lds.value, ws.value
+
+
+def config_table():
+    """The built-in tuned table as a list of (m, n_lo, n_hi, k, GemmConfig)."""
+    L = _lib.lib()
+    out = []
+    for i in range(L.tuna_config_table_size()):
+        m, lo, hi, k = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        cfg = GemmConfig()
+        _lib.check(L.tuna_config_table_entry(i, ctypes.byref(m), ctypes.byref(lo), ctypes.byref(hi), ctypes.byref(k),
+                                             ctypes.byref(cfg)))
+        out.append((m.value, lo.value, hi.value, k.value, cfg))
+    return out
+
+
+def _ptr_array(tensors):
+    arr = (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+    return ctypes.cast(arr, ctypes.POINTER(ctypes.c_void_p)), arr
+
+
+def time_matmul(q_list, absmax_list, x, c, o, m, n, k, config=None, decode_mode=_lib.DECODE_GEMM, warmup=10,
+                iters=100, use_graph=False) -> float:
+    """Milliseconds for `iters` GEMMs rotating over the weight sets, measured with HIP
+    events on the current stream (tuna_time_matmul).  Synchronises."""
+    assert len(q_list) == len(absmax_list) and len(q_list) > 0
+    qp, _qk = _ptr_array(q_list)
+    ap, _ak = _ptr_array(absmax_list)
+    ms = ctypes.c_float(0)
+    L = _lib.lib()
+    with torch.cuda.device(x.device):
+        rc = L.tuna_time_matmul(qp, ap, len(q_list), x.data_ptr(), c.data_ptr(), o.data_ptr(), int(m), int(n), int(k),
+                                ctypes.byref(config) if config is not None else None, int(decode_mode), int(warmup),
+                                int(iters), int(bool(use_graph)), _stream(x.device), ctypes.byref(ms))
+    _lib.check(rc)
+    return ms.value
+
+
+def time_dequant(q_list, absmax_list, c, o, m, k, warmup=5, iters=20) -> float:
+    qp, _qk = _ptr_array(q_list)
+    ap, _ak = _ptr_array(absmax_list)
+    ms = ctypes.c_float(0)
+    L = _lib.lib()
+    with torch.cuda.device(o.device):
+        rc = L.tuna_time_dequant(qp, ap, len(q_list), c.data_ptr(), o.data_ptr(), int(m), int(k), int(warmup),
+                                 int(iters), _stream(o.device), ctypes.byref(ms))
+    _lib.check(rc)
+    return ms.value
+
+
+def time_copy(src, dst, warmup=5, iters=20) -> float:
+    nbytes = src.numel() * src.element_size()
+    assert dst.numel() * dst.element_size() >= nbytes
+    ms = ctypes.c_float(0)
+    L = _lib.lib()
+    with torch.cuda.device(src.device):
+        rc = L.tuna_time_copy(src.data_ptr(), dst.data_ptr(), nbytes, int(warmup), int(iters), _stream(src.device),
+                              ctypes.byref(ms))
+    _lib.check(rc)
+    return ms.value
