@@ -1,0 +1,252 @@
+#!/usr/bin/env python3
+"""Benchmark of the FP16 x 4-bit GEMM on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one GEMM of the headline workload (Mistral-7B QKV projection at 16 tokens:
+out[16, 6144] = x[16, 4096] . W[6144, 4096]^T, BASELINE config 1) on one of a rotating set
+of distinct, HBM-resident weight matrices, so that neither L2 nor the 256 MB Infinity Cache
+can serve re-reads.  W warm-up steps, then exactly K timed steps bracketed by HIP events on
+the launch stream (tuna_time_matmul, inside the C library, so that no Python overhead sits
+between launches).  One JSON line is printed:
+
+  value        packed-weight bytes (m*k/2) per second, GB/s  - the roofline quantity
+  ms_per_step  milliseconds per GEMM (x1000 = the metric's "us/GEMM")
+  roofline     achieved / peak HBM bandwidth for the GEMM kernel (algorithmic bytes = m*k/2)
+  cpu_baseline the CPU oracle's dequantize-then-matmul on the same workload, host cores
+  shapes       the same measurement for every 16-token layer shape of the BASELINE configs
+  sweeps       Llama-70B 80-layer sweep (distinct weights per layer) and the token sweep
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+METRIC = "us/GEMM + HBM GB/s (frac of ~8 TB/s) at M=16, Mistral/Llama-70B shapes"
+HEADLINE = "mistral_qkv"
+TOKENS = 16
+CACHE_BYTES = 256 << 20  # Infinity Cache; the rotation streams at least twice this between re-uses
+
+# HBM bytes per launch of the GEMM kernel measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE,
+# each scaled by the same counter's reading for the copy kernel of known size); filled in from
+# the summaries under profiles/.  None = not measured for that shape.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def n_sets_for(bytes_per_set: int, cap_bytes: int) -> int:
+    n = max(2, -(-2 * CACHE_BYTES // bytes_per_set))
+    return max(2, min(n, max(2, cap_bytes // bytes_per_set)))
+
+
+def time_shape(ops, synth, torch, dev, m, n, k, steps, warmup, seed0=0, use_graph=False, cfg=None, sets=None):
+    """-> dict with us_per_gemm, GB/s, TFLOP/s, roofline fraction for one shape."""
+    bytes_w = m * k // 2
+    if sets is None:
+        ns = n_sets_for(bytes_w, 24 << 30)
+        sets = [synth.make_weights_torch(m, k, seed0 + i, dev) for i in range(ns)]
+    qs = [s[0] for s in sets]
+    ams = [s[1] for s in sets]
+    x = synth.make_x_torch(n, k, seed0, dev)
+    from tuna_amd.quantize import nf4_codebook
+
+    code = nf4_codebook(dev)
+    out = torch.empty((n, m), dtype=torch.float16, device=dev)
+    torch.cuda.synchronize()
+    ms = ops.time_matmul(qs, ams, x, code, out, m, n, k, config=cfg, warmup=warmup, iters=steps, use_graph=use_graph)
+    us = ms * 1000.0 / steps
+    gbs = bytes_w / (us * 1e-6) / 1e9
+    used, hit = ops.select_config(m, n, k)
+    return {
+        "m": m, "n": n, "k": k, "packed_bytes": bytes_w, "weight_sets": len(qs),
+        "us_per_gemm": round(us, 3), "gbs": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
+        "tflops": round(2.0 * m * n * k / (us * 1e-6) / 1e12, 2),
+        "config": (cfg or used).to_dict(), "config_from_table": bool(hit) if cfg is None else None,
+        "launch": "graph" if use_graph else "stream",
+    }
+
+
+def cpu_baseline(m, n, k, budget_s=12.0):
+    """The oracle's dequantize (D2) + fp32 matmul on the host cores (checker code timed as a
+    reported baseline only)."""
+    import numpy as np
+
+    from oracle import oracle as O
+    from tuna_amd.synth import make_inputs_np
+
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=0)
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        cores = os.cpu_count() or 1
+    cores = max(1, min(cores, O.max_threads() if O.max_threads() > 0 else cores))
+    xb = x.view(np.uint16)
+    # single-thread figure (one pass) and the all-cores figure (median over the budget)
+    _, td1, tm1, _ = O.cpu_baseline(q, xb, code, absmax, m, n, k, threads=1)
+    times, dec, mat = [], [], []
+    O.cpu_baseline(q, xb, code, absmax, m, n, k, threads=cores)  # warm-up
+    t_end = time.perf_counter() + budget_s
+    while time.perf_counter() < t_end or len(times) < 3:
+        _, td, tm, _ = O.cpu_baseline(q, xb, code, absmax, m, n, k, threads=cores)
+        times.append(td + tm)
+        dec.append(td)
+        mat.append(tm)
+        if len(times) >= 200:
+            break
+    med = float(np.median(times))
+    bytes_w = m * k // 2
+    return {
+        "value": round(bytes_w / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+        "sample": f"{len(times)} full GEMMs m={m} n={n} k={k} (decode to fp16, then fp32-accumulate matmul), "
+                  f"median of total; oracle/tuna_oracle.c with OpenMP",
+        "us_per_gemm": round(med * 1e6, 1), "us_decode": round(float(np.median(dec)) * 1e6, 1),
+        "us_matmul": round(float(np.median(mat)) * 1e6, 1),
+        "single_thread_us_per_gemm": round((td1 + tm1) * 1e6, 1),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--no-shapes", action="store_true", help="skip the per-shape table")
+    ap.add_argument("--no-sweeps", action="store_true", help="skip the 80-layer and token sweeps")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--only-headline", action="store_true", help="headline workload only (profiling runs)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+    if args.only_headline:
+        args.no_shapes = args.no_sweeps = args.no_cpu = True
+
+    import torch
+
+    from tuna_amd import ops, synth
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a HIP device", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    m, k = synth.SHAPES[HEADLINE]
+    n = TOKENS
+    res_stream = time_shape(ops, synth, torch, dev, m, n, k, args.steps, args.warmup, use_graph=False)
+    res_graph = time_shape(ops, synth, torch, dev, m, n, k, args.steps, args.warmup, use_graph=True)
+    head = res_graph if res_graph["us_per_gemm"] < res_stream["us_per_gemm"] else res_stream
+
+    line = {
+        "metric": METRIC,
+        "value": head["gbs"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(head["us_per_gemm"] / 1000.0, 6),
+        "us_per_gemm": head["us_per_gemm"],
+        "tflops": head["tflops"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"BASELINE config 1: Mistral-7B QKV projection, M={n} tokens, K={k}, N={m}; "
+                        f"uniform 4-bit codes, fp16 scales U(0.005,0.02), x ~ N(0,1)*0.1; "
+                        f"{head['weight_sets']} distinct weight matrices rotated",
+            "tile_config": head["config"],
+            "launch": head["launch"],
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": head["gbs"],
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(head["gbs"] / HBM_PEAK_GBS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(HEADLINE),
+            "kernel": "tuna::gemm_kernel",
+            "algorithmic_bytes_per_launch": head["packed_bytes"],
+            "avg_launch_us": head["us_per_gemm"],
+        },
+        "headline_stream_launch": res_stream,
+        "headline_graph_launch": res_graph,
+    }
+
+    if not args.no_shapes:
+        shapes = {}
+        steps = max(50, min(args.steps, 300))
+        for name, (sm, sk) in synth.SHAPES.items():
+            r_s = time_shape(ops, synth, torch, dev, sm, n, sk, steps, max(10, args.warmup // 5), seed0=1000)
+            r_g = time_shape(ops, synth, torch, dev, sm, n, sk, steps, max(10, args.warmup // 5), seed0=1000,
+                             use_graph=True)
+            best = r_g if r_g["us_per_gemm"] < r_s["us_per_gemm"] else r_s
+            best["us_stream"] = r_s["us_per_gemm"]
+            best["us_graph"] = r_g["us_per_gemm"]
+            shapes[name] = best
+            torch.cuda.empty_cache()
+        line["shapes"] = shapes
+        line["min_frac_hbm_over_shapes"] = min(v["frac_hbm"] for v in shapes.values())
+        # dequant kernel (k*m/2 bytes in, 2*k*m bytes out) on the 4096 x 4096 config
+        from tuna_amd.quantize import nf4_codebook
+
+        dm, dk = synth.SHAPES["mistral_attn_out"]
+        sets = [synth.make_weights_torch(dm, dk, 50 + i, dev) for i in range(8)]
+        img = torch.empty((dm, dk), dtype=torch.float16, device=dev)
+        ms = ops.time_dequant([s[0] for s in sets], [s[1] for s in sets], nf4_codebook(dev), img, dm, dk, 10, 100)
+        us = ms * 10.0
+        line["dequant"] = {"m": dm, "k": dk, "us": round(us, 2),
+                           "gbs_in_plus_out": round(2.5 * dm * dk / (us * 1e-6) / 1e9, 1),
+                           "frac_hbm": round(2.5 * dm * dk / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+
+    if not args.no_sweeps:
+        sweeps = {}
+        # Llama-70B decoder layer x 80 layers, distinct seeded weights per layer (34.2 GB resident)
+        names = ["llama70b_qkv", "llama70b_attn_out", "llama70b_gate_up", "llama70b_down"]
+        try:
+            layer_us = {}
+            total_bytes = 0
+            for nm in names:
+                sm, sk = synth.SHAPES[nm]
+                sets = [synth.make_weights_torch(sm, sk, 10_000 + layer, dev) for layer in range(80)]
+                r = time_shape(ops, synth, torch, dev, sm, n, sk, 160, 80, sets=sets, use_graph=True)
+                layer_us[nm] = r["us_per_gemm"]
+                total_bytes += sm * sk // 2
+                del sets
+                torch.cuda.empty_cache()
+            tot = sum(layer_us.values())
+            sweeps["llama70b_80_layers"] = {
+                "us_per_gemm": layer_us, "us_per_layer": round(tot, 2), "ms_80_layers": round(tot * 80 / 1000, 3),
+                "packed_bytes_per_layer": total_bytes, "gbs": round(total_bytes / (tot * 1e-6) / 1e9, 1),
+                "frac_hbm": round(total_bytes / (tot * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            }
+        except torch.OutOfMemoryError as e:  # pragma: no cover
+            sweeps["llama70b_80_layers"] = {"error": str(e)[:200]}
+        # token sweep on the Llama-70B layer set
+        tok = {}
+        for nt in (1, 16, 64, 256):
+            row = {}
+            for nm in names:
+                sm, sk = synth.SHAPES[nm]
+                r = time_shape(ops, synth, torch, dev, sm, nt, sk, 100, 20, seed0=2000, use_graph=True)
+                row[nm] = {"us": r["us_per_gemm"], "gbs": r["gbs"], "tflops": r["tflops"]}
+                torch.cuda.empty_cache()
+            tok[str(nt)] = row
+        sweeps["token_sweep_llama70b"] = tok
+        line["sweeps"] = sweeps
+
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(m, n, k)
+    else:
+        line["cpu_baseline"] = None
+
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

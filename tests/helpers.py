@@ -9,16 +9,25 @@ from tuna_amd.synth import make_inputs_np
 # outputs are sums of ~k zero-mean terms, so a few land arbitrarily close to zero, where a
 # pure ratio is meaningless; below FLOOR (0.1 % of the largest output) the error is measured
 # against that floor instead.
+#
+# Two floors are used.  Against the oracle GEMM with the SAME decode as the kernel (D1) the
+# floor is 1e-3: only accumulation order and the final fp16 rounding differ.  Against the
+# reference's dequantize-then-matmul (D2 weights) the floor is 5e-2: the reference's two
+# decodes differ by one fp16 ulp on ~20 % of the weights, which by itself moves exact
+# float64 outputs by 2.7e-4 of the largest output - 13 % of an output near zero under the
+# 1e-3 floor, 0.5 % under the 5e-2 floor (measured on the 4096 x 4096 config with the oracle
+# alone), so no kernel with the reference GEMM's decode can meet 1e-2 under a tighter floor.
 REL_TOL = 1e-2
 REL_FLOOR = 1e-3
+REL_FLOOR_D2 = 5e-2
 
 
-def rel_err(y, y_ref):
+def rel_err(y, y_ref, floor=REL_FLOOR):
     """Max relative error as defined above; y, y_ref are float64 arrays of one shape."""
     y = np.asarray(y, np.float64)
     y_ref = np.asarray(y_ref, np.float64)
     scale = np.abs(y_ref).max() if y_ref.size else 0.0
-    den = np.maximum(np.abs(y_ref), REL_FLOOR * scale)
+    den = np.maximum(np.abs(y_ref), floor * scale)
     den[den == 0] = 1.0
     return float((np.abs(y - y_ref) / den).max()) if y.size else 0.0
 
@@ -69,5 +78,5 @@ def run_dequant(q, code, absmax, m, k, decode_mode=2):
     return out.cpu().numpy().view(np.uint16)
 
 
-__all__ = ["O", "make_inputs_np", "rel_err", "REL_TOL", "f16_bits_to_f64", "ulp_diff_f16", "to_dev", "run_gemm",
+__all__ = ["O", "make_inputs_np", "rel_err", "REL_TOL", "REL_FLOOR_D2", "f16_bits_to_f64", "ulp_diff_f16", "to_dev", "run_gemm",
            "run_dequant"]

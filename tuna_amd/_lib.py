@@ -94,6 +94,12 @@ def lib():
             raise RuntimeError(
                 f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
                 "or `make -C tuna_amd/csrc`; tuna_amd has no non-HIP fallback")
+        # The HIP runtime must be the one PyTorch-ROCm already uses in this process (torch
+        # bundles its own libamdhip64): load torch first so that this library binds to it.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = ctypes.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(L, name)  # AttributeError if the library lacks a declared symbol

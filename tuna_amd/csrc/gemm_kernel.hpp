@@ -295,27 +295,36 @@ __global__ __launch_bounds__(MAXT) void gemm_kernel(const GemmArgs a)
     }
 
     // ---- reduce across the split_k workgroups through the workspace --------------------
+    // Partials travel as device-scope relaxed atomics (write-through stores, L2-bypassing
+    // loads): they are coherent across the 8 XCD L2s without the L2 write-back/invalidate
+    // that a device-scope release/acquire fence costs on every workgroup.  Order is given by
+    // "all my stores have completed" (workgroup-scope release = s_waitcnt vmcnt(0)) before
+    // the barrier that precedes the arrival counter's atomic increment.
     if (a.split_k > 1) {
         const size_t tile = (size_t)blockIdx.y * a.row_tiles + row_tile;
-        f32x4 *wst = reinterpret_cast<f32x4 *>(a.ws) + (tile * a.split_k * a.waves_m) * NACC * 64;
+        float *wst = a.ws + (tile * a.split_k * a.waves_m) * (size_t)(NACC * 256);
         if (wk == 0) {
-            f32x4 *dst = wst + ((size_t)(ks * a.waves_m + wm) * NACC) * 64 + lane;
+            float *dst = wst + ((size_t)(ks * a.waves_m + wm) * NACC) * 256 + lane;
 #pragma unroll
             for (int rw = 0; rw < RW; ++rw)
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
 #pragma unroll
-                    for (int tt = 0; tt < TT; ++tt) dst[((rw * 4 + j) * TT + tt) * 64] = acc[rw][j][tt];
+                    for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+                        for (int v = 0; v < 4; ++v)
+                            __hip_atomic_store(dst + (((rw * 4 + j) * TT + tt) * 4 + v) * 64, acc[rw][j][tt][v],
+                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         }
-        __threadfence();
         __syncthreads();
         volatile unsigned *ticket = reinterpret_cast<volatile unsigned *>(smem + a.lds_bytes - 16);
         if (tid == 0)
-            *ticket = __hip_atomic_fetch_add(a.counters + tile, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+            *ticket = __hip_atomic_fetch_add(a.counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (*ticket != (unsigned)(a.split_k - 1)) return;
-        __threadfence();
-        if (tid == 0) a.counters[tile] = 0u;  // ready for the next launch on this stream
+        // last workgroup of this tile: every partial is in memory; sum them in split order
+        if (tid == 0) __hip_atomic_store(a.counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (wk == 0) {
 #pragma unroll
             for (int rw = 0; rw < RW; ++rw)
@@ -324,14 +333,17 @@ __global__ __launch_bounds__(MAXT) void gemm_kernel(const GemmArgs a)
 #pragma unroll
                     for (int tt = 0; tt < TT; ++tt) acc[rw][j][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
             for (int s = 0; s < a.split_k; ++s) {
-                const f32x4 *src = wst + ((size_t)(s * a.waves_m + wm) * NACC) * 64 + lane;
+                const float *src = wst + ((size_t)(s * a.waves_m + wm) * NACC) * 256 + lane;
 #pragma unroll
                 for (int rw = 0; rw < RW; ++rw)
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
 #pragma unroll
                         for (int tt = 0; tt < TT; ++tt)
-                            acc[rw][j][tt] += __builtin_nontemporal_load(src + ((rw * 4 + j) * TT + tt) * 64);
+#pragma unroll
+                            for (int v = 0; v < 4; ++v)
+                                acc[rw][j][tt][v] += __hip_atomic_load(src + (((rw * 4 + j) * TT + tt) * 4 + v) * 64,
+                                                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
     }

@@ -16,14 +16,18 @@ struct Variant {
 #define V_TT(RW, U, MAXT) V(RW, U, 1, TUNA_DECODE_GEMM, MAXT), V(RW, U, 2, TUNA_DECODE_GEMM, MAXT), V(RW, U, 4, TUNA_DECODE_GEMM, MAXT)
 
 static const Variant kVariants[] = {
+    // Only variants that compile without register spills are listed (checked with
+    // -Rpass-analysis=kernel-resource-usage); tuna_amd/make_configs.py mirrors this list.
     // rows_per_wave = 64
     V_TT(1, 2, 512), V_TT(1, 4, 512), V_TT(1, 8, 512),
-    // rows_per_wave = 128 (prefetch 8 x 4 token tiles does not fit the register file)
-    V_TT(2, 2, 512), V_TT(2, 4, 512), V(2, 8, 1, TUNA_DECODE_GEMM, 512), V(2, 8, 2, TUNA_DECODE_GEMM, 512),
+    // rows_per_wave = 128
+    V(2, 2, 1, TUNA_DECODE_GEMM, 512), V(2, 2, 2, TUNA_DECODE_GEMM, 512),
+    V(2, 4, 1, TUNA_DECODE_GEMM, 512), V(2, 4, 2, TUNA_DECODE_GEMM, 512),
+    V(2, 8, 1, TUNA_DECODE_GEMM, 512),
     // rows_per_wave = 256
-    V(4, 2, 1, TUNA_DECODE_GEMM, 512), V(4, 2, 2, TUNA_DECODE_GEMM, 512), V(4, 4, 1, TUNA_DECODE_GEMM, 512),
+    V(4, 2, 1, TUNA_DECODE_GEMM, 512),
     // 16-wave workgroups (128 VGPRs per lane): single token tile only
-    V(1, 4, 1, TUNA_DECODE_GEMM, 1024), V(1, 8, 1, TUNA_DECODE_GEMM, 1024), V(2, 4, 1, TUNA_DECODE_GEMM, 1024),
+    V(1, 4, 1, TUNA_DECODE_GEMM, 1024), V(1, 8, 1, TUNA_DECODE_GEMM, 1024),
     // dequant-rounding decode (correctness mode, not tuned)
     V(1, 2, 1, TUNA_DECODE_DEQUANT, 512), V(1, 2, 2, TUNA_DECODE_DEQUANT, 512), V(1, 2, 4, TUNA_DECODE_DEQUANT, 512),
 };
