@@ -118,6 +118,9 @@ def main():
     ap.add_argument("--no-sweeps", action="store_true", help="skip the 80-layer and token sweeps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only-headline", action="store_true", help="headline workload only (profiling runs)")
+    ap.add_argument("--workload", default=HEADLINE, help="shape name timed as the headline (profiling runs)")
+    ap.add_argument("--tokens", type=int, default=TOKENS, help="token count of the headline workload")
+    ap.add_argument("--launch", choices=("both", "stream", "graph"), default="both")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
@@ -135,11 +138,15 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    m, k = synth.SHAPES[HEADLINE]
-    n = TOKENS
-    res_stream = time_shape(ops, synth, torch, dev, m, n, k, args.steps, args.warmup, use_graph=False)
-    res_graph = time_shape(ops, synth, torch, dev, m, n, k, args.steps, args.warmup, use_graph=True)
-    head = res_graph if res_graph["us_per_gemm"] < res_stream["us_per_gemm"] else res_stream
+    m, k = synth.SHAPES[args.workload]
+    n = args.tokens
+    res_stream = res_graph = None
+    if args.launch in ("both", "stream"):
+        res_stream = time_shape(ops, synth, torch, dev, m, n, k, args.steps, args.warmup, use_graph=False)
+    if args.launch in ("both", "graph"):
+        res_graph = time_shape(ops, synth, torch, dev, m, n, k, args.steps, args.warmup, use_graph=True)
+    cands = [r for r in (res_stream, res_graph) if r is not None]
+    head = min(cands, key=lambda r: r["us_per_gemm"])
 
     line = {
         "metric": METRIC,
@@ -157,7 +164,8 @@ def main():
         "dtype": "f16",
         "data": "synthetic",
         "config": {
-            "workload": f"BASELINE config 1: Mistral-7B QKV projection, M={n} tokens, K={k}, N={m}; "
+            "workload": f"{'BASELINE config 1: Mistral-7B QKV projection' if args.workload == HEADLINE else args.workload}, "
+                        f"M={n} tokens, K={k}, N={m}; "
                         f"uniform 4-bit codes, fp16 scales U(0.005,0.02), x ~ N(0,1)*0.1; "
                         f"{head['weight_sets']} distinct weight matrices rotated",
             "tile_config": head["config"],
@@ -169,7 +177,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(head["gbs"] / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(HEADLINE),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if n == TOKENS else None,
             "kernel": "tuna::gemm_kernel",
             "algorithmic_bytes_per_launch": head["packed_bytes"],
             "avg_launch_us": head["us_per_gemm"],

@@ -129,6 +129,12 @@ int tuna_time_dequant(const void *const *q_list, const void *const *absmax_list,
 int tuna_time_copy(const void *src, void *dst, size_t bytes, int warmup, int iters,
                    void *stream, float *elapsed_ms);
 
+/* Read-only streaming kernel over `bytes` bytes of `src` (16-byte multiples), `blocks`
+ * workgroups of 256 threads (0 = default): the ceiling a pure HBM reader reaches on the
+ * device, reported beside the GEMM's rate.  `sink` is 4 writable bytes. */
+int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int warmup, int iters,
+                   void *stream, float *elapsed_ms);
+
 /* Releases the library-owned split-K workspaces of the current device (synchronises
  * the device first). */
 int tuna_release_workspaces(void);

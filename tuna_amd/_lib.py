@@ -69,6 +69,7 @@ SIGNATURES = {
     "tuna_time_matmul": (_i, [_vpp, _vpp, _i, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_dequant": (_i, [_vpp, _vpp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_copy": (_i, [_vp, _vp, _sz, _i, _i, _vp, _fp]),
+    "tuna_time_read": (_i, [_vp, _vp, _sz, _i, _i, _i, _vp, _fp]),
     "tuna_release_workspaces": (_i, []),
 }
 

@@ -50,10 +50,21 @@ static int check_shape(int m, int n, int k)
     return TUNA_OK;
 }
 
+static inline bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+static inline int log2i(int v)
+{
+    int l = 0;
+    while ((1 << l) < v) ++l;
+    return l;
+}
+
 static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode, GemmPlan *plan)
 {
     int rc = check_shape(m, n, k);
     if (rc) return rc;
+    if ((unsigned long long)m * (unsigned long long)k / 2 >= (1ull << 32))
+        return fail(TUNA_ERR_UNSUPPORTED, "packed weights of %llu bytes exceed the kernel's 32-bit offsets",
+                    (unsigned long long)m * (unsigned long long)k / 2);
     if (decode != TUNA_DECODE_GEMM && decode != TUNA_DECODE_DEQUANT)
         return fail(TUNA_ERR_INVALID_ARG, "decode_mode %d is neither TUNA_DECODE_GEMM nor TUNA_DECODE_DEQUANT", decode);
     if (c.rows_per_wave != 64 && c.rows_per_wave != 128 && c.rows_per_wave != 256)
@@ -62,30 +73,42 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
         return fail(TUNA_ERR_UNSUPPORTED, "prefetch=%d (2, 4 or 8)", c.prefetch);
     if (c.token_tiles != 1 && c.token_tiles != 2 && c.token_tiles != 4)
         return fail(TUNA_ERR_UNSUPPORTED, "token_tiles=%d (1, 2 or 4)", c.token_tiles);
-    if (c.waves_m < 1 || c.waves_k < 1 || c.waves_m * c.waves_k * 64 > kMaxThreads)
-        return fail(TUNA_ERR_UNSUPPORTED, "waves_m=%d x waves_k=%d must give 1..16 waves", c.waves_m, c.waves_k);
+    if (!is_pow2(c.waves_m) || !is_pow2(c.waves_k) || c.waves_m * c.waves_k * 64 > kMaxThreads)
+        return fail(TUNA_ERR_UNSUPPORTED, "waves_m=%d and waves_k=%d must be powers of two with at most 16 waves", c.waves_m,
+                    c.waves_k);
     const int steps_total = ceil_div(k, kStepK);
     if (c.split_k < 1 || c.split_k > steps_total)
         return fail(TUNA_ERR_UNSUPPORTED, "split_k=%d must be in 1..%d for k=%d", c.split_k, steps_total, k);
-    if (c.x_chunk <= 0 || c.x_chunk % (kStepK * c.waves_k * c.prefetch) != 0)
-        return fail(TUNA_ERR_UNSUPPORTED, "x_chunk=%d must be a positive multiple of 32*waves_k*prefetch=%d", c.x_chunk,
+    if (!is_pow2(c.x_chunk) || c.x_chunk < kStepK * c.waves_k * c.prefetch)
+        return fail(TUNA_ERR_UNSUPPORTED, "x_chunk=%d must be a power of two >= 32*waves_k*prefetch=%d", c.x_chunk,
                     kStepK * c.waves_k * c.prefetch);
     const int rw = c.rows_per_wave / kRowsPerLoad;
     const int threads = c.waves_m * c.waves_k * 64;
-    if (!gemm_variant_exists(rw, c.prefetch, c.token_tiles, decode, threads))
+    const int rows_wg = c.rows_per_wave * c.waves_m;
+    if (c.x_chunk * c.token_tiles > 2 * threads)  // a chunk of x is staged as at most 4 pieces of 16 bytes per thread
+        return fail(TUNA_ERR_UNSUPPORTED, "x_chunk=%d x token_tiles=%d exceeds 2 x threads=%d", c.x_chunk, c.token_tiles,
+                    2 * threads);
+
+    const int nacc = rw * 4 * c.token_tiles;
+    const int lut = decode == TUNA_DECODE_GEMM ? kLutBytes : 64;
+    const size_t main_lds = (size_t)lut + (size_t)c.token_tiles * 16 * (size_t)c.x_chunk * 2;
+    const size_t red_lds = (size_t)c.waves_k * c.waves_m * nacc * 1024;
+    const size_t tile_lds = (size_t)c.token_tiles * 16 * (rows_wg + 8) * 2;
+    const size_t epi_lds = red_lds + tile_lds + 16;
+    const size_t lds = main_lds > epi_lds ? main_lds : epi_lds;
+    if (lds > (size_t)kLdsLimit)
+        return fail(TUNA_ERR_UNSUPPORTED, "config needs %zu bytes of LDS, the CU has %d", lds, kLdsLimit);
+
+    // Two workgroups per CU need <= 128 VGPRs each: take that variant when both fit in LDS.
+    int min_waves = threads > 512 ? 4 : 2;
+    if (threads <= 512 && 2 * lds <= (size_t)kLdsLimit &&
+        gemm_variant_exists(rw, c.prefetch, c.token_tiles, decode, threads, 4))
+        min_waves = 4;
+    if (!gemm_variant_exists(rw, c.prefetch, c.token_tiles, decode, threads, min_waves))
         return fail(TUNA_ERR_UNSUPPORTED,
                     "no kernel variant for rows_per_wave=%d prefetch=%d token_tiles=%d decode=%d threads=%d", c.rows_per_wave,
                     c.prefetch, c.token_tiles, decode, threads);
 
-    const int nacc = rw * 4 * c.token_tiles;
-    const int lut = decode == TUNA_DECODE_GEMM ? kLutBytes : 64;
-    const size_t main_lds = (size_t)lut + (size_t)c.token_tiles * 16 * ((size_t)c.x_chunk * 2 + 16);
-    const size_t red_lds = (size_t)(c.waves_k - 1) * c.waves_m * nacc * 1024;
-    const size_t lds = (main_lds > red_lds ? main_lds : red_lds) + 16;
-    if (lds > (size_t)kLdsLimit)
-        return fail(TUNA_ERR_UNSUPPORTED, "config needs %zu bytes of LDS, the CU has %d", lds, kLdsLimit);
-
-    const int rows_wg = c.rows_per_wave * c.waves_m;
     const int row_tiles = ceil_div(m, rows_wg);
     const int tok_chunks = ceil_div(n, 16 * c.token_tiles);
     if (tok_chunks > 65535) return fail(TUNA_ERR_UNSUPPORTED, "n=%d needs %d token chunks (max 65535)", n, tok_chunks);
@@ -97,6 +120,7 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     p.prefetch = c.prefetch;
     p.token_tiles = c.token_tiles;
     p.decode = decode;
+    p.min_waves = min_waves;
     p.threads = threads;
     p.lds_bytes = lds;
     p.grid = dim3((unsigned)(row_tiles * c.split_k), (unsigned)tok_chunks, 1);
@@ -108,13 +132,17 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     a.k = k;
     a.waves_m = c.waves_m;
     a.waves_k = c.waves_k;
+    a.wm_log2 = log2i(c.waves_m);
+    a.wk_log2 = log2i(c.waves_k);
     a.split_k = c.split_k;
     a.steps_total = steps_total;
     a.steps_per_split = ceil_div(steps_total, c.split_k);
     a.chunk_steps = c.x_chunk / kStepK;
+    a.chunk_log2 = log2i(a.chunk_steps);
     a.row_tiles = row_tiles;
     a.xcd_swizzle = c.xcd_swizzle ? 1 : 0;
     a.lds_bytes = (int)lds;
+    a.red_bytes = (int)red_lds;
     return TUNA_OK;
 }
 
@@ -124,10 +152,10 @@ static tuna_gemm_config derive_config(int m, int n, int k)
 {
     tuna_gemm_config c;
     c.token_tiles = n <= 16 ? 1 : (n <= 32 ? 2 : 4);
-    c.rows_per_wave = (m >= 16384 && c.token_tiles == 1) ? 128 : 64;
+    c.rows_per_wave = 64;
     c.waves_m = 2;
     c.waves_k = 4;
-    c.prefetch = 4;
+    c.prefetch = c.token_tiles == 4 ? 2 : 4;
     c.xcd_swizzle = 0;
     const int steps = ceil_div(k, kStepK);
     const int row_tiles = ceil_div(m, c.rows_per_wave * c.waves_m);
@@ -138,9 +166,9 @@ static tuna_gemm_config derive_config(int m, int n, int k)
     if (split < 1) split = 1;
     c.split_k = split;
     const int sps = ceil_div(steps, split);
-    int chunk_steps = round_up(sps, group);
-    const int cap = round_up(32 / c.token_tiles, group);  // keeps table + x within the 160 KB of LDS
-    if (chunk_steps > cap) chunk_steps = cap;
+    int chunk_steps = group;                                 // power of two
+    const int cap = 16 / c.token_tiles > group ? 16 / c.token_tiles : group;  // <= 16 KB of x per chunk
+    while (chunk_steps < sps && chunk_steps * 2 <= cap) chunk_steps *= 2;
     c.x_chunk = chunk_steps * kStepK;
     return c;
 }
@@ -234,6 +262,11 @@ static int check_ptr(const void *p, const char *name, size_t align)
     return TUNA_OK;
 }
 
+#ifdef TUNA_TRACE
+static unsigned long long *g_trace = nullptr;
+extern "C" __attribute__((visibility("default"))) void tuna_set_trace(void *p) { g_trace = static_cast<unsigned long long *>(p); }
+#endif
+
 static int matmul_impl(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n, int k,
                        const tuna_gemm_config *cfg, int decode, hipStream_t stream)
 {
@@ -249,7 +282,6 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
         if (decode != TUNA_DECODE_GEMM) {  // the dequant-rounding variants exist for one tile shape only
             c.rows_per_wave = 64;
             c.prefetch = 2;
-            c.x_chunk = round_up(c.x_chunk, kStepK * c.waves_k * c.prefetch);
         }
     }
     GemmPlan plan;
@@ -265,6 +297,9 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
         plan.args.ws = w.ws;
         plan.args.counters = w.counters;
     }
+#ifdef TUNA_TRACE
+    plan.args.trace = g_trace;
+#endif
     hipError_t e = launch_gemm(plan, stream);
     if (e != hipSuccess) return hip_fail(e, "gemm launch");
     return TUNA_OK;
@@ -471,6 +506,19 @@ TUNA_EXPORT int tuna_time_copy(const void *src, void *dst, size_t bytes, int war
     auto launch = [&](int, hipStream_t s) {
         hipError_t e = launch_copy(src, dst, bytes, s);
         return e == hipSuccess ? (int)TUNA_OK : hip_fail(e, "copy launch");
+    };
+    return time_loop(launch, 1, warmup, iters, 0, static_cast<hipStream_t>(stream), elapsed_ms);
+}
+
+TUNA_EXPORT int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int warmup, int iters, void *stream,
+                               float *elapsed_ms)
+{
+    int rc;
+    if ((rc = check_ptr(src, "src", 16)) || (rc = check_ptr(sink, "sink", 4))) return rc;
+    if (bytes == 0 || bytes % 16) return fail(TUNA_ERR_INVALID_ARG, "bytes must be a positive multiple of 16");
+    auto launch = [&](int, hipStream_t s) {
+        hipError_t e = launch_read(src, sink, bytes, blocks, s);
+        return e == hipSuccess ? (int)TUNA_OK : hip_fail(e, "read launch");
     };
     return time_loop(launch, 1, warmup, iters, 0, static_cast<hipStream_t>(stream), elapsed_ms);
 }

@@ -102,6 +102,34 @@ __global__ __launch_bounds__(256) void copy_kernel(const u32x4 *__restrict__ src
         __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
+// Read-only stream: the ceiling a pure HBM reader reaches on this device (8 loads of 16
+// bytes in flight per lane, 8 KB per wave and step, blocks walk the buffer in lockstep).
+__global__ __launch_bounds__(256) void read_kernel(const u32x4 *__restrict__ src, uint32_t *__restrict__ sink, size_t n16)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    u32x4 acc = u32x4{0u, 0u, 0u, 0u};
+    for (; i + 7 * stride < n16; i += 8 * stride) {
+        u32x4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc ^= v[u];
+    }
+    for (; i < n16; i += stride) acc ^= __builtin_nontemporal_load(src + i);
+    const uint32_t r = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+    if (r == 0x9e3779b9u) sink[0] = r;  // practically never: keeps the loads alive
+}
+
+hipError_t launch_read(const void *src, void *sink, size_t bytes, int blocks, hipStream_t stream)
+{
+    const size_t n16 = bytes / 16;
+    if (blocks <= 0) blocks = 256 * 8;
+    hipLaunchKernelGGL(read_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, reinterpret_cast<const u32x4 *>(src),
+                       reinterpret_cast<uint32_t *>(sink), n16);
+    return hipGetLastError();
+}
+
 hipError_t launch_copy(const void *src, void *dst, size_t bytes, hipStream_t stream)
 {
     const size_t n16 = bytes / 16;

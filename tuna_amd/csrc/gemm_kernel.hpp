@@ -19,7 +19,9 @@
 //   * Packed weights are used exactly once, so they go global -> registers through a
 //     ring of `U` k-steps per wave (nontemporal loads); there is nothing to share in LDS.
 //   * Activations are re-used by every wave: the workgroup stages its k-slice of x in
-//     LDS in chunks and each wave reads its B fragments with ds_read_b128.
+//     LDS in chunks, as 16-byte pieces ordered [8-k slot][token], so that both the staging
+//     writes and the ds_read_b128 of a B fragment (16 lanes = 16 tokens of one slot = 256
+//     contiguous bytes) are bank-conflict free without padding.
 //   * Decode: the codebook is a run-time input, so it is a table.  LDS holds, for every
 //     byte value, the half2 {code[hi nibble], code[lo nibble]} replicated once per lane
 //     (row stride 256 B).  A lane's address is (byte << 8) | (lane << 2), built by one
@@ -27,11 +29,13 @@
 //     data.  One v_pk_mul_f16 applies the row's fp16 scale - the same single fp16
 //     rounding as the reference's `smemCode.get(nib) * absMax` (kernel.cu:2178-2192).
 //     Cost: 1 perm + 1 ds_read_b32 + 1 pk_mul per two weights.
-//   * Split-K: waves_k waves of a workgroup cover interleaved k-steps and are summed in
-//     LDS in a fixed order; split_k workgroups write fp32 partials to a workspace and the
-//     last one to arrive (device-scope counter) sums them in split order and stores fp16.
-//     No atomics on the output (unlike kernel.cu:2739-2745), no pre-zeroing, and the
-//     result does not depend on arrival order.
+//   * Split-K: waves_k waves of a workgroup cover interleaved k-steps; their accumulators
+//     meet in LDS and every thread sums a 1/waves_k share in wave order.  split_k
+//     workgroups write those fp32 sums to a workspace and the last one to arrive
+//     (device-scope counter) adds them in split order.  The fp16 result is transposed
+//     through LDS and stored with 16-byte, fully coalesced writes.  No atomics on the
+//     output (unlike kernel.cu:2739-2745), no pre-zeroing, and the result does not depend
+//     on arrival order.
 #pragma once
 #include "tuna_internal.h"
 
@@ -62,14 +66,23 @@ __device__ __forceinline__ f16x8 decode_dword(uint32_t d, const unsigned char *l
         const uint32_t a3 = __builtin_amdgcn_perm(d, lane4, 0x0c0c0700u);
         // The table starts at LDS address 0 (the kernel has no static LDS), so the
         // permuted value IS the LDS address: no base add per lookup.
+#if defined(TUNA_ABLATE) && TUNA_ABLATE == 1  /* development only: no table reads */
+        const uint32_t t0 = a0, t1 = a1, t2 = a2, t3 = a3;
+#else
         const uint32_t t0 = *reinterpret_cast<const lds_u32 *>((uintptr_t)a0);
         const uint32_t t1 = *reinterpret_cast<const lds_u32 *>((uintptr_t)a1);
         const uint32_t t2 = *reinterpret_cast<const lds_u32 *>((uintptr_t)a2);
         const uint32_t t3 = *reinterpret_cast<const lds_u32 *>((uintptr_t)a3);
+#endif
+#if defined(TUNA_ABLATE) && TUNA_ABLATE == 2  /* development only: no scale multiply */
+        const f16x2 h0 = __builtin_bit_cast(f16x2, t0), h1 = __builtin_bit_cast(f16x2, t1);
+        const f16x2 h2 = __builtin_bit_cast(f16x2, t2), h3 = __builtin_bit_cast(f16x2, t3);
+#else
         const f16x2 h0 = __builtin_bit_cast(f16x2, t0) * sc16;
         const f16x2 h1 = __builtin_bit_cast(f16x2, t1) * sc16;
         const f16x2 h2 = __builtin_bit_cast(f16x2, t2) * sc16;
         const f16x2 h3 = __builtin_bit_cast(f16x2, t3) * sc16;
+#endif
         f16x8 r;
         r[0] = h0[0]; r[1] = h0[1]; r[2] = h1[0]; r[3] = h1[1];
         r[4] = h2[0]; r[5] = h2[1]; r[6] = h3[0]; r[7] = h3[1];
@@ -87,20 +100,68 @@ __device__ __forceinline__ f16x8 decode_dword(uint32_t d, const unsigned char *l
     }
 }
 
-template <int RW, int U, int TT, int DEC, int MAXT>
-__global__ __launch_bounds__(MAXT) void gemm_kernel(const GemmArgs a)
+// x staging, global -> registers -> LDS, in batches of kXBatch 16-byte pieces per thread.
+// Piece p of a chunk is token row (p % (16*TT)), 8-k slot (p / (16*TT)) and lives at LDS
+// byte 16*p.  All loads of a batch are issued before the first LDS write (addresses are
+// clamped so the loads are unconditional; invalid pieces are zeroed by a select).
+constexpr int kXBatch = 4;
+
+struct XStage {
+    u32x4 v[kXBatch];
+};
+
+template <int TT>
+__device__ __forceinline__ void x_stage_load(XStage &st, const f16 *xg, int base, int nthreads, int tid, int pieces,
+                                             int tok0, int kbase, int n, int k)
+{
+#pragma unroll
+    for (int b = 0; b < kXBatch; ++b) {
+        const int p = min(base + b * nthreads + tid, pieces - 1);
+        const int r = p & (16 * TT - 1);
+        const int c8 = p / (16 * TT);
+        const int tok = min(tok0 + r, n - 1);
+        const int kk = min(kbase + c8 * 8, k - 8);
+        st.v[b] = *reinterpret_cast<const u32x4 *>(xg + (size_t)tok * k + kk);
+    }
+}
+
+template <int TT>
+__device__ __forceinline__ void x_stage_store(const XStage &st, unsigned char *xs, int base, int nthreads, int tid,
+                                              int pieces, int tok0, int kbase, int n, int k)
+{
+#pragma unroll
+    for (int b = 0; b < kXBatch; ++b) {
+        const int p = base + b * nthreads + tid;
+        if (p < pieces) {
+            const int r = p & (16 * TT - 1);
+            const int c8 = p / (16 * TT);
+            const bool ok = (tok0 + r < n) && (kbase + c8 * 8 < k);
+            *reinterpret_cast<u32x4 *>(xs + (size_t)p * 16) = ok ? st.v[b] : u32x4{0u, 0u, 0u, 0u};
+        }
+    }
+}
+
+template <int RW, int U, int TT, int DEC, int MAXT, int MINW>
+__global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    constexpr int NACC = RW * 4 * TT;
+    constexpr int NACC = RW * 4 * TT;  // float4 accumulator planes per lane
     constexpr int LUT_B = (DEC == TUNA_DECODE_GEMM) ? kLutBytes : 64;
 
     const int tid = threadIdx.x;
+#ifdef TUNA_TRACE
+#define TUNA_MARK(i) if (a.trace && tid == 0) a.trace[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + (i)] = wall_clock64();
+#else
+#define TUNA_MARK(i)
+#endif
+    TUNA_MARK(0)
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wk = wave % a.waves_k;
-    const int wm = wave / a.waves_k;
+    const int wk = wave & (a.waves_k - 1);
+    const int wm = wave >> a.wk_log2;
     const int i16 = lane & 15;
     const int g = lane >> 4;
+    const int nthreads = (int)blockDim.x;
 
     int id = blockIdx.x;
     if (a.xcd_swizzle) {
@@ -110,22 +171,14 @@ __global__ __launch_bounds__(MAXT) void gemm_kernel(const GemmArgs a)
     const int row_tile = id / a.split_k;
     const int ks = id - row_tile * a.split_k;
     const int tok0 = blockIdx.y * (TT * 16);
-    const int row0 = (row_tile * a.waves_m + wm) * (RW * kRowsPerLoad);
+    const int rows_wg = a.waves_m * (RW * kRowsPerLoad);
+    const int row0 = row_tile * rows_wg + wm * (RW * kRowsPerLoad);  // first weight row of this wave
 
     const int sb = ks * a.steps_per_split;
     const int se = min(a.steps_total, sb + a.steps_per_split);
     const int nsteps = max(se - sb, 0);
-    const int n_it = nsteps > wk ? (nsteps - wk + a.waves_k - 1) / a.waves_k : 0;
+    const int n_it = nsteps > wk ? (nsteps - wk + a.waves_k - 1) >> a.wk_log2 : 0;
 
-    // ---- packed-weight stream: per-lane base pointers and the prefetch ring ----------
-    const int kb_total = a.k >> 3;
-    const int mb_last = (a.m >> 3) - 1;
-    const unsigned char *wp[RW];
-#pragma unroll
-    for (int rw = 0; rw < RW; ++rw) {
-        const int mb = min(((row0 + rw * kRowsPerLoad) >> 3) + (i16 >> 1), mb_last);
-        wp[rw] = a.q + ((size_t)mb * (size_t)kb_total) * 32 + (i16 & 1) * 16;
-    }
     // Small operands first, all unconditional, so that every later wait on them can be an
     // exact s_waitcnt vmcnt(N) that leaves the weight prefetches in flight.
     const float code_lane = a.code[lane & 15];
@@ -138,21 +191,44 @@ __global__ __launch_bounds__(MAXT) void gemm_kernel(const GemmArgs a)
             sc32[rw][j] = a.absmax[min(row, a.m - 1)];  // rows past m are never stored
         }
 
+    // ---- packed-weight stream ------------------------------------------------------------
+    // address = q + [uniform: 128 bytes per k-step] + [per lane: block row, row half, g]:
+    // the uniform part rides in SGPRs, so a load costs no vector ALU work.
+    const int kb_total = a.k >> 3;
+    const int mb_last = (a.m >> 3) - 1;
+    const int g_last = min(g, kb_total - 1 - (a.steps_total - 1) * 4);  // last k-step may be short
+    uint32_t lb[RW], lb_last[RW];
+#pragma unroll
+    for (int rw = 0; rw < RW; ++rw) {
+        const int mb = min(((row0 + rw * kRowsPerLoad) >> 3) + (i16 >> 1), mb_last);
+        const uint32_t rowb = (uint32_t)mb * (uint32_t)kb_total * 32u + (uint32_t)(i16 & 1) * 16u;
+        lb[rw] = rowb + (uint32_t)g * 32u;
+        lb_last[rw] = rowb + (uint32_t)g_last * 32u;
+    }
     u32x4 wq[U][RW];
-    const int kstride = a.waves_k * 4;  // block columns between this wave's consecutive steps
-    const int kb_first = (sb + wk) * 4 + g;
+    const int s_first = sb + wk;            // this wave's first k-step
+    const int s_stride = a.waves_k;         // k-steps between its consecutive iterations
     // Unconditional by design: a load whose step lies beyond this wave's share is clamped
-    // to a valid block column and its data is never used.  Only loads that are always
-    // issued let the compiler count outstanding loads exactly (s_waitcnt vmcnt(N > 0)).
+    // to the last k-step and its data is never used.  Only loads that are always issued
+    // let the compiler count outstanding loads exactly (s_waitcnt vmcnt(N > 0)).
 #define TUNA_LOAD_STEP(u, it)                                                                  \
     {                                                                                          \
-        const int kb_ = min(kb_first + (it) * kstride, kb_total - 1);                          \
-        _Pragma("unroll") for (int rw = 0; rw < RW; ++rw) wq[u][rw] =                          \
-            __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wp[rw] + (size_t)kb_ * 32)); \
+        const int s_ = min(s_first + (it) * s_stride, a.steps_total - 1);                      \
+        const unsigned char *base_ = a.q + (size_t)s_ * 128;                                   \
+        const bool last_ = s_ == a.steps_total - 1;                                            \
+        _Pragma("unroll") for (int rw = 0; rw < RW; ++rw) wq[u][rw] = __builtin_nontemporal_load( \
+            reinterpret_cast<const u32x4 *>(base_ + (last_ ? lb_last[rw] : lb[rw])));          \
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) TUNA_LOAD_STEP(u, u)
 
+    // first batch of the first x chunk: in flight while the decode table is built
+    const f16 *xg = reinterpret_cast<const f16 *>(a.x);
+    const int x_pieces = (TT * 16 * 4) << a.chunk_log2;  // 16-byte pieces per chunk
+    XStage xst;
+    x_stage_load<TT>(xst, xg, 0, nthreads, tid, x_pieces, tok0, sb * kStepK, a.n, a.k);
+
+    TUNA_MARK(1)
     // ---- per-row scales (fp16 like the reference's staging, kernel.cu:2770) -----------
     f16x2 sc16[RW][4];
 #pragma unroll
@@ -170,7 +246,8 @@ __global__ __launch_bounds__(MAXT) void gemm_kernel(const GemmArgs a)
         // entries are gathered across lanes, no memory traffic.
         // piece p: 16 bytes of row (p >> 4); all 64 slots of a row hold the same half2
         const int code_bits = (int)f16_bits((f16)code_lane);
-        for (int p = tid; p < kLutBytes / 16; p += blockDim.x) {
+#pragma unroll 4
+        for (int p = tid; p < kLutBytes / 16; p += nthreads) {
             const int e = p >> 4;
             const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute((e >> 4) << 2, code_bits);
             const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute((e & 15) << 2, code_bits);
@@ -181,11 +258,9 @@ __global__ __launch_bounds__(MAXT) void gemm_kernel(const GemmArgs a)
         if (tid < 16) reinterpret_cast<float *>(lut)[tid] = code_lane;
     }
     const uint32_t lane4 = (uint32_t)lane << 2;
+    TUNA_MARK(2)
 
-    // ---- x staging ----------------------------------------------------------------------
     unsigned char *xs = smem + LUT_B;
-    const int xs_stride = a.chunk_steps * 64 + 16;  // bytes per token row (+16: bank skew)
-    const f16 *xg = reinterpret_cast<const f16 *>(a.x);
 
     f32x4 acc[RW][4][TT];
 #pragma unroll
@@ -200,7 +275,7 @@ __global__ __launch_bounds__(MAXT) void gemm_kernel(const GemmArgs a)
     {                                                                                          \
         f16x8 b_[TT];                                                                          \
         _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) b_[tt] =                             \
-            *reinterpret_cast<const f16x8 *>(xb + tt * 16 * xs_stride + (xoff));               \
+            *reinterpret_cast<const f16x8 *>(xb + tt * 256 + (xoff));                          \
         _Pragma("unroll") for (int rw = 0; rw < RW; ++rw) _Pragma("unroll") for (int j = 0; j < 4; ++j) \
         {                                                                                      \
             const f16x8 av_ = decode_dword<DEC>(wq[u][rw][j], lut, lane4, sc16[rw][j], sc32[rw][j]); \
@@ -209,169 +284,171 @@ __global__ __launch_bounds__(MAXT) void gemm_kernel(const GemmArgs a)
         }                                                                                      \
     }
 
-    const int ipc = a.chunk_steps / a.waves_k;  // iterations per chunk per wave (multiple of U)
-    const int n_chunks = (nsteps + a.chunk_steps - 1) / a.chunk_steps;
-    const int wstep = a.waves_k * 64;           // LDS bytes between this wave's consecutive steps
-    int it = 0;                                 // this wave's next iteration (multiple of U)
+    // One group = U consecutive iterations of this wave: every ring slot is consumed and
+    // refilled, no branches inside (refill addresses are clamped, see TUNA_LOAD_STEP).
+#define TUNA_GROUP()                                                                            \
+    {                                                                                          \
+        _Pragma("unroll") for (int u = 0; u < U; ++u)                                          \
+        {                                                                                      \
+            TUNA_CONSUME(u, (it + u) * wstep)                                                  \
+            TUNA_LOAD_STEP(u, it + u + U)                                                      \
+            /* keep the refill right behind its consume: the scheduler would otherwise sink */ \
+            /* all U loads to the end of the group and empty the ring every group */           \
+            __builtin_amdgcn_sched_barrier(0);                                                 \
+        }                                                                                      \
+        it += U;                                                                               \
+    }
+
+    const int ipc = a.chunk_steps >> a.wk_log2;  // iterations per chunk per wave (multiple of U)
+    const int n_chunks = (nsteps + a.chunk_steps - 1) >> a.chunk_log2;
+    const int wstep = a.waves_k * (1024 * TT);   // LDS bytes between this wave's consecutive steps
+    int it = 0;                                  // this wave's next iteration (multiple of U)
+
+    // chunk 0 of x: loaded above, written here
+    if (n_chunks > 0) x_stage_store<TT>(xst, xs, 0, nthreads, tid, x_pieces, tok0, sb * kStepK, a.n, a.k);
+    __syncthreads();
+    TUNA_MARK(3)
+
     for (int c = 0; c < n_chunks; ++c) {
-        if (c) __syncthreads();
-        {
-            const int kbase = (sb + c * a.chunk_steps) * kStepK;
-            const int xc8 = a.chunk_steps * 4;  // 16-byte pieces per token row
-            for (int r = wave; r < TT * 16; r += (int)(blockDim.x >> 6)) {
-                const int tok = tok0 + r;
-                for (int c8 = lane; c8 < xc8; c8 += 64) {
-                    const int kk = kbase + c8 * 8;
-                    u32x4 v = u32x4{0u, 0u, 0u, 0u};
-                    if (tok < a.n && kk < a.k)
-                        v = *reinterpret_cast<const u32x4 *>(xg + (size_t)tok * a.k + kk);
-                    *reinterpret_cast<u32x4 *>(xs + r * xs_stride + c8 * 16) = v;
-                }
-            }
-        }
-        __syncthreads();
         const int it_chunk0 = c * ipc;
-        const int it_end = min(it_chunk0 + ipc, n_it);
-        const unsigned char *xb = xs + i16 * xs_stride + g * 16 + wk * 64 - it_chunk0 * wstep;
-        // steady state: every slot is consumed and refilled, no branches inside the group
-        while (it + U <= it_end && it + 2 * U <= n_it) {
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                TUNA_CONSUME(u, (it + u) * wstep)
-                TUNA_LOAD_STEP(u, it + u + U)
-                // keep the refill right behind its consume: the scheduler would otherwise
-                // sink all U loads to the end of the group and empty the ring every group
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            it += U;
-        }
-        if (it + U <= it_end && it + U == n_it) {
-            // last full group of the wave: drain the ring, nothing left to fetch
-#pragma unroll
-            for (int u = 0; u < U; ++u) TUNA_CONSUME(u, (it + u) * wstep)
-            it += U;
+        const bool has_next = c + 1 < n_chunks;
+        // B fragment of lane (token i16, k-group g), local step sl: slot sl*4+g, piece slot*16*TT + i16
+        const unsigned char *xb = xs + g * (256 * TT) + i16 * 16 + wk * (1024 * TT) - it_chunk0 * wstep;
+        if (has_next) {
+            // A chunk with a successor is full: every wave owns all ipc iterations of it.
+            const int it_peel = it_chunk0 + ipc - U;
+            while (it < it_peel) TUNA_GROUP()
+            // Last group of the chunk: the next chunk of x is fetched into registers first, so
+            // that after the group exactly U*RW younger loads are in flight and the wait before
+            // the LDS write below is an exact vmcnt, not a drain of the weight ring.
+            const int kbase = (sb + (c + 1) * a.chunk_steps) * kStepK;
+            x_stage_load<TT>(xst, xg, 0, nthreads, tid, x_pieces, tok0, kbase, a.n, a.k);
+            TUNA_GROUP()
+            __syncthreads();  // every wave is done reading chunk c
+            x_stage_store<TT>(xst, xs, 0, nthreads, tid, x_pieces, tok0, kbase, a.n, a.k);
+            __syncthreads();
         } else {
-            // ragged tail (fewer than U steps left in the wave or in the chunk)
-            while (it < it_end) {
+            const int it_end = min(it_chunk0 + ipc, n_it);
+            // steady state while both the group and its refills lie inside this wave's share
+            while (it + U <= it_end && it + 2 * U <= n_it) TUNA_GROUP()
+            if (it + U <= it_end && it + U == n_it) {
+                // last full group of the wave: drain the ring, nothing left to fetch
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    if (it + u < it_end) {
-                        TUNA_CONSUME(u, (it + u) * wstep)
-                        if (it + u + U < n_it) TUNA_LOAD_STEP(u, it + u + U)
-                    }
-                }
+                for (int u = 0; u < U; ++u) TUNA_CONSUME(u, (it + u) * wstep)
                 it += U;
+            } else {
+                // ragged tail (fewer than U steps left in the wave or in the chunk)
+                while (it < it_end) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        if (it + u < it_end) {
+                            TUNA_CONSUME(u, (it + u) * wstep)
+                            if (it + u + U < n_it) TUNA_LOAD_STEP(u, it + u + U)
+                        }
+                    }
+                    it += U;
+                }
             }
         }
     }
+#undef TUNA_GROUP
 #undef TUNA_CONSUME
 #undef TUNA_LOAD_STEP
+    TUNA_MARK(4)
 
-    // ---- reduce the waves_k partial sums of the workgroup in LDS, fixed order ---------
-    f32x4 *red = reinterpret_cast<f32x4 *>(smem);
-    if (a.waves_k > 1) {
-        __syncthreads();  // table and x are dead from here on
-        if (wk > 0) {
-            f32x4 *dst = red + ((size_t)((wk - 1) * a.waves_m + wm) * NACC) * 64 + lane;
+    // ---- workgroup reduction: accumulators meet in LDS, every thread sums a share ------
+    // A wave's accumulators are the float array [plane][lane][4] (NACC*256 floats); thread
+    // (wk, lane) of row group wm owns floats f = (i*waves_k + wk)*64 + lane, i < nf.
+    __syncthreads();  // table and x are dead from here on
+    {
+        f32x4 *dst = reinterpret_cast<f32x4 *>(smem) + (size_t)(wm * a.waves_k + wk) * (NACC * 64) + lane;
 #pragma unroll
-            for (int rw = 0; rw < RW; ++rw)
+        for (int rw = 0; rw < RW; ++rw)
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < 4; ++j)
 #pragma unroll
-                    for (int tt = 0; tt < TT; ++tt) dst[((rw * 4 + j) * TT + tt) * 64] = acc[rw][j][tt];
-        }
-        __syncthreads();
-        if (wk == 0) {
-            for (int w = 1; w < a.waves_k; ++w) {
-                const f32x4 *src = red + ((size_t)((w - 1) * a.waves_m + wm) * NACC) * 64 + lane;
-#pragma unroll
-                for (int rw = 0; rw < RW; ++rw)
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-#pragma unroll
-                        for (int tt = 0; tt < TT; ++tt) acc[rw][j][tt] += src[((rw * 4 + j) * TT + tt) * 64];
-            }
-        }
+                for (int tt = 0; tt < TT; ++tt) dst[((rw * 4 + j) * TT + tt) * 64] = acc[rw][j][tt];
+    }
+    __syncthreads();
+    TUNA_MARK(5)
+    const float *redf = reinterpret_cast<const float *>(smem) + (size_t)wm * a.waves_k * (NACC * 256);
+    const int nf = (NACC * 4) >> a.wk_log2;
+    f16 *tile = reinterpret_cast<f16 *>(smem + a.red_bytes);  // [token][rows_wg + 8] fp16
+    const int tile_ld = rows_wg + 8;
+    // float f = (plane*64 + l)*4 + v is token (plane % TT)*16 + l%16, weight row
+    // (plane / (4*TT))*64 + 16*(l/16) + 4*v + (plane / TT) % 4 of the wave
+#define TUNA_TILE_PUT(f, val)                                                                   \
+    {                                                                                          \
+        const int pl_ = (f) >> 8, l_ = ((f) >> 2) & 63, v_ = (f) & 3;                          \
+        const int tok_ = (pl_ % TT) * 16 + (l_ & 15);                                          \
+        const int row_ = wm * (RW * kRowsPerLoad) + (pl_ / (4 * TT)) * 64 + (l_ >> 4) * 16 + v_ * 4 + (pl_ / TT) % 4; \
+        tile[tok_ * tile_ld + row_] = (f16)(val);                                              \
     }
 
-    // ---- reduce across the split_k workgroups through the workspace --------------------
-    // Partials travel as device-scope relaxed atomics (write-through stores, L2-bypassing
-    // loads): they are coherent across the 8 XCD L2s without the L2 write-back/invalidate
-    // that a device-scope release/acquire fence costs on every workgroup.  Order is given by
-    // "all my stores have completed" (workgroup-scope release = s_waitcnt vmcnt(0)) before
-    // the barrier that precedes the arrival counter's atomic increment.
-    if (a.split_k > 1) {
-        const size_t tile = (size_t)blockIdx.y * a.row_tiles + row_tile;
-        float *wst = a.ws + (tile * a.split_k * a.waves_m) * (size_t)(NACC * 256);
-        if (wk == 0) {
-            float *dst = wst + ((size_t)(ks * a.waves_m + wm) * NACC) * 256 + lane;
-#pragma unroll
-            for (int rw = 0; rw < RW; ++rw)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-#pragma unroll
-                    for (int tt = 0; tt < TT; ++tt)
-#pragma unroll
-                        for (int v = 0; v < 4; ++v)
-                            __hip_atomic_store(dst + (((rw * 4 + j) * TT + tt) * 4 + v) * 64, acc[rw][j][tt][v],
-                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    if (a.split_k == 1) {
+        for (int i = 0; i < nf; ++i) {
+            const int f = ((i << a.wk_log2) + wk) * 64 + lane;
+            float s = 0.f;
+            for (int w = 0; w < a.waves_k; ++w) s += redf[(size_t)w * (NACC * 256) + f];
+            TUNA_TILE_PUT(f, s)
         }
+    } else {
+        // Partials travel as device-scope relaxed atomics (write-through stores, L2-bypassing
+        // loads): coherent across the 8 XCD L2s without the L2 write-back/invalidate that a
+        // device-scope release/acquire fence costs on every workgroup.  Order is given by
+        // "all my stores have completed" (workgroup-scope release = s_waitcnt vmcnt(0))
+        // before the barrier that precedes the arrival counter's increment.
+        const size_t tile_id = (size_t)blockIdx.y * a.row_tiles + row_tile;
+        float *wst = a.ws + (tile_id * a.split_k * a.waves_m) * (size_t)(NACC * 256);
+        float *mine = wst + ((size_t)ks * a.waves_m + wm) * (NACC * 256);
+        for (int i = 0; i < nf; ++i) {
+            const int f = ((i << a.wk_log2) + wk) * 64 + lane;
+            float s = 0.f;
+            for (int w = 0; w < a.waves_k; ++w) s += redf[(size_t)w * (NACC * 256) + f];
+            __hip_atomic_store(mine + f, s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
+        TUNA_MARK(6)
         volatile unsigned *ticket = reinterpret_cast<volatile unsigned *>(smem + a.lds_bytes - 16);
         if (tid == 0)
-            *ticket = __hip_atomic_fetch_add(a.counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *ticket = __hip_atomic_fetch_add(a.counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
+        TUNA_MARK(7)
         if (*ticket != (unsigned)(a.split_k - 1)) return;
-        // last workgroup of this tile: every partial is in memory; sum them in split order
-        if (tid == 0) __hip_atomic_store(a.counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (wk == 0) {
-#pragma unroll
-            for (int rw = 0; rw < RW; ++rw)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-#pragma unroll
-                    for (int tt = 0; tt < TT; ++tt) acc[rw][j][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
-            for (int s = 0; s < a.split_k; ++s) {
-                const float *src = wst + ((size_t)(s * a.waves_m + wm) * NACC) * 256 + lane;
-#pragma unroll
-                for (int rw = 0; rw < RW; ++rw)
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-#pragma unroll
-                        for (int tt = 0; tt < TT; ++tt)
-#pragma unroll
-                            for (int v = 0; v < 4; ++v)
-                                acc[rw][j][tt][v] += __hip_atomic_load(src + (((rw * 4 + j) * TT + tt) * 4 + v) * 64,
-                                                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
+        // last workgroup of this tile: every partial is in memory; add them in split order
+        if (tid == 0) __hip_atomic_store(a.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int i = 0; i < nf; ++i) {
+            const int f = ((i << a.wk_log2) + wk) * 64 + lane;
+            const float *src = wst + (size_t)wm * (NACC * 256) + f;
+            float s = 0.f;
+            for (int sp = 0; sp < a.split_k; ++sp)
+                s += __hip_atomic_load(src + (size_t)sp * a.waves_m * (NACC * 256), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+            TUNA_TILE_PUT(f, s)
         }
     }
+#undef TUNA_TILE_PUT
+    __syncthreads();
+    TUNA_MARK(8)
 
-    // ---- store: lane (token i16, group g) owns 16 consecutive output features ---------
-    if (wk == 0) {
+    // ---- store the [tokens][rows_wg] fp16 tile: 16 bytes per thread, rows contiguous ---
+    {
         f16 *outp = reinterpret_cast<f16 *>(a.out);
-#pragma unroll
-        for (int tt = 0; tt < TT; ++tt) {
-            const int tok = tok0 + tt * 16 + i16;
-            if (tok >= a.n) continue;
-#pragma unroll
-            for (int rw = 0; rw < RW; ++rw) {
-                const int rb = row0 + rw * kRowsPerLoad + g * 16;
-                f16x8 lo, hi;
-#pragma unroll
-                for (int v = 0; v < 2; ++v)
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        lo[v * 4 + j] = (f16)acc[rw][j][tt][v];
-                        hi[v * 4 + j] = (f16)acc[rw][j][tt][v + 2];
-                    }
-                f16 *dst = outp + (size_t)tok * a.m + rb;
-                if (rb + 8 <= a.m) *reinterpret_cast<f16x8 *>(dst) = lo;
-                if (rb + 16 <= a.m) *reinterpret_cast<f16x8 *>(dst + 8) = hi;
-            }
+        constexpr int RW_LOG2 = RW == 1 ? 0 : (RW == 2 ? 1 : 2);
+        const int r8_log2 = a.wm_log2 + RW_LOG2 + 3;  // log2(rows_wg / 8)
+        const int pieces = (TT * 16) << r8_log2;
+        for (int p = tid; p < pieces; p += nthreads) {
+            const int tok = p >> r8_log2;
+            const int r8 = p & ((1 << r8_log2) - 1);
+            const int row = row_tile * rows_wg + r8 * 8;
+            if (tok0 + tok < a.n && row + 8 <= a.m)
+                *reinterpret_cast<u32x4 *>(outp + (size_t)(tok0 + tok) * a.m + row) =
+                    *reinterpret_cast<const u32x4 *>(tile + tok * tile_ld + r8 * 8);
         }
     }
+    TUNA_MARK(9)
+#undef TUNA_MARK
 }
 
 }  // namespace tuna

@@ -8,46 +8,48 @@ namespace tuna {
 typedef void (*GemmKernelFn)(const GemmArgs);
 
 struct Variant {
-    int rw, u, tt, dec, maxt;
+    int rw, u, tt, dec, maxt, minw;
     GemmKernelFn fn;
 };
 
-#define V(RW, U, TT, DEC, MAXT) {RW, U, TT, DEC, MAXT, gemm_kernel<RW, U, TT, DEC, MAXT>}
-#define V_TT(RW, U, MAXT) V(RW, U, 1, TUNA_DECODE_GEMM, MAXT), V(RW, U, 2, TUNA_DECODE_GEMM, MAXT), V(RW, U, 4, TUNA_DECODE_GEMM, MAXT)
+#define V(RW, U, TT, DEC, MAXT, MINW) {RW, U, TT, DEC, MAXT, MINW, gemm_kernel<RW, U, TT, DEC, MAXT, MINW>}
+#define G TUNA_DECODE_GEMM
 
+// Only variants that compile with no (or a handful of) register spills are listed;
+// tuna_amd/make_configs.py mirrors this list.
+//   MAXT 512 / MINW 2 : up to 8 waves per workgroup, up to 256 VGPRs
+//   MAXT 512 / MINW 4 : up to 8 waves, at most 128 VGPRs, so that two workgroups share a CU
+//   MAXT 1024 / MINW 4: 16-wave workgroups
 static const Variant kVariants[] = {
-    // Only variants that compile without register spills are listed (checked with
-    // -Rpass-analysis=kernel-resource-usage); tuna_amd/make_configs.py mirrors this list.
-    // rows_per_wave = 64
-    V_TT(1, 2, 512), V_TT(1, 4, 512), V_TT(1, 8, 512),
-    // rows_per_wave = 128
-    V(2, 2, 1, TUNA_DECODE_GEMM, 512), V(2, 2, 2, TUNA_DECODE_GEMM, 512),
-    V(2, 4, 1, TUNA_DECODE_GEMM, 512), V(2, 4, 2, TUNA_DECODE_GEMM, 512),
-    V(2, 8, 1, TUNA_DECODE_GEMM, 512),
-    // rows_per_wave = 256
-    V(4, 2, 1, TUNA_DECODE_GEMM, 512),
-    // 16-wave workgroups (128 VGPRs per lane): single token tile only
-    V(1, 4, 1, TUNA_DECODE_GEMM, 1024), V(1, 8, 1, TUNA_DECODE_GEMM, 1024),
+    V(1, 2, 1, G, 512, 2), V(1, 2, 2, G, 512, 2), V(1, 2, 4, G, 512, 2),
+    V(1, 4, 1, G, 512, 2), V(1, 4, 2, G, 512, 2),
+    V(1, 8, 1, G, 512, 2), V(1, 8, 2, G, 512, 2),
+    V(2, 2, 1, G, 512, 2),
+    V(2, 4, 1, G, 512, 2),
+    V(1, 2, 1, G, 512, 4), V(1, 4, 1, G, 512, 4),
+    V(1, 2, 1, G, 1024, 4), V(1, 4, 1, G, 1024, 4),
     // dequant-rounding decode (correctness mode, not tuned)
-    V(1, 2, 1, TUNA_DECODE_DEQUANT, 512), V(1, 2, 2, TUNA_DECODE_DEQUANT, 512), V(1, 2, 4, TUNA_DECODE_DEQUANT, 512),
+    V(1, 2, 1, TUNA_DECODE_DEQUANT, 512, 2), V(1, 2, 2, TUNA_DECODE_DEQUANT, 512, 2),
+    V(1, 2, 4, TUNA_DECODE_DEQUANT, 512, 2),
 };
 #undef V
-#undef V_TT
+#undef G
 static constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
-static const Variant *find_variant(int rw, int u, int tt, int dec, int threads)
+static const Variant *find_variant(int rw, int u, int tt, int dec, int threads, int minw)
 {
     const int maxt = threads <= 512 ? 512 : 1024;
+    if (maxt == 1024) minw = 4;
     for (int i = 0; i < kNumVariants; ++i) {
         const Variant &v = kVariants[i];
-        if (v.rw == rw && v.u == u && v.tt == tt && v.dec == dec && v.maxt == maxt) return &v;
+        if (v.rw == rw && v.u == u && v.tt == tt && v.dec == dec && v.maxt == maxt && v.minw == minw) return &v;
     }
     return nullptr;
 }
 
-bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads)
+bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves)
 {
-    return find_variant(rw, prefetch, token_tiles, decode, threads) != nullptr;
+    return find_variant(rw, prefetch, token_tiles, decode, threads, min_waves) != nullptr;
 }
 
 // Dynamic LDS above 64 KB needs a one-time opt-in per kernel and device.
@@ -56,7 +58,7 @@ static unsigned char g_attr_done[16][kNumVariants];
 
 hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
 {
-    const Variant *v = find_variant(plan.rw, plan.prefetch, plan.token_tiles, plan.decode, plan.threads);
+    const Variant *v = find_variant(plan.rw, plan.prefetch, plan.token_tiles, plan.decode, plan.threads, plan.min_waves);
     if (!v) return hipErrorInvalidConfiguration;
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);

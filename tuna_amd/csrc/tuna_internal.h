@@ -28,13 +28,19 @@ struct GemmArgs {
     float *ws;           // split-K partial sums (library owned), may be null if split_k == 1
     unsigned *counters;  // one arrival counter per (token chunk, row tile), zero between launches
     int m, n, k;
-    int waves_m, waves_k, split_k;
+    int waves_m, waves_k, split_k;  // waves_m and waves_k are powers of two
+    int wm_log2, wk_log2;
     int steps_total;      // ceil(k / 32)
     int steps_per_split;  // k-steps owned by one workgroup
-    int chunk_steps;      // k-steps of x staged in LDS at a time
+    int chunk_steps;      // k-steps of x staged in LDS at a time (power of two)
+    int chunk_log2;
     int row_tiles;        // workgroups along m
     int xcd_swizzle;
     int lds_bytes;        // dynamic LDS size of the launch (last 16 bytes: arrival ticket)
+    int red_bytes;        // bytes of the workgroup reduction area = offset of the fp16 output tile
+#ifdef TUNA_TRACE
+    unsigned long long *trace;  // development builds only: 16 timestamps per workgroup
+#endif
 };
 
 struct GemmPlan {
@@ -42,6 +48,7 @@ struct GemmPlan {
     dim3 grid;
     int threads;
     int rw, prefetch, token_tiles, decode;
+    int min_waves;  // waves per SIMD the variant is compiled for (2: <=256 VGPRs, 4: <=128)
     size_t lds_bytes;
     size_t ws_bytes;
     size_t n_counters;
@@ -49,12 +56,13 @@ struct GemmPlan {
 
 // gemm_kernel.hip
 hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream);
-bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads);
+bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves);
 
 // dequant_kernel.hip
 hipError_t launch_dequant(const uint8_t *q, const float *absmax, const float *code, void *out,
                           int m, int k, int decode, hipStream_t stream);
 hipError_t launch_copy(const void *src, void *dst, size_t bytes, hipStream_t stream);
+hipError_t launch_read(const void *src, void *sink, size_t bytes, int blocks, hipStream_t stream);
 
 // config_table.cpp
 struct TableEntry {

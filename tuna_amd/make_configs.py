@@ -42,11 +42,16 @@ LUT_BYTES = 256 * 64 * 4
 LDS_LIMIT = 160 * 1024
 STEP_K = 32
 
-# (rows_per_wave / 64, prefetch, token_tiles) variants compiled for <= 512 and for
-# 1024 threads per workgroup; must match kVariants in csrc/gemm_launch.hip
-VARIANTS_512 = {(1, 2, 1), (1, 2, 2), (1, 2, 4), (1, 4, 1), (1, 4, 2), (1, 4, 4), (1, 8, 1), (1, 8, 2), (1, 8, 4),
-                (2, 2, 1), (2, 2, 2), (2, 4, 1), (2, 4, 2), (2, 8, 1), (4, 2, 1)}
-VARIANTS_1024 = {(1, 4, 1), (1, 8, 1)}
+# (rows_per_wave / 64, prefetch, token_tiles) variants compiled for <= 8 waves (<= 256 VGPRs),
+# for <= 8 waves with <= 128 VGPRs (two workgroups per CU) and for 16-wave workgroups;
+# must match kVariants in csrc/gemm_launch.hip
+VARIANTS_512 = {(1, 2, 1), (1, 2, 2), (1, 2, 4), (1, 4, 1), (1, 4, 2), (1, 8, 1), (1, 8, 2), (2, 2, 1), (2, 4, 1)}
+VARIANTS_512_2WG = {(1, 2, 1), (1, 4, 1)}
+VARIANTS_1024 = {(1, 2, 1), (1, 4, 1)}
+
+
+def _pow2(v: int) -> bool:
+    return v > 0 and (v & (v - 1)) == 0
 
 
 def bucket_of(n: int):
@@ -73,24 +78,35 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
     if c["token_tiles"] not in (1, 2, 4):
         raise ValueError("token_tiles must be 1, 2 or 4")
     wm, wk = c["waves_m"], c["waves_k"]
-    if wm < 1 or wk < 1 or wm * wk > 16:
-        raise ValueError("waves_m * waves_k must be 1..16")
+    if not _pow2(wm) or not _pow2(wk) or wm * wk > 16:
+        raise ValueError("waves_m and waves_k must be powers of two with waves_m * waves_k <= 16")
+    if m * k // 2 >= 1 << 32:
+        raise ValueError("packed weights exceed the kernel's 32-bit offsets")
     steps = -(-k // STEP_K)
     if not 1 <= c["split_k"] <= steps:
         raise ValueError(f"split_k must be in 1..{steps}")
     unit = STEP_K * wk * c["prefetch"]
-    if c["x_chunk"] <= 0 or c["x_chunk"] % unit:
-        raise ValueError(f"x_chunk must be a positive multiple of {unit}")
+    if not _pow2(c["x_chunk"]) or c["x_chunk"] < unit:
+        raise ValueError(f"x_chunk must be a power of two >= {unit}")
     rw = c["rows_per_wave"] // 64
     key = (rw, c["prefetch"], c["token_tiles"])
     threads = 64 * wm * wk
     if key not in (VARIANTS_512 if threads <= 512 else VARIANTS_1024):
         raise ValueError(f"no kernel variant {key} for {threads} threads")
+    if c["x_chunk"] * c["token_tiles"] > 2 * threads:
+        raise ValueError("x_chunk * token_tiles exceeds 2 * threads (x staging is at most 4 pieces per thread)")
+    if lds_bytes(c) > LDS_LIMIT:
+        raise ValueError(f"needs {lds_bytes(c)} bytes of LDS (limit {LDS_LIMIT})")
+
+
+def lds_bytes(c: dict) -> int:
+    """Dynamic LDS of a launch: max(decode table + x chunk, reduction area + output tile)."""
+    rw = c["rows_per_wave"] // 64
     nacc = rw * 4 * c["token_tiles"]
-    main = LUT_BYTES + c["token_tiles"] * 16 * (c["x_chunk"] * 2 + 16)
-    red = (wk - 1) * wm * nacc * 1024
-    if max(main, red) + 16 > LDS_LIMIT:
-        raise ValueError(f"needs {max(main, red) + 16} bytes of LDS (limit {LDS_LIMIT})")
+    main = LUT_BYTES + c["token_tiles"] * 16 * c["x_chunk"] * 2
+    red = c["waves_k"] * c["waves_m"] * nacc * 1024
+    tile = c["token_tiles"] * 16 * (c["rows_per_wave"] * c["waves_m"] + 8) * 2
+    return max(main, red + tile + 16)
 
 
 def generate(param_map: dict) -> str:

@@ -167,3 +167,16 @@ def time_copy(src, dst, warmup=5, iters=20) -> float:
                               ctypes.byref(ms))
     _lib.check(rc)
     return ms.value
+
+
+def time_read(src, blocks=0, warmup=5, iters=20) -> float:
+    """Milliseconds for `iters` read-only passes over `src` (tuna_time_read)."""
+    nbytes = src.numel() * src.element_size()
+    sink = torch.zeros(4, dtype=torch.int32, device=src.device)
+    ms = ctypes.c_float(0)
+    L = _lib.lib()
+    with torch.cuda.device(src.device):
+        rc = L.tuna_time_read(src.data_ptr(), sink.data_ptr(), nbytes, int(blocks), int(warmup), int(iters),
+                              _stream(src.device), ctypes.byref(ms))
+    _lib.check(rc)
+    return ms.value
