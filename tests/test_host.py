@@ -1,0 +1,226 @@
+"""CPU tests of the host side: C ABI surface, config table / generator / validation, tuner's
+search-space helpers, quantizer + packer, error behaviour without a GPU."""
+import ctypes
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    from tuna_amd import _lib
+
+    L = _lib.lib()
+    header = open(os.path.join(ROOT, "include", "tuna_amd.h")).read()
+    declared = set(re.findall(r"\b(tuna_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations parsed"
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    for name in declared:
+        assert hasattr(L, name), name
+    assert L.tuna_version() == 100
+    assert L.tuna_status_string(0) == b"ok"
+    assert L.tuna_status_string(2) == b"unsupported shape or config"
+
+
+def test_config_struct_matches_header():
+    from tuna_amd._lib import GemmConfig
+
+    header = open(os.path.join(ROOT, "include", "tuna_amd.h")).read()
+    body = header[header.index("typedef struct tuna_gemm_config"):header.index("} tuna_gemm_config;")]
+    fields = re.findall(r"int32_t\s+([a-z_]+);", body)
+    assert tuple(fields) == GemmConfig.FIELDS
+    assert ctypes.sizeof(GemmConfig) == 4 * len(fields)
+
+
+def test_select_config_is_host_only_and_every_table_entry_validates():
+    from tuna_amd import make_configs, ops
+
+    table = ops.config_table()
+    with open(os.path.join(ROOT, "tuna_amd", "configs", "param_map.json")) as f:
+        pm = json.load(f)
+    assert len(table) == len(pm)
+    for m, lo, hi, k, cfg in table:
+        key = f"{m}_{make_configs.bucket_of(lo)}_{k}"
+        assert key in pm
+        assert cfg.to_dict() == {f: pm[key][f] for f in cfg.FIELDS}
+        for n in (lo, hi):
+            ops.validate_config(m, n, k, cfg)                      # the C side accepts it
+            got, hit = ops.select_config(m, n, k)
+            assert hit and got.to_dict() == cfg.to_dict()
+        make_configs.validate(m, make_configs.bucket_of(lo), k, cfg.to_dict())  # and the generator's twin
+        lds, ws = ops.config_footprint(m, lo, k, cfg)
+        assert lds == make_configs.lds_bytes(cfg.to_dict()) and lds <= 160 * 1024
+
+
+@pytest.mark.parametrize("shape", [(8, 1, 8), (64, 16, 64), (4096, 16, 4104), (1000 * 8, 3, 40), (12288, 100, 4096),
+                                   (8192, 256, 8192), (8192, 4096, 1024), (229376, 128, 4096)])
+def test_derived_config_is_valid_for_any_shape(shape):
+    from tuna_amd import ops
+
+    cfg, _ = ops.select_config(*shape)
+    ops.validate_config(*shape, cfg)
+    lds, ws = ops.config_footprint(*shape, cfg)
+    assert 0 < lds <= 160 * 1024
+
+
+def test_token_buckets_follow_the_reference_dispatcher():
+    from tuna_amd import make_configs as mc
+
+    edges = {1: (1, 15), 16: (16, 31), 32: (32, 63), 64: (64, 127), 128: (128, 255), 256: (256, 511),
+             512: (512, 768), 1024: (769, 1024), 2048: (1025, 128000)}
+    assert mc.N_BUCKETS == edges
+    for n, want in [(1, 1), (15, 1), (16, 16), (31, 16), (32, 32), (768, 512), (769, 1024), (1025, 2048),
+                    (128000, 2048)]:
+        assert mc.bucket_of(n) == want
+    with pytest.raises(ValueError):
+        mc.bucket_of(128001)
+
+
+def test_invalid_configs_are_rejected_by_both_validators():
+    from tuna_amd import make_configs as mc
+    from tuna_amd import ops
+
+    good = dict(rows_per_wave=64, waves_m=2, waves_k=4, split_k=2, prefetch=4, x_chunk=512, token_tiles=1,
+                xcd_swizzle=0)
+    ops.validate_config(4096, 16, 4096, ops.GemmConfig.from_dict(good))
+    mc.validate(4096, 16, 4096, good)
+    bad = [dict(rows_per_wave=96), dict(prefetch=3), dict(token_tiles=3), dict(waves_m=3), dict(waves_k=32),
+           dict(waves_m=8, waves_k=4), dict(split_k=0), dict(split_k=129), dict(x_chunk=500), dict(x_chunk=256),
+           dict(x_chunk=1 << 16), dict(rows_per_wave=256, prefetch=8)]
+    for delta in bad:
+        c = dict(good, **delta)
+        with pytest.raises(ops.TunaError):
+            ops.validate_config(4096, 16, 4096, ops.GemmConfig.from_dict(c))
+        with pytest.raises(ValueError):
+            mc.validate(4096, 16, 4096, c)
+    for m, n, k in [(4100, 16, 4096), (4096, 16, 4100), (0, 16, 8), (8, 0, 8)]:
+        with pytest.raises(ops.TunaError):
+            ops.validate_config(m, n, k, ops.GemmConfig.from_dict(good))
+
+
+def test_generator_output_and_its_refusal_of_inconsistent_entries(tmp_path):
+    from tuna_amd import make_configs as mc
+
+    pm = {"4096_16_4096": dict(rows_per_wave=64, waves_m=1, waves_k=8, split_k=4, prefetch=2, x_chunk=1024,
+                               token_tiles=1, xcd_swizzle=1, us=9.9),
+          "4096_1_4096": dict(rows_per_wave=64, waves_m=1, waves_k=8, split_k=4, prefetch=2, x_chunk=1024,
+                              token_tiles=1, xcd_swizzle=0)}
+    text = mc.generate(pm)
+    assert "{4096, 16, 31, 4096, {64, 1, 8, 4, 2, 1024, 1, 1}}" in text
+    assert "{4096, 1, 15, 4096, {64, 1, 8, 4, 2, 1024, 1, 0}}" in text
+    assert "kConfigTableSize = 2" in text
+    # the checked-in table is what the generator produces from the checked-in json
+    with open(os.path.join(ROOT, "tuna_amd", "configs", "param_map.json")) as f:
+        real = json.load(f)
+    with open(os.path.join(ROOT, "tuna_amd", "csrc", "config_table.cpp")) as f:
+        assert f.read() == mc.generate(real)
+    # an entry like the reference's gemm_229376_4096_16 (thread count inconsistent with its warp grid) is refused
+    pm["229376_16_4096"] = dict(pm["4096_16_4096"], waves_m=8, waves_k=8)
+    with pytest.raises(ValueError, match="229376_16_4096"):
+        mc.generate(pm)
+    pm.pop("229376_16_4096")
+    pm["4096_17_4096"] = pm["4096_16_4096"]  # not a bucket key
+    with pytest.raises(ValueError):
+        mc.generate(pm)
+
+
+def test_tuner_repair_seeds_and_mutation_stay_valid():
+    import random
+
+    from tuna_amd import make_configs as mc
+    from tuna_amd import tuner
+
+    rng = random.Random(0)
+    for (m, n, k) in [(4096, 16, 4096), (229376, 16, 4096), (8192, 64, 28672), (8192, 1, 8192)]:
+        nk = mc.bucket_of(n)
+        pool = tuner.seeds(m, nk, k)
+        assert len(pool) > 20
+        for c in pool:
+            mc.validate(m, nk, k, c)
+        c = pool[0]
+        for _ in range(200):
+            d = tuner.mutate(c, rng, m, nk, k)
+            if d is not None:
+                mc.validate(m, nk, k, d)
+                c = d
+            e = tuner.crossover(c, rng.choice(pool), rng, m, nk, k)
+            if e is not None:
+                mc.validate(m, nk, k, e)
+    assert tuner.repair(dict(rows_per_wave=64, waves_m=8, waves_k=8, split_k=1, prefetch=2, x_chunk=512,
+                             token_tiles=1, xcd_swizzle=0), 4096, 16, 4096) is None
+
+
+def test_quantizer_matches_nearest_code_and_layout():
+    import torch
+
+    from oracle import oracle as O
+    from tuna_amd.quantize import quantize_blockwise_dynamic_4bit, unpack_codes
+
+    torch.manual_seed(0)
+    m, k = 64, 256
+    w = (torch.randn(m, k) * 0.05).half()
+    q, (absmax, code) = quantize_blockwise_dynamic_4bit(w, block_size=k, preprocess=True)
+    assert q.shape == (m // 8, k // 8, 32) and q.dtype == torch.uint8
+    assert absmax.dtype == torch.float32 and absmax.shape == (m,)
+    assert torch.equal(absmax, w.abs().amax(dim=1).float())
+    codes = unpack_codes(q, m, k).numpy()
+    # brute-force nearest entry (lowest index on ties) in float32, like the reference's argmin
+    norm = (w / absmax[:, None]).float().numpy()
+    cb = O.nf4_codebook()
+    want = np.abs(norm[:, :, None] - cb[None, None, :]).argmin(axis=2)
+    assert np.array_equal(codes, want)
+    # the packed bytes mean the same thing to the oracle
+    assert np.array_equal(O.unpack(q.numpy(), m, k), codes)
+    # unpacked variant returns flat codes
+    flat, _ = quantize_blockwise_dynamic_4bit(w, block_size=k, preprocess=False)
+    assert np.array_equal(flat.numpy().reshape(m, k), codes)
+    # decoded weights approximate the originals within half the widest code gap times absmax
+    img = O.dequant(q.numpy(), absmax.numpy(), cb, m, k, mode=O.D2).view(np.float16).astype(np.float32)
+    gap = np.diff(cb).max() / 2
+    assert (np.abs(img - w.float().numpy()) <= gap * absmax.numpy()[:, None] + 1e-3).all()
+
+
+def test_ops_reject_bad_arguments_without_touching_a_gpu():
+    import torch
+
+    from tuna_amd import ops
+
+    x = torch.zeros((16, 64), dtype=torch.float16)
+    q = torch.zeros((8, 8, 32), dtype=torch.uint8)
+    s = torch.ones(64)
+    c = torch.zeros(16)
+    o = torch.zeros((16, 64), dtype=torch.float16)
+    with pytest.raises(ValueError, match="HIP device"):
+        ops.matmul(x, q, s, c, o, 64, 16, 64)      # CPU tensors: there is no CPU fallback
+    with pytest.raises(ValueError):
+        ops.matmul(x, q, s, c, o, 60, 16, 64)
+    with pytest.raises(ValueError, match="HIP device"):
+        ops.dequant(q, s, c, torch.zeros((64, 64), dtype=torch.float16), 64, 64)
+
+
+def test_drop_in_module_has_the_reference_signatures():
+    import inspect
+
+    import tuna
+
+    assert list(inspect.signature(tuna.matmul).parameters)[:8] == ["x", "q", "s", "c", "o", "m", "n", "k"]
+    assert list(inspect.signature(tuna.dequant).parameters)[:6] == ["q", "absmax", "codebook", "o", "m", "k"]
+
+
+def test_synthetic_inputs_are_deterministic_and_in_range():
+    from tuna_amd.synth import SHAPES, make_inputs_np
+
+    a = make_inputs_np(64, 16, 128, seed=3)
+    b = make_inputs_np(64, 16, 128, seed=3)
+    for u, v in zip(a, b):
+        assert np.array_equal(u, v)
+    q, x, code, absmax = a
+    assert q.dtype == np.uint8 and q.shape == (8, 16, 32)
+    assert x.dtype == np.float16 and absmax.dtype == np.float32 and code.dtype == np.float32
+    assert (absmax >= 0.004999).all() and (absmax <= 0.02001).all()
+    assert np.array_equal(absmax, absmax.astype(np.float16).astype(np.float32))  # fp16-representable scales
+    assert len(SHAPES) == 10 and SHAPES["mistral_qkv"] == (6144, 4096)

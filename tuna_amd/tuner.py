@@ -37,6 +37,13 @@ GENES = {
 N_CU = 256
 
 
+def _pow2_floor(v: int) -> int:
+    p = 1
+    while p * 2 <= v:
+        p *= 2
+    return p
+
+
 def repair(c: dict, m: int, n_key: int, k: int):
     """Make a raw gene vector a valid config for the shape, or return None."""
     c = dict(c)
@@ -47,38 +54,43 @@ def repair(c: dict, m: int, n_key: int, k: int):
     # token tiles: never more tiles than the bucket's largest token count needs
     need = 1 if hi <= 16 or lo < 16 else (2 if lo < 32 else 4)
     c["token_tiles"] = min(c["token_tiles"], need)
-    unit = c["waves_k"] * c["prefetch"]          # k-steps per ring turn of the workgroup
+    threads = 64 * c["waves_m"] * c["waves_k"]
+    unit = 32 * c["waves_k"] * c["prefetch"]      # smallest x chunk: one ring turn of the workgroup
     c["split_k"] = max(1, min(int(c["split_k"]), steps))
     sps = -(-steps // c["split_k"])
-    # x chunk: a multiple of `unit` steps, at most what the split needs, within LDS
-    chunk_steps = max(unit, min(int(c.get("x_chunk", 1024)) // 32 // unit * unit, -(-sps // unit) * unit))
-    c["x_chunk"] = chunk_steps * 32
+    # x chunk: a power of two in [unit, 2*threads/token_tiles], no larger than the split needs
+    hi_chunk = _pow2_floor(max(unit, 2 * threads // c["token_tiles"]))
+    want = max(unit, min(_pow2_floor(max(int(c.get("x_chunk", 1024)), 1)), hi_chunk))
+    while want // 2 >= unit and want // 2 >= sps * 32:
+        want //= 2
+    c["x_chunk"] = want
     while True:
         try:
             make_configs.validate(m, n_key, k, c)
             return c
         except ValueError as e:
-            if "LDS" in str(e) and c["x_chunk"] > unit * 32:
-                c["x_chunk"] -= unit * 32
+            if "LDS" in str(e) and c["x_chunk"] // 2 >= unit:
+                c["x_chunk"] //= 2
                 continue
             return None
 
 
 def seeds(m: int, n_key: int, k: int):
     """Hand-derived starting points: fill the 256 CUs with 1-2 workgroups each."""
-    steps = -(-k // 32)
     out = []
-    for rpw in (64, 128, 256):
-        for wm, wk in ((1, 4), (1, 8), (2, 4), (2, 2), (4, 2), (1, 16), (2, 8), (4, 4), (4, 1), (8, 1)):
+    for rpw in (64, 128):
+        for wm, wk in ((1, 4), (1, 8), (2, 4), (2, 2), (4, 2), (1, 16), (2, 8), (4, 4), (4, 1), (8, 1), (1, 2)):
             row_tiles = -(-m // (rpw * wm))
             for target in (N_CU, 2 * N_CU, 4 * N_CU):
                 split = max(1, round(target / row_tiles))
                 for pf in (2, 4, 8):
                     for tt in (1, 2, 4):
-                        c = repair(dict(rows_per_wave=rpw, waves_m=wm, waves_k=wk, split_k=split, prefetch=pf,
-                                        x_chunk=min(2048, 32 * steps), token_tiles=tt, xcd_swizzle=0), m, n_key, k)
-                        if c is not None:
-                            out.append(c)
+                        for xc in (256, 512, 1024, 2048):
+                            for sw in (0, 1):
+                                c = repair(dict(rows_per_wave=rpw, waves_m=wm, waves_k=wk, split_k=split, prefetch=pf,
+                                                x_chunk=xc, token_tiles=tt, xcd_swizzle=sw), m, n_key, k)
+                                if c is not None:
+                                    out.append(c)
     uniq = {json.dumps(c, sort_keys=True): c for c in out}
     return list(uniq.values())
 
@@ -90,7 +102,7 @@ def mutate(c: dict, rng: random.Random, m, n_key, k):
         if gene == "split_k":
             c["split_k"] = max(1, int(round(c["split_k"] * rng.choice((0.5, 0.75, 1.25, 1.5, 2.0)) + rng.choice((-1, 0, 1)))))
         elif gene == "x_chunk":
-            c["x_chunk"] = max(32, int(c["x_chunk"] * rng.choice((0.5, 2.0))))
+            c["x_chunk"] = max(64, int(c["x_chunk"] * rng.choice((0.5, 2.0))))
         else:
             c[gene] = rng.choice(GENES[gene])
     return repair(c, m, n_key, k)
