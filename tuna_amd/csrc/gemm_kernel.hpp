@@ -270,6 +270,9 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 #pragma unroll
             for (int tt = 0; tt < TT; ++tt) acc[rw][j][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+#ifndef TUNA_DWORD_GROUP
+#define TUNA_DWORD_GROUP 0
+#endif
     // One k-step of this wave: B fragments from LDS, decode 4*RW dwords, 4*RW*TT MFMAs.
 #define TUNA_CONSUME(u, xoff)                                                                   \
     {                                                                                          \
@@ -281,6 +284,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
             const f16x8 av_ = decode_dword<DEC>(wq[u][rw][j], lut, lane4, sc16[rw][j], sc32[rw][j]); \
             _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) acc[rw][j][tt] =                 \
                 __builtin_amdgcn_mfma_f32_16x16x32_f16(av_, b_[tt], acc[rw][j][tt], 0, 0, 0);  \
+            if (TUNA_DWORD_GROUP > 0 && (j % TUNA_DWORD_GROUP) == TUNA_DWORD_GROUP - 1) __builtin_amdgcn_sched_barrier(0); \
         }                                                                                      \
     }
 
