@@ -139,12 +139,15 @@ CONFIGS = [
     dict(rows_per_wave=128, waves_m=2, waves_k=4, prefetch=4, x_chunk=1024, split_k=2),
     dict(rows_per_wave=128, waves_m=2, waves_k=2, prefetch=2, x_chunk=128),
     dict(rows_per_wave=128, waves_m=1, waves_k=1, prefetch=2, x_chunk=64, split_k=4, xcd_swizzle=1),
-    dict(waves_m=4, waves_k=4, prefetch=4, x_chunk=512, split_k=2, xcd_swizzle=1),  # 16 waves
+    dict(waves_m=4, waves_k=4, prefetch=2, x_chunk=512, split_k=2, xcd_swizzle=1),  # 16 waves
     dict(rows_per_wave=64, waves_m=1, waves_k=16, prefetch=2, x_chunk=2048),        # 16 waves along k
     dict(token_tiles=2, split_k=2, prefetch=2, x_chunk=256),
     dict(token_tiles=4, waves_m=2, waves_k=2, prefetch=2, x_chunk=128, split_k=5),
     dict(waves_m=1, waves_k=4, prefetch=4, x_chunk=512, split_k=7),                 # 4-wave workgroups
-    dict(waves_m=8, waves_k=1, prefetch=2, x_chunk=64),                             # no k split, many x chunks
+    dict(waves_m=8, waves_k=1, prefetch=2, x_chunk=64),                             # no k split: store from registers
+    dict(waves_m=16, waves_k=1, prefetch=2, x_chunk=64, xcd_swizzle=1),
+    dict(rows_per_wave=128, waves_m=4, waves_k=1, prefetch=2, x_chunk=64),
+    dict(token_tiles=2, waves_m=4, waves_k=1, prefetch=4, x_chunk=128),
     dict(waves_m=2, waves_k=2, prefetch=2, x_chunk=128, split_k=1),                 # many x chunks per workgroup
 ]
 

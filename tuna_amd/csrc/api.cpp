@@ -89,21 +89,24 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
         return fail(TUNA_ERR_UNSUPPORTED, "x_chunk=%d x token_tiles=%d exceeds 2 x threads=%d", c.x_chunk, c.token_tiles,
                     2 * threads);
 
+    // LDS = decode table + work area; the work area holds the x chunk in the main loop and, in
+    // the epilogue, two alternating buffers of one accumulator plane (1 KB) of every wave.
     const int nacc = rw * 4 * c.token_tiles;
     const int lut = decode == TUNA_DECODE_GEMM ? kLutBytes : 64;
-    const size_t main_lds = (size_t)lut + (size_t)c.token_tiles * 16 * (size_t)c.x_chunk * 2;
-    const size_t red_lds = (size_t)c.waves_k * c.waves_m * nacc * 1024;
-    const size_t tile_lds = (size_t)c.token_tiles * 16 * (rows_wg + 8) * 2;
-    const size_t epi_lds = red_lds + tile_lds + 16;
-    const size_t lds = main_lds > epi_lds ? main_lds : epi_lds;
+    const size_t x_lds = (size_t)c.token_tiles * 16 * (size_t)c.x_chunk * 2;
+    const size_t red_lds = (size_t)2 * c.waves_k * c.waves_m * 1024;
+    const size_t lds = (size_t)lut + (x_lds > red_lds ? x_lds : red_lds);
     if (lds > (size_t)kLdsLimit)
         return fail(TUNA_ERR_UNSUPPORTED, "config needs %zu bytes of LDS, the CU has %d", lds, kLdsLimit);
 
     // Two workgroups per CU need <= 128 VGPRs each: take that variant when both fit in LDS.
     int min_waves = threads > 512 ? 4 : 2;
+    int wgs_per_cu = 1;
     if (threads <= 512 && 2 * lds <= (size_t)kLdsLimit &&
-        gemm_variant_exists(rw, c.prefetch, c.token_tiles, decode, threads, 4))
+        gemm_variant_exists(rw, c.prefetch, c.token_tiles, decode, threads, 4)) {
         min_waves = 4;
+        wgs_per_cu = 2;
+    }
     if (!gemm_variant_exists(rw, c.prefetch, c.token_tiles, decode, threads, min_waves))
         return fail(TUNA_ERR_UNSUPPORTED,
                     "no kernel variant for rows_per_wave=%d prefetch=%d token_tiles=%d decode=%d threads=%d", c.rows_per_wave,
@@ -121,6 +124,7 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     p.token_tiles = c.token_tiles;
     p.decode = decode;
     p.min_waves = min_waves;
+    p.wgs_per_cu = wgs_per_cu;
     p.threads = threads;
     p.lds_bytes = lds;
     p.grid = dim3((unsigned)(row_tiles * c.split_k), (unsigned)tok_chunks, 1);
@@ -143,6 +147,8 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     a.xcd_swizzle = c.xcd_swizzle ? 1 : 0;
     a.lds_bytes = (int)lds;
     a.red_bytes = (int)red_lds;
+    a.planes_log2 = 0;
+    a.tiles_total = row_tiles * c.split_k;
     return TUNA_OK;
 }
 

@@ -29,11 +29,17 @@
 //     data.  One v_pk_mul_f16 applies the row's fp16 scale - the same single fp16
 //     rounding as the reference's `smemCode.get(nib) * absMax` (kernel.cu:2178-2192).
 //     Cost: 1 perm + 1 ds_read_b32 + 1 pk_mul per two weights.
+//   * Persistent workgroups: the grid is at most (CUs x workgroups per CU); a workgroup
+//     builds the decode table once and then walks tiles (row tile, k split) with stride
+//     gridDim.x.  The next tile's scales, weight ring and first x chunk are requested
+//     BEFORE the current tile's reduction and store, so the HBM stream never idles between
+//     tiles and the epilogue's latency is hidden behind the loads already in flight.
 //   * Split-K: waves_k waves of a workgroup cover interleaved k-steps; their accumulators
 //     meet in LDS and every thread sums a 1/waves_k share in wave order.  split_k
 //     workgroups write those fp32 sums to a workspace and the last one to arrive
-//     (device-scope counter) adds them in split order.  The fp16 result is transposed
-//     through LDS and stored with 16-byte, fully coalesced writes.  No atomics on the
+//     (device-scope counter) adds them in split order.  After the four planes of a 64-row
+//     group a thread owns 4 consecutive output features of one token: 8-byte stores, 32
+//     contiguous bytes per 4 lanes.  No atomics on the
 //     output (unlike kernel.cu:2739-2745), no pre-zeroing, and the result does not depend
 //     on arrival order.
 #pragma once
@@ -43,6 +49,7 @@ namespace tuna {
 
 typedef _Float16 f16;
 typedef f16 f16x2 __attribute__((ext_vector_type(2)));
+typedef f16 f16x4 __attribute__((ext_vector_type(4)));
 typedef f16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -150,10 +157,11 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 
     const int tid = threadIdx.x;
 #ifdef TUNA_TRACE
-#define TUNA_MARK(i) if (a.trace && tid == 0) a.trace[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + (i)] = wall_clock64();
+#define TUNA_MARK(i) if (a.trace && tid == 0 && tile_iter < 8) a.trace[((size_t)blockIdx.x * 8 + tile_iter) * 16 + (i)] = wall_clock64();
 #else
 #define TUNA_MARK(i)
 #endif
+    int tile_iter = 0;
     TUNA_MARK(0)
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -162,55 +170,38 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     const int i16 = lane & 15;
     const int g = lane >> 4;
     const int nthreads = (int)blockDim.x;
-
-    int id = blockIdx.x;
-    if (a.xcd_swizzle) {
-        const int total = gridDim.x;
-        if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
-    }
-    const int row_tile = id / a.split_k;
-    const int ks = id - row_tile * a.split_k;
     const int tok0 = blockIdx.y * (TT * 16);
     const int rows_wg = a.waves_m * (RW * kRowsPerLoad);
-    const int row0 = row_tile * rows_wg + wm * (RW * kRowsPerLoad);  // first weight row of this wave
-
-    const int sb = ks * a.steps_per_split;
-    const int se = min(a.steps_total, sb + a.steps_per_split);
-    const int nsteps = max(se - sb, 0);
-    const int n_it = nsteps > wk ? (nsteps - wk + a.waves_k - 1) >> a.wk_log2 : 0;
-
-    // Small operands first, all unconditional, so that every later wait on them can be an
-    // exact s_waitcnt vmcnt(N) that leaves the weight prefetches in flight.
-    const float code_lane = a.code[lane & 15];
-    float sc32[RW][4];
-#pragma unroll
-    for (int rw = 0; rw < RW; ++rw)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int row = row0 + rw * kRowsPerLoad + i16 * 4 + j;
-            sc32[rw][j] = a.absmax[min(row, a.m - 1)];  // rows past m are never stored
-        }
-
-    // ---- packed-weight stream ------------------------------------------------------------
-    // address = q + [uniform: 128 bytes per k-step] + [per lane: block row, row half, g]:
-    // the uniform part rides in SGPRs, so a load costs no vector ALU work.
     const int kb_total = a.k >> 3;
     const int mb_last = (a.m >> 3) - 1;
     const int g_last = min(g, kb_total - 1 - (a.steps_total - 1) * 4);  // last k-step may be short
+    const f16 *xg = reinterpret_cast<const f16 *>(a.x);
+    const int x_pieces = (TT * 16 * 4) << a.chunk_log2;  // 16-byte pieces per x chunk
+    const int s_stride = a.waves_k;                      // k-steps between a wave's consecutive iterations
+
+    // LDS: [decode table | work area].  The work area holds the x chunk during a tile's main
+    // loop and the reduction planes + fp16 output tile during its epilogue; the table is never
+    // overwritten, it serves every tile of this workgroup.
+    unsigned char *lut = smem;
+    unsigned char *work = smem + LUT_B;
+    const uint32_t lane4 = (uint32_t)lane << 2;
+
+    // ---- persistent tile walk -------------------------------------------------------------
+    int wg = blockIdx.x;
+    const int n_wg = gridDim.x;
+    if (a.xcd_swizzle && (n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
+
+    // state of the tile being fetched / computed
+    int row_tile = 0, ks = 0, sb = 0, nsteps = 0, n_it = 0, s_first = 0;
     uint32_t lb[RW], lb_last[RW];
-#pragma unroll
-    for (int rw = 0; rw < RW; ++rw) {
-        const int mb = min(((row0 + rw * kRowsPerLoad) >> 3) + (i16 >> 1), mb_last);
-        const uint32_t rowb = (uint32_t)mb * (uint32_t)kb_total * 32u + (uint32_t)(i16 & 1) * 16u;
-        lb[rw] = rowb + (uint32_t)g * 32u;
-        lb_last[rw] = rowb + (uint32_t)g_last * 32u;
-    }
+    float sc32[RW][4];
     u32x4 wq[U][RW];
-    const int s_first = sb + wk;            // this wave's first k-step
-    const int s_stride = a.waves_k;         // k-steps between its consecutive iterations
+    XStage xst;
+
     // Unconditional by design: a load whose step lies beyond this wave's share is clamped
     // to the last k-step and its data is never used.  Only loads that are always issued
     // let the compiler count outstanding loads exactly (s_waitcnt vmcnt(N > 0)).
+    // address = q + [uniform: 128 bytes per k-step, in SGPRs] + [per lane: block row, half, g]
 #define TUNA_LOAD_STEP(u, it)                                                                  \
     {                                                                                          \
         const int s_ = min(s_first + (it) * s_stride, a.steps_total - 1);                      \
@@ -219,28 +210,40 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
         _Pragma("unroll") for (int rw = 0; rw < RW; ++rw) wq[u][rw] = __builtin_nontemporal_load( \
             reinterpret_cast<const u32x4 *>(base_ + (last_ ? lb_last[rw] : lb[rw])));          \
     }
-#pragma unroll
-    for (int u = 0; u < U; ++u) TUNA_LOAD_STEP(u, u)
 
-    // first batch of the first x chunk: in flight while the decode table is built
-    const f16 *xg = reinterpret_cast<const f16 *>(a.x);
-    const int x_pieces = (TT * 16 * 4) << a.chunk_log2;  // 16-byte pieces per chunk
-    XStage xst;
-    x_stage_load<TT>(xst, xg, 0, nthreads, tid, x_pieces, tok0, sb * kStepK, a.n, a.k);
+    // Request what tile `t` needs from HBM first: scales and the weight ring.  (The first x
+    // chunk comes from L2 and is requested at the start of the tile, behind these loads: it
+    // would cost 16 registers across the previous tile's epilogue.)
+#define TUNA_TILE_FETCH(t)                                                                      \
+    {                                                                                          \
+        row_tile = (t) / a.split_k;                                                            \
+        ks = (t) - row_tile * a.split_k;                                                       \
+        const int row0_ = row_tile * rows_wg + wm * (RW * kRowsPerLoad);                       \
+        sb = ks * a.steps_per_split;                                                           \
+        nsteps = max(min(a.steps_total, sb + a.steps_per_split) - sb, 0);                      \
+        n_it = nsteps > wk ? (nsteps - wk + a.waves_k - 1) >> a.wk_log2 : 0;                   \
+        s_first = sb + wk;                                                                     \
+        _Pragma("unroll") for (int rw = 0; rw < RW; ++rw)                                      \
+        {                                                                                      \
+            _Pragma("unroll") for (int j = 0; j < 4; ++j)                                      \
+            {                                                                                  \
+                const int row_ = row0_ + rw * kRowsPerLoad + i16 * 4 + j;                      \
+                sc32[rw][j] = a.absmax[min(row_, a.m - 1)]; /* rows past m are never stored */ \
+            }                                                                                  \
+            const int mb_ = min(((row0_ + rw * kRowsPerLoad) >> 3) + (i16 >> 1), mb_last);     \
+            const uint32_t rowb_ = (uint32_t)mb_ * (uint32_t)kb_total * 32u + (uint32_t)(i16 & 1) * 16u; \
+            lb[rw] = rowb_ + (uint32_t)g * 32u;                                                \
+            lb_last[rw] = rowb_ + (uint32_t)g_last * 32u;                                      \
+        }                                                                                      \
+        _Pragma("unroll") for (int u = 0; u < U; ++u) TUNA_LOAD_STEP(u, u)                     \
+    }
 
+    int t = wg;
+    const float code_lane = a.code[lane & 15];
+    if (t < a.tiles_total) TUNA_TILE_FETCH(t)
     TUNA_MARK(1)
-    // ---- per-row scales (fp16 like the reference's staging, kernel.cu:2770) -----------
-    f16x2 sc16[RW][4];
-#pragma unroll
-    for (int rw = 0; rw < RW; ++rw)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const f16 h = (f16)sc32[rw][j];
-            sc16[rw][j] = f16x2{h, h};
-        }
 
-    // ---- decode table -------------------------------------------------------------------
-    unsigned char *lut = smem;
+    // ---- decode table, once per workgroup ------------------------------------------------
     if constexpr (DEC == TUNA_DECODE_GEMM) {
         // Lane l holds fp16(code[l % 16]) (kernel.cu:2800 rounds the codebook to fp16);
         // entries are gathered across lanes, no memory traffic.
@@ -257,18 +260,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     } else {
         if (tid < 16) reinterpret_cast<float *>(lut)[tid] = code_lane;
     }
-    const uint32_t lane4 = (uint32_t)lane << 2;
     TUNA_MARK(2)
-
-    unsigned char *xs = smem + LUT_B;
-
-    f32x4 acc[RW][4][TT];
-#pragma unroll
-    for (int rw = 0; rw < RW; ++rw)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int tt = 0; tt < TT; ++tt) acc[rw][j][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
 #ifndef TUNA_DWORD_GROUP
 #define TUNA_DWORD_GROUP 0
@@ -281,13 +273,11 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
             *reinterpret_cast<const f16x8 *>(xb + tt * 256 + (xoff));                          \
         _Pragma("unroll") for (int rw = 0; rw < RW; ++rw) _Pragma("unroll") for (int j = 0; j < 4; ++j) \
         {                                                                                      \
-            const f16x8 av_ = decode_dword<DEC>(wq[u][rw][j], lut, lane4, sc16[rw][j], sc32[rw][j]); \
+            const f16x8 av_ = decode_dword<DEC>(wq[u][rw][j], lut, lane4, sc16[rw][j], sc32c[rw][j]); \
             _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) acc[rw][j][tt] =                 \
                 __builtin_amdgcn_mfma_f32_16x16x32_f16(av_, b_[tt], acc[rw][j][tt], 0, 0, 0);  \
-            if (TUNA_DWORD_GROUP > 0 && (j % TUNA_DWORD_GROUP) == TUNA_DWORD_GROUP - 1) __builtin_amdgcn_sched_barrier(0); \
         }                                                                                      \
     }
-
     // One group = U consecutive iterations of this wave: every ring slot is consumed and
     // refilled, no branches inside (refill addresses are clamped, see TUNA_LOAD_STEP).
 #define TUNA_GROUP()                                                                            \
@@ -304,154 +294,227 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     }
 
     const int ipc = a.chunk_steps >> a.wk_log2;  // iterations per chunk per wave (multiple of U)
-    const int n_chunks = (nsteps + a.chunk_steps - 1) >> a.chunk_log2;
     const int wstep = a.waves_k * (1024 * TT);   // LDS bytes between this wave's consecutive steps
-    int it = 0;                                  // this wave's next iteration (multiple of U)
 
-    // chunk 0 of x: loaded above, written here
-    if (n_chunks > 0) x_stage_store<TT>(xst, xs, 0, nthreads, tid, x_pieces, tok0, sb * kStepK, a.n, a.k);
-    __syncthreads();
-    TUNA_MARK(3)
-
-    for (int c = 0; c < n_chunks; ++c) {
-        const int it_chunk0 = c * ipc;
-        const bool has_next = c + 1 < n_chunks;
-        // B fragment of lane (token i16, k-group g), local step sl: slot sl*4+g, piece slot*16*TT + i16
-        const unsigned char *xb = xs + g * (256 * TT) + i16 * 16 + wk * (1024 * TT) - it_chunk0 * wstep;
-        if (has_next) {
-            // A chunk with a successor is full: every wave owns all ipc iterations of it.
-            const int it_peel = it_chunk0 + ipc - U;
-            while (it < it_peel) TUNA_GROUP()
-            // Last group of the chunk: the next chunk of x is fetched into registers first, so
-            // that after the group exactly U*RW younger loads are in flight and the wait before
-            // the LDS write below is an exact vmcnt, not a drain of the weight ring.
-            const int kbase = (sb + (c + 1) * a.chunk_steps) * kStepK;
-            x_stage_load<TT>(xst, xg, 0, nthreads, tid, x_pieces, tok0, kbase, a.n, a.k);
-            TUNA_GROUP()
-            __syncthreads();  // every wave is done reading chunk c
-            x_stage_store<TT>(xst, xs, 0, nthreads, tid, x_pieces, tok0, kbase, a.n, a.k);
-            __syncthreads();
-        } else {
-            const int it_end = min(it_chunk0 + ipc, n_it);
-            // steady state while both the group and its refills lie inside this wave's share
-            while (it + U <= it_end && it + 2 * U <= n_it) TUNA_GROUP()
-            if (it + U <= it_end && it + U == n_it) {
-                // last full group of the wave: drain the ring, nothing left to fetch
+    for (; t < a.tiles_total; t += n_wg) {
+        // ---- this tile's scales (fp16 like the reference's staging, kernel.cu:2770) -------
+        f16x2 sc16[RW][4];
+        float sc32c[RW][4];
 #pragma unroll
-                for (int u = 0; u < U; ++u) TUNA_CONSUME(u, (it + u) * wstep)
-                it += U;
-            } else {
-                // ragged tail (fewer than U steps left in the wave or in the chunk)
-                while (it < it_end) {
+        for (int rw = 0; rw < RW; ++rw)
 #pragma unroll
-                    for (int u = 0; u < U; ++u) {
-                        if (it + u < it_end) {
-                            TUNA_CONSUME(u, (it + u) * wstep)
-                            if (it + u + U < n_it) TUNA_LOAD_STEP(u, it + u + U)
-                        }
-                    }
-                    it += U;
-                }
+            for (int j = 0; j < 4; ++j) {
+                const f16 h = (f16)sc32[rw][j];
+                sc16[rw][j] = f16x2{h, h};
+                sc32c[rw][j] = sc32[rw][j];
             }
-        }
-    }
-#undef TUNA_GROUP
-#undef TUNA_CONSUME
-#undef TUNA_LOAD_STEP
-    TUNA_MARK(4)
-
-    // ---- workgroup reduction: accumulators meet in LDS, every thread sums a share ------
-    // A wave's accumulators are the float array [plane][lane][4] (NACC*256 floats); thread
-    // (wk, lane) of row group wm owns floats f = (i*waves_k + wk)*64 + lane, i < nf.
-    __syncthreads();  // table and x are dead from here on
-    {
-        f32x4 *dst = reinterpret_cast<f32x4 *>(smem) + (size_t)(wm * a.waves_k + wk) * (NACC * 64) + lane;
+        f32x4 acc[RW][4][TT];
 #pragma unroll
         for (int rw = 0; rw < RW; ++rw)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int tt = 0; tt < TT; ++tt) dst[((rw * 4 + j) * TT + tt) * 64] = acc[rw][j][tt];
-    }
-    __syncthreads();
-    TUNA_MARK(5)
-    const float *redf = reinterpret_cast<const float *>(smem) + (size_t)wm * a.waves_k * (NACC * 256);
-    const int nf = (NACC * 4) >> a.wk_log2;
-    f16 *tile = reinterpret_cast<f16 *>(smem + a.red_bytes);  // [token][rows_wg + 8] fp16
-    const int tile_ld = rows_wg + 8;
-    // float f = (plane*64 + l)*4 + v is token (plane % TT)*16 + l%16, weight row
-    // (plane / (4*TT))*64 + 16*(l/16) + 4*v + (plane / TT) % 4 of the wave
-#define TUNA_TILE_PUT(f, val)                                                                   \
-    {                                                                                          \
-        const int pl_ = (f) >> 8, l_ = ((f) >> 2) & 63, v_ = (f) & 3;                          \
-        const int tok_ = (pl_ % TT) * 16 + (l_ & 15);                                          \
-        const int row_ = wm * (RW * kRowsPerLoad) + (pl_ / (4 * TT)) * 64 + (l_ >> 4) * 16 + v_ * 4 + (pl_ / TT) % 4; \
-        tile[tok_ * tile_ld + row_] = (f16)(val);                                              \
-    }
+                for (int tt = 0; tt < TT; ++tt) acc[rw][j][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    if (a.split_k == 1) {
-        for (int i = 0; i < nf; ++i) {
-            const int f = ((i << a.wk_log2) + wk) * 64 + lane;
-            float s = 0.f;
-            for (int w = 0; w < a.waves_k; ++w) s += redf[(size_t)w * (NACC * 256) + f];
-            TUNA_TILE_PUT(f, s)
+        const int cur_row_tile = row_tile, cur_ks = ks, cur_sb = sb;
+        const int n_chunks = (nsteps + a.chunk_steps - 1) >> a.chunk_log2;
+        int it = 0;  // this wave's next iteration (multiple of U)
+
+        // chunk 0 of x; the work area is free again once every wave has left the previous
+        // tile's epilogue
+        x_stage_load<TT>(xst, xg, 0, nthreads, tid, x_pieces, tok0, cur_sb * kStepK, a.n, a.k);
+        __syncthreads();
+        if (n_chunks > 0) x_stage_store<TT>(xst, work, 0, nthreads, tid, x_pieces, tok0, cur_sb * kStepK, a.n, a.k);
+        __syncthreads();
+        TUNA_MARK(3)
+
+        for (int c = 0; c < n_chunks; ++c) {
+            const int it_chunk0 = c * ipc;
+            const bool has_next = c + 1 < n_chunks;
+            // B fragment of lane (token i16, k-group g), local step sl: slot sl*4+g, piece slot*16*TT + i16
+            const unsigned char *xb = work + g * (256 * TT) + i16 * 16 + wk * (1024 * TT) - it_chunk0 * wstep;
+            if (has_next) {
+                // A chunk with a successor is full: every wave owns all ipc iterations of it.
+                const int it_peel = it_chunk0 + ipc - U;
+                while (it < it_peel) TUNA_GROUP()
+                // Last group of the chunk: the next chunk of x is fetched into registers first, so
+                // that after the group exactly U*RW younger loads are in flight and the wait before
+                // the LDS write below is an exact vmcnt, not a drain of the weight ring.
+                const int kbase = (cur_sb + (c + 1) * a.chunk_steps) * kStepK;
+                x_stage_load<TT>(xst, xg, 0, nthreads, tid, x_pieces, tok0, kbase, a.n, a.k);
+                TUNA_GROUP()
+                __syncthreads();  // every wave is done reading chunk c
+                x_stage_store<TT>(xst, work, 0, nthreads, tid, x_pieces, tok0, kbase, a.n, a.k);
+                __syncthreads();
+            } else {
+                const int it_end = min(it_chunk0 + ipc, n_it);
+                // steady state while both the group and its refills lie inside this wave's share
+                while (it + U <= it_end && it + 2 * U <= n_it) TUNA_GROUP()
+                if (it + U <= it_end && it + U == n_it) {
+                    // last full group of the wave: drain the ring, nothing left to fetch
+#pragma unroll
+                    for (int u = 0; u < U; ++u) TUNA_CONSUME(u, (it + u) * wstep)
+                    it += U;
+                } else {
+                    // ragged tail (fewer than U steps left in the wave or in the chunk)
+                    while (it < it_end) {
+#pragma unroll
+                        for (int u = 0; u < U; ++u) {
+                            if (it + u < it_end) {
+                                TUNA_CONSUME(u, (it + u) * wstep)
+                                if (it + u + U < n_it) TUNA_LOAD_STEP(u, it + u + U)
+                            }
+                        }
+                        it += U;
+                    }
+                }
+            }
         }
-    } else {
-        // Partials travel as device-scope relaxed atomics (write-through stores, L2-bypassing
-        // loads): coherent across the 8 XCD L2s without the L2 write-back/invalidate that a
-        // device-scope release/acquire fence costs on every workgroup.  Order is given by
-        // "all my stores have completed" (workgroup-scope release = s_waitcnt vmcnt(0))
-        // before the barrier that precedes the arrival counter's increment.
-        const size_t tile_id = (size_t)blockIdx.y * a.row_tiles + row_tile;
+        TUNA_MARK(4)
+
+        // ---- next tile: get its loads going before this tile's reduction and store ---------
+        if (t + n_wg < a.tiles_total) TUNA_TILE_FETCH(t + n_wg)
+
+        // ---- workgroup reduction and store, one accumulator plane per pass ------------------
+        // A plane is one float4 per lane = 256 floats [lane][4].  The waves_k waves of a row
+        // group put their copies of a plane side by side in LDS (two buffers alternate, so one
+        // barrier per plane) and thread (wk, lane) sums the floats f = (i*waves_k + wk)*64 + lane
+        // of it in wave order.  Float f = l*4 + v of the plane of MFMA j is token l%16 and
+        // weight row 16*(l/16) + 4*v + j of the wave's 64: after the four planes j = 0..3 a
+        // thread owns 4 consecutive output features of one token and stores them as 8 bytes.
+        // The per-thread index arithmetic does not depend on the tile; an opaque copy of the
+        // lane id keeps the compiler from hoisting it out of the tile loop into registers that
+        // would stay live across the main loop.
+        int lane_e = lane, wk_e = wk, wm_e = wm;
+        asm volatile("" : "+v"(lane_e));
+        asm volatile("" : "+s"(wk_e), "+s"(wm_e));
+        const size_t plane_floats = (size_t)(a.waves_m * a.waves_k) * 256;  // one buffer
+        float *redf = reinterpret_cast<float *>(work);
+        const size_t tile_id = (size_t)blockIdx.y * a.row_tiles + cur_row_tile;
+        // workspace of a tile: [split][wm][rw][tt][f][j] floats
         float *wst = a.ws + (tile_id * a.split_k * a.waves_m) * (size_t)(NACC * 256);
-        float *mine = wst + ((size_t)ks * a.waves_m + wm) * (NACC * 256);
-        for (int i = 0; i < nf; ++i) {
-            const int f = ((i << a.wk_log2) + wk) * 64 + lane;
-            float s = 0.f;
-            for (int w = 0; w < a.waves_k; ++w) s += redf[(size_t)w * (NACC * 256) + f];
-            __hip_atomic_store(mine + f, s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __syncthreads();
-        TUNA_MARK(6)
-        volatile unsigned *ticket = reinterpret_cast<volatile unsigned *>(smem + a.lds_bytes - 16);
-        if (tid == 0)
-            *ticket = __hip_atomic_fetch_add(a.counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        TUNA_MARK(7)
-        if (*ticket != (unsigned)(a.split_k - 1)) return;
-        // last workgroup of this tile: every partial is in memory; add them in split order
-        if (tid == 0) __hip_atomic_store(a.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        for (int i = 0; i < nf; ++i) {
-            const int f = ((i << a.wk_log2) + wk) * 64 + lane;
-            const float *src = wst + (size_t)wm * (NACC * 256) + f;
-            float s = 0.f;
-            for (int sp = 0; sp < a.split_k; ++sp)
-                s += __hip_atomic_load(src + (size_t)sp * a.waves_m * (NACC * 256), __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
-            TUNA_TILE_PUT(f, s)
-        }
-    }
-#undef TUNA_TILE_PUT
-    __syncthreads();
-    TUNA_MARK(8)
-
-    // ---- store the [tokens][rows_wg] fp16 tile: 16 bytes per thread, rows contiguous ---
-    {
+        float *mine = wst + ((size_t)cur_ks * a.waves_m + wm_e) * (NACC * 256);
         f16 *outp = reinterpret_cast<f16 *>(a.out);
-        constexpr int RW_LOG2 = RW == 1 ? 0 : (RW == 2 ? 1 : 2);
-        const int r8_log2 = a.wm_log2 + RW_LOG2 + 3;  // log2(rows_wg / 8)
-        const int pieces = (TT * 16) << r8_log2;
-        for (int p = tid; p < pieces; p += nthreads) {
-            const int tok = p >> r8_log2;
-            const int r8 = p & ((1 << r8_log2) - 1);
-            const int row = row_tile * rows_wg + r8 * 8;
-            if (tok0 + tok < a.n && row + 8 <= a.m)
-                *reinterpret_cast<u32x4 *>(outp + (size_t)(tok0 + tok) * a.m + row) =
-                    *reinterpret_cast<const u32x4 *>(tile + tok * tile_ld + r8 * 8);
+        bool write_out = true;
+        if (a.waves_k == 1 && a.split_k == 1) {
+            // No k split at all: the wave's accumulators are final.  Lane (token i16, group g)
+            // owns 16 consecutive output features, acc[rw][j][tt][v] being feature 4*v + j of
+            // them: two 16-byte stores per 64-row group, no LDS, no barrier.
+#pragma unroll
+            for (int tt = 0; tt < TT; ++tt) {
+                const int tok = tok0 + tt * 16 + (lane_e & 15);
+#pragma unroll
+                for (int rw = 0; rw < RW; ++rw) {
+                    const int rb = cur_row_tile * rows_wg + wm_e * (RW * kRowsPerLoad) + rw * 64 + (lane_e >> 4) * 16;
+                    f16x8 lo, hi;
+#pragma unroll
+                    for (int v = 0; v < 2; ++v)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            lo[v * 4 + j] = (f16)acc[rw][j][tt][v];
+                            hi[v * 4 + j] = (f16)acc[rw][j][tt][v + 2];
+                        }
+                    f16 *dst = outp + (size_t)tok * a.m + rb;
+                    if (tok < a.n && rb + 8 <= a.m) *reinterpret_cast<f16x8 *>(dst) = lo;
+                    if (tok < a.n && rb + 16 <= a.m) *reinterpret_cast<f16x8 *>(dst + 8) = hi;
+                }
+            }
+            ++tile_iter;
+            continue;
         }
+        __syncthreads();  // every wave has left the main loop: the work area is free
+#pragma unroll
+        for (int rw = 0; rw < RW; ++rw)
+#pragma unroll
+            for (int tt = 0; tt < TT; ++tt) {
+                float o[4][4];  // [i][j]
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float *buf = redf + ((rw * TT + tt) * 4 + j) % 2 * plane_floats;
+                    reinterpret_cast<f32x4 *>(buf)[(size_t)(wm_e * a.waves_k + wk_e) * 64 + lane_e] = acc[rw][j][tt];
+                    __syncthreads();
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int f = ((i << a.wk_log2) + wk_e) * 64 + lane_e;
+                        float sum = 0.f;
+                        if (f < 256)
+                            for (int w = 0; w < a.waves_k; ++w) sum += buf[(size_t)(wm_e * a.waves_k + w) * 256 + f];
+                        o[i][j] = sum;
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int f = ((i << a.wk_log2) + wk_e) * 64 + lane_e;
+                    if (f >= 256) continue;
+                    if (a.split_k == 1) {
+                        const int l = f >> 2, v = f & 3;
+                        const int tok = tok0 + tt * 16 + (l & 15);
+                        const int row = cur_row_tile * rows_wg + wm_e * (RW * kRowsPerLoad) + rw * 64 + (l >> 4) * 16 + v * 4;
+                        if (tok < a.n && row + 4 <= a.m) {
+                            f16x4 h = {(f16)o[i][0], (f16)o[i][1], (f16)o[i][2], (f16)o[i][3]};
+                            *reinterpret_cast<f16x4 *>(outp + (size_t)tok * a.m + row) = h;
+                        }
+                    } else {
+                        float *dst = mine + ((size_t)(rw * TT + tt) * 256 + f) * 4;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            __hip_atomic_store(dst + j, o[i][j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                }
+            }
+        TUNA_MARK(5)
+
+        if (a.split_k > 1) {
+            // Partials travel as device-scope relaxed atomics (write-through stores, L2-bypassing
+            // loads): coherent across the 8 XCD L2s without the L2 write-back/invalidate that a
+            // device-scope release/acquire fence costs on every workgroup.  Order is given by
+            // "all my stores have completed" (an explicit s_waitcnt vmcnt(0)) before the barrier
+            // that precedes the arrival counter's increment.
+            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): a workgroup-scope fence does not wait for global stores
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __syncthreads();  // also: every read of the reduction buffers is done
+            TUNA_MARK(6)
+            volatile unsigned *ticket = reinterpret_cast<volatile unsigned *>(work);
+            if (wk_e + wm_e == 0 && lane_e == 0)
+                *ticket = __hip_atomic_fetch_add(a.counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            TUNA_MARK(7)
+            write_out = *ticket == (unsigned)(a.split_k - 1);
+            if (write_out) {
+                // last workgroup of this tile: every partial is in memory; add them in split order
+                if (wk_e + wm_e == 0 && lane_e == 0)
+                    __hip_atomic_store(a.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (int rt = 0; rt < RW * TT; ++rt)
+                    for (int i = 0; i < 4; ++i) {
+                        const int f = ((i << a.wk_log2) + wk_e) * 64 + lane_e;
+                        if (f >= 256) break;
+                        const float *src = wst + (size_t)wm_e * (NACC * 256) + ((size_t)rt * 256 + f) * 4;
+                        float s4[4] = {0.f, 0.f, 0.f, 0.f};
+                        for (int sp = 0; sp < a.split_k; ++sp) {
+                            const float *sps = src + (size_t)sp * a.waves_m * (NACC * 256);
+#pragma unroll
+                            for (int j = 0; j < 4; ++j)
+                                s4[j] += __hip_atomic_load(sps + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        }
+                        const int rw = rt / TT, tt = rt % TT;
+                        const int l = f >> 2, v = f & 3;
+                        const int tok = tok0 + tt * 16 + (l & 15);
+                        const int row = cur_row_tile * rows_wg + wm_e * (RW * kRowsPerLoad) + rw * 64 + (l >> 4) * 16 + v * 4;
+                        if (tok < a.n && row + 4 <= a.m) {
+                            f16x4 h = {(f16)s4[0], (f16)s4[1], (f16)s4[2], (f16)s4[3]};
+                            *reinterpret_cast<f16x4 *>(outp + (size_t)tok * a.m + row) = h;
+                        }
+                    }
+            }
+        }
+        TUNA_MARK(8)
+        TUNA_MARK(9)
+        ++tile_iter;
     }
-    TUNA_MARK(9)
+#undef TUNA_GROUP
+#undef TUNA_CONSUME
+#undef TUNA_TILE_FETCH
+#undef TUNA_LOAD_STEP
 #undef TUNA_MARK
 }
 

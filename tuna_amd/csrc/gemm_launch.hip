@@ -15,20 +15,20 @@ struct Variant {
 #define V(RW, U, TT, DEC, MAXT, MINW) {RW, U, TT, DEC, MAXT, MINW, gemm_kernel<RW, U, TT, DEC, MAXT, MINW>}
 #define G TUNA_DECODE_GEMM
 
-// Only variants that compile with no (or a handful of) register spills are listed;
+// Only variants whose main loop compiles without register spills are listed (a spill in the
+// loop is a scratch access that drains the prefetch ring); the 4-token-tile variants are the
+// exception: they spill a few values and are kept so that 33+ tokens take one pass;
 // tuna_amd/make_configs.py mirrors this list.
 //   MAXT 512 / MINW 2 : up to 8 waves per workgroup, up to 256 VGPRs
 //   MAXT 512 / MINW 4 : up to 8 waves, at most 128 VGPRs, so that two workgroups share a CU
 //   MAXT 1024 / MINW 4: 16-wave workgroups
 static const Variant kVariants[] = {
     V(1, 2, 1, G, 512, 2), V(1, 2, 2, G, 512, 2), V(1, 2, 4, G, 512, 2),
-    V(1, 4, 1, G, 512, 2), V(1, 4, 2, G, 512, 2), V(1, 4, 4, G, 512, 2),
+    V(1, 4, 1, G, 512, 2), V(1, 4, 2, G, 512, 2),
     V(1, 8, 1, G, 512, 2), V(1, 8, 2, G, 512, 2),
-    V(2, 2, 1, G, 512, 2), V(2, 2, 2, G, 512, 2),
-    V(2, 4, 1, G, 512, 2), V(2, 4, 2, G, 512, 2),
-    V(2, 8, 1, G, 512, 2), V(4, 2, 1, G, 512, 2),
-    V(1, 2, 1, G, 512, 4), V(1, 4, 1, G, 512, 4), V(1, 8, 1, G, 512, 4), V(1, 2, 2, G, 512, 4), V(2, 2, 1, G, 512, 4), V(2, 4, 1, G, 512, 4),
-    V(1, 2, 1, G, 1024, 4), V(1, 4, 1, G, 1024, 4), V(1, 8, 1, G, 1024, 4), V(2, 2, 1, G, 1024, 4),
+    V(2, 2, 1, G, 512, 2), V(2, 4, 1, G, 512, 2),
+    V(1, 2, 1, G, 512, 4),
+    V(1, 2, 1, G, 1024, 4),
     // dequant-rounding decode (correctness mode, not tuned)
     V(1, 2, 1, TUNA_DECODE_DEQUANT, 512, 2), V(1, 2, 2, TUNA_DECODE_DEQUANT, 512, 2),
     V(1, 2, 4, TUNA_DECODE_DEQUANT, 512, 2),
@@ -56,6 +56,7 @@ bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int 
 // Dynamic LDS above 64 KB needs a one-time opt-in per kernel and device.
 static std::mutex g_attr_mutex;
 static unsigned char g_attr_done[16][kNumVariants];
+static int g_cu_count[16];
 
 hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
 {
@@ -66,8 +67,16 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
     const int vi = (int)(v - kVariants);
+    int cus;
     {
         std::lock_guard<std::mutex> lock(g_attr_mutex);
+        if (!g_cu_count[dev]) {
+            int n = 0;
+            e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+            if (e != hipSuccess) return e;
+            g_cu_count[dev] = n > 0 ? n : 256;
+        }
+        cus = g_cu_count[dev];
         if (!g_attr_done[dev][vi]) {
             e = hipFuncSetAttribute(reinterpret_cast<const void *>(v->fn),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
@@ -75,7 +84,11 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
             g_attr_done[dev][vi] = 1;
         }
     }
-    hipLaunchKernelGGL(v->fn, plan.grid, dim3(plan.threads), plan.lds_bytes, stream, plan.args);
+    // persistent workgroups: as many as the device holds at once, each walks tiles with this stride
+    dim3 grid = plan.grid;
+    const unsigned slots = (unsigned)(cus * plan.wgs_per_cu);
+    if (grid.x > slots) grid.x = slots;
+    hipLaunchKernelGGL(v->fn, grid, dim3(plan.threads), plan.lds_bytes, stream, plan.args);
     return hipGetLastError();
 }
 

@@ -37,7 +37,9 @@ struct GemmArgs {
     int row_tiles;        // workgroups along m
     int xcd_swizzle;
     int lds_bytes;        // dynamic LDS size of the launch (last 16 bytes: arrival ticket)
-    int red_bytes;        // bytes of the workgroup reduction area = offset of the fp16 output tile
+    int red_bytes;        // bytes of the reduction area in the LDS work area = offset of the fp16 output tile
+    int planes_log2;      // log2(accumulator planes reduced per epilogue pass)
+    int tiles_total;      // row_tiles * split_k: tiles walked by the persistent workgroups
 #ifdef TUNA_TRACE
     unsigned long long *trace;  // development builds only: 16 timestamps per workgroup
 #endif
@@ -49,6 +51,7 @@ struct GemmPlan {
     int threads;
     int rw, prefetch, token_tiles, decode;
     int min_waves;  // waves per SIMD the variant is compiled for (2: <=256 VGPRs, 4: <=128)
+    int wgs_per_cu; // workgroups of this launch that fit on one CU (LDS and registers)
     size_t lds_bytes;
     size_t ws_bytes;
     size_t n_counters;

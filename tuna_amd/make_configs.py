@@ -46,8 +46,8 @@ STEP_K = 32
 # for <= 8 waves with <= 128 VGPRs (two workgroups per CU) and for 16-wave workgroups;
 # must match kVariants in csrc/gemm_launch.hip
 VARIANTS_512 = {(1, 2, 1), (1, 2, 2), (1, 2, 4), (1, 4, 1), (1, 4, 2), (1, 8, 1), (1, 8, 2), (2, 2, 1), (2, 4, 1)}
-VARIANTS_512_2WG = {(1, 2, 1), (1, 4, 1)}
-VARIANTS_1024 = {(1, 2, 1), (1, 4, 1)}
+VARIANTS_512_2WG = {(1, 2, 1)}
+VARIANTS_1024 = {(1, 2, 1)}
 
 
 def _pow2(v: int) -> bool:
@@ -100,13 +100,10 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
 
 
 def lds_bytes(c: dict) -> int:
-    """Dynamic LDS of a launch: max(decode table + x chunk, reduction area + output tile)."""
-    rw = c["rows_per_wave"] // 64
-    nacc = rw * 4 * c["token_tiles"]
-    main = LUT_BYTES + c["token_tiles"] * 16 * c["x_chunk"] * 2
-    red = c["waves_k"] * c["waves_m"] * nacc * 1024
-    tile = c["token_tiles"] * 16 * (c["rows_per_wave"] * c["waves_m"] + 8) * 2
-    return max(main, red + tile + 16)
+    """Dynamic LDS of a launch: decode table + max(x chunk, two reduction buffers of one plane per wave)."""
+    x = c["token_tiles"] * 16 * c["x_chunk"] * 2
+    red = 2 * c["waves_k"] * c["waves_m"] * 1024
+    return LUT_BYTES + max(x, red)
 
 
 def generate(param_map: dict) -> str:

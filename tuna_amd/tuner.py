@@ -79,7 +79,8 @@ def seeds(m: int, n_key: int, k: int):
     """Hand-derived starting points: fill the 256 CUs with 1-2 workgroups each."""
     out = []
     for rpw in (64, 128):
-        for wm, wk in ((1, 4), (1, 8), (2, 4), (2, 2), (4, 2), (1, 16), (2, 8), (4, 4), (4, 1), (8, 1), (1, 2)):
+        for wm, wk in ((1, 4), (1, 8), (2, 4), (2, 2), (4, 2), (1, 16), (2, 8), (4, 4), (4, 1), (8, 1), (1, 2), (16, 1),
+                       (8, 2), (2, 1)):
             row_tiles = -(-m // (rpw * wm))
             for target in (N_CU, 2 * N_CU, 4 * N_CU):
                 split = max(1, round(target / row_tiles))
