@@ -94,7 +94,10 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     const int nacc = rw * 4 * c.token_tiles;
     const int lut = decode == TUNA_DECODE_GEMM ? kLutBytes : 64;
     const size_t x_lds = (size_t)c.token_tiles * 16 * (size_t)c.x_chunk * 2;
-    const size_t red_lds = (size_t)2 * c.waves_k * c.waves_m * 1024;
+    // (eight planes = two buffers of four when the x chunk leaves that much room anyway)
+    const size_t plane_lds = (size_t)c.waves_k * c.waves_m * 1024;
+    const int planes_log2 = x_lds >= 8 * plane_lds ? 2 : 0;
+    const size_t red_lds = 2 * plane_lds << planes_log2;
     const size_t lds = (size_t)lut + (x_lds > red_lds ? x_lds : red_lds);
     if (lds > (size_t)kLdsLimit)
         return fail(TUNA_ERR_UNSUPPORTED, "config needs %zu bytes of LDS, the CU has %d", lds, kLdsLimit);
@@ -147,7 +150,7 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     a.xcd_swizzle = c.xcd_swizzle ? 1 : 0;
     a.lds_bytes = (int)lds;
     a.red_bytes = (int)red_lds;
-    a.planes_log2 = 0;
+    a.planes_log2 = planes_log2;
     a.tiles_total = row_tiles * c.split_k;
     return TUNA_OK;
 }

@@ -194,7 +194,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     // state of the tile being fetched / computed
     int row_tile = 0, ks = 0, sb = 0, nsteps = 0, n_it = 0, s_first = 0;
     uint32_t lb[RW], lb_last[RW];
-    float sc32[RW][4];
     u32x4 wq[U][RW];
     XStage xst;
 
@@ -211,9 +210,10 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
             reinterpret_cast<const u32x4 *>(base_ + (last_ ? lb_last[rw] : lb[rw])));          \
     }
 
-    // Request what tile `t` needs from HBM first: scales and the weight ring.  (The first x
-    // chunk comes from L2 and is requested at the start of the tile, behind these loads: it
-    // would cost 16 registers across the previous tile's epilogue.)
+    // Request what tile `t` streams from HBM first: the weight ring.  (The row scales and the
+    // first x chunk are small and mostly L2 hits; they are requested at the start of the tile,
+    // behind these loads: prefetched here they would cost 20 registers across the previous
+    // tile's epilogue.)
 #define TUNA_TILE_FETCH(t)                                                                      \
     {                                                                                          \
         row_tile = (t) / a.split_k;                                                            \
@@ -225,11 +225,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
         s_first = sb + wk;                                                                     \
         _Pragma("unroll") for (int rw = 0; rw < RW; ++rw)                                      \
         {                                                                                      \
-            _Pragma("unroll") for (int j = 0; j < 4; ++j)                                      \
-            {                                                                                  \
-                const int row_ = row0_ + rw * kRowsPerLoad + i16 * 4 + j;                      \
-                sc32[rw][j] = a.absmax[min(row_, a.m - 1)]; /* rows past m are never stored */ \
-            }                                                                                  \
             const int mb_ = min(((row0_ + rw * kRowsPerLoad) >> 3) + (i16 >> 1), mb_last);     \
             const uint32_t rowb_ = (uint32_t)mb_ * (uint32_t)kb_total * 32u + (uint32_t)(i16 & 1) * 16u; \
             lb[rw] = rowb_ + (uint32_t)g * 32u;                                                \
@@ -297,16 +292,27 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     const int wstep = a.waves_k * (1024 * TT);   // LDS bytes between this wave's consecutive steps
 
     for (; t < a.tiles_total; t += n_wg) {
-        // ---- this tile's scales (fp16 like the reference's staging, kernel.cu:2770) -------
-        f16x2 sc16[RW][4];
+        // ---- this tile's scales (fp16 like the reference's staging, kernel.cu:2770) and the
+        //      first x chunk: both requested now, behind the ring loads already in flight
         float sc32c[RW][4];
+        {
+            const int row0_ = row_tile * rows_wg + wm * (RW * kRowsPerLoad);
+#pragma unroll
+            for (int rw = 0; rw < RW; ++rw)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int row_ = row0_ + rw * kRowsPerLoad + i16 * 4 + j;
+                    sc32c[rw][j] = a.absmax[min(row_, a.m - 1)];  // rows past m are never stored
+                }
+        }
+        x_stage_load<TT>(xst, xg, 0, nthreads, tid, x_pieces, tok0, sb * kStepK, a.n, a.k);
+        f16x2 sc16[RW][4];
 #pragma unroll
         for (int rw = 0; rw < RW; ++rw)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const f16 h = (f16)sc32[rw][j];
+                const f16 h = (f16)sc32c[rw][j];
                 sc16[rw][j] = f16x2{h, h};
-                sc32c[rw][j] = sc32[rw][j];
             }
         f32x4 acc[RW][4][TT];
 #pragma unroll
@@ -320,9 +326,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
         const int n_chunks = (nsteps + a.chunk_steps - 1) >> a.chunk_log2;
         int it = 0;  // this wave's next iteration (multiple of U)
 
-        // chunk 0 of x; the work area is free again once every wave has left the previous
-        // tile's epilogue
-        x_stage_load<TT>(xst, xg, 0, nthreads, tid, x_pieces, tok0, cur_sb * kStepK, a.n, a.k);
+        // the work area is free again once every wave has left the previous tile's epilogue
         __syncthreads();
         if (n_chunks > 0) x_stage_store<TT>(xst, work, 0, nthreads, tid, x_pieces, tok0, cur_sb * kStepK, a.n, a.k);
         __syncthreads();
@@ -375,10 +379,11 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
         // ---- next tile: get its loads going before this tile's reduction and store ---------
         if (t + n_wg < a.tiles_total) TUNA_TILE_FETCH(t + n_wg)
 
-        // ---- workgroup reduction and store, one accumulator plane per pass ------------------
+        // ---- workgroup reduction and store ---------------------------------------------------
         // A plane is one float4 per lane = 256 floats [lane][4].  The waves_k waves of a row
         // group put their copies of a plane side by side in LDS (two buffers alternate, so one
-        // barrier per plane) and thread (wk, lane) sums the floats f = (i*waves_k + wk)*64 + lane
+        // barrier per plane - or per four planes when the work area holds eight of them) and
+        // thread (wk, lane) sums the floats f = (i*waves_k + wk)*64 + lane
         // of it in wave order.  Float f = l*4 + v of the plane of MFMA j is token l%16 and
         // weight row 16*(l/16) + 4*v + j of the wave's 64: after the four planes j = 0..3 a
         // thread owns 4 consecutive output features of one token and stores them as 8 bytes.
@@ -428,18 +433,39 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 #pragma unroll
             for (int tt = 0; tt < TT; ++tt) {
                 float o[4][4];  // [i][j]
+                if (a.planes_log2 == 2) {
+                    // the work area holds all four planes of a row group at once: one barrier
+                    float *buf = redf + (size_t)((rw * TT + tt) % 2) * 4 * plane_floats;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    float *buf = redf + ((rw * TT + tt) * 4 + j) % 2 * plane_floats;
-                    reinterpret_cast<f32x4 *>(buf)[(size_t)(wm_e * a.waves_k + wk_e) * 64 + lane_e] = acc[rw][j][tt];
+                    for (int j = 0; j < 4; ++j)
+                        reinterpret_cast<f32x4 *>(buf + j * plane_floats)[(size_t)(wm_e * a.waves_k + wk_e) * 64 + lane_e] =
+                            acc[rw][j][tt];
                     __syncthreads();
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int f = ((i << a.wk_log2) + wk_e) * 64 + lane_e;
-                        float sum = 0.f;
-                        if (f < 256)
-                            for (int w = 0; w < a.waves_k; ++w) sum += buf[(size_t)(wm_e * a.waves_k + w) * 256 + f];
-                        o[i][j] = sum;
+                    for (int j = 0; j < 4; ++j)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int f = ((i << a.wk_log2) + wk_e) * 64 + lane_e;
+                            float sum = 0.f;
+                            if (f < 256)
+                                for (int w = 0; w < a.waves_k; ++w)
+                                    sum += buf[j * plane_floats + (size_t)(wm_e * a.waves_k + w) * 256 + f];
+                            o[i][j] = sum;
+                        }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        float *buf = redf + ((rw * TT + tt) * 4 + j) % 2 * plane_floats;
+                        reinterpret_cast<f32x4 *>(buf)[(size_t)(wm_e * a.waves_k + wk_e) * 64 + lane_e] = acc[rw][j][tt];
+                        __syncthreads();
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int f = ((i << a.wk_log2) + wk_e) * 64 + lane_e;
+                            float sum = 0.f;
+                            if (f < 256)
+                                for (int w = 0; w < a.waves_k; ++w) sum += buf[(size_t)(wm_e * a.waves_k + w) * 256 + f];
+                            o[i][j] = sum;
+                        }
                     }
                 }
 #pragma unroll

@@ -27,8 +27,8 @@ static const Variant kVariants[] = {
     V(1, 4, 1, G, 512, 2), V(1, 4, 2, G, 512, 2),
     V(1, 8, 1, G, 512, 2), V(1, 8, 2, G, 512, 2),
     V(2, 2, 1, G, 512, 2), V(2, 4, 1, G, 512, 2),
-    V(1, 2, 1, G, 512, 4),
-    V(1, 2, 1, G, 1024, 4),
+    V(1, 2, 1, G, 512, 4), V(1, 4, 1, G, 512, 4),
+    V(1, 2, 1, G, 1024, 4), V(1, 4, 1, G, 1024, 4),
     // dequant-rounding decode (correctness mode, not tuned)
     V(1, 2, 1, TUNA_DECODE_DEQUANT, 512, 2), V(1, 2, 2, TUNA_DECODE_DEQUANT, 512, 2),
     V(1, 2, 4, TUNA_DECODE_DEQUANT, 512, 2),

@@ -37,7 +37,7 @@ struct GemmArgs {
     int row_tiles;        // workgroups along m
     int xcd_swizzle;
     int lds_bytes;        // dynamic LDS size of the launch (last 16 bytes: arrival ticket)
-    int red_bytes;        // bytes of the reduction area in the LDS work area = offset of the fp16 output tile
+    int red_bytes;        // bytes of the reduction buffers in the LDS work area
     int planes_log2;      // log2(accumulator planes reduced per epilogue pass)
     int tiles_total;      // row_tiles * split_k: tiles walked by the persistent workgroups
 #ifdef TUNA_TRACE

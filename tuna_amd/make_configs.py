@@ -46,8 +46,8 @@ STEP_K = 32
 # for <= 8 waves with <= 128 VGPRs (two workgroups per CU) and for 16-wave workgroups;
 # must match kVariants in csrc/gemm_launch.hip
 VARIANTS_512 = {(1, 2, 1), (1, 2, 2), (1, 2, 4), (1, 4, 1), (1, 4, 2), (1, 8, 1), (1, 8, 2), (2, 2, 1), (2, 4, 1)}
-VARIANTS_512_2WG = {(1, 2, 1)}
-VARIANTS_1024 = {(1, 2, 1)}
+VARIANTS_512_2WG = {(1, 2, 1), (1, 4, 1)}
+VARIANTS_1024 = {(1, 2, 1), (1, 4, 1)}
 
 
 def _pow2(v: int) -> bool:
