@@ -61,7 +61,9 @@ typedef struct tuna_gemm_config {
     int32_t waves_k;       /* waves along k inside the workgroup (reduced in LDS)     */
     int32_t split_k;       /* workgroups along k (reduced through the workspace)      */
     int32_t prefetch;      /* 2, 4 or 8: k-steps of packed weights in flight per wave */
-    int32_t x_chunk;       /* k elements of x staged in LDS at a time (multiple of 32*waves_k*prefetch) */
+    int32_t x_chunk;       /* k elements of x staged in LDS at a time: a power of two, at least
+                              32*waves_k*prefetch, and x_chunk*token_tiles at most 2x the workgroup's
+                              threads (4x with prefetch 8)                            */
     int32_t token_tiles;   /* 1, 2 or 4: 16-token MFMA tiles per pass over the weights */
     int32_t xcd_swizzle;   /* 1: remap workgroup ids so neighbours share an XCD       */
 } tuna_gemm_config;

@@ -85,20 +85,27 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     const int rw = c.rows_per_wave / kRowsPerLoad;
     const int threads = c.waves_m * c.waves_k * 64;
     const int rows_wg = c.rows_per_wave * c.waves_m;
-    if (c.x_chunk * c.token_tiles > 2 * threads)  // a chunk of x is staged as at most 4 pieces of 16 bytes per thread
-        return fail(TUNA_ERR_UNSUPPORTED, "x_chunk=%d x token_tiles=%d exceeds 2 x threads=%d", c.x_chunk, c.token_tiles,
-                    2 * threads);
+    // a chunk of x is staged as at most 4 (prefetch 8: 8) pieces of 16 bytes per thread
+    const int x_cap = (c.prefetch == 8 ? 4 : 2) * threads;
+    if (c.x_chunk * c.token_tiles > x_cap)
+        return fail(TUNA_ERR_UNSUPPORTED, "x_chunk=%d x token_tiles=%d exceeds %d for %d threads and prefetch %d", c.x_chunk,
+                    c.token_tiles, x_cap, threads, c.prefetch);
 
     // LDS = decode table + work area; the work area holds the x chunk in the main loop and, in
     // the epilogue, two alternating buffers of one accumulator plane (1 KB) of every wave.
     const int nacc = rw * 4 * c.token_tiles;
     const int lut = decode == TUNA_DECODE_GEMM ? kLutBytes : 64;
     const size_t x_lds = (size_t)c.token_tiles * 16 * (size_t)c.x_chunk * 2;
-    // (eight planes = two buffers of four when the x chunk leaves that much room anyway)
+    // Two buffers of four planes (one barrier per 64-row group instead of four) are used when
+    // they cost no occupancy: the x chunk leaves that much room anyway, or the config cannot
+    // put two workgroups on a CU in the first place.
     const size_t plane_lds = (size_t)c.waves_k * c.waves_m * 1024;
-    const int planes_log2 = x_lds >= 8 * plane_lds ? 2 : 0;
+    const size_t lds_small = (size_t)lut + (x_lds > 2 * plane_lds ? x_lds : 2 * plane_lds);
+    const size_t lds_big = (size_t)lut + (x_lds > 8 * plane_lds ? x_lds : 8 * plane_lds);
+    const bool two_wgs_possible = threads <= 512 && 2 * lds_small <= (size_t)kLdsLimit;
+    const int planes_log2 = (lds_big <= (size_t)kLdsLimit && (lds_big == lds_small || !two_wgs_possible)) ? 2 : 0;
     const size_t red_lds = 2 * plane_lds << planes_log2;
-    const size_t lds = (size_t)lut + (x_lds > red_lds ? x_lds : red_lds);
+    const size_t lds = planes_log2 ? lds_big : lds_small;
     if (lds > (size_t)kLdsLimit)
         return fail(TUNA_ERR_UNSUPPORTED, "config needs %zu bytes of LDS, the CU has %d", lds, kLdsLimit);
 

@@ -107,22 +107,22 @@ __device__ __forceinline__ f16x8 decode_dword(uint32_t d, const unsigned char *l
     }
 }
 
-// x staging, global -> registers -> LDS, in batches of kXBatch 16-byte pieces per thread.
+// x staging, global -> registers -> LDS, XB 16-byte pieces per thread (4, or 8 for the deepest
+// prefetch ring, whose smallest chunk is twice as long).
 // Piece p of a chunk is token row (p % (16*TT)), 8-k slot (p / (16*TT)) and lives at LDS
 // byte 16*p.  All loads of a batch are issued before the first LDS write (addresses are
 // clamped so the loads are unconditional; invalid pieces are zeroed by a select).
-constexpr int kXBatch = 4;
-
+template <int XB>
 struct XStage {
-    u32x4 v[kXBatch];
+    u32x4 v[XB];
 };
 
-template <int TT>
-__device__ __forceinline__ void x_stage_load(XStage &st, const f16 *xg, int base, int nthreads, int tid, int pieces,
+template <int TT, int XB>
+__device__ __forceinline__ void x_stage_load(XStage<XB> &st, const f16 *xg, int base, int nthreads, int tid, int pieces,
                                              int tok0, int kbase, int n, int k)
 {
 #pragma unroll
-    for (int b = 0; b < kXBatch; ++b) {
+    for (int b = 0; b < XB; ++b) {
         const int p = min(base + b * nthreads + tid, pieces - 1);
         const int r = p & (16 * TT - 1);
         const int c8 = p / (16 * TT);
@@ -132,12 +132,12 @@ __device__ __forceinline__ void x_stage_load(XStage &st, const f16 *xg, int base
     }
 }
 
-template <int TT>
-__device__ __forceinline__ void x_stage_store(const XStage &st, unsigned char *xs, int base, int nthreads, int tid,
+template <int TT, int XB>
+__device__ __forceinline__ void x_stage_store(const XStage<XB> &st, unsigned char *xs, int base, int nthreads, int tid,
                                               int pieces, int tok0, int kbase, int n, int k)
 {
 #pragma unroll
-    for (int b = 0; b < kXBatch; ++b) {
+    for (int b = 0; b < XB; ++b) {
         const int p = base + b * nthreads + tid;
         if (p < pieces) {
             const int r = p & (16 * TT - 1);
@@ -195,7 +195,8 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     int row_tile = 0, ks = 0, sb = 0, nsteps = 0, n_it = 0, s_first = 0;
     uint32_t lb[RW], lb_last[RW];
     u32x4 wq[U][RW];
-    XStage xst;
+    constexpr int XB = U == 8 ? 8 : 4;
+    XStage<XB> xst;
 
     // Unconditional by design: a load whose step lies beyond this wave's share is clamped
     // to the last k-step and its data is never used.  Only loads that are always issued
@@ -233,29 +234,23 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
         _Pragma("unroll") for (int u = 0; u < U; ++u) TUNA_LOAD_STEP(u, u)                     \
     }
 
+    // The small operands of a tile: row scales and the first x chunk (mostly L2 hits).
+#define TUNA_TILE_SMALL_LOADS()                                                                 \
+    {                                                                                          \
+        const int row0_ = row_tile * rows_wg + wm * (RW * kRowsPerLoad);                       \
+        _Pragma("unroll") for (int rw = 0; rw < RW; ++rw) _Pragma("unroll") for (int j = 0; j < 4; ++j) \
+        {                                                                                      \
+            const int row_ = row0_ + rw * kRowsPerLoad + i16 * 4 + j;                          \
+            sc32c[rw][j] = a.absmax[min(row_, a.m - 1)]; /* rows past m are never stored */    \
+        }                                                                                      \
+        x_stage_load<TT, XB>(xst, xg, 0, nthreads, tid, x_pieces, tok0, sb * kStepK, a.n, a.k);    \
+    }
+
     int t = wg;
     const float code_lane = a.code[lane & 15];
     if (t < a.tiles_total) TUNA_TILE_FETCH(t)
     TUNA_MARK(1)
 
-    // ---- decode table, once per workgroup ------------------------------------------------
-    if constexpr (DEC == TUNA_DECODE_GEMM) {
-        // Lane l holds fp16(code[l % 16]) (kernel.cu:2800 rounds the codebook to fp16);
-        // entries are gathered across lanes, no memory traffic.
-        // piece p: 16 bytes of row (p >> 4); all 64 slots of a row hold the same half2
-        const int code_bits = (int)f16_bits((f16)code_lane);
-#pragma unroll 4
-        for (int p = tid; p < kLutBytes / 16; p += nthreads) {
-            const int e = p >> 4;
-            const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute((e >> 4) << 2, code_bits);
-            const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute((e & 15) << 2, code_bits);
-            const uint32_t v = hi | (lo << 16);
-            reinterpret_cast<u32x4 *>(lut)[p] = u32x4{v, v, v, v};
-        }
-    } else {
-        if (tid < 16) reinterpret_cast<float *>(lut)[tid] = code_lane;
-    }
-    TUNA_MARK(2)
 
 #ifndef TUNA_DWORD_GROUP
 #define TUNA_DWORD_GROUP 0
@@ -293,19 +288,30 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 
     for (; t < a.tiles_total; t += n_wg) {
         // ---- this tile's scales (fp16 like the reference's staging, kernel.cu:2770) and the
-        //      first x chunk: both requested now, behind the ring loads already in flight
+        //      first x chunk, requested behind the ring loads already in flight
         float sc32c[RW][4];
-        {
-            const int row0_ = row_tile * rows_wg + wm * (RW * kRowsPerLoad);
-#pragma unroll
-            for (int rw = 0; rw < RW; ++rw)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int row_ = row0_ + rw * kRowsPerLoad + i16 * 4 + j;
-                    sc32c[rw][j] = a.absmax[min(row_, a.m - 1)];  // rows past m are never stored
+        TUNA_TILE_SMALL_LOADS()
+        if (tile_iter == 0) {
+            // (placed here so that the first tile's loads are all in flight while it is built)
+            // ---- decode table, once per workgroup ------------------------------------------------
+            if constexpr (DEC == TUNA_DECODE_GEMM) {
+                // Lane l holds fp16(code[l % 16]) (kernel.cu:2800 rounds the codebook to fp16);
+                // entries are gathered across lanes, no memory traffic.
+                // piece p: 16 bytes of row (p >> 4); all 64 slots of a row hold the same half2
+                const int code_bits = (int)f16_bits((f16)code_lane);
+#pragma unroll 4
+                for (int p = tid; p < kLutBytes / 16; p += nthreads) {
+                    const int e = p >> 4;
+                    const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute((e >> 4) << 2, code_bits);
+                    const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute((e & 15) << 2, code_bits);
+                    const uint32_t v = hi | (lo << 16);
+                    reinterpret_cast<u32x4 *>(lut)[p] = u32x4{v, v, v, v};
                 }
+            } else {
+                if (tid < 16) reinterpret_cast<float *>(lut)[tid] = code_lane;
+            }
         }
-        x_stage_load<TT>(xst, xg, 0, nthreads, tid, x_pieces, tok0, sb * kStepK, a.n, a.k);
+        TUNA_MARK(2)
         f16x2 sc16[RW][4];
 #pragma unroll
         for (int rw = 0; rw < RW; ++rw)
@@ -328,7 +334,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 
         // the work area is free again once every wave has left the previous tile's epilogue
         __syncthreads();
-        if (n_chunks > 0) x_stage_store<TT>(xst, work, 0, nthreads, tid, x_pieces, tok0, cur_sb * kStepK, a.n, a.k);
+        if (n_chunks > 0) x_stage_store<TT, XB>(xst, work, 0, nthreads, tid, x_pieces, tok0, cur_sb * kStepK, a.n, a.k);
         __syncthreads();
         TUNA_MARK(3)
 
@@ -345,10 +351,10 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                 // that after the group exactly U*RW younger loads are in flight and the wait before
                 // the LDS write below is an exact vmcnt, not a drain of the weight ring.
                 const int kbase = (cur_sb + (c + 1) * a.chunk_steps) * kStepK;
-                x_stage_load<TT>(xst, xg, 0, nthreads, tid, x_pieces, tok0, kbase, a.n, a.k);
+                x_stage_load<TT, XB>(xst, xg, 0, nthreads, tid, x_pieces, tok0, kbase, a.n, a.k);
                 TUNA_GROUP()
                 __syncthreads();  // every wave is done reading chunk c
-                x_stage_store<TT>(xst, work, 0, nthreads, tid, x_pieces, tok0, kbase, a.n, a.k);
+                x_stage_store<TT, XB>(xst, work, 0, nthreads, tid, x_pieces, tok0, kbase, a.n, a.k);
                 __syncthreads();
             } else {
                 const int it_end = min(it_chunk0 + ipc, n_it);
@@ -540,6 +546,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 #undef TUNA_GROUP
 #undef TUNA_CONSUME
 #undef TUNA_TILE_FETCH
+#undef TUNA_TILE_SMALL_LOADS
 #undef TUNA_LOAD_STEP
 #undef TUNA_MARK
 }

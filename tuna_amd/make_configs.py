@@ -93,17 +93,24 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
     threads = 64 * wm * wk
     if key not in (VARIANTS_512 if threads <= 512 else VARIANTS_1024):
         raise ValueError(f"no kernel variant {key} for {threads} threads")
-    if c["x_chunk"] * c["token_tiles"] > 2 * threads:
-        raise ValueError("x_chunk * token_tiles exceeds 2 * threads (x staging is at most 4 pieces per thread)")
+    if c["x_chunk"] * c["token_tiles"] > (4 if c["prefetch"] == 8 else 2) * threads:
+        raise ValueError("x_chunk * token_tiles too large for the x staging (4 pieces per thread, 8 with prefetch 8)")
     if lds_bytes(c) > LDS_LIMIT:
         raise ValueError(f"needs {lds_bytes(c)} bytes of LDS (limit {LDS_LIMIT})")
 
 
 def lds_bytes(c: dict) -> int:
-    """Dynamic LDS of a launch: decode table + max(x chunk, two reduction buffers of one plane per wave)."""
+    """Dynamic LDS of a launch: decode table + max(x chunk, reduction buffers).
+
+    The reduction buffers are 2 x 1 plane (1 KB) per wave, or 2 x 4 planes when that costs no
+    occupancy (mirrors plan_gemm in csrc/api.cpp)."""
+    threads = 64 * c["waves_k"] * c["waves_m"]
     x = c["token_tiles"] * 16 * c["x_chunk"] * 2
-    red = 2 * c["waves_k"] * c["waves_m"] * 1024
-    return LUT_BYTES + max(x, red)
+    plane = c["waves_k"] * c["waves_m"] * 1024
+    small = LUT_BYTES + max(x, 2 * plane)
+    big = LUT_BYTES + max(x, 8 * plane)
+    two_wgs = threads <= 512 and 2 * small <= LDS_LIMIT
+    return big if big <= LDS_LIMIT and (big == small or not two_wgs) else small
 
 
 def generate(param_map: dict) -> str:

@@ -59,7 +59,7 @@ def repair(c: dict, m: int, n_key: int, k: int):
     c["split_k"] = max(1, min(int(c["split_k"]), steps))
     sps = -(-steps // c["split_k"])
     # x chunk: a power of two in [unit, 2*threads/token_tiles], no larger than the split needs
-    hi_chunk = _pow2_floor(max(unit, 2 * threads // c["token_tiles"]))
+    hi_chunk = _pow2_floor(max(unit, (4 if c["prefetch"] == 8 else 2) * threads // c["token_tiles"]))
     want = max(unit, min(_pow2_floor(max(int(c.get("x_chunk", 1024)), 1)), hi_chunk))
     while want // 2 >= unit and want // 2 >= sps * 32:
         want //= 2
