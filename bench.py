@@ -26,6 +26,12 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+# Kernel arguments placed in device memory by the HIP runtime instead of host memory: the
+# command processor then reads them locally, which takes about 1 us off every launch of a
+# 10 us kernel.  A runtime setting of the process (read when HIP initialises), recommended
+# for serving processes; the caller's own value wins.
+os.environ.setdefault("HIP_FORCE_DEV_KERNARG", "1")
+
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 METRIC = "us/GEMM + HBM GB/s (frac of ~8 TB/s) at M=16, Mistral/Llama-70B shapes"
 HEADLINE = "mistral_qkv"
@@ -121,6 +127,9 @@ def main():
     ap.add_argument("--workload", default=HEADLINE, help="shape name timed as the headline (profiling runs)")
     ap.add_argument("--tokens", type=int, default=TOKENS, help="token count of the headline workload")
     ap.add_argument("--launch", choices=("both", "stream", "graph"), default="both")
+    ap.add_argument("--copy-yardstick", type=int, default=0, metavar="MIB",
+                    help="also launch the plain copy kernel over MIB mebibytes (counter runs: the known-traffic "
+                         "launch the HBM counters of the GEMM kernel are scaled by)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
@@ -185,6 +194,15 @@ def main():
         "headline_stream_launch": res_stream,
         "headline_graph_launch": res_graph,
     }
+
+    if args.copy_yardstick > 0:
+        nb = args.copy_yardstick << 20
+        src = torch.full((nb,), 7, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        ms = ops.time_copy(src, dst, warmup=2, iters=10)
+        line["copy_yardstick"] = {"bytes_read": nb, "bytes_written": nb, "us": round(ms * 100.0, 2),
+                                  "gbs_read_plus_write": round(2 * nb / (ms * 1e-4) / 1e9, 1)}
+        del src, dst
 
     if not args.no_shapes:
         shapes = {}
