@@ -57,15 +57,21 @@ enum { TUNA_DECODE_GEMM = 1, TUNA_DECODE_DEQUANT = 2 };
  * rows_per_wave*waves_m rows and a 1/split_k share of k.                          */
 typedef struct tuna_gemm_config {
     int32_t rows_per_wave; /* 64, 128 or 256: 128-bit loads per lane per k-step x 64 */
-    int32_t waves_m;       /* waves along the weight rows                             */
-    int32_t waves_k;       /* waves along k inside the workgroup (reduced in LDS)     */
-    int32_t split_k;       /* workgroups along k (reduced through the workspace)      */
+    int32_t waves_m;       /* waves along the weight rows (any count; waves_m*waves_k <= 16) */
+    int32_t waves_k;       /* waves along k inside the workgroup, a power of two (reduced in LDS) */
+    int32_t split_k;       /* workgroups along k (reduced through the workspace); 0 = balanced:
+                              the k ranges of all row tiles, laid end to end, are divided
+                              evenly over the workgroups the device holds at once      */
     int32_t prefetch;      /* 2, 4 or 8: k-steps of packed weights in flight per wave */
     int32_t x_chunk;       /* k elements of x staged in LDS at a time: a power of two, at least
                               32*waves_k*prefetch, and x_chunk*token_tiles at most 2x the workgroup's
                               threads (4x with prefetch 8)                            */
     int32_t token_tiles;   /* 1, 2 or 4: 16-token MFMA tiles per pass over the weights */
     int32_t xcd_swizzle;   /* 1: remap workgroup ids so neighbours share an XCD       */
+    int32_t k_stagger;     /* row tile r starts r*k_stagger k-steps into its k range and wraps
+                              around (0: every row tile starts at the front).  When k*4 bytes,
+                              the distance between block rows, is a large power of two, tiles
+                              walking in lockstep keep hitting the same memory channels  */
 } tuna_gemm_config;
 
 int tuna_version(void);
@@ -108,6 +114,19 @@ int tuna_validate_config(int m, int n, int k, const tuna_gemm_config *cfg);
 /* Dynamic LDS bytes and workspace bytes a launch of `cfg` needs. */
 int tuna_config_footprint(int m, int n, int k, const tuna_gemm_config *cfg,
                           size_t *lds_bytes, size_t *workspace_bytes);
+/* How a launch of `cfg` divides the work (host only, no device needed): the segments
+ * workgroup `workgroup` of `n_workgroups` walks (0 = as many as the launch would start on
+ * a 256-CU device), four ints each: row tile, first k-step (32 k each), k-steps, and the
+ * slot of its partial sums (-1: the segment is a whole row tile and writes the output
+ * itself).  At most max_segments are written; *n_segments is the full count.  No counterpart
+ * in the reference, whose grid is one threadblock per tile (kernel.cu:2962-3007). */
+int tuna_config_segments(int m, int n, int k, const tuna_gemm_config *cfg, int n_workgroups,
+                         int workgroup, int *segments, int max_segments, int *n_segments);
+/* Balanced split only (split_k == 0): the workgroups whose partial sums make up row tile
+ * `row_tile`, first_workgroup .. first_workgroup + count - 1 in k order, and the slot the
+ * first of them used (all later ones use slot 0).  With a fixed split: -1, split_k, 0. */
+int tuna_config_contributors(int m, int n, int k, const tuna_gemm_config *cfg, int n_workgroups,
+                             int row_tile, int *first_workgroup, int *count, int *first_slot);
 /* Enumerate the built-in table: entry i -> its shape key and config. */
 int tuna_config_table_size(void);
 int tuna_config_table_entry(int i, int *m, int *n_lo, int *n_hi, int *k, tuna_gemm_config *cfg);

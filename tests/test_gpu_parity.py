@@ -149,6 +149,27 @@ CONFIGS = [
     dict(rows_per_wave=128, waves_m=4, waves_k=1, prefetch=2, x_chunk=64),
     dict(token_tiles=2, waves_m=4, waves_k=1, prefetch=4, x_chunk=128),
     dict(waves_m=2, waves_k=2, prefetch=2, x_chunk=128, split_k=1),                 # many x chunks per workgroup
+    # workgroups of 3, 5, 7 ... waves along the rows (row tiles that are not a power of two)
+    dict(waves_m=7, waves_k=1, prefetch=2, x_chunk=64),
+    dict(waves_m=3, waves_k=4, prefetch=2, x_chunk=256, split_k=2),
+    dict(waves_m=7, waves_k=2, prefetch=2, x_chunk=256, xcd_swizzle=1),
+    dict(waves_m=5, waves_k=2, prefetch=4, x_chunk=256, split_k=0),
+    # staggered start of the k walk per row tile (wraps around inside the segment)
+    dict(k_stagger=1),
+    dict(k_stagger=3, split_k=2, prefetch=2, x_chunk=256),
+    dict(k_stagger=5, waves_m=1, waves_k=8, prefetch=2, x_chunk=512, split_k=3, xcd_swizzle=1),
+    dict(k_stagger=1, waves_m=8, waves_k=1, prefetch=2, x_chunk=64),
+    dict(k_stagger=7, waves_m=7, waves_k=2, prefetch=4, x_chunk=256),
+    dict(k_stagger=2, token_tiles=2, waves_m=4, waves_k=1, prefetch=4, x_chunk=128),
+    dict(k_stagger=9, split_k=0, waves_m=2, waves_k=4, prefetch=2, x_chunk=256),
+    dict(k_stagger=4096, rows_per_wave=128, waves_m=2, waves_k=2, prefetch=2, x_chunk=128),
+    # balanced split (split_k = 0): k ranges of all row tiles divided evenly over the workgroups
+    dict(split_k=0),
+    dict(split_k=0, waves_m=1, waves_k=8, prefetch=2, x_chunk=512, xcd_swizzle=1),
+    dict(split_k=0, waves_m=8, waves_k=1, prefetch=2, x_chunk=64, xcd_swizzle=1),
+    dict(split_k=0, waves_m=4, waves_k=4, prefetch=2, x_chunk=512),                 # 16 waves
+    dict(split_k=0, token_tiles=2, waves_m=2, waves_k=4, prefetch=4, x_chunk=512),
+    dict(split_k=0, rows_per_wave=128, waves_m=2, waves_k=2, prefetch=2, x_chunk=128),
 ]
 
 
@@ -165,20 +186,41 @@ def test_gemm_every_config_family(ci, m, n, k):
     assert e <= REL_TOL, e
 
 
+@pytest.mark.parametrize("ckw", [
+    dict(split_k=0, waves_m=1, waves_k=2, prefetch=2, x_chunk=128),     # 2400 units: ~4.7 per workgroup
+    dict(split_k=0, waves_m=2, waves_k=1, prefetch=2, x_chunk=64, xcd_swizzle=1),
+    dict(split_k=0, waves_m=1, waves_k=4, prefetch=4, x_chunk=512),     # one unit per row tile: whole tiles only
+])
+def test_balanced_split_walks_whole_and_partial_row_tiles(ckw):
+    """More row tiles than workgroups: a workgroup's share is a tail of one row tile, whole
+    row tiles and a head of another.  Full comparison with the oracle, and the same bits on
+    a second launch (workspace slots and arrival counters are left reusable)."""
+    m, n, k = 38400, 16, 512
+    c = cfg(**ckw)
+    print(f"balanced {c.to_dict()} m={m} n={n} k={k}", flush=True)
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=21)
+    got = run_gemm(q, x, code, absmax, m, n, k, config=c, prefill=float("nan"))
+    ref = O.gemm_f64(q, x, code, absmax, m, n, k, mode=O.D1)
+    e = rel_err(f16_bits_to_f64(got), ref)
+    assert e <= REL_TOL, e
+    again = run_gemm(q, x, code, absmax, m, n, k, config=c, prefill=float("nan"))
+    assert np.array_equal(got, again)
+
+
 def test_split_k_is_deterministic_and_order_independent():
     """Same launch twice: identical bits (no atomics).  Different split counts: only fp32
     re-association noise, i.e. at most 1 fp16 ulp apart after the final rounding."""
     m, n, k = 2048, 16, 4096
     q, x, code, absmax = make_inputs_np(m, n, k, seed=11)
     outs = {}
-    for s in (1, 2, 4, 8, 16):
+    for s in (1, 2, 4, 8, 16, 0):
         c = cfg(split_k=s, x_chunk=512)
         a = run_gemm(q, x, code, absmax, m, n, k, config=c)
         for _ in range(3):
             b = run_gemm(q, x, code, absmax, m, n, k, config=c, prefill=float("nan"))
             assert np.array_equal(a, b), s
         outs[s] = a
-    for s in (2, 4, 8, 16):
+    for s in (2, 4, 8, 16, 0):
         assert ulp_diff_f16(outs[1], outs[s]) <= 1, s
 
 

@@ -88,8 +88,8 @@ def test_invalid_configs_are_rejected_by_both_validators():
                 xcd_swizzle=0)
     ops.validate_config(4096, 16, 4096, ops.GemmConfig.from_dict(good))
     mc.validate(4096, 16, 4096, good)
-    bad = [dict(rows_per_wave=96), dict(prefetch=3), dict(token_tiles=3), dict(waves_m=3), dict(waves_k=32),
-           dict(waves_m=8, waves_k=4), dict(split_k=0), dict(split_k=129), dict(x_chunk=500), dict(x_chunk=256),
+    bad = [dict(rows_per_wave=96), dict(prefetch=3), dict(token_tiles=3), dict(waves_m=0), dict(waves_k=3), dict(waves_k=32),
+           dict(waves_m=8, waves_k=4), dict(split_k=-1), dict(split_k=129), dict(x_chunk=500), dict(x_chunk=256),
            dict(x_chunk=1 << 16), dict(rows_per_wave=256, prefetch=8)]
     for delta in bad:
         c = dict(good, **delta)
@@ -108,10 +108,10 @@ def test_generator_output_and_its_refusal_of_inconsistent_entries(tmp_path):
     pm = {"4096_16_4096": dict(rows_per_wave=64, waves_m=1, waves_k=8, split_k=4, prefetch=2, x_chunk=1024,
                                token_tiles=1, xcd_swizzle=1, us=9.9),
           "4096_1_4096": dict(rows_per_wave=64, waves_m=1, waves_k=8, split_k=4, prefetch=2, x_chunk=1024,
-                              token_tiles=1, xcd_swizzle=0)}
+                              token_tiles=1, xcd_swizzle=0, k_stagger=3)}
     text = mc.generate(pm)
-    assert "{4096, 16, 31, 4096, {64, 1, 8, 4, 2, 1024, 1, 1}}" in text
-    assert "{4096, 1, 15, 4096, {64, 1, 8, 4, 2, 1024, 1, 0}}" in text
+    assert "{4096, 16, 31, 4096, {64, 1, 8, 4, 2, 1024, 1, 1, 0}}" in text     # k_stagger defaults to 0
+    assert "{4096, 1, 15, 4096, {64, 1, 8, 4, 2, 1024, 1, 0, 3}}" in text
     assert "kConfigTableSize = 2" in text
     # the checked-in table is what the generator produces from the checked-in json
     with open(os.path.join(ROOT, "tuna_amd", "configs", "param_map.json")) as f:
@@ -224,3 +224,102 @@ def test_synthetic_inputs_are_deterministic_and_in_range():
     assert (absmax >= 0.004999).all() and (absmax <= 0.02001).all()
     assert np.array_equal(absmax, absmax.astype(np.float16).astype(np.float32))  # fp16-representable scales
     assert len(SHAPES) == 10 and SHAPES["mistral_qkv"] == (6144, 4096)
+
+
+# ---------------------------------------------------------------------------------------
+# balanced split (split_k = 0): the partition arithmetic the kernel and the host share
+# ---------------------------------------------------------------------------------------
+def _balanced_cfg(**kw):
+    from tuna_amd import ops
+
+    base = dict(rows_per_wave=64, waves_m=1, waves_k=8, split_k=0, prefetch=2, x_chunk=1024, token_tiles=1, xcd_swizzle=1)
+    base.update(kw)
+    return ops.GemmConfig.from_dict(base)
+
+
+@pytest.mark.parametrize("m,k,cfgkw,nwgs", [
+    (6144, 4096, {}, (256, 512, 96, 7, 1)),
+    (4096, 4096, dict(waves_k=4, prefetch=4, x_chunk=512), (512, 100)),
+    (57344, 8192, dict(waves_m=4, waves_k=4, x_chunk=1024), (256, 255, 33)),
+    (229376, 4096, dict(waves_m=8, waves_k=1, x_chunk=512), (512, 256)),
+    (4096, 14336, dict(waves_k=8, prefetch=4), (256, 300)),
+    (72, 200, dict(waves_k=2, x_chunk=128), (256, 3, 1)),     # ragged rows and k
+    (8192, 28672, dict(waves_m=2, waves_k=8, x_chunk=1024), (256, 511)),
+])
+def test_balanced_split_partitions_every_k_step_once(m, k, cfgkw, nwgs):
+    """Every (row tile, k-step) is covered by exactly one segment; a row tile's partial
+    segments are consecutive workgroups in k order with the slots the finishing workgroup
+    assumes; whole row tiles have a single owner.  Checked through the C ABI, whose
+    arithmetic is the inline code the kernel compiles too."""
+    from tuna_amd import ops
+
+    cfg = _balanced_cfg(**cfgkw)
+    steps = -(-k // 32)
+    rows_wg = cfg.rows_per_wave * cfg.waves_m
+    row_tiles = -(-m // rows_wg)
+    for nw in nwgs:
+        segs = {}
+        n_launch = None
+        # the library clamps the workgroup count to what the launch would start
+        w = 0
+        while True:
+            try:
+                sg = ops.config_segments(m, 16, k, cfg, nw, w)
+            except ops.TunaError:
+                break
+            segs[w] = sg
+            w += 1
+        n_launch = w
+        assert 1 <= n_launch <= nw
+        cover = np.zeros((row_tiles, steps), dtype=np.int32)
+        per_tile = {}
+        for w, sg in segs.items():
+            partial_slots = []
+            for (rt, sb, ns, part) in sg:
+                assert 0 <= rt < row_tiles and ns > 0 and sb >= 0 and sb + ns <= steps
+                cover[rt, sb:sb + ns] += 1
+                per_tile.setdefault(rt, []).append((sb, w, part, ns))
+                if part >= 0:
+                    partial_slots.append(part)
+                else:
+                    assert sb == 0 and ns == steps
+            assert len(partial_slots) == len(set(partial_slots)) <= 2     # a workgroup owns two slots
+        assert (cover == 1).all()
+        # balance: workgroups differ by at most one unit (+ a ragged last unit)
+        unit = cfg.waves_k * cfg.prefetch
+        loads = [sum(s[2] for s in sg) for sg in segs.values()]
+        assert max(loads) - min(loads) <= 2 * unit
+        for rt, lst in per_tile.items():
+            lst.sort()
+            first_wg, count, first_slot = ops.config_contributors(m, 16, k, cfg, nw, rt)
+            if len(lst) == 1:
+                assert lst[0][2] == -1
+                continue
+            assert count == len(lst)
+            assert [w for _, w, _, _ in lst] == list(range(first_wg, first_wg + count))
+            assert lst[0][2] == first_slot
+            assert all(part == 0 for _, _, part, _ in lst[1:])
+
+
+def test_fixed_split_segments_match_the_grid():
+    from tuna_amd import ops
+
+    cfg = _balanced_cfg(split_k=4)
+    segs = [ops.config_segments(6144, 16, 4096, cfg, 0, w) for w in range(8)]
+    assert segs[0][0] == (0, 0, 32, 0) and segs[5][0] == (1, 32, 32, 1)
+    assert ops.config_contributors(6144, 16, 4096, cfg, 0, 3) == (-1, 4, 0)
+
+
+def test_gpu_parity_config_families_are_valid_configs():
+    """The config families the GPU parity tests launch are accepted by the host validator for
+    both of their shapes (a rejected config would fail the GPU test for the wrong reason)."""
+    import importlib.util
+
+    from tuna_amd import ops
+
+    spec = importlib.util.spec_from_file_location("gpu_parity_cases", os.path.join(ROOT, "tests", "test_gpu_parity.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    for kw in mod.CONFIGS:
+        for shape in ((1024, 16, 2048), (520, 37, 1096)):
+            ops.validate_config(*shape, mod.cfg(**kw))

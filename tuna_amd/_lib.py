@@ -35,6 +35,7 @@ class GemmConfig(ctypes.Structure):
         ("x_chunk", ctypes.c_int32),
         ("token_tiles", ctypes.c_int32),
         ("xcd_swizzle", ctypes.c_int32),
+        ("k_stagger", ctypes.c_int32),
     ]
 
     FIELDS = tuple(f for f, _ in _fields_)
@@ -44,7 +45,7 @@ class GemmConfig(ctypes.Structure):
 
     @classmethod
     def from_dict(cls, d):
-        return cls(**{f: int(d[f]) for f in cls.FIELDS})
+        return cls(**{f: int(d.get(f, 0) if f == "k_stagger" else d[f]) for f in cls.FIELDS})
 
 
 # name -> (restype, argtypes); also the list of symbols the header declares
@@ -64,6 +65,8 @@ SIGNATURES = {
     "tuna_select_config": (_i, [_i, _i, _i, _cfgp, _ip]),
     "tuna_validate_config": (_i, [_i, _i, _i, _cfgp]),
     "tuna_config_footprint": (_i, [_i, _i, _i, _cfgp, ctypes.POINTER(_sz), ctypes.POINTER(_sz)]),
+    "tuna_config_segments": (_i, [_i, _i, _i, _cfgp, _i, _i, _ip, _i, _ip]),
+    "tuna_config_contributors": (_i, [_i, _i, _i, _cfgp, _i, _i, _ip, _ip, _ip]),
     "tuna_config_table_size": (_i, []),
     "tuna_config_table_entry": (_i, [_i, _ip, _ip, _ip, _ip, _cfgp]),
     "tuna_time_matmul": (_i, [_vpp, _vpp, _i, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _i, _i, _i, _vp, _fp]),

@@ -36,7 +36,6 @@ static int hip_fail(hipError_t e, const char *what)
 }
 
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
-static inline int round_up(int a, int b) { return ceil_div(a, b) * b; }
 
 // ---------------------------------------------------------------------------------------
 // config validation and launch planning
@@ -73,15 +72,16 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
         return fail(TUNA_ERR_UNSUPPORTED, "prefetch=%d (2, 4 or 8)", c.prefetch);
     if (c.token_tiles != 1 && c.token_tiles != 2 && c.token_tiles != 4)
         return fail(TUNA_ERR_UNSUPPORTED, "token_tiles=%d (1, 2 or 4)", c.token_tiles);
-    if (!is_pow2(c.waves_m) || !is_pow2(c.waves_k) || c.waves_m * c.waves_k * 64 > kMaxThreads)
-        return fail(TUNA_ERR_UNSUPPORTED, "waves_m=%d and waves_k=%d must be powers of two with at most 16 waves", c.waves_m,
-                    c.waves_k);
+    if (c.waves_m < 1 || !is_pow2(c.waves_k) || c.waves_m * c.waves_k * 64 > kMaxThreads)
+        return fail(TUNA_ERR_UNSUPPORTED, "waves_m=%d must be at least 1 and waves_k=%d a power of two, with at most 16 waves",
+                    c.waves_m, c.waves_k);
     const int steps_total = ceil_div(k, kStepK);
-    if (c.split_k < 1 || c.split_k > steps_total)
-        return fail(TUNA_ERR_UNSUPPORTED, "split_k=%d must be in 1..%d for k=%d", c.split_k, steps_total, k);
+    if (c.split_k < 0 || c.split_k > steps_total)
+        return fail(TUNA_ERR_UNSUPPORTED, "split_k=%d must be in 0..%d for k=%d (0 = balanced)", c.split_k, steps_total, k);
     if (!is_pow2(c.x_chunk) || c.x_chunk < kStepK * c.waves_k * c.prefetch)
         return fail(TUNA_ERR_UNSUPPORTED, "x_chunk=%d must be a power of two >= 32*waves_k*prefetch=%d", c.x_chunk,
                     kStepK * c.waves_k * c.prefetch);
+    if (c.k_stagger < 0 || c.k_stagger > 4096) return fail(TUNA_ERR_UNSUPPORTED, "k_stagger=%d must be in 0..4096", c.k_stagger);
     const int rw = c.rows_per_wave / kRowsPerLoad;
     const int threads = c.waves_m * c.waves_k * 64;
     const int rows_wg = c.rows_per_wave * c.waves_m;
@@ -127,6 +127,24 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     if (tok_chunks > 65535) return fail(TUNA_ERR_UNSUPPORTED, "n=%d needs %d token chunks (max 65535)", n, tok_chunks);
     if ((long long)row_tiles * c.split_k > 0x7fffffffLL) return fail(TUNA_ERR_UNSUPPORTED, "grid too large");
 
+    // Balanced split (split_k == 0): the k ranges of all row tiles, cut into units of one ring
+    // turn of the workgroup (coarser if the unit count would overflow the kernel's 32-bit
+    // arithmetic), are divided evenly over the workgroups the device holds at once.
+    const bool balanced = c.split_k == 0;
+    const int slots = kMaxCus * wgs_per_cu;
+    int unit_log2 = log2i(c.waves_k) + log2i(c.prefetch);
+    int units_per_tile = 0;
+    long long units_total = 0;
+    if (balanced) {
+        for (;; ++unit_log2) {
+            units_per_tile = ceil_div(steps_total, 1 << unit_log2);
+            units_total = (long long)row_tiles * units_per_tile;
+            if ((units_total + 1) * slots < 0x7fffffffLL) break;
+            if (units_per_tile == 1) return fail(TUNA_ERR_UNSUPPORTED, "too many row tiles (%d) for a balanced split", row_tiles);
+        }
+    }
+    const unsigned grid_x = balanced ? (unsigned)(units_total < slots ? units_total : slots) : (unsigned)(row_tiles * c.split_k);
+
     GemmPlan &p = *plan;
     memset(&p, 0, sizeof(p));
     p.rw = rw;
@@ -137,24 +155,30 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     p.wgs_per_cu = wgs_per_cu;
     p.threads = threads;
     p.lds_bytes = lds;
-    p.grid = dim3((unsigned)(row_tiles * c.split_k), (unsigned)tok_chunks, 1);
-    p.ws_bytes = c.split_k > 1 ? (size_t)tok_chunks * row_tiles * c.split_k * c.waves_m * nacc * 1024 : 0;
-    p.n_counters = c.split_k > 1 ? (size_t)tok_chunks * row_tiles : 0;
+    p.grid = dim3(grid_x, (unsigned)tok_chunks, 1);
+    // partial sums: one segment is waves_m * nacc planes of 1 KB; two slots per workgroup when balanced
+    if (balanced) p.ws_bytes = (size_t)tok_chunks * grid_x * 2 * c.waves_m * nacc * 1024;
+    else p.ws_bytes = c.split_k > 1 ? (size_t)tok_chunks * row_tiles * c.split_k * c.waves_m * nacc * 1024 : 0;
+    p.n_counters = c.split_k != 1 ? (size_t)tok_chunks * row_tiles : 0;
     GemmArgs &a = p.args;
     a.m = m;
     a.n = n;
     a.k = k;
     a.waves_m = c.waves_m;
     a.waves_k = c.waves_k;
-    a.wm_log2 = log2i(c.waves_m);
     a.wk_log2 = log2i(c.waves_k);
     a.split_k = c.split_k;
     a.steps_total = steps_total;
-    a.steps_per_split = ceil_div(steps_total, c.split_k);
+    a.steps_per_split = balanced ? steps_total : ceil_div(steps_total, c.split_k);
+    a.balanced = balanced ? 1 : 0;
+    a.unit_log2 = unit_log2;
+    a.units_per_tile = units_per_tile;
+    a.units_total = (int)units_total;
     a.chunk_steps = c.x_chunk / kStepK;
     a.chunk_log2 = log2i(a.chunk_steps);
     a.row_tiles = row_tiles;
     a.xcd_swizzle = c.xcd_swizzle ? 1 : 0;
+    a.k_stagger = c.k_stagger;
     a.lds_bytes = (int)lds;
     a.red_bytes = (int)red_lds;
     a.planes_log2 = planes_log2;
@@ -173,6 +197,7 @@ static tuna_gemm_config derive_config(int m, int n, int k)
     c.waves_k = 4;
     c.prefetch = c.token_tiles == 4 ? 2 : 4;
     c.xcd_swizzle = 0;
+    c.k_stagger = 1;
     const int steps = ceil_div(k, kStepK);
     const int row_tiles = ceil_div(m, c.rows_per_wave * c.waves_m);
     const int group = c.waves_k * c.prefetch;  // k-steps one workgroup consumes per ring turn
@@ -475,6 +500,77 @@ TUNA_EXPORT int tuna_config_footprint(int m, int n, int k, const tuna_gemm_confi
     if (rc) return rc;
     if (lds_bytes) *lds_bytes = plan.lds_bytes;
     if (workspace_bytes) *workspace_bytes = plan.ws_bytes;
+    return TUNA_OK;
+}
+
+TUNA_EXPORT int tuna_config_segments(int m, int n, int k, const tuna_gemm_config *cfg, int n_workgroups, int workgroup,
+                                     int *segments, int max_segments, int *n_segments)
+{
+    if (!cfg || !n_segments) return fail(TUNA_ERR_INVALID_ARG, "cfg or n_segments is null");
+    GemmPlan plan;
+    int rc = plan_gemm(m, n, k, *cfg, TUNA_DECODE_GEMM, &plan);
+    if (rc) return rc;
+    const GemmArgs &a = plan.args;
+    int nw = n_workgroups > 0 ? n_workgroups : (int)plan.grid.x;
+    const int cap = kMaxCus * plan.wgs_per_cu;
+    if (nw > cap) nw = cap;
+    if (nw > (int)plan.grid.x) nw = (int)plan.grid.x;
+    if (workgroup < 0 || workgroup >= nw) return fail(TUNA_ERR_INVALID_ARG, "workgroup %d outside 0..%d", workgroup, nw - 1);
+    int count = 0;
+    auto emit = [&](int row_tile, int sb, int nsteps, int part) {
+        if (segments && count < max_segments) {
+            segments[4 * count + 0] = row_tile;
+            segments[4 * count + 1] = sb;
+            segments[4 * count + 2] = nsteps;
+            segments[4 * count + 3] = part;
+        }
+        ++count;
+    };
+    if (a.balanced) {
+        const int t_begin = balanced_begin((unsigned)workgroup, (unsigned)nw, (unsigned)a.units_total);
+        const int t_end = balanced_begin((unsigned)workgroup + 1u, (unsigned)nw, (unsigned)a.units_total);
+        for (int t = t_begin; t < t_end;) {
+            const Segment sg = balanced_segment(t, t_begin, t_end, a.units_per_tile, a.unit_log2, a.steps_total);
+            emit(sg.row_tile, sg.sb, sg.nsteps, sg.part);
+            t = sg.next;
+        }
+    } else {
+        for (int t = workgroup; t < a.tiles_total; t += nw) {
+            const int row_tile = t / a.split_k, ks = t - row_tile * a.split_k;
+            const int sb = ks * a.steps_per_split;
+            int nsteps = (a.steps_total < sb + a.steps_per_split ? a.steps_total : sb + a.steps_per_split) - sb;
+            if (nsteps < 0) nsteps = 0;
+            emit(row_tile, sb, nsteps, a.split_k == 1 ? -1 : ks);
+        }
+    }
+    *n_segments = count;
+    return TUNA_OK;
+}
+
+TUNA_EXPORT int tuna_config_contributors(int m, int n, int k, const tuna_gemm_config *cfg, int n_workgroups, int row_tile,
+                                         int *first_workgroup, int *count, int *first_slot)
+{
+    if (!cfg || !first_workgroup || !count || !first_slot) return fail(TUNA_ERR_INVALID_ARG, "null argument");
+    GemmPlan plan;
+    int rc = plan_gemm(m, n, k, *cfg, TUNA_DECODE_GEMM, &plan);
+    if (rc) return rc;
+    const GemmArgs &a = plan.args;
+    if (row_tile < 0 || row_tile >= a.row_tiles) return fail(TUNA_ERR_INVALID_ARG, "row_tile %d outside 0..%d", row_tile, a.row_tiles - 1);
+    if (!a.balanced) {
+        *first_workgroup = -1;
+        *count = a.split_k;
+        *first_slot = 0;
+        return TUNA_OK;
+    }
+    int nw = n_workgroups > 0 ? n_workgroups : (int)plan.grid.x;
+    const int cap = kMaxCus * plan.wgs_per_cu;
+    if (nw > cap) nw = cap;
+    if (nw > (int)plan.grid.x) nw = (int)plan.grid.x;
+    unsigned lo, cnt, slot;
+    balanced_contributors((unsigned)row_tile, (unsigned)a.units_per_tile, (unsigned)a.units_total, (unsigned)nw, &lo, &cnt, &slot);
+    *first_workgroup = (int)lo;
+    *count = (int)cnt;
+    *first_slot = (int)slot;
     return TUNA_OK;
 }
 

@@ -117,9 +117,21 @@ struct XStage {
     u32x4 v[XB];
 };
 
+// Where a segment's k range [hi_k - span_k, hi_k) starts: the walk begins rot_k elements into
+// it and wraps around (all in k elements, multiples of 32).
+struct KRot {
+    int rot_k, hi_k, span_k;
+};
+
+__device__ __forceinline__ int k_physical(int k_logical, const KRot &kr)
+{
+    const int kp = k_logical + kr.rot_k;
+    return kp >= kr.hi_k ? kp - kr.span_k : kp;
+}
+
 template <int TT, int XB>
 __device__ __forceinline__ void x_stage_load(XStage<XB> &st, const f16 *xg, int base, int nthreads, int tid, int pieces,
-                                             int tok0, int kbase, int n, int k)
+                                             int tok0, int kbase, int n, int k, const KRot &kr)
 {
 #pragma unroll
     for (int b = 0; b < XB; ++b) {
@@ -127,14 +139,14 @@ __device__ __forceinline__ void x_stage_load(XStage<XB> &st, const f16 *xg, int 
         const int r = p & (16 * TT - 1);
         const int c8 = p / (16 * TT);
         const int tok = min(tok0 + r, n - 1);
-        const int kk = min(kbase + c8 * 8, k - 8);
+        const int kk = min(k_physical(kbase + c8 * 8, kr), k - 8);
         st.v[b] = *reinterpret_cast<const u32x4 *>(xg + (size_t)tok * k + kk);
     }
 }
 
 template <int TT, int XB>
 __device__ __forceinline__ void x_stage_store(const XStage<XB> &st, unsigned char *xs, int base, int nthreads, int tid,
-                                              int pieces, int tok0, int kbase, int n, int k)
+                                              int pieces, int tok0, int kbase, int n, int k, const KRot &kr)
 {
 #pragma unroll
     for (int b = 0; b < XB; ++b) {
@@ -142,7 +154,8 @@ __device__ __forceinline__ void x_stage_store(const XStage<XB> &st, unsigned cha
         if (p < pieces) {
             const int r = p & (16 * TT - 1);
             const int c8 = p / (16 * TT);
-            const bool ok = (tok0 + r < n) && (kbase + c8 * 8 < k);
+            const int kl = kbase + c8 * 8;
+            const bool ok = (tok0 + r < n) && kl < kr.hi_k && k_physical(kl, kr) < k;
             *reinterpret_cast<u32x4 *>(xs + (size_t)p * 16) = ok ? st.v[b] : u32x4{0u, 0u, 0u, 0u};
         }
     }
@@ -191,20 +204,33 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     const int n_wg = gridDim.x;
     if (a.xcd_swizzle && (n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
 
+    // The walk.  Fixed split: tile t = (row tile, k split) for t = wg, wg + n_wg, ... below
+    // row_tiles * split_k.  Balanced split: the k range of every row tile is cut into units
+    // of 2^unit_log2 k-steps, all units of all row tiles form one sequence, workgroup w owns
+    // units [w*T/n_wg, (w+1)*T/n_wg) of it and walks them as segments that end at row tile
+    // boundaries.  `part` is the segment's slot among the partial sums of its row tile
+    // (-1: the segment is the whole row tile, its sums are final).
+    int t_begin = wg, t_end = a.tiles_total;
+    if (a.balanced) {
+        t_begin = balanced_begin((unsigned)wg, (unsigned)n_wg, (unsigned)a.units_total);
+        t_end = balanced_begin((unsigned)wg + 1u, (unsigned)n_wg, (unsigned)a.units_total);
+    }
     // state of the tile being fetched / computed
-    int row_tile = 0, ks = 0, sb = 0, nsteps = 0, n_it = 0, s_first = 0;
+    int row_tile = 0, part = -1, sb = 0, nsteps = 0, n_it = 0, s_first = 0, t_next = 0;
+    int seg_hi = 0, s_clamp = 0, rot = 0;
     uint32_t lb[RW], lb_last[RW];
     u32x4 wq[U][RW];
     constexpr int XB = U == 8 ? 8 : 4;
     XStage<XB> xst;
 
     // Unconditional by design: a load whose step lies beyond this wave's share is clamped
-    // to the last k-step and its data is never used.  Only loads that are always issued
+    // to the segment's last k-step and its data is never used.  Only loads that are always issued
     // let the compiler count outstanding loads exactly (s_waitcnt vmcnt(N > 0)).
     // address = q + [uniform: 128 bytes per k-step, in SGPRs] + [per lane: block row, half, g]
 #define TUNA_LOAD_STEP(u, it)                                                                  \
     {                                                                                          \
-        const int s_ = min(s_first + (it) * s_stride, a.steps_total - 1);                      \
+        int s_ = min(s_first + (it) * s_stride, s_clamp) + rot;                                \
+        if (s_ >= seg_hi) s_ -= nsteps;                                                        \
         const unsigned char *base_ = a.q + (size_t)s_ * 128;                                   \
         const bool last_ = s_ == a.steps_total - 1;                                            \
         _Pragma("unroll") for (int rw = 0; rw < RW; ++rw) wq[u][rw] = __builtin_nontemporal_load( \
@@ -217,13 +243,28 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     // tile's epilogue.)
 #define TUNA_TILE_FETCH(t)                                                                      \
     {                                                                                          \
-        row_tile = (t) / a.split_k;                                                            \
-        ks = (t) - row_tile * a.split_k;                                                       \
+        if (a.balanced) {                                                                      \
+            const Segment sg_ = balanced_segment((t), t_begin, t_end, a.units_per_tile, a.unit_log2, a.steps_total); \
+            row_tile = sg_.row_tile;                                                           \
+            sb = sg_.sb;                                                                       \
+            nsteps = sg_.nsteps;                                                               \
+            part = sg_.part;                                                                   \
+            t_next = sg_.next;                                                                 \
+        } else {                                                                               \
+            row_tile = (t) / a.split_k;                                                        \
+            part = (t) - row_tile * a.split_k;                                                 \
+            sb = part * a.steps_per_split;                                                     \
+            nsteps = max(min(a.steps_total, sb + a.steps_per_split) - sb, 0);                  \
+            if (a.split_k == 1) part = -1;                                                     \
+            t_next = (t) + n_wg;                                                               \
+        }                                                                                      \
         const int row0_ = row_tile * rows_wg + wm * (RW * kRowsPerLoad);                       \
-        sb = ks * a.steps_per_split;                                                           \
-        nsteps = max(min(a.steps_total, sb + a.steps_per_split) - sb, 0);                      \
         n_it = nsteps > wk ? (nsteps - wk + a.waves_k - 1) >> a.wk_log2 : 0;                   \
         s_first = sb + wk;                                                                     \
+        /* stagger: this row tile walks its k range starting rot steps in, wrapping around */  \
+        seg_hi = sb + nsteps;                                                                  \
+        s_clamp = min(seg_hi, a.steps_total) - 1;                                              \
+        rot = (a.k_stagger && nsteps > 1) ? (int)(((unsigned)row_tile * (unsigned)a.k_stagger) % (unsigned)nsteps) : 0; \
         _Pragma("unroll") for (int rw = 0; rw < RW; ++rw)                                      \
         {                                                                                      \
             const int mb_ = min(((row0_ + rw * kRowsPerLoad) >> 3) + (i16 >> 1), mb_last);     \
@@ -243,12 +284,13 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
             const int row_ = row0_ + rw * kRowsPerLoad + i16 * 4 + j;                          \
             sc32c[rw][j] = a.absmax[min(row_, a.m - 1)]; /* rows past m are never stored */    \
         }                                                                                      \
-        x_stage_load<TT, XB>(xst, xg, 0, nthreads, tid, x_pieces, tok0, sb * kStepK, a.n, a.k);    \
+        krot = KRot{rot * kStepK, seg_hi * kStepK, nsteps * kStepK};                           \
+        x_stage_load<TT, XB>(xst, xg, 0, nthreads, tid, x_pieces, tok0, sb * kStepK, a.n, a.k, krot); \
     }
 
-    int t = wg;
+    int t = t_begin;
     const float code_lane = a.code[lane & 15];
-    if (t < a.tiles_total) TUNA_TILE_FETCH(t)
+    if (t < t_end) TUNA_TILE_FETCH(t)
     TUNA_MARK(1)
 
 
@@ -286,10 +328,11 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     const int ipc = a.chunk_steps >> a.wk_log2;  // iterations per chunk per wave (multiple of U)
     const int wstep = a.waves_k * (1024 * TT);   // LDS bytes between this wave's consecutive steps
 
-    for (; t < a.tiles_total; t += n_wg) {
+    while (t < t_end) {
         // ---- this tile's scales (fp16 like the reference's staging, kernel.cu:2770) and the
         //      first x chunk, requested behind the ring loads already in flight
         float sc32c[RW][4];
+        KRot krot;
         TUNA_TILE_SMALL_LOADS()
         if (tile_iter == 0) {
             // (placed here so that the first tile's loads are all in flight while it is built)
@@ -328,13 +371,13 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 #pragma unroll
                 for (int tt = 0; tt < TT; ++tt) acc[rw][j][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-        const int cur_row_tile = row_tile, cur_ks = ks, cur_sb = sb;
+        const int cur_row_tile = row_tile, cur_part = part, cur_sb = sb;
         const int n_chunks = (nsteps + a.chunk_steps - 1) >> a.chunk_log2;
         int it = 0;  // this wave's next iteration (multiple of U)
 
         // the work area is free again once every wave has left the previous tile's epilogue
         __syncthreads();
-        if (n_chunks > 0) x_stage_store<TT, XB>(xst, work, 0, nthreads, tid, x_pieces, tok0, cur_sb * kStepK, a.n, a.k);
+        if (n_chunks > 0) x_stage_store<TT, XB>(xst, work, 0, nthreads, tid, x_pieces, tok0, cur_sb * kStepK, a.n, a.k, krot);
         __syncthreads();
         TUNA_MARK(3)
 
@@ -351,10 +394,10 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                 // that after the group exactly U*RW younger loads are in flight and the wait before
                 // the LDS write below is an exact vmcnt, not a drain of the weight ring.
                 const int kbase = (cur_sb + (c + 1) * a.chunk_steps) * kStepK;
-                x_stage_load<TT, XB>(xst, xg, 0, nthreads, tid, x_pieces, tok0, kbase, a.n, a.k);
+                x_stage_load<TT, XB>(xst, xg, 0, nthreads, tid, x_pieces, tok0, kbase, a.n, a.k, krot);
                 TUNA_GROUP()
                 __syncthreads();  // every wave is done reading chunk c
-                x_stage_store<TT, XB>(xst, work, 0, nthreads, tid, x_pieces, tok0, kbase, a.n, a.k);
+                x_stage_store<TT, XB>(xst, work, 0, nthreads, tid, x_pieces, tok0, kbase, a.n, a.k, krot);
                 __syncthreads();
             } else {
                 const int it_end = min(it_chunk0 + ipc, n_it);
@@ -383,7 +426,8 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
         TUNA_MARK(4)
 
         // ---- next tile: get its loads going before this tile's reduction and store ---------
-        if (t + n_wg < a.tiles_total) TUNA_TILE_FETCH(t + n_wg)
+        t = t_next;
+        if (t < t_end) TUNA_TILE_FETCH(t)
 
         // ---- workgroup reduction and store ---------------------------------------------------
         // A plane is one float4 per lane = 256 floats [lane][4].  The waves_k waves of a row
@@ -402,12 +446,41 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
         const size_t plane_floats = (size_t)(a.waves_m * a.waves_k) * 256;  // one buffer
         float *redf = reinterpret_cast<float *>(work);
         const size_t tile_id = (size_t)blockIdx.y * a.row_tiles + cur_row_tile;
-        // workspace of a tile: [split][wm][rw][tt][f][j] floats
-        float *wst = a.ws + (tile_id * a.split_k * a.waves_m) * (size_t)(NACC * 256);
-        float *mine = wst + ((size_t)cur_ks * a.waves_m + wm_e) * (NACC * 256);
+        // Partial sums of a segment: [wm][rw][tt][f][j] floats.  Fixed split: the row tile's
+        // split_k segments lie side by side in split order.  Balanced split: a workgroup owns
+        // two slots (a workgroup has at most two segments that are not whole row tiles: the
+        // one that starts at its first unit - slot 0 - and the one that ends at its last -
+        // slot 1).  The contributors of a row tile are consecutive workgroups in k order, and
+        // only the first of them can have used its slot 1.  Contributor c of this row tile is
+        // at src0 + c*src_stride - (c > 0 ? src_adj : 0).
+        const bool partial = cur_part >= 0;
+        const size_t seg_floats = (size_t)a.waves_m * (NACC * 256);
+        const float *src0 = a.ws;
+        size_t src_stride = 0, src_adj = 0;
+        float *mine = a.ws;
+        unsigned n_contrib = 1;
+        if (partial) {
+            if (a.balanced) {
+                const unsigned nw = (unsigned)n_wg;
+                unsigned w_lo, first_slot;
+                balanced_contributors((unsigned)cur_row_tile, (unsigned)a.units_per_tile, (unsigned)a.units_total, nw, &w_lo,
+                                      &n_contrib, &first_slot);
+                float *wsy = a.ws + (size_t)blockIdx.y * nw * 2 * seg_floats;
+                src0 = wsy + ((size_t)w_lo * 2 + first_slot) * seg_floats;
+                src_stride = 2 * seg_floats;
+                src_adj = first_slot * seg_floats;
+                mine = wsy + ((size_t)wg * 2 + (unsigned)cur_part) * seg_floats + (size_t)wm_e * (NACC * 256);
+            } else {
+                float *wst = a.ws + (tile_id * a.split_k) * seg_floats;
+                src0 = wst;
+                src_stride = seg_floats;
+                mine = wst + (size_t)cur_part * seg_floats + (size_t)wm_e * (NACC * 256);
+                n_contrib = (unsigned)a.split_k;
+            }
+        }
         f16 *outp = reinterpret_cast<f16 *>(a.out);
         bool write_out = true;
-        if (a.waves_k == 1 && a.split_k == 1) {
+        if (a.waves_k == 1 && !partial) {
             // No k split at all: the wave's accumulators are final.  Lane (token i16, group g)
             // owns 16 consecutive output features, acc[rw][j][tt][v] being feature 4*v + j of
             // them: two 16-byte stores per 64-row group, no LDS, no barrier.
@@ -478,7 +551,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                 for (int i = 0; i < 4; ++i) {
                     const int f = ((i << a.wk_log2) + wk_e) * 64 + lane_e;
                     if (f >= 256) continue;
-                    if (a.split_k == 1) {
+                    if (!partial) {
                         const int l = f >> 2, v = f & 3;
                         const int tok = tok0 + tt * 16 + (l & 15);
                         const int row = cur_row_tile * rows_wg + wm_e * (RW * kRowsPerLoad) + rw * 64 + (l >> 4) * 16 + v * 4;
@@ -496,7 +569,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
             }
         TUNA_MARK(5)
 
-        if (a.split_k > 1) {
+        if (partial) {
             // Partials travel as device-scope relaxed atomics (write-through stores, L2-bypassing
             // loads): coherent across the 8 XCD L2s without the L2 write-back/invalidate that a
             // device-scope release/acquire fence costs on every workgroup.  Order is given by
@@ -511,19 +584,19 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                 *ticket = __hip_atomic_fetch_add(a.counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __syncthreads();
             TUNA_MARK(7)
-            write_out = *ticket == (unsigned)(a.split_k - 1);
+            write_out = *ticket == n_contrib - 1u;
             if (write_out) {
-                // last workgroup of this tile: every partial is in memory; add them in split order
+                // last workgroup of this row tile: every partial is in memory; add them in k order
                 if (wk_e + wm_e == 0 && lane_e == 0)
                     __hip_atomic_store(a.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 for (int rt = 0; rt < RW * TT; ++rt)
                     for (int i = 0; i < 4; ++i) {
                         const int f = ((i << a.wk_log2) + wk_e) * 64 + lane_e;
                         if (f >= 256) break;
-                        const float *src = wst + (size_t)wm_e * (NACC * 256) + ((size_t)rt * 256 + f) * 4;
+                        const float *src = src0 + (size_t)wm_e * (NACC * 256) + ((size_t)rt * 256 + f) * 4;
                         float s4[4] = {0.f, 0.f, 0.f, 0.f};
-                        for (int sp = 0; sp < a.split_k; ++sp) {
-                            const float *sps = src + (size_t)sp * a.waves_m * (NACC * 256);
+                        for (unsigned sp = 0; sp < n_contrib; ++sp) {
+                            const float *sps = src + (size_t)sp * src_stride - (sp ? src_adj : 0);
 #pragma unroll
                             for (int j = 0; j < 4; ++j)
                                 s4[j] += __hip_atomic_load(sps + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -17,6 +17,7 @@ constexpr int kLdsLimit = 160 * 1024;
 constexpr int kStepK = 32;          // k per MFMA step (v_mfma_f32_16x16x32_f16)
 constexpr int kRowsPerLoad = 64;    // weight rows covered by one 128-bit load per lane
 constexpr int kMaxThreads = 1024;
+constexpr int kMaxCus = 256;        // compute units of the largest gfx950 part: bounds the persistent grid
 
 // Everything a GEMM launch needs, filled by the host from a tuna_gemm_config.
 struct GemmArgs {
@@ -28,22 +29,75 @@ struct GemmArgs {
     float *ws;           // split-K partial sums (library owned), may be null if split_k == 1
     unsigned *counters;  // one arrival counter per (token chunk, row tile), zero between launches
     int m, n, k;
-    int waves_m, waves_k, split_k;  // waves_m and waves_k are powers of two
-    int wm_log2, wk_log2;
+    int waves_m, waves_k, split_k;  // waves_k is a power of two, waves_m any count
+    int wk_log2;
     int steps_total;      // ceil(k / 32)
     int steps_per_split;  // k-steps owned by one workgroup
     int chunk_steps;      // k-steps of x staged in LDS at a time (power of two)
     int chunk_log2;
     int row_tiles;        // workgroups along m
     int xcd_swizzle;
+    int k_stagger;        // k-steps by which consecutive row tiles start later in their k range (0: none)
     int lds_bytes;        // dynamic LDS size of the launch (last 16 bytes: arrival ticket)
     int red_bytes;        // bytes of the reduction buffers in the LDS work area
     int planes_log2;      // log2(accumulator planes reduced per epilogue pass)
     int tiles_total;      // row_tiles * split_k: tiles walked by the persistent workgroups
+    int balanced;         // 1: balanced split (config split_k == 0), the fields below apply
+    int unit_log2;        // log2(k-steps per unit), a unit being what the split is made of
+    int units_per_tile;   // ceil(steps_total / unit)
+    int units_total;      // row_tiles * units_per_tile; (units_total + 1) * gridDim.x < 2^31
 #ifdef TUNA_TRACE
     unsigned long long *trace;  // development builds only: 16 timestamps per workgroup
 #endif
 };
+
+// ---------------------------------------------------------------------------------------
+// Balanced split: arithmetic shared by the kernel and the host (tuna_config_segments).
+// The k range of every row tile is cut into units of 2^unit_log2 k-steps; the T units of all
+// row tiles form one sequence; workgroup w of nw owns units [floor(w*T/nw), floor((w+1)*T/nw))
+// and walks them as segments that end at row tile boundaries.  (T + 1) * nw < 2^31.
+// ---------------------------------------------------------------------------------------
+struct Segment {
+    int row_tile;  // row tile of the segment
+    int sb;        // first k-step
+    int nsteps;    // k-steps (the last unit of a row tile may be short)
+    int part;      // -1: the whole row tile (sums are final); 0 / 1: the workgroup's partial-sum slot
+    int next;      // cursor of the workgroup's next segment
+};
+
+__host__ __device__ inline int balanced_begin(unsigned w, unsigned nw, unsigned T) { return (int)((w * T) / nw); }
+
+// Segment that starts at unit u of the workgroup owning units [t_begin, t_end).
+__host__ __device__ inline Segment balanced_segment(int u, int t_begin, int t_end, int units_per_tile, int unit_log2,
+                                                    int steps_total)
+{
+    Segment s;
+    s.row_tile = (int)((unsigned)u / (unsigned)units_per_tile);
+    const int u_in = u - s.row_tile * units_per_tile;
+    const int left_tile = units_per_tile - u_in, left_wg = t_end - u;
+    const int seg = left_wg < left_tile ? left_wg : left_tile;
+    s.sb = u_in << unit_log2;
+    const int want = seg << unit_log2, have = steps_total - s.sb;
+    s.nsteps = want < have ? want : have;
+    s.part = seg == units_per_tile ? -1 : (u == t_begin ? 0 : 1);
+    s.next = u + seg;
+    return s;
+}
+
+// Contributors of a row tile: workgroups w_lo .. w_lo + n - 1, in k order; first_slot is the
+// slot contributor 0 used (every later contributor starts the row tile's share at its own
+// first unit, so it used slot 0).
+__host__ __device__ inline void balanced_contributors(unsigned row_tile, unsigned units_per_tile, unsigned T, unsigned nw,
+                                                      unsigned *w_lo, unsigned *n, unsigned *first_slot)
+{
+    const unsigned u0 = row_tile * units_per_tile, u1 = u0 + units_per_tile - 1u;
+    // the workgroup that owns unit u is the largest w with floor(w*T/nw) <= u
+    const unsigned lo = ((u0 + 1u) * nw - 1u) / T;
+    const unsigned hi = ((u1 + 1u) * nw - 1u) / T;
+    *w_lo = lo;
+    *n = hi - lo + 1u;
+    *first_slot = (lo * T) / nw < u0 ? 1u : 0u;
+}
 
 struct GemmPlan {
     GemmArgs args;

@@ -36,7 +36,7 @@ N_BUCKETS = {
 }
 
 FIELDS = ("rows_per_wave", "waves_m", "waves_k", "split_k", "prefetch", "x_chunk",
-          "token_tiles", "xcd_swizzle")
+          "token_tiles", "xcd_swizzle", "k_stagger")
 
 LUT_BYTES = 256 * 64 * 4
 LDS_LIMIT = 160 * 1024
@@ -64,6 +64,7 @@ def bucket_of(n: int):
 
 def validate(m: int, n_key: int, k: int, c: dict) -> None:
     """Raise ValueError unless config `c` can run shape (m, n in bucket n_key, k)."""
+    c = {"k_stagger": 0, **c}  # entries written before the field existed
     missing = [f for f in FIELDS if f not in c]
     if missing:
         raise ValueError(f"missing fields {missing}")
@@ -78,13 +79,13 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
     if c["token_tiles"] not in (1, 2, 4):
         raise ValueError("token_tiles must be 1, 2 or 4")
     wm, wk = c["waves_m"], c["waves_k"]
-    if not _pow2(wm) or not _pow2(wk) or wm * wk > 16:
-        raise ValueError("waves_m and waves_k must be powers of two with waves_m * waves_k <= 16")
+    if wm < 1 or not _pow2(wk) or wm * wk > 16:
+        raise ValueError("waves_m must be >= 1 and waves_k a power of two, with waves_m * waves_k <= 16")
     if m * k // 2 >= 1 << 32:
         raise ValueError("packed weights exceed the kernel's 32-bit offsets")
     steps = -(-k // STEP_K)
-    if not 1 <= c["split_k"] <= steps:
-        raise ValueError(f"split_k must be in 1..{steps}")
+    if not 0 <= c["split_k"] <= steps:
+        raise ValueError(f"split_k must be in 0..{steps} (0 = balanced split)")
     unit = STEP_K * wk * c["prefetch"]
     if not _pow2(c["x_chunk"]) or c["x_chunk"] < unit:
         raise ValueError(f"x_chunk must be a power of two >= {unit}")
@@ -95,6 +96,8 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
         raise ValueError(f"no kernel variant {key} for {threads} threads")
     if c["x_chunk"] * c["token_tiles"] > (4 if c["prefetch"] == 8 else 2) * threads:
         raise ValueError("x_chunk * token_tiles too large for the x staging (4 pieces per thread, 8 with prefetch 8)")
+    if not 0 <= c["k_stagger"] <= 4096:
+        raise ValueError("k_stagger must be in 0..4096")
     if lds_bytes(c) > LDS_LIMIT:
         raise ValueError(f"needs {lds_bytes(c)} bytes of LDS (limit {LDS_LIMIT})")
 
@@ -123,7 +126,7 @@ def generate(param_map: dict) -> str:
         except ValueError as e:
             raise ValueError(f"param_map entry {key}: {e}") from None
         lo, hi = N_BUCKETS[n]
-        vals = ", ".join(str(int(c[f])) for f in FIELDS)
+        vals = ", ".join(str(int(c.get(f, 0))) for f in FIELDS)
         rows.append(f"    {{{m}, {lo}, {hi}, {k}, {{{vals}}}}},  // {key}")
     body = "\n".join(rows)
     return f"""// GENERATED by tuna_amd/make_configs.py from tuna_amd/configs/param_map.json - do not edit.
@@ -135,7 +138,7 @@ namespace tuna {{
 
 const TableEntry kConfigTable[] = {{
 {body}
-    {{0, 0, 0, 0, {{0, 0, 0, 0, 0, 0, 0, 0}}}},  // sentinel (not counted)
+    {{0, 0, 0, 0, {{0, 0, 0, 0, 0, 0, 0, 0, 0}}}},  // sentinel (not counted)
 }};
 const int kConfigTableSize = {len(rows)};
 

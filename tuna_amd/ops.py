@@ -110,6 +110,28 @@ def config_footprint(m: int, n: int, k: int, cfg: GemmConfig):
     return lds.value, ws.value
 
 
+def config_segments(m: int, n: int, k: int, cfg: GemmConfig, n_workgroups: int = 0, workgroup: int = 0):
+    """Segments (row tile, first k-step, k-steps, partial-sum slot or -1) that workgroup
+    `workgroup` of `n_workgroups` walks in a launch of `cfg`.  Host only."""
+    L = _lib.lib()
+    cnt = ctypes.c_int(0)
+    _lib.check(L.tuna_config_segments(int(m), int(n), int(k), ctypes.byref(cfg), int(n_workgroups), int(workgroup),
+                                      None, 0, ctypes.byref(cnt)))
+    buf = (ctypes.c_int * (4 * max(cnt.value, 1)))()
+    _lib.check(L.tuna_config_segments(int(m), int(n), int(k), ctypes.byref(cfg), int(n_workgroups), int(workgroup),
+                                      buf, cnt.value, ctypes.byref(cnt)))
+    return [tuple(buf[4 * i:4 * i + 4]) for i in range(cnt.value)]
+
+
+def config_contributors(m: int, n: int, k: int, cfg: GemmConfig, n_workgroups: int, row_tile: int):
+    """(first workgroup, count, slot of the first) of the partial sums of a row tile under a
+    balanced split; (-1, split_k, 0) under a fixed split.  Host only."""
+    a, b, c = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+    _lib.check(_lib.lib().tuna_config_contributors(int(m), int(n), int(k), ctypes.byref(cfg), int(n_workgroups),
+                                                   int(row_tile), ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))
+    return a.value, b.value, c.value
+
+
 def config_table():
     """The built-in tuned table as a list of (m, n_lo, n_hi, k, GemmConfig)."""
     L = _lib.lib()

@@ -28,11 +28,12 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 
 GENES = {
     "rows_per_wave": (64, 128, 256),
-    "waves_m": (1, 2, 4, 8),
+    "waves_m": (1, 2, 3, 4, 5, 6, 7, 8),
     "waves_k": (1, 2, 4, 8, 16),
     "prefetch": (2, 4, 8),
     "token_tiles": (1, 2, 4),
     "xcd_swizzle": (0, 1),
+    "k_stagger": (0, 1, 1, 2, 3, 5, 8, 16),
 }
 N_CU = 256
 
@@ -47,6 +48,7 @@ def _pow2_floor(v: int) -> int:
 def repair(c: dict, m: int, n_key: int, k: int):
     """Make a raw gene vector a valid config for the shape, or return None."""
     c = dict(c)
+    c.setdefault("k_stagger", 0)
     steps = -(-k // 32)
     if c["waves_m"] * c["waves_k"] > 16:
         return None
@@ -56,8 +58,8 @@ def repair(c: dict, m: int, n_key: int, k: int):
     c["token_tiles"] = min(c["token_tiles"], need)
     threads = 64 * c["waves_m"] * c["waves_k"]
     unit = 32 * c["waves_k"] * c["prefetch"]      # smallest x chunk: one ring turn of the workgroup
-    c["split_k"] = max(1, min(int(c["split_k"]), steps))
-    sps = -(-steps // c["split_k"])
+    c["split_k"] = max(0, min(int(c["split_k"]), steps))    # 0 = balanced split
+    sps = -(-steps // max(1, c["split_k"]))
     # x chunk: a power of two in [unit, 2*threads/token_tiles], no larger than the split needs
     hi_chunk = _pow2_floor(max(unit, (4 if c["prefetch"] == 8 else 2) * threads // c["token_tiles"]))
     want = max(unit, min(_pow2_floor(max(int(c.get("x_chunk", 1024)), 1)), hi_chunk))
@@ -80,16 +82,16 @@ def seeds(m: int, n_key: int, k: int):
     out = []
     for rpw in (64, 128):
         for wm, wk in ((1, 4), (1, 8), (2, 4), (2, 2), (4, 2), (1, 16), (2, 8), (4, 4), (4, 1), (8, 1), (1, 2), (16, 1),
-                       (8, 2), (2, 1)):
+                       (8, 2), (2, 1), (7, 1), (7, 2), (14, 1), (3, 4), (3, 2), (5, 2), (6, 2), (5, 1), (6, 1), (3, 1)):
             row_tiles = -(-m // (rpw * wm))
-            for target in (N_CU, 2 * N_CU, 4 * N_CU):
-                split = max(1, round(target / row_tiles))
+            for target in (0, N_CU, 2 * N_CU, 4 * N_CU):
+                split = max(1, round(target / row_tiles)) if target else 0
                 for pf in (2, 4, 8):
                     for tt in (1, 2, 4):
                         for xc in (256, 512, 1024, 2048):
-                            for sw in (0, 1):
+                            for sw, stg in ((0, 0), (1, 0), (1, 1), (0, 1)):
                                 c = repair(dict(rows_per_wave=rpw, waves_m=wm, waves_k=wk, split_k=split, prefetch=pf,
-                                                x_chunk=xc, token_tiles=tt, xcd_swizzle=sw), m, n_key, k)
+                                                x_chunk=xc, token_tiles=tt, xcd_swizzle=sw, k_stagger=stg), m, n_key, k)
                                 if c is not None:
                                     out.append(c)
     uniq = {json.dumps(c, sort_keys=True): c for c in out}
@@ -101,7 +103,12 @@ def mutate(c: dict, rng: random.Random, m, n_key, k):
     for _ in range(rng.choice((1, 1, 2))):
         gene = rng.choice(list(GENES) + ["split_k", "split_k", "x_chunk"])
         if gene == "split_k":
-            c["split_k"] = max(1, int(round(c["split_k"] * rng.choice((0.5, 0.75, 1.25, 1.5, 2.0)) + rng.choice((-1, 0, 1)))))
+            if rng.random() < 0.2:
+                c["split_k"] = 0                                   # balanced split
+            elif c["split_k"] == 0:
+                c["split_k"] = rng.choice((1, 2, 4, 8))
+            else:
+                c["split_k"] = max(1, int(round(c["split_k"] * rng.choice((0.5, 0.75, 1.25, 1.5, 2.0)) + rng.choice((-1, 0, 1)))))
         elif gene == "x_chunk":
             c["x_chunk"] = max(64, int(c["x_chunk"] * rng.choice((0.5, 2.0))))
         else:
