@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A "step" is one GEMM of the headline workload (Mistral-7B QKV projection at 16 tokens:
-out[16, 6144] = x[16, 4096] . W[6144, 4096]^T, BASELINE config 1) on one of a rotating set
+out[16, 6144] = x[16, 4096] . W[6144, 4096]^T, benchmark configuration 1) on one of a rotating set
 of distinct, HBM-resident weight matrices, so that neither L2 nor the 256 MB Infinity Cache
 can serve re-reads.  W warm-up steps, then exactly K timed steps bracketed by HIP events on
 the launch stream (tuna_time_matmul, inside the C library, so that no Python overhead sits
@@ -14,7 +14,7 @@ between launches).  One JSON line is printed:
   ms_per_step  milliseconds per GEMM (x1000 = the metric's "us/GEMM")
   roofline     achieved / peak HBM bandwidth for the GEMM kernel (algorithmic bytes = m*k/2)
   cpu_baseline the CPU oracle's dequantize-then-matmul on the same workload, host cores
-  shapes       the same measurement for every 16-token layer shape of the BASELINE configs
+  shapes       the same measurement for every 16-token layer shape of the benchmark configurations
   sweeps       Llama-70B 80-layer sweep (distinct weights per layer) and the token sweep
 """
 import argparse
@@ -177,7 +177,7 @@ def main():
         "dtype": "f16",
         "data": "synthetic",
         "config": {
-            "workload": f"{'BASELINE config 1: Mistral-7B QKV projection' if args.workload == HEADLINE else args.workload}, "
+            "workload": f"{'benchmark config 1: Mistral-7B QKV projection' if args.workload == HEADLINE else args.workload}, "
                         f"M={n} tokens, K={k}, N={m}; "
                         f"uniform 4-bit codes, fp16 scales U(0.005,0.02), x ~ N(0,1)*0.1; "
                         f"{head['weight_sets']} distinct weight matrices rotated",

@@ -112,7 +112,7 @@ def test_gemm_matches_oracle_small(m, n, k):
 
 @pytest.mark.parametrize("name", ["mistral_attn_out", "mistral_qkv"])
 def test_gemm_matches_oracle_full_config(name):
-    """BASELINE configs 0 and 1 in full (all rows), seed 0."""
+    """Benchmark configurations 0 and 1 in full (all rows), seed 0."""
     from tuna_amd.synth import SHAPES
 
     m, k = SHAPES[name]
@@ -238,7 +238,7 @@ def test_gemm_linearity_and_zero():
     assert np.array_equal(y2[normal], 2 * y1[normal])
 
 
-# ----------------------------------------------------------------------------- BASELINE sizes
+# ----------------------------------------------------------------------------- full benchmark sizes
 
 @pytest.mark.parametrize("name", list(__import__("tuna_amd.synth", fromlist=["SHAPES"]).SHAPES))
 def test_baseline_shapes_row_subset_and_readout(name):
@@ -293,7 +293,7 @@ def test_baseline_shapes_row_subset_and_readout(name):
 
 @pytest.mark.parametrize("n", [1, 64, 256])
 def test_token_sweep_llama_attn_out(n):
-    """The M sweep {1, 16, 64, 256} of BASELINE config 3 on the attention out-proj shape
+    """The M sweep {1, 16, 64, 256} of benchmark configuration 3 on the attention out-proj shape
     (16 is covered above), checked on a row subset."""
     import torch
 

@@ -9,7 +9,7 @@ import numpy as np
 
 from .quantize import NF4_CODE
 
-# (name, m = output features, k) of the 16-token layer shapes; BASELINE order
+# (name, m = output features, k) of the 16-token layer shapes, in the order of the benchmark configurations
 SHAPES = {
     "mistral_attn_out": (4096, 4096),
     "mistral_qkv": (6144, 4096),

@@ -12,7 +12,7 @@ Search: a seeded population of hand-derived configs, then generations of
 (tournament selection -> crossover -> mutation -> validity repair), every candidate timed on
 the GPU with HIP events over rotating, cache-defeating weight sets (tuna_time_matmul).
 
-    python -m tuna_amd.tuner --tokens 16 --shapes all --generations 6 --out gpurun_out/param_map.json
+    python -m tuna_amd.tuner --tokens 16 --shapes all --generations 6 --out tuned/param_map.json
 """
 import argparse
 import json
@@ -210,7 +210,7 @@ def main(argv=None):
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--base", default=os.path.join(HERE, "configs", "param_map.json"),
                     help="existing param_map.json to update")
-    ap.add_argument("--out", default="gpurun_out/param_map.json")
+    ap.add_argument("--out", default="tuned/param_map.json")
     ap.add_argument("--eval", default=None, help="JSON config: just time it on the given shapes and exit")
     args = ap.parse_args(argv)
 
