@@ -107,6 +107,17 @@ __device__ __forceinline__ f16x8 decode_dword(uint32_t d, const unsigned char *l
     }
 }
 
+// One 16-byte device-coherent store of partial sums: the write-through form (sc1) the
+// compiler emits for a relaxed device-scope atomic store, which it only offers 4 bytes wide
+// (four of those cost four 32-byte-granular writes to memory for every 16 bytes).  The
+// caller orders it with an explicit s_waitcnt vmcnt(0) before signalling.
+__device__ __forceinline__ void store_partial(float *dst, f32x4 v)
+{
+    // the s_nop covers the wait state a store wider than 8 bytes needs before its data
+    // registers may be overwritten (the compiler does not see inside the asm)
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 0" : : "v"(dst), "v"(v) : "memory");
+}
+
 // x staging, global -> registers -> LDS, XB 16-byte pieces per thread (4, or 8 for the deepest
 // prefetch ring, whose smallest chunk is twice as long).
 // Piece p of a chunk is token row (p % (16*TT)), 8-k slot (p / (16*TT)) and lives at LDS
@@ -561,9 +572,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                         }
                     } else {
                         float *dst = mine + ((size_t)(rw * TT + tt) * 256 + f) * 4;
-#pragma unroll
-                        for (int j = 0; j < 4; ++j)
-                            __hip_atomic_store(dst + j, o[i][j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        store_partial(dst, f32x4{o[i][0], o[i][1], o[i][2], o[i][3]});
                     }
                 }
             }
