@@ -225,14 +225,19 @@ def main():
         # dequant kernel (k*m/2 bytes in, 2*k*m bytes out) on the 4096 x 4096 config
         from tuna_amd.quantize import nf4_codebook
 
-        dm, dk = synth.SHAPES["mistral_attn_out"]
-        sets = [synth.make_weights_torch(dm, dk, 50 + i, dev) for i in range(8)]
-        img = torch.empty((dm, dk), dtype=torch.float16, device=dev)
-        ms = ops.time_dequant([s[0] for s in sets], [s[1] for s in sets], nf4_codebook(dev), img, dm, dk, 10, 100)
-        us = ms * 10.0
-        line["dequant"] = {"m": dm, "k": dk, "us": round(us, 2),
-                           "gbs_in_plus_out": round(2.5 * dm * dk / (us * 1e-6) / 1e9, 1),
-                           "frac_hbm": round(2.5 * dm * dk / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+        deq = {}
+        for nm in ("mistral_attn_out", "mistral_gate_up", "llama70b_down"):
+            dm, dk = synth.SHAPES[nm]
+            sets = [synth.make_weights_torch(dm, dk, 50 + i, dev) for i in range(max(2, min(8, (1 << 30) // (dm * dk // 2))))]
+            img = torch.empty((dm, dk), dtype=torch.float16, device=dev)
+            ms = ops.time_dequant([s[0] for s in sets], [s[1] for s in sets], nf4_codebook(dev), img, dm, dk, 10, 100)
+            us = ms * 10.0
+            deq[nm] = {"m": dm, "k": dk, "us": round(us, 2),
+                       "gbs_in_plus_out": round(2.5 * dm * dk / (us * 1e-6) / 1e9, 1),
+                       "frac_hbm": round(2.5 * dm * dk / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+            del sets, img
+            torch.cuda.empty_cache()
+        line["dequant"] = deq
 
     if not args.no_sweeps:
         sweeps = {}

@@ -118,6 +118,62 @@ __device__ __forceinline__ void store_partial(float *dst, f32x4 v)
     asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 0" : : "v"(dst), "v"(v) : "memory");
 }
 
+// Cross-wave sum of NP accumulator planes for thread (wk, lane) of a row group.  A plane
+// buffer holds, per wave of the row group, 256 floats; the thread sums float
+// f = (i*WK + wk)*64 + lane of every wave, in wave order, for each i with f < 256.  WK (the
+// number of waves along k) is a template argument so that all WK*NP loads of a thread are
+// issued before the first add: with a run-time wave count the loop took one LDS round trip
+// per wave and plane (32 of them, 1.3 us, for 8 waves).
+template <int WK, int NP>
+__device__ __forceinline__ void sum_planes(const float *buf, size_t plane_floats, int wm, int wk, int lane,
+                                           float (&o)[4][4], int j0)
+{
+    constexpr int NI = WK >= 4 ? 1 : 4 / WK;                        // values of i that can give f < 256
+    constexpr int JB = 32 / (WK * NI) < NP ? (32 / (WK * NI) > 0 ? 32 / (WK * NI) : 1) : NP;  // planes per batch of <= 32 loads
+    const float *base = buf + (size_t)wm * (WK * 256);
+    if (WK > 4 && wk >= 4) return;  // (wave-uniform) the 256 floats of a plane are owned by waves 0..3
+#pragma unroll
+    for (int jb = 0; jb < NP; jb += JB) {
+        float v[JB][NI][WK];
+#pragma unroll
+        for (int j = 0; j < JB; ++j)
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                const int f = min((i * WK + wk) * 64 + lane, 255);  // clamped: unused sums are discarded by the caller
+#pragma unroll
+                for (int w = 0; w < WK; ++w) v[j][i][w] = base[(jb + j) * plane_floats + (size_t)w * 256 + f];
+            }
+        // all loads of the batch before the first add (the scheduler otherwise pairs each load
+        // with its add to save registers, which is the serial chain again)
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < JB; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float sum = 0.f;
+                if (i < NI) {
+#pragma unroll
+                    for (int w = 0; w < WK; ++w) sum += v[j][i < NI ? i : 0][w];
+                }
+                o[i][j0 + jb + j] = sum;
+            }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+template <int NP>
+__device__ __forceinline__ void sum_planes_any(int wk_log2, const float *buf, size_t plane_floats, int wm, int wk, int lane,
+                                               float (&o)[4][4], int j0)
+{
+    switch (wk_log2) {
+    case 0: sum_planes<1, NP>(buf, plane_floats, wm, wk, lane, o, j0); break;
+    case 1: sum_planes<2, NP>(buf, plane_floats, wm, wk, lane, o, j0); break;
+    case 2: sum_planes<4, NP>(buf, plane_floats, wm, wk, lane, o, j0); break;
+    case 3: sum_planes<8, NP>(buf, plane_floats, wm, wk, lane, o, j0); break;
+    default: sum_planes<16, NP>(buf, plane_floats, wm, wk, lane, o, j0); break;
+    }
+}
+
 // x staging, global -> registers -> LDS, XB 16-byte pieces per thread (4, or 8 for the deepest
 // prefetch ring, whose smallest chunk is twice as long).
 // Piece p of a chunk is token row (p % (16*TT)), 8-k slot (p / (16*TT)) and lives at LDS
@@ -435,6 +491,11 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
             }
         }
         TUNA_MARK(4)
+#ifdef TUNA_TRACE
+        if (a.trace && lane == 0 && tile_iter < 8) {  // latest wave of the workgroup out of the main loop
+            atomicMax(&a.trace[((size_t)blockIdx.x * 8 + tile_iter) * 16 + 10], (unsigned long long)wall_clock64());
+        }
+#endif
 
         // ---- next tile: get its loads going before this tile's reduction and store ---------
         t = t_next;
@@ -518,6 +579,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
             continue;
         }
         __syncthreads();  // every wave has left the main loop: the work area is free
+        TUNA_MARK(11)
 #pragma unroll
         for (int rw = 0; rw < RW; ++rw)
 #pragma unroll
@@ -531,31 +593,16 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                         reinterpret_cast<f32x4 *>(buf + j * plane_floats)[(size_t)(wm_e * a.waves_k + wk_e) * 64 + lane_e] =
                             acc[rw][j][tt];
                     __syncthreads();
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const int f = ((i << a.wk_log2) + wk_e) * 64 + lane_e;
-                            float sum = 0.f;
-                            if (f < 256)
-                                for (int w = 0; w < a.waves_k; ++w)
-                                    sum += buf[j * plane_floats + (size_t)(wm_e * a.waves_k + w) * 256 + f];
-                            o[i][j] = sum;
-                        }
+                    TUNA_MARK(12)
+                    sum_planes_any<4>(a.wk_log2, buf, plane_floats, wm_e, wk_e, lane_e, o, 0);
+                    TUNA_MARK(13)
                 } else {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         float *buf = redf + ((rw * TT + tt) * 4 + j) % 2 * plane_floats;
                         reinterpret_cast<f32x4 *>(buf)[(size_t)(wm_e * a.waves_k + wk_e) * 64 + lane_e] = acc[rw][j][tt];
                         __syncthreads();
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const int f = ((i << a.wk_log2) + wk_e) * 64 + lane_e;
-                            float sum = 0.f;
-                            if (f < 256)
-                                for (int w = 0; w < a.waves_k; ++w) sum += buf[(size_t)(wm_e * a.waves_k + w) * 256 + f];
-                            o[i][j] = sum;
-                        }
+                        sum_planes_any<1>(a.wk_log2, buf, plane_floats, wm_e, wk_e, lane_e, o, j);
                     }
                 }
 #pragma unroll
@@ -603,12 +650,25 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                         const int f = ((i << a.wk_log2) + wk_e) * 64 + lane_e;
                         if (f >= 256) break;
                         const float *src = src0 + (size_t)wm_e * (NACC * 256) + ((size_t)rt * 256 + f) * 4;
+                        // four contributors per round trip (indices are clamped so that the loads
+                        // are unconditional and all in flight together); summed in k order
                         float s4[4] = {0.f, 0.f, 0.f, 0.f};
-                        for (unsigned sp = 0; sp < n_contrib; ++sp) {
-                            const float *sps = src + (size_t)sp * src_stride - (sp ? src_adj : 0);
+                        for (unsigned sp0 = 0; sp0 < n_contrib; sp0 += 4) {
+                            float pv[4][4];
 #pragma unroll
-                            for (int j = 0; j < 4; ++j)
-                                s4[j] += __hip_atomic_load(sps + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            for (unsigned b = 0; b < 4; ++b) {
+                                const unsigned sp = min(sp0 + b, n_contrib - 1u);
+                                const float *sps = src + (size_t)sp * src_stride - (sp ? src_adj : 0);
+#pragma unroll
+                                for (int j = 0; j < 4; ++j)
+                                    pv[b][j] = __hip_atomic_load(sps + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            }
+#pragma unroll
+                            for (unsigned b = 0; b < 4; ++b)
+                                if (sp0 + b < n_contrib) {
+#pragma unroll
+                                    for (int j = 0; j < 4; ++j) s4[j] += pv[b][j];
+                                }
                         }
                         const int rw = rt / TT, tt = rt % TT;
                         const int l = f >> 2, v = f & 3;
