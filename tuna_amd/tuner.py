@@ -159,10 +159,10 @@ class Evaluator:
         return self.cache[key]
 
 
-def tune_shape(m, n, k, generations=6, population=24, seed=0, log=print, max_seed_evals=120):
+def tune_shape(m, n, k, generations=6, population=24, seed=0, log=print, max_seed_evals=120, iters=60):
     rng = random.Random(seed * 7919 + m * 31 + k)
     n_key = make_configs.bucket_of(n)
-    ev = Evaluator(m, n, k)
+    ev = Evaluator(m, n, k, iters=iters, warmup=max(2, iters // 6))
     pool = seeds(m, n_key, k)
     rng.shuffle(pool)
     pool = pool[:max_seed_evals]
@@ -194,7 +194,7 @@ def tune_shape(m, n, k, generations=6, population=24, seed=0, log=print, max_see
     top = sorted(((t, s) for s, t in ev.cache.items()))[:5]
     ev2 = Evaluator.__new__(Evaluator)
     ev2.__dict__.update(ev.__dict__)
-    ev2.cache, ev2.iters, ev2.warmup = {}, 300, 30
+    ev2.cache, ev2.iters, ev2.warmup = {}, 5 * iters, max(2, iters // 2)
     final = sorted((ev2(json.loads(s)), s) for _, s in top)
     log(f"  final: {final[0][0]:.2f} us {final[0][1]}  ({len(ev.cache)} configs tried)")
     return json.loads(final[0][1]), final[0][0]
@@ -208,6 +208,7 @@ def main(argv=None):
     ap.add_argument("--population", type=int, default=24)
     ap.add_argument("--max-seed-evals", type=int, default=120)
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--iters", type=int, default=60, help="timed launches per candidate (fewer for large token counts)")
     ap.add_argument("--base", default=os.path.join(HERE, "configs", "param_map.json"),
                     help="existing param_map.json to update")
     ap.add_argument("--out", default="tuned/param_map.json")
@@ -245,7 +246,8 @@ def main(argv=None):
             t0 = time.time()
             print(f"tuning {name} m={m} n={n} k={k}", flush=True)
             best, us = tune_shape(m, n, k, args.generations, args.population, args.seed,
-                                  log=lambda s: print(s, flush=True), max_seed_evals=args.max_seed_evals)
+                                  log=lambda s: print(s, flush=True), max_seed_evals=args.max_seed_evals,
+                                  iters=args.iters)
             key = f"{m}_{make_configs.bucket_of(n)}_{k}"
             best = dict(best)
             best["us"] = round(us, 3)
