@@ -93,6 +93,23 @@ int tuna_matmul_ex(const void *q, const void *x, const void *code, const void *a
                    void *out, int m, int n, int k, const tuna_gemm_config *cfg,
                    int decode_mode, void *stream);
 
+/* Grouped GEMM (mixture of experts with per-expert token lists) in one launch.  The weights
+ * are n_groups (<= 64) matrices of m_group rows stacked along m - q [n_groups*m_group/8, k/8,
+ * 32], absmax [n_groups*m_group] - exactly the layout of the dense stacked call.  x [n_total,
+ * k] holds the activation rows sorted by group: group e owns rows token_offsets[e] ..
+ * token_offsets[e+1]-1 (token_offsets: HOST array of n_groups+1 non-decreasing ints, read
+ * during the call; n_total = token_offsets[n_groups]).  out [n_total, m_group]:
+ *   out[t, r] = x[t, :] . decode(W_e)[r, :]   for t in group e.
+ * Groups without tokens are skipped: their weights are not read.  m_group must be a multiple
+ * of 64 (of the config's rows per workgroup if cfg is given; NULL = table lookup on
+ * (n_groups*m_group, largest group, k)).  No counterpart in the reference, whose 8-expert
+ * benchmark applies every expert to every token (README.md:16-18); this is the op a
+ * router-driven Mixtral layer needs. */
+int tuna_matmul_grouped(const void *q, const void *x, const void *code, const void *absmax,
+                        void *out, int m_group, int n_groups, int k,
+                        const int32_t *token_offsets, const tuna_gemm_config *cfg,
+                        int decode_mode, void *stream);
+
 /* out[m, k] fp16 row-major = decode(q, code, absmax), TUNA_DECODE_DEQUANT rounding.
  * Replaces  void dequantize_wrapper(void *q, void *a, void *c, void *o, const int m,
  * const int k, cudaStream_t)  (kernel.cu:3243, declared extension.cpp:24). */

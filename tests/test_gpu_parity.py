@@ -349,3 +349,80 @@ def test_errors_raise_instead_of_silent_noop():
         ops.matmul(x, q, s, c, o, m, n, k, config=cfg(x_chunk=1 << 20))  # exceeds LDS
     ops.matmul(x, q, s, c, o, m, n, k)               # and the valid call still works
     torch.cuda.synchronize()
+
+
+# ----------------------------------------------------------------------------- grouped GEMM (per-expert token lists)
+def _run_grouped(q, x, code, absmax, m_group, n_groups, k, offsets, config=None):
+    import torch
+
+    from tuna_amd import ops
+
+    dq, dx, dc, da = to_dev(q, x, code, absmax)
+    n_total = offsets[-1]
+    out = torch.full((max(n_total, 1), m_group), float("nan"), dtype=torch.float16, device="cuda")[:n_total]
+    ops.matmul_grouped(dx, dq, da, dc, out, m_group, n_groups, k, offsets, config=config)
+    torch.cuda.synchronize()
+    return out.cpu().numpy().view(np.uint16)
+
+
+def _grouped_reference(q, x, code, absmax, m_group, n_groups, k, offsets):
+    """Per expert: the oracle's dense GEMM on that expert's packed rows and tokens."""
+    n_total = offsets[-1]
+    ref = np.zeros((n_total, m_group), dtype=np.float64)
+    qb = q.reshape(n_groups, m_group // 8, k // 8, 32)
+    for e in range(n_groups):
+        lo, hi = offsets[e], offsets[e + 1]
+        if hi > lo:
+            ref[lo:hi] = O.gemm_f64(np.ascontiguousarray(qb[e]), np.ascontiguousarray(x[lo:hi]), code,
+                                    np.ascontiguousarray(absmax[e * m_group:(e + 1) * m_group]), m_group, hi - lo, k, mode=O.D1)
+    return ref
+
+
+@pytest.mark.parametrize("m_group,n_groups,k,counts,ckw", [
+    (256, 8, 1024, [4, 4, 4, 4, 4, 4, 4, 4], None),
+    (256, 8, 1024, [0, 7, 0, 16, 1, 0, 3, 5], None),                       # empty experts are skipped
+    (512, 4, 2048, [16, 0, 0, 16], dict(split_k=2, x_chunk=512)),
+    (512, 4, 2048, [3, 20, 0, 9], dict(token_tiles=2, split_k=2, prefetch=2, x_chunk=256)),   # 20 tokens: two token tiles
+    (384, 5, 1096, [2, 0, 33, 1, 6], dict(waves_m=3, waves_k=2, prefetch=2, x_chunk=128)),     # ragged k, 3 token chunks
+    (1024, 3, 512, [5, 5, 5], dict(waves_m=8, waves_k=1, prefetch=2, x_chunk=64)),            # register-store epilogue
+    (256, 6, 2048, [1, 0, 2, 0, 0, 9], dict(split_k=0, waves_m=1, waves_k=4, prefetch=2, x_chunk=256)),  # balanced split
+    (128, 64, 256, [i % 3 for i in range(64)], None),                      # 64 experts
+])
+def test_grouped_gemm_matches_per_expert_oracle(m_group, n_groups, k, counts, ckw):
+    offsets = [0]
+    for c in counts:
+        offsets.append(offsets[-1] + c)
+    n_total = offsets[-1]
+    m = m_group * n_groups
+    config = cfg(**ckw) if ckw else None
+    print(f"grouped m_group={m_group} n_groups={n_groups} k={k} counts={counts} cfg={ckw}", flush=True)
+    q, x, code, absmax = make_inputs_np(m, n_total, k, seed=77)
+    got = _run_grouped(q, x, code, absmax, m_group, n_groups, k, offsets, config)
+    ref = _grouped_reference(q, x, code, absmax, m_group, n_groups, k, offsets)
+    assert not np.isnan(f16_bits_to_f64(got)).any()          # every output row was written
+    e = rel_err(f16_bits_to_f64(got), ref)
+    assert e <= REL_TOL, e
+
+
+def test_grouped_gemm_with_one_group_equals_dense_bits():
+    """One group owning every token is the dense GEMM: identical bits."""
+    m, n, k = 1024, 16, 2048
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=5)
+    c = cfg(split_k=2)
+    dense = run_gemm(q, x, code, absmax, m, n, k, config=c)
+    grouped = _run_grouped(q, x, code, absmax, m, 1, k, [0, n], c)
+    assert np.array_equal(dense, grouped)
+
+
+def test_grouped_gemm_rejects_bad_arguments():
+    import torch
+
+    from tuna_amd import ops
+
+    q, x, code, absmax = make_inputs_np(512, 8, 256, seed=1)
+    dq, dx, dc, da = to_dev(q, x, code, absmax)
+    out = torch.empty((8, 256), dtype=torch.float16, device="cuda")
+    with pytest.raises(ops.TunaError):
+        ops.matmul_grouped(dx, dq, da, dc, out, 256, 2, 256, [0, 9, 8])         # decreasing offsets
+    with pytest.raises(ops.TunaError):
+        ops.matmul_grouped(dx, dq, da, dc, out, 256, 2, 256, [0, 4, 8], config=cfg(waves_m=8, waves_k=1, prefetch=2, x_chunk=64))  # 512-row tiles straddle groups

@@ -57,7 +57,7 @@ static inline int log2i(int v)
     return l;
 }
 
-static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode, GemmPlan *plan)
+static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode, GemmPlan *plan, int grouped = 0)
 {
     int rc = check_shape(m, n, k);
     if (rc) return rc;
@@ -113,14 +113,14 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     int min_waves = threads > 512 ? 4 : 2;
     int wgs_per_cu = 1;
     if (threads <= 512 && 2 * lds <= (size_t)kLdsLimit &&
-        gemm_variant_exists(rw, c.prefetch, c.token_tiles, decode, threads, 4)) {
+        gemm_variant_exists(rw, c.prefetch, c.token_tiles, decode, threads, 4, grouped)) {
         min_waves = 4;
         wgs_per_cu = 2;
     }
-    if (!gemm_variant_exists(rw, c.prefetch, c.token_tiles, decode, threads, min_waves))
+    if (!gemm_variant_exists(rw, c.prefetch, c.token_tiles, decode, threads, min_waves, grouped))
         return fail(TUNA_ERR_UNSUPPORTED,
-                    "no kernel variant for rows_per_wave=%d prefetch=%d token_tiles=%d decode=%d threads=%d", c.rows_per_wave,
-                    c.prefetch, c.token_tiles, decode, threads);
+                    "no %skernel variant for rows_per_wave=%d prefetch=%d token_tiles=%d decode=%d threads=%d",
+                    grouped ? "grouped " : "", c.rows_per_wave, c.prefetch, c.token_tiles, decode, threads);
 
     const int row_tiles = ceil_div(m, rows_wg);
     const int tok_chunks = ceil_div(n, 16 * c.token_tiles);
@@ -346,6 +346,81 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
     return TUNA_OK;
 }
 
+// Grouped GEMM: n_groups stacked weight matrices of m_group rows, group e applied to the
+// activation rows offsets[e] .. offsets[e+1]-1 only.  The offsets are a host array: they are
+// validated here and travel to the kernel as launch arguments (no device buffer, no copy).
+static int matmul_grouped_impl(const void *q, const void *x, const void *code, const void *absmax, void *out, int m_group,
+                               int n_groups, int k, const int32_t *offsets, const tuna_gemm_config *cfg, int decode,
+                               hipStream_t stream)
+{
+    int rc;
+    if (n_groups < 1 || n_groups > kMaxGroups)
+        return fail(TUNA_ERR_INVALID_ARG, "n_groups=%d must be in 1..%d", n_groups, kMaxGroups);
+    if (!offsets) return fail(TUNA_ERR_INVALID_ARG, "token_offsets is null");
+    if (m_group <= 0 || (long long)m_group * n_groups > 0x7fffffffLL)
+        return fail(TUNA_ERR_INVALID_ARG, "m_group=%d x n_groups=%d out of range", m_group, n_groups);
+    if (offsets[0] < 0) return fail(TUNA_ERR_INVALID_ARG, "token_offsets[0]=%d is negative", offsets[0]);
+    int max_tok = 0;
+    for (int e = 0; e < n_groups; ++e) {
+        const int cnt = offsets[e + 1] - offsets[e];
+        if (cnt < 0) return fail(TUNA_ERR_INVALID_ARG, "token_offsets must not decrease (group %d)", e);
+        if (cnt > max_tok) max_tok = cnt;
+    }
+    const int n_total = offsets[n_groups];
+    const int m = m_group * n_groups;
+    if ((rc = check_shape(m, n_total > 0 ? n_total : 1, k))) return rc;
+    if (m_group % kRowsPerLoad) return fail(TUNA_ERR_UNSUPPORTED, "m_group=%d must be a multiple of %d", m_group, kRowsPerLoad);
+    if (max_tok == 0) return TUNA_OK;  // no group has a token: nothing to compute, nothing to write
+    if ((rc = check_ptr(q, "q", 16)) || (rc = check_ptr(x, "x", 16)) || (rc = check_ptr(code, "code", 4)) ||
+        (rc = check_ptr(absmax, "absmax", 4)) || (rc = check_ptr(out, "out", 16)))
+        return rc;
+    tuna_gemm_config c;
+    if (cfg) c = *cfg;
+    else {
+        select_config(m, max_tok, k, &c, nullptr);
+        // the grouped kernels exist for 64 rows per wave and rings of 2 or 4 k-steps
+        c.rows_per_wave = kRowsPerLoad;
+        if (c.prefetch > 4) c.prefetch = 4;
+        // row tiles must not straddle groups: shrink the workgroup's row count until it divides m_group
+        while (m_group % (c.rows_per_wave * c.waves_m)) {
+            if (c.rows_per_wave > kRowsPerLoad) c.rows_per_wave /= 2;
+            else --c.waves_m;
+        }
+        const int x_cap = (c.prefetch == 8 ? 4 : 2) * c.waves_m * c.waves_k * 64;
+        while (c.x_chunk * c.token_tiles > x_cap && c.x_chunk / 2 >= kStepK * c.waves_k * c.prefetch) c.x_chunk /= 2;
+        if (decode != TUNA_DECODE_GEMM) {
+            c.rows_per_wave = 64;
+            c.prefetch = 2;
+        }
+    }
+    if (m_group % (c.rows_per_wave * c.waves_m))
+        return fail(TUNA_ERR_UNSUPPORTED, "rows per workgroup (%d) must divide m_group=%d", c.rows_per_wave * c.waves_m, m_group);
+    GemmPlan plan;
+    if ((rc = plan_gemm(m, max_tok, k, c, decode, &plan, 1))) return rc;
+    GemmArgs &a = plan.args;
+    a.q = static_cast<const uint8_t *>(q);
+    a.x = x;
+    a.code = static_cast<const float *>(code);
+    a.absmax = static_cast<const float *>(absmax);
+    a.out = out;
+    a.n = n_total;
+    a.group_rows = m_group;
+    a.n_groups = n_groups;
+    for (int e = 0; e <= n_groups; ++e) a.tok_off[e] = offsets[e];
+    if (plan.ws_bytes) {
+        Workspace w;
+        if ((rc = get_workspace(stream, plan.ws_bytes, plan.n_counters, &w))) return rc;
+        a.ws = w.ws;
+        a.counters = w.counters;
+    }
+#ifdef TUNA_TRACE
+    a.trace = g_trace;
+#endif
+    hipError_t e = launch_gemm(plan, stream);
+    if (e != hipSuccess) return hip_fail(e, "grouped gemm launch");
+    return TUNA_OK;
+}
+
 static int dequant_impl(const void *q, const void *absmax, const void *code, void *out, int m, int k, int decode,
                         hipStream_t stream)
 {
@@ -463,6 +538,14 @@ TUNA_EXPORT int tuna_matmul_ex(const void *q, const void *x, const void *code, c
                                int k, const tuna_gemm_config *cfg, int decode_mode, void *stream)
 {
     return matmul_impl(q, x, code, absmax, out, m, n, k, cfg, decode_mode, static_cast<hipStream_t>(stream));
+}
+
+TUNA_EXPORT int tuna_matmul_grouped(const void *q, const void *x, const void *code, const void *absmax, void *out,
+                                    int m_group, int n_groups, int k, const int32_t *token_offsets,
+                                    const tuna_gemm_config *cfg, int decode_mode, void *stream)
+{
+    return matmul_grouped_impl(q, x, code, absmax, out, m_group, n_groups, k, token_offsets, cfg, decode_mode,
+                               static_cast<hipStream_t>(stream));
 }
 
 TUNA_EXPORT int tuna_dequant(const void *q, const void *absmax, const void *code, void *out, int m, int k, void *stream)

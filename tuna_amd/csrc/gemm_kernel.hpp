@@ -124,12 +124,27 @@ __device__ __forceinline__ void store_partial(float *dst, f32x4 v)
 // number of waves along k) is a template argument so that all WK*NP loads of a thread are
 // issued before the first add: with a run-time wave count the loop took one LDS round trip
 // per wave and plane (32 of them, 1.3 us, for 8 waves).
-template <int WK, int NP>
+template <int WK, int NP, int LIM>
 __device__ __forceinline__ void sum_planes(const float *buf, size_t plane_floats, int wm, int wk, int lane,
                                            float (&o)[4][4], int j0)
 {
+    if constexpr (LIM == 0) {
+        // register-starved variants (two workgroups per CU): one LDS round trip at a time
+#pragma unroll
+        for (int j = 0; j < NP; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int f = (i * WK + wk) * 64 + lane;
+                float sum = 0.f;
+                if (f < 256)
+                    for (int w = 0; w < WK; ++w) sum += buf[j * plane_floats + (size_t)(wm * WK + w) * 256 + f];
+                o[i][j0 + j] = sum;
+            }
+        return;
+    }
     constexpr int NI = WK >= 4 ? 1 : 4 / WK;                        // values of i that can give f < 256
-    constexpr int JB = 32 / (WK * NI) < NP ? (32 / (WK * NI) > 0 ? 32 / (WK * NI) : 1) : NP;  // planes per batch of <= 32 loads
+    constexpr int LIM1 = LIM > 0 ? LIM : 1;
+    constexpr int JB = LIM1 / (WK * NI) < NP ? (LIM1 / (WK * NI) > 0 ? LIM1 / (WK * NI) : 1) : NP;  // planes per batch of <= LIM loads
     const float *base = buf + (size_t)wm * (WK * 256);
     if (WK > 4 && wk >= 4) return;  // (wave-uniform) the 256 floats of a plane are owned by waves 0..3
 #pragma unroll
@@ -161,16 +176,16 @@ __device__ __forceinline__ void sum_planes(const float *buf, size_t plane_floats
     }
 }
 
-template <int NP>
+template <int NP, int LIM>
 __device__ __forceinline__ void sum_planes_any(int wk_log2, const float *buf, size_t plane_floats, int wm, int wk, int lane,
                                                float (&o)[4][4], int j0)
 {
     switch (wk_log2) {
-    case 0: sum_planes<1, NP>(buf, plane_floats, wm, wk, lane, o, j0); break;
-    case 1: sum_planes<2, NP>(buf, plane_floats, wm, wk, lane, o, j0); break;
-    case 2: sum_planes<4, NP>(buf, plane_floats, wm, wk, lane, o, j0); break;
-    case 3: sum_planes<8, NP>(buf, plane_floats, wm, wk, lane, o, j0); break;
-    default: sum_planes<16, NP>(buf, plane_floats, wm, wk, lane, o, j0); break;
+    case 0: sum_planes<1, NP, LIM>(buf, plane_floats, wm, wk, lane, o, j0); break;
+    case 1: sum_planes<2, NP, LIM>(buf, plane_floats, wm, wk, lane, o, j0); break;
+    case 2: sum_planes<4, NP, LIM>(buf, plane_floats, wm, wk, lane, o, j0); break;
+    case 3: sum_planes<8, NP, LIM>(buf, plane_floats, wm, wk, lane, o, j0); break;
+    default: sum_planes<16, NP, LIM>(buf, plane_floats, wm, wk, lane, o, j0); break;
     }
 }
 
@@ -228,12 +243,13 @@ __device__ __forceinline__ void x_stage_store(const XStage<XB> &st, unsigned cha
     }
 }
 
-template <int RW, int U, int TT, int DEC, int MAXT, int MINW>
+template <int RW, int U, int TT, int DEC, int MAXT, int MINW, bool GRP>
 __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int NACC = RW * 4 * TT;  // float4 accumulator planes per lane
     constexpr int LUT_B = (DEC == TUNA_DECODE_GEMM) ? kLutBytes : 64;
+    constexpr int RED_LIM = MINW >= 4 ? 0 : 32;  // LDS loads in flight per thread in the cross-wave sums (0: unbatched)
 
     const int tid = threadIdx.x;
 #ifdef TUNA_TRACE
@@ -250,7 +266,10 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     const int i16 = lane & 15;
     const int g = lane >> 4;
     const int nthreads = (int)blockDim.x;
-    const int tok0 = blockIdx.y * (TT * 16);
+    // tokens of the tile being fetched / computed: [tok0, min(tok0 + 16*TT, n_tok)); rows of
+    // `out` are out_ld long and the tile's group starts at weight row out_row0
+    int tok0 = blockIdx.y * (TT * 16), n_tok = a.n, out_row0 = 0;
+    const int out_ld = GRP ? a.group_rows : a.m;
     const int rows_wg = a.waves_m * (RW * kRowsPerLoad);
     const int kb_total = a.k >> 3;
     const int mb_last = (a.m >> 3) - 1;
@@ -304,6 +323,26 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
             reinterpret_cast<const u32x4 *>(base_ + (last_ ? lb_last[rw] : lb[rw])));          \
     }
 
+    // Grouped launches: a tile whose group has no tokens in this token chunk is not walked at
+    // all (its weights are never read).  Advances `t` to the workgroup's next tile with work.
+#define TUNA_SKIP_EMPTY(t)                                                                      \
+    if constexpr (GRP) {                                                                        \
+        while ((t) < t_end) {                                                                  \
+            int rt_, nx_;                                                                      \
+            if (a.balanced) {                                                                  \
+                const Segment sg_ = balanced_segment((t), t_begin, t_end, a.units_per_tile, a.unit_log2, a.steps_total); \
+                rt_ = sg_.row_tile;                                                            \
+                nx_ = sg_.next;                                                                \
+            } else {                                                                           \
+                rt_ = (t) / a.split_k;                                                         \
+                nx_ = (t) + n_wg;                                                              \
+            }                                                                                  \
+            const int e_ = (rt_ * rows_wg) / a.group_rows;                                     \
+            if (a.tok_off[e_] + (int)blockIdx.y * (TT * 16) < a.tok_off[e_ + 1]) break;        \
+            (t) = nx_;                                                                         \
+        }                                                                                      \
+    }
+
     // Request what tile `t` streams from HBM first: the weight ring.  (The row scales and the
     // first x chunk are small and mostly L2 hits; they are requested at the start of the tile,
     // behind these loads: prefetched here they would cost 20 registers across the previous
@@ -326,6 +365,12 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
             t_next = (t) + n_wg;                                                               \
         }                                                                                      \
         const int row0_ = row_tile * rows_wg + wm * (RW * kRowsPerLoad);                       \
+        if constexpr (GRP) {                                                                    \
+            const int e_ = (row_tile * rows_wg) / a.group_rows;                                \
+            tok0 = a.tok_off[e_] + (int)blockIdx.y * (TT * 16);                                \
+            n_tok = a.tok_off[e_ + 1];                                                         \
+            out_row0 = e_ * a.group_rows;                                                      \
+        }                                                                                      \
         n_it = nsteps > wk ? (nsteps - wk + a.waves_k - 1) >> a.wk_log2 : 0;                   \
         s_first = sb + wk;                                                                     \
         /* stagger: this row tile walks its k range starting rot steps in, wrapping around */  \
@@ -352,11 +397,12 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
             sc32c[rw][j] = a.absmax[min(row_, a.m - 1)]; /* rows past m are never stored */    \
         }                                                                                      \
         krot = KRot{rot * kStepK, seg_hi * kStepK, nsteps * kStepK};                           \
-        x_stage_load<TT, XB>(xst, xg, 0, nthreads, tid, x_pieces, tok0, sb * kStepK, a.n, a.k, krot); \
+        x_stage_load<TT, XB>(xst, xg, 0, nthreads, tid, x_pieces, tok0, sb * kStepK, n_tok, a.k, krot); \
     }
 
     int t = t_begin;
     const float code_lane = a.code[lane & 15];
+    TUNA_SKIP_EMPTY(t)
     if (t < t_end) TUNA_TILE_FETCH(t)
     TUNA_MARK(1)
 
@@ -439,12 +485,13 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                 for (int tt = 0; tt < TT; ++tt) acc[rw][j][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
         const int cur_row_tile = row_tile, cur_part = part, cur_sb = sb;
+        const int cur_tok0 = tok0, cur_ntok = n_tok, cur_out_row0 = out_row0;
         const int n_chunks = (nsteps + a.chunk_steps - 1) >> a.chunk_log2;
         int it = 0;  // this wave's next iteration (multiple of U)
 
         // the work area is free again once every wave has left the previous tile's epilogue
         __syncthreads();
-        if (n_chunks > 0) x_stage_store<TT, XB>(xst, work, 0, nthreads, tid, x_pieces, tok0, cur_sb * kStepK, a.n, a.k, krot);
+        if (n_chunks > 0) x_stage_store<TT, XB>(xst, work, 0, nthreads, tid, x_pieces, cur_tok0, cur_sb * kStepK, cur_ntok, a.k, krot);
         __syncthreads();
         TUNA_MARK(3)
 
@@ -461,10 +508,10 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                 // that after the group exactly U*RW younger loads are in flight and the wait before
                 // the LDS write below is an exact vmcnt, not a drain of the weight ring.
                 const int kbase = (cur_sb + (c + 1) * a.chunk_steps) * kStepK;
-                x_stage_load<TT, XB>(xst, xg, 0, nthreads, tid, x_pieces, tok0, kbase, a.n, a.k, krot);
+                x_stage_load<TT, XB>(xst, xg, 0, nthreads, tid, x_pieces, cur_tok0, kbase, cur_ntok, a.k, krot);
                 TUNA_GROUP()
                 __syncthreads();  // every wave is done reading chunk c
-                x_stage_store<TT, XB>(xst, work, 0, nthreads, tid, x_pieces, tok0, kbase, a.n, a.k, krot);
+                x_stage_store<TT, XB>(xst, work, 0, nthreads, tid, x_pieces, cur_tok0, kbase, cur_ntok, a.k, krot);
                 __syncthreads();
             } else {
                 const int it_end = min(it_chunk0 + ipc, n_it);
@@ -499,6 +546,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 
         // ---- next tile: get its loads going before this tile's reduction and store ---------
         t = t_next;
+        TUNA_SKIP_EMPTY(t)
         if (t < t_end) TUNA_TILE_FETCH(t)
 
         // ---- workgroup reduction and store ---------------------------------------------------
@@ -558,7 +606,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
             // them: two 16-byte stores per 64-row group, no LDS, no barrier.
 #pragma unroll
             for (int tt = 0; tt < TT; ++tt) {
-                const int tok = tok0 + tt * 16 + (lane_e & 15);
+                const int tok = cur_tok0 + tt * 16 + (lane_e & 15);
 #pragma unroll
                 for (int rw = 0; rw < RW; ++rw) {
                     const int rb = cur_row_tile * rows_wg + wm_e * (RW * kRowsPerLoad) + rw * 64 + (lane_e >> 4) * 16;
@@ -570,9 +618,9 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                             lo[v * 4 + j] = (f16)acc[rw][j][tt][v];
                             hi[v * 4 + j] = (f16)acc[rw][j][tt][v + 2];
                         }
-                    f16 *dst = outp + (size_t)tok * a.m + rb;
-                    if (tok < a.n && rb + 8 <= a.m) *reinterpret_cast<f16x8 *>(dst) = lo;
-                    if (tok < a.n && rb + 16 <= a.m) *reinterpret_cast<f16x8 *>(dst + 8) = hi;
+                    f16 *dst = outp + (size_t)tok * out_ld + (rb - cur_out_row0);
+                    if (tok < cur_ntok && rb + 8 <= a.m) *reinterpret_cast<f16x8 *>(dst) = lo;
+                    if (tok < cur_ntok && rb + 16 <= a.m) *reinterpret_cast<f16x8 *>(dst + 8) = hi;
                 }
             }
             ++tile_iter;
@@ -594,7 +642,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                             acc[rw][j][tt];
                     __syncthreads();
                     TUNA_MARK(12)
-                    sum_planes_any<4>(a.wk_log2, buf, plane_floats, wm_e, wk_e, lane_e, o, 0);
+                    sum_planes_any<4, RED_LIM>(a.wk_log2, buf, plane_floats, wm_e, wk_e, lane_e, o, 0);
                     TUNA_MARK(13)
                 } else {
 #pragma unroll
@@ -602,7 +650,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                         float *buf = redf + ((rw * TT + tt) * 4 + j) % 2 * plane_floats;
                         reinterpret_cast<f32x4 *>(buf)[(size_t)(wm_e * a.waves_k + wk_e) * 64 + lane_e] = acc[rw][j][tt];
                         __syncthreads();
-                        sum_planes_any<1>(a.wk_log2, buf, plane_floats, wm_e, wk_e, lane_e, o, j);
+                        sum_planes_any<1, RED_LIM>(a.wk_log2, buf, plane_floats, wm_e, wk_e, lane_e, o, j);
                     }
                 }
 #pragma unroll
@@ -611,11 +659,11 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                     if (f >= 256) continue;
                     if (!partial) {
                         const int l = f >> 2, v = f & 3;
-                        const int tok = tok0 + tt * 16 + (l & 15);
+                        const int tok = cur_tok0 + tt * 16 + (l & 15);
                         const int row = cur_row_tile * rows_wg + wm_e * (RW * kRowsPerLoad) + rw * 64 + (l >> 4) * 16 + v * 4;
-                        if (tok < a.n && row + 4 <= a.m) {
+                        if (tok < cur_ntok && row + 4 <= a.m) {
                             f16x4 h = {(f16)o[i][0], (f16)o[i][1], (f16)o[i][2], (f16)o[i][3]};
-                            *reinterpret_cast<f16x4 *>(outp + (size_t)tok * a.m + row) = h;
+                            *reinterpret_cast<f16x4 *>(outp + (size_t)tok * out_ld + (row - cur_out_row0)) = h;
                         }
                     } else {
                         float *dst = mine + ((size_t)(rw * TT + tt) * 256 + f) * 4;
@@ -650,13 +698,14 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                         const int f = ((i << a.wk_log2) + wk_e) * 64 + lane_e;
                         if (f >= 256) break;
                         const float *src = src0 + (size_t)wm_e * (NACC * 256) + ((size_t)rt * 256 + f) * 4;
-                        // four contributors per round trip (indices are clamped so that the loads
+                        // several contributors per round trip (indices are clamped so that the loads
                         // are unconditional and all in flight together); summed in k order
                         float s4[4] = {0.f, 0.f, 0.f, 0.f};
-                        for (unsigned sp0 = 0; sp0 < n_contrib; sp0 += 4) {
-                            float pv[4][4];
+                        constexpr unsigned FB = 4;
+                        for (unsigned sp0 = 0; sp0 < n_contrib; sp0 += FB) {
+                            float pv[FB][4];
 #pragma unroll
-                            for (unsigned b = 0; b < 4; ++b) {
+                            for (unsigned b = 0; b < FB; ++b) {
                                 const unsigned sp = min(sp0 + b, n_contrib - 1u);
                                 const float *sps = src + (size_t)sp * src_stride - (sp ? src_adj : 0);
 #pragma unroll
@@ -664,7 +713,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                                     pv[b][j] = __hip_atomic_load(sps + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                             }
 #pragma unroll
-                            for (unsigned b = 0; b < 4; ++b)
+                            for (unsigned b = 0; b < FB; ++b)
                                 if (sp0 + b < n_contrib) {
 #pragma unroll
                                     for (int j = 0; j < 4; ++j) s4[j] += pv[b][j];
@@ -672,11 +721,11 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                         }
                         const int rw = rt / TT, tt = rt % TT;
                         const int l = f >> 2, v = f & 3;
-                        const int tok = tok0 + tt * 16 + (l & 15);
+                        const int tok = cur_tok0 + tt * 16 + (l & 15);
                         const int row = cur_row_tile * rows_wg + wm_e * (RW * kRowsPerLoad) + rw * 64 + (l >> 4) * 16 + v * 4;
-                        if (tok < a.n && row + 4 <= a.m) {
+                        if (tok < cur_ntok && row + 4 <= a.m) {
                             f16x4 h = {(f16)s4[0], (f16)s4[1], (f16)s4[2], (f16)s4[3]};
-                            *reinterpret_cast<f16x4 *>(outp + (size_t)tok * a.m + row) = h;
+                            *reinterpret_cast<f16x4 *>(outp + (size_t)tok * out_ld + (row - cur_out_row0)) = h;
                         }
                     }
             }
@@ -688,6 +737,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 #undef TUNA_GROUP
 #undef TUNA_CONSUME
 #undef TUNA_TILE_FETCH
+#undef TUNA_SKIP_EMPTY
 #undef TUNA_TILE_SMALL_LOADS
 #undef TUNA_LOAD_STEP
 #undef TUNA_MARK

@@ -8,11 +8,12 @@ namespace tuna {
 typedef void (*GemmKernelFn)(const GemmArgs);
 
 struct Variant {
-    int rw, u, tt, dec, maxt, minw;
+    int rw, u, tt, dec, maxt, minw, grouped;
     GemmKernelFn fn;
 };
 
-#define V(RW, U, TT, DEC, MAXT, MINW) {RW, U, TT, DEC, MAXT, MINW, gemm_kernel<RW, U, TT, DEC, MAXT, MINW>}
+#define V(RW, U, TT, DEC, MAXT, MINW) {RW, U, TT, DEC, MAXT, MINW, 0, gemm_kernel<RW, U, TT, DEC, MAXT, MINW, false>}
+#define VG(RW, U, TT, DEC, MAXT, MINW) {RW, U, TT, DEC, MAXT, MINW, 1, gemm_kernel<RW, U, TT, DEC, MAXT, MINW, true>}
 #define G TUNA_DECODE_GEMM
 
 // Only variants whose main loop compiles without register spills are listed (a spill in the
@@ -32,25 +33,32 @@ static const Variant kVariants[] = {
     // dequant-rounding decode (correctness mode, not tuned)
     V(1, 2, 1, TUNA_DECODE_DEQUANT, 512, 2), V(1, 2, 2, TUNA_DECODE_DEQUANT, 512, 2),
     V(1, 2, 4, TUNA_DECODE_DEQUANT, 512, 2),
+    // grouped launches (per-group token lists): 64 rows per wave only
+    VG(1, 2, 1, G, 512, 2), VG(1, 2, 2, G, 512, 2), VG(1, 2, 4, G, 512, 2), VG(1, 4, 1, G, 512, 2), VG(1, 4, 2, G, 512, 2),
+    VG(1, 2, 1, G, 512, 4), VG(1, 4, 1, G, 512, 4), VG(1, 2, 1, G, 1024, 4), VG(1, 4, 1, G, 1024, 4),
+    VG(1, 2, 1, TUNA_DECODE_DEQUANT, 512, 2), VG(1, 2, 2, TUNA_DECODE_DEQUANT, 512, 2),
+    VG(1, 2, 4, TUNA_DECODE_DEQUANT, 512, 2),
 };
 #undef V
+#undef VG
 #undef G
 static constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
-static const Variant *find_variant(int rw, int u, int tt, int dec, int threads, int minw)
+static const Variant *find_variant(int rw, int u, int tt, int dec, int threads, int minw, int grouped)
 {
     const int maxt = threads <= 512 ? 512 : 1024;
     if (maxt == 1024) minw = 4;
     for (int i = 0; i < kNumVariants; ++i) {
         const Variant &v = kVariants[i];
-        if (v.rw == rw && v.u == u && v.tt == tt && v.dec == dec && v.maxt == maxt && v.minw == minw) return &v;
+        if (v.rw == rw && v.u == u && v.tt == tt && v.dec == dec && v.maxt == maxt && v.minw == minw && v.grouped == grouped)
+            return &v;
     }
     return nullptr;
 }
 
-bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves)
+bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves, int grouped)
 {
-    return find_variant(rw, prefetch, token_tiles, decode, threads, min_waves) != nullptr;
+    return find_variant(rw, prefetch, token_tiles, decode, threads, min_waves, grouped) != nullptr;
 }
 
 // Dynamic LDS above 64 KB needs a one-time opt-in per kernel and device.
@@ -60,7 +68,8 @@ static int g_cu_count[16];
 
 hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
 {
-    const Variant *v = find_variant(plan.rw, plan.prefetch, plan.token_tiles, plan.decode, plan.threads, plan.min_waves);
+    const Variant *v = find_variant(plan.rw, plan.prefetch, plan.token_tiles, plan.decode, plan.threads, plan.min_waves,
+                                    plan.args.group_rows ? 1 : 0);
     if (!v) return hipErrorInvalidConfiguration;
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);

@@ -17,6 +17,7 @@ constexpr int kLdsLimit = 160 * 1024;
 constexpr int kStepK = 32;          // k per MFMA step (v_mfma_f32_16x16x32_f16)
 constexpr int kRowsPerLoad = 64;    // weight rows covered by one 128-bit load per lane
 constexpr int kMaxThreads = 1024;
+constexpr int kMaxGroups = 64;      // experts per grouped launch (their token offsets travel as kernel arguments)
 constexpr int kMaxCus = 256;        // compute units of the largest gfx950 part: bounds the persistent grid
 
 // Everything a GEMM launch needs, filled by the host from a tuna_gemm_config.
@@ -46,6 +47,13 @@ struct GemmArgs {
     int unit_log2;        // log2(k-steps per unit), a unit being what the split is made of
     int units_per_tile;   // ceil(steps_total / unit)
     int units_total;      // row_tiles * units_per_tile; (units_total + 1) * gridDim.x < 2^31
+    // grouped (mixture-of-experts) launches: the weight rows are n_groups stacked matrices of
+    // group_rows rows each; group e multiplies only the activation rows tok_off[e] ..
+    // tok_off[e+1]-1 and writes out[token, row - e*group_rows] (leading dimension group_rows).
+    // group_rows == 0: one dense GEMM.  Row tiles never straddle groups.
+    int group_rows;
+    int n_groups;
+    int tok_off[kMaxGroups + 1];
 #ifdef TUNA_TRACE
     unsigned long long *trace;  // development builds only: 16 timestamps per workgroup
 #endif
@@ -113,7 +121,7 @@ struct GemmPlan {
 
 // gemm_kernel.hip
 hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream);
-bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves);
+bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves, int grouped);
 
 // dequant_kernel.hip
 hipError_t launch_dequant(const uint8_t *q, const float *absmax, const float *code, void *out,

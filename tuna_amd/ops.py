@@ -66,6 +66,37 @@ def matmul(x, q, s, c, o, m: int, n: int, k: int, config: GemmConfig = None,
     _lib.check(rc)
 
 
+def matmul_grouped(x, q, s, c, o, m_group: int, n_groups: int, k: int, token_offsets, config: GemmConfig = None,
+                   decode_mode: int = _lib.DECODE_GEMM) -> None:
+    """Grouped GEMM (mixture of experts): o[t, :] = x[t, :] @ decode(W_e)^T for the tokens t of
+    group e, token_offsets[e] <= t < token_offsets[e+1] (tuna_matmul_grouped).
+
+    x fp16 [n_total, k], rows sorted by group; q uint8 [n_groups*m_group/8, k/8, 32] and s fp32
+    [n_groups*m_group]: the groups' weights stacked along m; o fp16 [n_total, m_group];
+    token_offsets: n_groups+1 non-decreasing host ints.  Groups without tokens cost nothing.
+    """
+    m_group, n_groups, k = int(m_group), int(n_groups), int(k)
+    offs = [int(v) for v in token_offsets]
+    if len(offs) != n_groups + 1:
+        raise ValueError(f"token_offsets needs {n_groups + 1} entries, got {len(offs)}")
+    n_total = offs[-1]
+    m = m_group * n_groups
+    _require(x, "x", torch.float16, n_total * k)
+    _require(q, "q", torch.uint8, m * k // 2)
+    _require(s, "s", torch.float32, m)
+    _require(c, "c", torch.float32, 16)
+    _require(o, "o", torch.float16, n_total * m_group)
+    for name, t in (("q", q), ("s", s), ("c", c), ("o", o)):
+        if t.device != x.device:
+            raise ValueError(f"{name} is on {t.device}, x on {x.device}")
+    arr = (ctypes.c_int * (n_groups + 1))(*offs)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().tuna_matmul_grouped(q.data_ptr(), x.data_ptr(), c.data_ptr(), s.data_ptr(), o.data_ptr(), m_group,
+                                            n_groups, k, arr, ctypes.byref(config) if config is not None else None,
+                                            int(decode_mode), _stream(x.device))
+    _lib.check(rc)
+
+
 def dequant(q, absmax, codebook, o, m: int, k: int, decode_mode: int = _lib.DECODE_DEQUANT) -> None:
     """o[m, k] = decode(q, codebook, absmax) as fp16  (extension.cpp:40-49)."""
     m, k = int(m), int(k)
