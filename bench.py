@@ -239,6 +239,33 @@ def main():
             torch.cuda.empty_cache()
         line["dequant"] = deq
 
+    if not args.no_shapes:
+        # Mixtral gate+up with a router: 16 tokens x top-2 = 32 (token, expert) rows spread over the 8
+        # experts; each expert multiplies only its own rows (grouped GEMM, one launch).  "dense" is
+        # the reference's all-experts-on-all-tokens reading of the same weights.
+        from tuna_amd.quantize import nf4_codebook
+
+        gm, gk = 28672, 4096
+        sets = [synth.make_weights_torch(8 * gm, gk, 4000 + i, dev) for i in range(3)]
+        moe = {}
+        for label, counts in (("balanced_4_per_expert", [4] * 8), ("skewed", [9, 0, 6, 1, 0, 11, 5, 0]),
+                              ("two_experts", [16, 0, 0, 0, 16, 0, 0, 0])):
+            offs = [0]
+            for cnt in counts:
+                offs.append(offs[-1] + cnt)
+            xg = synth.make_x_torch(offs[-1], gk, 7, dev)
+            og = torch.empty((offs[-1], gm), dtype=torch.float16, device=dev)
+            ms = ops.time_matmul_grouped([s_[0] for s_ in sets], [s_[1] for s_ in sets], xg, nf4_codebook(dev), og, gm, 8, gk,
+                                         offs, warmup=10, iters=100, use_graph=True)
+            us = ms * 10.0
+            active = sum(1 for cnt in counts if cnt)
+            moe[label] = {"tokens_per_expert": counts, "us": round(us, 2), "active_experts": active,
+                          "packed_bytes_read": active * gm * gk // 2,
+                          "gbs": round(active * gm * gk / 2 / (us * 1e-6) / 1e9, 1)}
+        del sets
+        torch.cuda.empty_cache()
+        line["mixtral_gate_up_routed"] = moe
+
     if not args.no_sweeps:
         sweeps = {}
         # Llama-70B decoder layer x 80 layers, distinct seeded weights per layer (34.2 GB resident)

@@ -158,6 +158,12 @@ int tuna_time_matmul(const void *const *q_list, const void *const *absmax_list, 
                      const void *x, const void *code, void *out, int m, int n, int k,
                      const tuna_gemm_config *cfg, int decode_mode, int warmup, int iters,
                      int use_graph, void *stream, float *elapsed_ms);
+/* Same protocol for the grouped GEMM. */
+int tuna_time_matmul_grouped(const void *const *q_list, const void *const *absmax_list, int n_sets,
+                             const void *x, const void *code, void *out, int m_group, int n_groups,
+                             int k, const int32_t *token_offsets, const tuna_gemm_config *cfg,
+                             int decode_mode, int warmup, int iters, int use_graph, void *stream,
+                             float *elapsed_ms);
 /* Same protocol for the dequant kernel. */
 int tuna_time_dequant(const void *const *q_list, const void *const *absmax_list, int n_sets,
                       const void *code, void *out, int m, int k, int warmup, int iters,

@@ -186,31 +186,63 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     return TUNA_OK;
 }
 
-// A config for shapes the tuned table does not cover: 8-wave workgroups, enough
-// workgroups along k to occupy the 256 CUs, x staged 1024 k at a time.
+// A config for shapes the tuned table does not cover, following what the tuner finds on the
+// tuned shapes: many rows -> wide row tiles without any k split (accumulators stored straight
+// from registers); few rows -> one 64-row group per workgroup, 8 waves along k and enough
+// workgroups along k to occupy the CUs.  Rings of 2 k-steps: those variants never spill.
 static tuna_gemm_config derive_config(int m, int n, int k)
 {
     tuna_gemm_config c;
-    c.token_tiles = n <= 16 ? 1 : (n <= 32 ? 2 : 4);
+    c.token_tiles = n <= 16 ? 1 : 2;  // more tokens loop over gridDim.y (the 4-tile variants spill)
     c.rows_per_wave = 64;
-    c.waves_m = 2;
-    c.waves_k = 4;
-    c.prefetch = c.token_tiles == 4 ? 2 : 4;
-    c.xcd_swizzle = 0;
+    c.prefetch = 2;
+    c.xcd_swizzle = 1;
     c.k_stagger = 1;
     const int steps = ceil_div(k, kStepK);
+    const int groups64 = ceil_div(m, kRowsPerLoad);
+    if (groups64 >= 2048) {
+        c.waves_m = 8, c.waves_k = 1;
+    } else if (groups64 >= 512) {
+        c.waves_m = 4, c.waves_k = 4;
+    } else if (groups64 >= 256) {
+        c.waves_m = 2, c.waves_k = 8;
+    } else {
+        c.waves_m = 1, c.waves_k = 8;
+    }
+    if (c.token_tiles > 1 && c.waves_m * c.waves_k > 8) c.waves_k /= 2;  // 16-wave variants exist for one token tile only
     const int row_tiles = ceil_div(m, c.rows_per_wave * c.waves_m);
     const int group = c.waves_k * c.prefetch;  // k-steps one workgroup consumes per ring turn
-    int split = (512 + row_tiles / 2) / row_tiles;
-    const int max_split = steps / group > 0 ? steps / group : 1;
+    const int threads = c.waves_m * c.waves_k * 64;
+    auto set_chunk = [&](int sps) {
+        // x chunk: as long as the staging allows (4 pieces per thread), at most 1024 k, no longer than the split
+        // ... and, with more row tiles than CUs, short enough (16 KB) for two workgroups to share a CU
+        const int cap_k = (row_tiles > kMaxCus && threads <= 512) ? 512 / c.token_tiles : 1024;
+        int chunk_steps = group;  // power of two
+        while (chunk_steps < sps && chunk_steps * 2 * kStepK * c.token_tiles <= 2 * threads && chunk_steps * 2 * kStepK <= cap_k)
+            chunk_steps *= 2;
+        c.x_chunk = chunk_steps * kStepK;
+    };
+    // k split.  More row tiles than workgroup slots: none.  Otherwise the largest split that still
+    // fits one round of tiles, if that fills at least half of the slots (measured: a half-empty
+    // round of whole tiles beats the alternative); if no such split exists the k ranges are divided
+    // evenly instead (balanced split), which costs a partial-sum epilogue in every workgroup but
+    // leaves no CU idle.
+    const int max_split = steps / (2 * group) > 0 ? steps / (2 * group) : 1;  // at least two ring turns per workgroup
+    c.split_k = 1;
+    set_chunk(steps);
+    GemmPlan plan;
+    if (plan_gemm(m, n, k, c, TUNA_DECODE_GEMM, &plan) != TUNA_OK) return c;
+    const int slots = kMaxCus * plan.wgs_per_cu;
+    if (row_tiles >= slots) return c;
+    int split = slots / row_tiles;
     if (split > max_split) split = max_split;
     if (split < 1) split = 1;
-    c.split_k = split;
-    const int sps = ceil_div(steps, split);
-    int chunk_steps = group;                                 // power of two
-    const int cap = 16 / c.token_tiles > group ? 16 / c.token_tiles : group;  // <= 16 KB of x per chunk
-    while (chunk_steps < sps && chunk_steps * 2 <= cap) chunk_steps *= 2;
-    c.x_chunk = chunk_steps * kStepK;
+    if ((double)row_tiles * split >= 0.5 * slots) {
+        c.split_k = split;
+        set_chunk(ceil_div(steps, split));
+    } else if (steps >= 2 * group) {
+        c.split_k = 0;
+    }
     return c;
 }
 
@@ -370,43 +402,49 @@ static int matmul_grouped_impl(const void *q, const void *x, const void *code, c
     const int m = m_group * n_groups;
     if ((rc = check_shape(m, n_total > 0 ? n_total : 1, k))) return rc;
     if (m_group % kRowsPerLoad) return fail(TUNA_ERR_UNSUPPORTED, "m_group=%d must be a multiple of %d", m_group, kRowsPerLoad);
+    if ((unsigned long long)m * (unsigned long long)k / 2 >= (1ull << 32))
+        return fail(TUNA_ERR_UNSUPPORTED, "packed weights of %llu bytes exceed the kernel's 32-bit offsets",
+                    (unsigned long long)m * (unsigned long long)k / 2);
     if (max_tok == 0) return TUNA_OK;  // no group has a token: nothing to compute, nothing to write
     if ((rc = check_ptr(q, "q", 16)) || (rc = check_ptr(x, "x", 16)) || (rc = check_ptr(code, "code", 4)) ||
         (rc = check_ptr(absmax, "absmax", 4)) || (rc = check_ptr(out, "out", 16)))
         return rc;
+    // Only groups with tokens are walked: the launch is planned for their rows alone.
+    int n_active = 0;
+    unsigned char act[kMaxGroups];
+    for (int e = 0; e < n_groups; ++e)
+        if (offsets[e + 1] > offsets[e]) act[n_active++] = (unsigned char)e;
+    const int m_active = m_group * n_active;
     tuna_gemm_config c;
     if (cfg) c = *cfg;
     else {
-        select_config(m, max_tok, k, &c, nullptr);
+        select_config(m_active, max_tok, k, &c, nullptr);
         // the grouped kernels exist for 64 rows per wave and rings of 2 or 4 k-steps
         c.rows_per_wave = kRowsPerLoad;
         if (c.prefetch > 4) c.prefetch = 4;
         // row tiles must not straddle groups: shrink the workgroup's row count until it divides m_group
-        while (m_group % (c.rows_per_wave * c.waves_m)) {
-            if (c.rows_per_wave > kRowsPerLoad) c.rows_per_wave /= 2;
-            else --c.waves_m;
-        }
-        const int x_cap = (c.prefetch == 8 ? 4 : 2) * c.waves_m * c.waves_k * 64;
+        while (m_group % (c.rows_per_wave * c.waves_m)) --c.waves_m;
+        const int x_cap = 2 * c.waves_m * c.waves_k * 64;
         while (c.x_chunk * c.token_tiles > x_cap && c.x_chunk / 2 >= kStepK * c.waves_k * c.prefetch) c.x_chunk /= 2;
-        if (decode != TUNA_DECODE_GEMM) {
-            c.rows_per_wave = 64;
-            c.prefetch = 2;
-        }
+        if (decode != TUNA_DECODE_GEMM) c.prefetch = 2;
     }
     if (m_group % (c.rows_per_wave * c.waves_m))
         return fail(TUNA_ERR_UNSUPPORTED, "rows per workgroup (%d) must divide m_group=%d", c.rows_per_wave * c.waves_m, m_group);
     GemmPlan plan;
-    if ((rc = plan_gemm(m, max_tok, k, c, decode, &plan, 1))) return rc;
+    if ((rc = plan_gemm(m_active, max_tok, k, c, decode, &plan, 1))) return rc;
     GemmArgs &a = plan.args;
     a.q = static_cast<const uint8_t *>(q);
     a.x = x;
     a.code = static_cast<const float *>(code);
     a.absmax = static_cast<const float *>(absmax);
     a.out = out;
+    a.m = m;  // bounds of q and absmax: all groups
     a.n = n_total;
     a.group_rows = m_group;
     a.n_groups = n_groups;
+    a.tiles_per_group = m_group / (c.rows_per_wave * c.waves_m);
     for (int e = 0; e <= n_groups; ++e) a.tok_off[e] = offsets[e];
+    for (int e = 0; e < n_active; ++e) a.act[e] = act[e];
     if (plan.ws_bytes) {
         Workspace w;
         if ((rc = get_workspace(stream, plan.ws_bytes, plan.n_counters, &w))) return rc;
@@ -678,6 +716,19 @@ TUNA_EXPORT int tuna_time_matmul(const void *const *q_list, const void *const *a
     if (!q_list || !absmax_list) return fail(TUNA_ERR_INVALID_ARG, "q_list / absmax_list is null");
     auto launch = [&](int set, hipStream_t s) {
         return matmul_impl(q_list[set], x, code, absmax_list[set], out, m, n, k, cfg, decode_mode, s);
+    };
+    return time_loop(launch, n_sets, warmup, iters, use_graph, static_cast<hipStream_t>(stream), elapsed_ms);
+}
+
+TUNA_EXPORT int tuna_time_matmul_grouped(const void *const *q_list, const void *const *absmax_list, int n_sets, const void *x,
+                                         const void *code, void *out, int m_group, int n_groups, int k,
+                                         const int32_t *token_offsets, const tuna_gemm_config *cfg, int decode_mode,
+                                         int warmup, int iters, int use_graph, void *stream, float *elapsed_ms)
+{
+    if (!q_list || !absmax_list) return fail(TUNA_ERR_INVALID_ARG, "q_list / absmax_list is null");
+    auto launch = [&](int set, hipStream_t s) {
+        return matmul_grouped_impl(q_list[set], x, code, absmax_list[set], out, m_group, n_groups, k, token_offsets, cfg,
+                                   decode_mode, s);
     };
     return time_loop(launch, n_sets, warmup, iters, use_graph, static_cast<hipStream_t>(stream), elapsed_ms);
 }

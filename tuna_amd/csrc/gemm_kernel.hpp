@@ -303,7 +303,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     }
     // state of the tile being fetched / computed
     int row_tile = 0, part = -1, sb = 0, nsteps = 0, n_it = 0, s_first = 0, t_next = 0;
-    int seg_hi = 0, s_clamp = 0, rot = 0;
+    int seg_hi = 0, s_clamp = 0, rot = 0, row_base = 0;
     uint32_t lb[RW], lb_last[RW];
     u32x4 wq[U][RW];
     constexpr int XB = U == 8 ? 8 : 4;
@@ -337,7 +337,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                 rt_ = (t) / a.split_k;                                                         \
                 nx_ = (t) + n_wg;                                                              \
             }                                                                                  \
-            const int e_ = (rt_ * rows_wg) / a.group_rows;                                     \
+            const int e_ = a.act[rt_ / a.tiles_per_group];                                     \
             if (a.tok_off[e_] + (int)blockIdx.y * (TT * 16) < a.tok_off[e_ + 1]) break;        \
             (t) = nx_;                                                                         \
         }                                                                                      \
@@ -364,13 +364,17 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
             if (a.split_k == 1) part = -1;                                                     \
             t_next = (t) + n_wg;                                                               \
         }                                                                                      \
-        const int row0_ = row_tile * rows_wg + wm * (RW * kRowsPerLoad);                       \
+        row_base = row_tile * rows_wg;                                                         \
         if constexpr (GRP) {                                                                    \
-            const int e_ = (row_tile * rows_wg) / a.group_rows;                                \
+            /* row tiles count over the groups that have tokens only (a.act lists them) */     \
+            const int slot_ = row_tile / a.tiles_per_group;                                    \
+            const int e_ = a.act[slot_];                                                       \
             tok0 = a.tok_off[e_] + (int)blockIdx.y * (TT * 16);                                \
             n_tok = a.tok_off[e_ + 1];                                                         \
             out_row0 = e_ * a.group_rows;                                                      \
+            row_base = out_row0 + (row_tile - slot_ * a.tiles_per_group) * rows_wg;            \
         }                                                                                      \
+        const int row0_ = row_base + wm * (RW * kRowsPerLoad);                                 \
         n_it = nsteps > wk ? (nsteps - wk + a.waves_k - 1) >> a.wk_log2 : 0;                   \
         s_first = sb + wk;                                                                     \
         /* stagger: this row tile walks its k range starting rot steps in, wrapping around */  \
@@ -390,7 +394,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     // The small operands of a tile: row scales and the first x chunk (mostly L2 hits).
 #define TUNA_TILE_SMALL_LOADS()                                                                 \
     {                                                                                          \
-        const int row0_ = row_tile * rows_wg + wm * (RW * kRowsPerLoad);                       \
+        const int row0_ = row_base + wm * (RW * kRowsPerLoad);                                 \
         _Pragma("unroll") for (int rw = 0; rw < RW; ++rw) _Pragma("unroll") for (int j = 0; j < 4; ++j) \
         {                                                                                      \
             const int row_ = row0_ + rw * kRowsPerLoad + i16 * 4 + j;                          \
@@ -485,7 +489,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                 for (int tt = 0; tt < TT; ++tt) acc[rw][j][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
         const int cur_row_tile = row_tile, cur_part = part, cur_sb = sb;
-        const int cur_tok0 = tok0, cur_ntok = n_tok, cur_out_row0 = out_row0;
+        const int cur_tok0 = tok0, cur_ntok = n_tok, cur_out_row0 = out_row0, cur_row_base = row_base;
         const int n_chunks = (nsteps + a.chunk_steps - 1) >> a.chunk_log2;
         int it = 0;  // this wave's next iteration (multiple of U)
 
@@ -609,7 +613,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                 const int tok = cur_tok0 + tt * 16 + (lane_e & 15);
 #pragma unroll
                 for (int rw = 0; rw < RW; ++rw) {
-                    const int rb = cur_row_tile * rows_wg + wm_e * (RW * kRowsPerLoad) + rw * 64 + (lane_e >> 4) * 16;
+                    const int rb = cur_row_base + wm_e * (RW * kRowsPerLoad) + rw * 64 + (lane_e >> 4) * 16;
                     f16x8 lo, hi;
 #pragma unroll
                     for (int v = 0; v < 2; ++v)
@@ -660,7 +664,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                     if (!partial) {
                         const int l = f >> 2, v = f & 3;
                         const int tok = cur_tok0 + tt * 16 + (l & 15);
-                        const int row = cur_row_tile * rows_wg + wm_e * (RW * kRowsPerLoad) + rw * 64 + (l >> 4) * 16 + v * 4;
+                        const int row = cur_row_base + wm_e * (RW * kRowsPerLoad) + rw * 64 + (l >> 4) * 16 + v * 4;
                         if (tok < cur_ntok && row + 4 <= a.m) {
                             f16x4 h = {(f16)o[i][0], (f16)o[i][1], (f16)o[i][2], (f16)o[i][3]};
                             *reinterpret_cast<f16x4 *>(outp + (size_t)tok * out_ld + (row - cur_out_row0)) = h;
@@ -722,7 +726,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                         const int rw = rt / TT, tt = rt % TT;
                         const int l = f >> 2, v = f & 3;
                         const int tok = cur_tok0 + tt * 16 + (l & 15);
-                        const int row = cur_row_tile * rows_wg + wm_e * (RW * kRowsPerLoad) + rw * 64 + (l >> 4) * 16 + v * 4;
+                        const int row = cur_row_base + wm_e * (RW * kRowsPerLoad) + rw * 64 + (l >> 4) * 16 + v * 4;
                         if (tok < cur_ntok && row + 4 <= a.m) {
                             f16x4 h = {(f16)s4[0], (f16)s4[1], (f16)s4[2], (f16)s4[3]};
                             *reinterpret_cast<f16x4 *>(outp + (size_t)tok * out_ld + (row - cur_out_row0)) = h;

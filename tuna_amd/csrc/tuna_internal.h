@@ -51,9 +51,13 @@ struct GemmArgs {
     // group_rows rows each; group e multiplies only the activation rows tok_off[e] ..
     // tok_off[e+1]-1 and writes out[token, row - e*group_rows] (leading dimension group_rows).
     // group_rows == 0: one dense GEMM.  Row tiles never straddle groups.
+    // Row tiles count over the groups that have tokens: row tile r belongs to group
+    // act[r / tiles_per_group].
     int group_rows;
     int n_groups;
+    int tiles_per_group;
     int tok_off[kMaxGroups + 1];
+    unsigned char act[kMaxGroups];
 #ifdef TUNA_TRACE
     unsigned long long *trace;  // development builds only: 16 timestamps per workgroup
 #endif

@@ -198,6 +198,25 @@ def time_matmul(q_list, absmax_list, x, c, o, m, n, k, config=None, decode_mode=
     return ms.value
 
 
+
+def time_matmul_grouped(q_list, absmax_list, x, c, o, m_group, n_groups, k, token_offsets, config=None,
+                        decode_mode=_lib.DECODE_GEMM, warmup=10, iters=100, use_graph=False) -> float:
+    """Milliseconds for `iters` grouped GEMMs rotating over the weight sets
+    (tuna_time_matmul_grouped).  Synchronises."""
+    assert len(q_list) == len(absmax_list) and len(q_list) > 0
+    qp, _qk = _ptr_array(q_list)
+    ap, _ak = _ptr_array(absmax_list)
+    arr = (ctypes.c_int * (int(n_groups) + 1))(*[int(v) for v in token_offsets])
+    ms = ctypes.c_float(0)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().tuna_time_matmul_grouped(qp, ap, len(q_list), x.data_ptr(), c.data_ptr(), o.data_ptr(), int(m_group),
+                                                 int(n_groups), int(k), arr,
+                                                 ctypes.byref(config) if config is not None else None, int(decode_mode),
+                                                 int(warmup), int(iters), int(bool(use_graph)), _stream(x.device),
+                                                 ctypes.byref(ms))
+    _lib.check(rc)
+    return ms.value
+
 def time_dequant(q_list, absmax_list, c, o, m, k, warmup=5, iters=20) -> float:
     qp, _qk = _ptr_array(q_list)
     ap, _ak = _ptr_array(absmax_list)
