@@ -323,3 +323,23 @@ def test_gpu_parity_config_families_are_valid_configs():
     for kw in mod.CONFIGS:
         for shape in ((1024, 16, 2048), (520, 37, 1096)):
             ops.validate_config(*shape, mod.cfg(**kw))
+
+
+def test_grouped_gemm_argument_checks_need_no_device():
+    """tuna_matmul_grouped validates the group description on the host before any HIP call."""
+    from tuna_amd import _lib
+
+    L = _lib.lib()
+
+    def call(m_group, n_groups, k, offsets):
+        arr = (ctypes.c_int * len(offsets))(*offsets)
+        return L.tuna_matmul_grouped(None, None, None, None, None, m_group, n_groups, k, arr, None, 1, None)
+
+    assert call(256, 0, 256, [0]) == 1                    # no groups
+    assert call(256, 65, 256, list(range(66))) == 1       # more than 64 groups
+    assert call(256, 2, 256, [0, 9, 8]) == 1              # decreasing offsets
+    assert call(256, 2, 256, [-1, 3, 8]) == 1             # negative start
+    assert call(100, 2, 256, [0, 4, 8]) in (1, 2)         # rows per group not a multiple of 64
+    assert b"" != L.tuna_last_error()
+    assert call(256, 2, 256, [0, 0, 0]) == 0              # no tokens anywhere: nothing to do, no pointer is touched
+    assert call(256, 2, 256, [0, 4, 8]) == 1              # tokens, but null pointers
