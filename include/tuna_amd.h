@@ -72,6 +72,10 @@ typedef struct tuna_gemm_config {
                               around (0: every row tile starts at the front).  When k*4 bytes,
                               the distance between block rows, is a large power of two, tiles
                               walking in lockstep keep hitting the same memory channels  */
+    int32_t lds_tile_rows; /* 0: streaming kernel (all fields above).  64, 128 or 256: the
+                              many-token kernel, which decodes a tile of this many weight rows
+                              once into LDS for token_tiles*16 (64, 128 or 256) tokens; only
+                              token_tiles and split_k (>= 1) are read besides                */
 } tuna_gemm_config;
 
 int tuna_version(void);

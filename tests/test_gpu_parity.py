@@ -426,3 +426,36 @@ def test_grouped_gemm_rejects_bad_arguments():
         ops.matmul_grouped(dx, dq, da, dc, out, 256, 2, 256, [0, 9, 8])         # decreasing offsets
     with pytest.raises(ops.TunaError):
         ops.matmul_grouped(dx, dq, da, dc, out, 256, 2, 256, [0, 4, 8], config=cfg(waves_m=8, waves_k=1, prefetch=2, x_chunk=64))  # 512-row tiles straddle groups
+
+
+# ----------------------------------------------------------------------------- many-token kernel (weights decoded once into LDS)
+TILED = [(256, 16), (256, 8), (256, 4), (128, 16), (128, 8), (64, 16), (64, 8)]   # (lds_tile_rows, token_tiles)
+
+
+@pytest.mark.parametrize("tile", TILED)
+@pytest.mark.parametrize("m,n,k,split", [(512, 256, 512, 1), (520, 300, 1096, 1), (256, 70, 2048, 4), (1024, 129, 200, 3)])
+def test_many_token_kernel_matches_oracle(tile, m, n, k, split):
+    """Every tile shape of the many-token kernel, ragged m / n / k and split-K, against the
+    oracle's float64 contraction of the same fp16 weights."""
+    rows, tt = tile
+    c = cfg(lds_tile_rows=rows, token_tiles=tt, split_k=split)
+    print(f"many-token tile {rows}x{16 * tt} m={m} n={n} k={k} split={split}", flush=True)
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=rows + tt + split)
+    got = run_gemm(q, x, code, absmax, m, n, k, config=c, prefill=float("nan"))
+    ref = O.gemm_f64(q, x, code, absmax, m, n, k, mode=O.D1)
+    e = rel_err(f16_bits_to_f64(got), ref)
+    assert e <= REL_TOL, e
+    again = run_gemm(q, x, code, absmax, m, n, k, config=c, prefill=float("nan"))
+    assert np.array_equal(got, again)
+
+
+def test_many_token_kernel_decode_readout_is_bit_exact():
+    """One-hot activations turn the GEMM into a readout of the decoded weights: bit-exact D1."""
+    m, k = 256, 256
+    q, _, code, absmax = make_inputs_np(m, 16, k, seed=9)
+    code = (np.random.default_rng(3).standard_normal(16)).astype(np.float32)
+    x = np.zeros((k, k), dtype=np.float16)
+    x[np.arange(k), np.arange(k)] = 1.0
+    got = run_gemm(q, x, code, absmax, m, k, k, config=cfg(lds_tile_rows=128, token_tiles=8), prefill=float("nan"))
+    want = O.dequant(q, absmax, code, m, k, mode=O.D1)          # [m, k] fp16 bits
+    assert np.array_equal(got.T, want)

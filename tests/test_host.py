@@ -110,8 +110,8 @@ def test_generator_output_and_its_refusal_of_inconsistent_entries(tmp_path):
           "4096_1_4096": dict(rows_per_wave=64, waves_m=1, waves_k=8, split_k=4, prefetch=2, x_chunk=1024,
                               token_tiles=1, xcd_swizzle=0, k_stagger=3)}
     text = mc.generate(pm)
-    assert "{4096, 16, 31, 4096, {64, 1, 8, 4, 2, 1024, 1, 1, 0}}" in text     # k_stagger defaults to 0
-    assert "{4096, 1, 15, 4096, {64, 1, 8, 4, 2, 1024, 1, 0, 3}}" in text
+    assert "{4096, 16, 31, 4096, {64, 1, 8, 4, 2, 1024, 1, 1, 0, 0}}" in text  # k_stagger, lds_tile_rows default to 0
+    assert "{4096, 1, 15, 4096, {64, 1, 8, 4, 2, 1024, 1, 0, 3, 0}}" in text
     assert "kConfigTableSize = 2" in text
     # the checked-in table is what the generator produces from the checked-in json
     with open(os.path.join(ROOT, "tuna_amd", "configs", "param_map.json")) as f:
@@ -323,6 +323,13 @@ def test_gpu_parity_config_families_are_valid_configs():
     for kw in mod.CONFIGS:
         for shape in ((1024, 16, 2048), (520, 37, 1096)):
             ops.validate_config(*shape, mod.cfg(**kw))
+    for rows, tt in mod.TILED:
+        for (m, n, k, split) in ((512, 256, 512, 1), (520, 300, 1096, 1), (256, 70, 2048, 4), (1024, 129, 200, 3)):
+            ops.validate_config(m, n, k, mod.cfg(lds_tile_rows=rows, token_tiles=tt, split_k=split))
+    with pytest.raises(ops.TunaError):
+        ops.validate_config(512, 256, 512, mod.cfg(lds_tile_rows=96, token_tiles=16))       # no such tile
+    with pytest.raises(ops.TunaError):
+        ops.validate_config(512, 256, 512, mod.cfg(lds_tile_rows=64, token_tiles=4))        # no 64 x 64 tile
 
 
 def test_grouped_gemm_argument_checks_need_no_device():

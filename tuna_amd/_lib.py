@@ -36,6 +36,7 @@ class GemmConfig(ctypes.Structure):
         ("token_tiles", ctypes.c_int32),
         ("xcd_swizzle", ctypes.c_int32),
         ("k_stagger", ctypes.c_int32),
+        ("lds_tile_rows", ctypes.c_int32),
     ]
 
     FIELDS = tuple(f for f, _ in _fields_)
@@ -45,7 +46,7 @@ class GemmConfig(ctypes.Structure):
 
     @classmethod
     def from_dict(cls, d):
-        return cls(**{f: int(d.get(f, 0) if f == "k_stagger" else d[f]) for f in cls.FIELDS})
+        return cls(**{f: int(d.get(f, 0) if f in ("k_stagger", "lds_tile_rows") else d[f]) for f in cls.FIELDS})
 
 
 # name -> (restype, argtypes); also the list of symbols the header declares

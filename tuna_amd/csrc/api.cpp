@@ -66,6 +66,7 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
                     (unsigned long long)m * (unsigned long long)k / 2);
     if (decode != TUNA_DECODE_GEMM && decode != TUNA_DECODE_DEQUANT)
         return fail(TUNA_ERR_INVALID_ARG, "decode_mode %d is neither TUNA_DECODE_GEMM nor TUNA_DECODE_DEQUANT", decode);
+    if (c.lds_tile_rows) return fail(TUNA_ERR_INVALID_ARG, "plan_gemm called with a many-token config");
     if (c.rows_per_wave != 64 && c.rows_per_wave != 128 && c.rows_per_wave != 256)
         return fail(TUNA_ERR_UNSUPPORTED, "rows_per_wave=%d (64, 128 or 256)", c.rows_per_wave);
     if (c.prefetch != 2 && c.prefetch != 4 && c.prefetch != 8)
@@ -186,6 +187,43 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     return TUNA_OK;
 }
 
+// Many-token kernel: checks and launch arguments for a config with lds_tile_rows != 0.
+struct TiledPlan {
+    TiledArgs args;
+    int tile_rows, tile_tokens;
+    size_t lds_bytes, ws_bytes, n_counters;
+};
+
+static int plan_tiled(int m, int n, int k, const tuna_gemm_config &c, int decode, TiledPlan *plan)
+{
+    int rc = check_shape(m, n, k);
+    if (rc) return rc;
+    if (decode != TUNA_DECODE_GEMM)
+        return fail(TUNA_ERR_UNSUPPORTED, "the many-token kernel implements TUNA_DECODE_GEMM only");
+    const int tile_tokens = 16 * c.token_tiles;
+    if (!tiled_variant_exists(c.lds_tile_rows, tile_tokens))
+        return fail(TUNA_ERR_UNSUPPORTED, "no many-token kernel for a %d x %d tile (rows x tokens)", c.lds_tile_rows, tile_tokens);
+    const int steps = ceil_div(k, 64);
+    if (c.split_k < 1 || c.split_k > steps)
+        return fail(TUNA_ERR_UNSUPPORTED, "split_k=%d must be in 1..%d for the many-token kernel", c.split_k, steps);
+    if (c.split_k > 65535 || ceil_div(n, tile_tokens) > 65535) return fail(TUNA_ERR_UNSUPPORTED, "grid too large");
+    memset(plan, 0, sizeof(*plan));
+    plan->tile_rows = c.lds_tile_rows;
+    plan->tile_tokens = tile_tokens;
+    plan->lds_bytes = tiled_lds_bytes(c.lds_tile_rows, tile_tokens);
+    const size_t tiles = (size_t)ceil_div(m, c.lds_tile_rows) * ceil_div(n, tile_tokens);
+    plan->ws_bytes = c.split_k > 1 ? tiles * c.split_k * (size_t)c.lds_tile_rows * tile_tokens * 4 : 0;
+    plan->n_counters = c.split_k > 1 ? tiles : 0;
+    TiledArgs &a = plan->args;
+    a.m = m;
+    a.n = n;
+    a.k = k;
+    a.steps_total = steps;
+    a.split_k = c.split_k;
+    a.steps_per_split = ceil_div(steps, c.split_k);
+    return TUNA_OK;
+}
+
 // A config for shapes the tuned table does not cover, following what the tuner finds on the
 // tuned shapes: many rows -> wide row tiles without any k split (accumulators stored straight
 // from registers); few rows -> one 64-row group per workgroup, 8 waves along k and enough
@@ -193,11 +231,27 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
 static tuna_gemm_config derive_config(int m, int n, int k)
 {
     tuna_gemm_config c;
+    if (n >= 128) {
+        // many tokens: the kernel that decodes each weight tile once into LDS; 128-token tiles,
+        // 256 rows (128 for few rows), k split until about one workgroup per CU
+        memset(&c, 0, sizeof(c));
+        c.rows_per_wave = 64, c.waves_m = 1, c.waves_k = 1, c.prefetch = 2, c.x_chunk = 64;
+        c.token_tiles = 8;
+        c.lds_tile_rows = m >= 16384 ? 256 : 128;
+        const long long tiles = (long long)ceil_div(m, c.lds_tile_rows) * ceil_div(n, 128);
+        const int steps64 = ceil_div(k, 64);
+        long long split = tiles >= 192 ? 1 : (kMaxCus + tiles / 2) / tiles;
+        if (split > steps64 / 8) split = steps64 / 8;
+        if (split < 1) split = 1;
+        c.split_k = (int)split;
+        return c;
+    }
     c.token_tiles = n <= 16 ? 1 : 2;  // more tokens loop over gridDim.y (the 4-tile variants spill)
     c.rows_per_wave = 64;
     c.prefetch = 2;
     c.xcd_swizzle = 1;
     c.k_stagger = 1;
+    c.lds_tile_rows = 0;
     const int steps = ceil_div(k, kStepK);
     const int groups64 = ceil_div(m, kRowsPerLoad);
     if (groups64 >= 2048) {
@@ -357,6 +411,24 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
             c.prefetch = 2;
         }
     }
+    if (c.lds_tile_rows) {
+        TiledPlan tp;
+        if ((rc = plan_tiled(m, n, k, c, decode, &tp))) return rc;
+        tp.args.q = static_cast<const uint8_t *>(q);
+        tp.args.x = x;
+        tp.args.code = static_cast<const float *>(code);
+        tp.args.absmax = static_cast<const float *>(absmax);
+        tp.args.out = out;
+        if (tp.ws_bytes) {
+            Workspace w;
+            if ((rc = get_workspace(stream, tp.ws_bytes, tp.n_counters, &w))) return rc;
+            tp.args.ws = w.ws;
+            tp.args.counters = w.counters;
+        }
+        hipError_t e = launch_gemm_tiled(tp.args, tp.tile_rows, tp.tile_tokens, stream);
+        if (e != hipSuccess) return hip_fail(e, "many-token gemm launch");
+        return TUNA_OK;
+    }
     GemmPlan plan;
     if ((rc = plan_gemm(m, n, k, c, decode, &plan))) return rc;
     plan.args.q = static_cast<const uint8_t *>(q);
@@ -419,6 +491,7 @@ static int matmul_grouped_impl(const void *q, const void *x, const void *code, c
     if (cfg) c = *cfg;
     else {
         select_config(m_active, max_tok, k, &c, nullptr);
+        if (c.lds_tile_rows) c = derive_config(m_active, 64, k);  // grouped launches use the streaming kernel
         // the grouped kernels exist for 64 rows per wave and rings of 2 or 4 k-steps
         c.rows_per_wave = kRowsPerLoad;
         if (c.prefetch > 4) c.prefetch = 4;
@@ -608,6 +681,10 @@ TUNA_EXPORT int tuna_select_config(int m, int n, int k, tuna_gemm_config *cfg, i
 TUNA_EXPORT int tuna_validate_config(int m, int n, int k, const tuna_gemm_config *cfg)
 {
     if (!cfg) return fail(TUNA_ERR_INVALID_ARG, "cfg is null");
+    if (cfg->lds_tile_rows) {
+        TiledPlan tp;
+        return plan_tiled(m, n, k, *cfg, TUNA_DECODE_GEMM, &tp);
+    }
     GemmPlan plan;
     return plan_gemm(m, n, k, *cfg, TUNA_DECODE_GEMM, &plan);
 }
@@ -616,6 +693,14 @@ TUNA_EXPORT int tuna_config_footprint(int m, int n, int k, const tuna_gemm_confi
                                       size_t *workspace_bytes)
 {
     if (!cfg) return fail(TUNA_ERR_INVALID_ARG, "cfg is null");
+    if (cfg->lds_tile_rows) {
+        TiledPlan tp;
+        int rc = plan_tiled(m, n, k, *cfg, TUNA_DECODE_GEMM, &tp);
+        if (rc) return rc;
+        if (lds_bytes) *lds_bytes = tp.lds_bytes;
+        if (workspace_bytes) *workspace_bytes = tp.ws_bytes;
+        return TUNA_OK;
+    }
     GemmPlan plan;
     int rc = plan_gemm(m, n, k, *cfg, TUNA_DECODE_GEMM, &plan);
     if (rc) return rc;

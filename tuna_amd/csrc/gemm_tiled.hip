@@ -1,0 +1,294 @@
+// FP16-activation x 4-bit-codebook-weight GEMM for MANY tokens (64 ... thousands) on gfx950.
+//
+//   out[n, m] = x[n, k] . W[m, k]^T,   W[r, c] = fp16(code[nib(r, c)]) *fp16 fp16(absmax[r])
+//
+// Counterpart of the reference's larger-n kernel configurations (kernel.cu:3037-3155 select
+// them by token bucket).  With many tokens the op is bound by the matrix cores and by the
+// decode, not by HBM, so unlike the streaming kernel (gemm_kernel.hpp: weights straight into
+// registers, every wave decodes what it multiplies) a weight is decoded ONCE per workgroup
+// tile and shared by all tokens of the tile through LDS:
+//
+//   * workgroup tile: BM = WM*TM*16 weight rows x BN = WN*TN*16 tokens, k in steps of 64;
+//     WM x WN waves, a wave owns TM x TN MFMA tiles (v_mfma_f32_16x16x32_f16, weights = A).
+//   * per k-step the 512 threads fetch BM x 64 packed weights (16 bytes per thread: 4
+//     consecutive rows x 8 k; 16 threads cover 256 contiguous bytes of a block row) and
+//     BN x 64 activations, two steps ahead, into registers;
+//   * decode through the same conflict-free byte-pair table as the streaming kernel
+//     (one v_perm_b32 + ds_read_b32 + v_pk_mul_f16 per two weights, bit-identical to
+//     kernel.cu:2178-2192), then one ds_write_b128 per decoded dword into the A tile;
+//   * A and X tiles are [row][64 k] fp16 = 128-byte rows whose eight 16-byte slots are
+//     XOR-swizzled with (row & 7): the decode writes, the activation writes and the
+//     ds_read_b128 fragment reads (8 lanes = 8 consecutive rows of one slot) all touch every
+//     bank exactly once - no padding, no bank conflicts;
+//   * fp32 accumulators stay in registers for the whole k range; a lane ends up with 4
+//     consecutive output features of one token per MFMA tile: 8-byte stores.
+#include "tuna_internal.h"
+
+namespace tuna {
+
+typedef _Float16 f16;
+typedef f16 f16x2 __attribute__((ext_vector_type(2)));
+typedef f16 f16x4 __attribute__((ext_vector_type(4)));
+typedef f16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) uint32_t lds_u32;
+
+constexpr int kTiledThreads = 512;
+constexpr int kTiledStepK = 64;
+
+template <int WM, int TM, int WN, int TN>
+__global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const TiledArgs a)
+{
+    static_assert(WM * WN * 64 == kTiledThreads, "8 waves");
+    constexpr int BM = WM * TM * 16;
+    constexpr int BN = WN * TN * 16;
+    constexpr int A_PIECES = BM * 2;                 // 16-byte packed pieces per k-step
+    constexpr int X_PER_THREAD = BN * 8 / kTiledThreads;  // 16-byte activation pieces per thread per k-step
+    static_assert(A_PIECES <= kTiledThreads && X_PER_THREAD >= 1, "tile shape");
+    extern __shared__ __align__(16) unsigned char smem[];
+    unsigned char *lut = smem;                       // byte-pair table at LDS address 0
+    unsigned char *a_tile = smem + kLutBytes;        // [BM][128 bytes]
+    unsigned char *x_tile = a_tile + BM * 128;       // [BN][128 bytes]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm_i = wave / WN, wn_i = wave % WN;
+    const int i16 = lane & 15, g = lane >> 4;
+    const uint32_t lane4 = (uint32_t)lane << 2;
+
+    const int row_base = blockIdx.x * BM;
+    const int tok_base = blockIdx.y * BN;
+    const int kb_total = a.k >> 3;
+    const int mb_last = (a.m >> 3) - 1;
+    const f16 *xg = reinterpret_cast<const f16 *>(a.x);
+
+    // ---- this thread's share of the loads ------------------------------------------------
+    // weights: piece tid = block row (tid / 16) of the tile, k-block (tid % 16) / 2 of the step,
+    // half tid % 2 (rows 4*half .. +3 of the block row)
+    const bool a_loader = tid < A_PIECES;
+    const int a_mbl = tid >> 4, a_kb = (tid & 15) >> 1, a_half = tid & 1;
+    const int a_mb = min((row_base >> 3) + a_mbl, mb_last);
+    const unsigned char *a_src = a.q + (size_t)a_mb * kb_total * 32 + a_half * 16;
+    const int a_row = a_mbl * 8 + a_half * 4;        // first of the 4 tile rows this thread decodes
+    f16x2 sc16[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const f16 h = (f16)a.absmax[min(row_base + a_row + j, a.m - 1)];
+        sc16[j] = f16x2{h, h};
+    }
+    // activations: piece p = tid + i*512: token p / 8 of the tile, 8-k slot p % 8 of the step
+    const f16 *x_src[X_PER_THREAD];
+    bool x_tok_ok[X_PER_THREAD];
+#pragma unroll
+    for (int i = 0; i < X_PER_THREAD; ++i) {
+        const int p = tid + i * kTiledThreads;
+        const int tok = tok_base + (p >> 3);
+        x_tok_ok[i] = tok < a.n;
+        x_src[i] = xg + (size_t)min(tok, a.n - 1) * a.k + (p & 7) * 8;
+    }
+
+    u32x4 wq[2];
+    u32x4 xr[2][X_PER_THREAD];
+    // Unconditional, clamped loads (exact s_waitcnt counts); what lies beyond k is zeroed in x.
+#define TUNA_TILED_LOAD(set, s)                                                                 \
+    {                                                                                          \
+        const int kb_ = min((s) * 8 + a_kb, kb_total - 1);                                     \
+        wq[set] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(a_src + (size_t)kb_ * 32)); \
+        _Pragma("unroll") for (int i = 0; i < X_PER_THREAD; ++i)                               \
+        {                                                                                      \
+            const int kk_ = min((s) * kTiledStepK, a.k - 8 - ((tid + i * kTiledThreads) & 7) * 8); \
+            xr[set][i] = *reinterpret_cast<const u32x4 *>(x_src[i] + kk_);                     \
+        }                                                                                      \
+    }
+
+    const int s0 = blockIdx.z * a.steps_per_split;
+    const int s1 = min(a.steps_total, s0 + a.steps_per_split);
+    TUNA_TILED_LOAD(0, min(s0, a.steps_total - 1))
+    TUNA_TILED_LOAD(1, min(s0 + 1, a.steps_total - 1))
+
+    // ---- decode table (as in the streaming kernel) ------------------------------------------
+    {
+        const int code_bits = (int)(uint32_t)__builtin_bit_cast(uint16_t, (f16)a.code[lane & 15]);
+#pragma unroll 4
+        for (int p = tid; p < kLutBytes / 16; p += kTiledThreads) {
+            const int e = p >> 4;
+            const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute((e >> 4) << 2, code_bits);
+            const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute((e & 15) << 2, code_bits);
+            const uint32_t v = hi | (lo << 16);
+            reinterpret_cast<u32x4 *>(lut)[p] = u32x4{v, v, v, v};
+        }
+    }
+
+    f32x4 acc[TM][TN];
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // fragment addresses: row (i16) of MFMA tile tm / tn, slot (kh*4 + g) ^ (row & 7)
+    const unsigned char *a_frag = a_tile + (wm_i * TM * 16 + i16) * 128;
+    const unsigned char *x_frag = x_tile + (wn_i * TN * 16 + i16) * 128;
+    const int sw = i16 & 7;
+
+    // One k-step: (barrier) decode + stage -> (refill registers two steps ahead) -> barrier -> MFMA
+#define TUNA_TILED_STEP(set, s)                                                                 \
+    {                                                                                          \
+        __syncthreads(); /* every wave has finished reading the previous step's tiles */       \
+        if (a_loader) {                                                                        \
+            _Pragma("unroll") for (int j = 0; j < 4; ++j)                                      \
+            {                                                                                  \
+                const uint32_t d_ = wq[set][j];                                                \
+                const uint32_t t0_ = *reinterpret_cast<const lds_u32 *>((uintptr_t)__builtin_amdgcn_perm(d_, lane4, 0x0c0c0400u)); \
+                const uint32_t t1_ = *reinterpret_cast<const lds_u32 *>((uintptr_t)__builtin_amdgcn_perm(d_, lane4, 0x0c0c0500u)); \
+                const uint32_t t2_ = *reinterpret_cast<const lds_u32 *>((uintptr_t)__builtin_amdgcn_perm(d_, lane4, 0x0c0c0600u)); \
+                const uint32_t t3_ = *reinterpret_cast<const lds_u32 *>((uintptr_t)__builtin_amdgcn_perm(d_, lane4, 0x0c0c0700u)); \
+                const f16x2 h0_ = __builtin_bit_cast(f16x2, t0_) * sc16[j], h1_ = __builtin_bit_cast(f16x2, t1_) * sc16[j]; \
+                const f16x2 h2_ = __builtin_bit_cast(f16x2, t2_) * sc16[j], h3_ = __builtin_bit_cast(f16x2, t3_) * sc16[j]; \
+                const f16x8 w_ = {h0_[0], h0_[1], h1_[0], h1_[1], h2_[0], h2_[1], h3_[0], h3_[1]}; \
+                const int r_ = a_row + j;                                                      \
+                *reinterpret_cast<f16x8 *>(a_tile + r_ * 128 + ((a_kb ^ (r_ & 7)) << 4)) = w_; \
+            }                                                                                  \
+        }                                                                                      \
+        _Pragma("unroll") for (int i = 0; i < X_PER_THREAD; ++i)                               \
+        {                                                                                      \
+            const int p_ = tid + i * kTiledThreads;                                            \
+            const int t_ = p_ >> 3, sl_ = p_ & 7;                                              \
+            const bool ok_ = x_tok_ok[i] && ((s) * kTiledStepK + sl_ * 8 < a.k);               \
+            *reinterpret_cast<u32x4 *>(x_tile + t_ * 128 + ((sl_ ^ (t_ & 7)) << 4)) = ok_ ? xr[set][i] : u32x4{0u, 0u, 0u, 0u}; \
+        }                                                                                      \
+        TUNA_TILED_LOAD(set, min((s) + 2, a.steps_total - 1))                                  \
+        __syncthreads();                                                                       \
+        _Pragma("unroll") for (int kh = 0; kh < 2; ++kh)                                       \
+        {                                                                                      \
+            const int slot_ = ((kh * 4 + g) ^ sw) << 4;                                        \
+            f16x8 bf_[TN];                                                                     \
+            _Pragma("unroll") for (int tn = 0; tn < TN; ++tn)                                  \
+                bf_[tn] = *reinterpret_cast<const f16x8 *>(x_frag + tn * (16 * 128) + slot_);  \
+            _Pragma("unroll") for (int tm = 0; tm < TM; ++tm)                                  \
+            {                                                                                  \
+                const f16x8 af_ = *reinterpret_cast<const f16x8 *>(a_frag + tm * (16 * 128) + slot_); \
+                _Pragma("unroll") for (int tn = 0; tn < TN; ++tn) acc[tm][tn] =                \
+                    __builtin_amdgcn_mfma_f32_16x16x32_f16(af_, bf_[tn], acc[tm][tn], 0, 0, 0); \
+            }                                                                                  \
+        }                                                                                      \
+    }
+
+    int s = s0;
+    for (; s + 1 < s1; s += 2) {
+        TUNA_TILED_STEP(0, s)
+        TUNA_TILED_STEP(1, s + 1)
+    }
+    if (s < s1) TUNA_TILED_STEP(0, s)
+#undef TUNA_TILED_STEP
+#undef TUNA_TILED_LOAD
+
+    // ---- epilogue -----------------------------------------------------------------------------
+    // acc[tm][tn][v] of lane l is weight row 4*(l/16) + v of MFMA tile tm, token l%16 of tile tn
+    f16 *outp = reinterpret_cast<f16 *>(a.out);
+    if (a.split_k == 1) {
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+            const int row = row_base + (wm_i * TM + tm) * 16 + g * 4;
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn) {
+                const int tok = tok_base + (wn_i * TN + tn) * 16 + i16;
+                if (tok < a.n && row + 4 <= a.m) {
+                    const f32x4 v = acc[tm][tn];
+                    *reinterpret_cast<f16x4 *>(outp + (size_t)tok * a.m + row) = f16x4{(f16)v[0], (f16)v[1], (f16)v[2], (f16)v[3]};
+                }
+            }
+        }
+        return;
+    }
+    // split-K: fp32 partial tiles [split][tile][wave][tm][tn][lane] as float4, the last workgroup of
+    // a tile to arrive adds them in split order (deterministic, no atomics on out)
+    const size_t tile_id = (size_t)blockIdx.y * gridDim.x + blockIdx.x;
+    constexpr size_t kTileF4 = (size_t)8 * TM * TN * 64;  // float4s per partial tile
+    f32x4 *ws4 = reinterpret_cast<f32x4 *>(a.ws);
+    f32x4 *mine = ws4 + (tile_id * a.split_k + blockIdx.z) * kTileF4 + (size_t)wave * (TM * TN * 64) + lane;
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+            const f32x4 v = acc[tm][tn];
+            asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 0" : : "v"(mine + (tm * TN + tn) * 64), "v"(v) : "memory");
+        }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the partial sums have left this CU
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    volatile unsigned *ticket = reinterpret_cast<volatile unsigned *>(a_tile);
+    if (tid == 0) *ticket = __hip_atomic_fetch_add(a.counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (*ticket != (unsigned)(a.split_k - 1)) return;
+    if (tid == 0) __hip_atomic_store(a.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const f32x4 *src = ws4 + tile_id * a.split_k * kTileF4 + (size_t)wave * (TM * TN * 64) + lane;
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+        const int row = row_base + (wm_i * TM + tm) * 16 + g * 4;
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+            const int tok = tok_base + (wn_i * TN + tn) * 16 + i16;
+            float s4[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int sp = 0; sp < a.split_k; ++sp) {
+                const float *p = reinterpret_cast<const float *>(src + (size_t)sp * kTileF4 + (tm * TN + tn) * 64);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) s4[j] += __hip_atomic_load(p + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            if (tok < a.n && row + 4 <= a.m)
+                *reinterpret_cast<f16x4 *>(outp + (size_t)tok * a.m + row) = f16x4{(f16)s4[0], (f16)s4[1], (f16)s4[2], (f16)s4[3]};
+        }
+    }
+}
+
+typedef void (*TiledFn)(const TiledArgs);
+struct TiledVariant {
+    int bm, bn;
+    TiledFn fn;
+};
+// (WM, TM, WN, TN): rows x tokens of the workgroup tile
+static const TiledVariant kTiled[] = {
+    {256, 256, gemm_tiled_kernel<2, 8, 4, 4>},
+    {256, 128, gemm_tiled_kernel<4, 4, 2, 4>},
+    {256, 64, gemm_tiled_kernel<4, 4, 2, 2>},
+    {128, 256, gemm_tiled_kernel<2, 4, 4, 4>},
+    {128, 128, gemm_tiled_kernel<2, 4, 4, 2>},
+    {64, 256, gemm_tiled_kernel<1, 4, 8, 2>},
+    {64, 128, gemm_tiled_kernel<1, 4, 8, 1>},
+};
+static constexpr int kNumTiled = sizeof(kTiled) / sizeof(kTiled[0]);
+
+bool tiled_variant_exists(int bm, int bn)
+{
+    for (int i = 0; i < kNumTiled; ++i)
+        if (kTiled[i].bm == bm && kTiled[i].bn == bn) return true;
+    return false;
+}
+
+size_t tiled_lds_bytes(int bm, int bn) { return (size_t)kLutBytes + (size_t)(bm + bn) * 128; }
+
+static unsigned char g_tiled_attr[16][kNumTiled];
+
+hipError_t launch_gemm_tiled(const TiledArgs &args, int bm, int bn, hipStream_t stream)
+{
+    int vi = -1;
+    for (int i = 0; i < kNumTiled; ++i)
+        if (kTiled[i].bm == bm && kTiled[i].bn == bn) vi = i;
+    if (vi < 0) return hipErrorInvalidConfiguration;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
+    if (!g_tiled_attr[dev][vi]) {  // dynamic LDS above 64 KB needs a one-time opt-in per kernel and device
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(kTiled[vi].fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kLdsLimit);
+        if (e != hipSuccess) return e;
+        g_tiled_attr[dev][vi] = 1;
+    }
+    const dim3 grid((unsigned)ceil_div_i(args.m, bm), (unsigned)ceil_div_i(args.n, bn), (unsigned)args.split_k);
+    hipLaunchKernelGGL(kTiled[vi].fn, grid, dim3(kTiledThreads), tiled_lds_bytes(bm, bn), stream, args);
+    return hipGetLastError();
+}
+
+}  // namespace tuna

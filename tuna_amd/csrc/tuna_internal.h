@@ -111,6 +111,24 @@ __host__ __device__ inline void balanced_contributors(unsigned row_tile, unsigne
     *first_slot = (lo * T) / nw < u0 ? 1u : 0u;
 }
 
+// Launch arguments of the many-token kernel (gemm_tiled.hip): weights decoded once per
+// workgroup tile into LDS.  k-steps are 64 long here.
+struct TiledArgs {
+    const uint8_t *q;
+    const void *x;
+    const float *code;
+    const float *absmax;
+    void *out;
+    float *ws;           // split-K partial tiles (library owned), unused if split_k == 1
+    unsigned *counters;  // one arrival counter per tile, zero between launches
+    int m, n, k;
+    int steps_total;      // ceil(k / 64)
+    int split_k;          // gridDim.z
+    int steps_per_split;
+};
+
+inline int ceil_div_i(int a, int b) { return (a + b - 1) / b; }
+
 struct GemmPlan {
     GemmArgs args;
     dim3 grid;
@@ -126,6 +144,11 @@ struct GemmPlan {
 // gemm_kernel.hip
 hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream);
 bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves, int grouped);
+
+// gemm_tiled.hip
+hipError_t launch_gemm_tiled(const TiledArgs &args, int tile_rows, int tile_tokens, hipStream_t stream);
+bool tiled_variant_exists(int tile_rows, int tile_tokens);
+size_t tiled_lds_bytes(int tile_rows, int tile_tokens);
 
 // dequant_kernel.hip
 hipError_t launch_dequant(const uint8_t *q, const float *absmax, const float *code, void *out,

@@ -36,7 +36,7 @@ N_BUCKETS = {
 }
 
 FIELDS = ("rows_per_wave", "waves_m", "waves_k", "split_k", "prefetch", "x_chunk",
-          "token_tiles", "xcd_swizzle", "k_stagger")
+          "token_tiles", "xcd_swizzle", "k_stagger", "lds_tile_rows")
 
 LUT_BYTES = 256 * 64 * 4
 LDS_LIMIT = 160 * 1024
@@ -48,6 +48,10 @@ STEP_K = 32
 VARIANTS_512 = {(1, 2, 1), (1, 2, 2), (1, 2, 4), (1, 4, 1), (1, 4, 2), (1, 8, 1), (1, 8, 2), (2, 2, 1), (2, 4, 1)}
 VARIANTS_512_2WG = {(1, 2, 1), (1, 4, 1)}
 VARIANTS_1024 = {(1, 2, 1), (1, 4, 1)}
+
+
+# (rows, tokens) tiles of the many-token kernel; must match kTiled in csrc/gemm_tiled.hip
+TILED_VARIANTS = {(256, 256), (256, 128), (256, 64), (128, 256), (128, 128), (64, 256), (64, 128)}
 
 
 def _pow2(v: int) -> bool:
@@ -64,7 +68,7 @@ def bucket_of(n: int):
 
 def validate(m: int, n_key: int, k: int, c: dict) -> None:
     """Raise ValueError unless config `c` can run shape (m, n in bucket n_key, k)."""
-    c = {"k_stagger": 0, **c}  # entries written before the field existed
+    c = {"k_stagger": 0, "lds_tile_rows": 0, **c}  # entries written before the fields existed
     missing = [f for f in FIELDS if f not in c]
     if missing:
         raise ValueError(f"missing fields {missing}")
@@ -72,6 +76,13 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
         raise ValueError("m and k must be positive multiples of 8")
     if n_key not in N_BUCKETS:
         raise ValueError(f"n={n_key} is not a bucket key {sorted(N_BUCKETS)}")
+    if c["lds_tile_rows"]:
+        # many-token kernel: only the tile shape and the split matter
+        if (c["lds_tile_rows"], 16 * c["token_tiles"]) not in TILED_VARIANTS:
+            raise ValueError(f"no many-token kernel for a {c['lds_tile_rows']} x {16 * c['token_tiles']} tile")
+        if not 1 <= c["split_k"] <= -(-k // 64):
+            raise ValueError("split_k of the many-token kernel must be in 1..ceil(k/64)")
+        return
     if c["rows_per_wave"] not in (64, 128, 256):
         raise ValueError("rows_per_wave must be 64, 128 or 256")
     if c["prefetch"] not in (2, 4, 8):
@@ -138,7 +149,7 @@ namespace tuna {{
 
 const TableEntry kConfigTable[] = {{
 {body}
-    {{0, 0, 0, 0, {{0, 0, 0, 0, 0, 0, 0, 0, 0}}}},  // sentinel (not counted)
+    {{0, 0, 0, 0, {{0, 0, 0, 0, 0, 0, 0, 0, 0, 0}}}},  // sentinel (not counted)
 }};
 const int kConfigTableSize = {len(rows)};
 

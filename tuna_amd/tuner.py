@@ -49,6 +49,13 @@ def repair(c: dict, m: int, n_key: int, k: int):
     """Make a raw gene vector a valid config for the shape, or return None."""
     c = dict(c)
     c.setdefault("k_stagger", 0)
+    c.setdefault("lds_tile_rows", 0)
+    if c["lds_tile_rows"]:
+        try:
+            make_configs.validate(m, n_key, k, c)
+            return c
+        except ValueError:
+            return None
     steps = -(-k // 32)
     if c["waves_m"] * c["waves_k"] > 16:
         return None
@@ -96,6 +103,31 @@ def seeds(m: int, n_key: int, k: int):
                                     out.append(c)
     uniq = {json.dumps(c, sort_keys=True): c for c in out}
     return list(uniq.values())
+
+
+def tiled_space(m: int, n_key: int, k: int):
+    """Every config of the many-token kernel (weights decoded once into LDS) worth timing for
+    the shape: tile shapes x k splits.  Small enough to time exhaustively."""
+    lo, _ = make_configs.N_BUCKETS[n_key]
+    if lo < 64:
+        return []
+    out = []
+    steps = -(-k // 64)
+    for rows, tokens in sorted(make_configs.TILED_VARIANTS):
+        if tokens > max(64, 2 * lo):
+            continue
+        tiles = -(-m // rows) * -(-lo // tokens)
+        for split in (1, 2, 3, 4, 6, 8, 12, 16, 24, 32):
+            if split > 1 and (steps // split < 4 or tiles * split > 4 * N_CU):
+                continue
+            c = dict(rows_per_wave=64, waves_m=1, waves_k=1, split_k=split, prefetch=2, x_chunk=64, token_tiles=tokens // 16,
+                     xcd_swizzle=0, k_stagger=0, lds_tile_rows=rows)
+            try:
+                make_configs.validate(m, n_key, k, c)
+            except ValueError:
+                continue
+            out.append(c)
+    return out
 
 
 def mutate(c: dict, rng: random.Random, m, n_key, k):
@@ -163,6 +195,11 @@ def tune_shape(m, n, k, generations=6, population=24, seed=0, log=print, max_see
     rng = random.Random(seed * 7919 + m * 31 + k)
     n_key = make_configs.bucket_of(n)
     ev = Evaluator(m, n, k, iters=iters, warmup=max(2, iters // 6))
+    if n_key >= 512:
+        # far beyond the streaming kernel's range: only the many-token kernel is searched
+        scored = sorted((ev(c), json.dumps(c, sort_keys=True)) for c in tiled_space(m, n_key, k))
+        log(f"  many-token kernel: {len(scored)} configs, best {scored[0][0]:.2f} us {scored[0][1]}")
+        return json.loads(scored[0][1]), scored[0][0]
     pool = seeds(m, n_key, k)
     rng.shuffle(pool)
     pool = pool[:max_seed_evals]
@@ -189,6 +226,8 @@ def tune_shape(m, n, k, generations=6, population=24, seed=0, log=print, max_see
         allc = sorted(((t, s) for s, t in ev.cache.items()))
         pop = [json.loads(s) for _, s in allc[:population]]
         log(f"  gen {gen}: {len(children)} new, best {allc[0][0]:.2f} us {allc[0][1]}")
+    for c in tiled_space(m, n_key, k):      # the other kernel family: timed exhaustively
+        ev(c)
     best_t, best_s = min(((t, s) for s, t in ev.cache.items()))
     # re-time the top few with more iterations to pick a stable winner
     top = sorted(((t, s) for s, t in ev.cache.items()))[:5]
