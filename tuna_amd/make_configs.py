@@ -118,6 +118,9 @@ def lds_bytes(c: dict) -> int:
 
     The reduction buffers are 2 x 1 plane (1 KB) per wave, or 2 x 4 planes when that costs no
     occupancy (mirrors plan_gemm in csrc/api.cpp)."""
+    if c.get("lds_tile_rows"):
+        # many-token kernel: decode table + weight tile + activation tile, 128 bytes per row
+        return LUT_BYTES + (c["lds_tile_rows"] + 16 * c["token_tiles"]) * 128
     threads = 64 * c["waves_k"] * c["waves_m"]
     x = c["token_tiles"] * 16 * c["x_chunk"] * 2
     plane = c["waves_k"] * c["waves_m"] * 1024
