@@ -429,7 +429,7 @@ def test_grouped_gemm_rejects_bad_arguments():
 
 
 # ----------------------------------------------------------------------------- many-token kernel (weights decoded once into LDS)
-TILED = [(256, 16), (256, 8), (256, 4), (128, 16), (128, 8), (64, 16), (64, 8)]   # (lds_tile_rows, token_tiles)
+TILED = [(256, 8), (256, 4), (128, 16), (128, 8), (64, 16), (64, 8)]   # (lds_tile_rows, token_tiles)
 
 
 @pytest.mark.parametrize("tile", TILED)

@@ -12,7 +12,11 @@
 //     WM x WN waves, a wave owns TM x TN MFMA tiles (v_mfma_f32_16x16x32_f16, weights = A).
 //   * per k-step the 512 threads fetch BM x 64 packed weights (16 bytes per thread: 4
 //     consecutive rows x 8 k; 16 threads cover 256 contiguous bytes of a block row) and
-//     BN x 64 activations, two steps ahead, into registers;
+//     BN x 64 activations into registers, four steps ahead of their use (HBM latency is
+//     longer than two steps of matrix work);
+//   * two LDS tile buffers: while the matrix cores work on step s from one buffer, step
+//     s+1 is decoded and staged into the other - one barrier per step, and the decode's
+//     VALU/LDS work runs in the shadow of the MFMAs of the other wave on the SIMD;
 //   * decode through the same conflict-free byte-pair table as the streaming kernel
 //     (one v_perm_b32 + ds_read_b32 + v_pk_mul_f16 per two weights, bit-identical to
 //     kernel.cu:2178-2192), then one ds_write_b128 per decoded dword into the A tile;
@@ -48,8 +52,9 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     static_assert(A_PIECES <= kTiledThreads && X_PER_THREAD >= 1, "tile shape");
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char *lut = smem;                       // byte-pair table at LDS address 0
-    unsigned char *a_tile = smem + kLutBytes;        // [BM][128 bytes]
-    unsigned char *x_tile = a_tile + BM * 128;       // [BN][128 bytes]
+    constexpr int BUF = (BM + BN) * 128;             // one buffer: weight tile [BM][128 B] + activation tile [BN][128 B]
+    unsigned char *a_tile = smem + kLutBytes;
+    unsigned char *x_tile = a_tile + BM * 128;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -89,8 +94,9 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
         x_src[i] = xg + (size_t)min(tok, a.n - 1) * a.k + (p & 7) * 8;
     }
 
-    u32x4 wq[2];
-    u32x4 xr[2][X_PER_THREAD];
+    constexpr int NSETS = 4;  // register sets: steps s .. s+3 in flight
+    u32x4 wq[NSETS];
+    u32x4 xr[NSETS][X_PER_THREAD];
     // Unconditional, clamped loads (exact s_waitcnt counts); what lies beyond k is zeroed in x.
 #define TUNA_TILED_LOAD(set, s)                                                                 \
     {                                                                                          \
@@ -105,8 +111,8 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
 
     const int s0 = blockIdx.z * a.steps_per_split;
     const int s1 = min(a.steps_total, s0 + a.steps_per_split);
-    TUNA_TILED_LOAD(0, min(s0, a.steps_total - 1))
-    TUNA_TILED_LOAD(1, min(s0 + 1, a.steps_total - 1))
+#pragma unroll
+    for (int u = 0; u < NSETS; ++u) TUNA_TILED_LOAD(u, min(s0 + u, a.steps_total - 1))
 
     // ---- decode table (as in the streaming kernel) ------------------------------------------
     {
@@ -132,10 +138,11 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     const unsigned char *x_frag = x_tile + (wn_i * TN * 16 + i16) * 128;
     const int sw = i16 & 7;
 
-    // One k-step: (barrier) decode + stage -> (refill registers two steps ahead) -> barrier -> MFMA
-#define TUNA_TILED_STEP(set, s)                                                                 \
+    // Stage k-step s from register set `set` into tile buffer `buf`: decode the packed weights,
+    // copy the activations (zero beyond n and k), then refill the set four steps ahead.
+#define TUNA_TILED_STAGE(set, buf, s)                                                            \
     {                                                                                          \
-        __syncthreads(); /* every wave has finished reading the previous step's tiles */       \
+        unsigned char *at_ = a_tile + (buf) * BUF, *xt_ = x_tile + (buf) * BUF;                \
         if (a_loader) {                                                                        \
             _Pragma("unroll") for (int j = 0; j < 4; ++j)                                      \
             {                                                                                  \
@@ -148,7 +155,7 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
                 const f16x2 h2_ = __builtin_bit_cast(f16x2, t2_) * sc16[j], h3_ = __builtin_bit_cast(f16x2, t3_) * sc16[j]; \
                 const f16x8 w_ = {h0_[0], h0_[1], h1_[0], h1_[1], h2_[0], h2_[1], h3_[0], h3_[1]}; \
                 const int r_ = a_row + j;                                                      \
-                *reinterpret_cast<f16x8 *>(a_tile + r_ * 128 + ((a_kb ^ (r_ & 7)) << 4)) = w_; \
+                *reinterpret_cast<f16x8 *>(at_ + r_ * 128 + ((a_kb ^ (r_ & 7)) << 4)) = w_;    \
             }                                                                                  \
         }                                                                                      \
         _Pragma("unroll") for (int i = 0; i < X_PER_THREAD; ++i)                               \
@@ -156,13 +163,16 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
             const int p_ = tid + i * kTiledThreads;                                            \
             const int t_ = p_ >> 3, sl_ = p_ & 7;                                              \
             const bool ok_ = x_tok_ok[i] && ((s) * kTiledStepK + sl_ * 8 < a.k);               \
-            *reinterpret_cast<u32x4 *>(x_tile + t_ * 128 + ((sl_ ^ (t_ & 7)) << 4)) = ok_ ? xr[set][i] : u32x4{0u, 0u, 0u, 0u}; \
+            *reinterpret_cast<u32x4 *>(xt_ + t_ * 128 + ((sl_ ^ (t_ & 7)) << 4)) = ok_ ? xr[set][i] : u32x4{0u, 0u, 0u, 0u}; \
         }                                                                                      \
-        TUNA_TILED_LOAD(set, min((s) + 2, a.steps_total - 1))                                  \
-        __syncthreads();                                                                       \
+        TUNA_TILED_LOAD(set, min((s) + NSETS, a.steps_total - 1))                              \
+    }
+    // The matrix work of one k-step from tile buffer `buf`.
+#define TUNA_TILED_MFMA(buf)                                                                     \
+    {                                                                                          \
         _Pragma("unroll") for (int kh = 0; kh < 2; ++kh)                                       \
         {                                                                                      \
-            const int slot_ = ((kh * 4 + g) ^ sw) << 4;                                        \
+            const int slot_ = (((kh * 4 + g) ^ sw) << 4) + (buf) * BUF;                        \
             f16x8 bf_[TN];                                                                     \
             _Pragma("unroll") for (int tn = 0; tn < TN; ++tn)                                  \
                 bf_[tn] = *reinterpret_cast<const f16x8 *>(x_frag + tn * (16 * 128) + slot_);  \
@@ -174,14 +184,32 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
             }                                                                                  \
         }                                                                                      \
     }
+    // iteration i (k-step s0 + i): stage step s0+i+1 into the other buffer, multiply from this one
+#define TUNA_TILED_ITER(i)                                                                       \
+    {                                                                                          \
+        TUNA_TILED_STAGE(((i) + 1) & 3, ((i) + 1) & 1, s + (i) + 1)                            \
+        TUNA_TILED_MFMA((i) & 1)                                                               \
+        __syncthreads(); /* the staged tiles are complete; this step's tiles are free */       \
+    }
 
     int s = s0;
-    for (; s + 1 < s1; s += 2) {
-        TUNA_TILED_STEP(0, s)
-        TUNA_TILED_STEP(1, s + 1)
+    __syncthreads();  // decode table complete
+    TUNA_TILED_STAGE(0, 0, s)
+    __syncthreads();
+    for (; s + 3 < s1; s += 4) {
+        TUNA_TILED_ITER(0)
+        TUNA_TILED_ITER(1)
+        TUNA_TILED_ITER(2)
+        TUNA_TILED_ITER(3)
     }
-    if (s < s1) TUNA_TILED_STEP(0, s)
-#undef TUNA_TILED_STEP
+    // tail: up to three more steps (the staging of a step past the end is harmless: its loads are
+    // clamped and nothing reads the tiles)
+    if (s < s1) TUNA_TILED_ITER(0)
+    if (s + 1 < s1) TUNA_TILED_ITER(1)
+    if (s + 2 < s1) TUNA_TILED_ITER(2)
+#undef TUNA_TILED_ITER
+#undef TUNA_TILED_MFMA
+#undef TUNA_TILED_STAGE
 #undef TUNA_TILED_LOAD
 
     // ---- epilogue -----------------------------------------------------------------------------
@@ -249,7 +277,6 @@ struct TiledVariant {
 };
 // (WM, TM, WN, TN): rows x tokens of the workgroup tile
 static const TiledVariant kTiled[] = {
-    {256, 256, gemm_tiled_kernel<2, 8, 4, 4>},
     {256, 128, gemm_tiled_kernel<4, 4, 2, 4>},
     {256, 64, gemm_tiled_kernel<4, 4, 2, 2>},
     {128, 256, gemm_tiled_kernel<2, 4, 4, 4>},
@@ -266,7 +293,7 @@ bool tiled_variant_exists(int bm, int bn)
     return false;
 }
 
-size_t tiled_lds_bytes(int bm, int bn) { return (size_t)kLutBytes + (size_t)(bm + bn) * 128; }
+size_t tiled_lds_bytes(int bm, int bn) { return (size_t)kLutBytes + 2 * (size_t)(bm + bn) * 128; }  // two tile buffers
 
 static unsigned char g_tiled_attr[16][kNumTiled];
 

@@ -51,7 +51,7 @@ VARIANTS_1024 = {(1, 2, 1), (1, 4, 1)}
 
 
 # (rows, tokens) tiles of the many-token kernel; must match kTiled in csrc/gemm_tiled.hip
-TILED_VARIANTS = {(256, 256), (256, 128), (256, 64), (128, 256), (128, 128), (64, 256), (64, 128)}
+TILED_VARIANTS = {(256, 128), (256, 64), (128, 256), (128, 128), (64, 256), (64, 128)}
 
 
 def _pow2(v: int) -> bool:
@@ -119,8 +119,8 @@ def lds_bytes(c: dict) -> int:
     The reduction buffers are 2 x 1 plane (1 KB) per wave, or 2 x 4 planes when that costs no
     occupancy (mirrors plan_gemm in csrc/api.cpp)."""
     if c.get("lds_tile_rows"):
-        # many-token kernel: decode table + weight tile + activation tile, 128 bytes per row
-        return LUT_BYTES + (c["lds_tile_rows"] + 16 * c["token_tiles"]) * 128
+        # many-token kernel: decode table + two buffers of (weight tile + activation tile), 128 bytes per row
+        return LUT_BYTES + 2 * (c["lds_tile_rows"] + 16 * c["token_tiles"]) * 128
     threads = 64 * c["waves_k"] * c["waves_m"]
     x = c["token_tiles"] * 16 * c["x_chunk"] * 2
     plane = c["waves_k"] * c["waves_m"] * 1024
