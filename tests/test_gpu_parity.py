@@ -459,3 +459,74 @@ def test_many_token_kernel_decode_readout_is_bit_exact():
     got = run_gemm(q, x, code, absmax, m, k, k, config=cfg(lds_tile_rows=128, token_tiles=8), prefill=float("nan"))
     want = O.dequant(q, absmax, code, m, k, mode=O.D1)          # [m, k] fp16 bits
     assert np.array_equal(got.T, want)
+
+
+# ----------------------------------------------------------------------------- stream capture / graph replay, several streams
+def test_graph_replay_matches_eager_for_split_k_and_many_token_configs():
+    """The ops are stream-ordered and capturable once their workspace exists: a captured graph
+    of three GEMMs (fixed split-K, balanced split, many-token kernel with split-K) is replayed
+    with new inputs written in place, with eager work and synchronisations in between, and
+    every replay must give the bits of the eager call."""
+    import torch
+
+    from tuna_amd import ops
+
+    m, n, k = 1024, 144, 2048
+    cfgs = [cfg(split_k=4, x_chunk=512), cfg(split_k=0, waves_m=1, waves_k=8, prefetch=2, x_chunk=512),
+            cfg(lds_tile_rows=128, token_tiles=8, split_k=2)]
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=31)
+    dq, dx, dc, da = to_dev(q, x, code, absmax)
+    outs = [torch.zeros((n, m), dtype=torch.float16, device="cuda") for _ in cfgs]
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for c, o in zip(cfgs, outs):          # first call on this stream allocates the split-K workspace
+            ops.matmul(dx, dq, da, dc, o, m, n, k, config=c)
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for c, o in zip(cfgs, outs):
+                ops.matmul(dx, dq, da, dc, o, m, n, k, config=c)
+    for rep in range(4):
+        _, x2, _, _ = make_inputs_np(m, n, k, seed=100 + rep)
+        dx.copy_(torch.from_numpy(x2).cuda())
+        for o in outs:
+            o.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        for c, g in zip(cfgs, got):
+            eager = torch.zeros((n, m), dtype=torch.float16, device="cuda")
+            ops.matmul(dx, dq, da, dc, eager, m, n, k, config=c)
+            torch.cuda.synchronize()
+            assert torch.equal(g.view(torch.int16), eager.view(torch.int16)), (rep, c.to_dict())
+
+
+def test_two_streams_do_not_share_split_k_partial_sums():
+    """Split-K GEMMs enqueued on two streams at once (each stream owns its workspace) give the
+    same bits as run alone."""
+    import torch
+
+    from tuna_amd import ops
+
+    m, n, k = 4096, 16, 4096
+    c = cfg(waves_m=1, waves_k=8, prefetch=2, x_chunk=1024, split_k=4, xcd_swizzle=1)
+    data = []
+    for seed in (41, 42):
+        q, x, code, absmax = make_inputs_np(m, n, k, seed=seed)
+        data.append(to_dev(q, x, code, absmax))
+    alone = []
+    for dq, dx, dc, da in data:
+        o = torch.zeros((n, m), dtype=torch.float16, device="cuda")
+        ops.matmul(dx, dq, da, dc, o, m, n, k, config=c)
+        torch.cuda.synchronize()
+        alone.append(o)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [torch.zeros((n, m), dtype=torch.float16, device="cuda") for _ in range(2)]
+    for _ in range(20):
+        for st, (dq, dx, dc, da), o in zip(streams, data, outs):
+            with torch.cuda.stream(st):
+                ops.matmul(dx, dq, da, dc, o, m, n, k, config=c)
+    torch.cuda.synchronize()
+    for o, ref in zip(outs, alone):
+        assert torch.equal(o.view(torch.int16), ref.view(torch.int16))
