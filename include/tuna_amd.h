@@ -125,6 +125,14 @@ int tuna_dequant(const void *q, const void *absmax, const void *code, void *out,
 int tuna_dequant_ex(const void *q, const void *absmax, const void *code, void *out,
                     int m, int k, int decode_mode, void *stream);
 
+/* Quantizer and packer on the device: fp16 weights w [m, k] row-major -> q [m/8, k/8, 32] and
+ * absmax fp32 [m] (one scale per weight row) for the 16-entry codebook `code`.  The
+ * arithmetic of the reference harness's quantize_blockwise_dynamic_4bit with block_size == k
+ * and preprocess=True (test.py:7-68): absmax = max |w|; index = argmin |fp32(w) / absmax -
+ * code[j]| in fp32, first index on ties; packing of test.py:55-65.  An all-zero row gets the
+ * index of code 7.  The reference has this only as Python on torch tensors. */
+int tuna_quantize(const void *w, const void *code, void *q, void *absmax, int m, int k, void *stream);
+
 /* Shape -> config.  Replaces the if-chain of kernel.cu:3018-3156 over the constants of
  * configs.cu:56-3331 by a table lookup on (m, n-bucket, k) with a derived fallback.
  * Runs on the host only (no device needed).  Returns 1 in *from_table when the shape

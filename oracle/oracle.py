@@ -61,6 +61,8 @@ def lib():
         L.orc_unpack.argtypes = [vp, vp, i32, i32]
         L.orc_dequant.restype = i32
         L.orc_dequant.argtypes = [vp, vp, vp, vp, i32, i32, i32]
+        L.orc_quantize.restype = i32
+        L.orc_quantize.argtypes = [vp, vp, vp, vp, i32, i32]
         L.orc_gemm.restype = i32
         L.orc_gemm.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32]
         L.orc_gemm_rows.restype = i32
@@ -162,6 +164,17 @@ def dequant(q, absmax, code, m, k, mode=D2) -> np.ndarray:
     if rc:
         raise ValueError(f"orc_dequant rc={rc}")
     return out
+
+
+def quantize(w_bits, code, m, k):
+    """fp16 bit patterns [m, k] -> (packed uint8 [m/8, k/8, 32], absmax float32 [m])."""
+    w_bits, code = _c(w_bits, np.uint16), _c(code, np.float32)
+    q = np.empty((m // 8, k // 8, 32), np.uint8)
+    absmax = np.empty(m, np.float32)
+    rc = lib().orc_quantize(_p(w_bits), _p(code), _p(q), _p(absmax), m, k)
+    if rc:
+        raise ValueError(f"orc_quantize rc={rc}")
+    return q, absmax
 
 
 def gemm(q, x, code, absmax, m, n, k, mode=D1, acc64=True, rows=None) -> np.ndarray:

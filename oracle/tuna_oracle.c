@@ -20,6 +20,11 @@
  *   orc_decode_d1 / orc_decode_d2 : exhaustive 16 codes x 65536 scales against
  *       numpy fp16 / fp32 arithmetic; known-answer rows for scale 0x211f
  *   orc_dequant : unpack + decode, checked against a numpy gather
+ *   orc_quantize : per-row absmax + nearest codebook entry + packing (test.py:7-68),
+ *       checked against numpy float32 division / |difference| / argmin (first index on
+ *       ties) incl. exact midpoints between codes, and against the round trip through
+ *       orc_dequant.  All-zero rows: the reference divides by zero and lets NaNs
+ *       decide (parity unpinned for that input); here such a row gets code 7 (0.0).
  *   orc_gemm*   : textbook contraction; checked against numpy float64 matmul,
  *       linearity, one-hot read-out of the decoded weights, row permutation
  */
@@ -223,6 +228,48 @@ ORC_API int orc_dequant(const uint8_t *q, const float *absmax, const float *code
             uint8_t b = q[q_offset(r, c, k)];
             uint8_t nib = (c & 1) ? (b & 15u) : (uint8_t)(b >> 4);
             out[(size_t)r * k + c] = lut[nib];
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Quantizer (test.py:7-68 with block_size == k): absmax[r] = max |w[r, :]| as   */
+/* fp32; normalized = fp32(w) / absmax (fp32 division, test.py:41: fp16 / fp32   */
+/* promotes to fp32); code index = argmin_j |normalized - code[j]| in fp32 with  */
+/* the first index on ties (torch.argmin, test.py:50-53); packed as test.py:55-65 */
+/* ------------------------------------------------------------------------- */
+ORC_API int orc_quantize(const uint16_t *w, const float *code, uint8_t *q, float *absmax, int m, int k)
+{
+    if (m <= 0 || k <= 0 || (m & 7) || (k & 7)) return 1;
+    memset(q, 0, (size_t)m * k / 2);
+#pragma omp parallel for schedule(static)
+    for (int mb = 0; mb < m / 8; mb++) {
+        for (int r8 = 0; r8 < 8; r8++) {
+            const int r = mb * 8 + r8;
+            float amax = 0.f;
+            for (int c = 0; c < k; c++) {
+                const float v = fabsf(orc_f16_to_f32(w[(size_t)r * k + c]));
+                if (v > amax) amax = v;
+            }
+            absmax[r] = amax;
+            for (int c = 0; c < k; c++) {
+                int best = 7;
+                if (amax > 0.f) {
+                    const volatile float nv = orc_f16_to_f32(w[(size_t)r * k + c]) / amax; /* fp32, no excess precision */
+                    float bd = 0.f;
+                    best = 0;
+                    for (int j = 0; j < 16; j++) {
+                        const volatile float d = fabsf(nv - code[j]);
+                        if (j == 0 || d < bd) {
+                            bd = d;
+                            best = j;
+                        }
+                    }
+                }
+                uint8_t *b = &q[q_offset(r, c, k)];
+                *b |= (c & 1) ? (uint8_t)best : (uint8_t)(best << 4);
+            }
         }
     }
     return 0;

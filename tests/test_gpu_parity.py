@@ -530,3 +530,57 @@ def test_two_streams_do_not_share_split_k_partial_sums():
     torch.cuda.synchronize()
     for o, ref in zip(outs, alone):
         assert torch.equal(o.view(torch.int16), ref.view(torch.int16))
+
+
+# ----------------------------------------------------------------------------- quantizer + packer on the device
+@pytest.mark.parametrize("m,k", [(8, 8), (64, 256), (72, 1096), (4096, 4096)])
+def test_device_quantizer_is_bit_exact(m, k):
+    """tuna_quantize against the oracle's quantizer: packed bytes and scales identical, for the
+    NF4 codebook and an arbitrary one, incl. all-zero rows, near-midpoint values, subnormals."""
+    import torch
+
+    from tuna_amd import ops
+
+    rng = np.random.default_rng(m + k)
+    from tuna_amd.quantize import NF4_CODE
+
+    code = np.array(NF4_CODE, np.float32)
+    w = (rng.standard_normal((m, k)) * 0.03).astype(np.float16)
+    if m >= 8 and k >= 16:
+        w[1] = 0
+        w[2] = 0
+        w[2, 5] = np.float16(-0.25)
+        mids = ((code[:-1] + code[1:]) / 2).astype(np.float32)
+        w[3, :15] = (mids * 0.5).astype(np.float16)
+        w[3, 15] = np.float16(0.5)
+        w[4] = np.float16(6e-8)
+        w[4, 0] = np.float16(-1.2e-7)
+    print(f"quantize m={m} k={k}", flush=True)
+    for cb in (code, rng.standard_normal(16).astype(np.float32)):
+        dw, dc = to_dev(w, cb)
+        q, absmax, _ = ops.quantize(dw, dc)
+        torch.cuda.synchronize()
+        q_ref, a_ref = O.quantize(w.view(np.uint16), cb, m, k)
+        assert np.array_equal(absmax.cpu().numpy(), a_ref)
+        assert np.array_equal(q.cpu().numpy(), q_ref)
+
+
+def test_quantize_then_matmul_end_to_end():
+    """Real fp16 weights -> device quantizer -> GEMM, against the fp32 product of the
+    dequantized weights (the reference harness's own flow, test.py:71-106)."""
+    import torch
+
+    from tuna_amd import ops
+
+    m, n, k = 1024, 16, 2048
+    rng = np.random.default_rng(12)
+    w = (rng.standard_normal((m, k)) * 0.02).astype(np.float16)
+    x = (rng.standard_normal((n, k)) * 0.1).astype(np.float16)
+    dw, dx = to_dev(w, x)
+    q, absmax, code = ops.quantize(dw)
+    out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+    ops.matmul(dx, q, absmax, code, out, m, n, k)
+    torch.cuda.synchronize()
+    ref = O.gemm_f64(q.cpu().numpy(), x, code.cpu().numpy(), absmax.cpu().numpy(), m, n, k, mode=O.D1)
+    e = rel_err(out.cpu().numpy().astype(np.float64), ref)
+    assert e <= REL_TOL, e

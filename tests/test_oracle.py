@@ -257,3 +257,68 @@ def test_golden_fixtures():
     assert np.array_equal(out, gm["out_d1"])
     out = O.gemm(gm["q"], gm["x"], cb, gm["absmax"], 256, 16, 128, mode=O.D2)
     assert np.array_equal(out, gm["out_d2"])
+
+
+# ----------------------------------------------------------------------------- quantizer
+def _quantize_numpy_model(w, code):
+    """Independent model of test.py:7-68 with one block per row: numpy float32 division,
+    |difference| in float32, argmin with the first index on ties, then the product's packer."""
+    from tuna_amd.quantize import pack_codes_np
+
+    wf = w.astype(np.float32)
+    a = np.abs(wf).max(axis=1)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        nv = (wf / a[:, None]).astype(np.float32)
+    d = np.abs((nv[None] - code[:, None, None]).astype(np.float32))
+    idx = d.argmin(axis=0).astype(np.uint8)
+    idx[a == 0] = 7                                   # all-zero rows: defined here, NaN-driven in the reference
+    return pack_codes_np(idx), a.astype(np.float32)
+
+
+def _quantizer_inputs(rng, m, k):
+    from tuna_amd.quantize import NF4_CODE
+
+    code = np.array(NF4_CODE, np.float32)
+    w = (rng.standard_normal((m, k)) * 0.03).astype(np.float16)
+    if m >= 8 and k >= 16:
+        w[1] = 0                                      # all-zero row
+        w[2] = 0
+        w[2, 5] = np.float16(-0.25)                   # a single non-zero: the negative extreme
+        mids = ((code[:-1] + code[1:]) / 2).astype(np.float32)
+        w[3, :15] = (mids * 0.5).astype(np.float16)   # (nearly) halfway between neighbouring codes
+        w[3, 15] = np.float16(0.5)
+        w[4] = np.float16(6e-8)                       # fp16 subnormals
+        w[4, 0] = np.float16(-1.2e-7)
+    return w, code
+
+
+@pytest.mark.parametrize("m,k", [(8, 8), (8, 16), (64, 256), (72, 1096)])
+def test_quantizer_oracle_matches_numpy_model(m, k):
+    rng = np.random.default_rng(m * 131 + k)
+    w, code = _quantizer_inputs(rng, m, k)
+    q, absmax = O.quantize(w.view(np.uint16), code, m, k)
+    q_ref, a_ref = _quantize_numpy_model(w, code)
+    assert np.array_equal(absmax, a_ref)
+    assert np.array_equal(q, q_ref)
+    # an arbitrary (unsorted) codebook is handled the same way
+    code2 = rng.standard_normal(16).astype(np.float32)
+    q2, _ = O.quantize(w.view(np.uint16), code2, m, k)
+    assert np.array_equal(q2, _quantize_numpy_model(w, code2)[0])
+
+
+def test_quantizer_round_trip_recovers_the_codes():
+    """Weights that are exactly code * scale quantize back to the same codes and scale
+    (code gaps are far larger than an fp16 rounding), and dequantize to the same weights."""
+    from tuna_amd.quantize import NF4_CODE, pack_codes_np
+
+    rng = np.random.default_rng(5)
+    m, k = 32, 128
+    code = np.array(NF4_CODE, np.float32)
+    idx = rng.integers(0, 16, size=(m, k)).astype(np.uint8)
+    idx[:, 0] = 15                                    # every row contains the extreme code: absmax = scale
+    scale = rng.uniform(0.005, 0.02, size=m).astype(np.float16).astype(np.float32)
+    w_bits = O.dequant(pack_codes_np(idx), scale, code, m, k, mode=O.D2)
+    q, absmax = O.quantize(w_bits, code, m, k)
+    assert np.array_equal(absmax, scale)
+    assert np.array_equal(q, pack_codes_np(idx))
+    assert np.array_equal(O.dequant(q, absmax, code, m, k, mode=O.D2), w_bits)

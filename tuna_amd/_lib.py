@@ -63,6 +63,7 @@ SIGNATURES = {
     "tuna_matmul_ex": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _vp]),
     "tuna_matmul_grouped": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _ip, _cfgp, _i, _vp]),
     "tuna_dequant": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "tuna_quantize": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "tuna_dequant_ex": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "tuna_select_config": (_i, [_i, _i, _i, _cfgp, _ip]),
     "tuna_validate_config": (_i, [_i, _i, _i, _cfgp]),

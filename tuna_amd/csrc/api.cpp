@@ -664,6 +664,19 @@ TUNA_EXPORT int tuna_dequant(const void *q, const void *absmax, const void *code
     return dequant_impl(q, absmax, code, out, m, k, TUNA_DECODE_DEQUANT, static_cast<hipStream_t>(stream));
 }
 
+TUNA_EXPORT int tuna_quantize(const void *w, const void *code, void *q, void *absmax, int m, int k, void *stream)
+{
+    int rc;
+    if ((rc = check_shape(m, 1, k))) return rc;
+    if ((rc = check_ptr(w, "w", 16)) || (rc = check_ptr(code, "code", 4)) || (rc = check_ptr(q, "q", 16)) ||
+        (rc = check_ptr(absmax, "absmax", 4)))
+        return rc;
+    hipError_t e = launch_quantize(w, static_cast<const float *>(code), q, static_cast<float *>(absmax), m, k,
+                                   static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "quantize launch");
+    return TUNA_OK;
+}
+
 TUNA_EXPORT int tuna_dequant_ex(const void *q, const void *absmax, const void *code, void *out, int m, int k,
                                 int decode_mode, void *stream)
 {

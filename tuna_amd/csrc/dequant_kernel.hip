@@ -141,4 +141,69 @@ hipError_t launch_copy(const void *src, void *dst, size_t bytes, hipStream_t str
     return hipGetLastError();
 }
 
+// fp16 weights [m, k] -> packed 4-bit codes + per-row absmax: the device form of the reference
+// harness's quantize_blockwise_dynamic_4bit with one scale per row (test.py:7-68).  Same
+// arithmetic: absmax = max |w| as fp32; normalized = fp32(w) / absmax with an fp32 division
+// (test.py:41, fp16 / fp32 promotes to fp32); index = argmin_j |normalized - code[j]| in
+// fp32, first index on ties (torch.argmin, test.py:50-53); nibble packing of test.py:55-65.
+// An all-zero row (the reference divides by zero there) gets index 7, the NF4 zero.
+// One workgroup per block row (8 weight rows): 32 threads per row, 16-byte reads; a thread
+// turns 8 consecutive k of one row into one dword of the 32-byte record.
+__global__ __launch_bounds__(256) void quantize_kernel(const f16 *__restrict__ w, const float *__restrict__ code,
+                                                       uint32_t *__restrict__ q32, float *__restrict__ absmax, int m, int k)
+{
+    __shared__ float cf[16];
+    const int tid = threadIdx.x;
+    if (tid < 16) cf[tid] = code[tid];
+    const int mb = blockIdx.x;
+    const int r8 = tid >> 5, j = tid & 31;
+    const int row = mb * 8 + r8;
+    const int kb_total = k >> 3;
+    const f16 *src = w + (size_t)row * k;
+    float amax = 0.f;
+    for (int kb = j; kb < kb_total; kb += 32) {
+        const f16x8 v = *reinterpret_cast<const f16x8 *>(src + kb * 8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf((float)v[e]));
+    }
+#pragma unroll
+    for (int off = 16; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 32));
+    if (j == 0) absmax[row] = amax;
+    __syncthreads();  // codebook in LDS
+    float c[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) c[i] = cf[i];
+    for (int kb = j; kb < kb_total; kb += 32) {
+        const f16x8 v = *reinterpret_cast<const f16x8 *>(src + kb * 8);
+        uint32_t d = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            uint32_t best = 7;
+            if (amax > 0.f) {
+                const float nv = __fdiv_rn((float)v[e], amax);
+                float bd = fabsf(__fsub_rn(nv, c[0]));
+                best = 0;
+#pragma unroll
+                for (int i = 1; i < 16; ++i) {
+                    const float dd = fabsf(__fsub_rn(nv, c[i]));
+                    if (dd < bd) {
+                        bd = dd;
+                        best = i;
+                    }
+                }
+            }
+            // byte e/2 of the dword; even column = high nibble
+            d |= best << (8 * (e >> 1) + 4 * (1 - (e & 1)));
+        }
+        q32[((size_t)mb * kb_total + kb) * 8 + r8] = d;
+    }
+}
+
+hipError_t launch_quantize(const void *w, const float *code, void *q, float *absmax, int m, int k, hipStream_t stream)
+{
+    hipLaunchKernelGGL(quantize_kernel, dim3((unsigned)(m / 8)), dim3(256), 0, stream, static_cast<const f16 *>(w), code,
+                       static_cast<uint32_t *>(q), absmax, m, k);
+    return hipGetLastError();
+}
+
 }  // namespace tuna

@@ -153,6 +153,7 @@ size_t tiled_lds_bytes(int tile_rows, int tile_tokens);
 // dequant_kernel.hip
 hipError_t launch_dequant(const uint8_t *q, const float *absmax, const float *code, void *out,
                           int m, int k, int decode, hipStream_t stream);
+hipError_t launch_quantize(const void *w, const float *code, void *q, float *absmax, int m, int k, hipStream_t stream);
 hipError_t launch_copy(const void *src, void *dst, size_t bytes, hipStream_t stream);
 hipError_t launch_read(const void *src, void *sink, size_t bytes, int blocks, hipStream_t stream);
 

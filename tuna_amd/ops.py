@@ -120,6 +120,29 @@ def dequant(q, absmax, codebook, o, m: int, k: int, decode_mode: int = _lib.DECO
     _lib.check(rc)
 
 
+def quantize(w, codebook=None):
+    """fp16 weights [m, k] on a HIP device -> (q uint8 [m/8, k/8, 32], absmax fp32 [m], codebook
+    fp32 [16]): the reference harness's quantizer + packer with one scale per row (test.py:7-68)
+    as one kernel (tuna_quantize).  `codebook` defaults to the NF4 constants."""
+    from .quantize import nf4_codebook
+
+    if w.dim() != 2:
+        raise ValueError("w must be [m, k]")
+    m, k = w.shape
+    if m % 8 or k % 8:
+        raise ValueError("m and k must be multiples of 8")
+    _require(w, "w", torch.float16, m * k)
+    code = nf4_codebook(w.device) if codebook is None else codebook
+    _require(code, "codebook", torch.float32, 16)
+    q = torch.empty((m // 8, k // 8, 32), dtype=torch.uint8, device=w.device)
+    absmax = torch.empty((m,), dtype=torch.float32, device=w.device)
+    with torch.cuda.device(w.device):
+        rc = _lib.lib().tuna_quantize(w.data_ptr(), code.data_ptr(), q.data_ptr(), absmax.data_ptr(), int(m), int(k),
+                                      _stream(w.device))
+    _lib.check(rc)
+    return q, absmax, code
+
+
 def select_config(m: int, n: int, k: int):
     """(GemmConfig, from_table) the library would use for shape (m, n, k).  Host only."""
     cfg = GemmConfig()
