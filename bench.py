@@ -238,6 +238,21 @@ def main():
             del sets, img
             torch.cuda.empty_cache()
         line["dequant"] = deq
+        # device quantizer + packer on one shape (fp16 weights read twice, packed bytes written once)
+        qm, qk = synth.SHAPES["mistral_attn_out"]
+        wq_ = (torch.randn((qm, qk), device=dev) * 0.02).to(torch.float16)
+        for _ in range(3):
+            ops.quantize(wq_)
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for _ in range(20):
+            ops.quantize(wq_)
+        ev1.record()
+        torch.cuda.synchronize()
+        us = ev0.elapsed_time(ev1) * 1000.0 / 20
+        line["quantize"] = {"m": qm, "k": qk, "us": round(us, 2), "gbs_fp16_in": round(2.0 * qm * qk / (us * 1e-6) / 1e9, 1)}
+        del wq_
 
     if not args.no_shapes:
         # Mixtral gate+up with a router: 16 tokens x top-2 = 32 (token, expert) rows spread over the 8
@@ -291,7 +306,7 @@ def main():
             sweeps["llama70b_80_layers"] = {"error": str(e)[:200]}
         # token sweep on the Llama-70B layer set
         tok = {}
-        for nt in (1, 16, 64, 256):
+        for nt in (1, 16, 64, 256, 1024):
             row = {}
             for nm in names:
                 sm, sk = synth.SHAPES[nm]
