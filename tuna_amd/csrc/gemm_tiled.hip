@@ -41,7 +41,7 @@ typedef __attribute__((address_space(3))) uint32_t lds_u32;
 constexpr int kTiledThreads = 512;
 constexpr int kTiledStepK = 64;
 
-template <int WM, int TM, int WN, int TN>
+template <int WM, int TM, int WN, int TN, int NSETS>
 __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const TiledArgs a)
 {
     static_assert(WM * WN * 64 == kTiledThreads, "8 waves");
@@ -94,7 +94,9 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
         x_src[i] = xg + (size_t)min(tok, a.n - 1) * a.k + (p & 7) * 8;
     }
 
-    constexpr int NSETS = 4;  // register sets: steps s .. s+3 in flight
+    // NSETS register sets: steps s .. s+NSETS-1 in flight (4; 8 for the 64-token tiles, whose steps
+    // are short against the HBM latency)
+    static_assert(NSETS == 4 || NSETS == 8, "register sets");
     u32x4 wq[NSETS];
     u32x4 xr[NSETS][X_PER_THREAD];
     // Unconditional, clamped loads (exact s_waitcnt counts); what lies beyond k is zeroed in x.
@@ -187,7 +189,7 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     // iteration i (k-step s0 + i): stage step s0+i+1 into the other buffer, multiply from this one
 #define TUNA_TILED_ITER(i)                                                                       \
     {                                                                                          \
-        TUNA_TILED_STAGE(((i) + 1) & 3, ((i) + 1) & 1, s + (i) + 1)                            \
+        TUNA_TILED_STAGE(((i) + 1) % NSETS, ((i) + 1) & 1, s + (i) + 1)                        \
         TUNA_TILED_MFMA((i) & 1)                                                               \
         __syncthreads(); /* the staged tiles are complete; this step's tiles are free */       \
     }
@@ -196,17 +198,15 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     __syncthreads();  // decode table complete
     TUNA_TILED_STAGE(0, 0, s)
     __syncthreads();
-    for (; s + 3 < s1; s += 4) {
-        TUNA_TILED_ITER(0)
-        TUNA_TILED_ITER(1)
-        TUNA_TILED_ITER(2)
-        TUNA_TILED_ITER(3)
+    for (; s + NSETS - 1 < s1; s += NSETS) {
+#pragma unroll
+        for (int it = 0; it < NSETS; ++it) TUNA_TILED_ITER(it)  // (`it`: the macros use `i` inside)
     }
-    // tail: up to three more steps (the staging of a step past the end is harmless: its loads are
-    // clamped and nothing reads the tiles)
-    if (s < s1) TUNA_TILED_ITER(0)
-    if (s + 1 < s1) TUNA_TILED_ITER(1)
-    if (s + 2 < s1) TUNA_TILED_ITER(2)
+    // tail: up to NSETS - 1 more steps (the staging of a step past the end is harmless: its loads
+    // are clamped and nothing reads the tiles)
+#pragma unroll
+    for (int it = 0; it < NSETS - 1; ++it)
+        if (s + it < s1) TUNA_TILED_ITER(it)
 #undef TUNA_TILED_ITER
 #undef TUNA_TILED_MFMA
 #undef TUNA_TILED_STAGE
@@ -277,12 +277,12 @@ struct TiledVariant {
 };
 // (WM, TM, WN, TN): rows x tokens of the workgroup tile
 static const TiledVariant kTiled[] = {
-    {256, 128, gemm_tiled_kernel<4, 4, 2, 4>},
-    {256, 64, gemm_tiled_kernel<4, 4, 2, 2>},
-    {128, 256, gemm_tiled_kernel<2, 4, 4, 4>},
-    {128, 128, gemm_tiled_kernel<2, 4, 4, 2>},
-    {64, 256, gemm_tiled_kernel<1, 4, 8, 2>},
-    {64, 128, gemm_tiled_kernel<1, 4, 8, 1>},
+    {256, 128, gemm_tiled_kernel<4, 4, 2, 4, 4>},
+    {256, 64, gemm_tiled_kernel<4, 4, 2, 2, 8>},
+    {128, 256, gemm_tiled_kernel<2, 4, 4, 4, 4>},
+    {128, 128, gemm_tiled_kernel<2, 4, 4, 2, 4>},
+    {64, 256, gemm_tiled_kernel<1, 4, 8, 2, 4>},
+    {64, 128, gemm_tiled_kernel<1, 4, 8, 1, 4>},
 };
 static constexpr int kNumTiled = sizeof(kTiled) / sizeof(kTiled[0]);
 
