@@ -73,23 +73,14 @@ __device__ __forceinline__ f16x8 decode_dword(uint32_t d, const unsigned char *l
         const uint32_t a3 = __builtin_amdgcn_perm(d, lane4, 0x0c0c0700u);
         // The table starts at LDS address 0 (the kernel has no static LDS), so the
         // permuted value IS the LDS address: no base add per lookup.
-#if defined(TUNA_ABLATE) && TUNA_ABLATE == 1  /* development only: no table reads */
-        const uint32_t t0 = a0, t1 = a1, t2 = a2, t3 = a3;
-#else
         const uint32_t t0 = *reinterpret_cast<const lds_u32 *>((uintptr_t)a0);
         const uint32_t t1 = *reinterpret_cast<const lds_u32 *>((uintptr_t)a1);
         const uint32_t t2 = *reinterpret_cast<const lds_u32 *>((uintptr_t)a2);
         const uint32_t t3 = *reinterpret_cast<const lds_u32 *>((uintptr_t)a3);
-#endif
-#if defined(TUNA_ABLATE) && TUNA_ABLATE == 2  /* development only: no scale multiply */
-        const f16x2 h0 = __builtin_bit_cast(f16x2, t0), h1 = __builtin_bit_cast(f16x2, t1);
-        const f16x2 h2 = __builtin_bit_cast(f16x2, t2), h3 = __builtin_bit_cast(f16x2, t3);
-#else
         const f16x2 h0 = __builtin_bit_cast(f16x2, t0) * sc16;
         const f16x2 h1 = __builtin_bit_cast(f16x2, t1) * sc16;
         const f16x2 h2 = __builtin_bit_cast(f16x2, t2) * sc16;
         const f16x2 h3 = __builtin_bit_cast(f16x2, t3) * sc16;
-#endif
         f16x8 r;
         r[0] = h0[0]; r[1] = h0[1]; r[2] = h1[0]; r[3] = h1[1];
         r[4] = h2[0]; r[5] = h2[1]; r[6] = h3[0]; r[7] = h3[1];
@@ -211,33 +202,43 @@ __device__ __forceinline__ int k_physical(int k_logical, const KRot &kr)
     return kp >= kr.hi_k ? kp - kr.span_k : kp;
 }
 
+// A workgroup has a multiple of 16*TT threads, so the XB pieces of a thread (p = tid + b*nthreads)
+// all belong to the same token row r = tid % (16*TT) and their 8-k slots differ by the uniform
+// nthreads / (16*TT): one row offset and one slot per thread are all that is kept in registers.
 template <int TT, int XB>
-__device__ __forceinline__ void x_stage_load(XStage<XB> &st, const f16 *xg, int base, int nthreads, int tid, int pieces,
-                                             int tok0, int kbase, int n, int k, const KRot &kr)
+__device__ __forceinline__ void x_stage_load(XStage<XB> &st, const f16 *xg, int nthreads, int tid, int tok0, int kbase, int n,
+                                             int k, const KRot &kr)
 {
+    const int r = tid & (16 * TT - 1);
+    const int c8k = (tid / (16 * TT)) * 8;
+    const int slot_step = nthreads / (16 * TT);
+    // uniform 64-bit base (the tile's first token row) + a 32-bit per-lane offset: a tile spans
+    // at most 16*TT rows, so the offset fits and no 64-bit address lives in vector registers.
+    // Rows past n and slots past the chunk or k are clamped here and zeroed by x_stage_store.
+    const unsigned char *row0 = reinterpret_cast<const unsigned char *>(xg + (size_t)tok0 * k);
+    const uint32_t row_off = (uint32_t)(min(r, n - 1 - tok0) * k);
 #pragma unroll
     for (int b = 0; b < XB; ++b) {
-        const int p = min(base + b * nthreads + tid, pieces - 1);
-        const int r = p & (16 * TT - 1);
-        const int c8 = p / (16 * TT);
-        const int tok = min(tok0 + r, n - 1);
-        const int kk = min(k_physical(kbase + c8 * 8, kr), k - 8);
-        st.v[b] = *reinterpret_cast<const u32x4 *>(xg + (size_t)tok * k + kk);
+        const int kb = kbase + b * slot_step * 8;  // uniform part of the piece's k: stays in scalar registers
+        const int kk = min(k_physical(kb + c8k, kr), k - 8);
+        st.v[b] = *reinterpret_cast<const u32x4 *>(row0 + (row_off + (uint32_t)kk) * 2u);
     }
 }
 
 template <int TT, int XB>
-__device__ __forceinline__ void x_stage_store(const XStage<XB> &st, unsigned char *xs, int base, int nthreads, int tid,
-                                              int pieces, int tok0, int kbase, int n, int k, const KRot &kr)
+__device__ __forceinline__ void x_stage_store(const XStage<XB> &st, unsigned char *xs, int nthreads, int tid, int pieces,
+                                              int tok0, int kbase, int n, int k, const KRot &kr)
 {
+    const int r = tid & (16 * TT - 1);
+    const int c8k = (tid / (16 * TT)) * 8;
+    const int slot_step = nthreads / (16 * TT);
+    const bool row_ok = tok0 + r < n;
 #pragma unroll
     for (int b = 0; b < XB; ++b) {
-        const int p = base + b * nthreads + tid;
+        const int p = b * nthreads + tid;
         if (p < pieces) {
-            const int r = p & (16 * TT - 1);
-            const int c8 = p / (16 * TT);
-            const int kl = kbase + c8 * 8;
-            const bool ok = (tok0 + r < n) && kl < kr.hi_k && k_physical(kl, kr) < k;
+            const int kl = (kbase + b * slot_step * 8) + c8k;
+            const bool ok = row_ok && kl < kr.hi_k && k_physical(kl, kr) < k;
             *reinterpret_cast<u32x4 *>(xs + (size_t)p * 16) = ok ? st.v[b] : u32x4{0u, 0u, 0u, 0u};
         }
     }
@@ -401,7 +402,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
             sc32c[rw][j] = a.absmax[min(row_, a.m - 1)]; /* rows past m are never stored */    \
         }                                                                                      \
         krot = KRot{rot * kStepK, seg_hi * kStepK, nsteps * kStepK};                           \
-        x_stage_load<TT, XB>(xst, xg, 0, nthreads, tid, x_pieces, tok0, sb * kStepK, n_tok, a.k, krot); \
+        x_stage_load<TT, XB>(xst, xg, nthreads, tid, tok0, sb * kStepK, n_tok, a.k, krot); \
     }
 
     int t = t_begin;
@@ -410,10 +411,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     if (t < t_end) TUNA_TILE_FETCH(t)
     TUNA_MARK(1)
 
-
-#ifndef TUNA_DWORD_GROUP
-#define TUNA_DWORD_GROUP 0
-#endif
     // One k-step of this wave: B fragments from LDS, decode 4*RW dwords, 4*RW*TT MFMAs.
 #define TUNA_CONSUME(u, xoff)                                                                   \
     {                                                                                          \
@@ -495,7 +492,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 
         // the work area is free again once every wave has left the previous tile's epilogue
         __syncthreads();
-        if (n_chunks > 0) x_stage_store<TT, XB>(xst, work, 0, nthreads, tid, x_pieces, cur_tok0, cur_sb * kStepK, cur_ntok, a.k, krot);
+        if (n_chunks > 0) x_stage_store<TT, XB>(xst, work, nthreads, tid, x_pieces, cur_tok0, cur_sb * kStepK, cur_ntok, a.k, krot);
         __syncthreads();
         TUNA_MARK(3)
 
@@ -512,10 +509,10 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                 // that after the group exactly U*RW younger loads are in flight and the wait before
                 // the LDS write below is an exact vmcnt, not a drain of the weight ring.
                 const int kbase = (cur_sb + (c + 1) * a.chunk_steps) * kStepK;
-                x_stage_load<TT, XB>(xst, xg, 0, nthreads, tid, x_pieces, cur_tok0, kbase, cur_ntok, a.k, krot);
+                x_stage_load<TT, XB>(xst, xg, nthreads, tid, cur_tok0, kbase, cur_ntok, a.k, krot);
                 TUNA_GROUP()
                 __syncthreads();  // every wave is done reading chunk c
-                x_stage_store<TT, XB>(xst, work, 0, nthreads, tid, x_pieces, cur_tok0, kbase, cur_ntok, a.k, krot);
+                x_stage_store<TT, XB>(xst, work, nthreads, tid, x_pieces, cur_tok0, kbase, cur_ntok, a.k, krot);
                 __syncthreads();
             } else {
                 const int it_end = min(it_chunk0 + ipc, n_it);
