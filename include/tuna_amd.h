@@ -51,6 +51,13 @@ enum {
  *                       reference dequant op writes (kernel.cu:3222-3228).        */
 enum { TUNA_DECODE_GEMM = 1, TUNA_DECODE_DEQUANT = 2 };
 
+/* What happens to the fp32 sums before they are stored (tuna_matmul_fused).
+ * TUNA_EPILOGUE_RESIDUAL : out = fp16(sum + residual), residual fp16 [n, m] (may be `out` itself).
+ * TUNA_EPILOGUE_SILU_MUL : for a combined gate+up projection whose weight rows are interleaved
+ *                          (row 2i = gate_i, row 2i+1 = up_i): out [n, m/2] with
+ *                          out[t, i] = fp16(silu(sum[t, 2i]) * sum[t, 2i+1]).               */
+enum { TUNA_EPILOGUE_NONE = 0, TUNA_EPILOGUE_RESIDUAL = 1, TUNA_EPILOGUE_SILU_MUL = 2 };
+
 /* Tile configuration of one GEMM launch: the CDNA4 counterpart of the reference's
  * KernelConfig (configs.cu:12-54).  A workgroup is waves_m x waves_k wave64s; a wave
  * owns rows_per_wave weight rows and walks k in steps of 32; the workgroup owns
@@ -96,6 +103,14 @@ int tuna_matmul(const void *q, const void *x, const void *code, const void *absm
 int tuna_matmul_ex(const void *q, const void *x, const void *code, const void *absmax,
                    void *out, int m, int n, int k, const tuna_gemm_config *cfg,
                    int decode_mode, void *stream);
+
+/* tuna_matmul_ex with a fused epilogue (the step after the GEMM in a decoder layer: the
+ * residual add after the attention-out / down projections, SiLU(gate) * up after the combined
+ * gate+up projection), saving a launch and a round trip of the activations through HBM.
+ * `residual` is read only with TUNA_EPILOGUE_RESIDUAL.  No counterpart in the reference. */
+int tuna_matmul_fused(const void *q, const void *x, const void *code, const void *absmax,
+                      void *out, int m, int n, int k, const tuna_gemm_config *cfg,
+                      int decode_mode, int epilogue, const void *residual, void *stream);
 
 /* Grouped GEMM (mixture of experts with per-expert token lists) in one launch.  The weights
  * are n_groups (<= 64) matrices of m_group rows stacked along m - q [n_groups*m_group/8, k/8,

@@ -584,3 +584,52 @@ def test_quantize_then_matmul_end_to_end():
     ref = O.gemm_f64(q.cpu().numpy(), x, code.cpu().numpy(), absmax.cpu().numpy(), m, n, k, mode=O.D1)
     e = rel_err(out.cpu().numpy().astype(np.float64), ref)
     assert e <= REL_TOL, e
+
+
+# ----------------------------------------------------------------------------- fused epilogues
+FUSED_CFGS = [
+    dict(),                                                              # in-workgroup k split, direct store
+    dict(split_k=3, x_chunk=512),                                        # cross-workgroup split: finishing workgroup stores
+    dict(waves_m=8, waves_k=1, prefetch=2, x_chunk=64),                  # register-store epilogue
+    dict(split_k=0, waves_m=1, waves_k=8, prefetch=2, x_chunk=512),      # balanced split
+    dict(lds_tile_rows=128, token_tiles=8, split_k=1),                   # many-token kernel
+    dict(lds_tile_rows=64, token_tiles=8, split_k=2),                    # many-token kernel, split-K
+]
+
+
+@pytest.mark.parametrize("ci", range(len(FUSED_CFGS)))
+def test_fused_residual_and_silu_mul_epilogues(ci):
+    """out = fp16(sum + residual) (also in place) and out = fp16(silu(gate) * up) on interleaved
+    gate/up rows, against the oracle's float64 sums pushed through the same formulas."""
+    import torch
+
+    from tuna_amd import _lib, ops
+
+    m, n, k = 1024, 48, 1096
+    c = cfg(**FUSED_CFGS[ci])
+    print(f"fused cfg#{ci} {c.to_dict()}", flush=True)
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=60 + ci)
+    rng = np.random.default_rng(ci)
+    res = (rng.standard_normal((n, m)) * 0.05).astype(np.float16)
+    ref = O.gemm_f64(q, x, code, absmax, m, n, k, mode=O.D1)
+    dq, dx, dc, da, dres = to_dev(q, x, code, absmax, res)
+    # residual, separate output
+    out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+    ops.matmul_fused(dx, dq, da, dc, out, m, n, k, _lib.EPILOGUE_RESIDUAL, residual=dres, config=c)
+    torch.cuda.synchronize()
+    want = ref + res.astype(np.float64)
+    assert rel_err(out.cpu().numpy().astype(np.float64), want) <= REL_TOL
+    # residual in place: out is the residual
+    inplace = dres.clone()
+    ops.matmul_fused(dx, dq, da, dc, inplace, m, n, k, _lib.EPILOGUE_RESIDUAL, residual=inplace, config=c)
+    torch.cuda.synchronize()
+    assert torch.equal(inplace.view(torch.int16), out.view(torch.int16))
+    # silu(gate) * up on interleaved rows
+    out2 = torch.full((n, m // 2), float("nan"), dtype=torch.float16, device="cuda")
+    ops.matmul_fused(dx, dq, da, dc, out2, m, n, k, _lib.EPILOGUE_SILU_MUL, config=c)
+    torch.cuda.synchronize()
+    g, u = ref[:, 0::2], ref[:, 1::2]
+    want2 = g / (1.0 + np.exp(-g)) * u
+    # a product of two sums that are each within tolerance: relative to an output, the error of a
+    # near-zero factor is amplified, so the floor of the metric is the wider one (5e-2 of the largest output)
+    assert rel_err(out2.cpu().numpy().astype(np.float64), want2, floor=REL_FLOOR_D2) <= REL_TOL

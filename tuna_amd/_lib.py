@@ -21,6 +21,7 @@ ERR_WORKSPACE = 5
 
 DECODE_GEMM = 1
 DECODE_DEQUANT = 2
+EPILOGUE_NONE, EPILOGUE_RESIDUAL, EPILOGUE_SILU_MUL = 0, 1, 2
 
 
 class GemmConfig(ctypes.Structure):
@@ -61,6 +62,7 @@ SIGNATURES = {
     "tuna_last_error": (ctypes.c_char_p, []),
     "tuna_matmul": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "tuna_matmul_ex": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _vp]),
+    "tuna_matmul_fused": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _i, _vp, _vp]),
     "tuna_matmul_grouped": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _ip, _cfgp, _i, _vp]),
     "tuna_dequant": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "tuna_quantize": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),

@@ -395,10 +395,14 @@ extern "C" __attribute__((visibility("default"))) void tuna_set_trace(void *p) {
 #endif
 
 static int matmul_impl(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n, int k,
-                       const tuna_gemm_config *cfg, int decode, hipStream_t stream)
+                       const tuna_gemm_config *cfg, int decode, hipStream_t stream, int epilogue = TUNA_EPILOGUE_NONE,
+                       const void *residual = nullptr)
 {
     int rc;
     if ((rc = check_shape(m, n, k))) return rc;
+    if (epilogue != TUNA_EPILOGUE_NONE && epilogue != TUNA_EPILOGUE_RESIDUAL && epilogue != TUNA_EPILOGUE_SILU_MUL)
+        return fail(TUNA_ERR_INVALID_ARG, "epilogue %d is not a TUNA_EPILOGUE_* value", epilogue);
+    if (epilogue == TUNA_EPILOGUE_RESIDUAL && (rc = check_ptr(residual, "residual", 8))) return rc;
     if ((rc = check_ptr(q, "q", 16)) || (rc = check_ptr(x, "x", 16)) || (rc = check_ptr(code, "code", 4)) ||
         (rc = check_ptr(absmax, "absmax", 4)) || (rc = check_ptr(out, "out", 16)))
         return rc;
@@ -419,6 +423,8 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
         tp.args.code = static_cast<const float *>(code);
         tp.args.absmax = static_cast<const float *>(absmax);
         tp.args.out = out;
+        tp.args.epilogue = epilogue;
+        tp.args.residual = residual;
         if (tp.ws_bytes) {
             Workspace w;
             if ((rc = get_workspace(stream, tp.ws_bytes, tp.n_counters, &w))) return rc;
@@ -436,6 +442,8 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
     plan.args.code = static_cast<const float *>(code);
     plan.args.absmax = static_cast<const float *>(absmax);
     plan.args.out = out;
+    plan.args.epilogue = epilogue;
+    plan.args.residual = residual;
     if (plan.ws_bytes) {
         Workspace w;
         if ((rc = get_workspace(stream, plan.ws_bytes, plan.n_counters, &w))) return rc;
@@ -649,6 +657,13 @@ TUNA_EXPORT int tuna_matmul_ex(const void *q, const void *x, const void *code, c
                                int k, const tuna_gemm_config *cfg, int decode_mode, void *stream)
 {
     return matmul_impl(q, x, code, absmax, out, m, n, k, cfg, decode_mode, static_cast<hipStream_t>(stream));
+}
+
+TUNA_EXPORT int tuna_matmul_fused(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n,
+                                  int k, const tuna_gemm_config *cfg, int decode_mode, int epilogue, const void *residual,
+                                  void *stream)
+{
+    return matmul_impl(q, x, code, absmax, out, m, n, k, cfg, decode_mode, static_cast<hipStream_t>(stream), epilogue, residual);
 }
 
 TUNA_EXPORT int tuna_matmul_grouped(const void *q, const void *x, const void *code, const void *absmax, void *out,

@@ -43,17 +43,10 @@
 //     output (unlike kernel.cu:2739-2745), no pre-zeroing, and the result does not depend
 //     on arrival order.
 #pragma once
-#include "tuna_internal.h"
+#include "epilogue.hpp"
 
 namespace tuna {
 
-typedef _Float16 f16;
-typedef f16 f16x2 __attribute__((ext_vector_type(2)));
-typedef f16 f16x4 __attribute__((ext_vector_type(4)));
-typedef f16 f16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) uint32_t lds_u32;
 
 __device__ __forceinline__ uint32_t f16_bits(f16 h)
 {
@@ -600,6 +593,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
             }
         }
         f16 *outp = reinterpret_cast<f16 *>(a.out);
+        const f16 *resp = reinterpret_cast<const f16 *>(a.residual);
         bool write_out = true;
         if (a.waves_k == 1 && !partial) {
             // No k split at all: the wave's accumulators are final.  Lane (token i16, group g)
@@ -611,17 +605,25 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 #pragma unroll
                 for (int rw = 0; rw < RW; ++rw) {
                     const int rb = cur_row_base + wm_e * (RW * kRowsPerLoad) + rw * 64 + (lane_e >> 4) * 16;
-                    f16x8 lo, hi;
+                    if (a.epilogue == TUNA_EPILOGUE_NONE) {
+                        f16x8 lo, hi;
 #pragma unroll
-                    for (int v = 0; v < 2; ++v)
+                        for (int v = 0; v < 2; ++v)
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            lo[v * 4 + j] = (f16)acc[rw][j][tt][v];
-                            hi[v * 4 + j] = (f16)acc[rw][j][tt][v + 2];
-                        }
-                    f16 *dst = outp + (size_t)tok * out_ld + (rb - cur_out_row0);
-                    if (tok < cur_ntok && rb + 8 <= a.m) *reinterpret_cast<f16x8 *>(dst) = lo;
-                    if (tok < cur_ntok && rb + 16 <= a.m) *reinterpret_cast<f16x8 *>(dst + 8) = hi;
+                            for (int j = 0; j < 4; ++j) {
+                                lo[v * 4 + j] = (f16)acc[rw][j][tt][v];
+                                hi[v * 4 + j] = (f16)acc[rw][j][tt][v + 2];
+                            }
+                        f16 *dst = outp + (size_t)tok * out_ld + (rb - cur_out_row0);
+                        if (tok < cur_ntok && rb + 8 <= a.m) *reinterpret_cast<f16x8 *>(dst) = lo;
+                        if (tok < cur_ntok && rb + 16 <= a.m) *reinterpret_cast<f16x8 *>(dst + 8) = hi;
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 4; ++v)
+                            if (tok < cur_ntok && rb + v * 4 + 4 <= a.m)
+                                store_features4(outp, resp, a.epilogue, (size_t)tok, out_ld, rb + v * 4 - cur_out_row0,
+                                                acc[rw][0][tt][v], acc[rw][1][tt][v], acc[rw][2][tt][v], acc[rw][3][tt][v]);
+                    }
                 }
             }
             ++tile_iter;
@@ -662,10 +664,9 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                         const int l = f >> 2, v = f & 3;
                         const int tok = cur_tok0 + tt * 16 + (l & 15);
                         const int row = cur_row_base + wm_e * (RW * kRowsPerLoad) + rw * 64 + (l >> 4) * 16 + v * 4;
-                        if (tok < cur_ntok && row + 4 <= a.m) {
-                            f16x4 h = {(f16)o[i][0], (f16)o[i][1], (f16)o[i][2], (f16)o[i][3]};
-                            *reinterpret_cast<f16x4 *>(outp + (size_t)tok * out_ld + (row - cur_out_row0)) = h;
-                        }
+                        if (tok < cur_ntok && row + 4 <= a.m)
+                            store_features4(outp, resp, a.epilogue, (size_t)tok, out_ld, row - cur_out_row0, o[i][0], o[i][1],
+                                            o[i][2], o[i][3]);
                     } else {
                         float *dst = mine + ((size_t)(rw * TT + tt) * 256 + f) * 4;
                         store_partial(dst, f32x4{o[i][0], o[i][1], o[i][2], o[i][3]});
@@ -724,10 +725,9 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                         const int l = f >> 2, v = f & 3;
                         const int tok = cur_tok0 + tt * 16 + (l & 15);
                         const int row = cur_row_base + wm_e * (RW * kRowsPerLoad) + rw * 64 + (l >> 4) * 16 + v * 4;
-                        if (tok < cur_ntok && row + 4 <= a.m) {
-                            f16x4 h = {(f16)s4[0], (f16)s4[1], (f16)s4[2], (f16)s4[3]};
-                            *reinterpret_cast<f16x4 *>(outp + (size_t)tok * out_ld + (row - cur_out_row0)) = h;
-                        }
+                        if (tok < cur_ntok && row + 4 <= a.m)
+                            store_features4(outp, resp, a.epilogue, (size_t)tok, out_ld, row - cur_out_row0, s4[0], s4[1], s4[2],
+                                            s4[3]);
                     }
             }
         }

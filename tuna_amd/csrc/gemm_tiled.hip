@@ -26,17 +26,10 @@
 //     bank exactly once - no padding, no bank conflicts;
 //   * fp32 accumulators stay in registers for the whole k range; a lane ends up with 4
 //     consecutive output features of one token per MFMA tile: 8-byte stores.
-#include "tuna_internal.h"
+#include "epilogue.hpp"
 
 namespace tuna {
 
-typedef _Float16 f16;
-typedef f16 f16x2 __attribute__((ext_vector_type(2)));
-typedef f16 f16x4 __attribute__((ext_vector_type(4)));
-typedef f16 f16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) uint32_t lds_u32;
 
 constexpr int kTiledThreads = 512;
 constexpr int kTiledStepK = 64;
@@ -215,6 +208,7 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     // ---- epilogue -----------------------------------------------------------------------------
     // acc[tm][tn][v] of lane l is weight row 4*(l/16) + v of MFMA tile tm, token l%16 of tile tn
     f16 *outp = reinterpret_cast<f16 *>(a.out);
+    const f16 *resp = reinterpret_cast<const f16 *>(a.residual);
     if (a.split_k == 1) {
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
@@ -224,7 +218,7 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
                 const int tok = tok_base + (wn_i * TN + tn) * 16 + i16;
                 if (tok < a.n && row + 4 <= a.m) {
                     const f32x4 v = acc[tm][tn];
-                    *reinterpret_cast<f16x4 *>(outp + (size_t)tok * a.m + row) = f16x4{(f16)v[0], (f16)v[1], (f16)v[2], (f16)v[3]};
+                    store_features4(outp, resp, a.epilogue, (size_t)tok, a.m, row, v[0], v[1], v[2], v[3]);
                 }
             }
         }
@@ -264,8 +258,7 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
 #pragma unroll
                 for (int j = 0; j < 4; ++j) s4[j] += __hip_atomic_load(p + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
-            if (tok < a.n && row + 4 <= a.m)
-                *reinterpret_cast<f16x4 *>(outp + (size_t)tok * a.m + row) = f16x4{(f16)s4[0], (f16)s4[1], (f16)s4[2], (f16)s4[3]};
+            if (tok < a.n && row + 4 <= a.m) store_features4(outp, resp, a.epilogue, (size_t)tok, a.m, row, s4[0], s4[1], s4[2], s4[3]);
         }
     }
 }

@@ -27,6 +27,8 @@ struct GemmArgs {
     const float *code;
     const float *absmax;
     void *out;
+    const void *residual;  // fp16, layout of out: added before the final rounding (TUNA_EPILOGUE_RESIDUAL)
+    int epilogue;          // TUNA_EPILOGUE_*
     float *ws;           // split-K partial sums (library owned), may be null if split_k == 1
     unsigned *counters;  // one arrival counter per (token chunk, row tile), zero between launches
     int m, n, k;
@@ -119,6 +121,8 @@ struct TiledArgs {
     const float *code;
     const float *absmax;
     void *out;
+    const void *residual;  // as in GemmArgs
+    int epilogue;
     float *ws;           // split-K partial tiles (library owned), unused if split_k == 1
     unsigned *counters;  // one arrival counter per tile, zero between launches
     int m, n, k;

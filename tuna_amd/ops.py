@@ -66,6 +66,32 @@ def matmul(x, q, s, c, o, m: int, n: int, k: int, config: GemmConfig = None,
     _lib.check(rc)
 
 
+def matmul_fused(x, q, s, c, o, m: int, n: int, k: int, epilogue: int, residual=None, config: GemmConfig = None,
+                 decode_mode: int = _lib.DECODE_GEMM) -> None:
+    """matmul with a fused epilogue (tuna_matmul_fused).
+
+    EPILOGUE_RESIDUAL: o[n, m] = fp16(x @ W^T + residual), residual fp16 [n, m] (may be o).
+    EPILOGUE_SILU_MUL: weight rows interleaved (2i: gate_i, 2i+1: up_i); o[n, m/2] =
+    fp16(silu(gate) * up)."""
+    m, n, k = int(m), int(n), int(k)
+    _require(x, "x", torch.float16, n * k)
+    _require(q, "q", torch.uint8, m * k // 2)
+    _require(s, "s", torch.float32, m)
+    _require(c, "c", torch.float32, 16)
+    _require(o, "o", torch.float16, n * (m // 2 if epilogue == _lib.EPILOGUE_SILU_MUL else m))
+    rp = None
+    if epilogue == _lib.EPILOGUE_RESIDUAL:
+        if residual is None:
+            raise ValueError("EPILOGUE_RESIDUAL needs a residual tensor")
+        _require(residual, "residual", torch.float16, n * m)
+        rp = residual.data_ptr()
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().tuna_matmul_fused(q.data_ptr(), x.data_ptr(), c.data_ptr(), s.data_ptr(), o.data_ptr(), m, n, k,
+                                          ctypes.byref(config) if config is not None else None, int(decode_mode),
+                                          int(epilogue), rp, _stream(x.device))
+    _lib.check(rc)
+
+
 def matmul_grouped(x, q, s, c, o, m_group: int, n_groups: int, k: int, token_offsets, config: GemmConfig = None,
                    decode_mode: int = _lib.DECODE_GEMM) -> None:
     """Grouped GEMM (mixture of experts): o[t, :] = x[t, :] @ decode(W_e)^T for the tokens t of
