@@ -43,8 +43,8 @@ CACHE_BYTES = 256 << 20  # Infinity Cache; the rotation streams at least twice t
 # the summaries under profiles/.  None = not measured for that shape.
 MEASURED_TRAFFIC_BYTES = {
     # workload: FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 (KiB -> bytes), profiles/gemm_kernel_hbm_traffic_counters.md
-    "mistral_qkv": int((7243.1 * 2.000 + 969.0 * 1.000) * 1024),
-    "mixtral_gate_up_8e": int((230451.8 * 2.000 + 7168.0 * 1.000) * 1024),
+    "mistral_qkv": int((7596.0 * 2.000 + 1735.5 * 1.000) * 1024),
+    "mixtral_gate_up_8e": int((230457.9 * 2.000 + 7168.0 * 1.000) * 1024),
 }
 
 
