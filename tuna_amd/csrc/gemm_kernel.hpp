@@ -30,18 +30,33 @@
 //     rounding as the reference's `smemCode.get(nib) * absMax` (kernel.cu:2178-2192).
 //     Cost: 1 perm + 1 ds_read_b32 + 1 pk_mul per two weights.
 //   * Persistent workgroups: the grid is at most (CUs x workgroups per CU); a workgroup
-//     builds the decode table once and then walks tiles (row tile, k split) with stride
-//     gridDim.x.  The next tile's scales, weight ring and first x chunk are requested
-//     BEFORE the current tile's reduction and store, so the HBM stream never idles between
-//     tiles and the epilogue's latency is hidden behind the loads already in flight.
-//   * Split-K: waves_k waves of a workgroup cover interleaved k-steps; their accumulators
-//     meet in LDS and every thread sums a 1/waves_k share in wave order.  split_k
-//     workgroups write those fp32 sums to a workspace and the last one to arrive
-//     (device-scope counter) adds them in split order.  After the four planes of a 64-row
-//     group a thread owns 4 consecutive output features of one token: 8-byte stores, 32
-//     contiguous bytes per 4 lanes.  No atomics on the
-//     output (unlike kernel.cu:2739-2745), no pre-zeroing, and the result does not depend
-//     on arrival order.
+//     builds the decode table once (while its first tile's loads are in flight) and then
+//     walks tiles (row tile, k segment).  The next tile's weight ring is requested BEFORE
+//     the current tile's reduction and store, so the HBM stream never idles between tiles;
+//     the small operands (row scales, first x chunk - mostly L2 hits) follow at the start of
+//     the tile, where they do not hold registers across the epilogue.
+//   * Split-K inside a workgroup: waves_k waves cover interleaved k-steps; their
+//     accumulators meet in LDS and every thread sums a 1/waves_k share in wave order.  After
+//     the four planes of a 64-row group a thread owns 4 consecutive output features of one
+//     token.  With waves_k == 1 and no k split the accumulators are stored straight from
+//     registers (16-byte stores, no LDS, no barrier).
+//   * Split-K across workgroups, two schemes.  Fixed (split_k >= 1): tile t is (row tile
+//     t / split_k, part t % split_k), parts of equal length.  Balanced (split_k == 0): the
+//     k-steps of all row tiles, in units of 2^unit_log2 steps, are laid end to end and cut
+//     into one contiguous range per workgroup, so every workgroup streams the same number
+//     of bytes; a range covers whole row tiles plus at most two partial segments.  Either
+//     way partial fp32 sums go to a workspace with device-coherent stores and the last
+//     contributor to arrive (device-scope ticket counter) adds them in k order.  No atomics
+//     on the output (unlike kernel.cu:2739-2745), no pre-zeroing, and the result does not
+//     depend on arrival order.
+//   * k_stagger: row tile r starts r * k_stagger steps into its k segment and wraps, so
+//     that workgroups running side by side do not all walk the same 2^n-strided columns of
+//     the weight matrix (and the same HBM channels) in lockstep.
+//   * GRP variants (grouped GEMM, one weight matrix per group of tokens): row tiles count
+//     over the groups that have tokens; the token range, output column base and weight rows
+//     of a tile come from the group's entry of the offset list in the kernel arguments.
+//   * The store applies the fused epilogue (none / + residual / SiLU(gate) * up on
+//     interleaved rows), see epilogue.hpp.
 #pragma once
 #include "epilogue.hpp"
 
