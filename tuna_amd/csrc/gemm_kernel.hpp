@@ -252,9 +252,15 @@ __device__ __forceinline__ void x_stage_store(const XStage<XB> &st, unsigned cha
     }
 }
 
-template <int RW, int U, int TT, int DEC, int MAXT, int MINW, bool GRP>
+// MODE 0: persistent workgroups walking tiles; 1: the same for grouped launches (GRP below);
+// 2: the launch has one workgroup per tile and a fixed split (ONE below) - no tile walk, no
+// balanced split: the lean path for the small shapes, whose time is instruction issue between
+// the first and the last memory access rather than bandwidth.
+template <int RW, int U, int TT, int DEC, int MAXT, int MINW, int MODE>
 __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 {
+    constexpr bool GRP = MODE == 1;
+    constexpr bool ONE = MODE == 2;
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int NACC = RW * 4 * TT;  // float4 accumulator planes per lane
     constexpr int LUT_B = (DEC == TUNA_DECODE_GEMM) ? kLutBytes : 64;
@@ -262,14 +268,34 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 
     const int tid = threadIdx.x;
 #ifdef TUNA_TRACE
-#define TUNA_MARK(i) if (a.trace && tid == 0 && tile_iter < 8) a.trace[((size_t)blockIdx.x * 8 + tile_iter) * 16 + (i)] = wall_clock64();
+    // development builds: timestamps of the first tile go to 128 bytes of LDS behind the launch's
+    // own (global stores up here would turn the codebook's scalar loads into vector loads) and
+    // are copied out at the end of the tile
+    const unsigned long long t_entry_ = wall_clock64();
+#define TUNA_MARK(i) if (tid == 0 && tile_iter == 0) reinterpret_cast<unsigned long long *>(smem + a.lds_bytes)[i] = (i) == 0 ? t_entry_ : wall_clock64();
 #else
 #define TUNA_MARK(i)
 #endif
     int tile_iter = 0;
+#ifdef TUNA_TRACE
+    if (tid < 32) reinterpret_cast<unsigned long long *>(smem + a.lds_bytes)[tid] = 0ull;
+#endif
     TUNA_MARK(0)
+    // Every kernel argument the first tile needs is requested here, in one batch with one wait:
+    // left to itself the compiler fetches them where they are first used, three to four
+    // dependent round trips to memory before the first weight load can be issued.  (Not a
+    // volatile asm: that would count as a store and turn the codebook's scalar loads below
+    // into vector loads.  Its result, zero, is folded into the wave index to pin it here.)
+    int args_here;
+    asm("s_mov_b32 %0, 0"
+        : "=s"(args_here)
+        : "s"(a.q), "s"(a.x), "s"(a.code), "s"(a.absmax), "s"(a.ws), "s"(a.counters), "s"(a.epilogue), "s"(a.m), "s"(a.n), "s"(a.k), "s"(a.waves_m), "s"(a.waves_k),
+          "s"(a.split_k), "s"(a.wk_log2), "s"(a.steps_total), "s"(a.steps_per_split), "s"(a.chunk_steps), "s"(a.chunk_log2),
+          "s"(a.row_tiles), "s"(a.xcd_swizzle), "s"(a.k_stagger), "s"(a.tiles_total), "s"(a.balanced), "s"(a.unit_log2),
+          "s"(a.units_per_tile), "s"(a.units_total), "s"(gridDim.x), "s"(blockDim.x));
+    const bool bal = ONE ? false : (a.balanced != 0);
     const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6) + args_here;
     const int wk = wave & (a.waves_k - 1);
     const int wm = wave >> a.wk_log2;
     const int i16 = lane & 15;
@@ -414,10 +440,65 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     }
 
     int t = t_begin;
-    const float code_lane = a.code[lane & 15];
+    // The 16 codes are uniform and read before the kernel's first store, so they come through
+    // the scalar cache: waiting for them does not wait for the weight loads (vector loads
+    // return in order).
+    const float *__restrict__ code_ptr = a.code;
+    float code_s[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) code_s[i] = code_ptr[i];
+    // scales and first x chunk of the tile about to be computed (requested right behind its
+    // weight ring: at the start for the first tile, after the epilogue for the following ones)
+    float sc32c[RW][4] = {};
+    KRot krot{0, 0, 0};
     TUNA_SKIP_EMPTY(t)
-    if (t < t_end) TUNA_TILE_FETCH(t)
-    TUNA_MARK(1)
+    if (t < t_end) {
+        TUNA_TILE_FETCH(t)
+#if defined(TUNA_TRACE) && TUNA_TRACE_EXP == 1
+        TUNA_MARK(16)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        TUNA_MARK(17)
+#endif
+        if constexpr (!GRP) TUNA_TILE_SMALL_LOADS()
+#if defined(TUNA_TRACE) && TUNA_TRACE_EXP == 2
+        TUNA_MARK(16)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        TUNA_MARK(17)
+#endif
+        TUNA_MARK(1)
+        // ---- decode table, once per workgroup, built while the first tile's loads are in flight
+        float code_lane = 0.f;  // (a select between two loads would be turned back into a vector load)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) code_lane = i16 == i ? code_s[i] : code_lane;
+        TUNA_MARK(14)
+        if constexpr (DEC == TUNA_DECODE_GEMM) {
+            // Lane l holds fp16(code[l % 16]) (kernel.cu:2800 rounds the codebook to fp16);
+            // entries are gathered across lanes, no memory traffic.
+            // piece p: 16 bytes of row (p >> 4); all 64 slots of a row hold the same half2
+            const int code_bits = (int)f16_bits((f16)code_lane);
+            TUNA_MARK(15)
+            // four pieces per thread and round: the eight cross-lane reads of a round are in
+            // flight together instead of one LDS round trip per piece
+            for (int p0 = tid; p0 < kLutBytes / 16; p0 += 4 * nthreads) {
+                uint32_t v[4];
+    #pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const int e = (p0 + b * nthreads) >> 4;
+                    const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute((e >> 4) << 2, code_bits);
+                    const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute((e & 15) << 2, code_bits);
+                    v[b] = hi | (lo << 16);
+                }
+    #pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const int p = p0 + b * nthreads;
+                    if (p < kLutBytes / 16) reinterpret_cast<u32x4 *>(lut)[p] = u32x4{v[b], v[b], v[b], v[b]};
+                }
+            }
+        } else {
+            if (tid < 16) reinterpret_cast<float *>(lut)[tid] = code_lane;
+        }
+        TUNA_MARK(2)
+    }
 
     // One k-step of this wave: B fragments from LDS, decode 4*RW dwords, 4*RW*TT MFMAs.
 #define TUNA_CONSUME(u, xoff)                                                                   \
@@ -451,32 +532,11 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     const int wstep = a.waves_k * (1024 * TT);   // LDS bytes between this wave's consecutive steps
 
     while (t < t_end) {
+        // (grouped variants request them here for every tile: with a second place of request
+        // the compiler keeps two copies of the staging registers)
+        if constexpr (GRP) TUNA_TILE_SMALL_LOADS()
         // ---- this tile's scales (fp16 like the reference's staging, kernel.cu:2770) and the
         //      first x chunk, requested behind the ring loads already in flight
-        float sc32c[RW][4];
-        KRot krot;
-        TUNA_TILE_SMALL_LOADS()
-        if (tile_iter == 0) {
-            // (placed here so that the first tile's loads are all in flight while it is built)
-            // ---- decode table, once per workgroup ------------------------------------------------
-            if constexpr (DEC == TUNA_DECODE_GEMM) {
-                // Lane l holds fp16(code[l % 16]) (kernel.cu:2800 rounds the codebook to fp16);
-                // entries are gathered across lanes, no memory traffic.
-                // piece p: 16 bytes of row (p >> 4); all 64 slots of a row hold the same half2
-                const int code_bits = (int)f16_bits((f16)code_lane);
-#pragma unroll 4
-                for (int p = tid; p < kLutBytes / 16; p += nthreads) {
-                    const int e = p >> 4;
-                    const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute((e >> 4) << 2, code_bits);
-                    const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute((e & 15) << 2, code_bits);
-                    const uint32_t v = hi | (lo << 16);
-                    reinterpret_cast<u32x4 *>(lut)[p] = u32x4{v, v, v, v};
-                }
-            } else {
-                if (tid < 16) reinterpret_cast<float *>(lut)[tid] = code_lane;
-            }
-        }
-        TUNA_MARK(2)
         f16x2 sc16[RW][4];
 #pragma unroll
         for (int rw = 0; rw < RW; ++rw)
@@ -548,15 +608,19 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
         }
         TUNA_MARK(4)
 #ifdef TUNA_TRACE
-        if (a.trace && lane == 0 && tile_iter < 8) {  // latest wave of the workgroup out of the main loop
-            atomicMax(&a.trace[((size_t)blockIdx.x * 8 + tile_iter) * 16 + 10], (unsigned long long)wall_clock64());
+        if (lane == 0 && tile_iter == 0) {  // latest wave of the workgroup out of the main loop
+            atomicMax(reinterpret_cast<unsigned long long *>(smem + a.lds_bytes) + 10, (unsigned long long)wall_clock64());
         }
 #endif
 
         // ---- next tile: get its loads going before this tile's reduction and store ---------
-        t = t_next;
-        TUNA_SKIP_EMPTY(t)
-        if (t < t_end) TUNA_TILE_FETCH(t)
+        if constexpr (ONE) {
+            t = t_end;
+        } else {
+            t = t_next;
+            TUNA_SKIP_EMPTY(t)
+            if (t < t_end) TUNA_TILE_FETCH(t)
+        }
 
         // ---- workgroup reduction and store ---------------------------------------------------
         // A plane is one float4 per lane = 256 floats [lane][4].  The waves_k waves of a row
@@ -641,7 +705,13 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                     }
                 }
             }
+#ifdef TUNA_TRACE
+            TUNA_MARK(9)
+            if (a.trace && tid < 32 && tile_iter == 0)
+                a.trace[(size_t)blockIdx.x * 8 * 16 + tid] = reinterpret_cast<unsigned long long *>(smem + a.lds_bytes)[tid];
+#endif
             ++tile_iter;
+            if constexpr (MODE == 0) if (t < t_end) TUNA_TILE_SMALL_LOADS()
             continue;
         }
         __syncthreads();  // every wave has left the main loop: the work area is free
@@ -748,7 +818,12 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
         }
         TUNA_MARK(8)
         TUNA_MARK(9)
+#ifdef TUNA_TRACE
+        if (a.trace && tid < 32 && tile_iter == 0)
+            a.trace[(size_t)blockIdx.x * 8 * 16 + tid] = reinterpret_cast<unsigned long long *>(smem + a.lds_bytes)[tid];
+#endif
         ++tile_iter;
+        if constexpr (MODE == 0) if (t < t_end) TUNA_TILE_SMALL_LOADS()
     }
 #undef TUNA_GROUP
 #undef TUNA_CONSUME

@@ -8,12 +8,13 @@ namespace tuna {
 typedef void (*GemmKernelFn)(const GemmArgs);
 
 struct Variant {
-    int rw, u, tt, dec, maxt, minw, grouped;
+    int rw, u, tt, dec, maxt, minw, mode;  // mode: 0 tile walk, 1 grouped tile walk, 2 one tile per workgroup
     GemmKernelFn fn;
 };
 
-#define V(RW, U, TT, DEC, MAXT, MINW) {RW, U, TT, DEC, MAXT, MINW, 0, gemm_kernel<RW, U, TT, DEC, MAXT, MINW, false>}
-#define VG(RW, U, TT, DEC, MAXT, MINW) {RW, U, TT, DEC, MAXT, MINW, 1, gemm_kernel<RW, U, TT, DEC, MAXT, MINW, true>}
+#define V(RW, U, TT, DEC, MAXT, MINW) {RW, U, TT, DEC, MAXT, MINW, 0, gemm_kernel<RW, U, TT, DEC, MAXT, MINW, 0>}
+#define VG(RW, U, TT, DEC, MAXT, MINW) {RW, U, TT, DEC, MAXT, MINW, 1, gemm_kernel<RW, U, TT, DEC, MAXT, MINW, 1>}
+#define V1(RW, U, TT, DEC, MAXT, MINW) {RW, U, TT, DEC, MAXT, MINW, 2, gemm_kernel<RW, U, TT, DEC, MAXT, MINW, 2>}
 #define G TUNA_DECODE_GEMM
 
 // Only variants whose main loop compiles without register spills are listed (a spill in the
@@ -38,19 +39,25 @@ static const Variant kVariants[] = {
     VG(1, 2, 1, G, 512, 4), VG(1, 4, 1, G, 512, 4), VG(1, 2, 1, G, 1024, 4), VG(1, 4, 1, G, 1024, 4),
     VG(1, 2, 1, TUNA_DECODE_DEQUANT, 512, 2), VG(1, 2, 2, TUNA_DECODE_DEQUANT, 512, 2),
     VG(1, 2, 4, TUNA_DECODE_DEQUANT, 512, 2),
+    // one workgroup per tile (launches that fit the device in one round, fixed split): optional
+    // twins of dense variants, picked by launch_gemm when they apply
+    V1(1, 2, 1, G, 512, 2), V1(1, 2, 2, G, 512, 2), V1(1, 4, 1, G, 512, 2), V1(1, 4, 2, G, 512, 2),
+    V1(1, 8, 1, G, 512, 2), V1(2, 2, 1, G, 512, 2), V1(2, 4, 1, G, 512, 2),
+    V1(1, 2, 1, G, 512, 4), V1(1, 4, 1, G, 512, 4), V1(1, 2, 1, G, 1024, 4), V1(1, 4, 1, G, 1024, 4),
 };
 #undef V
 #undef VG
+#undef V1
 #undef G
 static constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
-static const Variant *find_variant(int rw, int u, int tt, int dec, int threads, int minw, int grouped)
+static const Variant *find_variant(int rw, int u, int tt, int dec, int threads, int minw, int mode)
 {
     const int maxt = threads <= 512 ? 512 : 1024;
     if (maxt == 1024) minw = 4;
     for (int i = 0; i < kNumVariants; ++i) {
         const Variant &v = kVariants[i];
-        if (v.rw == rw && v.u == u && v.tt == tt && v.dec == dec && v.maxt == maxt && v.minw == minw && v.grouped == grouped)
+        if (v.rw == rw && v.u == u && v.tt == tt && v.dec == dec && v.maxt == maxt && v.minw == minw && v.mode == mode)
             return &v;
     }
     return nullptr;
@@ -68,14 +75,10 @@ static int g_cu_count[16];
 
 hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
 {
-    const Variant *v = find_variant(plan.rw, plan.prefetch, plan.token_tiles, plan.decode, plan.threads, plan.min_waves,
-                                    plan.args.group_rows ? 1 : 0);
-    if (!v) return hipErrorInvalidConfiguration;
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
-    const int vi = (int)(v - kVariants);
     int cus;
     {
         std::lock_guard<std::mutex> lock(g_attr_mutex);
@@ -86,6 +89,22 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
             g_cu_count[dev] = n > 0 ? n : 256;
         }
         cus = g_cu_count[dev];
+    }
+    const unsigned slots = (unsigned)(cus * plan.wgs_per_cu);
+    const Variant *v = find_variant(plan.rw, plan.prefetch, plan.token_tiles, plan.decode, plan.threads, plan.min_waves,
+                                    plan.args.group_rows ? 1 : 0);
+    if (!v) return hipErrorInvalidConfiguration;
+    // a dense launch with a fixed split whose tiles all fit the device at once needs no tile
+    // walk: its one-tile-per-workgroup twin, where there is one, computes the same sums
+    if (!plan.args.group_rows && !plan.args.balanced && plan.grid.x <= slots &&
+        plan.grid.x == (unsigned)plan.args.tiles_total) {
+        const Variant *v1 = find_variant(plan.rw, plan.prefetch, plan.token_tiles, plan.decode, plan.threads,
+                                         plan.min_waves, 2);
+        if (v1) v = v1;
+    }
+    const int vi = (int)(v - kVariants);
+    {
+        std::lock_guard<std::mutex> lock(g_attr_mutex);
         if (!g_attr_done[dev][vi]) {
             e = hipFuncSetAttribute(reinterpret_cast<const void *>(v->fn),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
@@ -95,9 +114,12 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
     }
     // persistent workgroups: as many as the device holds at once, each walks tiles with this stride
     dim3 grid = plan.grid;
-    const unsigned slots = (unsigned)(cus * plan.wgs_per_cu);
     if (grid.x > slots) grid.x = slots;
+#ifdef TUNA_TRACE
+    hipLaunchKernelGGL(v->fn, grid, dim3(plan.threads), plan.lds_bytes + 256, stream, plan.args);  // + timestamps
+#else
     hipLaunchKernelGGL(v->fn, grid, dim3(plan.threads), plan.lds_bytes, stream, plan.args);
+#endif
     return hipGetLastError();
 }
 
