@@ -206,6 +206,16 @@ int tuna_time_copy(const void *src, void *dst, size_t bytes, int warmup, int ite
 int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int warmup, int iters,
                    void *stream, float *elapsed_ms);
 
+/* Diagnostic switch, process-wide, default on: small dense launches that qualify (one
+ * workgroup per tile, power-of-two split, aligned shapes, up to 16 tokens per tile) run a
+ * kernel stripped of everything else the general one carries.  Both compute bit-identical
+ * results; turning it off is for A/B timing and for the test that checks exactly that.
+ * Returns the previous setting.  No counterpart in the reference. */
+int tuna_set_lean_kernels(int enabled);
+
+/* Diagnostic: how many GEMM launches of this process took that kernel so far. */
+unsigned long long tuna_lean_launches(void);
+
 /* Releases the library-owned split-K workspaces of the current device (synchronises
  * the device first). */
 int tuna_release_workspaces(void);

@@ -633,3 +633,55 @@ def test_fused_residual_and_silu_mul_epilogues(ci):
     # a product of two sums that are each within tolerance: relative to an output, the error of a
     # near-zero factor is amplified, so the floor of the metric is the wider one (5e-2 of the largest output)
     assert rel_err(out2.cpu().numpy().astype(np.float64), want2, floor=REL_FLOOR_D2) <= REL_TOL
+
+
+# ----------------------------------------------------------------------------- lean kernel
+LEAN_CASES = [
+    # m, n, k, config: launches that qualify for the stripped-down kernel
+    (1024, 16, 2048, dict(waves_m=2, waves_k=4, split_k=4, prefetch=2, x_chunk=512)),
+    (512, 5, 4096, dict(waves_m=1, waves_k=8, split_k=2, prefetch=4, x_chunk=1024)),      # 8 pieces of x per thread
+    (256, 16, 1024, dict(waves_m=4, waves_k=1, split_k=1, prefetch=2, x_chunk=64)),        # register-store epilogue
+    (256, 40, 512, dict(waves_m=1, waves_k=2, split_k=1, prefetch=2, x_chunk=128)),        # three token chunks, ragged
+    (1024, 16, 4096, dict(waves_m=1, waves_k=16, split_k=2, prefetch=2, x_chunk=2048)),    # 16 waves along k
+    (512, 16, 8192, dict(waves_m=1, waves_k=8, split_k=8, prefetch=4, x_chunk=1024, xcd_swizzle=1)),
+    (448, 1, 1024, dict(waves_m=7, waves_k=1, split_k=2, prefetch=8, x_chunk=256)),        # 7 waves, deepest ring
+    (128, 16, 256, dict(waves_m=1, waves_k=4, split_k=1, prefetch=2, x_chunk=256)),        # one ring turn per wave
+]
+
+
+@pytest.mark.parametrize("ci", range(len(LEAN_CASES)))
+def test_lean_kernel_equals_general_kernel_bit_for_bit(ci):
+    """Small aligned launches take a stripped-down kernel; it must give the bits of the general
+    kernel with the same config (same decode, same summation order), for the plain store and both
+    fused epilogues, and be within tolerance of the oracle."""
+    import torch
+
+    from tuna_amd import _lib, ops
+
+    m, n, k, kw = LEAN_CASES[ci]
+    c = cfg(**kw)
+    print(f"lean case#{ci} {m}x{n}x{k} {c.to_dict()}", flush=True)
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=80 + ci)
+    res = (np.random.default_rng(ci).standard_normal((n, m)) * 0.05).astype(np.float16)
+    dq, dx, dc, da, dres = to_dev(q, x, code, absmax, res)
+    outs = {}
+    prev = ops.set_lean_kernels(True)
+    try:
+        for lean in (True, False):
+            ops.set_lean_kernels(lean)
+            before = ops.lean_launches()
+            o_plain = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+            o_res = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+            o_silu = torch.full((n, m // 2), float("nan"), dtype=torch.float16, device="cuda")
+            ops.matmul(dx, dq, da, dc, o_plain, m, n, k, config=c)
+            ops.matmul_fused(dx, dq, da, dc, o_res, m, n, k, _lib.EPILOGUE_RESIDUAL, residual=dres, config=c)
+            ops.matmul_fused(dx, dq, da, dc, o_silu, m, n, k, _lib.EPILOGUE_SILU_MUL, config=c)
+            torch.cuda.synchronize()
+            assert ops.lean_launches() - before == (3 if lean else 0)   # the case really qualifies
+            outs[lean] = (o_plain, o_res, o_silu)
+    finally:
+        ops.set_lean_kernels(prev)
+    for a, b in zip(outs[True], outs[False]):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    ref = O.gemm_f64(q, x, code, absmax, m, n, k, mode=O.D1)
+    assert rel_err(outs[True][0].cpu().numpy().astype(np.float64), ref) <= REL_TOL

@@ -79,6 +79,8 @@ SIGNATURES = {
     "tuna_time_dequant": (_i, [_vpp, _vpp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_copy": (_i, [_vp, _vp, _sz, _i, _i, _vp, _fp]),
     "tuna_time_read": (_i, [_vp, _vp, _sz, _i, _i, _i, _vp, _fp]),
+    "tuna_set_lean_kernels": (_i, [_i]),
+    "tuna_lean_launches": (ctypes.c_ulonglong, []),
     "tuna_release_workspaces": (_i, []),
 }
 

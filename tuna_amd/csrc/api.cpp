@@ -169,6 +169,7 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     a.waves_k = c.waves_k;
     a.wk_log2 = log2i(c.waves_k);
     a.split_k = c.split_k;
+    a.split_log2 = (c.split_k > 0 && (c.split_k & (c.split_k - 1)) == 0) ? log2i(c.split_k) : -1;
     a.steps_total = steps_total;
     a.steps_per_split = balanced ? steps_total : ceil_div(steps_total, c.split_k);
     a.balanced = balanced ? 1 : 0;
@@ -881,6 +882,10 @@ TUNA_EXPORT int tuna_time_read(const void *src, void *sink, size_t bytes, int bl
     };
     return time_loop(launch, 1, warmup, iters, 0, static_cast<hipStream_t>(stream), elapsed_ms);
 }
+
+TUNA_EXPORT int tuna_set_lean_kernels(int enabled) { return tuna::set_lean_kernels(enabled); }
+
+TUNA_EXPORT unsigned long long tuna_lean_launches(void) { return tuna::lean_launches(); }
 
 TUNA_EXPORT int tuna_release_workspaces(void)
 {

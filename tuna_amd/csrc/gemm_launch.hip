@@ -1,7 +1,9 @@
 // Instantiations of the GEMM kernel and the variant dispatcher.
+#include <atomic>
 #include <mutex>
 
 #include "gemm_kernel.hpp"
+#include "gemm_lean.hpp"
 
 namespace tuna {
 
@@ -68,9 +70,60 @@ bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int 
     return find_variant(rw, prefetch, token_tiles, decode, threads, min_waves, grouped) != nullptr;
 }
 
+// ---- lean twins (gemm_lean.hpp) -------------------------------------------------------------
+struct LeanVariant {
+    int wk, u, maxt;
+    GemmKernelFn fn;
+};
+#define L5(WK, U) {WK, U, 512, gemm_lean_kernel<WK, U, 512, 2>}
+#define L10(WK, U) {WK, U, 1024, gemm_lean_kernel<WK, U, 1024, 4>}
+static const LeanVariant kLean[] = {
+    L5(1, 2), L5(1, 4), L5(1, 8), L5(2, 2), L5(2, 4), L5(2, 8), L5(4, 2), L5(4, 4), L5(4, 8), L5(8, 2), L5(8, 4), L5(8, 8),
+    L10(4, 2), L10(4, 4), L10(8, 2), L10(8, 4), L10(16, 2), L10(16, 4),
+};
+#undef L5
+#undef L10
+static constexpr int kNumLean = sizeof(kLean) / sizeof(kLean[0]);
+
+// The lean kernel's LDS: decode table + max(x slice of the split, reduction planes) + ticket.
+static size_t lean_lds_bytes(const GemmPlan &plan)
+{
+    const size_t x_bytes = (size_t)plan.args.steps_per_split * 1024;  // 16 tokens x 32 k x 2 bytes per k-step
+    const size_t red_bytes = (size_t)(plan.threads / 64) * 4096;
+    return (size_t)kLutBytes + (x_bytes > red_bytes ? x_bytes : red_bytes) + 16;
+}
+
+static std::atomic<int> g_lean_enabled{1};
+static std::atomic<unsigned long long> g_lean_launches{0};
+
+unsigned long long lean_launches() { return g_lean_launches.load(); }
+
+int set_lean_kernels(int enabled) { return g_lean_enabled.exchange(enabled ? 1 : 0); }
+
+// Launches the lean kernel computes exactly like the general one (conditions in gemm_lean.hpp).
+static const LeanVariant *lean_applies(const GemmPlan &plan, unsigned slots)
+{
+    const GemmArgs &a = plan.args;
+    if (!g_lean_enabled.load(std::memory_order_relaxed)) return nullptr;
+    if (a.group_rows || a.balanced || plan.rw != 1 || plan.token_tiles != 1 || plan.decode != TUNA_DECODE_GEMM) return nullptr;
+    if (a.split_log2 < 0 || a.k_stagger != 0) return nullptr;
+    if (plan.grid.x != (unsigned)a.tiles_total || plan.grid.x > slots) return nullptr;
+    if (a.k != a.steps_total * kStepK || a.steps_per_split * a.split_k != a.steps_total) return nullptr;
+    if (a.steps_per_split % (a.waves_k * plan.prefetch) != 0) return nullptr;
+    if (a.m % (a.waves_m * kRowsPerLoad) != 0) return nullptr;
+    if (a.steps_per_split * 64 > 8 * plan.threads) return nullptr;  // at most 8 pieces of x per thread
+    if (lean_lds_bytes(plan) > (size_t)kLdsLimit) return nullptr;
+    if (((uintptr_t)a.absmax & 15u) != 0) return nullptr;
+    const int maxt = plan.threads <= 512 ? 512 : 1024;
+    for (int i = 0; i < kNumLean; ++i)
+        if (kLean[i].wk == a.waves_k && kLean[i].u == plan.prefetch && kLean[i].maxt == maxt) return &kLean[i];
+    return nullptr;
+}
+
 // Dynamic LDS above 64 KB needs a one-time opt-in per kernel and device.
 static std::mutex g_attr_mutex;
 static unsigned char g_attr_done[16][kNumVariants];
+static unsigned char g_lean_attr_done[16][kNumLean];
 static int g_cu_count[16];
 
 hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
@@ -94,6 +147,21 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
     const Variant *v = find_variant(plan.rw, plan.prefetch, plan.token_tiles, plan.decode, plan.threads, plan.min_waves,
                                     plan.args.group_rows ? 1 : 0);
     if (!v) return hipErrorInvalidConfiguration;
+    if (const LeanVariant *lv = lean_applies(plan, slots)) {
+        const int li = (int)(lv - kLean);
+        {
+            std::lock_guard<std::mutex> lock(g_attr_mutex);
+            if (!g_lean_attr_done[dev][li]) {
+                e = hipFuncSetAttribute(reinterpret_cast<const void *>(lv->fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        kLdsLimit);
+                if (e != hipSuccess) return e;
+                g_lean_attr_done[dev][li] = 1;
+            }
+        }
+        hipLaunchKernelGGL(lv->fn, plan.grid, dim3(plan.threads), lean_lds_bytes(plan), stream, plan.args);
+        g_lean_launches.fetch_add(1, std::memory_order_relaxed);
+        return hipGetLastError();
+    }
     // a dense launch with a fixed split whose tiles all fit the device at once needs no tile
     // walk: its one-tile-per-workgroup twin, where there is one, computes the same sums
     if (!plan.args.group_rows && !plan.args.balanced && plan.grid.x <= slots &&

@@ -33,6 +33,7 @@ struct GemmArgs {
     unsigned *counters;  // one arrival counter per (token chunk, row tile), zero between launches
     int m, n, k;
     int waves_m, waves_k, split_k;  // waves_k is a power of two, waves_m any count
+    int split_log2;                 // log2(split_k) if it is a power of two, else -1
     int wk_log2;
     int steps_total;      // ceil(k / 32)
     int steps_per_split;  // k-steps owned by one workgroup
@@ -147,6 +148,8 @@ struct GemmPlan {
 
 // gemm_kernel.hip
 hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream);
+int set_lean_kernels(int enabled);  // returns the previous setting
+unsigned long long lean_launches();
 bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves, int grouped);
 
 // gemm_tiled.hip

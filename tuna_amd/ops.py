@@ -301,3 +301,14 @@ def time_read(src, blocks=0, warmup=5, iters=20) -> float:
                               _stream(src.device), ctypes.byref(ms))
     _lib.check(rc)
     return ms.value
+
+
+def set_lean_kernels(enabled: bool) -> bool:
+    """Diagnostic switch (tuna_set_lean_kernels): whether qualifying small launches use the
+    stripped-down kernel.  Results are bit-identical either way.  Returns the previous setting."""
+    return bool(_lib.lib().tuna_set_lean_kernels(int(bool(enabled))))
+
+
+def lean_launches() -> int:
+    """Diagnostic (tuna_lean_launches): GEMM launches of this process that took the stripped-down kernel."""
+    return int(_lib.lib().tuna_lean_launches())
