@@ -101,18 +101,24 @@ unsigned long long lean_launches() { return g_lean_launches.load(); }
 int set_lean_kernels(int enabled) { return g_lean_enabled.exchange(enabled ? 1 : 0); }
 
 // Launches the lean kernel computes exactly like the general one (conditions in gemm_lean.hpp).
-static const LeanVariant *lean_applies(const GemmPlan &plan, unsigned slots)
+static const LeanVariant *lean_applies(const GemmPlan &plan, int cus)
 {
     const GemmArgs &a = plan.args;
     if (!g_lean_enabled.load(std::memory_order_relaxed)) return nullptr;
     if (a.group_rows || a.balanced || plan.rw != 1 || plan.token_tiles != 1 || plan.decode != TUNA_DECODE_GEMM) return nullptr;
     if (a.split_log2 < 0 || a.k_stagger != 0) return nullptr;
-    if (plan.grid.x != (unsigned)a.tiles_total || plan.grid.x > slots) return nullptr;
+    if (plan.grid.x != (unsigned)a.tiles_total) return nullptr;
     if (a.k != a.steps_total * kStepK || a.steps_per_split * a.split_k != a.steps_total) return nullptr;
     if (a.steps_per_split % (a.waves_k * plan.prefetch) != 0) return nullptr;
     if (a.m % (a.waves_m * kRowsPerLoad) != 0) return nullptr;
     if (a.steps_per_split * 64 > 8 * plan.threads) return nullptr;  // at most 8 pieces of x per thread
     if (lean_lds_bytes(plan) > (size_t)kLdsLimit) return nullptr;
+    // all tiles at once: workgroups per CU by LDS and by registers (at most 96 per lane: five
+    // waves per SIMD); a launch of several rounds is what the tile walk of gemm_kernel is for
+    const int waves = plan.threads / 64;
+    const int by_lds = (int)((size_t)kLdsLimit / lean_lds_bytes(plan));
+    const int by_regs = 20 / waves > 0 ? 20 / waves : 1;
+    if ((long long)plan.grid.x > (long long)cus * (by_lds < by_regs ? by_lds : by_regs)) return nullptr;
     if (((uintptr_t)a.absmax & 15u) != 0) return nullptr;
     const int maxt = plan.threads <= 512 ? 512 : 1024;
     for (int i = 0; i < kNumLean; ++i)
@@ -147,7 +153,7 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
     const Variant *v = find_variant(plan.rw, plan.prefetch, plan.token_tiles, plan.decode, plan.threads, plan.min_waves,
                                     plan.args.group_rows ? 1 : 0);
     if (!v) return hipErrorInvalidConfiguration;
-    if (const LeanVariant *lv = lean_applies(plan, slots)) {
+    if (const LeanVariant *lv = lean_applies(plan, cus)) {
         const int li = (int)(lv - kLean);
         {
             std::lock_guard<std::mutex> lock(g_attr_mutex);

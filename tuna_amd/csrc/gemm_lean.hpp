@@ -46,6 +46,20 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
     unsigned char *work = smem + kLutBytes;
 
     const int tid = threadIdx.x;
+#ifdef TUNA_TRACE
+    // development builds: timestamps of wave 0 in scalar registers, written out at the end
+    unsigned long long tm_[10] = {};
+#define TUNA_LMARK(i) tm_[i] = wall_clock64();
+#define TUNA_LDUMP()                                                                            \
+    if (a.trace && tid == 0) {                                                                 \
+        tm_[9] = wall_clock64();                                                               \
+        for (int i_ = 0; i_ < 10; ++i_) a.trace[(size_t)blockIdx.x * 128 + i_] = tm_[i_];      \
+    }
+#else
+#define TUNA_LMARK(i)
+#define TUNA_LDUMP()
+#endif
+    TUNA_LMARK(0)
     const int lane = tid & 63;
     const int i16 = lane & 15;
     const int g = lane >> 4;
@@ -98,6 +112,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
             xv[b] = *reinterpret_cast<const u32x4 *>(xrow + (size_t)(min(x_slot0 + b * x_slot_step, x_slots - 1) - x_slot0) * 16);
     }
 
+    TUNA_LMARK(1)
     // ---- decode table (see gemm_kernel.hpp), built while the loads are in flight ------------
     {
         const int code_bits = (int)f16_bits((f16)code_lane);
@@ -117,6 +132,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
             }
         }
     }
+    TUNA_LMARK(2)
     f16x2 sc16[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -137,6 +153,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
         }
     }
     __syncthreads();
+    TUNA_LMARK(3)
 
     // ---- main loop: n_it / U ring turns, the last one without refills ------------------------
     f32x4 acc[4];
@@ -167,6 +184,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
 #pragma unroll
     for (int u = 0; u < U; ++u) TUNA_LEAN_CONSUME(u)
 #undef TUNA_LEAN_CONSUME
+    TUNA_LMARK(4)
 
     // ---- reduction and store (layouts of gemm_kernel) ----------------------------------------
     f16 *outp = reinterpret_cast<f16 *>(a.out);
@@ -207,6 +225,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
     __syncthreads();
     float o[4][4];
     sum_planes<WK, 4, 32>(redf, plane_floats, wm, wk, lane, o, 0);
+    TUNA_LMARK(5)
 
     const size_t seg_floats = (size_t)a.waves_m * 1024;  // partial sums of one workgroup: [wm][f][j]
     const size_t tile_id = (size_t)blockIdx.y * a.row_tiles + row_tile;
@@ -239,12 +258,20 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
+    TUNA_LMARK(6)
     volatile unsigned *ticket = reinterpret_cast<volatile unsigned *>(work);
     if (tid == 0) *ticket = __hip_atomic_fetch_add(a.counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    if (*ticket != (unsigned)a.split_k - 1u) return;
+    TUNA_LMARK(7)
+    if (*ticket != (unsigned)a.split_k - 1u) {
+        TUNA_LDUMP()
+        return;
+    }
     if (tid == 0) __hip_atomic_store(a.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (!owner) return;
+    if (!owner) {
+        TUNA_LDUMP()
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
         const int f = (i * WK + wk) * 64 + lane;
@@ -256,6 +283,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
 #pragma unroll
             for (int b = 0; b < 4; ++b) ps[b] = src + (size_t)min(sp0 + b, a.split_k - 1) * seg_floats;
             load_partials4(ps[0], ps[1], ps[2], ps[3], p[0], p[1], p[2], p[3]);
+            TUNA_LMARK(8)
 #pragma unroll
             for (int b = 0; b < 4; ++b)
                 if (sp0 + b < a.split_k) s4 += p[b];
@@ -266,6 +294,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
             store_features4(outp, resp, a.epilogue, (size_t)tok, out_ld, row0 + (l >> 4) * 16 + v * 4, s4[0], s4[1], s4[2],
                             s4[3]);
     }
+    TUNA_LDUMP()
 }
 
 }  // namespace tuna

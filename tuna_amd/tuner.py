@@ -130,6 +130,41 @@ def tiled_space(m: int, n_key: int, k: int):
     return out
 
 
+def lean_space(m: int, n_key: int, k: int):
+    """Every config whose launch takes the stripped-down kernel for small aligned launches
+    (gemm_lean.hpp; the conditions of lean_applies in gemm_launch.hip): 64 rows per wave, one
+    token tile, no stagger, a power-of-two split, whole ring turns, all tiles resident at once.
+    Small enough to time exhaustively."""
+    lo, _ = make_configs.N_BUCKETS[n_key]
+    if lo > 32 or k % 32:
+        return []
+    steps = k // 32
+    out = []
+    for wm in range(1, 17):
+        for wk in (1, 2, 4, 8, 16):
+            waves = wm * wk
+            if waves > 16 or m % (64 * wm):
+                continue
+            split = 1
+            while split <= steps:
+                sps = steps // split
+                if steps % split == 0 and sps * 64 <= 8 * 64 * waves:
+                    lds = 65536 + max(sps * 1024, waves * 4096) + 16
+                    wgs = min(make_configs.LDS_LIMIT // lds, max(1, 20 // waves)) if lds <= make_configs.LDS_LIMIT else 0
+                    if (m // (64 * wm)) * split <= N_CU * wgs:
+                        for pf in (2, 4, 8):
+                            if sps % (wk * pf):
+                                continue
+                            for sw in (0, 1):
+                                c = repair(dict(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=split, prefetch=pf,
+                                                x_chunk=32 * wk * pf, token_tiles=1, xcd_swizzle=sw, k_stagger=0), m, n_key, k)
+                                if c is not None and c["split_k"] == split and c["token_tiles"] == 1:
+                                    out.append(c)
+                split *= 2
+    uniq = {json.dumps(c, sort_keys=True): c for c in out}
+    return list(uniq.values())
+
+
 def mutate(c: dict, rng: random.Random, m, n_key, k):
     c = dict(c)
     for _ in range(rng.choice((1, 1, 2))):
@@ -202,7 +237,7 @@ def tune_shape(m, n, k, generations=6, population=24, seed=0, log=print, max_see
         return json.loads(scored[0][1]), scored[0][0]
     pool = seeds(m, n_key, k)
     rng.shuffle(pool)
-    pool = pool[:max_seed_evals]
+    pool = pool[:max_seed_evals] + lean_space(m, n_key, k)
     scored = sorted(((ev(c), json.dumps(c, sort_keys=True)) for c in pool))
     pop = [json.loads(s) for _, s in scored[:population]]
     log(f"  seeds: {len(pool)} evaluated, best {scored[0][0]:.2f} us {scored[0][1]}")
