@@ -685,3 +685,82 @@ def test_lean_kernel_equals_general_kernel_bit_for_bit(ci):
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
     ref = O.gemm_f64(q, x, code, absmax, m, n, k, mode=O.D1)
     assert rel_err(outs[True][0].cpu().numpy().astype(np.float64), ref) <= REL_TOL
+
+
+# ----------------------------------------------------------------------------- narrow-row kernel
+NARROW_CASES = [
+    # m, n, k, rows_per_wave, waves_k, prefetch
+    (256, 16, 1024, 16, 4, 2),
+    (256, 5, 4096, 32, 16, 8),      # one ring turn per wave, 1024 threads
+    (64, 40, 512, 32, 2, 2),        # three token chunks, the last one ragged
+    (48, 1, 2048, 16, 8, 4),        # three workgroups of 16 rows, one token
+    (512, 16, 8192, 32, 8, 4),
+    (128, 16, 64, 16, 1, 2),        # a single wave: two passes over the row pairs
+    (128, 33, 256, 32, 1, 2),
+    (4096, 16, 4096, 16, 16, 2),    # full-size attention output projection, 256 workgroups
+]
+
+
+def narrow_cfg(rows, wk, pf):
+    return cfg(rows_per_wave=rows, waves_m=1, waves_k=wk, split_k=1, prefetch=pf, x_chunk=32 * wk * pf, token_tiles=1)
+
+
+@pytest.mark.parametrize("ci", range(len(NARROW_CASES)))
+def test_narrow_row_kernel_matches_oracle(ci):
+    """rows_per_wave 16 / 32 selects the kernel with one workgroup per 16 / 32 weight rows and no
+    split across workgroups: plain store and both fused epilogues against the oracle's float64
+    sums, the rows outside the result untouched (NaN prefill)."""
+    import torch
+
+    from tuna_amd import _lib, ops
+
+    m, n, k, rows, wk, pf = NARROW_CASES[ci]
+    c = narrow_cfg(rows, wk, pf)
+    print(f"narrow case#{ci} {m}x{n}x{k} {c.to_dict()}", flush=True)
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=90 + ci)
+    res = (np.random.default_rng(ci).standard_normal((n, m)) * 0.05).astype(np.float16)
+    ref = O.gemm_f64(q, x, code, absmax, m, n, k, mode=O.D1)
+    dq, dx, dc, da, dres = to_dev(q, x, code, absmax, res)
+    pad = torch.full((n + 2, m), float("nan"), dtype=torch.float16, device="cuda")   # a guard row on either side
+    out = pad[1:n + 1]
+    ops.matmul(dx, dq, da, dc, out, m, n, k, config=c)
+    o_res = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+    o_silu = torch.full((n, m // 2), float("nan"), dtype=torch.float16, device="cuda")
+    ops.matmul_fused(dx, dq, da, dc, o_res, m, n, k, _lib.EPILOGUE_RESIDUAL, residual=dres, config=c)
+    ops.matmul_fused(dx, dq, da, dc, o_silu, m, n, k, _lib.EPILOGUE_SILU_MUL, config=c)
+    torch.cuda.synchronize()
+    assert rel_err(out.cpu().numpy().astype(np.float64), ref) <= REL_TOL
+    assert torch.isnan(pad[0]).all() and torch.isnan(pad[n + 1]).all()
+    assert rel_err(o_res.cpu().numpy().astype(np.float64), ref + res.astype(np.float64)) <= REL_TOL
+    g, u = ref[:, 0::2], ref[:, 1::2]
+    assert rel_err(o_silu.cpu().numpy().astype(np.float64), g / (1.0 + np.exp(-g)) * u, floor=REL_FLOOR_D2) <= REL_TOL
+    # repeatable bit for bit
+    again = torch.empty((n, m), dtype=torch.float16, device="cuda")
+    ops.matmul(dx, dq, da, dc, again, m, n, k, config=c)
+    torch.cuda.synchronize()
+    assert torch.equal(again.view(torch.int16), out.view(torch.int16))
+
+
+@pytest.mark.parametrize("rows,wk,pf", [(16, 4, 2), (32, 8, 4), (32, 16, 2)])
+def test_narrow_row_kernel_decode_readout_is_bit_exact(rows, wk, pf):
+    """One-hot activations read the narrow-row kernel's in-register decode out: the oracle's D1 image."""
+    m, k = 256, 2048
+    q, _, code, absmax = make_inputs_np(m, 16, k, seed=rows + wk)
+    want_img = O.dequant(q, absmax, code, m, k, mode=O.D1)
+    cols = np.random.default_rng(wk).choice(k, size=16, replace=False)
+    x = np.zeros((16, k), np.float16)
+    x[np.arange(16), cols] = 1.0
+    got = run_gemm(q, x, code, absmax, m, 16, k, config=narrow_cfg(rows, wk, pf))
+    assert np.array_equal(f16_bits_to_f64(got), f16_bits_to_f64(want_img[:, cols].T))
+
+
+def test_narrow_row_configs_that_do_not_fit_are_rejected():
+    from tuna_amd import ops
+
+    q, x, code, absmax = make_inputs_np(256, 16, 1024, seed=1)
+    for m, k, kw in [(264, 1024, dict()),                       # m not a multiple of the rows
+                     (256, 1000, dict()),                       # k not a multiple of 32 * waves_k * prefetch
+                     (256, 1024, dict(split_k=2)), (256, 1024, dict(waves_m=2)), (256, 1024, dict(token_tiles=2))]:
+        c = cfg(**{**dict(rows_per_wave=16, waves_m=1, waves_k=4, split_k=1, prefetch=2, x_chunk=256, token_tiles=1), **kw})
+        with pytest.raises(ops.TunaError):
+            ops.validate_config(m, 16, k, c)

@@ -315,7 +315,7 @@ def test_gpu_parity_config_families_are_valid_configs():
     both of their shapes (a rejected config would fail the GPU test for the wrong reason)."""
     import importlib.util
 
-    from tuna_amd import ops
+    from tuna_amd import make_configs, ops
 
     spec = importlib.util.spec_from_file_location("gpu_parity_cases", os.path.join(ROOT, "tests", "test_gpu_parity.py"))
     mod = importlib.util.module_from_spec(spec)
@@ -326,6 +326,14 @@ def test_gpu_parity_config_families_are_valid_configs():
     for rows, tt in mod.TILED:
         for (m, n, k, split) in ((512, 256, 512, 1), (520, 300, 1096, 1), (256, 70, 2048, 4), (1024, 129, 200, 3)):
             ops.validate_config(m, n, k, mod.cfg(lds_tile_rows=rows, token_tiles=tt, split_k=split))
+    for (m, n, k, rows, wk, pf) in mod.NARROW_CASES:
+        c = mod.narrow_cfg(rows, wk, pf)
+        ops.validate_config(m, n, k, c)
+        lds, ws = ops.config_footprint(m, n, k, c)
+        assert (lds, ws) == (make_configs.lds_bytes(c.to_dict()), 0)
+        make_configs.validate(m, make_configs.bucket_of(n), k, c.to_dict())
+        assert ops.config_segments(m, n, k, c, 0, m // rows - 1) == [(m // rows - 1, 0, k // 32, -1)]
+        assert ops.config_contributors(m, n, k, c, 0, 0) == (-1, 1, 0)
     with pytest.raises(ops.TunaError):
         ops.validate_config(512, 256, 512, mod.cfg(lds_tile_rows=96, token_tiles=16))       # no such tile
     with pytest.raises(ops.TunaError):

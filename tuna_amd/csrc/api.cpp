@@ -225,6 +225,48 @@ static int plan_tiled(int m, int n, int k, const tuna_gemm_config &c, int decode
     return TUNA_OK;
 }
 
+// Narrow-row kernel: checks and launch arguments for a config with rows_per_wave 16 or 32.
+struct NarrowPlan {
+    NarrowArgs args;
+    int rows, waves_k, prefetch;
+    size_t lds_bytes;
+};
+
+static inline bool is_narrow(const tuna_gemm_config &c) { return !c.lds_tile_rows && (c.rows_per_wave == 16 || c.rows_per_wave == 32); }
+
+static int plan_narrow(int m, int n, int k, const tuna_gemm_config &c, int decode, NarrowPlan *plan)
+{
+    int rc = check_shape(m, n, k);
+    if (rc) return rc;
+    if (decode != TUNA_DECODE_GEMM)
+        return fail(TUNA_ERR_UNSUPPORTED, "the narrow-row kernel (rows_per_wave 16, 32) implements TUNA_DECODE_GEMM only");
+    if ((unsigned long long)m * (unsigned long long)k / 2 >= (1ull << 32) || (unsigned long long)k * 32 >= (1ull << 32))
+        return fail(TUNA_ERR_UNSUPPORTED, "operands exceed the kernel's 32-bit offsets");
+    if (c.waves_m != 1 || c.split_k != 1 || c.token_tiles != 1 || c.k_stagger != 0)
+        return fail(TUNA_ERR_UNSUPPORTED,
+                    "rows_per_wave=%d needs waves_m=1, split_k=1, token_tiles=1, k_stagger=0 (got %d, %d, %d, %d)",
+                    c.rows_per_wave, c.waves_m, c.split_k, c.token_tiles, c.k_stagger);
+    if (!is_pow2(c.waves_k) || c.waves_k > 16 || !narrow_variant_exists(c.rows_per_wave, c.waves_k, c.prefetch))
+        return fail(TUNA_ERR_UNSUPPORTED, "no narrow-row kernel for rows_per_wave=%d waves_k=%d prefetch=%d", c.rows_per_wave,
+                    c.waves_k, c.prefetch);
+    if (m % c.rows_per_wave)
+        return fail(TUNA_ERR_UNSUPPORTED, "rows_per_wave=%d needs m=%d to be a multiple of it", c.rows_per_wave, m);
+    if (k % (kStepK * c.waves_k * c.prefetch))
+        return fail(TUNA_ERR_UNSUPPORTED, "rows_per_wave=%d needs k=%d to be a multiple of 32*waves_k*prefetch=%d",
+                    c.rows_per_wave, k, kStepK * c.waves_k * c.prefetch);
+    if (ceil_div(n, 16) > 65535) return fail(TUNA_ERR_UNSUPPORTED, "n=%d needs more than 65535 token chunks", n);
+    memset(plan, 0, sizeof(*plan));
+    plan->rows = c.rows_per_wave;
+    plan->waves_k = c.waves_k;
+    plan->prefetch = c.prefetch;
+    plan->lds_bytes = (size_t)kLutBytes + (size_t)c.waves_k * (c.rows_per_wave / 16) * 1024;
+    plan->args.m = m;
+    plan->args.n = n;
+    plan->args.k = k;
+    plan->args.n_it = k / kStepK / c.waves_k;
+    return TUNA_OK;
+}
+
 // A config for shapes the tuned table does not cover, following what the tuner finds on the
 // tuned shapes: many rows -> wide row tiles without any k split (accumulators stored straight
 // from registers); few rows -> one 64-row group per workgroup, 8 waves along k and enough
@@ -434,6 +476,21 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
         }
         hipError_t e = launch_gemm_tiled(tp.args, tp.tile_rows, tp.tile_tokens, stream);
         if (e != hipSuccess) return hip_fail(e, "many-token gemm launch");
+        return TUNA_OK;
+    }
+    if (is_narrow(c)) {
+        NarrowPlan np;
+        if ((rc = plan_narrow(m, n, k, c, decode, &np))) return rc;
+        if ((rc = check_ptr(absmax, "absmax", 8))) return rc;  // scales are read two rows at a time
+        np.args.q = static_cast<const uint8_t *>(q);
+        np.args.x = x;
+        np.args.code = static_cast<const float *>(code);
+        np.args.absmax = static_cast<const float *>(absmax);
+        np.args.out = out;
+        np.args.epilogue = epilogue;
+        np.args.residual = residual;
+        hipError_t e = launch_gemm_narrow(np.args, np.rows, np.waves_k, np.prefetch, stream);
+        if (e != hipSuccess) return hip_fail(e, "narrow-row gemm launch");
         return TUNA_OK;
     }
     GemmPlan plan;
@@ -714,6 +771,10 @@ TUNA_EXPORT int tuna_validate_config(int m, int n, int k, const tuna_gemm_config
         TiledPlan tp;
         return plan_tiled(m, n, k, *cfg, TUNA_DECODE_GEMM, &tp);
     }
+    if (is_narrow(*cfg)) {
+        NarrowPlan np;
+        return plan_narrow(m, n, k, *cfg, TUNA_DECODE_GEMM, &np);
+    }
     GemmPlan plan;
     return plan_gemm(m, n, k, *cfg, TUNA_DECODE_GEMM, &plan);
 }
@@ -730,6 +791,14 @@ TUNA_EXPORT int tuna_config_footprint(int m, int n, int k, const tuna_gemm_confi
         if (workspace_bytes) *workspace_bytes = tp.ws_bytes;
         return TUNA_OK;
     }
+    if (is_narrow(*cfg)) {
+        NarrowPlan np;
+        int rc = plan_narrow(m, n, k, *cfg, TUNA_DECODE_GEMM, &np);
+        if (rc) return rc;
+        if (lds_bytes) *lds_bytes = np.lds_bytes;
+        if (workspace_bytes) *workspace_bytes = 0;
+        return TUNA_OK;
+    }
     GemmPlan plan;
     int rc = plan_gemm(m, n, k, *cfg, TUNA_DECODE_GEMM, &plan);
     if (rc) return rc;
@@ -742,6 +811,21 @@ TUNA_EXPORT int tuna_config_segments(int m, int n, int k, const tuna_gemm_config
                                      int *segments, int max_segments, int *n_segments)
 {
     if (!cfg || !n_segments) return fail(TUNA_ERR_INVALID_ARG, "cfg or n_segments is null");
+    if (is_narrow(*cfg)) {  // one workgroup per row tile, the whole k range
+        NarrowPlan np;
+        int rc = plan_narrow(m, n, k, *cfg, TUNA_DECODE_GEMM, &np);
+        if (rc) return rc;
+        const int tiles = m / np.rows;
+        if (workgroup < 0 || workgroup >= tiles) return fail(TUNA_ERR_INVALID_ARG, "workgroup %d outside 0..%d", workgroup, tiles - 1);
+        if (segments && max_segments > 0) {
+            segments[0] = workgroup;
+            segments[1] = 0;
+            segments[2] = k / kStepK;
+            segments[3] = -1;
+        }
+        *n_segments = 1;
+        return TUNA_OK;
+    }
     GemmPlan plan;
     int rc = plan_gemm(m, n, k, *cfg, TUNA_DECODE_GEMM, &plan);
     if (rc) return rc;
@@ -786,6 +870,16 @@ TUNA_EXPORT int tuna_config_contributors(int m, int n, int k, const tuna_gemm_co
                                          int *first_workgroup, int *count, int *first_slot)
 {
     if (!cfg || !first_workgroup || !count || !first_slot) return fail(TUNA_ERR_INVALID_ARG, "null argument");
+    if (is_narrow(*cfg)) {
+        NarrowPlan np;
+        int rc = plan_narrow(m, n, k, *cfg, TUNA_DECODE_GEMM, &np);
+        if (rc) return rc;
+        if (row_tile < 0 || row_tile >= m / np.rows) return fail(TUNA_ERR_INVALID_ARG, "row_tile %d out of range", row_tile);
+        *first_workgroup = -1;
+        *count = 1;
+        *first_slot = 0;
+        return TUNA_OK;
+    }
     GemmPlan plan;
     int rc = plan_gemm(m, n, k, *cfg, TUNA_DECODE_GEMM, &plan);
     if (rc) return rc;

@@ -4,6 +4,7 @@
 
 #include "gemm_kernel.hpp"
 #include "gemm_lean.hpp"
+#include "gemm_narrow.hpp"
 
 namespace tuna {
 
@@ -194,6 +195,55 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
 #else
     hipLaunchKernelGGL(v->fn, grid, dim3(plan.threads), plan.lds_bytes, stream, plan.args);
 #endif
+    return hipGetLastError();
+}
+
+// ---- narrow-row kernel (gemm_narrow.hpp) ---------------------------------------------------------
+typedef void (*NarrowKernelFn)(const NarrowArgs);
+struct NarrowVariant {
+    int rows, wk, u;
+    NarrowKernelFn fn;
+};
+#define N(LW, WK, U) {16 * LW, WK, U, gemm_narrow_kernel<LW, WK, U>}
+static const NarrowVariant kNarrow[] = {
+    N(1, 4, 2),  N(1, 4, 4),  N(1, 4, 8),  N(1, 8, 2),  N(1, 8, 4),  N(1, 8, 8),  N(1, 16, 2), N(1, 16, 4), N(1, 16, 8),
+    N(2, 4, 2),  N(2, 4, 4),  N(2, 4, 8),  N(2, 8, 2),  N(2, 8, 4),  N(2, 8, 8),  N(2, 16, 2), N(2, 16, 4), N(2, 16, 8),
+    N(1, 1, 2),  N(1, 2, 2),  N(2, 1, 2),  N(2, 2, 2),
+};
+#undef N
+static constexpr int kNumNarrow = sizeof(kNarrow) / sizeof(kNarrow[0]);
+static unsigned char g_narrow_attr_done[16][kNumNarrow];
+
+static const NarrowVariant *find_narrow(int rows, int wk, int u)
+{
+    for (int i = 0; i < kNumNarrow; ++i)
+        if (kNarrow[i].rows == rows && kNarrow[i].wk == wk && kNarrow[i].u == u) return &kNarrow[i];
+    return nullptr;
+}
+
+bool narrow_variant_exists(int rows, int waves_k, int prefetch) { return find_narrow(rows, waves_k, prefetch) != nullptr; }
+
+hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int prefetch, hipStream_t stream)
+{
+    const NarrowVariant *v = find_narrow(rows, waves_k, prefetch);
+    if (!v) return hipErrorInvalidConfiguration;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
+    const int vi = (int)(v - kNarrow);
+    {
+        std::lock_guard<std::mutex> lock(g_attr_mutex);
+        if (!g_narrow_attr_done[dev][vi]) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(v->fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    kLdsLimit);
+            if (e != hipSuccess) return e;
+            g_narrow_attr_done[dev][vi] = 1;
+        }
+    }
+    const size_t lds = (size_t)kLutBytes + (size_t)waves_k * (rows / 16) * 1024;
+    const dim3 grid((unsigned)(args.m / rows), (unsigned)((args.n + 15) / 16), 1);
+    hipLaunchKernelGGL(v->fn, grid, dim3(waves_k * 64), lds, stream, args);
     return hipGetLastError();
 }
 

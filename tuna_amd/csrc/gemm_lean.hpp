@@ -80,17 +80,9 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
     const int row0 = row_base + wm * 64;
     const int n_it = a.steps_per_split >> WK_LOG2;  // k-steps per wave, a multiple of U
 
-    // ---- requests, in the order their data is needed back (vector loads return in order) ----
+    // ---- requests, in the order their data is needed back (vector loads return in order):
+    //      codebook, scales, x slice, first ring turn of weights -----------------------------------
     const float code_lane = a.code[i16];
-    const uint32_t kb_total = (uint32_t)a.k >> 3;
-    const uint32_t lb = ((uint32_t)(row0 >> 3) + (uint32_t)(i16 >> 1)) * kb_total * 32u + (uint32_t)(i16 & 1) * 16u +
-                        (uint32_t)g * 32u;
-    const unsigned char *qp = a.q + (size_t)(sb + wk) * 128;  // uniform; advances one ring turn per group
-    u32x4 wq[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-        wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(qp + (size_t)u * (WK * 128) + lb));
-    qp += (size_t)U * (WK * 128);
     const f32x4 sc32 = *reinterpret_cast<const f32x4 *>(a.absmax + row0 + i16 * 4);
     // x slice [16 tokens][k of this split]: piece p = tid + b*nthreads is token p % 16, 8-k slot
     // p / 16, LDS byte 16*p.  64 * steps_per_split pieces, at most 8 per thread.
@@ -112,6 +104,17 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
             xv[b] = *reinterpret_cast<const u32x4 *>(xrow + (size_t)(min(x_slot0 + b * x_slot_step, x_slots - 1) - x_slot0) * 16);
     }
 
+    // the weights last: x and the scales come from L2 and are needed first, the first ring turn
+    // comes from HBM and is needed once x is staged
+    const uint32_t kb_total = (uint32_t)a.k >> 3;
+    const uint32_t lb = ((uint32_t)(row0 >> 3) + (uint32_t)(i16 >> 1)) * kb_total * 32u + (uint32_t)(i16 & 1) * 16u +
+                        (uint32_t)g * 32u;
+    const unsigned char *qp = a.q + (size_t)(sb + wk) * 128;  // uniform; advances one ring turn per group
+    u32x4 wq[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+        wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(qp + (size_t)u * (WK * 128) + lb));
+    qp += (size_t)U * (WK * 128);
     TUNA_LMARK(1)
     // ---- decode table (see gemm_kernel.hpp), built while the loads are in flight ------------
     {

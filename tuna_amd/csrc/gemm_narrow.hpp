@@ -1,0 +1,190 @@
+// Narrow-row GEMM kernel for the smallest launches (gfx950, wave64): 16 or 32 weight rows per
+// workgroup, all waves of the workgroup along k, no split across workgroups.
+//
+// With 64 rows per wave a 4096..8192-row projection has only 64..128 row groups, so filling
+// 256 CUs takes a split of k across workgroups, and its hand-over (partial sums through
+// memory, an arrival counter, a finishing pass) costs three dependent round trips: 2 us of an
+// 8 us launch.  Here a workgroup owns 16*LW rows (LW = 1, 2): 256..512 workgroups from the
+// rows alone, the k range is divided over the WK waves of the workgroup, and the only
+// reduction is the one through LDS.
+//   * MFMA v_mfma_f32_16x16x32_f16 as in gemm_kernel.hpp (weights = A, activations = B).  Lane
+//     (i = lane % 16, g = lane / 16) loads LW consecutive dwords of one 8x8 block: weight rows
+//     LW*i + j, j < LW, of the workgroup's 16*LW, block column 4*step + g.  A wave instruction
+//     covers 2*LW block rows x 128 contiguous bytes.
+//   * Every wave has its own k range, so nothing of x is shared inside the workgroup: B fragments
+//     come straight from global memory (L2 hits: x is 128 KB per 16 tokens and read by everyone),
+//     one 16-byte load per lane and k-step, no staging, no barrier before the main loop.  Token
+//     rows past n are clamped, not zeroed: a B column only feeds its own output column, which is
+//     never stored.
+//   * Weights and B fragments travel through one ring of U k-steps per wave.
+//   * Decode table and decode as in gemm_kernel.hpp (bit-identical weights).
+//   * Reduction: the WK waves put their LW accumulator planes in LDS; each thread sums two
+//     adjacent output features of one token in wave order and stores them (fused epilogues of
+//     epilogue.hpp).  Deterministic; no workspace, no counters.
+// Requires k % (32*WK*U) == 0, m % (16*LW) == 0, dense launches, at most 16 tokens per
+// workgroup (more tokens: gridDim.y chunks).  Selected by rows_per_wave = 16 or 32 in the config.
+#pragma once
+#include "gemm_kernel.hpp"
+
+namespace tuna {
+
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+template <int LW, int WK, int U>
+__global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const NarrowArgs a)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    static_assert(LW == 1 || LW == 2, "16 or 32 rows per workgroup");
+    unsigned char *lut = smem;
+    float *red = reinterpret_cast<float *>(smem + kLutBytes);  // [wave][plane][lane][4]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int i16 = lane & 15;
+    const int g = lane >> 4;
+    const int wk = __builtin_amdgcn_readfirstlane(tid >> 6);
+    constexpr int nthreads = WK * 64;
+    const uint32_t lane4 = (uint32_t)lane << 2;
+    const int row0 = blockIdx.x * (16 * LW);
+    const int tok0 = blockIdx.y * 16;
+
+    // ---- requests: codebook and scales, then the first ring turn (x fragment, weights) --------
+    const float code_lane = a.code[i16];
+    float sc32[LW];
+    if constexpr (LW == 1) {
+        sc32[0] = a.absmax[row0 + i16];
+    } else {
+        const f32x2 s2 = *reinterpret_cast<const f32x2 *>(a.absmax + row0 + 2 * i16);
+        sc32[0] = s2[0];
+        sc32[1] = s2[1];
+    }
+    const uint32_t kb_total = (uint32_t)a.k >> 3;
+    // per lane: block row and dwords of the block (weights); token row and 8-k group (x)
+    const uint32_t lb = ((uint32_t)(row0 >> 3) + (uint32_t)((LW * i16) >> 3)) * kb_total * 32u +
+                        (uint32_t)((LW * i16) & 7) * 4u + (uint32_t)g * 32u;
+    const uint32_t xoff = ((uint32_t)min(i16, a.n - 1 - tok0) * (uint32_t)a.k + (uint32_t)g * 8u) * 2u;
+    // uniform: this wave's step 0; one ring turn further per group
+    const unsigned char *qp = a.q + (size_t)wk * 128;
+    const unsigned char *xp = reinterpret_cast<const unsigned char *>(a.x) + (size_t)tok0 * a.k * 2 + (size_t)wk * 64;
+    uint32_t wq[U][LW];
+    u32x4 xq[U];
+#define TUNA_NARROW_LOAD(u)                                                                     \
+    {                                                                                          \
+        xq[u] = *reinterpret_cast<const u32x4 *>(xp + (size_t)(u) * (WK * 64) + xoff);         \
+        if constexpr (LW == 1) {                                                               \
+            wq[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(qp + (size_t)(u) * (WK * 128) + lb)); \
+        } else {                                                                               \
+            const u32x2 w2_ = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(qp + (size_t)(u) * (WK * 128) + lb)); \
+            wq[u][0] = w2_[0];                                                                 \
+            wq[u][1] = w2_[1];                                                                 \
+        }                                                                                      \
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) TUNA_NARROW_LOAD(u)
+    qp += (size_t)U * (WK * 128);
+    xp += (size_t)U * (WK * 64);
+
+    // ---- decode table (see gemm_kernel.hpp), built while the loads are in flight ------------
+    {
+        const int code_bits = (int)f16_bits((f16)code_lane);
+        for (int p0 = tid; p0 < kLutBytes / 16; p0 += 4 * nthreads) {
+            uint32_t v[4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int e = (p0 + b * nthreads) >> 4;
+                const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute((e >> 4) << 2, code_bits);
+                const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute((e & 15) << 2, code_bits);
+                v[b] = hi | (lo << 16);
+            }
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int p = p0 + b * nthreads;
+                if (p < kLutBytes / 16) reinterpret_cast<u32x4 *>(lut)[p] = u32x4{v[b], v[b], v[b], v[b]};
+            }
+        }
+    }
+    f16x2 sc16[LW];
+#pragma unroll
+    for (int j = 0; j < LW; ++j) {
+        const f16 h = (f16)sc32[j];
+        sc16[j] = f16x2{h, h};
+    }
+    __syncthreads();  // the table is complete
+
+    // ---- main loop: n_it / U ring turns, the last one without refills ------------------------
+    f32x4 acc[LW];
+#pragma unroll
+    for (int j = 0; j < LW; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#define TUNA_NARROW_CONSUME(u)                                                                  \
+    {                                                                                          \
+        const f16x8 b_ = __builtin_bit_cast(f16x8, xq[u]);                                     \
+        _Pragma("unroll") for (int j = 0; j < LW; ++j)                                         \
+        {                                                                                      \
+            const f16x8 av_ = decode_dword<TUNA_DECODE_GEMM>(wq[u][j], lut, lane4, sc16[j], 0.f); \
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av_, b_, acc[j], 0, 0, 0);         \
+        }                                                                                      \
+    }
+    for (int it = U; it < a.n_it; it += U) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            TUNA_NARROW_CONSUME(u)
+            TUNA_NARROW_LOAD(u)
+            __builtin_amdgcn_sched_barrier(0);  // keep each refill right behind its consume
+        }
+        qp += (size_t)U * (WK * 128);
+        xp += (size_t)U * (WK * 64);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) TUNA_NARROW_CONSUME(u)
+#undef TUNA_NARROW_CONSUME
+#undef TUNA_NARROW_LOAD
+
+    // ---- reduction over the waves and store -----------------------------------------------------
+    // Plane j of a wave: lane l, element v is token l % 16, MFMA row 4*(l/16) + v, weight row
+    // LW*(MFMA row) + j of the workgroup's 16*LW.
+#pragma unroll
+    for (int j = 0; j < LW; ++j) reinterpret_cast<f32x4 *>(red)[(size_t)(wk * LW + j) * 64 + lane] = acc[j];
+    __syncthreads();
+    f16 *outp = reinterpret_cast<f16 *>(a.out);
+    const f16 *resp = reinterpret_cast<const f16 *>(a.residual);
+    constexpr int PAIRS = 128 * LW;  // pairs of adjacent rows x 16 tokens
+#pragma unroll
+    for (int p0 = 0; p0 < PAIRS; p0 += nthreads) {
+        const int pi = p0 + tid;
+        if (PAIRS % nthreads != 0 && pi >= PAIRS) break;
+        const int tk = pi / (8 * LW), rp = pi % (8 * LW);  // token, row pair: rows 2*rp and 2*rp + 1
+        // float index of row 2*rp in wave 0's planes; row 2*rp + 1 is the next element (LW 1) or
+        // the same element of the next plane (LW 2)
+        const int mr = LW == 1 ? 2 * rp : rp;
+        const int f0 = (((mr >> 2) * 16 + tk) << 2) + (mr & 3);
+        constexpr int f1_off = LW == 1 ? 1 : 256;
+        float v0[WK], v1[WK];
+#pragma unroll
+        for (int w = 0; w < WK; ++w) {
+            v0[w] = red[(size_t)w * (LW * 256) + f0];
+            v1[w] = red[(size_t)w * (LW * 256) + f0 + f1_off];
+        }
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int w = 0; w < WK; ++w) {
+            s0 += v0[w];
+            s1 += v1[w];
+        }
+        const int tok = tok0 + tk;
+        if (tok >= a.n) continue;
+        const int col = row0 + 2 * rp;
+        if (a.epilogue == TUNA_EPILOGUE_SILU_MUL) {
+            outp[(size_t)tok * (size_t)(a.m >> 1) + (col >> 1)] = (f16)silu_mul(s0, s1);
+        } else {
+            const size_t at = (size_t)tok * (size_t)a.m + col;
+            if (a.epilogue == TUNA_EPILOGUE_RESIDUAL) {
+                const f16x2 r = *reinterpret_cast<const f16x2 *>(resp + at);
+                s0 += (float)r[0], s1 += (float)r[1];
+            }
+            *reinterpret_cast<f16x2 *>(outp + at) = f16x2{(f16)s0, (f16)s1};
+        }
+    }
+}
+
+}  // namespace tuna

@@ -148,6 +148,20 @@ struct GemmPlan {
 
 // gemm_kernel.hip
 hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream);
+// Narrow-row kernel (gemm_narrow.hpp): 16 or 32 rows per workgroup, all waves along k.
+struct NarrowArgs {
+    const uint8_t *q;
+    const void *x;
+    const float *code;
+    const float *absmax;
+    void *out;
+    const void *residual;
+    int epilogue;
+    int m, n, k;
+    int n_it;  // k-steps per wave: k / 32 / waves
+};
+bool narrow_variant_exists(int rows, int waves_k, int prefetch);
+hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int prefetch, hipStream_t stream);
 int set_lean_kernels(int enabled);  // returns the previous setting
 unsigned long long lean_launches();
 bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves, int grouped);

@@ -50,6 +50,10 @@ VARIANTS_512_2WG = {(1, 2, 1), (1, 4, 1)}
 VARIANTS_1024 = {(1, 2, 1), (1, 4, 1)}
 
 
+# (rows, waves_k, prefetch) of the narrow-row kernel; must match kNarrow in csrc/gemm_launch.hip
+NARROW_VARIANTS = {(r, wk, pf) for r in (16, 32) for wk in (4, 8, 16) for pf in (2, 4, 8)} | {
+    (16, 1, 2), (16, 2, 2), (32, 1, 2), (32, 2, 2)}
+
 # (rows, tokens) tiles of the many-token kernel; must match kTiled in csrc/gemm_tiled.hip
 TILED_VARIANTS = {(256, 128), (256, 64), (128, 256), (128, 128), (64, 256), (64, 128)}
 
@@ -83,8 +87,19 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
         if not 1 <= c["split_k"] <= -(-k // 64):
             raise ValueError("split_k of the many-token kernel must be in 1..ceil(k/64)")
         return
+    if c["rows_per_wave"] in (16, 32):
+        # narrow-row kernel: one workgroup per 16 or 32 rows, all waves along k, no split
+        if (c["waves_m"], c["split_k"], c["token_tiles"], c["k_stagger"]) != (1, 1, 1, 0):
+            raise ValueError("rows_per_wave 16 or 32 needs waves_m=1, split_k=1, token_tiles=1, k_stagger=0")
+        if (c["rows_per_wave"], c["waves_k"], c["prefetch"]) not in NARROW_VARIANTS:
+            raise ValueError("no narrow-row kernel for this rows_per_wave / waves_k / prefetch")
+        if m % c["rows_per_wave"] or k % (STEP_K * c["waves_k"] * c["prefetch"]):
+            raise ValueError("rows_per_wave 16 or 32 needs m a multiple of it and k a multiple of 32*waves_k*prefetch")
+        if m * k // 2 >= 1 << 32 or k * 32 >= 1 << 32:
+            raise ValueError("operands exceed the kernel's 32-bit offsets")
+        return
     if c["rows_per_wave"] not in (64, 128, 256):
-        raise ValueError("rows_per_wave must be 64, 128 or 256")
+        raise ValueError("rows_per_wave must be 16, 32 (narrow-row kernel), 64, 128 or 256")
     if c["prefetch"] not in (2, 4, 8):
         raise ValueError("prefetch must be 2, 4 or 8")
     if c["token_tiles"] not in (1, 2, 4):
@@ -121,6 +136,9 @@ def lds_bytes(c: dict) -> int:
     if c.get("lds_tile_rows"):
         # many-token kernel: decode table + two buffers of (weight tile + activation tile), 128 bytes per row
         return LUT_BYTES + 2 * (c["lds_tile_rows"] + 16 * c["token_tiles"]) * 128
+    if c["rows_per_wave"] in (16, 32):
+        # narrow-row kernel: decode table + one accumulator plane (1 KB) per wave and 16 rows
+        return LUT_BYTES + c["waves_k"] * (c["rows_per_wave"] // 16) * 1024
     threads = 64 * c["waves_k"] * c["waves_m"]
     x = c["token_tiles"] * 16 * c["x_chunk"] * 2
     plane = c["waves_k"] * c["waves_m"] * 1024
