@@ -60,30 +60,38 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const NarrowArgs a
         sc32[1] = s2[1];
     }
     const uint32_t kb_total = (uint32_t)a.k >> 3;
-    // per lane: block row and dwords of the block (weights); token row and 8-k group (x)
+    // A wave walks k in double steps of 64 (two MFMAs): wave wk owns double steps wk, wk + WK, ...
+    // Within a double step the MFMA k slots are permuted so that lane group g holds the two
+    // adjacent 8-k blocks 2g and 2g + 1 (first and second MFMA): the four groups of a token row
+    // then read one whole 128-byte line of x between them instead of half of two lines.  The
+    // weights follow the same permutation (block column 8*dstep + 2g + half).
+    // per lane: block row and dwords of the block (weights); token row and 8-k block (x)
     const uint32_t lb = ((uint32_t)(row0 >> 3) + (uint32_t)((LW * i16) >> 3)) * kb_total * 32u +
-                        (uint32_t)((LW * i16) & 7) * 4u + (uint32_t)g * 32u;
-    const uint32_t xoff = ((uint32_t)min(i16, a.n - 1 - tok0) * (uint32_t)a.k + (uint32_t)g * 8u) * 2u;
-    // uniform: this wave's step 0; one ring turn further per group
-    const unsigned char *qp = a.q + (size_t)wk * 128;
-    const unsigned char *xp = reinterpret_cast<const unsigned char *>(a.x) + (size_t)tok0 * a.k * 2 + (size_t)wk * 64;
+                        (uint32_t)((LW * i16) & 7) * 4u + (uint32_t)g * 64u;
+    const uint32_t xoff = ((uint32_t)min(i16, a.n - 1 - tok0) * (uint32_t)a.k + (uint32_t)g * 16u) * 2u;
+    // uniform: this wave's double step 0; one ring turn (U/2 double steps) further per group
+    const unsigned char *qp = a.q + (size_t)wk * 256;
+    const unsigned char *xp = reinterpret_cast<const unsigned char *>(a.x) + (size_t)tok0 * a.k * 2 + (size_t)wk * 128;
     uint32_t wq[U][LW];
     u32x4 xq[U];
+    static_assert(U % 2 == 0, "whole double steps");
 #define TUNA_NARROW_LOAD(u)                                                                     \
     {                                                                                          \
-        xq[u] = *reinterpret_cast<const u32x4 *>(xp + (size_t)(u) * (WK * 64) + xoff);         \
+        const size_t xo_ = (size_t)((u) >> 1) * (WK * 128) + ((u) & 1) * 16;               \
+        const size_t qo_ = (size_t)((u) >> 1) * (WK * 256) + ((u) & 1) * 32;               \
+        xq[u] = *reinterpret_cast<const u32x4 *>(xp + xo_ + xoff);                             \
         if constexpr (LW == 1) {                                                               \
-            wq[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(qp + (size_t)(u) * (WK * 128) + lb)); \
+            wq[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(qp + qo_ + lb)); \
         } else {                                                                               \
-            const u32x2 w2_ = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(qp + (size_t)(u) * (WK * 128) + lb)); \
+            const u32x2 w2_ = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(qp + qo_ + lb)); \
             wq[u][0] = w2_[0];                                                                 \
             wq[u][1] = w2_[1];                                                                 \
         }                                                                                      \
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) TUNA_NARROW_LOAD(u)
-    qp += (size_t)U * (WK * 128);
-    xp += (size_t)U * (WK * 64);
+    qp += (size_t)(U / 2) * (WK * 256);
+    xp += (size_t)(U / 2) * (WK * 128);
 
     // ---- decode table (see gemm_kernel.hpp), built while the loads are in flight ------------
     {
@@ -132,8 +140,8 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const NarrowArgs a
             TUNA_NARROW_LOAD(u)
             __builtin_amdgcn_sched_barrier(0);  // keep each refill right behind its consume
         }
-        qp += (size_t)U * (WK * 128);
-        xp += (size_t)U * (WK * 64);
+        qp += (size_t)(U / 2) * (WK * 256);
+        xp += (size_t)(U / 2) * (WK * 128);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) TUNA_NARROW_CONSUME(u)

@@ -50,7 +50,7 @@ def repair(c: dict, m: int, n_key: int, k: int):
     c = dict(c)
     c.setdefault("k_stagger", 0)
     c.setdefault("lds_tile_rows", 0)
-    if c["lds_tile_rows"]:
+    if c["lds_tile_rows"] or c["rows_per_wave"] in (16, 32):
         try:
             make_configs.validate(m, n_key, k, c)
             return c
@@ -165,6 +165,25 @@ def lean_space(m: int, n_key: int, k: int):
     return list(uniq.values())
 
 
+def narrow_space(m: int, n_key: int, k: int):
+    """Every config of the narrow-row kernel (gemm_narrow.hpp: 16 or 32 rows per workgroup, all
+    waves along k, no split) the shape admits.  Small enough to time exhaustively."""
+    lo, _ = make_configs.N_BUCKETS[n_key]
+    if lo > 32:
+        return []
+    out = []
+    for rows, wk, pf in sorted(make_configs.NARROW_VARIANTS):
+        c = dict(rows_per_wave=rows, waves_m=1, waves_k=wk, split_k=1, prefetch=pf, x_chunk=32 * wk * pf, token_tiles=1,
+                 xcd_swizzle=0, k_stagger=0, lds_tile_rows=0)
+        try:
+            make_configs.validate(m, n_key, k, c)
+        except ValueError:
+            continue
+        if m // rows <= 8 * N_CU:
+            out.append(c)
+    return out
+
+
 def mutate(c: dict, rng: random.Random, m, n_key, k):
     c = dict(c)
     for _ in range(rng.choice((1, 1, 2))):
@@ -238,6 +257,8 @@ def tune_shape(m, n, k, generations=6, population=24, seed=0, log=print, max_see
     pool = seeds(m, n_key, k)
     rng.shuffle(pool)
     pool = pool[:max_seed_evals] + lean_space(m, n_key, k)
+    for c in narrow_space(m, n_key, k):     # a kernel family of its own: timed, not bred
+        ev(c)
     scored = sorted(((ev(c), json.dumps(c, sort_keys=True)) for c in pool))
     pop = [json.loads(s) for _, s in scored[:population]]
     log(f"  seeds: {len(pool)} evaluated, best {scored[0][0]:.2f} us {scored[0][1]}")
