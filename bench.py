@@ -160,6 +160,17 @@ def main():
         res_graph = time_shape(ops, synth, torch, dev, m, n, k, args.steps, args.warmup, use_graph=True)
     cands = [r for r in (res_stream, res_graph) if r is not None]
     head = min(cands, key=lambda r: r["us_per_gemm"])
+    # which kernel family the headline config runs (the profiles name the same kernel)
+    hc = head["config"]
+    if hc.get("lds_tile_rows"):
+        kernel_name = "tuna::gemm_tiled_kernel"
+    elif hc["rows_per_wave"] < 64:
+        kernel_name = "tuna::gemm_narrow_kernel"
+    else:
+        before = ops.lean_launches()
+        probe = time_shape(ops, synth, torch, dev, m, n, k, 2, 1, use_graph=False)
+        kernel_name = "tuna::gemm_lean_kernel" if ops.lean_launches() > before else "tuna::gemm_kernel"
+        del probe
 
     line = {
         "metric": METRIC,
@@ -191,7 +202,7 @@ def main():
             "unit": "GB/s",
             "frac": round(head["gbs"] / HBM_PEAK_GBS, 4),
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if n == TOKENS else None,
-            "kernel": "tuna::gemm_kernel",
+            "kernel": kernel_name,
             "algorithmic_bytes_per_launch": head["packed_bytes"],
             "avg_launch_us": head["us_per_gemm"],
         },
