@@ -42,9 +42,10 @@ CACHE_BYTES = 256 << 20  # Infinity Cache; the rotation streams at least twice t
 # each scaled by the same counter's reading for the copy kernel of known size); filled in from
 # the summaries under profiles/.  None = not measured for that shape.
 MEASURED_TRAFFIC_BYTES = {
-    # workload: FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 (KiB -> bytes), profiles/gemm_kernel_hbm_traffic_counters.md
-    "mistral_qkv": int((7596.0 * 2.000 + 1735.5 * 1.000) * 1024),
-    "mixtral_gate_up_8e": int((230457.9 * 2.000 + 7168.0 * 1.000) * 1024),
+    # workload: FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 (KiB -> bytes),
+    # profiles/gemm_narrow_kernel_and_gemm_kernel_hbm_traffic_counters.md
+    "mistral_qkv": int((6722.1 * 2.000 + 192.0 * 1.000) * 1024),
+    "mixtral_gate_up_8e": int((230488.3 * 2.000 + 7168.1 * 1.000) * 1024),
 }
 
 
