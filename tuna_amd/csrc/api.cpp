@@ -172,6 +172,7 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     a.split_log2 = (c.split_k > 0 && (c.split_k & (c.split_k - 1)) == 0) ? log2i(c.split_k) : -1;
     a.steps_total = steps_total;
     a.steps_per_split = balanced ? steps_total : ceil_div(steps_total, c.split_k);
+    a.x_slots_magic = (unsigned)((1ull << 32) / (4ull * (unsigned)a.steps_per_split)) + 1u;
     a.balanced = balanced ? 1 : 0;
     a.unit_log2 = unit_log2;
     a.units_per_tile = units_per_tile;

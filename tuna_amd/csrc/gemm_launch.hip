@@ -89,7 +89,7 @@ static constexpr int kNumLean = sizeof(kLean) / sizeof(kLean[0]);
 // The lean kernel's LDS: decode table + max(x slice of the split, reduction planes) + ticket.
 static size_t lean_lds_bytes(const GemmPlan &plan)
 {
-    const size_t x_bytes = (size_t)plan.args.steps_per_split * 1024;  // 16 tokens x 32 k x 2 bytes per k-step
+    const size_t x_bytes = (size_t)plan.args.steps_per_split * 1088;  // 4 slots of 16 tokens x 16 bytes + 16 bytes of padding per k-step
     const size_t red_bytes = (size_t)(plan.threads / 64) * 4096;
     return (size_t)kLutBytes + (x_bytes > red_bytes ? x_bytes : red_bytes) + 16;
 }

@@ -84,25 +84,35 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
     //      codebook, scales, x slice, first ring turn of weights -----------------------------------
     const float code_lane = a.code[i16];
     const f32x4 sc32 = *reinterpret_cast<const f32x4 *>(a.absmax + row0 + i16 * 4);
-    // x slice [16 tokens][k of this split]: piece p = tid + b*nthreads is token p % 16, 8-k slot
-    // p / 16, LDS byte 16*p.  64 * steps_per_split pieces, at most 8 per thread.
-    const int x_pieces = a.steps_per_split * 64;
-    const int xr = tid & 15;
-    const bool x_row_ok = tok0 + xr < a.n;
-    const unsigned char *xrow = reinterpret_cast<const unsigned char *>(a.x) +
-                                ((size_t)min(tok0 + xr, a.n - 1) * a.k + (size_t)sb * 32 + (size_t)(tid >> 4) * 8) * 2;
-    const int x_slots = a.steps_per_split * 4;  // 8-k slots of the slice
-    const int x_slot0 = tid >> 4, x_slot_step = nthreads >> 4;
+    // x slice [16 tokens][k of this split], in 16-byte pieces (one token, one 8-k slot).  Piece
+    // p = tid + b*nthreads is token p / x_slots, slot p % x_slots: consecutive lanes read
+    // consecutive bytes of one token row (a wave instruction that touches 16 rows instead costs
+    // three times the cycles in the address path).  In LDS slot s, token t sits at byte
+    // s*272 + t*16: the 16 tokens of a slot are one contiguous B-fragment row, and the 16-byte pad
+    // per slot spreads the staging writes (consecutive slots, same token) over all banks.
+    // 64 * steps_per_split pieces, at most 8 per thread.
+    const int x_slots = a.steps_per_split * 4;
+    const int x_pieces = x_slots * 16;
+    const unsigned char *xsl = reinterpret_cast<const unsigned char *>(a.x) + ((size_t)tok0 * a.k + (size_t)sb * 32) * 2;
+    const int n_rel = a.n - 1 - tok0;  // last valid token row of this tile, relative
     u32x4 xv[8];
+    uint32_t xl[8];  // LDS byte of each piece, bit 0: token row past n (store zeros); ~0u: no piece
     const bool x_long = x_pieces > 4 * nthreads;  // uniform
+#define TUNA_LEAN_XLOAD(b)                                                                      \
+    {                                                                                          \
+        const uint32_t p_ = min((uint32_t)(tid + (b) * nthreads), (uint32_t)x_pieces - 1u);    \
+        const uint32_t t_ = __umulhi(p_, (uint32_t)a.x_slots_magic);                           \
+        const uint32_t s_ = p_ - t_ * (uint32_t)x_slots;                                       \
+        xl[b] = (tid + (b) * nthreads) < x_pieces ? (s_ * 272u + t_ * 16u) | ((int)t_ > n_rel ? 1u : 0u) : ~0u; \
+        xv[b] = *reinterpret_cast<const u32x4 *>(xsl + ((size_t)min((int)t_, n_rel) * a.k + (size_t)s_ * 8) * 2); \
+    }
 #pragma unroll
-    for (int b = 0; b < 4; ++b)  // (clamped: a short slice has fewer than 4 pieces per thread)
-        xv[b] = *reinterpret_cast<const u32x4 *>(xrow + (size_t)(min(x_slot0 + b * x_slot_step, x_slots - 1) - x_slot0) * 16);
+    for (int b = 0; b < 4; ++b) TUNA_LEAN_XLOAD(b)
     if (x_long) {
 #pragma unroll
-        for (int b = 4; b < 8; ++b)
-            xv[b] = *reinterpret_cast<const u32x4 *>(xrow + (size_t)(min(x_slot0 + b * x_slot_step, x_slots - 1) - x_slot0) * 16);
+        for (int b = 4; b < 8; ++b) TUNA_LEAN_XLOAD(b)
     }
+#undef TUNA_LEAN_XLOAD
 
     // the weights last: x and the scales come from L2 and are needed first, the first ring turn
     // comes from HBM and is needed once x is staged
@@ -144,16 +154,12 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
     }
     // ---- x into LDS; one barrier publishes the table and the slice ---------------------------
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
-        const int p = tid + b * nthreads;
-        if (p < x_pieces) *reinterpret_cast<u32x4 *>(work + (size_t)p * 16) = x_row_ok ? xv[b] : u32x4{0u, 0u, 0u, 0u};
-    }
+    for (int b = 0; b < 4; ++b)
+        if (xl[b] != ~0u) *reinterpret_cast<u32x4 *>(work + (xl[b] & ~1u)) = (xl[b] & 1u) ? u32x4{0u, 0u, 0u, 0u} : xv[b];
     if (x_long) {
 #pragma unroll
-        for (int b = 4; b < 8; ++b) {
-            const int p = tid + b * nthreads;
-            if (p < x_pieces) *reinterpret_cast<u32x4 *>(work + (size_t)p * 16) = x_row_ok ? xv[b] : u32x4{0u, 0u, 0u, 0u};
-        }
+        for (int b = 4; b < 8; ++b)
+            if (xl[b] != ~0u) *reinterpret_cast<u32x4 *>(work + (xl[b] & ~1u)) = (xl[b] & 1u) ? u32x4{0u, 0u, 0u, 0u} : xv[b];
     }
     __syncthreads();
     TUNA_LMARK(3)
@@ -162,8 +168,8 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
     f32x4 acc[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const unsigned char *xb = work + g * 256 + i16 * 16 + wk * 1024;  // B fragment of this wave's step 0
-    constexpr int wstep = WK * 1024;                                   // LDS bytes between its consecutive steps
+    const unsigned char *xb = work + g * 272 + i16 * 16 + wk * 1088;  // B fragment of this wave's step 0 (4 slots of 272 bytes per step)
+    constexpr int wstep = WK * 1088;                                   // LDS bytes between its consecutive steps
 #define TUNA_LEAN_CONSUME(u)                                                                    \
     {                                                                                          \
         const f16x8 b_ = *reinterpret_cast<const f16x8 *>(xb + (u) * wstep);                   \
