@@ -72,9 +72,16 @@ bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int 
 }
 
 // ---- lean twins (gemm_lean.hpp) -------------------------------------------------------------
+typedef void (*LeanKernelFn)(const uint8_t *, const void *, const float *, const float *, int, int, int, unsigned, int, int,
+                             void *, const void *, float *, unsigned *, int
+#ifdef TUNA_TRACE
+                             ,
+                             unsigned long long *
+#endif
+);
 struct LeanVariant {
     int wk, u, maxt;
-    GemmKernelFn fn;
+    LeanKernelFn fn;
 };
 #define L5(WK, U) {WK, U, 512, gemm_lean_kernel<WK, U, 512, 2>}
 #define L10(WK, U) {WK, U, 1024, gemm_lean_kernel<WK, U, 1024, 4>}
@@ -114,6 +121,8 @@ static const LeanVariant *lean_applies(const GemmPlan &plan, int cus)
     if (a.m % (a.waves_m * kRowsPerLoad) != 0) return nullptr;
     if (a.steps_per_split * 64 > 8 * plan.threads) return nullptr;  // at most 8 pieces of x per thread
     if (lean_lds_bytes(plan) > (size_t)kLdsLimit) return nullptr;
+    if (plan.grid.x >= (1u << 19) || a.split_log2 > 15 || a.epilogue > 3) return nullptr;  // fields of the packed argument
+    if (a.k >= (1 << 23)) return nullptr;  // 24-bit row pitch in the x staging
     // all tiles at once: workgroups per CU by LDS and by registers (at most 96 per lane: five
     // waves per SIMD); a launch of several rounds is what the tile walk of gemm_kernel is for
     const int waves = plan.threads / 64;
@@ -165,7 +174,17 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
                 g_lean_attr_done[dev][li] = 1;
             }
         }
-        hipLaunchKernelGGL(lv->fn, plan.grid, dim3(plan.threads), lean_lds_bytes(plan), stream, plan.args);
+        const GemmArgs &a = plan.args;
+        const int swz = a.xcd_swizzle && plan.grid.x % 8 == 0;
+        const int packed = a.split_log2 | a.waves_m << 4 | a.epilogue << 9 | swz << 11 | (int)(plan.grid.x >> 3) << 12;
+        hipLaunchKernelGGL(lv->fn, plan.grid, dim3(plan.threads), lean_lds_bytes(plan), stream, a.q, a.x, a.code, a.absmax,
+                           a.k, a.n, a.steps_per_split, a.x_slots_magic, packed, a.m, a.out, a.residual, a.ws, a.counters,
+                           a.row_tiles
+#ifdef TUNA_TRACE
+                           ,
+                           a.trace
+#endif
+        );
         g_lean_launches.fetch_add(1, std::memory_order_relaxed);
         return hipGetLastError();
     }
@@ -199,7 +218,8 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
 }
 
 // ---- narrow-row kernel (gemm_narrow.hpp) ---------------------------------------------------------
-typedef void (*NarrowKernelFn)(const NarrowArgs);
+typedef void (*NarrowKernelFn)(const uint8_t *, const void *, const float *, const float *, int, int, int, int, void *, int,
+                               const void *);
 struct NarrowVariant {
     int rows, wk, u;
     NarrowKernelFn fn;
@@ -243,7 +263,8 @@ hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int
     }
     const size_t lds = (size_t)kLutBytes + (size_t)waves_k * (rows / 16) * 1024;
     const dim3 grid((unsigned)(args.m / rows), (unsigned)((args.n + 15) / 16), 1);
-    hipLaunchKernelGGL(v->fn, grid, dim3(waves_k * 64), lds, stream, args);
+    hipLaunchKernelGGL(v->fn, grid, dim3(waves_k * 64), lds, stream, args.q, args.x, args.code, args.absmax, args.k, args.n,
+                       args.n_it, args.m, args.out, args.epilogue, args.residual);
     return hipGetLastError();
 }
 

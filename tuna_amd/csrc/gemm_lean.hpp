@@ -36,9 +36,65 @@ __device__ __forceinline__ void load_partials4(const float *s0, const float *s1,
         : "memory");
 }
 
+// What the kernel needs of GemmArgs, as separate scalar arguments with the ones the first loads
+// use in front: the first 14 dwords of such arguments are preloaded into scalar registers with
+// the wave (build flag -amdgpu-kernarg-preload-count), a struct passed by value is fetched by
+// the kernel itself - a round trip to memory before anything else can start.
+struct LeanArgs {
+    const uint8_t *q;
+    const void *x;
+    const float *code;
+    const float *absmax;
+    int k, n, steps_per_split;
+    unsigned x_slots_magic;
+    int packed;  // split_log2 | waves_m << 4 | epilogue << 9 | swizzle << 11 | (workgroups / 8) << 12
+    int m;
+    void *out;
+    const void *residual;
+    float *ws;
+    unsigned *counters;
+    int row_tiles;
+#ifdef TUNA_TRACE
+    unsigned long long *trace;
+#endif
+};
+
 template <int WK, int U, int MAXT, int MINW>
-__global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
+__global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_q, const void *a_x, const float *a_code,
+                                                               const float *a_absmax, int a_k, int a_n, int a_sps,
+                                                               unsigned a_magic, int a_packed, int a_m, void *a_out,
+                                                               const void *a_residual, float *a_ws, unsigned *a_counters,
+                                                               int a_row_tiles
+#ifdef TUNA_TRACE
+                                                               ,
+                                                               unsigned long long *a_trace
+#endif
+)
 {
+    struct {
+        const uint8_t *q;
+        const void *x;
+        const float *code;
+        const float *absmax;
+        void *out;
+        const void *residual;
+        float *ws;
+        unsigned *counters;
+        int m, n, k, steps_per_split, row_tiles, split_log2, split_k, waves_m, xcd_swizzle, epilogue;
+        unsigned x_slots_magic;
+#ifdef TUNA_TRACE
+        unsigned long long *trace;
+#endif
+    } const a = {a_q,           a_x,          a_code,          a_absmax,
+                 a_out,         a_residual,   a_ws,            a_counters,
+                 a_m,           a_n,          a_k,             a_sps,
+                 a_row_tiles,   a_packed & 15, 1 << (a_packed & 15), (a_packed >> 4) & 31,
+                 (a_packed >> 11) & 1, (a_packed >> 9) & 3, a_magic
+#ifdef TUNA_TRACE
+                 ,
+                 a_trace
+#endif
+    };
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int WK_LOG2 = WK == 1 ? 0 : WK == 2 ? 1 : WK == 4 ? 2 : WK == 8 ? 3 : 4;
     constexpr int TT = 1;
@@ -66,12 +122,13 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wk = wave & (WK - 1);
     const int wm = wave >> WK_LOG2;
-    const int nthreads = (int)blockDim.x;
+    const int nthreads = a.waves_m * (WK * 64);  // (blockDim would be a fetch from the argument segment)
     const uint32_t lane4 = (uint32_t)lane << 2;
 
     int wg = blockIdx.x;
-    const int n_wg = gridDim.x;
-    if (a.xcd_swizzle && (n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
+    // (the host sets the swizzle bit only for a workgroup count that is a multiple of 8, and passes
+    // an eighth of the count: reading gridDim here would be a fetch from the argument segment)
+    if (a.xcd_swizzle) wg = (wg & 7) * (a_packed >> 12) + (wg >> 3);
     const int row_tile = wg >> a.split_log2;
     const int part = wg & (a.split_k - 1);
     const int sb = part * a.steps_per_split;  // first k-step of this workgroup
@@ -98,13 +155,24 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const GemmArgs a)
     u32x4 xv[8];
     uint32_t xl[8];  // LDS byte of each piece, bit 0: token row past n (store zeros); ~0u: no piece
     const bool x_long = x_pieces > 4 * nthreads;  // uniform
+    // (token, slot) of the thread's first piece by one division (multiplication by the host's
+    // reciprocal); the following pieces are nthreads further: a uniform number of token rows and
+    // slots, with one carry
+    const uint32_t x_dt = __umulhi((uint32_t)nthreads, a.x_slots_magic), x_ds = (uint32_t)nthreads - x_dt * (uint32_t)x_slots;
+    uint32_t x_t = __umulhi((uint32_t)tid, a.x_slots_magic), x_s = (uint32_t)tid - x_t * (uint32_t)x_slots;
+    // (32-bit offsets off the uniform base: 16 token rows of at most 2^26 k)
+    const uint32_t row_bytes = (uint32_t)a.k * 2u;
 #define TUNA_LEAN_XLOAD(b)                                                                      \
     {                                                                                          \
-        const uint32_t p_ = min((uint32_t)(tid + (b) * nthreads), (uint32_t)x_pieces - 1u);    \
-        const uint32_t t_ = __umulhi(p_, (uint32_t)a.x_slots_magic);                           \
-        const uint32_t s_ = p_ - t_ * (uint32_t)x_slots;                                       \
-        xl[b] = (tid + (b) * nthreads) < x_pieces ? (s_ * 272u + t_ * 16u) | ((int)t_ > n_rel ? 1u : 0u) : ~0u; \
-        xv[b] = *reinterpret_cast<const u32x4 *>(xsl + ((size_t)min((int)t_, n_rel) * a.k + (size_t)s_ * 8) * 2); \
+        const uint32_t tc_ = (uint32_t)min((int)min(x_t, 15u), n_rel); /* past the slice or past n: a valid row */ \
+        xl[b] = (tid + (b) * nthreads) < x_pieces ? (x_s * 272u + x_t * 16u) | ((int)x_t > n_rel ? 1u : 0u) : ~0u; \
+        xv[b] = *reinterpret_cast<const u32x4 *>(xsl + (__umul24(tc_, row_bytes) + x_s * 16u)); \
+        x_t += x_dt;                                                                           \
+        x_s += x_ds;                                                                           \
+        if (x_s >= (uint32_t)x_slots) {                                                        \
+            x_s -= (uint32_t)x_slots;                                                          \
+            ++x_t;                                                                             \
+        }                                                                                      \
     }
 #pragma unroll
     for (int b = 0; b < 4; ++b) TUNA_LEAN_XLOAD(b)

@@ -31,9 +31,24 @@ namespace tuna {
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
+// The arguments are separate scalars, the ones the first loads need in front: the first 16
+// dwords of a kernel's arguments can be preloaded into scalar registers with the wave (built
+// with -amdgpu-kernarg-preload-count=16), which takes the argument fetch - a round trip to
+// memory - off the start of every wave.  A struct passed by value is not preloaded.
 template <int LW, int WK, int U>
-__global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const NarrowArgs a)
+__global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q, const void *a_x, const float *a_code,
+                                                              const float *a_absmax, int a_k, int a_n, int a_n_it, int a_m,
+                                                              void *a_out, int a_epilogue, const void *a_residual)
 {
+    struct {
+        const uint8_t *q;
+        const void *x;
+        const float *code;
+        const float *absmax;
+        void *out;
+        const void *residual;
+        int epilogue, m, n, k, n_it;
+    } const a = {a_q, a_x, a_code, a_absmax, a_out, a_residual, a_epilogue, a_m, a_n, a_k, a_n_it};
     extern __shared__ __align__(16) unsigned char smem[];
     static_assert(LW == 1 || LW == 2, "16 or 32 rows per workgroup");
     unsigned char *lut = smem;
