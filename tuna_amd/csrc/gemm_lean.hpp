@@ -157,22 +157,25 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
     const bool x_long = x_pieces > 4 * nthreads;  // uniform
     // (token, slot) of the thread's first piece by one division (multiplication by the host's
     // reciprocal); the following pieces are nthreads further: a uniform number of token rows and
-    // slots, with one carry
+    // slots, with one carry.  The global and the LDS offset of a piece advance the same way.
+    // Rows past n are loaded from the last valid row (offsets clamped) and stored as zeros.
+    const uint32_t row_bytes = (uint32_t)a.k * 2u;  // (32-bit offsets off the uniform base: 16 rows of at most 2^23 k)
     const uint32_t x_dt = __umulhi((uint32_t)nthreads, a.x_slots_magic), x_ds = (uint32_t)nthreads - x_dt * (uint32_t)x_slots;
     uint32_t x_t = __umulhi((uint32_t)tid, a.x_slots_magic), x_s = (uint32_t)tid - x_t * (uint32_t)x_slots;
-    // (32-bit offsets off the uniform base: 16 token rows of at most 2^26 k)
-    const uint32_t row_bytes = (uint32_t)a.k * 2u;
+    uint32_t x_go = x_t * row_bytes + x_s * 16u, x_lo = x_s * 272u + x_t * 16u;
+    const uint32_t go_step = x_dt * row_bytes + x_ds * 16u, lo_step = x_ds * 272u + x_dt * 16u;  // uniform
+    const uint32_t go_carry = row_bytes - (uint32_t)x_slots * 16u, lo_carry = 16u - (uint32_t)x_slots * 272u;
+    const uint32_t go_max = (uint32_t)min(n_rel, 15) * row_bytes + (uint32_t)(x_slots - 1) * 16u;
 #define TUNA_LEAN_XLOAD(b)                                                                      \
     {                                                                                          \
-        const uint32_t tc_ = (uint32_t)min((int)min(x_t, 15u), n_rel); /* past the slice or past n: a valid row */ \
-        xl[b] = (tid + (b) * nthreads) < x_pieces ? (x_s * 272u + x_t * 16u) | ((int)x_t > n_rel ? 1u : 0u) : ~0u; \
-        xv[b] = *reinterpret_cast<const u32x4 *>(xsl + (__umul24(tc_, row_bytes) + x_s * 16u)); \
-        x_t += x_dt;                                                                           \
+        xl[b] = (tid + (b) * nthreads) < x_pieces ? x_lo | ((int)x_t > n_rel ? 1u : 0u) : ~0u;  \
+        xv[b] = *reinterpret_cast<const u32x4 *>(xsl + min(x_go, go_max));                     \
         x_s += x_ds;                                                                           \
-        if (x_s >= (uint32_t)x_slots) {                                                        \
-            x_s -= (uint32_t)x_slots;                                                          \
-            ++x_t;                                                                             \
-        }                                                                                      \
+        const bool carry_ = x_s >= (uint32_t)x_slots;                                          \
+        x_s -= carry_ ? (uint32_t)x_slots : 0u;                                                \
+        x_t += x_dt + (carry_ ? 1u : 0u);                                                      \
+        x_go += go_step + (carry_ ? go_carry : 0u);                                            \
+        x_lo += lo_step + (carry_ ? lo_carry : 0u);                                            \
     }
 #pragma unroll
     for (int b = 0; b < 4; ++b) TUNA_LEAN_XLOAD(b)
