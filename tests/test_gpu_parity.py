@@ -698,11 +698,15 @@ NARROW_CASES = [
     (128, 16, 64, 16, 1, 2),        # a single wave: two passes over the row pairs
     (128, 33, 256, 32, 1, 2),
     (4096, 16, 4096, 16, 16, 2),    # full-size attention output projection, 256 workgroups
+    (256, 16, 2048, 64, 8, 4),      # 64 rows per workgroup (waves_m = 0 selects the kernel)
+    (192, 19, 1024, 64, 4, 8),
+    (128, 7, 4096, 64, 16, 2),
 ]
 
 
 def narrow_cfg(rows, wk, pf):
-    return cfg(rows_per_wave=rows, waves_m=1, waves_k=wk, split_k=1, prefetch=pf, x_chunk=32 * wk * pf, token_tiles=1)
+    return cfg(rows_per_wave=rows, waves_m=0 if rows == 64 else 1, waves_k=wk, split_k=1, prefetch=pf, x_chunk=32 * wk * pf,
+               token_tiles=1)
 
 
 @pytest.mark.parametrize("ci", range(len(NARROW_CASES)))
@@ -741,7 +745,7 @@ def test_narrow_row_kernel_matches_oracle(ci):
     assert torch.equal(again.view(torch.int16), out.view(torch.int16))
 
 
-@pytest.mark.parametrize("rows,wk,pf", [(16, 4, 2), (32, 8, 4), (32, 16, 2)])
+@pytest.mark.parametrize("rows,wk,pf", [(16, 4, 2), (32, 8, 4), (32, 16, 2), (64, 8, 2)])
 def test_narrow_row_kernel_decode_readout_is_bit_exact(rows, wk, pf):
     """One-hot activations read the narrow-row kernel's in-register decode out: the oracle's D1 image."""
     m, k = 256, 2048

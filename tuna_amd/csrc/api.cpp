@@ -233,7 +233,11 @@ struct NarrowPlan {
     size_t lds_bytes;
 };
 
-static inline bool is_narrow(const tuna_gemm_config &c) { return !c.lds_tile_rows && (c.rows_per_wave == 16 || c.rows_per_wave == 32); }
+// rows_per_wave 16 or 32, or 64 with waves_m = 0 (64 rows with waves_m >= 1 is the streaming kernel)
+static inline bool is_narrow(const tuna_gemm_config &c)
+{
+    return !c.lds_tile_rows && (c.rows_per_wave == 16 || c.rows_per_wave == 32 || (c.rows_per_wave == 64 && c.waves_m == 0));
+}
 
 static int plan_narrow(int m, int n, int k, const tuna_gemm_config &c, int decode, NarrowPlan *plan)
 {
@@ -243,10 +247,11 @@ static int plan_narrow(int m, int n, int k, const tuna_gemm_config &c, int decod
         return fail(TUNA_ERR_UNSUPPORTED, "the narrow-row kernel (rows_per_wave 16, 32) implements TUNA_DECODE_GEMM only");
     if ((unsigned long long)m * (unsigned long long)k / 2 >= (1ull << 32) || (unsigned long long)k * 32 >= (1ull << 32))
         return fail(TUNA_ERR_UNSUPPORTED, "operands exceed the kernel's 32-bit offsets");
-    if (c.waves_m != 1 || c.split_k != 1 || c.token_tiles != 1 || c.k_stagger != 0)
+    if (c.waves_m != (c.rows_per_wave == 64 ? 0 : 1) || c.split_k != 1 || c.token_tiles != 1 || c.k_stagger != 0)
         return fail(TUNA_ERR_UNSUPPORTED,
-                    "rows_per_wave=%d needs waves_m=1, split_k=1, token_tiles=1, k_stagger=0 (got %d, %d, %d, %d)",
-                    c.rows_per_wave, c.waves_m, c.split_k, c.token_tiles, c.k_stagger);
+                    "the narrow-row kernel needs waves_m=1 (0 with rows_per_wave=64), split_k=1, token_tiles=1, k_stagger=0 "
+                    "(got %d, %d, %d, %d)",
+                    c.waves_m, c.split_k, c.token_tiles, c.k_stagger);
     if (!is_pow2(c.waves_k) || c.waves_k > 16 || !narrow_variant_exists(c.rows_per_wave, c.waves_k, c.prefetch))
         return fail(TUNA_ERR_UNSUPPORTED, "no narrow-row kernel for rows_per_wave=%d waves_k=%d prefetch=%d", c.rows_per_wave,
                     c.waves_k, c.prefetch);
@@ -482,7 +487,7 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
     if (is_narrow(c)) {
         NarrowPlan np;
         if ((rc = plan_narrow(m, n, k, c, decode, &np))) return rc;
-        if ((rc = check_ptr(absmax, "absmax", 8))) return rc;  // scales are read two rows at a time
+        if ((rc = check_ptr(absmax, "absmax", np.rows == 64 ? 16 : 8))) return rc;  // scales are read 2 or 4 rows at a time
         np.args.q = static_cast<const uint8_t *>(q);
         np.args.x = x;
         np.args.code = static_cast<const float *>(code);

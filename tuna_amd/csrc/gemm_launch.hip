@@ -229,6 +229,7 @@ static const NarrowVariant kNarrow[] = {
     N(1, 4, 2),  N(1, 4, 4),  N(1, 4, 8),  N(1, 8, 2),  N(1, 8, 4),  N(1, 8, 8),  N(1, 16, 2), N(1, 16, 4), N(1, 16, 8),
     N(2, 4, 2),  N(2, 4, 4),  N(2, 4, 8),  N(2, 8, 2),  N(2, 8, 4),  N(2, 8, 8),  N(2, 16, 2), N(2, 16, 4), N(2, 16, 8),
     N(1, 1, 2),  N(1, 2, 2),  N(2, 1, 2),  N(2, 2, 2),
+    N(4, 4, 2),  N(4, 4, 4),  N(4, 4, 8),  N(4, 8, 2),  N(4, 8, 4),  N(4, 8, 8),  N(4, 16, 2), N(4, 16, 4), N(4, 16, 8),
 };
 #undef N
 static constexpr int kNumNarrow = sizeof(kNarrow) / sizeof(kNarrow[0]);

@@ -1,10 +1,10 @@
-// Narrow-row GEMM kernel for the smallest launches (gfx950, wave64): 16 or 32 weight rows per
+// Narrow-row GEMM kernel for the smallest launches (gfx950, wave64): 16, 32 or 64 weight rows per
 // workgroup, all waves of the workgroup along k, no split across workgroups.
 //
 // With 64 rows per wave a 4096..8192-row projection has only 64..128 row groups, so filling
 // 256 CUs takes a split of k across workgroups, and its hand-over (partial sums through
 // memory, an arrival counter, a finishing pass) costs three dependent round trips: 2 us of an
-// 8 us launch.  Here a workgroup owns 16*LW rows (LW = 1, 2): 256..512 workgroups from the
+// 8 us launch.  Here a workgroup owns 16*LW rows (LW = 1, 2, 4): 256..512 workgroups from the
 // rows alone, the k range is divided over the WK waves of the workgroup, and the only
 // reduction is the one through LDS.
 //   * MFMA v_mfma_f32_16x16x32_f16 as in gemm_kernel.hpp (weights = A, activations = B).  Lane
@@ -22,7 +22,8 @@
 //     adjacent output features of one token in wave order and stores them (fused epilogues of
 //     epilogue.hpp).  Deterministic; no workspace, no counters.
 // Requires k % (32*WK*U) == 0, m % (16*LW) == 0, dense launches, at most 16 tokens per
-// workgroup (more tokens: gridDim.y chunks).  Selected by rows_per_wave = 16 or 32 in the config.
+// workgroup (more tokens: gridDim.y chunks).  Selected by rows_per_wave = 16 or 32 in the config,
+// or by rows_per_wave = 64 with waves_m = 0.
 #pragma once
 #include "gemm_kernel.hpp"
 
@@ -50,7 +51,7 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
         int epilogue, m, n, k, n_it;
     } const a = {a_q, a_x, a_code, a_absmax, a_out, a_residual, a_epilogue, a_m, a_n, a_k, a_n_it};
     extern __shared__ __align__(16) unsigned char smem[];
-    static_assert(LW == 1 || LW == 2, "16 or 32 rows per workgroup");
+    static_assert(LW == 1 || LW == 2 || LW == 4, "16, 32 or 64 rows per workgroup");
     unsigned char *lut = smem;
     float *red = reinterpret_cast<float *>(smem + kLutBytes);  // [wave][plane][lane][4]
 
@@ -69,10 +70,14 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     float sc32[LW];
     if constexpr (LW == 1) {
         sc32[0] = a.absmax[row0 + i16];
-    } else {
+    } else if constexpr (LW == 2) {
         const f32x2 s2 = *reinterpret_cast<const f32x2 *>(a.absmax + row0 + 2 * i16);
         sc32[0] = s2[0];
         sc32[1] = s2[1];
+    } else {
+        const f32x4 s4 = *reinterpret_cast<const f32x4 *>(a.absmax + row0 + 4 * i16);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sc32[j] = s4[j];
     }
     const uint32_t kb_total = (uint32_t)a.k >> 3;
     // A wave walks k in double steps of 64 (two MFMAs): wave wk owns double steps wk, wk + WK, ...
@@ -97,10 +102,13 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
         xq[u] = *reinterpret_cast<const u32x4 *>(xp + xo_ + xoff);                             \
         if constexpr (LW == 1) {                                                               \
             wq[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(qp + qo_ + lb)); \
-        } else {                                                                               \
+        } else if constexpr (LW == 2) {                                                        \
             const u32x2 w2_ = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(qp + qo_ + lb)); \
             wq[u][0] = w2_[0];                                                                 \
             wq[u][1] = w2_[1];                                                                 \
+        } else {                                                                               \
+            const u32x4 w4_ = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(qp + qo_ + lb)); \
+            _Pragma("unroll") for (int j = 0; j < 4; ++j) wq[u][j] = w4_[j];                   \
         }                                                                                      \
     }
 #pragma unroll
@@ -178,9 +186,9 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
         if (PAIRS % nthreads != 0 && pi >= PAIRS) break;
         const int tk = pi / (8 * LW), rp = pi % (8 * LW);  // token, row pair: rows 2*rp and 2*rp + 1
         // float index of row 2*rp in wave 0's planes; row 2*rp + 1 is the next element (LW 1) or
-        // the same element of the next plane (LW 2)
-        const int mr = LW == 1 ? 2 * rp : rp;
-        const int f0 = (((mr >> 2) * 16 + tk) << 2) + (mr & 3);
+        // the same element of the next plane (LW 2, 4)
+        const int mr = (2 * rp) / LW, j0 = (2 * rp) % LW;  // MFMA row and plane of row 2*rp
+        const int f0 = j0 * 256 + (((mr >> 2) * 16 + tk) << 2) + (mr & 3);
         constexpr int f1_off = LW == 1 ? 1 : 256;
         float v0[WK], v1[WK];
 #pragma unroll

@@ -51,7 +51,7 @@ VARIANTS_1024 = {(1, 2, 1), (1, 4, 1)}
 
 
 # (rows, waves_k, prefetch) of the narrow-row kernel; must match kNarrow in csrc/gemm_launch.hip
-NARROW_VARIANTS = {(r, wk, pf) for r in (16, 32) for wk in (4, 8, 16) for pf in (2, 4, 8)} | {
+NARROW_VARIANTS = {(r, wk, pf) for r in (16, 32, 64) for wk in (4, 8, 16) for pf in (2, 4, 8)} | {
     (16, 1, 2), (16, 2, 2), (32, 1, 2), (32, 2, 2)}
 
 # (rows, tokens) tiles of the many-token kernel; must match kTiled in csrc/gemm_tiled.hip
@@ -68,6 +68,11 @@ def bucket_of(n: int):
         if lo <= n <= hi:
             return key
     raise ValueError(f"n={n} outside every token bucket")
+
+
+def is_narrow(c: dict) -> bool:
+    """The config selects the narrow-row kernel: rows_per_wave 16 or 32, or 64 with waves_m 0."""
+    return not c.get("lds_tile_rows") and (c["rows_per_wave"] in (16, 32) or (c["rows_per_wave"] == 64 and c["waves_m"] == 0))
 
 
 def validate(m: int, n_key: int, k: int, c: dict) -> None:
@@ -87,10 +92,11 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
         if not 1 <= c["split_k"] <= -(-k // 64):
             raise ValueError("split_k of the many-token kernel must be in 1..ceil(k/64)")
         return
-    if c["rows_per_wave"] in (16, 32):
-        # narrow-row kernel: one workgroup per 16 or 32 rows, all waves along k, no split
-        if (c["waves_m"], c["split_k"], c["token_tiles"], c["k_stagger"]) != (1, 1, 1, 0):
-            raise ValueError("rows_per_wave 16 or 32 needs waves_m=1, split_k=1, token_tiles=1, k_stagger=0")
+    if is_narrow(c):
+        # narrow-row kernel: one workgroup per 16, 32 or 64 rows, all waves along k, no split
+        if (c["waves_m"], c["split_k"], c["token_tiles"], c["k_stagger"]) != (0 if c["rows_per_wave"] == 64 else 1, 1, 1, 0):
+            raise ValueError("the narrow-row kernel needs waves_m=1 (0 with rows_per_wave 64), split_k=1, token_tiles=1, "
+                             "k_stagger=0")
         if (c["rows_per_wave"], c["waves_k"], c["prefetch"]) not in NARROW_VARIANTS:
             raise ValueError("no narrow-row kernel for this rows_per_wave / waves_k / prefetch")
         if m % c["rows_per_wave"] or k % (STEP_K * c["waves_k"] * c["prefetch"]):
@@ -136,7 +142,7 @@ def lds_bytes(c: dict) -> int:
     if c.get("lds_tile_rows"):
         # many-token kernel: decode table + two buffers of (weight tile + activation tile), 128 bytes per row
         return LUT_BYTES + 2 * (c["lds_tile_rows"] + 16 * c["token_tiles"]) * 128
-    if c["rows_per_wave"] in (16, 32):
+    if is_narrow(c):
         # narrow-row kernel: decode table + one accumulator plane (1 KB) per wave and 16 rows
         return LUT_BYTES + c["waves_k"] * (c["rows_per_wave"] // 16) * 1024
     threads = 64 * c["waves_k"] * c["waves_m"]

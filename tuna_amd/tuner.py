@@ -50,7 +50,7 @@ def repair(c: dict, m: int, n_key: int, k: int):
     c = dict(c)
     c.setdefault("k_stagger", 0)
     c.setdefault("lds_tile_rows", 0)
-    if c["lds_tile_rows"] or c["rows_per_wave"] in (16, 32):
+    if c["lds_tile_rows"] or make_configs.is_narrow(c):
         try:
             make_configs.validate(m, n_key, k, c)
             return c
@@ -173,8 +173,8 @@ def narrow_space(m: int, n_key: int, k: int):
         return []
     out = []
     for rows, wk, pf in sorted(make_configs.NARROW_VARIANTS):
-        c = dict(rows_per_wave=rows, waves_m=1, waves_k=wk, split_k=1, prefetch=pf, x_chunk=32 * wk * pf, token_tiles=1,
-                 xcd_swizzle=0, k_stagger=0, lds_tile_rows=0)
+        c = dict(rows_per_wave=rows, waves_m=0 if rows == 64 else 1, waves_k=wk, split_k=1, prefetch=pf, x_chunk=32 * wk * pf,
+                 token_tiles=1, xcd_swizzle=0, k_stagger=0, lds_tile_rows=0)
         try:
             make_configs.validate(m, n_key, k, c)
         except ValueError:
