@@ -222,9 +222,9 @@ typedef void (*NarrowKernelFn)(const uint8_t *, const void *, const float *, con
                                const void *);
 struct NarrowVariant {
     int rows, wk, u;
-    NarrowKernelFn fn;
+    NarrowKernelFn fn, fn_perm;  // B fragments loaded per lane (up to 4 tokens) / contiguously and permuted
 };
-#define N(LW, WK, U) {16 * LW, WK, U, gemm_narrow_kernel<LW, WK, U>}
+#define N(LW, WK, U) {16 * LW, WK, U, gemm_narrow_kernel<LW, WK, U, false>, gemm_narrow_kernel<LW, WK, U, true>}
 static const NarrowVariant kNarrow[] = {
     N(1, 4, 2),  N(1, 4, 4),  N(1, 4, 8),  N(1, 8, 2),  N(1, 8, 4),  N(1, 8, 8),  N(1, 16, 2), N(1, 16, 4), N(1, 16, 8),
     N(2, 4, 2),  N(2, 4, 4),  N(2, 4, 8),  N(2, 8, 2),  N(2, 8, 4),  N(2, 8, 8),  N(2, 16, 2), N(2, 16, 4), N(2, 16, 8),
@@ -233,7 +233,7 @@ static const NarrowVariant kNarrow[] = {
 };
 #undef N
 static constexpr int kNumNarrow = sizeof(kNarrow) / sizeof(kNarrow[0]);
-static unsigned char g_narrow_attr_done[16][kNumNarrow];
+static unsigned char g_narrow_attr_done[16][kNumNarrow][2];
 
 static const NarrowVariant *find_narrow(int rows, int wk, int u)
 {
@@ -253,18 +253,19 @@ hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
     const int vi = (int)(v - kNarrow);
+    const int perm = args.n > 4;
+    const NarrowKernelFn fn = perm ? v->fn_perm : v->fn;
     {
         std::lock_guard<std::mutex> lock(g_attr_mutex);
-        if (!g_narrow_attr_done[dev][vi]) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(v->fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    kLdsLimit);
+        if (!g_narrow_attr_done[dev][vi][perm]) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
             if (e != hipSuccess) return e;
-            g_narrow_attr_done[dev][vi] = 1;
+            g_narrow_attr_done[dev][vi][perm] = 1;
         }
     }
     const size_t lds = (size_t)kLutBytes + (size_t)waves_k * (rows / 16) * 1024;
     const dim3 grid((unsigned)(args.m / rows), (unsigned)((args.n + 15) / 16), 1);
-    hipLaunchKernelGGL(v->fn, grid, dim3(waves_k * 64), lds, stream, args.q, args.x, args.code, args.absmax, args.k, args.n,
+    hipLaunchKernelGGL(fn, grid, dim3(waves_k * 64), lds, stream, args.q, args.x, args.code, args.absmax, args.k, args.n,
                        args.n_it, args.m, args.out, args.epilogue, args.residual);
     return hipGetLastError();
 }

@@ -13,9 +13,9 @@
 //     covers 2*LW block rows x 128 contiguous bytes.
 //   * Every wave has its own k range, so nothing of x is shared inside the workgroup: B fragments
 //     come straight from global memory (L2 hits: x is 128 KB per 16 tokens and read by everyone),
-//     one 16-byte load per lane and k-step, no staging, no barrier before the main loop.  Token
-//     rows past n are clamped, not zeroed: a B column only feeds its own output column, which is
-//     never stored.
+//     one 16-byte load per lane and k-step, loaded contiguously and moved to the lane that needs
+//     them by cross-lane reads; no staging, no barrier before the main loop.  Token rows past n
+//     are clamped, not zeroed: a B column only feeds its own output column, which is never stored.
 //   * Weights and B fragments travel through one ring of U k-steps per wave.
 //   * Decode table and decode as in gemm_kernel.hpp (bit-identical weights).
 //   * Reduction: the WK waves put their LW accumulator planes in LDS; each thread sums two
@@ -36,7 +36,7 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 // dwords of a kernel's arguments can be preloaded into scalar registers with the wave (built
 // with -amdgpu-kernarg-preload-count=16), which takes the argument fetch - a round trip to
 // memory - off the start of every wave.  A struct passed by value is not preloaded.
-template <int LW, int WK, int U>
+template <int LW, int WK, int U, bool PERM>
 __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q, const void *a_x, const float *a_code,
                                                               const float *a_absmax, int a_k, int a_n, int a_n_it, int a_m,
                                                               void *a_out, int a_epilogue, const void *a_residual)
@@ -80,15 +80,22 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
         for (int j = 0; j < 4; ++j) sc32[j] = s4[j];
     }
     const uint32_t kb_total = (uint32_t)a.k >> 3;
-    // A wave walks k in double steps of 64 (two MFMAs): wave wk owns double steps wk, wk + WK, ...
-    // Within a double step the MFMA k slots are permuted so that lane group g holds the two
-    // adjacent 8-k blocks 2g and 2g + 1 (first and second MFMA): the four groups of a token row
-    // then read one whole 128-byte line of x between them instead of half of two lines.  The
-    // weights follow the same permutation (block column 8*dstep + 2g + half).
-    // per lane: block row and dwords of the block (weights); token row and 8-k block (x)
+    // A wave walks k in double steps of 64 (two MFMAs, one 128-byte line of x per token): wave wk
+    // owns double steps wk, wk + WK, ...
+    // Weights, per lane: block row and dwords of the block, block column 4*step + g.
     const uint32_t lb = ((uint32_t)(row0 >> 3) + (uint32_t)((LW * i16) >> 3)) * kb_total * 32u +
-                        (uint32_t)((LW * i16) & 7) * 4u + (uint32_t)g * 64u;
-    const uint32_t xoff = ((uint32_t)min(i16, a.n - 1 - tok0) * (uint32_t)a.k + (uint32_t)g * 16u) * 2u;
+                        (uint32_t)((LW * i16) & 7) * 4u + (uint32_t)g * 32u;
+    // B fragments: the MFMA wants lane (token i16, group g) to hold x[token][32*step + 8g ..], i.e.
+    // four consecutive lanes on four different token rows - a wave instruction loading it that
+    // way touches 16 rows with no two neighbouring lanes on one line and takes about three times
+    // as long in the address path as a contiguous one.  PERM: lane l LOADS token l / 4, 8-k group
+    // l % 4 (each quad of lanes reads 64 contiguous bytes) and the fragment goes to the lane that
+    // needs it by a cross-lane read (ds_bpermute: no LDS memory, no barrier) when it is consumed:
+    // lane (i16, g) takes the piece lane 4*i16 + g loaded.  Without PERM every lane loads its own
+    // fragment: cheaper for one to four tokens, where the clamped rows coincide anyway.
+    const uint32_t xoff = PERM ? ((uint32_t)min(lane >> 2, a.n - 1 - tok0) * (uint32_t)a.k + (uint32_t)(lane & 3) * 8u) * 2u
+                               : ((uint32_t)min(i16, a.n - 1 - tok0) * (uint32_t)a.k + (uint32_t)g * 8u) * 2u;
+    const int x_src = (i16 * 4 + g) << 2;  // byte address of the source lane for ds_bpermute
     // uniform: this wave's double step 0; one ring turn (U/2 double steps) further per group
     const unsigned char *qp = a.q + (size_t)wk * 256;
     const unsigned char *xp = reinterpret_cast<const unsigned char *>(a.x) + (size_t)tok0 * a.k * 2 + (size_t)wk * 128;
@@ -97,8 +104,8 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     static_assert(U % 2 == 0, "whole double steps");
 #define TUNA_NARROW_LOAD(u)                                                                     \
     {                                                                                          \
-        const size_t xo_ = (size_t)((u) >> 1) * (WK * 128) + ((u) & 1) * 16;               \
-        const size_t qo_ = (size_t)((u) >> 1) * (WK * 256) + ((u) & 1) * 32;               \
+        const size_t xo_ = (size_t)((u) >> 1) * (WK * 128) + ((u) & 1) * 64;               \
+        const size_t qo_ = (size_t)((u) >> 1) * (WK * 256) + ((u) & 1) * 128;              \
         xq[u] = *reinterpret_cast<const u32x4 *>(xp + xo_ + xoff);                             \
         if constexpr (LW == 1) {                                                               \
             wq[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(qp + qo_ + lb)); \
@@ -149,7 +156,11 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     for (int j = 0; j < LW; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #define TUNA_NARROW_CONSUME(u)                                                                  \
     {                                                                                          \
-        const f16x8 b_ = __builtin_bit_cast(f16x8, xq[u]);                                     \
+        u32x4 xb_ = xq[u];                                                                     \
+        if constexpr (PERM) {                                                                  \
+            _Pragma("unroll") for (int e = 0; e < 4; ++e) xb_[e] = (uint32_t)__builtin_amdgcn_ds_bpermute(x_src, (int)xq[u][e]); \
+        }                                                                                      \
+        const f16x8 b_ = __builtin_bit_cast(f16x8, xb_);                                       \
         _Pragma("unroll") for (int j = 0; j < LW; ++j)                                         \
         {                                                                                      \
             const f16x8 av_ = decode_dword<TUNA_DECODE_GEMM>(wq[u][j], lut, lane4, sc16[j], 0.f); \
