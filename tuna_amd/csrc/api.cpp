@@ -83,6 +83,7 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
         return fail(TUNA_ERR_UNSUPPORTED, "x_chunk=%d must be a power of two >= 32*waves_k*prefetch=%d", c.x_chunk,
                     kStepK * c.waves_k * c.prefetch);
     if (c.k_stagger < 0 || c.k_stagger > 4096) return fail(TUNA_ERR_UNSUPPORTED, "k_stagger=%d must be in 0..4096", c.k_stagger);
+    if (k >= (1 << 23)) return fail(TUNA_ERR_UNSUPPORTED, "k=%d exceeds the 24-bit row pitch of the x staging", k);
     const int rw = c.rows_per_wave / kRowsPerLoad;
     const int threads = c.waves_m * c.waves_k * 64;
     const int rows_wg = c.rows_per_wave * c.waves_m;
@@ -96,7 +97,7 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     // the epilogue, two alternating buffers of one accumulator plane (1 KB) of every wave.
     const int nacc = rw * 4 * c.token_tiles;
     const int lut = decode == TUNA_DECODE_GEMM ? kLutBytes : 64;
-    const size_t x_lds = (size_t)c.token_tiles * 16 * (size_t)c.x_chunk * 2;
+    const size_t x_lds = (size_t)(c.x_chunk / 8) * (256 * (size_t)c.token_tiles + 16);  // 8-k slots of 16*token_tiles pieces + 16 bytes of padding
     // Two buffers of four planes (one barrier per 64-row group instead of four) are used when
     // they cost no occupancy: the x chunk leaves that much room anyway, or the config cannot
     // put two workgroups on a CU in the first place.
