@@ -701,12 +701,17 @@ NARROW_CASES = [
     (256, 16, 2048, 64, 8, 4),      # 64 rows per workgroup (waves_m = 0 selects the kernel)
     (192, 19, 1024, 64, 4, 8),
     (128, 7, 4096, 64, 16, 2),
+    # two and four 16-token tiles per workgroup (7th entry: token_tiles)
+    (256, 32, 1024, 32, 8, 2, 2),
+    (128, 50, 2048, 16, 4, 4, 4),   # 64 tokens per chunk, 50 present
+    (256, 100, 512, 64, 4, 2, 2),   # four chunks of 32, the last one ragged
+    (96, 64, 4096, 32, 8, 4, 4),
 ]
 
 
-def narrow_cfg(rows, wk, pf):
+def narrow_cfg(rows, wk, pf, tt=1):
     return cfg(rows_per_wave=rows, waves_m=0 if rows == 64 else 1, waves_k=wk, split_k=1, prefetch=pf, x_chunk=32 * wk * pf,
-               token_tiles=1)
+               token_tiles=tt)
 
 
 @pytest.mark.parametrize("ci", range(len(NARROW_CASES)))
@@ -718,8 +723,8 @@ def test_narrow_row_kernel_matches_oracle(ci):
 
     from tuna_amd import _lib, ops
 
-    m, n, k, rows, wk, pf = NARROW_CASES[ci]
-    c = narrow_cfg(rows, wk, pf)
+    m, n, k, rows, wk, pf = NARROW_CASES[ci][:6]
+    c = narrow_cfg(rows, wk, pf, *NARROW_CASES[ci][6:])
     print(f"narrow case#{ci} {m}x{n}x{k} {c.to_dict()}", flush=True)
     q, x, code, absmax = make_inputs_np(m, n, k, seed=90 + ci)
     res = (np.random.default_rng(ci).standard_normal((n, m)) * 0.05).astype(np.float16)
@@ -764,7 +769,7 @@ def test_narrow_row_configs_that_do_not_fit_are_rejected():
     q, x, code, absmax = make_inputs_np(256, 16, 1024, seed=1)
     for m, k, kw in [(264, 1024, dict()),                       # m not a multiple of the rows
                      (256, 1000, dict()),                       # k not a multiple of 32 * waves_k * prefetch
-                     (256, 1024, dict(split_k=2)), (256, 1024, dict(waves_m=2)), (256, 1024, dict(token_tiles=2))]:
+                     (256, 1024, dict(split_k=2)), (256, 1024, dict(waves_m=2)), (256, 1024, dict(token_tiles=3))]:
         c = cfg(**{**dict(rows_per_wave=16, waves_m=1, waves_k=4, split_k=1, prefetch=2, x_chunk=256, token_tiles=1), **kw})
         with pytest.raises(ops.TunaError):
             ops.validate_config(m, 16, k, c)

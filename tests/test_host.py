@@ -326,8 +326,9 @@ def test_gpu_parity_config_families_are_valid_configs():
     for rows, tt in mod.TILED:
         for (m, n, k, split) in ((512, 256, 512, 1), (520, 300, 1096, 1), (256, 70, 2048, 4), (1024, 129, 200, 3)):
             ops.validate_config(m, n, k, mod.cfg(lds_tile_rows=rows, token_tiles=tt, split_k=split))
-    for (m, n, k, rows, wk, pf) in mod.NARROW_CASES:
-        c = mod.narrow_cfg(rows, wk, pf)
+    for case in mod.NARROW_CASES:
+        m, n, k, rows, wk, pf = case[:6]
+        c = mod.narrow_cfg(rows, wk, pf, *case[6:])
         ops.validate_config(m, n, k, c)
         lds, ws = ops.config_footprint(m, n, k, c)
         assert (lds, ws) == (make_configs.lds_bytes(c.to_dict()), 0)

@@ -230,7 +230,7 @@ static int plan_tiled(int m, int n, int k, const tuna_gemm_config &c, int decode
 // Narrow-row kernel: checks and launch arguments for a config with rows_per_wave 16 or 32.
 struct NarrowPlan {
     NarrowArgs args;
-    int rows, waves_k, prefetch;
+    int rows, waves_k, prefetch, token_tiles;
     size_t lds_bytes;
 };
 
@@ -248,25 +248,25 @@ static int plan_narrow(int m, int n, int k, const tuna_gemm_config &c, int decod
         return fail(TUNA_ERR_UNSUPPORTED, "the narrow-row kernel (rows_per_wave 16, 32) implements TUNA_DECODE_GEMM only");
     if ((unsigned long long)m * (unsigned long long)k / 2 >= (1ull << 32) || (unsigned long long)k * 32 >= (1ull << 32))
         return fail(TUNA_ERR_UNSUPPORTED, "operands exceed the kernel's 32-bit offsets");
-    if (c.waves_m != (c.rows_per_wave == 64 ? 0 : 1) || c.split_k != 1 || c.token_tiles != 1 || c.k_stagger != 0)
+    if (c.waves_m != (c.rows_per_wave == 64 ? 0 : 1) || c.split_k != 1 || c.k_stagger != 0)
         return fail(TUNA_ERR_UNSUPPORTED,
-                    "the narrow-row kernel needs waves_m=1 (0 with rows_per_wave=64), split_k=1, token_tiles=1, k_stagger=0 "
-                    "(got %d, %d, %d, %d)",
-                    c.waves_m, c.split_k, c.token_tiles, c.k_stagger);
-    if (!is_pow2(c.waves_k) || c.waves_k > 16 || !narrow_variant_exists(c.rows_per_wave, c.waves_k, c.prefetch))
-        return fail(TUNA_ERR_UNSUPPORTED, "no narrow-row kernel for rows_per_wave=%d waves_k=%d prefetch=%d", c.rows_per_wave,
-                    c.waves_k, c.prefetch);
+                    "the narrow-row kernel needs waves_m=1 (0 with rows_per_wave=64), split_k=1, k_stagger=0 (got %d, %d, %d)",
+                    c.waves_m, c.split_k, c.k_stagger);
+    if (!is_pow2(c.waves_k) || c.waves_k > 16 || !narrow_variant_exists(c.rows_per_wave, c.waves_k, c.prefetch, c.token_tiles))
+        return fail(TUNA_ERR_UNSUPPORTED, "no narrow-row kernel for rows_per_wave=%d waves_k=%d prefetch=%d token_tiles=%d",
+                    c.rows_per_wave, c.waves_k, c.prefetch, c.token_tiles);
     if (m % c.rows_per_wave)
         return fail(TUNA_ERR_UNSUPPORTED, "rows_per_wave=%d needs m=%d to be a multiple of it", c.rows_per_wave, m);
     if (k % (kStepK * c.waves_k * c.prefetch))
         return fail(TUNA_ERR_UNSUPPORTED, "rows_per_wave=%d needs k=%d to be a multiple of 32*waves_k*prefetch=%d",
                     c.rows_per_wave, k, kStepK * c.waves_k * c.prefetch);
-    if (ceil_div(n, 16) > 65535) return fail(TUNA_ERR_UNSUPPORTED, "n=%d needs more than 65535 token chunks", n);
+    if (ceil_div(n, 16 * c.token_tiles) > 65535) return fail(TUNA_ERR_UNSUPPORTED, "n=%d needs more than 65535 token chunks", n);
     memset(plan, 0, sizeof(*plan));
+    plan->token_tiles = c.token_tiles;
     plan->rows = c.rows_per_wave;
     plan->waves_k = c.waves_k;
     plan->prefetch = c.prefetch;
-    plan->lds_bytes = (size_t)kLutBytes + (size_t)c.waves_k * (c.rows_per_wave / 16) * 1024;
+    plan->lds_bytes = (size_t)kLutBytes + (size_t)c.waves_k * (c.rows_per_wave / 16) * c.token_tiles * 1024;
     plan->args.m = m;
     plan->args.n = n;
     plan->args.k = k;
@@ -496,7 +496,7 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
         np.args.out = out;
         np.args.epilogue = epilogue;
         np.args.residual = residual;
-        hipError_t e = launch_gemm_narrow(np.args, np.rows, np.waves_k, np.prefetch, stream);
+        hipError_t e = launch_gemm_narrow(np.args, np.rows, np.waves_k, np.prefetch, np.token_tiles, stream);
         if (e != hipSuccess) return hip_fail(e, "narrow-row gemm launch");
         return TUNA_OK;
     }

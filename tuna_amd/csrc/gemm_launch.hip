@@ -221,32 +221,44 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
 typedef void (*NarrowKernelFn)(const uint8_t *, const void *, const float *, const float *, int, int, int, int, void *, int,
                                const void *);
 struct NarrowVariant {
-    int rows, wk, u;
+    int rows, wk, u, tt;
     NarrowKernelFn fn, fn_perm;  // B fragments loaded per lane (up to 4 tokens) / contiguously and permuted
 };
-#define N(LW, WK, U) {16 * LW, WK, U, gemm_narrow_kernel<LW, WK, U, false>, gemm_narrow_kernel<LW, WK, U, true>}
+#define N(LW, WK, U) {16 * LW, WK, U, 1, gemm_narrow_kernel<LW, WK, U, false, 1>, gemm_narrow_kernel<LW, WK, U, true, 1>}
+#define NT(LW, WK, U, TT) {16 * LW, WK, U, TT, gemm_narrow_kernel<LW, WK, U, true, TT>, gemm_narrow_kernel<LW, WK, U, true, TT>}
 static const NarrowVariant kNarrow[] = {
     N(1, 4, 2),  N(1, 4, 4),  N(1, 4, 8),  N(1, 8, 2),  N(1, 8, 4),  N(1, 8, 8),  N(1, 16, 2), N(1, 16, 4), N(1, 16, 8),
     N(2, 4, 2),  N(2, 4, 4),  N(2, 4, 8),  N(2, 8, 2),  N(2, 8, 4),  N(2, 8, 8),  N(2, 16, 2), N(2, 16, 4), N(2, 16, 8),
     N(1, 1, 2),  N(1, 2, 2),  N(2, 1, 2),  N(2, 2, 2),
     N(4, 4, 2),  N(4, 4, 4),  N(4, 4, 8),  N(4, 8, 2),  N(4, 8, 4),  N(4, 8, 8),  N(4, 16, 2), N(4, 16, 4), N(4, 16, 8),
+    // two and four token tiles per workgroup (17..64 tokens per pass over the weights)
+    NT(1, 4, 2, 2), NT(1, 4, 4, 2), NT(1, 8, 2, 2), NT(1, 8, 4, 2), NT(1, 16, 2, 2), NT(1, 16, 4, 2),
+    NT(2, 4, 2, 2), NT(2, 4, 4, 2), NT(2, 8, 2, 2), NT(2, 8, 4, 2), NT(2, 16, 2, 2), NT(2, 16, 4, 2),
+    NT(4, 4, 2, 2), NT(4, 4, 4, 2), NT(4, 8, 2, 2), NT(4, 8, 4, 2), NT(4, 16, 2, 2), NT(4, 16, 4, 2),
+    NT(1, 4, 2, 4), NT(1, 4, 4, 4), NT(1, 8, 2, 4), NT(1, 8, 4, 4),
+    NT(2, 4, 2, 4), NT(2, 4, 4, 4), NT(2, 8, 2, 4), NT(2, 8, 4, 4),
+    NT(4, 4, 2, 4), NT(4, 8, 2, 4),
 };
 #undef N
+#undef NT
 static constexpr int kNumNarrow = sizeof(kNarrow) / sizeof(kNarrow[0]);
 static unsigned char g_narrow_attr_done[16][kNumNarrow][2];
 
-static const NarrowVariant *find_narrow(int rows, int wk, int u)
+static const NarrowVariant *find_narrow(int rows, int wk, int u, int tt)
 {
     for (int i = 0; i < kNumNarrow; ++i)
-        if (kNarrow[i].rows == rows && kNarrow[i].wk == wk && kNarrow[i].u == u) return &kNarrow[i];
+        if (kNarrow[i].rows == rows && kNarrow[i].wk == wk && kNarrow[i].u == u && kNarrow[i].tt == tt) return &kNarrow[i];
     return nullptr;
 }
 
-bool narrow_variant_exists(int rows, int waves_k, int prefetch) { return find_narrow(rows, waves_k, prefetch) != nullptr; }
-
-hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int prefetch, hipStream_t stream)
+bool narrow_variant_exists(int rows, int waves_k, int prefetch, int token_tiles)
 {
-    const NarrowVariant *v = find_narrow(rows, waves_k, prefetch);
+    return find_narrow(rows, waves_k, prefetch, token_tiles) != nullptr;
+}
+
+hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int prefetch, int token_tiles, hipStream_t stream)
+{
+    const NarrowVariant *v = find_narrow(rows, waves_k, prefetch, token_tiles);
     if (!v) return hipErrorInvalidConfiguration;
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
@@ -263,8 +275,8 @@ hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int
             g_narrow_attr_done[dev][vi][perm] = 1;
         }
     }
-    const size_t lds = (size_t)kLutBytes + (size_t)waves_k * (rows / 16) * 1024;
-    const dim3 grid((unsigned)(args.m / rows), (unsigned)((args.n + 15) / 16), 1);
+    const size_t lds = (size_t)kLutBytes + (size_t)waves_k * (rows / 16) * token_tiles * 1024;
+    const dim3 grid((unsigned)(args.m / rows), (unsigned)((args.n + 16 * token_tiles - 1) / (16 * token_tiles)), 1);
     hipLaunchKernelGGL(fn, grid, dim3(waves_k * 64), lds, stream, args.q, args.x, args.code, args.absmax, args.k, args.n,
                        args.n_it, args.m, args.out, args.epilogue, args.residual);
     return hipGetLastError();

@@ -21,8 +21,9 @@
 //   * Reduction: the WK waves put their LW accumulator planes in LDS; each thread sums two
 //     adjacent output features of one token in wave order and stores them (fused epilogues of
 //     epilogue.hpp).  Deterministic; no workspace, no counters.
-// Requires k % (32*WK*U) == 0, m % (16*LW) == 0, dense launches, at most 16 tokens per
-// workgroup (more tokens: gridDim.y chunks).  Selected by rows_per_wave = 16 or 32 in the config,
+// Requires k % (32*WK*U) == 0, m % (16*LW) == 0, dense launches; a workgroup takes 16*TT tokens
+// (TT = token_tiles = 1, 2, 4: every decoded weight fragment feeds TT MFMAs), more tokens are
+// gridDim.y chunks.  Selected by rows_per_wave = 16 or 32 in the config,
 // or by rows_per_wave = 64 with waves_m = 0.
 #pragma once
 #include "gemm_kernel.hpp"
@@ -36,7 +37,7 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 // dwords of a kernel's arguments can be preloaded into scalar registers with the wave (built
 // with -amdgpu-kernarg-preload-count=16), which takes the argument fetch - a round trip to
 // memory - off the start of every wave.  A struct passed by value is not preloaded.
-template <int LW, int WK, int U, bool PERM>
+template <int LW, int WK, int U, bool PERM, int TT>
 __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q, const void *a_x, const float *a_code,
                                                               const float *a_absmax, int a_k, int a_n, int a_n_it, int a_m,
                                                               void *a_out, int a_epilogue, const void *a_residual)
@@ -53,7 +54,7 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     extern __shared__ __align__(16) unsigned char smem[];
     static_assert(LW == 1 || LW == 2 || LW == 4, "16, 32 or 64 rows per workgroup");
     unsigned char *lut = smem;
-    float *red = reinterpret_cast<float *>(smem + kLutBytes);  // [wave][plane][lane][4]
+    float *red = reinterpret_cast<float *>(smem + kLutBytes);  // [wave][row plane][token tile][lane][4]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -63,7 +64,7 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     constexpr int nthreads = WK * 64;
     const uint32_t lane4 = (uint32_t)lane << 2;
     const int row0 = blockIdx.x * (16 * LW);
-    const int tok0 = blockIdx.y * 16;
+    const int tok0 = blockIdx.y * (16 * TT);  // TT tiles of 16 tokens share every decoded weight fragment
 
     // ---- requests: codebook and scales, then the first ring turn (x fragment, weights) --------
     const float code_lane = a.code[i16];
@@ -93,20 +94,23 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     // needs it by a cross-lane read (ds_bpermute: no LDS memory, no barrier) when it is consumed:
     // lane (i16, g) takes the piece lane 4*i16 + g loaded.  Without PERM every lane loads its own
     // fragment: cheaper for one to four tokens, where the clamped rows coincide anyway.
-    const uint32_t xoff = PERM ? ((uint32_t)min(lane >> 2, a.n - 1 - tok0) * (uint32_t)a.k + (uint32_t)(lane & 3) * 8u) * 2u
-                               : ((uint32_t)min(i16, a.n - 1 - tok0) * (uint32_t)a.k + (uint32_t)g * 8u) * 2u;
+    uint32_t xoff[TT];
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt)
+        xoff[tt] = PERM ? ((uint32_t)min(tt * 16 + (lane >> 2), a.n - 1 - tok0) * (uint32_t)a.k + (uint32_t)(lane & 3) * 8u) * 2u
+                        : ((uint32_t)min(tt * 16 + i16, a.n - 1 - tok0) * (uint32_t)a.k + (uint32_t)g * 8u) * 2u;
     const int x_src = (i16 * 4 + g) << 2;  // byte address of the source lane for ds_bpermute
     // uniform: this wave's double step 0; one ring turn (U/2 double steps) further per group
     const unsigned char *qp = a.q + (size_t)wk * 256;
     const unsigned char *xp = reinterpret_cast<const unsigned char *>(a.x) + (size_t)tok0 * a.k * 2 + (size_t)wk * 128;
     uint32_t wq[U][LW];
-    u32x4 xq[U];
+    u32x4 xq[U][TT];
     static_assert(U % 2 == 0, "whole double steps");
 #define TUNA_NARROW_LOAD(u)                                                                     \
     {                                                                                          \
         const size_t xo_ = (size_t)((u) >> 1) * (WK * 128) + ((u) & 1) * 64;               \
         const size_t qo_ = (size_t)((u) >> 1) * (WK * 256) + ((u) & 1) * 128;              \
-        xq[u] = *reinterpret_cast<const u32x4 *>(xp + xo_ + xoff);                             \
+        _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) xq[u][tt] = *reinterpret_cast<const u32x4 *>(xp + xo_ + xoff[tt]); \
         if constexpr (LW == 1) {                                                               \
             wq[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(qp + qo_ + lb)); \
         } else if constexpr (LW == 2) {                                                        \
@@ -151,20 +155,27 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     __syncthreads();  // the table is complete
 
     // ---- main loop: n_it / U ring turns, the last one without refills ------------------------
-    f32x4 acc[LW];
+    f32x4 acc[LW][TT];
 #pragma unroll
-    for (int j = 0; j < LW; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < LW; ++j)
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) acc[j][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #define TUNA_NARROW_CONSUME(u)                                                                  \
     {                                                                                          \
-        u32x4 xb_ = xq[u];                                                                     \
-        if constexpr (PERM) {                                                                  \
-            _Pragma("unroll") for (int e = 0; e < 4; ++e) xb_[e] = (uint32_t)__builtin_amdgcn_ds_bpermute(x_src, (int)xq[u][e]); \
+        f16x8 b_[TT];                                                                          \
+        _Pragma("unroll") for (int tt = 0; tt < TT; ++tt)                                      \
+        {                                                                                      \
+            u32x4 xb_ = xq[u][tt];                                                             \
+            if constexpr (PERM) {                                                              \
+                _Pragma("unroll") for (int e = 0; e < 4; ++e) xb_[e] = (uint32_t)__builtin_amdgcn_ds_bpermute(x_src, (int)xq[u][tt][e]); \
+            }                                                                                  \
+            b_[tt] = __builtin_bit_cast(f16x8, xb_);                                           \
         }                                                                                      \
-        const f16x8 b_ = __builtin_bit_cast(f16x8, xb_);                                       \
         _Pragma("unroll") for (int j = 0; j < LW; ++j)                                         \
         {                                                                                      \
             const f16x8 av_ = decode_dword<TUNA_DECODE_GEMM>(wq[u][j], lut, lane4, sc16[j], 0.f); \
-            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av_, b_, acc[j], 0, 0, 0);         \
+            _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) acc[j][tt] =                     \
+                __builtin_amdgcn_mfma_f32_16x16x32_f16(av_, b_[tt], acc[j][tt], 0, 0, 0);      \
         }                                                                                      \
     }
     for (int it = U; it < a.n_it; it += U) {
@@ -183,29 +194,33 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
 #undef TUNA_NARROW_LOAD
 
     // ---- reduction over the waves and store -----------------------------------------------------
-    // Plane j of a wave: lane l, element v is token l % 16, MFMA row 4*(l/16) + v, weight row
-    // LW*(MFMA row) + j of the workgroup's 16*LW.
+    // Plane (j, tt) of a wave: lane l, element v is token 16*tt + l % 16, MFMA row 4*(l/16) + v,
+    // weight row LW*(MFMA row) + j of the workgroup's 16*LW.
 #pragma unroll
-    for (int j = 0; j < LW; ++j) reinterpret_cast<f32x4 *>(red)[(size_t)(wk * LW + j) * 64 + lane] = acc[j];
+    for (int j = 0; j < LW; ++j)
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt)
+            reinterpret_cast<f32x4 *>(red)[(size_t)((wk * LW + j) * TT + tt) * 64 + lane] = acc[j][tt];
     __syncthreads();
     f16 *outp = reinterpret_cast<f16 *>(a.out);
     const f16 *resp = reinterpret_cast<const f16 *>(a.residual);
-    constexpr int PAIRS = 128 * LW;  // pairs of adjacent rows x 16 tokens
+    constexpr int PAIRS = 128 * LW * TT;  // pairs of adjacent rows x 16*TT tokens
 #pragma unroll
     for (int p0 = 0; p0 < PAIRS; p0 += nthreads) {
         const int pi = p0 + tid;
         if (PAIRS % nthreads != 0 && pi >= PAIRS) break;
-        const int tk = pi / (8 * LW), rp = pi % (8 * LW);  // token, row pair: rows 2*rp and 2*rp + 1
+        const int tt = pi / (128 * LW);                                // token tile
+        const int tk = (pi / (8 * LW)) % 16, rp = pi % (8 * LW);       // token of the tile, row pair: rows 2*rp and 2*rp + 1
         // float index of row 2*rp in wave 0's planes; row 2*rp + 1 is the next element (LW 1) or
-        // the same element of the next plane (LW 2, 4)
+        // the same element of the next row plane (LW 2, 4)
         const int mr = (2 * rp) / LW, j0 = (2 * rp) % LW;  // MFMA row and plane of row 2*rp
-        const int f0 = j0 * 256 + (((mr >> 2) * 16 + tk) << 2) + (mr & 3);
-        constexpr int f1_off = LW == 1 ? 1 : 256;
+        const int f0 = (j0 * TT + tt) * 256 + (((mr >> 2) * 16 + tk) << 2) + (mr & 3);
+        constexpr int f1_off = LW == 1 ? 1 : TT * 256;
         float v0[WK], v1[WK];
 #pragma unroll
         for (int w = 0; w < WK; ++w) {
-            v0[w] = red[(size_t)w * (LW * 256) + f0];
-            v1[w] = red[(size_t)w * (LW * 256) + f0 + f1_off];
+            v0[w] = red[(size_t)w * (LW * TT * 256) + f0];
+            v1[w] = red[(size_t)w * (LW * TT * 256) + f0 + f1_off];
         }
         float s0 = 0.f, s1 = 0.f;
 #pragma unroll
@@ -213,7 +228,7 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
             s0 += v0[w];
             s1 += v1[w];
         }
-        const int tok = tok0 + tk;
+        const int tok = tok0 + tt * 16 + tk;
         if (tok >= a.n) continue;
         const int col = row0 + 2 * rp;
         if (a.epilogue == TUNA_EPILOGUE_SILU_MUL) {

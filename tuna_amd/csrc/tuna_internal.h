@@ -161,8 +161,8 @@ struct NarrowArgs {
     int m, n, k;
     int n_it;  // k-steps per wave: k / 32 / waves
 };
-bool narrow_variant_exists(int rows, int waves_k, int prefetch);
-hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int prefetch, hipStream_t stream);
+bool narrow_variant_exists(int rows, int waves_k, int prefetch, int token_tiles);
+hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int prefetch, int token_tiles, hipStream_t stream);
 int set_lean_kernels(int enabled);  // returns the previous setting
 unsigned long long lean_launches();
 bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves, int grouped);

@@ -50,9 +50,12 @@ VARIANTS_512_2WG = {(1, 2, 1), (1, 4, 1)}
 VARIANTS_1024 = {(1, 2, 1), (1, 4, 1)}
 
 
-# (rows, waves_k, prefetch) of the narrow-row kernel; must match kNarrow in csrc/gemm_launch.hip
-NARROW_VARIANTS = {(r, wk, pf) for r in (16, 32, 64) for wk in (4, 8, 16) for pf in (2, 4, 8)} | {
-    (16, 1, 2), (16, 2, 2), (32, 1, 2), (32, 2, 2)}
+# (rows, waves_k, prefetch, token_tiles) of the narrow-row kernel; must match kNarrow in csrc/gemm_launch.hip
+NARROW_VARIANTS = (
+    {(r, wk, pf, 1) for r in (16, 32, 64) for wk in (4, 8, 16) for pf in (2, 4, 8)}
+    | {(16, 1, 2, 1), (16, 2, 2, 1), (32, 1, 2, 1), (32, 2, 2, 1)}
+    | {(r, wk, pf, 2) for r in (16, 32, 64) for wk in (4, 8, 16) for pf in (2, 4)}
+    | {(r, wk, pf, 4) for r in (16, 32) for wk in (4, 8) for pf in (2, 4)} | {(64, 4, 2, 4), (64, 8, 2, 4)})
 
 # (rows, tokens) tiles of the many-token kernel; must match kTiled in csrc/gemm_tiled.hip
 TILED_VARIANTS = {(256, 128), (256, 64), (128, 256), (128, 128), (64, 256), (64, 128)}
@@ -94,11 +97,10 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
         return
     if is_narrow(c):
         # narrow-row kernel: one workgroup per 16, 32 or 64 rows, all waves along k, no split
-        if (c["waves_m"], c["split_k"], c["token_tiles"], c["k_stagger"]) != (0 if c["rows_per_wave"] == 64 else 1, 1, 1, 0):
-            raise ValueError("the narrow-row kernel needs waves_m=1 (0 with rows_per_wave 64), split_k=1, token_tiles=1, "
-                             "k_stagger=0")
-        if (c["rows_per_wave"], c["waves_k"], c["prefetch"]) not in NARROW_VARIANTS:
-            raise ValueError("no narrow-row kernel for this rows_per_wave / waves_k / prefetch")
+        if (c["waves_m"], c["split_k"], c["k_stagger"]) != (0 if c["rows_per_wave"] == 64 else 1, 1, 0):
+            raise ValueError("the narrow-row kernel needs waves_m=1 (0 with rows_per_wave 64), split_k=1, k_stagger=0")
+        if (c["rows_per_wave"], c["waves_k"], c["prefetch"], c["token_tiles"]) not in NARROW_VARIANTS:
+            raise ValueError("no narrow-row kernel for this rows_per_wave / waves_k / prefetch / token_tiles")
         if m % c["rows_per_wave"] or k % (STEP_K * c["waves_k"] * c["prefetch"]):
             raise ValueError("rows_per_wave 16 or 32 needs m a multiple of it and k a multiple of 32*waves_k*prefetch")
         if m * k // 2 >= 1 << 32 or k * 32 >= 1 << 32:
@@ -144,7 +146,7 @@ def lds_bytes(c: dict) -> int:
         return LUT_BYTES + 2 * (c["lds_tile_rows"] + 16 * c["token_tiles"]) * 128
     if is_narrow(c):
         # narrow-row kernel: decode table + one accumulator plane (1 KB) per wave and 16 rows
-        return LUT_BYTES + c["waves_k"] * (c["rows_per_wave"] // 16) * 1024
+        return LUT_BYTES + c["waves_k"] * (c["rows_per_wave"] // 16) * c["token_tiles"] * 1024
     threads = 64 * c["waves_k"] * c["waves_m"]
     x = (c["x_chunk"] // 8) * (256 * c["token_tiles"] + 16)   # 8-k slots of 16*token_tiles pieces + 16 bytes of padding
     plane = c["waves_k"] * c["waves_m"] * 1024

@@ -168,13 +168,15 @@ def lean_space(m: int, n_key: int, k: int):
 def narrow_space(m: int, n_key: int, k: int):
     """Every config of the narrow-row kernel (gemm_narrow.hpp: 16 or 32 rows per workgroup, all
     waves along k, no split) the shape admits.  Small enough to time exhaustively."""
-    lo, _ = make_configs.N_BUCKETS[n_key]
-    if lo > 32:
+    lo, hi = make_configs.N_BUCKETS[n_key]
+    if lo > 64:
         return []
     out = []
-    for rows, wk, pf in sorted(make_configs.NARROW_VARIANTS):
+    for rows, wk, pf, tt in sorted(make_configs.NARROW_VARIANTS):
+        if 16 * tt > max(16, hi) or (tt > 1 and 16 * (tt // 2) >= hi):   # no more token tiles than the bucket can fill
+            continue
         c = dict(rows_per_wave=rows, waves_m=0 if rows == 64 else 1, waves_k=wk, split_k=1, prefetch=pf, x_chunk=32 * wk * pf,
-                 token_tiles=1, xcd_swizzle=0, k_stagger=0, lds_tile_rows=0)
+                 token_tiles=tt, xcd_swizzle=0, k_stagger=0, lds_tile_rows=0)
         try:
             make_configs.validate(m, n_key, k, c)
         except ValueError:
