@@ -154,6 +154,34 @@ def test_tuner_repair_seeds_and_mutation_stay_valid():
                              token_tiles=1, xcd_swizzle=0), 4096, 16, 4096) is None
 
 
+def test_tuner_small_launch_config_spaces_are_valid_for_both_validators():
+    """The exhaustively timed config spaces of the lean and the narrow-row kernel: every member
+    passes the Python validator and the library's, narrow-row members report the footprint the
+    twin computes, and the spaces have the members the tuned table relies on."""
+    from tuna_amd import make_configs as mc
+    from tuna_amd import ops, tuner
+
+    for (m, n, k) in [(4096, 16, 4096), (6144, 1, 4096), (6144, 32, 4096), (8192, 64, 8192), (28672, 16, 4096)]:
+        nk = mc.bucket_of(n)
+        lean = tuner.lean_space(m, nk, k)
+        narrow = tuner.narrow_space(m, nk, k)
+        assert narrow and (lean or n >= 64)    # the lean kernel takes 16 tokens per pass: not offered from 64 tokens up
+        for c in lean + narrow:
+            mc.validate(m, nk, k, c)
+            ops.validate_config(m, n, k, ops.GemmConfig.from_dict(c))
+        for c in lean:
+            assert c["rows_per_wave"] == 64 and c["token_tiles"] == 1 and c["k_stagger"] == 0
+            assert c["split_k"] & (c["split_k"] - 1) == 0 and (k // 32) % (c["split_k"] * c["waves_k"] * c["prefetch"]) == 0
+        for c in narrow:
+            assert mc.is_narrow(c)
+            lds, ws = ops.config_footprint(m, n, k, ops.GemmConfig.from_dict(c))
+            assert (lds, ws) == (mc.lds_bytes(c), 0)
+        tiles = {c["token_tiles"] for c in narrow}
+        assert tiles == ({1} if n <= 16 else {1, 2} if n <= 32 else {1, 2, 4})
+    assert tuner.narrow_space(4096, 128, 4096) == [] and tuner.lean_space(4096, 128, 4096) == []
+    assert tuner.lean_space(4096, 16, 4104) == []       # k not a multiple of 32: no lean launch
+
+
 def test_quantizer_matches_nearest_code_and_layout():
     import torch
 
