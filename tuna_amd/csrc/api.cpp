@@ -97,7 +97,7 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     // the epilogue, two alternating buffers of one accumulator plane (1 KB) of every wave.
     const int nacc = rw * 4 * c.token_tiles;
     const int lut = decode == TUNA_DECODE_GEMM ? kLutBytes : 64;
-    const size_t x_lds = (size_t)(c.x_chunk / 8) * (256 * (size_t)c.token_tiles + 16);  // 8-k slots of 16*token_tiles pieces + 16 bytes of padding
+    const size_t x_lds = (size_t)c.token_tiles * 16 * (size_t)c.x_chunk * 2;
     // Two buffers of four planes (one barrier per 64-row group instead of four) are used when
     // they cost no occupancy: the x chunk leaves that much room anyway, or the config cannot
     // put two workgroups on a CU in the first place.
@@ -173,7 +173,6 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     a.split_log2 = (c.split_k > 0 && (c.split_k & (c.split_k - 1)) == 0) ? log2i(c.split_k) : -1;
     a.steps_total = steps_total;
     a.steps_per_split = balanced ? steps_total : ceil_div(steps_total, c.split_k);
-    a.x_slots_magic = (unsigned)((1ull << 32) / (4ull * (unsigned)a.steps_per_split)) + 1u;
     a.balanced = balanced ? 1 : 0;
     a.unit_log2 = unit_log2;
     a.units_per_tile = units_per_tile;

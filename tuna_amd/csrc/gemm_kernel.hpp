@@ -19,10 +19,11 @@
 //   * Packed weights are used exactly once, so they go global -> registers through a
 //     ring of `U` k-steps per wave (nontemporal loads); there is nothing to share in LDS.
 //   * Activations are re-used by every wave: the workgroup stages its k-slice of x in
-//     LDS in chunks, as 16-byte pieces ordered [8-k slot][token] with 16 bytes of padding per
-//     slot: the ds_read_b128 of a B fragment (16 lanes = 16 tokens of one slot = 256 contiguous
-//     bytes) is bank-conflict free, and so are the staging writes, whose lanes run along k
-//     (consecutive slots of one token row - the order in which global memory is read fastest).
+//     LDS in chunks, as 16-byte pieces ordered [8-k slot][token], so that the ds_read_b128 of
+//     a B fragment (16 lanes = 16 tokens of one slot = 256 contiguous bytes) is bank-conflict
+//     free without padding; the staging reads global memory with every quad of lanes on 64
+//     contiguous bytes of one token row and writes one k-step (4 slots x 16 tokens = 1 KB
+//     contiguous) per wave instruction.
 //   * Decode: the codebook is a run-time input, so it is a table.  LDS holds, for every
 //     byte value, the half2 {code[hi nibble], code[lo nibble]} replicated once per lane
 //     (row stride 256 B).  A lane's address is (byte << 8) | (lane << 2), built by one
@@ -211,53 +212,51 @@ __device__ __forceinline__ int k_physical(int k_logical, const KRot &kr)
     return kp >= kr.hi_k ? kp - kr.span_k : kp;
 }
 
-// Piece p = tid + b*nthreads of a chunk of 2^cs_log2 8-k slots is token row p >> cs_log2, slot
-// p & (2^cs_log2 - 1): consecutive lanes read consecutive 16 bytes of one token row.  (With
-// consecutive lanes on different token rows - the order the MFMA wants - a wave instruction
-// touches 16 rows with no two neighbouring lanes on one cache line and takes about three
-// times as long in the address path.)  In LDS slot s, token row r sits at byte
-// s*(256*TT + 16) + r*16: the rows of a slot are the contiguous B fragments of its TT token
-// tiles, and the 16-byte pad per slot spreads the staging writes (consecutive slots, same
-// row) over all banks.
-template <int TT>
-constexpr int kSlotBytes = 256 * TT + 16;
-
+// Piece p = tid + b*nthreads of a chunk: its lane (p % 64) picks token row lane / 4 of a 16-token
+// tile and 8-k group lane % 4 of a k-step, p / 64 picks the k-step and (TT > 1) the token tile.
+// Every quad of lanes reads 64 contiguous bytes of one token row - with neighbouring lanes on
+// different rows (the order the MFMA wants) a wave instruction takes about three times as long
+// in the address path - and a wave instruction writes the 16 rows x 4 slots of one k-step and
+// tile: with the layout byte = slot*(256*TT) + row*16 that is 4 runs of 256 contiguous bytes,
+// bank-conflict free without padding, and the 16 rows of a slot are a contiguous B fragment.
 template <int TT, int XB>
 __device__ __forceinline__ void x_stage_load(XStage<XB> &st, const f16 *xg, int nthreads, int tid, int tok0, int kbase, int n,
-                                             int k, const KRot &kr, int cs_log2)
+                                             int k, const KRot &kr)
 {
     // uniform 64-bit base (the tile's first token row) + a 32-bit per-lane offset: a tile spans
     // at most 16*TT rows of at most 2^23 k, so no 64-bit address lives in vector registers.
     // Rows past n and slots past the chunk or k are clamped here and zeroed by x_stage_store.
     const unsigned char *row0 = reinterpret_cast<const unsigned char *>(xg + (size_t)tok0 * k);
     const uint32_t row_bytes = (uint32_t)k * 2u;
-    const uint32_t r_max = (uint32_t)min(n - 1 - tok0, 16 * TT - 1);
-    const uint32_t s_mask = (1u << cs_log2) - 1u;
+    const int r_max = n - 1 - tok0;
     // (an opaque copy of the thread id: the per-piece offsets below do not depend on the chunk,
     // and hoisted out of the chunk loop they would sit in registers across the MFMA loop)
     asm volatile("" : "+v"(tid));
+    const int row_l = (tid & 63) >> 2, grp = tid & 3;
 #pragma unroll
     for (int b = 0; b < XB; ++b) {
-        const uint32_t p = (uint32_t)(tid + b * nthreads);
-        const int kk = min(k_physical(kbase + (int)(p & s_mask) * 8, kr), k - 8);
-        st.v[b] = *reinterpret_cast<const u32x4 *>(row0 + (__umul24(min(p >> cs_log2, r_max), row_bytes) + (uint32_t)kk * 2u));
+        const int wv = (tid + b * nthreads) >> 6;  // wave instruction of the chunk: k-step wv / TT, token tile wv % TT
+        const int row = (wv % TT) * 16 + row_l;
+        const int kk = min(k_physical(kbase + (wv / TT) * 32 + grp * 8, kr), k - 8);
+        st.v[b] = *reinterpret_cast<const u32x4 *>(row0 + (__umul24((uint32_t)min(row, r_max), row_bytes) + (uint32_t)kk * 2u));
     }
 }
 
 template <int TT, int XB>
 __device__ __forceinline__ void x_stage_store(const XStage<XB> &st, unsigned char *xs, int nthreads, int tid, int pieces,
-                                              int tok0, int kbase, int n, int k, const KRot &kr, int cs_log2)
+                                              int tok0, int kbase, int n, int k, const KRot &kr)
 {
-    const uint32_t s_mask = (1u << cs_log2) - 1u;
     asm volatile("" : "+v"(tid));  // (as in x_stage_load)
+    const int row_l = (tid & 63) >> 2, grp = tid & 3;
 #pragma unroll
     for (int b = 0; b < XB; ++b) {
-        const uint32_t p = (uint32_t)(b * nthreads + tid);
-        if (p < (uint32_t)pieces) {
-            const uint32_t s = p & s_mask, r = p >> cs_log2;
-            const int kl = kbase + (int)s * 8;
-            const bool ok = tok0 + (int)r < n && kl < kr.hi_k && k_physical(kl, kr) < k;
-            *reinterpret_cast<u32x4 *>(xs + s * (uint32_t)kSlotBytes<TT> + r * 16u) = ok ? st.v[b] : u32x4{0u, 0u, 0u, 0u};
+        const int p = b * nthreads + tid;
+        if (p < pieces) {
+            const int wv = p >> 6;
+            const int row = (wv % TT) * 16 + row_l, slot = (wv / TT) * 4 + grp;
+            const int kl = kbase + slot * 8;
+            const bool ok = tok0 + row < n && kl < kr.hi_k && k_physical(kl, kr) < k;
+            *reinterpret_cast<u32x4 *>(xs + slot * (256 * TT) + row * 16) = ok ? st.v[b] : u32x4{0u, 0u, 0u, 0u};
         }
     }
 }
@@ -446,7 +445,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
             sc32c[rw][j] = a.absmax[min(row_, a.m - 1)]; /* rows past m are never stored */    \
         }                                                                                      \
         krot = KRot{rot * kStepK, seg_hi * kStepK, nsteps * kStepK};                           \
-        x_stage_load<TT, XB>(xst, xg, nthreads, tid, tok0, sb * kStepK, n_tok, a.k, krot, a.chunk_log2 + 2); \
+        x_stage_load<TT, XB>(xst, xg, nthreads, tid, tok0, sb * kStepK, n_tok, a.k, krot); \
     }
 
     int t = t_begin;
@@ -539,7 +538,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     }
 
     const int ipc = a.chunk_steps >> a.wk_log2;  // iterations per chunk per wave (multiple of U)
-    const int wstep = a.waves_k * (4 * kSlotBytes<TT>);  // LDS bytes between this wave's consecutive steps (4 slots per step)
+    const int wstep = a.waves_k * (1024 * TT);   // LDS bytes between this wave's consecutive steps
 
     while (t < t_end) {
         // (grouped variants request them here for every tile: with a second place of request
@@ -570,15 +569,15 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 
         // the work area is free again once every wave has left the previous tile's epilogue
         __syncthreads();
-        if (n_chunks > 0) x_stage_store<TT, XB>(xst, work, nthreads, tid, x_pieces, cur_tok0, cur_sb * kStepK, cur_ntok, a.k, krot, a.chunk_log2 + 2);
+        if (n_chunks > 0) x_stage_store<TT, XB>(xst, work, nthreads, tid, x_pieces, cur_tok0, cur_sb * kStepK, cur_ntok, a.k, krot);
         __syncthreads();
         TUNA_MARK(3)
 
         for (int c = 0; c < n_chunks; ++c) {
             const int it_chunk0 = c * ipc;
             const bool has_next = c + 1 < n_chunks;
-            // B fragment of lane (token i16, k-group g), local step sl: slot sl*4+g, byte slot*kSlotBytes + i16*16
-            const unsigned char *xb = work + g * kSlotBytes<TT> + i16 * 16 + wk * (4 * kSlotBytes<TT>) - it_chunk0 * wstep;
+            // B fragment of lane (token i16, k-group g), local step sl: slot sl*4+g, piece slot*16*TT + i16
+            const unsigned char *xb = work + g * (256 * TT) + i16 * 16 + wk * (1024 * TT) - it_chunk0 * wstep;
             if (has_next) {
                 // A chunk with a successor is full: every wave owns all ipc iterations of it.
                 const int it_peel = it_chunk0 + ipc - U;
@@ -587,10 +586,10 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                 // that after the group exactly U*RW younger loads are in flight and the wait before
                 // the LDS write below is an exact vmcnt, not a drain of the weight ring.
                 const int kbase = (cur_sb + (c + 1) * a.chunk_steps) * kStepK;
-                x_stage_load<TT, XB>(xst, xg, nthreads, tid, cur_tok0, kbase, cur_ntok, a.k, krot, a.chunk_log2 + 2);
+                x_stage_load<TT, XB>(xst, xg, nthreads, tid, cur_tok0, kbase, cur_ntok, a.k, krot);
                 TUNA_GROUP()
                 __syncthreads();  // every wave is done reading chunk c
-                x_stage_store<TT, XB>(xst, work, nthreads, tid, x_pieces, cur_tok0, kbase, cur_ntok, a.k, krot, a.chunk_log2 + 2);
+                x_stage_store<TT, XB>(xst, work, nthreads, tid, x_pieces, cur_tok0, kbase, cur_ntok, a.k, krot);
                 __syncthreads();
             } else {
                 const int it_end = min(it_chunk0 + ipc, n_it);

@@ -72,7 +72,7 @@ bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int 
 }
 
 // ---- lean twins (gemm_lean.hpp) -------------------------------------------------------------
-typedef void (*LeanKernelFn)(const uint8_t *, const void *, const float *, const float *, int, int, int, unsigned, int, int,
+typedef void (*LeanKernelFn)(const uint8_t *, const void *, const float *, const float *, int, int, int, int, int,
                              void *, const void *, float *, unsigned *, int
 #ifdef TUNA_TRACE
                              ,
@@ -96,7 +96,7 @@ static constexpr int kNumLean = sizeof(kLean) / sizeof(kLean[0]);
 // The lean kernel's LDS: decode table + max(x slice of the split, reduction planes) + ticket.
 static size_t lean_lds_bytes(const GemmPlan &plan)
 {
-    const size_t x_bytes = (size_t)plan.args.steps_per_split * 1088;  // 4 slots of 16 tokens x 16 bytes + 16 bytes of padding per k-step
+    const size_t x_bytes = (size_t)plan.args.steps_per_split * 1024;  // 16 tokens x 32 k x 2 bytes per k-step
     const size_t red_bytes = (size_t)(plan.threads / 64) * 4096;
     return (size_t)kLutBytes + (x_bytes > red_bytes ? x_bytes : red_bytes) + 16;
 }
@@ -178,7 +178,7 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
         const int swz = a.xcd_swizzle && plan.grid.x % 8 == 0;
         const int packed = a.split_log2 | a.waves_m << 4 | a.epilogue << 9 | swz << 11 | (int)(plan.grid.x >> 3) << 12;
         hipLaunchKernelGGL(lv->fn, plan.grid, dim3(plan.threads), lean_lds_bytes(plan), stream, a.q, a.x, a.code, a.absmax,
-                           a.k, a.n, a.steps_per_split, a.x_slots_magic, packed, a.m, a.out, a.residual, a.ws, a.counters,
+                           a.k, a.n, a.steps_per_split, packed, a.m, a.out, a.residual, a.ws, a.counters,
                            a.row_tiles
 #ifdef TUNA_TRACE
                            ,

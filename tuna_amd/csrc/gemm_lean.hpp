@@ -46,7 +46,6 @@ struct LeanArgs {
     const float *code;
     const float *absmax;
     int k, n, steps_per_split;
-    unsigned x_slots_magic;
     int packed;  // split_log2 | waves_m << 4 | epilogue << 9 | swizzle << 11 | (workgroups / 8) << 12
     int m;
     void *out;
@@ -62,7 +61,7 @@ struct LeanArgs {
 template <int WK, int U, int MAXT, int MINW>
 __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_q, const void *a_x, const float *a_code,
                                                                const float *a_absmax, int a_k, int a_n, int a_sps,
-                                                               unsigned a_magic, int a_packed, int a_m, void *a_out,
+                                                               int a_packed, int a_m, void *a_out,
                                                                const void *a_residual, float *a_ws, unsigned *a_counters,
                                                                int a_row_tiles
 #ifdef TUNA_TRACE
@@ -81,7 +80,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
         float *ws;
         unsigned *counters;
         int m, n, k, steps_per_split, row_tiles, split_log2, split_k, waves_m, xcd_swizzle, epilogue;
-        unsigned x_slots_magic;
 #ifdef TUNA_TRACE
         unsigned long long *trace;
 #endif
@@ -89,7 +87,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
                  a_out,         a_residual,   a_ws,            a_counters,
                  a_m,           a_n,          a_k,             a_sps,
                  a_row_tiles,   a_packed & 15, 1 << (a_packed & 15), (a_packed >> 4) & 31,
-                 (a_packed >> 11) & 1, (a_packed >> 9) & 3, a_magic
+                 (a_packed >> 11) & 1, (a_packed >> 9) & 3
 #ifdef TUNA_TRACE
                  ,
                  a_trace
@@ -142,48 +140,29 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
     const float code_lane = a.code[i16];
     const f32x4 sc32 = *reinterpret_cast<const f32x4 *>(a.absmax + row0 + i16 * 4);
     // x slice [16 tokens][k of this split], in 16-byte pieces (one token, one 8-k slot).  Piece
-    // p = tid + b*nthreads is token p / x_slots, slot p % x_slots: consecutive lanes read
-    // consecutive bytes of one token row (a wave instruction that touches 16 rows instead costs
-    // three times the cycles in the address path).  In LDS slot s, token t sits at byte
-    // s*272 + t*16: the 16 tokens of a slot are one contiguous B-fragment row, and the 16-byte pad
-    // per slot spreads the staging writes (consecutive slots, same token) over all banks.
-    // 64 * steps_per_split pieces, at most 8 per thread.
-    const int x_slots = a.steps_per_split * 4;
-    const int x_pieces = x_slots * 16;
+    // p = tid + b*nthreads: lane p % 64 picks token lane / 4 and 8-k group lane % 4, p / 64 the
+    // k-step.  Every quad of lanes reads 64 contiguous bytes of one token row (neighbouring lanes
+    // on different rows would cost three times the cycles in the address path) and a wave
+    // instruction writes one k-step - 4 slots x 16 tokens, 1 KB contiguous - to LDS, where slot s,
+    // token t sits at byte s*256 + t*16: the 16 tokens of a slot are one B-fragment row.
+    // 64 * steps_per_split pieces, at most 8 per thread.  Rows past n: clamped loads, zeros stored.
+    const int x_steps = a.steps_per_split;
     const unsigned char *xsl = reinterpret_cast<const unsigned char *>(a.x) + ((size_t)tok0 * a.k + (size_t)sb * 32) * 2;
     const int n_rel = a.n - 1 - tok0;  // last valid token row of this tile, relative
+    const int x_row = lane >> 2, x_grp = lane & 3;
+    const bool x_row_ok = x_row <= n_rel;
+    const uint32_t x_lane_off = (uint32_t)min(x_row, n_rel) * ((uint32_t)a.k * 2u) + (uint32_t)x_grp * 16u;  // (k < 2^23)
+    const int x_wv0 = wave, x_dwv = nthreads >> 6;  // this wave's first k-step and the stride between its pieces
     u32x4 xv[8];
-    uint32_t xl[8];  // LDS byte of each piece, bit 0: token row past n (store zeros); ~0u: no piece
-    const bool x_long = x_pieces > 4 * nthreads;  // uniform
-    // (token, slot) of the thread's first piece by one division (multiplication by the host's
-    // reciprocal); the following pieces are nthreads further: a uniform number of token rows and
-    // slots, with one carry.  The global and the LDS offset of a piece advance the same way.
-    // Rows past n are loaded from the last valid row (offsets clamped) and stored as zeros.
-    const uint32_t row_bytes = (uint32_t)a.k * 2u;  // (32-bit offsets off the uniform base: 16 rows of at most 2^23 k)
-    const uint32_t x_dt = __umulhi((uint32_t)nthreads, a.x_slots_magic), x_ds = (uint32_t)nthreads - x_dt * (uint32_t)x_slots;
-    uint32_t x_t = __umulhi((uint32_t)tid, a.x_slots_magic), x_s = (uint32_t)tid - x_t * (uint32_t)x_slots;
-    uint32_t x_go = x_t * row_bytes + x_s * 16u, x_lo = x_s * 272u + x_t * 16u;
-    const uint32_t go_step = x_dt * row_bytes + x_ds * 16u, lo_step = x_ds * 272u + x_dt * 16u;  // uniform
-    const uint32_t go_carry = row_bytes - (uint32_t)x_slots * 16u, lo_carry = 16u - (uint32_t)x_slots * 272u;
-    const uint32_t go_max = (uint32_t)min(n_rel, 15) * row_bytes + (uint32_t)(x_slots - 1) * 16u;
-#define TUNA_LEAN_XLOAD(b)                                                                      \
-    {                                                                                          \
-        xl[b] = (tid + (b) * nthreads) < x_pieces ? x_lo | ((int)x_t > n_rel ? 1u : 0u) : ~0u;  \
-        xv[b] = *reinterpret_cast<const u32x4 *>(xsl + min(x_go, go_max));                     \
-        x_s += x_ds;                                                                           \
-        const bool carry_ = x_s >= (uint32_t)x_slots;                                          \
-        x_s -= carry_ ? (uint32_t)x_slots : 0u;                                                \
-        x_t += x_dt + (carry_ ? 1u : 0u);                                                      \
-        x_go += go_step + (carry_ ? go_carry : 0u);                                            \
-        x_lo += lo_step + (carry_ ? lo_carry : 0u);                                            \
-    }
+    const bool x_long = x_steps > 4 * x_dwv;  // uniform: more than 4 pieces per thread
 #pragma unroll
-    for (int b = 0; b < 4; ++b) TUNA_LEAN_XLOAD(b)
+    for (int b = 0; b < 4; ++b)  // (clamped: a short slice has fewer than 4 pieces per thread)
+        xv[b] = *reinterpret_cast<const u32x4 *>(xsl + (size_t)min(x_wv0 + b * x_dwv, x_steps - 1) * 64 + x_lane_off);
     if (x_long) {
 #pragma unroll
-        for (int b = 4; b < 8; ++b) TUNA_LEAN_XLOAD(b)
+        for (int b = 4; b < 8; ++b)
+            xv[b] = *reinterpret_cast<const u32x4 *>(xsl + (size_t)min(x_wv0 + b * x_dwv, x_steps - 1) * 64 + x_lane_off);
     }
-#undef TUNA_LEAN_XLOAD
 
     // the weights last: x and the scales come from L2 and are needed first, the first ring turn
     // comes from HBM and is needed once x is staged
@@ -224,13 +203,16 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
         sc16[j] = f16x2{h, h};
     }
     // ---- x into LDS; one barrier publishes the table and the slice ---------------------------
+    unsigned char *x_dst = work + x_grp * 256 + x_row * 16;
 #pragma unroll
     for (int b = 0; b < 4; ++b)
-        if (xl[b] != ~0u) *reinterpret_cast<u32x4 *>(work + (xl[b] & ~1u)) = (xl[b] & 1u) ? u32x4{0u, 0u, 0u, 0u} : xv[b];
+        if (x_wv0 + b * x_dwv < x_steps)
+            *reinterpret_cast<u32x4 *>(x_dst + (size_t)(x_wv0 + b * x_dwv) * 1024) = x_row_ok ? xv[b] : u32x4{0u, 0u, 0u, 0u};
     if (x_long) {
 #pragma unroll
         for (int b = 4; b < 8; ++b)
-            if (xl[b] != ~0u) *reinterpret_cast<u32x4 *>(work + (xl[b] & ~1u)) = (xl[b] & 1u) ? u32x4{0u, 0u, 0u, 0u} : xv[b];
+            if (x_wv0 + b * x_dwv < x_steps)
+                *reinterpret_cast<u32x4 *>(x_dst + (size_t)(x_wv0 + b * x_dwv) * 1024) = x_row_ok ? xv[b] : u32x4{0u, 0u, 0u, 0u};
     }
     __syncthreads();
     TUNA_LMARK(3)
@@ -239,8 +221,8 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
     f32x4 acc[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const unsigned char *xb = work + g * 272 + i16 * 16 + wk * 1088;  // B fragment of this wave's step 0 (4 slots of 272 bytes per step)
-    constexpr int wstep = WK * 1088;                                   // LDS bytes between its consecutive steps
+    const unsigned char *xb = work + g * 256 + i16 * 16 + wk * 1024;  // B fragment of this wave's step 0
+    constexpr int wstep = WK * 1024;                                   // LDS bytes between its consecutive steps
 #define TUNA_LEAN_CONSUME(u)                                                                    \
     {                                                                                          \
         const f16x8 b_ = *reinterpret_cast<const f16x8 *>(xb + (u) * wstep);                   \

@@ -34,7 +34,6 @@ struct GemmArgs {
     int m, n, k;
     int waves_m, waves_k, split_k;  // waves_k is a power of two, waves_m any count
     int split_log2;                 // log2(split_k) if it is a power of two, else -1
-    unsigned x_slots_magic;         // floor(2^32 / (4 * steps_per_split)) + 1: p / (4 * steps_per_split) == mulhi(p, magic) for p < 2^16
     int wk_log2;
     int steps_total;      // ceil(k / 32)
     int steps_per_split;  // k-steps owned by one workgroup

@@ -148,7 +148,7 @@ def lds_bytes(c: dict) -> int:
         # narrow-row kernel: decode table + one accumulator plane (1 KB) per wave and 16 rows
         return LUT_BYTES + c["waves_k"] * (c["rows_per_wave"] // 16) * c["token_tiles"] * 1024
     threads = 64 * c["waves_k"] * c["waves_m"]
-    x = (c["x_chunk"] // 8) * (256 * c["token_tiles"] + 16)   # 8-k slots of 16*token_tiles pieces + 16 bytes of padding
+    x = c["token_tiles"] * 16 * c["x_chunk"] * 2
     plane = c["waves_k"] * c["waves_m"] * 1024
     small = LUT_BYTES + max(x, 2 * plane)
     big = LUT_BYTES + max(x, 8 * plane)

@@ -149,7 +149,7 @@ def lean_space(m: int, n_key: int, k: int):
             while split <= steps:
                 sps = steps // split
                 if steps % split == 0 and sps * 64 <= 8 * 64 * waves:
-                    lds = 65536 + max(sps * 1088, waves * 4096) + 16
+                    lds = 65536 + max(sps * 1024, waves * 4096) + 16
                     wgs = min(make_configs.LDS_LIMIT // lds, max(1, 20 // waves)) if lds <= make_configs.LDS_LIMIT else 0
                     if (m // (64 * wm)) * split <= N_CU * wgs:
                         for pf in (2, 4, 8):
