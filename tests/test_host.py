@@ -178,6 +178,13 @@ def test_tuner_small_launch_config_spaces_are_valid_for_both_validators():
             assert (lds, ws) == (mc.lds_bytes(c), 0)
         tiles = {c["token_tiles"] for c in narrow}
         assert tiles == ({1} if n <= 16 else {1, 2} if n <= 32 else {1, 2, 4})
+    # 16 waves x 64 rows x 2 token tiles: 128 KB of reduction planes beside the 64 KB table - refused by both validators
+    big = dict(rows_per_wave=64, waves_m=0, waves_k=16, split_k=1, prefetch=2, x_chunk=1024, token_tiles=2, xcd_swizzle=0,
+               k_stagger=0, lds_tile_rows=0)
+    with pytest.raises(ValueError):
+        mc.validate(256, 32, 5120, big)
+    with pytest.raises(ops.TunaError):
+        ops.validate_config(256, 32, 5120, ops.GemmConfig.from_dict(big))
     assert tuner.narrow_space(4096, 128, 4096) == [] and tuner.lean_space(4096, 128, 4096) == []
     assert tuner.lean_space(4096, 16, 4104) == []       # k not a multiple of 32: no lean launch
 

@@ -266,6 +266,8 @@ static int plan_narrow(int m, int n, int k, const tuna_gemm_config &c, int decod
     plan->waves_k = c.waves_k;
     plan->prefetch = c.prefetch;
     plan->lds_bytes = (size_t)kLutBytes + (size_t)c.waves_k * (c.rows_per_wave / 16) * c.token_tiles * 1024;
+    if (plan->lds_bytes > (size_t)kLdsLimit)
+        return fail(TUNA_ERR_UNSUPPORTED, "config needs %zu bytes of LDS, the CU has %d", plan->lds_bytes, kLdsLimit);
     plan->args.m = m;
     plan->args.n = n;
     plan->args.k = k;

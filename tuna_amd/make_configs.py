@@ -105,6 +105,8 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
             raise ValueError("rows_per_wave 16 or 32 needs m a multiple of it and k a multiple of 32*waves_k*prefetch")
         if m * k // 2 >= 1 << 32 or k * 32 >= 1 << 32:
             raise ValueError("operands exceed the kernel's 32-bit offsets")
+        if lds_bytes(c) > LDS_LIMIT:
+            raise ValueError(f"needs {lds_bytes(c)} bytes of LDS (limit {LDS_LIMIT})")
         return
     if c["rows_per_wave"] not in (64, 128, 256):
         raise ValueError("rows_per_wave must be 16, 32 (narrow-row kernel), 64, 128 or 256")
