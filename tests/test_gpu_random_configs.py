@@ -1,0 +1,78 @@
+"""Seeded random launch configurations of the three streaming kernel families against the oracle.
+
+Every case draws a shape, a token count and a config from the same spaces the tuner searches
+(narrow-row variants, lean-kernel layouts, the general kernel's seed pool), keeps it only if the Python
+validator accepts it, and runs it through the C-ABI. A config the Python validator accepts but the library
+cannot launch, or a launch that differs from the oracle beyond the GEMM tolerance, fails the test.
+Output layout and rounding follow kernel.cu:2649-2754 (fp32 accumulate, one fp16 rounding).
+"""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import O, REL_TOL, make_inputs_np, rel_err, to_dev
+from tuna_amd import make_configs as mc
+from tuna_amd import ops, tuner
+
+pytestmark = pytest.mark.gpu
+
+TOKENS = [1, 2, 3, 4, 5, 7, 8, 15, 16, 17, 31, 32, 33, 48, 63, 64, 65, 100]
+
+
+def draw(rng):
+    kind = rng.choice(["narrow", "lean", "general"])
+    n = rng.choice(TOKENS)
+    bucket = mc.bucket_of(n)
+    if kind == "narrow":
+        rows, wk, pf, tt = rng.choice(sorted(mc.NARROW_VARIANTS))
+        m = rows * rng.randint(1, 12)
+        k = 32 * wk * pf * rng.randint(1, 6)
+        c = dict(rows_per_wave=rows, waves_m=0 if rows == 64 else 1, waves_k=wk, split_k=1, prefetch=pf,
+                 x_chunk=32 * wk * pf, token_tiles=tt, xcd_swizzle=0, k_stagger=0, lds_tile_rows=0)
+    elif kind == "lean":
+        wm, wk = rng.randint(1, 8), rng.choice([1, 2, 4, 8, 16])
+        if wm * wk > 16:
+            return None
+        pf, sp = rng.choice([2, 4, 8]), rng.choice([1, 2, 4, 8])
+        k = 32 * wk * pf * rng.randint(1, 4) * sp
+        m = 64 * wm * rng.randint(1, 6)
+        c = dict(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=sp, prefetch=pf, x_chunk=32 * wk * pf,
+                 token_tiles=1, xcd_swizzle=rng.choice([0, 1]), k_stagger=0, lds_tile_rows=0)
+        c = tuner.repair(c, m, bucket, k)
+        if c is None or c["token_tiles"] != 1 or c["split_k"] != sp:
+            return None
+    else:
+        m, k = 8 * rng.randint(1, 120), 8 * rng.randint(1, 400)
+        pool = tuner.seeds(m, bucket, k)
+        if not pool:
+            return None
+        c = rng.choice(pool)
+    try:
+        mc.validate(m, bucket, k, c)
+    except ValueError:
+        return None
+    return kind, m, n, k, c
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_configs_match_oracle(seed):
+    rng = random.Random(seed)
+    ran = {"narrow": 0, "lean": 0, "general": 0}
+    for case in range(45):
+        drawn = draw(rng)
+        if drawn is None:
+            continue
+        kind, m, n, k, c = drawn
+        q, x, code, absmax = make_inputs_np(m, n, k, seed=seed * 1000 + case)
+        want = O.gemm_f64(q, x, code, absmax, m, n, k, mode=O.D1)
+        dq, dx, dc, da = to_dev(q, x, code, absmax)
+        out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+        print(f"seed {seed} case {case} {kind} m={m} n={n} k={k} {c}", flush=True)
+        ops.matmul(dx, dq, da, dc, out, m, n, k, config=ops.GemmConfig.from_dict(c))
+        torch.cuda.synchronize()
+        err = rel_err(out.cpu().numpy().astype(np.float64), want)
+        assert err <= REL_TOL, (kind, m, n, k, c, err)     # max relative error 1e-2
+        ran[kind] += 1
+    assert all(v >= 3 for v in ran.values()), ran
