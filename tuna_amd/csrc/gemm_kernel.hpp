@@ -70,6 +70,10 @@ __device__ __forceinline__ uint32_t f16_bits(f16 h)
     return (uint32_t)__builtin_bit_cast(uint16_t, h);
 }
 
+// s_waitcnt immediate for "at most n vector memory operations outstanding", the other counters
+// unconstrained (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8).
+constexpr int wait_vmcnt(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
+
 // Decode one packed dword (one weight row, 8 consecutive k) into the MFMA A operand.
 template <int DEC>
 __device__ __forceinline__ f16x8 decode_dword(uint32_t d, const unsigned char *lut, uint32_t lane4,
@@ -570,6 +574,12 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
         // the work area is free again once every wave has left the previous tile's epilogue
         __syncthreads();
         if (n_chunks > 0) x_stage_store<TT, XB>(xst, work, nthreads, tid, x_pieces, cur_tok0, cur_sb * kStepK, cur_ntok, a.k, krot);
+        // The x pieces are the youngest loads in flight, so a thread that stored one has waited for
+        // everything; a thread with no piece to store has not, and the compiler then carries its
+        // staging registers as pending loads through the tile: reusing one of them inside the main
+        // loop gets a wait for ALL loads there, which empties the weight ring once per group.
+        // The explicit wait makes "nothing pending" a fact on every path.
+        __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));
         __syncthreads();
         TUNA_MARK(3)
 
@@ -589,6 +599,8 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                 x_stage_load<TT, XB>(xst, xg, nthreads, tid, cur_tok0, kbase, cur_ntok, a.k, krot);
                 TUNA_GROUP()
                 __syncthreads();  // every wave is done reading chunk c
+                // exactly the group's U*RW refills are younger than the x pieces (see above)
+                __builtin_amdgcn_s_waitcnt(wait_vmcnt(U * RW));
                 x_stage_store<TT, XB>(xst, work, nthreads, tid, x_pieces, cur_tok0, kbase, cur_ntok, a.k, krot);
                 __syncthreads();
             } else {
