@@ -76,3 +76,55 @@ def test_random_configs_match_oracle(seed):
         assert err <= REL_TOL, (kind, m, n, k, c, err)     # max relative error 1e-2
         ran[kind] += 1
     assert all(v >= 3 for v in ran.values()), ran
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_random_shapes_through_the_dispatcher_match_oracle(seed):
+    """No config: the library picks one for every shape and token count, tuned or not (m and k any
+    multiples of 8, 1..2500 tokens - every bucket of the dispatcher, kernel.cu:3022-3155)."""
+    from helpers import f16_bits_to_f64, run_gemm
+    rng = random.Random(seed)
+    for case in range(28):
+        n = rng.choice([1, 2, 9, 16, 17, 40, 64, 100, 128, 200, 256, 300, 512, 600, 769, 1025, 2500])
+        budget = 3e8 // n                                   # keeps the oracle's float64 GEMM in seconds
+        k = 8 * rng.randint(1, 600)
+        m = 8 * rng.randint(1, max(1, min(400, int(budget // k) // 8)))
+        q, x, code, absmax = make_inputs_np(m, n, k, seed=seed * 1000 + case)
+        print(f"seed {seed} case {case} dispatcher m={m} n={n} k={k}", flush=True)
+        got = run_gemm(q, x, code, absmax, m, n, k, prefill=float("nan"))
+        want = O.gemm_f64(q, x, code, absmax, m, n, k, mode=O.D1)
+        err = rel_err(f16_bits_to_f64(got), want)
+        assert err <= REL_TOL, (m, n, k, err)              # max relative error 1e-2
+
+
+def test_random_grouped_launches_match_per_group_oracle():
+    """Random group counts, sizes and token lists (empty groups included), no config."""
+    from helpers import f16_bits_to_f64
+    rng = random.Random(31)
+    for case in range(12):
+        n_groups = rng.choice([1, 2, 3, 8, 16])
+        m_group = 64 * rng.randint(1, 8)                 # groups are whole 64-row tiles
+        k = 8 * rng.randint(1, 300)
+        counts = [rng.choice([0, 0, 1, 3, 16, 17, 40]) for _ in range(n_groups)]
+        if sum(counts) == 0:
+            counts[rng.randrange(n_groups)] = 5
+        offsets = [0]
+        for c in counts:
+            offsets.append(offsets[-1] + c)
+        n_total, m = offsets[-1], m_group * n_groups
+        q, x, code, absmax = make_inputs_np(m, n_total, k, seed=3100 + case)
+        dq, dx, dc, da = to_dev(q, x, code, absmax)
+        out = torch.full((n_total, m_group), float("nan"), dtype=torch.float16, device="cuda")
+        print(f"grouped case {case} m_group={m_group} n_groups={n_groups} k={k} counts={counts}", flush=True)
+        ops.matmul_grouped(dx, dq, da, dc, out, m_group, n_groups, k, offsets)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy().astype(np.float64)
+        qb = q.reshape(n_groups, m_group // 8, k // 8, 32)
+        for e in range(n_groups):
+            lo, hi = offsets[e], offsets[e + 1]
+            if hi == lo:
+                continue
+            want = O.gemm_f64(np.ascontiguousarray(qb[e]), np.ascontiguousarray(x[lo:hi]), code,
+                              np.ascontiguousarray(absmax[e * m_group:(e + 1) * m_group]), m_group, hi - lo, k, mode=O.D1)
+            err = rel_err(got[lo:hi], want)
+            assert err <= REL_TOL, (case, e, err)
