@@ -103,10 +103,12 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     // put two workgroups on a CU in the first place.
     const size_t plane_lds = (size_t)c.waves_k * c.waves_m * 1024;
     const size_t lds_small = (size_t)lut + (x_lds > 2 * plane_lds ? x_lds : 2 * plane_lds);
-    const size_t lds_big = (size_t)lut + (x_lds > 8 * plane_lds ? x_lds : 8 * plane_lds);
+    // (a wave with a single 64-row group and token tile has nothing to alternate with: one buffer)
+    const size_t big_planes = nacc == 4 ? 4 : 8;
+    const size_t lds_big = (size_t)lut + (x_lds > big_planes * plane_lds ? x_lds : big_planes * plane_lds);
     const bool two_wgs_possible = threads <= 512 && 2 * lds_small <= (size_t)kLdsLimit;
     const int planes_log2 = (lds_big <= (size_t)kLdsLimit && (lds_big == lds_small || !two_wgs_possible)) ? 2 : 0;
-    const size_t red_lds = 2 * plane_lds << planes_log2;
+    const size_t red_lds = planes_log2 ? big_planes * plane_lds : 2 * plane_lds;
     const size_t lds = planes_log2 ? lds_big : lds_small;
     if (lds > (size_t)kLdsLimit)
         return fail(TUNA_ERR_UNSUPPORTED, "config needs %zu bytes of LDS, the CU has %d", lds, kLdsLimit);

@@ -141,8 +141,8 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
 def lds_bytes(c: dict) -> int:
     """Dynamic LDS of a launch: decode table + max(x chunk, reduction buffers).
 
-    The reduction buffers are 2 x 1 plane (1 KB) per wave, or 2 x 4 planes when that costs no
-    occupancy (mirrors plan_gemm in csrc/api.cpp)."""
+    The reduction buffers are 2 x 1 plane (1 KB) per wave, or 2 x 4 planes (1 x 4 for a wave with one
+    64-row group and token tile) when that costs no occupancy (mirrors plan_gemm in csrc/api.cpp)."""
     if c.get("lds_tile_rows"):
         # many-token kernel: decode table + two buffers of (weight tile + activation tile), 128 bytes per row
         return LUT_BYTES + 2 * (c["lds_tile_rows"] + 16 * c["token_tiles"]) * 128
@@ -153,7 +153,8 @@ def lds_bytes(c: dict) -> int:
     x = c["token_tiles"] * 16 * c["x_chunk"] * 2
     plane = c["waves_k"] * c["waves_m"] * 1024
     small = LUT_BYTES + max(x, 2 * plane)
-    big = LUT_BYTES + max(x, 8 * plane)
+    one_group = c["rows_per_wave"] == 64 and c["token_tiles"] == 1     # nothing to alternate with: one buffer
+    big = LUT_BYTES + max(x, (4 if one_group else 8) * plane)
     two_wgs = threads <= 512 and 2 * small <= LDS_LIMIT
     return big if big <= LDS_LIMIT and (big == small or not two_wgs) else small
 
