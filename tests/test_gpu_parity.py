@@ -687,6 +687,65 @@ def test_lean_kernel_equals_general_kernel_bit_for_bit(ci):
     assert rel_err(outs[True][0].cpu().numpy().astype(np.float64), ref) <= REL_TOL
 
 
+# ----------------------------------------------------------------------------- 17..64-token streaming kernel
+MID_CASES = [
+    # m, n, k, config of the launch, config of the general-kernel launch it is compared with (None: the same)
+    (512, 32, 512, dict(waves_m=8, waves_k=1, prefetch=2, token_tiles=2, x_chunk=256), None),
+    (1024, 17, 1024, dict(waves_m=8, waves_k=1, prefetch=4, token_tiles=2, x_chunk=512), None),       # ragged second tile
+    (2048, 30, 2048, dict(waves_m=8, waves_k=1, prefetch=8, token_tiles=2, x_chunk=512), None),
+    (512, 64, 512, dict(waves_m=4, waves_k=1, prefetch=2, token_tiles=4, x_chunk=128), None),
+    (1344, 100, 1024, dict(waves_m=7, waves_k=1, prefetch=2, token_tiles=2, x_chunk=256), None),      # 7 waves, 4 token chunks
+    # ring depths and workgroup sizes only this kernel has: the general kernel with ring 2 (and 8 waves)
+    # adds the same products in the same order
+    (1536, 50, 2048, dict(waves_m=8, waves_k=1, prefetch=8, token_tiles=4, x_chunk=256),
+     dict(waves_m=8, waves_k=1, prefetch=2, token_tiles=4, x_chunk=256)),
+    (4096, 32, 1024, dict(waves_m=16, waves_k=1, prefetch=4, token_tiles=2, x_chunk=512),
+     dict(waves_m=8, waves_k=1, prefetch=4, token_tiles=2, x_chunk=512)),
+    # more row tiles than CUs: the workgroups walk (296 tiles of 256 rows), one chunk of x per tile
+    (75776, 33, 256, dict(waves_m=4, waves_k=1, prefetch=2, token_tiles=4, x_chunk=128), None),
+]
+
+
+@pytest.mark.parametrize("ci", range(len(MID_CASES)))
+def test_mid_token_kernel_equals_general_kernel_bit_for_bit(ci):
+    """Dense unsplit launches with two or four token tiles take the 17..64-token streaming kernel;
+    it must give the bits of the general kernel (same decode, same summation order), for the plain
+    store and both fused epilogues, and be within tolerance of the oracle."""
+    import torch
+
+    from tuna_amd import _lib, ops
+
+    m, n, k, kw, kw_general = MID_CASES[ci]
+    c, cg = cfg(**kw), cfg(**(kw_general or kw))
+    print(f"mid case#{ci} {m}x{n}x{k} {c.to_dict()}", flush=True)
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=180 + ci)
+    res = (np.random.default_rng(ci).standard_normal((n, m)) * 0.05).astype(np.float16)
+    dq, dx, dc, da, dres = to_dev(q, x, code, absmax, res)
+    outs = {}
+    prev = ops.set_lean_kernels(True)
+    try:
+        for twin in (True, False):
+            ops.set_lean_kernels(twin)
+            before = ops.lean_launches()
+            o_plain = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+            o_res = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+            o_silu = torch.full((n, m // 2), float("nan"), dtype=torch.float16, device="cuda")
+            cc = c if twin else cg
+            ops.matmul(dx, dq, da, dc, o_plain, m, n, k, config=cc)
+            ops.matmul_fused(dx, dq, da, dc, o_res, m, n, k, _lib.EPILOGUE_RESIDUAL, residual=dres, config=cc)
+            ops.matmul_fused(dx, dq, da, dc, o_silu, m, n, k, _lib.EPILOGUE_SILU_MUL, config=cc)
+            torch.cuda.synchronize()
+            assert ops.lean_launches() - before == (3 if twin else 0)   # the case really qualifies
+            outs[twin] = (o_plain, o_res, o_silu)
+    finally:
+        ops.set_lean_kernels(prev)
+    for a, b in zip(outs[True], outs[False]):
+        assert not torch.isnan(a.float()).any()
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    ref = O.gemm_f64(q, x, code, absmax, m, n, k, mode=O.D1)
+    assert rel_err(outs[True][0].cpu().numpy().astype(np.float64), ref) <= REL_TOL   # max relative error 1e-2
+
+
 # ----------------------------------------------------------------------------- narrow-row kernel
 NARROW_CASES = [
     # m, n, k, rows_per_wave, waves_k, prefetch

@@ -185,6 +185,23 @@ def test_tuner_small_launch_config_spaces_are_valid_for_both_validators():
         mc.validate(256, 32, 5120, big)
     with pytest.raises(ops.TunaError):
         ops.validate_config(256, 32, 5120, ops.GemmConfig.from_dict(big))
+    # configs only the 17..64-token streaming kernel has (ring 8 with four token tiles, 16 waves with two): valid
+    # for both validators while the launch qualifies, refused by both when it does not (waves along k)
+    mid = dict(rows_per_wave=64, waves_m=8, waves_k=1, split_k=1, prefetch=8, x_chunk=256, token_tiles=4, xcd_swizzle=0,
+               k_stagger=0, lds_tile_rows=0)
+    for c, ok in ((mid, True), (dict(mid, waves_m=16, token_tiles=2, prefetch=4), True),
+                  (dict(mid, waves_m=4, waves_k=2), False), (dict(mid, k_stagger=3), False)):
+        assert mc.mid_applies(229376, 4096, c) == ok
+        if ok:
+            mc.validate(229376, 64 if c["token_tiles"] == 4 else 32, 4096, c)
+            ops.validate_config(229376, 64 if c["token_tiles"] == 4 else 32, 4096, ops.GemmConfig.from_dict(c))
+        else:
+            with pytest.raises(ValueError):
+                mc.validate(229376, 64, 4096, c)
+            with pytest.raises(ops.TunaError):
+                ops.validate_config(229376, 64, 4096, ops.GemmConfig.from_dict(c))
+    space = tuner.mid_space(229376, 64, 4096)
+    assert space and all(mc.mid_applies(229376, 4096, c) for c in space) and tuner.mid_space(229376, 16, 4096) == []
     assert tuner.narrow_space(4096, 128, 4096) == [] and tuner.lean_space(4096, 128, 4096) == []
     assert tuner.lean_space(4096, 16, 4104) == []       # k not a multiple of 32: no lean launch
 

@@ -121,10 +121,9 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
         min_waves = 4;
         wgs_per_cu = 2;
     }
-    if (!gemm_variant_exists(rw, c.prefetch, c.token_tiles, decode, threads, min_waves, grouped))
-        return fail(TUNA_ERR_UNSUPPORTED,
-                    "no %skernel variant for rows_per_wave=%d prefetch=%d token_tiles=%d decode=%d threads=%d",
-                    grouped ? "grouped " : "", c.rows_per_wave, c.prefetch, c.token_tiles, decode, threads);
+    // (a launch without a variant of the general kernel may still be one the 17..64-token streaming
+    // kernel takes: decided below, when the launch arguments are known)
+    const bool have_general = gemm_variant_exists(rw, c.prefetch, c.token_tiles, decode, threads, min_waves, grouped);
 
     const int row_tiles = ceil_div(m, rows_wg);
     const int tok_chunks = ceil_div(n, 16 * c.token_tiles);
@@ -188,6 +187,10 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     a.red_bytes = (int)red_lds;
     a.planes_log2 = planes_log2;
     a.tiles_total = row_tiles * c.split_k;
+    if (!have_general && (grouped || !mid_applies(*plan)))
+        return fail(TUNA_ERR_UNSUPPORTED,
+                    "no %skernel variant for rows_per_wave=%d prefetch=%d token_tiles=%d decode=%d threads=%d",
+                    grouped ? "grouped " : "", c.rows_per_wave, c.prefetch, c.token_tiles, decode, threads);
     return TUNA_OK;
 }
 

@@ -1,0 +1,93 @@
+// Instantiations and launcher of the 17..64-token streaming kernel (gemm_mid.hpp).
+#include <mutex>
+
+#include "gemm_mid.hpp"
+
+namespace tuna {
+
+typedef void (*MidKernelFn)(const uint8_t *, const void *, const float *, const float *, int, int, int, int, void *,
+                            const void *, int, int);
+struct MidVariant {
+    int u, tt, xb, maxt;
+    MidKernelFn fn;
+};
+#define M5(U, TT, XB) {U, TT, XB, 512, gemm_mid_kernel<U, TT, XB, 512, 2>}
+#define M10(U, TT, XB) {U, TT, XB, 1024, gemm_mid_kernel<U, TT, XB, 1024, 4>}
+static const MidVariant kMid[] = {
+    M5(2, 2, 4), M5(4, 2, 4), M5(8, 2, 4), M5(2, 2, 8), M5(4, 2, 8), M5(8, 2, 8),
+    M5(2, 4, 4), M5(4, 4, 4), M5(8, 4, 4), M5(2, 4, 8), M5(4, 4, 8), M5(8, 4, 8),
+    M10(2, 2, 4), M10(4, 2, 4),
+};
+#undef M5
+#undef M10
+static constexpr int kNumMid = sizeof(kMid) / sizeof(kMid[0]);
+
+// x chunk the kernel uses: the config's, capped so that two buffers fit beside the decode table.
+static int mid_x_chunk(const GemmPlan &plan)
+{
+    int xc = plan.args.chunk_steps * kStepK;
+    const int cap = (kLdsLimit - kLutBytes) / (2 * plan.token_tiles * 32);  // k per buffer
+    while (xc > cap) xc >>= 1;
+    return xc;
+}
+
+static const MidVariant *mid_variant(const GemmPlan &plan, int *xc_out)
+{
+    const GemmArgs &a = plan.args;
+    if (a.group_rows || a.balanced || plan.rw != 1 || plan.decode != TUNA_DECODE_GEMM) return nullptr;
+    if (plan.token_tiles != 2 && plan.token_tiles != 4) return nullptr;
+    if (a.waves_k != 1 || a.split_k != 1 || a.k_stagger != 0) return nullptr;
+    if (a.k != a.steps_total * kStepK || a.k >= (1 << 23)) return nullptr;
+    if (a.m % (a.waves_m * kRowsPerLoad) != 0 || a.waves_m > 16) return nullptr;
+    const int xc = mid_x_chunk(plan);
+    if (xc < plan.prefetch * kStepK || (xc & (xc - 1)) != 0 || a.k % xc != 0) return nullptr;
+    const int pieces = plan.token_tiles * 2 * xc;  // 16-byte pieces per chunk
+    const int per_thread = (pieces + plan.threads - 1) / plan.threads;
+    if (per_thread > 8) return nullptr;
+    const int xb = per_thread <= 4 ? 4 : 8;
+    const int maxt = plan.threads <= 512 ? 512 : 1024;
+    for (int i = 0; i < kNumMid; ++i)
+        if (kMid[i].u == plan.prefetch && kMid[i].tt == plan.token_tiles && kMid[i].xb == xb && kMid[i].maxt == maxt) {
+            *xc_out = xc;
+            return &kMid[i];
+        }
+    return nullptr;
+}
+
+bool mid_applies(const GemmPlan &plan)
+{
+    int xc;
+    return mid_variant(plan, &xc) != nullptr;
+}
+
+static std::mutex g_mid_mutex;
+static unsigned char g_mid_attr_done[16][kNumMid];
+
+hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t stream)
+{
+    int xc = 0;
+    const MidVariant *v = mid_variant(plan, &xc);
+    if (!v) return hipErrorInvalidConfiguration;
+    const int vi = (int)(v - kMid);
+    {
+        std::lock_guard<std::mutex> lock(g_mid_mutex);
+        if (!g_mid_attr_done[dev][vi]) {
+            hipError_t e =
+                hipFuncSetAttribute(reinterpret_cast<const void *>(v->fn), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
+            if (e != hipSuccess) return e;
+            g_mid_attr_done[dev][vi] = 1;
+        }
+    }
+    const GemmArgs &a = plan.args;
+    int xc_log2 = 0;
+    while ((1 << xc_log2) < xc) ++xc_log2;
+    const size_t lds = (size_t)kLutBytes + 2 * (size_t)plan.token_tiles * 32 * (size_t)xc;
+    dim3 grid = plan.grid;
+    grid.x = (unsigned)(a.row_tiles < cus ? a.row_tiles : cus);  // one workgroup per CU (LDS), walking row tiles
+    const int packed = a.waves_m | a.epilogue << 5 | xc_log2 << 8;
+    hipLaunchKernelGGL(v->fn, grid, dim3(plan.threads), lds, stream, a.q, a.x, a.code, a.absmax, a.k, a.n, a.m, packed, a.out,
+                       a.residual, a.row_tiles, (int)grid.x);
+    return hipGetLastError();
+}
+
+}  // namespace tuna

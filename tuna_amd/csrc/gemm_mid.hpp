@@ -1,0 +1,201 @@
+// Streaming GEMM kernel for 17..64 tokens per pass on shapes with many rows (gfx950, wave64).
+//
+// With two or four 16-token tiles per wave every decoded weight fragment feeds two or four
+// MFMAs and the launch sits between the bandwidth and the matrix-core bound: what counts is how
+// many weight loads a wave keeps in flight and how little else it does.  This kernel computes
+// exactly what gemm_kernel computes for one class of launches:
+//   * dense, no split of k at all (every wave owns 64 rows and walks the whole k range:
+//     waves_k = 1, split_k = 1), no stagger, m a multiple of the workgroup's rows, k a multiple
+//     of the x chunk, chunks of whole ring turns: no clamped or conditional weight loads, no
+//     tails, no cross-wave reduction (accumulators are final, stored from registers);
+//   * x chunks are double-buffered in LDS: chunk c + 1 is requested before chunk c is consumed
+//     and written to the other buffer after it, one barrier per chunk, and the weight ring runs
+//     on across chunk and tile boundaries' barriers without being emptied;
+//   * arguments as separate scalars (preloaded with the wave), persistent workgroups walking row
+//     tiles with a fixed stride, the decode table built once per workgroup.
+// Same operand mapping, decode and summation order as gemm_kernel (see gemm_kernel.hpp), so the
+// results are bit-identical to the general kernel run with the same config.  launch_gemm picks
+// it when the launch qualifies (mid_applies in gemm_launch.hip).
+#pragma once
+#include "gemm_kernel.hpp"
+
+namespace tuna {
+
+template <int U, int TT, int XB, int MAXT, int MINW>
+__global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q, const void *a_x, const float *a_code,
+                                                              const float *a_absmax, int a_k, int a_n, int a_m, int a_packed,
+                                                              void *a_out, const void *a_residual, int a_row_tiles,
+                                                              int a_n_wg)
+{
+    // a_packed = waves_m | epilogue << 5 | log2(x chunk in k) << 8
+    const int waves_m = a_packed & 31;
+    const int epilogue = (a_packed >> 5) & 7;
+    const int xc_log2 = (a_packed >> 8) & 31;
+    extern __shared__ __align__(16) unsigned char smem[];
+    unsigned char *lut = smem;
+    unsigned char *xbuf = smem + kLutBytes;  // two buffers of one x chunk: [slot][token tile][token][16 B]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int i16 = lane & 15;
+    const int g = lane >> 4;
+    const int wm = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nthreads = waves_m * 64;
+    const uint32_t lane4 = (uint32_t)lane << 2;
+    const int tok0 = blockIdx.y * (16 * TT);
+    const int xc = 1 << xc_log2;
+    const int chunk_steps = xc >> 5;                 // a multiple of U
+    const int n_chunks = a_k >> xc_log2;
+    const int n_steps = a_k >> 5;
+    const uint32_t kb_total = (uint32_t)a_k >> 3;
+    const uint32_t xbuf_bytes = (uint32_t)(TT * 32) << xc_log2;  // 16*TT tokens x xc k x 2 bytes
+    const int x_pieces = (int)(xbuf_bytes >> 4);
+    const f16 *xg = reinterpret_cast<const f16 *>(a_x);
+    const KRot krot{0, a_k, a_k};
+
+    const float code_lane = a_code[i16];
+    int tile = blockIdx.x;
+    // weights of this wave's rows: lane (i16, g) loads 16 bytes = dword j of row 4*i16 + j's 8 k
+    // (block row i16/2, second half of the block for odd i16), block column 4*step + g
+    uint32_t lb = 0;
+    u32x4 wq[U];
+    f32x4 sc32{0.f, 0.f, 0.f, 0.f};
+    XStage<XB> xst;
+#define TUNA_MID_TILE_FETCH(t)                                                                  \
+    {                                                                                          \
+        const int row0_ = (t) * (waves_m * 64) + wm * 64;                                      \
+        lb = ((uint32_t)(row0_ >> 3) + (uint32_t)(i16 >> 1)) * kb_total * 32u + (uint32_t)(i16 & 1) * 16u + (uint32_t)g * 32u; \
+        _Pragma("unroll") for (int u = 0; u < U; ++u) wq[u] =                                  \
+            __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(a_q + (size_t)u * 128 + lb)); \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) sc32[j] = a_absmax[row0_ + i16 * 4 + j];  \
+        x_stage_load<TT, XB>(xst, xg, nthreads, tid, tok0, 0, a_n, a_k, krot);                 \
+    }
+    if (tile < a_row_tiles) TUNA_MID_TILE_FETCH(tile)
+
+    // ---- decode table (see gemm_kernel.hpp), built while the first loads are in flight --------
+    {
+        const int code_bits = (int)f16_bits((f16)code_lane);
+        for (int p0 = tid; p0 < kLutBytes / 16; p0 += 4 * nthreads) {
+            uint32_t v[4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int e = (p0 + b * nthreads) >> 4;
+                const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute((e >> 4) << 2, code_bits);
+                const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute((e & 15) << 2, code_bits);
+                v[b] = hi | (lo << 16);
+            }
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int p = p0 + b * nthreads;
+                if (p < kLutBytes / 16) reinterpret_cast<u32x4 *>(lut)[p] = u32x4{v[b], v[b], v[b], v[b]};
+            }
+        }
+    }
+
+    f16 *outp = reinterpret_cast<f16 *>(a_out);
+    const f16 *resp = reinterpret_cast<const f16 *>(a_residual);
+    // B fragment of lane (token i16, k-group g), local step sl, token tile tt:
+    // slot sl*4 + g, byte slot*(256*TT) + tt*256 + i16*16
+    const uint32_t xb_lane = (uint32_t)g * (256 * TT) + (uint32_t)i16 * 16;
+
+    // One ring turn: U k-steps, each consumed (B fragments from LDS, 4 fragments decoded, 4*TT
+    // MFMAs) and refilled with step + U of this tile (the last turn re-reads the last step: in
+    // bounds, never consumed).
+#define TUNA_MID_GROUP(sl)                                                                      \
+    {                                                                                          \
+        _Pragma("unroll") for (int u = 0; u < U; ++u)                                          \
+        {                                                                                      \
+            f16x8 b_[TT];                                                                      \
+            _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) b_[tt] =                         \
+                *reinterpret_cast<const f16x8 *>(xb + (size_t)((sl) + u) * (1024 * TT) + tt * 256); \
+            _Pragma("unroll") for (int j = 0; j < 4; ++j)                                      \
+            {                                                                                  \
+                const f16x8 av_ = decode_dword<TUNA_DECODE_GEMM>(wq[u][j], lut, lane4, sc16[j], 0.f); \
+                _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) acc[j][tt] =                 \
+                    __builtin_amdgcn_mfma_f32_16x16x32_f16(av_, b_[tt], acc[j][tt], 0, 0, 0);  \
+            }                                                                                  \
+            const int s_ = min(step + u + U, n_steps - 1);                                     \
+            wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(qrow + (size_t)s_ * 128)); \
+            __builtin_amdgcn_sched_barrier(0); /* keep each refill right behind its consume */ \
+        }                                                                                      \
+        step += U;                                                                             \
+    }
+
+    while (tile < a_row_tiles) {
+        f16x2 sc16[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const f16 h = (f16)sc32[j];
+            sc16[j] = f16x2{h, h};
+        }
+        const int row0 = tile * (waves_m * 64) + wm * 64;
+        f32x4 acc[4][TT];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int tt = 0; tt < TT; ++tt) acc[j][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+        // chunk 0 of x into buffer 0 (every wave has left the previous tile's last chunk: the
+        // barrier that ends a chunk), then the table and the chunk are published together
+        x_stage_store<TT, XB>(xst, xbuf, nthreads, tid, x_pieces, tok0, 0, a_n, a_k, krot);
+        __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));  // (threads without a piece: see gemm_kernel.hpp)
+        __syncthreads();
+
+        const unsigned char *qrow = a_q + lb;
+        int step = 0;  // this wave's next k-step
+        for (int c = 0; c < n_chunks; ++c) {
+            const bool has_next = c + 1 < n_chunks;
+            // (unconditional - the last chunk requests itself again and drops it: behind a branch
+            // the compiler could not count these loads into the waits of the first ring turn)
+            x_stage_load<TT, XB>(xst, xg, nthreads, tid, tok0, min(c + 1, n_chunks - 1) << xc_log2, a_n, a_k, krot);
+            const unsigned char *xb = xbuf + (c & 1) * xbuf_bytes + xb_lane;
+            // (the first ring turn of a chunk is a copy of its own: there the x pieces just
+            // requested are in flight behind the ring, and only straight-line code lets the
+            // compiler count them into its waits instead of waiting them out)
+            TUNA_MID_GROUP(0)
+            for (int sl = U; sl < chunk_steps; sl += U) TUNA_MID_GROUP(sl)
+            if (has_next) {
+                // the other buffer was last read in chunk c - 1, which ended with a barrier
+                __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));  // exactly the last ring turn's refills are younger
+                x_stage_store<TT, XB>(xst, xbuf + ((c + 1) & 1) * xbuf_bytes, nthreads, tid, x_pieces, tok0, (c + 1) << xc_log2,
+                                      a_n, a_k, krot);
+            }
+            __syncthreads();
+        }
+
+        // ---- next tile's loads, then this tile's store ------------------------------------------
+        const int cur_row0 = row0;
+        tile += a_n_wg;
+        if (tile < a_row_tiles) TUNA_MID_TILE_FETCH(tile)
+        // Lane (token i16, group g) owns 16 consecutive output features, acc[j][tt][v] being
+        // feature 4*v + j of them: two 16-byte stores per token tile.
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) {
+            const int tok = tok0 + tt * 16 + i16;
+            const int rb = cur_row0 + g * 16;
+            if (tok >= a_n) continue;
+            if (epilogue == TUNA_EPILOGUE_NONE) {
+                f16x8 lo, hi;
+#pragma unroll
+                for (int v = 0; v < 2; ++v)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        lo[v * 4 + j] = (f16)acc[j][tt][v];
+                        hi[v * 4 + j] = (f16)acc[j][tt][v + 2];
+                    }
+                f16 *dst = outp + (size_t)tok * a_m + rb;
+                *reinterpret_cast<f16x8 *>(dst) = lo;
+                *reinterpret_cast<f16x8 *>(dst + 8) = hi;
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    store_features4(outp, resp, epilogue, (size_t)tok, a_m, rb + v * 4, acc[0][tt][v], acc[1][tt][v], acc[2][tt][v],
+                                    acc[3][tt][v]);
+            }
+        }
+    }
+#undef TUNA_MID_GROUP
+#undef TUNA_MID_TILE_FETCH
+}
+
+}  // namespace tuna

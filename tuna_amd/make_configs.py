@@ -50,6 +50,11 @@ VARIANTS_512_2WG = {(1, 2, 1), (1, 4, 1)}
 VARIANTS_1024 = {(1, 2, 1), (1, 4, 1)}
 
 
+# (prefetch, token_tiles, x pieces per thread, max threads) of the 17..64-token streaming kernel; must match
+# kMid in csrc/gemm_mid.hip
+MID_VARIANTS = ({(u, tt, xb, 512) for u in (2, 4, 8) for tt in (2, 4) for xb in (4, 8)}
+                | {(2, 2, 4, 1024), (4, 2, 4, 1024)})
+
 # (rows, waves_k, prefetch, token_tiles) of the narrow-row kernel; must match kNarrow in csrc/gemm_launch.hip
 NARROW_VARIANTS = (
     {(r, wk, pf, 1) for r in (16, 32, 64) for wk in (4, 8, 16) for pf in (2, 4, 8)}
@@ -128,7 +133,7 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
     rw = c["rows_per_wave"] // 64
     key = (rw, c["prefetch"], c["token_tiles"])
     threads = 64 * wm * wk
-    if key not in (VARIANTS_512 if threads <= 512 else VARIANTS_1024):
+    if key not in (VARIANTS_512 if threads <= 512 else VARIANTS_1024) and not mid_applies(m, k, c):
         raise ValueError(f"no kernel variant {key} for {threads} threads")
     if c["x_chunk"] * c["token_tiles"] > (4 if c["prefetch"] == 8 else 2) * threads:
         raise ValueError("x_chunk * token_tiles too large for the x staging (4 pieces per thread, 8 with prefetch 8)")
@@ -136,6 +141,27 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
         raise ValueError("k_stagger must be in 0..4096")
     if lds_bytes(c) > LDS_LIMIT:
         raise ValueError(f"needs {lds_bytes(c)} bytes of LDS (limit {LDS_LIMIT})")
+
+
+def mid_applies(m: int, k: int, c: dict) -> bool:
+    """True if a dense launch of this config is taken by the 17..64-token streaming kernel
+    (mirrors mid_variant in csrc/gemm_mid.hip)."""
+    tt, wm = c["token_tiles"], c["waves_m"]
+    if c["rows_per_wave"] != 64 or tt not in (2, 4) or c["waves_k"] != 1 or c["split_k"] != 1 or c["k_stagger"] != 0:
+        return False
+    if k % STEP_K or k >= 1 << 23 or wm > 16 or m % (64 * wm):
+        return False
+    xc = c["x_chunk"]
+    cap = (LDS_LIMIT - LUT_BYTES) // (2 * tt * 32)
+    while xc > cap:
+        xc //= 2
+    if xc < c["prefetch"] * STEP_K or k % xc:
+        return False
+    threads = 64 * wm
+    per_thread = -(-(tt * 2 * xc) // threads)
+    if per_thread > 8:
+        return False
+    return (c["prefetch"], tt, 4 if per_thread <= 4 else 8, 512 if threads <= 512 else 1024) in MID_VARIANTS
 
 
 def lds_bytes(c: dict) -> int:

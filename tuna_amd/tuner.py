@@ -165,6 +165,32 @@ def lean_space(m: int, n_key: int, k: int):
     return list(uniq.values())
 
 
+def mid_space(m: int, n_key: int, k: int):
+    """Every config whose launch takes the 17..64-token streaming kernel (gemm_mid.hpp; the
+    conditions of mid_variant in gemm_mid.hip): 64 rows per wave, all waves along m, no split,
+    no stagger, two or four token tiles.  Small enough to time exhaustively."""
+    lo, hi = make_configs.N_BUCKETS[n_key]
+    if lo < 17 or lo > 64:
+        return []
+    out = []
+    for tt in ((2,) if hi <= 32 else (4,) if lo > 32 else (2, 4)):
+        for wm in range(2, 17):
+            if m % (64 * wm):
+                continue
+            for pf in (2, 4, 8):
+                for xc in (128, 256, 512, 1024):
+                    for sw in (0, 1):
+                        c = dict(rows_per_wave=64, waves_m=wm, waves_k=1, split_k=1, prefetch=pf, x_chunk=xc, token_tiles=tt,
+                                 xcd_swizzle=sw, k_stagger=0, lds_tile_rows=0)
+                        try:
+                            make_configs.validate(m, n_key, k, c)
+                        except ValueError:
+                            continue
+                        if make_configs.mid_applies(m, k, c):
+                            out.append(c)
+    return out
+
+
 def narrow_space(m: int, n_key: int, k: int):
     """Every config of the narrow-row kernel (gemm_narrow.hpp: 16 or 32 rows per workgroup, all
     waves along k, no split) the shape admits.  Small enough to time exhaustively."""
@@ -258,7 +284,7 @@ def tune_shape(m, n, k, generations=6, population=24, seed=0, log=print, max_see
         return json.loads(scored[0][1]), scored[0][0]
     pool = seeds(m, n_key, k)
     rng.shuffle(pool)
-    pool = pool[:max_seed_evals] + lean_space(m, n_key, k)
+    pool = pool[:max_seed_evals] + lean_space(m, n_key, k) + mid_space(m, n_key, k)
     for c in narrow_space(m, n_key, k):     # a kernel family of its own: timed, not bred
         ev(c)
     scored = sorted(((ev(c), json.dumps(c, sort_keys=True)) for c in pool))
