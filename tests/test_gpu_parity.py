@@ -701,8 +701,14 @@ MID_CASES = [
      dict(waves_m=8, waves_k=1, prefetch=2, token_tiles=4, x_chunk=256)),
     (4096, 32, 1024, dict(waves_m=16, waves_k=1, prefetch=4, token_tiles=2, x_chunk=512),
      dict(waves_m=8, waves_k=1, prefetch=4, token_tiles=2, x_chunk=512)),
+    # waves along k: summed through LDS in wave order, as in the general kernel
+    (1024, 32, 1024, dict(waves_m=4, waves_k=2, prefetch=2, token_tiles=2, x_chunk=256), None),
+    (1024, 33, 2048, dict(waves_m=2, waves_k=4, prefetch=2, token_tiles=4, x_chunk=256), None),
+    (768, 40, 1024, dict(waves_m=3, waves_k=2, prefetch=4, token_tiles=2, x_chunk=256), None),       # 6 waves, 3 token chunks
+    (512, 64, 4096, dict(waves_m=1, waves_k=8, prefetch=2, token_tiles=2, x_chunk=512), None),       # 8 waves along k
     # more row tiles than CUs: the workgroups walk (296 tiles of 256 rows), one chunk of x per tile
     (75776, 33, 256, dict(waves_m=4, waves_k=1, prefetch=2, token_tiles=4, x_chunk=128), None),
+    (37888, 20, 512, dict(waves_m=2, waves_k=2, prefetch=2, token_tiles=2, x_chunk=128), None),      # the same with a reduction per tile
 ]
 
 

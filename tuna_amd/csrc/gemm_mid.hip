@@ -36,11 +36,12 @@ static const MidVariant *mid_variant(const GemmPlan &plan, int *xc_out)
     const GemmArgs &a = plan.args;
     if (a.group_rows || a.balanced || plan.rw != 1 || plan.decode != TUNA_DECODE_GEMM) return nullptr;
     if (plan.token_tiles != 2 && plan.token_tiles != 4) return nullptr;
-    if (a.waves_k != 1 || a.split_k != 1 || a.k_stagger != 0) return nullptr;
+    if (a.split_k != 1 || a.k_stagger != 0 || a.waves_k > 16 || (a.waves_k & (a.waves_k - 1)) != 0) return nullptr;
     if (a.k != a.steps_total * kStepK || a.k >= (1 << 23)) return nullptr;
-    if (a.m % (a.waves_m * kRowsPerLoad) != 0 || a.waves_m > 16) return nullptr;
+    if (a.m % (a.waves_m * kRowsPerLoad) != 0 || a.waves_m * a.waves_k > 16) return nullptr;
     const int xc = mid_x_chunk(plan);
-    if (xc < plan.prefetch * kStepK || (xc & (xc - 1)) != 0 || a.k % xc != 0) return nullptr;
+    // a chunk is whole ring turns of the workgroup: xc / 32 steps, waves_k * prefetch per turn
+    if (xc < a.waves_k * plan.prefetch * kStepK || (xc & (xc - 1)) != 0 || a.k % xc != 0) return nullptr;
     const int pieces = plan.token_tiles * 2 * xc;  // 16-byte pieces per chunk
     const int per_thread = (pieces + plan.threads - 1) / plan.threads;
     if (per_thread > 8) return nullptr;
@@ -81,10 +82,12 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
     const GemmArgs &a = plan.args;
     int xc_log2 = 0;
     while ((1 << xc_log2) < xc) ++xc_log2;
-    const size_t lds = (size_t)kLutBytes + 2 * (size_t)plan.token_tiles * 32 * (size_t)xc;
+    const size_t x_lds = 2 * (size_t)plan.token_tiles * 32 * (size_t)xc;   // two buffers of one chunk
+    const size_t red_lds = 2 * (size_t)(plan.threads / 64) * 1024;         // two buffers of one plane per wave
+    const size_t lds = (size_t)kLutBytes + (x_lds > red_lds ? x_lds : red_lds);
     dim3 grid = plan.grid;
     grid.x = (unsigned)(a.row_tiles < cus ? a.row_tiles : cus);  // one workgroup per CU (LDS), walking row tiles
-    const int packed = a.waves_m | a.epilogue << 5 | xc_log2 << 8;
+    const int packed = a.waves_m | a.epilogue << 5 | xc_log2 << 8 | a.wk_log2 << 13;
     hipLaunchKernelGGL(v->fn, grid, dim3(plan.threads), lds, stream, a.q, a.x, a.code, a.absmax, a.k, a.n, a.m, packed, a.out,
                        a.residual, a.row_tiles, (int)grid.x);
     return hipGetLastError();

@@ -4,10 +4,11 @@
 // MFMAs and the launch sits between the bandwidth and the matrix-core bound: what counts is how
 // many weight loads a wave keeps in flight and how little else it does.  This kernel computes
 // exactly what gemm_kernel computes for one class of launches:
-//   * dense, no split of k at all (every wave owns 64 rows and walks the whole k range:
-//     waves_k = 1, split_k = 1), no stagger, m a multiple of the workgroup's rows, k a multiple
-//     of the x chunk, chunks of whole ring turns: no clamped or conditional weight loads, no
-//     tails, no cross-wave reduction (accumulators are final, stored from registers);
+//   * dense, no split of k across workgroups (split_k = 1), no stagger, m a multiple of the
+//     workgroup's rows, k a multiple of the x chunk, chunks of whole ring turns of the workgroup:
+//     no clamped or conditional weight loads, no tails; with all waves along m the accumulators
+//     are final and stored from registers, with waves along k they are summed through LDS in
+//     wave order as in gemm_kernel;
 //   * x chunks are double-buffered in LDS: chunk c + 1 is requested before chunk c is consumed
 //     and written to the other buffer after it, one barrier per chunk, and the weight ring runs
 //     on across chunk and tile boundaries' barriers without being emptied;
@@ -27,10 +28,12 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
                                                               void *a_out, const void *a_residual, int a_row_tiles,
                                                               int a_n_wg)
 {
-    // a_packed = waves_m | epilogue << 5 | log2(x chunk in k) << 8
+    // a_packed = waves_m | epilogue << 5 | log2(x chunk in k) << 8 | log2(waves_k) << 13
     const int waves_m = a_packed & 31;
     const int epilogue = (a_packed >> 5) & 7;
     const int xc_log2 = (a_packed >> 8) & 31;
+    const int wk_log2 = (a_packed >> 13) & 7;
+    const int waves_k = 1 << wk_log2;
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char *lut = smem;
     unsigned char *xbuf = smem + kLutBytes;  // two buffers of one x chunk: [slot][token tile][token][16 B]
@@ -39,12 +42,14 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     const int lane = tid & 63;
     const int i16 = lane & 15;
     const int g = lane >> 4;
-    const int wm = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nthreads = waves_m * 64;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wk = wave & (waves_k - 1);  // wave (wm, wk): rows 64*wm.., k-steps wk, wk + waves_k, ...
+    const int wm = wave >> wk_log2;
+    const int nthreads = (waves_m * 64) << wk_log2;
     const uint32_t lane4 = (uint32_t)lane << 2;
     const int tok0 = blockIdx.y * (16 * TT);
     const int xc = 1 << xc_log2;
-    const int chunk_steps = xc >> 5;                 // a multiple of U
+    const int chunk_its = (xc >> 5) >> wk_log2;      // k-steps of one wave per chunk, a multiple of U
     const int n_chunks = a_k >> xc_log2;
     const int n_steps = a_k >> 5;
     const uint32_t kb_total = (uint32_t)a_k >> 3;
@@ -65,8 +70,8 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     {                                                                                          \
         const int row0_ = (t) * (waves_m * 64) + wm * 64;                                      \
         lb = ((uint32_t)(row0_ >> 3) + (uint32_t)(i16 >> 1)) * kb_total * 32u + (uint32_t)(i16 & 1) * 16u + (uint32_t)g * 32u; \
-        _Pragma("unroll") for (int u = 0; u < U; ++u) wq[u] =                                  \
-            __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(a_q + (size_t)u * 128 + lb)); \
+        _Pragma("unroll") for (int u = 0; u < U; ++u) wq[u] = __builtin_nontemporal_load(      \
+            reinterpret_cast<const u32x4 *>(a_q + (size_t)(wk + (u << wk_log2)) * 128 + lb));  \
         _Pragma("unroll") for (int j = 0; j < 4; ++j) sc32[j] = a_absmax[row0_ + i16 * 4 + j];  \
         x_stage_load<TT, XB>(xst, xg, nthreads, tid, tok0, 0, a_n, a_k, krot);                 \
     }
@@ -96,29 +101,30 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     const f16 *resp = reinterpret_cast<const f16 *>(a_residual);
     // B fragment of lane (token i16, k-group g), local step sl, token tile tt:
     // slot sl*4 + g, byte slot*(256*TT) + tt*256 + i16*16
-    const uint32_t xb_lane = (uint32_t)g * (256 * TT) + (uint32_t)i16 * 16;
+    const uint32_t xb_lane = (uint32_t)g * (256 * TT) + (uint32_t)i16 * 16 + (uint32_t)wk * (1024 * TT);
+    const uint32_t wstep = (uint32_t)(1024 * TT) << wk_log2;  // LDS bytes between this wave's consecutive steps
 
-    // One ring turn: U k-steps, each consumed (B fragments from LDS, 4 fragments decoded, 4*TT
-    // MFMAs) and refilled with step + U of this tile (the last turn re-reads the last step: in
-    // bounds, never consumed).
+    // One ring turn: U of this wave's k-steps, each consumed (B fragments from LDS, 4 fragments
+    // decoded, 4*TT MFMAs) and refilled with the wave's step U iterations on (the last turn
+    // re-reads the tile's last step: in bounds, never consumed).
 #define TUNA_MID_GROUP(sl)                                                                      \
     {                                                                                          \
         _Pragma("unroll") for (int u = 0; u < U; ++u)                                          \
         {                                                                                      \
             f16x8 b_[TT];                                                                      \
             _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) b_[tt] =                         \
-                *reinterpret_cast<const f16x8 *>(xb + (size_t)((sl) + u) * (1024 * TT) + tt * 256); \
+                *reinterpret_cast<const f16x8 *>(xb + (size_t)((sl) + u) * wstep + tt * 256);  \
             _Pragma("unroll") for (int j = 0; j < 4; ++j)                                      \
             {                                                                                  \
                 const f16x8 av_ = decode_dword<TUNA_DECODE_GEMM>(wq[u][j], lut, lane4, sc16[j], 0.f); \
                 _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) acc[j][tt] =                 \
                     __builtin_amdgcn_mfma_f32_16x16x32_f16(av_, b_[tt], acc[j][tt], 0, 0, 0);  \
             }                                                                                  \
-            const int s_ = min(step + u + U, n_steps - 1);                                     \
+            const int s_ = min(wk + ((it + u + U) << wk_log2), n_steps - 1);                   \
             wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(qrow + (size_t)s_ * 128)); \
             __builtin_amdgcn_sched_barrier(0); /* keep each refill right behind its consume */ \
         }                                                                                      \
-        step += U;                                                                             \
+        it += U;                                                                               \
     }
 
     while (tile < a_row_tiles) {
@@ -142,7 +148,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
         __syncthreads();
 
         const unsigned char *qrow = a_q + lb;
-        int step = 0;  // this wave's next k-step
+        int it = 0;  // this wave's next iteration (its k-step wk + it*waves_k)
         for (int c = 0; c < n_chunks; ++c) {
             const bool has_next = c + 1 < n_chunks;
             // (unconditional - the last chunk requests itself again and drops it: behind a branch
@@ -153,7 +159,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
             // requested are in flight behind the ring, and only straight-line code lets the
             // compiler count them into its waits instead of waiting them out)
             TUNA_MID_GROUP(0)
-            for (int sl = U; sl < chunk_steps; sl += U) TUNA_MID_GROUP(sl)
+            for (int sl = U; sl < chunk_its; sl += U) TUNA_MID_GROUP(sl)
             if (has_next) {
                 // the other buffer was last read in chunk c - 1, which ended with a barrier
                 __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));  // exactly the last ring turn's refills are younger
@@ -167,6 +173,38 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
         const int cur_row0 = row0;
         tile += a_n_wg;
         if (tile < a_row_tiles) TUNA_MID_TILE_FETCH(tile)
+        if (wk_log2 != 0) {
+            // Waves along k: every wave puts its copy of a plane (one float4 per lane) in LDS - two
+            // buffers alternate in the x area, free since the barrier that ended the last chunk -
+            // and thread (wk, lane) sums floats f = (i*waves_k + wk)*64 + lane of it in wave order:
+            // float f = l*4 + v of plane j is token l%16, weight row 16*(l/16) + 4*v + j of the wave's
+            // 64, so after the four planes a thread owns 4 consecutive features of one token.
+            float *redf = reinterpret_cast<float *>(xbuf);
+            const size_t plane_floats = (size_t)(waves_m << wk_log2) * 256;
+#pragma unroll
+            for (int tt = 0; tt < TT; ++tt) {
+                float o[4][4];  // [i][j]
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float *buf = redf + (size_t)((tt * 4 + j) & 1) * plane_floats;
+                    reinterpret_cast<f32x4 *>(buf)[(size_t)wave * 64 + lane] = acc[j][tt];
+                    __syncthreads();
+                    sum_planes_any<1, 32>(wk_log2, buf, plane_floats, wm, wk, lane, o, j);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int f = ((i << wk_log2) + wk) * 64 + lane;
+                    if (f >= 256) continue;
+                    const int l = f >> 2, v = f & 3;
+                    const int tok = tok0 + tt * 16 + (l & 15);
+                    if (tok < a_n)
+                        store_features4(outp, resp, epilogue, (size_t)tok, a_m, cur_row0 + (l >> 4) * 16 + v * 4, o[i][0], o[i][1],
+                                        o[i][2], o[i][3]);
+                }
+            }
+            __syncthreads();  // the x area is written again at the top of the next tile
+            continue;
+        }
         // Lane (token i16, group g) owns 16 consecutive output features, acc[j][tt][v] being
         // feature 4*v + j of them: two 16-byte stores per token tile.
 #pragma unroll

@@ -146,18 +146,18 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
 def mid_applies(m: int, k: int, c: dict) -> bool:
     """True if a dense launch of this config is taken by the 17..64-token streaming kernel
     (mirrors mid_variant in csrc/gemm_mid.hip)."""
-    tt, wm = c["token_tiles"], c["waves_m"]
-    if c["rows_per_wave"] != 64 or tt not in (2, 4) or c["waves_k"] != 1 or c["split_k"] != 1 or c["k_stagger"] != 0:
+    tt, wm, wk = c["token_tiles"], c["waves_m"], c["waves_k"]
+    if c["rows_per_wave"] != 64 or tt not in (2, 4) or c["split_k"] != 1 or c["k_stagger"] != 0:
         return False
-    if k % STEP_K or k >= 1 << 23 or wm > 16 or m % (64 * wm):
+    if k % STEP_K or k >= 1 << 23 or not _pow2(wk) or wm < 1 or wm * wk > 16 or m % (64 * wm):
         return False
     xc = c["x_chunk"]
     cap = (LDS_LIMIT - LUT_BYTES) // (2 * tt * 32)
     while xc > cap:
         xc //= 2
-    if xc < c["prefetch"] * STEP_K or k % xc:
+    if xc < wk * c["prefetch"] * STEP_K or k % xc:
         return False
-    threads = 64 * wm
+    threads = 64 * wm * wk
     per_thread = -(-(tt * 2 * xc) // threads)
     if per_thread > 8:
         return False

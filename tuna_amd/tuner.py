@@ -167,27 +167,28 @@ def lean_space(m: int, n_key: int, k: int):
 
 def mid_space(m: int, n_key: int, k: int):
     """Every config whose launch takes the 17..64-token streaming kernel (gemm_mid.hpp; the
-    conditions of mid_variant in gemm_mid.hip): 64 rows per wave, all waves along m, no split,
+    conditions of mid_variant in gemm_mid.hip): 64 rows per wave, no split across workgroups,
     no stagger, two or four token tiles.  Small enough to time exhaustively."""
     lo, hi = make_configs.N_BUCKETS[n_key]
     if lo < 17 or lo > 64:
         return []
     out = []
     for tt in ((2,) if hi <= 32 else (4,) if lo > 32 else (2, 4)):
-        for wm in range(2, 17):
-            if m % (64 * wm):
-                continue
-            for pf in (2, 4, 8):
-                for xc in (128, 256, 512, 1024):
-                    for sw in (0, 1):
-                        c = dict(rows_per_wave=64, waves_m=wm, waves_k=1, split_k=1, prefetch=pf, x_chunk=xc, token_tiles=tt,
-                                 xcd_swizzle=sw, k_stagger=0, lds_tile_rows=0)
-                        try:
-                            make_configs.validate(m, n_key, k, c)
-                        except ValueError:
-                            continue
-                        if make_configs.mid_applies(m, k, c):
-                            out.append(c)
+        for wm in range(1, 17):
+            for wk in (1, 2, 4, 8):
+                if m % (64 * wm) or wm * wk > 16 or wm * wk < 4:
+                    continue
+                for pf in (2, 4, 8):
+                    for xc in (128, 256, 512, 1024):
+                        for sw in (0, 1):
+                            c = dict(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=1, prefetch=pf, x_chunk=xc,
+                                     token_tiles=tt, xcd_swizzle=sw, k_stagger=0, lds_tile_rows=0)
+                            try:
+                                make_configs.validate(m, n_key, k, c)
+                            except ValueError:
+                                continue
+                            if make_configs.mid_applies(m, k, c):
+                                out.append(c)
     return out
 
 
