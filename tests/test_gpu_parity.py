@@ -687,7 +687,7 @@ def test_lean_kernel_equals_general_kernel_bit_for_bit(ci):
     assert rel_err(outs[True][0].cpu().numpy().astype(np.float64), ref) <= REL_TOL
 
 
-# ----------------------------------------------------------------------------- 17..64-token streaming kernel
+# ----------------------------------------------------------------------------- 17..128-token streaming kernel
 MID_CASES = [
     # m, n, k, config of the launch, config of the general-kernel launch it is compared with (None: the same)
     (512, 32, 512, dict(waves_m=8, waves_k=1, prefetch=2, token_tiles=2, x_chunk=256), None),
@@ -701,6 +701,11 @@ MID_CASES = [
      dict(waves_m=8, waves_k=1, prefetch=2, token_tiles=4, x_chunk=256)),
     (4096, 32, 1024, dict(waves_m=16, waves_k=1, prefetch=4, token_tiles=2, x_chunk=512),
      dict(waves_m=8, waves_k=1, prefetch=4, token_tiles=2, x_chunk=512)),
+    # eight token tiles (128 tokens per pass): a token's sums do not depend on the tile count
+    (1024, 128, 1024, dict(waves_m=8, waves_k=1, prefetch=2, token_tiles=8, x_chunk=128),
+     dict(waves_m=8, waves_k=1, prefetch=2, token_tiles=4, x_chunk=128)),
+    (768, 200, 512, dict(waves_m=4, waves_k=2, prefetch=2, token_tiles=8, x_chunk=128),
+     dict(waves_m=4, waves_k=2, prefetch=2, token_tiles=4, x_chunk=128)),                            # two passes, ragged
     # waves along k: summed through LDS in wave order, as in the general kernel
     (1024, 32, 1024, dict(waves_m=4, waves_k=2, prefetch=2, token_tiles=2, x_chunk=256), None),
     (1024, 33, 2048, dict(waves_m=2, waves_k=4, prefetch=2, token_tiles=4, x_chunk=256), None),
@@ -714,7 +719,7 @@ MID_CASES = [
 
 @pytest.mark.parametrize("ci", range(len(MID_CASES)))
 def test_mid_token_kernel_equals_general_kernel_bit_for_bit(ci):
-    """Dense unsplit launches with two or four token tiles take the 17..64-token streaming kernel;
+    """Dense unsplit launches with two or four token tiles take the 17..128-token streaming kernel;
     it must give the bits of the general kernel (same decode, same summation order), for the plain
     store and both fused epilogues, and be within tolerance of the oracle."""
     import torch

@@ -185,7 +185,7 @@ def test_tuner_small_launch_config_spaces_are_valid_for_both_validators():
         mc.validate(256, 32, 5120, big)
     with pytest.raises(ops.TunaError):
         ops.validate_config(256, 32, 5120, ops.GemmConfig.from_dict(big))
-    # configs only the 17..64-token streaming kernel has (ring 8 with four token tiles, 16 waves with two): valid
+    # configs only the 17..128-token streaming kernel has (ring 8 with four token tiles, 16 waves with two): valid
     # for both validators while the launch qualifies, refused by both when it does not (waves along k)
     mid = dict(rows_per_wave=64, waves_m=8, waves_k=1, split_k=1, prefetch=8, x_chunk=256, token_tiles=4, xcd_swizzle=0,
                k_stagger=0, lds_tile_rows=0)

@@ -71,8 +71,8 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
         return fail(TUNA_ERR_UNSUPPORTED, "rows_per_wave=%d (64, 128 or 256)", c.rows_per_wave);
     if (c.prefetch != 2 && c.prefetch != 4 && c.prefetch != 8)
         return fail(TUNA_ERR_UNSUPPORTED, "prefetch=%d (2, 4 or 8)", c.prefetch);
-    if (c.token_tiles != 1 && c.token_tiles != 2 && c.token_tiles != 4)
-        return fail(TUNA_ERR_UNSUPPORTED, "token_tiles=%d (1, 2 or 4)", c.token_tiles);
+    if (c.token_tiles != 1 && c.token_tiles != 2 && c.token_tiles != 4 && c.token_tiles != 8)
+        return fail(TUNA_ERR_UNSUPPORTED, "token_tiles=%d (1, 2, 4 or 8)", c.token_tiles);
     if (c.waves_m < 1 || !is_pow2(c.waves_k) || c.waves_m * c.waves_k * 64 > kMaxThreads)
         return fail(TUNA_ERR_UNSUPPORTED, "waves_m=%d must be at least 1 and waves_k=%d a power of two, with at most 16 waves",
                     c.waves_m, c.waves_k);

@@ -1,4 +1,4 @@
-// Instantiations and launcher of the 17..64-token streaming kernel (gemm_mid.hpp).
+// Instantiations and launcher of the 17..128-token streaming kernel (gemm_mid.hpp).
 #include <mutex>
 
 #include "gemm_mid.hpp"
@@ -16,6 +16,7 @@ struct MidVariant {
 static const MidVariant kMid[] = {
     M5(2, 2, 4), M5(4, 2, 4), M5(8, 2, 4), M5(2, 2, 8), M5(4, 2, 8), M5(8, 2, 8),
     M5(2, 4, 4), M5(4, 4, 4), M5(8, 4, 4), M5(2, 4, 8), M5(4, 4, 8), M5(8, 4, 8),
+    M5(2, 8, 4), M5(2, 8, 8),  // (deeper rings with eight token tiles spill inside the loop)
     M10(2, 2, 4), M10(4, 2, 4),
 };
 #undef M5
@@ -35,7 +36,7 @@ static const MidVariant *mid_variant(const GemmPlan &plan, int *xc_out)
 {
     const GemmArgs &a = plan.args;
     if (a.group_rows || a.balanced || plan.rw != 1 || plan.decode != TUNA_DECODE_GEMM) return nullptr;
-    if (plan.token_tiles != 2 && plan.token_tiles != 4) return nullptr;
+    if (plan.token_tiles != 2 && plan.token_tiles != 4 && plan.token_tiles != 8) return nullptr;
     if (a.split_k != 1 || a.k_stagger != 0 || a.waves_k > 16 || (a.waves_k & (a.waves_k - 1)) != 0) return nullptr;
     if (a.k != a.steps_total * kStepK || a.k >= (1 << 23)) return nullptr;
     if (a.m % (a.waves_m * kRowsPerLoad) != 0 || a.waves_m * a.waves_k > 16) return nullptr;

@@ -1,6 +1,6 @@
-// Streaming GEMM kernel for 17..64 tokens per pass on shapes with many rows (gfx950, wave64).
+// Streaming GEMM kernel for 17..128 tokens per pass on shapes with many rows (gfx950, wave64).
 //
-// With two or four 16-token tiles per wave every decoded weight fragment feeds two or four
+// With two, four or eight 16-token tiles per wave every decoded weight fragment feeds as many
 // MFMAs and the launch sits between the bandwidth and the matrix-core bound: what counts is how
 // many weight loads a wave keeps in flight and how little else it does.  This kernel computes
 // exactly what gemm_kernel computes for one class of launches:

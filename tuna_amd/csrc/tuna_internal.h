@@ -148,7 +148,7 @@ struct GemmPlan {
 
 // gemm_kernel.hip
 hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream);
-// 17..64-token streaming twin of the general kernel (gemm_mid.hpp) for the launches it applies to.
+// 17..128-token streaming twin of the general kernel (gemm_mid.hpp) for the launches it applies to.
 bool mid_applies(const GemmPlan &plan);
 hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t stream);
 // Narrow-row kernel (gemm_narrow.hpp): 16 or 32 rows per workgroup, all waves along k.

@@ -50,10 +50,10 @@ VARIANTS_512_2WG = {(1, 2, 1), (1, 4, 1)}
 VARIANTS_1024 = {(1, 2, 1), (1, 4, 1)}
 
 
-# (prefetch, token_tiles, x pieces per thread, max threads) of the 17..64-token streaming kernel; must match
+# (prefetch, token_tiles, x pieces per thread, max threads) of the 17..128-token streaming kernel; must match
 # kMid in csrc/gemm_mid.hip
 MID_VARIANTS = ({(u, tt, xb, 512) for u in (2, 4, 8) for tt in (2, 4) for xb in (4, 8)}
-                | {(2, 2, 4, 1024), (4, 2, 4, 1024)})
+                | {(2, 8, 4, 512), (2, 8, 8, 512), (2, 2, 4, 1024), (4, 2, 4, 1024)})
 
 # (rows, waves_k, prefetch, token_tiles) of the narrow-row kernel; must match kNarrow in csrc/gemm_launch.hip
 NARROW_VARIANTS = (
@@ -117,8 +117,8 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
         raise ValueError("rows_per_wave must be 16, 32 (narrow-row kernel), 64, 128 or 256")
     if c["prefetch"] not in (2, 4, 8):
         raise ValueError("prefetch must be 2, 4 or 8")
-    if c["token_tiles"] not in (1, 2, 4):
-        raise ValueError("token_tiles must be 1, 2 or 4")
+    if c["token_tiles"] not in (1, 2, 4, 8):
+        raise ValueError("token_tiles must be 1, 2, 4 or 8")
     wm, wk = c["waves_m"], c["waves_k"]
     if wm < 1 or not _pow2(wk) or wm * wk > 16:
         raise ValueError("waves_m must be >= 1 and waves_k a power of two, with waves_m * waves_k <= 16")
@@ -144,10 +144,10 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
 
 
 def mid_applies(m: int, k: int, c: dict) -> bool:
-    """True if a dense launch of this config is taken by the 17..64-token streaming kernel
+    """True if a dense launch of this config is taken by the 17..128-token streaming kernel
     (mirrors mid_variant in csrc/gemm_mid.hip)."""
     tt, wm, wk = c["token_tiles"], c["waves_m"], c["waves_k"]
-    if c["rows_per_wave"] != 64 or tt not in (2, 4) or c["split_k"] != 1 or c["k_stagger"] != 0:
+    if c["rows_per_wave"] != 64 or tt not in (2, 4, 8) or c["split_k"] != 1 or c["k_stagger"] != 0:
         return False
     if k % STEP_K or k >= 1 << 23 or not _pow2(wk) or wm < 1 or wm * wk > 16 or m % (64 * wm):
         return False

@@ -166,14 +166,14 @@ def lean_space(m: int, n_key: int, k: int):
 
 
 def mid_space(m: int, n_key: int, k: int):
-    """Every config whose launch takes the 17..64-token streaming kernel (gemm_mid.hpp; the
+    """Every config whose launch takes the 17..128-token streaming kernel (gemm_mid.hpp; the
     conditions of mid_variant in gemm_mid.hip): 64 rows per wave, no split across workgroups,
-    no stagger, two or four token tiles.  Small enough to time exhaustively."""
+    no stagger, two, four or eight token tiles.  Small enough to time exhaustively."""
     lo, hi = make_configs.N_BUCKETS[n_key]
-    if lo < 17 or lo > 64:
+    if lo < 17 or lo > 128:
         return []
     out = []
-    for tt in ((2,) if hi <= 32 else (4,) if lo > 32 else (2, 4)):
+    for tt in ((2,) if hi <= 32 else (4,) if hi <= 64 else (8,)):
         for wm in range(1, 17):
             for wk in (1, 2, 4, 8):
                 if m % (64 * wm) or wm * wk > 16 or wm * wk < 4:
