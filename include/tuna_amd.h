@@ -206,14 +206,18 @@ int tuna_time_copy(const void *src, void *dst, size_t bytes, int warmup, int ite
 int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int warmup, int iters,
                    void *stream, float *elapsed_ms);
 
-/* Diagnostic switch, process-wide, default on: small dense launches that qualify (one
- * workgroup per tile, power-of-two split, aligned shapes, up to 16 tokens per tile) run a
- * kernel stripped of everything else the general one carries.  Both compute bit-identical
- * results; turning it off is for A/B timing and for the test that checks exactly that.
- * Returns the previous setting.  No counterpart in the reference. */
+/* Diagnostic switch, process-wide, default on: dense launches that qualify run one of two
+ * kernels stripped of everything else the general one carries - small launches (one workgroup
+ * per tile, power-of-two split, aligned shapes, up to 16 tokens per tile) and launches with 2, 4
+ * or 8 token tiles and no split of k across workgroups (x chunks double-buffered in LDS).  Both
+ * compute the general kernel's results bit for bit; turning them off is for A/B timing and for
+ * the tests that check exactly that.  A config whose ring depth or token tile count only the
+ * second kernel has (prefetch 4 or 8 with 4 token tiles, 8 token tiles, 16 waves with 2 or more
+ * token tiles) runs it regardless of the switch.  Returns the previous setting.  No counterpart
+ * in the reference. */
 int tuna_set_lean_kernels(int enabled);
 
-/* Diagnostic: how many GEMM launches of this process took that kernel so far. */
+/* Diagnostic: how many GEMM launches of this process took one of those kernels so far. */
 unsigned long long tuna_lean_launches(void);
 
 /* Releases the library-owned split-K workspaces of the current device (synchronises
