@@ -55,8 +55,40 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     const uint32_t kb_total = (uint32_t)a_k >> 3;
     const uint32_t xbuf_bytes = (uint32_t)(TT * 32) << xc_log2;  // 16*TT tokens x xc k x 2 bytes
     const int x_pieces = (int)(xbuf_bytes >> 4);
-    const f16 *xg = reinterpret_cast<const f16 *>(a_x);
-    const KRot krot{0, a_k, a_k};
+    // x staging, global -> registers -> LDS: piece p = tid + b*nthreads of a chunk is (as in
+    // gemm_kernel.hpp) token row (p/64 % TT)*16 + lane/4, k-step p/64 / TT, 8-k group lane%4 - every
+    // quad of lanes reads 64 contiguous bytes of one token row, a wave instruction writes one k-step
+    // of one token tile.  Nothing of it depends on the chunk, so the byte offsets are formed once
+    // and a chunk costs XB loads with a uniform base plus XB LDS writes (there are registers to
+    // spare here; the general kernel recomputes them per chunk to save some).
+    uint32_t x_goff[XB], x_loff[XB];
+    uint32_t x_inchunk = 0, x_real = 0;  // bit b: piece b exists in a chunk / its token row exists
+    {
+        const int row_l = lane >> 2, grp = lane & 3;
+#pragma unroll
+        for (int b = 0; b < XB; ++b) {
+            const int p = tid + b * nthreads;
+            const int wv = p >> 6;
+            const int row = (wv % TT) * 16 + row_l, ks = wv / TT;
+            const bool in = p < x_pieces;
+            x_goff[b] = in ? ((uint32_t)min(row, a_n - 1 - tok0) * (uint32_t)a_k + (uint32_t)(ks * 32 + grp * 8)) * 2u : 0u;
+            x_loff[b] = (uint32_t)((ks * 4 + grp) * (256 * TT) + row * 16);
+            x_inchunk |= in ? 1u << b : 0u;
+            x_real |= (in && tok0 + row < a_n) ? 1u << b : 0u;
+        }
+    }
+    const unsigned char *x_tile = reinterpret_cast<const unsigned char *>(a_x) + (size_t)tok0 * a_k * 2;
+#define TUNA_MID_X_LOAD(kbase)                                                                  \
+    {                                                                                          \
+        const unsigned char *xc_ = x_tile + (size_t)(kbase) * 2;                               \
+        _Pragma("unroll") for (int b = 0; b < XB; ++b) xst.v[b] = *reinterpret_cast<const u32x4 *>(xc_ + x_goff[b]); \
+    }
+    // (rows past n are zeroed, as the general kernel does)
+#define TUNA_MID_X_STORE(buf)                                                                   \
+    {                                                                                          \
+        _Pragma("unroll") for (int b = 0; b < XB; ++b) if (x_inchunk >> b & 1u)                \
+            *reinterpret_cast<u32x4 *>((buf) + x_loff[b]) = (x_real >> b & 1u) ? xst.v[b] : u32x4{0u, 0u, 0u, 0u}; \
+    }
 
     const float code_lane = a_code[i16];
     int tile = blockIdx.x;
@@ -73,7 +105,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
         _Pragma("unroll") for (int u = 0; u < U; ++u) wq[u] = __builtin_nontemporal_load(      \
             reinterpret_cast<const u32x4 *>(a_q + (size_t)(wk + (u << wk_log2)) * 128 + lb));  \
         _Pragma("unroll") for (int j = 0; j < 4; ++j) sc32[j] = a_absmax[row0_ + i16 * 4 + j];  \
-        x_stage_load<TT, XB>(xst, xg, nthreads, tid, tok0, 0, a_n, a_k, krot);                 \
+        TUNA_MID_X_LOAD(0)                                                                     \
     }
     if (tile < a_row_tiles) TUNA_MID_TILE_FETCH(tile)
 
@@ -143,7 +175,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
 
         // chunk 0 of x into buffer 0 (every wave has left the previous tile's last chunk: the
         // barrier that ends a chunk), then the table and the chunk are published together
-        x_stage_store<TT, XB>(xst, xbuf, nthreads, tid, x_pieces, tok0, 0, a_n, a_k, krot);
+        TUNA_MID_X_STORE(xbuf)
         __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));  // (threads without a piece: see gemm_kernel.hpp)
         __syncthreads();
 
@@ -153,7 +185,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
             const bool has_next = c + 1 < n_chunks;
             // (unconditional - the last chunk requests itself again and drops it: behind a branch
             // the compiler could not count these loads into the waits of the first ring turn)
-            x_stage_load<TT, XB>(xst, xg, nthreads, tid, tok0, min(c + 1, n_chunks - 1) << xc_log2, a_n, a_k, krot);
+            TUNA_MID_X_LOAD(min(c + 1, n_chunks - 1) << xc_log2)
             const unsigned char *xb = xbuf + (c & 1) * xbuf_bytes + xb_lane;
             // (the first ring turn of a chunk is a copy of its own: there the x pieces just
             // requested are in flight behind the ring, and only straight-line code lets the
@@ -163,8 +195,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
             if (has_next) {
                 // the other buffer was last read in chunk c - 1, which ended with a barrier
                 __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));  // exactly the last ring turn's refills are younger
-                x_stage_store<TT, XB>(xst, xbuf + ((c + 1) & 1) * xbuf_bytes, nthreads, tid, x_pieces, tok0, (c + 1) << xc_log2,
-                                      a_n, a_k, krot);
+                TUNA_MID_X_STORE(xbuf + ((c + 1) & 1) * xbuf_bytes)
             }
             __syncthreads();
         }
@@ -233,6 +264,8 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
         }
     }
 #undef TUNA_MID_GROUP
+#undef TUNA_MID_X_LOAD
+#undef TUNA_MID_X_STORE
 #undef TUNA_MID_TILE_FETCH
 }
 
