@@ -173,7 +173,7 @@ def mid_space(m: int, n_key: int, k: int):
     if lo < 17 or lo > 128:
         return []
     out = []
-    for tt in ((2,) if hi <= 32 else (4,) if hi <= 64 else (8,)):
+    for tt in ((2,) if lo <= 32 else (4,) if lo <= 64 else (8,)):   # configs are tuned at the bucket's lower edge
         for wm in range(1, 17):
             for wk in (1, 2, 4, 8):
                 if m % (64 * wm) or wm * wk > 16 or wm * wk < 4:
