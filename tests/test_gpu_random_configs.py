@@ -1,7 +1,7 @@
-"""Seeded random launch configurations of the three streaming kernel families against the oracle.
+"""Seeded random launch configurations of the streaming kernel families against the oracle.
 
 Every case draws a shape, a token count and a config from the same spaces the tuner searches
-(narrow-row variants, lean-kernel layouts, the general kernel's seed pool), keeps it only if the Python
+(narrow-row variants, lean-kernel layouts, the general kernel's seed pool, the 17..128-token streaming kernel), keeps it only if the Python
 validator accepts it, and runs it through the C-ABI. A config the Python validator accepts but the library
 cannot launch, or a launch that differs from the oracle beyond the GEMM tolerance, fails the test.
 Output layout and rounding follow kernel.cu:2649-2754 (fp32 accumulate, one fp16 rounding).
@@ -22,9 +22,21 @@ TOKENS = [1, 2, 3, 4, 5, 7, 8, 15, 16, 17, 31, 32, 33, 48, 63, 64, 65, 100]
 
 
 def draw(rng):
-    kind = rng.choice(["narrow", "lean", "general"])
+    kind = rng.choice(["narrow", "lean", "general", "mid"])
     n = rng.choice(TOKENS)
     bucket = mc.bucket_of(n)
+    if kind == "mid":
+        wm, wk = rng.randint(1, 8), rng.choice([1, 2, 4])
+        xc = rng.choice([128, 256, 512])
+        c = dict(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=1, prefetch=rng.choice([2, 4, 8]), x_chunk=xc,
+                 token_tiles=rng.choice([2, 4, 8]), xcd_swizzle=rng.choice([0, 1]), k_stagger=0, lds_tile_rows=0)
+        m, k = 64 * wm * rng.randint(1, 6), xc * rng.randint(1, 4)
+        n = rng.choice([17, 20, 32, 33, 50, 64, 65, 100, 128, 130, 200])
+        try:
+            mc.validate(m, mc.bucket_of(n), k, c)
+        except ValueError:
+            return None
+        return (kind, m, n, k, c) if mc.mid_applies(m, k, c) else None
     if kind == "narrow":
         rows, wk, pf, tt = rng.choice(sorted(mc.NARROW_VARIANTS))
         m = rows * rng.randint(1, 12)
@@ -59,8 +71,8 @@ def draw(rng):
 @pytest.mark.parametrize("seed", [11, 12, 13])
 def test_random_configs_match_oracle(seed):
     rng = random.Random(seed)
-    ran = {"narrow": 0, "lean": 0, "general": 0}
-    for case in range(45):
+    ran = {"narrow": 0, "lean": 0, "general": 0, "mid": 0}
+    for case in range(60):
         drawn = draw(rng)
         if drawn is None:
             continue
