@@ -701,6 +701,9 @@ MID_CASES = [
      dict(waves_m=8, waves_k=1, prefetch=2, token_tiles=4, x_chunk=256)),
     (4096, 32, 1024, dict(waves_m=16, waves_k=1, prefetch=4, token_tiles=2, x_chunk=512),
      dict(waves_m=8, waves_k=1, prefetch=4, token_tiles=2, x_chunk=512)),
+    # one token tile (large shapes at up to 16 tokens; launches the lean kernel does not take: several tiles per CU)
+    (33280, 16, 1024, dict(waves_m=2, waves_k=4, prefetch=2, token_tiles=1, x_chunk=1024), None),
+    (38400, 9, 512, dict(waves_m=1, waves_k=1, prefetch=8, token_tiles=1, x_chunk=256), None),
     # eight token tiles (128 tokens per pass): a token's sums do not depend on the tile count
     (1024, 128, 1024, dict(waves_m=8, waves_k=1, prefetch=2, token_tiles=8, x_chunk=128),
      dict(waves_m=8, waves_k=1, prefetch=2, token_tiles=4, x_chunk=128)),

@@ -201,7 +201,9 @@ def test_tuner_small_launch_config_spaces_are_valid_for_both_validators():
             with pytest.raises(ops.TunaError):
                 ops.validate_config(229376, 64, 4096, ops.GemmConfig.from_dict(c))
     space = tuner.mid_space(229376, 64, 4096)
-    assert space and all(mc.mid_applies(229376, 4096, c) for c in space) and tuner.mid_space(229376, 16, 4096) == []
+    assert space and all(mc.mid_applies(229376, 4096, c) for c in space)
+    # one token tile: offered only where unsplit tiles fill the device (small shapes take the lean or narrow-row kernel)
+    assert tuner.mid_space(229376, 16, 4096) and tuner.mid_space(4096, 16, 4096) == [] and tuner.mid_space(4096, 256, 4096) == []
     assert tuner.narrow_space(4096, 128, 4096) == [] and tuner.lean_space(4096, 128, 4096) == []
     assert tuner.lean_space(4096, 16, 4104) == []       # k not a multiple of 32: no lean launch
 

@@ -18,6 +18,8 @@ static const MidVariant kMid[] = {
     M5(2, 4, 4), M5(4, 4, 4), M5(8, 4, 4), M5(2, 4, 8), M5(4, 4, 8), M5(8, 4, 8),
     M5(2, 8, 4), M5(2, 8, 8),  // (deeper rings with eight token tiles spill inside the loop)
     M10(2, 2, 4), M10(4, 2, 4),
+    // one token tile: the large shapes at up to 16 tokens (small launches take gemm_lean.hpp first)
+    M5(2, 1, 4), M5(4, 1, 4), M5(8, 1, 4), M5(2, 1, 8), M5(4, 1, 8), M5(8, 1, 8), M10(2, 1, 4), M10(4, 1, 4), M10(8, 1, 4),
 };
 #undef M5
 #undef M10
@@ -36,7 +38,7 @@ static const MidVariant *mid_variant(const GemmPlan &plan, int *xc_out)
 {
     const GemmArgs &a = plan.args;
     if (a.group_rows || a.balanced || plan.rw != 1 || plan.decode != TUNA_DECODE_GEMM) return nullptr;
-    if (plan.token_tiles != 2 && plan.token_tiles != 4 && plan.token_tiles != 8) return nullptr;
+    if (plan.token_tiles != 1 && plan.token_tiles != 2 && plan.token_tiles != 4 && plan.token_tiles != 8) return nullptr;
     if (a.split_k != 1 || a.k_stagger != 0 || a.waves_k > 16 || (a.waves_k & (a.waves_k - 1)) != 0) return nullptr;
     if (a.k != a.steps_total * kStepK || a.k >= (1 << 23)) return nullptr;
     if (a.m % (a.waves_m * kRowsPerLoad) != 0 || a.waves_m * a.waves_k > 16) return nullptr;

@@ -1,9 +1,10 @@
-// Streaming GEMM kernel for 17..128 tokens per pass on shapes with many rows (gfx950, wave64).
+// Streaming GEMM kernel for shapes with many rows, up to 128 tokens per pass (gfx950, wave64).
 //
 // With two, four or eight 16-token tiles per wave every decoded weight fragment feeds as many
 // MFMAs and the launch sits between the bandwidth and the matrix-core bound: what counts is how
-// many weight loads a wave keeps in flight and how little else it does.  This kernel computes
-// exactly what gemm_kernel computes for one class of launches:
+// many weight loads a wave keeps in flight and how little else it does.  (With one token tile it
+// is the general kernel without a split across workgroups, a tile walk to pay for or a stagger.)
+// This kernel computes exactly what gemm_kernel computes for one class of launches:
 //   * dense, no split of k across workgroups (split_k = 1), no stagger, m a multiple of the
 //     workgroup's rows, k a multiple of the x chunk, chunks of whole ring turns of the workgroup:
 //     no clamped or conditional weight loads, no tails; with all waves along m the accumulators

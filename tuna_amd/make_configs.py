@@ -53,7 +53,8 @@ VARIANTS_1024 = {(1, 2, 1), (1, 4, 1)}
 # (prefetch, token_tiles, x pieces per thread, max threads) of the 17..128-token streaming kernel; must match
 # kMid in csrc/gemm_mid.hip
 MID_VARIANTS = ({(u, tt, xb, 512) for u in (2, 4, 8) for tt in (2, 4) for xb in (4, 8)}
-                | {(2, 8, 4, 512), (2, 8, 8, 512), (2, 2, 4, 1024), (4, 2, 4, 1024)})
+                | {(2, 8, 4, 512), (2, 8, 8, 512), (2, 2, 4, 1024), (4, 2, 4, 1024)}
+                | {(u, 1, xb, 512) for u in (2, 4, 8) for xb in (4, 8)} | {(u, 1, 4, 1024) for u in (2, 4, 8)})
 
 # (rows, waves_k, prefetch, token_tiles) of the narrow-row kernel; must match kNarrow in csrc/gemm_launch.hip
 NARROW_VARIANTS = (
@@ -147,7 +148,7 @@ def mid_applies(m: int, k: int, c: dict) -> bool:
     """True if a dense launch of this config is taken by the 17..128-token streaming kernel
     (mirrors mid_variant in csrc/gemm_mid.hip)."""
     tt, wm, wk = c["token_tiles"], c["waves_m"], c["waves_k"]
-    if c["rows_per_wave"] != 64 or tt not in (2, 4, 8) or c["split_k"] != 1 or c["k_stagger"] != 0:
+    if c["rows_per_wave"] != 64 or tt not in (1, 2, 4, 8) or c["split_k"] != 1 or c["k_stagger"] != 0:
         return False
     if k % STEP_K or k >= 1 << 23 or not _pow2(wk) or wm < 1 or wm * wk > 16 or m % (64 * wm):
         return False

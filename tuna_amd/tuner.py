@@ -170,16 +170,18 @@ def mid_space(m: int, n_key: int, k: int):
     conditions of mid_variant in gemm_mid.hip): 64 rows per wave, no split across workgroups,
     no stagger, two, four or eight token tiles.  Small enough to time exhaustively."""
     lo, hi = make_configs.N_BUCKETS[n_key]
-    if lo < 17 or lo > 128:
+    if lo > 128:
         return []
     out = []
-    for tt in ((2,) if lo <= 32 else (4,) if lo <= 64 else (8,)):   # configs are tuned at the bucket's lower edge
+    for tt in ((1,) if lo <= 16 else (2,) if lo <= 32 else (4,) if lo <= 64 else (8,)):   # tuned at the bucket's lower edge
         for wm in range(1, 17):
             for wk in (1, 2, 4, 8):
                 if m % (64 * wm) or wm * wk > 16 or wm * wk < 4:
                     continue
+                if tt == 1 and (m // (64 * wm) < 100 or wm * wk < 8):
+                    continue        # one token tile: only launches that fill the device unsplit (others: lean, narrow-row)
                 for pf in (2, 4, 8):
-                    for xc in (128, 256, 512, 1024):
+                    for xc in (128, 256, 512, 1024, 2048):
                         for sw in (0, 1):
                             c = dict(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=1, prefetch=pf, x_chunk=xc,
                                      token_tiles=tt, xcd_swizzle=sw, k_stagger=0, lds_tile_rows=0)
