@@ -120,6 +120,18 @@ def cpu_baseline(m, n, k, budget_s=12.0):
     }
 
 
+def probe_is_mid(make_configs, m, k, c):
+    """True if an unsplit one-token-tile launch that took a twin took the streaming one: the lean kernel is
+    tried first and takes every launch whose tiles are all resident at once (lean_applies in gemm_launch.hip)."""
+    if not make_configs.mid_applies(m, k, {f: c.get(f, 0) for f in make_configs.FIELDS}):
+        return False
+    waves = c["waves_m"] * c["waves_k"]
+    sps = k // 32
+    lds = 65536 + max(sps * 1024, waves * 4096) + 16
+    slots = 256 * min(make_configs.LDS_LIMIT // lds, max(1, 20 // waves)) if lds <= make_configs.LDS_LIMIT else 0
+    return m // (64 * c["waves_m"]) > slots or sps * 64 > 8 * 64 * waves
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -170,7 +182,14 @@ def main():
     else:
         before = ops.lean_launches()
         probe = time_shape(ops, synth, torch, dev, m, n, k, 2, 1, use_graph=False)
-        kernel_name = "tuna::gemm_lean_kernel" if ops.lean_launches() > before else "tuna::gemm_kernel"
+        twin = ops.lean_launches() > before      # counts both stripped-down twins of the general kernel
+        from tuna_amd import make_configs
+        if twin and (hc.get("token_tiles", 1) > 1 or probe_is_mid(make_configs, m, k, hc)):
+            kernel_name = "tuna::gemm_mid_kernel"
+        elif twin:
+            kernel_name = "tuna::gemm_lean_kernel"
+        else:
+            kernel_name = "tuna::gemm_kernel"
         del probe
 
     line = {
