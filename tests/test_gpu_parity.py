@@ -701,6 +701,10 @@ MID_CASES = [
      dict(waves_m=8, waves_k=1, prefetch=2, token_tiles=4, x_chunk=256)),
     (4096, 32, 1024, dict(waves_m=16, waves_k=1, prefetch=4, token_tiles=2, x_chunk=512),
      dict(waves_m=8, waves_k=1, prefetch=4, token_tiles=2, x_chunk=512)),
+    # staggered k walk per row tile (wraps inside a chunk of x and inside a ring turn)
+    (2048, 32, 2048, dict(waves_m=4, waves_k=1, prefetch=2, token_tiles=2, x_chunk=256, k_stagger=3), None),
+    (1536, 64, 1024, dict(waves_m=2, waves_k=4, prefetch=2, token_tiles=4, x_chunk=256, k_stagger=5), None),
+    (16640, 16, 1024, dict(waves_m=1, waves_k=2, prefetch=4, token_tiles=1, x_chunk=256, k_stagger=2), None),   # 260 tiles
     # one token tile (large shapes at up to 16 tokens; launches the lean kernel does not take: several tiles per CU)
     (33280, 16, 1024, dict(waves_m=2, waves_k=4, prefetch=2, token_tiles=1, x_chunk=1024), None),
     (38400, 9, 512, dict(waves_m=1, waves_k=1, prefetch=8, token_tiles=1, x_chunk=256), None),

@@ -186,11 +186,11 @@ def test_tuner_small_launch_config_spaces_are_valid_for_both_validators():
     with pytest.raises(ops.TunaError):
         ops.validate_config(256, 32, 5120, ops.GemmConfig.from_dict(big))
     # configs only the 17..128-token streaming kernel has (ring 8 with four token tiles, 16 waves with two): valid
-    # for both validators while the launch qualifies, refused by both when it does not (waves along k)
+    # for both validators while the launch qualifies, refused by both when it does not (too many waves, a split)
     mid = dict(rows_per_wave=64, waves_m=8, waves_k=1, split_k=1, prefetch=8, x_chunk=256, token_tiles=4, xcd_swizzle=0,
                k_stagger=0, lds_tile_rows=0)
     for c, ok in ((mid, True), (dict(mid, waves_m=16, token_tiles=2, prefetch=4), True),
-                  (dict(mid, waves_m=4, waves_k=2), False), (dict(mid, k_stagger=3), False)):
+                  (dict(mid, k_stagger=3), True), (dict(mid, waves_m=4, waves_k=4), False), (dict(mid, split_k=2), False)):
         assert mc.mid_applies(229376, 4096, c) == ok
         if ok:
             mc.validate(229376, 64 if c["token_tiles"] == 4 else 32, 4096, c)

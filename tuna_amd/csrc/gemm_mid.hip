@@ -39,7 +39,8 @@ static const MidVariant *mid_variant(const GemmPlan &plan, int *xc_out)
     const GemmArgs &a = plan.args;
     if (a.group_rows || a.balanced || plan.rw != 1 || plan.decode != TUNA_DECODE_GEMM) return nullptr;
     if (plan.token_tiles != 1 && plan.token_tiles != 2 && plan.token_tiles != 4 && plan.token_tiles != 8) return nullptr;
-    if (a.split_k != 1 || a.k_stagger != 0 || a.waves_k > 16 || (a.waves_k & (a.waves_k - 1)) != 0) return nullptr;
+    if (a.split_k != 1 || a.k_stagger < 0 || a.k_stagger > 4096 || a.waves_k > 16 || (a.waves_k & (a.waves_k - 1)) != 0)
+        return nullptr;
     if (a.k != a.steps_total * kStepK || a.k >= (1 << 23)) return nullptr;
     if (a.m % (a.waves_m * kRowsPerLoad) != 0 || a.waves_m * a.waves_k > 16) return nullptr;
     const int xc = mid_x_chunk(plan);
@@ -90,7 +91,7 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
     const size_t lds = (size_t)kLutBytes + (x_lds > red_lds ? x_lds : red_lds);
     dim3 grid = plan.grid;
     grid.x = (unsigned)(a.row_tiles < cus ? a.row_tiles : cus);  // one workgroup per CU (LDS), walking row tiles
-    const int packed = a.waves_m | a.epilogue << 5 | xc_log2 << 8 | a.wk_log2 << 13;
+    const int packed = a.waves_m | a.epilogue << 5 | xc_log2 << 8 | a.wk_log2 << 13 | a.k_stagger << 16;
     hipLaunchKernelGGL(v->fn, grid, dim3(plan.threads), lds, stream, a.q, a.x, a.code, a.absmax, a.k, a.n, a.m, packed, a.out,
                        a.residual, a.row_tiles, (int)grid.x);
     return hipGetLastError();

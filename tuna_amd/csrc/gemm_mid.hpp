@@ -5,7 +5,7 @@
 // many weight loads a wave keeps in flight and how little else it does.  (With one token tile it
 // is the general kernel without a split across workgroups, a tile walk to pay for or a stagger.)
 // This kernel computes exactly what gemm_kernel computes for one class of launches:
-//   * dense, no split of k across workgroups (split_k = 1), no stagger, m a multiple of the
+//   * dense, no split of k across workgroups (split_k = 1), m a multiple of the
 //     workgroup's rows, k a multiple of the x chunk, chunks of whole ring turns of the workgroup:
 //     no clamped or conditional weight loads, no tails; with all waves along m the accumulators
 //     are final and stored from registers, with waves along k they are summed through LDS in
@@ -29,12 +29,13 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
                                                               void *a_out, const void *a_residual, int a_row_tiles,
                                                               int a_n_wg)
 {
-    // a_packed = waves_m | epilogue << 5 | log2(x chunk in k) << 8 | log2(waves_k) << 13
+    // a_packed = waves_m | epilogue << 5 | log2(x chunk in k) << 8 | log2(waves_k) << 13 | k_stagger << 16
     const int waves_m = a_packed & 31;
     const int epilogue = (a_packed >> 5) & 7;
     const int xc_log2 = (a_packed >> 8) & 31;
     const int wk_log2 = (a_packed >> 13) & 7;
     const int waves_k = 1 << wk_log2;
+    const unsigned k_stagger = (unsigned)a_packed >> 16;
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char *lut = smem;
     unsigned char *xbuf = smem + kLutBytes;  // two buffers of one x chunk: [slot][token tile][token][16 B]
@@ -62,7 +63,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     // of one token tile.  Nothing of it depends on the chunk, so the byte offsets are formed once
     // and a chunk costs XB loads with a uniform base plus XB LDS writes (there are registers to
     // spare here; the general kernel recomputes them per chunk to save some).
-    uint32_t x_goff[XB], x_loff[XB];
+    uint32_t x_goff[XB], x_loff[XB], x_kloc[XB];  // (x_kloc: the piece's k within its chunk, for the stagger's wrap)
     uint32_t x_inchunk = 0, x_real = 0;  // bit b: piece b exists in a chunk / its token row exists
     {
         const int row_l = lane >> 2, grp = lane & 3;
@@ -72,17 +73,24 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
             const int wv = p >> 6;
             const int row = (wv % TT) * 16 + row_l, ks = wv / TT;
             const bool in = p < x_pieces;
-            x_goff[b] = in ? ((uint32_t)min(row, a_n - 1 - tok0) * (uint32_t)a_k + (uint32_t)(ks * 32 + grp * 8)) * 2u : 0u;
+            x_kloc[b] = in ? (uint32_t)(ks * 32 + grp * 8) : 0u;
+            x_goff[b] = in ? ((uint32_t)min(row, a_n - 1 - tok0) * (uint32_t)a_k + x_kloc[b]) * 2u : 0u;
             x_loff[b] = (uint32_t)((ks * 4 + grp) * (256 * TT) + row * 16);
             x_inchunk |= in ? 1u << b : 0u;
             x_real |= (in && tok0 + row < a_n) ? 1u << b : 0u;
         }
     }
     const unsigned char *x_tile = reinterpret_cast<const unsigned char *>(a_x) + (size_t)tok0 * a_k * 2;
-#define TUNA_MID_X_LOAD(kbase)                                                                  \
+    // Chunk at logical k `kbase` of a tile whose walk starts rot_k elements into the k range and
+    // wraps around (stagger, as in gemm_kernel.hpp): physical k = logical + rot_k, minus k past the
+    // end - a piece is 8 k of one 32-k step and rot_k a multiple of 32, so no piece straddles the wrap.
+#define TUNA_MID_X_LOAD(kbase, rot_k)                                                           \
     {                                                                                          \
-        const unsigned char *xc_ = x_tile + (size_t)(kbase) * 2;                               \
-        _Pragma("unroll") for (int b = 0; b < XB; ++b) xst.v[b] = *reinterpret_cast<const u32x4 *>(xc_ + x_goff[b]); \
+        const uint32_t kb_ = (uint32_t)(kbase) + (uint32_t)(rot_k);                            \
+        const unsigned char *xc_ = x_tile + (size_t)kb_ * 2;                                   \
+        const uint32_t wrap_at_ = (uint32_t)a_k - kb_; /* pieces at or past it wrap (kb_ < 2k) */ \
+        _Pragma("unroll") for (int b = 0; b < XB; ++b) xst.v[b] = *reinterpret_cast<const u32x4 *>( \
+            xc_ + x_goff[b] - ((int32_t)(x_kloc[b] - wrap_at_) >= 0 ? (size_t)a_k * 2 : (size_t)0)); \
     }
     // (rows past n are zeroed, as the general kernel does)
 #define TUNA_MID_X_STORE(buf)                                                                   \
@@ -96,17 +104,24 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     // weights of this wave's rows: lane (i16, g) loads 16 bytes = dword j of row 4*i16 + j's 8 k
     // (block row i16/2, second half of the block for odd i16), block column 4*step + g
     uint32_t lb = 0;
+    int rot = 0;
     u32x4 wq[U];
     f32x4 sc32{0.f, 0.f, 0.f, 0.f};
     XStage<XB> xst;
 #define TUNA_MID_TILE_FETCH(t)                                                                  \
     {                                                                                          \
         const int row0_ = (t) * (waves_m * 64) + wm * 64;                                      \
+        /* stagger: row tile t walks k starting rot steps in, wrapping around (gemm_kernel.hpp) */ \
+        rot = (k_stagger && n_steps > 1) ? (int)(((unsigned)(t) * k_stagger) % (unsigned)n_steps) : 0; \
         lb = ((uint32_t)(row0_ >> 3) + (uint32_t)(i16 >> 1)) * kb_total * 32u + (uint32_t)(i16 & 1) * 16u + (uint32_t)g * 32u; \
-        _Pragma("unroll") for (int u = 0; u < U; ++u) wq[u] = __builtin_nontemporal_load(      \
-            reinterpret_cast<const u32x4 *>(a_q + (size_t)(wk + (u << wk_log2)) * 128 + lb));  \
+        _Pragma("unroll") for (int u = 0; u < U; ++u)                                          \
+        {                                                                                      \
+            int s_ = wk + (u << wk_log2) + rot;                                                \
+            if (s_ >= n_steps) s_ -= n_steps;                                                  \
+            wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(a_q + (size_t)s_ * 128 + lb)); \
+        }                                                                                      \
         _Pragma("unroll") for (int j = 0; j < 4; ++j) sc32[j] = a_absmax[row0_ + i16 * 4 + j];  \
-        TUNA_MID_X_LOAD(0)                                                                     \
+        TUNA_MID_X_LOAD(0, rot << 5)                                                           \
     }
     if (tile < a_row_tiles) TUNA_MID_TILE_FETCH(tile)
 
@@ -153,7 +168,8 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
                 _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) acc[j][tt] =                 \
                     __builtin_amdgcn_mfma_f32_16x16x32_f16(av_, b_[tt], acc[j][tt], 0, 0, 0);  \
             }                                                                                  \
-            const int s_ = min(wk + ((it + u + U) << wk_log2), n_steps - 1);                   \
+            int s_ = min(wk + ((it + u + U) << wk_log2), n_steps - 1) + cur_rot;               \
+            if (s_ >= n_steps) s_ -= n_steps;                                                  \
             wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(qrow + (size_t)s_ * 128)); \
             __builtin_amdgcn_sched_barrier(0); /* keep each refill right behind its consume */ \
         }                                                                                      \
@@ -181,12 +197,13 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
         __syncthreads();
 
         const unsigned char *qrow = a_q + lb;
+        const int cur_rot = rot;
         int it = 0;  // this wave's next iteration (its k-step wk + it*waves_k)
         for (int c = 0; c < n_chunks; ++c) {
             const bool has_next = c + 1 < n_chunks;
             // (unconditional - the last chunk requests itself again and drops it: behind a branch
             // the compiler could not count these loads into the waits of the first ring turn)
-            TUNA_MID_X_LOAD(min(c + 1, n_chunks - 1) << xc_log2)
+            TUNA_MID_X_LOAD(min(c + 1, n_chunks - 1) << xc_log2, cur_rot << 5)
             const unsigned char *xb = xbuf + (c & 1) * xbuf_bytes + xb_lane;
             // (the first ring turn of a chunk is a copy of its own: there the x pieces just
             // requested are in flight behind the ring, and only straight-line code lets the

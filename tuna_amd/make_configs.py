@@ -148,7 +148,7 @@ def mid_applies(m: int, k: int, c: dict) -> bool:
     """True if a dense launch of this config is taken by the 17..128-token streaming kernel
     (mirrors mid_variant in csrc/gemm_mid.hip)."""
     tt, wm, wk = c["token_tiles"], c["waves_m"], c["waves_k"]
-    if c["rows_per_wave"] != 64 or tt not in (1, 2, 4, 8) or c["split_k"] != 1 or c["k_stagger"] != 0:
+    if c["rows_per_wave"] != 64 or tt not in (1, 2, 4, 8) or c["split_k"] != 1 or not 0 <= c["k_stagger"] <= 4096:
         return False
     if k % STEP_K or k >= 1 << 23 or not _pow2(wk) or wm < 1 or wm * wk > 16 or m % (64 * wm):
         return False

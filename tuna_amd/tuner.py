@@ -167,8 +167,8 @@ def lean_space(m: int, n_key: int, k: int):
 
 def mid_space(m: int, n_key: int, k: int):
     """Every config whose launch takes the 17..128-token streaming kernel (gemm_mid.hpp; the
-    conditions of mid_variant in gemm_mid.hip): 64 rows per wave, no split across workgroups,
-    no stagger, two, four or eight token tiles.  Small enough to time exhaustively."""
+    conditions of mid_variant in gemm_mid.hip): 64 rows per wave, no split across workgroups.
+    Small enough to time exhaustively."""
     lo, hi = make_configs.N_BUCKETS[n_key]
     if lo > 128:
         return []
@@ -182,9 +182,9 @@ def mid_space(m: int, n_key: int, k: int):
                     continue        # one token tile: only launches that fill the device unsplit (others: lean, narrow-row)
                 for pf in (2, 4, 8):
                     for xc in (128, 256, 512, 1024, 2048):
-                        for sw in (0, 1):
+                        for sw, stg in ((0, 0), (1, 0), (0, 2), (0, 5)):
                             c = dict(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=1, prefetch=pf, x_chunk=xc,
-                                     token_tiles=tt, xcd_swizzle=sw, k_stagger=0, lds_tile_rows=0)
+                                     token_tiles=tt, xcd_swizzle=sw, k_stagger=stg, lds_tile_rows=0)
                             try:
                                 make_configs.validate(m, n_key, k, c)
                             except ValueError:
