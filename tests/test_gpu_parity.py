@@ -323,6 +323,41 @@ def test_token_sweep_llama_attn_out(n):
     assert e <= REL_TOL
 
 
+@pytest.mark.parametrize("n", [1, 16, 40, 100, 200, 300, 600, 1000, 1500])
+@pytest.mark.parametrize("m,k", [(2560, 2560), (2560, 10240), (7680, 2560), (10240, 2560)])
+def test_reference_table_2560_wide_shapes_every_bucket(m, k, n):
+    """The four 2560-wide shapes of the reference's table (param_map.json keys 2560_*_2560,
+    2560_*_10240, 7680_*_2560, 10240_*_2560; dispatched at kernel.cu:3022-3155) with the tuned
+    entry of every token bucket, checked against the oracle on a random subset of 8-row blocks."""
+    import torch
+
+    from tuna_amd import ops
+    from tuna_amd.quantize import nf4_codebook
+    from tuna_amd.synth import make_weights_torch, make_x_torch
+
+    _, hit = ops.select_config(m, n, k)
+    assert hit, "no tuned table entry"
+    print(f"2560-wide shape m={m} k={k} n={n}", flush=True)
+    dev = torch.device("cuda")
+    q, absmax = make_weights_torch(m, k, seed=m + n, device=dev)
+    x = make_x_torch(n, k, seed=k + n, device=dev)
+    code = nf4_codebook(dev)
+    out = torch.full((n, m), float("nan"), dtype=torch.float16, device=dev)
+    ops.matmul(x, q, absmax, code, out, m, n, k)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    rng = np.random.default_rng(m * 31 + k + n)
+    mbs = np.sort(rng.choice(m // 8, size=8, replace=False))
+    rows = (mbs[:, None] * 8 + np.arange(8)[None, :]).ravel()
+    q_sub = q[torch.from_numpy(mbs).to(dev)].cpu().numpy()
+    ref = O.gemm_f64(q_sub, x.cpu().numpy().view(np.uint16), code.cpu().numpy(), absmax.cpu().numpy()[rows],
+                     len(rows), n, k, mode=O.D1)
+    got = out.cpu().numpy().view(np.uint16)[:, rows]
+    e = rel_err(f16_bits_to_f64(got), ref)
+    print(f"  rel_err={e:.3e}", flush=True)
+    assert e <= REL_TOL
+
+
 # ----------------------------------------------------------------------------- error behaviour
 
 def test_errors_raise_instead_of_silent_noop():
