@@ -756,6 +756,12 @@ MID_CASES = [
     # more row tiles than CUs: the workgroups walk (296 tiles of 256 rows), one chunk of x per tile
     (75776, 33, 256, dict(waves_m=4, waves_k=1, prefetch=2, token_tiles=4, x_chunk=128), None),
     (37888, 20, 512, dict(waves_m=2, waves_k=2, prefetch=2, token_tiles=2, x_chunk=128), None),      # the same with a reduction per tile
+    # more (row tiles x token chunks) than CUs: walkers whose token chunks run side by side
+    (19200, 40, 256, dict(waves_m=1, waves_k=2, prefetch=2, token_tiles=2, x_chunk=128), None),      # 300 tiles x 2 chunks
+    (16640, 150, 256, dict(waves_m=2, waves_k=2, prefetch=2, token_tiles=2, x_chunk=128), None),     # 130 x 5, ragged last chunk
+    (2048, 1100, 512, dict(waves_m=1, waves_k=4, prefetch=2, token_tiles=2, x_chunk=256), None),     # 32 x 35: more workgroups than CUs
+    (51200, 300, 256, dict(waves_m=8, waves_k=1, prefetch=2, token_tiles=8, x_chunk=128),
+     dict(waves_m=8, waves_k=1, prefetch=2, token_tiles=4, x_chunk=128)),                            # 100 x 3, eight token tiles
 ]
 
 

@@ -203,7 +203,11 @@ def test_tuner_small_launch_config_spaces_are_valid_for_both_validators():
     space = tuner.mid_space(229376, 64, 4096)
     assert space and all(mc.mid_applies(229376, 4096, c) for c in space)
     # one token tile: offered only where unsplit tiles fill the device (small shapes take the lean or narrow-row kernel)
-    assert tuner.mid_space(229376, 16, 4096) and tuner.mid_space(4096, 16, 4096) == [] and tuner.mid_space(4096, 256, 4096) == []
+    assert tuner.mid_space(229376, 16, 4096) and tuner.mid_space(4096, 16, 4096) == []
+    # from 128 tokens on: passes of eight token tiles, timed for every larger bucket too
+    for n_key in (128, 256, 2048):
+        big = tuner.mid_space(57344, n_key, 8192)
+        assert big and all(c["token_tiles"] == 8 and mc.mid_applies(57344, 8192, c) for c in big)
     assert tuner.narrow_space(4096, 128, 4096) == [] and tuner.lean_space(4096, 128, 4096) == []
     assert tuner.lean_space(4096, 16, 4104) == []       # k not a multiple of 32: no lean launch
 

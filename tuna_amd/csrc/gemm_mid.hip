@@ -6,7 +6,7 @@
 namespace tuna {
 
 typedef void (*MidKernelFn)(const uint8_t *, const void *, const float *, const float *, int, int, int, int, void *,
-                            const void *, int, int);
+                            const void *, int, int, int);
 struct MidVariant {
     int u, tt, xb, maxt;
     MidKernelFn fn;
@@ -91,9 +91,30 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
     const size_t lds = (size_t)kLutBytes + (x_lds > red_lds ? x_lds : red_lds);
     dim3 grid = plan.grid;
     grid.x = (unsigned)(a.row_tiles < cus ? a.row_tiles : cus);  // one workgroup per CU (LDS), walking row tiles
+    // Several token chunks that do not all fit the device at once: rather than one round of row
+    // tile walkers per chunk (every round streams all weights from HBM again), fewer walkers whose
+    // token chunks run side by side and share the weights through the caches.  With a multiple of
+    // 8 walkers the chunks of a walker can sit on one XCD and share its L2 (the kernel's mapping
+    // for chunks > 0); where that would leave more than an eighth of the CUs idle (9 chunks: 24
+    // walkers, 216 workgroups) any walker count is used and the chunks of a walker are neighbours
+    // in launch order only (chunks < 0), which still shares through the memory-side cache.
+    // Mixtral gate+up, eight token tiles: 1024 tokens 1870 -> 1740 us, 2048 tokens 3746 -> 3520 us.
+    int chunks = 0, n_wg = (int)grid.x;
+    if (grid.y > 1 && (long long)a.row_tiles * (long long)grid.y > (long long)cus && grid.y <= 4096) {
+        const int c = (int)grid.y;
+        const int w8 = (cus / c) & ~7;
+        if (w8 >= 8 && (long long)w8 * c * 8 >= 7LL * cus) {
+            n_wg = w8;
+            chunks = c;
+        } else {
+            n_wg = cus / c > 0 ? cus / c : 1;
+            chunks = -c;
+        }
+        grid = dim3((unsigned)(n_wg * c), 1, 1);
+    }
     const int packed = a.waves_m | a.epilogue << 5 | xc_log2 << 8 | a.wk_log2 << 13 | a.k_stagger << 16;
     hipLaunchKernelGGL(v->fn, grid, dim3(plan.threads), lds, stream, a.q, a.x, a.code, a.absmax, a.k, a.n, a.m, packed, a.out,
-                       a.residual, a.row_tiles, (int)grid.x);
+                       a.residual, a.row_tiles, n_wg, chunks);
     return hipGetLastError();
 }
 

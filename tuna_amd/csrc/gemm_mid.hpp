@@ -27,7 +27,7 @@ template <int U, int TT, int XB, int MAXT, int MINW>
 __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q, const void *a_x, const float *a_code,
                                                               const float *a_absmax, int a_k, int a_n, int a_m, int a_packed,
                                                               void *a_out, const void *a_residual, int a_row_tiles,
-                                                              int a_n_wg)
+                                                              int a_n_wg, int a_chunks)
 {
     // a_packed = waves_m | epilogue << 5 | log2(x chunk in k) << 8 | log2(waves_k) << 13 | k_stagger << 16
     const int waves_m = a_packed & 31;
@@ -49,7 +49,24 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     const int wm = wave >> wk_log2;
     const int nthreads = (waves_m * 64) << wk_log2;
     const uint32_t lane4 = (uint32_t)lane << 2;
-    const int tok0 = blockIdx.y * (16 * TT);
+    // Which row tiles and which chunk of 16*TT tokens this workgroup takes.  a_chunks == 0: row tile
+    // walk from blockIdx.x, token chunk blockIdx.y.  Otherwise (launches of several rounds) a
+    // one-dimensional grid of a_n_wg walkers x |a_chunks| token chunks in which the token chunks of
+    // a walker run side by side: they stream the same weights at about the same time, so the
+    // weights come from HBM once per launch instead of once per token chunk.  a_chunks > 1: a_n_wg
+    // is a multiple of 8 and the chunks of a walker share an XCD and its L2 (workgroups are dealt to
+    // the 8 XCDs in turn, workgroup L sits on XCD L % 8); a_chunks < -1: they are neighbours in
+    // launch order.
+    int tile = blockIdx.x, tok_chunk = blockIdx.y;
+    if (a_chunks > 1) {
+        const unsigned slot = blockIdx.x >> 3;
+        tok_chunk = (int)(slot % (unsigned)a_chunks);
+        tile = (int)(slot / (unsigned)a_chunks) * 8 + (int)(blockIdx.x & 7);
+    } else if (a_chunks < -1) {
+        tok_chunk = (int)(blockIdx.x % (unsigned)(-a_chunks));
+        tile = (int)(blockIdx.x / (unsigned)(-a_chunks));
+    }
+    const int tok0 = tok_chunk * (16 * TT);
     const int xc = 1 << xc_log2;
     const int chunk_its = (xc >> 5) >> wk_log2;      // k-steps of one wave per chunk, a multiple of U
     const int n_chunks = a_k >> xc_log2;
@@ -100,7 +117,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     }
 
     const float code_lane = a_code[i16];
-    int tile = blockIdx.x;
     // weights of this wave's rows: lane (i16, g) loads 16 bytes = dword j of row 4*i16 + j's 8 k
     // (block row i16/2, second half of the block for odd i16), block column 4*step + g
     uint32_t lb = 0;

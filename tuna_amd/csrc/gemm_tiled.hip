@@ -56,8 +56,22 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     const int i16 = lane & 15, g = lane >> 4;
     const uint32_t lane4 = (uint32_t)lane << 2;
 
-    const int row_base = blockIdx.x * BM;
-    const int tok_base = blockIdx.y * BN;
+    // One-dimensional grid over (row tile, token tile) with the token tiles of a row tile next to
+    // each other in launch order, so that the workgroups resident at one time share their weights
+    // through the caches (rows-major order streams all weights from HBM once per token tile).  When
+    // the row tile count is a multiple of 8 the token tiles of a row tile also share an XCD and its
+    // L2: workgroups are dealt to the 8 XCDs in turn, workgroup L sits on XCD L % 8.
+    int row_tile, tok_tile;
+    if ((a.row_tiles & 7) == 0) {
+        const unsigned slot = blockIdx.x >> 3;
+        tok_tile = (int)(slot % (unsigned)a.tok_tiles);
+        row_tile = (int)(slot / (unsigned)a.tok_tiles) * 8 + (int)(blockIdx.x & 7);
+    } else {
+        tok_tile = (int)(blockIdx.x % (unsigned)a.tok_tiles);
+        row_tile = (int)(blockIdx.x / (unsigned)a.tok_tiles);
+    }
+    const int row_base = row_tile * BM;
+    const int tok_base = tok_tile * BN;
     const int kb_total = a.k >> 3;
     const int mb_last = (a.m >> 3) - 1;
     const f16 *xg = reinterpret_cast<const f16 *>(a.x);
@@ -226,7 +240,7 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     }
     // split-K: fp32 partial tiles [split][tile][wave][tm][tn][lane] as float4, the last workgroup of
     // a tile to arrive adds them in split order (deterministic, no atomics on out)
-    const size_t tile_id = (size_t)blockIdx.y * gridDim.x + blockIdx.x;
+    const size_t tile_id = (size_t)tok_tile * a.row_tiles + row_tile;
     constexpr size_t kTileF4 = (size_t)8 * TM * TN * 64;  // float4s per partial tile
     f32x4 *ws4 = reinterpret_cast<f32x4 *>(a.ws);
     f32x4 *mine = ws4 + (tile_id * a.split_k + blockIdx.z) * kTileF4 + (size_t)wave * (TM * TN * 64) + lane;
@@ -306,8 +320,12 @@ hipError_t launch_gemm_tiled(const TiledArgs &args, int bm, int bn, hipStream_t 
         if (e != hipSuccess) return e;
         g_tiled_attr[dev][vi] = 1;
     }
-    const dim3 grid((unsigned)ceil_div_i(args.m, bm), (unsigned)ceil_div_i(args.n, bn), (unsigned)args.split_k);
-    hipLaunchKernelGGL(kTiled[vi].fn, grid, dim3(kTiledThreads), tiled_lds_bytes(bm, bn), stream, args);
+    TiledArgs a = args;
+    a.row_tiles = ceil_div_i(args.m, bm);
+    a.tok_tiles = ceil_div_i(args.n, bn);
+    if ((long long)a.row_tiles * a.tok_tiles > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    const dim3 grid((unsigned)(a.row_tiles * a.tok_tiles), 1, (unsigned)args.split_k);
+    hipLaunchKernelGGL(kTiled[vi].fn, grid, dim3(kTiledThreads), tiled_lds_bytes(bm, bn), stream, a);
     return hipGetLastError();
 }
 

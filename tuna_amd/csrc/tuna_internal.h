@@ -130,6 +130,7 @@ struct TiledArgs {
     int steps_total;      // ceil(k / 64)
     int split_k;          // gridDim.z
     int steps_per_split;
+    int row_tiles, tok_tiles;  // gridDim.x = row_tiles * tok_tiles: token tiles of a row tile are launched together
 };
 
 inline int ceil_div_i(int a, int b) { return (a + b - 1) / b; }

@@ -170,10 +170,10 @@ def mid_space(m: int, n_key: int, k: int):
     conditions of mid_variant in gemm_mid.hip): 64 rows per wave, no split across workgroups.
     Small enough to time exhaustively."""
     lo, hi = make_configs.N_BUCKETS[n_key]
-    if lo > 128:
-        return []
     out = []
-    for tt in ((1,) if lo <= 16 else (2,) if lo <= 32 else (4,) if lo <= 64 else (8,)):   # tuned at the bucket's lower edge
+    # tuned at the bucket's lower edge; from 128 tokens on, passes of eight token tiles (on the
+    # largest shapes they beat the many-token kernel at every token count)
+    for tt in ((1,) if lo <= 16 else (2,) if lo <= 32 else (4,) if lo <= 64 else (8,)):
         for wm in range(1, 17):
             for wk in (1, 2, 4, 8):
                 if m % (64 * wm) or wm * wk > 16 or wm * wk < 4:
@@ -281,9 +281,10 @@ def tune_shape(m, n, k, generations=6, population=24, seed=0, log=print, max_see
     n_key = make_configs.bucket_of(n)
     ev = Evaluator(m, n, k, iters=iters, warmup=max(2, iters // 6))
     if n_key >= 512:
-        # far beyond the streaming kernel's range: only the many-token kernel is searched
-        scored = sorted((ev(c), json.dumps(c, sort_keys=True)) for c in tiled_space(m, n_key, k))
-        log(f"  many-token kernel: {len(scored)} configs, best {scored[0][0]:.2f} us {scored[0][1]}")
+        # far beyond the general kernel's range: the many-token kernel and the streaming kernel
+        # with eight token tiles per pass are timed exhaustively, nothing is bred
+        scored = sorted((ev(c), json.dumps(c, sort_keys=True)) for c in tiled_space(m, n_key, k) + mid_space(m, n_key, k))
+        log(f"  many-token + streaming kernel: {len(scored)} configs, best {scored[0][0]:.2f} us {scored[0][1]}")
         return json.loads(scored[0][1]), scored[0][0]
     pool = seeds(m, n_key, k)
     rng.shuffle(pool)
