@@ -356,15 +356,49 @@ static tuna_gemm_config derive_config(int m, int n, int k)
     return c;
 }
 
+// Whether config c can run the shape (the checks of the three planners).
+static bool config_runs(int m, int n, int k, const tuna_gemm_config &c)
+{
+    if (c.lds_tile_rows) {
+        TiledPlan tp;
+        return plan_tiled(m, n, k, c, TUNA_DECODE_GEMM, &tp) == TUNA_OK;
+    }
+    if (is_narrow(c)) {
+        NarrowPlan np;
+        return plan_narrow(m, n, k, c, TUNA_DECODE_GEMM, &np) == TUNA_OK;
+    }
+    GemmPlan plan;
+    return plan_gemm(m, n, k, c, TUNA_DECODE_GEMM, &plan) == TUNA_OK;
+}
+
+// The table's buckets are the reference dispatcher's (kernel.cu:3022-3155) and every entry is
+// tuned at the lower edge of its bucket.  A token count inside one of the buckets 16..31, 32..63,
+// 64..127 or 128..255 takes two passes over the weights with that entry (it covers the lower
+// edge in one) but one pass with the entry of the next bucket, which is tuned for more tokens per
+// pass: measured on six of the benchmark shapes, 17..255 tokens, the next bucket's entry is 15-40 %
+// faster (8192 x 8192 at 20 tokens 23.8 -> 14.8 us, 57344 x 8192 at 24 tokens 81 -> 57 us,
+// 229376 x 4096 at 100 tokens 297 -> 237 us), so such a count takes it when it can run the shape.
+// Up to 15 tokens and from 256 tokens the containing bucket's entry stays.
 static int select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_table)
 {
-    for (int i = 0; i < kConfigTableSize; ++i) {
+    const TableEntry *own = nullptr;
+    for (int i = 0; i < kConfigTableSize && !own; ++i) {
         const TableEntry &e = kConfigTable[i];
-        if (e.m == m && e.k == k && n >= e.n_lo && n <= e.n_hi) {
-            *cfg = e.cfg;
-            if (from_table) *from_table = 1;
-            return TUNA_OK;
+        if (e.m == m && e.k == k && n >= e.n_lo && n <= e.n_hi) own = &e;
+    }
+    if (own && n > own->n_lo && own->n_lo >= 16 && own->n_lo <= 128) {
+        for (int i = 0; i < kConfigTableSize; ++i) {
+            const TableEntry &e = kConfigTable[i];
+            if (e.m == m && e.k == k && e.n_lo == own->n_hi + 1) {
+                if (config_runs(m, n, k, e.cfg)) own = &e;
+                break;
+            }
         }
+    }
+    if (own) {
+        *cfg = own->cfg;
+        if (from_table) *from_table = 1;
+        return TUNA_OK;
     }
     *cfg = derive_config(m, n, k);
     if (from_table) *from_table = 0;

@@ -23,7 +23,16 @@
 
 namespace tuna {
 
-template <int U, int TT, int XB, int MAXT, int MINW>
+template <bool NT>
+__device__ __forceinline__ u32x4 load_weights(const u32x4 *p)
+{
+    if constexpr (NT) return __builtin_nontemporal_load(p);
+    else return *p;
+}
+
+// NT: weight loads carry the nontemporal hint (each byte is used once per launch).  Launches whose
+// token chunks share the weights through the caches (a_chunks != 0) run the twin without it.
+template <int U, int TT, int XB, int MAXT, int MINW, bool NT = true>
 __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q, const void *a_x, const float *a_code,
                                                               const float *a_absmax, int a_k, int a_n, int a_m, int a_packed,
                                                               void *a_out, const void *a_residual, int a_row_tiles,
@@ -134,7 +143,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
         {                                                                                      \
             int s_ = wk + (u << wk_log2) + rot;                                                \
             if (s_ >= n_steps) s_ -= n_steps;                                                  \
-            wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(a_q + (size_t)s_ * 128 + lb)); \
+            wq[u] = load_weights<NT>(reinterpret_cast<const u32x4 *>(a_q + (size_t)s_ * 128 + lb)); \
         }                                                                                      \
         _Pragma("unroll") for (int j = 0; j < 4; ++j) sc32[j] = a_absmax[row0_ + i16 * 4 + j];  \
         TUNA_MID_X_LOAD(0, rot << 5)                                                           \
@@ -186,7 +195,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
             }                                                                                  \
             int s_ = min(wk + ((it + u + U) << wk_log2), n_steps - 1) + cur_rot;               \
             if (s_ >= n_steps) s_ -= n_steps;                                                  \
-            wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(qrow + (size_t)s_ * 128)); \
+            wq[u] = load_weights<NT>(reinterpret_cast<const u32x4 *>(qrow + (size_t)s_ * 128)); \
             __builtin_amdgcn_sched_barrier(0); /* keep each refill right behind its consume */ \
         }                                                                                      \
         it += U;                                                                               \
