@@ -23,15 +23,6 @@
 
 namespace tuna {
 
-// Within a slot (8 k of one k-step) of the staged x the 16 tokens of a tile are stored at
-// token ^ x_swz(k-group): the staging writes come from quads of lanes that hold the four k-groups
-// of ONE token (that is what keeps their global reads contiguous), i.e. four pieces a multiple
-// of 256 bytes apart - without the swizzle all four on the same banks.  With it any 8 consecutive
-// lanes (2 tokens x 4 groups) hit 8 different 16-byte bank groups and any 16 consecutive lanes 16
-// different ones, whichever of the two widths the LDS works in; a B fragment read (16 lanes, one
-// group, 16 tokens) stays a permutation of 256 contiguous bytes.
-__device__ __forceinline__ int x_swz(int grp) { return ((grp & 1) ? 10 : 0) ^ ((grp & 2) << 1); }
-
 template <bool NT>
 __device__ __forceinline__ u32x4 load_weights(const u32x4 *p)
 {
@@ -110,7 +101,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
             const bool in = p < x_pieces;
             x_kloc[b] = in ? (uint32_t)(ks * 32 + grp * 8) : 0u;
             x_goff[b] = in ? ((uint32_t)min(row, a_n - 1 - tok0) * (uint32_t)a_k + x_kloc[b]) * 2u : 0u;
-            x_loff[b] = (uint32_t)((ks * 4 + grp) * (256 * TT) + (row ^ x_swz(grp)) * 16);
+            x_loff[b] = (uint32_t)((ks * 4 + grp) * (256 * TT) + row * 16);
             x_inchunk |= in ? 1u << b : 0u;
             x_real |= (in && tok0 + row < a_n) ? 1u << b : 0u;
         }
@@ -182,8 +173,8 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     f16 *outp = reinterpret_cast<f16 *>(a_out);
     const f16 *resp = reinterpret_cast<const f16 *>(a_residual);
     // B fragment of lane (token i16, k-group g), local step sl, token tile tt:
-    // slot sl*4 + g, byte slot*(256*TT) + tt*256 + (i16 ^ x_swz(g))*16
-    const uint32_t xb_lane = (uint32_t)g * (256 * TT) + (uint32_t)(i16 ^ x_swz(g)) * 16 + (uint32_t)wk * (1024 * TT);
+    // slot sl*4 + g, byte slot*(256*TT) + tt*256 + i16*16
+    const uint32_t xb_lane = (uint32_t)g * (256 * TT) + (uint32_t)i16 * 16 + (uint32_t)wk * (1024 * TT);
     const uint32_t wstep = (uint32_t)(1024 * TT) << wk_log2;  // LDS bytes between this wave's consecutive steps
 
     // One ring turn: U of this wave's k-steps, each consumed (B fragments from LDS, 4 fragments
