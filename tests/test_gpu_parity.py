@@ -358,6 +358,39 @@ def test_reference_table_2560_wide_shapes_every_bucket(m, k, n):
     assert e <= REL_TOL
 
 
+def test_derived_config_for_a_large_untuned_shape_with_many_tokens():
+    """A shape outside the table with many rows and 128+ tokens gets the streaming kernel with eight
+    token tiles (three passes of 128 tokens here, side by side); checked on a random subset of rows."""
+    import torch
+
+    from tuna_amd import ops
+    from tuna_amd.quantize import nf4_codebook
+    from tuna_amd.synth import make_weights_torch, make_x_torch
+
+    m, n, k = 66560, 300, 1024
+    cfg, hit = ops.select_config(m, n, k)
+    assert not hit and cfg.token_tiles == 8 and cfg.lds_tile_rows == 0
+    print(f"derived config m={m} n={n} k={k} {cfg.to_dict()}", flush=True)
+    dev = torch.device("cuda")
+    q, absmax = make_weights_torch(m, k, seed=5, device=dev)
+    x = make_x_torch(n, k, seed=6, device=dev)
+    code = nf4_codebook(dev)
+    out = torch.full((n, m), float("nan"), dtype=torch.float16, device=dev)
+    ops.matmul(x, q, absmax, code, out, m, n, k)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    rng = np.random.default_rng(11)
+    mbs = np.sort(rng.choice(m // 8, size=32, replace=False))
+    rows = (mbs[:, None] * 8 + np.arange(8)[None, :]).ravel()
+    q_sub = q[torch.from_numpy(mbs).to(dev)].cpu().numpy()
+    ref = O.gemm_f64(q_sub, x.cpu().numpy().view(np.uint16), code.cpu().numpy(), absmax.cpu().numpy()[rows],
+                     len(rows), n, k, mode=O.D1)
+    got = out.cpu().numpy().view(np.uint16)[:, rows]
+    e = rel_err(f16_bits_to_f64(got), ref)
+    print(f"  rel_err={e:.3e}", flush=True)
+    assert e <= REL_TOL
+
+
 # ----------------------------------------------------------------------------- error behaviour
 
 def test_errors_raise_instead_of_silent_noop():

@@ -284,9 +284,25 @@ static int plan_narrow(int m, int n, int k, const tuna_gemm_config &c, int decod
 // tuned shapes: many rows -> wide row tiles without any k split (accumulators stored straight
 // from registers); few rows -> one 64-row group per workgroup, 8 waves along k and enough
 // workgroups along k to occupy the CUs.  Rings of 2 k-steps: those variants never spill.
+static bool config_runs(int m, int n, int k, const tuna_gemm_config &c);
+
 static tuna_gemm_config derive_config(int m, int n, int k)
 {
     tuna_gemm_config c;
+    if (n >= 256 && m >= 24576 && m % 512 == 0 && k % 128 == 0) {
+        // many rows, several passes of 128 tokens: the streaming kernel with eight token tiles
+        // (64 rows per wave, no split), whose token chunks run side by side and share the
+        // weights - what the tuned entries of every shape from 28672 rows choose there.  8 waves
+        // along the rows, or 4 x 2 where 512-row tiles times token chunks would not fill the CUs.
+        // (Measured on 65536 x 4096, 24576 x 8192 and 40960 x 5120: 7-25 % faster than the
+        // many-token kernel from 300 tokens, slower up to 128 tokens, where it stays.)
+        memset(&c, 0, sizeof(c));
+        const long long chunks = ceil_div(n, 128);
+        c.rows_per_wave = 64, c.split_k = 1, c.prefetch = 2, c.x_chunk = 128, c.token_tiles = 8;
+        c.waves_m = (m / 512) * chunks >= 200 ? 8 : 4;
+        c.waves_k = 8 / c.waves_m;
+        if (config_runs(m, n, k, c)) return c;
+    }
     if (n >= 128) {
         // many tokens: the kernel that decodes each weight tile once into LDS; 128-token tiles,
         // 256 rows (128 for few rows), k split until about one workgroup per CU
