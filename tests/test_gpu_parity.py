@@ -358,8 +358,9 @@ def test_reference_table_2560_wide_shapes_every_bucket(m, k, n):
     assert e <= REL_TOL
 
 
-@pytest.mark.parametrize("n,tiles", [(50, 4), (100, 8), (300, 8)])
-def test_derived_config_for_a_large_untuned_shape_with_many_tokens(n, tiles):
+@pytest.mark.parametrize("m,k,n,tiles", [(66560, 1024, 50, 4), (66560, 1024, 100, 8), (66560, 1024, 300, 8),
+                                         (16384, 2048, 100, 4)])
+def test_derived_config_for_a_large_untuned_shape_with_many_tokens(m, k, n, tiles):
     """A shape outside the table with many rows and more than 32 tokens gets the streaming kernel
     with four or eight token tiles (one pass of 64 or 128 tokens, or three passes of 128 side by
     side); checked on a random subset of rows."""
@@ -369,7 +370,6 @@ def test_derived_config_for_a_large_untuned_shape_with_many_tokens(n, tiles):
     from tuna_amd.quantize import nf4_codebook
     from tuna_amd.synth import make_weights_torch, make_x_torch
 
-    m, k = 66560, 1024
     cfg, hit = ops.select_config(m, n, k)
     assert not hit and cfg.token_tiles == tiles and cfg.lds_tile_rows == 0
     print(f"derived config m={m} n={n} k={k} {cfg.to_dict()}", flush=True)

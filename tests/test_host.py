@@ -68,7 +68,7 @@ def test_select_config_is_host_only_and_every_table_entry_validates():
 
 
 @pytest.mark.parametrize("shape", [(8, 1, 8), (64, 16, 64), (4096, 16, 4104), (1000 * 8, 3, 40), (12288, 100, 4096),
-                                   (8192, 256, 8192), (8192, 4096, 1024), (229376, 128, 4096), (65536, 300, 4096), (24576, 256, 1024), (24576, 2000, 1024), (32768, 50, 2048)])
+                                   (8192, 256, 8192), (8192, 4096, 1024), (229376, 128, 4096), (65536, 300, 4096), (24576, 256, 1024), (24576, 2000, 1024), (32768, 50, 2048), (16384, 100, 8192), (12288, 128, 4096)])
 def test_derived_config_is_valid_for_any_shape(shape):
     from tuna_amd import ops
 
