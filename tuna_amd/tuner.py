@@ -173,7 +173,9 @@ def mid_space(m: int, n_key: int, k: int):
     out = []
     # tuned at the bucket's lower edge; from 128 tokens on, passes of eight token tiles (on the
     # largest shapes they beat the many-token kernel at every token count)
-    for tt in ((1,) if lo <= 16 else (2,) if lo <= 32 else (4,) if lo <= 64 else (8,)):
+    # (128 and 256 tokens: also passes of 32 and 64 tokens, which run side by side and share the
+    # weights when they all fit the device - the mid-size shapes prefer them)
+    for tt in ((1,) if lo <= 16 else (2,) if lo <= 32 else (4,) if lo <= 64 else (8, 4, 2) if lo <= 256 else (8,)):
         for wm in range(1, 17):
             for wk in (1, 2, 4, 8):
                 if m % (64 * wm) or wm * wk > 16 or wm * wk < 4:
