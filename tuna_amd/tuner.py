@@ -341,6 +341,9 @@ def main(argv=None):
     ap.add_argument("--base", default=os.path.join(HERE, "configs", "param_map.json"),
                     help="existing param_map.json to update")
     ap.add_argument("--out", default="tuned/param_map.json")
+    ap.add_argument("--replace-margin", type=float, default=0.98,
+                    help="an entry of --base is replaced only if the new config takes less than this fraction of its "
+                         "time, both timed on this box (0: always replace)")
     ap.add_argument("--eval", default=None, help="JSON config: just time it on the given shapes and exit")
     args = ap.parse_args(argv)
 
@@ -378,6 +381,22 @@ def main(argv=None):
                                   log=lambda s: print(s, flush=True), max_seed_evals=args.max_seed_evals,
                                   iters=args.iters)
             key = f"{m}_{make_configs.bucket_of(n)}_{k}"
+            old = param_map.get(key)
+            if old is not None and args.replace_margin > 0:
+                # Boxes differ by several per cent, so a time recorded with the existing entry says
+                # little: the entry is re-timed here, on this box, and kept unless the new config
+                # beats it by the margin.
+                c_old = {f: old.get(f, 0) for f in make_configs.FIELDS}
+                if c_old != {f: best.get(f, 0) for f in make_configs.FIELDS}:
+                    ev = Evaluator(m, n, k, iters=max(100, 2 * args.iters), warmup=15)
+                    t_old, t_new = ev(c_old), ev(dict(best))
+                    ev.cache.clear()
+                    t_old, t_new = min(t_old, ev(c_old)), min(t_new, ev(dict(best)))
+                    print(f"  existing entry {t_old:.2f} us, new config {t_new:.2f} us on this box", flush=True)
+                    if not t_new < args.replace_margin * t_old:
+                        print(f"  -> {key}: existing entry kept", flush=True)
+                        continue
+                    us = t_new
             best = dict(best)
             best["us"] = round(us, 3)
             best["gbs"] = round(m * k / 2 / us / 1e3, 1)
