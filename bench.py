@@ -230,6 +230,25 @@ def main():
         "headline_graph_launch": res_graph,
     }
 
+    # Yardsticks for the fixed cost of a launch, measured in the same run: back-to-back launches of a
+    # read kernel over 4 KB (nothing to stream: the time per launch is what any kernel pays on this box)
+    # and the rate of the same kernel over 512 MB.  A launch that streams the headline's packed bytes
+    # at that rate cannot take less than their sum.
+    if not args.only_headline:
+        tiny = torch.zeros(4096, dtype=torch.uint8, device=dev)
+        big = torch.full((512 << 20,), 3, dtype=torch.uint8, device=dev)
+        us_empty = ops.time_read(tiny, blocks=192, warmup=100, iters=1000) * 1000.0 / 1000
+        ms_big = ops.time_read(big, warmup=3, iters=10) / 10
+        rate = big.numel() / (ms_big * 1e-3) / 1e9
+        line["launch_floor"] = {
+            "empty_launch_us": round(us_empty, 3),
+            "read_kernel_gbs": round(rate, 1),
+            "headline_bytes_at_read_rate_us": round(head["packed_bytes"] / rate / 1e3, 3),
+            "floor_us": round(us_empty + head["packed_bytes"] / rate / 1e3, 3),
+        }
+        del tiny, big
+        torch.cuda.empty_cache()
+
     if args.copy_yardstick > 0:
         nb = args.copy_yardstick << 20
         src = torch.full((nb,), 7, dtype=torch.uint8, device=dev)
