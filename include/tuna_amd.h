@@ -144,8 +144,9 @@ int tuna_dequant_ex(const void *q, const void *absmax, const void *code, void *o
  * absmax fp32 [m] (one scale per weight row) for the 16-entry codebook `code`.  The
  * arithmetic of the reference harness's quantize_blockwise_dynamic_4bit with block_size == k
  * and preprocess=True (test.py:7-68): absmax = max |w|; index = argmin |fp32(w) / absmax -
- * code[j]| in fp32, first index on ties; packing of test.py:55-65.  An all-zero row gets the
- * index of code 7.  The reference has this only as Python on torch tensors. */
+ * code[j]| in fp32, first index on ties; packing of test.py:55-65.  An all-zero row gets index
+ * 0 throughout (0/0 makes every candidate NaN and torch.argmin then returns 0).  The reference
+ * has this only as Python on torch tensors. */
 int tuna_quantize(const void *w, const void *code, void *q, void *absmax, int m, int k, void *stream);
 
 /* Shape -> config.  Replaces the if-chain of kernel.cu:3018-3156 over the constants of
@@ -153,8 +154,18 @@ int tuna_quantize(const void *w, const void *code, void *q, void *absmax, int m,
  * Runs on the host only (no device needed).  Returns 1 in *from_table when the shape
  * hit a tuned entry. */
 int tuna_select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_table);
+/* The config tuna_matmul_ex(cfg = NULL, decode_mode) runs: the table lookup above for
+ * TUNA_DECODE_GEMM; for TUNA_DECODE_DEQUANT, whose kernel variants the table is not tuned for,
+ * always a derived config.  Host only. */
+int tuna_select_config_ex(int m, int n, int k, int decode_mode, tuna_gemm_config *cfg, int *from_table);
+/* The config tuna_matmul_grouped(cfg = NULL) runs for n_active groups with tokens, the largest
+ * of them with max_tokens.  Host only. */
+int tuna_select_config_grouped(int m_group, int n_active, int max_tokens, int k, int decode_mode,
+                               tuna_gemm_config *cfg);
 /* TUNA_OK if `cfg` can run shape (m, n, k); otherwise an error and tuna_last_error(). */
 int tuna_validate_config(int m, int n, int k, const tuna_gemm_config *cfg);
+/* Same for a decode mode (tuna_validate_config checks TUNA_DECODE_GEMM). */
+int tuna_validate_config_ex(int m, int n, int k, const tuna_gemm_config *cfg, int decode_mode);
 /* Dynamic LDS bytes and workspace bytes a launch of `cfg` needs. */
 int tuna_config_footprint(int m, int n, int k, const tuna_gemm_config *cfg,
                           size_t *lds_bytes, size_t *workspace_bytes);
@@ -175,53 +186,10 @@ int tuna_config_contributors(int m, int n, int k, const tuna_gemm_config *cfg, i
 int tuna_config_table_size(void);
 int tuna_config_table_entry(int i, int *m, int *n_lo, int *n_hi, int *k, tuna_gemm_config *cfg);
 
-/* Timing helper for the bench and the tuner: enqueues `warmup` untimed and `iters`
- * timed GEMMs on `stream`, launch i using weight set (i mod n_sets) of q_list /
- * absmax_list (rotating over distinct weights defeats the L2 / MALL caches), and
- * returns the elapsed milliseconds of the timed launches measured with HIP events
- * recorded on `stream`.  use_graph != 0 captures one rotation into a HIP graph and
- * replays it.  This call synchronises the host with `stream`. */
-int tuna_time_matmul(const void *const *q_list, const void *const *absmax_list, int n_sets,
-                     const void *x, const void *code, void *out, int m, int n, int k,
-                     const tuna_gemm_config *cfg, int decode_mode, int warmup, int iters,
-                     int use_graph, void *stream, float *elapsed_ms);
-/* Same protocol for the grouped GEMM. */
-int tuna_time_matmul_grouped(const void *const *q_list, const void *const *absmax_list, int n_sets,
-                             const void *x, const void *code, void *out, int m_group, int n_groups,
-                             int k, const int32_t *token_offsets, const tuna_gemm_config *cfg,
-                             int decode_mode, int warmup, int iters, int use_graph, void *stream,
-                             float *elapsed_ms);
-/* Same protocol for the dequant kernel. */
-int tuna_time_dequant(const void *const *q_list, const void *const *absmax_list, int n_sets,
-                      const void *code, void *out, int m, int k, int warmup, int iters,
-                      void *stream, float *elapsed_ms);
-/* Plain device-to-device copy kernel of `bytes` bytes (16-byte multiples), timed the
- * same way: the known-traffic yardstick the HBM counters are scaled against. */
-int tuna_time_copy(const void *src, void *dst, size_t bytes, int warmup, int iters,
-                   void *stream, float *elapsed_ms);
-
-/* Read-only streaming kernel over `bytes` bytes of `src` (16-byte multiples), `blocks`
- * workgroups of 256 threads (0 = default): the ceiling a pure HBM reader reaches on the
- * device, reported beside the GEMM's rate.  `sink` is 4 writable bytes. */
-int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int warmup, int iters,
-                   void *stream, float *elapsed_ms);
-
-/* Diagnostic switch, process-wide, default on: dense launches that qualify run one of two
- * kernels stripped of everything else the general one carries - small launches (one workgroup
- * per tile, power-of-two split, aligned shapes, up to 16 tokens per tile) and launches with 2, 4
- * or 8 token tiles and no split of k across workgroups (x chunks double-buffered in LDS).  Both
- * compute the general kernel's results bit for bit; turning them off is for A/B timing and for
- * the tests that check exactly that.  A config whose ring depth or token tile count only the
- * second kernel has (prefetch 4 or 8 with 4 token tiles, 8 token tiles, 16 waves with 2 or more
- * token tiles) runs it regardless of the switch.  Returns the previous setting.  No counterpart
- * in the reference. */
-int tuna_set_lean_kernels(int enabled);
-
-/* Diagnostic: how many GEMM launches of this process took one of those kernels so far. */
-unsigned long long tuna_lean_launches(void);
-
 /* Releases the library-owned split-K workspaces of the current device (synchronises
- * the device first). */
+ * the device first).  Until then a workspace that a launch has used is never freed or moved -
+ * HIP graphs captured earlier keep working when later launches need a larger one - so call this
+ * only when no captured graph that contains GEMMs of this library will be replayed again. */
 int tuna_release_workspaces(void);
 
 #ifdef __cplusplus

@@ -1,0 +1,66 @@
+/*
+ * tuna_amd - measurement and diagnostic entry points of libtuna_amd.so.
+ *
+ * These are tools for bench.py, the tuner and the tests: timing loops with HIP events on the
+ * launch stream, known-traffic yardstick kernels, and a switch between kernels that compute
+ * identical results.  None of them replaces an interface of the reference; the product's C ABI
+ * is tuna_amd.h.
+ */
+#ifndef TUNA_AMD_BENCH_H
+#define TUNA_AMD_BENCH_H
+
+#include "tuna_amd.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Timing helper for the bench and the tuner: enqueues `warmup` untimed and `iters`
+ * timed GEMMs on `stream`, launch i using weight set (i mod n_sets) of q_list /
+ * absmax_list (rotating over distinct weights defeats the L2 / MALL caches), and
+ * returns the elapsed milliseconds of the timed launches measured with HIP events
+ * recorded on `stream`.  use_graph != 0 captures one rotation into a HIP graph and
+ * replays it.  This call synchronises the host with `stream`. */
+int tuna_time_matmul(const void *const *q_list, const void *const *absmax_list, int n_sets,
+                     const void *x, const void *code, void *out, int m, int n, int k,
+                     const tuna_gemm_config *cfg, int decode_mode, int warmup, int iters,
+                     int use_graph, void *stream, float *elapsed_ms);
+/* Same protocol for the grouped GEMM. */
+int tuna_time_matmul_grouped(const void *const *q_list, const void *const *absmax_list, int n_sets,
+                             const void *x, const void *code, void *out, int m_group, int n_groups,
+                             int k, const int32_t *token_offsets, const tuna_gemm_config *cfg,
+                             int decode_mode, int warmup, int iters, int use_graph, void *stream,
+                             float *elapsed_ms);
+/* Same protocol for the dequant kernel. */
+int tuna_time_dequant(const void *const *q_list, const void *const *absmax_list, int n_sets,
+                      const void *code, void *out, int m, int k, int warmup, int iters,
+                      void *stream, float *elapsed_ms);
+/* Plain device-to-device copy kernel of `bytes` bytes (16-byte multiples), timed the
+ * same way: the known-traffic yardstick the HBM counters are scaled against. */
+int tuna_time_copy(const void *src, void *dst, size_t bytes, int warmup, int iters,
+                   void *stream, float *elapsed_ms);
+
+/* Read-only streaming kernel over `bytes` bytes of `src` (16-byte multiples), `blocks`
+ * workgroups of 256 threads (0 = default): the ceiling a pure HBM reader reaches on the
+ * device, reported beside the GEMM's rate.  `sink` is 4 writable bytes. */
+int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int warmup, int iters,
+                   void *stream, float *elapsed_ms);
+
+/* Diagnostic switch, process-wide, default on: dense launches that qualify run one of two
+ * kernels stripped of everything else the general one carries - small launches (one workgroup
+ * per tile, power-of-two split, aligned shapes, up to 16 tokens per tile) and launches with 2, 4
+ * or 8 token tiles and no split of k across workgroups (x chunks double-buffered in LDS).  Both
+ * compute the general kernel's results bit for bit; turning them off is for A/B timing and for
+ * the tests that check exactly that.  A config whose ring depth or token tile count only the
+ * second kernel has (prefetch 4 or 8 with 4 token tiles, 8 token tiles, 16 waves with 2 or more
+ * token tiles) runs it regardless of the switch.  Returns the previous setting.  No counterpart
+ * in the reference. */
+int tuna_set_lean_kernels(int enabled);
+
+/* Diagnostic: how many GEMM launches of this process took one of those kernels so far. */
+unsigned long long tuna_lean_launches(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TUNA_AMD_BENCH_H */

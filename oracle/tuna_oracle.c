@@ -23,8 +23,9 @@
  *   orc_quantize : per-row absmax + nearest codebook entry + packing (test.py:7-68),
  *       checked against numpy float32 division / |difference| / argmin (first index on
  *       ties) incl. exact midpoints between codes, and against the round trip through
- *       orc_dequant.  All-zero rows: the reference divides by zero and lets NaNs
- *       decide (parity unpinned for that input); here such a row gets code 7 (0.0).
+ *       orc_dequant.  All-zero rows: the reference divides by zero, every candidate
+ *       distance is NaN and torch.argmin over an all-NaN column returns index 0;
+ *       pinned by running that torch expression (CPU torch) in the test.
  *   orc_gemm*   : textbook contraction; checked against numpy float64 matmul,
  *       linearity, one-hot read-out of the decoded weights, row permutation
  */
@@ -254,7 +255,7 @@ ORC_API int orc_quantize(const uint16_t *w, const float *code, uint8_t *q, float
             }
             absmax[r] = amax;
             for (int c = 0; c < k; c++) {
-                int best = 7;
+                int best = 0; /* all-NaN candidates: torch.argmin returns index 0 */
                 if (amax > 0.f) {
                     const volatile float nv = orc_f16_to_f32(w[(size_t)r * k + c]) / amax; /* fp32, no excess precision */
                     float bd = 0.f;

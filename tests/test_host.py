@@ -15,7 +15,8 @@ def test_library_loads_and_exports_every_declared_symbol():
     from tuna_amd import _lib
 
     L = _lib.lib()
-    header = open(os.path.join(ROOT, "include", "tuna_amd.h")).read()
+    header = "".join(open(os.path.join(ROOT, "include", h)).read() for h in sorted(os.listdir(os.path.join(ROOT, "include")))
+                     if h.endswith(".h"))
     declared = set(re.findall(r"\b(tuna_[a-z0-9_]+)\s*\(", header))
     assert declared, "no declarations parsed"
     assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
@@ -430,3 +431,49 @@ def test_grouped_gemm_argument_checks_need_no_device():
     assert b"" != L.tuna_last_error()
     assert call(256, 2, 256, [0, 0, 0]) == 0              # no tokens anywhere: nothing to do, no pointer is touched
     assert call(256, 2, 256, [0, 4, 8]) == 1              # tokens, but null pointers
+
+
+def test_dequant_rounding_mode_gets_a_runnable_config_for_every_table_shape():
+    """tuna_matmul_ex(cfg=NULL, TUNA_DECODE_DEQUANT) must run every tuned shape: the table's entries
+    are for the GEMM's own decode (narrow-row, many-token and deep-ring entries have no variant
+    with the dequant rounding), so that mode takes a derived streaming config."""
+    from tuna_amd import _lib, ops
+
+    for m, lo, hi, k, _cfg in ops.config_table():
+        for n in sorted({lo, min(hi, lo + 7), min(hi, 4096)}):
+            c, hit = ops.select_config(m, n, k, _lib.DECODE_DEQUANT)
+            assert not hit
+            assert c.lds_tile_rows == 0 and c.rows_per_wave == 64 and c.prefetch == 2 and c.waves_m >= 1
+            assert c.waves_m * c.waves_k <= 8 and c.token_tiles in (1, 2, 4)
+            ops.validate_config(m, n, k, c, _lib.DECODE_DEQUANT)
+    # the GEMM's own decode still takes the table
+    c, hit = ops.select_config(6144, 16, 4096, _lib.DECODE_GEMM)
+    assert hit and c.rows_per_wave == 32
+    with pytest.raises(ops.TunaError):
+        ops.validate_config(6144, 16, 4096, c, _lib.DECODE_DEQUANT)   # narrow-row: GEMM decode only
+
+
+def test_grouped_launch_gets_a_runnable_config_for_every_table_shape():
+    """tuna_matmul_grouped(cfg=NULL) for every tuned shape split into 1, 2 or 8 groups, with all or
+    only some groups active: a config is found (no division by a zero waves_m of a narrow-row
+    entry, no TUNA_ERR_UNSUPPORTED), its row tile divides the group and it is a streaming config."""
+    from tuna_amd import _lib, ops
+
+    seen = 0
+    for m, lo, hi, k, _cfg in ops.config_table():
+        for groups in (1, 2, 8):
+            if m % (64 * groups):
+                continue
+            m_group = m // groups
+            for active in sorted({1, groups}):
+                for decode in (_lib.DECODE_GEMM, _lib.DECODE_DEQUANT):
+                    c = ops.select_config_grouped(m_group, active, lo, k, decode)
+                    assert c.lds_tile_rows == 0 and c.rows_per_wave == 64 and c.waves_m >= 1
+                    assert m_group % (64 * c.waves_m) == 0
+                    seen += 1
+    assert seen > 300
+    # the case that used to divide by zero: Mixtral down, all 8 experts active, 4 tokens each
+    c = ops.select_config_grouped(4096, 8, 4, 14336)
+    assert c.waves_m >= 1 and 4096 % (64 * c.waves_m) == 0
+    with pytest.raises(ops.TunaError):
+        ops.select_config_grouped(4000, 8, 4, 14336)                   # not a multiple of 64 rows

@@ -270,8 +270,7 @@ def _quantize_numpy_model(w, code):
     with np.errstate(divide="ignore", invalid="ignore"):
         nv = (wf / a[:, None]).astype(np.float32)
     d = np.abs((nv[None] - code[:, None, None]).astype(np.float32))
-    idx = d.argmin(axis=0).astype(np.uint8)
-    idx[a == 0] = 7                                   # all-zero rows: defined here, NaN-driven in the reference
+    idx = d.argmin(axis=0).astype(np.uint8)           # all-zero rows: every distance is NaN, argmin gives 0
     return pack_codes_np(idx), a.astype(np.float32)
 
 
@@ -304,6 +303,31 @@ def test_quantizer_oracle_matches_numpy_model(m, k):
     code2 = rng.standard_normal(16).astype(np.float32)
     q2, _ = O.quantize(w.view(np.uint16), code2, m, k)
     assert np.array_equal(q2, _quantize_numpy_model(w, code2)[0])
+
+
+def test_quantizer_oracle_matches_torch_semantics_incl_all_zero_rows():
+    """The reference's quantizer is torch code (test.py:41-53): fp16 / fp32 division, |a - b|, and
+    torch.argmin, whose result on an all-NaN column (an all-zero row divided by its absmax 0) is
+    index 0.  The same torch expressions on the CPU pin the oracle for that input too."""
+    import torch
+
+    rng = np.random.default_rng(77)
+    m, k = 16, 64
+    w, code = _quantizer_inputs(rng, m, k)
+    wt = torch.from_numpy(w.copy())
+    ct = torch.from_numpy(code.copy())
+    absmax = torch.max(wt.abs(), dim=1)[0].float()
+    normalized = torch.divide(wt, absmax.unsqueeze(-1)).flatten()
+    assert normalized.dtype == torch.float32
+    cand = torch.sub(normalized.unsqueeze(0), ct.unsqueeze(-1)).abs()
+    idx = torch.argmin(cand, keepdim=True, dim=0).flatten().to(torch.uint8).numpy().reshape(m, k)
+    assert (idx[1] == 0).all() and torch.isnan(normalized.reshape(m, k)[1]).all()   # the all-zero row
+    from tuna_amd.quantize import pack_codes_np
+
+    q, a = O.quantize(w.view(np.uint16), code, m, k)
+    assert np.array_equal(a, absmax.numpy())
+    assert np.array_equal(q, pack_codes_np(idx))
+    assert (q.reshape(m // 8, k // 8, 8, 4)[0, :, 1] == 0).all()                    # bytes 0x00, not 0x77
 
 
 def test_quantizer_round_trip_recovers_the_codes():

@@ -68,7 +68,10 @@ SIGNATURES = {
     "tuna_quantize": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "tuna_dequant_ex": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "tuna_select_config": (_i, [_i, _i, _i, _cfgp, _ip]),
+    "tuna_select_config_ex": (_i, [_i, _i, _i, _i, _cfgp, _ip]),
+    "tuna_select_config_grouped": (_i, [_i, _i, _i, _i, _i, _cfgp]),
     "tuna_validate_config": (_i, [_i, _i, _i, _cfgp]),
+    "tuna_validate_config_ex": (_i, [_i, _i, _i, _cfgp, _i]),
     "tuna_config_footprint": (_i, [_i, _i, _i, _cfgp, ctypes.POINTER(_sz), ctypes.POINTER(_sz)]),
     "tuna_config_segments": (_i, [_i, _i, _i, _cfgp, _i, _i, _ip, _i, _ip]),
     "tuna_config_contributors": (_i, [_i, _i, _i, _cfgp, _i, _i, _ip, _ip, _ip]),

@@ -259,6 +259,9 @@ static int plan_narrow(int m, int n, int k, const tuna_gemm_config &c, int decod
     if (!is_pow2(c.waves_k) || c.waves_k > 16 || !narrow_variant_exists(c.rows_per_wave, c.waves_k, c.prefetch, c.token_tiles))
         return fail(TUNA_ERR_UNSUPPORTED, "no narrow-row kernel for rows_per_wave=%d waves_k=%d prefetch=%d token_tiles=%d",
                     c.rows_per_wave, c.waves_k, c.prefetch, c.token_tiles);
+    if (c.x_chunk != kStepK * c.waves_k * c.prefetch)
+        return fail(TUNA_ERR_UNSUPPORTED, "the narrow-row kernel stages no x: x_chunk=%d must be 32*waves_k*prefetch=%d", c.x_chunk,
+                    kStepK * c.waves_k * c.prefetch);
     if (m % c.rows_per_wave)
         return fail(TUNA_ERR_UNSUPPORTED, "rows_per_wave=%d needs m=%d to be a multiple of it", c.rows_per_wave, m);
     if (k % (kStepK * c.waves_k * c.prefetch))
@@ -278,6 +281,69 @@ static int plan_narrow(int m, int n, int k, const tuna_gemm_config &c, int decod
     plan->args.k = k;
     plan->args.n_it = k / kStepK / c.waves_k;
     return TUNA_OK;
+}
+
+// The streaming-kernel branch of the derivation: 64 rows per wave, rings of 2 k-steps (those
+// variants never spill), one or two token tiles.  Many rows -> wide row tiles without any k split
+// (accumulators stored straight from registers); few rows -> one 64-row group per workgroup, 8
+// waves along k and enough workgroups along k to occupy the CUs.  The dequant-rounding variants
+// exist for up to 8 waves only.
+static tuna_gemm_config derive_streaming(int m, int n, int k, int decode)
+{
+    tuna_gemm_config c;
+    c.token_tiles = n <= 16 ? 1 : 2;  // more tokens loop over gridDim.y (the 4-tile variants spill)
+    c.rows_per_wave = 64;
+    c.prefetch = 2;
+    c.xcd_swizzle = 1;
+    c.k_stagger = 1;
+    c.lds_tile_rows = 0;
+    const int steps = ceil_div(k, kStepK);
+    const int groups64 = ceil_div(m, kRowsPerLoad);
+    if (groups64 >= 2048) {
+        c.waves_m = 8, c.waves_k = 1;
+    } else if (groups64 >= 512) {
+        c.waves_m = 4, c.waves_k = 4;
+    } else if (groups64 >= 256) {
+        c.waves_m = 2, c.waves_k = 8;
+    } else {
+        c.waves_m = 1, c.waves_k = 8;
+    }
+    // 16-wave variants exist for one token tile and the GEMM's own decode only
+    if ((c.token_tiles > 1 || decode != TUNA_DECODE_GEMM) && c.waves_m * c.waves_k > 8) c.waves_k /= 2;
+    const int row_tiles = ceil_div(m, c.rows_per_wave * c.waves_m);
+    const int group = c.waves_k * c.prefetch;  // k-steps one workgroup consumes per ring turn
+    const int threads = c.waves_m * c.waves_k * 64;
+    auto set_chunk = [&](int sps) {
+        // x chunk: as long as the staging allows (4 pieces per thread), at most 1024 k, no longer than the split
+        // ... and, with more row tiles than CUs, short enough (16 KB) for two workgroups to share a CU
+        const int cap_k = (row_tiles > kMaxCus && threads <= 512) ? 512 / c.token_tiles : 1024;
+        int chunk_steps = group;  // power of two
+        while (chunk_steps < sps && chunk_steps * 2 * kStepK * c.token_tiles <= 2 * threads && chunk_steps * 2 * kStepK <= cap_k)
+            chunk_steps *= 2;
+        c.x_chunk = chunk_steps * kStepK;
+    };
+    // k split.  More row tiles than workgroup slots: none.  Otherwise the largest split that still
+    // fits one round of tiles, if that fills at least half of the slots (measured: a half-empty
+    // round of whole tiles beats the alternative); if no such split exists the k ranges are divided
+    // evenly instead (balanced split), which costs a partial-sum epilogue in every workgroup but
+    // leaves no CU idle.
+    const int max_split = steps / (2 * group) > 0 ? steps / (2 * group) : 1;  // at least two ring turns per workgroup
+    c.split_k = 1;
+    set_chunk(steps);
+    GemmPlan plan;
+    if (plan_gemm(m, n, k, c, decode, &plan) != TUNA_OK) return c;
+    const int slots = kMaxCus * plan.wgs_per_cu;
+    if (row_tiles >= slots) return c;
+    int split = slots / row_tiles;
+    if (split > max_split) split = max_split;
+    if (split < 1) split = 1;
+    if ((double)row_tiles * split >= 0.5 * slots) {
+        c.split_k = split;
+        set_chunk(ceil_div(steps, split));
+    } else if (steps >= 2 * group) {
+        c.split_k = 0;
+    }
+    return c;
 }
 
 // A config for shapes the tuned table does not cover, following what the tuner finds on the
@@ -348,58 +414,7 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         c.split_k = (int)split;
         return c;
     }
-    c.token_tiles = n <= 16 ? 1 : 2;  // more tokens loop over gridDim.y (the 4-tile variants spill)
-    c.rows_per_wave = 64;
-    c.prefetch = 2;
-    c.xcd_swizzle = 1;
-    c.k_stagger = 1;
-    c.lds_tile_rows = 0;
-    const int steps = ceil_div(k, kStepK);
-    const int groups64 = ceil_div(m, kRowsPerLoad);
-    if (groups64 >= 2048) {
-        c.waves_m = 8, c.waves_k = 1;
-    } else if (groups64 >= 512) {
-        c.waves_m = 4, c.waves_k = 4;
-    } else if (groups64 >= 256) {
-        c.waves_m = 2, c.waves_k = 8;
-    } else {
-        c.waves_m = 1, c.waves_k = 8;
-    }
-    if (c.token_tiles > 1 && c.waves_m * c.waves_k > 8) c.waves_k /= 2;  // 16-wave variants exist for one token tile only
-    const int row_tiles = ceil_div(m, c.rows_per_wave * c.waves_m);
-    const int group = c.waves_k * c.prefetch;  // k-steps one workgroup consumes per ring turn
-    const int threads = c.waves_m * c.waves_k * 64;
-    auto set_chunk = [&](int sps) {
-        // x chunk: as long as the staging allows (4 pieces per thread), at most 1024 k, no longer than the split
-        // ... and, with more row tiles than CUs, short enough (16 KB) for two workgroups to share a CU
-        const int cap_k = (row_tiles > kMaxCus && threads <= 512) ? 512 / c.token_tiles : 1024;
-        int chunk_steps = group;  // power of two
-        while (chunk_steps < sps && chunk_steps * 2 * kStepK * c.token_tiles <= 2 * threads && chunk_steps * 2 * kStepK <= cap_k)
-            chunk_steps *= 2;
-        c.x_chunk = chunk_steps * kStepK;
-    };
-    // k split.  More row tiles than workgroup slots: none.  Otherwise the largest split that still
-    // fits one round of tiles, if that fills at least half of the slots (measured: a half-empty
-    // round of whole tiles beats the alternative); if no such split exists the k ranges are divided
-    // evenly instead (balanced split), which costs a partial-sum epilogue in every workgroup but
-    // leaves no CU idle.
-    const int max_split = steps / (2 * group) > 0 ? steps / (2 * group) : 1;  // at least two ring turns per workgroup
-    c.split_k = 1;
-    set_chunk(steps);
-    GemmPlan plan;
-    if (plan_gemm(m, n, k, c, TUNA_DECODE_GEMM, &plan) != TUNA_OK) return c;
-    const int slots = kMaxCus * plan.wgs_per_cu;
-    if (row_tiles >= slots) return c;
-    int split = slots / row_tiles;
-    if (split > max_split) split = max_split;
-    if (split < 1) split = 1;
-    if ((double)row_tiles * split >= 0.5 * slots) {
-        c.split_k = split;
-        set_chunk(ceil_div(steps, split));
-    } else if (steps >= 2 * group) {
-        c.split_k = 0;
-    }
-    return c;
+    return derive_streaming(m, n, k, TUNA_DECODE_GEMM);
 }
 
 // Whether config c can run the shape (the checks of the three planners).
@@ -451,8 +466,40 @@ static int select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_t
     return TUNA_OK;
 }
 
+// The config a launch without an explicit one runs.  The tuned table is for the GEMM's own decode;
+// the dequant rounding (a correctness mode) has variants of the general kernel only - 64 rows per
+// wave, rings of 2, up to 8 waves - so it always takes the derived streaming config.
+static int select_config_for(int m, int n, int k, int decode, tuna_gemm_config *cfg, int *from_table)
+{
+    if (decode == TUNA_DECODE_GEMM) return select_config(m, n, k, cfg, from_table);
+    *cfg = derive_streaming(m, n, k, decode);
+    if (from_table) *from_table = 0;
+    return TUNA_OK;
+}
+
+// The checks of the planner `c` belongs to, for a decode mode.
+static int validate_for(int m, int n, int k, const tuna_gemm_config &c, int decode)
+{
+    if (c.lds_tile_rows) {
+        TiledPlan tp;
+        return plan_tiled(m, n, k, c, decode, &tp);
+    }
+    if (is_narrow(c)) {
+        NarrowPlan np;
+        return plan_narrow(m, n, k, c, decode, &np);
+    }
+    GemmPlan plan;
+    return plan_gemm(m, n, k, c, decode, &plan);
+}
+
 // ---------------------------------------------------------------------------------------
-// split-K workspace: owned by the library, one per (device, stream), grown on demand
+// split-K workspace: owned by the library, one per (device, stream)
+//
+// A buffer that has been handed to a launch is never freed or moved before
+// tuna_release_workspaces: a HIP graph captured on the stream keeps the pointers in its kernel
+// nodes and may be replayed at any later time.  The first request allocates generously (64 MB of
+// partial sums and 64 K counters cover every entry of the tuned table); a larger request adds a
+// new buffer and retires the old one, which stays allocated for the graphs that know it.
 // ---------------------------------------------------------------------------------------
 
 struct Workspace {
@@ -460,10 +507,23 @@ struct Workspace {
     size_t ws_bytes = 0;
     unsigned *counters = nullptr;
     size_t n_counters = 0;
+    std::vector<void *> retired;  // outgrown buffers, kept for graphs captured while they were current
 };
+
+constexpr size_t kWsFirstBytes = (size_t)64 << 20;
+constexpr size_t kWsFirstCounters = (size_t)64 << 10;
 
 static std::mutex g_ws_mutex;
 static std::map<std::pair<int, hipStream_t>, Workspace> g_workspaces;
+
+// Size of the buffer that serves a request of `want` when `have` is current: unchanged if it
+// fits, otherwise at least the first-allocation size and at least twice the current one.
+static size_t grown_size(size_t have, size_t want, size_t first)
+{
+    if (want <= have) return have;
+    size_t s = have ? 2 * have : first;
+    return s > want ? s : want;
+}
 
 static int get_workspace(hipStream_t stream, size_t ws_bytes, size_t n_counters, Workspace *out)
 {
@@ -478,32 +538,46 @@ static int get_workspace(hipStream_t stream, size_t ws_bytes, size_t n_counters,
             return fail(TUNA_ERR_WORKSPACE,
                         "split-K workspace must grow (%zu bytes) while the stream is capturing; run the shape once before capture",
                         ws_bytes);
-        // hipFree waits for the device, so kernels still using the old buffers are done.
         if (w.ws_bytes < ws_bytes) {
-            size_t want = ws_bytes < (size_t)(8u << 20) ? (size_t)(8u << 20) : ws_bytes;
-            if (w.ws) (void)hipFree(w.ws);
-            w.ws = nullptr;
-            w.ws_bytes = 0;
-            e = hipMalloc(reinterpret_cast<void **>(&w.ws), want);
+            const size_t want = grown_size(w.ws_bytes, ws_bytes, kWsFirstBytes);
+            float *fresh = nullptr;
+            e = hipMalloc(reinterpret_cast<void **>(&fresh), want);
             if (e != hipSuccess) return fail(TUNA_ERR_WORKSPACE, "hipMalloc(%zu) for the split-K workspace: %s", want, hipGetErrorString(e));
+            if (w.ws) w.retired.push_back(w.ws);
+            w.ws = fresh;
             w.ws_bytes = want;
         }
         if (w.n_counters < n_counters) {
-            size_t want = n_counters < 16384 ? 16384 : n_counters;
-            if (w.counters) (void)hipFree(w.counters);
-            w.counters = nullptr;
-            w.n_counters = 0;
-            e = hipMalloc(reinterpret_cast<void **>(&w.counters), want * sizeof(unsigned));
+            const size_t want = grown_size(w.n_counters, n_counters, kWsFirstCounters);
+            unsigned *fresh = nullptr;
+            e = hipMalloc(reinterpret_cast<void **>(&fresh), want * sizeof(unsigned));
             if (e != hipSuccess) return fail(TUNA_ERR_WORKSPACE, "hipMalloc for the split-K counters: %s", hipGetErrorString(e));
-            e = hipMemset(w.counters, 0, want * sizeof(unsigned));  // kernels leave them at zero afterwards
-            if (e != hipSuccess) return hip_fail(e, "hipMemset(counters)");
+            e = hipMemset(fresh, 0, want * sizeof(unsigned));  // kernels leave them at zero afterwards
+            if (e != hipSuccess) {
+                (void)hipFree(fresh);
+                return hip_fail(e, "hipMemset(counters)");
+            }
             e = hipDeviceSynchronize();
-            if (e != hipSuccess) return hip_fail(e, "hipDeviceSynchronize");
+            if (e != hipSuccess) {
+                (void)hipFree(fresh);
+                return hip_fail(e, "hipDeviceSynchronize");
+            }
+            if (w.counters) w.retired.push_back(w.counters);
+            w.counters = fresh;
             w.n_counters = want;
         }
     }
     *out = w;
+    out->retired.clear();
     return TUNA_OK;
+}
+
+static void free_workspace(Workspace &w)
+{
+    if (w.ws) (void)hipFree(w.ws);
+    if (w.counters) (void)hipFree(w.counters);
+    for (void *p : w.retired) (void)hipFree(p);
+    w = Workspace();
 }
 
 static void drop_workspace(hipStream_t stream)
@@ -513,8 +587,7 @@ static void drop_workspace(hipStream_t stream)
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     auto it = g_workspaces.find(std::make_pair(dev, stream));
     if (it == g_workspaces.end()) return;
-    if (it->second.ws) (void)hipFree(it->second.ws);
-    if (it->second.counters) (void)hipFree(it->second.counters);
+    free_workspace(it->second);
     g_workspaces.erase(it);
 }
 
@@ -524,11 +597,6 @@ static int check_ptr(const void *p, const char *name, size_t align)
     if (reinterpret_cast<uintptr_t>(p) % align) return fail(TUNA_ERR_INVALID_ARG, "%s must be %zu-byte aligned", name, align);
     return TUNA_OK;
 }
-
-#ifdef TUNA_TRACE
-static unsigned long long *g_trace = nullptr;
-extern "C" __attribute__((visibility("default"))) void tuna_set_trace(void *p) { g_trace = static_cast<unsigned long long *>(p); }
-#endif
 
 static int matmul_impl(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n, int k,
                        const tuna_gemm_config *cfg, int decode, hipStream_t stream, int epilogue = TUNA_EPILOGUE_NONE,
@@ -544,13 +612,7 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
         return rc;
     tuna_gemm_config c;
     if (cfg) c = *cfg;
-    else {
-        select_config(m, n, k, &c, nullptr);
-        if (decode != TUNA_DECODE_GEMM) {  // the dequant-rounding variants exist for one tile shape only
-            c.rows_per_wave = 64;
-            c.prefetch = 2;
-        }
-    }
+    else select_config_for(m, n, k, decode, &c, nullptr);
     if (c.lds_tile_rows) {
         TiledPlan tp;
         if ((rc = plan_tiled(m, n, k, c, decode, &tp))) return rc;
@@ -601,12 +663,51 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
         plan.args.ws = w.ws;
         plan.args.counters = w.counters;
     }
-#ifdef TUNA_TRACE
-    plan.args.trace = g_trace;
-#endif
     hipError_t e = launch_gemm(plan, stream);
     if (e != hipSuccess) return hip_fail(e, "gemm launch");
     return TUNA_OK;
+}
+
+// Config of a grouped launch chosen by the library.  Candidates, in order: the tuned entry for the
+// active rows if it is a streaming config the grouped variants can run as it stands; the derived
+// streaming config with its row tile shrunk until it divides m_group; one 64-row group per
+// workgroup with 8 waves along k, which runs any shape.  Table entries are never patched: a
+// narrow-row, many-token or deep-ring entry has no grouped counterpart.
+static int grouped_config(int m_group, int m_active, int max_tok, int k, int decode, tuna_gemm_config *out, GemmPlan *plan)
+{
+    auto runs = [&](const tuna_gemm_config &c) {
+        if (c.lds_tile_rows || is_narrow(c) || c.waves_m < 1 || c.rows_per_wave != kRowsPerLoad) return false;
+        if (m_group % (c.rows_per_wave * c.waves_m)) return false;
+        return plan_gemm(m_active, max_tok, k, c, decode, plan, 1) == TUNA_OK;
+    };
+    tuna_gemm_config c;
+    if (decode == TUNA_DECODE_GEMM) {
+        select_config(m_active, max_tok, k, &c, nullptr);
+        if (runs(c)) {
+            *out = c;
+            return TUNA_OK;
+        }
+    }
+    c = derive_streaming(m_active, max_tok < 64 ? max_tok : 64, k, decode);
+    while (c.waves_m > 1 && m_group % (c.rows_per_wave * c.waves_m)) --c.waves_m;
+    {
+        const int x_cap = 2 * c.waves_m * c.waves_k * 64;
+        while (c.x_chunk * c.token_tiles > x_cap && c.x_chunk / 2 >= kStepK * c.waves_k * c.prefetch) c.x_chunk /= 2;
+    }
+    if (runs(c)) {
+        *out = c;
+        return TUNA_OK;
+    }
+    memset(&c, 0, sizeof(c));
+    c.rows_per_wave = kRowsPerLoad, c.waves_m = 1, c.waves_k = 8, c.split_k = 1, c.prefetch = 2, c.x_chunk = 512;
+    c.token_tiles = max_tok <= 16 ? 1 : 2;
+    c.xcd_swizzle = 1;
+    if (runs(c)) {
+        *out = c;
+        return TUNA_OK;
+    }
+    return fail(TUNA_ERR_UNSUPPORTED, "no grouped config for m_group=%d, %d active rows, %d tokens, k=%d: %s", m_group, m_active,
+                max_tok, k, std::string(g_error).c_str());
 }
 
 // Grouped GEMM: n_groups stacked weight matrices of m_group rows, group e applied to the
@@ -647,23 +748,17 @@ static int matmul_grouped_impl(const void *q, const void *x, const void *code, c
         if (offsets[e + 1] > offsets[e]) act[n_active++] = (unsigned char)e;
     const int m_active = m_group * n_active;
     tuna_gemm_config c;
-    if (cfg) c = *cfg;
-    else {
-        select_config(m_active, max_tok, k, &c, nullptr);
-        if (c.lds_tile_rows) c = derive_config(m_active, 64, k);  // grouped launches use the streaming kernel
-        // the grouped kernels exist for 64 rows per wave and rings of 2 or 4 k-steps
-        c.rows_per_wave = kRowsPerLoad;
-        if (c.prefetch > 4) c.prefetch = 4;
-        // row tiles must not straddle groups: shrink the workgroup's row count until it divides m_group
-        while (m_group % (c.rows_per_wave * c.waves_m)) --c.waves_m;
-        const int x_cap = 2 * c.waves_m * c.waves_k * 64;
-        while (c.x_chunk * c.token_tiles > x_cap && c.x_chunk / 2 >= kStepK * c.waves_k * c.prefetch) c.x_chunk /= 2;
-        if (decode != TUNA_DECODE_GEMM) c.prefetch = 2;
-    }
-    if (m_group % (c.rows_per_wave * c.waves_m))
-        return fail(TUNA_ERR_UNSUPPORTED, "rows per workgroup (%d) must divide m_group=%d", c.rows_per_wave * c.waves_m, m_group);
     GemmPlan plan;
-    if ((rc = plan_gemm(m_active, max_tok, k, c, decode, &plan, 1))) return rc;
+    if (cfg) {
+        c = *cfg;
+        if (c.lds_tile_rows || is_narrow(c) || c.waves_m < 1)
+            return fail(TUNA_ERR_UNSUPPORTED, "grouped launches run the streaming kernel: rows_per_wave 64, waves_m >= 1, no lds_tile_rows");
+        if (m_group % (c.rows_per_wave * c.waves_m))
+            return fail(TUNA_ERR_UNSUPPORTED, "rows per workgroup (%d) must divide m_group=%d", c.rows_per_wave * c.waves_m, m_group);
+        if ((rc = plan_gemm(m_active, max_tok, k, c, decode, &plan, 1))) return rc;
+    } else if ((rc = grouped_config(m_group, m_active, max_tok, k, decode, &c, &plan))) {
+        return rc;
+    }
     GemmArgs &a = plan.args;
     a.q = static_cast<const uint8_t *>(q);
     a.x = x;
@@ -683,9 +778,6 @@ static int matmul_grouped_impl(const void *q, const void *x, const void *code, c
         a.ws = w.ws;
         a.counters = w.counters;
     }
-#ifdef TUNA_TRACE
-    a.trace = g_trace;
-#endif
     hipError_t e = launch_gemm(plan, stream);
     if (e != hipSuccess) return hip_fail(e, "grouped gemm launch");
     return TUNA_OK;
@@ -857,19 +949,40 @@ TUNA_EXPORT int tuna_select_config(int m, int n, int k, tuna_gemm_config *cfg, i
     return select_config(m, n, k, cfg, from_table);
 }
 
+TUNA_EXPORT int tuna_select_config_ex(int m, int n, int k, int decode_mode, tuna_gemm_config *cfg, int *from_table)
+{
+    if (!cfg) return fail(TUNA_ERR_INVALID_ARG, "cfg is null");
+    if (decode_mode != TUNA_DECODE_GEMM && decode_mode != TUNA_DECODE_DEQUANT)
+        return fail(TUNA_ERR_INVALID_ARG, "decode_mode %d is neither TUNA_DECODE_GEMM nor TUNA_DECODE_DEQUANT", decode_mode);
+    int rc = check_shape(m, n, k);
+    if (rc) return rc;
+    return select_config_for(m, n, k, decode_mode, cfg, from_table);
+}
+
+TUNA_EXPORT int tuna_select_config_grouped(int m_group, int n_active, int max_tokens, int k, int decode_mode,
+                                           tuna_gemm_config *cfg)
+{
+    if (!cfg) return fail(TUNA_ERR_INVALID_ARG, "cfg is null");
+    if (m_group <= 0 || n_active < 1 || n_active > kMaxGroups || max_tokens < 1 || m_group % kRowsPerLoad ||
+        (long long)m_group * n_active > 0x7fffffffLL)
+        return fail(TUNA_ERR_INVALID_ARG, "m_group=%d (a positive multiple of %d), n_active=%d (1..%d), max_tokens=%d (>= 1)",
+                    m_group, kRowsPerLoad, n_active, kMaxGroups, max_tokens);
+    int rc = check_shape(m_group * n_active, max_tokens, k);
+    if (rc) return rc;
+    GemmPlan plan;
+    return grouped_config(m_group, m_group * n_active, max_tokens, k, decode_mode, cfg, &plan);
+}
+
 TUNA_EXPORT int tuna_validate_config(int m, int n, int k, const tuna_gemm_config *cfg)
 {
     if (!cfg) return fail(TUNA_ERR_INVALID_ARG, "cfg is null");
-    if (cfg->lds_tile_rows) {
-        TiledPlan tp;
-        return plan_tiled(m, n, k, *cfg, TUNA_DECODE_GEMM, &tp);
-    }
-    if (is_narrow(*cfg)) {
-        NarrowPlan np;
-        return plan_narrow(m, n, k, *cfg, TUNA_DECODE_GEMM, &np);
-    }
-    GemmPlan plan;
-    return plan_gemm(m, n, k, *cfg, TUNA_DECODE_GEMM, &plan);
+    return validate_for(m, n, k, *cfg, TUNA_DECODE_GEMM);
+}
+
+TUNA_EXPORT int tuna_validate_config_ex(int m, int n, int k, const tuna_gemm_config *cfg, int decode_mode)
+{
+    if (!cfg) return fail(TUNA_ERR_INVALID_ARG, "cfg is null");
+    return validate_for(m, n, k, *cfg, decode_mode);
 }
 
 TUNA_EXPORT int tuna_config_footprint(int m, int n, int k, const tuna_gemm_config *cfg, size_t *lds_bytes,
@@ -1084,8 +1197,7 @@ TUNA_EXPORT int tuna_release_workspaces(void)
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     for (auto it = g_workspaces.begin(); it != g_workspaces.end();) {
         if (it->first.first == dev) {
-            if (it->second.ws) (void)hipFree(it->second.ws);
-            if (it->second.counters) (void)hipFree(it->second.counters);
+            free_workspace(it->second);
             it = g_workspaces.erase(it);
         } else {
             ++it;

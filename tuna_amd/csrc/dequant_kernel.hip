@@ -146,7 +146,8 @@ hipError_t launch_copy(const void *src, void *dst, size_t bytes, hipStream_t str
 // arithmetic: absmax = max |w| as fp32; normalized = fp32(w) / absmax with an fp32 division
 // (test.py:41, fp16 / fp32 promotes to fp32); index = argmin_j |normalized - code[j]| in
 // fp32, first index on ties (torch.argmin, test.py:50-53); nibble packing of test.py:55-65.
-// An all-zero row (the reference divides by zero there) gets index 7, the NF4 zero.
+// An all-zero row gets index 0: the reference divides by zero there, every candidate distance is
+// NaN, and torch.argmin over an all-NaN column returns index 0 (test.py:41-53).
 // One workgroup per block row (8 weight rows): 32 threads per row, 16-byte reads; a thread
 // turns 8 consecutive k of one row into one dword of the 32-byte record.
 __global__ __launch_bounds__(256) void quantize_kernel(const f16 *__restrict__ w, const float *__restrict__ code,
@@ -178,7 +179,7 @@ __global__ __launch_bounds__(256) void quantize_kernel(const f16 *__restrict__ w
         uint32_t d = 0;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            uint32_t best = 7;
+            uint32_t best = 0;
             if (amax > 0.f) {
                 const float nv = __fdiv_rn((float)v[e], amax);
                 float bd = fabsf(__fsub_rn(nv, c[0]));

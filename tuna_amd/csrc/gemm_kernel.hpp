@@ -280,20 +280,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     constexpr int RED_LIM = MINW >= 4 ? 0 : 32;  // LDS loads in flight per thread in the cross-wave sums (0: unbatched)
 
     const int tid = threadIdx.x;
-#ifdef TUNA_TRACE
-    // development builds: timestamps of the first tile go to 128 bytes of LDS behind the launch's
-    // own (global stores up here would turn the codebook's scalar loads into vector loads) and
-    // are copied out at the end of the tile
-    const unsigned long long t_entry_ = wall_clock64();
-#define TUNA_MARK(i) if (tid == 0 && tile_iter == 0) reinterpret_cast<unsigned long long *>(smem + a.lds_bytes)[i] = (i) == 0 ? t_entry_ : wall_clock64();
-#else
-#define TUNA_MARK(i)
-#endif
-    int tile_iter = 0;
-#ifdef TUNA_TRACE
-    if (tid < 32) reinterpret_cast<unsigned long long *>(smem + a.lds_bytes)[tid] = 0ull;
-#endif
-    TUNA_MARK(0)
     // Every kernel argument the first tile needs is requested here, in one batch with one wait:
     // left to itself the compiler fetches them where they are first used, three to four
     // dependent round trips to memory before the first weight load can be issued.  (Not a
@@ -467,29 +453,16 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
     TUNA_SKIP_EMPTY(t)
     if (t < t_end) {
         TUNA_TILE_FETCH(t)
-#if defined(TUNA_TRACE) && TUNA_TRACE_EXP == 1
-        TUNA_MARK(16)
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        TUNA_MARK(17)
-#endif
         if constexpr (!GRP) TUNA_TILE_SMALL_LOADS()
-#if defined(TUNA_TRACE) && TUNA_TRACE_EXP == 2
-        TUNA_MARK(16)
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        TUNA_MARK(17)
-#endif
-        TUNA_MARK(1)
         // ---- decode table, once per workgroup, built while the first tile's loads are in flight
         float code_lane = 0.f;  // (a select between two loads would be turned back into a vector load)
 #pragma unroll
         for (int i = 0; i < 16; ++i) code_lane = i16 == i ? code_s[i] : code_lane;
-        TUNA_MARK(14)
         if constexpr (DEC == TUNA_DECODE_GEMM) {
             // Lane l holds fp16(code[l % 16]) (kernel.cu:2800 rounds the codebook to fp16);
             // entries are gathered across lanes, no memory traffic.
             // piece p: 16 bytes of row (p >> 4); all 64 slots of a row hold the same half2
             const int code_bits = (int)f16_bits((f16)code_lane);
-            TUNA_MARK(15)
             // four pieces per thread and round: the eight cross-lane reads of a round are in
             // flight together instead of one LDS round trip per piece
             for (int p0 = tid; p0 < kLutBytes / 16; p0 += 4 * nthreads) {
@@ -510,7 +483,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
         } else {
             if (tid < 16) reinterpret_cast<float *>(lut)[tid] = code_lane;
         }
-        TUNA_MARK(2)
     }
 
     // One k-step of this wave: B fragments from LDS, decode 4*RW dwords, 4*RW*TT MFMAs.
@@ -581,7 +553,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
         // The explicit wait makes "nothing pending" a fact on every path.
         __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));
         __syncthreads();
-        TUNA_MARK(3)
 
         for (int c = 0; c < n_chunks; ++c) {
             const int it_chunk0 = c * ipc;
@@ -627,12 +598,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                 }
             }
         }
-        TUNA_MARK(4)
-#ifdef TUNA_TRACE
-        if (lane == 0 && tile_iter == 0) {  // latest wave of the workgroup out of the main loop
-            atomicMax(reinterpret_cast<unsigned long long *>(smem + a.lds_bytes) + 10, (unsigned long long)wall_clock64());
-        }
-#endif
 
         // ---- next tile: get its loads going before this tile's reduction and store ---------
         if constexpr (ONE) {
@@ -726,17 +691,10 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                     }
                 }
             }
-#ifdef TUNA_TRACE
-            TUNA_MARK(9)
-            if (a.trace && tid < 32 && tile_iter == 0)
-                a.trace[(size_t)blockIdx.x * 8 * 16 + tid] = reinterpret_cast<unsigned long long *>(smem + a.lds_bytes)[tid];
-#endif
-            ++tile_iter;
             if constexpr (MODE == 0) if (t < t_end) TUNA_TILE_SMALL_LOADS()
             continue;
         }
         __syncthreads();  // every wave has left the main loop: the work area is free
-        TUNA_MARK(11)
 #pragma unroll
         for (int rw = 0; rw < RW; ++rw)
 #pragma unroll
@@ -750,9 +708,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                         reinterpret_cast<f32x4 *>(buf + j * plane_floats)[(size_t)(wm_e * a.waves_k + wk_e) * 64 + lane_e] =
                             acc[rw][j][tt];
                     __syncthreads();
-                    TUNA_MARK(12)
                     sum_planes_any<4, RED_LIM>(a.wk_log2, buf, plane_floats, wm_e, wk_e, lane_e, o, 0);
-                    TUNA_MARK(13)
                 } else {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
@@ -779,7 +735,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                     }
                 }
             }
-        TUNA_MARK(5)
 
         if (partial) {
             // Partials travel as device-scope relaxed atomics (write-through stores, L2-bypassing
@@ -790,12 +745,10 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
             __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): a workgroup-scope fence does not wait for global stores
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
             __syncthreads();  // also: every read of the reduction buffers is done
-            TUNA_MARK(6)
             volatile unsigned *ticket = reinterpret_cast<volatile unsigned *>(work);
             if (wk_e + wm_e == 0 && lane_e == 0)
                 *ticket = __hip_atomic_fetch_add(a.counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __syncthreads();
-            TUNA_MARK(7)
             write_out = *ticket == n_contrib - 1u;
             if (write_out) {
                 // last workgroup of this row tile: every partial is in memory; add them in k order
@@ -837,13 +790,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
                     }
             }
         }
-        TUNA_MARK(8)
-        TUNA_MARK(9)
-#ifdef TUNA_TRACE
-        if (a.trace && tid < 32 && tile_iter == 0)
-            a.trace[(size_t)blockIdx.x * 8 * 16 + tid] = reinterpret_cast<unsigned long long *>(smem + a.lds_bytes)[tid];
-#endif
-        ++tile_iter;
         if constexpr (MODE == 0) if (t < t_end) TUNA_TILE_SMALL_LOADS()
     }
 #undef TUNA_GROUP
@@ -852,7 +798,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_kernel(const GemmArgs a)
 #undef TUNA_SKIP_EMPTY
 #undef TUNA_TILE_SMALL_LOADS
 #undef TUNA_LOAD_STEP
-#undef TUNA_MARK
 }
 
 }  // namespace tuna

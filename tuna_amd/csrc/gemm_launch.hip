@@ -74,10 +74,6 @@ bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int 
 // ---- lean twins (gemm_lean.hpp) -------------------------------------------------------------
 typedef void (*LeanKernelFn)(const uint8_t *, const void *, const float *, const float *, int, int, int, int, int,
                              void *, const void *, float *, unsigned *, int
-#ifdef TUNA_TRACE
-                             ,
-                             unsigned long long *
-#endif
 );
 struct LeanVariant {
     int wk, u, maxt;
@@ -186,10 +182,6 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
         hipLaunchKernelGGL(lv->fn, plan.grid, dim3(plan.threads), lean_lds_bytes(plan), stream, a.q, a.x, a.code, a.absmax,
                            a.k, a.n, a.steps_per_split, packed, a.m, a.out, a.residual, a.ws, a.counters,
                            a.row_tiles
-#ifdef TUNA_TRACE
-                           ,
-                           a.trace
-#endif
         );
         g_lean_launches.fetch_add(1, std::memory_order_relaxed);
         return hipGetLastError();
@@ -215,11 +207,7 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
     // persistent workgroups: as many as the device holds at once, each walks tiles with this stride
     dim3 grid = plan.grid;
     if (grid.x > slots) grid.x = slots;
-#ifdef TUNA_TRACE
-    hipLaunchKernelGGL(v->fn, grid, dim3(plan.threads), plan.lds_bytes + 256, stream, plan.args);  // + timestamps
-#else
     hipLaunchKernelGGL(v->fn, grid, dim3(plan.threads), plan.lds_bytes, stream, plan.args);
-#endif
     return hipGetLastError();
 }
 

@@ -53,9 +53,6 @@ struct LeanArgs {
     float *ws;
     unsigned *counters;
     int row_tiles;
-#ifdef TUNA_TRACE
-    unsigned long long *trace;
-#endif
 };
 
 template <int WK, int U, int MAXT, int MINW>
@@ -64,10 +61,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
                                                                int a_packed, int a_m, void *a_out,
                                                                const void *a_residual, float *a_ws, unsigned *a_counters,
                                                                int a_row_tiles
-#ifdef TUNA_TRACE
-                                                               ,
-                                                               unsigned long long *a_trace
-#endif
 )
 {
     struct {
@@ -80,18 +73,11 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
         float *ws;
         unsigned *counters;
         int m, n, k, steps_per_split, row_tiles, split_log2, split_k, waves_m, xcd_swizzle, epilogue;
-#ifdef TUNA_TRACE
-        unsigned long long *trace;
-#endif
     } const a = {a_q,           a_x,          a_code,          a_absmax,
                  a_out,         a_residual,   a_ws,            a_counters,
                  a_m,           a_n,          a_k,             a_sps,
                  a_row_tiles,   a_packed & 15, 1 << (a_packed & 15), (a_packed >> 4) & 31,
                  (a_packed >> 11) & 1, (a_packed >> 9) & 3
-#ifdef TUNA_TRACE
-                 ,
-                 a_trace
-#endif
     };
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int WK_LOG2 = WK == 1 ? 0 : WK == 2 ? 1 : WK == 4 ? 2 : WK == 8 ? 3 : 4;
@@ -100,20 +86,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
     unsigned char *work = smem + kLutBytes;
 
     const int tid = threadIdx.x;
-#ifdef TUNA_TRACE
-    // development builds: timestamps of wave 0 in scalar registers, written out at the end
-    unsigned long long tm_[10] = {};
-#define TUNA_LMARK(i) tm_[i] = wall_clock64();
-#define TUNA_LDUMP()                                                                            \
-    if (a.trace && tid == 0) {                                                                 \
-        tm_[9] = wall_clock64();                                                               \
-        for (int i_ = 0; i_ < 10; ++i_) a.trace[(size_t)blockIdx.x * 128 + i_] = tm_[i_];      \
-    }
-#else
-#define TUNA_LMARK(i)
-#define TUNA_LDUMP()
-#endif
-    TUNA_LMARK(0)
     const int lane = tid & 63;
     const int i16 = lane & 15;
     const int g = lane >> 4;
@@ -175,7 +147,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
     for (int u = 0; u < U; ++u)
         wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(qp + (size_t)u * (WK * 128) + lb));
     qp += (size_t)U * (WK * 128);
-    TUNA_LMARK(1)
     // ---- decode table (see gemm_kernel.hpp), built while the loads are in flight ------------
     {
         const int code_bits = (int)f16_bits((f16)code_lane);
@@ -195,7 +166,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
             }
         }
     }
-    TUNA_LMARK(2)
     f16x2 sc16[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -215,7 +185,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
                 *reinterpret_cast<u32x4 *>(x_dst + (size_t)(x_wv0 + b * x_dwv) * 1024) = x_row_ok ? xv[b] : u32x4{0u, 0u, 0u, 0u};
     }
     __syncthreads();
-    TUNA_LMARK(3)
 
     // ---- main loop: n_it / U ring turns, the last one without refills ------------------------
     f32x4 acc[4];
@@ -246,7 +215,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
 #pragma unroll
     for (int u = 0; u < U; ++u) TUNA_LEAN_CONSUME(u)
 #undef TUNA_LEAN_CONSUME
-    TUNA_LMARK(4)
 
     // ---- reduction and store (layouts of gemm_kernel) ----------------------------------------
     f16 *outp = reinterpret_cast<f16 *>(a.out);
@@ -287,7 +255,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
     __syncthreads();
     float o[4][4];
     sum_planes<WK, 4, 32>(redf, plane_floats, wm, wk, lane, o, 0);
-    TUNA_LMARK(5)
 
     const size_t seg_floats = (size_t)a.waves_m * 1024;  // partial sums of one workgroup: [wm][f][j]
     const size_t tile_id = (size_t)blockIdx.y * a.row_tiles + row_tile;
@@ -320,18 +287,14 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
-    TUNA_LMARK(6)
     volatile unsigned *ticket = reinterpret_cast<volatile unsigned *>(work);
     if (tid == 0) *ticket = __hip_atomic_fetch_add(a.counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    TUNA_LMARK(7)
     if (*ticket != (unsigned)a.split_k - 1u) {
-        TUNA_LDUMP()
         return;
     }
     if (tid == 0) __hip_atomic_store(a.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (!owner) {
-        TUNA_LDUMP()
         return;
     }
 #pragma unroll
@@ -345,7 +308,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
 #pragma unroll
             for (int b = 0; b < 4; ++b) ps[b] = src + (size_t)min(sp0 + b, a.split_k - 1) * seg_floats;
             load_partials4(ps[0], ps[1], ps[2], ps[3], p[0], p[1], p[2], p[3]);
-            TUNA_LMARK(8)
 #pragma unroll
             for (int b = 0; b < 4; ++b)
                 if (sp0 + b < a.split_k) s4 += p[b];
@@ -356,7 +318,6 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_lean_kernel(const uint8_t *a_
             store_features4(outp, resp, a.epilogue, (size_t)tok, out_ld, row0 + (l >> 4) * 16 + v * 4, s4[0], s4[1], s4[2],
                             s4[3]);
     }
-    TUNA_LDUMP()
 }
 
 }  // namespace tuna

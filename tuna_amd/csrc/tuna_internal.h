@@ -5,6 +5,7 @@
 #include <stdint.h>
 
 #include "../../include/tuna_amd.h"
+#include "../../include/tuna_amd_bench.h"
 
 namespace tuna {
 
@@ -61,9 +62,6 @@ struct GemmArgs {
     int tiles_per_group;
     int tok_off[kMaxGroups + 1];
     unsigned char act[kMaxGroups];
-#ifdef TUNA_TRACE
-    unsigned long long *trace;  // development builds only: 16 timestamps per workgroup
-#endif
 };
 
 // ---------------------------------------------------------------------------------------

@@ -107,6 +107,8 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
             raise ValueError("the narrow-row kernel needs waves_m=1 (0 with rows_per_wave 64), split_k=1, k_stagger=0")
         if (c["rows_per_wave"], c["waves_k"], c["prefetch"], c["token_tiles"]) not in NARROW_VARIANTS:
             raise ValueError("no narrow-row kernel for this rows_per_wave / waves_k / prefetch / token_tiles")
+        if c["x_chunk"] != STEP_K * c["waves_k"] * c["prefetch"]:
+            raise ValueError("the narrow-row kernel stages no x: x_chunk must be 32*waves_k*prefetch, the k of one ring turn")
         if m % c["rows_per_wave"] or k % (STEP_K * c["waves_k"] * c["prefetch"]):
             raise ValueError("rows_per_wave 16 or 32 needs m a multiple of it and k a multiple of 32*waves_k*prefetch")
         if m * k // 2 >= 1 << 32 or k * 32 >= 1 << 32:

@@ -169,17 +169,26 @@ def quantize(w, codebook=None):
     return q, absmax, code
 
 
-def select_config(m: int, n: int, k: int):
+def select_config(m: int, n: int, k: int, decode_mode: int = _lib.DECODE_GEMM):
     """(GemmConfig, from_table) the library would use for shape (m, n, k).  Host only."""
     cfg = GemmConfig()
     hit = ctypes.c_int(0)
-    _lib.check(_lib.lib().tuna_select_config(int(m), int(n), int(k), ctypes.byref(cfg), ctypes.byref(hit)))
+    _lib.check(_lib.lib().tuna_select_config_ex(int(m), int(n), int(k), int(decode_mode), ctypes.byref(cfg),
+                                                ctypes.byref(hit)))
     return cfg, bool(hit.value)
 
 
-def validate_config(m: int, n: int, k: int, cfg: GemmConfig) -> None:
+def select_config_grouped(m_group: int, n_active: int, max_tokens: int, k: int, decode_mode: int = _lib.DECODE_GEMM):
+    """GemmConfig matmul_grouped(config=None) runs for n_active groups with tokens.  Host only."""
+    cfg = GemmConfig()
+    _lib.check(_lib.lib().tuna_select_config_grouped(int(m_group), int(n_active), int(max_tokens), int(k),
+                                                     int(decode_mode), ctypes.byref(cfg)))
+    return cfg
+
+
+def validate_config(m: int, n: int, k: int, cfg: GemmConfig, decode_mode: int = _lib.DECODE_GEMM) -> None:
     """Raises TunaError unless `cfg` can run shape (m, n, k).  Host only."""
-    _lib.check(_lib.lib().tuna_validate_config(int(m), int(n), int(k), ctypes.byref(cfg)))
+    _lib.check(_lib.lib().tuna_validate_config_ex(int(m), int(n), int(k), ctypes.byref(cfg), int(decode_mode)))
 
 
 def config_footprint(m: int, n: int, k: int, cfg: GemmConfig):
