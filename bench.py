@@ -38,15 +38,32 @@ HEADLINE = "mistral_qkv"
 TOKENS = 16
 CACHE_BYTES = 256 << 20  # Infinity Cache; the rotation streams at least twice this between re-uses
 
-# HBM bytes per launch of the GEMM kernel measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE,
-# each scaled by the same counter's reading for the copy kernel of known size); filled in from
-# the summaries under profiles/.  None = not measured for that shape.
-MEASURED_TRAFFIC_BYTES = {
-    # workload: FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 (KiB -> bytes),
+# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE in KiB per dispatch, each
+# scaled by the same counter's reading for the copy kernel of known size: factors 2.000 and 1.000), from the
+# summaries under profiles/.  Keyed by shape AND by the kernel the profile was taken of: when the table or
+# the dispatcher picks another kernel for the shape, the entry no longer applies and `traffic` is null.
+MEASURED_TRAFFIC = {
     # profiles/gemm_narrow_kernel_and_gemm_kernel_hbm_traffic_counters.md
-    "mistral_qkv": int((6702.5 * 2.000 + 192.0 * 1.000) * 1024),
-    "mixtral_gate_up_8e": int((230494.3 * 2.000 + 7168.1 * 1.000) * 1024),
+    ("mistral_qkv", "gemm_narrow_kernel<LW=2,WK=8,U=4,PERM=1,TT=1>"): (6702.5, 192.0),
+    ("mixtral_gate_up_8e", "gemm_kernel<RW=1,U=4,TT=1,DEC=1,1024 threads,4 waves/SIMD,MODE=2> split_k=1"): (230494.3, 7168.1),
 }
+
+
+def traffic_bytes(shape_name, kernel):
+    kib = MEASURED_TRAFFIC.get((shape_name, kernel))
+    return int((kib[0] * 2.000 + kib[1] * 1.000) * 1024) if kib else None
+
+
+def roofline_block(shape_name, r):
+    """The `roofline` object of one timed shape `r` (a time_shape result)."""
+    return {
+        "bound": "hbm", "achieved": r["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(r["gbs"] / HBM_PEAK_GBS, 4),
+        "traffic": traffic_bytes(shape_name, r["kernel"]) if r["n"] == TOKENS else None,
+        "kernel": "tuna::" + r["kernel"],
+        "algorithmic_bytes_per_launch": r["packed_bytes"],
+        "avg_launch_us": r["us_per_gemm"],
+    }
 
 
 def n_sets_for(bytes_per_set: int, cap_bytes: int) -> int:
@@ -54,8 +71,9 @@ def n_sets_for(bytes_per_set: int, cap_bytes: int) -> int:
     return max(2, min(n, max(2, cap_bytes // bytes_per_set)))
 
 
-def time_shape(ops, synth, torch, dev, m, n, k, steps, warmup, seed0=0, use_graph=False, cfg=None, sets=None):
-    """-> dict with us_per_gemm, GB/s, TFLOP/s, roofline fraction for one shape."""
+def time_shape(ops, synth, torch, dev, m, n, k, steps, warmup, seed0=0, use_graph=False, cfg=None, sets=None, settle=0):
+    """-> dict with us_per_gemm, GB/s, TFLOP/s, roofline fraction for one shape.  `settle` untimed
+    launches run before the warm-up (clocks and caches of a box that has just been idle)."""
     bytes_w = m * k // 2
     if sets is None:
         ns = n_sets_for(bytes_w, 24 << 30)
@@ -68,6 +86,8 @@ def time_shape(ops, synth, torch, dev, m, n, k, steps, warmup, seed0=0, use_grap
     code = nf4_codebook(dev)
     out = torch.empty((n, m), dtype=torch.float16, device=dev)
     torch.cuda.synchronize()
+    if settle > 0:
+        ops.time_matmul(qs, ams, x, code, out, m, n, k, config=cfg, warmup=0, iters=settle, use_graph=False)
     ms = ops.time_matmul(qs, ams, x, code, out, m, n, k, config=cfg, warmup=warmup, iters=steps, use_graph=use_graph)
     us = ms * 1000.0 / steps
     gbs = bytes_w / (us * 1e-6) / 1e9
@@ -78,6 +98,7 @@ def time_shape(ops, synth, torch, dev, m, n, k, steps, warmup, seed0=0, use_grap
         "tflops": round(2.0 * m * n * k / (us * 1e-6) / 1e12, 2),
         "config": (cfg or used).to_dict(), "config_from_table": bool(hit) if cfg is None else None,
         "launch": "graph" if use_graph else "stream",
+        "kernel": ops.describe_launch(m, n, k, cfg),
     }
 
 
@@ -112,24 +133,85 @@ def cpu_baseline(m, n, k, budget_s=12.0):
     bytes_w = m * k // 2
     return {
         "value": round(bytes_w / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-        "sample": f"{len(times)} full GEMMs m={m} n={n} k={k} (decode to fp16, then fp32-accumulate matmul), "
-                  f"median of total; oracle/tuna_oracle.c with OpenMP",
+        "sample": f"benchmark config 0, seed 0: {len(times)} full GEMMs m={m} n={n} k={k} (decode to fp16, then "
+                  f"fp32-accumulate matmul), median of total; oracle/tuna_oracle.c with OpenMP",
         "us_per_gemm": round(med * 1e6, 1), "us_decode": round(float(np.median(dec)) * 1e6, 1),
         "us_matmul": round(float(np.median(mat)) * 1e6, 1),
         "single_thread_us_per_gemm": round((td1 + tm1) * 1e6, 1),
     }
 
 
-def probe_is_mid(make_configs, m, k, c):
-    """True if an unsplit one-token-tile launch that took a twin took the streaming one: the lean kernel is
-    tried first and takes every launch whose tiles are all resident at once (lean_applies in gemm_launch.hip)."""
-    if not make_configs.mid_applies(m, k, {f: c.get(f, 0) for f in make_configs.FIELDS}):
-        return False
-    waves = c["waves_m"] * c["waves_k"]
-    sps = k // 32
-    lds = 65536 + max(sps * 1024, waves * 4096) + 16
-    slots = 256 * min(make_configs.LDS_LIMIT // lds, max(1, 20 // waves)) if lds <= make_configs.LDS_LIMIT else 0
-    return m // (64 * c["waves_m"]) > slots or sps * 64 > 8 * 64 * waves
+READ_VARIANTS = {0: "nontemporal x8", 1: "plain x8", 2: "nontemporal x16", 3: "plain x16", 4: "nontemporal x4", 5: "plain x4"}
+
+
+def read_sweep(ops, torch, dev, nbytes=2 << 30, iters=5):
+    """Rate of the read-only kernel over `nbytes` for every (workgroups, variant): {label: GB/s}."""
+    big = torch.full((nbytes,), 3, dtype=torch.uint8, device=dev)
+    out = {}
+    for variant, vname in READ_VARIANTS.items():
+        for blocks in (256, 512, 1024, 2048, 4096, 8192):
+            ms = ops.time_read(big, blocks=blocks, variant=variant, warmup=2, iters=iters) / iters
+            out[f"{vname}, {blocks} workgroups"] = round(nbytes / (ms * 1e-3) / 1e9, 1)
+    del big
+    torch.cuda.empty_cache()
+    return out
+
+
+def launch_floor(ops, torch, dev, headline_bytes):
+    tiny = torch.zeros(4096, dtype=torch.uint8, device=dev)
+    us_empty = ops.time_read(tiny, blocks=192, warmup=100, iters=1000) * 1000.0 / 1000
+    sweep = read_sweep(ops, torch, dev)
+    best = max(sweep, key=sweep.get)
+    rate = sweep[best]
+    return {
+        "empty_launch_us": round(us_empty, 3),
+        "read_kernel_gbs": rate,
+        "read_kernel_best": best,
+        "read_kernel_frac_of_peak": round(rate / HBM_PEAK_GBS, 4),
+        "read_kernel_sweep_gbs": sweep,
+        "headline_bytes_at_read_rate_us": round(headline_bytes / rate / 1e3, 3),
+        "floor_us": round(us_empty + headline_bytes / rate / 1e3, 3),
+    }
+
+
+def time_dequant_shapes(ops, synth, torch, dev, names=("mistral_attn_out", "mistral_gate_up", "llama70b_down")):
+    from tuna_amd.quantize import nf4_codebook
+
+    deq = {}
+    for nm in names:
+        dm, dk = synth.SHAPES[nm]
+        sets = [synth.make_weights_torch(dm, dk, 50 + i, dev) for i in range(max(2, min(8, (1 << 30) // (dm * dk // 2))))]
+        img = torch.empty((dm, dk), dtype=torch.float16, device=dev)
+        ms = ops.time_dequant([s[0] for s in sets], [s[1] for s in sets], nf4_codebook(dev), img, dm, dk, 10, 100)
+        us = ms * 10.0
+        gbs = 2.5 * dm * dk / (us * 1e-6) / 1e9
+        deq[nm] = {"m": dm, "k": dk, "us": round(us, 2), "gbs_in_plus_out": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
+                   "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "tuna::dequant_kernel",
+                                "algorithmic_bytes_per_launch": int(2.5 * dm * dk), "avg_launch_us": round(us, 2)}}
+        del sets, img
+        torch.cuda.empty_cache()
+    return deq
+
+
+def time_quantize(ops, synth, torch, dev):
+    qm, qk = synth.SHAPES["mistral_attn_out"]
+    wq_ = (torch.randn((qm, qk), device=dev) * 0.02).to(torch.float16)
+    for _ in range(3):
+        ops.quantize(wq_)
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(20):
+        ops.quantize(wq_)
+    ev1.record()
+    torch.cuda.synchronize()
+    us = ev0.elapsed_time(ev1) * 1000.0 / 20
+    gbs = 2.5 * qm * qk / (us * 1e-6) / 1e9       # fp16 weights in (2 bytes each), packed codes out (half a byte each)
+    return {"m": qm, "k": qk, "us": round(us, 2), "gbs_fp16_in": round(2.0 * qm * qk / (us * 1e-6) / 1e9, 1),
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "tuna::quantize_kernel",
+                         "algorithmic_bytes_per_launch": int(2.5 * qm * qk), "avg_launch_us": round(us, 2)}}
 
 
 def main():
@@ -144,6 +226,10 @@ def main():
     ap.add_argument("--workload", default=HEADLINE, help="shape name timed as the headline (profiling runs)")
     ap.add_argument("--tokens", type=int, default=TOKENS, help="token count of the headline workload")
     ap.add_argument("--launch", choices=("both", "stream", "graph"), default="both")
+    ap.add_argument("--settle", type=int, default=300,
+                    help="untimed launches before the warm-up of the headline (a box that was idle ramps its clocks)")
+    ap.add_argument("--only", choices=("read", "dequant", "quantize"), default=None,
+                    help="profiling runs: launch only the read-kernel sweep / the dequant kernel / the quantizer")
     ap.add_argument("--copy-yardstick", type=int, default=0, metavar="MIB",
                     help="also launch the plain copy kernel over MIB mebibytes (counter runs: the known-traffic "
                          "launch the HBM counters of the GEMM kernel are scaled by)")
@@ -164,34 +250,25 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.only:
+        if args.only == "read":
+            res = {"read_kernel_sweep_gbs": read_sweep(ops, torch, dev)}
+        elif args.only == "dequant":
+            res = {"dequant": time_dequant_shapes(ops, synth, torch, dev)}
+        else:
+            res = {"quantize": time_quantize(ops, synth, torch, dev)}
+        print(json.dumps(res))
+        return
+
     m, k = synth.SHAPES[args.workload]
     n = args.tokens
     res_stream = res_graph = None
     if args.launch in ("both", "stream"):
-        res_stream = time_shape(ops, synth, torch, dev, m, n, k, args.steps, args.warmup, use_graph=False)
+        res_stream = time_shape(ops, synth, torch, dev, m, n, k, args.steps, args.warmup, use_graph=False, settle=args.settle)
     if args.launch in ("both", "graph"):
-        res_graph = time_shape(ops, synth, torch, dev, m, n, k, args.steps, args.warmup, use_graph=True)
+        res_graph = time_shape(ops, synth, torch, dev, m, n, k, args.steps, args.warmup, use_graph=True, settle=args.settle)
     cands = [r for r in (res_stream, res_graph) if r is not None]
     head = min(cands, key=lambda r: r["us_per_gemm"])
-    # which kernel family the headline config runs (the profiles name the same kernel)
-    hc = head["config"]
-    if hc.get("lds_tile_rows"):
-        kernel_name = "tuna::gemm_tiled_kernel"
-    elif hc["rows_per_wave"] < 64:
-        kernel_name = "tuna::gemm_narrow_kernel"
-    else:
-        before = ops.lean_launches()
-        probe = time_shape(ops, synth, torch, dev, m, n, k, 2, 1, use_graph=False)
-        twin = ops.lean_launches() > before      # counts both stripped-down twins of the general kernel
-        from tuna_amd import make_configs
-        if twin and (hc.get("token_tiles", 1) > 1 or probe_is_mid(make_configs, m, k, hc)):
-            kernel_name = "tuna::gemm_mid_kernel"
-        elif twin:
-            kernel_name = "tuna::gemm_lean_kernel"
-        else:
-            kernel_name = "tuna::gemm_kernel"
-        del probe
-
     line = {
         "metric": METRIC,
         "value": head["gbs"],
@@ -215,39 +292,18 @@ def main():
             "tile_config": head["config"],
             "launch": head["launch"],
         },
-        "roofline": {
-            "bound": "hbm",
-            "achieved": head["gbs"],
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": round(head["gbs"] / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if n == TOKENS else None,
-            "kernel": kernel_name,
-            "algorithmic_bytes_per_launch": head["packed_bytes"],
-            "avg_launch_us": head["us_per_gemm"],
-        },
+        "roofline": roofline_block(args.workload, head),
         "headline_stream_launch": res_stream,
         "headline_graph_launch": res_graph,
     }
 
     # Yardsticks for the fixed cost of a launch, measured in the same run: back-to-back launches of a
     # read kernel over 4 KB (nothing to stream: the time per launch is what any kernel pays on this box)
-    # and the rate of the same kernel over 512 MB.  A launch that streams the headline's packed bytes
-    # at that rate cannot take less than their sum.
+    # and the best rate a read-only kernel reaches over 2 GB (sweep over workgroup counts, loads in flight
+    # and nontemporal / plain loads).  A launch that streams the headline's packed bytes at that rate
+    # cannot take less than their sum.
     if not args.only_headline:
-        tiny = torch.zeros(4096, dtype=torch.uint8, device=dev)
-        big = torch.full((512 << 20,), 3, dtype=torch.uint8, device=dev)
-        us_empty = ops.time_read(tiny, blocks=192, warmup=100, iters=1000) * 1000.0 / 1000
-        ms_big = ops.time_read(big, warmup=3, iters=10) / 10
-        rate = big.numel() / (ms_big * 1e-3) / 1e9
-        line["launch_floor"] = {
-            "empty_launch_us": round(us_empty, 3),
-            "read_kernel_gbs": round(rate, 1),
-            "headline_bytes_at_read_rate_us": round(head["packed_bytes"] / rate / 1e3, 3),
-            "floor_us": round(us_empty + head["packed_bytes"] / rate / 1e3, 3),
-        }
-        del tiny, big
-        torch.cuda.empty_cache()
+        line["launch_floor"] = launch_floor(ops, torch, dev, head["packed_bytes"])
 
     if args.copy_yardstick > 0:
         nb = args.copy_yardstick << 20
@@ -268,41 +324,13 @@ def main():
             best = r_g if r_g["us_per_gemm"] < r_s["us_per_gemm"] else r_s
             best["us_stream"] = r_s["us_per_gemm"]
             best["us_graph"] = r_g["us_per_gemm"]
+            best["roofline"] = roofline_block(name, best)
             shapes[name] = best
             torch.cuda.empty_cache()
         line["shapes"] = shapes
         line["min_frac_hbm_over_shapes"] = min(v["frac_hbm"] for v in shapes.values())
-        # dequant kernel (k*m/2 bytes in, 2*k*m bytes out) on the 4096 x 4096 config
-        from tuna_amd.quantize import nf4_codebook
-
-        deq = {}
-        for nm in ("mistral_attn_out", "mistral_gate_up", "llama70b_down"):
-            dm, dk = synth.SHAPES[nm]
-            sets = [synth.make_weights_torch(dm, dk, 50 + i, dev) for i in range(max(2, min(8, (1 << 30) // (dm * dk // 2))))]
-            img = torch.empty((dm, dk), dtype=torch.float16, device=dev)
-            ms = ops.time_dequant([s[0] for s in sets], [s[1] for s in sets], nf4_codebook(dev), img, dm, dk, 10, 100)
-            us = ms * 10.0
-            deq[nm] = {"m": dm, "k": dk, "us": round(us, 2),
-                       "gbs_in_plus_out": round(2.5 * dm * dk / (us * 1e-6) / 1e9, 1),
-                       "frac_hbm": round(2.5 * dm * dk / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
-            del sets, img
-            torch.cuda.empty_cache()
-        line["dequant"] = deq
-        # device quantizer + packer on one shape (fp16 weights read twice, packed bytes written once)
-        qm, qk = synth.SHAPES["mistral_attn_out"]
-        wq_ = (torch.randn((qm, qk), device=dev) * 0.02).to(torch.float16)
-        for _ in range(3):
-            ops.quantize(wq_)
-        torch.cuda.synchronize()
-        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        ev0.record()
-        for _ in range(20):
-            ops.quantize(wq_)
-        ev1.record()
-        torch.cuda.synchronize()
-        us = ev0.elapsed_time(ev1) * 1000.0 / 20
-        line["quantize"] = {"m": qm, "k": qk, "us": round(us, 2), "gbs_fp16_in": round(2.0 * qm * qk / (us * 1e-6) / 1e9, 1)}
-        del wq_
+        line["dequant"] = time_dequant_shapes(ops, synth, torch, dev)
+        line["quantize"] = time_quantize(ops, synth, torch, dev)
 
     if not args.no_shapes:
         # Mixtral gate+up with a router: 16 tokens x top-2 = 32 (token, expert) rows spread over the 8
@@ -368,7 +396,9 @@ def main():
         line["sweeps"] = sweeps
 
     if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline(m, n, k)
+        # benchmark configuration 0: the CPU path on the Mistral attention out-proj shape, 16 tokens, seed 0
+        cm, ck = synth.SHAPES["mistral_attn_out"]
+        line["cpu_baseline"] = cpu_baseline(cm, TOKENS, ck)
     else:
         line["cpu_baseline"] = None
 

@@ -41,10 +41,19 @@ int tuna_time_copy(const void *src, void *dst, size_t bytes, int warmup, int ite
                    void *stream, float *elapsed_ms);
 
 /* Read-only streaming kernel over `bytes` bytes of `src` (16-byte multiples), `blocks`
- * workgroups of 256 threads (0 = default): the ceiling a pure HBM reader reaches on the
- * device, reported beside the GEMM's rate.  `sink` is 4 writable bytes. */
-int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int warmup, int iters,
-                   void *stream, float *elapsed_ms);
+ * workgroups of 256 threads (0 = 2048): the ceiling a pure HBM reader reaches on the device,
+ * reported beside the GEMM's rate.  `variant`: 0 nontemporal loads, 8 in flight per lane;
+ * 1 plain loads, 8; 2 nontemporal, 16; 3 plain, 16; 4 nontemporal, 4; 5 plain, 4.  `sink` is
+ * 4 writable bytes. */
+int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int variant, int warmup,
+                   int iters, void *stream, float *elapsed_ms);
+
+/* Name and template arguments of the kernel a GEMM launch would start (cfg NULL = the library's
+ * choice), e.g. "gemm_narrow_kernel<LW=2,WK=8,U=4,PERM=1,TT=1>": what the bench writes beside a
+ * timing so that it can be matched with a profile.  Host only; with a device present the
+ * device's CU count decides between twins, otherwise 256 CUs are assumed. */
+int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config *cfg, int decode_mode,
+                         char *buf, size_t len);
 
 /* Diagnostic switch, process-wide, default on: dense launches that qualify run one of two
  * kernels stripped of everything else the general one carries - small launches (one workgroup

@@ -81,7 +81,8 @@ SIGNATURES = {
     "tuna_time_matmul_grouped": (_i, [_vpp, _vpp, _i, _vp, _vp, _vp, _i, _i, _i, _ip, _cfgp, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_dequant": (_i, [_vpp, _vpp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_copy": (_i, [_vp, _vp, _sz, _i, _i, _vp, _fp]),
-    "tuna_time_read": (_i, [_vp, _vp, _sz, _i, _i, _i, _vp, _fp]),
+    "tuna_time_read": (_i, [_vp, _vp, _sz, _i, _i, _i, _i, _vp, _fp]),
+    "tuna_describe_launch": (_i, [_i, _i, _i, _cfgp, _i, ctypes.c_char_p, _sz]),
     "tuna_set_lean_kernels": (_i, [_i]),
     "tuna_lean_launches": (ctypes.c_ulonglong, []),
     "tuna_release_workspaces": (_i, []),

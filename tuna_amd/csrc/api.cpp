@@ -1170,17 +1170,49 @@ TUNA_EXPORT int tuna_time_copy(const void *src, void *dst, size_t bytes, int war
     return time_loop(launch, 1, warmup, iters, 0, static_cast<hipStream_t>(stream), elapsed_ms);
 }
 
-TUNA_EXPORT int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int warmup, int iters, void *stream,
-                               float *elapsed_ms)
+TUNA_EXPORT int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int variant, int warmup, int iters,
+                               void *stream, float *elapsed_ms)
 {
     int rc;
     if ((rc = check_ptr(src, "src", 16)) || (rc = check_ptr(sink, "sink", 4))) return rc;
     if (bytes == 0 || bytes % 16) return fail(TUNA_ERR_INVALID_ARG, "bytes must be a positive multiple of 16");
+    if (variant < 0 || variant > 5) return fail(TUNA_ERR_INVALID_ARG, "variant %d outside 0..5", variant);
     auto launch = [&](int, hipStream_t s) {
-        hipError_t e = launch_read(src, sink, bytes, blocks, s);
+        hipError_t e = launch_read(src, sink, bytes, blocks, variant, s);
         return e == hipSuccess ? (int)TUNA_OK : hip_fail(e, "read launch");
     };
     return time_loop(launch, 1, warmup, iters, 0, static_cast<hipStream_t>(stream), elapsed_ms);
+}
+
+TUNA_EXPORT int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config *cfg, int decode_mode, char *buf, size_t len)
+{
+    if (!buf || len < 16) return fail(TUNA_ERR_INVALID_ARG, "buf is null or shorter than 16 bytes");
+    int rc = check_shape(m, n, k);
+    if (rc) return rc;
+    tuna_gemm_config c;
+    if (cfg) c = *cfg;
+    else select_config_for(m, n, k, decode_mode, &c, nullptr);
+    if (c.lds_tile_rows) {
+        TiledPlan tp;
+        if ((rc = plan_tiled(m, n, k, c, decode_mode, &tp))) return rc;
+        snprintf(buf, len, "gemm_tiled_kernel<%d rows x %d tokens> split_k=%d", tp.tile_rows, tp.tile_tokens, c.split_k);
+        return TUNA_OK;
+    }
+    if (is_narrow(c)) {
+        NarrowPlan np;
+        if ((rc = plan_narrow(m, n, k, c, decode_mode, &np))) return rc;
+        describe_narrow_launch(np.rows, np.waves_k, np.prefetch, np.token_tiles, n, buf, len);
+        return TUNA_OK;
+    }
+    GemmPlan plan;
+    if ((rc = plan_gemm(m, n, k, c, decode_mode, &plan))) return rc;
+    int cus = kMaxCus, dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+        cus = v;
+    else
+        (void)hipGetLastError();
+    describe_gemm_launch(plan, cus, buf, len);
+    return TUNA_OK;
 }
 
 TUNA_EXPORT int tuna_set_lean_kernels(int enabled) { return tuna::set_lean_kernels(enabled); }

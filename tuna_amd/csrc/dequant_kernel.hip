@@ -102,31 +102,44 @@ __global__ __launch_bounds__(256) void copy_kernel(const u32x4 *__restrict__ src
         __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
-// Read-only stream: the ceiling a pure HBM reader reaches on this device (8 loads of 16
-// bytes in flight per lane, 8 KB per wave and step, blocks walk the buffer in lockstep).
+// Read-only stream: the ceiling a pure HBM reader reaches on this device.  UNROLL loads of 16
+// bytes in flight per lane (UNROLL * 4 KB per workgroup and step), blocks walk the buffer in
+// lockstep; NT selects nontemporal (streaming) or plain loads.
+template <int UNROLL, bool NT>
 __global__ __launch_bounds__(256) void read_kernel(const u32x4 *__restrict__ src, uint32_t *__restrict__ sink, size_t n16)
 {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     u32x4 acc = u32x4{0u, 0u, 0u, 0u};
-    for (; i + 7 * stride < n16; i += 8 * stride) {
-        u32x4 v[8];
+    for (; i + (UNROLL - 1) * stride < n16; i += UNROLL * stride) {
+        u32x4 v[UNROLL];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+        for (int u = 0; u < UNROLL; ++u) v[u] = NT ? __builtin_nontemporal_load(src + i + u * stride) : src[i + u * stride];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) acc ^= v[u];
+        for (int u = 0; u < UNROLL; ++u) acc ^= v[u];
     }
-    for (; i < n16; i += stride) acc ^= __builtin_nontemporal_load(src + i);
+    for (; i < n16; i += stride) acc ^= NT ? __builtin_nontemporal_load(src + i) : src[i];
     const uint32_t r = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
     if (r == 0x9e3779b9u) sink[0] = r;  // practically never: keeps the loads alive
 }
 
-hipError_t launch_read(const void *src, void *sink, size_t bytes, int blocks, hipStream_t stream)
+// variant: 0 nontemporal x8 (default), 1 plain x8, 2 nontemporal x16, 3 plain x16, 4 nontemporal x4, 5 plain x4
+hipError_t launch_read(const void *src, void *sink, size_t bytes, int blocks, int variant, hipStream_t stream)
 {
     const size_t n16 = bytes / 16;
     if (blocks <= 0) blocks = 256 * 8;
-    hipLaunchKernelGGL(read_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, reinterpret_cast<const u32x4 *>(src),
-                       reinterpret_cast<uint32_t *>(sink), n16);
+    const u32x4 *s = reinterpret_cast<const u32x4 *>(src);
+    uint32_t *k = reinterpret_cast<uint32_t *>(sink);
+    const dim3 grid((unsigned)blocks), block(256);
+    switch (variant) {
+    case 0: hipLaunchKernelGGL((read_kernel<8, true>), grid, block, 0, stream, s, k, n16); break;
+    case 1: hipLaunchKernelGGL((read_kernel<8, false>), grid, block, 0, stream, s, k, n16); break;
+    case 2: hipLaunchKernelGGL((read_kernel<16, true>), grid, block, 0, stream, s, k, n16); break;
+    case 3: hipLaunchKernelGGL((read_kernel<16, false>), grid, block, 0, stream, s, k, n16); break;
+    case 4: hipLaunchKernelGGL((read_kernel<4, true>), grid, block, 0, stream, s, k, n16); break;
+    case 5: hipLaunchKernelGGL((read_kernel<4, false>), grid, block, 0, stream, s, k, n16); break;
+    default: return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

@@ -1,5 +1,6 @@
 // Instantiations of the GEMM kernel and the variant dispatcher.
 #include <atomic>
+#include <cstdio>
 #include <mutex>
 
 #include "gemm_kernel.hpp"
@@ -211,6 +212,28 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
     return hipGetLastError();
 }
 
+void describe_gemm_launch(const GemmPlan &plan, int cus, char *buf, size_t len)
+{
+    const unsigned slots = (unsigned)(cus * plan.wgs_per_cu);
+    const Variant *v = find_variant(plan.rw, plan.prefetch, plan.token_tiles, plan.decode, plan.threads, plan.min_waves,
+                                    plan.args.group_rows ? 1 : 0);
+    if ((!v || g_lean_enabled.load(std::memory_order_relaxed)) && mid_describe(plan, buf, len)) return;
+    if (!v) {
+        snprintf(buf, len, "none");
+        return;
+    }
+    if (const LeanVariant *lv = lean_applies(plan, cus)) {
+        snprintf(buf, len, "gemm_lean_kernel<WK=%d,U=%d,%d threads> split_k=%d", lv->wk, lv->u, lv->maxt, plan.args.split_k);
+        return;
+    }
+    int mode = v->mode;
+    if (!plan.args.group_rows && !plan.args.balanced && plan.grid.x <= slots && plan.grid.x == (unsigned)plan.args.tiles_total &&
+        find_variant(plan.rw, plan.prefetch, plan.token_tiles, plan.decode, plan.threads, plan.min_waves, 2))
+        mode = 2;
+    snprintf(buf, len, "gemm_kernel<RW=%d,U=%d,TT=%d,DEC=%d,%d threads,%d waves/SIMD,MODE=%d> split_k=%d", v->rw, v->u, v->tt,
+             v->dec, v->maxt, v->minw, mode, plan.args.split_k);
+}
+
 // ---- narrow-row kernel (gemm_narrow.hpp) ---------------------------------------------------------
 typedef void (*NarrowKernelFn)(const uint8_t *, const void *, const float *, const float *, int, int, int, int, void *, int,
                                const void *);
@@ -248,6 +271,12 @@ static const NarrowVariant *find_narrow(int rows, int wk, int u, int tt)
 bool narrow_variant_exists(int rows, int waves_k, int prefetch, int token_tiles)
 {
     return find_narrow(rows, waves_k, prefetch, token_tiles) != nullptr;
+}
+
+void describe_narrow_launch(int rows, int waves_k, int prefetch, int token_tiles, int n, char *buf, size_t len)
+{
+    snprintf(buf, len, "gemm_narrow_kernel<LW=%d,WK=%d,U=%d,PERM=%d,TT=%d>", rows / 16, waves_k, prefetch,
+             (n > 4 || token_tiles > 1) ? 1 : 0, token_tiles);
 }
 
 hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int prefetch, int token_tiles, hipStream_t stream)

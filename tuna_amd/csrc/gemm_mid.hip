@@ -1,4 +1,5 @@
 // Instantiations and launcher of the 17..128-token streaming kernel (gemm_mid.hpp).
+#include <cstdio>
 #include <mutex>
 
 #include "gemm_mid.hpp"
@@ -66,6 +67,15 @@ bool mid_applies(const GemmPlan &plan)
 {
     int xc;
     return mid_variant(plan, &xc) != nullptr;
+}
+
+bool mid_describe(const GemmPlan &plan, char *buf, size_t len)
+{
+    int xc;
+    const MidVariant *v = mid_variant(plan, &xc);
+    if (!v) return false;
+    snprintf(buf, len, "gemm_mid_kernel<U=%d,TT=%d,XB=%d,%d threads> x_chunk=%d", v->u, v->tt, v->xb, v->maxt, xc);
+    return true;
 }
 
 static std::mutex g_mid_mutex;

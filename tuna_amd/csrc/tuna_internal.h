@@ -150,6 +150,10 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream);
 // 17..128-token streaming twin of the general kernel (gemm_mid.hpp) for the launches it applies to.
 bool mid_applies(const GemmPlan &plan);
 hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t stream);
+bool mid_describe(const GemmPlan &plan, char *buf, size_t len);
+// Name and template arguments of the kernel launch_gemm would start for `plan` on a device of `cus` CUs.
+void describe_gemm_launch(const GemmPlan &plan, int cus, char *buf, size_t len);
+void describe_narrow_launch(int rows, int waves_k, int prefetch, int token_tiles, int n, char *buf, size_t len);
 // Narrow-row kernel (gemm_narrow.hpp): 16 or 32 rows per workgroup, all waves along k.
 struct NarrowArgs {
     const uint8_t *q;
@@ -178,7 +182,7 @@ hipError_t launch_dequant(const uint8_t *q, const float *absmax, const float *co
                           int m, int k, int decode, hipStream_t stream);
 hipError_t launch_quantize(const void *w, const float *code, void *q, float *absmax, int m, int k, hipStream_t stream);
 hipError_t launch_copy(const void *src, void *dst, size_t bytes, hipStream_t stream);
-hipError_t launch_read(const void *src, void *sink, size_t bytes, int blocks, hipStream_t stream);
+hipError_t launch_read(const void *src, void *sink, size_t bytes, int blocks, int variant, hipStream_t stream);
 
 // config_table.cpp
 struct TableEntry {

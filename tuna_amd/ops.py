@@ -299,17 +299,25 @@ def time_copy(src, dst, warmup=5, iters=20) -> float:
     return ms.value
 
 
-def time_read(src, blocks=0, warmup=5, iters=20) -> float:
+def time_read(src, blocks=0, variant=0, warmup=5, iters=20) -> float:
     """Milliseconds for `iters` read-only passes over `src` (tuna_time_read)."""
     nbytes = src.numel() * src.element_size()
     sink = torch.zeros(4, dtype=torch.int32, device=src.device)
     ms = ctypes.c_float(0)
     L = _lib.lib()
     with torch.cuda.device(src.device):
-        rc = L.tuna_time_read(src.data_ptr(), sink.data_ptr(), nbytes, int(blocks), int(warmup), int(iters),
+        rc = L.tuna_time_read(src.data_ptr(), sink.data_ptr(), nbytes, int(blocks), int(variant), int(warmup), int(iters),
                               _stream(src.device), ctypes.byref(ms))
     _lib.check(rc)
     return ms.value
+
+
+def describe_launch(m: int, n: int, k: int, config: GemmConfig = None, decode_mode: int = _lib.DECODE_GEMM) -> str:
+    """Name and template arguments of the kernel a GEMM launch would start (tuna_describe_launch)."""
+    buf = ctypes.create_string_buffer(256)
+    _lib.check(_lib.lib().tuna_describe_launch(int(m), int(n), int(k), ctypes.byref(config) if config is not None else None,
+                                               int(decode_mode), buf, 256))
+    return buf.value.decode()
 
 
 def set_lean_kernels(enabled: bool) -> bool:
