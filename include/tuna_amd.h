@@ -104,6 +104,30 @@ int tuna_matmul_ex(const void *q, const void *x, const void *code, const void *a
                    void *out, int m, int n, int k, const tuna_gemm_config *cfg,
                    int decode_mode, void *stream);
 
+/* Bytes of split-K partial sums the static scratch of tuna_matmul_static holds (plus 65536
+ * arrival counters). */
+#define TUNA_STATIC_WORKSPACE_BYTES (16u << 20)
+
+/* Optional one-time set-up on the current device: resolves the device address of the static
+ * scratch that tuna_matmul_static uses.  tuna_matmul_static does the same on its first call on
+ * a device; calling this first keeps even that step out of the caller's critical section. */
+int tuna_init(void);
+
+/* tuna_matmul_ex for callers that cannot allocate: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Where
+ * tuna_matmul_ex takes the split-K partial sums and arrival counters of a launch from a
+ * library-owned workspace that is allocated on first use, this entry point takes them from a
+ * fixed array in device memory that is part of the loaded library (16 MB + 256 KB, held on
+ * every GPU the library runs on until the process ends) and calls no allocating routine.  A
+ * launch that needs more than TUNA_STATIC_WORKSPACE_BYTES of partial sums or more than 65536
+ * counters fails with TUNA_ERR_WORKSPACE.  All calls on one GPU share that GPU's array: calls
+ * that may overlap (different streams) race; calls on one stream are ordered and safe.  The
+ * kernels return the counters they used to zero, so nothing is cleared between calls.  Results
+ * are those of tuna_matmul_ex, bit for bit. */
+int tuna_matmul_static(const void *q, const void *x, const void *code, const void *absmax,
+                       void *out, int m, int n, int k, const tuna_gemm_config *cfg,
+                       int decode_mode, void *stream);
+
 /* tuna_matmul_ex with a fused epilogue (the step after the GEMM in a decoder layer: the
  * residual add after the attention-out / down projections, SiLU(gate) * up after the combined
  * gate+up projection), saving a launch and a round trip of the activations through HBM.

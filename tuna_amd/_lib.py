@@ -62,6 +62,8 @@ SIGNATURES = {
     "tuna_last_error": (ctypes.c_char_p, []),
     "tuna_matmul": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "tuna_matmul_ex": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _vp]),
+    "tuna_init": (_i, []),
+    "tuna_matmul_static": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _vp]),
     "tuna_matmul_fused": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _i, _vp, _vp]),
     "tuna_matmul_grouped": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _ip, _cfgp, _i, _vp]),
     "tuna_dequant": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),

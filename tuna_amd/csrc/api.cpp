@@ -591,6 +591,64 @@ static void drop_workspace(hipStream_t stream)
     g_workspaces.erase(it);
 }
 
+// ---------------------------------------------------------------------------------------
+// Static scratch for tuna_matmul_static: the split-K partial sums and arrival counters of a
+// launch in device memory that exists from module load on, so that the call allocates nothing.
+// Every device the library runs on holds its own copy of the array at its own address until the
+// process ends; the host-side name is a stand-in, the address comes from hipGetSymbolAddress
+// (once per device, with that device current).
+// ---------------------------------------------------------------------------------------
+constexpr size_t kStaticCounters = (size_t)64 << 10;                       // arrival counters (4 bytes each) in front
+constexpr size_t kStaticWsBytes = (size_t)TUNA_STATIC_WORKSPACE_BYTES;     // partial sums behind them
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kStaticCounters * sizeof(unsigned) + kStaticWsBytes];
+
+static std::mutex g_scratch_mutex;
+static unsigned char *g_scratch_ptr[16];  // per device: address of that device's copy of `scratch`
+
+static int static_scratch(unsigned char **out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    if (dev < 0 || dev >= 16) return fail(TUNA_ERR_NO_DEVICE, "device index %d outside 0..15", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+        if (!p) return fail(TUNA_ERR_WORKSPACE, "hipGetSymbolAddress returned no address for the static scratch");
+        // The array is zero when the module is loaded and every launch returns the counters it
+        // used to zero, so nothing needs clearing here or between calls.
+        g_scratch_ptr[dev] = static_cast<unsigned char *>(p);
+    }
+    *out = g_scratch_ptr[dev];
+    return TUNA_OK;
+}
+
+// Where a launch gets its partial-sum buffer and counters from.
+static int provide_workspace(bool use_static, hipStream_t stream, size_t ws_bytes, size_t n_counters, float **ws, unsigned **counters)
+{
+    if (!use_static) {
+        Workspace w;
+        int rc = get_workspace(stream, ws_bytes, n_counters, &w);
+        if (rc) return rc;
+        *ws = w.ws;
+        *counters = w.counters;
+        return TUNA_OK;
+    }
+    if (ws_bytes > kStaticWsBytes || n_counters > kStaticCounters)
+        return fail(TUNA_ERR_WORKSPACE,
+                    "this launch needs %zu bytes of partial sums and %zu counters; the static scratch holds %zu bytes and %zu counters "
+                    "(use tuna_matmul_ex, whose workspace grows)",
+                    ws_bytes, n_counters, kStaticWsBytes, kStaticCounters);
+    unsigned char *base = nullptr;
+    int rc = static_scratch(&base);
+    if (rc) return rc;
+    *counters = reinterpret_cast<unsigned *>(base);
+    *ws = reinterpret_cast<float *>(base + kStaticCounters * sizeof(unsigned));
+    return TUNA_OK;
+}
+
 static int check_ptr(const void *p, const char *name, size_t align)
 {
     if (!p) return fail(TUNA_ERR_INVALID_ARG, "%s is null", name);
@@ -600,7 +658,7 @@ static int check_ptr(const void *p, const char *name, size_t align)
 
 static int matmul_impl(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n, int k,
                        const tuna_gemm_config *cfg, int decode, hipStream_t stream, int epilogue = TUNA_EPILOGUE_NONE,
-                       const void *residual = nullptr)
+                       const void *residual = nullptr, bool static_ws = false)
 {
     int rc;
     if ((rc = check_shape(m, n, k))) return rc;
@@ -623,12 +681,8 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
         tp.args.out = out;
         tp.args.epilogue = epilogue;
         tp.args.residual = residual;
-        if (tp.ws_bytes) {
-            Workspace w;
-            if ((rc = get_workspace(stream, tp.ws_bytes, tp.n_counters, &w))) return rc;
-            tp.args.ws = w.ws;
-            tp.args.counters = w.counters;
-        }
+        if (tp.ws_bytes && (rc = provide_workspace(static_ws, stream, tp.ws_bytes, tp.n_counters, &tp.args.ws, &tp.args.counters)))
+            return rc;
         hipError_t e = launch_gemm_tiled(tp.args, tp.tile_rows, tp.tile_tokens, stream);
         if (e != hipSuccess) return hip_fail(e, "many-token gemm launch");
         return TUNA_OK;
@@ -657,12 +711,8 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
     plan.args.out = out;
     plan.args.epilogue = epilogue;
     plan.args.residual = residual;
-    if (plan.ws_bytes) {
-        Workspace w;
-        if ((rc = get_workspace(stream, plan.ws_bytes, plan.n_counters, &w))) return rc;
-        plan.args.ws = w.ws;
-        plan.args.counters = w.counters;
-    }
+    if (plan.ws_bytes && (rc = provide_workspace(static_ws, stream, plan.ws_bytes, plan.n_counters, &plan.args.ws, &plan.args.counters)))
+        return rc;
     hipError_t e = launch_gemm(plan, stream);
     if (e != hipSuccess) return hip_fail(e, "gemm launch");
     return TUNA_OK;
@@ -900,6 +950,19 @@ TUNA_EXPORT int tuna_matmul_ex(const void *q, const void *x, const void *code, c
                                int k, const tuna_gemm_config *cfg, int decode_mode, void *stream)
 {
     return matmul_impl(q, x, code, absmax, out, m, n, k, cfg, decode_mode, static_cast<hipStream_t>(stream));
+}
+
+TUNA_EXPORT int tuna_init(void)
+{
+    unsigned char *p = nullptr;
+    return static_scratch(&p);
+}
+
+TUNA_EXPORT int tuna_matmul_static(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n,
+                                   int k, const tuna_gemm_config *cfg, int decode_mode, void *stream)
+{
+    return matmul_impl(q, x, code, absmax, out, m, n, k, cfg, decode_mode, static_cast<hipStream_t>(stream), TUNA_EPILOGUE_NONE,
+                       nullptr, true);
 }
 
 TUNA_EXPORT int tuna_matmul_fused(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n,

@@ -66,6 +66,24 @@ def matmul(x, q, s, c, o, m: int, n: int, k: int, config: GemmConfig = None,
     _lib.check(rc)
 
 
+def matmul_static(x, q, s, c, o, m: int, n: int, k: int, config: GemmConfig = None,
+                  decode_mode: int = _lib.DECODE_GEMM) -> None:
+    """matmul through tuna_matmul_static: same result, but the split-K partial sums live in a fixed
+    array of the loaded library instead of an allocated workspace (for callers that cannot
+    allocate).  Raises TunaError (ERR_WORKSPACE) if the launch needs more than that array holds."""
+    m, n, k = int(m), int(n), int(k)
+    _require(x, "x", torch.float16, n * k)
+    _require(q, "q", torch.uint8, m * k // 2)
+    _require(s, "s", torch.float32, m)
+    _require(c, "c", torch.float32, 16)
+    _require(o, "o", torch.float16, n * m)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().tuna_matmul_static(q.data_ptr(), x.data_ptr(), c.data_ptr(), s.data_ptr(), o.data_ptr(), m, n, k,
+                                           ctypes.byref(config) if config is not None else None, int(decode_mode),
+                                           _stream(x.device))
+    _lib.check(rc)
+
+
 def matmul_fused(x, q, s, c, o, m: int, n: int, k: int, epilogue: int, residual=None, config: GemmConfig = None,
                  decode_mode: int = _lib.DECODE_GEMM) -> None:
     """matmul with a fused epilogue (tuna_matmul_fused).
