@@ -136,6 +136,32 @@ int tuna_matmul_fused(const void *q, const void *x, const void *code, const void
                       void *out, int m, int n, int k, const tuna_gemm_config *cfg,
                       int decode_mode, int epilogue, const void *residual, void *stream);
 
+/* One GEMM of a batch: the arguments of tuna_matmul. */
+typedef struct tuna_gemm_problem {
+    const void *q;      /* uint8 [m/8, k/8, 32] */
+    const void *x;      /* fp16  [n, k]         */
+    const void *code;   /* fp32  [16]           */
+    const void *absmax; /* fp32  [m]            */
+    void *out;          /* fp16  [n, m]         */
+    int32_t m, n, k;
+} tuna_gemm_problem;
+
+/* `count` independent GEMMs in one call - the projections of a decoder layer that do not feed
+ * one another (Q, K and V kept separate; gate and up), the experts of a mixture, the layers of
+ * a benchmark sweep (README.md:25-27 totals are layers x four GEMMs).  `problems` is a host
+ * array read during the call.  Runs of up to 32 consecutive problems with at most 16 tokens
+ * each, rows in multiples of 64, k in multiples of 256 or more, 16-byte aligned scales and one
+ * shared codebook become ONE launch of persistent workgroups: the k ranges of all row tiles of
+ * all problems are laid end to end and divided evenly over the compute units, a workgroup
+ * streams its share without a gap between problems, and the per-launch fixed time (about 2.5
+ * us kernel-to-kernel, the ramp of the memory system, the uneven finish) is paid once per batch
+ * instead of once per GEMM.  Results are deterministic and within the GEMM's tolerance of
+ * tuna_matmul's (the summation order differs where tuna_matmul uses another kernel).  Problems
+ * that do not qualify are launched one by one, exactly as tuna_matmul would.  Ordering is that
+ * of one call on `stream`; no problem may read what another one writes.  All problems are
+ * checked before anything is enqueued.  No counterpart in the reference. */
+int tuna_matmul_multi(const tuna_gemm_problem *problems, int count, void *stream);
+
 /* Grouped GEMM (mixture of experts with per-expert token lists) in one launch.  The weights
  * are n_groups (<= 64) matrices of m_group rows stacked along m - q [n_groups*m_group/8, k/8,
  * 32], absmax [n_groups*m_group] - exactly the layout of the dense stacked call.  x [n_total,

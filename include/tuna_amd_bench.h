@@ -25,6 +25,10 @@ int tuna_time_matmul(const void *const *q_list, const void *const *absmax_list, 
                      const void *x, const void *code, void *out, int m, int n, int k,
                      const tuna_gemm_config *cfg, int decode_mode, int warmup, int iters,
                      int use_graph, void *stream, float *elapsed_ms);
+/* Same protocol for tuna_matmul_multi: `problems` holds n_sets batches of `count` problems each,
+ * iteration i is one call with batch (i mod n_sets); the time is that of `iters` calls. */
+int tuna_time_matmul_multi(const tuna_gemm_problem *problems, int n_sets, int count, int warmup,
+                           int iters, int use_graph, void *stream, float *elapsed_ms);
 /* Same protocol for the grouped GEMM. */
 int tuna_time_matmul_grouped(const void *const *q_list, const void *const *absmax_list, int n_sets,
                              const void *x, const void *code, void *out, int m_group, int n_groups,
@@ -54,6 +58,13 @@ int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int va
  * device's CU count decides between twins, otherwise 256 CUs are assumed. */
 int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config *cfg, int decode_mode,
                          char *buf, size_t len);
+
+/* Diagnostic override of the batched kernel's workgroup shape (tuna_matmul_multi): waves along the
+ * rows (1, 2, 4, 8 or 16 of the workgroup's 16 waves; 0 = the library's choice) and ring depth
+ * (2 or 4; 0 = the library's choice).  For A/B timing. */
+int tuna_set_multi_shape(int waves_m, int prefetch);
+/* Diagnostic: launches of the batched kernel so far in this process. */
+unsigned long long tuna_multi_launches(void);
 
 /* Diagnostic switch, process-wide, default on: dense launches that qualify run one of two
  * kernels stripped of everything else the general one carries - small launches (one workgroup

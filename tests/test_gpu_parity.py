@@ -1038,3 +1038,169 @@ def test_captured_graph_survives_growth_of_the_split_k_workspace():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out.view(torch.int16), eager.view(torch.int16))
+
+
+# ----------------------------------------------------------------------------- several GEMMs in one call
+def _multi_problems(shapes, seed0):
+    import torch
+
+    probs, host = [], []
+    dc = None
+    for i, (m, n, k) in enumerate(shapes):
+        q, x, code, absmax = make_inputs_np(m, n, k, seed=seed0 + i)
+        dq, dx, dc_i, da = to_dev(q, x, code, absmax)
+        dc = dc_i if dc is None else dc       # one codebook tensor for the batch (one decode table per launch)
+        out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+        probs.append((dx, dq, da, dc, out, m, n, k))
+        host.append((q, x, code, absmax))
+    return probs, host
+
+
+def _check_against_oracle(host, got_bits, m, n, k, seed, n_rows=256):
+    q, x, code, absmax = host
+    rng = np.random.default_rng(seed)
+    rows = np.sort(rng.choice(m, size=min(n_rows, m), replace=False)).astype(np.int32)
+    ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1, rows=rows)
+    return rel_err(f16_bits_to_f64(got_bits[:, rows]), ref)
+
+
+def test_matmul_multi_matches_the_oracle_and_separate_calls():
+    """tuna_matmul_multi on a mixed batch: five problems that the batched persistent kernel takes
+    in one launch (1..16 tokens, tuned and untuned shapes, k up to 14336), one it cannot take
+    (40 tokens, ragged sizes) and one more behind it.  Every output is checked against the oracle
+    (row subset), agrees with a separate tuna_matmul call within the same tolerance (the batched
+    kernel sums in another order), and a second call gives the same bits again."""
+    import torch
+
+    from tuna_amd import _lib, ops
+
+    shapes = [(4096, 16, 4096), (6144, 16, 4096), (4096, 16, 14336), (1024, 5, 2048), (8192, 1, 8192), (520, 40, 1096),
+              (10240, 16, 8192)]
+    probs, host = _multi_problems(shapes, 300)
+    want = []
+    for (dx, dq, da, dc, _o, m, n, k) in probs:
+        o = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+        ops.matmul(dx, dq, da, dc, o, m, n, k)
+        want.append(o)
+    torch.cuda.synchronize()
+    first = None
+    for rep in range(2):
+        for p in probs:
+            p[4].fill_(float("nan"))
+        before = _lib.lib().tuna_multi_launches()
+        ops.matmul_multi(probs)
+        torch.cuda.synchronize()
+        assert _lib.lib().tuna_multi_launches() == before + 1          # problems 0..4 in one launch, the rest one by one
+        got = [p[4].cpu().numpy().view(np.uint16).copy() for p in probs]
+        for i, ((m, n, k), g, w) in enumerate(zip(shapes, got, want)):
+            assert not np.isnan(g.view(np.float16)).any(), (rep, i)
+            e = _check_against_oracle(host[i], g, m, n, k, seed=i)
+            print(f"  multi problem {i} {m}x{n}x{k}: rel_err={e:.3e}", flush=True)
+            assert e <= REL_TOL, (rep, i, e)
+            assert rel_err(f16_bits_to_f64(g), w.float().cpu().numpy().astype(np.float64)) <= REL_TOL
+        for i in (5, 6):                                               # launched as tuna_matmul would: identical bits
+            assert np.array_equal(got[i], want[i].cpu().numpy().view(np.uint16))
+        if first is None:
+            first = got
+        else:
+            assert all(np.array_equal(a, b) for a, b in zip(first, got))   # deterministic
+    ops.matmul_multi([])                      # an empty batch is a no-op
+    ops.matmul_multi(probs[:1])               # a batch of one is a plain call
+    torch.cuda.synchronize()
+    assert torch.equal(probs[0][4].view(torch.int16), want[0].view(torch.int16))
+
+
+@pytest.mark.parametrize("waves_m,prefetch", [(4, 2), (4, 4), (2, 2), (2, 4), (8, 2), (8, 4), (1, 2), (16, 2)])
+def test_matmul_multi_every_workgroup_shape_and_decode_readout(waves_m, prefetch):
+    """The batched kernel with every workgroup shape it has (waves along rows x ring depth): oracle
+    check on a batch whose shares cut row tiles at many places, and the one-hot read-out of the
+    in-register decode (bit-exact whatever the split, since every partial sum but one is zero)."""
+    import torch
+
+    from tuna_amd import _lib, ops
+
+    L = _lib.lib()
+    shapes = [(2048, 16, 4096), (1024, 7, 8192), (3072, 16, 2048), (1024, 1, 4096)]
+    probs, host = _multi_problems(shapes, 330)
+    L.tuna_set_multi_shape(waves_m, prefetch)
+    try:
+        before = L.tuna_multi_launches()
+        ops.matmul_multi(probs)
+        torch.cuda.synchronize()
+        assert L.tuna_multi_launches() == before + 1
+        for i, (m, n, k) in enumerate(shapes):
+            g = probs[i][4].cpu().numpy().view(np.uint16)
+            assert not np.isnan(g.view(np.float16)).any()
+            e = _check_against_oracle(host[i], g, m, n, k, seed=i, n_rows=128)
+            assert e <= REL_TOL, (i, e)
+        # one-hot activations: out[t, r] must be the decoded weight W[r, col_t], bit for bit
+        rng = np.random.default_rng(5)
+        for i, (m, n, k) in enumerate(shapes):
+            cols = rng.choice(k, size=n, replace=False)
+            xh = np.zeros((n, k), np.float16)
+            xh[np.arange(n), cols] = 1.0
+            probs[i][0].copy_(torch.from_numpy(xh).cuda())
+            probs[i][4].fill_(float("nan"))
+        ops.matmul_multi(probs)
+        torch.cuda.synchronize()
+        rng = np.random.default_rng(5)
+        for i, (m, n, k) in enumerate(shapes):
+            cols = rng.choice(k, size=n, replace=False)
+            q, _x, code, absmax = host[i]
+            img = O.dequant(q, absmax, code, m, k, mode=O.D1)
+            assert np.array_equal(probs[i][4].cpu().numpy().view(np.uint16), img[:, cols].T), i
+    finally:
+        L.tuna_set_multi_shape(0, 0)
+
+
+def test_matmul_multi_checks_every_problem_before_launching_any():
+    import torch
+
+    from tuna_amd import ops
+
+    probs, _ = _multi_problems([(512, 16, 1024), (256, 16, 512)], 310)
+    bad = list(probs[1])
+    bad[5] = 260                              # m not a multiple of 8: caught by the library, not by the wrapper
+    arr = ops.problem_array(probs)
+    arr[1].m = 260
+    from tuna_amd import _lib
+
+    rc = _lib.lib().tuna_matmul_multi(arr, 2, None)
+    assert rc == _lib.ERR_INVALID_ARG
+    torch.cuda.synchronize()
+    assert torch.isnan(probs[0][4]).all()     # nothing ran
+
+
+def test_matmul_multi_in_a_captured_graph_replays_correctly():
+    """A captured tuna_matmul_multi call replayed several times with fresh activations, eager work
+    in between: every replay equals the eager call (the batched kernel's workspace and counters
+    are those of the capture stream, allocated by the eager call before the capture)."""
+    import torch
+
+    from tuna_amd import ops
+
+    shapes = [(4096, 16, 4096), (1024, 16, 2048), (4096, 16, 14336), (2048, 16, 1024), (8192, 16, 8192)]
+    probs, _ = _multi_problems(shapes, 320)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        ops.matmul_multi(probs)               # eager once: the stream's workspace exists afterwards
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            ops.matmul_multi(probs)
+    for rep in range(3):
+        for i, p in enumerate(probs):
+            _, x2, _, _ = make_inputs_np(p[5], p[6], p[7], seed=900 + 10 * rep + i)
+            p[0].copy_(torch.from_numpy(x2).cuda())
+            p[4].fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [p[4].clone() for p in probs]
+        for p in probs:
+            p[4].fill_(float("nan"))
+        ops.matmul_multi(probs)               # the same batch eagerly: identical bits
+        torch.cuda.synchronize()
+        for p, g in zip(probs, got):
+            assert not torch.isnan(g).any()
+            assert torch.equal(g.view(torch.int16), p[4].view(torch.int16)), rep

@@ -50,6 +50,13 @@ class GemmConfig(ctypes.Structure):
         return cls(**{f: int(d.get(f, 0) if f in ("k_stagger", "lds_tile_rows") else d[f]) for f in cls.FIELDS})
 
 
+class GemmProblem(ctypes.Structure):
+    """Mirror of ``tuna_gemm_problem`` (include/tuna_amd.h)."""
+
+    _fields_ = [("q", ctypes.c_void_p), ("x", ctypes.c_void_p), ("code", ctypes.c_void_p), ("absmax", ctypes.c_void_p),
+                ("out", ctypes.c_void_p), ("m", ctypes.c_int32), ("n", ctypes.c_int32), ("k", ctypes.c_int32)]
+
+
 # name -> (restype, argtypes); also the list of symbols the header declares
 _vp, _i, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
 _cfgp = ctypes.POINTER(GemmConfig)
@@ -65,6 +72,7 @@ SIGNATURES = {
     "tuna_init": (_i, []),
     "tuna_matmul_static": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _vp]),
     "tuna_matmul_fused": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _i, _vp, _vp]),
+    "tuna_matmul_multi": (_i, [ctypes.POINTER(GemmProblem), _i, _vp]),
     "tuna_matmul_grouped": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _ip, _cfgp, _i, _vp]),
     "tuna_dequant": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "tuna_quantize": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
@@ -80,11 +88,14 @@ SIGNATURES = {
     "tuna_config_table_size": (_i, []),
     "tuna_config_table_entry": (_i, [_i, _ip, _ip, _ip, _ip, _cfgp]),
     "tuna_time_matmul": (_i, [_vpp, _vpp, _i, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _i, _i, _i, _vp, _fp]),
+    "tuna_time_matmul_multi": (_i, [ctypes.POINTER(GemmProblem), _i, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_matmul_grouped": (_i, [_vpp, _vpp, _i, _vp, _vp, _vp, _i, _i, _i, _ip, _cfgp, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_dequant": (_i, [_vpp, _vpp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_copy": (_i, [_vp, _vp, _sz, _i, _i, _vp, _fp]),
     "tuna_time_read": (_i, [_vp, _vp, _sz, _i, _i, _i, _i, _vp, _fp]),
     "tuna_describe_launch": (_i, [_i, _i, _i, _cfgp, _i, ctypes.c_char_p, _sz]),
+    "tuna_set_multi_shape": (_i, [_i, _i]),
+    "tuna_multi_launches": (ctypes.c_ulonglong, []),
     "tuna_set_lean_kernels": (_i, [_i]),
     "tuna_lean_launches": (ctypes.c_ulonglong, []),
     "tuna_release_workspaces": (_i, []),

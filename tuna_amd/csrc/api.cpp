@@ -4,6 +4,7 @@
 // Replaces the reference's host dispatcher (kernel.cu:2962-3156: requiredSmem,
 // LAUNCH_KERNEL_IF_CONDITION and the 122-arm if-chain in wrapper) and
 // dequantize_wrapper (kernel.cu:3243-3253).
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -13,6 +14,7 @@
 #include <utility>
 #include <vector>
 
+#include "gemm_multi.hpp"
 #include "tuna_internal.h"
 
 namespace tuna {
@@ -833,6 +835,114 @@ static int matmul_grouped_impl(const void *q, const void *x, const void *code, c
     return TUNA_OK;
 }
 
+// ---------------------------------------------------------------------------------------
+// Several independent GEMMs in one call: batches of up to kMaxMultiProblems problems that the
+// batched persistent kernel can run (gemm_multi.hpp) are one launch each; anything else is
+// launched problem by problem on the same stream.
+// ---------------------------------------------------------------------------------------
+static std::atomic<int> g_multi_waves_m{0}, g_multi_prefetch{0};  // 0: the library's choice (diagnostic override)
+static std::atomic<unsigned long long> g_multi_launches{0};
+
+struct MultiPlan {
+    MultiArgs args;
+    int prefetch;
+    size_t ws_bytes, n_counters;
+};
+
+// Whether problems[0..count) can run as one launch on a device of `cus` compute units; fills `plan`.
+static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, MultiPlan *plan)
+{
+    if (count < 2 || count > kMaxMultiProblems || cus < 1) return false;
+    int waves_m = g_multi_waves_m.load(std::memory_order_relaxed);
+    int prefetch = g_multi_prefetch.load(std::memory_order_relaxed);
+    if (!prefetch) prefetch = 2;
+    if (!multi_variant_exists(prefetch)) return false;
+    if (!waves_m) {
+        // 256-row tiles (4 x 4 waves) when every problem allows, else narrower tiles and more waves along k
+        waves_m = 4;
+        for (int i = 0; i < count; ++i)
+            while (waves_m > 1 && problems[i].m % (64 * waves_m)) waves_m >>= 1;
+    }
+    if (waves_m != 1 && waves_m != 2 && waves_m != 4 && waves_m != 8 && waves_m != 16) return false;
+    const int waves_k = 16 / waves_m;
+    if ((32 / waves_k) % prefetch) return false;  // an x chunk of 32 k-steps is whole ring turns of every wave
+    const int unit_steps = waves_k * prefetch;
+    MultiArgs &a = plan->args;
+    memset(&a, 0, sizeof(a));
+    long long units = 0, tiles = 0;
+    for (int i = 0; i < count; ++i) {
+        const tuna_gemm_problem &p = problems[i];
+        if (p.n > 16 || p.m % (64 * waves_m) || p.k % (kStepK * unit_steps)) return false;
+        if ((unsigned long long)p.m * (unsigned long long)p.k / 2 >= (1ull << 32) || p.k >= (1 << 23)) return false;
+        if (reinterpret_cast<uintptr_t>(p.absmax) % 16) return false;
+        if (p.code != problems[0].code) return false;  // one decode table per launch
+        MultiProblem &mp = a.prob[i];
+        mp.q = static_cast<const uint8_t *>(p.q);
+        mp.x = p.x;
+        mp.absmax = static_cast<const float *>(p.absmax);
+        mp.out = p.out;
+        mp.m = p.m, mp.n = p.n, mp.k = p.k;
+        mp.units_per_tile = p.k / (kStepK * unit_steps);
+        mp.unit_begin = (int)units;
+        mp.tile_begin = (int)tiles;
+        const long long row_tiles = p.m / (64 * waves_m);
+        units += row_tiles * mp.units_per_tile;
+        tiles += row_tiles;
+        if ((units + 1) * cus >= 0x7fffffffLL) return false;
+    }
+    int n_wg = units < cus ? (int)units : cus;
+    a.code = static_cast<const float *>(problems[0].code);
+    a.n_problems = count;
+    a.units_total = (int)units;
+    a.waves_m = waves_m;
+    a.wk_log2 = log2i(waves_k);
+    a.n_wg = n_wg;
+    a.swizzle = (n_wg % 8 == 0) ? 1 : 0;
+    plan->prefetch = prefetch;
+    plan->ws_bytes = (size_t)n_wg * 2 * waves_m * 4096;
+    plan->n_counters = (size_t)tiles;
+    return true;
+}
+
+static int matmul_multi_impl(const tuna_gemm_problem *problems, int count, hipStream_t stream)
+{
+    if (count < 0 || (count > 0 && !problems)) return fail(TUNA_ERR_INVALID_ARG, "problems is null or count=%d negative", count);
+    if (count == 0) return TUNA_OK;
+    int rc;
+    // every problem is checked before anything is enqueued: a bad one must not leave half a batch behind
+    for (int i = 0; i < count; ++i) {
+        const tuna_gemm_problem &p = problems[i];
+        if ((rc = check_shape(p.m, p.n, p.k))) return rc;
+        if ((rc = check_ptr(p.q, "q", 16)) || (rc = check_ptr(p.x, "x", 16)) || (rc = check_ptr(p.code, "code", 4)) ||
+            (rc = check_ptr(p.absmax, "absmax", 4)) || (rc = check_ptr(p.out, "out", 16)))
+            return rc;
+        tuna_gemm_config c;
+        select_config(p.m, p.n, p.k, &c, nullptr);
+        if ((rc = validate_for(p.m, p.n, p.k, c, TUNA_DECODE_GEMM))) return rc;
+    }
+    int dev = 0, cus = 0;
+    hipError_t e = device_cus(&dev, &cus);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    for (int first = 0; first < count;) {
+        // the longest run of problems from `first` that one launch can take
+        MultiPlan plan;
+        int take = count - first < kMaxMultiProblems ? count - first : kMaxMultiProblems;
+        while (take >= 2 && !plan_multi(problems + first, take, cus, &plan)) --take;
+        if (take >= 2) {
+            if ((rc = provide_workspace(false, stream, plan.ws_bytes, plan.n_counters, &plan.args.ws, &plan.args.counters))) return rc;
+            e = launch_gemm_multi(plan.args, plan.prefetch, dev, stream);
+            if (e != hipSuccess) return hip_fail(e, "batched gemm launch");
+            g_multi_launches.fetch_add(1, std::memory_order_relaxed);
+            first += take;
+            continue;
+        }
+        const tuna_gemm_problem &p = problems[first];
+        if ((rc = matmul_impl(p.q, p.x, p.code, p.absmax, p.out, p.m, p.n, p.k, nullptr, TUNA_DECODE_GEMM, stream))) return rc;
+        ++first;
+    }
+    return TUNA_OK;
+}
+
 static int dequant_impl(const void *q, const void *absmax, const void *code, void *out, int m, int k, int decode,
                         hipStream_t stream)
 {
@@ -970,6 +1080,11 @@ TUNA_EXPORT int tuna_matmul_fused(const void *q, const void *x, const void *code
                                   void *stream)
 {
     return matmul_impl(q, x, code, absmax, out, m, n, k, cfg, decode_mode, static_cast<hipStream_t>(stream), epilogue, residual);
+}
+
+TUNA_EXPORT int tuna_matmul_multi(const tuna_gemm_problem *problems, int count, void *stream)
+{
+    return matmul_multi_impl(problems, count, static_cast<hipStream_t>(stream));
 }
 
 TUNA_EXPORT int tuna_matmul_grouped(const void *q, const void *x, const void *code, const void *absmax, void *out,
@@ -1197,6 +1312,14 @@ TUNA_EXPORT int tuna_time_matmul(const void *const *q_list, const void *const *a
     return time_loop(launch, n_sets, warmup, iters, use_graph, static_cast<hipStream_t>(stream), elapsed_ms);
 }
 
+TUNA_EXPORT int tuna_time_matmul_multi(const tuna_gemm_problem *problems, int n_sets, int count, int warmup, int iters,
+                                       int use_graph, void *stream, float *elapsed_ms)
+{
+    if (!problems || count < 1) return fail(TUNA_ERR_INVALID_ARG, "problems is null or count < 1");
+    auto launch = [&](int set, hipStream_t s) { return matmul_multi_impl(problems + (size_t)set * count, count, s); };
+    return time_loop(launch, n_sets, warmup, iters, use_graph, static_cast<hipStream_t>(stream), elapsed_ms);
+}
+
 TUNA_EXPORT int tuna_time_matmul_grouped(const void *const *q_list, const void *const *absmax_list, int n_sets, const void *x,
                                          const void *code, void *out, int m_group, int n_groups, int k,
                                          const int32_t *token_offsets, const tuna_gemm_config *cfg, int decode_mode,
@@ -1277,6 +1400,15 @@ TUNA_EXPORT int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config
     describe_gemm_launch(plan, cus, buf, len);
     return TUNA_OK;
 }
+
+TUNA_EXPORT int tuna_set_multi_shape(int waves_m, int prefetch)
+{
+    g_multi_waves_m.store(waves_m);
+    g_multi_prefetch.store(prefetch);
+    return TUNA_OK;
+}
+
+TUNA_EXPORT unsigned long long tuna_multi_launches(void) { return g_multi_launches.load(); }
 
 TUNA_EXPORT int tuna_set_lean_kernels(int enabled) { return tuna::set_lean_kernels(enabled); }
 

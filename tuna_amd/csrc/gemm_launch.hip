@@ -139,23 +139,29 @@ static unsigned char g_attr_done[16][kNumVariants];
 static unsigned char g_lean_attr_done[16][kNumLean];
 static int g_cu_count[16];
 
-hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
+hipError_t device_cus(int *dev_out, int *cus_out)
 {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
-    int cus;
-    {
-        std::lock_guard<std::mutex> lock(g_attr_mutex);
-        if (!g_cu_count[dev]) {
-            int n = 0;
-            e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
-            if (e != hipSuccess) return e;
-            g_cu_count[dev] = n > 0 ? n : 256;
-        }
-        cus = g_cu_count[dev];
+    std::lock_guard<std::mutex> lock(g_attr_mutex);
+    if (!g_cu_count[dev]) {
+        int n = 0;
+        e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+        if (e != hipSuccess) return e;
+        g_cu_count[dev] = n > 0 ? n : 256;
     }
+    *dev_out = dev;
+    *cus_out = g_cu_count[dev];
+    return hipSuccess;
+}
+
+hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
+{
+    int dev = 0, cus = 0;
+    hipError_t e = device_cus(&dev, &cus);
+    if (e != hipSuccess) return e;
     const unsigned slots = (unsigned)(cus * plan.wgs_per_cu);
     const Variant *v = find_variant(plan.rw, plan.prefetch, plan.token_tiles, plan.decode, plan.threads, plan.min_waves,
                                     plan.args.group_rows ? 1 : 0);

@@ -172,6 +172,14 @@ int set_lean_kernels(int enabled);  // returns the previous setting
 unsigned long long lean_launches();
 bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves, int grouped);
 
+// gemm_multi.hip: several 1..16-token GEMMs in one launch of persistent workgroups (gemm_multi.hpp)
+struct MultiArgs;
+bool multi_variant_exists(int prefetch);
+size_t multi_lds_bytes();
+hipError_t launch_gemm_multi(const MultiArgs &args, int prefetch, int dev, hipStream_t stream);
+// Compute units of the current device (cached); *dev receives its index.
+hipError_t device_cus(int *dev, int *cus);
+
 // gemm_tiled.hip
 hipError_t launch_gemm_tiled(const TiledArgs &args, int tile_rows, int tile_tokens, hipStream_t stream);
 bool tiled_variant_exists(int tile_rows, int tile_tokens);

@@ -110,6 +110,32 @@ def matmul_fused(x, q, s, c, o, m: int, n: int, k: int, epilogue: int, residual=
     _lib.check(rc)
 
 
+def problem_array(problems):
+    """ctypes array of GemmProblem for matmul_multi / time_matmul_multi from (x, q, s, c, o, m, n, k) tuples."""
+    arr = (_lib.GemmProblem * len(problems))()
+    for i, (x, q, s, c, o, m, n, k) in enumerate(problems):
+        m, n, k = int(m), int(n), int(k)
+        _require(x, "x", torch.float16, n * k)
+        _require(q, "q", torch.uint8, m * k // 2)
+        _require(s, "s", torch.float32, m)
+        _require(c, "c", torch.float32, 16)
+        _require(o, "o", torch.float16, n * m)
+        arr[i] = _lib.GemmProblem(q.data_ptr(), x.data_ptr(), c.data_ptr(), s.data_ptr(), o.data_ptr(), m, n, k)
+    return arr
+
+
+def matmul_multi(problems) -> None:
+    """Several independent GEMMs in one call (tuna_matmul_multi): `problems` is a list of
+    (x, q, s, c, o, m, n, k) tuples, each with the meaning of matmul's arguments."""
+    if not problems:
+        return
+    arr = problem_array(problems)
+    dev = problems[0][0].device
+    with torch.cuda.device(dev):
+        rc = _lib.lib().tuna_matmul_multi(arr, len(problems), _stream(dev))
+    _lib.check(rc)
+
+
 def matmul_grouped(x, q, s, c, o, m_group: int, n_groups: int, k: int, token_offsets, config: GemmConfig = None,
                    decode_mode: int = _lib.DECODE_GEMM) -> None:
     """Grouped GEMM (mixture of experts): o[t, :] = x[t, :] @ decode(W_e)^T for the tokens t of
@@ -292,6 +318,21 @@ def time_matmul_grouped(q_list, absmax_list, x, c, o, m_group, n_groups, k, toke
                                                  ctypes.byref(ms))
     _lib.check(rc)
     return ms.value
+
+def time_matmul_multi(batches, warmup=10, iters=100, use_graph=False) -> float:
+    """Milliseconds for `iters` matmul_multi calls rotating over `batches` (equally long lists of
+    (x, q, s, c, o, m, n, k) problems), HIP events on the current stream (tuna_time_matmul_multi)."""
+    count = len(batches[0])
+    assert count > 0 and all(len(b) == count for b in batches)
+    arr = problem_array([p for b in batches for p in b])
+    dev = batches[0][0][0].device
+    ms = ctypes.c_float(0)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().tuna_time_matmul_multi(arr, len(batches), count, int(warmup), int(iters), int(bool(use_graph)),
+                                               _stream(dev), ctypes.byref(ms))
+    _lib.check(rc)
+    return ms.value
+
 
 def time_dequant(q_list, absmax_list, c, o, m, k, warmup=5, iters=20) -> float:
     qp, _qk = _ptr_array(q_list)
