@@ -63,6 +63,9 @@ int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config *cfg, int d
  * rows (1, 2, 4, 8 or 16 of the workgroup's 16 waves; 0 = the library's choice) and ring depth
  * (2 or 4; 0 = the library's choice).  For A/B timing. */
 int tuna_set_multi_shape(int waves_m, int prefetch);
+/* Diagnostic: the shortest run of problems tuna_matmul_multi hands to the batched kernel
+ * (default 2; 1 sends single problems through it as well).  Returns the previous value. */
+int tuna_set_multi_min_batch(int count);
 /* Diagnostic: launches of the batched kernel so far in this process. */
 unsigned long long tuna_multi_launches(void);
 

@@ -95,6 +95,7 @@ SIGNATURES = {
     "tuna_time_read": (_i, [_vp, _vp, _sz, _i, _i, _i, _i, _vp, _fp]),
     "tuna_describe_launch": (_i, [_i, _i, _i, _cfgp, _i, ctypes.c_char_p, _sz]),
     "tuna_set_multi_shape": (_i, [_i, _i]),
+    "tuna_set_multi_min_batch": (_i, [_i]),
     "tuna_multi_launches": (ctypes.c_ulonglong, []),
     "tuna_set_lean_kernels": (_i, [_i]),
     "tuna_lean_launches": (ctypes.c_ulonglong, []),

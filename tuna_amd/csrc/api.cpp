@@ -842,6 +842,7 @@ static int matmul_grouped_impl(const void *q, const void *x, const void *code, c
 // ---------------------------------------------------------------------------------------
 static std::atomic<int> g_multi_waves_m{0}, g_multi_prefetch{0};  // 0: the library's choice (diagnostic override)
 static std::atomic<unsigned long long> g_multi_launches{0};
+static std::atomic<int> g_multi_min_batch{2};  // batches shorter than this are launched problem by problem
 
 struct MultiPlan {
     MultiArgs args;
@@ -852,7 +853,7 @@ struct MultiPlan {
 // Whether problems[0..count) can run as one launch on a device of `cus` compute units; fills `plan`.
 static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, MultiPlan *plan)
 {
-    if (count < 2 || count > kMaxMultiProblems || cus < 1) return false;
+    if (count < g_multi_min_batch.load(std::memory_order_relaxed) || count > kMaxMultiProblems || cus < 1) return false;
     int waves_m = g_multi_waves_m.load(std::memory_order_relaxed);
     int prefetch = g_multi_prefetch.load(std::memory_order_relaxed);
     if (!prefetch) prefetch = 2;
@@ -883,14 +884,21 @@ static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, Mu
         mp.out = p.out;
         mp.m = p.m, mp.n = p.n, mp.k = p.k;
         mp.units_per_tile = p.k / (kStepK * unit_steps);
-        mp.unit_begin = (int)units;
+        a.unit_begin[i] = (int)units;
         mp.tile_begin = (int)tiles;
         const long long row_tiles = p.m / (64 * waves_m);
         units += row_tiles * mp.units_per_tile;
         tiles += row_tiles;
         if ((units + 1) * cus >= 0x7fffffffLL) return false;
     }
+    for (int i = count; i < kMaxMultiProblems; ++i) a.unit_begin[i] = 0x7fffffff;
     int n_wg = units < cus ? (int)units : cus;
+    if (n_wg > kMaxCus) n_wg = kMaxCus;
+    for (int w = 0, p = 0; w < n_wg; ++w) {
+        const long long first = (long long)w * units / n_wg;  // balanced_begin
+        while (p + 1 < count && first >= a.unit_begin[p + 1]) ++p;
+        a.first_problem[w] = (unsigned char)p;
+    }
     a.code = static_cast<const float *>(problems[0].code);
     a.n_problems = count;
     a.units_total = (int)units;
@@ -927,8 +935,8 @@ static int matmul_multi_impl(const tuna_gemm_problem *problems, int count, hipSt
         // the longest run of problems from `first` that one launch can take
         MultiPlan plan;
         int take = count - first < kMaxMultiProblems ? count - first : kMaxMultiProblems;
-        while (take >= 2 && !plan_multi(problems + first, take, cus, &plan)) --take;
-        if (take >= 2) {
+        while (take >= 1 && !plan_multi(problems + first, take, cus, &plan)) --take;
+        if (take >= 1) {
             if ((rc = provide_workspace(false, stream, plan.ws_bytes, plan.n_counters, &plan.args.ws, &plan.args.counters))) return rc;
             e = launch_gemm_multi(plan.args, plan.prefetch, dev, stream);
             if (e != hipSuccess) return hip_fail(e, "batched gemm launch");
@@ -1406,6 +1414,11 @@ TUNA_EXPORT int tuna_set_multi_shape(int waves_m, int prefetch)
     g_multi_waves_m.store(waves_m);
     g_multi_prefetch.store(prefetch);
     return TUNA_OK;
+}
+
+TUNA_EXPORT int tuna_set_multi_min_batch(int count)
+{
+    return g_multi_min_batch.exchange(count < 1 ? 1 : count);
 }
 
 TUNA_EXPORT unsigned long long tuna_multi_launches(void) { return g_multi_launches.load(); }

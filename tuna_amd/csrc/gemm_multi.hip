@@ -22,7 +22,7 @@ bool multi_variant_exists(int prefetch)
     return false;
 }
 
-size_t multi_lds_bytes() { return (size_t)kLutBytes + 2 * 32 * 1024 + 16; }
+size_t multi_lds_bytes() { return (size_t)kLutBytes + 2 * 32 * 1024 + 32 * 1024; }  // table, two x buffers, reduction area
 
 hipError_t launch_gemm_multi(const MultiArgs &args, int prefetch, int dev, hipStream_t stream)
 {

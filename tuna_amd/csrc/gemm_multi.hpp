@@ -15,7 +15,10 @@
 //     tile, or another problem - so that segment's first weights are in registers when its loop
 //     begins, and the reduction and store of the finished segment run under loads in flight.
 //   * x: the segment's k range in chunks of 1024 k, double-buffered in LDS as in gemm_mid.hpp
-//     ([8-k slot][token] pieces: conflict-free writes and B-fragment reads).
+//     ([8-k slot][token] pieces: conflict-free writes and B-fragment reads).  The last chunk of a
+//     segment prefetches the first chunk and the scales of the next segment instead, so a segment
+//     switch is an ordinary chunk switch and the reduction of the finished segment (through an LDS
+//     area of its own, two accumulator planes at a time) is the only work between two main loops.
 //   * A segment that is a whole row tile stores its output; a partial one hands its fp32 sums over
 //     through the workspace (write-through stores, explicit wait, arrival ticket) and the last of
 //     the row tile's contributors to arrive adds them in k order: deterministic, no atomics on the
@@ -36,9 +39,8 @@ struct MultiProblem {
     void *out;
     int m, n, k;
     int units_per_tile;  // k / (32 * waves_k * U)
-    int unit_begin;      // first unit of this problem in the batch's sequence
     int tile_begin;      // id of its first row tile (arrival counters)
-    int pad0, pad1;
+    int pad0, pad1, pad2;
 };
 
 struct MultiArgs {
@@ -50,10 +52,15 @@ struct MultiArgs {
     int waves_m, wk_log2;
     int n_wg;
     int swizzle;         // n_wg is a multiple of 8: consecutive shares sit on one XCD
+    // first unit of every problem in the batch's sequence, and the problem that holds the first unit of
+    // every workgroup: a workgroup finds the problem of a unit by walking on from there (its share
+    // rarely spans more than two problems), not through a chain of dependent fetches from problem 0
+    int unit_begin[kMaxMultiProblems];
+    unsigned char first_problem[kMaxCus];
     MultiProblem prob[kMaxMultiProblems];
 };
 
-template <int U>
+template <int U, bool DEFER = true>
 __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
 {
     constexpr int XB = 2;                  // 16-byte x pieces per thread and chunk: 16 tokens x 1024 k x 2 B / 1024 threads
@@ -61,8 +68,11 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
     constexpr uint32_t kXBuf = 32 * 1024;  // bytes of one x buffer
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char *lut = smem;
-    unsigned char *xbuf = smem + kLutBytes;                // two x buffers; the reduction planes after a segment's loop
-    volatile unsigned *ticket = reinterpret_cast<volatile unsigned *>(smem + kLutBytes + 2 * kXBuf);
+    unsigned char *xbuf = smem + kLutBytes;  // two x buffers
+    // reduction area: two accumulator planes of all 16 waves (32 KB); its first two words double as the
+    // arrival tickets of the hand-over, which are written only after every sum has been read
+    float *redf = reinterpret_cast<float *>(smem + kLutBytes + 2 * kXBuf);
+    volatile unsigned *ticket = reinterpret_cast<volatile unsigned *>(redf);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -102,10 +112,11 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         int u0;       // first unit of the row tile in the batch's sequence
         int upt;      // units per row tile
     };
-    int p_scan = 0;  // problem of the last segment looked up (segments are looked up in order)
+    int p_scan = a.first_problem[wg];  // problem of the last segment looked up (segments are looked up in order)
     auto seg_at = [&](int u) {
-        while (p_scan + 1 < a.n_problems && u >= a.prob[p_scan + 1].unit_begin) ++p_scan;
+        while (p_scan + 1 < a.n_problems && u >= a.unit_begin[p_scan + 1]) ++p_scan;
         const MultiProblem &pr = a.prob[p_scan];
+        const int unit_begin_p = a.unit_begin[p_scan];
         Seg s;
         s.q = pr.q;
         s.x = reinterpret_cast<const unsigned char *>(pr.x);
@@ -113,7 +124,7 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         s.out = reinterpret_cast<f16 *>(pr.out);
         s.m = pr.m, s.n = pr.n, s.k = pr.k;
         s.upt = pr.units_per_tile;
-        const int ul = u - pr.unit_begin;
+        const int ul = u - unit_begin_p;
         const int row_tile = (int)((unsigned)ul / (unsigned)s.upt);
         const int u_in = ul - row_tile * s.upt;
         const int left_tile = s.upt - u_in, left_wg = t_end - u;
@@ -136,34 +147,29 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
     u32x4 wq[U];
     u32x4 xv[XB];
     f32x4 sc32;
-    // x chunk `c` of segment s: piece b of this thread is k-step (tid + b*1024) / 64 of the chunk, token
-    // row lane / 4, 8-k group lane % 4 (every quad of lanes reads 64 contiguous bytes of one token row).
-    // Steps past the segment's end or k are clamped to valid addresses; their data is never read.
+    // x chunk `c` of segment sg (its steps 32c .. 32c+31 in walking order): piece b of this thread is
+    // k-step (tid + b*1024) / 64 of the chunk, token row lane / 4, 8-k group lane % 4 (every quad of
+    // lanes reads 64 contiguous bytes of one token row).
     const int x_row = lane >> 2, x_grp = lane & 3;
-#define TUNA_MULTI_X_LOAD(s, c)                                                                 \
+#define TUNA_MULTI_X_LOAD(sg, c)                                                                \
     {                                                                                          \
-        const uint32_t row_off_ = (uint32_t)min(x_row, (s).n - 1) * ((uint32_t)(s).k * 2u);    \
+        const uint32_t row_off_ = (uint32_t)min(x_row, (sg).n - 1) * ((uint32_t)(sg).k * 2u);  \
         _Pragma("unroll") for (int b = 0; b < XB; ++b)                                         \
         {                                                                                      \
-            const int ks_ = (tid + b * 1024) >> 6;                                             \
-            const int kk_ = min(((s).sb + (c) * kChunkSteps + ks_) * 32 + x_grp * 8, (s).k - 8); \
-            xv[b] = *reinterpret_cast<const u32x4 *>((s).x + row_off_ + (uint32_t)kk_ * 2u);   \
+            /* steps past the segment's end: clamped to a valid address, never read */         \
+            const int p_ = min((c) * kChunkSteps + ((tid + b * 1024) >> 6), (sg).nsteps - 1);  \
+            xv[b] = *reinterpret_cast<const u32x4 *>((sg).x + row_off_ + (uint32_t)(((sg).sb + p_) * 32 + x_grp * 8) * 2u); \
         }                                                                                      \
     }
-    // (token rows past n are zeroed: they feed output columns that are never stored, but must not be NaN-free garbage either way)
-#define TUNA_MULTI_X_STORE(s, buf)                                                              \
+    // (token rows past n are zeroed, as the other kernels do; they feed output columns that are never stored)
+#define TUNA_MULTI_X_STORE(n_, buf)                                                             \
     {                                                                                          \
-        const bool ok_ = x_row < (s).n;                                                        \
+        const bool ok_ = x_row < (n_);                                                         \
         _Pragma("unroll") for (int b = 0; b < XB; ++b)                                         \
         {                                                                                      \
             const int ks_ = (tid + b * 1024) >> 6;                                             \
             *reinterpret_cast<u32x4 *>((buf) + (ks_ * 4 + x_grp) * 256 + x_row * 16) = ok_ ? xv[b] : u32x4{0u, 0u, 0u, 0u}; \
         }                                                                                      \
-    }
-#define TUNA_MULTI_SMALL_LOADS(s)                                                               \
-    {                                                                                          \
-        sc32 = *reinterpret_cast<const f32x4 *>((s).absmax + (s).row0 + wm * 64 + i16 * 4);    \
-        TUNA_MULTI_X_LOAD(s, 0)                                                                \
     }
 
     const float code_lane = a.code[i16];
@@ -174,7 +180,8 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
 #pragma unroll
         for (int u = 0; u < U; ++u) wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(qp + (size_t)u * wq_stride + lb));
     }
-    TUNA_MULTI_SMALL_LOADS(cur)
+    sc32 = *reinterpret_cast<const f32x4 *>(cur.absmax + cur.row0 + wm * 64 + i16 * 4);
+    TUNA_MULTI_X_LOAD(cur, 0)
 
     // ---- decode table (see gemm_kernel.hpp), built while the first loads are in flight --------
     {
@@ -192,11 +199,52 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
             for (int b = 0; b < 4; ++b) reinterpret_cast<u32x4 *>(lut)[p0 + b * 1024] = u32x4{v[b], v[b], v[b], v[b]};
         }
     }
+    // chunk 0 of the first segment into buffer 0; one barrier publishes it and the table
+    TUNA_MULTI_X_STORE(cur.n, xbuf)
+    __syncthreads();
+    uint32_t xsel = 0;  // buffer that holds the chunk about to be consumed
 
     const uint32_t xb_lane = (uint32_t)g * 256u + (uint32_t)i16 * 16u + (uint32_t)wk * 1024u;
     const uint32_t wstep = 1024u << wk_log2;  // LDS bytes between this wave's consecutive k-steps
     const size_t seg_floats = (size_t)a.waves_m * 1024;
     const size_t plane_floats = (size_t)16 * 256;  // one accumulator plane of all 16 waves
+
+    // partial segments waiting for their hand-over, by slot (n_contrib == 0: none)
+    struct Pending {
+        f16 *out;
+        int m, n, row0, tile_id;
+        unsigned w_lo, n_contrib, first_slot;
+    };
+    Pending pend0 = {}, pend1 = {};
+    // Last contributor of a row tile: every partial is in memory; add them in k order and store.
+    auto finish = [&](const Pending &pd) {
+        if (tid == 0) __hip_atomic_store(a.counters + pd.tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int f = ((i << wk_log2) + wk) * 64 + lane;
+            if (f >= 256) continue;
+            const float *src = a.ws + ((size_t)pd.w_lo * 2 + pd.first_slot) * seg_floats + (size_t)wm * 1024 + (size_t)f * 4;
+            f32x4 s4 = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (unsigned sp0 = 0; sp0 < pd.n_contrib; sp0 += 4) {  // four contributors per round trip, summed in k order
+                f32x4 pv[4];
+                const float *ps[4];
+#pragma unroll
+                for (unsigned b = 0; b < 4; ++b) {
+                    const unsigned sp = min(sp0 + b, pd.n_contrib - 1u);
+                    ps[b] = src + (size_t)sp * 2 * seg_floats - (sp ? (size_t)pd.first_slot * seg_floats : (size_t)0);
+                }
+                load_partials4(ps[0], ps[1], ps[2], ps[3], pv[0], pv[1], pv[2], pv[3]);
+#pragma unroll
+                for (unsigned b = 0; b < 4; ++b)
+                    if (sp0 + b < pd.n_contrib) s4 += pv[b];
+            }
+            const int l = f >> 2, v = f & 3;
+            const int tok = l & 15;
+            if (tok < pd.n)
+                store_features4(pd.out, nullptr, TUNA_EPILOGUE_NONE, (size_t)tok, pd.m, pd.row0 + wm * 64 + (l >> 4) * 16 + v * 4, s4[0],
+                                s4[1], s4[2], s4[3]);
+        }
+    };
 
     for (;;) {
         const bool has_next = cur.next < t_end;
@@ -214,10 +262,6 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-        // chunk 0 into buffer 0: the x area is free (the barrier that ended the previous segment)
-        TUNA_MULTI_X_STORE(cur, xbuf)
-        __syncthreads();
-
         const int n_it = cur.nsteps >> wk_log2;                                  // this wave's iterations, a multiple of U
         const int n_chunks = (cur.nsteps + kChunkSteps - 1) / kChunkSteps;
         // refills: iteration it + U of this segment; in the last ring turn the first U iterations of
@@ -230,8 +274,16 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         int it = 0;
         for (int c = 0; c < n_chunks; ++c) {
             const bool more = c + 1 < n_chunks;
-            TUNA_MULTI_X_LOAD(cur, more ? c + 1 : c)
-            const unsigned char *xb = xbuf + (c & 1) * kXBuf + xb_lane;
+            // the chunk behind this one: of this segment, or - in its last chunk - the first one of
+            // the next segment together with that segment's scales (no next segment: this chunk
+            // again, dropped).  One unconditional batch of loads either way.
+            if (more) {
+                TUNA_MULTI_X_LOAD(cur, c + 1)
+            } else {
+                TUNA_MULTI_X_LOAD(nxt, has_next ? 0 : c)
+                sc32 = *reinterpret_cast<const f32x4 *>(nxt.absmax + nxt.row0 + wm * 64 + i16 * 4);
+            }
+            const unsigned char *xb = xbuf + xsel * kXBuf + xb_lane;
             const int its = min(chunk_its, n_it - it);
             for (int sl = 0; sl < its; sl += U) {
                 if (it + U >= n_it) {
@@ -252,23 +304,27 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
                 rp += (size_t)U * wq_stride;
                 it += U;
             }
-            if (more) TUNA_MULTI_X_STORE(cur, xbuf + ((c + 1) & 1) * kXBuf)
+            // the other buffer was last read in the previous chunk, which ended with a barrier
+            TUNA_MULTI_X_STORE(more ? cur.n : nxt.n, xbuf + (xsel ^ 1u) * kXBuf)
             __syncthreads();
+            xsel ^= 1u;
         }
 
-        // ---- the next segment's scales and first x chunk, behind its ring loads --------------------
-        const Seg done = cur;
-        if (has_next) TUNA_MULTI_SMALL_LOADS(nxt)
-
-        // ---- reduction over the waves along k (layouts of gemm_kernel.hpp) and store ------------------
-        float *redf = reinterpret_cast<float *>(xbuf);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) reinterpret_cast<f32x4 *>(redf + j * plane_floats)[(size_t)wave * 64 + lane] = acc[j];
-        __syncthreads();
+        // ---- reduction over the waves along k (layouts of gemm_kernel.hpp), two planes at a time ----
+        // (the area was last read before a chunk barrier of this segment; the next segment's first
+        // chunk is already staged, so its main loop starts right behind the stores below)
         float o[4][4];
-        sum_planes_any<4, 32>(wk_log2, redf, plane_floats, wm, wk, lane, o, 0);
-        const bool partial = done.part >= 0;
-        float *mine = a.ws + ((size_t)wg * 2 + (size_t)(partial ? done.part : 0)) * seg_floats + (size_t)wm * 1024;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            if (h) __syncthreads();  // the first half's sums have been read
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                reinterpret_cast<f32x4 *>(redf + j * plane_floats)[(size_t)wave * 64 + lane] = acc[2 * h + j];
+            __syncthreads();
+            sum_planes_any<2, 32>(wk_log2, redf, plane_floats, wm, wk, lane, o, 2 * h);
+        }
+        const bool partial = cur.part >= 0;
+        float *mine = a.ws + ((size_t)wg * 2 + (size_t)(partial ? cur.part : 0)) * seg_floats + (size_t)wm * 1024;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int f = ((i << wk_log2) + wk) * 64 + lane;
@@ -276,65 +332,59 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
             if (!partial) {
                 const int l = f >> 2, v = f & 3;
                 const int tok = l & 15;
-                if (tok < done.n)
-                    store_features4(done.out, nullptr, TUNA_EPILOGUE_NONE, (size_t)tok, done.m, done.row0 + wm * 64 + (l >> 4) * 16 + v * 4,
+                if (tok < cur.n)
+                    store_features4(cur.out, nullptr, TUNA_EPILOGUE_NONE, (size_t)tok, cur.m, cur.row0 + wm * 64 + (l >> 4) * 16 + v * 4,
                                     o[i][0], o[i][1], o[i][2], o[i][3]);
             } else {
                 store_partial(mine + (size_t)f * 4, f32x4{o[i][0], o[i][1], o[i][2], o[i][3]});
             }
         }
         if (partial) {
-            // hand-over (see gemm_kernel.hpp): stores complete, barrier, arrival ticket, the last one sums
-            unsigned w_lo, n_contrib, first_slot;
-            {
-                const unsigned T = (unsigned)a.units_total, nw = (unsigned)a.n_wg;
-                const unsigned u0 = (unsigned)done.u0, u1 = u0 + (unsigned)done.upt - 1u;
-                w_lo = ((u0 + 1u) * nw - 1u) / T;
-                n_contrib = ((u1 + 1u) * nw - 1u) / T - w_lo + 1u;
-                first_slot = (w_lo * T) / nw < u0 ? 1u : 0u;
-            }
-            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-            __syncthreads();
-            if (tid == 0) *ticket = __hip_atomic_fetch_add(a.counters + done.tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __syncthreads();
-            if (*ticket == n_contrib - 1u) {
-                if (tid == 0) __hip_atomic_store(a.counters + done.tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int f = ((i << wk_log2) + wk) * 64 + lane;
-                    if (f >= 256) continue;
-                    const float *src = a.ws + ((size_t)w_lo * 2 + first_slot) * seg_floats + (size_t)wm * 1024 + (size_t)f * 4;
-                    f32x4 s4 = f32x4{0.f, 0.f, 0.f, 0.f};
-                    for (unsigned sp0 = 0; sp0 < n_contrib; sp0 += 4) {  // four contributors per round trip, summed in k order
-                        f32x4 pv[4];
-                        const float *ps[4];
-#pragma unroll
-                        for (unsigned b = 0; b < 4; ++b) {
-                            const unsigned sp = min(sp0 + b, n_contrib - 1u);
-                            ps[b] = src + (size_t)sp * 2 * seg_floats - (sp ? (size_t)first_slot * seg_floats : (size_t)0);
-                        }
-                        load_partials4(ps[0], ps[1], ps[2], ps[3], pv[0], pv[1], pv[2], pv[3]);
-#pragma unroll
-                        for (unsigned b = 0; b < 4; ++b)
-                            if (sp0 + b < n_contrib) s4 += pv[b];
-                    }
-                    const int l = f >> 2, v = f & 3;
-                    const int tok = l & 15;
-                    if (tok < done.n)
-                        store_features4(done.out, nullptr, TUNA_EPILOGUE_NONE, (size_t)tok, done.m,
-                                        done.row0 + wm * 64 + (l >> 4) * 16 + v * 4, s4[0], s4[1], s4[2], s4[3]);
-                }
+            Pending pd;
+            pd.out = cur.out;
+            pd.m = cur.m, pd.n = cur.n, pd.row0 = cur.row0, pd.tile_id = cur.tile_id;
+            const unsigned T = (unsigned)a.units_total, nw = (unsigned)a.n_wg;
+            const unsigned u0 = (unsigned)cur.u0, u1 = u0 + (unsigned)cur.upt - 1u;
+            pd.w_lo = ((u0 + 1u) * nw - 1u) / T;
+            pd.n_contrib = ((u1 + 1u) * nw - 1u) / T - pd.w_lo + 1u;
+            pd.first_slot = (pd.w_lo * T) / nw < u0 ? 1u : 0u;
+            if constexpr (DEFER) {
+                // left to the end of the workgroup's share, where its at most two partial segments (slots 0
+                // and 1) are handed over together
+                if (cur.part == 0) pend0 = pd;  // (two named copies: an array indexed by the slot would live in scratch memory)
+                else pend1 = pd;
+            } else {
+                __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): a workgroup-scope fence does not wait for global stores
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                __syncthreads();  // also: every sum has been read, the ticket word is free
+                if (tid == 0) ticket[0] = __hip_atomic_fetch_add(a.counters + pd.tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __syncthreads();
+                if (ticket[0] == pd.n_contrib - 1u) finish(pd);
             }
         }
         if (!has_next) break;
-        __syncthreads();  // every read of the reduction planes is done: the x area may be written again
         cur = nxt;
         lb = lb_next;
     }
+
+    // ---- hand-over of the partial segments (see gemm_kernel.hpp): stores complete, barrier, arrival
+    //      tickets, and for every row tile whose last contributor this workgroup is, the sum in k order
+    if constexpr (DEFER) {
+        if (pend0.n_contrib | pend1.n_contrib) {
+            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): a workgroup-scope fence does not wait for global stores
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __syncthreads();  // also: every sum has been read, the ticket words are free
+            if (tid == 0 && pend0.n_contrib)
+                ticket[0] = __hip_atomic_fetch_add(a.counters + pend0.tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (tid == 64 && pend1.n_contrib)  // (another wave: the two round trips overlap)
+                ticket[1] = __hip_atomic_fetch_add(a.counters + pend1.tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            if (pend0.n_contrib && ticket[0] == pend0.n_contrib - 1u) finish(pend0);
+            if (pend1.n_contrib && ticket[1] == pend1.n_contrib - 1u) finish(pend1);
+        }
+    }
 #undef TUNA_MULTI_X_LOAD
 #undef TUNA_MULTI_X_STORE
-#undef TUNA_MULTI_SMALL_LOADS
 }
 
 }  // namespace tuna
