@@ -1204,3 +1204,36 @@ def test_matmul_multi_in_a_captured_graph_replays_correctly():
         for p, g in zip(probs, got):
             assert not torch.isnan(g).any()
             assert torch.equal(g.view(torch.int16), p[4].view(torch.int16)), rep
+
+
+@pytest.mark.parametrize("m,n,k,ckw", [
+    (1024, 16, 2048, dict(waves_m=4, waves_k=4, prefetch=2, x_chunk=512)),
+    (2048, 7, 4096, dict(waves_m=4, waves_k=4, prefetch=4, x_chunk=1024)),
+    (1024, 16, 8192, dict(waves_m=2, waves_k=8, prefetch=2, x_chunk=512)),
+    (4096, 1, 2048, dict(waves_m=8, waves_k=2, prefetch=4, x_chunk=256)),
+    (3072, 16, 14336, dict(waves_m=1, waves_k=16, prefetch=2, x_chunk=1024)),
+])
+def test_balanced_split_through_the_batched_kernel_equals_general_kernel_bit_for_bit(m, n, k, ckw):
+    """A balanced split over 16-wave workgroups is run by the batched kernel as a batch of one.  It
+    walks the segments gemm_kernel's balanced split walks, in the same order, and sums in the same
+    order: identical bits (the general kernel is reached with the twins switched off), and both agree
+    with the oracle."""
+    import torch
+
+    from tuna_amd import _lib, ops
+
+    c = cfg(split_k=0, **ckw)
+    assert ops.describe_launch(m, n, k, c).startswith("gemm_multi_kernel")
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=m + k)
+    before = _lib.lib().tuna_multi_launches()
+    got = run_gemm(q, x, code, absmax, m, n, k, config=c, prefill=float("nan"))
+    assert _lib.lib().tuna_multi_launches() == before + 1
+    prev = ops.set_lean_kernels(False)
+    try:
+        assert ops.describe_launch(m, n, k, c).startswith("gemm_kernel")
+        general = run_gemm(q, x, code, absmax, m, n, k, config=c, prefill=float("nan"))
+    finally:
+        ops.set_lean_kernels(prev)
+    assert np.array_equal(got, general)
+    ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1)
+    assert rel_err(f16_bits_to_f64(got), ref) <= REL_TOL

@@ -658,6 +658,99 @@ static int check_ptr(const void *p, const char *name, size_t align)
     return TUNA_OK;
 }
 
+// ---------------------------------------------------------------------------------------
+// Several independent GEMMs in one call: batches of up to kMaxMultiProblems problems that the
+// batched persistent kernel can run (gemm_multi.hpp) are one launch each; anything else is
+// launched problem by problem on the same stream.
+// ---------------------------------------------------------------------------------------
+static std::atomic<int> g_multi_waves_m{0}, g_multi_prefetch{0};  // 0: the library's choice (diagnostic override)
+static std::atomic<unsigned long long> g_multi_launches{0};
+static std::atomic<int> g_multi_min_batch{2};  // batches shorter than this are launched problem by problem
+
+struct MultiPlan {
+    MultiArgs args;
+    int prefetch;
+    size_t ws_bytes, n_counters;
+};
+
+// Whether problems[0..count) can run as one launch on a device of `cus` compute units; fills `plan`.
+// waves_m / prefetch: 0 = chosen here.
+static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, MultiPlan *plan, int waves_m = 0, int prefetch = 0)
+{
+    if (count < 1 || count > kMaxMultiProblems || cus < 1) return false;
+    if (!waves_m) waves_m = g_multi_waves_m.load(std::memory_order_relaxed);
+    if (!prefetch) prefetch = g_multi_prefetch.load(std::memory_order_relaxed);
+    if (!prefetch) {
+        // deeper rings pay on long streams; short batches finish sooner with fewer bytes requested ahead
+        unsigned long long bytes = 0;
+        for (int i = 0; i < count; ++i) bytes += (unsigned long long)problems[i].m * (unsigned long long)problems[i].k / 2;
+        prefetch = bytes >= (200ull << 20) ? 4 : 2;
+    }
+    if (!multi_variant_exists(prefetch)) return false;
+    if (!waves_m) {
+        // 256-row tiles (4 x 4 waves) when every problem allows, else narrower tiles and more waves along k
+        waves_m = 4;
+        for (int i = 0; i < count; ++i)
+            while (waves_m > 1 && problems[i].m % (64 * waves_m)) waves_m >>= 1;
+    }
+    if (waves_m != 1 && waves_m != 2 && waves_m != 4 && waves_m != 8 && waves_m != 16) return false;
+    const int waves_k = 16 / waves_m;
+    if ((32 / waves_k) % prefetch) return false;  // an x chunk of 32 k-steps is whole ring turns of every wave
+    const int unit_steps = waves_k * prefetch;
+    MultiArgs &a = plan->args;
+    memset(&a, 0, sizeof(a));
+    long long units = 0, tiles = 0;
+    for (int i = 0; i < count; ++i) {
+        const tuna_gemm_problem &p = problems[i];
+        if (p.n > 16 || p.m % (64 * waves_m) || p.k % (kStepK * unit_steps)) return false;
+        if ((unsigned long long)p.m * (unsigned long long)p.k / 2 >= (1ull << 32) || p.k >= (1 << 23)) return false;
+        if (reinterpret_cast<uintptr_t>(p.absmax) % 16) return false;
+        if (p.code != problems[0].code) return false;  // one decode table per launch
+        MultiProblem &mp = a.prob[i];
+        mp.q = static_cast<const uint8_t *>(p.q);
+        mp.x = p.x;
+        mp.absmax = static_cast<const float *>(p.absmax);
+        mp.out = p.out;
+        mp.m = p.m, mp.n = p.n, mp.k = p.k;
+        mp.units_per_tile = p.k / (kStepK * unit_steps);
+        a.unit_begin[i] = (int)units;
+        mp.tile_begin = (int)tiles;
+        const long long row_tiles = p.m / (64 * waves_m);
+        units += row_tiles * mp.units_per_tile;
+        tiles += row_tiles;
+        if ((units + 1) * cus >= 0x7fffffffLL) return false;
+    }
+    for (int i = count; i < kMaxMultiProblems; ++i) a.unit_begin[i] = 0x7fffffff;
+    int n_wg = units < cus ? (int)units : cus;
+    if (n_wg > kMaxCus) n_wg = kMaxCus;
+    for (int w = 0, p = 0; w < n_wg; ++w) {
+        const long long first = (long long)w * units / n_wg;  // balanced_begin
+        while (p + 1 < count && first >= a.unit_begin[p + 1]) ++p;
+        a.first_problem[w] = (unsigned char)p;
+    }
+    a.code = static_cast<const float *>(problems[0].code);
+    a.n_problems = count;
+    a.units_total = (int)units;
+    a.waves_m = waves_m;
+    a.wk_log2 = log2i(waves_k);
+    a.n_wg = n_wg;
+    a.swizzle = (n_wg % 8 == 0) ? 1 : 0;
+    plan->prefetch = prefetch;
+    plan->ws_bytes = (size_t)n_wg * 2 * waves_m * 4096;
+    plan->n_counters = (size_t)tiles;
+    return true;
+}
+
+// A dense launch the batched kernel (gemm_multi.hpp) takes as a batch of one: balanced split, 64 rows
+// per wave, 16 waves, one token tile, the GEMM's own decode, no fused epilogue.  (plan_multi checks
+// the shape's alignment.)  Off with the diagnostic switch that turns the other twins off.
+static bool stream_applies(const tuna_gemm_config &c, int n, int decode, int epilogue)
+{
+    return c.split_k == 0 && !c.lds_tile_rows && c.rows_per_wave == kRowsPerLoad && c.waves_m >= 1 && c.waves_m * c.waves_k == 16 &&
+           c.token_tiles == 1 && n <= 16 && decode == TUNA_DECODE_GEMM && epilogue == TUNA_EPILOGUE_NONE &&
+           (c.prefetch == 2 || c.prefetch == 4) && set_lean_kernels(-1) != 0;
+}
+
 static int matmul_impl(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n, int k,
                        const tuna_gemm_config *cfg, int decode, hipStream_t stream, int epilogue = TUNA_EPILOGUE_NONE,
                        const void *residual = nullptr, bool static_ws = false)
@@ -706,6 +799,22 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
     }
     GemmPlan plan;
     if ((rc = plan_gemm(m, n, k, c, decode, &plan))) return rc;
+    if (stream_applies(c, n, decode, epilogue)) {
+        // a balanced split over 16-wave workgroups: the batched kernel with a batch of one walks the same
+        // segments as gemm_kernel's balanced split and keeps its weight ring full across them
+        int dev = 0, cus = 0;
+        hipError_t e = device_cus(&dev, &cus);
+        if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+        const tuna_gemm_problem one = {q, x, code, absmax, out, m, n, k};
+        MultiPlan mp;
+        if (plan_multi(&one, 1, cus, &mp, c.waves_m, c.prefetch)) {
+            if ((rc = provide_workspace(static_ws, stream, mp.ws_bytes, mp.n_counters, &mp.args.ws, &mp.args.counters))) return rc;
+            e = launch_gemm_multi(mp.args, mp.prefetch, dev, stream);
+            if (e != hipSuccess) return hip_fail(e, "gemm launch");
+            g_multi_launches.fetch_add(1, std::memory_order_relaxed);
+            return TUNA_OK;
+        }
+    }
     plan.args.q = static_cast<const uint8_t *>(q);
     plan.args.x = x;
     plan.args.code = static_cast<const float *>(code);
@@ -835,83 +944,6 @@ static int matmul_grouped_impl(const void *q, const void *x, const void *code, c
     return TUNA_OK;
 }
 
-// ---------------------------------------------------------------------------------------
-// Several independent GEMMs in one call: batches of up to kMaxMultiProblems problems that the
-// batched persistent kernel can run (gemm_multi.hpp) are one launch each; anything else is
-// launched problem by problem on the same stream.
-// ---------------------------------------------------------------------------------------
-static std::atomic<int> g_multi_waves_m{0}, g_multi_prefetch{0};  // 0: the library's choice (diagnostic override)
-static std::atomic<unsigned long long> g_multi_launches{0};
-static std::atomic<int> g_multi_min_batch{2};  // batches shorter than this are launched problem by problem
-
-struct MultiPlan {
-    MultiArgs args;
-    int prefetch;
-    size_t ws_bytes, n_counters;
-};
-
-// Whether problems[0..count) can run as one launch on a device of `cus` compute units; fills `plan`.
-static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, MultiPlan *plan)
-{
-    if (count < g_multi_min_batch.load(std::memory_order_relaxed) || count > kMaxMultiProblems || cus < 1) return false;
-    int waves_m = g_multi_waves_m.load(std::memory_order_relaxed);
-    int prefetch = g_multi_prefetch.load(std::memory_order_relaxed);
-    if (!prefetch) prefetch = 2;
-    if (!multi_variant_exists(prefetch)) return false;
-    if (!waves_m) {
-        // 256-row tiles (4 x 4 waves) when every problem allows, else narrower tiles and more waves along k
-        waves_m = 4;
-        for (int i = 0; i < count; ++i)
-            while (waves_m > 1 && problems[i].m % (64 * waves_m)) waves_m >>= 1;
-    }
-    if (waves_m != 1 && waves_m != 2 && waves_m != 4 && waves_m != 8 && waves_m != 16) return false;
-    const int waves_k = 16 / waves_m;
-    if ((32 / waves_k) % prefetch) return false;  // an x chunk of 32 k-steps is whole ring turns of every wave
-    const int unit_steps = waves_k * prefetch;
-    MultiArgs &a = plan->args;
-    memset(&a, 0, sizeof(a));
-    long long units = 0, tiles = 0;
-    for (int i = 0; i < count; ++i) {
-        const tuna_gemm_problem &p = problems[i];
-        if (p.n > 16 || p.m % (64 * waves_m) || p.k % (kStepK * unit_steps)) return false;
-        if ((unsigned long long)p.m * (unsigned long long)p.k / 2 >= (1ull << 32) || p.k >= (1 << 23)) return false;
-        if (reinterpret_cast<uintptr_t>(p.absmax) % 16) return false;
-        if (p.code != problems[0].code) return false;  // one decode table per launch
-        MultiProblem &mp = a.prob[i];
-        mp.q = static_cast<const uint8_t *>(p.q);
-        mp.x = p.x;
-        mp.absmax = static_cast<const float *>(p.absmax);
-        mp.out = p.out;
-        mp.m = p.m, mp.n = p.n, mp.k = p.k;
-        mp.units_per_tile = p.k / (kStepK * unit_steps);
-        a.unit_begin[i] = (int)units;
-        mp.tile_begin = (int)tiles;
-        const long long row_tiles = p.m / (64 * waves_m);
-        units += row_tiles * mp.units_per_tile;
-        tiles += row_tiles;
-        if ((units + 1) * cus >= 0x7fffffffLL) return false;
-    }
-    for (int i = count; i < kMaxMultiProblems; ++i) a.unit_begin[i] = 0x7fffffff;
-    int n_wg = units < cus ? (int)units : cus;
-    if (n_wg > kMaxCus) n_wg = kMaxCus;
-    for (int w = 0, p = 0; w < n_wg; ++w) {
-        const long long first = (long long)w * units / n_wg;  // balanced_begin
-        while (p + 1 < count && first >= a.unit_begin[p + 1]) ++p;
-        a.first_problem[w] = (unsigned char)p;
-    }
-    a.code = static_cast<const float *>(problems[0].code);
-    a.n_problems = count;
-    a.units_total = (int)units;
-    a.waves_m = waves_m;
-    a.wk_log2 = log2i(waves_k);
-    a.n_wg = n_wg;
-    a.swizzle = (n_wg % 8 == 0) ? 1 : 0;
-    plan->prefetch = prefetch;
-    plan->ws_bytes = (size_t)n_wg * 2 * waves_m * 4096;
-    plan->n_counters = (size_t)tiles;
-    return true;
-}
-
 static int matmul_multi_impl(const tuna_gemm_problem *problems, int count, hipStream_t stream)
 {
     if (count < 0 || (count > 0 && !problems)) return fail(TUNA_ERR_INVALID_ARG, "problems is null or count=%d negative", count);
@@ -935,8 +967,9 @@ static int matmul_multi_impl(const tuna_gemm_problem *problems, int count, hipSt
         // the longest run of problems from `first` that one launch can take
         MultiPlan plan;
         int take = count - first < kMaxMultiProblems ? count - first : kMaxMultiProblems;
-        while (take >= 1 && !plan_multi(problems + first, take, cus, &plan)) --take;
-        if (take >= 1) {
+        const int min_batch = g_multi_min_batch.load(std::memory_order_relaxed);
+        while (take >= min_batch && !plan_multi(problems + first, take, cus, &plan)) --take;
+        if (take >= min_batch) {
             if ((rc = provide_workspace(false, stream, plan.ws_bytes, plan.n_counters, &plan.args.ws, &plan.args.counters))) return rc;
             e = launch_gemm_multi(plan.args, plan.prefetch, dev, stream);
             if (e != hipSuccess) return hip_fail(e, "batched gemm launch");
@@ -1400,6 +1433,14 @@ TUNA_EXPORT int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config
     }
     GemmPlan plan;
     if ((rc = plan_gemm(m, n, k, c, decode_mode, &plan))) return rc;
+    if (stream_applies(c, n, decode_mode, TUNA_EPILOGUE_NONE)) {
+        const tuna_gemm_problem one = {buf, buf, buf, nullptr, buf, m, n, k};  // (only sizes and alignment are looked at)
+        MultiPlan mp;
+        if (plan_multi(&one, 1, kMaxCus, &mp, c.waves_m, c.prefetch)) {
+            snprintf(buf, len, "gemm_multi_kernel<U=%d> waves_m=%d waves_k=%d", mp.prefetch, c.waves_m, c.waves_k);
+            return TUNA_OK;
+        }
+    }
     int cus = kMaxCus, dev = 0, v = 0;
     if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
         cus = v;
@@ -1423,7 +1464,7 @@ TUNA_EXPORT int tuna_set_multi_min_batch(int count)
 
 TUNA_EXPORT unsigned long long tuna_multi_launches(void) { return g_multi_launches.load(); }
 
-TUNA_EXPORT int tuna_set_lean_kernels(int enabled) { return tuna::set_lean_kernels(enabled); }
+TUNA_EXPORT int tuna_set_lean_kernels(int enabled) { return tuna::set_lean_kernels(enabled ? 1 : 0); }
 
 TUNA_EXPORT unsigned long long tuna_lean_launches(void) { return tuna::lean_launches(); }
 

@@ -103,7 +103,10 @@ static std::atomic<unsigned long long> g_lean_launches{0};
 
 unsigned long long lean_launches() { return g_lean_launches.load(); }
 
-int set_lean_kernels(int enabled) { return g_lean_enabled.exchange(enabled ? 1 : 0); }
+int set_lean_kernels(int enabled)  // negative: query only
+{
+    return enabled < 0 ? g_lean_enabled.load() : g_lean_enabled.exchange(enabled ? 1 : 0);
+}
 
 // Launches the lean kernel computes exactly like the general one (conditions in gemm_lean.hpp).
 static const LeanVariant *lean_applies(const GemmPlan &plan, int cus)
