@@ -214,6 +214,43 @@ def time_quantize(ops, synth, torch, dev):
                          "algorithmic_bytes_per_launch": int(2.5 * qm * qk), "avg_launch_us": round(us, 2)}}
 
 
+def multi_layer_sweep(ops, synth, torch, dev, names, n, layers, iters=None, seed0=10_000):
+    """`layers` calls of tuna_matmul_multi, each with the GEMMs `names` of one layer (distinct seeded weights per
+    layer), back to back: us per call, packed-weight GB/s.  The independent-problems reading of a layer: what
+    a benchmark sweep or a batch of unrelated projections can use; a real decoder layer's GEMMs feed one another."""
+    from tuna_amd.quantize import nf4_codebook
+
+    code = nf4_codebook(dev)
+    batches, total_bytes = [], 0
+    xs = {nm: synth.make_x_torch(n, synth.SHAPES[nm][1], seed0, dev) for nm in names}
+    outs = [torch.empty((n, synth.SHAPES[nm][0]), dtype=torch.float16, device=dev) for nm in names]  # one per problem of a launch
+    for layer in range(layers):
+        b = []
+        for j, nm in enumerate(names):
+            m, k = synth.SHAPES[nm]
+            q, a = synth.make_weights_torch(m, k, seed0 + layer * len(names) + j, dev)
+            b.append((xs[nm], q, a, code, outs[j], m, n, k))
+        batches.append(b)
+    total_bytes = sum(synth.SHAPES[nm][0] * synth.SHAPES[nm][1] // 2 for nm in names)
+    iters = iters or 2 * layers
+    best = None
+    for use_graph in (False, True):
+        ms = ops.time_matmul_multi(batches, warmup=layers, iters=iters, use_graph=use_graph)
+        us = ms * 1000.0 / iters
+        if best is None or us < best[0]:
+            best = (us, "graph" if use_graph else "stream")
+    us = best[0]
+    del batches
+    torch.cuda.empty_cache()
+    return {
+        "launch": "multi", "gemms_per_launch": len(names), "us_per_launch": round(us, 2),
+        "us_per_gemm_mean": round(us / len(names), 3), "ms_all": round(us * layers / 1000, 3),
+        "packed_bytes_per_launch": total_bytes, "gbs": round(total_bytes / (us * 1e-6) / 1e9, 1),
+        "frac_hbm": round(total_bytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "enqueue": best[1],
+        "kernel": "tuna::gemm_multi_kernel",
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -329,6 +366,16 @@ def main():
             torch.cuda.empty_cache()
         line["shapes"] = shapes
         line["min_frac_hbm_over_shapes"] = min(v["frac_hbm"] for v in shapes.values())
+        # every shape again as batches of 8 independent problems per launch (tuna_matmul_multi, distinct weights):
+        # what the per-launch fixed time costs each shape, beside the one-GEMM-per-launch numbers above
+        shapes_multi = {}
+        for name in synth.SHAPES:
+            sets = max(2, min(16, (4 << 30) // (8 * synth.SHAPES[name][0] * synth.SHAPES[name][1] // 2)))
+            r = multi_layer_sweep(ops, synth, torch, dev, [name] * 8, n, layers=sets, iters=max(20, 2 * sets), seed0=3000)
+            shapes_multi[name] = {"launch": "multi", "gemms_per_launch": 8, "us_per_gemm": r["us_per_gemm_mean"],
+                                  "gbs": r["gbs"], "frac_hbm": r["frac_hbm"], "enqueue": r["enqueue"], "kernel": r["kernel"]}
+        line["shapes_multi_x8"] = shapes_multi
+        line["min_frac_hbm_over_shapes_multi_x8"] = min(v["frac_hbm"] for v in shapes_multi.values())
         line["dequant"] = time_dequant_shapes(ops, synth, torch, dev)
         line["quantize"] = time_quantize(ops, synth, torch, dev)
 
@@ -382,6 +429,11 @@ def main():
             }
         except torch.OutOfMemoryError as e:  # pragma: no cover
             sweeps["llama70b_80_layers"] = {"error": str(e)[:200]}
+        # the same 80 layers with the four GEMMs of a layer in ONE launch (tuna_matmul_multi): one call per layer
+        try:
+            sweeps["llama70b_80_layers_multi"] = multi_layer_sweep(ops, synth, torch, dev, names, n, layers=80)
+        except torch.OutOfMemoryError as e:  # pragma: no cover
+            sweeps["llama70b_80_layers_multi"] = {"error": str(e)[:200]}
         # token sweep on the Llama-70B layer set
         tok = {}
         for nt in (1, 16, 64, 256, 1024):
