@@ -195,23 +195,43 @@ def time_dequant_shapes(ops, synth, torch, dev, names=("mistral_attn_out", "mist
 
 
 def time_quantize(ops, synth, torch, dev):
+    """Device quantizer + packer (fp16 weights in, packed codes and scales out) on 4096 x 4096, per-row and
+    per-64 scales: back-to-back launches through the C ABI on preallocated buffers, HIP events around them."""
+    import ctypes
+
+    from tuna_amd import _lib
+    from tuna_amd.quantize import nf4_codebook
+
     qm, qk = synth.SHAPES["mistral_attn_out"]
-    wq_ = (torch.randn((qm, qk), device=dev) * 0.02).to(torch.float16)
-    for _ in range(3):
-        ops.quantize(wq_)
-    torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    ev0.record()
-    for _ in range(20):
-        ops.quantize(wq_)
-    ev1.record()
-    torch.cuda.synchronize()
-    us = ev0.elapsed_time(ev1) * 1000.0 / 20
-    gbs = 2.5 * qm * qk / (us * 1e-6) / 1e9       # fp16 weights in (2 bytes each), packed codes out (half a byte each)
-    return {"m": qm, "k": qk, "us": round(us, 2), "gbs_fp16_in": round(2.0 * qm * qk / (us * 1e-6) / 1e9, 1),
-            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "tuna::quantize_kernel",
-                         "algorithmic_bytes_per_launch": int(2.5 * qm * qk), "avg_launch_us": round(us, 2)}}
+    L = _lib.lib()
+    code = nf4_codebook(dev)
+    ws = [(torch.randn((qm, qk), device=dev) * 0.02).to(torch.float16) for _ in range(16)]   # 16 x 33.5 MB: beyond the caches
+    q = torch.empty((qm // 8, qk // 8, 32), dtype=torch.uint8, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    res = {}
+    for label, bs in (("per_row", qk), ("per_64", 64)):
+        absmax = torch.empty((qm * (qk // bs),), dtype=torch.float32, device=dev)
+        def launch(i):
+            _lib.check(L.tuna_quantize_blockwise(ws[i % len(ws)].data_ptr(), code.data_ptr(), q.data_ptr(), absmax.data_ptr(), qm, qk,
+                                                 bs, stream))
+        for i in range(5):
+            launch(i)
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        iters = 100
+        ev0.record()
+        for i in range(iters):
+            launch(i)
+        ev1.record()
+        torch.cuda.synchronize()
+        us = ev0.elapsed_time(ev1) * 1000.0 / iters
+        nbytes = 2.5 * qm * qk + 4 * qm * (qk // bs)    # fp16 in, half a byte per weight and the scales out
+        gbs = nbytes / (us * 1e-6) / 1e9
+        res[label] = {"m": qm, "k": qk, "block_size": bs, "us": round(us, 2), "gbs_fp16_in": round(2.0 * qm * qk / (us * 1e-6) / 1e9, 1),
+                      "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                   "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "tuna::quantize_kernel",
+                                   "algorithmic_bytes_per_launch": int(nbytes), "avg_launch_us": round(us, 2)}}
+    return res
 
 
 def multi_layer_sweep(ops, synth, torch, dev, names, n, layers, iters=None, seed0=10_000):

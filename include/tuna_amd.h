@@ -199,6 +199,23 @@ int tuna_dequant_ex(const void *q, const void *absmax, const void *code, void *o
  * has this only as Python on torch tensors. */
 int tuna_quantize(const void *w, const void *code, void *q, void *absmax, int m, int k, void *stream);
 
+/* Scale blocks finer than a row.  The reference's quantizer takes a block_size (test.py:7-17): the
+ * weights, flattened row-major, are cut into blocks of block_size elements with one absmax each,
+ * so for k a multiple of block_size element (r, c) uses absmax[r * (k/block_size) + c/block_size];
+ * its kernels only ever run block_size == k (test.py:81, kernel.cu:2904).  The three entry points
+ * below take absmax fp32 [m, k/block_size] in that layout; block_size == k is the plain op.
+ *   tuna_quantize_blockwise : block_size 8, 16, 32, 64, 128, 256 or k.
+ *   tuna_dequant_blockwise  : any multiple of 8 that divides k.
+ *   tuna_matmul_blockwise   : block_size 64, 128, 256, ... (a multiple of 64 that divides k) with m
+ *                             a multiple of 16 and k of 256; TUNA_DECODE_GEMM rounding,
+ *                             fp16(code) * fp16(absmax of the block), as in tuna_matmul.       */
+int tuna_quantize_blockwise(const void *w, const void *code, void *q, void *absmax, int m, int k,
+                            int block_size, void *stream);
+int tuna_dequant_blockwise(const void *q, const void *absmax, const void *code, void *out, int m, int k,
+                           int block_size, int decode_mode, void *stream);
+int tuna_matmul_blockwise(const void *q, const void *x, const void *code, const void *absmax,
+                          void *out, int m, int n, int k, int block_size, void *stream);
+
 /* Shape -> config.  Replaces the if-chain of kernel.cu:3018-3156 over the constants of
  * configs.cu:56-3331 by a table lookup on (m, n-bucket, k) with a derived fallback.
  * Runs on the host only (no device needed).  Returns 1 in *from_table when the shape

@@ -59,6 +59,14 @@ int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int va
 int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config *cfg, int decode_mode,
                          char *buf, size_t len);
 
+/* Self-test of the quantizer's division: the kernel divides by a block's maximum with a refined
+ * reciprocal and one fused correction instead of the general IEEE sequence; this runs that
+ * division for every pair of fp16 values (w, a) with a > 0 finite and |w| <= a - all the quotients
+ * the quantizer can form - against the IEEE division on the device (zeros of either sign count as
+ * equal: the quotient is only ever compared or subtracted from).  `counts`: two zeroed device
+ * uint64; counts[0] receives the pairs checked, counts[1] the mismatches. */
+int tuna_selftest_quantizer_division(void *counts, void *stream);
+
 /* Diagnostic override of the batched kernel's workgroup shape (tuna_matmul_multi): waves along the
  * rows (1, 2, 4, 8 or 16 of the workgroup's 16 waves; 0 = the library's choice) and ring depth
  * (2 or 4; 0 = the library's choice).  For A/B timing. */

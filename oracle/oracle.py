@@ -63,6 +63,12 @@ def lib():
         L.orc_dequant.argtypes = [vp, vp, vp, vp, i32, i32, i32]
         L.orc_quantize.restype = i32
         L.orc_quantize.argtypes = [vp, vp, vp, vp, i32, i32]
+        L.orc_quantize_blk.restype = i32
+        L.orc_quantize_blk.argtypes = [vp, vp, vp, vp, i32, i32, i32]
+        L.orc_dequant_blk.restype = i32
+        L.orc_dequant_blk.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32]
+        L.orc_gemm_rows_f64_blk.restype = i32
+        L.orc_gemm_rows_f64_blk.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp, i32]
         L.orc_gemm.restype = i32
         L.orc_gemm.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32]
         L.orc_gemm_rows.restype = i32
@@ -156,25 +162,29 @@ def unpack(q: np.ndarray, m: int, k: int) -> np.ndarray:
     return codes
 
 
-def dequant(q, absmax, code, m, k, mode=D2) -> np.ndarray:
-    """-> fp16 bit patterns uint16 [m, k]."""
+def dequant(q, absmax, code, m, k, mode=D2, block_size=None) -> np.ndarray:
+    """-> fp16 bit patterns uint16 [m, k].  block_size: weights per scale along a row (absmax is then
+    [m, k/block_size]); None = one scale per row."""
     q, absmax, code = _c(q, np.uint8), _c(absmax, np.float32), _c(code, np.float32)
+    bs = k if block_size is None else int(block_size)
+    assert absmax.size == m * (k // bs)
     out = np.empty((m, k), np.uint16)
-    rc = lib().orc_dequant(_p(q), _p(absmax), _p(code), _p(out), m, k, mode)
+    rc = lib().orc_dequant_blk(_p(q), _p(absmax), _p(code), _p(out), m, k, mode, bs)
     if rc:
         raise ValueError(f"orc_dequant rc={rc}")
     return out
 
 
-def quantize(w_bits, code, m, k):
-    """fp16 bit patterns [m, k] -> (packed uint8 [m/8, k/8, 32], absmax float32 [m])."""
+def quantize(w_bits, code, m, k, block_size=None):
+    """fp16 bit patterns [m, k] -> (packed uint8 [m/8, k/8, 32], absmax float32 [m] or [m, k/block_size])."""
     w_bits, code = _c(w_bits, np.uint16), _c(code, np.float32)
+    bs = k if block_size is None else int(block_size)
     q = np.empty((m // 8, k // 8, 32), np.uint8)
-    absmax = np.empty(m, np.float32)
-    rc = lib().orc_quantize(_p(w_bits), _p(code), _p(q), _p(absmax), m, k)
+    absmax = np.empty(m * (k // bs), np.float32)
+    rc = lib().orc_quantize_blk(_p(w_bits), _p(code), _p(q), _p(absmax), m, k, bs)
     if rc:
         raise ValueError(f"orc_quantize rc={rc}")
-    return q, absmax
+    return q, (absmax if block_size is None else absmax.reshape(m, k // bs))
 
 
 def gemm(q, x, code, absmax, m, n, k, mode=D1, acc64=True, rows=None) -> np.ndarray:
@@ -195,17 +205,19 @@ def gemm(q, x, code, absmax, m, n, k, mode=D1, acc64=True, rows=None) -> np.ndar
     return out
 
 
-def gemm_f64(q, x, code, absmax, m, n, k, mode=D1, rows=None) -> np.ndarray:
-    """Un-rounded float64 sums, [n, m] (or [n, len(rows)])."""
+def gemm_f64(q, x, code, absmax, m, n, k, mode=D1, rows=None, block_size=None) -> np.ndarray:
+    """Un-rounded float64 sums, [n, m] (or [n, len(rows)]).  block_size as in dequant."""
     q, absmax, code = _c(q, np.uint8), _c(absmax, np.float32), _c(code, np.float32)
     x = _c(x, np.uint16)
+    bs = k if block_size is None else int(block_size)
+    assert absmax.size == m * (k // bs)
     if rows is None:
         rows_a, nr, rp = None, m, None
     else:
         rows_a = np.ascontiguousarray(rows, np.int32)
         nr, rp = len(rows_a), _p(rows_a)
     out = np.empty((n, nr), np.float64)
-    rc = lib().orc_gemm_rows_f64(_p(q), _p(x), _p(code), _p(absmax), _p(out), m, n, k, mode, rp, nr)
+    rc = lib().orc_gemm_rows_f64_blk(_p(q), _p(x), _p(code), _p(absmax), _p(out), m, n, k, mode, bs, rp, nr)
     if rc:
         raise ValueError(f"orc_gemm_rows_f64 rc={rc}")
     return out

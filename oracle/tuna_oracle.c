@@ -26,6 +26,10 @@
  *       orc_dequant.  All-zero rows: the reference divides by zero, every candidate
  *       distance is NaN and torch.argmin over an all-NaN column returns index 0;
  *       pinned by running that torch expression (CPU torch) in the test.
+ *   *_blk       : the same functions with one scale per block of block_size consecutive weights
+ *       of a row (test.py:7-17 layout); block_size == k is the plain function.  Checked against
+ *       numpy gathers / matmul with the scales expanded per element, and the quantizer against
+ *       the torch expressions of test.py:15-53 run on the CPU with block_size < k.
  *   orc_gemm*   : textbook contraction; checked against numpy float64 matmul,
  *       linearity, one-hot read-out of the decoded weights, row permutation
  */
@@ -215,17 +219,30 @@ static void build_row_lut(uint16_t lut[16], const float *code, float absmax, int
         lut[i] = (mode == ORC_D1) ? orc_decode_d1(code[i], absmax) : orc_decode_d2(code[i], absmax);
 }
 
+/* Scale blocks.  The reference's quantizer takes a block_size (test.py:7-9): the weights, flattened
+ * row-major, are cut into blocks of block_size elements and every block gets its own absmax
+ * (test.py:15-17), i.e. element (r, c) of an [m, k] matrix with k a multiple of block_size uses
+ * absmax[(r*k + c) / block_size] = absmax[r * (k/block_size) + c / block_size].  The reference's
+ * kernels only ever run block_size == k (one scale per row: kernel.cu:2904 indexes absmax by row,
+ * test.py:81); the *_blk functions below restate the same arithmetic for finer blocks and the
+ * plain functions are their block_size == k case. */
+static inline float blk_scale(const float *absmax, int r, int c, int k, int bs)
+{
+    return absmax[(size_t)r * (size_t)(k / bs) + (size_t)(c / bs)];
+}
+
 /* out[m, k] fp16 row-major (kernel.cu:3238); mode selects D1 or D2 */
-ORC_API int orc_dequant(const uint8_t *q, const float *absmax, const float *code,
-                        uint16_t *out, int m, int k, int mode)
+ORC_API int orc_dequant_blk(const uint8_t *q, const float *absmax, const float *code,
+                            uint16_t *out, int m, int k, int mode, int bs)
 {
     if (m <= 0 || k <= 0 || (m & 7) || (k & 7)) return 1;
     if (mode != ORC_D1 && mode != ORC_D2) return 2;
+    if (bs <= 0 || k % bs) return 5;
 #pragma omp parallel for schedule(static)
     for (int r = 0; r < m; r++) {
         uint16_t lut[16];
-        build_row_lut(lut, code, absmax[r], mode);
         for (int c = 0; c < k; c++) {
+            if (c % bs == 0) build_row_lut(lut, code, blk_scale(absmax, r, c, k, bs), mode);
             uint8_t b = q[q_offset(r, c, k)];
             uint8_t nib = (c & 1) ? (b & 15u) : (uint8_t)(b >> 4);
             out[(size_t)r * k + c] = lut[nib];
@@ -234,46 +251,60 @@ ORC_API int orc_dequant(const uint8_t *q, const float *absmax, const float *code
     return 0;
 }
 
+ORC_API int orc_dequant(const uint8_t *q, const float *absmax, const float *code,
+                        uint16_t *out, int m, int k, int mode)
+{
+    return orc_dequant_blk(q, absmax, code, out, m, k, mode, k);
+}
+
 /* ------------------------------------------------------------------------- */
 /* Quantizer (test.py:7-68 with block_size == k): absmax[r] = max |w[r, :]| as   */
 /* fp32; normalized = fp32(w) / absmax (fp32 division, test.py:41: fp16 / fp32   */
 /* promotes to fp32); code index = argmin_j |normalized - code[j]| in fp32 with  */
 /* the first index on ties (torch.argmin, test.py:50-53); packed as test.py:55-65 */
 /* ------------------------------------------------------------------------- */
-ORC_API int orc_quantize(const uint16_t *w, const float *code, uint8_t *q, float *absmax, int m, int k)
+ORC_API int orc_quantize_blk(const uint16_t *w, const float *code, uint8_t *q, float *absmax, int m, int k, int bs)
 {
     if (m <= 0 || k <= 0 || (m & 7) || (k & 7)) return 1;
+    if (bs <= 0 || k % bs) return 5;
+    const int nb = k / bs;
     memset(q, 0, (size_t)m * k / 2);
 #pragma omp parallel for schedule(static)
     for (int mb = 0; mb < m / 8; mb++) {
         for (int r8 = 0; r8 < 8; r8++) {
             const int r = mb * 8 + r8;
-            float amax = 0.f;
-            for (int c = 0; c < k; c++) {
-                const float v = fabsf(orc_f16_to_f32(w[(size_t)r * k + c]));
-                if (v > amax) amax = v;
-            }
-            absmax[r] = amax;
-            for (int c = 0; c < k; c++) {
-                int best = 0; /* all-NaN candidates: torch.argmin returns index 0 */
-                if (amax > 0.f) {
-                    const volatile float nv = orc_f16_to_f32(w[(size_t)r * k + c]) / amax; /* fp32, no excess precision */
-                    float bd = 0.f;
-                    best = 0;
-                    for (int j = 0; j < 16; j++) {
-                        const volatile float d = fabsf(nv - code[j]);
-                        if (j == 0 || d < bd) {
-                            bd = d;
-                            best = j;
+            for (int b0 = 0; b0 < nb; b0++) {
+                float amax = 0.f;
+                for (int c = b0 * bs; c < (b0 + 1) * bs; c++) {
+                    const float v = fabsf(orc_f16_to_f32(w[(size_t)r * k + c]));
+                    if (v > amax) amax = v;
+                }
+                absmax[(size_t)r * nb + b0] = amax;
+                for (int c = b0 * bs; c < (b0 + 1) * bs; c++) {
+                    int best = 0; /* all-NaN candidates: torch.argmin returns index 0 */
+                    if (amax > 0.f) {
+                        const volatile float nv = orc_f16_to_f32(w[(size_t)r * k + c]) / amax; /* fp32, no excess precision */
+                        float bd = 0.f;
+                        for (int j = 0; j < 16; j++) {
+                            const volatile float d = fabsf(nv - code[j]);
+                            if (j == 0 || d < bd) {
+                                bd = d;
+                                best = j;
+                            }
                         }
                     }
+                    uint8_t *b = &q[q_offset(r, c, k)];
+                    *b |= (c & 1) ? (uint8_t)best : (uint8_t)(best << 4);
                 }
-                uint8_t *b = &q[q_offset(r, c, k)];
-                *b |= (c & 1) ? (uint8_t)best : (uint8_t)(best << 4);
             }
         }
     }
     return 0;
+}
+
+ORC_API int orc_quantize(const uint16_t *w, const float *code, uint8_t *q, float *absmax, int m, int k)
+{
+    return orc_quantize_blk(w, code, q, absmax, m, k, k);
 }
 
 /* ------------------------------------------------------------------------- */
@@ -340,32 +371,41 @@ ORC_API int orc_gemm(const uint8_t *q, const uint16_t *x, const float *code,
 
 /* Same contraction with the exact double sums returned (no final rounding):
  * lets tests measure the GPU's error against the un-rounded value. */
-ORC_API int orc_gemm_rows_f64(const uint8_t *q, const uint16_t *x, const float *code,
-                              const float *absmax, double *out, int m, int n, int k,
-                              int mode, const int32_t *rows, int n_rows)
+ORC_API int orc_gemm_rows_f64_blk(const uint8_t *q, const uint16_t *x, const float *code,
+                                  const float *absmax, double *out, int m, int n, int k,
+                                  int mode, int bs, const int32_t *rows, int n_rows)
 {
     if (m <= 0 || k <= 0 || n < 0 || (m & 7) || (k & 7)) return 1;
     if (mode != ORC_D1 && mode != ORC_D2) return 2;
+    if (bs <= 0 || k % bs) return 5;
     int nr = rows ? n_rows : m;
     int bad = 0;
 #pragma omp parallel for schedule(static)
     for (int ri = 0; ri < nr; ri++) {
         int r = rows ? rows[ri] : ri;
         if (r < 0 || r >= m) { bad = 1; continue; }
+        double *w = (double *)malloc((size_t)k * sizeof(double));
         uint16_t lut[16];
-        double lutd[16];
-        build_row_lut(lut, code, absmax[r], mode);
-        for (int i = 0; i < 16; i++) lutd[i] = (double)orc_f16_to_f32(lut[i]);
+        for (int c = 0; c < k; c++) {
+            if (c % bs == 0) build_row_lut(lut, code, blk_scale(absmax, r, c, k, bs), mode);
+            uint8_t b = q[q_offset(r, c, k)];
+            w[c] = (double)orc_f16_to_f32(lut[(c & 1) ? (b & 15u) : (b >> 4)]);
+        }
         for (int t = 0; t < n; t++) {
             double s = 0.0;
-            for (int c = 0; c < k; c++) {
-                uint8_t b = q[q_offset(r, c, k)];
-                s += (double)orc_f16_to_f32(x[(size_t)t * k + c]) * lutd[(c & 1) ? (b & 15u) : (b >> 4)];
-            }
+            for (int c = 0; c < k; c++) s += (double)orc_f16_to_f32(x[(size_t)t * k + c]) * w[c];
             out[(size_t)t * nr + ri] = s;
         }
+        free(w);
     }
     return bad ? 4 : 0;
+}
+
+ORC_API int orc_gemm_rows_f64(const uint8_t *q, const uint16_t *x, const float *code,
+                              const float *absmax, double *out, int m, int n, int k,
+                              int mode, const int32_t *rows, int n_rows)
+{
+    return orc_gemm_rows_f64_blk(q, x, code, absmax, out, m, n, k, mode, k, rows, n_rows);
 }
 
 /* ------------------------------------------------------------------------- */

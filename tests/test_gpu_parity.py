@@ -1237,3 +1237,147 @@ def test_balanced_split_through_the_batched_kernel_equals_general_kernel_bit_for
     assert np.array_equal(got, general)
     ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1)
     assert rel_err(f16_bits_to_f64(got), ref) <= REL_TOL
+
+
+# ----------------------------------------------------------------------------- scale blocks finer than a row
+@pytest.mark.parametrize("m,k,bs", [(8, 64, 8), (64, 256, 64), (72, 1152, 128), (136, 1032, 24), (4096, 4096, 64), (4096, 4096, 128)])
+@pytest.mark.parametrize("mode", [O.D2, O.D1])
+def test_blockwise_dequant_bit_exact(m, k, bs, mode):
+    import torch
+
+    from tuna_amd import ops
+
+    rng = np.random.default_rng(m + k + bs)
+    q = rng.integers(0, 256, size=(m // 8, k // 8, 32), dtype=np.uint8)
+    code = O.nf4_codebook()
+    absmax = rng.uniform(0.004, 0.03, size=(m, k // bs)).astype(np.float32)
+    dq, dc, da = to_dev(q, code, absmax)
+    out = torch.full((m, k), float("nan"), dtype=torch.float16, device="cuda")
+    ops.dequant(dq, da, dc, out, m, k, decode_mode=mode, block_size=bs)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), O.dequant(q, absmax, code, m, k, mode=mode, block_size=bs))
+
+
+@pytest.mark.parametrize("m,k,bs", [(8, 64, 8), (64, 256, 64), (72, 1096, None), (72, 1024, 128), (4096, 4096, 64), (4096, 4096, 128),
+                                    (4096, 4096, None), (512, 8192, None), (64, 14336, 256), (256, 14336, None)])
+def test_device_quantizer_blockwise_and_every_row_length_is_bit_exact(m, k, bs):
+    """The rewritten quantizer kernel (rows held in registers up to k = 4096, two passes beyond; block
+    maxima by shuffles; binary search for sorted codebooks) against the oracle: packed bytes and
+    scales identical, for per-row and per-block scales, incl. zero rows / blocks, near-midpoint
+    inputs, fp16 subnormals, and an unsorted codebook (the 16-comparison path)."""
+    import torch
+
+    from tuna_amd import ops
+
+    rng = np.random.default_rng(m * 7 + k + (bs or 0))
+    w = (rng.standard_normal((m, k)) * 0.03).astype(np.float16)
+    code = O.nf4_codebook()
+    w[1] = 0
+    w[2, :] = 0
+    w[2, 5] = np.float16(-0.25)
+    mids = ((code[:-1] + code[1:]) / 2).astype(np.float32)
+    w[3, :15] = (mids * 0.5).astype(np.float16)
+    w[3, 15] = np.float16(0.5)
+    w[4] = np.float16(6e-8)
+    if bs:
+        w[5, bs:2 * bs] = 0
+    for cb in (code, rng.standard_normal(16).astype(np.float32), np.sort(rng.standard_normal(16)).astype(np.float32)):
+        dw, dc = to_dev(w, cb)
+        q, a, _ = ops.quantize(dw, dc, block_size=bs)
+        torch.cuda.synchronize()
+        q_ref, a_ref = O.quantize(w.view(np.uint16), cb, m, k, block_size=bs)
+        assert np.array_equal(a.cpu().numpy(), a_ref)
+        assert np.array_equal(q.cpu().numpy(), q_ref)
+
+
+@pytest.mark.parametrize("m,n,k,bs", [(64, 16, 256, 64), (256, 5, 1024, 128), (1024, 16, 4096, 64), (512, 37, 2048, 256),
+                                      (4096, 16, 4096, 128), (2048, 1, 8192, 64)])
+def test_blockwise_gemm_matches_oracle_and_reads_out_the_decode(m, n, k, bs):
+    """tuna_matmul_blockwise: one scale per `bs` weights of a row.  Against the oracle's float64 sums
+    over the blockwise D1 weights, and bit-exact through one-hot activations (out[t, r] = the decoded
+    weight W[r, col_t] with its block's scale)."""
+    import torch
+
+    from tuna_amd import ops
+
+    rng = np.random.default_rng(m + n + k + bs)
+    q, x, code, _ = make_inputs_np(m, n, k, seed=m + bs)
+    absmax = rng.uniform(0.005, 0.02, size=(m, k // bs)).astype(np.float16).astype(np.float32)
+    dq, dx, dc, da = to_dev(q, x, code, absmax)
+    out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+    ops.matmul_blockwise(dx, dq, da, dc, out, m, n, k, bs)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().view(np.uint16)
+    assert not np.isnan(got.view(np.float16)).any()
+    rows = np.sort(rng.choice(m, size=min(m, 256), replace=False)).astype(np.int32)
+    ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1, rows=rows, block_size=bs)
+    e = rel_err(f16_bits_to_f64(got[:, rows]), ref)
+    assert e <= REL_TOL, e
+    cols = rng.choice(k, size=n, replace=False)
+    xh = np.zeros((n, k), np.float16)
+    xh[np.arange(n), cols] = 1.0
+    dxh, = to_dev(xh)
+    ops.matmul_blockwise(dxh, dq, da, dc, out, m, n, k, bs)
+    torch.cuda.synchronize()
+    img = O.dequant(q, absmax, code, m, k, mode=O.D1, block_size=bs)
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), img[:, cols].T)
+
+
+def test_blockwise_entry_points_reject_what_they_cannot_run():
+    import torch
+
+    from tuna_amd import ops
+
+    q, x, code, _ = make_inputs_np(64, 16, 512, seed=1)
+    dq, dx, dc = to_dev(q, x, code)
+    da = torch.ones((64, 512 // 32), dtype=torch.float32, device="cuda")
+    out = torch.zeros((16, 64), dtype=torch.float16, device="cuda")
+    with pytest.raises(ops.TunaError):
+        ops.matmul_blockwise(dx, dq, da, dc, out, 64, 16, 512, 32)          # GEMM blocks start at 64
+    w = torch.zeros((64, 768), dtype=torch.float16, device="cuda")
+    with pytest.raises(ops.TunaError):
+        ops.quantize(w, dc, block_size=384)                                 # quantizer blocks: 8..256 (powers of two) or k
+    ops.quantize(w, dc, block_size=768)                                     # == k: the per-row op
+    torch.cuda.synchronize()
+
+
+def test_quantizer_division_is_the_ieee_division_for_every_quotient_it_can_form():
+    """The quantizer divides by a block's maximum with a refined reciprocal and one fused correction.
+    Every pair of fp16 values (w, a), a > 0 finite, |w| <= a - 1.0e9 pairs, all there are - gives
+    the bits of the IEEE fp32 division."""
+    import torch
+
+    from tuna_amd import _lib
+
+    counts = torch.zeros(2, dtype=torch.int64, device="cuda")
+    _lib.check(_lib.lib().tuna_selftest_quantizer_division(counts.data_ptr(), None))
+    torch.cuda.synchronize()
+    n, bad = (int(v) for v in counts.cpu())
+    assert n == sum(2 * a + 2 for a in range(1, 0x7c00))      # for magnitude a: the bit patterns 0 .. a with either sign
+    assert bad == 0, f"{bad} of {n} quotients differ from the IEEE division"
+
+
+def test_quantizer_every_fp16_value_against_the_oracle():
+    """Rows that hold every fp16 value up to their maximum (k = 65536, per-row scale: the two-pass
+    variant) for maxima from the subnormals to 65504, and the same values with one scale per 64
+    (different maxima per block): packed bytes and scales identical to the oracle's."""
+    import torch
+
+    from tuna_amd import ops
+
+    rng = np.random.default_rng(3)
+    allbits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    maxima = np.array([0x3c00, 0x3999, 0x2266, 0x0001, 0x0155, 0x7bff, 0x5640, 0x1c03], np.uint16)   # 1.0, 0.7, 0.0125, ...
+    w = np.zeros((8, 65536), np.uint16)
+    for r, a in enumerate(maxima):
+        row = allbits.copy()
+        row[(row & 0x7fff) > a] = 0                       # larger magnitudes, infinities and NaNs out
+        w[r] = rng.permutation(row)
+    code = O.nf4_codebook()
+    dw, dc = to_dev(w.view(np.float16), code)
+    for bs in (None, 64, 256):
+        q, a, _ = ops.quantize(dw, dc, block_size=bs)
+        torch.cuda.synchronize()
+        q_ref, a_ref = O.quantize(w, code, 8, 65536, block_size=bs)
+        assert np.array_equal(a.cpu().numpy(), a_ref)
+        assert np.array_equal(q.cpu().numpy(), q_ref), bs

@@ -346,3 +346,52 @@ def test_quantizer_round_trip_recovers_the_codes():
     assert np.array_equal(absmax, scale)
     assert np.array_equal(q, pack_codes_np(idx))
     assert np.array_equal(O.dequant(q, absmax, code, m, k, mode=O.D2), w_bits)
+
+
+# ----------------------------------------------------------------------------- scale blocks finer than a row
+@pytest.mark.parametrize("bs", [8, 64, 128, 256])
+def test_blockwise_dequant_and_gemm_against_numpy(bs):
+    """One scale per block of `bs` weights of a row, absmax [m, k/bs] (the quantizer's layout,
+    test.py:15-17): dequant against a numpy gather with the scales expanded per element and the
+    elementwise decode (pinned exhaustively above), the GEMM against numpy float64 matmul."""
+    rng = np.random.default_rng(bs)
+    m, n, k = 64, 5, 512
+    idx = rng.integers(0, 16, size=(m, k)).astype(np.uint8)
+    q = O.pack(idx)
+    code = O.nf4_codebook()
+    absmax = rng.uniform(0.004, 0.03, size=(m, k // bs)).astype(np.float32)
+    per_elem = np.repeat(absmax, bs, axis=1)                       # [m, k]
+    for mode in (O.D1, O.D2):
+        want = O.decode(code[idx].ravel(), per_elem.ravel(), mode).reshape(m, k)
+        got = O.dequant(q, absmax, code, m, k, mode=mode, block_size=bs)
+        assert np.array_equal(got, want)
+        x = (rng.standard_normal((n, k)) * 0.1).astype(np.float16)
+        ref = x.astype(np.float64) @ want.view(np.float16).astype(np.float64).T
+        got64 = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=mode, block_size=bs)
+        assert np.allclose(got64, ref, rtol=1e-12, atol=1e-12)
+    # block_size == k is the per-row function
+    a_row = rng.uniform(0.004, 0.03, size=m).astype(np.float32)
+    assert np.array_equal(O.dequant(q, a_row, code, m, k, block_size=k), O.dequant(q, a_row, code, m, k))
+
+
+@pytest.mark.parametrize("bs", [8, 64, 128])
+def test_blockwise_quantizer_oracle_matches_torch_semantics(bs):
+    """The reference's quantizer with block_size < k is torch code (test.py:15-53); the product's
+    torch restatement of it (tuna_amd/quantize.py) run on the CPU pins the oracle's blockwise
+    quantizer, including a block of zeros (index 0) and near-midpoint inputs."""
+    import torch
+
+    from tuna_amd.quantize import quantize_blockwise_dynamic_4bit
+
+    rng = np.random.default_rng(100 + bs)
+    m, k = 16, 256
+    w, code = _quantizer_inputs(rng, m, k)
+    w[5, bs:2 * bs] = 0                                            # one all-zero block inside a non-zero row
+    qt, (at, _c) = quantize_blockwise_dynamic_4bit(torch.from_numpy(w.copy()), block_size=bs, preprocess=True)
+    q, a = O.quantize(w.view(np.uint16), code, m, k, block_size=bs)
+    assert np.array_equal(a.ravel(), at.numpy())
+    assert np.array_equal(q, qt.numpy())
+    # round trip: dequant of the quantized weights stays within half the widest code gap of the block's scale
+    img = O.dequant(q, a, code, m, k, mode=O.D2, block_size=bs).view(np.float16).astype(np.float32)
+    gap = np.diff(code).max() / 2
+    assert (np.abs(img - w.astype(np.float32)) <= gap * np.repeat(a, bs, axis=1) + 1e-6).all()

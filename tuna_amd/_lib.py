@@ -76,6 +76,9 @@ SIGNATURES = {
     "tuna_matmul_grouped": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _ip, _cfgp, _i, _vp]),
     "tuna_dequant": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "tuna_quantize": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "tuna_quantize_blockwise": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "tuna_dequant_blockwise": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "tuna_matmul_blockwise": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "tuna_dequant_ex": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "tuna_select_config": (_i, [_i, _i, _i, _cfgp, _ip]),
     "tuna_select_config_ex": (_i, [_i, _i, _i, _i, _cfgp, _ip]),
@@ -94,6 +97,7 @@ SIGNATURES = {
     "tuna_time_copy": (_i, [_vp, _vp, _sz, _i, _i, _vp, _fp]),
     "tuna_time_read": (_i, [_vp, _vp, _sz, _i, _i, _i, _i, _vp, _fp]),
     "tuna_describe_launch": (_i, [_i, _i, _i, _cfgp, _i, ctypes.c_char_p, _sz]),
+    "tuna_selftest_quantizer_division": (_i, [_vp, _vp]),
     "tuna_set_multi_shape": (_i, [_i, _i]),
     "tuna_set_multi_min_batch": (_i, [_i]),
     "tuna_multi_launches": (ctypes.c_ulonglong, []),

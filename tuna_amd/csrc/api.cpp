@@ -984,19 +984,44 @@ static int matmul_multi_impl(const tuna_gemm_problem *problems, int count, hipSt
     return TUNA_OK;
 }
 
-static int dequant_impl(const void *q, const void *absmax, const void *code, void *out, int m, int k, int decode,
+// Scale blocks: one absmax per block_size consecutive weights of a row (absmax [m, k/block_size], the
+// layout of the reference's quantizer for block_size < k, test.py:15-17); block_size == k is one per row.
+static int check_block_size(int k, int bs, bool pow2_up_to_256)
+{
+    if (bs == k) return TUNA_OK;
+    if (bs < 8 || (bs & 7) || k % bs) return fail(TUNA_ERR_INVALID_ARG, "block_size=%d must be a multiple of 8 that divides k=%d", bs, k);
+    if (pow2_up_to_256 && (!is_pow2(bs) || bs > 256))
+        return fail(TUNA_ERR_UNSUPPORTED, "block_size=%d: the quantizer takes 8, 16, 32, 64, 128, 256 or k", bs);
+    return TUNA_OK;
+}
+
+static int dequant_impl(const void *q, const void *absmax, const void *code, void *out, int m, int k, int bs, int decode,
                         hipStream_t stream)
 {
     int rc;
     if ((rc = check_shape(m, 1, k))) return rc;
     if (decode != TUNA_DECODE_GEMM && decode != TUNA_DECODE_DEQUANT)
         return fail(TUNA_ERR_INVALID_ARG, "decode_mode %d is neither TUNA_DECODE_GEMM nor TUNA_DECODE_DEQUANT", decode);
+    if ((rc = check_block_size(k, bs, false))) return rc;
     if ((rc = check_ptr(q, "q", 16)) || (rc = check_ptr(absmax, "absmax", 4)) || (rc = check_ptr(code, "code", 4)) ||
         (rc = check_ptr(out, "out", 16)))
         return rc;
     hipError_t e = launch_dequant(static_cast<const uint8_t *>(q), static_cast<const float *>(absmax),
-                                  static_cast<const float *>(code), out, m, k, decode, stream);
+                                  static_cast<const float *>(code), out, m, k, bs, decode, stream);
     if (e != hipSuccess) return hip_fail(e, "dequant launch");
+    return TUNA_OK;
+}
+
+static int quantize_impl(const void *w, const void *code, void *q, void *absmax, int m, int k, int bs, hipStream_t stream)
+{
+    int rc;
+    if ((rc = check_shape(m, 1, k))) return rc;
+    if ((rc = check_block_size(k, bs, true))) return rc;
+    if ((rc = check_ptr(w, "w", 16)) || (rc = check_ptr(code, "code", 4)) || (rc = check_ptr(q, "q", 16)) ||
+        (rc = check_ptr(absmax, "absmax", 4)))
+        return rc;
+    hipError_t e = launch_quantize(w, static_cast<const float *>(code), q, static_cast<float *>(absmax), m, k, bs, stream);
+    if (e != hipSuccess) return hip_fail(e, "quantize launch");
     return TUNA_OK;
 }
 
@@ -1138,26 +1163,60 @@ TUNA_EXPORT int tuna_matmul_grouped(const void *q, const void *x, const void *co
 
 TUNA_EXPORT int tuna_dequant(const void *q, const void *absmax, const void *code, void *out, int m, int k, void *stream)
 {
-    return dequant_impl(q, absmax, code, out, m, k, TUNA_DECODE_DEQUANT, static_cast<hipStream_t>(stream));
+    return dequant_impl(q, absmax, code, out, m, k, k, TUNA_DECODE_DEQUANT, static_cast<hipStream_t>(stream));
 }
 
 TUNA_EXPORT int tuna_quantize(const void *w, const void *code, void *q, void *absmax, int m, int k, void *stream)
 {
+    return quantize_impl(w, code, q, absmax, m, k, k, static_cast<hipStream_t>(stream));
+}
+
+TUNA_EXPORT int tuna_quantize_blockwise(const void *w, const void *code, void *q, void *absmax, int m, int k, int block_size,
+                                        void *stream)
+{
+    return quantize_impl(w, code, q, absmax, m, k, block_size, static_cast<hipStream_t>(stream));
+}
+
+TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n,
+                                      int k, int block_size, void *stream)
+{
+    if (block_size == k) return matmul_impl(q, x, code, absmax, out, m, n, k, nullptr, TUNA_DECODE_GEMM, static_cast<hipStream_t>(stream));
     int rc;
-    if ((rc = check_shape(m, 1, k))) return rc;
-    if ((rc = check_ptr(w, "w", 16)) || (rc = check_ptr(code, "code", 4)) || (rc = check_ptr(q, "q", 16)) ||
-        (rc = check_ptr(absmax, "absmax", 4)))
+    if ((rc = check_shape(m, n, k))) return rc;
+    if (block_size < 64 || !is_pow2(block_size) || k % block_size)
+        return fail(TUNA_ERR_UNSUPPORTED, "block_size=%d: the GEMM takes 64, 128, 256, ... (a power of two that divides k=%d) or k",
+                    block_size, k);
+    if (m % 16 || k % 256)
+        return fail(TUNA_ERR_UNSUPPORTED, "scale blocks need m a multiple of 16 and k of 256 (m=%d, k=%d)", m, k);
+    if ((unsigned long long)m * (unsigned long long)k / 2 >= (1ull << 32) || (unsigned long long)k * 32 >= (1ull << 32))
+        return fail(TUNA_ERR_UNSUPPORTED, "operands exceed the kernel's 32-bit offsets");
+    if ((n + 15) / 16 > 65535) return fail(TUNA_ERR_UNSUPPORTED, "n=%d needs more than 65535 token chunks", n);
+    if ((rc = check_ptr(q, "q", 16)) || (rc = check_ptr(x, "x", 16)) || (rc = check_ptr(code, "code", 4)) ||
+        (rc = check_ptr(absmax, "absmax", 4)) || (rc = check_ptr(out, "out", 16)))
         return rc;
-    hipError_t e = launch_quantize(w, static_cast<const float *>(code), q, static_cast<float *>(absmax), m, k,
-                                   static_cast<hipStream_t>(stream));
-    if (e != hipSuccess) return hip_fail(e, "quantize launch");
+    NarrowArgs a;
+    memset(&a, 0, sizeof(a));
+    a.q = static_cast<const uint8_t *>(q);
+    a.x = x;
+    a.code = static_cast<const float *>(code);
+    a.absmax = static_cast<const float *>(absmax);
+    a.out = out;
+    a.m = m, a.n = n, a.k = k;
+    hipError_t e = launch_gemm_blockwise(a, log2i(block_size) - 6, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "blockwise gemm launch");
     return TUNA_OK;
+}
+
+TUNA_EXPORT int tuna_dequant_blockwise(const void *q, const void *absmax, const void *code, void *out, int m, int k,
+                                       int block_size, int decode_mode, void *stream)
+{
+    return dequant_impl(q, absmax, code, out, m, k, block_size, decode_mode, static_cast<hipStream_t>(stream));
 }
 
 TUNA_EXPORT int tuna_dequant_ex(const void *q, const void *absmax, const void *code, void *out, int m, int k,
                                 int decode_mode, void *stream)
 {
-    return dequant_impl(q, absmax, code, out, m, k, decode_mode, static_cast<hipStream_t>(stream));
+    return dequant_impl(q, absmax, code, out, m, k, k, decode_mode, static_cast<hipStream_t>(stream));
 }
 
 TUNA_EXPORT int tuna_select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_table)
@@ -1379,7 +1438,7 @@ TUNA_EXPORT int tuna_time_dequant(const void *const *q_list, const void *const *
 {
     if (!q_list || !absmax_list) return fail(TUNA_ERR_INVALID_ARG, "q_list / absmax_list is null");
     auto launch = [&](int set, hipStream_t s) {
-        return dequant_impl(q_list[set], absmax_list[set], code, out, m, k, TUNA_DECODE_DEQUANT, s);
+        return dequant_impl(q_list[set], absmax_list[set], code, out, m, k, k, TUNA_DECODE_DEQUANT, s);
     };
     return time_loop(launch, n_sets, warmup, iters, 0, static_cast<hipStream_t>(stream), elapsed_ms);
 }
@@ -1447,6 +1506,15 @@ TUNA_EXPORT int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config
     else
         (void)hipGetLastError();
     describe_gemm_launch(plan, cus, buf, len);
+    return TUNA_OK;
+}
+
+TUNA_EXPORT int tuna_selftest_quantizer_division(void *counts, void *stream)
+{
+    int rc = check_ptr(counts, "counts", 8);
+    if (rc) return rc;
+    hipError_t e = launch_division_selftest(static_cast<unsigned long long *>(counts), static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "selftest launch");
     return TUNA_OK;
 }
 

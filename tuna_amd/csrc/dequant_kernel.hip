@@ -23,11 +23,13 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kDqUnroll = 4;  // 1 KB chunks per wave
 
-template <int DEC>
+// BLK: one scale per `bs` consecutive weights of a row, absmax [m, k/bs] (the layout the reference's
+// quantizer writes for block_size < k, test.py:15-17); otherwise one scale per row.
+template <int DEC, bool BLK>
 __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t *__restrict__ q,
                                                       const float *__restrict__ absmax,
                                                       const float *__restrict__ code,
-                                                      f16 *__restrict__ out, int m, int k)
+                                                      f16 *__restrict__ out, int m, int k, int bs)
 {
     __shared__ float cf[16];
     __shared__ f16 ch[16];
@@ -44,13 +46,16 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t *__restrict_
     if (mb >= (m >> 3)) return;
     const int half = lane & 1;
     const int kb_lane = blockIdx.x * (32 * kDqUnroll) + (lane >> 1);
+    const int nblk = BLK ? k / bs : 1;
 
     float s32[4];
     f16 s16[4];
+    if constexpr (!BLK) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        s32[j] = absmax[mb * 8 + half * 4 + j];
-        s16[j] = (f16)s32[j];
+        for (int j = 0; j < 4; ++j) {
+            s32[j] = absmax[mb * 8 + half * 4 + j];
+            s16[j] = (f16)s32[j];
+        }
     }
     const uint8_t *src = q + ((size_t)mb * kb_total) * 32 + half * 16;
     u32x4 w[kDqUnroll];
@@ -63,6 +68,14 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t *__restrict_
     for (int u = 0; u < kDqUnroll; ++u) {
         const int kb = kb_lane + u * 32;
         if (kb >= kb_total) continue;
+        if constexpr (BLK) {
+            const int blk = (kb * 8) / bs;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                s32[j] = absmax[(size_t)(mb * 8 + half * 4 + j) * nblk + blk];
+                s16[j] = (f16)s32[j];
+            }
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const uint32_t d = w[u][j];
@@ -81,16 +94,22 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t *__restrict_
 }
 
 hipError_t launch_dequant(const uint8_t *q, const float *absmax, const float *code, void *out,
-                          int m, int k, int decode, hipStream_t stream)
+                          int m, int k, int bs, int decode, hipStream_t stream)
 {
     const int kb_total = k >> 3;
     dim3 grid((kb_total + 32 * kDqUnroll - 1) / (32 * kDqUnroll), ((m >> 3) + 3) / 4, 1);
-    if (decode == TUNA_DECODE_DEQUANT)
-        hipLaunchKernelGGL(dequant_kernel<TUNA_DECODE_DEQUANT>, grid, dim3(256), 0, stream, q, absmax, code,
-                           reinterpret_cast<f16 *>(out), m, k);
-    else
-        hipLaunchKernelGGL(dequant_kernel<TUNA_DECODE_GEMM>, grid, dim3(256), 0, stream, q, absmax, code,
-                           reinterpret_cast<f16 *>(out), m, k);
+    f16 *o = reinterpret_cast<f16 *>(out);
+    if (bs == k) {
+        if (decode == TUNA_DECODE_DEQUANT)
+            hipLaunchKernelGGL((dequant_kernel<TUNA_DECODE_DEQUANT, false>), grid, dim3(256), 0, stream, q, absmax, code, o, m, k, bs);
+        else
+            hipLaunchKernelGGL((dequant_kernel<TUNA_DECODE_GEMM, false>), grid, dim3(256), 0, stream, q, absmax, code, o, m, k, bs);
+    } else {
+        if (decode == TUNA_DECODE_DEQUANT)
+            hipLaunchKernelGGL((dequant_kernel<TUNA_DECODE_DEQUANT, true>), grid, dim3(256), 0, stream, q, absmax, code, o, m, k, bs);
+        else
+            hipLaunchKernelGGL((dequant_kernel<TUNA_DECODE_GEMM, true>), grid, dim3(256), 0, stream, q, absmax, code, o, m, k, bs);
+    }
     return hipGetLastError();
 }
 
@@ -154,69 +173,255 @@ hipError_t launch_copy(const void *src, void *dst, size_t bytes, hipStream_t str
     return hipGetLastError();
 }
 
-// fp16 weights [m, k] -> packed 4-bit codes + per-row absmax: the device form of the reference
-// harness's quantize_blockwise_dynamic_4bit with one scale per row (test.py:7-68).  Same
-// arithmetic: absmax = max |w| as fp32; normalized = fp32(w) / absmax with an fp32 division
-// (test.py:41, fp16 / fp32 promotes to fp32); index = argmin_j |normalized - code[j]| in
-// fp32, first index on ties (torch.argmin, test.py:50-53); nibble packing of test.py:55-65.
-// An all-zero row gets index 0: the reference divides by zero there, every candidate distance is
-// NaN, and torch.argmin over an all-NaN column returns index 0 (test.py:41-53).
-// One workgroup per block row (8 weight rows): 32 threads per row, 16-byte reads; a thread
-// turns 8 consecutive k of one row into one dword of the 32-byte record.
-__global__ __launch_bounds__(256) void quantize_kernel(const f16 *__restrict__ w, const float *__restrict__ code,
-                                                       uint32_t *__restrict__ q32, float *__restrict__ absmax, int m, int k)
+// fp16 weights [m, k] -> packed 4-bit codes + absmax: the device form of the reference harness's
+// quantize_blockwise_dynamic_4bit (test.py:7-68).  Same arithmetic: absmax = max |w| over a block of
+// `bs` consecutive weights of a row as fp32 (bs == k: one scale per row, what the kernels of the
+// reference run); normalized = fp32(w) / absmax with an fp32 division (test.py:41, fp16 / fp32
+// promotes to fp32); index = argmin_j |normalized - code[j]| in fp32, first index on ties
+// (torch.argmin, test.py:50-53); nibble packing of test.py:55-65.  A block of zeros gets index 0: the
+// reference divides by zero there, every candidate distance is NaN, and torch.argmin over an all-NaN
+// column returns index 0.
+//
+// One workgroup per block row (8 weight rows), 64 threads per row, 16-byte reads (a row's threads
+// read 1 KB contiguous).  NP > 0: the whole row (k <= 512*NP) is read once into registers, all
+// loads in flight together, so the op streams the weights exactly once; NP == 0: two passes (the
+// second mostly from cache).  Block maxima come from shuffles inside the row's 64 threads.  For a
+// codebook that is sorted with gaps wide enough that fp32 rounding cannot reorder distances, the
+// nearest entry is found by a 4-step binary search over the 15 decision boundaries between
+// neighbouring entries (each the smallest fp32 value the argmin gives to the upper entry, found by
+// bisection with the argmin's own arithmetic once per workgroup) - the argmin's result, since
+// |nv - c| is monotonic in c on either side of nv; any other codebook takes the 16 comparisons.
+// The division by the block maximum is a multiply by its refined reciprocal and one fused correction.  A thread's dword (one row, 8
+// consecutive k) is written through a 2 KB LDS tile so that the stores are 16 bytes per lane and
+// contiguous (the records of 64 block columns), not 4 bytes at a stride of 32.
+// fp32(w) / a, correctly rounded, for the quotients this kernel forms: w an fp16 value, a the
+// largest |fp16| of its block, so |w| <= a and both are normal binary32 numbers (or w is zero).
+// y is the reciprocal of a refined once from v_rcp_f32 (computed once per block); the quotient is one
+// multiply and one fused correction step.  No denormal-mode switches, no scaling: the ranges rule
+// out what the general division sequence guards against.  Equality with the IEEE division is
+// checked for every pair (w, a) of fp16 values with |w| <= a in tests/test_gpu_parity.py.
+__device__ __forceinline__ float refined_rcp(float a)
 {
-    __shared__ float cf[16];
+    const float y = __builtin_amdgcn_rcpf(a);
+    return __builtin_fmaf(__builtin_fmaf(-a, y, 1.0f), y, y);
+}
+
+__device__ __forceinline__ float div_by_block_max(float w, float a, float y)
+{
+    const float q = w * y;
+    return __builtin_fmaf(__builtin_fmaf(-q, a, w), y, q);
+}
+
+// Nearest entry of a sorted codebook: bnd[i] (i = 0..14) is the smallest binary32 value that the
+// argmin assigns to entry i + 1 rather than entry i, so the index is the number of boundaries <= nv:
+// a 4-step binary search, as a tree of selects over the 15 values (uniform, held in registers).
+__device__ __forceinline__ uint32_t nearest_sorted(float nv, const float (&b)[15])
+{
+    const bool b3 = nv >= b[7];
+    const float t2 = b3 ? b[11] : b[3];
+    const float u3 = b3 ? b[13] : b[5], v3 = b3 ? b[9] : b[1];
+    const float p4 = b3 ? b[14] : b[6], q4 = b3 ? b[12] : b[4], r4 = b3 ? b[10] : b[2], s4 = b3 ? b[8] : b[0];
+    const bool b2 = nv >= t2;
+    const float t3 = b2 ? u3 : v3;
+    const float x4 = b2 ? p4 : r4, y4 = b2 ? q4 : s4;
+    const bool b1 = nv >= t3;
+    const float t4 = b1 ? x4 : y4;
+    const bool b0 = nv >= t4;
+    return (b3 ? 8u : 0u) + (b2 ? 4u : 0u) + (b1 ? 2u : 0u) + (b0 ? 1u : 0u);  // a NaN nv ends at 0 like the argmin
+}
+
+__device__ __forceinline__ uint32_t nearest_any(float nv, const float (&c)[16])
+{
+    float bd = fabsf(__fsub_rn(nv, c[0]));
+    uint32_t best = 0;
+#pragma unroll
+    for (int i = 1; i < 16; ++i) {
+        const float dd = fabsf(__fsub_rn(nv, c[i]));
+        if (dd < bd) {
+            bd = dd;
+            best = i;
+        }
+    }
+    return best;
+}
+
+// Smallest binary32 v in [lo, hi] for which the argmin prefers hi: |v - hi| < |v - lo| in fp32
+// arithmetic (ties keep the lower index).  The predicate is monotonic in v (both rounded differences
+// are), so a bisection over the bit patterns finds it; lo < hi, and it holds at v = hi.
+__device__ inline float decision_boundary(float lo, float hi)
+{
+    auto key = [](float f) {  // order-preserving map of finite floats to integers
+        const int64_t i = (int64_t)__builtin_bit_cast(int32_t, f);
+        return i < 0 ? -(i & 0x7fffffff) : i;
+    };
+    auto unkey = [](int64_t k) {
+        const uint32_t i = k < 0 ? (uint32_t)(-k) | 0x80000000u : (uint32_t)k;
+        return __builtin_bit_cast(float, i);
+    };
+    int64_t a = key(lo), b = key(hi);  // predicate false at a (distance 0 to lo), true at b
+    while (b - a > 1) {
+        const int64_t mid = a + ((b - a) >> 1);
+        const float v = unkey(mid);
+        if (fabsf(__fsub_rn(v, hi)) < fabsf(__fsub_rn(v, lo))) b = mid;
+        else a = mid;
+    }
+    return unkey(b);
+}
+
+template <int NP>
+__global__ __launch_bounds__(512) void quantize_kernel(const f16 *__restrict__ w, const float *__restrict__ code,
+                                                       uint32_t *__restrict__ q32, float *__restrict__ absmax, int m, int k,
+                                                       int bs)
+{
+    __shared__ float cs[16], bs_[15];
+    __shared__ int fast_s;
+    constexpr int TPR = 64;  // threads per weight row: a row's threads read 1 KB contiguous
+    __shared__ __align__(16) uint32_t tile[2][TPR * 8];  // [buffer][block column of the step (64)][row (8)]
     const int tid = threadIdx.x;
-    if (tid < 16) cf[tid] = code[tid];
+    if (tid < 16) cs[tid] = code[tid];
+    __syncthreads();
+    if (tid == 0) {
+        // sorted, and every gap far above the rounding of a difference (|nv| <= 1, so a difference is
+        // at most 1 + max|c| and its rounding error below 2^-23 of that)
+        float cmax = fmaxf(fabsf(cs[0]), fabsf(cs[15]));
+        const float thr = (1.0f + cmax) * 9.5367431640625e-7f;  // 2^-20
+        int ok = 1;
+        for (int i = 0; i < 15; ++i) ok &= (cs[i + 1] - cs[i] >= thr) ? 1 : 0;
+        fast_s = ok && cmax < 3.0e38f;
+    }
+    __syncthreads();
+    const bool fast = fast_s != 0;
+    if (fast && tid < 15) bs_[tid] = decision_boundary(cs[tid], cs[tid + 1]);
+    __syncthreads();
+    float c[16], bnd[15];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) c[i] = cs[i];
+#pragma unroll
+    for (int i = 0; i < 15; ++i) bnd[i] = fast ? bs_[i] : 0.f;
+
     const int mb = blockIdx.x;
-    const int r8 = tid >> 5, j = tid & 31;
+    const int r8 = tid / TPR, j = tid % TPR;
     const int row = mb * 8 + r8;
     const int kb_total = k >> 3;
+    const int n_steps = (kb_total + TPR - 1) / TPR;  // steps of 64 block columns
     const f16 *src = w + (size_t)row * k;
-    float amax = 0.f;
-    for (int kb = j; kb < kb_total; kb += 32) {
-        const f16x8 v = *reinterpret_cast<const f16x8 *>(src + kb * 8);
+    const bool by_row = bs == k;
+    const int lanes_blk = by_row ? TPR : bs >> 3;  // threads that share a scale (a power of two <= 32)
+    const int nblk = k / bs;
+
+    f16x8 v[NP > 0 ? NP : 1];
+    float row_max = 0.f;
+    if constexpr (NP > 0) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf((float)v[e]));
-    }
-#pragma unroll
-    for (int off = 16; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 32));
-    if (j == 0) absmax[row] = amax;
-    __syncthreads();  // codebook in LDS
-    float c[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) c[i] = cf[i];
-    for (int kb = j; kb < kb_total; kb += 32) {
-        const f16x8 v = *reinterpret_cast<const f16x8 *>(src + kb * 8);
-        uint32_t d = 0;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            uint32_t best = 0;
-            if (amax > 0.f) {
-                const float nv = __fdiv_rn((float)v[e], amax);
-                float bd = fabsf(__fsub_rn(nv, c[0]));
-                best = 0;
-#pragma unroll
-                for (int i = 1; i < 16; ++i) {
-                    const float dd = fabsf(__fsub_rn(nv, c[i]));
-                    if (dd < bd) {
-                        bd = dd;
-                        best = i;
-                    }
-                }
-            }
-            // byte e/2 of the dword; even column = high nibble
-            d |= best << (8 * (e >> 1) + 4 * (1 - (e & 1)));
+        for (int i = 0; i < NP; ++i) {
+            const int kb = i * TPR + j;
+            v[i] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            if (kb < kb_total) v[i] = *reinterpret_cast<const f16x8 *>(src + (size_t)kb * 8);
         }
-        q32[((size_t)mb * kb_total + kb) * 8 + r8] = d;
+    }
+    if (by_row) {
+        if constexpr (NP > 0) {
+#pragma unroll
+            for (int i = 0; i < NP; ++i)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) row_max = fmaxf(row_max, fabsf((float)v[i][e]));
+        } else {
+            for (int kb = j; kb < kb_total; kb += TPR) {
+                const f16x8 t = *reinterpret_cast<const f16x8 *>(src + (size_t)kb * 8);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) row_max = fmaxf(row_max, fabsf((float)t[e]));
+            }
+        }
+#pragma unroll
+        for (int off = TPR / 2; off >= 1; off >>= 1) row_max = fmaxf(row_max, __shfl_xor(row_max, off, TPR));
+        if (j == 0) absmax[row] = row_max;
+    }
+
+    // one step: 64 block columns of the 8 rows -> 2 KB of packed records
+    auto step = [&](int st, f16x8 t) {
+        const int kb = st * TPR + j;
+        float amax = row_max;
+        if (!by_row) {
+            amax = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf((float)t[e]));
+            for (int off = 1; off < lanes_blk; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, TPR));
+            if (kb < kb_total && (j & (lanes_blk - 1)) == 0) absmax[(size_t)row * nblk + (kb * 8) / bs] = amax;
+        }
+        uint32_t d = 0;
+        if (amax > 0.f) {  // (a block of zeros: every index 0)
+            const float y = refined_rcp(amax);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float nv = div_by_block_max((float)t[e], amax, y);
+                const uint32_t best = fast ? nearest_sorted(nv, bnd) : nearest_any(nv, c);
+                d |= best << (8 * (e >> 1) + 4 * (1 - (e & 1)));  // byte e/2 of the dword; even column = high nibble
+            }
+        }
+        uint32_t *tb = tile[st & 1];
+        tb[j * 8 + r8] = d;
+        __syncthreads();  // (the other buffer was read before the previous step's barrier)
+        if (tid < 2 * TPR) {
+            const int kb0 = st * TPR;
+            const int kbw = kb0 + (tid >> 1);  // block column of the 16 bytes this thread writes
+            if (kbw < kb_total)
+                *reinterpret_cast<u32x4 *>(q32 + ((size_t)mb * kb_total + kb0) * 8 + tid * 4) = *reinterpret_cast<const u32x4 *>(tb + tid * 4);
+        }
+    };
+    if constexpr (NP > 0) {
+        // (fully unrolled: an array indexed by a loop counter would live in scratch memory)
+#pragma unroll
+        for (int st = 0; st < NP; ++st)
+            if (st < n_steps) step(st, v[st]);  // (uniform: every thread of the workgroup takes the same steps)
+    } else {
+        for (int st = 0; st < n_steps; ++st) {
+            const int kb = st * TPR + j;
+            f16x8 t = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            if (kb < kb_total) t = *reinterpret_cast<const f16x8 *>(src + (size_t)kb * 8);
+            step(st, t);
+        }
     }
 }
 
-hipError_t launch_quantize(const void *w, const float *code, void *q, float *absmax, int m, int k, hipStream_t stream)
+// Self-test of div_by_block_max: every pair of fp16 values (w, a) with a > 0 finite and |w| <= a,
+// against the IEEE division (zeros of either sign count as equal).  One workgroup per value of a;
+// counts[0] += pairs, counts[1] += mismatches.
+__global__ __launch_bounds__(256) void division_selftest_kernel(unsigned long long *counts)
 {
-    hipLaunchKernelGGL(quantize_kernel, dim3((unsigned)(m / 8)), dim3(256), 0, stream, static_cast<const f16 *>(w), code,
-                       static_cast<uint32_t *>(q), absmax, m, k);
+    const uint16_t abits = (uint16_t)(blockIdx.x + 1);  // 0x0001 .. 0x7bff: every positive finite fp16
+    const float a = (float)__builtin_bit_cast(f16, abits);
+    const float y = refined_rcp(a);
+    unsigned long long n = 0, bad = 0;
+    for (uint32_t wb = threadIdx.x; wb < 65536u; wb += 256u) {
+        const uint16_t mag = (uint16_t)(wb & 0x7fffu);
+        if (mag > abits) continue;  // |w| > a, infinities, NaNs
+        const float w = (float)__builtin_bit_cast(f16, (uint16_t)wb);
+        const float got = div_by_block_max(w, a, y), want = __fdiv_rn(w, a);
+        ++n;
+        // (a zero quotient may come out with the other sign: -0 / a is -0, the correction step gives +0;
+        // every later use of the quotient is a comparison or a difference, where the two are one value)
+        const bool same = __builtin_bit_cast(uint32_t, got) == __builtin_bit_cast(uint32_t, want) || (got == 0.f && want == 0.f);
+        bad += same ? 0u : 1u;
+    }
+    atomicAdd(counts, n);
+    if (bad) atomicAdd(counts + 1, bad);
+}
+
+hipError_t launch_division_selftest(unsigned long long *counts, hipStream_t stream)
+{
+    hipLaunchKernelGGL(division_selftest_kernel, dim3(0x7bff), dim3(256), 0, stream, counts);
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize(const void *w, const float *code, void *q, float *absmax, int m, int k, int bs, hipStream_t stream)
+{
+    const f16 *wp = static_cast<const f16 *>(w);
+    uint32_t *qp = static_cast<uint32_t *>(q);
+    const dim3 grid((unsigned)(m / 8)), block(512);
+    if (k <= 512 * 4) hipLaunchKernelGGL(quantize_kernel<4>, grid, block, 0, stream, wp, code, qp, absmax, m, k, bs);
+    else if (k <= 512 * 8) hipLaunchKernelGGL(quantize_kernel<8>, grid, block, 0, stream, wp, code, qp, absmax, m, k, bs);
+    else if (k <= 512 * 16) hipLaunchKernelGGL(quantize_kernel<16>, grid, block, 0, stream, wp, code, qp, absmax, m, k, bs);
+    else hipLaunchKernelGGL(quantize_kernel<0>, grid, block, 0, stream, wp, code, qp, absmax, m, k, bs);
     return hipGetLastError();
 }
 

@@ -245,7 +245,7 @@ void describe_gemm_launch(const GemmPlan &plan, int cus, char *buf, size_t len)
 
 // ---- narrow-row kernel (gemm_narrow.hpp) ---------------------------------------------------------
 typedef void (*NarrowKernelFn)(const uint8_t *, const void *, const float *, const float *, int, int, int, int, void *, int,
-                               const void *);
+                               const void *, int, int);
 struct NarrowVariant {
     int rows, wk, u, tt;
     NarrowKernelFn fn, fn_perm;  // B fragments loaded per lane (up to 4 tokens) / contiguously and permuted
@@ -310,7 +310,35 @@ hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int
     const size_t lds = (size_t)kLutBytes + (size_t)waves_k * (rows / 16) * token_tiles * 1024;
     const dim3 grid((unsigned)(args.m / rows), (unsigned)((args.n + 16 * token_tiles - 1) / (16 * token_tiles)), 1);
     hipLaunchKernelGGL(fn, grid, dim3(waves_k * 64), lds, stream, args.q, args.x, args.code, args.absmax, args.k, args.n,
-                       args.n_it, args.m, args.out, args.epilogue, args.residual);
+                       args.n_it, args.m, args.out, args.epilogue, args.residual, 0, 1);
+    return hipGetLastError();
+}
+
+// Scale blocks finer than a row: the narrow-row kernel's BLK variant, 16 rows per workgroup, 4 waves
+// along k, ring of 2.  block = 64 << blk_shift weights per scale.
+hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, hipStream_t stream)
+{
+    constexpr int WK = 4, U = 2;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
+    const int perm = args.n > 4;
+    const NarrowKernelFn fn = perm ? gemm_narrow_kernel<1, WK, U, true, 1, true> : gemm_narrow_kernel<1, WK, U, false, 1, true>;
+    static unsigned char done[16][2];
+    {
+        std::lock_guard<std::mutex> lock(g_attr_mutex);
+        if (!done[dev][perm]) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
+            if (e != hipSuccess) return e;
+            done[dev][perm] = 1;
+        }
+    }
+    const size_t lds = (size_t)kLutBytes + (size_t)WK * 1024;
+    const dim3 grid((unsigned)(args.m / 16), (unsigned)((args.n + 15) / 16), 1);
+    const int nblk = args.k >> (6 + blk_shift);
+    hipLaunchKernelGGL(fn, grid, dim3(WK * 64), lds, stream, args.q, args.x, args.code, args.absmax, args.k, args.n,
+                       args.k / kStepK / WK, args.m, args.out, TUNA_EPILOGUE_NONE, nullptr, blk_shift, nblk);
     return hipGetLastError();
 }
 

@@ -21,6 +21,11 @@
 //   * Reduction: the WK waves put their LW accumulator planes in LDS; each thread sums two
 //     adjacent output features of one token in wave order and stores them (fused epilogues of
 //     epilogue.hpp).  Deterministic; no workspace, no counters.
+//   * BLK variants: one scale per block of 64 << blk_shift consecutive weights of a row, absmax
+//     [m, k / block] (the layout the reference's quantizer writes for block_size < k, test.py:15-17).
+//     A wave's double step of 64 k lies inside one block; the scales of a ring slot's block travel
+//     through the ring with its weights and are rounded to fp16 when the slot is consumed - the
+//     decode is fp16(code) * fp16(absmax of the block), the GEMM's rounding with a finer scale.
 // Requires k % (32*WK*U) == 0, m % (16*LW) == 0, dense launches; a workgroup takes 16*TT tokens
 // (TT = token_tiles = 1, 2, 4: every decoded weight fragment feeds TT MFMAs), more tokens are
 // gridDim.y chunks.  Selected by rows_per_wave = 16 or 32 in the config,
@@ -37,10 +42,11 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 // dwords of a kernel's arguments can be preloaded into scalar registers with the wave (built
 // with -amdgpu-kernarg-preload-count=16), which takes the argument fetch - a round trip to
 // memory - off the start of every wave.  A struct passed by value is not preloaded.
-template <int LW, int WK, int U, bool PERM, int TT>
+template <int LW, int WK, int U, bool PERM, int TT, bool BLK = false>
 __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q, const void *a_x, const float *a_code,
                                                               const float *a_absmax, int a_k, int a_n, int a_n_it, int a_m,
-                                                              void *a_out, int a_epilogue, const void *a_residual)
+                                                              void *a_out, int a_epilogue, const void *a_residual,
+                                                              int a_blk_shift, int a_nblk)
 {
     struct {
         const uint8_t *q;
@@ -68,8 +74,10 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
 
     // ---- requests: codebook and scales, then the first ring turn (x fragment, weights) --------
     const float code_lane = a.code[i16];
-    float sc32[LW];
-    if constexpr (LW == 1) {
+    float sc32[LW] = {};
+    if constexpr (BLK) {
+        // (per block: loaded with the ring below)
+    } else if constexpr (LW == 1) {
         sc32[0] = a.absmax[row0 + i16];
     } else if constexpr (LW == 2) {
         const f32x2 s2 = *reinterpret_cast<const f32x2 *>(a.absmax + row0 + 2 * i16);
@@ -105,11 +113,19 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     const unsigned char *xp = reinterpret_cast<const unsigned char *>(a.x) + (size_t)tok0 * a.k * 2 + (size_t)wk * 128;
     uint32_t wq[U][LW];
     u32x4 xq[U][TT];
+    float sq[BLK ? U : 1][LW];  // BLK: the scales of the ring slot's block
+    // BLK: lane's first scale, and the double step of ring slot 0 in the turn being loaded
+    const float *sp = a.absmax + (size_t)(row0 + LW * i16) * (size_t)(BLK ? a_nblk : 1);
+    int dstep = wk;
     static_assert(U % 2 == 0, "whole double steps");
 #define TUNA_NARROW_LOAD(u)                                                                     \
     {                                                                                          \
         const size_t xo_ = (size_t)((u) >> 1) * (WK * 128) + ((u) & 1) * 64;               \
         const size_t qo_ = (size_t)((u) >> 1) * (WK * 256) + ((u) & 1) * 128;              \
+        if constexpr (BLK) {                                                                   \
+            const int blk_ = (dstep + ((u) >> 1) * WK) >> a_blk_shift;                         \
+            _Pragma("unroll") for (int j = 0; j < LW; ++j) sq[u][j] = sp[(size_t)j * a_nblk + blk_]; \
+        }                                                                                      \
         _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) xq[u][tt] = *reinterpret_cast<const u32x4 *>(xp + xo_ + xoff[tt]); \
         if constexpr (LW == 1) {                                                               \
             wq[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(qp + qo_ + lb)); \
@@ -126,6 +142,7 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     for (int u = 0; u < U; ++u) TUNA_NARROW_LOAD(u)
     qp += (size_t)(U / 2) * (WK * 256);
     xp += (size_t)(U / 2) * (WK * 128);
+    dstep += (U / 2) * WK;
 
     // ---- decode table (see gemm_kernel.hpp), built while the loads are in flight ------------
     {
@@ -173,7 +190,12 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
         }                                                                                      \
         _Pragma("unroll") for (int j = 0; j < LW; ++j)                                         \
         {                                                                                      \
-            const f16x8 av_ = decode_dword<TUNA_DECODE_GEMM>(wq[u][j], lut, lane4, sc16[j], 0.f); \
+            f16x2 s_ = sc16[j];                                                                \
+            if constexpr (BLK) {                                                               \
+                const f16 h_ = (f16)sq[u][j];                                                  \
+                s_ = f16x2{h_, h_};                                                            \
+            }                                                                                  \
+            const f16x8 av_ = decode_dword<TUNA_DECODE_GEMM>(wq[u][j], lut, lane4, s_, 0.f);   \
             _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) acc[j][tt] =                     \
                 __builtin_amdgcn_mfma_f32_16x16x32_f16(av_, b_[tt], acc[j][tt], 0, 0, 0);      \
         }                                                                                      \
@@ -187,6 +209,7 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
         }
         qp += (size_t)(U / 2) * (WK * 256);
         xp += (size_t)(U / 2) * (WK * 128);
+        dstep += (U / 2) * WK;
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) TUNA_NARROW_CONSUME(u)

@@ -168,6 +168,7 @@ struct NarrowArgs {
 };
 bool narrow_variant_exists(int rows, int waves_k, int prefetch, int token_tiles);
 hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int prefetch, int token_tiles, hipStream_t stream);
+hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, hipStream_t stream);
 int set_lean_kernels(int enabled);  // returns the previous setting
 unsigned long long lean_launches();
 bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves, int grouped);
@@ -187,9 +188,11 @@ size_t tiled_lds_bytes(int tile_rows, int tile_tokens);
 
 // dequant_kernel.hip
 hipError_t launch_dequant(const uint8_t *q, const float *absmax, const float *code, void *out,
-                          int m, int k, int decode, hipStream_t stream);
-hipError_t launch_quantize(const void *w, const float *code, void *q, float *absmax, int m, int k, hipStream_t stream);
+                          int m, int k, int block_size, int decode, hipStream_t stream);
+hipError_t launch_quantize(const void *w, const float *code, void *q, float *absmax, int m, int k, int block_size,
+                           hipStream_t stream);
 hipError_t launch_copy(const void *src, void *dst, size_t bytes, hipStream_t stream);
+hipError_t launch_division_selftest(unsigned long long *counts, hipStream_t stream);
 hipError_t launch_read(const void *src, void *sink, size_t bytes, int blocks, int variant, hipStream_t stream);
 
 // config_table.cpp

@@ -167,13 +167,18 @@ def matmul_grouped(x, q, s, c, o, m_group: int, n_groups: int, k: int, token_off
     _lib.check(rc)
 
 
-def dequant(q, absmax, codebook, o, m: int, k: int, decode_mode: int = _lib.DECODE_DEQUANT) -> None:
-    """o[m, k] = decode(q, codebook, absmax) as fp16  (extension.cpp:40-49)."""
+def dequant(q, absmax, codebook, o, m: int, k: int, decode_mode: int = _lib.DECODE_DEQUANT, block_size: int = None) -> None:
+    """o[m, k] = decode(q, codebook, absmax) as fp16  (extension.cpp:40-49).  block_size: weights per
+    scale along a row, absmax [m, k/block_size] (the quantizer's layout for block_size < k,
+    test.py:15-17); None = one scale per row."""
     m, k = int(m), int(k)
     if m <= 0 or k <= 0 or m % 8 or k % 8:
         raise ValueError(f"m and k must be positive multiples of 8 (m={m}, k={k})")
+    bs = k if block_size is None else int(block_size)
+    if bs <= 0 or k % bs:
+        raise ValueError(f"block_size={bs} must divide k={k}")
     _require(q, "q", torch.uint8, m * k // 2)
-    _require(absmax, "absmax", torch.float32, m)
+    _require(absmax, "absmax", torch.float32, m * (k // bs))
     _require(codebook, "codebook", torch.float32, 16)
     _require(o, "o", torch.float16, m * k)
     for name, t in (("absmax", absmax), ("codebook", codebook), ("o", o)):
@@ -181,7 +186,10 @@ def dequant(q, absmax, codebook, o, m: int, k: int, decode_mode: int = _lib.DECO
             raise ValueError(f"{name} is on {t.device}, q on {q.device}")
     L = _lib.lib()
     with torch.cuda.device(q.device):
-        if decode_mode == _lib.DECODE_DEQUANT:
+        if bs != k:
+            rc = L.tuna_dequant_blockwise(q.data_ptr(), absmax.data_ptr(), codebook.data_ptr(), o.data_ptr(), m, k, bs,
+                                          int(decode_mode), _stream(q.device))
+        elif decode_mode == _lib.DECODE_DEQUANT:
             rc = L.tuna_dequant(q.data_ptr(), absmax.data_ptr(), codebook.data_ptr(), o.data_ptr(), m, k,
                                 _stream(q.device))
         else:
@@ -190,10 +198,28 @@ def dequant(q, absmax, codebook, o, m: int, k: int, decode_mode: int = _lib.DECO
     _lib.check(rc)
 
 
-def quantize(w, codebook=None):
-    """fp16 weights [m, k] on a HIP device -> (q uint8 [m/8, k/8, 32], absmax fp32 [m], codebook
-    fp32 [16]): the reference harness's quantizer + packer with one scale per row (test.py:7-68)
-    as one kernel (tuna_quantize).  `codebook` defaults to the NF4 constants."""
+def matmul_blockwise(x, q, s, c, o, m: int, n: int, k: int, block_size: int) -> None:
+    """matmul with one scale per block_size consecutive weights of a row: s fp32 [m, k/block_size]
+    (tuna_matmul_blockwise)."""
+    m, n, k, bs = int(m), int(n), int(k), int(block_size)
+    if bs <= 0 or k % bs:
+        raise ValueError(f"block_size={bs} must divide k={k}")
+    _require(x, "x", torch.float16, n * k)
+    _require(q, "q", torch.uint8, m * k // 2)
+    _require(s, "s", torch.float32, m * (k // bs))
+    _require(c, "c", torch.float32, 16)
+    _require(o, "o", torch.float16, n * m)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().tuna_matmul_blockwise(q.data_ptr(), x.data_ptr(), c.data_ptr(), s.data_ptr(), o.data_ptr(), m, n, k, bs,
+                                              _stream(x.device))
+    _lib.check(rc)
+
+
+def quantize(w, codebook=None, block_size: int = None):
+    """fp16 weights [m, k] on a HIP device -> (q uint8 [m/8, k/8, 32], absmax fp32 [m] - or
+    [m, k/block_size] - and codebook fp32 [16]): the reference harness's quantizer + packer
+    (test.py:7-68) as one kernel (tuna_quantize / tuna_quantize_blockwise).  `codebook` defaults to
+    the NF4 constants, block_size to k (one scale per row, what the GEMM of the reference runs)."""
     from .quantize import nf4_codebook
 
     if w.dim() != 2:
@@ -201,14 +227,17 @@ def quantize(w, codebook=None):
     m, k = w.shape
     if m % 8 or k % 8:
         raise ValueError("m and k must be multiples of 8")
+    bs = k if block_size is None else int(block_size)
+    if bs <= 0 or k % bs:
+        raise ValueError(f"block_size={bs} must divide k={k}")
     _require(w, "w", torch.float16, m * k)
     code = nf4_codebook(w.device) if codebook is None else codebook
     _require(code, "codebook", torch.float32, 16)
     q = torch.empty((m // 8, k // 8, 32), dtype=torch.uint8, device=w.device)
-    absmax = torch.empty((m,), dtype=torch.float32, device=w.device)
+    absmax = torch.empty((m,) if block_size is None else (m, k // bs), dtype=torch.float32, device=w.device)
     with torch.cuda.device(w.device):
-        rc = _lib.lib().tuna_quantize(w.data_ptr(), code.data_ptr(), q.data_ptr(), absmax.data_ptr(), int(m), int(k),
-                                      _stream(w.device))
+        rc = _lib.lib().tuna_quantize_blockwise(w.data_ptr(), code.data_ptr(), q.data_ptr(), absmax.data_ptr(), int(m), int(k),
+                                                bs, _stream(w.device))
     _lib.check(rc)
     return q, absmax, code
 
