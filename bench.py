@@ -157,6 +157,16 @@ def read_sweep(ops, torch, dev, nbytes=2 << 30, iters=5):
     return out
 
 
+def copy_yardstick(ops, torch, dev, mib):
+    """The plain copy kernel over `mib` mebibytes: the known-traffic launch the HBM counters are scaled by."""
+    nb = mib << 20
+    src = torch.full((nb,), 7, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    ms = ops.time_copy(src, dst, warmup=2, iters=10)
+    return {"bytes_read": nb, "bytes_written": nb, "us": round(ms * 100.0, 2),
+            "gbs_read_plus_write": round(2 * nb / (ms * 1e-4) / 1e9, 1)}
+
+
 def launch_floor(ops, torch, dev, headline_bytes):
     tiny = torch.zeros(4096, dtype=torch.uint8, device=dev)
     us_empty = ops.time_read(tiny, blocks=192, warmup=100, iters=1000) * 1000.0 / 1000
@@ -285,8 +295,9 @@ def main():
     ap.add_argument("--launch", choices=("both", "stream", "graph"), default="both")
     ap.add_argument("--settle", type=int, default=300,
                     help="untimed launches before the warm-up of the headline (a box that was idle ramps its clocks)")
-    ap.add_argument("--only", choices=("read", "dequant", "quantize"), default=None,
-                    help="profiling runs: launch only the read-kernel sweep / the dequant kernel / the quantizer")
+    ap.add_argument("--only", choices=("read", "dequant", "quantize", "multi"), default=None,
+                    help="profiling runs: launch only the read-kernel sweep / the dequant kernel / the quantizer / "
+                         "the Llama-70B layer set through tuna_matmul_multi (16 layers)")
     ap.add_argument("--copy-yardstick", type=int, default=0, metavar="MIB",
                     help="also launch the plain copy kernel over MIB mebibytes (counter runs: the known-traffic "
                          "launch the HBM counters of the GEMM kernel are scaled by)")
@@ -312,8 +323,13 @@ def main():
             res = {"read_kernel_sweep_gbs": read_sweep(ops, torch, dev)}
         elif args.only == "dequant":
             res = {"dequant": time_dequant_shapes(ops, synth, torch, dev)}
-        else:
+        elif args.only == "quantize":
             res = {"quantize": time_quantize(ops, synth, torch, dev)}
+        else:
+            names = ["llama70b_qkv", "llama70b_attn_out", "llama70b_gate_up", "llama70b_down"]
+            res = {"llama70b_layers_multi": multi_layer_sweep(ops, synth, torch, dev, names, args.tokens, layers=16)}
+        if args.copy_yardstick > 0:
+            res["copy_yardstick"] = copy_yardstick(ops, torch, dev, args.copy_yardstick)
         print(json.dumps(res))
         return
 
@@ -363,13 +379,7 @@ def main():
         line["launch_floor"] = launch_floor(ops, torch, dev, head["packed_bytes"])
 
     if args.copy_yardstick > 0:
-        nb = args.copy_yardstick << 20
-        src = torch.full((nb,), 7, dtype=torch.uint8, device=dev)
-        dst = torch.empty_like(src)
-        ms = ops.time_copy(src, dst, warmup=2, iters=10)
-        line["copy_yardstick"] = {"bytes_read": nb, "bytes_written": nb, "us": round(ms * 100.0, 2),
-                                  "gbs_read_plus_write": round(2 * nb / (ms * 1e-4) / 1e9, 1)}
-        del src, dst
+        line["copy_yardstick"] = copy_yardstick(ops, torch, dev, args.copy_yardstick)
 
     if not args.no_shapes:
         shapes = {}
