@@ -43,9 +43,10 @@ CACHE_BYTES = 256 << 20  # Infinity Cache; the rotation streams at least twice t
 # summaries under profiles/.  Keyed by shape AND by the kernel the profile was taken of: when the table or
 # the dispatcher picks another kernel for the shape, the entry no longer applies and `traffic` is null.
 MEASURED_TRAFFIC = {
-    # profiles/gemm_narrow_kernel_and_gemm_kernel_hbm_traffic_counters.md
-    ("mistral_qkv", "gemm_narrow_kernel<LW=2,WK=8,U=4,PERM=1,TT=1>"): (6702.5, 192.0),
-    ("mixtral_gate_up_8e", "gemm_kernel<RW=1,U=4,TT=1,DEC=1,1024 threads,4 waves/SIMD,MODE=2> split_k=1"): (230494.3, 7168.1),
+    # profiles/gemm_narrow_kernel_mistral_qkv_kernel_trace.md
+    ("mistral_qkv", "gemm_narrow_kernel<LW=2,WK=8,U=4,PERM=1,TT=1>"): (6700.5, 192.0),
+    # profiles/gemm_lean_kernel_llama70b_qkv_kernel_trace_and_counters.md
+    ("llama70b_qkv", "gemm_lean_kernel<WK=4,U=2,1024 threads> split_k=4"): (22857.5, 2886.2),
 }
 
 
