@@ -139,14 +139,16 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
         /* stagger: row tile t walks k starting rot steps in, wrapping around (gemm_kernel.hpp) */ \
         rot = (k_stagger && n_steps > 1) ? (int)(((unsigned)(t) * k_stagger) % (unsigned)n_steps) : 0; \
         lb = ((uint32_t)(row0_ >> 3) + (uint32_t)(i16 >> 1)) * kb_total * 32u + (uint32_t)(i16 & 1) * 16u + (uint32_t)g * 32u; \
+        /* x and the scales first: vector loads return in order, and the tile's first barrier */ \
+        /* waits for the x pieces only - the first ring turn stays in flight across it */        \
+        TUNA_MID_X_LOAD(0, rot << 5)                                                           \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) sc32[j] = a_absmax[row0_ + i16 * 4 + j];  \
         _Pragma("unroll") for (int u = 0; u < U; ++u)                                          \
         {                                                                                      \
             int s_ = wk + (u << wk_log2) + rot;                                                \
             if (s_ >= n_steps) s_ -= n_steps;                                                  \
             wq[u] = load_weights<NT>(reinterpret_cast<const u32x4 *>(a_q + (size_t)s_ * 128 + lb)); \
         }                                                                                      \
-        _Pragma("unroll") for (int j = 0; j < 4; ++j) sc32[j] = a_absmax[row0_ + i16 * 4 + j];  \
-        TUNA_MID_X_LOAD(0, rot << 5)                                                           \
     }
     if (tile < a_row_tiles) TUNA_MID_TILE_FETCH(tile)
 
@@ -218,7 +220,9 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
         // chunk 0 of x into buffer 0 (every wave has left the previous tile's last chunk: the
         // barrier that ends a chunk), then the table and the chunk are published together
         TUNA_MID_X_STORE(xbuf)
-        __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));  // (threads without a piece: see gemm_kernel.hpp)
+        // (threads without a piece to store have not waited for theirs, see gemm_kernel.hpp; the U
+        // weight loads of the ring are younger than every x piece and may stay in flight)
+        __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));
         __syncthreads();
 
         const unsigned char *qrow = a_q + lb;

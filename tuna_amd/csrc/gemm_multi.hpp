@@ -151,14 +151,14 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
     // k-step (tid + b*1024) / 64 of the chunk, token row lane / 4, 8-k group lane % 4 (every quad of
     // lanes reads 64 contiguous bytes of one token row).
     const int x_row = lane >> 2, x_grp = lane & 3;
-#define TUNA_MULTI_X_LOAD(sg, c)                                                                \
+#define TUNA_MULTI_X_LOAD(x_, n_, k_, sb_, nsteps_, c)                                           \
     {                                                                                          \
-        const uint32_t row_off_ = (uint32_t)min(x_row, (sg).n - 1) * ((uint32_t)(sg).k * 2u);  \
+        const uint32_t row_off_ = (uint32_t)min(x_row, (n_) - 1) * ((uint32_t)(k_) * 2u);      \
         _Pragma("unroll") for (int b = 0; b < XB; ++b)                                         \
         {                                                                                      \
             /* steps past the segment's end: clamped to a valid address, never read */         \
-            const int p_ = min((c) * kChunkSteps + ((tid + b * 1024) >> 6), (sg).nsteps - 1);  \
-            xv[b] = *reinterpret_cast<const u32x4 *>((sg).x + row_off_ + (uint32_t)(((sg).sb + p_) * 32 + x_grp * 8) * 2u); \
+            const int p_ = min((c) * kChunkSteps + ((tid + b * 1024) >> 6), (nsteps_) - 1);    \
+            xv[b] = *reinterpret_cast<const u32x4 *>((x_) + row_off_ + (uint32_t)(((sb_) + p_) * 32 + x_grp * 8) * 2u); \
         }                                                                                      \
     }
     // (token rows past n are zeroed, as the other kernels do; they feed output columns that are never stored)
@@ -175,13 +175,15 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
     const float code_lane = a.code[i16];
     Seg cur = seg_at(t_begin);
     uint32_t lb = lane_base(cur);
+    // x and the scales first: vector loads return in order, and the first barrier then waits for the x
+    // pieces only while the first ring turn stays in flight across it
+    TUNA_MULTI_X_LOAD(cur.x, cur.n, cur.k, cur.sb, cur.nsteps, 0)
+    sc32 = *reinterpret_cast<const f32x4 *>(cur.absmax + cur.row0 + wm * 64 + i16 * 4);
     {
         const unsigned char *qp = cur.q + (size_t)(cur.sb + wk) * 128;
 #pragma unroll
         for (int u = 0; u < U; ++u) wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(qp + (size_t)u * wq_stride + lb));
     }
-    sc32 = *reinterpret_cast<const f32x4 *>(cur.absmax + cur.row0 + wm * 64 + i16 * 4);
-    TUNA_MULTI_X_LOAD(cur, 0)
 
     // ---- decode table (see gemm_kernel.hpp), built while the first loads are in flight --------
     {
@@ -272,43 +274,58 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
                                                 : cur.q + (size_t)(cur.sb + wk) * 128 + (size_t)(n_it - U) * wq_stride;
         const uint32_t rlb_last = has_next ? lb_next : lb;
         int it = 0;
+        // the scales of the next segment (without one: this segment's again), needed when this one ends
+        const f32x4 sc_next = *reinterpret_cast<const f32x4 *>(nxt.absmax + nxt.row0 + wm * 64 + i16 * 4);
+        // One ring turn: U of this wave's k-steps consumed and refilled; the refills of the segment's
+        // last turn are the first steps of the next segment.
+#define TUNA_MULTI_TURN(sl)                                                                     \
+    {                                                                                          \
+        if (it + U >= n_it) {                                                                  \
+            rp = rp_last;                                                                      \
+            rlb = rlb_last;                                                                    \
+        }                                                                                      \
+        _Pragma("unroll") for (int u = 0; u < U; ++u)                                          \
+        {                                                                                      \
+            const f16x8 b_ = *reinterpret_cast<const f16x8 *>(xb + (size_t)((sl) + u) * wstep); \
+            _Pragma("unroll") for (int j = 0; j < 4; ++j)                                      \
+            {                                                                                  \
+                const f16x8 av_ = decode_dword<TUNA_DECODE_GEMM>(wq[u][j], lut, lane4, sc16[j], 0.f); \
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av_, b_, acc[j], 0, 0, 0);     \
+            }                                                                                  \
+            wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(rp + (size_t)u * wq_stride + rlb)); \
+            __builtin_amdgcn_sched_barrier(0); /* keep each refill right behind its consume */ \
+        }                                                                                      \
+        rp += (size_t)U * wq_stride;                                                           \
+        it += U;                                                                               \
+    }
         for (int c = 0; c < n_chunks; ++c) {
             const bool more = c + 1 < n_chunks;
             // the chunk behind this one: of this segment, or - in its last chunk - the first one of
-            // the next segment together with that segment's scales (no next segment: this chunk
-            // again, dropped).  One unconditional batch of loads either way.
-            if (more) {
-                TUNA_MULTI_X_LOAD(cur, c + 1)
-            } else {
-                TUNA_MULTI_X_LOAD(nxt, has_next ? 0 : c)
-                sc32 = *reinterpret_cast<const f32x4 *>(nxt.absmax + nxt.row0 + wm * 64 + i16 * 4);
+            // the next segment (no next segment: this chunk again, dropped).  Uniform parameters and
+            // ONE unconditional batch of loads: behind a branch the compiler could not count these
+            // loads into the waits of the ring and would wait for everything in flight instead.
+            {
+                const unsigned char *x_ = more ? cur.x : nxt.x;
+                const int xn_ = more ? cur.n : nxt.n, xk_ = more ? cur.k : nxt.k, xsb_ = more ? cur.sb : nxt.sb;
+                const int xns_ = more ? cur.nsteps : nxt.nsteps, xc_ = more ? c + 1 : (has_next ? 0 : c);
+                TUNA_MULTI_X_LOAD(x_, xn_, xk_, xsb_, xns_, xc_)
             }
             const unsigned char *xb = xbuf + xsel * kXBuf + xb_lane;
             const int its = min(chunk_its, n_it - it);
-            for (int sl = 0; sl < its; sl += U) {
-                if (it + U >= n_it) {
-                    rp = rp_last;
-                    rlb = rlb_last;
-                }
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const f16x8 b_ = *reinterpret_cast<const f16x8 *>(xb + (size_t)(sl + u) * wstep);
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const f16x8 av_ = decode_dword<TUNA_DECODE_GEMM>(wq[u][j], lut, lane4, sc16[j], 0.f);
-                        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av_, b_, acc[j], 0, 0, 0);
-                    }
-                    wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(rp + (size_t)u * wq_stride + rlb));
-                    __builtin_amdgcn_sched_barrier(0);  // keep each refill right behind its consume
-                }
-                rp += (size_t)U * wq_stride;
-                it += U;
-            }
-            // the other buffer was last read in the previous chunk, which ended with a barrier
+            // (the first ring turn of a chunk is a copy of its own: there the x pieces just requested
+            // are in flight behind the ring, and only straight-line code lets the compiler count them
+            // into its waits)
+            TUNA_MULTI_TURN(0)
+            for (int sl = U; sl < its; sl += U) TUNA_MULTI_TURN(sl)
+            // the other buffer was last read in the previous chunk, which ended with a barrier;
+            // exactly the last ring turn's U refills are younger than the x pieces
+            __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));
             TUNA_MULTI_X_STORE(more ? cur.n : nxt.n, xbuf + (xsel ^ 1u) * kXBuf)
             __syncthreads();
             xsel ^= 1u;
         }
+#undef TUNA_MULTI_TURN
+        sc32 = sc_next;
 
         // ---- reduction over the waves along k (layouts of gemm_kernel.hpp), two planes at a time ----
         // (the area was last read before a chunk barrier of this segment; the next segment's first
