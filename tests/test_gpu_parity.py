@@ -871,6 +871,52 @@ def test_mid_token_kernel_equals_general_kernel_bit_for_bit(ci):
     assert rel_err(outs[True][0].cpu().numpy().astype(np.float64), ref) <= REL_TOL   # max relative error 1e-2
 
 
+LDS_PATH_CASES = [
+    # m, n, k, waves_m, waves_k, prefetch, x_chunk, k_stagger
+    (1024, 16, 4096, 16, 1, 4, 1024, 2),      # all waves along the rows (chunks of 512 k beside the rings)
+    (2048, 16, 8192, 4, 4, 2, 1024, 2),       # waves along k: sums through LDS
+    (512, 5, 2048, 2, 8, 2, 512, 0),
+    (256 * 300, 16, 1024, 4, 4, 2, 1024, 3),  # more row tiles than compute units: workgroups that walk two tiles
+    (1024 * 260, 3, 512, 16, 1, 2, 512, 1),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("ci", range(len(LDS_PATH_CASES)))
+def test_weights_staged_through_lds_equal_the_register_ring_bit_for_bit(ci):
+    """The diagnostic switch that stages the packed weights (and x, and the scales) through LDS with
+    global -> LDS loads runs the same arithmetic in the same order: equal bits, and the launch
+    description says which path ran."""
+    import torch
+
+    from tuna_amd import ops
+
+    m, n, k, wm, wk, pf, xc, st = LDS_PATH_CASES[ci]
+    c = cfg(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=1, prefetch=pf, x_chunk=xc, k_stagger=st)
+    print(f"lds path case#{ci} {m}x{n}x{k} {c.to_dict()}", flush=True)
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=700 + ci)
+    dq, dx, dc, da = to_dev(q, x, code, absmax)
+    outs = {}
+    prev = ops.set_weight_path(False)
+    try:
+        for staged in (False, True):
+            ops.set_weight_path(staged)
+            d = ops.describe_launch(m, n, k, c)
+            assert d.startswith("gemm_mid_kernel") and (("through LDS" in d) == staged), d
+            o = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+            ops.matmul(dx, dq, da, dc, o, m, n, k, config=c)
+            ops.matmul(dx, dq, da, dc, o, m, n, k, config=c)   # twice: the second launch finds LDS-independent state
+            torch.cuda.synchronize()
+            outs[staged] = o
+    finally:
+        ops.set_weight_path(prev)
+    assert not torch.isnan(outs[True].float()).any()
+    assert torch.equal(outs[True].view(torch.int16), outs[False].view(torch.int16))
+    rows = np.random.default_rng(ci).choice(m, size=min(m, 256), replace=False).astype(np.int32)
+    ref = O.gemm_f64(q, x, code, absmax, m, n, k, mode=O.D1, rows=rows)
+    assert rel_err(outs[True].cpu().numpy().astype(np.float64)[:, rows], ref) <= REL_TOL   # max relative error 1e-2
+
+
 # ----------------------------------------------------------------------------- narrow-row kernel
 NARROW_CASES = [
     # m, n, k, rows_per_wave, waves_k, prefetch

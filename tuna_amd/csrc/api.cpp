@@ -1533,6 +1533,7 @@ TUNA_EXPORT int tuna_set_multi_min_batch(int count)
 TUNA_EXPORT unsigned long long tuna_multi_launches(void) { return g_multi_launches.load(); }
 
 TUNA_EXPORT int tuna_set_lean_kernels(int enabled) { return tuna::set_lean_kernels(enabled ? 1 : 0); }
+TUNA_EXPORT int tuna_set_weight_path(int through_lds) { return tuna::set_weight_path(through_lds ? 1 : 0); }
 
 TUNA_EXPORT unsigned long long tuna_lean_launches(void) { return tuna::lean_launches(); }
 

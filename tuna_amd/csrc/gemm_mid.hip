@@ -1,4 +1,5 @@
 // Instantiations and launcher of the 17..128-token streaming kernel (gemm_mid.hpp).
+#include <atomic>
 #include <cstdio>
 #include <mutex>
 
@@ -12,28 +13,45 @@ struct MidVariant {
     int u, tt, xb, maxt;
     MidKernelFn fn;
     MidKernelFn fn_shared;  // twin without the nontemporal hint on the weight loads (token chunks side by side), or null
+    MidKernelFn fn_lds;     // twin with the packed weights staged through LDS (diagnostic switch), or null
 };
-#define M5(U, TT, XB) {U, TT, XB, 512, gemm_mid_kernel<U, TT, XB, 512, 2>, nullptr}
-#define M5S(U, TT, XB) {U, TT, XB, 512, gemm_mid_kernel<U, TT, XB, 512, 2>, gemm_mid_kernel<U, TT, XB, 512, 2, false>}
-#define M10(U, TT, XB) {U, TT, XB, 1024, gemm_mid_kernel<U, TT, XB, 1024, 4>, nullptr}
+#define M5(U, TT, XB) {U, TT, XB, 512, gemm_mid_kernel<U, TT, XB, 512, 2>, nullptr, nullptr}
+#define M5S(U, TT, XB) {U, TT, XB, 512, gemm_mid_kernel<U, TT, XB, 512, 2>, gemm_mid_kernel<U, TT, XB, 512, 2, false>, nullptr}
+#define M10(U, TT, XB) {U, TT, XB, 1024, gemm_mid_kernel<U, TT, XB, 1024, 4>, nullptr, nullptr}
+#define M10L(U, TT, XB) {U, TT, XB, 1024, gemm_mid_kernel<U, TT, XB, 1024, 4>, nullptr, gemm_mid_kernel<U, TT, XB, 1024, 4, true, true>}
 static const MidVariant kMid[] = {
     M5(2, 2, 4), M5(4, 2, 4), M5(8, 2, 4), M5(2, 2, 8), M5(4, 2, 8), M5(8, 2, 8),
     M5(2, 4, 4), M5(4, 4, 4), M5(8, 4, 4), M5(2, 4, 8), M5(4, 4, 8), M5(8, 4, 8),
     M5S(2, 8, 4), M5S(2, 8, 8),  // (deeper rings with eight token tiles spill inside the loop)
     M10(2, 2, 4), M10(4, 2, 4),
     // one token tile: the large shapes at up to 16 tokens (small launches take gemm_lean.hpp first)
-    M5(2, 1, 4), M5(4, 1, 4), M5(8, 1, 4), M5(2, 1, 8), M5(4, 1, 8), M5(8, 1, 8), M10(2, 1, 4), M10(4, 1, 4), M10(8, 1, 4),
+    M5(2, 1, 4), M5(4, 1, 4), M5(8, 1, 4), M5(2, 1, 8), M5(4, 1, 8), M5(8, 1, 8), M10L(2, 1, 4), M10L(4, 1, 4), M10(8, 1, 4),
 };
 #undef M5
 #undef M5S
 #undef M10
+#undef M10L
 static constexpr int kNumMid = sizeof(kMid) / sizeof(kMid[0]);
 
-// x chunk the kernel uses: the config's, capped so that two buffers fit beside the decode table.
+// Diagnostic switch: 1 = launches that have an LDS-staged twin run it (tuna_set_weight_path).
+static std::atomic<int> g_weight_path{0};
+int set_weight_path(int path)
+{
+    return path < 0 ? g_weight_path.load(std::memory_order_relaxed) : g_weight_path.exchange(path ? 1 : 0, std::memory_order_relaxed);
+}
+static bool lds_path(const GemmPlan &plan)
+{
+    return g_weight_path.load(std::memory_order_relaxed) != 0 && plan.token_tiles == 1 && plan.threads == 1024 &&
+           (plan.prefetch == 2 || plan.prefetch == 4);
+}
+
+// x chunk the kernel uses: the config's, capped so that two buffers fit beside the decode table
+// (and, for the LDS-staged twin, the waves' weight rings).
 static int mid_x_chunk(const GemmPlan &plan)
 {
     int xc = plan.args.chunk_steps * kStepK;
-    const int cap = (kLdsLimit - kLutBytes) / (2 * plan.token_tiles * 32);  // k per buffer
+    const int ring = lds_path(plan) ? (plan.threads / 64) * plan.prefetch * 1024 : 0;
+    const int cap = (kLdsLimit - kLutBytes - ring) / (2 * plan.token_tiles * 32);  // k per buffer
     while (xc > cap) xc >>= 1;
     return xc;
 }
@@ -74,7 +92,8 @@ bool mid_describe(const GemmPlan &plan, char *buf, size_t len)
     int xc;
     const MidVariant *v = mid_variant(plan, &xc);
     if (!v) return false;
-    snprintf(buf, len, "gemm_mid_kernel<U=%d,TT=%d,XB=%d,%d threads> x_chunk=%d", v->u, v->tt, v->xb, v->maxt, xc);
+    snprintf(buf, len, "gemm_mid_kernel<U=%d,TT=%d,XB=%d,%d threads%s> x_chunk=%d", v->u, v->tt, v->xb, v->maxt,
+             (lds_path(plan) && v->fn_lds) ? ",weights through LDS" : "", xc);
     return true;
 }
 
@@ -95,6 +114,9 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
             if (e == hipSuccess && v->fn_shared)
                 e = hipFuncSetAttribute(reinterpret_cast<const void *>(v->fn_shared), hipFuncAttributeMaxDynamicSharedMemorySize,
                                         kLdsLimit);
+            if (e == hipSuccess && v->fn_lds)
+                e = hipFuncSetAttribute(reinterpret_cast<const void *>(v->fn_lds), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        kLdsLimit);
             if (e != hipSuccess) return e;
             g_mid_attr_done[dev][vi] = 1;
         }
@@ -104,7 +126,11 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
     while ((1 << xc_log2) < xc) ++xc_log2;
     const size_t x_lds = 2 * (size_t)plan.token_tiles * 32 * (size_t)xc;   // two buffers of one chunk
     const size_t red_lds = 2 * (size_t)(plan.threads / 64) * 1024;         // two buffers of one plane per wave
-    const size_t lds = (size_t)kLutBytes + (x_lds > red_lds ? x_lds : red_lds);
+    const bool staged = lds_path(plan) && v->fn_lds;
+    const size_t lds = (size_t)kLutBytes + (staged ? x_lds + (size_t)(plan.threads / 64) * plan.prefetch * 1024
+                                                   : (x_lds > red_lds ? x_lds : red_lds));
+    // (the twin counts on one or two x pieces per wave and chunk: chunks of 512 or 1024 k)
+    if (staged && (x_lds < red_lds || lds > (size_t)kLdsLimit || (xc != 512 && xc != 1024))) return hipErrorInvalidConfiguration;
     dim3 grid = plan.grid;
     grid.x = (unsigned)(a.row_tiles < cus ? a.row_tiles : cus);  // one workgroup per CU (LDS), walking row tiles
     // Several token chunks that do not all fit the device at once: rather than one round of row
@@ -131,7 +157,7 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
     const int packed = a.waves_m | a.epilogue << 5 | xc_log2 << 8 | a.wk_log2 << 13 | a.k_stagger << 16;
     // weights that sibling workgroups re-read stay in the caches longer without the nontemporal hint
     // (Mixtral gate+up, 1024 tokens: 1745 -> 1687 us)
-    const MidKernelFn fn = (chunks && v->fn_shared) ? v->fn_shared : v->fn;
+    const MidKernelFn fn = staged ? v->fn_lds : (chunks && v->fn_shared) ? v->fn_shared : v->fn;
     hipLaunchKernelGGL(fn, grid, dim3(plan.threads), lds, stream, a.q, a.x, a.code, a.absmax, a.k, a.n, a.m, packed, a.out,
                        a.residual, a.row_tiles, n_wg, chunks);
     return hipGetLastError();

@@ -30,9 +30,45 @@ __device__ __forceinline__ u32x4 load_weights(const u32x4 *p)
     else return *p;
 }
 
+// Packed weights through LDS instead of registers (LDSW variants): one 16-byte global -> LDS load per
+// lane (global_load_lds_dwordx4: the data goes from the memory pipeline into LDS without passing a
+// register; lane l's bytes land at the slot's base + 16*l) and, when the slot is consumed, one
+// ds_read_b128 of the same bytes.  A pure transit buffer: the same global access pattern, ring depth
+// and waits as the register ring, which is what makes the two comparable.
+template <bool NT>
+__device__ __forceinline__ void load_weights_to_lds(const unsigned char *p, unsigned char *slot)
+{
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(p),
+                                     (__attribute__((address_space(3))) void *)(slot), 16, 0, NT ? 2 : 0);
+}
+
+// With global -> LDS loads in flight the compiler makes every LDS store and every workgroup fence
+// wait for ALL of them (they are LDS writes it cannot tell apart from the x staging area), which
+// would empty the ring at every chunk switch; and it waits for everything, too, before it uses a
+// register loaded from global memory while such loads are in flight.  The LDSW variants therefore
+// bring x into LDS the same way (lane (token, 8-k group) fetches its own B-fragment piece of a
+// k-step, so a wave instruction fills one k-step of the chunk buffer), build the decode table with
+// stores the compiler does not look into, and synchronise with a bare barrier behind an explicit
+// wait for the wave's own LDS operations; the waits for the loads are written out where a slot or
+// a chunk is used.
+__device__ __forceinline__ void lds_store16_opaque(unsigned char *p, u32x4 v)
+{
+    const uint32_t a = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)p;
+    asm volatile("ds_write_b128 %0, %1" ::"v"(a), "v"(v) : "memory");
+}
+__device__ __forceinline__ void barrier_lds_only()
+{
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's LDS stores have been performed
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" ::: "memory");
+}
+
 // NT: weight loads carry the nontemporal hint (each byte is used once per launch).  Launches whose
 // token chunks share the weights through the caches (a_chunks != 0) run the twin without it.
-template <int U, int TT, int XB, int MAXT, int MINW, bool NT = true>
+template <int U, int TT, int XB, int MAXT, int MINW, bool NT = true, bool LDSW = false>
 __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q, const void *a_x, const float *a_code,
                                                               const float *a_absmax, int a_k, int a_n, int a_m, int a_packed,
                                                               void *a_out, const void *a_residual, int a_row_tiles,
@@ -122,10 +158,43 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
 #define TUNA_MID_X_STORE(buf)                                                                   \
     {                                                                                          \
         _Pragma("unroll") for (int b = 0; b < XB; ++b) if (x_inchunk >> b & 1u)                \
-            *reinterpret_cast<u32x4 *>((buf) + x_loff[b]) = (x_real >> b & 1u) ? xst.v[b] : u32x4{0u, 0u, 0u, 0u}; \
+        {                                                                                      \
+            const u32x4 v_ = (x_real >> b & 1u) ? xst.v[b] : u32x4{0u, 0u, 0u, 0u};            \
+            *reinterpret_cast<u32x4 *>((buf) + x_loff[b]) = v_;                                \
+        }                                                                                      \
     }
 
-    const float code_lane = a_code[i16];
+    // LDSW: chunk `kbase` of x straight into `buf`: k-step wave + b*(waves of the workgroup) of the
+    // chunk, b < xdma_n (a uniform count of 1 or 2: the explicit waits below count on it); token rows
+    // past n are clamped (their output columns are never stored)
+    const int xdma_n = LDSW ? max(1, (xc >> 5) / (nthreads >> 6)) : 0;
+    const uint32_t xdma_lane = LDSW ? ((uint32_t)min(i16, a_n - 1 - tok0) * (uint32_t)a_k + (uint32_t)g * 8u) * 2u : 0u;
+#define TUNA_MID_X_DMA(buf, kbase, rot_steps)                                                   \
+    {                                                                                          \
+        for (int b = 0; b < xdma_n; ++b) {                                                     \
+            const int ks_ = min(wave + b * (nthreads >> 6), (xc >> 5) - 1);                    \
+            int s_ = ((kbase) >> 5) + ks_ + (rot_steps);                                       \
+            if (s_ >= n_steps) s_ -= n_steps;                                                  \
+            load_weights_to_lds<false>(x_tile + (size_t)s_ * 64 + xdma_lane, (buf) + ks_ * 1024); \
+        }                                                                                      \
+    }
+
+    float code_lane;
+    if constexpr (LDSW) {
+        // through the scalar cache: a vector load here would be one more thing in flight that the
+        // compiler waits for by waiting for everything
+        // (uniform, read before the kernel's first store; the selection starts from a constant: a
+        // select between two loads would be turned back into one vector load)
+        const float *__restrict__ code_ptr = a_code;
+        float cs[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) cs[j] = code_ptr[j];
+        code_lane = 0.f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) code_lane = i16 == j ? cs[j] : code_lane;
+    } else {
+        code_lane = a_code[i16];
+    }
     // weights of this wave's rows: lane (i16, g) loads 16 bytes = dword j of row 4*i16 + j's 8 k
     // (block row i16/2, second half of the block for odd i16), block column 4*step + g
     uint32_t lb = 0;
@@ -141,14 +210,36 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
         lb = ((uint32_t)(row0_ >> 3) + (uint32_t)(i16 >> 1)) * kb_total * 32u + (uint32_t)(i16 & 1) * 16u + (uint32_t)g * 32u; \
         /* x and the scales first: vector loads return in order, and the tile's first barrier */ \
         /* waits for the x pieces only - the first ring turn stays in flight across it */        \
-        TUNA_MID_X_LOAD(0, rot << 5)                                                           \
-        _Pragma("unroll") for (int j = 0; j < 4; ++j) sc32[j] = a_absmax[row0_ + i16 * 4 + j];  \
+        if constexpr (!LDSW) TUNA_MID_X_LOAD(0, rot << 5)                                      \
+        if constexpr (!LDSW) {                                                                 \
+            _Pragma("unroll") for (int j = 0; j < 4; ++j) sc32[j] = a_absmax[row0_ + i16 * 4 + j]; \
+        }                                                                                      \
         _Pragma("unroll") for (int u = 0; u < U; ++u)                                          \
         {                                                                                      \
             int s_ = wk + (u << wk_log2) + rot;                                                \
             if (s_ >= n_steps) s_ -= n_steps;                                                  \
-            wq[u] = load_weights<NT>(reinterpret_cast<const u32x4 *>(a_q + (size_t)s_ * 128 + lb)); \
+            if constexpr (LDSW) load_weights_to_lds<NT>(a_q + (size_t)s_ * 128 + lb, wring + u * 1024); \
+            else wq[u] = load_weights<NT>(reinterpret_cast<const u32x4 *>(a_q + (size_t)s_ * 128 + lb)); \
         }                                                                                      \
+    }
+    // LDSW: this wave's ring of U slots of 1 KB, behind the two x buffers
+    unsigned char *wring = xbuf + 2 * ((uint32_t)(TT * 32) << xc_log2) + wave * (U * 1024);
+    bool first_tile = true;
+    // LDSW: chunk 0 of tile t into buffer 0 and the lane's four scales into this wave's KB of buffer 1
+    // (free until chunk 1 is requested; read back at the top of the tile)
+#define TUNA_MID_TOP_DMA(t, rot_steps)                                                          \
+    {                                                                                          \
+        TUNA_MID_X_DMA(xbuf, 0, rot_steps)                                                     \
+        load_weights_to_lds<false>(reinterpret_cast<const unsigned char *>(a_absmax + (t) * (waves_m * 64) + wm * 64 + i16 * 4), \
+                                   xbuf + ((uint32_t)(TT * 32) << xc_log2) + wave * 1024);     \
+    }
+    if constexpr (LDSW) {
+        // the first tile's ahead of its ring (later tiles: at the top of the tile, when the
+        // reduction has left the x area)
+        if (tile < a_row_tiles) {
+            const int rot0_ = (k_stagger && n_steps > 1) ? (int)(((unsigned)tile * k_stagger) % (unsigned)n_steps) : 0;
+            TUNA_MID_TOP_DMA(tile, rot0_)
+        }
     }
     if (tile < a_row_tiles) TUNA_MID_TILE_FETCH(tile)
 
@@ -167,7 +258,10 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
 #pragma unroll
             for (int b = 0; b < 4; ++b) {
                 const int p = p0 + b * nthreads;
-                if (p < kLutBytes / 16) reinterpret_cast<u32x4 *>(lut)[p] = u32x4{v[b], v[b], v[b], v[b]};
+                if (p < kLutBytes / 16) {
+                    if constexpr (LDSW) lds_store16_opaque(lut + (size_t)p * 16, u32x4{v[b], v[b], v[b], v[b]});
+                    else reinterpret_cast<u32x4 *>(lut)[p] = u32x4{v[b], v[b], v[b], v[b]};
+                }
             }
         }
     }
@@ -182,10 +276,18 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     // One ring turn: U of this wave's k-steps, each consumed (B fragments from LDS, 4 fragments
     // decoded, 4*TT MFMAs) and refilled with the wave's step U iterations on (the last turn
     // re-reads the tile's last step: in bounds, never consumed).
-#define TUNA_MID_GROUP(sl)                                                                      \
+#define TUNA_MID_GROUP(sl, first)                                                               \
     {                                                                                          \
         _Pragma("unroll") for (int u = 0; u < U; ++u)                                          \
         {                                                                                      \
+            if constexpr (LDSW) {                                                              \
+                /* the slot's load has landed: U - 1 younger ring loads, in a chunk's first turn */ \
+                /* also the XB x pieces just requested, may stay in flight */                  \
+                if (!(first)) __builtin_amdgcn_s_waitcnt(wait_vmcnt(U - 1));                   \
+                else if (xdma_n == 2) __builtin_amdgcn_s_waitcnt(wait_vmcnt(U + 1));           \
+                else __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));                                \
+                wq[u] = *reinterpret_cast<const u32x4 *>(wring + u * 1024 + lane * 16);        \
+            }                                                                                  \
             f16x8 b_[TT];                                                                      \
             _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) b_[tt] =                         \
                 *reinterpret_cast<const f16x8 *>(xb + (size_t)((sl) + u) * wstep + tt * 256);  \
@@ -197,13 +299,29 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
             }                                                                                  \
             int s_ = min(wk + ((it + u + U) << wk_log2), n_steps - 1) + cur_rot;               \
             if (s_ >= n_steps) s_ -= n_steps;                                                  \
-            wq[u] = load_weights<NT>(reinterpret_cast<const u32x4 *>(qrow + (size_t)s_ * 128)); \
+            if constexpr (LDSW) {                                                              \
+                /* behind the MFMAs that used the slot's bytes: the slot is free */            \
+                __builtin_amdgcn_sched_barrier(0);                                             \
+                load_weights_to_lds<NT>(qrow + (size_t)s_ * 128, wring + u * 1024);            \
+            } else {                                                                           \
+                wq[u] = load_weights<NT>(reinterpret_cast<const u32x4 *>(qrow + (size_t)s_ * 128)); \
+            }                                                                                  \
             __builtin_amdgcn_sched_barrier(0); /* keep each refill right behind its consume */ \
         }                                                                                      \
         it += U;                                                                               \
     }
 
     while (tile < a_row_tiles) {
+        if constexpr (LDSW) {
+            if (first_tile) {
+                __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));  // chunk 0 and the scales are older than the ring's U loads
+            } else {
+                TUNA_MID_TOP_DMA(tile, rot)
+                __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));
+            }
+            first_tile = false;
+            sc32 = *reinterpret_cast<const f32x4 *>(xbuf + ((uint32_t)(TT * 32) << xc_log2) + wave * 1024 + lane * 16);
+        }
         f16x2 sc16[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -219,11 +337,15 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
 
         // chunk 0 of x into buffer 0 (every wave has left the previous tile's last chunk: the
         // barrier that ends a chunk), then the table and the chunk are published together
-        TUNA_MID_X_STORE(xbuf)
-        // (threads without a piece to store have not waited for theirs, see gemm_kernel.hpp; the U
-        // weight loads of the ring are younger than every x piece and may stay in flight)
-        __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));
-        __syncthreads();
+        if constexpr (LDSW) {
+            barrier_lds_only();  // (every wave has waited for its pieces of chunk 0 and read its scales)
+        } else {
+            TUNA_MID_X_STORE(xbuf)
+            // (threads without a piece to store have not waited for theirs, see gemm_kernel.hpp; the U
+            // weight loads of the ring are younger than every x piece and may stay in flight)
+            __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));
+            __syncthreads();
+        }
 
         const unsigned char *qrow = a_q + lb;
         const int cur_rot = rot;
@@ -232,19 +354,29 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
             const bool has_next = c + 1 < n_chunks;
             // (unconditional - the last chunk requests itself again and drops it: behind a branch
             // the compiler could not count these loads into the waits of the first ring turn)
-            TUNA_MID_X_LOAD(min(c + 1, n_chunks - 1) << xc_log2, cur_rot << 5)
+            if constexpr (LDSW) {
+                // (the other buffer was last read in chunk c - 1, which ended with a barrier)
+                TUNA_MID_X_DMA(xbuf + ((c + 1) & 1) * xbuf_bytes, min(c + 1, n_chunks - 1) << xc_log2, cur_rot)
+            } else {
+                TUNA_MID_X_LOAD(min(c + 1, n_chunks - 1) << xc_log2, cur_rot << 5)
+            }
             const unsigned char *xb = xbuf + (c & 1) * xbuf_bytes + xb_lane;
             // (the first ring turn of a chunk is a copy of its own: there the x pieces just
             // requested are in flight behind the ring, and only straight-line code lets the
             // compiler count them into its waits instead of waiting them out)
-            TUNA_MID_GROUP(0)
-            for (int sl = U; sl < chunk_its; sl += U) TUNA_MID_GROUP(sl)
-            if (has_next) {
-                // the other buffer was last read in chunk c - 1, which ended with a barrier
-                __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));  // exactly the last ring turn's refills are younger
-                TUNA_MID_X_STORE(xbuf + ((c + 1) & 1) * xbuf_bytes)
+            TUNA_MID_GROUP(0, true)
+            for (int sl = U; sl < chunk_its; sl += U) TUNA_MID_GROUP(sl, false)
+            if constexpr (LDSW) {
+                __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));  // this wave's pieces of the next chunk have landed
+                barrier_lds_only();
+            } else {
+                if (has_next) {
+                    // the other buffer was last read in chunk c - 1, which ended with a barrier
+                    __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));  // exactly the last ring turn's refills are younger
+                    TUNA_MID_X_STORE(xbuf + ((c + 1) & 1) * xbuf_bytes)
+                }
+                __syncthreads();
             }
-            __syncthreads();
         }
 
         // ---- next tile's loads, then this tile's store ------------------------------------------
@@ -313,6 +445,8 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
 #undef TUNA_MID_GROUP
 #undef TUNA_MID_X_LOAD
 #undef TUNA_MID_X_STORE
+#undef TUNA_MID_X_DMA
+#undef TUNA_MID_TOP_DMA
 #undef TUNA_MID_TILE_FETCH
 }
 

@@ -170,6 +170,7 @@ bool narrow_variant_exists(int rows, int waves_k, int prefetch, int token_tiles)
 hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int prefetch, int token_tiles, hipStream_t stream);
 hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, hipStream_t stream);
 int set_lean_kernels(int enabled);  // returns the previous setting
+int set_weight_path(int path);      // gemm_mid.hip; negative: query
 unsigned long long lean_launches();
 bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves, int grouped);
 

@@ -414,6 +414,12 @@ def set_lean_kernels(enabled: bool) -> bool:
     return bool(_lib.lib().tuna_set_lean_kernels(int(bool(enabled))))
 
 
+def set_weight_path(through_lds: bool) -> bool:
+    """Diagnostic switch (tuna_set_weight_path): unsplit 16-wave launches of up to 16 tokens stage the
+    packed weights through LDS instead of registers.  Bit-identical results.  Returns the previous setting."""
+    return bool(_lib.lib().tuna_set_weight_path(int(bool(through_lds))))
+
+
 def lean_launches() -> int:
     """Diagnostic (tuna_lean_launches): GEMM launches of this process that took the stripped-down kernel."""
     return int(_lib.lib().tuna_lean_launches())
