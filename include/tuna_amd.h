@@ -82,7 +82,10 @@ typedef struct tuna_gemm_config {
     int32_t lds_tile_rows; /* 0: streaming kernel (all fields above).  64, 128 or 256: the
                               many-token kernel, which decodes a tile of this many weight rows
                               once into LDS for token_tiles*16 (64, 128 or 256) tokens; only
-                              token_tiles and split_k (>= 1) are read besides                */
+                              token_tiles, split_k (>= 1) and rows_per_wave are read besides:
+                              rows_per_wave == 32 multiplies with 32 x 32 x 16 MFMA tiles
+                              (tiles of at least 32 tokens), any other value with 16 x 16 x 32
+                              (the reference's counterpart: its MMA shapes, kernel.cu:411-465) */
 } tuna_gemm_config;
 
 int tuna_version(void);

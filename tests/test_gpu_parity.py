@@ -550,6 +550,30 @@ def test_many_token_kernel_matches_oracle(tile, m, n, k, split):
     assert np.array_equal(got, again)
 
 
+@pytest.mark.parametrize("tile", [t for t in TILED if t != (64, 8)])
+@pytest.mark.parametrize("m,n,k,split", [(512, 256, 512, 1), (520, 300, 1096, 1), (256, 70, 2048, 4), (1024, 129, 200, 3)])
+def test_many_token_kernel_with_32x32_mfma_tiles_matches_oracle(tile, m, n, k, split):
+    """The same tiles multiplied with v_mfma_f32_32x32x16_f16 (rows_per_wave = 32 in a many-token
+    config): ragged m / n / k and split-K against the oracle's float64 sums, run-to-run identical,
+    and within fp32 summation-order noise of the 16 x 16 x 32 variant."""
+    from tuna_amd import ops
+
+    rows, tt = tile
+    c32 = cfg(lds_tile_rows=rows, token_tiles=tt, split_k=split, rows_per_wave=32)
+    c16 = cfg(lds_tile_rows=rows, token_tiles=tt, split_k=split)
+    assert "mfma 32x32x16" in ops.describe_launch(m, n, k, c32) and "mfma" not in ops.describe_launch(m, n, k, c16)
+    print(f"many-token tile {rows}x{16 * tt} with 32x32 MFMA tiles, m={m} n={n} k={k} split={split}", flush=True)
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=rows + tt + split)
+    got = run_gemm(q, x, code, absmax, m, n, k, config=c32, prefill=float("nan"))
+    ref = O.gemm_f64(q, x, code, absmax, m, n, k, mode=O.D1)
+    e = rel_err(f16_bits_to_f64(got), ref)
+    assert e <= REL_TOL, e                                   # max relative error 1e-2
+    again = run_gemm(q, x, code, absmax, m, n, k, config=c32, prefill=float("nan"))
+    assert np.array_equal(got, again)
+    other = run_gemm(q, x, code, absmax, m, n, k, config=c16, prefill=float("nan"))
+    assert rel_err(f16_bits_to_f64(got), f16_bits_to_f64(other)) <= 2e-3   # one fp16 ulp of the larger outputs
+
+
 def test_many_token_kernel_decode_readout_is_bit_exact():
     """One-hot activations turn the GEMM into a readout of the decoded weights: bit-exact D1."""
     m, k = 256, 256
@@ -560,6 +584,8 @@ def test_many_token_kernel_decode_readout_is_bit_exact():
     got = run_gemm(q, x, code, absmax, m, k, k, config=cfg(lds_tile_rows=128, token_tiles=8), prefill=float("nan"))
     want = O.dequant(q, absmax, code, m, k, mode=O.D1)          # [m, k] fp16 bits
     assert np.array_equal(got.T, want)
+    got32 = run_gemm(q, x, code, absmax, m, k, k, config=cfg(lds_tile_rows=128, token_tiles=8, rows_per_wave=32), prefill=float("nan"))
+    assert np.array_equal(got32.T, want)                        # 32 x 32 x 16 MFMA tiles: the same read-out
 
 
 # ----------------------------------------------------------------------------- stream capture / graph replay, several streams

@@ -200,6 +200,7 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
 struct TiledPlan {
     TiledArgs args;
     int tile_rows, tile_tokens;
+    bool mfma32;  // rows_per_wave == 32 in a many-token config: 32 x 32 x 16 MFMAs instead of 16 x 16 x 32
     size_t lds_bytes, ws_bytes, n_counters;
 };
 
@@ -210,8 +211,10 @@ static int plan_tiled(int m, int n, int k, const tuna_gemm_config &c, int decode
     if (decode != TUNA_DECODE_GEMM)
         return fail(TUNA_ERR_UNSUPPORTED, "the many-token kernel implements TUNA_DECODE_GEMM only");
     const int tile_tokens = 16 * c.token_tiles;
-    if (!tiled_variant_exists(c.lds_tile_rows, tile_tokens))
-        return fail(TUNA_ERR_UNSUPPORTED, "no many-token kernel for a %d x %d tile (rows x tokens)", c.lds_tile_rows, tile_tokens);
+    const bool mfma32 = c.rows_per_wave == 32;
+    if (!tiled_variant_exists(c.lds_tile_rows, tile_tokens, mfma32))
+        return fail(TUNA_ERR_UNSUPPORTED, "no many-token kernel for a %d x %d tile (rows x tokens)%s", c.lds_tile_rows, tile_tokens,
+                    mfma32 ? " with 32 x 32 MFMA tiles" : "");
     const int steps = ceil_div(k, 64);
     if (c.split_k < 1 || c.split_k > steps)
         return fail(TUNA_ERR_UNSUPPORTED, "split_k=%d must be in 1..%d for the many-token kernel", c.split_k, steps);
@@ -219,6 +222,7 @@ static int plan_tiled(int m, int n, int k, const tuna_gemm_config &c, int decode
     memset(plan, 0, sizeof(*plan));
     plan->tile_rows = c.lds_tile_rows;
     plan->tile_tokens = tile_tokens;
+    plan->mfma32 = mfma32;
     plan->lds_bytes = tiled_lds_bytes(c.lds_tile_rows, tile_tokens);
     const size_t tiles = (size_t)ceil_div(m, c.lds_tile_rows) * ceil_div(n, tile_tokens);
     plan->ws_bytes = c.split_k > 1 ? tiles * c.split_k * (size_t)c.lds_tile_rows * tile_tokens * 4 : 0;
@@ -778,7 +782,7 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
         tp.args.residual = residual;
         if (tp.ws_bytes && (rc = provide_workspace(static_ws, stream, tp.ws_bytes, tp.n_counters, &tp.args.ws, &tp.args.counters)))
             return rc;
-        hipError_t e = launch_gemm_tiled(tp.args, tp.tile_rows, tp.tile_tokens, stream);
+        hipError_t e = launch_gemm_tiled(tp.args, tp.tile_rows, tp.tile_tokens, tp.mfma32, stream);
         if (e != hipSuccess) return hip_fail(e, "many-token gemm launch");
         return TUNA_OK;
     }
@@ -1481,7 +1485,8 @@ TUNA_EXPORT int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config
     if (c.lds_tile_rows) {
         TiledPlan tp;
         if ((rc = plan_tiled(m, n, k, c, decode_mode, &tp))) return rc;
-        snprintf(buf, len, "gemm_tiled_kernel<%d rows x %d tokens> split_k=%d", tp.tile_rows, tp.tile_tokens, c.split_k);
+        snprintf(buf, len, "gemm_tiled_kernel<%d rows x %d tokens%s> split_k=%d", tp.tile_rows, tp.tile_tokens,
+                 tp.mfma32 ? ",mfma 32x32x16" : "", c.split_k);
         return TUNA_OK;
     }
     if (is_narrow(c)) {

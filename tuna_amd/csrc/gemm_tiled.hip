@@ -26,6 +26,14 @@
 //     bank exactly once - no padding, no bank conflicts;
 //   * fp32 accumulators stay in registers for the whole k range; a lane ends up with 4
 //     consecutive output features of one token per MFMA tile: 8-byte stores.
+//   * M32 variants multiply with v_mfma_f32_32x32x16_f16 instead (the counterpart of the reference's
+//     wider MMA shapes, kernel.cu:411-465): a wave's TM x TN tiles of 16 x 16 become (TM/2) x (TN/2)
+//     tiles of 32 x 32, a k-step of 64 is four MFMA steps of 16 instead of two of 32.  Lane l
+//     supplies row / token l % 32 and the 8 k of half l / 32 of the step: the same 16-byte
+//     fragment reads from the same tiles (8 consecutive lanes still read 8 consecutive rows of one
+//     slot), half as many MFMA instructions for the same bytes read from LDS.  The sums are the
+//     same products added in another order, so results differ from the 16 x 16 variants in the
+//     last bits of the fp32 accumulation only.
 #include "epilogue.hpp"
 
 namespace tuna {
@@ -34,10 +42,13 @@ namespace tuna {
 constexpr int kTiledThreads = 512;
 constexpr int kTiledStepK = 64;
 
-template <int WM, int TM, int WN, int TN, int NSETS>
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+template <int WM, int TM, int WN, int TN, int NSETS, bool M32 = false>
 __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const TiledArgs a)
 {
     static_assert(WM * WN * 64 == kTiledThreads, "8 waves");
+    static_assert(!M32 || (TM % 2 == 0 && TN % 2 == 0), "32 x 32 MFMA tiles pair up the 16 x 16 ones");
     constexpr int BM = WM * TM * 16;
     constexpr int BN = WN * TN * 16;
     constexpr int A_PIECES = BM * 2;                 // 16-byte packed pieces per k-step
@@ -136,16 +147,32 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
         }
     }
 
-    f32x4 acc[TM][TN];
+    // Accumulators as TM * TN float4 "slots" in both variants.  16 x 16 tiles: slot tm * TN + tn, element
+    // v of lane l is weight row 16*tm + 4*(l/16) + v, token 16*tn + l%16.  32 x 32 tiles: tile t holds 16
+    // floats per lane, float 4*q + v being weight row 8*q + 4*(l/32) + v, token l%32 of the tile; its
+    // four float4s are the slots 4*t + q.
+    constexpr int TM2 = M32 ? TM / 2 : 1, TN2 = M32 ? TN / 2 : 1;
+    f32x4 acc[M32 ? 1 : TM][M32 ? 1 : TN];
+    f32x16 acc32[TM2][TN2];
+    if constexpr (M32) {
 #pragma unroll
-    for (int tm = 0; tm < TM; ++tm)
+        for (int tm = 0; tm < TM2; ++tm)
 #pragma unroll
-        for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int tn = 0; tn < TN2; ++tn)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc32[tm][tn][e] = 0.f;
+    } else {
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn) acc[tm][tn] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    const int i32 = lane & 31, h32 = lane >> 5;
 
     // fragment addresses: row (i16) of MFMA tile tm / tn, slot (kh*4 + g) ^ (row & 7)
-    const unsigned char *a_frag = a_tile + (wm_i * TM * 16 + i16) * 128;
-    const unsigned char *x_frag = x_tile + (wn_i * TN * 16 + i16) * 128;
-    const int sw = i16 & 7;
+    const unsigned char *a_frag = a_tile + (wm_i * TM * 16 + (M32 ? i32 : i16)) * 128;
+    const unsigned char *x_frag = x_tile + (wn_i * TN * 16 + (M32 ? i32 : i16)) * 128;
+    const int sw = (M32 ? i32 : i16) & 7;
 
     // Stage k-step s from register set `set` into tile buffer `buf`: decode the packed weights,
     // copy the activations (zero beyond n and k), then refill the set four steps ahead.
@@ -179,6 +206,21 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     // The matrix work of one k-step from tile buffer `buf`.
 #define TUNA_TILED_MFMA(buf)                                                                     \
     {                                                                                          \
+        if constexpr (M32) {                                                                   \
+            _Pragma("unroll") for (int kq = 0; kq < 4; ++kq)                                   \
+            {                                                                                  \
+                const int slot_ = (((kq * 2 + h32) ^ sw) << 4) + (buf) * BUF;                  \
+                f16x8 bf_[TN2];                                                                \
+                _Pragma("unroll") for (int tn = 0; tn < TN2; ++tn)                             \
+                    bf_[tn] = *reinterpret_cast<const f16x8 *>(x_frag + tn * (32 * 128) + slot_); \
+                _Pragma("unroll") for (int tm = 0; tm < TM2; ++tm)                             \
+                {                                                                              \
+                    const f16x8 af_ = *reinterpret_cast<const f16x8 *>(a_frag + tm * (32 * 128) + slot_); \
+                    _Pragma("unroll") for (int tn = 0; tn < TN2; ++tn) acc32[tm][tn] =         \
+                        __builtin_amdgcn_mfma_f32_32x32x16_f16(af_, bf_[tn], acc32[tm][tn], 0, 0, 0); \
+                }                                                                              \
+            }                                                                                  \
+        } else                                                                                 \
         _Pragma("unroll") for (int kh = 0; kh < 2; ++kh)                                       \
         {                                                                                      \
             const int slot_ = (((kh * 4 + g) ^ sw) << 4) + (buf) * BUF;                        \
@@ -220,20 +262,33 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
 #undef TUNA_TILED_LOAD
 
     // ---- epilogue -----------------------------------------------------------------------------
-    // acc[tm][tn][v] of lane l is weight row 4*(l/16) + v of MFMA tile tm, token l%16 of tile tn
+    // slot sl = tm * TN + tn (see the accumulators above): its float4 of this lane, first weight row, token
+    auto slot_value = [&](int sl) {
+        if constexpr (M32) {
+            const int t32 = sl >> 2, q = sl & 3;  // slots of a 32 x 32 tile are consecutive here: sl = tile * 4 + q
+            const f32x16 &t = acc32[t32 / TN2][t32 % TN2];
+            return f32x4{t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
+        } else {
+            return acc[sl / TN][sl % TN];
+        }
+    };
+    auto slot_row = [&](int sl) {
+        if constexpr (M32) return row_base + wm_i * TM * 16 + ((sl >> 2) / TN2) * 32 + (sl & 3) * 8 + h32 * 4;
+        else return row_base + (wm_i * TM + sl / TN) * 16 + g * 4;
+    };
+    auto slot_tok = [&](int sl) {
+        if constexpr (M32) return tok_base + wn_i * TN * 16 + ((sl >> 2) % TN2) * 32 + i32;
+        else return tok_base + (wn_i * TN + sl % TN) * 16 + i16;
+    };
     f16 *outp = reinterpret_cast<f16 *>(a.out);
     const f16 *resp = reinterpret_cast<const f16 *>(a.residual);
     if (a.split_k == 1) {
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm) {
-            const int row = row_base + (wm_i * TM + tm) * 16 + g * 4;
-#pragma unroll
-            for (int tn = 0; tn < TN; ++tn) {
-                const int tok = tok_base + (wn_i * TN + tn) * 16 + i16;
-                if (tok < a.n && row + 4 <= a.m) {
-                    const f32x4 v = acc[tm][tn];
-                    store_features4(outp, resp, a.epilogue, (size_t)tok, a.m, row, v[0], v[1], v[2], v[3]);
-                }
+        for (int sl = 0; sl < TM * TN; ++sl) {
+            const int row = slot_row(sl), tok = slot_tok(sl);
+            if (tok < a.n && row + 4 <= a.m) {
+                const f32x4 v = slot_value(sl);
+                store_features4(outp, resp, a.epilogue, (size_t)tok, a.m, row, v[0], v[1], v[2], v[3]);
             }
         }
         return;
@@ -245,12 +300,10 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     f32x4 *ws4 = reinterpret_cast<f32x4 *>(a.ws);
     f32x4 *mine = ws4 + (tile_id * a.split_k + blockIdx.z) * kTileF4 + (size_t)wave * (TM * TN * 64) + lane;
 #pragma unroll
-    for (int tm = 0; tm < TM; ++tm)
-#pragma unroll
-        for (int tn = 0; tn < TN; ++tn) {
-            const f32x4 v = acc[tm][tn];
-            asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 0" : : "v"(mine + (tm * TN + tn) * 64), "v"(v) : "memory");
-        }
+    for (int sl = 0; sl < TM * TN; ++sl) {
+        const f32x4 v = slot_value(sl);
+        asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 0" : : "v"(mine + sl * 64), "v"(v) : "memory");
+    }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the partial sums have left this CU
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
@@ -261,19 +314,15 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     if (tid == 0) __hip_atomic_store(a.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const f32x4 *src = ws4 + tile_id * a.split_k * kTileF4 + (size_t)wave * (TM * TN * 64) + lane;
 #pragma unroll
-    for (int tm = 0; tm < TM; ++tm) {
-        const int row = row_base + (wm_i * TM + tm) * 16 + g * 4;
+    for (int sl = 0; sl < TM * TN; ++sl) {
+        const int row = slot_row(sl), tok = slot_tok(sl);
+        float s4[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int sp = 0; sp < a.split_k; ++sp) {
+            const float *p = reinterpret_cast<const float *>(src + (size_t)sp * kTileF4 + sl * 64);
 #pragma unroll
-        for (int tn = 0; tn < TN; ++tn) {
-            const int tok = tok_base + (wn_i * TN + tn) * 16 + i16;
-            float s4[4] = {0.f, 0.f, 0.f, 0.f};
-            for (int sp = 0; sp < a.split_k; ++sp) {
-                const float *p = reinterpret_cast<const float *>(src + (size_t)sp * kTileF4 + (tm * TN + tn) * 64);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) s4[j] += __hip_atomic_load(p + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            if (tok < a.n && row + 4 <= a.m) store_features4(outp, resp, a.epilogue, (size_t)tok, a.m, row, s4[0], s4[1], s4[2], s4[3]);
+            for (int j = 0; j < 4; ++j) s4[j] += __hip_atomic_load(p + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+        if (tok < a.n && row + 4 <= a.m) store_features4(outp, resp, a.epilogue, (size_t)tok, a.m, row, s4[0], s4[1], s4[2], s4[3]);
     }
 }
 
@@ -281,51 +330,53 @@ typedef void (*TiledFn)(const TiledArgs);
 struct TiledVariant {
     int bm, bn;
     TiledFn fn;
+    TiledFn fn32;  // the same tile with 32 x 32 x 16 MFMAs, or null
 };
 // (WM, TM, WN, TN): rows x tokens of the workgroup tile
 static const TiledVariant kTiled[] = {
-    {256, 128, gemm_tiled_kernel<4, 4, 2, 4, 4>},
-    {256, 64, gemm_tiled_kernel<4, 4, 2, 2, 8>},
-    {128, 256, gemm_tiled_kernel<2, 4, 4, 4, 4>},
-    {128, 128, gemm_tiled_kernel<2, 4, 4, 2, 4>},
-    {64, 256, gemm_tiled_kernel<1, 4, 8, 2, 4>},
-    {64, 128, gemm_tiled_kernel<1, 4, 8, 1, 4>},
+    {256, 128, gemm_tiled_kernel<4, 4, 2, 4, 4>, gemm_tiled_kernel<4, 4, 2, 4, 4, true>},
+    {256, 64, gemm_tiled_kernel<4, 4, 2, 2, 8>, gemm_tiled_kernel<4, 4, 2, 2, 8, true>},
+    {128, 256, gemm_tiled_kernel<2, 4, 4, 4, 4>, gemm_tiled_kernel<2, 4, 4, 4, 4, true>},
+    {128, 128, gemm_tiled_kernel<2, 4, 4, 2, 4>, gemm_tiled_kernel<2, 4, 4, 2, 4, true>},
+    {64, 256, gemm_tiled_kernel<1, 4, 8, 2, 4>, gemm_tiled_kernel<1, 4, 8, 2, 4, true>},
+    {64, 128, gemm_tiled_kernel<1, 4, 8, 1, 4>, nullptr},
 };
 static constexpr int kNumTiled = sizeof(kTiled) / sizeof(kTiled[0]);
 
-bool tiled_variant_exists(int bm, int bn)
+bool tiled_variant_exists(int bm, int bn, bool mfma32)
 {
     for (int i = 0; i < kNumTiled; ++i)
-        if (kTiled[i].bm == bm && kTiled[i].bn == bn) return true;
+        if (kTiled[i].bm == bm && kTiled[i].bn == bn) return !mfma32 || kTiled[i].fn32 != nullptr;
     return false;
 }
 
 size_t tiled_lds_bytes(int bm, int bn) { return (size_t)kLutBytes + 2 * (size_t)(bm + bn) * 128; }  // two tile buffers
 
-static unsigned char g_tiled_attr[16][kNumTiled];
+static unsigned char g_tiled_attr[16][kNumTiled][2];
 
-hipError_t launch_gemm_tiled(const TiledArgs &args, int bm, int bn, hipStream_t stream)
+hipError_t launch_gemm_tiled(const TiledArgs &args, int bm, int bn, bool mfma32, hipStream_t stream)
 {
     int vi = -1;
     for (int i = 0; i < kNumTiled; ++i)
         if (kTiled[i].bm == bm && kTiled[i].bn == bn) vi = i;
     if (vi < 0) return hipErrorInvalidConfiguration;
+    const TiledFn fn = mfma32 ? kTiled[vi].fn32 : kTiled[vi].fn;
+    if (!fn) return hipErrorInvalidConfiguration;
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
-    if (!g_tiled_attr[dev][vi]) {  // dynamic LDS above 64 KB needs a one-time opt-in per kernel and device
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(kTiled[vi].fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                kLdsLimit);
+    if (!g_tiled_attr[dev][vi][mfma32]) {  // dynamic LDS above 64 KB needs a one-time opt-in per kernel and device
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
         if (e != hipSuccess) return e;
-        g_tiled_attr[dev][vi] = 1;
+        g_tiled_attr[dev][vi][mfma32] = 1;
     }
     TiledArgs a = args;
     a.row_tiles = ceil_div_i(args.m, bm);
     a.tok_tiles = ceil_div_i(args.n, bn);
     if ((long long)a.row_tiles * a.tok_tiles > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     const dim3 grid((unsigned)(a.row_tiles * a.tok_tiles), 1, (unsigned)args.split_k);
-    hipLaunchKernelGGL(kTiled[vi].fn, grid, dim3(kTiledThreads), tiled_lds_bytes(bm, bn), stream, a);
+    hipLaunchKernelGGL(fn, grid, dim3(kTiledThreads), tiled_lds_bytes(bm, bn), stream, a);
     return hipGetLastError();
 }
 

@@ -183,8 +183,8 @@ hipError_t launch_gemm_multi(const MultiArgs &args, int prefetch, int dev, hipSt
 hipError_t device_cus(int *dev, int *cus);
 
 // gemm_tiled.hip
-hipError_t launch_gemm_tiled(const TiledArgs &args, int tile_rows, int tile_tokens, hipStream_t stream);
-bool tiled_variant_exists(int tile_rows, int tile_tokens);
+hipError_t launch_gemm_tiled(const TiledArgs &args, int tile_rows, int tile_tokens, bool mfma32, hipStream_t stream);
+bool tiled_variant_exists(int tile_rows, int tile_tokens, bool mfma32);
 size_t tiled_lds_bytes(int tile_rows, int tile_tokens);
 
 // dequant_kernel.hip

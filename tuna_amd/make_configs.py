@@ -98,6 +98,8 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
         # many-token kernel: only the tile shape and the split matter
         if (c["lds_tile_rows"], 16 * c["token_tiles"]) not in TILED_VARIANTS:
             raise ValueError(f"no many-token kernel for a {c['lds_tile_rows']} x {16 * c['token_tiles']} tile")
+        if c["rows_per_wave"] == 32 and (c["lds_tile_rows"], 16 * c["token_tiles"]) == (64, 128):
+            raise ValueError("the 64 x 128 tile has no 32 x 32 MFMA variant (one 16-token tile per wave)")
         if not 1 <= c["split_k"] <= -(-k // 64):
             raise ValueError("split_k of the many-token kernel must be in 1..ceil(k/64)")
         return

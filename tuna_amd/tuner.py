@@ -120,13 +120,14 @@ def tiled_space(m: int, n_key: int, k: int):
         for split in (1, 2, 3, 4, 6, 8, 12, 16, 24, 32):
             if split > 1 and (steps // split < 4 or tiles * split > 4 * N_CU):
                 continue
-            c = dict(rows_per_wave=64, waves_m=1, waves_k=1, split_k=split, prefetch=2, x_chunk=64, token_tiles=tokens // 16,
-                     xcd_swizzle=0, k_stagger=0, lds_tile_rows=rows)
-            try:
-                make_configs.validate(m, n_key, k, c)
-            except ValueError:
-                continue
-            out.append(c)
+            for mfma_rows in (64, 32):   # 16 x 16 x 32 MFMA tiles (any value but 32) / 32 x 32 x 16
+                c = dict(rows_per_wave=mfma_rows, waves_m=1, waves_k=1, split_k=split, prefetch=2, x_chunk=64,
+                         token_tiles=tokens // 16, xcd_swizzle=0, k_stagger=0, lds_tile_rows=rows)
+                try:
+                    make_configs.validate(m, n_key, k, c)
+                except ValueError:
+                    continue
+                out.append(c)
     return out
 
 
