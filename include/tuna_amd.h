@@ -79,7 +79,11 @@ typedef struct tuna_gemm_config {
                               around (0: every row tile starts at the front).  When k*4 bytes,
                               the distance between block rows, is a large power of two, tiles
                               walking in lockstep keep hitting the same memory channels  */
-    int32_t lds_tile_rows; /* 0: streaming kernel (all fields above).  64, 128 or 256: the
+    int32_t lds_tile_rows; /* 0: streaming kernel (all fields above).  -1: the same, with the packed
+                              weights, x and scales staged through LDS by global -> LDS loads
+                              (the reference's weight path, kernel.cu:1997-2042) instead of
+                              registers: same results bit for bit; for unsplit 16-wave launches
+                              of up to 16 tokens with prefetch 2 or 4.  64, 128 or 256: the
                               many-token kernel, which decodes a tile of this many weight rows
                               once into LDS for token_tiles*16 (64, 128 or 256) tokens; only
                               token_tiles, split_k (>= 1) and rows_per_wave are read besides:

@@ -922,22 +922,26 @@ def test_weights_staged_through_lds_equal_the_register_ring_bit_for_bit(ci):
     print(f"lds path case#{ci} {m}x{n}x{k} {c.to_dict()}", flush=True)
     q, x, code, absmax = make_inputs_np(m, n, k, seed=700 + ci)
     dq, dx, dc, da = to_dev(q, x, code, absmax)
+    c_lds = cfg(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=1, prefetch=pf, x_chunk=xc, k_stagger=st, lds_tile_rows=-1)
     outs = {}
     prev = ops.set_weight_path(False)
     try:
-        for staged in (False, True):
+        # the register ring, the diagnostic switch, and a config that asks for the LDS path itself
+        for mode, (staged, cc) in {"registers": (False, c), "switch": (True, c), "config": (False, c_lds)}.items():
             ops.set_weight_path(staged)
-            d = ops.describe_launch(m, n, k, c)
-            assert d.startswith("gemm_mid_kernel") and (("through LDS" in d) == staged), d
+            d = ops.describe_launch(m, n, k, cc)
+            assert d.startswith("gemm_mid_kernel") and (("through LDS" in d) == (mode != "registers")), d
             o = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
-            ops.matmul(dx, dq, da, dc, o, m, n, k, config=c)
-            ops.matmul(dx, dq, da, dc, o, m, n, k, config=c)   # twice: the second launch finds LDS-independent state
+            ops.matmul(dx, dq, da, dc, o, m, n, k, config=cc)
+            ops.matmul(dx, dq, da, dc, o, m, n, k, config=cc)   # twice: the second launch finds LDS-independent state
             torch.cuda.synchronize()
-            outs[staged] = o
+            outs[mode] = o
     finally:
         ops.set_weight_path(prev)
-    assert not torch.isnan(outs[True].float()).any()
-    assert torch.equal(outs[True].view(torch.int16), outs[False].view(torch.int16))
+    assert not torch.isnan(outs["switch"].float()).any()
+    assert torch.equal(outs["switch"].view(torch.int16), outs["registers"].view(torch.int16))
+    assert torch.equal(outs["config"].view(torch.int16), outs["registers"].view(torch.int16))
+    outs = {True: outs["config"]}
     rows = np.random.default_rng(ci).choice(m, size=min(m, 256), replace=False).astype(np.int32)
     ref = O.gemm_f64(q, x, code, absmax, m, n, k, mode=O.D1, rows=rows)
     assert rel_err(outs[True].cpu().numpy().astype(np.float64)[:, rows], ref) <= REL_TOL   # max relative error 1e-2

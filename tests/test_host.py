@@ -222,6 +222,22 @@ def test_tuner_small_launch_config_spaces_are_valid_for_both_validators():
         assert big and all(mc.mid_applies(57344, 8192, c) for c in big)
         # 128 and 256 tokens: also passes of 32 and 64 tokens (they share the weights when they all fit the device)
         assert {c["token_tiles"] for c in big} == ({8, 4, 2} if n_key <= 256 else {8})
+    # packed weights staged through LDS (lds_tile_rows = -1): offered for 16-wave launches with one token tile, valid
+    # for both validators exactly where the twin exists
+    sp16 = tuner.mid_space(229376, 16, 4096)
+    lds = [c for c in sp16 if c["lds_tile_rows"] == -1]
+    assert lds and all(c["waves_m"] * c["waves_k"] == 16 and c["prefetch"] in (2, 4) and c["token_tiles"] == 1 for c in lds)
+    for c in lds[:40]:
+        mc.validate(229376, 16, 4096, c)
+        ops.validate_config(229376, 16, 4096, ops.GemmConfig.from_dict(c))
+        assert "weights through LDS" in ops.describe_launch(229376, 16, 4096, ops.GemmConfig.from_dict(c))
+    assert all(c["lds_tile_rows"] == 0 for c in tuner.mid_space(229376, 64, 4096))
+    for bad in (dict(lds[0], waves_m=8, waves_k=1), dict(lds[0], prefetch=8, x_chunk=1024), dict(lds[0], token_tiles=2),
+                dict(lds[0], split_k=2), dict(lds[0], lds_tile_rows=-2)):
+        with pytest.raises(ValueError):
+            mc.validate(229376, 16 if bad["token_tiles"] == 1 else 32, 4096, bad)
+        with pytest.raises(ops.TunaError):
+            ops.validate_config(229376, 16 if bad["token_tiles"] == 1 else 32, 4096, ops.GemmConfig.from_dict(bad))
     assert tuner.narrow_space(4096, 128, 4096) == [] and tuner.lean_space(4096, 128, 4096) == []
     assert tuner.lean_space(4096, 16, 4104) == []       # k not a multiple of 32: no lean launch
 

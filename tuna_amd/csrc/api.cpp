@@ -68,7 +68,8 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
                     (unsigned long long)m * (unsigned long long)k / 2);
     if (decode != TUNA_DECODE_GEMM && decode != TUNA_DECODE_DEQUANT)
         return fail(TUNA_ERR_INVALID_ARG, "decode_mode %d is neither TUNA_DECODE_GEMM nor TUNA_DECODE_DEQUANT", decode);
-    if (c.lds_tile_rows) return fail(TUNA_ERR_INVALID_ARG, "plan_gemm called with a many-token config");
+    if (c.lds_tile_rows > 0) return fail(TUNA_ERR_INVALID_ARG, "plan_gemm called with a many-token config");
+    if (c.lds_tile_rows < -1) return fail(TUNA_ERR_INVALID_ARG, "lds_tile_rows=%d (0, -1, 64, 128 or 256)", c.lds_tile_rows);
     if (c.rows_per_wave != 64 && c.rows_per_wave != 128 && c.rows_per_wave != 256)
         return fail(TUNA_ERR_UNSUPPORTED, "rows_per_wave=%d (64, 128 or 256)", c.rows_per_wave);
     if (c.prefetch != 2 && c.prefetch != 4 && c.prefetch != 8)
@@ -158,6 +159,7 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
     p.decode = decode;
     p.min_waves = min_waves;
     p.wgs_per_cu = wgs_per_cu;
+    p.lds_weights = c.lds_tile_rows == -1 ? 1 : 0;
     p.threads = threads;
     p.lds_bytes = lds;
     p.grid = dim3(grid_x, (unsigned)tok_chunks, 1);
@@ -193,6 +195,11 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
         return fail(TUNA_ERR_UNSUPPORTED,
                     "no %skernel variant for rows_per_wave=%d prefetch=%d token_tiles=%d decode=%d threads=%d",
                     grouped ? "grouped " : "", c.rows_per_wave, c.prefetch, c.token_tiles, decode, threads);
+    if (p.lds_weights && (grouped || !mid_lds_applies(*plan)))
+        return fail(TUNA_ERR_UNSUPPORTED,
+                    "lds_tile_rows=-1 (packed weights through LDS) needs a dense unsplit launch of 16 waves, 64 rows per wave, one "
+                    "token tile, prefetch 2 or 4, the GEMM's own decode, m a multiple of 64*waves_m and x chunks of 512 or 1024 k "
+                    "that divide k and leave room for the rings");
     return TUNA_OK;
 }
 
@@ -426,7 +433,7 @@ static tuna_gemm_config derive_config(int m, int n, int k)
 // Whether config c can run the shape (the checks of the three planners).
 static bool config_runs(int m, int n, int k, const tuna_gemm_config &c)
 {
-    if (c.lds_tile_rows) {
+    if (c.lds_tile_rows > 0) {
         TiledPlan tp;
         return plan_tiled(m, n, k, c, TUNA_DECODE_GEMM, &tp) == TUNA_OK;
     }
@@ -486,7 +493,7 @@ static int select_config_for(int m, int n, int k, int decode, tuna_gemm_config *
 // The checks of the planner `c` belongs to, for a decode mode.
 static int validate_for(int m, int n, int k, const tuna_gemm_config &c, int decode)
 {
-    if (c.lds_tile_rows) {
+    if (c.lds_tile_rows > 0) {
         TiledPlan tp;
         return plan_tiled(m, n, k, c, decode, &tp);
     }
@@ -770,7 +777,7 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
     tuna_gemm_config c;
     if (cfg) c = *cfg;
     else select_config_for(m, n, k, decode, &c, nullptr);
-    if (c.lds_tile_rows) {
+    if (c.lds_tile_rows > 0) {
         TiledPlan tp;
         if ((rc = plan_tiled(m, n, k, c, decode, &tp))) return rc;
         tp.args.q = static_cast<const uint8_t *>(q);
@@ -1271,7 +1278,7 @@ TUNA_EXPORT int tuna_config_footprint(int m, int n, int k, const tuna_gemm_confi
                                       size_t *workspace_bytes)
 {
     if (!cfg) return fail(TUNA_ERR_INVALID_ARG, "cfg is null");
-    if (cfg->lds_tile_rows) {
+    if (cfg->lds_tile_rows > 0) {
         TiledPlan tp;
         int rc = plan_tiled(m, n, k, *cfg, TUNA_DECODE_GEMM, &tp);
         if (rc) return rc;
@@ -1482,7 +1489,7 @@ TUNA_EXPORT int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config
     tuna_gemm_config c;
     if (cfg) c = *cfg;
     else select_config_for(m, n, k, decode_mode, &c, nullptr);
-    if (c.lds_tile_rows) {
+    if (c.lds_tile_rows > 0) {
         TiledPlan tp;
         if ((rc = plan_tiled(m, n, k, c, decode_mode, &tp))) return rc;
         snprintf(buf, len, "gemm_tiled_kernel<%d rows x %d tokens%s> split_k=%d", tp.tile_rows, tp.tile_tokens,

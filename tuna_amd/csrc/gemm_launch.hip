@@ -169,7 +169,7 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
     const Variant *v = find_variant(plan.rw, plan.prefetch, plan.token_tiles, plan.decode, plan.threads, plan.min_waves,
                                     plan.args.group_rows ? 1 : 0);
     // (deeper rings with four token tiles exist in the 17..128-token streaming kernel only)
-    if ((!v || g_lean_enabled.load(std::memory_order_relaxed)) && mid_applies(plan)) {
+    if ((!v || plan.lds_weights || g_lean_enabled.load(std::memory_order_relaxed)) && mid_applies(plan)) {
         e = launch_gemm_mid(plan, dev, cus, stream);
         if (e == hipSuccess) g_lean_launches.fetch_add(1, std::memory_order_relaxed);
         return e;

@@ -41,8 +41,8 @@ int set_weight_path(int path)
 }
 static bool lds_path(const GemmPlan &plan)
 {
-    return g_weight_path.load(std::memory_order_relaxed) != 0 && plan.token_tiles == 1 && plan.threads == 1024 &&
-           (plan.prefetch == 2 || plan.prefetch == 4);
+    return (plan.lds_weights || g_weight_path.load(std::memory_order_relaxed) != 0) && plan.token_tiles == 1 &&
+           plan.threads == 1024 && (plan.prefetch == 2 || plan.prefetch == 4);
 }
 
 // x chunk the kernel uses: the config's, capped so that two buffers fit beside the decode table
@@ -85,6 +85,15 @@ bool mid_applies(const GemmPlan &plan)
 {
     int xc;
     return mid_variant(plan, &xc) != nullptr;
+}
+
+bool mid_lds_applies(const GemmPlan &plan)
+{
+    int xc;
+    const MidVariant *v = mid_variant(plan, &xc);
+    if (!v || !v->fn_lds || !lds_path(plan) || (xc != 512 && xc != 1024)) return false;
+    const size_t x_lds = 2 * (size_t)32 * (size_t)xc, red_lds = 2 * (size_t)(plan.threads / 64) * 1024;
+    return x_lds >= red_lds && (size_t)kLutBytes + x_lds + (size_t)(plan.threads / 64) * plan.prefetch * 1024 <= (size_t)kLdsLimit;
 }
 
 bool mid_describe(const GemmPlan &plan, char *buf, size_t len)

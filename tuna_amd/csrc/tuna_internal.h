@@ -140,6 +140,7 @@ struct GemmPlan {
     int rw, prefetch, token_tiles, decode;
     int min_waves;  // waves per SIMD the variant is compiled for (2: <=256 VGPRs, 4: <=128)
     int wgs_per_cu; // workgroups of this launch that fit on one CU (LDS and registers)
+    int lds_weights; // the config asks for the packed weights staged through LDS (lds_tile_rows == -1)
     size_t lds_bytes;
     size_t ws_bytes;
     size_t n_counters;
@@ -149,6 +150,7 @@ struct GemmPlan {
 hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream);
 // 17..128-token streaming twin of the general kernel (gemm_mid.hpp) for the launches it applies to.
 bool mid_applies(const GemmPlan &plan);
+bool mid_lds_applies(const GemmPlan &plan);  // ... with the packed weights staged through LDS
 hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t stream);
 bool mid_describe(const GemmPlan &plan, char *buf, size_t len);
 // Name and template arguments of the kernel launch_gemm would start for `plan` on a device of `cus` CUs.

@@ -81,7 +81,7 @@ def bucket_of(n: int):
 
 def is_narrow(c: dict) -> bool:
     """The config selects the narrow-row kernel: rows_per_wave 16 or 32, or 64 with waves_m 0."""
-    return not c.get("lds_tile_rows") and (c["rows_per_wave"] in (16, 32) or (c["rows_per_wave"] == 64 and c["waves_m"] == 0))
+    return c.get("lds_tile_rows", 0) == 0 and (c["rows_per_wave"] in (16, 32) or (c["rows_per_wave"] == 64 and c["waves_m"] == 0))
 
 
 def validate(m: int, n_key: int, k: int, c: dict) -> None:
@@ -94,7 +94,9 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
         raise ValueError("m and k must be positive multiples of 8")
     if n_key not in N_BUCKETS:
         raise ValueError(f"n={n_key} is not a bucket key {sorted(N_BUCKETS)}")
-    if c["lds_tile_rows"]:
+    if c["lds_tile_rows"] not in (0, -1, 64, 128, 256):
+        raise ValueError("lds_tile_rows must be 0, -1 (packed weights through LDS), 64, 128 or 256")
+    if c["lds_tile_rows"] > 0:
         # many-token kernel: only the tile shape and the split matter
         if (c["lds_tile_rows"], 16 * c["token_tiles"]) not in TILED_VARIANTS:
             raise ValueError(f"no many-token kernel for a {c['lds_tile_rows']} x {16 * c['token_tiles']} tile")
@@ -146,6 +148,27 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
         raise ValueError("k_stagger must be in 0..4096")
     if lds_bytes(c) > LDS_LIMIT:
         raise ValueError(f"needs {lds_bytes(c)} bytes of LDS (limit {LDS_LIMIT})")
+    if c["lds_tile_rows"] == -1 and not mid_lds_applies(m, k, c):
+        raise ValueError("lds_tile_rows -1 needs an unsplit 16-wave launch with one token tile, prefetch 2 or 4 and "
+                         "x chunks of 512 or 1024 k that leave room for the weight rings")
+
+
+def mid_lds_applies(m: int, k: int, c: dict) -> bool:
+    """True if the streaming kernel's twin with the packed weights staged through LDS takes a dense
+    launch of this config (mirrors mid_lds_applies in csrc/gemm_mid.hip)."""
+    wm, wk, pf = c["waves_m"], c["waves_k"], c["prefetch"]
+    if c["rows_per_wave"] != 64 or c["token_tiles"] != 1 or c["split_k"] != 1 or wm * wk != 16 or pf not in (2, 4):
+        return False
+    if k % STEP_K or k >= 1 << 23 or not _pow2(wk) or m % (64 * wm) or not 0 <= c["k_stagger"] <= 4096:
+        return False
+    ring = 16 * pf * 1024
+    xc = c["x_chunk"]
+    cap = (LDS_LIMIT - LUT_BYTES - ring) // (2 * 32)
+    while xc > cap:
+        xc //= 2
+    if xc not in (512, 1024) or xc < wk * pf * STEP_K or k % xc:
+        return False
+    return 2 * 32 * xc >= 2 * 16 * 1024 and LUT_BYTES + 2 * 32 * xc + ring <= LDS_LIMIT
 
 
 def mid_applies(m: int, k: int, c: dict) -> bool:
@@ -174,7 +197,7 @@ def lds_bytes(c: dict) -> int:
 
     The reduction buffers are 2 x 1 plane (1 KB) per wave, or 2 x 4 planes (1 x 4 for a wave with one
     64-row group and token tile) when that costs no occupancy (mirrors plan_gemm in csrc/api.cpp)."""
-    if c.get("lds_tile_rows"):
+    if c.get("lds_tile_rows", 0) > 0:
         # many-token kernel: decode table + two buffers of (weight tile + activation tile), 128 bytes per row
         return LUT_BYTES + 2 * (c["lds_tile_rows"] + 16 * c["token_tiles"]) * 128
     if is_narrow(c):

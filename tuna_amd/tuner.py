@@ -50,7 +50,7 @@ def repair(c: dict, m: int, n_key: int, k: int):
     c = dict(c)
     c.setdefault("k_stagger", 0)
     c.setdefault("lds_tile_rows", 0)
-    if c["lds_tile_rows"] or make_configs.is_narrow(c):
+    if c["lds_tile_rows"] > 0 or make_configs.is_narrow(c):
         try:
             make_configs.validate(m, n_key, k, c)
             return c
@@ -194,6 +194,10 @@ def mid_space(m: int, n_key: int, k: int):
                                 continue
                             if make_configs.mid_applies(m, k, c):
                                 out.append(c)
+                                # the same launch with the packed weights staged through LDS, where that twin exists
+                                cl = dict(c, lds_tile_rows=-1)
+                                if make_configs.mid_lds_applies(m, k, cl):
+                                    out.append(cl)
     return out
 
 
