@@ -47,6 +47,8 @@ MEASURED_TRAFFIC = {
     ("mistral_qkv", "gemm_narrow_kernel<LW=2,WK=8,U=4,PERM=1,TT=1>"): (6700.5, 192.0),
     # profiles/gemm_lean_kernel_llama70b_qkv_kernel_trace_and_counters.md
     ("llama70b_qkv", "gemm_lean_kernel<WK=4,U=2,1024 threads> split_k=4"): (22857.5, 2886.2),
+    # profiles/gemm_mid_kernel_weights_through_lds_vs_registers.md
+    ("llama70b_gate_up", "gemm_mid_kernel<U=4,TT=1,XB=4,1024 threads,weights through LDS> x_chunk=512"): (116009.3, 1792.0),
 }
 
 
@@ -101,6 +103,27 @@ def time_shape(ops, synth, torch, dev, m, n, k, steps, warmup, seed0=0, use_grap
         "launch": "graph" if use_graph else "stream",
         "kernel": ops.describe_launch(m, n, k, cfg),
     }
+
+
+def mfma_shapes(ops, synth, torch, dev, tokens):
+    """The many-token kernel's 256 x 128 tile with v_mfma_f32_16x16x32_f16 and with v_mfma_f32_32x32x16_f16
+    (rows_per_wave 64 / 32 in the config), same inputs, alternating, on two Llama-70B shapes."""
+    out = {}
+    for name in ("llama70b_gate_up", "llama70b_qkv"):
+        m, k = synth.SHAPES[name]
+        sets = [synth.make_weights_torch(m, k, 40 + i, dev) for i in range(3)]
+        row = {}
+        for rep in range(2):
+            for label, rpw in (("mfma_16x16x32", 64), ("mfma_32x32x16", 32)):
+                c = ops.GemmConfig(rows_per_wave=rpw, waves_m=1, waves_k=1, split_k=1, prefetch=2, x_chunk=64, token_tiles=8,
+                                   xcd_swizzle=0, k_stagger=0, lds_tile_rows=256)
+                r = time_shape(ops, synth, torch, dev, m, tokens, k, 20, 5, cfg=c, sets=sets)
+                if label not in row or r["us_per_gemm"] < row[label]["us"]:
+                    row[label] = {"us": r["us_per_gemm"], "tflops": r["tflops"], "kernel": r["kernel"]}
+        out[name] = {"tokens": tokens, **row}
+        del sets
+        torch.cuda.empty_cache()
+    return out
 
 
 def cpu_baseline(m, n, k, budget_s=12.0):
@@ -296,9 +319,13 @@ def main():
     ap.add_argument("--launch", choices=("both", "stream", "graph"), default="both")
     ap.add_argument("--settle", type=int, default=300,
                     help="untimed launches before the warm-up of the headline (a box that was idle ramps its clocks)")
-    ap.add_argument("--only", choices=("read", "dequant", "quantize", "multi"), default=None,
+    ap.add_argument("--only", choices=("read", "dequant", "quantize", "multi", "mfma"), default=None,
                     help="profiling runs: launch only the read-kernel sweep / the dequant kernel / the quantizer / "
-                         "the Llama-70B layer set through tuna_matmul_multi (16 layers)")
+                         "the Llama-70B layer set through tuna_matmul_multi (16 layers) / the many-token kernel with "
+                         "16x16x32 and with 32x32x16 MFMA tiles (Llama-70B gate+up and QKV, --tokens, default 1024)")
+    ap.add_argument("--weight-path", choices=("table", "registers", "lds"), default="table",
+                    help="headline workload: the table's config as it is, or with the packed weights forced through "
+                         "registers / staged through LDS (lds_tile_rows 0 / -1; A/B runs of the two weight paths)")
     ap.add_argument("--copy-yardstick", type=int, default=0, metavar="MIB",
                     help="also launch the plain copy kernel over MIB mebibytes (counter runs: the known-traffic "
                          "launch the HBM counters of the GEMM kernel are scaled by)")
@@ -326,6 +353,8 @@ def main():
             res = {"dequant": time_dequant_shapes(ops, synth, torch, dev)}
         elif args.only == "quantize":
             res = {"quantize": time_quantize(ops, synth, torch, dev)}
+        elif args.only == "mfma":
+            res = {"many_token_kernel_mfma_shapes": mfma_shapes(ops, synth, torch, dev, 1024 if args.tokens == TOKENS else args.tokens)}
         else:
             names = ["llama70b_qkv", "llama70b_attn_out", "llama70b_gate_up", "llama70b_down"]
             res = {"llama70b_layers_multi": multi_layer_sweep(ops, synth, torch, dev, names, args.tokens, layers=16)}
@@ -336,11 +365,18 @@ def main():
 
     m, k = synth.SHAPES[args.workload]
     n = args.tokens
+    head_cfg = None
+    if args.weight_path != "table":
+        head_cfg, _ = ops.select_config(m, n, k)
+        head_cfg.lds_tile_rows = -1 if args.weight_path == "lds" else 0
+        ops.validate_config(m, n, k, head_cfg)   # raises where the shape's config has no such twin
     res_stream = res_graph = None
     if args.launch in ("both", "stream"):
-        res_stream = time_shape(ops, synth, torch, dev, m, n, k, args.steps, args.warmup, use_graph=False, settle=args.settle)
+        res_stream = time_shape(ops, synth, torch, dev, m, n, k, args.steps, args.warmup, use_graph=False, cfg=head_cfg,
+                                settle=args.settle)
     if args.launch in ("both", "graph"):
-        res_graph = time_shape(ops, synth, torch, dev, m, n, k, args.steps, args.warmup, use_graph=True, settle=args.settle)
+        res_graph = time_shape(ops, synth, torch, dev, m, n, k, args.steps, args.warmup, use_graph=True, cfg=head_cfg,
+                               settle=args.settle)
     cands = [r for r in (res_stream, res_graph) if r is not None]
     head = min(cands, key=lambda r: r["us_per_gemm"])
     line = {
