@@ -92,7 +92,7 @@ int tuna_set_lean_kernels(int enabled);
 unsigned long long tuna_lean_launches(void);
 
 /* Diagnostic switch, process-wide, default 0: with 1, unsplit 16-wave launches of up to 16 tokens
- * (the streaming kernel of gemm_mid.hpp with ring depth 2 or 4) stage the packed weights through
+ * and 8- or 16-wave launches with more token tiles (the streaming kernel of gemm_mid.hpp, ring depth 2 or 4) stage the packed weights through
  * LDS (global_load_lds_dwordx4 into a per-wave ring, ds_read_b128 when a slot is consumed) instead
  * of loading them into registers.  Same access pattern, ring depth, arithmetic and results; it
  * exists so that the two weight paths can be timed against each other on one box (the reference

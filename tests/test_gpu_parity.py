@@ -904,6 +904,13 @@ LDS_PATH_CASES = [
     (512, 5, 2048, 2, 8, 2, 512, 0),
     (256 * 300, 16, 1024, 4, 4, 2, 1024, 3),  # more row tiles than compute units: workgroups that walk two tiles
     (1024 * 260, 3, 512, 16, 1, 2, 512, 1),
+    # two, four and eight token tiles per pass (9th entry), 8 and 16 waves
+    (512, 32, 4096, 2, 4, 4, 512, 1, 2),
+    (2048, 27, 2048, 4, 4, 2, 512, 0, 2),      # 16 waves, ragged token count
+    (1024, 40, 2048, 4, 2, 4, 256, 2, 4),
+    (2048, 100, 1024, 8, 1, 2, 128, 0, 8),     # one pass of 128 tokens, 100 present
+    (1024, 300, 1024, 4, 2, 2, 128, 3, 8),     # three token chunks
+    (512 * 70, 1100, 512, 8, 1, 2, 128, 0, 8), # 70 row tiles x 9 token chunks: chunks of a walker side by side
 ]
 
 
@@ -917,12 +924,14 @@ def test_weights_staged_through_lds_equal_the_register_ring_bit_for_bit(ci):
 
     from tuna_amd import ops
 
-    m, n, k, wm, wk, pf, xc, st = LDS_PATH_CASES[ci]
-    c = cfg(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=1, prefetch=pf, x_chunk=xc, k_stagger=st)
+    m, n, k, wm, wk, pf, xc, st = LDS_PATH_CASES[ci][:8]
+    tt = LDS_PATH_CASES[ci][8] if len(LDS_PATH_CASES[ci]) > 8 else 1
+    c = cfg(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=1, prefetch=pf, x_chunk=xc, k_stagger=st, token_tiles=tt)
     print(f"lds path case#{ci} {m}x{n}x{k} {c.to_dict()}", flush=True)
     q, x, code, absmax = make_inputs_np(m, n, k, seed=700 + ci)
     dq, dx, dc, da = to_dev(q, x, code, absmax)
-    c_lds = cfg(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=1, prefetch=pf, x_chunk=xc, k_stagger=st, lds_tile_rows=-1)
+    c_lds = cfg(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=1, prefetch=pf, x_chunk=xc, k_stagger=st, token_tiles=tt,
+                lds_tile_rows=-1)
     outs = {}
     prev = ops.set_weight_path(False)
     try:

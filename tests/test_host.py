@@ -231,13 +231,21 @@ def test_tuner_small_launch_config_spaces_are_valid_for_both_validators():
         mc.validate(229376, 16, 4096, c)
         ops.validate_config(229376, 16, 4096, ops.GemmConfig.from_dict(c))
         assert "weights through LDS" in ops.describe_launch(229376, 16, 4096, ops.GemmConfig.from_dict(c))
-    assert all(c["lds_tile_rows"] == 0 for c in tuner.mid_space(229376, 64, 4096))
-    for bad in (dict(lds[0], waves_m=8, waves_k=1), dict(lds[0], prefetch=8, x_chunk=1024), dict(lds[0], token_tiles=2),
+    # ... and for the passes of 32 ... 128 tokens (8 or 16 waves, ring 2 or 4; ring 2 with eight token tiles)
+    for n_key in (64, 128):
+        sp = [c for c in tuner.mid_space(229376, n_key, 4096) if c["lds_tile_rows"] == -1]
+        assert sp and all(c["waves_m"] * c["waves_k"] in (8, 16) and c["prefetch"] in (2, 4) for c in sp)
+        assert all(c["prefetch"] == 2 for c in sp if c["token_tiles"] == 8)
+        for c in sp[:40]:
+            mc.validate(229376, n_key, 4096, c)
+            ops.validate_config(229376, n_key, 4096, ops.GemmConfig.from_dict(c))
+            assert "weights through LDS" in ops.describe_launch(229376, n_key, 4096, ops.GemmConfig.from_dict(c))
+    for bad in (dict(lds[0], waves_m=4, waves_k=1), dict(lds[0], prefetch=8, x_chunk=1024), dict(lds[0], token_tiles=8, prefetch=4),
                 dict(lds[0], split_k=2), dict(lds[0], lds_tile_rows=-2)):
         with pytest.raises(ValueError):
-            mc.validate(229376, 16 if bad["token_tiles"] == 1 else 32, 4096, bad)
+            mc.validate(229376, 16 if bad["token_tiles"] == 1 else 128, 4096, bad)
         with pytest.raises(ops.TunaError):
-            ops.validate_config(229376, 16 if bad["token_tiles"] == 1 else 32, 4096, ops.GemmConfig.from_dict(bad))
+            ops.validate_config(229376, 16 if bad["token_tiles"] == 1 else 128, 4096, ops.GemmConfig.from_dict(bad))
     assert tuner.narrow_space(4096, 128, 4096) == [] and tuner.lean_space(4096, 128, 4096) == []
     assert tuner.lean_space(4096, 16, 4104) == []       # k not a multiple of 32: no lean launch
 

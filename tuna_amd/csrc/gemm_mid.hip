@@ -13,22 +13,27 @@ struct MidVariant {
     int u, tt, xb, maxt;
     MidKernelFn fn;
     MidKernelFn fn_shared;  // twin without the nontemporal hint on the weight loads (token chunks side by side), or null
-    MidKernelFn fn_lds;     // twin with the packed weights staged through LDS (diagnostic switch), or null
+    MidKernelFn fn_lds;     // twin with the packed weights staged through LDS (lds_tile_rows = -1 or the diagnostic switch), or null
+    MidKernelFn fn_lds_shared;  // ... without the nontemporal hint, or null
 };
-#define M5(U, TT, XB) {U, TT, XB, 512, gemm_mid_kernel<U, TT, XB, 512, 2>, nullptr, nullptr}
-#define M5S(U, TT, XB) {U, TT, XB, 512, gemm_mid_kernel<U, TT, XB, 512, 2>, gemm_mid_kernel<U, TT, XB, 512, 2, false>, nullptr}
-#define M10(U, TT, XB) {U, TT, XB, 1024, gemm_mid_kernel<U, TT, XB, 1024, 4>, nullptr, nullptr}
-#define M10L(U, TT, XB) {U, TT, XB, 1024, gemm_mid_kernel<U, TT, XB, 1024, 4>, nullptr, gemm_mid_kernel<U, TT, XB, 1024, 4, true, true>}
+#define M5(U, TT, XB) {U, TT, XB, 512, gemm_mid_kernel<U, TT, XB, 512, 2>, nullptr, nullptr, nullptr}
+#define M5L(U, TT, XB) {U, TT, XB, 512, gemm_mid_kernel<U, TT, XB, 512, 2>, nullptr, gemm_mid_kernel<U, TT, XB, 512, 2, true, true>, nullptr}
+#define M5SL(U, TT, XB)                                                                                             \
+    {U, TT, XB, 512, gemm_mid_kernel<U, TT, XB, 512, 2>, gemm_mid_kernel<U, TT, XB, 512, 2, false>,                \
+     gemm_mid_kernel<U, TT, XB, 512, 2, true, true>, gemm_mid_kernel<U, TT, XB, 512, 2, false, true>}
+#define M10(U, TT, XB) {U, TT, XB, 1024, gemm_mid_kernel<U, TT, XB, 1024, 4>, nullptr, nullptr, nullptr}
+#define M10L(U, TT, XB) {U, TT, XB, 1024, gemm_mid_kernel<U, TT, XB, 1024, 4>, nullptr, gemm_mid_kernel<U, TT, XB, 1024, 4, true, true>, nullptr}
 static const MidVariant kMid[] = {
-    M5(2, 2, 4), M5(4, 2, 4), M5(8, 2, 4), M5(2, 2, 8), M5(4, 2, 8), M5(8, 2, 8),
-    M5(2, 4, 4), M5(4, 4, 4), M5(8, 4, 4), M5(2, 4, 8), M5(4, 4, 8), M5(8, 4, 8),
-    M5S(2, 8, 4), M5S(2, 8, 8),  // (deeper rings with eight token tiles spill inside the loop)
-    M10(2, 2, 4), M10(4, 2, 4),
+    M5L(2, 2, 4), M5L(4, 2, 4), M5(8, 2, 4), M5(2, 2, 8), M5(4, 2, 8), M5(8, 2, 8),
+    M5L(2, 4, 4), M5L(4, 4, 4), M5(8, 4, 4), M5L(2, 4, 8), M5L(4, 4, 8), M5(8, 4, 8),
+    M5SL(2, 8, 4), M5SL(2, 8, 8),  // (deeper rings with eight token tiles spill inside the loop)
+    M10L(2, 2, 4), M10L(4, 2, 4),
     // one token tile: the large shapes at up to 16 tokens (small launches take gemm_lean.hpp first)
     M5(2, 1, 4), M5(4, 1, 4), M5(8, 1, 4), M5(2, 1, 8), M5(4, 1, 8), M5(8, 1, 8), M10L(2, 1, 4), M10L(4, 1, 4), M10(8, 1, 4),
 };
 #undef M5
-#undef M5S
+#undef M5L
+#undef M5SL
 #undef M10
 #undef M10L
 static constexpr int kNumMid = sizeof(kMid) / sizeof(kMid[0]);
@@ -41,8 +46,8 @@ int set_weight_path(int path)
 }
 static bool lds_path(const GemmPlan &plan)
 {
-    return (plan.lds_weights || g_weight_path.load(std::memory_order_relaxed) != 0) && plan.token_tiles == 1 &&
-           plan.threads == 1024 && (plan.prefetch == 2 || plan.prefetch == 4);
+    return (plan.lds_weights || g_weight_path.load(std::memory_order_relaxed) != 0) && (plan.threads == 512 || plan.threads == 1024) &&
+           (plan.prefetch == 2 || plan.prefetch == 4);
 }
 
 // x chunk the kernel uses: the config's, capped so that two buffers fit beside the decode table
@@ -50,7 +55,7 @@ static bool lds_path(const GemmPlan &plan)
 static int mid_x_chunk(const GemmPlan &plan)
 {
     int xc = plan.args.chunk_steps * kStepK;
-    const int ring = lds_path(plan) ? (plan.threads / 64) * plan.prefetch * 1024 : 0;
+    const int ring = lds_path(plan) ? (plan.threads / 64) * plan.prefetch * 1024 : 0;  // (twins without an LDS variant: a smaller chunk than they need, harmless)
     const int cap = (kLdsLimit - kLutBytes - ring) / (2 * plan.token_tiles * 32);  // k per buffer
     while (xc > cap) xc >>= 1;
     return xc;
@@ -91,9 +96,12 @@ bool mid_lds_applies(const GemmPlan &plan)
 {
     int xc;
     const MidVariant *v = mid_variant(plan, &xc);
-    if (!v || !v->fn_lds || !lds_path(plan) || (xc != 512 && xc != 1024)) return false;
-    const size_t x_lds = 2 * (size_t)32 * (size_t)xc, red_lds = 2 * (size_t)(plan.threads / 64) * 1024;
-    return x_lds >= red_lds && (size_t)kLutBytes + x_lds + (size_t)(plan.threads / 64) * plan.prefetch * 1024 <= (size_t)kLdsLimit;
+    if (!v || !v->fn_lds || !lds_path(plan)) return false;
+    // x pieces (one wave instruction per k-step and token tile) per wave and chunk: 1, 2 or 4
+    const int pieces = (xc / 32) * plan.token_tiles, waves = plan.threads / 64;
+    if (pieces % waves != 0 || (pieces / waves != 1 && pieces / waves != 2 && pieces / waves != 4)) return false;
+    const size_t x_lds = 2 * (size_t)plan.token_tiles * 32 * (size_t)xc, red_lds = 2 * (size_t)waves * 1024;
+    return x_lds >= red_lds && (size_t)kLutBytes + x_lds + (size_t)waves * plan.prefetch * 1024 <= (size_t)kLdsLimit;
 }
 
 bool mid_describe(const GemmPlan &plan, char *buf, size_t len)
@@ -102,7 +110,7 @@ bool mid_describe(const GemmPlan &plan, char *buf, size_t len)
     const MidVariant *v = mid_variant(plan, &xc);
     if (!v) return false;
     snprintf(buf, len, "gemm_mid_kernel<U=%d,TT=%d,XB=%d,%d threads%s> x_chunk=%d", v->u, v->tt, v->xb, v->maxt,
-             (lds_path(plan) && v->fn_lds) ? ",weights through LDS" : "", xc);
+             mid_lds_applies(plan) ? ",weights through LDS" : "", xc);
     return true;
 }
 
@@ -126,6 +134,9 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
             if (e == hipSuccess && v->fn_lds)
                 e = hipFuncSetAttribute(reinterpret_cast<const void *>(v->fn_lds), hipFuncAttributeMaxDynamicSharedMemorySize,
                                         kLdsLimit);
+            if (e == hipSuccess && v->fn_lds_shared)
+                e = hipFuncSetAttribute(reinterpret_cast<const void *>(v->fn_lds_shared), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        kLdsLimit);
             if (e != hipSuccess) return e;
             g_mid_attr_done[dev][vi] = 1;
         }
@@ -135,11 +146,10 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
     while ((1 << xc_log2) < xc) ++xc_log2;
     const size_t x_lds = 2 * (size_t)plan.token_tiles * 32 * (size_t)xc;   // two buffers of one chunk
     const size_t red_lds = 2 * (size_t)(plan.threads / 64) * 1024;         // two buffers of one plane per wave
-    const bool staged = lds_path(plan) && v->fn_lds;
+    const bool staged = mid_lds_applies(plan);
     const size_t lds = (size_t)kLutBytes + (staged ? x_lds + (size_t)(plan.threads / 64) * plan.prefetch * 1024
                                                    : (x_lds > red_lds ? x_lds : red_lds));
-    // (the twin counts on one or two x pieces per wave and chunk: chunks of 512 or 1024 k)
-    if (staged && (x_lds < red_lds || lds > (size_t)kLdsLimit || (xc != 512 && xc != 1024))) return hipErrorInvalidConfiguration;
+    if (plan.lds_weights && !staged) return hipErrorInvalidConfiguration;
     dim3 grid = plan.grid;
     grid.x = (unsigned)(a.row_tiles < cus ? a.row_tiles : cus);  // one workgroup per CU (LDS), walking row tiles
     // Several token chunks that do not all fit the device at once: rather than one round of row
@@ -166,7 +176,8 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
     const int packed = a.waves_m | a.epilogue << 5 | xc_log2 << 8 | a.wk_log2 << 13 | a.k_stagger << 16;
     // weights that sibling workgroups re-read stay in the caches longer without the nontemporal hint
     // (Mixtral gate+up, 1024 tokens: 1745 -> 1687 us)
-    const MidKernelFn fn = staged ? v->fn_lds : (chunks && v->fn_shared) ? v->fn_shared : v->fn;
+    const MidKernelFn fn = staged ? ((chunks && v->fn_lds_shared) ? v->fn_lds_shared : v->fn_lds)
+                                  : (chunks && v->fn_shared) ? v->fn_shared : v->fn;
     hipLaunchKernelGGL(fn, grid, dim3(plan.threads), lds, stream, a.q, a.x, a.code, a.absmax, a.k, a.n, a.m, packed, a.out,
                        a.residual, a.row_tiles, n_wg, chunks);
     return hipGetLastError();

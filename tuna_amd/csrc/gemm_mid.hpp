@@ -164,18 +164,22 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
         }                                                                                      \
     }
 
-    // LDSW: chunk `kbase` of x straight into `buf`: k-step wave + b*(waves of the workgroup) of the
-    // chunk, b < xdma_n (a uniform count of 1 or 2: the explicit waits below count on it); token rows
-    // past n are clamped (their output columns are never stored)
-    const int xdma_n = LDSW ? max(1, (xc >> 5) / (nthreads >> 6)) : 0;
-    const uint32_t xdma_lane = LDSW ? ((uint32_t)min(i16, a_n - 1 - tok0) * (uint32_t)a_k + (uint32_t)g * 8u) * 2u : 0u;
+    // LDSW: chunk `kbase` of x straight into `buf`, one wave instruction per k-step and token tile: piece
+    // i = wave + b*(waves of the workgroup), b < xdma_n (a uniform count of 1, 2 or 4: the explicit waits
+    // below count on it), is k-step i / TT, token tile i % TT, and lands at buf + i KB; lane (token i16,
+    // 8-k group g) fetches its own B-fragment piece.  Token rows past n are clamped (their output
+    // columns are never stored).
+    const int xdma_n = LDSW ? max(1, ((xc >> 5) * TT) / (nthreads >> 6)) : 0;
 #define TUNA_MID_X_DMA(buf, kbase, rot_steps)                                                   \
     {                                                                                          \
-        for (int b = 0; b < xdma_n; ++b) {                                                     \
-            const int ks_ = min(wave + b * (nthreads >> 6), (xc >> 5) - 1);                    \
+        _Pragma("unroll 1") for (int b = 0; b < xdma_n; ++b)                                  \
+        {                                                                                      \
+            const int i_ = min(wave + b * (nthreads >> 6), (xc >> 5) * TT - 1);                \
+            const int ks_ = i_ / TT, tt_ = i_ % TT;                                            \
             int s_ = ((kbase) >> 5) + ks_ + (rot_steps);                                       \
             if (s_ >= n_steps) s_ -= n_steps;                                                  \
-            load_weights_to_lds<false>(x_tile + (size_t)s_ * 64 + xdma_lane, (buf) + ks_ * 1024); \
+            const uint32_t lane_ = ((uint32_t)min(tt_ * 16 + i16, a_n - 1 - tok0) * (uint32_t)a_k + (uint32_t)g * 8u) * 2u; \
+            load_weights_to_lds<false>(x_tile + (size_t)s_ * 64 + lane_, (buf) + i_ * 1024);   \
         }                                                                                      \
     }
 
@@ -270,7 +274,9 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     const f16 *resp = reinterpret_cast<const f16 *>(a_residual);
     // B fragment of lane (token i16, k-group g), local step sl, token tile tt:
     // slot sl*4 + g, byte slot*(256*TT) + tt*256 + i16*16
-    const uint32_t xb_lane = (uint32_t)g * (256 * TT) + (uint32_t)i16 * 16 + (uint32_t)wk * (1024 * TT);
+    // (LDSW: a KB per k-step and token tile, lane l's piece at 16*l)
+    const uint32_t xb_lane = (LDSW ? (uint32_t)lane * 16 : (uint32_t)g * (256 * TT) + (uint32_t)i16 * 16) + (uint32_t)wk * (1024 * TT);
+    constexpr uint32_t xb_tile = LDSW ? 1024 : 256;  // bytes between the token tiles of a k-step
     const uint32_t wstep = (uint32_t)(1024 * TT) << wk_log2;  // LDS bytes between this wave's consecutive steps
 
     // One ring turn: U of this wave's k-steps, each consumed (B fragments from LDS, 4 fragments
@@ -284,13 +290,14 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
                 /* the slot's load has landed: U - 1 younger ring loads, in a chunk's first turn */ \
                 /* also the XB x pieces just requested, may stay in flight */                  \
                 if (!(first)) __builtin_amdgcn_s_waitcnt(wait_vmcnt(U - 1));                   \
+                else if (xdma_n == 4) __builtin_amdgcn_s_waitcnt(wait_vmcnt(U + 3));           \
                 else if (xdma_n == 2) __builtin_amdgcn_s_waitcnt(wait_vmcnt(U + 1));           \
                 else __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));                                \
                 wq[u] = *reinterpret_cast<const u32x4 *>(wring + u * 1024 + lane * 16);        \
             }                                                                                  \
             f16x8 b_[TT];                                                                      \
             _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) b_[tt] =                         \
-                *reinterpret_cast<const f16x8 *>(xb + (size_t)((sl) + u) * wstep + tt * 256);  \
+                *reinterpret_cast<const f16x8 *>(xb + (size_t)((sl) + u) * wstep + tt * xb_tile); \
             _Pragma("unroll") for (int j = 0; j < 4; ++j)                                      \
             {                                                                                  \
                 const f16x8 av_ = decode_dword<TUNA_DECODE_GEMM>(wq[u][j], lut, lane4, sc16[j], 0.f); \

@@ -149,47 +149,58 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
     if lds_bytes(c) > LDS_LIMIT:
         raise ValueError(f"needs {lds_bytes(c)} bytes of LDS (limit {LDS_LIMIT})")
     if c["lds_tile_rows"] == -1 and not mid_lds_applies(m, k, c):
-        raise ValueError("lds_tile_rows -1 needs an unsplit 16-wave launch with one token tile, prefetch 2 or 4 and "
-                         "x chunks of 512 or 1024 k that leave room for the weight rings")
+        raise ValueError("lds_tile_rows -1 needs an unsplit launch of 8 or 16 waves the streaming kernel takes, prefetch 2 or 4 "
+                         "(2 with eight token tiles) and x chunks that leave room for the weight rings")
+
+
+# (prefetch, token_tiles, x pieces per thread, max threads) of the streaming kernel's twins that stage the packed
+# weights through LDS; must match the fn_lds entries of kMid in csrc/gemm_mid.hip
+MID_LDS_VARIANTS = ({(u, 2, 4, 512) for u in (2, 4)} | {(u, 4, xb, 512) for u in (2, 4) for xb in (4, 8)}
+                    | {(2, 8, 4, 512), (2, 8, 8, 512), (2, 2, 4, 1024), (4, 2, 4, 1024), (2, 1, 4, 1024), (4, 1, 4, 1024)})
+
+
+def _mid_variant(m: int, k: int, c: dict, lds_path: bool):
+    """(variant key, x chunk) of the streaming kernel for a dense launch of this config, or None
+    (mirrors mid_variant and mid_x_chunk in csrc/gemm_mid.hip)."""
+    tt, wm, wk = c["token_tiles"], c["waves_m"], c["waves_k"]
+    if c["rows_per_wave"] != 64 or tt not in (1, 2, 4, 8) or c["split_k"] != 1 or not 0 <= c["k_stagger"] <= 4096:
+        return None
+    if k % STEP_K or k >= 1 << 23 or not _pow2(wk) or wm < 1 or wm * wk > 16 or m % (64 * wm):
+        return None
+    threads = 64 * wm * wk
+    ring = (threads // 64) * c["prefetch"] * 1024 if lds_path and threads in (512, 1024) and c["prefetch"] in (2, 4) else 0
+    xc = c["x_chunk"]
+    cap = (LDS_LIMIT - LUT_BYTES - ring) // (2 * tt * 32)
+    while xc > cap:
+        xc //= 2
+    if xc < wk * c["prefetch"] * STEP_K or k % xc:
+        return None
+    per_thread = -(-(tt * 2 * xc) // threads)
+    if per_thread > 8:
+        return None
+    key = (c["prefetch"], tt, 4 if per_thread <= 4 else 8, 512 if threads <= 512 else 1024)
+    return (key, xc) if key in MID_VARIANTS else None
 
 
 def mid_lds_applies(m: int, k: int, c: dict) -> bool:
     """True if the streaming kernel's twin with the packed weights staged through LDS takes a dense
     launch of this config (mirrors mid_lds_applies in csrc/gemm_mid.hip)."""
-    wm, wk, pf = c["waves_m"], c["waves_k"], c["prefetch"]
-    if c["rows_per_wave"] != 64 or c["token_tiles"] != 1 or c["split_k"] != 1 or wm * wk != 16 or pf not in (2, 4):
+    v = _mid_variant(m, k, c, True)
+    threads = 64 * c["waves_m"] * c["waves_k"]
+    if v is None or v[0] not in MID_LDS_VARIANTS or threads not in (512, 1024):
         return False
-    if k % STEP_K or k >= 1 << 23 or not _pow2(wk) or m % (64 * wm) or not 0 <= c["k_stagger"] <= 4096:
+    xc, tt, waves = v[1], c["token_tiles"], threads // 64
+    pieces = (xc // 32) * tt
+    if pieces % waves or pieces // waves not in (1, 2, 4):
         return False
-    ring = 16 * pf * 1024
-    xc = c["x_chunk"]
-    cap = (LDS_LIMIT - LUT_BYTES - ring) // (2 * 32)
-    while xc > cap:
-        xc //= 2
-    if xc not in (512, 1024) or xc < wk * pf * STEP_K or k % xc:
-        return False
-    return 2 * 32 * xc >= 2 * 16 * 1024 and LUT_BYTES + 2 * 32 * xc + ring <= LDS_LIMIT
+    x_lds, red_lds = 2 * tt * 32 * xc, 2 * waves * 1024
+    return x_lds >= red_lds and LUT_BYTES + x_lds + waves * c["prefetch"] * 1024 <= LDS_LIMIT
 
 
 def mid_applies(m: int, k: int, c: dict) -> bool:
     """True if a dense launch of this config is taken by the 17..128-token streaming kernel
     (mirrors mid_variant in csrc/gemm_mid.hip)."""
-    tt, wm, wk = c["token_tiles"], c["waves_m"], c["waves_k"]
-    if c["rows_per_wave"] != 64 or tt not in (1, 2, 4, 8) or c["split_k"] != 1 or not 0 <= c["k_stagger"] <= 4096:
-        return False
-    if k % STEP_K or k >= 1 << 23 or not _pow2(wk) or wm < 1 or wm * wk > 16 or m % (64 * wm):
-        return False
-    xc = c["x_chunk"]
-    cap = (LDS_LIMIT - LUT_BYTES) // (2 * tt * 32)
-    while xc > cap:
-        xc //= 2
-    if xc < wk * c["prefetch"] * STEP_K or k % xc:
-        return False
-    threads = 64 * wm * wk
-    per_thread = -(-(tt * 2 * xc) // threads)
-    if per_thread > 8:
-        return False
-    return (c["prefetch"], tt, 4 if per_thread <= 4 else 8, 512 if threads <= 512 else 1024) in MID_VARIANTS
+    return _mid_variant(m, k, c, c.get("lds_tile_rows", 0) == -1) is not None
 
 
 def lds_bytes(c: dict) -> int:

@@ -196,8 +196,11 @@ def mid_space(m: int, n_key: int, k: int):
                                 out.append(c)
                                 # the same launch with the packed weights staged through LDS, where that twin exists
                                 cl = dict(c, lds_tile_rows=-1)
-                                if make_configs.mid_lds_applies(m, k, cl):
+                                try:
+                                    make_configs.validate(m, n_key, k, cl)
                                     out.append(cl)
+                                except ValueError:
+                                    pass
     return out
 
 
