@@ -71,6 +71,10 @@ int tuna_selftest_quantizer_division(void *counts, void *stream);
  * rows (1, 2, 4, 8 or 16 of the workgroup's 16 waves; 0 = the library's choice) and ring depth
  * (2 or 4; 0 = the library's choice).  For A/B timing. */
 int tuna_set_multi_shape(int waves_m, int prefetch);
+/* Switch, process-wide: batches that run with a ring of 2 stage the packed weights and x through LDS
+ * (global -> LDS loads, as the LDS-staged twins of the streaming kernel do) instead of registers.
+ * Bit-identical results; for A/B timing.  Returns the previous setting. */
+int tuna_set_multi_weight_path(int through_lds);
 /* Diagnostic: the shortest run of problems tuna_matmul_multi hands to the batched kernel
  * (default 2; 1 sends single problems through it as well).  Returns the previous value. */
 int tuna_set_multi_min_batch(int count);

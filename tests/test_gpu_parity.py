@@ -1126,6 +1126,49 @@ def test_captured_graph_survives_growth_of_the_split_k_workspace():
 
 
 # ----------------------------------------------------------------------------- several GEMMs in one call
+@pytest.mark.parametrize("shapes", [
+    [(4096, 16, 4096), (6144, 16, 4096), (4096, 16, 14336), (1024, 5, 2048), (8192, 1, 8192)],   # row tiles of 256, k of 512 ... 14336
+    [(10240, 16, 8192), (8192, 16, 8192), (57344, 16, 8192), (8192, 16, 28672)],                   # a Llama-70B layer
+    [(128, 16, 1024), (640, 3, 512), (384, 16, 2560)],                                             # 128-row tiles, short k, ragged shares
+    [(8192, 16, 28672)],                                                                           # a batch of one
+])
+def test_matmul_multi_with_weights_through_lds_gives_the_register_paths_bits(shapes):
+    """The batched kernel's twin that stages packed weights and x through LDS (global -> LDS loads, x
+    chunks of 512 k) adds the same products in the same order: equal bits, on batches that exercise
+    whole and partial row tiles, segment switches across problems and the deferred hand-over."""
+    import torch
+
+    from tuna_amd import _lib
+
+    L = _lib.lib()
+    probs, host = _multi_problems(shapes, 900)
+    outs = {}
+    prev_min = L.tuna_set_multi_min_batch(1)
+    prev = L.tuna_set_multi_weight_path(0)
+    L.tuna_set_multi_shape(0, 2)              # the LDS twin exists for the ring of two
+    try:
+        from tuna_amd import ops
+        for lds in (0, 1):
+            L.tuna_set_multi_weight_path(lds)
+            for rep in range(2):
+                for p in probs:
+                    p[4].fill_(float("nan"))
+                before = L.tuna_multi_launches()
+                ops.matmul_multi(probs)
+                torch.cuda.synchronize()
+                assert L.tuna_multi_launches() == before + 1
+            outs[lds] = [p[4].clone() for p in probs]
+    finally:
+        L.tuna_set_multi_weight_path(prev)
+        L.tuna_set_multi_min_batch(prev_min)
+        L.tuna_set_multi_shape(0, 0)
+    for i, (a, b) in enumerate(zip(outs[0], outs[1])):
+        assert not torch.isnan(b.float()).any(), i
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16)), i
+    m, n, k = shapes[0]
+    assert _check_against_oracle(host[0], outs[1][0].cpu().numpy().view(np.uint16), m, n, k, seed=1) <= REL_TOL   # max relative error 1e-2
+
+
 def _multi_problems(shapes, seed0):
     import torch
 

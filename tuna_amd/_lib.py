@@ -103,6 +103,7 @@ SIGNATURES = {
     "tuna_multi_launches": (ctypes.c_ulonglong, []),
     "tuna_set_lean_kernels": (_i, [_i]),
     "tuna_set_weight_path": (_i, [_i]),
+    "tuna_set_multi_weight_path": (_i, [_i]),
     "tuna_lean_launches": (ctypes.c_ulonglong, []),
     "tuna_release_workspaces": (_i, []),
 }

@@ -675,6 +675,7 @@ static int check_ptr(const void *p, const char *name, size_t align)
 // launched problem by problem on the same stream.
 // ---------------------------------------------------------------------------------------
 static std::atomic<int> g_multi_waves_m{0}, g_multi_prefetch{0};  // 0: the library's choice (diagnostic override)
+static std::atomic<int> g_multi_lds{0};  // batches with a ring of 2 stage weights and x through LDS (tuna_set_multi_weight_path)
 static std::atomic<unsigned long long> g_multi_launches{0};
 static std::atomic<int> g_multi_min_batch{2};  // batches shorter than this are launched problem by problem
 
@@ -691,18 +692,26 @@ static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, Mu
     if (count < 1 || count > kMaxMultiProblems || cus < 1) return false;
     if (!waves_m) waves_m = g_multi_waves_m.load(std::memory_order_relaxed);
     if (!prefetch) prefetch = g_multi_prefetch.load(std::memory_order_relaxed);
-    if (!prefetch) {
-        // deeper rings pay on long streams; short batches finish sooner with fewer bytes requested ahead
-        unsigned long long bytes = 0;
-        for (int i = 0; i < count; ++i) bytes += (unsigned long long)problems[i].m * (unsigned long long)problems[i].k / 2;
-        prefetch = bytes >= (200ull << 20) ? 4 : 2;
-    }
+    // (a ring of two: with every wait of the ring exact it streams as fast as a ring of four on the longest
+    // batches and faster on the others - fewer bytes requested ahead at a segment switch)
+    if (!prefetch) prefetch = 2;
     if (!multi_variant_exists(prefetch)) return false;
     if (!waves_m) {
         // 256-row tiles (4 x 4 waves) when every problem allows, else narrower tiles and more waves along k
         waves_m = 4;
         for (int i = 0; i < count; ++i)
             while (waves_m > 1 && problems[i].m % (64 * waves_m)) waves_m >>= 1;
+        // fewer 256-row tiles than workgroups: every tile would be shared by several workgroups and handed
+        // over through memory; 128-row tiles (2 x 8 waves) give a workgroup whole tiles more often
+        if (waves_m == 4) {
+            long long tiles = 0;
+            bool k_ok = true;
+            for (int i = 0; i < count; ++i) {
+                tiles += problems[i].m / 256;
+                k_ok = k_ok && problems[i].k % (kStepK * 8 * prefetch) == 0;
+            }
+            if (tiles < cus && k_ok) waves_m = 2;
+        }
     }
     if (waves_m != 1 && waves_m != 2 && waves_m != 4 && waves_m != 8 && waves_m != 16) return false;
     const int waves_k = 16 / waves_m;
@@ -746,7 +755,10 @@ static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, Mu
     a.wk_log2 = log2i(waves_k);
     a.n_wg = n_wg;
     a.swizzle = (n_wg % 8 == 0) ? 1 : 0;
-    plan->prefetch = prefetch;
+    // variant -2: ring of 2 with weights and x staged through LDS (x chunks of 512 k: every wave needs a whole
+    // number of ring turns per chunk, so at most 8 waves along k)
+    const bool lds = g_multi_lds.load(std::memory_order_relaxed) != 0 && prefetch == 2 && waves_k <= 8 && multi_variant_exists(-2);
+    plan->prefetch = lds ? -2 : prefetch;
     plan->ws_bytes = (size_t)n_wg * 2 * waves_m * 4096;
     plan->n_counters = (size_t)tiles;
     return true;
@@ -1536,6 +1548,8 @@ TUNA_EXPORT int tuna_set_multi_shape(int waves_m, int prefetch)
     g_multi_prefetch.store(prefetch);
     return TUNA_OK;
 }
+
+TUNA_EXPORT int tuna_set_multi_weight_path(int through_lds) { return g_multi_lds.exchange(through_lds ? 1 : 0); }
 
 TUNA_EXPORT int tuna_set_multi_min_batch(int count)
 {

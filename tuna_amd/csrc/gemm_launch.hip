@@ -1,7 +1,6 @@
 // Instantiations of the GEMM kernel and the variant dispatcher.
 #include <atomic>
 #include <cstdio>
-#include <mutex>
 
 #include "gemm_kernel.hpp"
 #include "gemm_lean.hpp"
@@ -137,10 +136,9 @@ static const LeanVariant *lean_applies(const GemmPlan &plan, int cus)
 }
 
 // Dynamic LDS above 64 KB needs a one-time opt-in per kernel and device.
-static std::mutex g_attr_mutex;
-static unsigned char g_attr_done[16][kNumVariants];
-static unsigned char g_lean_attr_done[16][kNumLean];
-static int g_cu_count[16];
+static OptInFlag g_attr_done[16][kNumVariants];
+static OptInFlag g_lean_attr_done[16][kNumLean];
+static std::atomic<int> g_cu_count[16];
 
 hipError_t device_cus(int *dev_out, int *cus_out)
 {
@@ -148,15 +146,15 @@ hipError_t device_cus(int *dev_out, int *cus_out)
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
-    std::lock_guard<std::mutex> lock(g_attr_mutex);
-    if (!g_cu_count[dev]) {
-        int n = 0;
+    int n = g_cu_count[dev].load(std::memory_order_relaxed);
+    if (!n) {
         e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
         if (e != hipSuccess) return e;
-        g_cu_count[dev] = n > 0 ? n : 256;
+        if (n <= 0) n = 256;
+        g_cu_count[dev].store(n, std::memory_order_relaxed);
     }
     *dev_out = dev;
-    *cus_out = g_cu_count[dev];
+    *cus_out = n;
     return hipSuccess;
 }
 
@@ -177,15 +175,7 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
     if (!v) return hipErrorInvalidConfiguration;
     if (const LeanVariant *lv = lean_applies(plan, cus)) {
         const int li = (int)(lv - kLean);
-        {
-            std::lock_guard<std::mutex> lock(g_attr_mutex);
-            if (!g_lean_attr_done[dev][li]) {
-                e = hipFuncSetAttribute(reinterpret_cast<const void *>(lv->fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                        kLdsLimit);
-                if (e != hipSuccess) return e;
-                g_lean_attr_done[dev][li] = 1;
-            }
-        }
+        if ((e = ensure_lds_opt_in(g_lean_attr_done[dev][li], reinterpret_cast<const void *>(lv->fn))) != hipSuccess) return e;
         const GemmArgs &a = plan.args;
         const int swz = a.xcd_swizzle && plan.grid.x % 8 == 0;
         const int packed = a.split_log2 | a.waves_m << 4 | a.epilogue << 9 | swz << 11 | (int)(plan.grid.x >> 3) << 12;
@@ -205,15 +195,7 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
         if (v1) v = v1;
     }
     const int vi = (int)(v - kVariants);
-    {
-        std::lock_guard<std::mutex> lock(g_attr_mutex);
-        if (!g_attr_done[dev][vi]) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(v->fn),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
-            if (e != hipSuccess) return e;
-            g_attr_done[dev][vi] = 1;
-        }
-    }
+    if ((e = ensure_lds_opt_in(g_attr_done[dev][vi], reinterpret_cast<const void *>(v->fn))) != hipSuccess) return e;
     // persistent workgroups: as many as the device holds at once, each walks tiles with this stride
     dim3 grid = plan.grid;
     if (grid.x > slots) grid.x = slots;
@@ -268,7 +250,7 @@ static const NarrowVariant kNarrow[] = {
 #undef N
 #undef NT
 static constexpr int kNumNarrow = sizeof(kNarrow) / sizeof(kNarrow[0]);
-static unsigned char g_narrow_attr_done[16][kNumNarrow][2];
+static OptInFlag g_narrow_attr_done[16][kNumNarrow][2];
 
 static const NarrowVariant *find_narrow(int rows, int wk, int u, int tt)
 {
@@ -299,14 +281,7 @@ hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int
     const int vi = (int)(v - kNarrow);
     const int perm = args.n > 4;
     const NarrowKernelFn fn = perm ? v->fn_perm : v->fn;
-    {
-        std::lock_guard<std::mutex> lock(g_attr_mutex);
-        if (!g_narrow_attr_done[dev][vi][perm]) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
-            if (e != hipSuccess) return e;
-            g_narrow_attr_done[dev][vi][perm] = 1;
-        }
-    }
+    if ((e = ensure_lds_opt_in(g_narrow_attr_done[dev][vi][perm], reinterpret_cast<const void *>(fn))) != hipSuccess) return e;
     const size_t lds = (size_t)kLutBytes + (size_t)waves_k * (rows / 16) * token_tiles * 1024;
     const dim3 grid((unsigned)(args.m / rows), (unsigned)((args.n + 16 * token_tiles - 1) / (16 * token_tiles)), 1);
     hipLaunchKernelGGL(fn, grid, dim3(waves_k * 64), lds, stream, args.q, args.x, args.code, args.absmax, args.k, args.n,
@@ -325,15 +300,8 @@ hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, hipStrea
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
     const int perm = args.n > 4;
     const NarrowKernelFn fn = perm ? gemm_narrow_kernel<1, WK, U, true, 1, true> : gemm_narrow_kernel<1, WK, U, false, 1, true>;
-    static unsigned char done[16][2];
-    {
-        std::lock_guard<std::mutex> lock(g_attr_mutex);
-        if (!done[dev][perm]) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
-            if (e != hipSuccess) return e;
-            done[dev][perm] = 1;
-        }
-    }
+    static OptInFlag done[16][2];
+    if ((e = ensure_lds_opt_in(done[dev][perm], reinterpret_cast<const void *>(fn))) != hipSuccess) return e;
     const size_t lds = (size_t)kLutBytes + (size_t)WK * 1024;
     const dim3 grid((unsigned)(args.m / 16), (unsigned)((args.n + 15) / 16), 1);
     const int nblk = args.k >> (6 + blk_shift);

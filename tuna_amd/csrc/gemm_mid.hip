@@ -1,7 +1,6 @@
 // Instantiations and launcher of the 17..128-token streaming kernel (gemm_mid.hpp).
 #include <atomic>
 #include <cstdio>
-#include <mutex>
 
 #include "gemm_mid.hpp"
 
@@ -114,8 +113,8 @@ bool mid_describe(const GemmPlan &plan, char *buf, size_t len)
     return true;
 }
 
-static std::mutex g_mid_mutex;
-static unsigned char g_mid_attr_done[16][kNumMid];
+// (the opt-in to more than 64 KB of dynamic LDS, once per variant and device: see ensure_lds_opt_in)
+static OptInFlag g_mid_attr_done[16][kNumMid];
 
 hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t stream)
 {
@@ -123,23 +122,13 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
     const MidVariant *v = mid_variant(plan, &xc);
     if (!v) return hipErrorInvalidConfiguration;
     const int vi = (int)(v - kMid);
-    {
-        std::lock_guard<std::mutex> lock(g_mid_mutex);
-        if (!g_mid_attr_done[dev][vi]) {
-            hipError_t e =
-                hipFuncSetAttribute(reinterpret_cast<const void *>(v->fn), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
-            if (e == hipSuccess && v->fn_shared)
-                e = hipFuncSetAttribute(reinterpret_cast<const void *>(v->fn_shared), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                        kLdsLimit);
-            if (e == hipSuccess && v->fn_lds)
-                e = hipFuncSetAttribute(reinterpret_cast<const void *>(v->fn_lds), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                        kLdsLimit);
-            if (e == hipSuccess && v->fn_lds_shared)
-                e = hipFuncSetAttribute(reinterpret_cast<const void *>(v->fn_lds_shared), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                        kLdsLimit);
+    if (!g_mid_attr_done[dev][vi].load(std::memory_order_acquire)) {
+        for (const MidKernelFn f : {v->fn, v->fn_shared, v->fn_lds, v->fn_lds_shared}) {
+            if (!f) continue;
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(f), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
             if (e != hipSuccess) return e;
-            g_mid_attr_done[dev][vi] = 1;
         }
+        g_mid_attr_done[dev][vi].store(1, std::memory_order_release);
     }
     const GemmArgs &a = plan.args;
     int xc_log2 = 0;

@@ -23,10 +23,15 @@
 //     through the workspace (write-through stores, explicit wait, arrival ticket) and the last of
 //     the row tile's contributors to arrive adds them in k order: deterministic, no atomics on the
 //     output, counters return to zero (the scheme of gemm_kernel.hpp's balanced split).
+//   * LDSW variants (ring of 2): packed weights and x go global -> LDS with global_load_lds_dwordx4 as in
+//     the LDSW twins of gemm_mid.hpp (per-wave weight ring read back with ds_read_b128, x chunks of
+//     512 k straight into the chunk buffer, every wait for a load written out, bare barriers, stores
+//     into LDS the compiler does not look into).  Same arithmetic in the same order: same bits.
 // Requires, for every problem: n <= 16, m a multiple of 64*waves_m, k a multiple of
 // 32*waves_k*U, 16-byte aligned scales; the host falls back to separate launches otherwise.
 #pragma once
 #include "gemm_lean.hpp"
+#include "gemm_mid.hpp"
 
 namespace tuna {
 
@@ -60,18 +65,19 @@ struct MultiArgs {
     MultiProblem prob[kMaxMultiProblems];
 };
 
-template <int U, bool DEFER = true>
+template <int U, bool DEFER = true, bool LDSW = false>
 __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
 {
+    static_assert(!LDSW || U == 2, "LDS is full with a ring of two: table 64 KB, x 2 x 16 KB, rings 32 KB, reduction 32 KB");
     constexpr int XB = 2;                  // 16-byte x pieces per thread and chunk: 16 tokens x 1024 k x 2 B / 1024 threads
-    constexpr int kChunkSteps = 32;        // k-steps per x chunk
-    constexpr uint32_t kXBuf = 32 * 1024;  // bytes of one x buffer
+    constexpr int kChunkSteps = LDSW ? 16 : 32;                 // k-steps per x chunk (LDSW: one wave instruction per wave)
+    constexpr uint32_t kXBuf = (LDSW ? 16 : 32) * 1024;         // bytes of one x buffer
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char *lut = smem;
     unsigned char *xbuf = smem + kLutBytes;  // two x buffers
     // reduction area: two accumulator planes of all 16 waves (32 KB); its first two words double as the
     // arrival tickets of the hand-over, which are written only after every sum has been read
-    float *redf = reinterpret_cast<float *>(smem + kLutBytes + 2 * kXBuf);
+    float *redf = reinterpret_cast<float *>(smem + kLutBytes + 2 * kXBuf + (LDSW ? 16 * U * 1024 : 0));
     volatile unsigned *ticket = reinterpret_cast<volatile unsigned *>(redf);
 
     const int tid = threadIdx.x;
@@ -79,6 +85,8 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
     const int i16 = lane & 15;
     const int g = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // LDSW: behind the x buffers the waves' weight rings, U slots of 1 KB each
+    unsigned char *wring = smem + kLutBytes + 2 * kXBuf + wave * (U * 1024);
     const int wk_log2 = a.wk_log2;
     const int waves_k = 1 << wk_log2;
     const int wk = wave & (waves_k - 1);
@@ -172,14 +180,43 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         }                                                                                      \
     }
 
-    const float code_lane = a.code[i16];
+    // LDSW: chunk `c` straight into `buf`, k-step `wave` of the chunk per wave; lane (token i16, 8-k group g)
+    // fetches its own B-fragment piece (token rows past n: clamped, their output columns are never stored)
+#define TUNA_MULTI_X_DMA(x_, n_, k_, sb_, nsteps_, c, buf)                                       \
+    {                                                                                          \
+        const int p_ = min((c) * kChunkSteps + wave, (nsteps_) - 1);                           \
+        load_weights_to_lds<false>((x_) + (uint32_t)min(i16, (n_) - 1) * ((uint32_t)(k_) * 2u) + (uint32_t)(((sb_) + p_) * 32 + g * 8) * 2u, \
+                                   (buf) + wave * 1024);                                       \
+    }
+
+    float code_lane;
+    if constexpr (LDSW) {
+        // through the scalar cache (see gemm_mid.hpp: no vector load into a register while global -> LDS loads fly)
+        const float *__restrict__ code_ptr = a.code;
+        float cs[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) cs[j] = code_ptr[j];
+        code_lane = 0.f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) code_lane = i16 == j ? cs[j] : code_lane;
+    } else {
+        code_lane = a.code[i16];
+    }
     Seg cur = seg_at(t_begin);
     uint32_t lb = lane_base(cur);
     // x and the scales first: vector loads return in order, and the first barrier then waits for the x
     // pieces only while the first ring turn stays in flight across it
-    TUNA_MULTI_X_LOAD(cur.x, cur.n, cur.k, cur.sb, cur.nsteps, 0)
-    sc32 = *reinterpret_cast<const f32x4 *>(cur.absmax + cur.row0 + wm * 64 + i16 * 4);
-    {
+    if constexpr (LDSW) {
+        TUNA_MULTI_X_DMA(cur.x, cur.n, cur.k, cur.sb, cur.nsteps, 0, xbuf)
+        // the first segment's scales into this wave's KB of x buffer 1, free until chunk 1 is requested
+        load_weights_to_lds<false>(reinterpret_cast<const unsigned char *>(cur.absmax + cur.row0 + wm * 64 + i16 * 4),
+                                   xbuf + kXBuf + wave * 1024);
+        const unsigned char *qp = cur.q + (size_t)(cur.sb + wk) * 128;
+#pragma unroll
+        for (int u = 0; u < U; ++u) load_weights_to_lds<true>(qp + (size_t)u * wq_stride + lb, wring + u * 1024);
+    } else {
+        TUNA_MULTI_X_LOAD(cur.x, cur.n, cur.k, cur.sb, cur.nsteps, 0)
+        sc32 = *reinterpret_cast<const f32x4 *>(cur.absmax + cur.row0 + wm * 64 + i16 * 4);
         const unsigned char *qp = cur.q + (size_t)(cur.sb + wk) * 128;
 #pragma unroll
         for (int u = 0; u < U; ++u) wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(qp + (size_t)u * wq_stride + lb));
@@ -198,15 +235,25 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
                 v[b] = hi | (lo << 16);
             }
 #pragma unroll
-            for (int b = 0; b < 4; ++b) reinterpret_cast<u32x4 *>(lut)[p0 + b * 1024] = u32x4{v[b], v[b], v[b], v[b]};
+            for (int b = 0; b < 4; ++b) {
+                if constexpr (LDSW) lds_store16_opaque(lut + (size_t)(p0 + b * 1024) * 16, u32x4{v[b], v[b], v[b], v[b]});
+                else reinterpret_cast<u32x4 *>(lut)[p0 + b * 1024] = u32x4{v[b], v[b], v[b], v[b]};
+            }
         }
     }
     // chunk 0 of the first segment into buffer 0; one barrier publishes it and the table
-    TUNA_MULTI_X_STORE(cur.n, xbuf)
-    __syncthreads();
+    if constexpr (LDSW) {
+        __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));  // chunk 0 and the scales are older than the ring's U loads
+        sc32 = *reinterpret_cast<const f32x4 *>(xbuf + kXBuf + wave * 1024 + lane * 16);
+        barrier_lds_only();
+    } else {
+        TUNA_MULTI_X_STORE(cur.n, xbuf)
+        __syncthreads();
+    }
     uint32_t xsel = 0;  // buffer that holds the chunk about to be consumed
 
-    const uint32_t xb_lane = (uint32_t)g * 256u + (uint32_t)i16 * 16u + (uint32_t)wk * 1024u;
+    // (LDSW: a KB per k-step, lane l's piece at 16*l)
+    const uint32_t xb_lane = (LDSW ? (uint32_t)lane * 16u : (uint32_t)g * 256u + (uint32_t)i16 * 16u) + (uint32_t)wk * 1024u;
     const uint32_t wstep = 1024u << wk_log2;  // LDS bytes between this wave's consecutive k-steps
     const size_t seg_floats = (size_t)a.waves_m * 1024;
     const size_t plane_floats = (size_t)16 * 256;  // one accumulator plane of all 16 waves
@@ -278,7 +325,7 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         const f32x4 sc_next = *reinterpret_cast<const f32x4 *>(nxt.absmax + nxt.row0 + wm * 64 + i16 * 4);
         // One ring turn: U of this wave's k-steps consumed and refilled; the refills of the segment's
         // last turn are the first steps of the next segment.
-#define TUNA_MULTI_TURN(sl)                                                                     \
+#define TUNA_MULTI_TURN(sl, first)                                                              \
     {                                                                                          \
         if (it + U >= n_it) {                                                                  \
             rp = rp_last;                                                                      \
@@ -286,13 +333,26 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         }                                                                                      \
         _Pragma("unroll") for (int u = 0; u < U; ++u)                                          \
         {                                                                                      \
+            if constexpr (LDSW) {                                                              \
+                /* the slot's load has landed: U - 1 younger ring loads and, in a chunk's first */ \
+                /* turn, the x piece just requested (and the next segment's scales) may fly on */ \
+                if (!(first)) __builtin_amdgcn_s_waitcnt(wait_vmcnt(U - 1));                   \
+                else if (c == 0) __builtin_amdgcn_s_waitcnt(wait_vmcnt(U + 1));                \
+                else __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));                                \
+                wq[u] = *reinterpret_cast<const u32x4 *>(wring + u * 1024 + lane * 16);        \
+            }                                                                                  \
             const f16x8 b_ = *reinterpret_cast<const f16x8 *>(xb + (size_t)((sl) + u) * wstep); \
             _Pragma("unroll") for (int j = 0; j < 4; ++j)                                      \
             {                                                                                  \
                 const f16x8 av_ = decode_dword<TUNA_DECODE_GEMM>(wq[u][j], lut, lane4, sc16[j], 0.f); \
                 acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av_, b_, acc[j], 0, 0, 0);     \
             }                                                                                  \
-            wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(rp + (size_t)u * wq_stride + rlb)); \
+            if constexpr (LDSW) {                                                              \
+                __builtin_amdgcn_sched_barrier(0); /* behind the MFMAs that used the slot's bytes */ \
+                load_weights_to_lds<true>(rp + (size_t)u * wq_stride + rlb, wring + u * 1024); \
+            } else {                                                                           \
+                wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(rp + (size_t)u * wq_stride + rlb)); \
+            }                                                                                  \
             __builtin_amdgcn_sched_barrier(0); /* keep each refill right behind its consume */ \
         }                                                                                      \
         rp += (size_t)U * wq_stride;                                                           \
@@ -308,20 +368,29 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
                 const unsigned char *x_ = more ? cur.x : nxt.x;
                 const int xn_ = more ? cur.n : nxt.n, xk_ = more ? cur.k : nxt.k, xsb_ = more ? cur.sb : nxt.sb;
                 const int xns_ = more ? cur.nsteps : nxt.nsteps, xc_ = more ? c + 1 : (has_next ? 0 : c);
-                TUNA_MULTI_X_LOAD(x_, xn_, xk_, xsb_, xns_, xc_)
+                if constexpr (LDSW) {
+                    // (the other buffer was last read in the previous chunk, which ended with a barrier)
+                    TUNA_MULTI_X_DMA(x_, xn_, xk_, xsb_, xns_, xc_, xbuf + (xsel ^ 1u) * kXBuf)
+                } else {
+                    TUNA_MULTI_X_LOAD(x_, xn_, xk_, xsb_, xns_, xc_)
+                }
             }
             const unsigned char *xb = xbuf + xsel * kXBuf + xb_lane;
             const int its = min(chunk_its, n_it - it);
             // (the first ring turn of a chunk is a copy of its own: there the x pieces just requested
             // are in flight behind the ring, and only straight-line code lets the compiler count them
             // into its waits)
-            TUNA_MULTI_TURN(0)
-            for (int sl = U; sl < its; sl += U) TUNA_MULTI_TURN(sl)
+            TUNA_MULTI_TURN(0, true)
+            for (int sl = U; sl < its; sl += U) TUNA_MULTI_TURN(sl, false)
             // the other buffer was last read in the previous chunk, which ended with a barrier;
             // exactly the last ring turn's U refills are younger than the x pieces
             __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));
-            TUNA_MULTI_X_STORE(more ? cur.n : nxt.n, xbuf + (xsel ^ 1u) * kXBuf)
-            __syncthreads();
+            if constexpr (LDSW) {
+                barrier_lds_only();
+            } else {
+                TUNA_MULTI_X_STORE(more ? cur.n : nxt.n, xbuf + (xsel ^ 1u) * kXBuf)
+                __syncthreads();
+            }
             xsel ^= 1u;
         }
 #undef TUNA_MULTI_TURN
@@ -333,11 +402,18 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         float o[4][4];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            if (h) __syncthreads();  // the first half's sums have been read
+            if (h) {  // the first half's sums have been read
+                if constexpr (LDSW) barrier_lds_only();
+                else __syncthreads();
+            }
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                reinterpret_cast<f32x4 *>(redf + j * plane_floats)[(size_t)wave * 64 + lane] = acc[2 * h + j];
-            __syncthreads();
+            for (int j = 0; j < 2; ++j) {
+                float *dst = redf + j * plane_floats + ((size_t)wave * 64 + lane) * 4;
+                if constexpr (LDSW) lds_store16_opaque(reinterpret_cast<unsigned char *>(dst), __builtin_bit_cast(u32x4, acc[2 * h + j]));
+                else *reinterpret_cast<f32x4 *>(dst) = acc[2 * h + j];
+            }
+            if constexpr (LDSW) barrier_lds_only();
+            else __syncthreads();
             sum_planes_any<2, 32>(wk_log2, redf, plane_floats, wm, wk, lane, o, 2 * h);
         }
         const bool partial = cur.part >= 0;
@@ -401,6 +477,7 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         }
     }
 #undef TUNA_MULTI_X_LOAD
+#undef TUNA_MULTI_X_DMA
 #undef TUNA_MULTI_X_STORE
 }
 

@@ -352,7 +352,7 @@ bool tiled_variant_exists(int bm, int bn, bool mfma32)
 
 size_t tiled_lds_bytes(int bm, int bn) { return (size_t)kLutBytes + 2 * (size_t)(bm + bn) * 128; }  // two tile buffers
 
-static unsigned char g_tiled_attr[16][kNumTiled][2];
+static OptInFlag g_tiled_attr[16][kNumTiled][2];
 
 hipError_t launch_gemm_tiled(const TiledArgs &args, int bm, int bn, bool mfma32, hipStream_t stream)
 {
@@ -366,11 +366,7 @@ hipError_t launch_gemm_tiled(const TiledArgs &args, int bm, int bn, bool mfma32,
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
-    if (!g_tiled_attr[dev][vi][mfma32]) {  // dynamic LDS above 64 KB needs a one-time opt-in per kernel and device
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
-        if (e != hipSuccess) return e;
-        g_tiled_attr[dev][vi][mfma32] = 1;
-    }
+    if ((e = ensure_lds_opt_in(g_tiled_attr[dev][vi][mfma32], reinterpret_cast<const void *>(fn))) != hipSuccess) return e;
     TiledArgs a = args;
     a.row_tiles = ceil_div_i(args.m, bm);
     a.tok_tiles = ceil_div_i(args.n, bn);

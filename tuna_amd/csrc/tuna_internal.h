@@ -4,6 +4,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/tuna_amd.h"
 #include "../../include/tuna_amd_bench.h"
 
@@ -15,6 +17,18 @@ namespace tuna {
 // its own bank column, whatever the data.
 constexpr int kLutBytes = 256 * 64 * 4;
 constexpr int kLdsLimit = 160 * 1024;
+
+// Dynamic LDS above 64 KB needs a one-time opt-in per kernel and device.  `done` is read without a
+// lock on every launch; the attribute call is idempotent, so threads racing on a kernel's first
+// launch may both make it.
+typedef std::atomic<unsigned char> OptInFlag;
+inline hipError_t ensure_lds_opt_in(OptInFlag &done, const void *kernel)
+{
+    if (done.load(std::memory_order_acquire)) return hipSuccess;
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
+    if (e == hipSuccess) done.store(1, std::memory_order_release);
+    return e;
+}
 constexpr int kStepK = 32;          // k per MFMA step (v_mfma_f32_16x16x32_f16)
 constexpr int kRowsPerLoad = 64;    // weight rows covered by one 128-bit load per lane
 constexpr int kMaxThreads = 1024;
