@@ -74,9 +74,11 @@ def n_sets_for(bytes_per_set: int, cap_bytes: int) -> int:
     return max(2, min(n, max(2, cap_bytes // bytes_per_set)))
 
 
-def time_shape(ops, synth, torch, dev, m, n, k, steps, warmup, seed0=0, use_graph=False, cfg=None, sets=None, settle=0):
+def time_shape(ops, synth, torch, dev, m, n, k, steps, warmup, seed0=0, use_graph=False, cfg=None, sets=None, settle=0,
+               settle_ms=0.0):
     """-> dict with us_per_gemm, GB/s, TFLOP/s, roofline fraction for one shape.  `settle` untimed
-    launches run before the warm-up (clocks and caches of a box that has just been idle)."""
+    launches run before the warm-up (clocks and caches of a box that has just been idle); `settle_ms`
+    asks for that many milliseconds of them instead (the count comes from a five-launch estimate)."""
     bytes_w = m * k // 2
     if sets is None:
         ns = n_sets_for(bytes_w, 24 << 30)
@@ -89,6 +91,9 @@ def time_shape(ops, synth, torch, dev, m, n, k, steps, warmup, seed0=0, use_grap
     code = nf4_codebook(dev)
     out = torch.empty((n, m), dtype=torch.float16, device=dev)
     torch.cuda.synchronize()
+    if settle_ms > 0:
+        est = ops.time_matmul(qs, ams, x, code, out, m, n, k, config=cfg, warmup=1, iters=5, use_graph=False) / 5.0
+        settle = max(settle, min(20000, int(settle_ms / max(est, 1e-4)) + 1))
     if settle > 0:
         ops.time_matmul(qs, ams, x, code, out, m, n, k, config=cfg, warmup=0, iters=settle, use_graph=False)
     ms = ops.time_matmul(qs, ams, x, code, out, m, n, k, config=cfg, warmup=warmup, iters=steps, use_graph=use_graph)
@@ -422,7 +427,7 @@ def main():
         shapes = {}
         steps = max(50, min(args.steps, 300))
         for name, (sm, sk) in synth.SHAPES.items():
-            r_s = time_shape(ops, synth, torch, dev, sm, n, sk, steps, max(10, args.warmup // 5), seed0=1000)
+            r_s = time_shape(ops, synth, torch, dev, sm, n, sk, steps, max(10, args.warmup // 5), seed0=1000, settle_ms=10.0)
             r_g = time_shape(ops, synth, torch, dev, sm, n, sk, steps, max(10, args.warmup // 5), seed0=1000,
                              use_graph=True)
             best = r_g if r_g["us_per_gemm"] < r_s["us_per_gemm"] else r_s
@@ -507,7 +512,7 @@ def main():
             row = {}
             for nm in names:
                 sm, sk = synth.SHAPES[nm]
-                r = time_shape(ops, synth, torch, dev, sm, nt, sk, 100, 20, seed0=2000, use_graph=True)
+                r = time_shape(ops, synth, torch, dev, sm, nt, sk, 100, 20, seed0=2000, use_graph=True, settle_ms=25.0)
                 row[nm] = {"us": r["us_per_gemm"], "gbs": r["gbs"], "tflops": r["tflops"]}
                 torch.cuda.empty_cache()
             tok[str(nt)] = row

@@ -286,7 +286,7 @@ class Evaluator:
         return self.cache[key]
 
 
-def tune_shape(m, n, k, generations=6, population=24, seed=0, log=print, max_seed_evals=120, iters=60):
+def tune_shape(m, n, k, generations=6, population=24, seed=0, log=print, max_seed_evals=120, iters=60, extra=()):
     rng = random.Random(seed * 7919 + m * 31 + k)
     n_key = make_configs.bucket_of(n)
     ev = Evaluator(m, n, k, iters=iters, warmup=max(2, iters // 6))
@@ -299,6 +299,9 @@ def tune_shape(m, n, k, generations=6, population=24, seed=0, log=print, max_see
     pool = seeds(m, n_key, k)
     rng.shuffle(pool)
     pool = pool[:max_seed_evals] + lean_space(m, n_key, k) + mid_space(m, n_key, k)
+    # the winners of the other token buckets of this (m, k), where they are valid here: a config tuned
+    # for 16 tokens also runs one token, and is sometimes what the bucket should have
+    pool += [c for c in (repair(dict(e), m, n_key, k) for e in extra) if c is not None]
     for c in narrow_space(m, n_key, k):     # a kernel family of its own: timed, not bred
         ev(c)
     scored = sorted(((ev(c), json.dumps(c, sort_keys=True)) for c in pool))
@@ -385,9 +388,11 @@ def main(argv=None):
         for n in tokens:
             t0 = time.time()
             print(f"tuning {name} m={m} n={n} k={k}", flush=True)
+            others = [{f: e.get(f, 0) for f in make_configs.FIELDS} for key_, e in param_map.items()
+                      if key_.split("_")[0] == str(m) and key_.split("_")[2] == str(k)]
             best, us = tune_shape(m, n, k, args.generations, args.population, args.seed,
                                   log=lambda s: print(s, flush=True), max_seed_evals=args.max_seed_evals,
-                                  iters=args.iters)
+                                  iters=args.iters, extra=others)
             key = f"{m}_{make_configs.bucket_of(n)}_{k}"
             old = param_map.get(key)
             if old is not None and args.replace_margin > 0:
