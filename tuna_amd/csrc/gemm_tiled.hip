@@ -43,6 +43,7 @@ constexpr int kTiledThreads = 512;
 constexpr int kTiledStepK = 64;
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t tiled_u32x2 __attribute__((ext_vector_type(2)));
 
 template <int WM, int TM, int WN, int TN, int NSETS, bool M32 = false>
 __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const TiledArgs a)
@@ -51,9 +52,12 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     static_assert(!M32 || (TM % 2 == 0 && TN % 2 == 0), "32 x 32 MFMA tiles pair up the 16 x 16 ones");
     constexpr int BM = WM * TM * 16;
     constexpr int BN = WN * TN * 16;
-    constexpr int A_PIECES = BM * 2;                 // 16-byte packed pieces per k-step
-    constexpr int X_PER_THREAD = BN * 8 / kTiledThreads;  // 16-byte activation pieces per thread per k-step
-    static_assert(A_PIECES <= kTiledThreads && X_PER_THREAD >= 1, "tile shape");
+    constexpr int DW = BM / 64;            // packed dwords (weight rows of one 8-k block) a thread decodes per k-step
+    constexpr int P = 8 / DW;              // threads per 32-byte block of the packed layout
+    constexpr int L = 4 * DW;              // table lookups (byte pairs) per thread and k-step
+    constexpr int X_PER_THREAD = BN / 64;  // 16-byte activation pieces per thread per k-step
+    static_assert(DW == 1 || DW == 2 || DW == 4, "64, 128 or 256 weight rows per workgroup");
+    static_assert(X_PER_THREAD >= 1, "tile shape");
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char *lut = smem;                       // byte-pair table at LDS address 0
     constexpr int BUF = (BM + BN) * 128;             // one buffer: weight tile [BM][128 B] + activation tile [BN][128 B]
@@ -88,16 +92,16 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     const f16 *xg = reinterpret_cast<const f16 *>(a.x);
 
     // ---- this thread's share of the loads ------------------------------------------------
-    // weights: piece tid = block row (tid / 16) of the tile, k-block (tid % 16) / 2 of the step,
-    // half tid % 2 (rows 4*half .. +3 of the block row)
-    const bool a_loader = tid < A_PIECES;
-    const int a_mbl = tid >> 4, a_kb = (tid & 15) >> 1, a_half = tid & 1;
+    // weights: every thread takes DW consecutive rows of one 8 x 8 block per k-step - block row
+    // tid / (8 P) of the tile, k-block (tid / P) % 8 of the step, rows DW * (tid % P) .. of the block:
+    // a wave's load covers whole 32-byte blocks, 8 P consecutive threads 256 contiguous bytes
+    const int a_piece = tid % P, a_kb = (tid / P) & 7, a_mbl = tid / (8 * P);
     const int a_mb = min((row_base >> 3) + a_mbl, mb_last);
-    const unsigned char *a_src = a.q + (size_t)a_mb * kb_total * 32 + a_half * 16;
-    const int a_row = a_mbl * 8 + a_half * 4;        // first of the 4 tile rows this thread decodes
-    f16x2 sc16[4];
+    const unsigned char *a_src = a.q + (size_t)a_mb * kb_total * 32 + a_piece * (4 * DW);
+    const int a_row = a_mbl * 8 + a_piece * DW;      // first of the DW tile rows this thread decodes
+    f16x2 sc16[DW];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < DW; ++j) {
         const f16 h = (f16)a.absmax[min(row_base + a_row + j, a.m - 1)];
         sc16[j] = f16x2{h, h};
     }
@@ -115,24 +119,41 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     // NSETS register sets: steps s .. s+NSETS-1 in flight (4; 8 for the 64-token tiles, whose steps
     // are short against the HBM latency)
     static_assert(NSETS == 4 || NSETS == 8, "register sets");
-    u32x4 wq[NSETS];
-    u32x4 xr[NSETS][X_PER_THREAD];
+    // (256-token tiles keep two sets of activations: four would not leave room for both halves' fragments, and
+    // activations come from the L2, not from HBM)
+    constexpr int XSETS = X_PER_THREAD == 4 ? 2 : NSETS;
+    uint32_t wq[NSETS][DW];
+    u32x4 xr[XSETS][X_PER_THREAD];
     // Unconditional, clamped loads (exact s_waitcnt counts); what lies beyond k is zeroed in x.
 #define TUNA_TILED_LOAD(set, s)                                                                 \
     {                                                                                          \
         const int kb_ = min((s) * 8 + a_kb, kb_total - 1);                                     \
-        wq[set] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(a_src + (size_t)kb_ * 32)); \
-        _Pragma("unroll") for (int i = 0; i < X_PER_THREAD; ++i)                               \
-        {                                                                                      \
-            const int kk_ = min((s) * kTiledStepK, a.k - 8 - ((tid + i * kTiledThreads) & 7) * 8); \
-            xr[set][i] = *reinterpret_cast<const u32x4 *>(x_src[i] + kk_);                     \
+        const unsigned char *p_ = a_src + (size_t)kb_ * 32;                                    \
+        if constexpr (DW == 4) {                                                               \
+            const u32x4 w_ = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p_));  \
+            _Pragma("unroll") for (int j = 0; j < 4; ++j) wq[set][j] = w_[j];                  \
+        } else if constexpr (DW == 2) {                                                        \
+            const tiled_u32x2 w_ = __builtin_nontemporal_load(reinterpret_cast<const tiled_u32x2 *>(p_)); \
+            wq[set][0] = w_[0];                                                                \
+            wq[set][DW - 1] = w_[1];                                                           \
+        } else {                                                                               \
+            wq[set][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(p_));   \
         }                                                                                      \
+    }
+#define TUNA_TILED_LOAD_X(set, s)                                                               \
+    _Pragma("unroll") for (int i = 0; i < X_PER_THREAD; ++i)                                   \
+    {                                                                                          \
+        const int kk_ = min((s) * kTiledStepK, a.k - 8 - ((tid + i * kTiledThreads) & 7) * 8); \
+        xr[set][i] = *reinterpret_cast<const u32x4 *>(x_src[i] + kk_);                         \
     }
 
     const int s0 = blockIdx.z * a.steps_per_split;
     const int s1 = min(a.steps_total, s0 + a.steps_per_split);
 #pragma unroll
-    for (int u = 0; u < NSETS; ++u) TUNA_TILED_LOAD(u, min(s0 + u, a.steps_total - 1))
+    for (int u = 0; u < NSETS; ++u) {
+        TUNA_TILED_LOAD(u, min(s0 + u, a.steps_total - 1))
+        if (u < XSETS) TUNA_TILED_LOAD_X(u, min(s0 + u, a.steps_total - 1))
+    }
 
     // ---- decode table (as in the streaming kernel) ------------------------------------------
     {
@@ -174,91 +195,150 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     const unsigned char *x_frag = x_tile + (wn_i * TN * 16 + (M32 ? i32 : i16)) * 128;
     const int sw = (M32 ? i32 : i16) & 7;
 
-    // Stage k-step s from register set `set` into tile buffer `buf`: decode the packed weights,
-    // copy the activations (zero beyond n and k), then refill the set four steps ahead.
-#define TUNA_TILED_STAGE(set, buf, s)                                                            \
-    {                                                                                          \
-        unsigned char *at_ = a_tile + (buf) * BUF, *xt_ = x_tile + (buf) * BUF;                \
-        if (a_loader) {                                                                        \
-            _Pragma("unroll") for (int j = 0; j < 4; ++j)                                      \
-            {                                                                                  \
-                const uint32_t d_ = wq[set][j];                                                \
-                const uint32_t t0_ = *reinterpret_cast<const lds_u32 *>((uintptr_t)__builtin_amdgcn_perm(d_, lane4, 0x0c0c0400u)); \
-                const uint32_t t1_ = *reinterpret_cast<const lds_u32 *>((uintptr_t)__builtin_amdgcn_perm(d_, lane4, 0x0c0c0500u)); \
-                const uint32_t t2_ = *reinterpret_cast<const lds_u32 *>((uintptr_t)__builtin_amdgcn_perm(d_, lane4, 0x0c0c0600u)); \
-                const uint32_t t3_ = *reinterpret_cast<const lds_u32 *>((uintptr_t)__builtin_amdgcn_perm(d_, lane4, 0x0c0c0700u)); \
-                const f16x2 h0_ = __builtin_bit_cast(f16x2, t0_) * sc16[j], h1_ = __builtin_bit_cast(f16x2, t1_) * sc16[j]; \
-                const f16x2 h2_ = __builtin_bit_cast(f16x2, t2_) * sc16[j], h3_ = __builtin_bit_cast(f16x2, t3_) * sc16[j]; \
-                const f16x8 w_ = {h0_[0], h0_[1], h1_[0], h1_[1], h2_[0], h2_[1], h3_[0], h3_[1]}; \
-                const int r_ = a_row + j;                                                      \
-                *reinterpret_cast<f16x8 *>(at_ + r_ * 128 + ((a_kb ^ (r_ & 7)) << 4)) = w_;    \
-            }                                                                                  \
-        }                                                                                      \
-        _Pragma("unroll") for (int i = 0; i < X_PER_THREAD; ++i)                               \
-        {                                                                                      \
-            const int p_ = tid + i * kTiledThreads;                                            \
-            const int t_ = p_ >> 3, sl_ = p_ & 7;                                              \
-            const bool ok_ = x_tok_ok[i] && ((s) * kTiledStepK + sl_ * 8 < a.k);               \
-            *reinterpret_cast<u32x4 *>(xt_ + t_ * 128 + ((sl_ ^ (t_ & 7)) << 4)) = ok_ ? xr[set][i] : u32x4{0u, 0u, 0u, 0u}; \
-        }                                                                                      \
-        TUNA_TILED_LOAD(set, min((s) + NSETS, a.steps_total - 1))                              \
-    }
-    // The matrix work of one k-step from tile buffer `buf`.
-#define TUNA_TILED_MFMA(buf)                                                                     \
+    // ---- the pieces of one k-step --------------------------------------------------------------
+    // A k-step of 64 is two halves of 32 k.  Fragments of half h of a step, TM of the weight tile and TN
+    // of the activation tile (32 x 32 tiles: two k-quarters of TM/2 and TN/2):
+    f16x8 fa[2][TM], fb[2][TN];
+#define TUNA_TILED_READ(h, buf)                                                                  \
     {                                                                                          \
         if constexpr (M32) {                                                                   \
-            _Pragma("unroll") for (int kq = 0; kq < 4; ++kq)                                   \
+            _Pragma("unroll") for (int kk = 0; kk < 2; ++kk)                                   \
             {                                                                                  \
-                const int slot_ = (((kq * 2 + h32) ^ sw) << 4) + (buf) * BUF;                  \
-                f16x8 bf_[TN2];                                                                \
+                const int slot_ = (((((h) * 2 + kk) * 2 + h32) ^ sw) << 4) + (buf) * BUF;      \
                 _Pragma("unroll") for (int tn = 0; tn < TN2; ++tn)                             \
-                    bf_[tn] = *reinterpret_cast<const f16x8 *>(x_frag + tn * (32 * 128) + slot_); \
+                    fb[h][kk * TN2 + tn] = *reinterpret_cast<const f16x8 *>(x_frag + tn * (32 * 128) + slot_); \
                 _Pragma("unroll") for (int tm = 0; tm < TM2; ++tm)                             \
-                {                                                                              \
-                    const f16x8 af_ = *reinterpret_cast<const f16x8 *>(a_frag + tm * (32 * 128) + slot_); \
-                    _Pragma("unroll") for (int tn = 0; tn < TN2; ++tn) acc32[tm][tn] =         \
-                        __builtin_amdgcn_mfma_f32_32x32x16_f16(af_, bf_[tn], acc32[tm][tn], 0, 0, 0); \
-                }                                                                              \
+                    fa[h][kk * TM2 + tm] = *reinterpret_cast<const f16x8 *>(a_frag + tm * (32 * 128) + slot_); \
             }                                                                                  \
-        } else                                                                                 \
-        _Pragma("unroll") for (int kh = 0; kh < 2; ++kh)                                       \
-        {                                                                                      \
-            const int slot_ = (((kh * 4 + g) ^ sw) << 4) + (buf) * BUF;                        \
-            f16x8 bf_[TN];                                                                     \
+        } else {                                                                               \
+            const int slot_ = ((((h) * 4 + g) ^ sw) << 4) + (buf) * BUF;                       \
             _Pragma("unroll") for (int tn = 0; tn < TN; ++tn)                                  \
-                bf_[tn] = *reinterpret_cast<const f16x8 *>(x_frag + tn * (16 * 128) + slot_);  \
+                fb[h][tn] = *reinterpret_cast<const f16x8 *>(x_frag + tn * (16 * 128) + slot_); \
             _Pragma("unroll") for (int tm = 0; tm < TM; ++tm)                                  \
-            {                                                                                  \
-                const f16x8 af_ = *reinterpret_cast<const f16x8 *>(a_frag + tm * (16 * 128) + slot_); \
-                _Pragma("unroll") for (int tn = 0; tn < TN; ++tn) acc[tm][tn] =                \
-                    __builtin_amdgcn_mfma_f32_16x16x32_f16(af_, bf_[tn], acc[tm][tn], 0, 0, 0); \
-            }                                                                                  \
+                fa[h][tm] = *reinterpret_cast<const f16x8 *>(a_frag + tm * (16 * 128) + slot_); \
         }                                                                                      \
     }
-    // iteration i (k-step s0 + i): stage step s0+i+1 into the other buffer, multiply from this one
-#define TUNA_TILED_ITER(i)                                                                       \
+    // MFMA q of the NM of a half
+    constexpr int NM = M32 ? 2 * TM2 * TN2 : TM * TN;
+    constexpr int QS = NM / 4;
+#define TUNA_TILED_MFMA1(h, q)                                                                   \
     {                                                                                          \
-        TUNA_TILED_STAGE(((i) + 1) % NSETS, ((i) + 1) & 1, s + (i) + 1)                        \
-        TUNA_TILED_MFMA((i) & 1)                                                               \
+        if constexpr (M32) {                                                                   \
+            const int kk_ = (q) / (TM2 * TN2), tm_ = ((q) % (TM2 * TN2)) / TN2, tn_ = (q) % TN2; \
+            acc32[tm_][tn_] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[h][kk_ * TM2 + tm_], fb[h][kk_ * TN2 + tn_], \
+                                                                     acc32[tm_][tn_], 0, 0, 0); \
+        } else {                                                                               \
+            acc[(q) / TN][(q) % TN] =                                                          \
+                __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[h][(q) / TN], fb[h][(q) % TN], acc[(q) / TN][(q) % TN], 0, 0, 0); \
+        }                                                                                      \
+    }
+    // Staging of a k-step from register set `set`: the table reads of its L byte pairs ...
+    uint32_t lt[L];
+    f16x2 hh[L];
+#define TUNA_TILED_LUT(set)                                                                      \
+    _Pragma("unroll") for (int j = 0; j < DW; ++j)                                             \
+    {                                                                                          \
+        const uint32_t d_ = wq[set][j];                                                        \
+        lt[4 * j + 0] = *reinterpret_cast<const lds_u32 *>((uintptr_t)__builtin_amdgcn_perm(d_, lane4, 0x0c0c0400u)); \
+        lt[4 * j + 1] = *reinterpret_cast<const lds_u32 *>((uintptr_t)__builtin_amdgcn_perm(d_, lane4, 0x0c0c0500u)); \
+        lt[4 * j + 2] = *reinterpret_cast<const lds_u32 *>((uintptr_t)__builtin_amdgcn_perm(d_, lane4, 0x0c0c0600u)); \
+        lt[4 * j + 3] = *reinterpret_cast<const lds_u32 *>((uintptr_t)__builtin_amdgcn_perm(d_, lane4, 0x0c0c0700u)); \
+    }
+    // ... the scaling of pair l (bit-identical to kernel.cu:2178-2192), the fourth pair of a dword storing
+    // its eight weights into row a_row + l / 4 of weight tile `buf` ...
+#define TUNA_TILED_DECODE(l, buf)                                                                \
+    {                                                                                          \
+        hh[l] = __builtin_bit_cast(f16x2, lt[l]) * sc16[(l) >> 2];                             \
+        if (((l) & 3) == 3) {                                                                  \
+            const int r_ = a_row + ((l) >> 2);                                                 \
+            const f16x8 w_ = {hh[(l) - 3][0], hh[(l) - 3][1], hh[(l) - 2][0], hh[(l) - 2][1],  \
+                              hh[(l) - 1][0], hh[(l) - 1][1], hh[l][0],       hh[l][1]};       \
+            *reinterpret_cast<f16x8 *>(a_tile + (buf) * BUF + r_ * 128 + ((a_kb ^ (r_ & 7)) << 4)) = w_; \
+        }                                                                                      \
+    }
+    // ... and activation piece i of step s (zero beyond n and k) into activation tile `buf`.
+#define TUNA_TILED_XSTAGE(set, i, buf, s)                                                        \
+    {                                                                                          \
+        const int p_ = tid + (i) * kTiledThreads;                                              \
+        const int t_ = p_ >> 3, sl_ = p_ & 7;                                                  \
+        const bool ok_ = x_tok_ok[i] && ((s) * kTiledStepK + sl_ * 8 < a.k);                   \
+        *reinterpret_cast<u32x4 *>(x_tile + (buf) * BUF + t_ * 128 + ((sl_ ^ (t_ & 7)) << 4)) = \
+            ok_ ? xr[set][i] : u32x4{0u, 0u, 0u, 0u};                                          \
+    }
+    // Iteration i of a tile's k-steps, k-step `step`, whose tiles are complete in buffer i & 1 (a barrier
+    // has passed).  The matrix cores must not wait for the staging of the next step, nor for the
+    // fragments of this one, so the order is written out and pinned:
+    //   fragments of this step's first half are requested, and the table reads of step + 1;
+    //   the MFMAs of the PREVIOUS step's second half run meanwhile (their fragments were read before the
+    //     barrier), with the scaling and the weight-tile stores of step + 1 between them;
+    //   fragments of this step's second half are requested;
+    //   the MFMAs of this step's first half run, with the activation stores of step + 1 and the
+    //     refill of the register set between them;
+    //   barrier.
+    // FIRST: no previous step.  The second half of the last step follows the loop.
+#define TUNA_TILED_ITER(i, step, FIRST)                                                          \
+    {                                                                                          \
+        const int set_ = ((i) + 1) % NSETS, xset_ = ((i) + 1) % XSETS, cur_ = (i) & 1, nxt_ = cur_ ^ 1; \
+        TUNA_TILED_READ(0, cur_)                                                               \
+        TUNA_TILED_LUT(set_)                                                                   \
+        __builtin_amdgcn_sched_barrier(0);                                                     \
+        _Pragma("unroll") for (int q = 0; q < NM; ++q)                                         \
+        {                                                                                      \
+            if (!(FIRST)) TUNA_TILED_MFMA1(1, q)                                               \
+            /* (none behind the first quarter of the MFMAs: the table reads are still on their way) */ \
+            _Pragma("unroll") for (int l = max(q - QS, 0) * L / (NM - QS); l < max(q - QS + 1, 0) * L / (NM - QS); ++l) \
+                TUNA_TILED_DECODE(l, nxt_)                                                     \
+            __builtin_amdgcn_sched_barrier(0);                                                 \
+        }                                                                                      \
+        TUNA_TILED_READ(1, cur_)                                                               \
+        __builtin_amdgcn_sched_barrier(0);                                                     \
+        _Pragma("unroll") for (int q = 0; q < NM; ++q)                                         \
+        {                                                                                      \
+            TUNA_TILED_MFMA1(0, q)                                                             \
+            _Pragma("unroll") for (int xi = 0; xi < X_PER_THREAD; ++xi)                        \
+                if (q == xi * NM / X_PER_THREAD) TUNA_TILED_XSTAGE(xset_, xi, nxt_, (step) + 1) \
+            if (q == NM - 1) {                                                                 \
+                /* (activations first: the wait for them two steps on then leaves this step's weights in flight) */ \
+                TUNA_TILED_LOAD_X(xset_, min((step) + 1 + XSETS, a.steps_total - 1))           \
+                TUNA_TILED_LOAD(set_, min((step) + 1 + NSETS, a.steps_total - 1))              \
+            }                                                                                  \
+            __builtin_amdgcn_sched_barrier(0);                                                 \
+        }                                                                                      \
         __syncthreads(); /* the staged tiles are complete; this step's tiles are free */       \
     }
 
     int s = s0;
     __syncthreads();  // decode table complete
-    TUNA_TILED_STAGE(0, 0, s)
+    // the first step, staged with nothing to hide behind
+    TUNA_TILED_LUT(0)
+#pragma unroll
+    for (int l = 0; l < L; ++l) TUNA_TILED_DECODE(l, 0)
+#pragma unroll
+    for (int xi = 0; xi < X_PER_THREAD; ++xi) TUNA_TILED_XSTAGE(0, xi, 0, s)
+    TUNA_TILED_LOAD(0, min(s + NSETS, a.steps_total - 1))
+    TUNA_TILED_LOAD_X(0, min(s + XSETS, a.steps_total - 1))
     __syncthreads();
+    TUNA_TILED_ITER(0, s, true)
+    ++s;
     for (; s + NSETS - 1 < s1; s += NSETS) {
 #pragma unroll
-        for (int it = 0; it < NSETS; ++it) TUNA_TILED_ITER(it)  // (`it`: the macros use `i` inside)
+        for (int it = 0; it < NSETS; ++it) TUNA_TILED_ITER(it + 1, s + it, false)
     }
     // tail: up to NSETS - 1 more steps (the staging of a step past the end is harmless: its loads
     // are clamped and nothing reads the tiles)
 #pragma unroll
     for (int it = 0; it < NSETS - 1; ++it)
-        if (s + it < s1) TUNA_TILED_ITER(it)
+        if (s + it < s1) TUNA_TILED_ITER(it + 1, s + it, false)
+    // second half of the last step
+#pragma unroll
+    for (int q = 0; q < NM; ++q) TUNA_TILED_MFMA1(1, q)
 #undef TUNA_TILED_ITER
-#undef TUNA_TILED_MFMA
-#undef TUNA_TILED_STAGE
+#undef TUNA_TILED_XSTAGE
+#undef TUNA_TILED_DECODE
+#undef TUNA_TILED_LUT
+#undef TUNA_TILED_MFMA1
+#undef TUNA_TILED_READ
+#undef TUNA_TILED_LOAD_X
 #undef TUNA_TILED_LOAD
 
     // ---- epilogue -----------------------------------------------------------------------------
