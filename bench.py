@@ -213,6 +213,23 @@ def launch_floor(ops, torch, dev, headline_bytes):
     }
 
 
+def unit_rates(ops, dev):
+    """Yardsticks of the many-token kernels: what the matrix cores and the LDS of this box deliver to the MFMA
+    shapes and LDS access patterns those kernels use (best of three timings each)."""
+    names = ["mfma_16x16x32_f16_one_wave_per_simd_tflops", "mfma_16x16x32_f16_two_waves_per_simd_tflops",
+             "mfma_32x32x16_f16_one_wave_per_simd_tflops", "lds_fragment_reads_b128_bytes_per_clk_per_cu",
+             "lds_table_reads_b32_bytes_per_clk_per_cu", "lds_tile_writes_b128_bytes_per_clk_per_cu"]
+    out = {}
+    for unit, nm in enumerate(names):
+        best = 0.0
+        for _ in range(3):
+            ms, work = ops.time_unit_rate(unit, dev, warmup=1, iters=4)
+            best = max(best, work * 4 / (ms * 1e-3))
+        out[nm] = round(best / 1e12, 1) if unit < 3 else round(best / 256 / 2.4e9, 1)
+    out["note"] = "LDS rates per compute unit at the 2.4 GHz peak clock, 256 compute units"
+    return out
+
+
 def time_dequant_shapes(ops, synth, torch, dev, names=("mistral_attn_out", "mistral_gate_up", "llama70b_down")):
     from tuna_amd.quantize import nf4_codebook
 
@@ -324,10 +341,11 @@ def main():
     ap.add_argument("--launch", choices=("both", "stream", "graph"), default="both")
     ap.add_argument("--settle", type=int, default=300,
                     help="untimed launches before the warm-up of the headline (a box that was idle ramps its clocks)")
-    ap.add_argument("--only", choices=("read", "dequant", "quantize", "multi", "mfma"), default=None,
+    ap.add_argument("--only", choices=("read", "dequant", "quantize", "multi", "mfma", "rates"), default=None,
                     help="profiling runs: launch only the read-kernel sweep / the dequant kernel / the quantizer / "
                          "the Llama-70B layer set through tuna_matmul_multi (16 layers) / the many-token kernel with "
-                         "16x16x32 and with 32x32x16 MFMA tiles (Llama-70B gate+up and QKV, --tokens, default 1024)")
+                         "16x16x32 and with 32x32x16 MFMA tiles (Llama-70B gate+up and QKV, --tokens, default 1024) / the "
+                         "matrix-core and LDS yardstick kernels")
     ap.add_argument("--weight-path", choices=("table", "registers", "lds"), default="table",
                     help="headline workload: the table's config as it is, or with the packed weights forced through "
                          "registers / staged through LDS (lds_tile_rows 0 / -1; A/B runs of the two weight paths)")
@@ -358,6 +376,8 @@ def main():
             res = {"dequant": time_dequant_shapes(ops, synth, torch, dev)}
         elif args.only == "quantize":
             res = {"quantize": time_quantize(ops, synth, torch, dev)}
+        elif args.only == "rates":
+            res = {"unit_rates": unit_rates(ops, dev)}
         elif args.only == "mfma":
             res = {"many_token_kernel_mfma_shapes": mfma_shapes(ops, synth, torch, dev, 1024 if args.tokens == TOKENS else args.tokens)}
         else:
@@ -419,6 +439,7 @@ def main():
     # cannot take less than their sum.
     if not args.only_headline:
         line["launch_floor"] = launch_floor(ops, torch, dev, head["packed_bytes"])
+        line["unit_rates"] = unit_rates(ops, dev)
 
     if args.copy_yardstick > 0:
         line["copy_yardstick"] = copy_yardstick(ops, torch, dev, args.copy_yardstick)

@@ -52,6 +52,16 @@ int tuna_time_copy(const void *src, void *dst, size_t bytes, int warmup, int ite
 int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int variant, int warmup,
                    int iters, void *stream, float *elapsed_ms);
 
+/* What the matrix cores and the LDS deliver on this device, the yardsticks of the many-token kernels as the
+ * read kernel is that of the streaming ones.  unit 0 / 1: independent v_mfma_f32_16x16x32_f16 back to back from
+ * one / two waves per SIMD (16 accumulators each); 2: v_mfma_f32_32x32x16_f16 from one wave per SIMD (4
+ * accumulators); 3: 16-byte LDS reads in the pattern of an MFMA fragment read from a tile of 128-byte rows; 4:
+ * 4-byte LDS reads in the pattern of the byte-pair decode table; 5: 16-byte LDS writes in the pattern of the
+ * decoded weight tile (3..5 with 8 waves per compute unit).  One workgroup per compute unit (two for unit 1).
+ * *work_per_launch receives the flops (0..2) or LDS bytes (3..5) of one launch; `sink`: 8 writable bytes. */
+int tuna_time_unit_rate(int unit, void *sink, int warmup, int iters, void *stream, float *elapsed_ms,
+                        double *work_per_launch);
+
 /* Name and template arguments of the kernel a GEMM launch would start (cfg NULL = the library's
  * choice), e.g. "gemm_narrow_kernel<LW=2,WK=8,U=4,PERM=1,TT=1>": what the bench writes beside a
  * timing so that it can be matched with a profile.  Host only; with a device present the

@@ -96,6 +96,7 @@ SIGNATURES = {
     "tuna_time_dequant": (_i, [_vpp, _vpp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_copy": (_i, [_vp, _vp, _sz, _i, _i, _vp, _fp]),
     "tuna_time_read": (_i, [_vp, _vp, _sz, _i, _i, _i, _i, _vp, _fp]),
+    "tuna_time_unit_rate": (_i, [_i, _vp, _i, _i, _vp, _fp, ctypes.POINTER(ctypes.c_double)]),
     "tuna_describe_launch": (_i, [_i, _i, _i, _cfgp, _i, ctypes.c_char_p, _sz]),
     "tuna_selftest_quantizer_division": (_i, [_vp, _vp]),
     "tuna_set_multi_shape": (_i, [_i, _i]),

@@ -1493,6 +1493,23 @@ TUNA_EXPORT int tuna_time_read(const void *src, void *sink, size_t bytes, int bl
     return time_loop(launch, 1, warmup, iters, 0, static_cast<hipStream_t>(stream), elapsed_ms);
 }
 
+TUNA_EXPORT int tuna_time_unit_rate(int unit, void *sink, int warmup, int iters, void *stream, float *elapsed_ms,
+                                    double *work_per_launch)
+{
+    int rc;
+    if ((rc = check_ptr(sink, "sink", 4))) return rc;
+    if (unit < 0 || unit > 5) return fail(TUNA_ERR_INVALID_ARG, "unit %d outside 0..5", unit);
+    if (!work_per_launch) return fail(TUNA_ERR_INVALID_ARG, "work_per_launch is null");
+    int dev = 0, cus = 0;
+    hipError_t e = device_cus(&dev, &cus);
+    if (e != hipSuccess) return hip_fail(e, "device query");
+    auto launch = [&](int, hipStream_t s) {
+        hipError_t e2 = launch_unit_rate(unit, cus, static_cast<uint32_t *>(sink), work_per_launch, s);
+        return e2 == hipSuccess ? (int)TUNA_OK : hip_fail(e2, "unit-rate launch");
+    };
+    return time_loop(launch, 1, warmup, iters, 0, static_cast<hipStream_t>(stream), elapsed_ms);
+}
+
 TUNA_EXPORT int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config *cfg, int decode_mode, char *buf, size_t len)
 {
     if (!buf || len < 16) return fail(TUNA_ERR_INVALID_ARG, "buf is null or shorter than 16 bytes");

@@ -162,6 +162,128 @@ hipError_t launch_read(const void *src, void *sink, size_t bytes, int blocks, in
     return hipGetLastError();
 }
 
+// ---- unit rates: what the matrix cores and the LDS of this device deliver to the access patterns the
+// many-token kernel uses, measured the way the read kernel measures HBM --------------------------------
+typedef float rate_f32x16 __attribute__((ext_vector_type(16)));
+typedef float rate_f32x4 __attribute__((ext_vector_type(4)));
+constexpr int kRateIters = 4096;
+
+// Independent MFMAs back to back, nothing else: NACC accumulators per wave, 4 waves per workgroup.
+template <bool M32, int NACC>
+__global__ __launch_bounds__(256) void mfma_rate_kernel(uint32_t *sink)
+{
+    f16x8 a, b;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        a[e] = (f16)(0.001f * (float)threadIdx.x + (float)e);
+        b[e] = (f16)(0.5f * (float)e);
+    }
+    float s = 0.f;
+    if constexpr (M32) {
+        rate_f32x16 acc[NACC];
+#pragma unroll
+        for (int i = 0; i < NACC; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
+        for (int it = 0; it < kRateIters; ++it)
+#pragma unroll
+            for (int i = 0; i < NACC; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i], 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < NACC; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s += acc[i][e];
+    } else {
+        rate_f32x4 acc[NACC];
+#pragma unroll
+        for (int i = 0; i < NACC; ++i) acc[i] = rate_f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int it = 0; it < kRateIters; ++it)
+#pragma unroll
+            for (int i = 0; i < NACC; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[i], 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < NACC; ++i) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+    }
+    if (s == 12345.678f) sink[0] = 1u;  // practically never: keeps the chain alive
+}
+
+// LDS traffic of 8 waves per CU, eight accesses per wave and iteration, addresses opaque to the compiler.
+// MODE 0: 16-byte reads the way a wave reads an MFMA fragment from a tile of 128-byte rows (lane = row 0..15 x
+// k-group, slot ^ (row & 7)); 1: 4-byte reads the way the decode reads the byte-pair table ((byte << 8) | (lane
+// << 2), byte from a counter); 2: 16-byte writes the way the decoded weights are stored (4 rows x 8 k-blocks
+// per 32 lanes).
+template <int MODE>
+__global__ __launch_bounds__(512) void lds_rate_kernel(uint32_t *sink)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    for (int i = threadIdx.x; i < 65536 / 4; i += 512) reinterpret_cast<uint32_t *>(smem)[i] = (uint32_t)i;
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t s = 0;
+    if constexpr (MODE == 0) {
+        const int row = lane & 15, g = lane >> 4;
+        const uint32_t base = (uint32_t)(row * 128 + ((g ^ (row & 7)) << 4) + wave * 4096);
+        for (int it = 0; it < kRateIters; ++it)
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                uint32_t off = (base + r * 2048 + (it & 1) * 32768) & 65535u;
+                asm volatile("" : "+v"(off));
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(smem + off);
+                s += v[0] ^ v[1] ^ v[2] ^ v[3];
+            }
+    } else if constexpr (MODE == 1) {
+        for (int it = 0; it < kRateIters; ++it)
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                uint32_t off = ((uint32_t)((it * 8 + r + wave * 31) & 255) << 8) | ((uint32_t)lane << 2);
+                asm volatile("" : "+v"(off));
+                s += *reinterpret_cast<const uint32_t *>(smem + off);
+            }
+    } else {
+        const int half = lane & 1, kb = (lane >> 1) & 7, mbl = lane >> 4;
+        u32x4 v = {(uint32_t)threadIdx.x, 1u, 2u, 3u};
+        for (int it = 0; it < kRateIters; ++it) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                const int row = mbl * 8 + half * 4 + (r & 3);
+                uint32_t off = (uint32_t)(row * 128 + ((kb ^ (row & 7)) << 4) + wave * 4096 + ((it + (r >> 2)) & 1) * 32768) & 65535u;
+                asm volatile("" : "+v"(off));
+                *reinterpret_cast<u32x4 *>(smem + off) = v;
+            }
+            v[0] += 1u;
+        }
+        __syncthreads();
+        s = smem[threadIdx.x];
+    }
+    if (s == 0x9e3779b9u && sink[1] == 77u) sink[0] = s;  // practically never
+}
+
+// unit: 0 / 1 v_mfma_f32_16x16x32_f16 with one / two waves per SIMD (16 accumulators), 2 v_mfma_f32_32x32x16_f16
+// (one wave per SIMD, 4 accumulators); 3 LDS fragment reads, 4 LDS table reads, 5 LDS tile writes.  *work =
+// flops (0..2) or bytes (3..5) of one launch on `cus` compute units.
+hipError_t launch_unit_rate(int unit, int cus, uint32_t *sink, double *work, hipStream_t stream)
+{
+    static OptInFlag attr[16][3];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
+    switch (unit) {
+    case 0: hipLaunchKernelGGL((mfma_rate_kernel<false, 16>), dim3(cus), dim3(256), 0, stream, sink); *work = (double)cus * 4 * kRateIters * 16 * 16384.0; break;
+    case 1: hipLaunchKernelGGL((mfma_rate_kernel<false, 16>), dim3(2 * cus), dim3(256), 0, stream, sink); *work = (double)cus * 8 * kRateIters * 16 * 16384.0; break;
+    case 2: hipLaunchKernelGGL((mfma_rate_kernel<true, 4>), dim3(cus), dim3(256), 0, stream, sink); *work = (double)cus * 4 * kRateIters * 4 * 32768.0; break;
+    case 3:
+        if ((e = ensure_lds_opt_in(attr[dev][0], reinterpret_cast<const void *>(lds_rate_kernel<0>))) != hipSuccess) return e;
+        hipLaunchKernelGGL(lds_rate_kernel<0>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 16.0; break;
+    case 4:
+        if ((e = ensure_lds_opt_in(attr[dev][1], reinterpret_cast<const void *>(lds_rate_kernel<1>))) != hipSuccess) return e;
+        hipLaunchKernelGGL(lds_rate_kernel<1>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 4.0; break;
+    case 5:
+        if ((e = ensure_lds_opt_in(attr[dev][2], reinterpret_cast<const void *>(lds_rate_kernel<2>))) != hipSuccess) return e;
+        hipLaunchKernelGGL(lds_rate_kernel<2>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 16.0; break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 hipError_t launch_copy(const void *src, void *dst, size_t bytes, hipStream_t stream)
 {
     const size_t n16 = bytes / 16;

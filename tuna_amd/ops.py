@@ -400,6 +400,19 @@ def time_read(src, blocks=0, variant=0, warmup=5, iters=20) -> float:
     return ms.value
 
 
+def time_unit_rate(unit: int, device, warmup=2, iters=5):
+    """(milliseconds for `iters` launches, flops or LDS bytes per launch) of one of the matrix-core / LDS
+    yardstick kernels (tuna_time_unit_rate)."""
+    sink = torch.zeros(4, dtype=torch.int32, device=device)
+    ms = ctypes.c_float(0)
+    work = ctypes.c_double(0)
+    with torch.cuda.device(device):
+        rc = _lib.lib().tuna_time_unit_rate(int(unit), sink.data_ptr(), int(warmup), int(iters), _stream(device),
+                                            ctypes.byref(ms), ctypes.byref(work))
+    _lib.check(rc)
+    return ms.value, work.value
+
+
 def describe_launch(m: int, n: int, k: int, config: GemmConfig = None, decode_mode: int = _lib.DECODE_GEMM) -> str:
     """Name and template arguments of the kernel a GEMM launch would start (tuna_describe_launch)."""
     buf = ctypes.create_string_buffer(256)
