@@ -15,6 +15,8 @@
 //     multiply (TUNA_DECODE_GEMM, kernel.cu:2178-2192).
 #include "tuna_internal.h"
 
+#include <type_traits>
+
 namespace tuna {
 
 typedef _Float16 f16;
@@ -337,7 +339,7 @@ __device__ __forceinline__ float div_by_block_max(float w, float a, float y)
 // Nearest entry of a sorted codebook: bnd[i] (i = 0..14) is the smallest binary32 value that the
 // argmin assigns to entry i + 1 rather than entry i, so the index is the number of boundaries <= nv:
 // a 4-step binary search, as a tree of selects over the 15 values (uniform, held in registers).
-__device__ __forceinline__ uint32_t nearest_sorted(float nv, const float (&b)[15])
+__device__ __forceinline__ uint32_t nearest_sorted(float nv, const float (&b)[16])
 {
     const bool b3 = nv >= b[7];
     const float t2 = b3 ? b[11] : b[3];
@@ -350,6 +352,32 @@ __device__ __forceinline__ uint32_t nearest_sorted(float nv, const float (&b)[15
     const float t4 = b1 ? x4 : y4;
     const bool b0 = nv >= t4;
     return (b3 ? 8u : 0u) + (b2 ? 4u : 0u) + (b1 ? 2u : 0u) + (b0 ? 1u : 0u);  // a NaN nv ends at 0 like the argmin
+}
+
+// The same count of boundaries <= nv without the search: the quotients lie in [-1, 1], cut into 128 buckets
+// of 1/64; when no two boundaries share a bucket, a bucket knows how many boundaries lie below it and the one
+// boundary (if any) inside it, and the index is that count plus one comparison.  bucket_of is monotonic in
+// nv (a fused multiply-add, a clamp, a truncation), so every value of a lower bucket is below the boundary
+// of a higher one and vice versa: the result is the binary search's for every nv, NaN included (bucket 0, the
+// comparison false, index 0).  Two LDS tables in the lane-private layout of the GEMM's decode table (entry e
+// of lane l at (e << 8) | (l << 2), resp. (e << 6) | l: no bank conflicts whatever the data).
+constexpr int kQuantBuckets = 129;
+constexpr int kQuantBndBytes = kQuantBuckets * 256;  // fp32 boundary of the bucket, +inf if none
+constexpr int kQuantLoBytes = kQuantBuckets * 64;    // boundaries below the bucket, one byte
+typedef __attribute__((address_space(3))) unsigned char lds_u8;
+typedef __attribute__((address_space(3))) uint32_t lds_word;
+
+__device__ __forceinline__ uint32_t bucket_of(float nv)
+{
+    return (uint32_t)__builtin_amdgcn_fmed3f(__builtin_fmaf(nv, 64.0f, 64.0f), 0.0f, 128.0f);
+}
+
+__device__ __forceinline__ uint32_t nearest_bucketed(float nv, uint32_t bnd_lane, uint32_t lo_lane)
+{
+    const uint32_t e = bucket_of(nv);
+    const float b = __builtin_bit_cast(float, *reinterpret_cast<const lds_word *>((uintptr_t)((e << 8) + bnd_lane)));
+    const uint32_t lo = *reinterpret_cast<const lds_u8 *>((uintptr_t)((e << 6) + lo_lane));
+    return lo + (nv >= b ? 1u : 0u);
 }
 
 __device__ __forceinline__ uint32_t nearest_any(float nv, const float (&c)[16])
@@ -391,12 +419,13 @@ __device__ inline float decision_boundary(float lo, float hi)
 }
 
 template <int NP>
-__global__ __launch_bounds__(512) void quantize_kernel(const f16 *__restrict__ w, const float *__restrict__ code,
+__global__ __launch_bounds__(512, NP == 16 ? 2 : 4) void quantize_kernel(const f16 *__restrict__ w, const float *__restrict__ code,
                                                        uint32_t *__restrict__ q32, float *__restrict__ absmax, int m, int k,
                                                        int bs)
 {
     __shared__ float cs[16], bs_[15];
-    __shared__ int fast_s;
+    __shared__ int fast_s, tab_s, jb_s[15];
+    extern __shared__ __align__(16) unsigned char qtab[];  // bucket tables: boundaries, then counts
     constexpr int TPR = 64;  // threads per weight row: a row's threads read 1 KB contiguous
     __shared__ __align__(16) uint32_t tile[2][TPR * 8];  // [buffer][block column of the step (64)][row (8)]
     const int tid = threadIdx.x;
@@ -415,13 +444,49 @@ __global__ __launch_bounds__(512) void quantize_kernel(const f16 *__restrict__ w
     const bool fast = fast_s != 0;
     if (fast && tid < 15) bs_[tid] = decision_boundary(cs[tid], cs[tid + 1]);
     __syncthreads();
-    float c[16], bnd[15];
+    // bucket tables, if every boundary is finite and has a bucket of its own
+    if (tid == 0) {
+        int ok = fast ? 1 : 0;
+        for (int i = 0; i < 15 && ok; ++i) {
+            jb_s[i] = (int)bucket_of(bs_[i]);
+            ok &= (fabsf(bs_[i]) < 3.0e38f) && (i == 0 || jb_s[i] > jb_s[i - 1]) ? 1 : 0;
+        }
+        tab_s = ok;
+    }
+    __syncthreads();
+    const bool tabled = tab_s != 0;
+    const uint32_t tab0 = (uint32_t)(uintptr_t)(lds_u8 *)qtab;
+    const uint32_t bnd_lane = tab0 + ((uint32_t)(tid & 63) << 2);
+    const uint32_t lo_lane = tab0 + (uint32_t)kQuantBndBytes + (uint32_t)(tid & 63);
+    if (tabled) {
+        for (int p = tid; p < kQuantBndBytes / 16; p += 512) {  // 16 stores of 16 bytes per bucket
+            const int e = p >> 4;
+            float b = __builtin_inff();
 #pragma unroll
-    for (int i = 0; i < 16; ++i) c[i] = cs[i];
+            for (int i = 0; i < 15; ++i) b = jb_s[i] == e ? bs_[i] : b;
+            const uint32_t u = __builtin_bit_cast(uint32_t, b);
+            reinterpret_cast<u32x4 *>(qtab)[p] = u32x4{u, u, u, u};
+        }
+        for (int p = tid; p < kQuantLoBytes / 16; p += 512) {   // 4 stores of 16 bytes per bucket
+            const int e = p >> 2;
+            uint32_t n = 0;
 #pragma unroll
-    for (int i = 0; i < 15; ++i) bnd[i] = fast ? bs_[i] : 0.f;
+            for (int i = 0; i < 15; ++i) n += jb_s[i] < e ? 1u : 0u;
+            n *= 0x01010101u;
+            reinterpret_cast<u32x4 *>(qtab + kQuantBndBytes)[p] = u32x4{n, n, n, n};
+        }
+    }
+    __syncthreads();
 
-    const int mb = blockIdx.x;
+    // The block rows, with the nearest-entry rule as a compile-time choice (the three loops share nothing
+    // but their registers: the table path must not carry the 15 boundaries of the search).  MODE 0: bucket
+    // tables; 1: binary search over the boundaries; 2: the 16 comparisons.
+    auto run = [&](auto mode_tag) {
+    constexpr int MODE = decltype(mode_tag)::value;
+    float c[16];  // MODE 1: the boundaries; MODE 2: the codebook
+#pragma unroll
+    for (int i = 0; i < 16; ++i) c[i] = MODE == 1 ? (i < 15 ? bs_[i] : 0.f) : MODE == 2 ? cs[i] : 0.f;
+    for (int mb = blockIdx.x; mb < (m >> 3); mb += gridDim.x) {
     const int r8 = tid / TPR, j = tid % TPR;
     const int row = mb * 8 + r8;
     const int kb_total = k >> 3;
@@ -476,7 +541,10 @@ __global__ __launch_bounds__(512) void quantize_kernel(const f16 *__restrict__ w
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const float nv = div_by_block_max((float)t[e], amax, y);
-                const uint32_t best = fast ? nearest_sorted(nv, bnd) : nearest_any(nv, c);
+                uint32_t best;
+                if constexpr (MODE == 0) best = nearest_bucketed(nv, bnd_lane, lo_lane);
+                else if constexpr (MODE == 1) best = nearest_sorted(nv, c);
+                else best = nearest_any(nv, c);
                 d |= best << (8 * (e >> 1) + 4 * (1 - (e & 1)));  // byte e/2 of the dword; even column = high nibble
             }
         }
@@ -503,6 +571,12 @@ __global__ __launch_bounds__(512) void quantize_kernel(const f16 *__restrict__ w
             step(st, t);
         }
     }
+    __syncthreads();  // (the next block row's first step reuses the tile buffer the last step may still be read from)
+    }
+    };
+    if (tabled) run(std::integral_constant<int, 0>{});
+    else if (fast) run(std::integral_constant<int, 1>{});
+    else run(std::integral_constant<int, 2>{});
 }
 
 // Self-test of div_by_block_max: every pair of fp16 values (w, a) with a > 0 finite and |w| <= a,
@@ -539,11 +613,18 @@ hipError_t launch_quantize(const void *w, const float *code, void *q, float *abs
 {
     const f16 *wp = static_cast<const f16 *>(w);
     uint32_t *qp = static_cast<uint32_t *>(q);
-    const dim3 grid((unsigned)(m / 8)), block(512);
-    if (k <= 512 * 4) hipLaunchKernelGGL(quantize_kernel<4>, grid, block, 0, stream, wp, code, qp, absmax, m, k, bs);
-    else if (k <= 512 * 8) hipLaunchKernelGGL(quantize_kernel<8>, grid, block, 0, stream, wp, code, qp, absmax, m, k, bs);
-    else if (k <= 512 * 16) hipLaunchKernelGGL(quantize_kernel<16>, grid, block, 0, stream, wp, code, qp, absmax, m, k, bs);
-    else hipLaunchKernelGGL(quantize_kernel<0>, grid, block, 0, stream, wp, code, qp, absmax, m, k, bs);
+    // one workgroup per block row up to three per compute unit (what fits beside the bucket tables), which then
+    // walk the block rows: the tables are built once per workgroup
+    int dev = 0, cus = 0;
+    hipError_t e = device_cus(&dev, &cus);
+    if (e != hipSuccess) return e;
+    const int rows8 = m / 8;
+    const dim3 grid((unsigned)(rows8 < 3 * cus ? rows8 : 3 * cus)), block(512);
+    const size_t lds = (size_t)kQuantBndBytes + kQuantLoBytes;
+    if (k <= 512 * 4) hipLaunchKernelGGL(quantize_kernel<4>, grid, block, lds, stream, wp, code, qp, absmax, m, k, bs);
+    else if (k <= 512 * 8) hipLaunchKernelGGL(quantize_kernel<8>, grid, block, lds, stream, wp, code, qp, absmax, m, k, bs);
+    else if (k <= 512 * 16) hipLaunchKernelGGL(quantize_kernel<16>, grid, block, lds, stream, wp, code, qp, absmax, m, k, bs);
+    else hipLaunchKernelGGL(quantize_kernel<0>, grid, block, lds, stream, wp, code, qp, absmax, m, k, bs);
     return hipGetLastError();
 }
 
