@@ -63,7 +63,10 @@ enum { TUNA_EPILOGUE_NONE = 0, TUNA_EPILOGUE_RESIDUAL = 1, TUNA_EPILOGUE_SILU_MU
  * owns rows_per_wave weight rows and walks k in steps of 32; the workgroup owns
  * rows_per_wave*waves_m rows and a 1/split_k share of k.                          */
 typedef struct tuna_gemm_config {
-    int32_t rows_per_wave; /* 64, 128 or 256: 128-bit loads per lane per k-step x 64 */
+    int32_t rows_per_wave; /* 64, 128 or 256: 128-bit loads per lane per k-step x 64.  16, 24 or 32 (with
+                              waves_m 1), or 64 with waves_m 0: the narrow-row kernel - that many rows per
+                              workgroup, every wave along k, no split (m a multiple of it; 24 is a 32-row
+                              tile three quarters full, for row counts that make 256 tiles of 24) */
     int32_t waves_m;       /* waves along the weight rows (any count; waves_m*waves_k <= 16) */
     int32_t waves_k;       /* waves along k inside the workgroup, a power of two (reduced in LDS) */
     int32_t split_k;       /* workgroups along k (reduced through the workspace); 0 = balanced:

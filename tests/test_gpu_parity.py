@@ -970,6 +970,9 @@ NARROW_CASES = [
     (256, 16, 2048, 64, 8, 4),      # 64 rows per workgroup (waves_m = 0 selects the kernel)
     (192, 19, 1024, 64, 4, 8),
     (128, 7, 4096, 64, 16, 2),
+    (6144, 16, 4096, 24, 8, 4),     # 24 rows per workgroup: a 32-row tile three quarters full, 256 workgroups
+    (72, 3, 1024, 24, 8, 2),        # three such workgroups, the last block row of the matrix in the last one
+    (240, 11, 2048, 24, 16, 4),
     # two and four 16-token tiles per workgroup (7th entry: token_tiles)
     (256, 32, 1024, 32, 8, 2, 2),
     (128, 50, 2048, 16, 4, 4, 4),   # 64 tokens per chunk, 50 present
@@ -1019,10 +1022,10 @@ def test_narrow_row_kernel_matches_oracle(ci):
     assert torch.equal(again.view(torch.int16), out.view(torch.int16))
 
 
-@pytest.mark.parametrize("rows,wk,pf", [(16, 4, 2), (32, 8, 4), (32, 16, 2), (64, 8, 2)])
+@pytest.mark.parametrize("rows,wk,pf", [(16, 4, 2), (32, 8, 4), (32, 16, 2), (64, 8, 2), (24, 8, 8)])
 def test_narrow_row_kernel_decode_readout_is_bit_exact(rows, wk, pf):
     """One-hot activations read the narrow-row kernel's in-register decode out: the oracle's D1 image."""
-    m, k = 256, 2048
+    m, k = (264 if rows == 24 else 256), 2048
     q, _, code, absmax = make_inputs_np(m, 16, k, seed=rows + wk)
     want_img = O.dequant(q, absmax, code, m, k, mode=O.D1)
     cols = np.random.default_rng(wk).choice(k, size=16, replace=False)

@@ -254,7 +254,8 @@ struct NarrowPlan {
 // rows_per_wave 16 or 32, or 64 with waves_m = 0 (64 rows with waves_m >= 1 is the streaming kernel)
 static inline bool is_narrow(const tuna_gemm_config &c)
 {
-    return !c.lds_tile_rows && (c.rows_per_wave == 16 || c.rows_per_wave == 32 || (c.rows_per_wave == 64 && c.waves_m == 0));
+    return !c.lds_tile_rows &&
+           (c.rows_per_wave == 16 || c.rows_per_wave == 24 || c.rows_per_wave == 32 || (c.rows_per_wave == 64 && c.waves_m == 0));
 }
 
 static int plan_narrow(int m, int n, int k, const tuna_gemm_config &c, int decode, NarrowPlan *plan)
@@ -286,7 +287,7 @@ static int plan_narrow(int m, int n, int k, const tuna_gemm_config &c, int decod
     plan->rows = c.rows_per_wave;
     plan->waves_k = c.waves_k;
     plan->prefetch = c.prefetch;
-    plan->lds_bytes = (size_t)kLutBytes + (size_t)c.waves_k * (c.rows_per_wave / 16) * c.token_tiles * 1024;
+    plan->lds_bytes = (size_t)kLutBytes + (size_t)c.waves_k * ((c.rows_per_wave + 15) / 16) * c.token_tiles * 1024;
     if (plan->lds_bytes > (size_t)kLdsLimit)
         return fail(TUNA_ERR_UNSUPPORTED, "config needs %zu bytes of LDS, the CU has %d", plan->lds_bytes, kLdsLimit);
     plan->args.m = m;

@@ -234,6 +234,7 @@ struct NarrowVariant {
 };
 #define N(LW, WK, U) {16 * LW, WK, U, 1, gemm_narrow_kernel<LW, WK, U, false, 1>, gemm_narrow_kernel<LW, WK, U, true, 1>}
 #define NT(LW, WK, U, TT) {16 * LW, WK, U, TT, gemm_narrow_kernel<LW, WK, U, true, TT>, gemm_narrow_kernel<LW, WK, U, true, TT>}
+#define N24(WK, U) {24, WK, U, 1, gemm_narrow_kernel<2, WK, U, false, 1, false, 24>, gemm_narrow_kernel<2, WK, U, true, 1, false, 24>}
 static const NarrowVariant kNarrow[] = {
     N(1, 4, 2),  N(1, 4, 4),  N(1, 4, 8),  N(1, 8, 2),  N(1, 8, 4),  N(1, 8, 8),  N(1, 16, 2), N(1, 16, 4), N(1, 16, 8),
     N(2, 4, 2),  N(2, 4, 4),  N(2, 4, 8),  N(2, 8, 2),  N(2, 8, 4),  N(2, 8, 8),  N(2, 16, 2), N(2, 16, 4), N(2, 16, 8),
@@ -246,9 +247,12 @@ static const NarrowVariant kNarrow[] = {
     NT(1, 4, 2, 4), NT(1, 4, 4, 4), NT(1, 8, 2, 4), NT(1, 8, 4, 4),
     NT(2, 4, 2, 4), NT(2, 4, 4, 4), NT(2, 8, 2, 4), NT(2, 8, 4, 4),
     NT(4, 4, 2, 4), NT(4, 8, 2, 4),
+    // 24 rows per workgroup (a 32-row tile three quarters full): row counts that are 256 tiles of 24 but 192 of 32
+    N24(8, 2), N24(8, 4), N24(8, 8), N24(16, 2), N24(16, 4),
 };
 #undef N
 #undef NT
+#undef N24
 static constexpr int kNumNarrow = sizeof(kNarrow) / sizeof(kNarrow[0]);
 static OptInFlag g_narrow_attr_done[16][kNumNarrow][2];
 
@@ -266,8 +270,8 @@ bool narrow_variant_exists(int rows, int waves_k, int prefetch, int token_tiles)
 
 void describe_narrow_launch(int rows, int waves_k, int prefetch, int token_tiles, int n, char *buf, size_t len)
 {
-    snprintf(buf, len, "gemm_narrow_kernel<LW=%d,WK=%d,U=%d,PERM=%d,TT=%d>", rows / 16, waves_k, prefetch,
-             (n > 4 || token_tiles > 1) ? 1 : 0, token_tiles);
+    snprintf(buf, len, "gemm_narrow_kernel<LW=%d,WK=%d,U=%d,PERM=%d,TT=%d%s>", (rows + 15) / 16, waves_k, prefetch,
+             (n > 4 || token_tiles > 1) ? 1 : 0, token_tiles, rows == 24 ? ",ROWS=24" : "");
 }
 
 hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int prefetch, int token_tiles, hipStream_t stream)
@@ -282,7 +286,7 @@ hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int
     const int perm = args.n > 4;
     const NarrowKernelFn fn = perm ? v->fn_perm : v->fn;
     if ((e = ensure_lds_opt_in(g_narrow_attr_done[dev][vi][perm], reinterpret_cast<const void *>(fn))) != hipSuccess) return e;
-    const size_t lds = (size_t)kLutBytes + (size_t)waves_k * (rows / 16) * token_tiles * 1024;
+    const size_t lds = (size_t)kLutBytes + (size_t)waves_k * ((rows + 15) / 16) * token_tiles * 1024;
     const dim3 grid((unsigned)(args.m / rows), (unsigned)((args.n + 16 * token_tiles - 1) / (16 * token_tiles)), 1);
     hipLaunchKernelGGL(fn, grid, dim3(waves_k * 64), lds, stream, args.q, args.x, args.code, args.absmax, args.k, args.n,
                        args.n_it, args.m, args.out, args.epilogue, args.residual, 0, 1);

@@ -42,7 +42,7 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 // dwords of a kernel's arguments can be preloaded into scalar registers with the wave (built
 // with -amdgpu-kernarg-preload-count=16), which takes the argument fetch - a round trip to
 // memory - off the start of every wave.  A struct passed by value is not preloaded.
-template <int LW, int WK, int U, bool PERM, int TT, bool BLK = false>
+template <int LW, int WK, int U, bool PERM, int TT, bool BLK = false, int ROWS = 16 * LW>
 __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q, const void *a_x, const float *a_code,
                                                               const float *a_absmax, int a_k, int a_n, int a_n_it, int a_m,
                                                               void *a_out, int a_epilogue, const void *a_residual,
@@ -59,6 +59,7 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     } const a = {a_q, a_x, a_code, a_absmax, a_out, a_residual, a_epilogue, a_m, a_n, a_k, a_n_it};
     extern __shared__ __align__(16) unsigned char smem[];
     static_assert(LW == 1 || LW == 2 || LW == 4, "16, 32 or 64 rows per workgroup");
+    static_assert(ROWS % 8 == 0 && ROWS % LW == 0 && ROWS <= 16 * LW && ROWS > 8 * LW, "rows of a partly filled tile");
     unsigned char *lut = smem;
     float *red = reinterpret_cast<float *>(smem + kLutBytes);  // [wave][row plane][token tile][lane][4]
 
@@ -69,7 +70,10 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     const int wk = __builtin_amdgcn_readfirstlane(tid >> 6);
     constexpr int nthreads = WK * 64;
     const uint32_t lane4 = (uint32_t)lane << 2;
-    const int row0 = blockIdx.x * (16 * LW);
+    const int row0 = blockIdx.x * ROWS;
+    // ROWS < 16 * LW (24 rows with LW = 2: 6144 rows make 256 workgroups instead of 192): the lanes whose rows lie
+    // beyond the tile load the rows of other lanes again - valid addresses, sums nobody stores
+    const int ia = ROWS == 16 * LW ? i16 : (i16 < ROWS / LW ? i16 : i16 - ROWS / LW);
     const int tok0 = blockIdx.y * (16 * TT);  // TT tiles of 16 tokens share every decoded weight fragment
 
     // ---- requests: codebook and scales, then the first ring turn (x fragment, weights) --------
@@ -78,13 +82,13 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     if constexpr (BLK) {
         // (per block: loaded with the ring below)
     } else if constexpr (LW == 1) {
-        sc32[0] = a.absmax[row0 + i16];
+        sc32[0] = a.absmax[row0 + ia];
     } else if constexpr (LW == 2) {
-        const f32x2 s2 = *reinterpret_cast<const f32x2 *>(a.absmax + row0 + 2 * i16);
+        const f32x2 s2 = *reinterpret_cast<const f32x2 *>(a.absmax + row0 + 2 * ia);
         sc32[0] = s2[0];
         sc32[1] = s2[1];
     } else {
-        const f32x4 s4 = *reinterpret_cast<const f32x4 *>(a.absmax + row0 + 4 * i16);
+        const f32x4 s4 = *reinterpret_cast<const f32x4 *>(a.absmax + row0 + 4 * ia);
 #pragma unroll
         for (int j = 0; j < 4; ++j) sc32[j] = s4[j];
     }
@@ -92,8 +96,8 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     // A wave walks k in double steps of 64 (two MFMAs, one 128-byte line of x per token): wave wk
     // owns double steps wk, wk + WK, ...
     // Weights, per lane: block row and dwords of the block, block column 4*step + g.
-    const uint32_t lb = ((uint32_t)(row0 >> 3) + (uint32_t)((LW * i16) >> 3)) * kb_total * 32u +
-                        (uint32_t)((LW * i16) & 7) * 4u + (uint32_t)g * 32u;
+    const uint32_t lb = ((uint32_t)(row0 >> 3) + (uint32_t)((LW * ia) >> 3)) * kb_total * 32u +
+                        (uint32_t)((LW * ia) & 7) * 4u + (uint32_t)g * 32u;
     // B fragments: the MFMA wants lane (token i16, group g) to hold x[token][32*step + 8g ..], i.e.
     // four consecutive lanes on four different token rows - a wave instruction loading it that
     // way touches 16 rows with no two neighbouring lanes on one line and takes about three times
@@ -115,7 +119,7 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     u32x4 xq[U][TT];
     float sq[BLK ? U : 1][LW];  // BLK: the scales of the ring slot's block
     // BLK: lane's first scale, and the double step of ring slot 0 in the turn being loaded
-    const float *sp = a.absmax + (size_t)(row0 + LW * i16) * (size_t)(BLK ? a_nblk : 1);
+    const float *sp = a.absmax + (size_t)(row0 + LW * ia) * (size_t)(BLK ? a_nblk : 1);
     int dstep = wk;
     static_assert(U % 2 == 0, "whole double steps");
 #define TUNA_NARROW_LOAD(u)                                                                     \
@@ -252,7 +256,7 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
             s1 += v1[w];
         }
         const int tok = tok0 + tt * 16 + tk;
-        if (tok >= a.n) continue;
+        if (tok >= a.n || (ROWS != 16 * LW && 2 * rp >= ROWS)) continue;
         const int col = row0 + 2 * rp;
         if (a.epilogue == TUNA_EPILOGUE_SILU_MUL) {
             outp[(size_t)tok * (size_t)(a.m >> 1) + (col >> 1)] = (f16)silu_mul(s0, s1);

@@ -61,7 +61,8 @@ NARROW_VARIANTS = (
     {(r, wk, pf, 1) for r in (16, 32, 64) for wk in (4, 8, 16) for pf in (2, 4, 8)}
     | {(16, 1, 2, 1), (16, 2, 2, 1), (32, 1, 2, 1), (32, 2, 2, 1)}
     | {(r, wk, pf, 2) for r in (16, 32, 64) for wk in (4, 8, 16) for pf in (2, 4)}
-    | {(r, wk, pf, 4) for r in (16, 32) for wk in (4, 8) for pf in (2, 4)} | {(64, 4, 2, 4), (64, 8, 2, 4)})
+    | {(r, wk, pf, 4) for r in (16, 32) for wk in (4, 8) for pf in (2, 4)} | {(64, 4, 2, 4), (64, 8, 2, 4)}
+    | {(24, 8, 2, 1), (24, 8, 4, 1), (24, 8, 8, 1), (24, 16, 2, 1), (24, 16, 4, 1)})
 
 # (rows, tokens) tiles of the many-token kernel; must match kTiled in csrc/gemm_tiled.hip
 TILED_VARIANTS = {(256, 128), (256, 64), (128, 256), (128, 128), (64, 256), (64, 128)}
@@ -80,8 +81,8 @@ def bucket_of(n: int):
 
 
 def is_narrow(c: dict) -> bool:
-    """The config selects the narrow-row kernel: rows_per_wave 16 or 32, or 64 with waves_m 0."""
-    return c.get("lds_tile_rows", 0) == 0 and (c["rows_per_wave"] in (16, 32) or (c["rows_per_wave"] == 64 and c["waves_m"] == 0))
+    """The config selects the narrow-row kernel: rows_per_wave 16, 24 or 32, or 64 with waves_m 0."""
+    return c.get("lds_tile_rows", 0) == 0 and (c["rows_per_wave"] in (16, 24, 32) or (c["rows_per_wave"] == 64 and c["waves_m"] == 0))
 
 
 def validate(m: int, n_key: int, k: int, c: dict) -> None:
@@ -114,14 +115,14 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
         if c["x_chunk"] != STEP_K * c["waves_k"] * c["prefetch"]:
             raise ValueError("the narrow-row kernel stages no x: x_chunk must be 32*waves_k*prefetch, the k of one ring turn")
         if m % c["rows_per_wave"] or k % (STEP_K * c["waves_k"] * c["prefetch"]):
-            raise ValueError("rows_per_wave 16 or 32 needs m a multiple of it and k a multiple of 32*waves_k*prefetch")
+            raise ValueError("rows_per_wave 16, 24 or 32 needs m a multiple of it and k a multiple of 32*waves_k*prefetch")
         if m * k // 2 >= 1 << 32 or k * 32 >= 1 << 32:
             raise ValueError("operands exceed the kernel's 32-bit offsets")
         if lds_bytes(c) > LDS_LIMIT:
             raise ValueError(f"needs {lds_bytes(c)} bytes of LDS (limit {LDS_LIMIT})")
         return
     if c["rows_per_wave"] not in (64, 128, 256):
-        raise ValueError("rows_per_wave must be 16, 32 (narrow-row kernel), 64, 128 or 256")
+        raise ValueError("rows_per_wave must be 16, 24, 32 (narrow-row kernel), 64, 128 or 256")
     if c["prefetch"] not in (2, 4, 8):
         raise ValueError("prefetch must be 2, 4 or 8")
     if c["token_tiles"] not in (1, 2, 4, 8):
@@ -213,7 +214,7 @@ def lds_bytes(c: dict) -> int:
         return LUT_BYTES + 2 * (c["lds_tile_rows"] + 16 * c["token_tiles"]) * 128
     if is_narrow(c):
         # narrow-row kernel: decode table + one accumulator plane (1 KB) per wave and 16 rows
-        return LUT_BYTES + c["waves_k"] * (c["rows_per_wave"] // 16) * c["token_tiles"] * 1024
+        return LUT_BYTES + c["waves_k"] * ((c["rows_per_wave"] + 15) // 16) * c["token_tiles"] * 1024
     threads = 64 * c["waves_k"] * c["waves_m"]
     x = c["token_tiles"] * 16 * c["x_chunk"] * 2
     plane = c["waves_k"] * c["waves_m"] * 1024
