@@ -427,7 +427,9 @@ __global__ __launch_bounds__(512, NP == 16 ? 2 : 4) void quantize_kernel(const f
     __shared__ int fast_s, tab_s, jb_s[15];
     extern __shared__ __align__(16) unsigned char qtab[];  // bucket tables: boundaries, then counts
     constexpr int TPR = 64;  // threads per weight row: a row's threads read 1 KB contiguous
-    __shared__ __align__(16) uint32_t tile[2][TPR * 8];  // [buffer][block column of the step (64)][row (8)]
+    // records of the block row being assembled: [step][block column of the step (64)][row (8)] - all NP steps
+    // of a row held in registers (one barrier per block row), or two buffers of one step each (NP == 0)
+    __shared__ __align__(16) uint32_t tile[NP > 0 ? NP : 2][TPR * 8];
     const int tid = threadIdx.x;
     if (tid < 16) cs[tid] = code[tid];
     __syncthreads();
@@ -486,6 +488,8 @@ __global__ __launch_bounds__(512, NP == 16 ? 2 : 4) void quantize_kernel(const f
     float c[16];  // MODE 1: the boundaries; MODE 2: the codebook
 #pragma unroll
     for (int i = 0; i < 16; ++i) c[i] = MODE == 1 ? (i < 15 ? bs_[i] : 0.f) : MODE == 2 ? cs[i] : 0.f;
+    constexpr bool AHEAD = NP > 0 && NP <= 8;
+    f16x8 v[NP > 0 ? NP : 1];
     for (int mb = blockIdx.x; mb < (m >> 3); mb += gridDim.x) {
     const int r8 = tid / TPR, j = tid % TPR;
     const int row = mb * 8 + r8;
@@ -496,14 +500,28 @@ __global__ __launch_bounds__(512, NP == 16 ? 2 : 4) void quantize_kernel(const f
     const int lanes_blk = by_row ? TPR : bs >> 3;  // threads that share a scale (a power of two <= 32)
     const int nblk = k / bs;
 
-    f16x8 v[NP > 0 ? NP : 1];
     float row_max = 0.f;
     if constexpr (NP > 0) {
+        if (!AHEAD || mb == (int)blockIdx.x) {
 #pragma unroll
-        for (int i = 0; i < NP; ++i) {
-            const int kb = i * TPR + j;
-            v[i] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-            if (kb < kb_total) v[i] = *reinterpret_cast<const f16x8 *>(src + (size_t)kb * 8);
+            for (int i = 0; i < NP; ++i) {
+                const int kb = i * TPR + j;
+                v[i] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                if (kb < kb_total) v[i] = *reinterpret_cast<const f16x8 *>(src + (size_t)kb * 8);
+            }
+        }
+    }
+    // the next block row's weights are requested before this one's arithmetic (registers for both up to NP = 8)
+    f16x8 vn[AHEAD ? NP : 1];
+    if constexpr (AHEAD) {
+        if (mb + (int)gridDim.x < (m >> 3)) {
+            const f16 *srcn = src + (size_t)gridDim.x * 8 * k;
+#pragma unroll
+            for (int i = 0; i < NP; ++i) {
+                const int kb = i * TPR + j;
+                vn[i] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                if (kb < kb_total) vn[i] = *reinterpret_cast<const f16x8 *>(srcn + (size_t)kb * 8);
+            }
         }
     }
     if (by_row) {
@@ -548,14 +566,18 @@ __global__ __launch_bounds__(512, NP == 16 ? 2 : 4) void quantize_kernel(const f
                 d |= best << (8 * (e >> 1) + 4 * (1 - (e & 1)));  // byte e/2 of the dword; even column = high nibble
             }
         }
-        uint32_t *tb = tile[st & 1];
-        tb[j * 8 + r8] = d;
-        __syncthreads();  // (the other buffer was read before the previous step's barrier)
-        if (tid < 2 * TPR) {
-            const int kb0 = st * TPR;
-            const int kbw = kb0 + (tid >> 1);  // block column of the 16 bytes this thread writes
-            if (kbw < kb_total)
-                *reinterpret_cast<u32x4 *>(q32 + ((size_t)mb * kb_total + kb0) * 8 + tid * 4) = *reinterpret_cast<const u32x4 *>(tb + tid * 4);
+        if constexpr (NP > 0) {
+            tile[st][j * 8 + r8] = d;  // (stored after the block row's last step)
+        } else {
+            uint32_t *tb = tile[st & 1];
+            tb[j * 8 + r8] = d;
+            __syncthreads();  // (the other buffer was read before the previous step's barrier)
+            if (tid < 2 * TPR) {
+                const int kb0 = st * TPR;
+                const int kbw = kb0 + (tid >> 1);  // block column of the 16 bytes this thread writes
+                if (kbw < kb_total)
+                    *reinterpret_cast<u32x4 *>(q32 + ((size_t)mb * kb_total + kb0) * 8 + tid * 4) = *reinterpret_cast<const u32x4 *>(tb + tid * 4);
+            }
         }
     };
     if constexpr (NP > 0) {
@@ -563,6 +585,19 @@ __global__ __launch_bounds__(512, NP == 16 ? 2 : 4) void quantize_kernel(const f
 #pragma unroll
         for (int st = 0; st < NP; ++st)
             if (st < n_steps) step(st, v[st]);  // (uniform: every thread of the workgroup takes the same steps)
+        __syncthreads();  // the block row's records are complete
+        // 16 bytes per thread and pass: the records of NP * 64 block columns, contiguous in the packed layout
+#pragma unroll
+        for (int p = tid; p < NP * 2 * TPR; p += 512) {
+            const int kbw = p >> 1;  // block column of the 16 bytes this thread writes
+            if (kbw < kb_total)
+                *reinterpret_cast<u32x4 *>(q32 + (size_t)mb * kb_total * 8 + (size_t)p * 4) =
+                    *reinterpret_cast<const u32x4 *>(&tile[0][0] + p * 4);
+        }
+        if constexpr (AHEAD) {
+#pragma unroll
+            for (int i = 0; i < NP; ++i) v[i] = vn[i];
+        }
     } else {
         for (int st = 0; st < n_steps; ++st) {
             const int kb = st * TPR + j;
@@ -571,7 +606,7 @@ __global__ __launch_bounds__(512, NP == 16 ? 2 : 4) void quantize_kernel(const f
             step(st, t);
         }
     }
-    __syncthreads();  // (the next block row's first step reuses the tile buffer the last step may still be read from)
+    __syncthreads();  // (the next block row writes the tile buffers this one's stores read)
     }
     };
     if (tabled) run(std::integral_constant<int, 0>{});
