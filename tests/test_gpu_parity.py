@@ -534,10 +534,14 @@ TILED = [(256, 8), (256, 4), (128, 16), (128, 8), (64, 16), (64, 8)]   # (lds_ti
 
 
 @pytest.mark.parametrize("tile", TILED)
-@pytest.mark.parametrize("m,n,k,split", [(512, 256, 512, 1), (520, 300, 1096, 1), (256, 70, 2048, 4), (1024, 129, 200, 3)])
+@pytest.mark.parametrize("m,n,k,split", [(512, 256, 512, 1), (520, 300, 1096, 1), (256, 70, 2048, 4), (1024, 129, 200, 3),
+                                         (256, 40, 64, 1), (264, 130, 192, 1), (512, 64, 320, 1), (256, 200, 576, 1),
+                                         (128, 260, 1088, 1), (256, 33, 1408, 2)])
 def test_many_token_kernel_matches_oracle(tile, m, n, k, split):
     """Every tile shape of the many-token kernel, ragged m / n / k and split-K, against the
-    oracle's float64 contraction of the same fp16 weights."""
+    oracle's float64 contraction of the same fp16 weights; k ranges of 1, 2, 3, 5, 9, 11, 17 and 18 steps per
+    workgroup (the loop is unrolled by the four or eight register sets: every length of its tail, a split that
+    gets no step at all)."""
     rows, tt = tile
     c = cfg(lds_tile_rows=rows, token_tiles=tt, split_k=split)
     print(f"many-token tile {rows}x{16 * tt} m={m} n={n} k={k} split={split}", flush=True)
