@@ -354,30 +354,31 @@ __device__ __forceinline__ uint32_t nearest_sorted(float nv, const float (&b)[16
     return (b3 ? 8u : 0u) + (b2 ? 4u : 0u) + (b1 ? 2u : 0u) + (b0 ? 1u : 0u);  // a NaN nv ends at 0 like the argmin
 }
 
-// The same count of boundaries <= nv without the search: the quotients lie in [-1, 1], cut into 128 buckets
-// of 1/64; when no two boundaries share a bucket, a bucket knows how many boundaries lie below it and the one
+// The same count of boundaries <= nv without the search: the quotients lie in [-1, 1], cut into 64 buckets
+// of 1/32; when no two boundaries share a bucket, a bucket knows how many boundaries lie below it and the one
 // boundary (if any) inside it, and the index is that count plus one comparison.  bucket_of is monotonic in
 // nv (a fused multiply-add, a clamp, a truncation), so every value of a lower bucket is below the boundary
 // of a higher one and vice versa: the result is the binary search's for every nv, NaN included (bucket 0, the
-// comparison false, index 0).  Two LDS tables in the lane-private layout of the GEMM's decode table (entry e
-// of lane l at (e << 8) | (l << 2), resp. (e << 6) | l: no bank conflicts whatever the data).
-constexpr int kQuantBuckets = 129;
-constexpr int kQuantBndBytes = kQuantBuckets * 256;  // fp32 boundary of the bucket, +inf if none
-constexpr int kQuantLoBytes = kQuantBuckets * 64;    // boundaries below the bucket, one byte
+// comparison false, index 0).  One LDS table of {boundary, count} pairs in the lane-private layout of the
+// GEMM's decode table (entry e of lane l at (e << 9) | (l << 3): one 8-byte read, no bank conflicts whatever
+// the data).
+constexpr int kQuantBuckets = 65;
+constexpr int kQuantTabBytes = kQuantBuckets * 512;  // per bucket and lane: fp32 boundary (+inf if none), boundaries below it
 typedef __attribute__((address_space(3))) unsigned char lds_u8;
-typedef __attribute__((address_space(3))) uint32_t lds_word;
+typedef uint32_t quant_u32x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) quant_u32x2 lds_pair;
 
 __device__ __forceinline__ uint32_t bucket_of(float nv)
 {
-    return (uint32_t)__builtin_amdgcn_fmed3f(__builtin_fmaf(nv, 64.0f, 64.0f), 0.0f, 128.0f);
+    return (uint32_t)__builtin_amdgcn_fmed3f(__builtin_fmaf(nv, 32.0f, 32.0f), 0.0f, 64.0f);
 }
 
-__device__ __forceinline__ uint32_t nearest_bucketed(float nv, uint32_t bnd_lane, uint32_t lo_lane)
+__device__ __forceinline__ uint32_t nearest_bucketed(float nv, uint32_t tab_lane)
 {
     const uint32_t e = bucket_of(nv);
-    const float b = __builtin_bit_cast(float, *reinterpret_cast<const lds_word *>((uintptr_t)((e << 8) + bnd_lane)));
-    const uint32_t lo = *reinterpret_cast<const lds_u8 *>((uintptr_t)((e << 6) + lo_lane));
-    return lo + (nv >= b ? 1u : 0u);
+    const quant_u32x2 t = *reinterpret_cast<const lds_pair *>((uintptr_t)((e << 9) + tab_lane));
+    const uint32_t bnd_bits = t[0], below = t[1];
+    return below + (nv >= __builtin_bit_cast(float, bnd_bits) ? 1u : 0u);
 }
 
 __device__ __forceinline__ uint32_t nearest_any(float nv, const float (&c)[16])
@@ -397,26 +398,57 @@ __device__ __forceinline__ uint32_t nearest_any(float nv, const float (&c)[16])
 
 // Smallest binary32 v in [lo, hi] for which the argmin prefers hi: |v - hi| < |v - lo| in fp32
 // arithmetic (ties keep the lower index).  The predicate is monotonic in v (both rounded differences
-// are), so a bisection over the bit patterns finds it; lo < hi, and it holds at v = hi.
+// are), so a bisection over the bit patterns finds it; lo < hi finite, and it holds at v = hi.  Two probes
+// 64 patterns either side of the rounded midpoint come first: the boundary lies between them unless the
+// midpoint is tiny against the gap, and the bisection then takes 7 steps instead of 31.
 __device__ inline float decision_boundary(float lo, float hi)
 {
-    auto key = [](float f) {  // order-preserving map of finite floats to integers
-        const int64_t i = (int64_t)__builtin_bit_cast(int32_t, f);
+    auto key = [](float f) {  // order-preserving map of finite floats to integers (both zeros -> 0)
+        const int32_t i = __builtin_bit_cast(int32_t, f);
         return i < 0 ? -(i & 0x7fffffff) : i;
     };
-    auto unkey = [](int64_t k) {
+    auto unkey = [](int32_t k) {
         const uint32_t i = k < 0 ? (uint32_t)(-k) | 0x80000000u : (uint32_t)k;
         return __builtin_bit_cast(float, i);
     };
-    int64_t a = key(lo), b = key(hi);  // predicate false at a (distance 0 to lo), true at b
-    while (b - a > 1) {
-        const int64_t mid = a + ((b - a) >> 1);
-        const float v = unkey(mid);
-        if (fabsf(__fsub_rn(v, hi)) < fabsf(__fsub_rn(v, lo))) b = mid;
+    auto prefers_hi = [&](int32_t kv) {
+        const float v = unkey(kv);
+        return fabsf(__fsub_rn(v, hi)) < fabsf(__fsub_rn(v, lo));
+    };
+    int32_t a = key(lo), b = key(hi);  // predicate false at a (distance 0 to lo), true at b; b - a < 2^32
+    const int32_t mid0 = key(0.5f * lo + 0.5f * hi);
+#pragma unroll
+    for (int side = -1; side <= 1; side += 2) {
+        const int64_t want = (int64_t)mid0 + side * 64;
+        if (want > (int64_t)a && want < (int64_t)b) {
+            const int32_t p = (int32_t)want;
+            if (prefers_hi(p)) b = p;
+            else a = p;
+        }
+    }
+    while ((uint32_t)b - (uint32_t)a > 1u) {
+        const int32_t mid = (int32_t)((uint32_t)a + (((uint32_t)b - (uint32_t)a) >> 1));
+        if (prefers_hi(mid)) b = mid;
         else a = mid;
     }
     return unkey(b);
 }
+
+// max(acc, |t|) over eight fp16 values, two at a time: the magnitudes are the bit patterns with the sign
+// cleared, packed maxima never round, and the conversion to fp32 at the end is exact - the maximum the
+// reference forms in fp32, at one instruction per weight.  (NaN is skipped by either form of the maximum.)
+typedef f16 quant_f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ quant_f16x2 pk_absmax8(quant_f16x2 acc, f16x8 t)
+{
+    const u32x4 b = __builtin_bit_cast(u32x4, t) & 0x7fff7fffu;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t pair = b[i];  // (a bit_cast of the vector element itself reads element 0)
+        acc = __builtin_elementwise_max(acc, __builtin_bit_cast(quant_f16x2, pair));
+    }
+    return acc;
+}
+__device__ __forceinline__ float pk_absmax_value(quant_f16x2 acc) { return fmaxf((float)acc[0], (float)acc[1]); }
 
 template <int NP>
 __global__ __launch_bounds__(512, NP == 16 ? 2 : 4) void quantize_kernel(const f16 *__restrict__ w, const float *__restrict__ code,
@@ -425,7 +457,8 @@ __global__ __launch_bounds__(512, NP == 16 ? 2 : 4) void quantize_kernel(const f
 {
     __shared__ float cs[16], bs_[15];
     __shared__ int fast_s, tab_s, jb_s[15];
-    extern __shared__ __align__(16) unsigned char qtab[];  // bucket tables: boundaries, then counts
+    __shared__ uint32_t pair_s[kQuantBuckets][2];
+    extern __shared__ __align__(16) unsigned char qtab[];  // bucket table
     constexpr int TPR = 64;  // threads per weight row: a row's threads read 1 KB contiguous
     // records of the block row being assembled: [step][block column of the step (64)][row (8)] - all NP steps
     // of a row held in registers (one barrier per block row), or two buffers of one step each (NP == 0)
@@ -458,24 +491,23 @@ __global__ __launch_bounds__(512, NP == 16 ? 2 : 4) void quantize_kernel(const f
     __syncthreads();
     const bool tabled = tab_s != 0;
     const uint32_t tab0 = (uint32_t)(uintptr_t)(lds_u8 *)qtab;
-    const uint32_t bnd_lane = tab0 + ((uint32_t)(tid & 63) << 2);
-    const uint32_t lo_lane = tab0 + (uint32_t)kQuantBndBytes + (uint32_t)(tid & 63);
+    const uint32_t tab_lane = tab0 + ((uint32_t)(tid & 63) << 3);
     if (tabled) {
-        for (int p = tid; p < kQuantBndBytes / 16; p += 512) {  // 16 stores of 16 bytes per bucket
-            const int e = p >> 4;
+        if (tid < kQuantBuckets) {  // a bucket's pair: its boundary (+inf: none) and the boundaries below it
             float b = __builtin_inff();
-#pragma unroll
-            for (int i = 0; i < 15; ++i) b = jb_s[i] == e ? bs_[i] : b;
-            const uint32_t u = __builtin_bit_cast(uint32_t, b);
-            reinterpret_cast<u32x4 *>(qtab)[p] = u32x4{u, u, u, u};
-        }
-        for (int p = tid; p < kQuantLoBytes / 16; p += 512) {   // 4 stores of 16 bytes per bucket
-            const int e = p >> 2;
             uint32_t n = 0;
 #pragma unroll
-            for (int i = 0; i < 15; ++i) n += jb_s[i] < e ? 1u : 0u;
-            n *= 0x01010101u;
-            reinterpret_cast<u32x4 *>(qtab + kQuantBndBytes)[p] = u32x4{n, n, n, n};
+            for (int i = 0; i < 15; ++i) {
+                b = jb_s[i] == tid ? bs_[i] : b;
+                n += jb_s[i] < tid ? 1u : 0u;
+            }
+            pair_s[tid][0] = __builtin_bit_cast(uint32_t, b);
+            pair_s[tid][1] = n;
+        }
+        __syncthreads();
+        for (int p = tid; p < kQuantTabBytes / 16; p += 512) {  // 32 stores of 16 bytes (two lanes' pairs) per bucket
+            const uint32_t u = pair_s[p >> 5][0], n = pair_s[p >> 5][1];
+            reinterpret_cast<u32x4 *>(qtab)[p] = u32x4{u, n, u, n};
         }
     }
     __syncthreads();
@@ -525,18 +557,14 @@ __global__ __launch_bounds__(512, NP == 16 ? 2 : 4) void quantize_kernel(const f
         }
     }
     if (by_row) {
+        quant_f16x2 pm = quant_f16x2{(f16)0.f, (f16)0.f};
         if constexpr (NP > 0) {
 #pragma unroll
-            for (int i = 0; i < NP; ++i)
-#pragma unroll
-                for (int e = 0; e < 8; ++e) row_max = fmaxf(row_max, fabsf((float)v[i][e]));
+            for (int i = 0; i < NP; ++i) pm = pk_absmax8(pm, v[i]);
         } else {
-            for (int kb = j; kb < kb_total; kb += TPR) {
-                const f16x8 t = *reinterpret_cast<const f16x8 *>(src + (size_t)kb * 8);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) row_max = fmaxf(row_max, fabsf((float)t[e]));
-            }
+            for (int kb = j; kb < kb_total; kb += TPR) pm = pk_absmax8(pm, *reinterpret_cast<const f16x8 *>(src + (size_t)kb * 8));
         }
+        row_max = pk_absmax_value(pm);
 #pragma unroll
         for (int off = TPR / 2; off >= 1; off >>= 1) row_max = fmaxf(row_max, __shfl_xor(row_max, off, TPR));
         if (j == 0) absmax[row] = row_max;
@@ -547,9 +575,7 @@ __global__ __launch_bounds__(512, NP == 16 ? 2 : 4) void quantize_kernel(const f
         const int kb = st * TPR + j;
         float amax = row_max;
         if (!by_row) {
-            amax = 0.f;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf((float)t[e]));
+            amax = pk_absmax_value(pk_absmax8(quant_f16x2{(f16)0.f, (f16)0.f}, t));
             for (int off = 1; off < lanes_blk; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, TPR));
             if (kb < kb_total && (j & (lanes_blk - 1)) == 0) absmax[(size_t)row * nblk + (kb * 8) / bs] = amax;
         }
@@ -560,7 +586,7 @@ __global__ __launch_bounds__(512, NP == 16 ? 2 : 4) void quantize_kernel(const f
             for (int e = 0; e < 8; ++e) {
                 const float nv = div_by_block_max((float)t[e], amax, y);
                 uint32_t best;
-                if constexpr (MODE == 0) best = nearest_bucketed(nv, bnd_lane, lo_lane);
+                if constexpr (MODE == 0) best = nearest_bucketed(nv, tab_lane);
                 else if constexpr (MODE == 1) best = nearest_sorted(nv, c);
                 else best = nearest_any(nv, c);
                 d |= best << (8 * (e >> 1) + 4 * (1 - (e & 1)));  // byte e/2 of the dword; even column = high nibble
@@ -655,7 +681,7 @@ hipError_t launch_quantize(const void *w, const float *code, void *q, float *abs
     if (e != hipSuccess) return e;
     const int rows8 = m / 8;
     const dim3 grid((unsigned)(rows8 < 3 * cus ? rows8 : 3 * cus)), block(512);
-    const size_t lds = (size_t)kQuantBndBytes + kQuantLoBytes;
+    const size_t lds = (size_t)kQuantTabBytes;
     if (k <= 512 * 4) hipLaunchKernelGGL(quantize_kernel<4>, grid, block, lds, stream, wp, code, qp, absmax, m, k, bs);
     else if (k <= 512 * 8) hipLaunchKernelGGL(quantize_kernel<8>, grid, block, lds, stream, wp, code, qp, absmax, m, k, bs);
     else if (k <= 512 * 16) hipLaunchKernelGGL(quantize_kernel<16>, grid, block, lds, stream, wp, code, qp, absmax, m, k, bs);
