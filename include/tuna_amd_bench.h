@@ -85,6 +85,16 @@ int tuna_set_multi_shape(int waves_m, int prefetch);
  * (global -> LDS loads, as the LDS-staged twins of the streaming kernel do) instead of registers.
  * Bit-identical results; for A/B timing.  Returns the previous setting. */
 int tuna_set_multi_weight_path(int through_lds);
+/* Diagnostic switch, process-wide, default 1: tuna_matmul_blockwise runs launches of up to 16 tokens and at least 20 MB
+ * of packed weights whose shape allows (m a multiple of 64, k of 256 and of the block) through the scale-block variant
+ * of the batched streaming kernel as a batch of one; 2: every launch whose shape allows, whatever its size; 0: always
+ * the narrow-row kernel's variants.  Both decode fp16(code) * fp16(absmax of the block); the sums differ in summation
+ * order only.  Returns the previous setting. */
+int tuna_set_blockwise_stream(int enabled);
+/* Diagnostic override of the kernel variant tuna_matmul_blockwise runs: rows per workgroup (16, 32 or 64), waves along k
+ * (4, 8 or 16) and ring depth (2 or 4); all zero = the library's choice.  TUNA_ERR_INVALID_ARG if no such variant is built;
+ * a variant that does not fit a later call's shape makes that call fail with TUNA_ERR_UNSUPPORTED.  For A/B timing. */
+int tuna_set_blockwise_shape(int rows, int waves_k, int prefetch);
 /* Diagnostic: the shortest run of problems tuna_matmul_multi hands to the batched kernel
  * (default 2; 1 sends single problems through it as well).  Returns the previous value. */
 int tuna_set_multi_min_batch(int count);

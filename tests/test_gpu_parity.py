@@ -1458,6 +1458,54 @@ def test_blockwise_gemm_matches_oracle_and_reads_out_the_decode(m, n, k, bs):
     assert np.array_equal(out.cpu().numpy().view(np.uint16), img[:, cols].T)
 
 
+@pytest.mark.parametrize("m,n,k,bs", [(256, 16, 1280, 64), (128, 7, 1536, 64), (512, 16, 4096, 128), (1024, 1, 2048, 256),
+                                      (256, 16, 2048, 512), (768, 13, 5120, 64), (4096, 16, 4096, 64), (8192, 16, 8192, 64)])
+def test_blockwise_gemm_through_the_batched_streaming_kernel(m, n, k, bs):
+    """The scale-block variant of the batched streaming kernel (tuna_matmul_blockwise takes it from 20 MB of packed
+    weights; the switch sends every shape it can plan there): against the oracle's float64 sums over the blockwise D1
+    weights on a row sample, bit-exact through one-hot activations (every scale block of every sampled column read
+    out), and run-to-run identical.  k ranges that are not whole x chunks, 128-row tiles, blocks longer than a chunk,
+    shares that split row tiles (hand-over through the workspace)."""
+    import torch
+
+    from tuna_amd import _lib, ops
+
+    rng = np.random.default_rng(m + n + k + bs + 1)
+    q, x, code, _ = make_inputs_np(m, n, k, seed=m + bs + 1)
+    absmax = rng.uniform(0.005, 0.02, size=(m, k // bs)).astype(np.float16).astype(np.float32)
+    dq, dx, dc, da = to_dev(q, x, code, absmax)
+    out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+    L = _lib.lib()
+    prev = L.tuna_set_blockwise_stream(2)
+    launches = L.tuna_multi_launches()
+    try:
+        print(f"blockwise through the batched kernel m={m} n={n} k={k} block={bs}", flush=True)
+        ops.matmul_blockwise(dx, dq, da, dc, out, m, n, k, bs)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy().view(np.uint16)
+        assert L.tuna_multi_launches() == launches + 1     # the batched kernel ran it
+        assert not np.isnan(got.view(np.float16)).any()
+        rows = np.sort(rng.choice(m, size=min(m, 192), replace=False)).astype(np.int32)
+        ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1, rows=rows, block_size=bs)
+        e = rel_err(f16_bits_to_f64(got[:, rows]), ref)
+        assert e <= REL_TOL, e
+        again = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+        ops.matmul_blockwise(dx, dq, da, dc, again, m, n, k, bs)
+        torch.cuda.synchronize()
+        assert np.array_equal(again.cpu().numpy().view(np.uint16), got)
+        img = O.dequant(q, absmax, code, m, k, mode=O.D1, block_size=bs)
+        for rep in range(2):
+            cols = rng.choice(k, size=n, replace=False)
+            xh = np.zeros((n, k), np.float16)
+            xh[np.arange(n), cols] = 1.0
+            dxh, = to_dev(xh)
+            ops.matmul_blockwise(dxh, dq, da, dc, out, m, n, k, bs)
+            torch.cuda.synchronize()
+            assert np.array_equal(out.cpu().numpy().view(np.uint16), img[:, cols].T)
+    finally:
+        L.tuna_set_blockwise_stream(prev)
+
+
 def test_blockwise_entry_points_reject_what_they_cannot_run():
     import torch
 

@@ -101,6 +101,8 @@ SIGNATURES = {
     "tuna_selftest_quantizer_division": (_i, [_vp, _vp]),
     "tuna_set_multi_shape": (_i, [_i, _i]),
     "tuna_set_multi_min_batch": (_i, [_i]),
+    "tuna_set_blockwise_shape": (_i, [_i, _i, _i]),
+    "tuna_set_blockwise_stream": (_i, [_i]),
     "tuna_multi_launches": (ctypes.c_ulonglong, []),
     "tuna_set_lean_kernels": (_i, [_i]),
     "tuna_set_weight_path": (_i, [_i]),

@@ -676,6 +676,7 @@ static int check_ptr(const void *p, const char *name, size_t align)
 // launched problem by problem on the same stream.
 // ---------------------------------------------------------------------------------------
 static std::atomic<int> g_multi_waves_m{0}, g_multi_prefetch{0};  // 0: the library's choice (diagnostic override)
+static std::atomic<int> g_blockwise_stream{1};  // tuna_matmul_blockwise takes the batched kernel's scale-block variant where it can
 static std::atomic<int> g_multi_lds{0};  // batches with a ring of 2 stage weights and x through LDS (tuna_set_multi_weight_path)
 static std::atomic<unsigned long long> g_multi_launches{0};
 static std::atomic<int> g_multi_min_batch{2};  // batches shorter than this are launched problem by problem
@@ -688,15 +689,18 @@ struct MultiPlan {
 
 // Whether problems[0..count) can run as one launch on a device of `cus` compute units; fills `plan`.
 // waves_m / prefetch: 0 = chosen here.
-static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, MultiPlan *plan, int waves_m = 0, int prefetch = 0)
+// blk_shift >= 0: every problem's absmax is [m, k / (64 << blk_shift)], one scale per block of a row (the BLK variants).
+static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, MultiPlan *plan, int waves_m = 0, int prefetch = 0,
+                       int blk_shift = -1)
 {
     if (count < 1 || count > kMaxMultiProblems || cus < 1) return false;
+    const bool blk = blk_shift >= 0;
     if (!waves_m) waves_m = g_multi_waves_m.load(std::memory_order_relaxed);
     if (!prefetch) prefetch = g_multi_prefetch.load(std::memory_order_relaxed);
     // (a ring of two: with every wait of the ring exact it streams as fast as a ring of four on the longest
     // batches and faster on the others - fewer bytes requested ahead at a segment switch)
     if (!prefetch) prefetch = 2;
-    if (!multi_variant_exists(prefetch)) return false;
+    if (!multi_variant_exists(blk ? 10 + prefetch : prefetch)) return false;
     if (!waves_m) {
         // 256-row tiles (4 x 4 waves) when every problem allows, else narrower tiles and more waves along k
         waves_m = 4;
@@ -715,8 +719,10 @@ static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, Mu
         }
     }
     if (waves_m != 1 && waves_m != 2 && waves_m != 4 && waves_m != 8 && waves_m != 16) return false;
+    if (blk && waves_m > 4) return false;  // the scale buffers hold 256 rows
     const int waves_k = 16 / waves_m;
-    if ((32 / waves_k) % prefetch) return false;  // an x chunk of 32 k-steps is whole ring turns of every wave
+    // an x chunk of 32 k-steps (16 with scale blocks) is whole ring turns of every wave
+    if (((blk ? 16 : 32) / waves_k) % prefetch || (blk ? 16 : 32) < waves_k * prefetch) return false;
     const int unit_steps = waves_k * prefetch;
     MultiArgs &a = plan->args;
     memset(&a, 0, sizeof(a));
@@ -725,7 +731,8 @@ static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, Mu
         const tuna_gemm_problem &p = problems[i];
         if (p.n > 16 || p.m % (64 * waves_m) || p.k % (kStepK * unit_steps)) return false;
         if ((unsigned long long)p.m * (unsigned long long)p.k / 2 >= (1ull << 32) || p.k >= (1 << 23)) return false;
-        if (reinterpret_cast<uintptr_t>(p.absmax) % 16) return false;
+        if (reinterpret_cast<uintptr_t>(p.absmax) % (blk ? 4 : 16)) return false;
+        if (blk && (p.k % (64 << blk_shift) || p.k / (64 << blk_shift) < 2)) return false;
         if (p.code != problems[0].code) return false;  // one decode table per launch
         MultiProblem &mp = a.prob[i];
         mp.q = static_cast<const uint8_t *>(p.q);
@@ -756,10 +763,11 @@ static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, Mu
     a.wk_log2 = log2i(waves_k);
     a.n_wg = n_wg;
     a.swizzle = (n_wg % 8 == 0) ? 1 : 0;
+    a.blk_shift = blk ? blk_shift : 0;
     // variant -2: ring of 2 with weights and x staged through LDS (x chunks of 512 k: every wave needs a whole
     // number of ring turns per chunk, so at most 8 waves along k)
-    const bool lds = g_multi_lds.load(std::memory_order_relaxed) != 0 && prefetch == 2 && waves_k <= 8 && multi_variant_exists(-2);
-    plan->prefetch = lds ? -2 : prefetch;
+    const bool lds = !blk && g_multi_lds.load(std::memory_order_relaxed) != 0 && prefetch == 2 && waves_k <= 8 && multi_variant_exists(-2);
+    plan->prefetch = blk ? 10 + prefetch : lds ? -2 : prefetch;
     plan->ws_bytes = (size_t)n_wg * 2 * waves_m * 4096;
     plan->n_counters = (size_t)tiles;
     return true;
@@ -1218,6 +1226,31 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
     if ((rc = check_ptr(q, "q", 16)) || (rc = check_ptr(x, "x", 16)) || (rc = check_ptr(code, "code", 4)) ||
         (rc = check_ptr(absmax, "absmax", 4)) || (rc = check_ptr(out, "out", 16)))
         return rc;
+    // Up to 16 tokens, aligned shapes: the batched streaming kernel's scale-block variant as a batch of one (balanced
+    // split over one workgroup per compute unit).  Everything else: the narrow-row kernel's.
+    // (below about 20 MB of packed weights the narrow-row kernel's single pass is faster: 12.1 against 16.1 us on
+    // 6144 x 4096, 21.4 against 16.5 us on 4096 x 14336)
+    const int stream_mode = g_blockwise_stream.load(std::memory_order_relaxed);
+    if (n <= 16 && (stream_mode == 2 || (stream_mode == 1 && (long long)m * k / 2 >= (20ll << 20)))) {
+        int dev = 0, cus = 0;
+        hipError_t e = device_cus(&dev, &cus);
+        if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+        const tuna_gemm_problem one = {q, x, code, absmax, out, m, n, k};
+        MultiPlan plan;
+        // the batched kernel's own choice of tile height (256 rows, 128 where those are fewer than workgroups), ring of two;
+        // then whatever height the row count allows
+        bool ok = plan_multi(&one, 1, cus, &plan, 0, 0, log2i(block_size) - 6);
+        for (int wm = 4; wm >= 1 && !ok; wm >>= 1) ok = plan_multi(&one, 1, cus, &plan, wm, 2, log2i(block_size) - 6);
+        if (ok) {
+            if ((rc = provide_workspace(false, static_cast<hipStream_t>(stream), plan.ws_bytes, plan.n_counters, &plan.args.ws,
+                                        &plan.args.counters)))
+                return rc;
+            e = launch_gemm_multi(plan.args, plan.prefetch, dev, static_cast<hipStream_t>(stream));
+            if (e != hipSuccess) return hip_fail(e, "blockwise gemm launch");
+            g_multi_launches.fetch_add(1, std::memory_order_relaxed);
+            return TUNA_OK;
+        }
+    }
     NarrowArgs a;
     memset(&a, 0, sizeof(a));
     a.q = static_cast<const uint8_t *>(q);
@@ -1509,6 +1542,18 @@ TUNA_EXPORT int tuna_time_unit_rate(int unit, void *sink, int warmup, int iters,
         return e2 == hipSuccess ? (int)TUNA_OK : hip_fail(e2, "unit-rate launch");
     };
     return time_loop(launch, 1, warmup, iters, 0, static_cast<hipStream_t>(stream), elapsed_ms);
+}
+
+TUNA_EXPORT int tuna_set_blockwise_stream(int enabled)
+{
+    return g_blockwise_stream.exchange(enabled < 0 ? 0 : enabled > 2 ? 2 : enabled, std::memory_order_relaxed);
+}
+
+TUNA_EXPORT int tuna_set_blockwise_shape(int rows, int waves_k, int prefetch)
+{
+    if (set_blockwise_shape(rows, waves_k, prefetch))
+        return fail(TUNA_ERR_INVALID_ARG, "no blockwise GEMM variant with %d rows, %d waves, ring %d", rows, waves_k, prefetch);
+    return TUNA_OK;
 }
 
 TUNA_EXPORT int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config *cfg, int decode_mode, char *buf, size_t len)

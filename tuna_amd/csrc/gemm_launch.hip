@@ -293,24 +293,90 @@ hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int
     return hipGetLastError();
 }
 
-// Scale blocks finer than a row: the narrow-row kernel's BLK variant, 16 rows per workgroup, 4 waves
-// along k, ring of 2.  block = 64 << blk_shift weights per scale.
+// Scale blocks finer than a row: the narrow-row kernel's BLK variants (the scales of a ring slot's block travel
+// through the ring with its weights).  block = 64 << blk_shift weights per scale.
+struct BlockwiseVariant {
+    int rows, wk, u;
+    NarrowKernelFn fn, fn_perm;
+};
+#define B(LW, WK, U) {16 * LW, WK, U, gemm_narrow_kernel<LW, WK, U, false, 1, true>, gemm_narrow_kernel<LW, WK, U, true, 1, true>}
+static const BlockwiseVariant kBlockwise[] = {
+    B(1, 4, 2), B(1, 8, 4), B(1, 16, 2), B(2, 8, 2), B(2, 8, 4), B(2, 16, 2), B(4, 4, 4), B(4, 8, 2), B(4, 8, 4), B(4, 16, 2),
+};
+#undef B
+static constexpr int kNumBlockwise = sizeof(kBlockwise) / sizeof(kBlockwise[0]);
+static std::atomic<int> g_blockwise_shape[3];  // diagnostic override: rows, waves_k, ring depth (0: the library's choice)
+
+int set_blockwise_shape(int rows, int waves_k, int prefetch)
+{
+    if (rows || waves_k || prefetch) {
+        bool found = false;
+        for (int i = 0; i < kNumBlockwise; ++i)
+            found |= kBlockwise[i].rows == rows && kBlockwise[i].wk == waves_k && kBlockwise[i].u == prefetch;
+        if (!found) return -1;
+    }
+    g_blockwise_shape[0].store(rows);
+    g_blockwise_shape[1].store(waves_k);
+    g_blockwise_shape[2].store(prefetch);
+    return 0;
+}
+
+static bool blockwise_fits(const BlockwiseVariant &v, int m, int k) { return m % v.rows == 0 && k % (kStepK * v.wk * v.u) == 0; }
+
+// The library's choice: the widest tile that still gives three workgroups per four compute units (measured on the
+// benchmark shapes with a scale per 64 weights).
+static const BlockwiseVariant *choose_blockwise(int m, int k, int cus)
+{
+    const int ov_rows = g_blockwise_shape[0].load();
+    if (ov_rows) {
+        const int wk = g_blockwise_shape[1].load(), u = g_blockwise_shape[2].load();
+        for (int i = 0; i < kNumBlockwise; ++i)
+            if (kBlockwise[i].rows == ov_rows && kBlockwise[i].wk == wk && kBlockwise[i].u == u && blockwise_fits(kBlockwise[i], m, k))
+                return &kBlockwise[i];
+        return nullptr;
+    }
+    static const int pref[][3] = {{64, 8, 4}, {64, 8, 2}, {32, 8, 4}, {32, 8, 2}, {16, 8, 4}, {16, 4, 2}};
+    const BlockwiseVariant *fallback = nullptr;
+    for (const auto &p : pref)
+        for (int i = 0; i < kNumBlockwise; ++i) {
+            const BlockwiseVariant &v = kBlockwise[i];
+            if (v.rows != p[0] || v.wk != p[1] || v.u != p[2] || !blockwise_fits(v, m, k)) continue;
+            if (!fallback) fallback = &v;
+            if (m / v.rows >= cus * 3 / 4) return &v;
+        }
+    if (fallback) {  // fewer row tiles than compute units at every height: the narrowest tile that fits
+        for (int i = 0; i < kNumBlockwise; ++i)
+            if (blockwise_fits(kBlockwise[i], m, k) && kBlockwise[i].rows < fallback->rows) fallback = &kBlockwise[i];
+    }
+    return fallback;
+}
+
+bool blockwise_describe(int m, int n, int k, char *buf, size_t len)
+{
+    const BlockwiseVariant *v = choose_blockwise(m, k, kMaxCus);
+    if (!v) return false;
+    snprintf(buf, len, "gemm_narrow_kernel<LW=%d,WK=%d,U=%d,PERM=%d,TT=1,BLK>", v->rows / 16, v->wk, v->u, n > 4 ? 1 : 0);
+    return true;
+}
+
 hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, hipStream_t stream)
 {
-    constexpr int WK = 4, U = 2;
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
+    int dev = 0, cus = 0;
+    hipError_t e = device_cus(&dev, &cus);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
+    const BlockwiseVariant *v = choose_blockwise(args.m, args.k, cus);
+    if (!v) return hipErrorInvalidConfiguration;
+    const int vi = (int)(v - kBlockwise);
     const int perm = args.n > 4;
-    const NarrowKernelFn fn = perm ? gemm_narrow_kernel<1, WK, U, true, 1, true> : gemm_narrow_kernel<1, WK, U, false, 1, true>;
-    static OptInFlag done[16][2];
-    if ((e = ensure_lds_opt_in(done[dev][perm], reinterpret_cast<const void *>(fn))) != hipSuccess) return e;
-    const size_t lds = (size_t)kLutBytes + (size_t)WK * 1024;
-    const dim3 grid((unsigned)(args.m / 16), (unsigned)((args.n + 15) / 16), 1);
+    const NarrowKernelFn fn = perm ? v->fn_perm : v->fn;
+    static OptInFlag done[16][kNumBlockwise][2];
+    if ((e = ensure_lds_opt_in(done[dev][vi][perm], reinterpret_cast<const void *>(fn))) != hipSuccess) return e;
+    const size_t lds = (size_t)kLutBytes + (size_t)v->wk * (v->rows / 16) * 1024;
+    const dim3 grid((unsigned)(args.m / v->rows), (unsigned)((args.n + 15) / 16), 1);
     const int nblk = args.k >> (6 + blk_shift);
-    hipLaunchKernelGGL(fn, grid, dim3(WK * 64), lds, stream, args.q, args.x, args.code, args.absmax, args.k, args.n,
-                       args.k / kStepK / WK, args.m, args.out, TUNA_EPILOGUE_NONE, nullptr, blk_shift, nblk);
+    hipLaunchKernelGGL(fn, grid, dim3(v->wk * 64), lds, stream, args.q, args.x, args.code, args.absmax, args.k, args.n,
+                       args.k / kStepK / v->wk, args.m, args.out, TUNA_EPILOGUE_NONE, nullptr, blk_shift, nblk);
     return hipGetLastError();
 }
 

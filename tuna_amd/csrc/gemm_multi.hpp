@@ -27,6 +27,11 @@
 //     the LDSW twins of gemm_mid.hpp (per-wave weight ring read back with ds_read_b128, x chunks of
 //     512 k straight into the chunk buffer, every wait for a load written out, bare barriers, stores
 //     into LDS the compiler does not look into).  Same arithmetic in the same order: same bits.
+//   * BLK variants: one scale per block of 64 << blk_shift weights of a row (absmax [m, k / block]) instead of one per
+//     row.  x chunks of 512 k; beside each x chunk the scales of the workgroup's rows for the chunk's blocks are
+//     staged in LDS ([block of the chunk][row]: coalesced 8-byte reads of a row's consecutive blocks, one 16-byte
+//     LDS read of a lane's four rows per k-step) and rounded to fp16 when a step is decoded: the decode is
+//     fp16(code) * fp16(absmax of the block), the GEMM's rounding with a finer scale.
 // Requires, for every problem: n <= 16, m a multiple of 64*waves_m, k a multiple of
 // 32*waves_k*U, 16-byte aligned scales; the host falls back to separate launches otherwise.
 #pragma once
@@ -57,6 +62,7 @@ struct MultiArgs {
     int waves_m, wk_log2;
     int n_wg;
     int swizzle;         // n_wg is a multiple of 8: consecutive shares sit on one XCD
+    int blk_shift;       // BLK variants: a scale per 64 << blk_shift weights of a row (every problem of the launch)
     // first unit of every problem in the batch's sequence, and the problem that holds the first unit of
     // every workgroup: a workgroup finds the problem of a unit by walking on from there (its share
     // rarely spans more than two problems), not through a chain of dependent fetches from problem 0
@@ -65,19 +71,22 @@ struct MultiArgs {
     MultiProblem prob[kMaxMultiProblems];
 };
 
-template <int U, bool DEFER = true, bool LDSW = false>
+template <int U, bool DEFER = true, bool LDSW = false, bool BLK = false>
 __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
 {
     static_assert(!LDSW || U == 2, "LDS is full with a ring of two: table 64 KB, x 2 x 16 KB, rings 32 KB, reduction 32 KB");
-    constexpr int XB = 2;                  // 16-byte x pieces per thread and chunk: 16 tokens x 1024 k x 2 B / 1024 threads
-    constexpr int kChunkSteps = LDSW ? 16 : 32;                 // k-steps per x chunk (LDSW: one wave instruction per wave)
-    constexpr uint32_t kXBuf = (LDSW ? 16 : 32) * 1024;         // bytes of one x buffer
+    static_assert(!(LDSW && BLK), "scale blocks: register-staged variants only");
+    constexpr int XB = BLK ? 1 : 2;        // 16-byte x pieces per thread and chunk: 16 tokens x 1024 (BLK: 512) k x 2 B / 1024 threads
+    constexpr int kChunkSteps = (LDSW || BLK) ? 16 : 32;        // k-steps per x chunk (LDSW: one wave instruction per wave)
+    constexpr uint32_t kXBuf = ((LDSW || BLK) ? 16 : 32) * 1024;  // bytes of one x buffer
+    constexpr uint32_t kSBuf = BLK ? 8 * 256 * 4 : 0;           // BLK: bytes of one scale buffer, [block of the chunk (8)][row (256)]
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char *lut = smem;
     unsigned char *xbuf = smem + kLutBytes;  // two x buffers
+    unsigned char *sbuf = smem + kLutBytes + 2 * kXBuf;  // BLK: two scale buffers
     // reduction area: two accumulator planes of all 16 waves (32 KB); its first two words double as the
     // arrival tickets of the hand-over, which are written only after every sum has been read
-    float *redf = reinterpret_cast<float *>(smem + kLutBytes + 2 * kXBuf + (LDSW ? 16 * U * 1024 : 0));
+    float *redf = reinterpret_cast<float *>(smem + kLutBytes + 2 * kXBuf + 2 * kSBuf + (LDSW ? 16 * U * 1024 : 0));
     volatile unsigned *ticket = reinterpret_cast<volatile unsigned *>(redf);
 
     const int tid = threadIdx.x;
@@ -180,6 +189,26 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         }                                                                                      \
     }
 
+    // BLK: the scales of the workgroup's rows for the blocks chunk `c` of a segment touches - thread (row tid / 4,
+    // pair tid % 4) fetches blocks 2 * pair and 2 * pair + 1 behind the chunk's first block (a quad of lanes reads
+    // 32 contiguous bytes of a row of absmax; block indices clamped to the row, rows to the tile: duplicates)
+    const int s_row = min(tid >> 2, rows_wg - 1), s_pair = tid & 3;
+    const int blk_sh = a.blk_shift + 1;  // log2(k-steps per scale block)
+    float sv[2];
+#define TUNA_MULTI_S_LOAD(absmax_, k_, row0_, sb_, nsteps_, c)                                   \
+    {                                                                                          \
+        const int nblk_ = (k_) >> (5 + blk_sh);                                                \
+        const int b0_ = ((sb_) + min((c) * kChunkSteps, (nsteps_) - 1)) >> blk_sh;             \
+        const float *sp_ = (absmax_) + (size_t)((row0_) + s_row) * (size_t)nblk_;              \
+        sv[0] = sp_[min(b0_ + 2 * s_pair, nblk_ - 1)];                                         \
+        sv[1] = sp_[min(b0_ + 2 * s_pair + 1, nblk_ - 1)];                                     \
+    }
+#define TUNA_MULTI_S_STORE(buf)                                                                 \
+    {                                                                                          \
+        reinterpret_cast<float *>(buf)[(2 * s_pair) * 256 + (tid >> 2)] = sv[0];               \
+        reinterpret_cast<float *>(buf)[(2 * s_pair + 1) * 256 + (tid >> 2)] = sv[1];           \
+    }
+
     // LDSW: chunk `c` straight into `buf`, k-step `wave` of the chunk per wave; lane (token i16, 8-k group g)
     // fetches its own B-fragment piece (token rows past n: clamped, their output columns are never stored)
 #define TUNA_MULTI_X_DMA(x_, n_, k_, sb_, nsteps_, c, buf)                                       \
@@ -216,7 +245,8 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         for (int u = 0; u < U; ++u) load_weights_to_lds<true>(qp + (size_t)u * wq_stride + lb, wring + u * 1024);
     } else {
         TUNA_MULTI_X_LOAD(cur.x, cur.n, cur.k, cur.sb, cur.nsteps, 0)
-        sc32 = *reinterpret_cast<const f32x4 *>(cur.absmax + cur.row0 + wm * 64 + i16 * 4);
+        if constexpr (BLK) TUNA_MULTI_S_LOAD(cur.absmax, cur.k, cur.row0, cur.sb, cur.nsteps, 0)
+        else sc32 = *reinterpret_cast<const f32x4 *>(cur.absmax + cur.row0 + wm * 64 + i16 * 4);
         const unsigned char *qp = cur.q + (size_t)(cur.sb + wk) * 128;
 #pragma unroll
         for (int u = 0; u < U; ++u) wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(qp + (size_t)u * wq_stride + lb));
@@ -248,6 +278,7 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         barrier_lds_only();
     } else {
         TUNA_MULTI_X_STORE(cur.n, xbuf)
+        if constexpr (BLK) TUNA_MULTI_S_STORE(sbuf)
         __syncthreads();
     }
     uint32_t xsel = 0;  // buffer that holds the chunk about to be consumed
@@ -302,10 +333,12 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         const uint32_t lb_next = lane_base(nxt);
 
         f16x2 sc16[4];
+        if constexpr (!BLK) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const f16 h = (f16)sc32[j];
-            sc16[j] = f16x2{h, h};
+            for (int j = 0; j < 4; ++j) {
+                const f16 h = (f16)sc32[j];
+                sc16[j] = f16x2{h, h};
+            }
         }
         f32x4 acc[4];
 #pragma unroll
@@ -322,7 +355,8 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         const uint32_t rlb_last = has_next ? lb_next : lb;
         int it = 0;
         // the scales of the next segment (without one: this segment's again), needed when this one ends
-        const f32x4 sc_next = *reinterpret_cast<const f32x4 *>(nxt.absmax + nxt.row0 + wm * 64 + i16 * 4);
+        f32x4 sc_next = f32x4{0.f, 0.f, 0.f, 0.f};
+        if constexpr (!BLK) sc_next = *reinterpret_cast<const f32x4 *>(nxt.absmax + nxt.row0 + wm * 64 + i16 * 4);
         // One ring turn: U of this wave's k-steps consumed and refilled; the refills of the segment's
         // last turn are the first steps of the next segment.
 #define TUNA_MULTI_TURN(sl, first)                                                              \
@@ -342,6 +376,16 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
                 wq[u] = *reinterpret_cast<const u32x4 *>(wring + u * 1024 + lane * 16);        \
             }                                                                                  \
             const f16x8 b_ = *reinterpret_cast<const f16x8 *>(xb + (size_t)((sl) + u) * wstep); \
+            if constexpr (BLK) {                                                               \
+                /* the step's scale block, counted from the chunk's first one */               \
+                const int rel_ = ((sbc + (((sl) + u) << wk_log2) + wk) >> blk_sh) - (sbc >> blk_sh); \
+                const f32x4 s4_ = *reinterpret_cast<const f32x4 *>(sb_lane + (size_t)rel_ * 1024); \
+                _Pragma("unroll") for (int j = 0; j < 4; ++j)                                  \
+                {                                                                              \
+                    const f16 h_ = (f16)s4_[j];                                                \
+                    sc16[j] = f16x2{h_, h_};                                                   \
+                }                                                                              \
+            }                                                                                  \
             _Pragma("unroll") for (int j = 0; j < 4; ++j)                                      \
             {                                                                                  \
                 const f16x8 av_ = decode_dword<TUNA_DECODE_GEMM>(wq[u][j], lut, lane4, sc16[j], 0.f); \
@@ -373,9 +417,17 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
                     TUNA_MULTI_X_DMA(x_, xn_, xk_, xsb_, xns_, xc_, xbuf + (xsel ^ 1u) * kXBuf)
                 } else {
                     TUNA_MULTI_X_LOAD(x_, xn_, xk_, xsb_, xns_, xc_)
+                    if constexpr (BLK) {
+                        const float *am_ = more ? cur.absmax : nxt.absmax;
+                        const int row0_ = more ? cur.row0 : nxt.row0;
+                        TUNA_MULTI_S_LOAD(am_, xk_, row0_, xsb_, xns_, xc_)
+                    }
                 }
             }
             const unsigned char *xb = xbuf + xsel * kXBuf + xb_lane;
+            // BLK: this lane's four rows in the scale buffer of the chunk, and the chunk's first k-step
+            const unsigned char *sb_lane = sbuf + xsel * kSBuf + (size_t)(wm * 64 + i16 * 4) * 4;
+            const int sbc = cur.sb + c * kChunkSteps;
             const int its = min(chunk_its, n_it - it);
             // (the first ring turn of a chunk is a copy of its own: there the x pieces just requested
             // are in flight behind the ring, and only straight-line code lets the compiler count them
@@ -389,6 +441,7 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
                 barrier_lds_only();
             } else {
                 TUNA_MULTI_X_STORE(more ? cur.n : nxt.n, xbuf + (xsel ^ 1u) * kXBuf)
+                if constexpr (BLK) TUNA_MULTI_S_STORE(sbuf + (xsel ^ 1u) * kSBuf)
                 __syncthreads();
             }
             xsel ^= 1u;
@@ -479,6 +532,8 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
 #undef TUNA_MULTI_X_LOAD
 #undef TUNA_MULTI_X_DMA
 #undef TUNA_MULTI_X_STORE
+#undef TUNA_MULTI_S_LOAD
+#undef TUNA_MULTI_S_STORE
 }
 
 }  // namespace tuna
