@@ -298,6 +298,45 @@ def time_quantize(ops, synth, torch, dev):
     return res
 
 
+def time_blockwise(ops, synth, torch, dev, names=("mistral_qkv", "mistral_gate_up", "llama70b_qkv", "llama70b_gate_up", "llama70b_down"),
+                   block_size=64, tokens=16):
+    """tuna_matmul_blockwise (one fp32 scale per `block_size` weights of a row, the layout of block-quantized NF4
+    checkpoints) on some of the 16-token shapes: back-to-back calls through the C ABI over rotating weights, HIP
+    events around them on torch's stream (which the calls launch on).  Algorithmic bytes: packed weights + scales."""
+    from tuna_amd.quantize import nf4_codebook
+
+    code = nf4_codebook(dev)
+    out = {}
+    for nm in names:
+        m, k = synth.SHAPES[nm]
+        nsets = max(2, min(24, int(600e6 // (m * k // 2))))
+        sets = [synth.make_weights_torch(m, k, 70 + i, dev) for i in range(nsets)]
+        scales = [torch.rand((m, k // block_size), dtype=torch.float32, device=dev) * 0.015 + 0.005 for _ in range(nsets)]
+        x = synth.make_x_torch(tokens, k, 3, dev)
+        o = torch.empty((tokens, m), dtype=torch.float16, device=dev)
+        for i in range(50):
+            ops.matmul_blockwise(x, sets[i % nsets][0], scales[i % nsets], code, o, m, tokens, k, block_size)
+        torch.cuda.synchronize()
+        iters = 300
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for i in range(iters):
+            ops.matmul_blockwise(x, sets[i % nsets][0], scales[i % nsets], code, o, m, tokens, k, block_size)
+        ev1.record()
+        torch.cuda.synchronize()
+        us = ev0.elapsed_time(ev1) * 1000.0 / iters
+        nbytes = m * k // 2 + 4 * m * (k // block_size)
+        gbs = nbytes / (us * 1e-6) / 1e9
+        out[nm] = {"m": m, "k": k, "block_size": block_size, "us": round(us, 2),
+                   "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                                "kernel": "tuna::gemm_multi_kernel (scale blocks)" if m * k // 2 >= 20 << 20 else "tuna::gemm_narrow_kernel (scale blocks)",
+                                "algorithmic_bytes_per_launch": nbytes, "avg_launch_us": round(us, 2)}}
+        del sets, scales
+        torch.cuda.empty_cache()
+    return out
+
+
 def multi_layer_sweep(ops, synth, torch, dev, names, n, layers, iters=None, seed0=10_000):
     """`layers` calls of tuna_matmul_multi, each with the GEMMs `names` of one layer (distinct seeded weights per
     layer), back to back: us per call, packed-weight GB/s.  The independent-problems reading of a layer: what
@@ -349,11 +388,11 @@ def main():
     ap.add_argument("--launch", choices=("both", "stream", "graph"), default="both")
     ap.add_argument("--settle", type=int, default=300,
                     help="untimed launches before the warm-up of the headline (a box that was idle ramps its clocks)")
-    ap.add_argument("--only", choices=("read", "dequant", "quantize", "multi", "mfma", "rates"), default=None,
+    ap.add_argument("--only", choices=("read", "dequant", "quantize", "multi", "mfma", "rates", "blockwise"), default=None,
                     help="profiling runs: launch only the read-kernel sweep / the dequant kernel / the quantizer / "
                          "the Llama-70B layer set through tuna_matmul_multi (16 layers) / the many-token kernel with "
                          "16x16x32 and with 32x32x16 MFMA tiles (Llama-70B gate+up and QKV, --tokens, default 1024) / the "
-                         "matrix-core and LDS yardstick kernels")
+                         "matrix-core and LDS yardstick kernels / the blockwise GEMM (a scale per 64 weights)")
     ap.add_argument("--weight-path", choices=("table", "registers", "lds"), default="table",
                     help="headline workload: the table's config as it is, or with the packed weights forced through "
                          "registers / staged through LDS (lds_tile_rows 0 / -1; A/B runs of the two weight paths)")
@@ -386,6 +425,8 @@ def main():
             res = {"quantize": time_quantize(ops, synth, torch, dev)}
         elif args.only == "rates":
             res = {"unit_rates": unit_rates(ops, dev)}
+        elif args.only == "blockwise":
+            res = {"blockwise_gemm_block_64": time_blockwise(ops, synth, torch, dev)}
         elif args.only == "mfma":
             res = {"many_token_kernel_mfma_shapes": mfma_shapes(ops, synth, torch, dev, 1024 if args.tokens == TOKENS else args.tokens)}
         else:
@@ -479,6 +520,7 @@ def main():
         line["min_frac_hbm_over_shapes_multi_x8"] = min(v["frac_hbm"] for v in shapes_multi.values())
         line["dequant"] = time_dequant_shapes(ops, synth, torch, dev)
         line["quantize"] = time_quantize(ops, synth, torch, dev)
+        line["blockwise_gemm_block_64"] = time_blockwise(ops, synth, torch, dev)
 
     if not args.no_shapes:
         # Mixtral gate+up with a router: 16 tokens x top-2 = 32 (token, expert) rows spread over the 8
