@@ -171,6 +171,11 @@ typedef struct tuna_gemm_problem {
  * of one call on `stream`; no problem may read what another one writes.  All problems are
  * checked before anything is enqueued.  No counterpart in the reference. */
 int tuna_matmul_multi(const tuna_gemm_problem *problems, int count, void *stream);
+/* The same for weights with one scale per block_size (64, 128, 256, ...) consecutive weights of a row: every
+ * problem's absmax is fp32 [m, k / block_size] (the layout tuna_quantize_blockwise writes, the reference
+ * quantizer's for block_size < k, test.py:7-17), 4-byte aligned.  Problems that do not qualify for the batched
+ * launch are run one by one as tuna_matmul_blockwise would.  No counterpart in the reference's kernels. */
+int tuna_matmul_multi_blockwise(const tuna_gemm_problem *problems, int count, int block_size, void *stream);
 
 /* Grouped GEMM (mixture of experts with per-expert token lists) in one launch.  The weights
  * are n_groups (<= 64) matrices of m_group rows stacked along m - q [n_groups*m_group/8, k/8,

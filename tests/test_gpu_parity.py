@@ -1506,6 +1506,78 @@ def test_blockwise_gemm_through_the_batched_streaming_kernel(m, n, k, bs):
         L.tuna_set_blockwise_stream(prev)
 
 
+def test_matmul_multi_blockwise_matches_the_oracle_and_separate_calls():
+    """tuna_matmul_multi_blockwise: four problems with a scale per 64 weights in one launch of the batched kernel, one
+    it cannot take (40 tokens) and one more behind it; every output against the oracle's float64 sums over the blockwise
+    D1 weights (row sample), within tolerance of a separate tuna_matmul_blockwise call, one-hot read-outs bit-exact, and
+    the same bits on a second call."""
+    import torch
+
+    from tuna_amd import _lib, ops
+
+    bs = 64
+    shapes = [(1024, 16, 2048), (2048, 16, 1024), (512, 3, 4096), (4096, 16, 4096), (256, 40, 1024), (768, 16, 1536)]
+    rng = np.random.default_rng(77)
+    probs, host = [], []
+    dc = None
+    for i, (m, n, k) in enumerate(shapes):
+        q, x, code, _ = make_inputs_np(m, n, k, seed=500 + i)
+        absmax = rng.uniform(0.005, 0.02, size=(m, k // bs)).astype(np.float16).astype(np.float32)
+        dq, dx, dc_i, da = to_dev(q, x, code, absmax)
+        dc = dc_i if dc is None else dc
+        out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+        probs.append((dx, dq, da, dc, out, m, n, k))
+        host.append((q, x, code, absmax))
+    want = []
+    for (dx, dq, da, dcc, _o, m, n, k) in probs:
+        o = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+        ops.matmul_blockwise(dx, dq, da, dcc, o, m, n, k, bs)
+        want.append(o)
+    torch.cuda.synchronize()
+    first = None
+    for rep in range(2):
+        for p in probs:
+            p[4].fill_(float("nan"))
+        before = _lib.lib().tuna_multi_launches()
+        ops.matmul_multi(probs, block_size=bs)
+        torch.cuda.synchronize()
+        assert _lib.lib().tuna_multi_launches() == before + 1      # problems 0..3 in one launch, the rest one by one
+        got = [p[4].cpu().numpy().view(np.uint16).copy() for p in probs]
+        for i, ((m, n, k), g, w) in enumerate(zip(shapes, got, want)):
+            assert not np.isnan(g.view(np.float16)).any(), (rep, i)
+            q, x, code, absmax = host[i]
+            rows = np.sort(np.random.default_rng(i).choice(m, size=min(m, 192), replace=False)).astype(np.int32)
+            ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1, rows=rows, block_size=bs)
+            e = rel_err(f16_bits_to_f64(g[:, rows]), ref)
+            assert e <= REL_TOL, (rep, i, e)
+            assert rel_err(f16_bits_to_f64(g), w.float().cpu().numpy().astype(np.float64)) <= REL_TOL
+        for i in (4, 5):
+            assert np.array_equal(got[i], want[i].cpu().numpy().view(np.uint16))
+        if first is None:
+            first = got
+        else:
+            assert all(np.array_equal(a, b) for a, b in zip(first, got))
+    # one-hot activations read the decode out of the batched launch: every problem's image, its blocks' scales included
+    hot = []
+    for i, (m, n, k) in enumerate(shapes[:4]):
+        cols = rng.choice(k, size=n, replace=False)
+        xh = np.zeros((n, k), np.float16)
+        xh[np.arange(n), cols] = 1.0
+        dxh, = to_dev(xh)
+        hot.append((dxh,) + probs[i][1:])
+        hot[-1][4].fill_(float("nan"))
+        hot[-1] = hot[-1] + (cols,)
+    ops.matmul_multi([h[:8] for h in hot], block_size=bs)
+    torch.cuda.synchronize()
+    for i, h in enumerate(hot):
+        q, _, code, absmax = host[i]
+        m, n, k = shapes[i]
+        img = O.dequant(q, absmax, code, m, k, mode=O.D1, block_size=bs)
+        assert np.array_equal(h[4].cpu().numpy().view(np.uint16), img[:, h[8]].T), i
+    arr = ops.problem_array(probs[:2], bs)
+    assert _lib.lib().tuna_matmul_multi_blockwise(arr, 2, 32, ops._stream(probs[0][0].device)) == _lib.ERR_UNSUPPORTED   # blocks start at 64
+
+
 def test_blockwise_entry_points_reject_what_they_cannot_run():
     import torch
 

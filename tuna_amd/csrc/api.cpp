@@ -976,6 +976,9 @@ static int matmul_grouped_impl(const void *q, const void *x, const void *code, c
     return TUNA_OK;
 }
 
+extern "C" int tuna_matmul_blockwise(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n,
+                                     int k, int block_size, void *stream);
+
 static int matmul_multi_impl(const tuna_gemm_problem *problems, int count, hipStream_t stream)
 {
     if (count < 0 || (count > 0 && !problems)) return fail(TUNA_ERR_INVALID_ARG, "problems is null or count=%d negative", count);
@@ -1183,6 +1186,52 @@ TUNA_EXPORT int tuna_matmul_fused(const void *q, const void *x, const void *code
 TUNA_EXPORT int tuna_matmul_multi(const tuna_gemm_problem *problems, int count, void *stream)
 {
     return matmul_multi_impl(problems, count, static_cast<hipStream_t>(stream));
+}
+
+TUNA_EXPORT int tuna_matmul_multi_blockwise(const tuna_gemm_problem *problems, int count, int block_size, void *stream)
+{
+    if (count < 0 || (count > 0 && !problems)) return fail(TUNA_ERR_INVALID_ARG, "problems is null or count=%d negative", count);
+    if (count == 0) return TUNA_OK;
+    if (block_size < 64 || !is_pow2(block_size))
+        return fail(TUNA_ERR_UNSUPPORTED, "block_size=%d: the batched blockwise GEMM takes 64, 128, 256, ...", block_size);
+    int rc;
+    // every problem is checked before anything is enqueued: a bad one must not leave half a batch behind
+    for (int i = 0; i < count; ++i) {
+        const tuna_gemm_problem &p = problems[i];
+        if ((rc = check_shape(p.m, p.n, p.k))) return rc;
+        if (p.k % block_size || p.k / block_size < 2 || p.m % 16 || p.k % 256)
+            return fail(TUNA_ERR_UNSUPPORTED, "problem %d: scale blocks of %d need k=%d a multiple of them (at least two), m=%d of 16, k of 256",
+                        i, block_size, p.k, p.m);
+        if ((unsigned long long)p.m * (unsigned long long)p.k / 2 >= (1ull << 32) || (unsigned long long)p.k * 32 >= (1ull << 32))
+            return fail(TUNA_ERR_UNSUPPORTED, "problem %d: operands exceed the kernel's 32-bit offsets", i);
+        if ((p.n + 15) / 16 > 65535) return fail(TUNA_ERR_UNSUPPORTED, "problem %d: n=%d needs more than 65535 token chunks", i, p.n);
+        if ((rc = check_ptr(p.q, "q", 16)) || (rc = check_ptr(p.x, "x", 16)) || (rc = check_ptr(p.code, "code", 4)) ||
+            (rc = check_ptr(p.absmax, "absmax", 4)) || (rc = check_ptr(p.out, "out", 16)))
+            return rc;
+    }
+    int dev = 0, cus = 0;
+    hipError_t e = device_cus(&dev, &cus);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int shift = log2i(block_size) - 6;
+    for (int first = 0; first < count;) {
+        MultiPlan plan;
+        int take = count - first < kMaxMultiProblems ? count - first : kMaxMultiProblems;
+        const int min_batch = g_multi_min_batch.load(std::memory_order_relaxed);
+        while (take >= min_batch && !plan_multi(problems + first, take, cus, &plan, 0, 0, shift)) --take;
+        if (take >= min_batch) {
+            if ((rc = provide_workspace(false, st, plan.ws_bytes, plan.n_counters, &plan.args.ws, &plan.args.counters))) return rc;
+            e = launch_gemm_multi(plan.args, plan.prefetch, dev, st);
+            if (e != hipSuccess) return hip_fail(e, "batched blockwise gemm launch");
+            g_multi_launches.fetch_add(1, std::memory_order_relaxed);
+            first += take;
+            continue;
+        }
+        const tuna_gemm_problem &p = problems[first];
+        if ((rc = tuna_matmul_blockwise(p.q, p.x, p.code, p.absmax, p.out, p.m, p.n, p.k, block_size, stream))) return rc;
+        ++first;
+    }
+    return TUNA_OK;
 }
 
 TUNA_EXPORT int tuna_matmul_grouped(const void *q, const void *x, const void *code, const void *absmax, void *out,

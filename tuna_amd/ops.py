@@ -110,29 +110,36 @@ def matmul_fused(x, q, s, c, o, m: int, n: int, k: int, epilogue: int, residual=
     _lib.check(rc)
 
 
-def problem_array(problems):
-    """ctypes array of GemmProblem for matmul_multi / time_matmul_multi from (x, q, s, c, o, m, n, k) tuples."""
+def problem_array(problems, block_size: int = None):
+    """ctypes array of GemmProblem for matmul_multi / time_matmul_multi from (x, q, s, c, o, m, n, k) tuples
+    (block_size: s is [m, k / block_size])."""
     arr = (_lib.GemmProblem * len(problems))()
     for i, (x, q, s, c, o, m, n, k) in enumerate(problems):
         m, n, k = int(m), int(n), int(k)
         _require(x, "x", torch.float16, n * k)
         _require(q, "q", torch.uint8, m * k // 2)
-        _require(s, "s", torch.float32, m)
+        _require(s, "s", torch.float32, m if block_size is None else m * (k // int(block_size)))
         _require(c, "c", torch.float32, 16)
         _require(o, "o", torch.float16, n * m)
         arr[i] = _lib.GemmProblem(q.data_ptr(), x.data_ptr(), c.data_ptr(), s.data_ptr(), o.data_ptr(), m, n, k)
     return arr
 
 
-def matmul_multi(problems) -> None:
+def matmul_multi(problems, block_size: int = None) -> None:
     """Several independent GEMMs in one call (tuna_matmul_multi): `problems` is a list of
-    (x, q, s, c, o, m, n, k) tuples, each with the meaning of matmul's arguments."""
+    (x, q, s, c, o, m, n, k) tuples, each with the meaning of matmul's arguments.  With block_size every s is
+    [m, k / block_size], one scale per block of a row (tuna_matmul_multi_blockwise)."""
     if not problems:
         return
-    arr = problem_array(problems)
+    if block_size is not None and (int(block_size) <= 0 or any(int(p[7]) % int(block_size) for p in problems)):
+        raise ValueError(f"block_size={block_size} must divide every k")
+    arr = problem_array(problems, block_size)
     dev = problems[0][0].device
     with torch.cuda.device(dev):
-        rc = _lib.lib().tuna_matmul_multi(arr, len(problems), _stream(dev))
+        if block_size is None:
+            rc = _lib.lib().tuna_matmul_multi(arr, len(problems), _stream(dev))
+        else:
+            rc = _lib.lib().tuna_matmul_multi_blockwise(arr, len(problems), int(block_size), _stream(dev))
     _lib.check(rc)
 
 
