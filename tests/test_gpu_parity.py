@@ -1459,13 +1459,15 @@ def test_blockwise_gemm_matches_oracle_and_reads_out_the_decode(m, n, k, bs):
 
 
 @pytest.mark.parametrize("m,n,k,bs", [(256, 16, 1280, 64), (128, 7, 1536, 64), (512, 16, 4096, 128), (1024, 1, 2048, 256),
-                                      (256, 16, 2048, 512), (768, 13, 5120, 64), (4096, 16, 4096, 64), (8192, 16, 8192, 64)])
+                                      (256, 16, 2048, 512), (768, 13, 5120, 64), (4096, 16, 4096, 64), (8192, 16, 8192, 64),
+                                      (512, 37, 2048, 256), (256, 100, 1024, 64), (256, 530, 512, 64)])
 def test_blockwise_gemm_through_the_batched_streaming_kernel(m, n, k, bs):
     """The scale-block variant of the batched streaming kernel (tuna_matmul_blockwise takes it from 20 MB of packed
     weights; the switch sends every shape it can plan there): against the oracle's float64 sums over the blockwise D1
     weights on a row sample, bit-exact through one-hot activations (every scale block of every sampled column read
     out), and run-to-run identical.  k ranges that are not whole x chunks, 128-row tiles, blocks longer than a chunk,
-    shares that split row tiles (hand-over through the workspace)."""
+    shares that split row tiles (hand-over through the workspace); more than 16 tokens run as the token chunks of a
+    batch, 32 chunks to a launch."""
     import torch
 
     from tuna_amd import _lib, ops
@@ -1483,7 +1485,7 @@ def test_blockwise_gemm_through_the_batched_streaming_kernel(m, n, k, bs):
         ops.matmul_blockwise(dx, dq, da, dc, out, m, n, k, bs)
         torch.cuda.synchronize()
         got = out.cpu().numpy().view(np.uint16)
-        assert L.tuna_multi_launches() == launches + 1     # the batched kernel ran it
+        assert L.tuna_multi_launches() == launches + -(-(-(-n // 16)) // 32)     # the batched kernel ran it
         assert not np.isnan(got.view(np.float16)).any()
         rows = np.sort(rng.choice(m, size=min(m, 192), replace=False)).astype(np.int32)
         ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1, rows=rows, block_size=bs)
@@ -1495,6 +1497,8 @@ def test_blockwise_gemm_through_the_batched_streaming_kernel(m, n, k, bs):
         assert np.array_equal(again.cpu().numpy().view(np.uint16), got)
         img = O.dequant(q, absmax, code, m, k, mode=O.D1, block_size=bs)
         for rep in range(2):
+            if n > k:
+                break
             cols = rng.choice(k, size=n, replace=False)
             xh = np.zeros((n, k), np.float16)
             xh[np.arange(n), cols] = 1.0

@@ -1275,28 +1275,49 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
     if ((rc = check_ptr(q, "q", 16)) || (rc = check_ptr(x, "x", 16)) || (rc = check_ptr(code, "code", 4)) ||
         (rc = check_ptr(absmax, "absmax", 4)) || (rc = check_ptr(out, "out", 16)))
         return rc;
-    // Up to 16 tokens, aligned shapes: the batched streaming kernel's scale-block variant as a batch of one (balanced
-    // split over one workgroup per compute unit).  Everything else: the narrow-row kernel's.
-    // (below about 20 MB of packed weights the narrow-row kernel's single pass is faster: 12.1 against 16.1 us on
-    // 6144 x 4096, 21.4 against 16.5 us on 4096 x 14336)
+    // Aligned shapes from about 20 MB of packed weights: the batched streaming kernel's scale-block variant, a batch of
+    // one for up to 16 tokens (balanced split over one workgroup per compute unit), the token chunks of 16 as the
+    // problems of a batch beyond that (every chunk streams the weights again, in one launch per 32 chunks).
+    // Everything else: the narrow-row kernel's variants.
+    // (below that size the narrow-row kernel's single pass is faster: 12.1 against 16.1 us on 6144 x 4096, 21.4
+    // against 16.5 us on 4096 x 14336)
     const int stream_mode = g_blockwise_stream.load(std::memory_order_relaxed);
-    if (n <= 16 && (stream_mode == 2 || (stream_mode == 1 && (long long)m * k / 2 >= (20ll << 20)))) {
+    if (stream_mode == 2 || (stream_mode == 1 && (long long)m * k / 2 >= (20ll << 20))) {
         int dev = 0, cus = 0;
         hipError_t e = device_cus(&dev, &cus);
         if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
-        const tuna_gemm_problem one = {q, x, code, absmax, out, m, n, k};
-        MultiPlan plan;
-        // the batched kernel's own choice of tile height (256 rows, 128 where those are fewer than workgroups), ring of two;
-        // then whatever height the row count allows
-        bool ok = plan_multi(&one, 1, cus, &plan, 0, 0, log2i(block_size) - 6);
-        for (int wm = 4; wm >= 1 && !ok; wm >>= 1) ok = plan_multi(&one, 1, cus, &plan, wm, 2, log2i(block_size) - 6);
-        if (ok) {
-            if ((rc = provide_workspace(false, static_cast<hipStream_t>(stream), plan.ws_bytes, plan.n_counters, &plan.args.ws,
-                                        &plan.args.counters)))
-                return rc;
-            e = launch_gemm_multi(plan.args, plan.prefetch, dev, static_cast<hipStream_t>(stream));
-            if (e != hipSuccess) return hip_fail(e, "blockwise gemm launch");
-            g_multi_launches.fetch_add(1, std::memory_order_relaxed);
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        const int shift = log2i(block_size) - 6;
+        const int chunks = (n + 15) / 16;
+        // batch `c0 / 32` of the token chunks as a list of problems, planned for this device
+        auto plan_batch = [&](int c0, MultiPlan *plan) {
+            const int cnt = chunks - c0 < kMaxMultiProblems ? chunks - c0 : kMaxMultiProblems;
+            tuna_gemm_problem probs[kMaxMultiProblems];
+            for (int c = 0; c < cnt; ++c) {
+                const int t0 = (c0 + c) * 16;
+                probs[c] = {q, static_cast<const char *>(x) + (size_t)t0 * k * 2, code, absmax,
+                            static_cast<char *>(out) + (size_t)t0 * m * 2, m, n - t0 < 16 ? n - t0 : 16, k};
+            }
+            // the batched kernel's own choice of tile height (256 rows, 128 where those are fewer than workgroups), ring of
+            // two; then whatever height the row count allows
+            bool ok = plan_multi(probs, cnt, cus, plan, 0, 0, shift);
+            for (int wm = 4; wm >= 1 && !ok; wm >>= 1) ok = plan_multi(probs, cnt, cus, plan, wm, 2, shift);
+            return ok;
+        };
+        bool planned_all = true;  // (nothing is enqueued unless every batch of chunks can run here)
+        for (int c0 = 0; c0 < chunks && planned_all; c0 += kMaxMultiProblems) {
+            MultiPlan plan;
+            planned_all = plan_batch(c0, &plan);
+        }
+        if (planned_all) {
+            for (int c0 = 0; c0 < chunks; c0 += kMaxMultiProblems) {
+                MultiPlan plan;
+                if (!plan_batch(c0, &plan)) return fail(TUNA_ERR_UNSUPPORTED, "blockwise gemm: a batch of token chunks stopped planning");
+                if ((rc = provide_workspace(false, st, plan.ws_bytes, plan.n_counters, &plan.args.ws, &plan.args.counters))) return rc;
+                e = launch_gemm_multi(plan.args, plan.prefetch, dev, st);
+                if (e != hipSuccess) return hip_fail(e, "blockwise gemm launch");
+                g_multi_launches.fetch_add(1, std::memory_order_relaxed);
+            }
             return TUNA_OK;
         }
     }
