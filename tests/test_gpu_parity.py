@@ -1510,6 +1510,48 @@ def test_blockwise_gemm_through_the_batched_streaming_kernel(m, n, k, bs):
         L.tuna_set_blockwise_stream(prev)
 
 
+@pytest.mark.parametrize("m,n,k,bs", [(512, 64, 1024, 64), (528, 130, 2048, 128), (1024, 300, 4096, 64), (256, 1024, 512, 256),
+                                      (4096, 33, 4096, 64), (272, 200, 1280, 64)])
+def test_blockwise_gemm_with_many_tokens_through_the_many_token_kernel(m, n, k, bs):
+    """From 33 tokens tuna_matmul_blockwise decodes a weight tile once per workgroup with the scale of each k-step's block
+    (the many-token kernel's scale-block variants): against the oracle's float64 sums over the blockwise D1 weights (row
+    sample), bit-exact through one-hot activations, run-to-run identical; ragged m / n, k ranges of 8 to 64 steps."""
+    import torch
+
+    from tuna_amd import _lib, ops
+
+    rng = np.random.default_rng(m + n + k + bs + 2)
+    q, x, code, _ = make_inputs_np(m, n, k, seed=m + bs + 2)
+    absmax = rng.uniform(0.005, 0.02, size=(m, k // bs)).astype(np.float16).astype(np.float32)
+    dq, dx, dc, da = to_dev(q, x, code, absmax)
+    out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+    L = _lib.lib()
+    before = L.tuna_blockwise_launches(2)
+    print(f"blockwise through the many-token kernel m={m} n={n} k={k} block={bs}", flush=True)
+    ops.matmul_blockwise(dx, dq, da, dc, out, m, n, k, bs)
+    torch.cuda.synchronize()
+    assert L.tuna_blockwise_launches(2) == before + 1
+    got = out.cpu().numpy().view(np.uint16)
+    assert not np.isnan(got.view(np.float16)).any()
+    rows = np.sort(rng.choice(m, size=min(m, 128), replace=False)).astype(np.int32)
+    ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1, rows=rows, block_size=bs)
+    e = rel_err(f16_bits_to_f64(got[:, rows]), ref)
+    assert e <= REL_TOL, e
+    again = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+    ops.matmul_blockwise(dx, dq, da, dc, again, m, n, k, bs)
+    torch.cuda.synchronize()
+    assert np.array_equal(again.cpu().numpy().view(np.uint16), got)
+    nh = min(n, k)
+    cols = rng.choice(k, size=nh, replace=False)
+    xh = np.zeros((n, k), np.float16)
+    xh[np.arange(nh), cols] = 1.0
+    dxh, = to_dev(xh)
+    ops.matmul_blockwise(dxh, dq, da, dc, out, m, n, k, bs)
+    torch.cuda.synchronize()
+    img = O.dequant(q, absmax, code, m, k, mode=O.D1, block_size=bs)
+    assert np.array_equal(out.cpu().numpy().view(np.uint16)[:nh], img[:, cols].T)
+
+
 def test_matmul_multi_blockwise_matches_the_oracle_and_separate_calls():
     """tuna_matmul_multi_blockwise: four problems with a scale per 64 weights in one launch of the batched kernel, one
     it cannot take (40 tokens) and one more behind it; every output against the oracle's float64 sums over the blockwise

@@ -104,6 +104,7 @@ SIGNATURES = {
     "tuna_set_multi_min_batch": (_i, [_i]),
     "tuna_set_blockwise_shape": (_i, [_i, _i, _i]),
     "tuna_set_blockwise_stream": (_i, [_i]),
+    "tuna_blockwise_launches": (ctypes.c_ulonglong, [_i]),
     "tuna_multi_launches": (ctypes.c_ulonglong, []),
     "tuna_set_lean_kernels": (_i, [_i]),
     "tuna_set_weight_path": (_i, [_i]),

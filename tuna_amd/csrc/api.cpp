@@ -676,6 +676,7 @@ static int check_ptr(const void *p, const char *name, size_t align)
 // launched problem by problem on the same stream.
 // ---------------------------------------------------------------------------------------
 static std::atomic<int> g_multi_waves_m{0}, g_multi_prefetch{0};  // 0: the library's choice (diagnostic override)
+static std::atomic<unsigned long long> g_blockwise_launches[3];  // by kernel: narrow-row, batched streaming, many-token
 static std::atomic<int> g_blockwise_stream{1};  // tuna_matmul_blockwise takes the batched kernel's scale-block variant where it can
 static std::atomic<int> g_multi_lds{0};  // batches with a ring of 2 stage weights and x through LDS (tuna_set_multi_weight_path)
 static std::atomic<unsigned long long> g_multi_launches{0};
@@ -1275,13 +1276,50 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
     if ((rc = check_ptr(q, "q", 16)) || (rc = check_ptr(x, "x", 16)) || (rc = check_ptr(code, "code", 4)) ||
         (rc = check_ptr(absmax, "absmax", 4)) || (rc = check_ptr(out, "out", 16)))
         return rc;
+    // From 33 tokens: the many-token kernel's scale-block variants (the weights are decoded once per workgroup tile,
+    // with the scale of the k-step's block) - the tile the per-row table has for the shape and token count if that is a
+    // many-token entry, else 256 rows x 64 tokens up to 64 tokens, 128 x 128 up to 128 and 128 x 256 beyond.
+    const int stream_mode = g_blockwise_stream.load(std::memory_order_relaxed);
+    if (n > 32 && stream_mode == 1) {
+        tuna_gemm_config c;
+        select_config(m, n, k, &c, nullptr);
+        if (c.lds_tile_rows <= 0 || !tiled_variant_exists(c.lds_tile_rows, 16 * c.token_tiles, false)) {
+            c.lds_tile_rows = n > 64 ? 128 : 256;
+            c.token_tiles = n > 128 ? 16 : n > 64 ? 8 : 4;
+            // fewer tiles than compute units: split k until the launch fills them (at least eight k-steps per workgroup)
+            int dev_ = 0, cus_ = kMaxCus;
+            (void)device_cus(&dev_, &cus_);
+            const long long tiles = (long long)ceil_div(m, c.lds_tile_rows) * ceil_div(n, 16 * c.token_tiles);
+            const int steps = ceil_div(k, 64);
+            long long split = tiles > 0 ? cus_ / tiles : 1;
+            if (split > steps / 8) split = steps / 8;
+            c.split_k = split < 1 ? 1 : (int)split;
+        }
+        c.rows_per_wave = 64;  // (16 x 16 x 32 MFMA tiles: the scale-block variants exist for those)
+        TiledPlan tp;
+        if (plan_tiled(m, n, k, c, TUNA_DECODE_GEMM, &tp) == TUNA_OK) {
+            hipStream_t st = static_cast<hipStream_t>(stream);
+            tp.args.q = static_cast<const uint8_t *>(q);
+            tp.args.x = x;
+            tp.args.code = static_cast<const float *>(code);
+            tp.args.absmax = static_cast<const float *>(absmax);
+            tp.args.out = out;
+            tp.args.epilogue = TUNA_EPILOGUE_NONE;
+            tp.args.residual = nullptr;
+            tp.args.blk_shift = log2i(block_size) - 6;
+            if (tp.ws_bytes && (rc = provide_workspace(false, st, tp.ws_bytes, tp.n_counters, &tp.args.ws, &tp.args.counters))) return rc;
+            hipError_t e = launch_gemm_tiled(tp.args, tp.tile_rows, tp.tile_tokens, false, st, true);
+            if (e != hipSuccess) return hip_fail(e, "many-token blockwise gemm launch");
+            g_blockwise_launches[2].fetch_add(1, std::memory_order_relaxed);
+            return TUNA_OK;
+        }
+    }
     // Aligned shapes from about 20 MB of packed weights: the batched streaming kernel's scale-block variant, a batch of
     // one for up to 16 tokens (balanced split over one workgroup per compute unit), the token chunks of 16 as the
     // problems of a batch beyond that (every chunk streams the weights again, in one launch per 32 chunks).
     // Everything else: the narrow-row kernel's variants.
     // (below that size the narrow-row kernel's single pass is faster: 12.1 against 16.1 us on 6144 x 4096, 21.4
     // against 16.5 us on 4096 x 14336)
-    const int stream_mode = g_blockwise_stream.load(std::memory_order_relaxed);
     if (stream_mode == 2 || (stream_mode == 1 && (long long)m * k / 2 >= (20ll << 20))) {
         int dev = 0, cus = 0;
         hipError_t e = device_cus(&dev, &cus);
@@ -1317,10 +1355,12 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
                 e = launch_gemm_multi(plan.args, plan.prefetch, dev, st);
                 if (e != hipSuccess) return hip_fail(e, "blockwise gemm launch");
                 g_multi_launches.fetch_add(1, std::memory_order_relaxed);
+                g_blockwise_launches[1].fetch_add(1, std::memory_order_relaxed);
             }
             return TUNA_OK;
         }
     }
+    g_blockwise_launches[0].fetch_add(1, std::memory_order_relaxed);
     NarrowArgs a;
     memset(&a, 0, sizeof(a));
     a.q = static_cast<const uint8_t *>(q);
@@ -1612,6 +1652,11 @@ TUNA_EXPORT int tuna_time_unit_rate(int unit, void *sink, int warmup, int iters,
         return e2 == hipSuccess ? (int)TUNA_OK : hip_fail(e2, "unit-rate launch");
     };
     return time_loop(launch, 1, warmup, iters, 0, static_cast<hipStream_t>(stream), elapsed_ms);
+}
+
+TUNA_EXPORT unsigned long long tuna_blockwise_launches(int kernel)
+{
+    return kernel >= 0 && kernel < 3 ? g_blockwise_launches[kernel].load(std::memory_order_relaxed) : 0ull;
 }
 
 TUNA_EXPORT int tuna_set_blockwise_stream(int enabled)

@@ -45,7 +45,7 @@ constexpr int kTiledStepK = 64;
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t tiled_u32x2 __attribute__((ext_vector_type(2)));
 
-template <int WM, int TM, int WN, int TN, int NSETS, bool M32 = false>
+template <int WM, int TM, int WN, int TN, int NSETS, bool M32 = false, bool BLK = false>
 __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const TiledArgs a)
 {
     static_assert(WM * WN * 64 == kTiledThreads, "8 waves");
@@ -99,11 +99,18 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     const int a_mb = min((row_base >> 3) + a_mbl, mb_last);
     const unsigned char *a_src = a.q + (size_t)a_mb * kb_total * 32 + a_piece * (4 * DW);
     const int a_row = a_mbl * 8 + a_piece * DW;      // first of the DW tile rows this thread decodes
+    // one scale per row - or (BLK) per block of 64 << blk_shift weights of a row: a k-step of 64 lies inside one
+    // block, its scales travel through the register sets with its weights
     f16x2 sc16[DW];
+    const float *sc_src[DW];
+    const int nblk = BLK ? a.k >> (6 + a.blk_shift) : 1;
 #pragma unroll
     for (int j = 0; j < DW; ++j) {
-        const f16 h = (f16)a.absmax[min(row_base + a_row + j, a.m - 1)];
-        sc16[j] = f16x2{h, h};
+        sc_src[j] = a.absmax + (size_t)min(row_base + a_row + j, a.m - 1) * (size_t)nblk;
+        if constexpr (!BLK) {
+            const f16 h = (f16)sc_src[j][0];
+            sc16[j] = f16x2{h, h};
+        }
     }
     // activations: piece p = tid + i*512: token p / 8 of the tile, 8-k slot p % 8 of the step
     const f16 *x_src[X_PER_THREAD];
@@ -123,12 +130,17 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     // activations come from the L2, not from HBM)
     constexpr int XSETS = X_PER_THREAD == 4 ? 2 : NSETS;
     uint32_t wq[NSETS][DW];
+    float sq[BLK ? NSETS : 1][DW];
     u32x4 xr[XSETS][X_PER_THREAD];
     // Unconditional, clamped loads (exact s_waitcnt counts); what lies beyond k is zeroed in x.
 #define TUNA_TILED_LOAD(set, s)                                                                 \
     {                                                                                          \
         const int kb_ = min((s) * 8 + a_kb, kb_total - 1);                                     \
         const unsigned char *p_ = a_src + (size_t)kb_ * 32;                                    \
+        if constexpr (BLK) {                                                                   \
+            const int blk_ = min((s) >> a.blk_shift, nblk - 1);                                \
+            _Pragma("unroll") for (int j = 0; j < DW; ++j) sq[set][j] = sc_src[j][blk_];       \
+        }                                                                                      \
         if constexpr (DW == 4) {                                                               \
             const u32x4 w_ = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p_));  \
             _Pragma("unroll") for (int j = 0; j < 4; ++j) wq[set][j] = w_[j];                  \
@@ -239,6 +251,10 @@ __global__ __launch_bounds__(kTiledThreads, 2) void gemm_tiled_kernel(const Tile
     _Pragma("unroll") for (int j = 0; j < DW; ++j)                                             \
     {                                                                                          \
         const uint32_t d_ = wq[set][j];                                                        \
+        if constexpr (BLK) {                                                                   \
+            const f16 h_ = (f16)sq[set][j];                                                    \
+            sc16[j] = f16x2{h_, h_};                                                           \
+        }                                                                                      \
         lt[4 * j + 0] = *reinterpret_cast<const lds_u32 *>((uintptr_t)__builtin_amdgcn_perm(d_, lane4, 0x0c0c0400u)); \
         lt[4 * j + 1] = *reinterpret_cast<const lds_u32 *>((uintptr_t)__builtin_amdgcn_perm(d_, lane4, 0x0c0c0500u)); \
         lt[4 * j + 2] = *reinterpret_cast<const lds_u32 *>((uintptr_t)__builtin_amdgcn_perm(d_, lane4, 0x0c0c0600u)); \
@@ -410,16 +426,17 @@ typedef void (*TiledFn)(const TiledArgs);
 struct TiledVariant {
     int bm, bn;
     TiledFn fn;
-    TiledFn fn32;  // the same tile with 32 x 32 x 16 MFMAs, or null
+    TiledFn fn32;   // the same tile with 32 x 32 x 16 MFMAs, or null
+    TiledFn fn_blk; // the same tile (16 x 16 x 32 MFMAs) with a scale per block of a row
 };
 // (WM, TM, WN, TN): rows x tokens of the workgroup tile
 static const TiledVariant kTiled[] = {
-    {256, 128, gemm_tiled_kernel<4, 4, 2, 4, 4>, gemm_tiled_kernel<4, 4, 2, 4, 4, true>},
-    {256, 64, gemm_tiled_kernel<4, 4, 2, 2, 8>, gemm_tiled_kernel<4, 4, 2, 2, 8, true>},
-    {128, 256, gemm_tiled_kernel<2, 4, 4, 4, 4>, gemm_tiled_kernel<2, 4, 4, 4, 4, true>},
-    {128, 128, gemm_tiled_kernel<2, 4, 4, 2, 4>, gemm_tiled_kernel<2, 4, 4, 2, 4, true>},
-    {64, 256, gemm_tiled_kernel<1, 4, 8, 2, 4>, gemm_tiled_kernel<1, 4, 8, 2, 4, true>},
-    {64, 128, gemm_tiled_kernel<1, 4, 8, 1, 4>, nullptr},
+    {256, 128, gemm_tiled_kernel<4, 4, 2, 4, 4>, gemm_tiled_kernel<4, 4, 2, 4, 4, true>, gemm_tiled_kernel<4, 4, 2, 4, 4, false, true>},
+    {256, 64, gemm_tiled_kernel<4, 4, 2, 2, 8>, gemm_tiled_kernel<4, 4, 2, 2, 8, true>, gemm_tiled_kernel<4, 4, 2, 2, 8, false, true>},
+    {128, 256, gemm_tiled_kernel<2, 4, 4, 4, 4>, gemm_tiled_kernel<2, 4, 4, 4, 4, true>, gemm_tiled_kernel<2, 4, 4, 4, 4, false, true>},
+    {128, 128, gemm_tiled_kernel<2, 4, 4, 2, 4>, gemm_tiled_kernel<2, 4, 4, 2, 4, true>, gemm_tiled_kernel<2, 4, 4, 2, 4, false, true>},
+    {64, 256, gemm_tiled_kernel<1, 4, 8, 2, 4>, gemm_tiled_kernel<1, 4, 8, 2, 4, true>, gemm_tiled_kernel<1, 4, 8, 2, 4, false, true>},
+    {64, 128, gemm_tiled_kernel<1, 4, 8, 1, 4>, nullptr, gemm_tiled_kernel<1, 4, 8, 1, 4, false, true>},
 };
 static constexpr int kNumTiled = sizeof(kTiled) / sizeof(kTiled[0]);
 
@@ -432,21 +449,21 @@ bool tiled_variant_exists(int bm, int bn, bool mfma32)
 
 size_t tiled_lds_bytes(int bm, int bn) { return (size_t)kLutBytes + 2 * (size_t)(bm + bn) * 128; }  // two tile buffers
 
-static OptInFlag g_tiled_attr[16][kNumTiled][2];
+static OptInFlag g_tiled_attr[16][kNumTiled][3];
 
-hipError_t launch_gemm_tiled(const TiledArgs &args, int bm, int bn, bool mfma32, hipStream_t stream)
+hipError_t launch_gemm_tiled(const TiledArgs &args, int bm, int bn, bool mfma32, hipStream_t stream, bool scale_blocks)
 {
     int vi = -1;
     for (int i = 0; i < kNumTiled; ++i)
         if (kTiled[i].bm == bm && kTiled[i].bn == bn) vi = i;
-    if (vi < 0) return hipErrorInvalidConfiguration;
-    const TiledFn fn = mfma32 ? kTiled[vi].fn32 : kTiled[vi].fn;
+    if (vi < 0 || (scale_blocks && mfma32)) return hipErrorInvalidConfiguration;
+    const TiledFn fn = scale_blocks ? kTiled[vi].fn_blk : mfma32 ? kTiled[vi].fn32 : kTiled[vi].fn;
     if (!fn) return hipErrorInvalidConfiguration;
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
-    if ((e = ensure_lds_opt_in(g_tiled_attr[dev][vi][mfma32], reinterpret_cast<const void *>(fn))) != hipSuccess) return e;
+    if ((e = ensure_lds_opt_in(g_tiled_attr[dev][vi][scale_blocks ? 2 : mfma32], reinterpret_cast<const void *>(fn))) != hipSuccess) return e;
     TiledArgs a = args;
     a.row_tiles = ceil_div_i(args.m, bm);
     a.tok_tiles = ceil_div_i(args.n, bn);

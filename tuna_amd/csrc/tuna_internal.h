@@ -143,6 +143,7 @@ struct TiledArgs {
     int split_k;          // gridDim.z
     int steps_per_split;
     int row_tiles, tok_tiles;  // gridDim.x = row_tiles * tok_tiles: token tiles of a row tile are launched together
+    int blk_shift;        // scale-block variants: absmax is [m, k / (64 << blk_shift)], one scale per block of a row
 };
 
 inline int ceil_div_i(int a, int b) { return (a + b - 1) / b; }
@@ -201,7 +202,8 @@ hipError_t launch_gemm_multi(const MultiArgs &args, int prefetch, int dev, hipSt
 hipError_t device_cus(int *dev, int *cus);
 
 // gemm_tiled.hip
-hipError_t launch_gemm_tiled(const TiledArgs &args, int tile_rows, int tile_tokens, bool mfma32, hipStream_t stream);
+hipError_t launch_gemm_tiled(const TiledArgs &args, int tile_rows, int tile_tokens, bool mfma32, hipStream_t stream,
+                             bool scale_blocks = false);
 bool tiled_variant_exists(int tile_rows, int tile_tokens, bool mfma32);
 size_t tiled_lds_bytes(int tile_rows, int tile_tokens);
 
