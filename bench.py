@@ -226,7 +226,8 @@ def unit_rates(ops, dev):
     shapes and LDS access patterns those kernels use (best of three timings each)."""
     names = ["mfma_16x16x32_f16_one_wave_per_simd_tflops", "mfma_16x16x32_f16_two_waves_per_simd_tflops",
              "mfma_32x32x16_f16_one_wave_per_simd_tflops", "lds_fragment_reads_b128_bytes_per_clk_per_cu",
-             "lds_table_reads_b32_bytes_per_clk_per_cu", "lds_tile_writes_b128_bytes_per_clk_per_cu"]
+             "lds_table_reads_b32_bytes_per_clk_per_cu", "lds_tile_writes_b128_bytes_per_clk_per_cu",
+             "lds_tile_writes_b64_bytes_per_clk_per_cu", "lds_linear_writes_b128_bytes_per_clk_per_cu"]
     out = {}
     for unit, nm in enumerate(names):
         best = 0.0

@@ -57,8 +57,9 @@ int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int va
  * one / two waves per SIMD (16 accumulators each); 2: v_mfma_f32_32x32x16_f16 from one wave per SIMD (4
  * accumulators); 3: 16-byte LDS reads in the pattern of an MFMA fragment read from a tile of 128-byte rows; 4:
  * 4-byte LDS reads in the pattern of the byte-pair decode table; 5: 16-byte LDS writes in the pattern of the
- * decoded weight tile (3..5 with 8 waves per compute unit).  One workgroup per compute unit (two for unit 1).
- * *work_per_launch receives the flops (0..2) or LDS bytes (3..5) of one launch; `sink`: 8 writable bytes. */
+ * decoded weight tile; 6: the same bytes as pairs of 8-byte writes; 7: 16-byte writes at consecutive addresses
+ * (3..7 with 8 waves per compute unit).  One workgroup per compute unit (two for unit 1).
+ * *work_per_launch receives the flops (0..2) or LDS bytes (3..7) of one launch; `sink`: 8 writable bytes. */
 int tuna_time_unit_rate(int unit, void *sink, int warmup, int iters, void *stream, float *elapsed_ms,
                         double *work_per_launch);
 

@@ -168,6 +168,7 @@ hipError_t launch_read(const void *src, void *sink, size_t bytes, int blocks, in
 // many-token kernel uses, measured the way the read kernel measures HBM --------------------------------
 typedef float rate_f32x16 __attribute__((ext_vector_type(16)));
 typedef float rate_f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t rate_u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kRateIters = 4096;
 
 // Independent MFMAs back to back, nothing else: NACC accumulators per wave, 4 waves per workgroup.
@@ -211,7 +212,7 @@ __global__ __launch_bounds__(256) void mfma_rate_kernel(uint32_t *sink)
 // MODE 0: 16-byte reads the way a wave reads an MFMA fragment from a tile of 128-byte rows (lane = row 0..15 x
 // k-group, slot ^ (row & 7)); 1: 4-byte reads the way the decode reads the byte-pair table ((byte << 8) | (lane
 // << 2), byte from a counter); 2: 16-byte writes the way the decoded weights are stored (4 rows x 8 k-blocks
-// per 32 lanes).
+// per 32 lanes); 3: the same bytes as two 8-byte writes each; 4: 16-byte writes at consecutive addresses.
 template <int MODE>
 __global__ __launch_bounds__(512) void lds_rate_kernel(uint32_t *sink)
 {
@@ -239,6 +240,34 @@ __global__ __launch_bounds__(512) void lds_rate_kernel(uint32_t *sink)
                 asm volatile("" : "+v"(off));
                 s += *reinterpret_cast<const uint32_t *>(smem + off);
             }
+    } else if constexpr (MODE == 3) {
+        const int half = lane & 1, kb = (lane >> 1) & 7, mbl = lane >> 4;
+        rate_u32x2 v = {(uint32_t)threadIdx.x, 1u};
+        for (int it = 0; it < kRateIters; ++it) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = mbl * 8 + half * 4 + ((r >> 1) & 3);
+                uint32_t off = (uint32_t)(row * 128 + ((kb ^ (row & 7)) << 4) + (r & 1) * 8 + wave * 4096 + ((it + (r >> 3)) & 1) * 32768) & 65535u;
+                asm volatile("" : "+v"(off));
+                *reinterpret_cast<rate_u32x2 *>(smem + off) = v;
+            }
+            v[0] += 1u;
+        }
+        __syncthreads();
+        s = smem[threadIdx.x];
+    } else if constexpr (MODE == 4) {
+        u32x4 v = {(uint32_t)threadIdx.x, 1u, 2u, 3u};
+        for (int it = 0; it < kRateIters; ++it) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                uint32_t off = (uint32_t)(lane * 16 + r * 1024 + wave * 8192) & 65535u;
+                asm volatile("" : "+v"(off));
+                *reinterpret_cast<u32x4 *>(smem + off) = v;
+            }
+            v[0] += 1u;
+        }
+        __syncthreads();
+        s = smem[threadIdx.x];
     } else {
         const int half = lane & 1, kb = (lane >> 1) & 7, mbl = lane >> 4;
         u32x4 v = {(uint32_t)threadIdx.x, 1u, 2u, 3u};
@@ -259,11 +288,12 @@ __global__ __launch_bounds__(512) void lds_rate_kernel(uint32_t *sink)
 }
 
 // unit: 0 / 1 v_mfma_f32_16x16x32_f16 with one / two waves per SIMD (16 accumulators), 2 v_mfma_f32_32x32x16_f16
-// (one wave per SIMD, 4 accumulators); 3 LDS fragment reads, 4 LDS table reads, 5 LDS tile writes.  *work =
-// flops (0..2) or bytes (3..5) of one launch on `cus` compute units.
+// (one wave per SIMD, 4 accumulators); 3 LDS fragment reads, 4 LDS table reads, 5 LDS tile writes, 6 the tile
+// writes as 8-byte halves, 7 16-byte writes at consecutive addresses.  *work = flops (0..2) or bytes (3..7) of
+// one launch on `cus` compute units.
 hipError_t launch_unit_rate(int unit, int cus, uint32_t *sink, double *work, hipStream_t stream)
 {
-    static OptInFlag attr[16][3];
+    static OptInFlag attr[16][5];
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
@@ -281,6 +311,12 @@ hipError_t launch_unit_rate(int unit, int cus, uint32_t *sink, double *work, hip
     case 5:
         if ((e = ensure_lds_opt_in(attr[dev][2], reinterpret_cast<const void *>(lds_rate_kernel<2>))) != hipSuccess) return e;
         hipLaunchKernelGGL(lds_rate_kernel<2>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 16.0; break;
+    case 6:
+        if ((e = ensure_lds_opt_in(attr[dev][3], reinterpret_cast<const void *>(lds_rate_kernel<3>))) != hipSuccess) return e;
+        hipLaunchKernelGGL(lds_rate_kernel<3>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 16.0; break;
+    case 7:
+        if ((e = ensure_lds_opt_in(attr[dev][4], reinterpret_cast<const void *>(lds_rate_kernel<4>))) != hipSuccess) return e;
+        hipLaunchKernelGGL(lds_rate_kernel<4>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 16.0; break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
