@@ -578,6 +578,46 @@ def test_many_token_kernel_with_32x32_mfma_tiles_matches_oracle(tile, m, n, k, s
     assert rel_err(f16_bits_to_f64(got), f16_bits_to_f64(other)) <= 2e-3   # one fp16 ulp of the larger outputs
 
 
+@pytest.mark.parametrize("mfma_rows", [64, 32])
+@pytest.mark.parametrize("m,n,k,split", [(512, 256, 512, 1), (520, 300, 1088, 1), (256, 70, 2048, 4), (1024, 129, 192, 3),
+                                         (256, 40, 64, 1), (264, 130, 192, 1), (512, 600, 320, 1), (768, 513, 576, 2),
+                                         (256, 256, 128, 1), (1280, 1024, 256, 1)])
+def test_many_token_kernel_with_the_256_x_256_tile_matches_oracle_and_the_smaller_tiles(mfma_rows, m, n, k, split):
+    """The 256 x 256 tile (one wave per SIMD, a wave owns 128 x 128) with both MFMA shapes: ragged m and n,
+    split-K with a remainder, k ranges of 1 ... 32 steps per workgroup (its loop is unrolled by two: odd and even
+    lengths), against the oracle's float64 sums; run-to-run identical; and, unsplit, the bits of the 128 x 128
+    tile with the same MFMA shape (the same products added in the same order)."""
+    from tuna_amd import ops
+
+    c = cfg(lds_tile_rows=256, token_tiles=16, split_k=split, rows_per_wave=mfma_rows)
+    assert "gemm_wide_kernel" in ops.describe_launch(m, n, k, c)
+    print(f"many-token tile 256x256 mfma_rows={mfma_rows} m={m} n={n} k={k} split={split}", flush=True)
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=m + n + split)
+    got = run_gemm(q, x, code, absmax, m, n, k, config=c, prefill=float("nan"))
+    ref = O.gemm_f64(q, x, code, absmax, m, n, k, mode=O.D1)
+    e = rel_err(f16_bits_to_f64(got), ref)
+    assert e <= REL_TOL, e                                   # max relative error 1e-2
+    again = run_gemm(q, x, code, absmax, m, n, k, config=c, prefill=float("nan"))
+    assert np.array_equal(got, again)
+    if split == 1:
+        small = run_gemm(q, x, code, absmax, m, n, k, config=cfg(lds_tile_rows=128, token_tiles=8, rows_per_wave=mfma_rows),
+                         prefill=float("nan"))
+        assert np.array_equal(got, small)
+
+
+def test_the_256_x_256_tile_rejects_k_that_is_not_a_multiple_of_64():
+    import torch
+
+    from tuna_amd import ops
+
+    m, n, k = 256, 256, 200
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=2)
+    dq, dx, dc, da = to_dev(q, x, code, absmax)
+    out = torch.empty((n, m), dtype=torch.float16, device="cuda")
+    with pytest.raises(ops.TunaError):
+        ops.matmul(dx, dq, da, dc, out, m, n, k, config=cfg(lds_tile_rows=256, token_tiles=16))
+
+
 def test_many_token_kernel_decode_readout_is_bit_exact():
     """One-hot activations turn the GEMM into a readout of the decoded weights: bit-exact D1."""
     m, k = 256, 256
@@ -590,6 +630,10 @@ def test_many_token_kernel_decode_readout_is_bit_exact():
     assert np.array_equal(got.T, want)
     got32 = run_gemm(q, x, code, absmax, m, k, k, config=cfg(lds_tile_rows=128, token_tiles=8, rows_per_wave=32), prefill=float("nan"))
     assert np.array_equal(got32.T, want)                        # 32 x 32 x 16 MFMA tiles: the same read-out
+    for mfma_rows in (64, 32):                                  # the 256 x 256 tile, both MFMA shapes
+        wide = run_gemm(q, x, code, absmax, m, k, k, config=cfg(lds_tile_rows=256, token_tiles=16, rows_per_wave=mfma_rows),
+                        prefill=float("nan"))
+        assert np.array_equal(wide.T, want)
 
 
 # ----------------------------------------------------------------------------- stream capture / graph replay, several streams
@@ -725,6 +769,8 @@ FUSED_CFGS = [
     dict(split_k=0, waves_m=1, waves_k=8, prefetch=2, x_chunk=512),      # balanced split
     dict(lds_tile_rows=128, token_tiles=8, split_k=1),                   # many-token kernel
     dict(lds_tile_rows=64, token_tiles=8, split_k=2),                    # many-token kernel, split-K
+    dict(lds_tile_rows=256, token_tiles=16, split_k=1),                  # 256 x 256 tile
+    dict(lds_tile_rows=256, token_tiles=16, split_k=2, rows_per_wave=32),  # 256 x 256 tile, 32 x 32 MFMA tiles, split-K
 ]
 
 
@@ -737,6 +783,8 @@ def test_fused_residual_and_silu_mul_epilogues(ci):
     from tuna_amd import _lib, ops
 
     m, n, k = 1024, 48, 1096
+    if FUSED_CFGS[ci].get("lds_tile_rows") == 256:
+        k = 1088                                                         # that tile takes k in multiples of 64
     c = cfg(**FUSED_CFGS[ci])
     print(f"fused cfg#{ci} {c.to_dict()}", flush=True)
     q, x, code, absmax = make_inputs_np(m, n, k, seed=60 + ci)

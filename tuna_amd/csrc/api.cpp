@@ -222,6 +222,9 @@ static int plan_tiled(int m, int n, int k, const tuna_gemm_config &c, int decode
     if (!tiled_variant_exists(c.lds_tile_rows, tile_tokens, mfma32))
         return fail(TUNA_ERR_UNSUPPORTED, "no many-token kernel for a %d x %d tile (rows x tokens)%s", c.lds_tile_rows, tile_tokens,
                     mfma32 ? " with 32 x 32 MFMA tiles" : "");
+    if (c.lds_tile_rows == 256 && tile_tokens == 256 &&
+        (k % 64 != 0 || (unsigned long long)m * (unsigned)k / 2 >= (1ull << 32) || (unsigned long long)n * (unsigned)k * 2 >= (1ull << 32)))
+        return fail(TUNA_ERR_UNSUPPORTED, "the 256 x 256 many-token tile needs k a multiple of 64 and q and x below 4 GB");
     const int steps = ceil_div(k, 64);
     if (c.split_k < 1 || c.split_k > steps)
         return fail(TUNA_ERR_UNSUPPORTED, "split_k=%d must be in 1..%d for the many-token kernel", c.split_k, steps);
@@ -1642,7 +1645,7 @@ TUNA_EXPORT int tuna_time_unit_rate(int unit, void *sink, int warmup, int iters,
 {
     int rc;
     if ((rc = check_ptr(sink, "sink", 4))) return rc;
-    if (unit < 0 || unit > 7) return fail(TUNA_ERR_INVALID_ARG, "unit %d outside 0..7", unit);
+    if (unit < 0 || unit > 13) return fail(TUNA_ERR_INVALID_ARG, "unit %d outside 0..13", unit);
     if (!work_per_launch) return fail(TUNA_ERR_INVALID_ARG, "work_per_launch is null");
     int dev = 0, cus = 0;
     hipError_t e = device_cus(&dev, &cus);
@@ -1682,8 +1685,9 @@ TUNA_EXPORT int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config
     if (c.lds_tile_rows > 0) {
         TiledPlan tp;
         if ((rc = plan_tiled(m, n, k, c, decode_mode, &tp))) return rc;
-        snprintf(buf, len, "gemm_tiled_kernel<%d rows x %d tokens%s> split_k=%d", tp.tile_rows, tp.tile_tokens,
-                 tp.mfma32 ? ",mfma 32x32x16" : "", c.split_k);
+        const bool wide = tp.tile_rows == 256 && tp.tile_tokens == 256;  // gemm_wide.hip: one wave per SIMD
+        snprintf(buf, len, "%s<%d rows x %d tokens%s> split_k=%d", wide ? "gemm_wide_kernel" : "gemm_tiled_kernel", tp.tile_rows,
+                 tp.tile_tokens, tp.mfma32 ? ",mfma 32x32x16" : "", c.split_k);
         return TUNA_OK;
     }
     if (is_narrow(c)) {

@@ -171,16 +171,28 @@ typedef float rate_f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t rate_u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kRateIters = 4096;
 
-// Independent MFMAs back to back, nothing else: NACC accumulators per wave, 4 waves per workgroup.
-template <bool M32, int NACC>
+// Independent MFMAs back to back, nothing else: NACC accumulators per wave, 4 waves per workgroup.  RANDOM: the
+// operands are four + four registers of pseudo-random fp16 values in (-1, 1) instead of one pair of small
+// regular numbers - what the matrix cores draw, and the clock they are then given, depends on the bits that toggle.
+template <bool M32, int NACC, bool RANDOM = false>
 __global__ __launch_bounds__(256) void mfma_rate_kernel(uint32_t *sink)
 {
-    f16x8 a, b;
+    constexpr int NOP = RANDOM ? 4 : 1;
+    f16x8 a[NOP], b[NOP];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        a[e] = (f16)(0.001f * (float)threadIdx.x + (float)e);
-        b[e] = (f16)(0.5f * (float)e);
-    }
+    for (int o = 0; o < NOP; ++o)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if constexpr (RANDOM) {
+                uint32_t h = (threadIdx.x * 8u + e + o * 4099u + blockIdx.x * 131071u) * 2654435761u;
+                h ^= h >> 15, h *= 2246822519u, h ^= h >> 13;
+                a[o][e] = (f16)((float)(int)(h & 0xffffu) * (1.0f / 32768.0f) - 1.0f);
+                b[o][e] = (f16)((float)(int)(h >> 16) * (1.0f / 32768.0f) - 1.0f);
+            } else {
+                a[o][e] = (f16)(0.001f * (float)threadIdx.x + (float)e);
+                b[o][e] = (f16)(0.5f * (float)e);
+            }
+        }
     float s = 0.f;
     if constexpr (M32) {
         rate_f32x16 acc[NACC];
@@ -190,7 +202,8 @@ __global__ __launch_bounds__(256) void mfma_rate_kernel(uint32_t *sink)
             for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
         for (int it = 0; it < kRateIters; ++it)
 #pragma unroll
-            for (int i = 0; i < NACC; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i], 0, 0, 0);
+            for (int i = 0; i < NACC; ++i)
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[(i >> 2) % NOP], b[i % NOP], acc[i], 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < NACC; ++i)
 #pragma unroll
@@ -201,7 +214,8 @@ __global__ __launch_bounds__(256) void mfma_rate_kernel(uint32_t *sink)
         for (int i = 0; i < NACC; ++i) acc[i] = rate_f32x4{0.f, 0.f, 0.f, 0.f};
         for (int it = 0; it < kRateIters; ++it)
 #pragma unroll
-            for (int i = 0; i < NACC; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[i], 0, 0, 0);
+            for (int i = 0; i < NACC; ++i)
+                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[(i >> 2) % NOP], b[i % NOP], acc[i], 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < NACC; ++i) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
     }
@@ -237,6 +251,15 @@ __global__ __launch_bounds__(512) void lds_rate_kernel(uint32_t *sink)
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
                 uint32_t off = ((uint32_t)((it * 8 + r + wave * 31) & 255) << 8) | ((uint32_t)lane << 2);
+                asm volatile("" : "+v"(off));
+                s += *reinterpret_cast<const uint32_t *>(smem + off);
+            }
+    } else if constexpr (MODE == 5 || MODE == 6) {
+        constexpr int REP = MODE == 5 ? 32 : 16;  // lanes that have a copy of the table of their own
+        for (int it = 0; it < kRateIters; ++it)
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                uint32_t off = ((uint32_t)(((it * 8 + r) * 37 + wave * 31 + lane * lane * 13 + (lane >> 3)) & 255) * (REP * 4)) | ((uint32_t)(lane % REP) << 2);
                 asm volatile("" : "+v"(off));
                 s += *reinterpret_cast<const uint32_t *>(smem + off);
             }
@@ -293,7 +316,7 @@ __global__ __launch_bounds__(512) void lds_rate_kernel(uint32_t *sink)
 // one launch on `cus` compute units.
 hipError_t launch_unit_rate(int unit, int cus, uint32_t *sink, double *work, hipStream_t stream)
 {
-    static OptInFlag attr[16][5];
+    static OptInFlag attr[16][7];
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
@@ -317,6 +340,16 @@ hipError_t launch_unit_rate(int unit, int cus, uint32_t *sink, double *work, hip
     case 7:
         if ((e = ensure_lds_opt_in(attr[dev][4], reinterpret_cast<const void *>(lds_rate_kernel<4>))) != hipSuccess) return e;
         hipLaunchKernelGGL(lds_rate_kernel<4>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 16.0; break;
+    case 10: hipLaunchKernelGGL((mfma_rate_kernel<true, 16, true>), dim3(cus), dim3(256), 0, stream, sink); *work = (double)cus * 4 * kRateIters * 16 * 32768.0; break;
+    case 11: hipLaunchKernelGGL((mfma_rate_kernel<false, 16, true>), dim3(2 * cus), dim3(256), 0, stream, sink); *work = (double)cus * 8 * kRateIters * 16 * 16384.0; break;
+    case 12: hipLaunchKernelGGL((mfma_rate_kernel<false, 16, true>), dim3(cus), dim3(256), 0, stream, sink); *work = (double)cus * 4 * kRateIters * 16 * 16384.0; break;
+    case 13: hipLaunchKernelGGL((mfma_rate_kernel<true, 16, true>), dim3(2 * cus), dim3(256), 0, stream, sink); *work = (double)cus * 8 * kRateIters * 16 * 32768.0; break;
+    case 8:
+        if ((e = ensure_lds_opt_in(attr[dev][5], reinterpret_cast<const void *>(lds_rate_kernel<5>))) != hipSuccess) return e;
+        hipLaunchKernelGGL(lds_rate_kernel<5>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 4.0; break;
+    case 9:
+        if ((e = ensure_lds_opt_in(attr[dev][6], reinterpret_cast<const void *>(lds_rate_kernel<6>))) != hipSuccess) return e;
+        hipLaunchKernelGGL(lds_rate_kernel<6>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 4.0; break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

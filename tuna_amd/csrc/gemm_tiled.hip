@@ -442,17 +442,23 @@ static constexpr int kNumTiled = sizeof(kTiled) / sizeof(kTiled[0]);
 
 bool tiled_variant_exists(int bm, int bn, bool mfma32)
 {
+    if (bm == 256 && bn == 256) return true;  // gemm_wide.hip
     for (int i = 0; i < kNumTiled; ++i)
         if (kTiled[i].bm == bm && kTiled[i].bn == bn) return !mfma32 || kTiled[i].fn32 != nullptr;
     return false;
 }
 
-size_t tiled_lds_bytes(int bm, int bn) { return (size_t)kLutBytes + 2 * (size_t)(bm + bn) * 128; }  // two tile buffers
+size_t tiled_lds_bytes(int bm, int bn)
+{
+    if (bm == 256 && bn == 256) return wide_lds_bytes();
+    return (size_t)kLutBytes + 2 * (size_t)(bm + bn) * 128;  // two tile buffers
+}
 
 static OptInFlag g_tiled_attr[16][kNumTiled][3];
 
 hipError_t launch_gemm_tiled(const TiledArgs &args, int bm, int bn, bool mfma32, hipStream_t stream, bool scale_blocks)
 {
+    if (bm == 256 && bn == 256) return !scale_blocks ? launch_gemm_wide(args, mfma32, stream) : hipErrorInvalidConfiguration;
     int vi = -1;
     for (int i = 0; i < kNumTiled; ++i)
         if (kTiled[i].bm == bm && kTiled[i].bn == bn) vi = i;

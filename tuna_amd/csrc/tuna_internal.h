@@ -204,6 +204,9 @@ hipError_t device_cus(int *dev, int *cus);
 // gemm_tiled.hip
 hipError_t launch_gemm_tiled(const TiledArgs &args, int tile_rows, int tile_tokens, bool mfma32, hipStream_t stream,
                              bool scale_blocks = false);
+// 256 x 256 tile, one wave per SIMD (gemm_wide.hip): reached through launch_gemm_tiled
+size_t wide_lds_bytes();
+hipError_t launch_gemm_wide(const TiledArgs &args, bool mfma32, hipStream_t stream);
 bool tiled_variant_exists(int tile_rows, int tile_tokens, bool mfma32);
 size_t tiled_lds_bytes(int tile_rows, int tile_tokens);
 

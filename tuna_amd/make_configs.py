@@ -64,8 +64,10 @@ NARROW_VARIANTS = (
     | {(r, wk, pf, 4) for r in (16, 32) for wk in (4, 8) for pf in (2, 4)} | {(64, 4, 2, 4), (64, 8, 2, 4)}
     | {(24, 8, 2, 1), (24, 8, 4, 1), (24, 8, 8, 1), (24, 16, 2, 1), (24, 16, 4, 1)})
 
-# (rows, tokens) tiles of the many-token kernel; must match kTiled in csrc/gemm_tiled.hip
-TILED_VARIANTS = {(256, 128), (256, 64), (128, 256), (128, 128), (64, 256), (64, 128)}
+# (rows, tokens) tiles of the many-token kernels; must match kTiled in csrc/gemm_tiled.hip, plus the 256 x 256 tile
+# of csrc/gemm_wide.hip (one wave per SIMD; k a multiple of 64)
+TILED_VARIANTS = {(256, 256), (256, 128), (256, 64), (128, 256), (128, 128), (64, 256), (64, 128)}
+WIDE_LUT_BYTES = 256 * 32 * 4
 
 
 def _pow2(v: int) -> bool:
@@ -105,6 +107,8 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
             raise ValueError("the 64 x 128 tile has no 32 x 32 MFMA variant (one 16-token tile per wave)")
         if not 1 <= c["split_k"] <= -(-k // 64):
             raise ValueError("split_k of the many-token kernel must be in 1..ceil(k/64)")
+        if (c["lds_tile_rows"], 16 * c["token_tiles"]) == (256, 256) and k % 64:
+            raise ValueError("the 256 x 256 many-token tile needs k a multiple of 64")
         return
     if is_narrow(c):
         # narrow-row kernel: one workgroup per 16, 32 or 64 rows, all waves along k, no split
@@ -211,7 +215,8 @@ def lds_bytes(c: dict) -> int:
     64-row group and token tile) when that costs no occupancy (mirrors plan_gemm in csrc/api.cpp)."""
     if c.get("lds_tile_rows", 0) > 0:
         # many-token kernel: decode table + two buffers of (weight tile + activation tile), 128 bytes per row
-        return LUT_BYTES + 2 * (c["lds_tile_rows"] + 16 * c["token_tiles"]) * 128
+        wide = (c["lds_tile_rows"], 16 * c["token_tiles"]) == (256, 256)
+        return (WIDE_LUT_BYTES if wide else LUT_BYTES) + 2 * (c["lds_tile_rows"] + 16 * c["token_tiles"]) * 128
     if is_narrow(c):
         # narrow-row kernel: decode table + one accumulator plane (1 KB) per wave and 16 rows
         return LUT_BYTES + c["waves_k"] * ((c["rows_per_wave"] + 15) // 16) * c["token_tiles"] * 1024
