@@ -57,9 +57,14 @@ int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int va
  * one / two waves per SIMD (16 accumulators each); 2: v_mfma_f32_32x32x16_f16 from one wave per SIMD (4
  * accumulators); 3: 16-byte LDS reads in the pattern of an MFMA fragment read from a tile of 128-byte rows; 4:
  * 4-byte LDS reads in the pattern of the byte-pair decode table; 5: 16-byte LDS writes in the pattern of the
- * decoded weight tile; 6: the same bytes as pairs of 8-byte writes; 7: 16-byte writes at consecutive addresses
- * (3..7 with 8 waves per compute unit).  One workgroup per compute unit (two for unit 1).
- * *work_per_launch receives the flops (0..2) or LDS bytes (3..7) of one launch; `sink`: 8 writable bytes. */
+ * decoded weight tile; 6: the same bytes as pairs of 8-byte writes; 7: 16-byte writes at consecutive addresses;
+ * 8 / 9: the table reads of 4 with one copy of the table per 32 / 16 lanes instead of per 64, a pseudo-random byte
+ * per lane (3..9 with 8 waves per compute unit); 10 / 13: v_mfma_f32_32x32x16_f16 from one / two waves per SIMD and
+ * 12 / 11: v_mfma_f32_16x16x32_f16 from one / two waves per SIMD, 16 accumulators, with four + four operand
+ * registers of pseudo-random fp16 values in (-1, 1) - the rate the matrix cores sustain on real data, which is
+ * well below the rate on the regular operands of units 0..2.  One workgroup per compute unit (two for units 1,
+ * 11, 13).  *work_per_launch receives the flops (0..2, 10..13) or LDS bytes (3..9) of one launch; `sink`: 8
+ * writable bytes. */
 int tuna_time_unit_rate(int unit, void *sink, int warmup, int iters, void *stream, float *elapsed_ms,
                         double *work_per_launch);
 

@@ -222,9 +222,8 @@ static int plan_tiled(int m, int n, int k, const tuna_gemm_config &c, int decode
     if (!tiled_variant_exists(c.lds_tile_rows, tile_tokens, mfma32))
         return fail(TUNA_ERR_UNSUPPORTED, "no many-token kernel for a %d x %d tile (rows x tokens)%s", c.lds_tile_rows, tile_tokens,
                     mfma32 ? " with 32 x 32 MFMA tiles" : "");
-    if (c.lds_tile_rows == 256 && tile_tokens == 256 &&
-        (k % 64 != 0 || (unsigned long long)m * (unsigned)k / 2 >= (1ull << 32) || (unsigned long long)n * (unsigned)k * 2 >= (1ull << 32)))
-        return fail(TUNA_ERR_UNSUPPORTED, "the 256 x 256 many-token tile needs k a multiple of 64 and q and x below 4 GB");
+    if (c.lds_tile_rows == 256 && tile_tokens == 256 && k % 64 != 0)
+        return fail(TUNA_ERR_UNSUPPORTED, "the 256 x 256 many-token tile needs k a multiple of 64");
     const int steps = ceil_div(k, 64);
     if (c.split_k < 1 || c.split_k > steps)
         return fail(TUNA_ERR_UNSUPPORTED, "split_k=%d must be in 1..%d for the many-token kernel", c.split_k, steps);

@@ -226,7 +226,8 @@ __global__ __launch_bounds__(256) void mfma_rate_kernel(uint32_t *sink)
 // MODE 0: 16-byte reads the way a wave reads an MFMA fragment from a tile of 128-byte rows (lane = row 0..15 x
 // k-group, slot ^ (row & 7)); 1: 4-byte reads the way the decode reads the byte-pair table ((byte << 8) | (lane
 // << 2), byte from a counter); 2: 16-byte writes the way the decoded weights are stored (4 rows x 8 k-blocks
-// per 32 lanes); 3: the same bytes as two 8-byte writes each; 4: 16-byte writes at consecutive addresses.
+// per 32 lanes); 3: the same bytes as two 8-byte writes each; 4: 16-byte writes at consecutive addresses; 5 / 6:
+// the table reads of 1 with one copy of the table per 32 / 16 lanes and a pseudo-random byte per lane.
 template <int MODE>
 __global__ __launch_bounds__(512) void lds_rate_kernel(uint32_t *sink)
 {
@@ -312,8 +313,9 @@ __global__ __launch_bounds__(512) void lds_rate_kernel(uint32_t *sink)
 
 // unit: 0 / 1 v_mfma_f32_16x16x32_f16 with one / two waves per SIMD (16 accumulators), 2 v_mfma_f32_32x32x16_f16
 // (one wave per SIMD, 4 accumulators); 3 LDS fragment reads, 4 LDS table reads, 5 LDS tile writes, 6 the tile
-// writes as 8-byte halves, 7 16-byte writes at consecutive addresses.  *work = flops (0..2) or bytes (3..7) of
-// one launch on `cus` compute units.
+// writes as 8-byte halves, 7 16-byte writes at consecutive addresses, 8 / 9 table reads with a copy of the table
+// per 32 / 16 lanes; 10 / 13 32x32x16 and 12 / 11 16x16x32 MFMAs on pseudo-random operands from one / two waves per
+// SIMD.  *work = flops (0..2, 10..13) or bytes (3..9) of one launch on `cus` compute units.
 hipError_t launch_unit_rate(int unit, int cus, uint32_t *sink, double *work, hipStream_t stream)
 {
     static OptInFlag attr[16][7];

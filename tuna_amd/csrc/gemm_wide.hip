@@ -24,7 +24,7 @@
 //     contiguous bytes of a block row's k-step; weights and activations come through buffer loads (descriptor in
 //     scalar registers, one 32-bit offset per lane, the k-step as a scalar offset): no 64-bit address
 //     arithmetic in the loop, which a single wave per SIMD would pay for in MFMA issue slots.
-// k must be a multiple of 64 and q and x smaller than 4 GB (32-bit offsets from uniform bases); the host checks.
+// k must be a multiple of 64; the host checks.
 //
 // Decode and rounding are those of the other kernels (bit-identical to kernel.cu:2178-2192); the sums are the
 // same products in the same order as the variants of gemm_tiled.hip with the same MFMA shape.
@@ -75,10 +75,11 @@ __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(const TiledA
     const int mb_last = (a.m >> 3) - 1;
 
     // weights: thread -> block row tid / 8 of the tile, k-block tid % 8 of the step (rows beyond the matrix are
-    // clamped: their products are never stored).  Addresses are a uniform base that advances with the k-step
-    // plus a 32-bit offset per thread: no 64-bit vector arithmetic in the loop, short address operands.
+    // clamped: their products are never stored).  Addresses are a uniform base - the tile's first block row, first
+    // token - that advances with the k-step, plus a 32-bit offset per thread inside the tile: no 64-bit vector
+    // arithmetic in the loop, short address operands, no limit on the size of q or x.
     const int a_kb = tid & 7, a_mbl = tid >> 3;
-    const uint32_t a_off = ((uint32_t)min((row_base >> 3) + a_mbl, mb_last) * (uint32_t)kb_total + (uint32_t)a_kb) * 32u;
+    const uint32_t a_off = ((uint32_t)(min((row_base >> 3) + a_mbl, mb_last) - (row_base >> 3)) * (uint32_t)kb_total + (uint32_t)a_kb) * 32u;
     f16x2 sc16[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -92,7 +93,7 @@ __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(const TiledA
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int tok = tok_base + (tid >> 3) + 32 * i;
-        x_off[i] = ((uint32_t)min(tok, a.n - 1) * (uint32_t)a.k + (uint32_t)(tid & 7) * 8u) * 2u;
+        x_off[i] = ((uint32_t)(min(tok, a.n - 1) - tok_base) * (uint32_t)a.k + (uint32_t)(tid & 7) * 8u) * 2u;
     }
     unsigned char *x_dst = x_tile + (tid >> 3) * 128 + (((tid & 7) ^ ((tid >> 3) & 7)) << 4);  // piece i: + i * 4096
 
@@ -100,10 +101,12 @@ __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(const TiledA
     u32x4 xr[XSETS][8];
     // buffer loads: descriptor + 32-bit offset per lane + uniform offset of the k-step (weights without the
     // nontemporal hint: the token tiles of a row tile run side by side and share them through the L2)
-    const __amdgpu_buffer_rsrc_t q_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(a.q), 0, (int)((uint32_t)a.m * (uint32_t)(a.k >> 1)), 0x00020000);
-    const __amdgpu_buffer_rsrc_t x_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(a.x), 0, (int)((uint32_t)a.n * (uint32_t)a.k * 2u), 0x00020000);
+    const size_t q_rest = (size_t)(a.m - row_base) * (size_t)(a.k >> 1), x_rest = (size_t)(a.n - tok_base) * (size_t)a.k * 2;
+    const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t *>(a.q) + (size_t)(row_base >> 3) * kb_total * 32, 0, (int)(uint32_t)min(q_rest, (size_t)0xffffffffu), 0x00020000);
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        reinterpret_cast<unsigned char *>(const_cast<void *>(a.x)) + (size_t)tok_base * a.k * 2, 0,
+        (int)(uint32_t)min(x_rest, (size_t)0xffffffffu), 0x00020000);
 #define TUNA_WIDE_LOAD(set, s)                                                                  \
     {                                                                                          \
         wq[set][0] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, (int)a_off, (s) * 256, 0);  \
