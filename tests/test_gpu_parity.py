@@ -389,6 +389,45 @@ def test_reference_table_2560_wide_shapes_every_bucket(m, k, n):
     assert e <= REL_TOL
 
 
+@pytest.mark.parametrize("m,k,n,split", [(12288, 1024, 1000, 1), (5120, 4096, 1300, 2), (5120, 1024, 1300, None)])
+def test_derived_config_for_an_untuned_shape_with_very_many_tokens(m, k, n, split):
+    """A shape outside the table with 768 tokens or more gets the 256 x 256 many-token tile when its tiles fill the
+    device (192 tiles; 120 tiles with the k range split in two; not with 120 tiles and a short k), through the plain
+    entry point; checked on a random subset of rows."""
+    import torch
+
+    from tuna_amd import ops
+    from tuna_amd.quantize import nf4_codebook
+    from tuna_amd.synth import make_weights_torch, make_x_torch
+
+    cfg, hit = ops.select_config(m, n, k)
+    assert not hit
+    if split is None:
+        assert (cfg.lds_tile_rows, cfg.token_tiles) != (256, 16)
+    else:
+        assert (cfg.lds_tile_rows, cfg.token_tiles, cfg.split_k) == (256, 16, split)
+        assert "gemm_wide_kernel" in ops.describe_launch(m, n, k, None)
+    print(f"derived config m={m} n={n} k={k} {cfg.to_dict()}", flush=True)
+    dev = torch.device("cuda")
+    q, absmax = make_weights_torch(m, k, seed=7, device=dev)
+    x = make_x_torch(n, k, seed=8, device=dev)
+    code = nf4_codebook(dev)
+    out = torch.full((n, m), float("nan"), dtype=torch.float16, device=dev)
+    ops.matmul(x, q, absmax, code, out, m, n, k)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    rng = np.random.default_rng(13)
+    mbs = np.sort(rng.choice(m // 8, size=16, replace=False))
+    rows = (mbs[:, None] * 8 + np.arange(8)[None, :]).ravel()
+    q_sub = q[torch.from_numpy(mbs).to(dev)].cpu().numpy()
+    ref = O.gemm_f64(q_sub, x.cpu().numpy().view(np.uint16), code.cpu().numpy(), absmax.cpu().numpy()[rows],
+                     len(rows), n, k, mode=O.D1)
+    got = out.cpu().numpy().view(np.uint16)[:, rows]
+    e = rel_err(f16_bits_to_f64(got), ref)
+    print(f"  rel_err={e:.3e}", flush=True)
+    assert e <= REL_TOL                                      # max relative error 1e-2
+
+
 @pytest.mark.parametrize("m,k,n,tiles", [(66560, 1024, 50, 4), (66560, 1024, 100, 8), (66560, 1024, 300, 8),
                                          (16384, 2048, 100, 4)])
 def test_derived_config_for_a_large_untuned_shape_with_many_tokens(m, k, n, tiles):
@@ -1559,11 +1598,12 @@ def test_blockwise_gemm_through_the_batched_streaming_kernel(m, n, k, bs):
 
 
 @pytest.mark.parametrize("m,n,k,bs", [(512, 64, 1024, 64), (528, 130, 2048, 128), (1024, 300, 4096, 64), (256, 1024, 512, 256),
-                                      (4096, 33, 4096, 64), (272, 200, 1280, 64)])
+                                      (4096, 33, 4096, 64), (272, 200, 1280, 64), (12288, 1000, 1024, 64)])
 def test_blockwise_gemm_with_many_tokens_through_the_many_token_kernel(m, n, k, bs):
     """From 33 tokens tuna_matmul_blockwise decodes a weight tile once per workgroup with the scale of each k-step's block
     (the many-token kernel's scale-block variants): against the oracle's float64 sums over the blockwise D1 weights (row
-    sample), bit-exact through one-hot activations, run-to-run identical; ragged m / n, k ranges of 8 to 64 steps."""
+    sample), bit-exact through one-hot activations, run-to-run identical; ragged m / n, k ranges of 8 to 64 steps; the
+    last case is a shape whose per-row config is the 256 x 256 tile, which has no scale-block variant."""
     import torch
 
     from tuna_amd import _lib, ops

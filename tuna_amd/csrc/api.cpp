@@ -415,6 +415,21 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         c.token_tiles = 4;
         if (config_runs(m, n, k, c)) return c;
     }
+    if (n >= 768 && k % 64 == 0) {
+        // very many tokens: the 256 x 256 tile (one wave per SIMD) where it fills the device - from about 150
+        // tiles, or from 90 with the k range split in two when that leaves 32 steps per workgroup.  Measured on
+        // 12288 x 6144, 5120 x 5120, 16384 x 8192, 3072 x 9216 and 20480 x 5120 at 1024..8192 tokens: 5-38 %
+        // faster than the 128-token tiles below from 150 tiles (12288 x 6144 at 4096 tokens 842 -> 526 us),
+        // 10 % with the split at 96 tiles, slower at 80.
+        const long long tiles = (long long)ceil_div(m, 256) * ceil_div(n, 256);
+        const int split = tiles >= 150 ? 1 : (tiles >= 90 && k >= 64 * 64) ? 2 : 0;
+        if (split) {
+            memset(&c, 0, sizeof(c));
+            c.rows_per_wave = 64, c.waves_m = 1, c.waves_k = 1, c.prefetch = 2, c.x_chunk = 64;
+            c.token_tiles = 16, c.lds_tile_rows = 256, c.split_k = split;
+            return c;
+        }
+    }
     if (n >= 128) {
         // many tokens: the kernel that decodes each weight tile once into LDS; 128-token tiles,
         // 256 rows (128 for few rows), k split until about one workgroup per CU
@@ -1285,7 +1300,9 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
     if (n > 32 && stream_mode == 1) {
         tuna_gemm_config c;
         select_config(m, n, k, &c, nullptr);
-        if (c.lds_tile_rows <= 0 || !tiled_variant_exists(c.lds_tile_rows, 16 * c.token_tiles, false)) {
+        // (the 256 x 256 tile has no scale-block variant: its threads have no registers left for eight more scales)
+        if (c.lds_tile_rows <= 0 || !tiled_variant_exists(c.lds_tile_rows, 16 * c.token_tiles, false) ||
+            (c.lds_tile_rows == 256 && c.token_tiles == 16)) {
             c.lds_tile_rows = n > 64 ? 128 : 256;
             c.token_tiles = n > 128 ? 16 : n > 64 ? 8 : 4;
             // fewer tiles than compute units: split k until the launch fills them (at least eight k-steps per workgroup)
