@@ -354,6 +354,41 @@ def test_token_sweep_llama70b_layer_set(name, n):
     assert e <= REL_TOL
 
 
+@pytest.mark.parametrize("name,n", [("mistral_attn_out", 3072), ("mistral_down", 3100), ("llama70b_qkv", 4096)])
+def test_token_counts_far_into_the_last_bucket_take_the_256_x_256_tile(name, n):
+    """The last bucket of the table is open-ended and tuned at 2048 tokens; from 3072 tokens a shape of fewer than
+    24576 rows runs the 256 x 256 many-token tile through the plain entry point.  Row-subset check against the oracle."""
+    import torch
+
+    from tuna_amd import ops
+    from tuna_amd.quantize import nf4_codebook
+    from tuna_amd.synth import SHAPES, make_weights_torch, make_x_torch
+
+    m, k = SHAPES[name]
+    used, hit = ops.select_config(m, n, k)
+    assert hit and (used.lds_tile_rows, used.token_tiles) == (256, 16)
+    assert "gemm_wide_kernel" in ops.describe_launch(m, n, k, None)
+    print(f"last bucket {name} m={m} k={k} n={n}", flush=True)
+    dev = torch.device("cuda")
+    q, absmax = make_weights_torch(m, k, seed=n, device=dev)
+    x = make_x_torch(n, k, seed=n + 1, device=dev)
+    code = nf4_codebook(dev)
+    out = torch.full((n, m), float("nan"), dtype=torch.float16, device=dev)
+    ops.matmul(x, q, absmax, code, out, m, n, k)
+    torch.cuda.synchronize()
+    assert not torch.isnan(out).any()                       # every output was written
+    rng = np.random.default_rng(n)
+    mbs = np.sort(rng.choice(m // 8, size=4, replace=False))
+    rows = (mbs[:, None] * 8 + np.arange(8)[None, :]).ravel()
+    q_sub = q[torch.from_numpy(mbs).to(dev)].cpu().numpy()
+    ref = O.gemm_f64(q_sub, x.cpu().numpy().view(np.uint16), code.cpu().numpy(), absmax.cpu().numpy()[rows],
+                     len(rows), n, k, mode=O.D1)
+    got = out[:, torch.from_numpy(rows).to(dev)].cpu().numpy().view(np.uint16)
+    e = rel_err(f16_bits_to_f64(got), ref)
+    print(f"  rel_err={e:.3e}", flush=True)
+    assert e <= REL_TOL                                      # max relative error 1e-2
+
+
 @pytest.mark.parametrize("n", [1, 16, 40, 100, 200, 300, 600, 1000, 1500])
 @pytest.mark.parametrize("m,k", [(2560, 2560), (2560, 10240), (7680, 2560), (10240, 2560)])
 def test_reference_table_2560_wide_shapes_every_bucket(m, k, n):

@@ -470,7 +470,7 @@ static bool config_runs(int m, int n, int k, const tuna_gemm_config &c)
 // pass: measured on six of the benchmark shapes, 17..255 tokens, the next bucket's entry is 15-40 %
 // faster (8192 x 8192 at 20 tokens 23.8 -> 14.8 us, 57344 x 8192 at 24 tokens 81 -> 57 us,
 // 229376 x 4096 at 100 tokens 297 -> 237 us), so such a count takes it when it can run the shape.
-// Up to 15 tokens and from 256 tokens the containing bucket's entry stays.
+// Up to 15 tokens and from 256 tokens the containing bucket's entry stays (but see the last bucket below).
 static int select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_table)
 {
     const TableEntry *own = nullptr;
@@ -489,6 +489,16 @@ static int select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_t
     }
     if (own) {
         *cfg = own->cfg;
+        // The last bucket is open-ended and tuned at 2048 tokens.  From 3072 tokens a shape of fewer than 24576 rows
+        // takes the 256 x 256 many-token tile whatever its entry says, when that tile fills the device: measured on
+        // six benchmark shapes at 3072..8192 tokens it equals or beats every other entry there (4096 x 4096 at 8192
+        // tokens 336 -> 255 us, 4096 x 14336 at 4096 tokens 469 -> 392 us, 10240 x 8192 at 8192 tokens 1582 -> 1200 us).
+        if (n >= 3072 && m < 24576 && k % 64 == 0 && !(cfg->lds_tile_rows == 256 && cfg->token_tiles == 16) &&
+            (long long)ceil_div(m, 256) * ceil_div(n, 256) >= 150) {
+            memset(cfg, 0, sizeof(*cfg));
+            cfg->rows_per_wave = 64, cfg->waves_m = 1, cfg->waves_k = 1, cfg->prefetch = 2, cfg->x_chunk = 64;
+            cfg->token_tiles = 16, cfg->lds_tile_rows = 256, cfg->split_k = 1;
+        }
         if (from_table) *from_table = 1;
         return TUNA_OK;
     }
