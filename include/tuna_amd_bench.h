@@ -62,9 +62,10 @@ int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int va
  * per lane (3..9 with 8 waves per compute unit); 10 / 13: v_mfma_f32_32x32x16_f16 from one / two waves per SIMD and
  * 12 / 11: v_mfma_f32_16x16x32_f16 from one / two waves per SIMD, 16 accumulators, with four + four operand
  * registers of pseudo-random fp16 values in (-1, 1) - the rate the matrix cores sustain on real data, which is
- * well below the rate on the regular operands of units 0..2.  One workgroup per compute unit (two for units 1,
- * 11, 13).  *work_per_launch receives the flops (0..2, 10..13) or LDS bytes (3..9) of one launch; `sink`: 8
- * writable bytes. */
+ * well below the rate on the regular operands of units 0..2; 14 / 15 / 16: units 4 / 3 / 5 with 16 waves per
+ * compute unit (8 waves do not keep enough reads in flight to saturate the LDS).  One workgroup per compute unit
+ * (two for units 1, 11, 13).  *work_per_launch receives the flops (0..2, 10..13) or LDS bytes (3..9, 14..16) of
+ * one launch; `sink`: 8 writable bytes. */
 int tuna_time_unit_rate(int unit, void *sink, int warmup, int iters, void *stream, float *elapsed_ms,
                         double *work_per_launch);
 

@@ -222,17 +222,18 @@ __global__ __launch_bounds__(256) void mfma_rate_kernel(uint32_t *sink)
     if (s == 12345.678f) sink[0] = 1u;  // practically never: keeps the chain alive
 }
 
-// LDS traffic of 8 waves per CU, eight accesses per wave and iteration, addresses opaque to the compiler.
+// LDS traffic of 8 (THREADS = 1024: 16) waves per CU, eight accesses per wave and iteration, addresses opaque to
+// the compiler.
 // MODE 0: 16-byte reads the way a wave reads an MFMA fragment from a tile of 128-byte rows (lane = row 0..15 x
 // k-group, slot ^ (row & 7)); 1: 4-byte reads the way the decode reads the byte-pair table ((byte << 8) | (lane
 // << 2), byte from a counter); 2: 16-byte writes the way the decoded weights are stored (4 rows x 8 k-blocks
 // per 32 lanes); 3: the same bytes as two 8-byte writes each; 4: 16-byte writes at consecutive addresses; 5 / 6:
 // the table reads of 1 with one copy of the table per 32 / 16 lanes and a pseudo-random byte per lane.
-template <int MODE>
-__global__ __launch_bounds__(512) void lds_rate_kernel(uint32_t *sink)
+template <int MODE, int THREADS = 512>
+__global__ __launch_bounds__(THREADS) void lds_rate_kernel(uint32_t *sink)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    for (int i = threadIdx.x; i < 65536 / 4; i += 512) reinterpret_cast<uint32_t *>(smem)[i] = (uint32_t)i;
+    for (int i = threadIdx.x; i < 65536 / 4; i += THREADS) reinterpret_cast<uint32_t *>(smem)[i] = (uint32_t)i;
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint32_t s = 0;
@@ -315,10 +316,11 @@ __global__ __launch_bounds__(512) void lds_rate_kernel(uint32_t *sink)
 // (one wave per SIMD, 4 accumulators); 3 LDS fragment reads, 4 LDS table reads, 5 LDS tile writes, 6 the tile
 // writes as 8-byte halves, 7 16-byte writes at consecutive addresses, 8 / 9 table reads with a copy of the table
 // per 32 / 16 lanes; 10 / 13 32x32x16 and 12 / 11 16x16x32 MFMAs on pseudo-random operands from one / two waves per
-// SIMD.  *work = flops (0..2, 10..13) or bytes (3..9) of one launch on `cus` compute units.
+// SIMD; 14 / 15 / 16: units 4 / 3 / 5 from 16 waves per compute unit.  *work = flops (0..2, 10..13) or bytes
+// (3..9, 14..16) of one launch on `cus` compute units.
 hipError_t launch_unit_rate(int unit, int cus, uint32_t *sink, double *work, hipStream_t stream)
 {
-    static OptInFlag attr[16][7];
+    static OptInFlag attr[16][10];
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
@@ -346,6 +348,15 @@ hipError_t launch_unit_rate(int unit, int cus, uint32_t *sink, double *work, hip
     case 11: hipLaunchKernelGGL((mfma_rate_kernel<false, 16, true>), dim3(2 * cus), dim3(256), 0, stream, sink); *work = (double)cus * 8 * kRateIters * 16 * 16384.0; break;
     case 12: hipLaunchKernelGGL((mfma_rate_kernel<false, 16, true>), dim3(cus), dim3(256), 0, stream, sink); *work = (double)cus * 4 * kRateIters * 16 * 16384.0; break;
     case 13: hipLaunchKernelGGL((mfma_rate_kernel<true, 16, true>), dim3(2 * cus), dim3(256), 0, stream, sink); *work = (double)cus * 8 * kRateIters * 16 * 32768.0; break;
+    case 14:
+        if ((e = ensure_lds_opt_in(attr[dev][7], reinterpret_cast<const void *>(lds_rate_kernel<1, 1024>))) != hipSuccess) return e;
+        hipLaunchKernelGGL((lds_rate_kernel<1, 1024>), dim3(cus), dim3(1024), 65536, stream, sink); *work = (double)cus * 1024 * kRateIters * 8 * 4.0; break;
+    case 15:
+        if ((e = ensure_lds_opt_in(attr[dev][8], reinterpret_cast<const void *>(lds_rate_kernel<0, 1024>))) != hipSuccess) return e;
+        hipLaunchKernelGGL((lds_rate_kernel<0, 1024>), dim3(cus), dim3(1024), 65536, stream, sink); *work = (double)cus * 1024 * kRateIters * 8 * 16.0; break;
+    case 16:
+        if ((e = ensure_lds_opt_in(attr[dev][9], reinterpret_cast<const void *>(lds_rate_kernel<2, 1024>))) != hipSuccess) return e;
+        hipLaunchKernelGGL((lds_rate_kernel<2, 1024>), dim3(cus), dim3(1024), 65536, stream, sink); *work = (double)cus * 1024 * kRateIters * 8 * 16.0; break;
     case 8:
         if ((e = ensure_lds_opt_in(attr[dev][5], reinterpret_cast<const void *>(lds_rate_kernel<5>))) != hipSuccess) return e;
         hipLaunchKernelGGL(lds_rate_kernel<5>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 4.0; break;
