@@ -435,6 +435,19 @@ def test_gpu_parity_config_families_are_valid_configs():
         make_configs.validate(m, make_configs.bucket_of(n), k, c.to_dict())
         assert ops.config_segments(m, n, k, c, 0, m // rows - 1) == [(m // rows - 1, 0, k // 32, -1)]
         assert ops.config_contributors(m, n, k, c, 0, 0) == (-1, 1, 0)
+    # the 256 x 256 tile (a kernel of its own): both MFMA shapes, split-K, k in multiples of 64 only; 160 KB of LDS
+    # (32 KB table + two buffers of 512 rows) in the C planner and in the generator's twin
+    for mfma_rows in (64, 32):
+        for (m, n, k, split) in ((512, 256, 512, 1), (520, 300, 1088, 1), (256, 70, 2048, 4), (1024, 129, 192, 3)):
+            c = mod.cfg(lds_tile_rows=256, token_tiles=16, split_k=split, rows_per_wave=mfma_rows)
+            ops.validate_config(m, n, k, c)
+            lds, _ = ops.config_footprint(m, n, k, c)
+            assert lds == make_configs.lds_bytes(c.to_dict()) == 160 * 1024
+            make_configs.validate(m, make_configs.bucket_of(n), k, c.to_dict())
+    with pytest.raises(ops.TunaError):
+        ops.validate_config(512, 256, 520, mod.cfg(lds_tile_rows=256, token_tiles=16))      # k not a multiple of 64
+    with pytest.raises(ValueError):
+        make_configs.validate(512, 256, 520, mod.cfg(lds_tile_rows=256, token_tiles=16).to_dict())
     with pytest.raises(ops.TunaError):
         ops.validate_config(512, 256, 512, mod.cfg(lds_tile_rows=96, token_tiles=16))       # no such tile
     with pytest.raises(ops.TunaError):
