@@ -424,6 +424,45 @@ def test_reference_table_2560_wide_shapes_every_bucket(m, k, n):
     assert e <= REL_TOL
 
 
+@pytest.mark.parametrize("m,k,n,kernel", [(5120, 5120, 16, "gemm_narrow_kernel"), (2048, 2048, 3, "gemm_narrow_kernel"),
+                                           (11008, 4096, 9, "gemm_narrow_kernel"), (3072, 8192, 16, "gemm_lean_kernel"),
+                                           (20480, 5120, 1, "gemm_lean_kernel"), (22016, 4096, 16, "weights through LDS"),
+                                           (37888, 3584, 12, "weights through LDS"), (4096, 11008, 16, "gemm_kernel")])
+def test_derived_configs_for_untuned_shapes_up_to_16_tokens(m, k, n, kernel):
+    """Shapes outside the table at up to 16 tokens: one round of narrow-row workgroups where a tile height gives one,
+    the streaming kernel with the weights through LDS for many rows, the lean split-K kernel where k divides in
+    powers of two, the general kernel otherwise - each through the plain entry point, on a random subset of rows."""
+    import torch
+
+    from tuna_amd import ops
+    from tuna_amd.quantize import nf4_codebook
+    from tuna_amd.synth import make_weights_torch, make_x_torch
+
+    cfg, hit = ops.select_config(m, n, k)
+    assert not hit
+    desc = ops.describe_launch(m, n, k, None)
+    print(f"derived config m={m} n={n} k={k}: {desc}", flush=True)
+    assert kernel in desc
+    dev = torch.device("cuda")
+    q, absmax = make_weights_torch(m, k, seed=m + n, device=dev)
+    x = make_x_torch(n, k, seed=k + n, device=dev)
+    code = nf4_codebook(dev)
+    out = torch.full((n, m), float("nan"), dtype=torch.float16, device=dev)
+    ops.matmul(x, q, absmax, code, out, m, n, k)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    rng = np.random.default_rng(m + k + n)
+    mbs = np.sort(rng.choice(m // 8, size=32, replace=False))
+    rows = (mbs[:, None] * 8 + np.arange(8)[None, :]).ravel()
+    q_sub = q[torch.from_numpy(mbs).to(dev)].cpu().numpy()
+    ref = O.gemm_f64(q_sub, x.cpu().numpy().view(np.uint16), code.cpu().numpy(), absmax.cpu().numpy()[rows],
+                     len(rows), n, k, mode=O.D1)
+    got = out.cpu().numpy().view(np.uint16)[:, rows]
+    e = rel_err(f16_bits_to_f64(got), ref)
+    print(f"  rel_err={e:.3e}", flush=True)
+    assert e <= REL_TOL                                      # max relative error 1e-2
+
+
 @pytest.mark.parametrize("m,k,n,split", [(12288, 1024, 1000, 1), (5120, 4096, 1300, 2), (5120, 1024, 1300, None)])
 def test_derived_config_for_an_untuned_shape_with_very_many_tokens(m, k, n, split):
     """A shape outside the table with 768 tokens or more gets the 256 x 256 many-token tile when its tiles fill the

@@ -349,13 +349,21 @@ static tuna_gemm_config derive_streaming(int m, int n, int k, int decode)
     GemmPlan plan;
     if (plan_gemm(m, n, k, c, decode, &plan) != TUNA_OK) return c;
     const int slots = kMaxCus * plan.wgs_per_cu;
-    if (row_tiles >= slots) return c;
+    // (an unsplit launch takes the streaming twin only with chunks that divide k: 3584 = 7 x 512, not 3.5 x 1024)
+    auto dividing_chunk = [&]() {
+        while (c.x_chunk > group * kStepK && k % c.x_chunk != 0) c.x_chunk /= 2;
+    };
+    if (row_tiles >= slots) {
+        dividing_chunk();
+        return c;
+    }
     int split = slots / row_tiles;
     if (split > max_split) split = max_split;
     if (split < 1) split = 1;
     if ((double)row_tiles * split >= 0.5 * slots) {
         c.split_k = split;
         set_chunk(ceil_div(steps, split));
+        if (split == 1) dividing_chunk();
     } else if (steps >= 2 * group) {
         c.split_k = 0;
     }
@@ -371,6 +379,74 @@ static bool config_runs(int m, int n, int k, const tuna_gemm_config &c);
 static tuna_gemm_config derive_config(int m, int n, int k)
 {
     tuna_gemm_config c;
+    if (n <= 16) {
+        // One round of workgroups of the narrow-row kernel (a workgroup owns 64, 32, 24 or 16 rows over the whole
+        // k range, all waves along k: no partial sums leave the workgroup) when some tile height gives 150..300
+        // of them - what the tuner finds on such shapes (3584 x 3584, 4608 x 3584, 5120 x 5120, 8192 x 4096,
+        // 11008 x 4096, 15360 x 5120, 16384 x 4096, 16384 x 8192: 6.5..18.2 us, 20-35 % under the streaming
+        // derivation below).  A workgroup reads all of x, 64 / rows times its weight bytes, so tiles of fewer than
+        // 64 rows are taken up to k = 8192 and of fewer than 32 up to k = 4096 only (5120 x 13824 in 32-row tiles:
+        // 20.9 us against 18.4).
+        static const int kRows[4] = {64, 32, 24, 16};
+        static const int kRing[5][2] = {{8, 4}, {4, 8}, {8, 2}, {4, 4}, {4, 2}};  // waves along k, ring depth
+        // (second pass, shapes of up to 8 MB that no tile height brings into that range: 96..600 workgroups - 2048 x 2048
+        // as 128 workgroups of 16 rows 3.9 us against 9.0, 8960 x 1536 as 280 of 32 rows 6.0 against 7.9)
+        for (int pass = 0; pass < 2; ++pass) {
+            const int lo = pass ? 96 : 150, hi = pass ? 600 : 300;
+            if (pass && (long long)m * k > (8ll << 21)) break;  // 8 MB of packed weights
+            for (int ri = 0; ri < 4; ++ri) {
+                const int r = kRows[ri];
+                if (m % r != 0 || m / r < lo || m / r > hi || (r < 32 && k > 4096) || (r < 64 && k > 8192)) continue;
+                if (!pass && r == 64 && m / r > 260) continue;  // (two 64-row tiles on some CUs: the streaming twin below)
+                for (int gi = 0; gi < 5; ++gi) {
+                    if (k % (32 * kRing[gi][0] * kRing[gi][1]) != 0) continue;
+                    memset(&c, 0, sizeof(c));
+                    c.rows_per_wave = r, c.waves_m = r == 64 ? 0 : 1, c.waves_k = kRing[gi][0], c.prefetch = kRing[gi][1];
+                    c.split_k = 1, c.token_tiles = 1, c.x_chunk = 32 * c.waves_k * c.prefetch;
+                    if (config_runs(m, n, k, c)) return c;
+                }
+            }
+        }
+        // Many rows (from 330 groups of 64): the streaming kernel, unsplit, with the packed weights staged through LDS,
+        // 16 waves as 2 x 8 (4 x 4 from 576 groups), chunks of 512 k, a staggered walk - what the tuner finds from
+        // 22016 x 4096 to 49152 x 6144 (14.3, 15.9, 19.3, 30.5 us against 18.1, 19.4, 22.0, 34.1 of the configs below).
+        const int groups = m / 64;
+        if (m % 256 == 0 && groups >= 330 && k % 512 == 0) {
+            memset(&c, 0, sizeof(c));
+            c.rows_per_wave = 64, c.split_k = 1, c.token_tiles = 1, c.x_chunk = 512, c.xcd_swizzle = 1, c.k_stagger = 2;
+            c.lds_tile_rows = -1;
+            if (groups >= 576) c.waves_m = 4, c.waves_k = 4, c.prefetch = k >= 3072 ? 4 : 2;
+            else c.waves_m = 2, c.waves_k = 8, c.prefetch = 2;
+            if (config_runs(m, n, k, c)) return c;
+        }
+        // Otherwise one round of 140..260 workgroups of the lean split-K kernel (one workgroup per row tile and
+        // power-of-two k slice, no staggered walk) where k divides that way: the few-row shapes the streaming
+        // derivation below gives the general kernel with an odd split (4096 x 8192 and 3072 x 8192: 12.2 -> 8.4 us),
+        // and mid-size shapes of many rows (20480 x 5120: 19.1 -> 17.5 us).  The most workgroups win, then the
+        // narrower row tile.
+        static const int kLeanShape[9][3] = {{1, 16, 2}, {1, 8, 4}, {1, 8, 2}, {2, 8, 2}, {2, 4, 4}, {2, 4, 2}, {4, 4, 4}, {4, 4, 2}, {4, 2, 4}};
+        tuna_gemm_config best;
+        long long best_wgs = 0;
+        for (int li = 0; li < 9; ++li) {
+            const int wm = kLeanShape[li][0], wk = kLeanShape[li][1], pf = kLeanShape[li][2];
+            if (m % (64 * wm) != 0 || k % 32 != 0) continue;
+            const int steps = k / 32;
+            for (int split = 1; split <= 16; split *= 2) {
+                const long long wgs = (long long)(m / (64 * wm)) * split;
+                if (wgs < 140 || wgs > 260 || wgs <= best_wgs) continue;
+                if (steps % split != 0 || (steps / split) % (wk * pf) != 0) continue;
+                memset(&c, 0, sizeof(c));
+                c.rows_per_wave = 64, c.waves_m = wm, c.waves_k = wk, c.prefetch = pf, c.split_k = split;
+                c.token_tiles = 1, c.xcd_swizzle = 1;
+                c.x_chunk = 32 * wk * pf;
+                while (c.x_chunk * 2 <= 1024 && (k / split) % (c.x_chunk * 2) == 0) c.x_chunk *= 2;
+                GemmPlan plan;
+                if (plan_gemm(m, n, k, c, TUNA_DECODE_GEMM, &plan) != TUNA_OK || !launch_is_lean(plan, kMaxCus)) continue;
+                best = c, best_wgs = wgs;
+            }
+        }
+        if (best_wgs) return best;
+    }
     if (n >= 256 && m >= 24576 && m % 512 == 0 && k % 128 == 0) {
         // many rows, several passes of 128 tokens: the streaming kernel with eight token tiles
         // (64 rows per wave, no split), whose token chunks run side by side and share the

@@ -135,6 +135,10 @@ static const LeanVariant *lean_applies(const GemmPlan &plan, int cus)
     return nullptr;
 }
 
+// Whether a planned launch would take the lean kernel on a device of `cus` compute units (the host's derivation of
+// configs asks: only configs that do are worth proposing for the shapes it proposes them for).
+bool launch_is_lean(const GemmPlan &plan, int cus) { return lean_applies(plan, cus) != nullptr; }
+
 // Dynamic LDS above 64 KB needs a one-time opt-in per kernel and device.
 static OptInFlag g_attr_done[16][kNumVariants];
 static OptInFlag g_lean_attr_done[16][kNumLean];

@@ -191,6 +191,7 @@ bool blockwise_describe(int m, int n, int k, char *buf, size_t len);
 int set_lean_kernels(int enabled);  // returns the previous setting
 int set_weight_path(int path);      // gemm_mid.hip; negative: query
 unsigned long long lean_launches();
+bool launch_is_lean(const GemmPlan &plan, int cus);  // the planned launch would take the lean kernel
 bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves, int grouped);
 
 // gemm_multi.hip: several 1..16-token GEMMs in one launch of persistent workgroups (gemm_multi.hpp)
