@@ -429,6 +429,21 @@ def test_reference_table_2560_wide_shapes_every_bucket(m, k, n):
                                            (20480, 5120, 1, "gemm_lean_kernel"), (22016, 4096, 16, "weights through LDS"),
                                            (37888, 3584, 12, "weights through LDS"), (4096, 11008, 16, "gemm_kernel")])
 def test_derived_configs_for_untuned_shapes_up_to_16_tokens(m, k, n, kernel):
+    _check_derived(m, k, n, kernel)
+
+
+@pytest.mark.parametrize("m,k,n,kernel", [(8192, 3072, 64, "gemm_narrow_kernel"), (5120, 5120, 20, "gemm_narrow_kernel"),
+                                           (4096, 12288, 32, "gemm_lean_kernel"), (12288, 4096, 64, "weights through LDS"),
+                                           (37888, 3584, 40, "weights through LDS"), (3072, 8192, 128, "weights through LDS"),
+                                           (5120, 5120, 200, "gemm_mid_kernel"), (12288, 4096, 300, "128 rows x 256 tokens"),
+                                           (3072, 8192, 512, "128 rows x 128 tokens")])
+def test_derived_configs_for_untuned_shapes_from_17_to_512_tokens(m, k, n, kernel):
+    """The same for 17..512 tokens: narrow-row and lean workgroups with the token passes side by side in the grid,
+    the streaming kernel with 16, 32 or 64 tokens per pass, the many-token tiles."""
+    _check_derived(m, k, n, kernel)
+
+
+def _check_derived(m, k, n, kernel):
     """Shapes outside the table at up to 16 tokens: one round of narrow-row workgroups where a tile height gives one,
     the streaming kernel with the weights through LDS for many rows, the lean split-K kernel where k divides in
     powers of two, the general kernel otherwise - each through the plain entry point, on a random subset of rows."""
@@ -515,7 +530,7 @@ def test_derived_config_for_a_large_untuned_shape_with_many_tokens(m, k, n, tile
     from tuna_amd.synth import make_weights_torch, make_x_torch
 
     cfg, hit = ops.select_config(m, n, k)
-    assert not hit and cfg.token_tiles == tiles and cfg.lds_tile_rows == 0
+    assert not hit and cfg.token_tiles == tiles and cfg.lds_tile_rows in (0, -1)   # (-1: the packed weights through LDS)
     print(f"derived config m={m} n={n} k={k} {cfg.to_dict()}", flush=True)
     dev = torch.device("cuda")
     q, absmax = make_weights_torch(m, k, seed=5, device=dev)

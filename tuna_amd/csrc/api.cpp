@@ -379,61 +379,74 @@ static bool config_runs(int m, int n, int k, const tuna_gemm_config &c);
 static tuna_gemm_config derive_config(int m, int n, int k)
 {
     tuna_gemm_config c;
-    if (n <= 16) {
+    if (n <= 64) {
         // One round of workgroups of the narrow-row kernel (a workgroup owns 64, 32, 24 or 16 rows over the whole
         // k range, all waves along k: no partial sums leave the workgroup) when some tile height gives 150..300
         // of them - what the tuner finds on such shapes (3584 x 3584, 4608 x 3584, 5120 x 5120, 8192 x 4096,
-        // 11008 x 4096, 15360 x 5120, 16384 x 4096, 16384 x 8192: 6.5..18.2 us, 20-35 % under the streaming
-        // derivation below).  A workgroup reads all of x, 64 / rows times its weight bytes, so tiles of fewer than
-        // 64 rows are taken up to k = 8192 and of fewer than 32 up to k = 4096 only (5120 x 13824 in 32-row tiles:
-        // 20.9 us against 18.4).
+        // 11008 x 4096, 15360 x 5120, 16384 x 4096, 16384 x 8192 at 16 tokens: 6.5..18.2 us, 20-35 % under the
+        // streaming derivation below).  A workgroup reads all of x, 64 / rows times its weight bytes, so tiles of
+        // fewer than 64 rows are taken up to k = 8192 and of fewer than 32 up to k = 4096 only (5120 x 13824 in
+        // 32-row tiles: 20.9 us against 18.4).  17..64 tokens: the same with one or two token tiles per pass, the
+        // passes side by side in the grid, so that rows x passes make the round (8192 x 3072 at 64 tokens as
+        // 128 x 2 workgroups 11.4 us against 27.6; 64- and 32-row tiles only).
+        // (Second pass, shapes of up to 8 MB at up to 16 tokens that no tile height brings into that range: 96..600
+        // workgroups - 2048 x 2048 as 128 workgroups of 16 rows 3.9 us against 9.0, 8960 x 1536 as 280 of 32 rows
+        // 6.0 against 7.9.)
         static const int kRows[4] = {64, 32, 24, 16};
         static const int kRing[5][2] = {{8, 4}, {4, 8}, {8, 2}, {4, 4}, {4, 2}};  // waves along k, ring depth
-        // (second pass, shapes of up to 8 MB that no tile height brings into that range: 96..600 workgroups - 2048 x 2048
-        // as 128 workgroups of 16 rows 3.9 us against 9.0, 8960 x 1536 as 280 of 32 rows 6.0 against 7.9)
-        for (int pass = 0; pass < 2; ++pass) {
+        for (int pass = 0; pass < (n <= 16 ? 2 : 1); ++pass) {
             const int lo = pass ? 96 : 150, hi = pass ? 600 : 300;
             if (pass && (long long)m * k > (8ll << 21)) break;  // 8 MB of packed weights
-            for (int ri = 0; ri < 4; ++ri) {
+            for (int ri = 0; ri < (n <= 16 ? 4 : 2); ++ri) {
                 const int r = kRows[ri];
-                if (m % r != 0 || m / r < lo || m / r > hi || (r < 32 && k > 4096) || (r < 64 && k > 8192)) continue;
-                if (!pass && r == 64 && m / r > 260) continue;  // (two 64-row tiles on some CUs: the streaming twin below)
-                for (int gi = 0; gi < 5; ++gi) {
-                    if (k % (32 * kRing[gi][0] * kRing[gi][1]) != 0) continue;
-                    memset(&c, 0, sizeof(c));
-                    c.rows_per_wave = r, c.waves_m = r == 64 ? 0 : 1, c.waves_k = kRing[gi][0], c.prefetch = kRing[gi][1];
-                    c.split_k = 1, c.token_tiles = 1, c.x_chunk = 32 * c.waves_k * c.prefetch;
-                    if (config_runs(m, n, k, c)) return c;
+                if (m % r != 0 || (r < 32 && k > 4096) || (r < 64 && k > 8192)) continue;
+                for (int tt = n <= 16 ? 1 : 2; tt >= 1; --tt) {
+                    const long long wgs = (long long)(m / r) * ceil_div(n, 16 * tt);
+                    if (wgs < lo || wgs > hi) continue;
+                    if (!pass && n <= 16 && r == 64 && wgs > 260) continue;  // (two 64-row tiles on some CUs: the streaming twin below)
+                    for (int gi = 0; gi < 5; ++gi) {
+                        if (k % (32 * kRing[gi][0] * kRing[gi][1]) != 0 || (tt > 1 && kRing[gi][1] > 4)) continue;
+                        memset(&c, 0, sizeof(c));
+                        c.rows_per_wave = r, c.waves_m = r == 64 ? 0 : 1, c.waves_k = kRing[gi][0], c.prefetch = kRing[gi][1];
+                        c.split_k = 1, c.token_tiles = tt, c.x_chunk = 32 * c.waves_k * c.prefetch;
+                        if (config_runs(m, n, k, c)) return c;
+                    }
                 }
             }
         }
-        // Many rows (from 330 groups of 64): the streaming kernel, unsplit, with the packed weights staged through LDS,
-        // 16 waves as 2 x 8 (4 x 4 from 576 groups), chunks of 512 k, a staggered walk - what the tuner finds from
-        // 22016 x 4096 to 49152 x 6144 (14.3, 15.9, 19.3, 30.5 us against 18.1, 19.4, 22.0, 34.1 of the configs below).
+        // Many rows (from 330 groups of 64; from 170 at 17..64 tokens): the streaming kernel, unsplit, with the packed
+        // weights staged through LDS, 16 waves as 2 x 8 (4 x 4 from 576 groups), chunks of 512 k, a staggered walk -
+        // what the tuner finds from 22016 x 4096 to 49152 x 6144 (16 tokens: 14.3, 15.9, 19.3, 30.5 us against 18.1,
+        // 19.4, 22.0, 34.1 of the configs below); 17..64 tokens in passes of 32 side by side (12288 x 4096 at 64
+        // tokens 19.3 us against 32.0, 16384 x 8192 31.7 against 57.0), 33..64 tokens on 576 groups or more in one
+        // pass of 64 with 4 x 2 waves (37888 x 3584: 41.2 against 57.2).
         const int groups = m / 64;
-        if (m % 256 == 0 && groups >= 330 && k % 512 == 0) {
+        if (m % 256 == 0 && groups >= (n <= 16 ? 330 : 170) && k % 512 == 0) {
             memset(&c, 0, sizeof(c));
-            c.rows_per_wave = 64, c.split_k = 1, c.token_tiles = 1, c.x_chunk = 512, c.xcd_swizzle = 1, c.k_stagger = 2;
+            c.rows_per_wave = 64, c.split_k = 1, c.token_tiles = n <= 16 ? 1 : 2, c.x_chunk = 512, c.xcd_swizzle = 1, c.k_stagger = 2;
             c.lds_tile_rows = -1;
-            if (groups >= 576) c.waves_m = 4, c.waves_k = 4, c.prefetch = k >= 3072 ? 4 : 2;
+            if (groups >= 576 && n > 32) c.waves_m = 4, c.waves_k = 2, c.prefetch = 2, c.token_tiles = 4, c.x_chunk = 256;
+            else if (groups >= 576) c.waves_m = 4, c.waves_k = 4, c.prefetch = (n <= 16 && k >= 3072) ? 4 : 2, c.x_chunk = n <= 16 ? 512 : 256;
             else c.waves_m = 2, c.waves_k = 8, c.prefetch = 2;
             if (config_runs(m, n, k, c)) return c;
         }
-        // Otherwise one round of 140..260 workgroups of the lean split-K kernel (one workgroup per row tile and
-        // power-of-two k slice, no staggered walk) where k divides that way: the few-row shapes the streaming
-        // derivation below gives the general kernel with an odd split (4096 x 8192 and 3072 x 8192: 12.2 -> 8.4 us),
+        // Otherwise one round of 140..260 workgroups (..300 with the 16-token passes of 17..64 tokens side by side)
+        // of the lean split-K kernel (one workgroup per row tile and power-of-two k slice, no staggered walk) where k
+        // divides that way: the few-row shapes the streaming derivation below gives the general kernel with an odd
+        // split (4096 x 8192 and 3072 x 8192 at 16 tokens: 12.2 -> 8.4 us; 4096 x 12288 at 32 tokens 21.0 -> 14.4),
         // and mid-size shapes of many rows (20480 x 5120: 19.1 -> 17.5 us).  The most workgroups win, then the
         // narrower row tile.
         static const int kLeanShape[9][3] = {{1, 16, 2}, {1, 8, 4}, {1, 8, 2}, {2, 8, 2}, {2, 4, 4}, {2, 4, 2}, {4, 4, 4}, {4, 4, 2}, {4, 2, 4}};
         tuna_gemm_config best;
         long long best_wgs = 0;
-        for (int li = 0; li < 9; ++li) {
+        const int passes16 = ceil_div(n, 16);
+        for (int li = 0; li < 9 && passes16 <= 2; ++li) {
             const int wm = kLeanShape[li][0], wk = kLeanShape[li][1], pf = kLeanShape[li][2];
             if (m % (64 * wm) != 0 || k % 32 != 0) continue;
             const int steps = k / 32;
             for (int split = 1; split <= 16; split *= 2) {
-                const long long wgs = (long long)(m / (64 * wm)) * split;
-                if (wgs < 140 || wgs > 260 || wgs <= best_wgs) continue;
+                const long long wgs = (long long)(m / (64 * wm)) * split * passes16;
+                if (wgs < 140 || wgs > (passes16 > 1 ? 300 : 260) || wgs <= best_wgs) continue;
                 if (steps % split != 0 || (steps / split) % (wk * pf) != 0) continue;
                 memset(&c, 0, sizeof(c));
                 c.rows_per_wave = 64, c.waves_m = wm, c.waves_k = wk, c.prefetch = pf, c.split_k = split;
@@ -446,6 +459,27 @@ static tuna_gemm_config derive_config(int m, int n, int k)
             }
         }
         if (best_wgs) return best;
+    }
+    if (n > 64 && n <= 256 && k % 512 == 0) {
+        // 65..256 tokens: the streaming kernel with the weights through LDS, 16 waves (8 with four token tiles), the
+        // passes of 16, 32 or 64 tokens side by side in the grid (they share the weights through the L2), the tile
+        // height and the tokens per pass chosen so that row tiles x passes make one round of 150..300 workgroups -
+        // what the tuner finds on 3072 x 8192, 4096 x 12288, 5120 x 5120, 12288 x 4096 and 16384 x 8192 (128 tokens:
+        // 22.8, 32.9, 21.1, 27.3, 53.2 us against 60.3, 49.8, 37.2, 33.2, 57.3 of the rules below, which split k for
+        // the many-token kernel there).
+        static const int kTokWm[6][2] = {{4, 2}, {4, 4}, {2, 2}, {2, 4}, {1, 2}, {1, 4}};  // token tiles per pass, waves along the rows
+        for (int ci = 0; ci < 6; ++ci) {
+            const int tt = kTokWm[ci][0], wm = kTokWm[ci][1];
+            if (m % (64 * wm) != 0) continue;
+            const long long wgs = (long long)(m / (64 * wm)) * ceil_div(n, 16 * tt);
+            if (wgs < 150 || wgs > 300) continue;
+            for (int lds = -1; lds <= 0; ++lds) {
+                memset(&c, 0, sizeof(c));
+                c.rows_per_wave = 64, c.waves_m = wm, c.waves_k = (tt == 4 ? 8 : 16) / wm, c.prefetch = 2, c.split_k = 1;
+                c.token_tiles = tt, c.x_chunk = tt == 4 ? 256 : 512, c.xcd_swizzle = 1, c.lds_tile_rows = lds;
+                if (config_runs(m, n, k, c)) return c;
+            }
+        }
     }
     if (n >= 256 && m >= 24576 && m % 512 == 0 && k % 128 == 0) {
         // many rows, several passes of 128 tokens: the streaming kernel with eight token tiles
@@ -513,9 +547,11 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         c.rows_per_wave = 64, c.waves_m = 1, c.waves_k = 1, c.prefetch = 2, c.x_chunk = 64;
         c.token_tiles = 8;
         c.lds_tile_rows = m >= 16384 ? 256 : 128;
-        const long long tiles = (long long)ceil_div(m, c.lds_tile_rows) * ceil_div(n, 128);
+        // (from 257 tokens 128 x 256 tiles when they fill the device: 12288 x 4096 at 512 tokens 62.7 us against 82.9)
+        if (n > 256 && (long long)ceil_div(m, 128) * ceil_div(n, 256) >= 150) c.lds_tile_rows = 128, c.token_tiles = 16;
+        const long long tiles = (long long)ceil_div(m, c.lds_tile_rows) * ceil_div(n, 16 * c.token_tiles);
         const int steps64 = ceil_div(k, 64);
-        long long split = tiles >= 192 ? 1 : (kMaxCus + tiles / 2) / tiles;
+        long long split = tiles >= 150 ? 1 : kMaxCus / tiles;
         if (split > steps64 / 8) split = steps64 / 8;
         if (split < 1) split = 1;
         c.split_k = (int)split;
