@@ -69,6 +69,10 @@ int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int va
 int tuna_time_unit_rate(int unit, void *sink, int warmup, int iters, void *stream, float *elapsed_ms,
                         double *work_per_launch);
 
+/* The config the library derives for a shape when its table has no entry for it - also for shapes that have
+ * one: what the tuner seeds its search with, and what a table entry has to beat.  Host only. */
+int tuna_derive_config(int m, int n, int k, tuna_gemm_config *cfg);
+
 /* Name and template arguments of the kernel a GEMM launch would start (cfg NULL = the library's
  * choice), e.g. "gemm_narrow_kernel<LW=2,WK=8,U=4,PERM=1,TT=1>": what the bench writes beside a
  * timing so that it can be matched with a profile.  Host only; with a device present the

@@ -83,6 +83,7 @@ SIGNATURES = {
     "tuna_dequant_ex": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "tuna_select_config": (_i, [_i, _i, _i, _cfgp, _ip]),
     "tuna_select_config_ex": (_i, [_i, _i, _i, _i, _cfgp, _ip]),
+    "tuna_derive_config": (_i, [_i, _i, _i, _cfgp]),
     "tuna_select_config_grouped": (_i, [_i, _i, _i, _i, _i, _cfgp]),
     "tuna_validate_config": (_i, [_i, _i, _i, _cfgp]),
     "tuna_validate_config_ex": (_i, [_i, _i, _i, _cfgp, _i]),

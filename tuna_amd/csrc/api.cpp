@@ -1535,6 +1535,15 @@ TUNA_EXPORT int tuna_select_config(int m, int n, int k, tuna_gemm_config *cfg, i
     return select_config(m, n, k, cfg, from_table);
 }
 
+TUNA_EXPORT int tuna_derive_config(int m, int n, int k, tuna_gemm_config *cfg)
+{
+    if (!cfg) return fail(TUNA_ERR_INVALID_ARG, "cfg is null");
+    int rc = check_shape(m, n, k);
+    if (rc) return rc;
+    *cfg = derive_config(m, n, k);
+    return TUNA_OK;
+}
+
 TUNA_EXPORT int tuna_select_config_ex(int m, int n, int k, int decode_mode, tuna_gemm_config *cfg, int *from_table)
 {
     if (!cfg) return fail(TUNA_ERR_INVALID_ARG, "cfg is null");

@@ -258,6 +258,14 @@ def select_config(m: int, n: int, k: int, decode_mode: int = _lib.DECODE_GEMM):
     return cfg, bool(hit.value)
 
 
+def derive_config(m: int, n: int, k: int):
+    """GemmConfig the library derives for shape (m, n, k) when the table has no entry (also for shapes that have
+    one: the tuner's seed, and what an entry has to beat).  Host only."""
+    cfg = GemmConfig()
+    _lib.check(_lib.lib().tuna_derive_config(int(m), int(n), int(k), ctypes.byref(cfg)))
+    return cfg
+
+
 def select_config_grouped(m_group: int, n_active: int, max_tokens: int, k: int, decode_mode: int = _lib.DECODE_GEMM):
     """GemmConfig matmul_grouped(config=None) runs for n_active groups with tokens.  Host only."""
     cfg = GemmConfig()

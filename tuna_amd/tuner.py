@@ -290,15 +290,17 @@ def tune_shape(m, n, k, generations=6, population=24, seed=0, log=print, max_see
     rng = random.Random(seed * 7919 + m * 31 + k)
     n_key = make_configs.bucket_of(n)
     ev = Evaluator(m, n, k, iters=iters, warmup=max(2, iters // 6))
+    # what the library would run without a table entry: a tuned entry is never worse than that
+    derived = [ev.ops.derive_config(m, n, k).to_dict()]
     if n_key >= 512:
         # far beyond the general kernel's range: the many-token kernel and the streaming kernel
         # with eight token tiles per pass are timed exhaustively, nothing is bred
-        scored = sorted((ev(c), json.dumps(c, sort_keys=True)) for c in tiled_space(m, n_key, k) + mid_space(m, n_key, k))
+        scored = sorted((ev(c), json.dumps(c, sort_keys=True)) for c in tiled_space(m, n_key, k) + mid_space(m, n_key, k) + derived)
         log(f"  many-token + streaming kernel: {len(scored)} configs, best {scored[0][0]:.2f} us {scored[0][1]}")
         return json.loads(scored[0][1]), scored[0][0]
     pool = seeds(m, n_key, k)
     rng.shuffle(pool)
-    pool = pool[:max_seed_evals] + lean_space(m, n_key, k) + mid_space(m, n_key, k)
+    pool = pool[:max_seed_evals] + lean_space(m, n_key, k) + mid_space(m, n_key, k) + derived
     # the winners of the other token buckets of this (m, k), where they are valid here: a config tuned
     # for 16 tokens also runs one token, and is sometimes what the bucket should have
     pool += [c for c in (repair(dict(e), m, n_key, k) for e in extra) if c is not None]
