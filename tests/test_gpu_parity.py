@@ -478,10 +478,10 @@ def _check_derived(m, k, n, kernel):
     assert e <= REL_TOL                                      # max relative error 1e-2
 
 
-@pytest.mark.parametrize("m,k,n,split", [(12288, 1024, 1000, 1), (5120, 4096, 1300, 2), (5120, 1024, 1300, None)])
+@pytest.mark.parametrize("m,k,n,split", [(12288, 1024, 1000, 1), (5120, 8192, 1300, 2), (5120, 4096, 1300, None)])
 def test_derived_config_for_an_untuned_shape_with_very_many_tokens(m, k, n, split):
     """A shape outside the table with 768 tokens or more gets the 256 x 256 many-token tile when its tiles fill the
-    device (192 tiles; 120 tiles with the k range split in two; not with 120 tiles and a short k), through the plain
+    device (192 tiles; 120 tiles with the k range split in two; not with 120 tiles and k below 8192), through the plain
     entry point; checked on a random subset of rows."""
     import torch
 

@@ -527,12 +527,13 @@ static tuna_gemm_config derive_config(int m, int n, int k)
     }
     if (n >= 768 && k % 64 == 0) {
         // very many tokens: the 256 x 256 tile (one wave per SIMD) where it fills the device - from about 150
-        // tiles, or from 90 with the k range split in two when that leaves 32 steps per workgroup.  Measured on
+        // tiles, or from 90 with the k range split in two when k is 8192 or more (with k = 4096 the split loses:
+        // 6144 x 4096 at 800 tokens 103 us against 63 of the 128-token tiles).  Measured on
         // 12288 x 6144, 5120 x 5120, 16384 x 8192, 3072 x 9216 and 20480 x 5120 at 1024..8192 tokens: 5-38 %
         // faster than the 128-token tiles below from 150 tiles (12288 x 6144 at 4096 tokens 842 -> 526 us),
         // 10 % with the split at 96 tiles, slower at 80.
         const long long tiles = (long long)ceil_div(m, 256) * ceil_div(n, 256);
-        const int split = tiles >= 150 ? 1 : (tiles >= 90 && k >= 64 * 64) ? 2 : 0;
+        const int split = tiles >= 150 ? 1 : (tiles >= 90 && k >= 8192) ? 2 : 0;
         if (split) {
             memset(&c, 0, sizeof(c));
             c.rows_per_wave = 64, c.waves_m = 1, c.waves_k = 1, c.prefetch = 2, c.x_chunk = 64;
