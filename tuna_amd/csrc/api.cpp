@@ -583,7 +583,7 @@ static bool config_runs(int m, int n, int k, const tuna_gemm_config &c)
 // pass: measured on six of the benchmark shapes, 17..255 tokens, the next bucket's entry is 15-40 %
 // faster (8192 x 8192 at 20 tokens 23.8 -> 14.8 us, 57344 x 8192 at 24 tokens 81 -> 57 us,
 // 229376 x 4096 at 100 tokens 297 -> 237 us), so such a count takes it when it can run the shape.
-// Up to 15 tokens and from 256 tokens the containing bucket's entry stays (but see the last bucket below).
+// Up to 9 tokens and from 256 tokens the containing bucket's entry stays (but see the last bucket below).
 static int select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_table)
 {
     const TableEntry *own = nullptr;
@@ -591,7 +591,10 @@ static int select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_t
         const TableEntry &e = kConfigTable[i];
         if (e.m == m && e.k == k && n >= e.n_lo && n <= e.n_hi) own = &e;
     }
-    if (own && n > own->n_lo && own->n_lo >= 16 && own->n_lo <= 128) {
+    // The first bucket (1..15 tokens) is tuned at one token: from 10 tokens the 16-token entry is the better one too
+    // (ten benchmark shapes at 12 / 15 tokens: 3 % / 9 % less time in sum, 8192 x 28672 at 15 tokens 36.1 -> 28.9 us;
+    // at 8 tokens they are even, at 4 the one-token entry wins).
+    if (own && ((n > own->n_lo && own->n_lo >= 16 && own->n_lo <= 128) || (own->n_lo == 1 && n >= 10))) {
         for (int i = 0; i < kConfigTableSize; ++i) {
             const TableEntry &e = kConfigTable[i];
             if (e.m == m && e.k == k && e.n_lo == own->n_hi + 1) {
