@@ -318,10 +318,11 @@ def test_baseline_shapes_row_subset_and_readout(name):
     assert torch.equal(out.float(), img[:, cols].t().float())
 
 
-@pytest.mark.parametrize("n", [1, 64, 256, 1024])
+@pytest.mark.parametrize("n", [1, 13, 64, 256, 1024])
 @pytest.mark.parametrize("name", ["llama70b_qkv", "llama70b_attn_out", "llama70b_gate_up", "llama70b_down"])
 def test_token_sweep_llama70b_layer_set(name, n):
-    """The M sweep of benchmark configuration 3 ({1, 16, 64, 256}, plus the 1024 the bench also times)
+    """The M sweep of benchmark configuration 3 ({1, 16, 64, 256}, plus the 1024 the bench also times and 13,
+    which the dispatcher serves with the 16-token entry)
     on all four Llama-70B shapes with the tuned table's entries - narrow-row, lean, streaming and
     many-token kernels at their real sizes - checked on a row subset (16 tokens is covered above)."""
     import torch
