@@ -310,10 +310,13 @@ def time_quantize(ops, synth, torch, dev):
 def time_blockwise(ops, synth, torch, dev, names=("mistral_qkv", "mistral_gate_up", "llama70b_qkv", "llama70b_gate_up", "llama70b_down"),
                    block_size=64, tokens=16):
     """tuna_matmul_blockwise (one fp32 scale per `block_size` weights of a row, the layout of block-quantized NF4
-    checkpoints) on some of the 16-token shapes: back-to-back calls through the C ABI over rotating weights, HIP
-    events around them on torch's stream (which the calls launch on).  Algorithmic bytes: packed weights + scales."""
+    checkpoints) on some of the 16-token shapes: calls through the C ABI over rotating weights, recorded once into a
+    HIP graph and replayed (a call from Python costs about 10 us, more than the smaller launches take), HIP events
+    around the replays on torch's stream.  Algorithmic bytes: packed weights + scales."""
+    from tuna_amd import _lib
     from tuna_amd.quantize import nf4_codebook
 
+    L = _lib.lib()
     code = nf4_codebook(dev)
     out = {}
     for nm in names:
@@ -323,23 +326,38 @@ def time_blockwise(ops, synth, torch, dev, names=("mistral_qkv", "mistral_gate_u
         scales = [torch.rand((m, k // block_size), dtype=torch.float32, device=dev) * 0.015 + 0.005 for _ in range(nsets)]
         x = synth.make_x_torch(tokens, k, 3, dev)
         o = torch.empty((tokens, m), dtype=torch.float16, device=dev)
-        for i in range(50):
-            ops.matmul_blockwise(x, sets[i % nsets][0], scales[i % nsets], code, o, m, tokens, k, block_size)
+        before = [L.tuna_blockwise_launches(i) for i in range(3)]
+        calls = 4 * nsets
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            for i in range(nsets):  # (the library's workspace exists before the capture starts)
+                ops.matmul_blockwise(x, sets[i][0], scales[i], code, o, m, tokens, k, block_size)
+            side.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(calls):
+                    ops.matmul_blockwise(x, sets[i % nsets][0], scales[i % nsets], code, o, m, tokens, k, block_size)
         torch.cuda.synchronize()
-        iters = 300
+        took = [L.tuna_blockwise_launches(i) - before[i] for i in range(3)]
+        kernel = ("tuna::gemm_narrow_kernel", "tuna::gemm_multi_kernel", "tuna::gemm_tiled_kernel")[took.index(max(took))]
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        replays = max(3, 300 // calls)
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         ev0.record()
-        for i in range(iters):
-            ops.matmul_blockwise(x, sets[i % nsets][0], scales[i % nsets], code, o, m, tokens, k, block_size)
+        for _ in range(replays):
+            graph.replay()
         ev1.record()
         torch.cuda.synchronize()
-        us = ev0.elapsed_time(ev1) * 1000.0 / iters
+        us = ev0.elapsed_time(ev1) * 1000.0 / (replays * calls)
+        del graph
         nbytes = m * k // 2 + 4 * m * (k // block_size)
         gbs = nbytes / (us * 1e-6) / 1e9
         out[nm] = {"m": m, "k": k, "block_size": block_size, "us": round(us, 2),
                    "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                 "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                                "kernel": "tuna::gemm_multi_kernel (scale blocks)" if m * k // 2 >= 20 << 20 else "tuna::gemm_narrow_kernel (scale blocks)",
+                                "kernel": kernel + " (scale blocks)",
                                 "algorithmic_bytes_per_launch": nbytes, "avg_launch_us": round(us, 2)}}
         del sets, scales
         torch.cuda.empty_cache()

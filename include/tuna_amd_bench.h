@@ -97,15 +97,21 @@ int tuna_set_multi_shape(int waves_m, int prefetch);
  * Bit-identical results; for A/B timing.  Returns the previous setting. */
 int tuna_set_multi_weight_path(int through_lds);
 /* Diagnostic switch, process-wide, default 1: tuna_matmul_blockwise runs launches of more than 32 tokens through the
- * many-token kernel's scale-block variants, and launches of at least 20 MB of packed weights whose shape allows (m a
- * multiple of 64, k of 256 and of the block) through the scale-block variant of the batched streaming kernel (a batch of
- * one up to 16 tokens, the token chunks as a batch beyond); 2: the batched streaming kernel for every launch it can plan,
+ * many-token kernel's scale-block variants, and large launches whose shape allows (m a multiple of 64, k of 256 and of
+ * the block; 17 to 32 tokens from 20 MB of packed weights, 9 to 16 tokens from 100 MB or from 20 MB when k >= 12288,
+ * 5 to 8 tokens from 100 MB, 1 to 4 tokens from 256 MB) through the scale-block variant of the batched streaming kernel
+ * (a batch of one up to 16 tokens, the token chunks as a batch beyond); 2: the batched streaming kernel for every launch it can plan,
  * whatever its size and token count; 0: always the narrow-row kernel's variants.  All decode fp16(code) * fp16(absmax of
  * the block); the sums differ in summation order only.  Returns the previous setting. */
 int tuna_set_blockwise_stream(int enabled);
 /* Diagnostic: tuna_matmul_blockwise calls so far in this process that ran the narrow-row kernel (kernel 0), launches of
  * the batched streaming kernel (1) and calls that ran the many-token kernel (2) on their behalf. */
 unsigned long long tuna_blockwise_launches(int kernel);
+/* A/B switch of the narrow-row blockwise GEMM, process-wide: 1 (default) copies a workgroup's scales into LDS once and
+ * reads them from there (when they fit beside the decode table), 0 reads them from memory with every ring slot.
+ * Bit-identical results.  Returns the previous setting. */
+int tuna_set_blockwise_scales_lds(int enabled);
+
 /* Diagnostic override of the kernel variant tuna_matmul_blockwise runs: rows per workgroup (16, 32 or 64), waves along k
  * (4, 8 or 16) and ring depth (2 or 4); all zero = the library's choice.  TUNA_ERR_INVALID_ARG if no such variant is built;
  * a variant that does not fit a later call's shape makes that call fail with TUNA_ERR_UNSUPPORTED.  For A/B timing. */

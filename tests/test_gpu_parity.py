@@ -1635,6 +1635,62 @@ def test_blockwise_gemm_matches_oracle_and_reads_out_the_decode(m, n, k, bs):
     assert np.array_equal(out.cpu().numpy().view(np.uint16), img[:, cols].T)
 
 
+@pytest.mark.parametrize("m,n,k,bs,shape", [
+    (256, 16, 28672, 64, None),          # 16-row tiles, 7168 scales per workgroup: two rounds of the prologue copy
+    (1024, 16, 8192, 64, (64, 8, 4)),    # 64-row tiles, 8192 scales: two rounds
+    (1024, 5, 4096, 64, (64, 8, 2)),     # exactly one full round
+    (512, 37, 2048, 128, (32, 8, 4)),    # three token chunks, ragged last
+    (512, 1, 4096, 512, (32, 16, 2)),    # few long blocks
+    (256, 16, 1536, 64, (16, 4, 2)),     # k range of three ring turns
+    (128, 9, 28672, 64, (64, 8, 4)),     # 64 rows x 449 floats do not fit beside the table: scales stay in memory
+    (2560, 16, 10240, 64, None),         # 160 tiles of 16 rows
+])
+def test_blockwise_narrow_kernel_with_scales_in_lds_and_in_memory(m, n, k, bs, shape):
+    """The narrow-row kernel's scale-block variants stage the workgroup's scales in LDS when they fit and read them
+    from memory per ring slot when they do not (or when the switch says so): both orders of reading the same scales
+    give identical bits, match the oracle's float64 sums, and read the decoded weights out exactly."""
+    import torch
+
+    from tuna_amd import _lib, ops
+
+    rng = np.random.default_rng(m + n + k + bs + 2)
+    q, x, code, _ = make_inputs_np(m, n, k, seed=m + bs + 2)
+    absmax = rng.uniform(0.005, 0.02, size=(m, k // bs)).astype(np.float16).astype(np.float32)
+    dq, dx, dc, da = to_dev(q, x, code, absmax)
+    L = _lib.lib()
+    prev_stream = L.tuna_set_blockwise_stream(0)
+    prev_lds = L.tuna_set_blockwise_scales_lds(1)
+    if shape:
+        assert L.tuna_set_blockwise_shape(*shape) == 0
+    try:
+        print(f"blockwise narrow rows m={m} n={n} k={k} block={bs} variant={shape}", flush=True)
+        cols = rng.choice(k, size=n, replace=False)
+        xh = np.zeros((n, k), np.float16)
+        xh[np.arange(n), cols] = 1.0
+        dxh, = to_dev(xh)
+        img = O.dequant(q, absmax, code, m, k, mode=O.D1, block_size=bs)
+        got = {}
+        for lds in (1, 0):
+            L.tuna_set_blockwise_scales_lds(lds)
+            out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+            ops.matmul_blockwise(dx, dq, da, dc, out, m, n, k, bs)
+            torch.cuda.synchronize()
+            got[lds] = out.cpu().numpy().view(np.uint16)
+            ops.matmul_blockwise(dxh, dq, da, dc, out, m, n, k, bs)
+            torch.cuda.synchronize()
+            assert np.array_equal(out.cpu().numpy().view(np.uint16), img[:, cols].T), lds
+        assert not np.isnan(got[1].view(np.float16)).any()
+        assert np.array_equal(got[1], got[0])
+        rows = np.sort(rng.choice(m, size=min(m, 128), replace=False)).astype(np.int32)
+        ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1, rows=rows, block_size=bs)
+        e = rel_err(f16_bits_to_f64(got[1][:, rows]), ref)
+        assert e <= REL_TOL, e
+    finally:
+        L.tuna_set_blockwise_shape(0, 0, 0)
+        L.tuna_set_blockwise_scales_lds(prev_lds)
+        L.tuna_set_blockwise_stream(prev_stream)
+
+
 @pytest.mark.parametrize("m,n,k,bs", [(256, 16, 1280, 64), (128, 7, 1536, 64), (512, 16, 4096, 128), (1024, 1, 2048, 256),
                                       (256, 16, 2048, 512), (768, 13, 5120, 64), (4096, 16, 4096, 64), (8192, 16, 8192, 64),
                                       (512, 37, 2048, 256), (256, 100, 1024, 64), (256, 530, 512, 64)])

@@ -84,6 +84,7 @@ SIGNATURES = {
     "tuna_select_config": (_i, [_i, _i, _i, _cfgp, _ip]),
     "tuna_select_config_ex": (_i, [_i, _i, _i, _i, _cfgp, _ip]),
     "tuna_derive_config": (_i, [_i, _i, _i, _cfgp]),
+    "tuna_set_blockwise_scales_lds": (_i, [_i]),
     "tuna_select_config_grouped": (_i, [_i, _i, _i, _i, _i, _cfgp]),
     "tuna_validate_config": (_i, [_i, _i, _i, _cfgp]),
     "tuna_validate_config_ex": (_i, [_i, _i, _i, _cfgp, _i]),

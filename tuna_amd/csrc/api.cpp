@@ -1459,13 +1459,19 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
             return TUNA_OK;
         }
     }
-    // Aligned shapes from about 20 MB of packed weights: the batched streaming kernel's scale-block variant, a batch of
-    // one for up to 16 tokens (balanced split over one workgroup per compute unit), the token chunks of 16 as the
-    // problems of a batch beyond that (every chunk streams the weights again, in one launch per 32 chunks).
-    // Everything else: the narrow-row kernel's variants.
-    // (below that size the narrow-row kernel's single pass is faster: 12.1 against 16.1 us on 6144 x 4096, 21.4
-    // against 16.5 us on 4096 x 14336)
-    if (stream_mode == 2 || (stream_mode == 1 && (long long)m * k / 2 >= (20ll << 20))) {
+    // Large aligned shapes: the batched streaming kernel's scale-block variant, a batch of one for up to 16 tokens
+    // (balanced split over one workgroup per compute unit), the token chunks of 16 as the problems of a batch beyond
+    // that (every chunk streams the weights again, in one launch per 32 chunks).  Everything else: the narrow-row
+    // kernel's variants, whose single pass with the workgroup's scales in LDS is faster below these sizes.  Measured
+    // at 16 tokens, narrow against streaming: 8.7 / 15.5 us on 6144 x 4096, 14.1 / 16.3 on 8192 x 8192, 19.4 / 20.9 on
+    // 10240 x 8192, 22.4 / 24.2 on 28672 x 4096, but 18.5 / 16.5 on 4096 x 14336, 44 / 35 on 8192 x 28672 and 75 / 66 on
+    // 57344 x 8192; at one token the narrow kernel wins up to 57344 x 8192 (63 / 65) and loses on 229376 x 4096
+    // (117 / 102); at 32 tokens it wins on 6144 x 4096 only.
+    const long long packed_bytes = (long long)m * k / 2;
+    const bool stream_wins = n > 16  ? packed_bytes >= (20ll << 20)
+                             : n > 4 ? packed_bytes >= (100ll << 20) || (n > 8 && k >= 12288 && packed_bytes >= (20ll << 20))
+                                     : packed_bytes >= (256ll << 20);
+    if (stream_mode == 2 || (stream_mode == 1 && stream_wins)) {
         int dev = 0, cus = 0;
         hipError_t e = device_cus(&dev, &cus);
         if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
@@ -1817,6 +1823,8 @@ TUNA_EXPORT int tuna_set_blockwise_stream(int enabled)
 {
     return g_blockwise_stream.exchange(enabled < 0 ? 0 : enabled > 2 ? 2 : enabled, std::memory_order_relaxed);
 }
+
+TUNA_EXPORT int tuna_set_blockwise_scales_lds(int enabled) { return set_blockwise_scales_lds(enabled); }
 
 TUNA_EXPORT int tuna_set_blockwise_shape(int rows, int waves_k, int prefetch)
 {

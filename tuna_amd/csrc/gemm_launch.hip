@@ -231,7 +231,7 @@ void describe_gemm_launch(const GemmPlan &plan, int cus, char *buf, size_t len)
 
 // ---- narrow-row kernel (gemm_narrow.hpp) ---------------------------------------------------------
 typedef void (*NarrowKernelFn)(const uint8_t *, const void *, const float *, const float *, int, int, int, int, void *, int,
-                               const void *, int, int);
+                               const void *, int, int, int);
 struct NarrowVariant {
     int rows, wk, u, tt;
     NarrowKernelFn fn, fn_perm;  // B fragments loaded per lane (up to 4 tokens) / contiguously and permuted
@@ -293,7 +293,7 @@ hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int
     const size_t lds = (size_t)kLutBytes + (size_t)waves_k * ((rows + 15) / 16) * token_tiles * 1024;
     const dim3 grid((unsigned)(args.m / rows), (unsigned)((args.n + 16 * token_tiles - 1) / (16 * token_tiles)), 1);
     hipLaunchKernelGGL(fn, grid, dim3(waves_k * 64), lds, stream, args.q, args.x, args.code, args.absmax, args.k, args.n,
-                       args.n_it, args.m, args.out, args.epilogue, args.residual, 0, 1);
+                       args.n_it, args.m, args.out, args.epilogue, args.residual, 0, 1, 0);
     return hipGetLastError();
 }
 
@@ -310,6 +310,9 @@ static const BlockwiseVariant kBlockwise[] = {
 #undef B
 static constexpr int kNumBlockwise = sizeof(kBlockwise) / sizeof(kBlockwise[0]);
 static std::atomic<int> g_blockwise_shape[3];  // diagnostic override: rows, waves_k, ring depth (0: the library's choice)
+static std::atomic<int> g_blockwise_scales_lds{1};  // A/B switch: the workgroup's scales staged in LDS (1) or read from memory per step (0)
+
+int set_blockwise_scales_lds(int enabled) { return g_blockwise_scales_lds.exchange(enabled ? 1 : 0); }
 
 int set_blockwise_shape(int rows, int waves_k, int prefetch)
 {
@@ -327,9 +330,14 @@ int set_blockwise_shape(int rows, int waves_k, int prefetch)
 
 static bool blockwise_fits(const BlockwiseVariant &v, int m, int k) { return m % v.rows == 0 && k % (kStepK * v.wk * v.u) == 0; }
 
-// The library's choice: the widest tile that still gives three workgroups per four compute units (measured on the
-// benchmark shapes with a scale per 64 weights).
-static const BlockwiseVariant *choose_blockwise(int m, int k, int cus)
+// LDS of a variant's launch without the scales, and the bytes its workgroup's scales take there (rows of nblk + 1 floats)
+static size_t blockwise_base_lds(const BlockwiseVariant &v) { return (size_t)kLutBytes + (size_t)v.wk * (v.rows / 16) * 1024; }
+static size_t blockwise_scale_bytes(const BlockwiseVariant &v, int nblk) { return (size_t)v.rows * (size_t)(nblk + 1) * 4; }
+
+// The library's choice: the widest tile that still gives nine workgroups per sixteen compute units and whose scales
+// fit in LDS (measured on the benchmark shapes and three 2560-wide ones with a scale per 64 weights: one round of
+// 144 to 256 wide workgroups beats two rounds of narrower ones, and scales read from memory cost 1.4 to 2x).
+static const BlockwiseVariant *choose_blockwise(int m, int k, int nblk, int cus)
 {
     const int ov_rows = g_blockwise_shape[0].load();
     if (ov_rows) {
@@ -340,24 +348,25 @@ static const BlockwiseVariant *choose_blockwise(int m, int k, int cus)
         return nullptr;
     }
     static const int pref[][3] = {{64, 8, 4}, {64, 8, 2}, {32, 8, 4}, {32, 8, 2}, {16, 8, 4}, {16, 4, 2}};
-    const BlockwiseVariant *fallback = nullptr;
-    for (const auto &p : pref)
-        for (int i = 0; i < kNumBlockwise; ++i) {
-            const BlockwiseVariant &v = kBlockwise[i];
-            if (v.rows != p[0] || v.wk != p[1] || v.u != p[2] || !blockwise_fits(v, m, k)) continue;
-            if (!fallback) fallback = &v;
-            if (m / v.rows >= cus * 3 / 4) return &v;
-        }
-    if (fallback) {  // fewer row tiles than compute units at every height: the narrowest tile that fits
-        for (int i = 0; i < kNumBlockwise; ++i)
-            if (blockwise_fits(kBlockwise[i], m, k) && kBlockwise[i].rows < fallback->rows) fallback = &kBlockwise[i];
+    for (int need_lds = 1; need_lds >= 0; --need_lds) {
+        const BlockwiseVariant *fallback = nullptr;
+        for (const auto &p : pref)
+            for (int i = 0; i < kNumBlockwise; ++i) {
+                const BlockwiseVariant &v = kBlockwise[i];
+                if (v.rows != p[0] || v.wk != p[1] || v.u != p[2] || !blockwise_fits(v, m, k)) continue;
+                if (need_lds && blockwise_base_lds(v) + blockwise_scale_bytes(v, nblk) > (size_t)kLdsLimit) continue;
+                if (m / v.rows >= cus * 9 / 16) return &v;
+                // fewer row tiles than that at every height: the narrowest tile that fits, the deeper ring first
+                if (!fallback || v.rows < fallback->rows) fallback = &v;
+            }
+        if (fallback) return fallback;
     }
-    return fallback;
+    return nullptr;
 }
 
 bool blockwise_describe(int m, int n, int k, char *buf, size_t len)
 {
-    const BlockwiseVariant *v = choose_blockwise(m, k, kMaxCus);
+    const BlockwiseVariant *v = choose_blockwise(m, k, k / 64, kMaxCus);
     if (!v) return false;
     snprintf(buf, len, "gemm_narrow_kernel<LW=%d,WK=%d,U=%d,PERM=%d,TT=1,BLK>", v->rows / 16, v->wk, v->u, n > 4 ? 1 : 0);
     return true;
@@ -369,18 +378,22 @@ hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, hipStrea
     hipError_t e = device_cus(&dev, &cus);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
-    const BlockwiseVariant *v = choose_blockwise(args.m, args.k, cus);
+    const int nblk = args.k >> (6 + blk_shift);
+    const BlockwiseVariant *v = choose_blockwise(args.m, args.k, nblk, cus);
     if (!v) return hipErrorInvalidConfiguration;
     const int vi = (int)(v - kBlockwise);
     const int perm = args.n > 4;
     const NarrowKernelFn fn = perm ? v->fn_perm : v->fn;
     static OptInFlag done[16][kNumBlockwise][2];
     if ((e = ensure_lds_opt_in(done[dev][vi][perm], reinterpret_cast<const void *>(fn))) != hipSuccess) return e;
-    const size_t lds = (size_t)kLutBytes + (size_t)v->wk * (v->rows / 16) * 1024;
+    size_t lds = blockwise_base_lds(*v);
     const dim3 grid((unsigned)(args.m / v->rows), (unsigned)((args.n + 15) / 16), 1);
-    const int nblk = args.k >> (6 + blk_shift);
+    // the workgroup's scales in LDS when they fit beside the table and the reduction planes
+    const size_t scale_bytes = blockwise_scale_bytes(*v, nblk);
+    const int slds = g_blockwise_scales_lds.load(std::memory_order_relaxed) && lds + scale_bytes <= (size_t)kLdsLimit;
+    if (slds) lds += scale_bytes;
     hipLaunchKernelGGL(fn, grid, dim3(v->wk * 64), lds, stream, args.q, args.x, args.code, args.absmax, args.k, args.n,
-                       args.k / kStepK / v->wk, args.m, args.out, TUNA_EPILOGUE_NONE, nullptr, blk_shift, nblk);
+                       args.k / kStepK / v->wk, args.m, args.out, TUNA_EPILOGUE_NONE, nullptr, blk_shift, nblk, slds);
     return hipGetLastError();
 }
 

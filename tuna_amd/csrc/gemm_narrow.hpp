@@ -26,6 +26,11 @@
 //     A wave's double step of 64 k lies inside one block; the scales of a ring slot's block travel
 //     through the ring with its weights and are rounded to fp16 when the slot is consumed - the
 //     decode is fp16(code) * fp16(absmax of the block), the GEMM's rounding with a finer scale.
+//     The workgroup's scales ([rows][k / block], contiguous in memory) are copied into LDS once at
+//     the start (a_slds; rows one float apart from a multiple of the bank count) and read from
+//     there when a ring slot is refilled: a wave's scale load from global memory touches sixteen
+//     cache lines for sixteen values, as much address work as sixteen weight loads.  Without
+//     a_slds (slices that do not fit beside table and reduction planes) they come from memory.
 // Requires k % (32*WK*U) == 0, m % (16*LW) == 0, dense launches; a workgroup takes 16*TT tokens
 // (TT = token_tiles = 1, 2, 4: every decoded weight fragment feeds TT MFMAs), more tokens are
 // gridDim.y chunks.  Selected by rows_per_wave = 16 or 32 in the config,
@@ -46,7 +51,7 @@ template <int LW, int WK, int U, bool PERM, int TT, bool BLK = false, int ROWS =
 __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q, const void *a_x, const float *a_code,
                                                               const float *a_absmax, int a_k, int a_n, int a_n_it, int a_m,
                                                               void *a_out, int a_epilogue, const void *a_residual,
-                                                              int a_blk_shift, int a_nblk)
+                                                              int a_blk_shift, int a_nblk, int a_slds)
 {
     struct {
         const uint8_t *q;
@@ -62,6 +67,7 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     static_assert(ROWS % 8 == 0 && ROWS % LW == 0 && ROWS <= 16 * LW && ROWS > 8 * LW, "rows of a partly filled tile");
     unsigned char *lut = smem;
     float *red = reinterpret_cast<float *>(smem + kLutBytes);  // [wave][row plane][token tile][lane][4]
+    float *sbuf = red + WK * LW * TT * 256;  // BLK with a_slds: [row][a_nblk + 1] scales of the workgroup
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -128,7 +134,13 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
         const size_t qo_ = (size_t)((u) >> 1) * (WK * 256) + ((u) & 1) * 128;              \
         if constexpr (BLK) {                                                                   \
             const int blk_ = (dstep + ((u) >> 1) * WK) >> a_blk_shift;                         \
-            _Pragma("unroll") for (int j = 0; j < LW; ++j) sq[u][j] = sp[(size_t)j * a_nblk + blk_]; \
+            if (a_slds) {                                                                      \
+                if (dstep != wk) {                                                             \
+                    _Pragma("unroll") for (int j = 0; j < LW; ++j) sq[u][j] = sbuf[(LW * ia + j) * (a_nblk + 1) + blk_]; \
+                }                                                                              \
+            } else {                                                                           \
+                _Pragma("unroll") for (int j = 0; j < LW; ++j) sq[u][j] = sp[(size_t)j * a_nblk + blk_]; \
+            }                                                                                  \
         }                                                                                      \
         _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) xq[u][tt] = *reinterpret_cast<const u32x4 *>(xp + xo_ + xoff[tt]); \
         if constexpr (LW == 1) {                                                               \
@@ -147,6 +159,18 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     qp += (size_t)(U / 2) * (WK * 256);
     xp += (size_t)(U / 2) * (WK * 128);
     dstep += (U / 2) * WK;
+    // BLK, scales through LDS: the first eight scales per thread of the workgroup's slice are requested here and
+    // stored behind the table build; longer slices follow in further rounds
+    constexpr int SB = 8;
+    float sv[BLK ? SB : 1];
+    const int s_count = BLK ? ROWS * a_nblk : 0;
+    const float *s_src = a.absmax + (size_t)row0 * (size_t)(BLK ? a_nblk : 1);
+    if constexpr (BLK) {
+        if (a_slds) {
+#pragma unroll
+            for (int i = 0; i < SB; ++i) sv[i] = s_src[min(tid + i * nthreads, s_count - 1)];
+        }
+    }
 
     // ---- decode table (see gemm_kernel.hpp), built while the loads are in flight ------------
     {
@@ -173,7 +197,36 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
         const f16 h = (f16)sc32[j];
         sc16[j] = f16x2{h, h};
     }
-    __syncthreads();  // the table is complete
+    if constexpr (BLK) {
+        if (a_slds) {
+            const int pitch = a_nblk + 1;
+            for (int base = 0; base < s_count; base += SB * nthreads) {
+                if (base) {
+#pragma unroll
+                    for (int i = 0; i < SB; ++i) sv[i] = s_src[min(base + tid + i * nthreads, s_count - 1)];
+                }
+#pragma unroll
+                for (int i = 0; i < SB; ++i) {
+                    const int idx = base + tid + i * nthreads;
+                    const int r = idx / a_nblk;
+                    if (idx < s_count) sbuf[r * pitch + (idx - r * a_nblk)] = sv[i];
+                }
+            }
+        }
+    }
+    __syncthreads();  // the table (and the scales) are complete
+    if constexpr (BLK) {
+        if (a_slds) {
+            // the first ring turn's scales (its weights were requested before the scales were in LDS)
+            const float *sl = sbuf + LW * ia * (a_nblk + 1);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int blk_ = (wk + (u >> 1) * WK) >> a_blk_shift;
+#pragma unroll
+                for (int j = 0; j < LW; ++j) sq[u][j] = sl[j * (a_nblk + 1) + blk_];
+            }
+        }
+    }
 
     // ---- main loop: n_it / U ring turns, the last one without refills ------------------------
     f32x4 acc[LW][TT];
