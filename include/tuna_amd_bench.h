@@ -98,7 +98,7 @@ int tuna_set_multi_shape(int waves_m, int prefetch);
 int tuna_set_multi_weight_path(int through_lds);
 /* Diagnostic switch, process-wide, default 1: tuna_matmul_blockwise runs launches of more than 32 tokens through the
  * many-token kernel's scale-block variants, and large launches whose shape allows (m a multiple of 64, k of 256 and of
- * the block; 17 to 32 tokens from 20 MB of packed weights, 9 to 16 tokens from 100 MB or from 20 MB when k >= 12288,
+ * the block; 17 to 32 tokens from 100 MB of packed weights, from 40 MB when k > 4096 and from 12 MB when k > 8192, 9 to 16 tokens from 100 MB or from 20 MB when k >= 12288,
  * 5 to 8 tokens from 100 MB, 1 to 4 tokens from 256 MB) through the scale-block variant of the batched streaming kernel
  * (a batch of one up to 16 tokens, the token chunks as a batch beyond); 2: the batched streaming kernel for every launch it can plan,
  * whatever its size and token count; 0: always the narrow-row kernel's variants.  All decode fp16(code) * fp16(absmax of

@@ -1644,6 +1644,11 @@ def test_blockwise_gemm_matches_oracle_and_reads_out_the_decode(m, n, k, bs):
     (256, 16, 1536, 64, (16, 4, 2)),     # k range of three ring turns
     (128, 9, 28672, 64, (64, 8, 4)),     # 64 rows x 449 floats do not fit beside the table: scales stay in memory
     (2560, 16, 10240, 64, None),         # 160 tiles of 16 rows
+    (1024, 32, 4096, 64, (64, 8, 4)),    # two token tiles per workgroup, 64 rows
+    (512, 23, 2048, 64, (32, 8, 2)),     # two token tiles, the second ragged
+    (256, 70, 1024, 128, (16, 4, 2)),    # three passes of two token tiles, the last with one
+    (768, 32, 8192, 64, None),           # two token tiles, the library's choice of rows
+    (256, 32, 28672, 64, (64, 8, 4)),    # two token tiles, scales in memory (they do not fit in LDS)
 ])
 def test_blockwise_narrow_kernel_with_scales_in_lds_and_in_memory(m, n, k, bs, shape):
     """The narrow-row kernel's scale-block variants stage the workgroup's scales in LDS when they fit and read them

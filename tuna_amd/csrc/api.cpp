@@ -1466,9 +1466,12 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
     // at 16 tokens, narrow against streaming: 8.7 / 15.5 us on 6144 x 4096, 14.1 / 16.3 on 8192 x 8192, 19.4 / 20.9 on
     // 10240 x 8192, 22.4 / 24.2 on 28672 x 4096, but 18.5 / 16.5 on 4096 x 14336, 44 / 35 on 8192 x 28672 and 75 / 66 on
     // 57344 x 8192; at one token the narrow kernel wins up to 57344 x 8192 (63 / 65) and loses on 229376 x 4096
-    // (117 / 102); at 32 tokens it wins on 6144 x 4096 only.
+    // (117 / 102); at 32 tokens, with two token tiles per workgroup, 11.9 / 16.9 on 6144 x 4096, 20.3 / 24.6 on
+    // 8192 x 8192, 30.9 / 38.7 on 28672 x 4096, 21.4 / 28.3 on 13824 x 5120, but 37.2 / 30.4 on 10240 x 8192, 29.6 / 22.7
+    // on 4096 x 14336, 22.1 / 18.3 on 2560 x 10240, 134 / 106 on 32768 x 14336 and 131 / 108 on 57344 x 8192.
     const long long packed_bytes = (long long)m * k / 2;
-    const bool stream_wins = n > 16  ? packed_bytes >= (20ll << 20)
+    const bool stream_wins = n > 16  ? packed_bytes >= (100ll << 20) || (k > 8192 && packed_bytes >= (12ll << 20)) ||
+                                           (k > 4096 && packed_bytes >= (40ll << 20))
                              : n > 4 ? packed_bytes >= (100ll << 20) || (n > 8 && k >= 12288 && packed_bytes >= (20ll << 20))
                                      : packed_bytes >= (256ll << 20);
     if (stream_mode == 2 || (stream_mode == 1 && stream_wins)) {

@@ -300,14 +300,18 @@ hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int
 // Scale blocks finer than a row: the narrow-row kernel's BLK variants (the scales of a ring slot's block travel
 // through the ring with its weights).  block = 64 << blk_shift weights per scale.
 struct BlockwiseVariant {
-    int rows, wk, u;
+    int rows, wk, u, tt;
     NarrowKernelFn fn, fn_perm;
 };
-#define B(LW, WK, U) {16 * LW, WK, U, gemm_narrow_kernel<LW, WK, U, false, 1, true>, gemm_narrow_kernel<LW, WK, U, true, 1, true>}
+#define B(LW, WK, U) {16 * LW, WK, U, 1, gemm_narrow_kernel<LW, WK, U, false, 1, true>, gemm_narrow_kernel<LW, WK, U, true, 1, true>}
+#define B2(LW, WK, U) {16 * LW, WK, U, 2, gemm_narrow_kernel<LW, WK, U, true, 2, true>, gemm_narrow_kernel<LW, WK, U, true, 2, true>}
 static const BlockwiseVariant kBlockwise[] = {
     B(1, 4, 2), B(1, 8, 4), B(1, 16, 2), B(2, 8, 2), B(2, 8, 4), B(2, 16, 2), B(4, 4, 4), B(4, 8, 2), B(4, 8, 4), B(4, 16, 2),
+    // two token tiles per workgroup: 17..32 tokens in one pass over the weights
+    B2(1, 4, 2), B2(1, 8, 4), B2(2, 8, 2), B2(2, 8, 4), B2(4, 8, 2), B2(4, 8, 4),
 };
 #undef B
+#undef B2
 static constexpr int kNumBlockwise = sizeof(kBlockwise) / sizeof(kBlockwise[0]);
 static std::atomic<int> g_blockwise_shape[3];  // diagnostic override: rows, waves_k, ring depth (0: the library's choice)
 static std::atomic<int> g_blockwise_scales_lds{1};  // A/B switch: the workgroup's scales staged in LDS (1) or read from memory per step (0)
@@ -319,7 +323,7 @@ int set_blockwise_shape(int rows, int waves_k, int prefetch)
     if (rows || waves_k || prefetch) {
         bool found = false;
         for (int i = 0; i < kNumBlockwise; ++i)
-            found |= kBlockwise[i].rows == rows && kBlockwise[i].wk == waves_k && kBlockwise[i].u == prefetch;
+            found |= kBlockwise[i].tt == 1 && kBlockwise[i].rows == rows && kBlockwise[i].wk == waves_k && kBlockwise[i].u == prefetch;
         if (!found) return -1;
     }
     g_blockwise_shape[0].store(rows);
@@ -331,20 +335,22 @@ int set_blockwise_shape(int rows, int waves_k, int prefetch)
 static bool blockwise_fits(const BlockwiseVariant &v, int m, int k) { return m % v.rows == 0 && k % (kStepK * v.wk * v.u) == 0; }
 
 // LDS of a variant's launch without the scales, and the bytes its workgroup's scales take there (rows of nblk + 1 floats)
-static size_t blockwise_base_lds(const BlockwiseVariant &v) { return (size_t)kLutBytes + (size_t)v.wk * (v.rows / 16) * 1024; }
+static size_t blockwise_base_lds(const BlockwiseVariant &v) { return (size_t)kLutBytes + (size_t)v.wk * (v.rows / 16) * v.tt * 1024; }
 static size_t blockwise_scale_bytes(const BlockwiseVariant &v, int nblk) { return (size_t)v.rows * (size_t)(nblk + 1) * 4; }
 
 // The library's choice: the widest tile that still gives nine workgroups per sixteen compute units and whose scales
 // fit in LDS (measured on the benchmark shapes and three 2560-wide ones with a scale per 64 weights: one round of
 // 144 to 256 wide workgroups beats two rounds of narrower ones, and scales read from memory cost 1.4 to 2x).
-static const BlockwiseVariant *choose_blockwise(int m, int k, int nblk, int cus)
+static const BlockwiseVariant *choose_blockwise(int m, int k, int nblk, int cus, int tt)
 {
     const int ov_rows = g_blockwise_shape[0].load();
     if (ov_rows) {
         const int wk = g_blockwise_shape[1].load(), u = g_blockwise_shape[2].load();
-        for (int i = 0; i < kNumBlockwise; ++i)
-            if (kBlockwise[i].rows == ov_rows && kBlockwise[i].wk == wk && kBlockwise[i].u == u && blockwise_fits(kBlockwise[i], m, k))
-                return &kBlockwise[i];
+        for (int t = tt; t >= 1; --t)  // (the two-tile twin of the named shape where one is built)
+            for (int i = 0; i < kNumBlockwise; ++i)
+                if (kBlockwise[i].tt == t && kBlockwise[i].rows == ov_rows && kBlockwise[i].wk == wk && kBlockwise[i].u == u &&
+                    blockwise_fits(kBlockwise[i], m, k))
+                    return &kBlockwise[i];
         return nullptr;
     }
     static const int pref[][3] = {{64, 8, 4}, {64, 8, 2}, {32, 8, 4}, {32, 8, 2}, {16, 8, 4}, {16, 4, 2}};
@@ -353,7 +359,7 @@ static const BlockwiseVariant *choose_blockwise(int m, int k, int nblk, int cus)
         for (const auto &p : pref)
             for (int i = 0; i < kNumBlockwise; ++i) {
                 const BlockwiseVariant &v = kBlockwise[i];
-                if (v.rows != p[0] || v.wk != p[1] || v.u != p[2] || !blockwise_fits(v, m, k)) continue;
+                if (v.tt != tt || v.rows != p[0] || v.wk != p[1] || v.u != p[2] || !blockwise_fits(v, m, k)) continue;
                 if (need_lds && blockwise_base_lds(v) + blockwise_scale_bytes(v, nblk) > (size_t)kLdsLimit) continue;
                 if (m / v.rows >= cus * 9 / 16) return &v;
                 // fewer row tiles than that at every height: the narrowest tile that fits, the deeper ring first
@@ -361,14 +367,14 @@ static const BlockwiseVariant *choose_blockwise(int m, int k, int nblk, int cus)
             }
         if (fallback) return fallback;
     }
-    return nullptr;
+    return tt > 1 ? choose_blockwise(m, k, nblk, cus, 1) : nullptr;  // (shapes only the 16-row, 4-wave tile of one token tile fits)
 }
 
 bool blockwise_describe(int m, int n, int k, char *buf, size_t len)
 {
-    const BlockwiseVariant *v = choose_blockwise(m, k, k / 64, kMaxCus);
+    const BlockwiseVariant *v = choose_blockwise(m, k, k / 64, kMaxCus, n > 16 ? 2 : 1);
     if (!v) return false;
-    snprintf(buf, len, "gemm_narrow_kernel<LW=%d,WK=%d,U=%d,PERM=%d,TT=1,BLK>", v->rows / 16, v->wk, v->u, n > 4 ? 1 : 0);
+    snprintf(buf, len, "gemm_narrow_kernel<LW=%d,WK=%d,U=%d,PERM=%d,TT=%d,BLK>", v->rows / 16, v->wk, v->u, n > 4 ? 1 : 0, v->tt);
     return true;
 }
 
@@ -379,7 +385,7 @@ hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, hipStrea
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
     const int nblk = args.k >> (6 + blk_shift);
-    const BlockwiseVariant *v = choose_blockwise(args.m, args.k, nblk, cus);
+    const BlockwiseVariant *v = choose_blockwise(args.m, args.k, nblk, cus, args.n > 16 ? 2 : 1);
     if (!v) return hipErrorInvalidConfiguration;
     const int vi = (int)(v - kBlockwise);
     const int perm = args.n > 4;
@@ -387,7 +393,7 @@ hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, hipStrea
     static OptInFlag done[16][kNumBlockwise][2];
     if ((e = ensure_lds_opt_in(done[dev][vi][perm], reinterpret_cast<const void *>(fn))) != hipSuccess) return e;
     size_t lds = blockwise_base_lds(*v);
-    const dim3 grid((unsigned)(args.m / v->rows), (unsigned)((args.n + 15) / 16), 1);
+    const dim3 grid((unsigned)(args.m / v->rows), (unsigned)((args.n + 16 * v->tt - 1) / (16 * v->tt)), 1);
     // the workgroup's scales in LDS when they fit beside the table and the reduction planes
     const size_t scale_bytes = blockwise_scale_bytes(*v, nblk);
     const int slds = g_blockwise_scales_lds.load(std::memory_order_relaxed) && lds + scale_bytes <= (size_t)kLdsLimit;
