@@ -1035,14 +1035,23 @@ MID_CASES = [
     (2048, 1100, 512, dict(waves_m=1, waves_k=4, prefetch=2, token_tiles=2, x_chunk=256), None),     # 32 x 35: more workgroups than CUs
     (51200, 300, 256, dict(waves_m=8, waves_k=1, prefetch=2, token_tiles=8, x_chunk=128),
      dict(waves_m=8, waves_k=1, prefetch=2, token_tiles=4, x_chunk=128)),                            # 100 x 3, eight token tiles
+    # k split across workgroups: the parts of a row tile meet through the workspace, summed in k order
+    (1024, 32, 4096, dict(waves_m=4, waves_k=2, prefetch=2, token_tiles=2, x_chunk=256, split_k=2), None),
+    (1024, 33, 2048, dict(waves_m=2, waves_k=4, prefetch=2, token_tiles=4, x_chunk=256, split_k=4), None),   # two chunks per part, ragged
+    (512, 64, 4096, dict(waves_m=1, waves_k=8, prefetch=2, token_tiles=2, x_chunk=512, split_k=8), None),    # one chunk per part, two token chunks
+    (1024, 64, 2048, dict(waves_m=4, waves_k=1, prefetch=2, token_tiles=4, x_chunk=128, split_k=4), None),   # all waves along the rows
+    (37888, 20, 512, dict(waves_m=2, waves_k=2, prefetch=2, token_tiles=2, x_chunk=128, split_k=2), None),   # 592 (tile, part) pairs: walkers
+    (16640, 150, 256, dict(waves_m=2, waves_k=2, prefetch=2, token_tiles=2, x_chunk=128, split_k=2), None),  # 260 pairs x 5 token chunks side by side
+    (2048, 100, 8192, dict(waves_m=2, waves_k=4, prefetch=2, token_tiles=4, x_chunk=256, split_k=16), None), # 16 parts: four round trips of four
 ]
 
 
 @pytest.mark.parametrize("ci", range(len(MID_CASES)))
 def test_mid_token_kernel_equals_general_kernel_bit_for_bit(ci):
-    """Dense unsplit launches with two or four token tiles take the 17..128-token streaming kernel;
-    it must give the bits of the general kernel (same decode, same summation order), for the plain
-    store and both fused epilogues, and be within tolerance of the oracle."""
+    """Dense launches with two, four or eight token tiles, unsplit or with k split into a power of two of
+    equal parts, take the 17..128-token streaming kernel; it must give the bits of the general kernel (same
+    decode, same summation order), for the plain store and both fused epilogues, and be within tolerance of
+    the oracle."""
     import torch
 
     from tuna_amd import _lib, ops
@@ -1092,6 +1101,10 @@ LDS_PATH_CASES = [
     (2048, 100, 1024, 8, 1, 2, 128, 0, 8),     # one pass of 128 tokens, 100 present
     (1024, 300, 1024, 4, 2, 2, 128, 3, 8),     # three token chunks
     (512 * 70, 1100, 512, 8, 1, 2, 128, 0, 8), # 70 row tiles x 9 token chunks: chunks of a walker side by side
+    # k split across workgroups (10th entry)
+    (1024, 64, 4096, 2, 4, 2, 256, 0, 4, 4),
+    (2048, 32, 8192, 4, 4, 2, 512, 0, 2, 2),   # 16 waves
+    (512 * 70, 40, 1024, 4, 2, 4, 256, 0, 2, 4),  # 140 row tiles x 4 parts: walkers
 ]
 
 
@@ -1107,11 +1120,12 @@ def test_weights_staged_through_lds_equal_the_register_ring_bit_for_bit(ci):
 
     m, n, k, wm, wk, pf, xc, st = LDS_PATH_CASES[ci][:8]
     tt = LDS_PATH_CASES[ci][8] if len(LDS_PATH_CASES[ci]) > 8 else 1
-    c = cfg(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=1, prefetch=pf, x_chunk=xc, k_stagger=st, token_tiles=tt)
+    split = LDS_PATH_CASES[ci][9] if len(LDS_PATH_CASES[ci]) > 9 else 1
+    c = cfg(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=split, prefetch=pf, x_chunk=xc, k_stagger=st, token_tiles=tt)
     print(f"lds path case#{ci} {m}x{n}x{k} {c.to_dict()}", flush=True)
     q, x, code, absmax = make_inputs_np(m, n, k, seed=700 + ci)
     dq, dx, dc, da = to_dev(q, x, code, absmax)
-    c_lds = cfg(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=1, prefetch=pf, x_chunk=xc, k_stagger=st, token_tiles=tt,
+    c_lds = cfg(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=split, prefetch=pf, x_chunk=xc, k_stagger=st, token_tiles=tt,
                 lds_tile_rows=-1)
     outs = {}
     prev = ops.set_weight_path(False)

@@ -19,23 +19,6 @@
 
 namespace tuna {
 
-// Four 16-byte device-coherent loads of partial sums (the counterpart of store_partial) and the
-// wait for them, in one statement: the compiler does not know that the results arrive later,
-// so nothing of its own may come between the loads and the wait.
-__device__ __forceinline__ void load_partials4(const float *s0, const float *s1, const float *s2, const float *s3, f32x4 &p0,
-                                               f32x4 &p1, f32x4 &p2, f32x4 &p3)
-{
-    asm volatile(
-        "global_load_dwordx4 %0, %4, off sc1\n\t"
-        "global_load_dwordx4 %1, %5, off sc1\n\t"
-        "global_load_dwordx4 %2, %6, off sc1\n\t"
-        "global_load_dwordx4 %3, %7, off sc1\n\t"
-        "s_waitcnt vmcnt(0)"
-        : "=&v"(p0), "=&v"(p1), "=&v"(p2), "=&v"(p3)
-        : "v"(s0), "v"(s1), "v"(s2), "v"(s3)
-        : "memory");
-}
-
 // What the kernel needs of GemmArgs, as separate scalar arguments with the ones the first loads
 // use in front: the first 14 dwords of such arguments are preloaded into scalar registers with
 // the wave (build flag -amdgpu-kernarg-preload-count), a struct passed by value is fetched by

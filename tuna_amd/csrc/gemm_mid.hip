@@ -7,31 +7,42 @@
 namespace tuna {
 
 typedef void (*MidKernelFn)(const uint8_t *, const void *, const float *, const float *, int, int, int, int, void *,
-                            const void *, int, int, int);
+                            const void *, int, int, int, float *, unsigned *, int);
 struct MidVariant {
     int u, tt, xb, maxt;
     MidKernelFn fn;
     MidKernelFn fn_shared;  // twin without the nontemporal hint on the weight loads (token chunks side by side), or null
     MidKernelFn fn_lds;     // twin with the packed weights staged through LDS (lds_tile_rows = -1 or the diagnostic switch), or null
     MidKernelFn fn_lds_shared;  // ... without the nontemporal hint, or null
+    MidKernelFn fn_split;      // twin for k split across workgroups, or null
+    MidKernelFn fn_split_lds;  // ... with the packed weights staged through LDS, or null
 };
 #define M5(U, TT, XB) {U, TT, XB, 512, gemm_mid_kernel<U, TT, XB, 512, 2>, nullptr, nullptr, nullptr}
 #define M5L(U, TT, XB) {U, TT, XB, 512, gemm_mid_kernel<U, TT, XB, 512, 2>, nullptr, gemm_mid_kernel<U, TT, XB, 512, 2, true, true>, nullptr}
+#define M5LS(U, TT, XB)                                                                                             \
+    {U, TT, XB, 512, gemm_mid_kernel<U, TT, XB, 512, 2>, nullptr, gemm_mid_kernel<U, TT, XB, 512, 2, true, true>, nullptr, \
+     gemm_mid_kernel<U, TT, XB, 512, 2, true, false, true>, gemm_mid_kernel<U, TT, XB, 512, 2, true, true, true>}
 #define M5SL(U, TT, XB)                                                                                             \
     {U, TT, XB, 512, gemm_mid_kernel<U, TT, XB, 512, 2>, gemm_mid_kernel<U, TT, XB, 512, 2, false>,                \
      gemm_mid_kernel<U, TT, XB, 512, 2, true, true>, gemm_mid_kernel<U, TT, XB, 512, 2, false, true>}
 #define M10(U, TT, XB) {U, TT, XB, 1024, gemm_mid_kernel<U, TT, XB, 1024, 4>, nullptr, nullptr, nullptr}
 #define M10L(U, TT, XB) {U, TT, XB, 1024, gemm_mid_kernel<U, TT, XB, 1024, 4>, nullptr, gemm_mid_kernel<U, TT, XB, 1024, 4, true, true>, nullptr}
+#define M10LS(U, TT, XB)                                                                                            \
+    {U, TT, XB, 1024, gemm_mid_kernel<U, TT, XB, 1024, 4>, nullptr, gemm_mid_kernel<U, TT, XB, 1024, 4, true, true>, nullptr, \
+     gemm_mid_kernel<U, TT, XB, 1024, 4, true, false, true>, gemm_mid_kernel<U, TT, XB, 1024, 4, true, true, true>}
 static const MidVariant kMid[] = {
-    M5L(2, 2, 4), M5L(4, 2, 4), M5(8, 2, 4), M5(2, 2, 8), M5(4, 2, 8), M5(8, 2, 8),
-    M5L(2, 4, 4), M5L(4, 4, 4), M5(8, 4, 4), M5L(2, 4, 8), M5L(4, 4, 8), M5(8, 4, 8),
+    // (the ...S entries also have twins for k split across workgroups)
+    M5LS(2, 2, 4), M5LS(4, 2, 4), M5(8, 2, 4), M5(2, 2, 8), M5(4, 2, 8), M5(8, 2, 8),
+    M5LS(2, 4, 4), M5LS(4, 4, 4), M5(8, 4, 4), M5LS(2, 4, 8), M5LS(4, 4, 8), M5(8, 4, 8),
     M5SL(2, 8, 4), M5SL(2, 8, 8),  // (deeper rings with eight token tiles spill inside the loop)
-    M10L(2, 2, 4), M10L(4, 2, 4),
+    M10LS(2, 2, 4), M10LS(4, 2, 4),
     // one token tile: the large shapes at up to 16 tokens (small launches take gemm_lean.hpp first)
     M5(2, 1, 4), M5(4, 1, 4), M5(8, 1, 4), M5(2, 1, 8), M5(4, 1, 8), M5(8, 1, 8), M10L(2, 1, 4), M10L(4, 1, 4), M10(8, 1, 4),
 };
 #undef M5
 #undef M5L
+#undef M5LS
+#undef M10LS
 #undef M5SL
 #undef M10
 #undef M10L
@@ -65,13 +76,15 @@ static const MidVariant *mid_variant(const GemmPlan &plan, int *xc_out)
     const GemmArgs &a = plan.args;
     if (a.group_rows || a.balanced || plan.rw != 1 || plan.decode != TUNA_DECODE_GEMM) return nullptr;
     if (plan.token_tiles != 1 && plan.token_tiles != 2 && plan.token_tiles != 4 && plan.token_tiles != 8) return nullptr;
-    if (a.split_k != 1 || a.k_stagger < 0 || a.k_stagger > 4096 || a.waves_k > 16 || (a.waves_k & (a.waves_k - 1)) != 0)
-        return nullptr;
+    if (a.k_stagger < 0 || a.k_stagger > 4096 || a.waves_k > 16 || (a.waves_k & (a.waves_k - 1)) != 0) return nullptr;
+    // k split across workgroups: a power of two of equal parts, two or more token tiles (one token tile: the lean
+    // kernel's launches), no stagger
+    if (a.split_k != 1 && (a.split_log2 < 1 || a.split_log2 > 8 || plan.token_tiles < 2 || a.k_stagger != 0)) return nullptr;
     if (a.k != a.steps_total * kStepK || a.k >= (1 << 23)) return nullptr;
     if (a.m % (a.waves_m * kRowsPerLoad) != 0 || a.waves_m * a.waves_k > 16) return nullptr;
     const int xc = mid_x_chunk(plan);
     // a chunk is whole ring turns of the workgroup: xc / 32 steps, waves_k * prefetch per turn
-    if (xc < a.waves_k * plan.prefetch * kStepK || (xc & (xc - 1)) != 0 || a.k % xc != 0) return nullptr;
+    if (xc < a.waves_k * plan.prefetch * kStepK || (xc & (xc - 1)) != 0 || a.k % (xc * a.split_k) != 0) return nullptr;
     const int pieces = plan.token_tiles * 2 * xc;  // 16-byte pieces per chunk
     const int per_thread = (pieces + plan.threads - 1) / plan.threads;
     if (per_thread > 8) return nullptr;
@@ -79,6 +92,7 @@ static const MidVariant *mid_variant(const GemmPlan &plan, int *xc_out)
     const int maxt = plan.threads <= 512 ? 512 : 1024;
     for (int i = 0; i < kNumMid; ++i)
         if (kMid[i].u == plan.prefetch && kMid[i].tt == plan.token_tiles && kMid[i].xb == xb && kMid[i].maxt == maxt) {
+            if (a.split_k != 1 && !kMid[i].fn_split) return nullptr;
             *xc_out = xc;
             return &kMid[i];
         }
@@ -108,8 +122,9 @@ bool mid_describe(const GemmPlan &plan, char *buf, size_t len)
     int xc;
     const MidVariant *v = mid_variant(plan, &xc);
     if (!v) return false;
-    snprintf(buf, len, "gemm_mid_kernel<U=%d,TT=%d,XB=%d,%d threads%s> x_chunk=%d", v->u, v->tt, v->xb, v->maxt,
-             mid_lds_applies(plan) ? ",weights through LDS" : "", xc);
+    int used = snprintf(buf, len, "gemm_mid_kernel<U=%d,TT=%d,XB=%d,%d threads%s> x_chunk=%d", v->u, v->tt, v->xb, v->maxt,
+                        mid_lds_applies(plan) ? ",weights through LDS" : "", xc);
+    if (plan.args.split_k > 1 && used > 0 && (size_t)used < len) snprintf(buf + used, len - used, " split_k=%d", plan.args.split_k);
     return true;
 }
 
@@ -123,7 +138,7 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
     if (!v) return hipErrorInvalidConfiguration;
     const int vi = (int)(v - kMid);
     if (!g_mid_attr_done[dev][vi].load(std::memory_order_acquire)) {
-        for (const MidKernelFn f : {v->fn, v->fn_shared, v->fn_lds, v->fn_lds_shared}) {
+        for (const MidKernelFn f : {v->fn, v->fn_shared, v->fn_lds, v->fn_lds_shared, v->fn_split, v->fn_split_lds}) {
             if (!f) continue;
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(f), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
             if (e != hipSuccess) return e;
@@ -140,7 +155,9 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
                                                    : (x_lds > red_lds ? x_lds : red_lds));
     if (plan.lds_weights && !staged) return hipErrorInvalidConfiguration;
     dim3 grid = plan.grid;
-    grid.x = (unsigned)(a.row_tiles < cus ? a.row_tiles : cus);  // one workgroup per CU (LDS), walking row tiles
+    const int split_log2 = a.split_k > 1 ? a.split_log2 : 0;
+    const int walk_tiles = a.row_tiles << split_log2;  // (row tile, part of k) pairs
+    grid.x = (unsigned)(walk_tiles < cus ? walk_tiles : cus);  // one workgroup per CU (LDS), walking row tiles
     // Several token chunks that do not all fit the device at once: rather than one round of row
     // tile walkers per chunk (every round streams all weights from HBM again), fewer walkers whose
     // token chunks run side by side and share the weights through the caches.  With a multiple of
@@ -150,7 +167,7 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
     // in launch order only (chunks < 0), which still shares through the memory-side cache.
     // Mixtral gate+up, eight token tiles: 1024 tokens 1870 -> 1740 us, 2048 tokens 3746 -> 3520 us.
     int chunks = 0, n_wg = (int)grid.x;
-    if (grid.y > 1 && (long long)a.row_tiles * (long long)grid.y > (long long)cus && grid.y <= 4096) {
+    if (grid.y > 1 && (long long)walk_tiles * (long long)grid.y > (long long)cus && grid.y <= 4096) {
         const int c = (int)grid.y;
         const int w8 = (cus / c) & ~7;
         if (w8 >= 8 && (long long)w8 * c * 8 >= 7LL * cus) {
@@ -165,10 +182,11 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
     const int packed = a.waves_m | a.epilogue << 5 | xc_log2 << 8 | a.wk_log2 << 13 | a.k_stagger << 16;
     // weights that sibling workgroups re-read stay in the caches longer without the nontemporal hint
     // (Mixtral gate+up, 1024 tokens: 1745 -> 1687 us)
-    const MidKernelFn fn = staged ? ((chunks && v->fn_lds_shared) ? v->fn_lds_shared : v->fn_lds)
-                                  : (chunks && v->fn_shared) ? v->fn_shared : v->fn;
+    const MidKernelFn fn = split_log2 ? (staged ? v->fn_split_lds : v->fn_split)
+                           : staged   ? ((chunks && v->fn_lds_shared) ? v->fn_lds_shared : v->fn_lds)
+                                      : (chunks && v->fn_shared) ? v->fn_shared : v->fn;
     hipLaunchKernelGGL(fn, grid, dim3(plan.threads), lds, stream, a.q, a.x, a.code, a.absmax, a.k, a.n, a.m, packed, a.out,
-                       a.residual, a.row_tiles, n_wg, chunks);
+                       a.residual, walk_tiles, n_wg, chunks, a.ws, a.counters, split_log2);
     return hipGetLastError();
 }
 

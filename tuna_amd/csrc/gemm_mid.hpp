@@ -5,11 +5,15 @@
 // many weight loads a wave keeps in flight and how little else it does.  (With one token tile it
 // is the general kernel without a split across workgroups, a tile walk to pay for or a stagger.)
 // This kernel computes exactly what gemm_kernel computes for one class of launches:
-//   * dense, no split of k across workgroups (split_k = 1), m a multiple of the
-//     workgroup's rows, k a multiple of the x chunk, chunks of whole ring turns of the workgroup:
-//     no clamped or conditional weight loads, no tails; with all waves along m the accumulators
-//     are final and stored from registers, with waves along k they are summed through LDS in
-//     wave order as in gemm_kernel;
+//   * dense, m a multiple of the workgroup's rows, k a multiple of the x chunk, chunks of whole
+//     ring turns of the workgroup: no clamped or conditional weight loads, no tails; with all
+//     waves along m the accumulators are final and stored from registers, with waves along k they
+//     are summed through LDS in wave order as in gemm_kernel;
+//   * k unsplit, or (two or more token tiles, no stagger) split into a power of two of equal parts
+//     of whole x chunks: a workgroup then walks (row tile, part) pairs, and the parts of a row tile
+//     meet through the workspace as in gemm_kernel - partial sums stored, an arrival ticket per
+//     tile, the last arrival adds the parts in k order and stores the outputs.  No workgroup
+//     waits for another;
 //   * x chunks are double-buffered in LDS: chunk c + 1 is requested before chunk c is consumed
 //     and written to the other buffer after it, one barrier per chunk, and the weight ring runs
 //     on across chunk and tile boundaries' barriers without being emptied;
@@ -68,11 +72,13 @@ __device__ __forceinline__ void barrier_lds_only()
 
 // NT: weight loads carry the nontemporal hint (each byte is used once per launch).  Launches whose
 // token chunks share the weights through the caches (a_chunks != 0) run the twin without it.
-template <int U, int TT, int XB, int MAXT, int MINW, bool NT = true, bool LDSW = false>
+// SPLIT: the twin for launches with k split across workgroups (the unsplit kernels carry none of its code).
+template <int U, int TT, int XB, int MAXT, int MINW, bool NT = true, bool LDSW = false, bool SPLIT = false>
 __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q, const void *a_x, const float *a_code,
                                                               const float *a_absmax, int a_k, int a_n, int a_m, int a_packed,
                                                               void *a_out, const void *a_residual, int a_row_tiles,
-                                                              int a_n_wg, int a_chunks)
+                                                              int a_n_wg, int a_chunks, float *a_ws, unsigned *a_counters,
+                                                              int a_split_log2)
 {
     // a_packed = waves_m | epilogue << 5 | log2(x chunk in k) << 8 | log2(waves_k) << 13 | k_stagger << 16
     const int waves_m = a_packed & 31;
@@ -114,8 +120,12 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     const int tok0 = tok_chunk * (16 * TT);
     const int xc = 1 << xc_log2;
     const int chunk_its = (xc >> 5) >> wk_log2;      // k-steps of one wave per chunk, a multiple of U
-    const int n_chunks = a_k >> xc_log2;
-    const int n_steps = a_k >> 5;
+    // k split across workgroups (a_split_log2 != 0): a_row_tiles counts (row tile, part) pairs, pair t is row tile
+    // t >> a_split_log2, part t & (parts - 1); n_steps, n_chunks and k_len are those of one part
+    const int split_log2 = SPLIT ? a_split_log2 : 0;
+    const int k_len = a_k >> split_log2;
+    const int n_chunks = k_len >> xc_log2;
+    const int n_steps = k_len >> 5;
     const uint32_t kb_total = (uint32_t)a_k >> 3;
     const uint32_t xbuf_bytes = (uint32_t)(TT * 32) << xc_log2;  // 16*TT tokens x xc k x 2 bytes
     const int x_pieces = (int)(xbuf_bytes >> 4);
@@ -146,13 +156,13 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     // Chunk at logical k `kbase` of a tile whose walk starts rot_k elements into the k range and
     // wraps around (stagger, as in gemm_kernel.hpp): physical k = logical + rot_k, minus k past the
     // end - a piece is 8 k of one 32-k step and rot_k a multiple of 32, so no piece straddles the wrap.
-#define TUNA_MID_X_LOAD(kbase, rot_k)                                                           \
+#define TUNA_MID_X_LOAD(kbase, rot_k, part_k)                                                   \
     {                                                                                          \
         const uint32_t kb_ = (uint32_t)(kbase) + (uint32_t)(rot_k);                            \
-        const unsigned char *xc_ = x_tile + (size_t)kb_ * 2;                                   \
-        const uint32_t wrap_at_ = (uint32_t)a_k - kb_; /* pieces at or past it wrap (kb_ < 2k) */ \
+        const unsigned char *xc_ = x_tile + (size_t)(kb_ + (uint32_t)(part_k)) * 2;            \
+        const uint32_t wrap_at_ = (uint32_t)k_len - kb_; /* pieces at or past it wrap (kb_ < 2k) */ \
         _Pragma("unroll") for (int b = 0; b < XB; ++b) xst.v[b] = *reinterpret_cast<const u32x4 *>( \
-            xc_ + x_goff[b] - ((int32_t)(x_kloc[b] - wrap_at_) >= 0 ? (size_t)a_k * 2 : (size_t)0)); \
+            xc_ + x_goff[b] - ((int32_t)(x_kloc[b] - wrap_at_) >= 0 ? (size_t)k_len * 2 : (size_t)0)); \
     }
     // (rows past n are zeroed, as the general kernel does)
 #define TUNA_MID_X_STORE(buf)                                                                   \
@@ -170,7 +180,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     // 8-k group g) fetches its own B-fragment piece.  Token rows past n are clamped (their output
     // columns are never stored).
     const int xdma_n = LDSW ? max(1, ((xc >> 5) * TT) / (nthreads >> 6)) : 0;
-#define TUNA_MID_X_DMA(buf, kbase, rot_steps)                                                   \
+#define TUNA_MID_X_DMA(buf, kbase, rot_steps, part_steps)                                       \
     {                                                                                          \
         _Pragma("unroll 1") for (int b = 0; b < xdma_n; ++b)                                  \
         {                                                                                      \
@@ -178,6 +188,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
             const int ks_ = i_ / TT, tt_ = i_ % TT;                                            \
             int s_ = ((kbase) >> 5) + ks_ + (rot_steps);                                       \
             if (s_ >= n_steps) s_ -= n_steps;                                                  \
+            s_ += (part_steps);                                                                \
             const uint32_t lane_ = ((uint32_t)min(tt_ * 16 + i16, a_n - 1 - tok0) * (uint32_t)a_k + (uint32_t)g * 8u) * 2u; \
             load_weights_to_lds<false>(x_tile + (size_t)s_ * 64 + lane_, (buf) + i_ * 1024);   \
         }                                                                                      \
@@ -203,18 +214,20 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     // (block row i16/2, second half of the block for odd i16), block column 4*step + g
     uint32_t lb = 0;
     int rot = 0;
+    int ps = 0;  // first k-step of the tile's part
     u32x4 wq[U];
     f32x4 sc32{0.f, 0.f, 0.f, 0.f};
     XStage<XB> xst;
 #define TUNA_MID_TILE_FETCH(t)                                                                  \
     {                                                                                          \
-        const int row0_ = (t) * (waves_m * 64) + wm * 64;                                      \
+        const int row0_ = ((t) >> split_log2) * (waves_m * 64) + wm * 64;                      \
+        ps = ((t) & ((1 << split_log2) - 1)) * n_steps;                                        \
         /* stagger: row tile t walks k starting rot steps in, wrapping around (gemm_kernel.hpp) */ \
         rot = (k_stagger && n_steps > 1) ? (int)(((unsigned)(t) * k_stagger) % (unsigned)n_steps) : 0; \
         lb = ((uint32_t)(row0_ >> 3) + (uint32_t)(i16 >> 1)) * kb_total * 32u + (uint32_t)(i16 & 1) * 16u + (uint32_t)g * 32u; \
         /* x and the scales first: vector loads return in order, and the tile's first barrier */ \
         /* waits for the x pieces only - the first ring turn stays in flight across it */        \
-        if constexpr (!LDSW) TUNA_MID_X_LOAD(0, rot << 5)                                      \
+        if constexpr (!LDSW) TUNA_MID_X_LOAD(0, rot << 5, ps << 5)                             \
         if constexpr (!LDSW) {                                                                 \
             _Pragma("unroll") for (int j = 0; j < 4; ++j) sc32[j] = a_absmax[row0_ + i16 * 4 + j]; \
         }                                                                                      \
@@ -222,6 +235,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
         {                                                                                      \
             int s_ = wk + (u << wk_log2) + rot;                                                \
             if (s_ >= n_steps) s_ -= n_steps;                                                  \
+            s_ += ps;                                                                          \
             if constexpr (LDSW) load_weights_to_lds<NT>(a_q + (size_t)s_ * 128 + lb, wring + u * 1024); \
             else wq[u] = load_weights<NT>(reinterpret_cast<const u32x4 *>(a_q + (size_t)s_ * 128 + lb)); \
         }                                                                                      \
@@ -233,8 +247,8 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     // (free until chunk 1 is requested; read back at the top of the tile)
 #define TUNA_MID_TOP_DMA(t, rot_steps)                                                          \
     {                                                                                          \
-        TUNA_MID_X_DMA(xbuf, 0, rot_steps)                                                     \
-        load_weights_to_lds<false>(reinterpret_cast<const unsigned char *>(a_absmax + (t) * (waves_m * 64) + wm * 64 + i16 * 4), \
+        TUNA_MID_X_DMA(xbuf, 0, rot_steps, ((t) & ((1 << split_log2) - 1)) * n_steps)          \
+        load_weights_to_lds<false>(reinterpret_cast<const unsigned char *>(a_absmax + ((t) >> split_log2) * (waves_m * 64) + wm * 64 + i16 * 4), \
                                    xbuf + ((uint32_t)(TT * 32) << xc_log2) + wave * 1024);     \
     }
     if constexpr (LDSW) {
@@ -335,7 +349,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
             const f16 h = (f16)sc32[j];
             sc16[j] = f16x2{h, h};
         }
-        const int row0 = tile * (waves_m * 64) + wm * 64;
+        const int row0 = (tile >> split_log2) * (waves_m * 64) + wm * 64;
         f32x4 acc[4][TT];
 #pragma unroll
         for (int j = 0; j < 4; ++j)
@@ -354,8 +368,9 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
             __syncthreads();
         }
 
-        const unsigned char *qrow = a_q + lb;
+        const unsigned char *qrow = a_q + lb + (size_t)ps * 128;
         const int cur_rot = rot;
+        const int cur_ps = ps;
         int it = 0;  // this wave's next iteration (its k-step wk + it*waves_k)
         for (int c = 0; c < n_chunks; ++c) {
             const bool has_next = c + 1 < n_chunks;
@@ -363,9 +378,9 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
             // the compiler could not count these loads into the waits of the first ring turn)
             if constexpr (LDSW) {
                 // (the other buffer was last read in chunk c - 1, which ended with a barrier)
-                TUNA_MID_X_DMA(xbuf + ((c + 1) & 1) * xbuf_bytes, min(c + 1, n_chunks - 1) << xc_log2, cur_rot)
+                TUNA_MID_X_DMA(xbuf + ((c + 1) & 1) * xbuf_bytes, min(c + 1, n_chunks - 1) << xc_log2, cur_rot, cur_ps)
             } else {
-                TUNA_MID_X_LOAD(min(c + 1, n_chunks - 1) << xc_log2, cur_rot << 5)
+                TUNA_MID_X_LOAD(min(c + 1, n_chunks - 1) << xc_log2, cur_rot << 5, cur_ps << 5)
             }
             const unsigned char *xb = xbuf + (c & 1) * xbuf_bytes + xb_lane;
             // (the first ring turn of a chunk is a copy of its own: there the x pieces just
@@ -388,9 +403,10 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
 
         // ---- next tile's loads, then this tile's store ------------------------------------------
         const int cur_row0 = row0;
+        const int cur_tile = tile;
         tile += a_n_wg;
         if (tile < a_row_tiles) TUNA_MID_TILE_FETCH(tile)
-        if (wk_log2 != 0) {
+        if (wk_log2 != 0 || split_log2 != 0) {
             // Waves along k: every wave puts its copy of a plane (one float4 per lane) in LDS - two
             // buffers alternate in the x area, free since the barrier that ended the last chunk -
             // and thread (wk, lane) sums floats f = (i*waves_k + wk)*64 + lane of it in wave order:
@@ -398,6 +414,11 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
             // 64, so after the four planes a thread owns 4 consecutive features of one token.
             float *redf = reinterpret_cast<float *>(xbuf);
             const size_t plane_floats = (size_t)(waves_m << wk_log2) * 256;
+            // split: this wave row's partial sums of part p of the tile at wst + p * seg_floats, as [token tile][f] float4s
+            const size_t seg_floats = (size_t)waves_m * (TT * 1024);
+            const size_t tile_id = (size_t)tok_chunk * (size_t)(a_row_tiles >> split_log2) + (size_t)(cur_tile >> split_log2);
+            float *wst = a_ws + (tile_id << split_log2) * seg_floats + (size_t)wm * (TT * 1024);
+            const int part = cur_tile & ((1 << split_log2) - 1);
 #pragma unroll
             for (int tt = 0; tt < TT; ++tt) {
                 float o[4][4];  // [i][j]
@@ -412,11 +433,52 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
                 for (int i = 0; i < 4; ++i) {
                     const int f = ((i << wk_log2) + wk) * 64 + lane;
                     if (f >= 256) continue;
+                    if (split_log2 != 0) {
+                        store_partial(wst + (size_t)part * seg_floats + (size_t)(tt * 256 + f) * 4,
+                                      f32x4{o[i][0], o[i][1], o[i][2], o[i][3]});
+                        continue;
+                    }
                     const int l = f >> 2, v = f & 3;
                     const int tok = tok0 + tt * 16 + (l & 15);
                     if (tok < a_n)
                         store_features4(outp, resp, epilogue, (size_t)tok, a_m, cur_row0 + (l >> 4) * 16 + v * 4, o[i][0], o[i][1],
                                         o[i][2], o[i][3]);
+                }
+            }
+            if (split_log2 != 0) {
+                // hand-over (see gemm_kernel): stores complete, barrier (also: every read of the reduction
+                // buffers is done), arrival ticket, the last arrival adds the parts in k order
+                __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                __syncthreads();
+                volatile unsigned *ticket = reinterpret_cast<volatile unsigned *>(xbuf);
+                if (tid == 0) *ticket = __hip_atomic_fetch_add(a_counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __syncthreads();
+                const int parts = 1 << split_log2;
+                if (*ticket == (unsigned)parts - 1u) {
+                    if (tid == 0) __hip_atomic_store(a_counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    for (int tt = 0; tt < TT; ++tt)
+                        for (int i = 0; i < 4; ++i) {
+                            const int f = ((i << wk_log2) + wk) * 64 + lane;
+                            if (f >= 256) break;
+                            const float *src = wst + (size_t)(tt * 256 + f) * 4;
+                            f32x4 s4 = f32x4{0.f, 0.f, 0.f, 0.f};
+                            for (int sp0 = 0; sp0 < parts; sp0 += 4) {  // four contributors per round trip
+                                f32x4 p[4];
+                                const float *psrc[4];
+#pragma unroll
+                                for (int b = 0; b < 4; ++b) psrc[b] = src + (size_t)min(sp0 + b, parts - 1) * seg_floats;
+                                load_partials4(psrc[0], psrc[1], psrc[2], psrc[3], p[0], p[1], p[2], p[3]);
+#pragma unroll
+                                for (int b = 0; b < 4; ++b)
+                                    if (sp0 + b < parts) s4 += p[b];
+                            }
+                            const int l = f >> 2, v = f & 3;
+                            const int tok = tok0 + tt * 16 + (l & 15);
+                            if (tok < a_n)
+                                store_features4(outp, resp, epilogue, (size_t)tok, a_m, cur_row0 + (l >> 4) * 16 + v * 4, s4[0],
+                                                s4[1], s4[2], s4[3]);
+                        }
                 }
             }
             __syncthreads();  // the x area is written again at the top of the next tile

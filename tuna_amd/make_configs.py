@@ -56,6 +56,10 @@ MID_VARIANTS = ({(u, tt, xb, 512) for u in (2, 4, 8) for tt in (2, 4) for xb in 
                 | {(2, 8, 4, 512), (2, 8, 8, 512), (2, 2, 4, 1024), (4, 2, 4, 1024)}
                 | {(u, 1, xb, 512) for u in (2, 4, 8) for xb in (4, 8)} | {(u, 1, 4, 1024) for u in (2, 4, 8)})
 
+# ... of those, the ones with a twin for k split across workgroups (fn_split of kMid)
+MID_SPLIT_VARIANTS = ({(u, tt, xb, 512) for u in (2, 4) for (tt, xb) in ((2, 4), (4, 4), (4, 8))}
+                      | {(2, 2, 4, 1024), (4, 2, 4, 1024)})
+
 # (rows, waves_k, prefetch, token_tiles) of the narrow-row kernel; must match kNarrow in csrc/gemm_launch.hip
 NARROW_VARIANTS = (
     {(r, wk, pf, 1) for r in (16, 32, 64) for wk in (4, 8, 16) for pf in (2, 4, 8)}
@@ -168,7 +172,11 @@ def _mid_variant(m: int, k: int, c: dict, lds_path: bool):
     """(variant key, x chunk) of the streaming kernel for a dense launch of this config, or None
     (mirrors mid_variant and mid_x_chunk in csrc/gemm_mid.hip)."""
     tt, wm, wk = c["token_tiles"], c["waves_m"], c["waves_k"]
-    if c["rows_per_wave"] != 64 or tt not in (1, 2, 4, 8) or c["split_k"] != 1 or not 0 <= c["k_stagger"] <= 4096:
+    if c["rows_per_wave"] != 64 or tt not in (1, 2, 4, 8) or not 0 <= c["k_stagger"] <= 4096:
+        return None
+    split = c["split_k"]
+    # k split across workgroups: 2..256 equal parts, a power of two, two or more token tiles, no stagger
+    if split != 1 and (not _pow2(split) or split > 256 or tt < 2 or c["k_stagger"] != 0):
         return None
     if k % STEP_K or k >= 1 << 23 or not _pow2(wk) or wm < 1 or wm * wk > 16 or m % (64 * wm):
         return None
@@ -178,12 +186,14 @@ def _mid_variant(m: int, k: int, c: dict, lds_path: bool):
     cap = (LDS_LIMIT - LUT_BYTES - ring) // (2 * tt * 32)
     while xc > cap:
         xc //= 2
-    if xc < wk * c["prefetch"] * STEP_K or k % xc:
+    if xc < wk * c["prefetch"] * STEP_K or k % (xc * split):
         return None
     per_thread = -(-(tt * 2 * xc) // threads)
     if per_thread > 8:
         return None
     key = (c["prefetch"], tt, 4 if per_thread <= 4 else 8, 512 if threads <= 512 else 1024)
+    if split != 1 and key not in MID_SPLIT_VARIANTS:
+        return None
     return (key, xc) if key in MID_VARIANTS else None
 
 

@@ -168,8 +168,8 @@ def lean_space(m: int, n_key: int, k: int):
 
 def mid_space(m: int, n_key: int, k: int):
     """Every config whose launch takes the 17..128-token streaming kernel (gemm_mid.hpp; the
-    conditions of mid_variant in gemm_mid.hip): 64 rows per wave, no split across workgroups.
-    Small enough to time exhaustively."""
+    conditions of mid_variant in gemm_mid.hip): 64 rows per wave, k unsplit or split into a power of two
+    of parts.  Small enough to time exhaustively."""
     lo, hi = make_configs.N_BUCKETS[n_key]
     out = []
     # tuned at the bucket's lower edge; from 128 tokens on, passes of eight token tiles (on the
@@ -186,21 +186,26 @@ def mid_space(m: int, n_key: int, k: int):
                 for pf in (2, 4, 8):
                     for xc in (128, 256, 512, 1024, 2048):
                         for sw, stg in ((0, 0), (1, 0), (0, 2), (0, 5)):
-                            c = dict(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=1, prefetch=pf, x_chunk=xc,
-                                     token_tiles=tt, xcd_swizzle=sw, k_stagger=stg, lds_tile_rows=0)
-                            try:
-                                make_configs.validate(m, n_key, k, c)
-                            except ValueError:
-                                continue
-                            if make_configs.mid_applies(m, k, c):
-                                out.append(c)
-                                # the same launch with the packed weights staged through LDS, where that twin exists
-                                cl = dict(c, lds_tile_rows=-1)
+                            # k split across workgroups (two or more token tiles, no stagger): where the row tiles
+                            # alone leave compute units idle, up to about two rounds of workgroups
+                            for split in (1, 2, 4, 8, 16):
+                                if split > 1 and (tt < 2 or stg or (m // (64 * wm)) * (split // 2) >= 2 * N_CU):
+                                    continue
+                                c = dict(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=split, prefetch=pf, x_chunk=xc,
+                                         token_tiles=tt, xcd_swizzle=sw, k_stagger=stg, lds_tile_rows=0)
                                 try:
-                                    make_configs.validate(m, n_key, k, cl)
-                                    out.append(cl)
+                                    make_configs.validate(m, n_key, k, c)
                                 except ValueError:
-                                    pass
+                                    continue
+                                if make_configs.mid_applies(m, k, c):
+                                    out.append(c)
+                                    # the same launch with the packed weights staged through LDS, where that twin exists
+                                    cl = dict(c, lds_tile_rows=-1)
+                                    try:
+                                        make_configs.validate(m, n_key, k, cl)
+                                        out.append(cl)
+                                    except ValueError:
+                                        pass
     return out
 
 
