@@ -85,8 +85,9 @@ typedef struct tuna_gemm_config {
     int32_t lds_tile_rows; /* 0: streaming kernel (all fields above).  -1: the same, with the packed
                               weights, x and scales staged through LDS by global -> LDS loads
                               (the reference's weight path, kernel.cu:1997-2042) instead of
-                              registers: same results bit for bit; for unsplit launches of 8 or 16
-                              waves with prefetch 2 or 4 (2 with eight token tiles).  64, 128 or 256: the
+                              registers: same results bit for bit; for launches of 8 or 16 waves
+                              with prefetch 2 or 4 (2 with eight token tiles), k unsplit or, with
+                              two or four token tiles, split into a power of two of equal parts.  64, 128 or 256: the
                               many-token kernel, which decodes a tile of this many weight rows
                               once into LDS for token_tiles*16 (64, 128 or 256) tokens; only
                               token_tiles, split_k (>= 1) and rows_per_wave are read besides:

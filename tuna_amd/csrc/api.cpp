@@ -197,9 +197,9 @@ static int plan_gemm(int m, int n, int k, const tuna_gemm_config &c, int decode,
                     grouped ? "grouped " : "", c.rows_per_wave, c.prefetch, c.token_tiles, decode, threads);
     if (p.lds_weights && (grouped || !mid_lds_applies(*plan)))
         return fail(TUNA_ERR_UNSUPPORTED,
-                    "lds_tile_rows=-1 (packed weights through LDS) needs a dense unsplit launch of 8 or 16 waves, 64 rows per wave, "
-                    "prefetch 2 or 4 (2 with eight token tiles), the GEMM's own decode, m a multiple of 64*waves_m and x chunks "
-                    "that divide k and leave room for the rings");
+                    "lds_tile_rows=-1 (packed weights through LDS) needs a dense launch of 8 or 16 waves, 64 rows per wave, prefetch 2 "
+                    "or 4 (2 with eight token tiles), the GEMM's own decode, m a multiple of 64*waves_m, x chunks that divide k "
+                    "(k/split_k for a power-of-two split with two or four token tiles; no other split) and leave room for the rings");
     return TUNA_OK;
 }
 

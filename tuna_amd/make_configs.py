@@ -158,7 +158,7 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
     if lds_bytes(c) > LDS_LIMIT:
         raise ValueError(f"needs {lds_bytes(c)} bytes of LDS (limit {LDS_LIMIT})")
     if c["lds_tile_rows"] == -1 and not mid_lds_applies(m, k, c):
-        raise ValueError("lds_tile_rows -1 needs an unsplit launch of 8 or 16 waves the streaming kernel takes, prefetch 2 or 4 "
+        raise ValueError("lds_tile_rows -1 needs a launch of 8 or 16 waves the streaming kernel takes, prefetch 2 or 4 "
                          "(2 with eight token tiles) and x chunks that leave room for the weight rings")
 
 
