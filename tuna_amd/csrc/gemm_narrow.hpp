@@ -67,7 +67,8 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     static_assert(ROWS % 8 == 0 && ROWS % LW == 0 && ROWS <= 16 * LW && ROWS > 8 * LW, "rows of a partly filled tile");
     unsigned char *lut = smem;
     float *red = reinterpret_cast<float *>(smem + kLutBytes);  // [wave][row plane][token tile][lane][4]
-    float *sbuf = red + WK * LW * TT * 256;  // BLK with a_slds: [row][a_nblk + 1] scales of the workgroup
+    // BLK with a_slds: [row][a_nblk + 1] scales of the workgroup, each rounded to fp16 and stored twice in a dword
+    uint32_t *sbuf = reinterpret_cast<uint32_t *>(red + WK * LW * TT * 256);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -123,7 +124,11 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     const unsigned char *xp = reinterpret_cast<const unsigned char *>(a.x) + (size_t)tok0 * a.k * 2 + (size_t)wk * 128;
     uint32_t wq[U][LW];
     u32x4 xq[U][TT];
-    float sq[BLK ? U : 1][LW];  // BLK: the scales of the ring slot's block
+    uint32_t sq[BLK ? U : 1][LW];  // BLK: the scales of the ring slot's block, rounded to fp16, twice in a dword
+    const auto pack_scale = [](float s_) {
+        const uint32_t h_ = (uint32_t)f16_bits((f16)s_);
+        return h_ | (h_ << 16);
+    };
     // BLK: lane's first scale, and the double step of ring slot 0 in the turn being loaded
     const float *sp = a.absmax + (size_t)(row0 + LW * ia) * (size_t)(BLK ? a_nblk : 1);
     int dstep = wk;
@@ -135,11 +140,13 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
         if constexpr (BLK) {                                                                   \
             const int blk_ = (dstep + ((u) >> 1) * WK) >> a_blk_shift;                         \
             if (a_slds) {                                                                      \
+                /* (the two slots of a double step lie in one block: the second copies the first) */ \
                 if (dstep != wk) {                                                             \
-                    _Pragma("unroll") for (int j = 0; j < LW; ++j) sq[u][j] = sbuf[(LW * ia + j) * (a_nblk + 1) + blk_]; \
+                    _Pragma("unroll") for (int j = 0; j < LW; ++j) sq[u][j] =                  \
+                        ((u) & 1) ? sq[(u) & ~1][j] : sbuf[(LW * ia + j) * (a_nblk + 1) + blk_]; \
                 }                                                                              \
             } else {                                                                           \
-                _Pragma("unroll") for (int j = 0; j < LW; ++j) sq[u][j] = sp[(size_t)j * a_nblk + blk_]; \
+                _Pragma("unroll") for (int j = 0; j < LW; ++j) sq[u][j] = pack_scale(sp[(size_t)j * a_nblk + blk_]); \
             }                                                                                  \
         }                                                                                      \
         _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) xq[u][tt] = *reinterpret_cast<const u32x4 *>(xp + xo_ + xoff[tt]); \
@@ -209,7 +216,7 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
                 for (int i = 0; i < SB; ++i) {
                     const int idx = base + tid + i * nthreads;
                     const int r = idx / a_nblk;
-                    if (idx < s_count) sbuf[r * pitch + (idx - r * a_nblk)] = sv[i];
+                    if (idx < s_count) sbuf[r * pitch + (idx - r * a_nblk)] = pack_scale(sv[i]);
                 }
             }
         }
@@ -218,7 +225,7 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
     if constexpr (BLK) {
         if (a_slds) {
             // the first ring turn's scales (its weights were requested before the scales were in LDS)
-            const float *sl = sbuf + LW * ia * (a_nblk + 1);
+            const uint32_t *sl = sbuf + LW * ia * (a_nblk + 1);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int blk_ = (wk + (u >> 1) * WK) >> a_blk_shift;
@@ -248,10 +255,7 @@ __global__ __launch_bounds__(WK * 64) void gemm_narrow_kernel(const uint8_t *a_q
         _Pragma("unroll") for (int j = 0; j < LW; ++j)                                         \
         {                                                                                      \
             f16x2 s_ = sc16[j];                                                                \
-            if constexpr (BLK) {                                                               \
-                const f16 h_ = (f16)sq[u][j];                                                  \
-                s_ = f16x2{h_, h_};                                                            \
-            }                                                                                  \
+            if constexpr (BLK) s_ = __builtin_bit_cast(f16x2, sq[u][j]);                       \
             const f16x8 av_ = decode_dword<TUNA_DECODE_GEMM>(wq[u][j], lut, lane4, s_, 0.f);   \
             _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) acc[j][tt] =                     \
                 __builtin_amdgcn_mfma_f32_16x16x32_f16(av_, b_[tt], acc[j][tt], 0, 0, 0);      \
