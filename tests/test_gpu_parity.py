@@ -109,6 +109,89 @@ def test_gemm_with_dequant_rounding_through_the_dispatcher_on_benchmark_configs(
     assert np.array_equal(got_h, img[:, cols].T)
 
 
+def _random_shapes(count, seed, m_step, k_step):
+    """Seeded shapes no table entry has: m and k multiples of the given steps, a token count from every bucket."""
+    rng = np.random.default_rng(seed)
+    tokens = [1, 2, 3, 5, 8, 11, 13, 16, 17, 24, 31, 32, 40, 63, 64, 65, 100, 128, 130, 200, 256, 300, 511, 512, 700, 1030]
+    out = []
+    for i in range(count):
+        # about a third each: small, one-pass sized (8 .. 60 MB packed) and long-k shapes
+        kind = i % 3
+        if kind == 0:
+            m, k = int(rng.integers(1, 40)) * m_step, int(rng.integers(1, 24)) * k_step
+        elif kind == 1:
+            m, k = int(rng.integers(2048 // m_step, 12288 // m_step)) * m_step, int(rng.integers(2048 // k_step, 6144 // k_step)) * k_step
+        else:
+            m, k = int(rng.integers(1024 // m_step, 4096 // m_step)) * m_step, int(rng.integers(8192 // k_step, 20480 // k_step)) * k_step
+        n = tokens[int(rng.integers(0, len(tokens)))]
+        if m * n > 6_000_000:     # keeps the output and the oracle's sample small
+            n = tokens[int(rng.integers(0, 12))]
+        out.append((m, n, k))
+    return out
+
+
+@pytest.mark.parametrize("m,n,k", _random_shapes(36, 20240607, 8, 8) + _random_shapes(24, 77, 64, 256))
+def test_gemm_through_the_dispatcher_on_random_shapes(m, n, k):
+    """tuna_matmul without a config on seeded random shapes (multiples of 8, and multiples of 64 x 256 that the
+    streaming kernels' derived configs take): whatever kernel the dispatcher picks, every output is written, a
+    row sample matches the oracle's float64 sums, and one-hot activations read the decoded weights out exactly."""
+    print(f"random shape m={m} n={n} k={k}", flush=True)
+    from tuna_amd import ops
+
+    print("  " + ops.describe_launch(m, n, k, None), flush=True)
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=m + 3 * n + 7 * k)
+    got = run_gemm(q, x, code, absmax, m, n, k, prefill=float("nan"))
+    assert not np.isnan(f16_bits_to_f64(got)).any()
+    rng = np.random.default_rng(m + n)
+    rows = np.sort(rng.choice(m, size=min(m, 96), replace=False)).astype(np.int32)
+    ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1, rows=rows)
+    e = rel_err(f16_bits_to_f64(got[:, rows]), ref)
+    assert e <= REL_TOL, e
+    nh = min(n, k)
+    cols = rng.choice(k, size=nh, replace=False)
+    xh = np.zeros((n, k), np.float16)
+    xh[np.arange(nh), cols] = 1.0
+    got_h = run_gemm(q, xh, code, absmax, m, n, k)
+    img = O.dequant(q, absmax, code, m, k, mode=O.D1)
+    assert np.array_equal(got_h[:nh], img[:, cols].T)
+    assert not got_h[nh:].any() or np.array_equal(got_h[nh:] & 0x7fff, np.zeros_like(got_h[nh:]))
+
+
+@pytest.mark.parametrize("m,n,k", _random_shapes(30, 4242, 16, 256))
+def test_blockwise_gemm_through_the_dispatcher_on_random_shapes(m, n, k):
+    """tuna_matmul_blockwise (a scale per 64 or 128 weights) on seeded random shapes, routed by the library
+    between the narrow-row, batched streaming and many-token kernels: complete output, oracle on a row sample,
+    exact read-out of the decoded weights."""
+    import torch
+
+    from tuna_amd import ops
+
+    bs = 64 if (m // 16) % 2 else 128
+    print(f"random blockwise shape m={m} n={n} k={k} block={bs}", flush=True)
+    rng = np.random.default_rng(m + n + k)
+    q, x, code, _ = make_inputs_np(m, n, k, seed=m + 5 * n + k)
+    absmax = rng.uniform(0.005, 0.02, size=(m, k // bs)).astype(np.float16).astype(np.float32)
+    dq, dx, dc, da = to_dev(q, x, code, absmax)
+    out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+    ops.matmul_blockwise(dx, dq, da, dc, out, m, n, k, bs)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().view(np.uint16)
+    assert not np.isnan(got.view(np.float16)).any()
+    rows = np.sort(rng.choice(m, size=min(m, 96), replace=False)).astype(np.int32)
+    ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1, rows=rows, block_size=bs)
+    e = rel_err(f16_bits_to_f64(got[:, rows]), ref)
+    assert e <= REL_TOL, e
+    nh = min(n, k)
+    cols = rng.choice(k, size=nh, replace=False)
+    xh = np.zeros((n, k), np.float16)
+    xh[np.arange(nh), cols] = 1.0
+    dxh, = to_dev(xh)
+    ops.matmul_blockwise(dxh, dq, da, dc, out, m, n, k, bs)
+    torch.cuda.synchronize()
+    img = O.dequant(q, absmax, code, m, k, mode=O.D1, block_size=bs)
+    assert np.array_equal(out.cpu().numpy().view(np.uint16)[:nh], img[:, cols].T)
+
+
 SMALL = [
     # m, n, k
     (8, 1, 8), (8, 16, 8), (64, 16, 64), (72, 3, 40), (136, 16, 1032), (256, 16, 128),
