@@ -203,10 +203,14 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         sv[0] = sp_[min(b0_ + 2 * s_pair, nblk_ - 1)];                                         \
         sv[1] = sp_[min(b0_ + 2 * s_pair + 1, nblk_ - 1)];                                     \
     }
+    /* (stored rounded to fp16, twice in a dword: what the decode multiplies with) */
 #define TUNA_MULTI_S_STORE(buf)                                                                 \
     {                                                                                          \
-        reinterpret_cast<float *>(buf)[(2 * s_pair) * 256 + (tid >> 2)] = sv[0];               \
-        reinterpret_cast<float *>(buf)[(2 * s_pair + 1) * 256 + (tid >> 2)] = sv[1];           \
+        _Pragma("unroll") for (int e_ = 0; e_ < 2; ++e_)                                       \
+        {                                                                                      \
+            const uint32_t h_ = (uint32_t)f16_bits((f16)sv[e_]);                               \
+            reinterpret_cast<uint32_t *>(buf)[(2 * s_pair + e_) * 256 + (tid >> 2)] = h_ | (h_ << 16); \
+        }                                                                                      \
     }
 
     // LDSW: chunk `c` straight into `buf`, k-step `wave` of the chunk per wave; lane (token i16, 8-k group g)
@@ -379,11 +383,11 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
             if constexpr (BLK) {                                                               \
                 /* the step's scale block, counted from the chunk's first one */               \
                 const int rel_ = ((sbc + (((sl) + u) << wk_log2) + wk) >> blk_sh) - (sbc >> blk_sh); \
-                const f32x4 s4_ = *reinterpret_cast<const f32x4 *>(sb_lane + (size_t)rel_ * 1024); \
+                const u32x4 s4_ = *reinterpret_cast<const u32x4 *>(sb_lane + (size_t)rel_ * 1024); \
                 _Pragma("unroll") for (int j = 0; j < 4; ++j)                                  \
                 {                                                                              \
-                    const f16 h_ = (f16)s4_[j];                                                \
-                    sc16[j] = f16x2{h_, h_};                                                   \
+                    const uint32_t e_ = s4_[j]; /* (a copy: bit_cast of a vector element reads element 0) */ \
+                    sc16[j] = __builtin_bit_cast(f16x2, e_);                                   \
                 }                                                                              \
             }                                                                                  \
             _Pragma("unroll") for (int j = 0; j < 4; ++j)                                      \
