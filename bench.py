@@ -326,7 +326,7 @@ def time_blockwise(ops, synth, torch, dev, names=("mistral_qkv", "mistral_gate_u
         scales = [torch.rand((m, k // block_size), dtype=torch.float32, device=dev) * 0.015 + 0.005 for _ in range(nsets)]
         x = synth.make_x_torch(tokens, k, 3, dev)
         o = torch.empty((tokens, m), dtype=torch.float16, device=dev)
-        before = [L.tuna_blockwise_launches(i) for i in range(3)]
+        before = [L.tuna_blockwise_launches(i) for i in range(4)]
         calls = 4 * nsets
         side = torch.cuda.Stream()
         with torch.cuda.stream(side):
@@ -338,8 +338,8 @@ def time_blockwise(ops, synth, torch, dev, names=("mistral_qkv", "mistral_gate_u
                 for i in range(calls):
                     ops.matmul_blockwise(x, sets[i % nsets][0], scales[i % nsets], code, o, m, tokens, k, block_size)
         torch.cuda.synchronize()
-        took = [L.tuna_blockwise_launches(i) - before[i] for i in range(3)]
-        kernel = ("tuna::gemm_narrow_kernel", "tuna::gemm_multi_kernel", "tuna::gemm_tiled_kernel")[took.index(max(took))]
+        took = [L.tuna_blockwise_launches(i) - before[i] for i in range(4)]
+        kernel = ("tuna::gemm_narrow_kernel", "tuna::gemm_multi_kernel", "tuna::gemm_tiled_kernel", "tuna::gemm_mid_kernel")[took.index(max(took))]
         for _ in range(3):
             graph.replay()
         torch.cuda.synchronize()

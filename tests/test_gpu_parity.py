@@ -1845,6 +1845,54 @@ def test_blockwise_gemm_through_the_batched_streaming_kernel(m, n, k, bs):
         L.tuna_set_blockwise_stream(prev)
 
 
+@pytest.mark.parametrize("m,n,k,bs", [(256, 16, 1024, 64), (512, 7, 2048, 64), (1024, 16, 4096, 128), (2048, 1, 8192, 64),
+                                      (256 * 70, 16, 1024, 64), (768, 13, 5120, 64), (512, 16, 8192, 4096), (1024, 16, 2048, 1024),
+                                      (4096, 16, 4096, 64), (16384, 16, 4096, 64), (28672, 16, 4096, 64)])
+def test_blockwise_gemm_through_the_streaming_kernel(m, n, k, bs):
+    """The scale-block twin of the streaming kernel (tuna_matmul_blockwise takes it for the largest shapes at up to 16
+    tokens; the switch sends every launch it can plan there, with the per-row table's workgroup shape or four waves
+    by four): oracle on a row sample, exact read-out of the decoded weights with random scales per block (blocks
+    shorter and longer than an x chunk, workgroups that walk several row tiles), run-to-run identical."""
+    import torch
+
+    from tuna_amd import _lib, ops
+
+    rng = np.random.default_rng(m + n + k + bs + 3)
+    q, x, code, _ = make_inputs_np(m, n, k, seed=m + bs + 3)
+    absmax = rng.uniform(0.005, 0.02, size=(m, k // bs)).astype(np.float16).astype(np.float32)
+    dq, dx, dc, da = to_dev(q, x, code, absmax)
+    L = _lib.lib()
+    prev = L.tuna_set_blockwise_stream(3)
+    before = L.tuna_blockwise_launches(3)
+    try:
+        print(f"blockwise through the streaming kernel m={m} n={n} k={k} block={bs}", flush=True)
+        out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+        ops.matmul_blockwise(dx, dq, da, dc, out, m, n, k, bs)
+        torch.cuda.synchronize()
+        assert L.tuna_blockwise_launches(3) == before + 1     # that kernel ran it
+        got = out.cpu().numpy().view(np.uint16)
+        assert not np.isnan(got.view(np.float16)).any()
+        rows = np.sort(rng.choice(m, size=min(m, 160), replace=False)).astype(np.int32)
+        ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1, rows=rows, block_size=bs)
+        e = rel_err(f16_bits_to_f64(got[:, rows]), ref)
+        assert e <= REL_TOL, e
+        again = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+        ops.matmul_blockwise(dx, dq, da, dc, again, m, n, k, bs)
+        torch.cuda.synchronize()
+        assert np.array_equal(again.cpu().numpy().view(np.uint16), got)
+        img = O.dequant(q, absmax, code, m, k, mode=O.D1, block_size=bs)
+        for rep in range(2):
+            cols = rng.choice(k, size=n, replace=False)
+            xh = np.zeros((n, k), np.float16)
+            xh[np.arange(n), cols] = 1.0
+            dxh, = to_dev(xh)
+            ops.matmul_blockwise(dxh, dq, da, dc, out, m, n, k, bs)
+            torch.cuda.synchronize()
+            assert np.array_equal(out.cpu().numpy().view(np.uint16), img[:, cols].T)
+    finally:
+        L.tuna_set_blockwise_stream(prev)
+
+
 @pytest.mark.parametrize("m,n,k,bs", [(512, 64, 1024, 64), (528, 130, 2048, 128), (1024, 300, 4096, 64), (256, 1024, 512, 256),
                                       (4096, 33, 4096, 64), (272, 200, 1280, 64), (12288, 1000, 1024, 64)])
 def test_blockwise_gemm_with_many_tokens_through_the_many_token_kernel(m, n, k, bs):

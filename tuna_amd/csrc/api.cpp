@@ -819,7 +819,7 @@ static int check_ptr(const void *p, const char *name, size_t align)
 // launched problem by problem on the same stream.
 // ---------------------------------------------------------------------------------------
 static std::atomic<int> g_multi_waves_m{0}, g_multi_prefetch{0};  // 0: the library's choice (diagnostic override)
-static std::atomic<unsigned long long> g_blockwise_launches[3];  // by kernel: narrow-row, batched streaming, many-token
+static std::atomic<unsigned long long> g_blockwise_launches[4];  // by kernel: narrow-row, batched streaming, many-token, streaming
 static std::atomic<int> g_blockwise_stream{1};  // tuna_matmul_blockwise takes the batched kernel's scale-block variant where it can
 static std::atomic<int> g_multi_lds{0};  // batches with a ring of 2 stage weights and x through LDS (tuna_set_multi_weight_path)
 static std::atomic<unsigned long long> g_multi_launches{0};
@@ -1402,6 +1402,17 @@ TUNA_EXPORT int tuna_quantize_blockwise(const void *w, const void *code, void *q
     return quantize_impl(w, code, q, absmax, m, k, block_size, static_cast<hipStream_t>(stream));
 }
 
+// Shapes on which the streaming kernel's scale-block twin beats the narrow-row and the batched kernel at up to 16
+// tokens: many rows (it does not split k) and 48 to 400 MB of packed weights.  Measured with a scale per 64 weights,
+// us, twin / narrow-row / batched: 62.2 / 77.4 / 74.6 on 57344 x 8192, 21.8 / 23.4 / 25.4 on 28672 x 4096,
+// 62.8 / 73.1 / 67.3 on 32768 x 14336, but 132 / 148 / 114 on 229376 x 4096 (whose per-row entry staggers the k walk
+// of its row tiles, which the twin does not).
+static bool mid_blockwise_wins(int m, int k)
+{
+    const long long packed_bytes = (long long)m * k / 2;
+    return m >= 16384 && packed_bytes >= (48ll << 20) && packed_bytes < (400ll << 20);
+}
+
 TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n,
                                       int k, int block_size, void *stream)
 {
@@ -1470,6 +1481,47 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
     // 8192 x 8192, 30.9 / 38.7 on 28672 x 4096, 21.4 / 28.3 on 13824 x 5120, but 37.2 / 30.4 on 10240 x 8192, 29.6 / 22.7
     // on 4096 x 14336, 22.1 / 18.3 on 2560 x 10240, 134 / 106 on 32768 x 14336 and 131 / 108 on 57344 x 8192.
     const long long packed_bytes = (long long)m * k / 2;
+    // Up to 16 tokens, shapes whose per-row table entry is an unsplit launch of the streaming kernel (the large ones):
+    // that kernel's scale-block twin with the entry's workgroup shape, ring and x chunk (register ring, no stagger).
+    if (n <= 16 && (stream_mode == 3 || (stream_mode == 1 && mid_blockwise_wins(m, k)))) {
+        tuna_gemm_config c;
+        select_config(m, n, k, &c, nullptr);
+        const bool entry_fits = c.lds_tile_rows <= 0 && c.rows_per_wave == 64 && c.token_tiles == 1 && c.split_k == 1 &&
+                                c.waves_m * c.waves_k >= 8 && (c.prefetch == 2 || c.prefetch == 4);
+        for (int attempt = entry_fits ? 0 : 1; attempt < 2; ++attempt) {
+            if (attempt == 1) {  // no such entry (or it does not fit the scale buffers): four waves along the rows, four along k
+                c.rows_per_wave = 64;
+                c.waves_m = m % 256 == 0 ? 4 : m % 128 == 0 ? 2 : 1;
+                c.waves_k = 16 / c.waves_m > 8 ? 8 : 16 / c.waves_m;
+                c.split_k = 1;
+                c.prefetch = 2;
+                c.x_chunk = 512;
+                c.token_tiles = 1;
+                c.xcd_swizzle = 0;
+            }
+            c.lds_tile_rows = 0;
+            c.k_stagger = 0;
+            GemmPlan plan;
+            const int shift = log2i(block_size) - 6;
+            if (m % (64 * c.waves_m) != 0 || plan_gemm(m, n, k, c, TUNA_DECODE_GEMM, &plan) != TUNA_OK ||
+                !mid_blockwise_applies(plan, shift))
+                continue;
+            int dev = 0, cus = 0;
+            hipError_t e = device_cus(&dev, &cus);
+            if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+            plan.args.q = static_cast<const uint8_t *>(q);
+            plan.args.x = x;
+            plan.args.code = static_cast<const float *>(code);
+            plan.args.absmax = static_cast<const float *>(absmax);
+            plan.args.out = out;
+            plan.args.epilogue = TUNA_EPILOGUE_NONE;
+            plan.args.residual = nullptr;
+            e = launch_gemm_mid_blockwise(plan, shift, dev, cus, static_cast<hipStream_t>(stream));
+            if (e != hipSuccess) return hip_fail(e, "streaming blockwise gemm launch");
+            g_blockwise_launches[3].fetch_add(1, std::memory_order_relaxed);
+            return TUNA_OK;
+        }
+    }
     const bool stream_wins = n > 16  ? packed_bytes >= (100ll << 20) || (k > 8192 && packed_bytes >= (12ll << 20)) ||
                                            (k > 4096 && packed_bytes >= (40ll << 20))
                              : n > 4 ? packed_bytes >= (100ll << 20) || (n > 8 && k >= 12288 && packed_bytes >= (20ll << 20))
@@ -1819,12 +1871,12 @@ TUNA_EXPORT int tuna_time_unit_rate(int unit, void *sink, int warmup, int iters,
 
 TUNA_EXPORT unsigned long long tuna_blockwise_launches(int kernel)
 {
-    return kernel >= 0 && kernel < 3 ? g_blockwise_launches[kernel].load(std::memory_order_relaxed) : 0ull;
+    return kernel >= 0 && kernel < 4 ? g_blockwise_launches[kernel].load(std::memory_order_relaxed) : 0ull;
 }
 
 TUNA_EXPORT int tuna_set_blockwise_stream(int enabled)
 {
-    return g_blockwise_stream.exchange(enabled < 0 ? 0 : enabled > 2 ? 2 : enabled, std::memory_order_relaxed);
+    return g_blockwise_stream.exchange(enabled < 0 ? 0 : enabled > 3 ? 3 : enabled, std::memory_order_relaxed);
 }
 
 TUNA_EXPORT int tuna_set_blockwise_scales_lds(int enabled) { return set_blockwise_scales_lds(enabled); }

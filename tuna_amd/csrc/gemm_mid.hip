@@ -7,7 +7,7 @@
 namespace tuna {
 
 typedef void (*MidKernelFn)(const uint8_t *, const void *, const float *, const float *, int, int, int, int, void *,
-                            const void *, int, int, int, float *, unsigned *, int);
+                            const void *, int, int, int, float *, unsigned *, int, int);
 struct MidVariant {
     int u, tt, xb, maxt;
     MidKernelFn fn;
@@ -186,7 +186,73 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
                            : staged   ? ((chunks && v->fn_lds_shared) ? v->fn_lds_shared : v->fn_lds)
                                       : (chunks && v->fn_shared) ? v->fn_shared : v->fn;
     hipLaunchKernelGGL(fn, grid, dim3(plan.threads), lds, stream, a.q, a.x, a.code, a.absmax, a.k, a.n, a.m, packed, a.out,
-                       a.residual, walk_tiles, n_wg, chunks, a.ws, a.counters, split_log2);
+                       a.residual, walk_tiles, n_wg, chunks, a.ws, a.counters, split_log2, 0);
+    return hipGetLastError();
+}
+
+// ---- scale blocks finer than a row: the BLK twins (one token tile, register ring) ---------------------------------
+struct MidBlkVariant {
+    int u, maxt;
+    MidKernelFn fn;
+};
+static const MidBlkVariant kMidBlk[] = {
+    {2, 512, gemm_mid_kernel<2, 1, 4, 512, 2, true, false, false, true>},
+    {4, 512, gemm_mid_kernel<4, 1, 4, 512, 2, true, false, false, true>},
+    {2, 1024, gemm_mid_kernel<2, 1, 4, 1024, 4, true, false, false, true>},
+    {4, 1024, gemm_mid_kernel<4, 1, 4, 1024, 4, true, false, false, true>},
+};
+static constexpr int kNumMidBlk = sizeof(kMidBlk) / sizeof(kMidBlk[0]);
+static OptInFlag g_mid_blk_attr_done[16][kNumMidBlk];
+
+// The BLK twin for a planned launch (an unsplit, unstaggered config of one token tile the streaming kernel takes, up
+// to four scales per thread and chunk), its x chunk and LDS size; null if there is none.
+static const MidBlkVariant *mid_blk_variant(const GemmPlan &plan, int blk_shift, int *xc_out, size_t *lds_out)
+{
+    const GemmArgs &a = plan.args;
+    int xc = 0;
+    if (plan.token_tiles != 1 || a.split_k != 1 || a.k_stagger != 0 || plan.lds_weights || !mid_variant(plan, &xc)) return nullptr;
+    if (a.n > 16 || a.k % (64 << blk_shift) != 0) return nullptr;
+    const int pieces = 2 * xc;  // 16-byte x pieces per chunk (one token tile)
+    if ((pieces + plan.threads - 1) / plan.threads > 4) return nullptr;
+    const int rows_wg = a.waves_m * 64;
+    const int nbc = xc >> (6 + blk_shift) > 0 ? xc >> (6 + blk_shift) : 1;  // scale blocks per chunk
+    if ((long long)rows_wg * nbc > (plan.threads > 512 ? 2LL : 4LL) * plan.threads) return nullptr;  // scales per thread and chunk
+    const size_t x_lds = 2 * (size_t)32 * (size_t)xc, s_lds = 2 * (size_t)nbc * (size_t)(rows_wg + 4) * 4;
+    const size_t red_lds = 2 * (size_t)(plan.threads / 64) * 1024;
+    const size_t lds = (size_t)kLutBytes + (x_lds + s_lds > red_lds ? x_lds + s_lds : red_lds);
+    if (lds > (size_t)kLdsLimit) return nullptr;
+    const int maxt = plan.threads <= 512 ? 512 : 1024;
+    for (int i = 0; i < kNumMidBlk; ++i)
+        if (kMidBlk[i].u == plan.prefetch && kMidBlk[i].maxt == maxt) {
+            *xc_out = xc;
+            *lds_out = lds;
+            return &kMidBlk[i];
+        }
+    return nullptr;
+}
+
+bool mid_blockwise_applies(const GemmPlan &plan, int blk_shift)
+{
+    int xc;
+    size_t lds;
+    return mid_blk_variant(plan, blk_shift, &xc, &lds) != nullptr;
+}
+
+hipError_t launch_gemm_mid_blockwise(const GemmPlan &plan, int blk_shift, int dev, int cus, hipStream_t stream)
+{
+    int xc = 0;
+    size_t lds = 0;
+    const MidBlkVariant *v = mid_blk_variant(plan, blk_shift, &xc, &lds);
+    if (!v) return hipErrorInvalidConfiguration;
+    hipError_t e = ensure_lds_opt_in(g_mid_blk_attr_done[dev][(int)(v - kMidBlk)], reinterpret_cast<const void *>(v->fn));
+    if (e != hipSuccess) return e;
+    const GemmArgs &a = plan.args;
+    int xc_log2 = 0;
+    while ((1 << xc_log2) < xc) ++xc_log2;
+    const int n_wg = a.row_tiles < cus ? a.row_tiles : cus;  // one workgroup per CU, walking row tiles
+    const int packed = a.waves_m | a.epilogue << 5 | xc_log2 << 8 | a.wk_log2 << 13;
+    hipLaunchKernelGGL(v->fn, dim3((unsigned)n_wg, 1, 1), dim3(plan.threads), lds, stream, a.q, a.x, a.code, a.absmax, a.k, a.n, a.m,
+                       packed, a.out, a.residual, a.row_tiles, n_wg, 0, nullptr, nullptr, 0, blk_shift);
     return hipGetLastError();
 }
 

@@ -73,13 +73,18 @@ __device__ __forceinline__ void barrier_lds_only()
 // NT: weight loads carry the nontemporal hint (each byte is used once per launch).  Launches whose
 // token chunks share the weights through the caches (a_chunks != 0) run the twin without it.
 // SPLIT: the twin for launches with k split across workgroups (the unsplit kernels carry none of its code).
-template <int U, int TT, int XB, int MAXT, int MINW, bool NT = true, bool LDSW = false, bool SPLIT = false>
+// BLK: one scale per block of 64 << a_blk_shift weights of a row (absmax [m, k / block]) instead of one per row:
+// beside every x chunk the scales of the workgroup's rows for the chunk's blocks are staged in LDS (rounded to
+// fp16, twice in a dword, as [block of the chunk][row]; two buffers, switched with the x buffers), and a lane reads
+// its four rows' scales of a k-step's block with one 16-byte LDS read.  Register ring, no stagger, no split.
+template <int U, int TT, int XB, int MAXT, int MINW, bool NT = true, bool LDSW = false, bool SPLIT = false, bool BLK = false>
 __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q, const void *a_x, const float *a_code,
                                                               const float *a_absmax, int a_k, int a_n, int a_m, int a_packed,
                                                               void *a_out, const void *a_residual, int a_row_tiles,
                                                               int a_n_wg, int a_chunks, float *a_ws, unsigned *a_counters,
-                                                              int a_split_log2)
+                                                              int a_split_log2, int a_blk_shift)
 {
+    static_assert(!BLK || (!LDSW && !SPLIT), "scale blocks: register ring, unsplit");
     // a_packed = waves_m | epilogue << 5 | log2(x chunk in k) << 8 | log2(waves_k) << 13 | k_stagger << 16
     const int waves_m = a_packed & 31;
     const int epilogue = (a_packed >> 5) & 7;
@@ -151,6 +156,37 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
             x_inchunk |= in ? 1u << b : 0u;
             x_real |= (in && tok0 + row < a_n) ? 1u << b : 0u;
         }
+    }
+    // BLK: scale s = tid + i * nthreads (i < SB) of a chunk is row s >> nbc_log2 of the workgroup's, block
+    // s & (nbc - 1) of the chunk's nbc (consecutive lanes read consecutive blocks of a row); stored at
+    // [block][row] with rows padded by 4 so that the lanes of a store hit different banks
+    constexpr int SB = MAXT > 512 ? 2 : 4;  // (the 1024-thread twins have 128 registers per lane)
+    const int blk_log2 = BLK ? 6 + a_blk_shift : 0;                       // log2(weights per scale)
+    const int nbc_log2 = BLK ? max(xc_log2 - blk_log2, 0) : 0;          // log2(blocks per chunk)
+    const int s_pitch = waves_m * 64 + 4;                               // dwords between the blocks of a buffer
+    const int s_count = BLK ? (waves_m * 64) << nbc_log2 : 0;           // scales per chunk
+    const uint32_t sbuf_bytes = BLK ? ((uint32_t)s_pitch << nbc_log2) * 4u : 0u;
+    unsigned char *sbuf = xbuf + 2 * xbuf_bytes;                        // two scale buffers behind the x buffers
+    float sv[BLK ? SB : 1];
+    const int nblk = BLK ? a_k >> blk_log2 : 1;                         // scales per row
+#define TUNA_MID_S_LOAD(row0_wg, kbase)                                                          \
+    if constexpr (BLK) {                                                                       \
+        const float *sp_ = a_absmax + (size_t)(row0_wg) * (size_t)nblk + ((kbase) >> blk_log2); \
+        _Pragma("unroll") for (int i = 0; i < SB; ++i)                                         \
+        {                                                                                      \
+            const int s_ = min(tid + i * nthreads, s_count - 1);                               \
+            sv[i] = sp_[(size_t)(s_ >> nbc_log2) * (size_t)nblk + (s_ & ((1 << nbc_log2) - 1))]; \
+        }                                                                                      \
+    }
+#define TUNA_MID_S_STORE(buf)                                                                   \
+    if constexpr (BLK) {                                                                       \
+        _Pragma("unroll") for (int i = 0; i < SB; ++i)                                         \
+        {                                                                                      \
+            const int s_ = tid + i * nthreads;                                                 \
+            const uint32_t h_ = (uint32_t)f16_bits((f16)sv[i]);                                \
+            if (s_ < s_count)                                                                  \
+                reinterpret_cast<uint32_t *>(buf)[(s_ & ((1 << nbc_log2) - 1)) * s_pitch + (s_ >> nbc_log2)] = h_ | (h_ << 16); \
+        }                                                                                      \
     }
     const unsigned char *x_tile = reinterpret_cast<const unsigned char *>(a_x) + (size_t)tok0 * a_k * 2;
     // Chunk at logical k `kbase` of a tile whose walk starts rot_k elements into the k range and
@@ -228,7 +264,9 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
         /* x and the scales first: vector loads return in order, and the tile's first barrier */ \
         /* waits for the x pieces only - the first ring turn stays in flight across it */        \
         if constexpr (!LDSW) TUNA_MID_X_LOAD(0, rot << 5, ps << 5)                             \
-        if constexpr (!LDSW) {                                                                 \
+        if constexpr (BLK) {                                                                   \
+            TUNA_MID_S_LOAD(((t) >> split_log2) * (waves_m * 64), 0)                           \
+        } else if constexpr (!LDSW) {                                                          \
             _Pragma("unroll") for (int j = 0; j < 4; ++j) sc32[j] = a_absmax[row0_ + i16 * 4 + j]; \
         }                                                                                      \
         _Pragma("unroll") for (int u = 0; u < U; ++u)                                          \
@@ -312,6 +350,16 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
             f16x8 b_[TT];                                                                      \
             _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) b_[tt] =                         \
                 *reinterpret_cast<const f16x8 *>(xb + (size_t)((sl) + u) * wstep + tt * xb_tile); \
+            if constexpr (BLK) {                                                               \
+                /* the block of this wave's k-step (sl + u) of the chunk, counted from the chunk's first */ \
+                const int rel_ = min(((((sl) + u) << wk_log2) + wk) >> (blk_log2 - 5), (1 << nbc_log2) - 1); \
+                const u32x4 s4_ = *reinterpret_cast<const u32x4 *>(sb_lane + (size_t)rel_ * (size_t)(s_pitch * 4)); \
+                _Pragma("unroll") for (int j = 0; j < 4; ++j)                                  \
+                {                                                                              \
+                    const uint32_t e_ = s4_[j]; /* (a copy: bit_cast of a vector element reads element 0) */ \
+                    sc16[j] = __builtin_bit_cast(f16x2, e_);                                   \
+                }                                                                              \
+            }                                                                                  \
             _Pragma("unroll") for (int j = 0; j < 4; ++j)                                      \
             {                                                                                  \
                 const f16x8 av_ = decode_dword<TUNA_DECODE_GEMM>(wq[u][j], lut, lane4, sc16[j], 0.f); \
@@ -362,6 +410,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
             barrier_lds_only();  // (every wave has waited for its pieces of chunk 0 and read its scales)
         } else {
             TUNA_MID_X_STORE(xbuf)
+            TUNA_MID_S_STORE(sbuf)
             // (threads without a piece to store have not waited for theirs, see gemm_kernel.hpp; the U
             // weight loads of the ring are younger than every x piece and may stay in flight)
             __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));
@@ -381,8 +430,11 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
                 TUNA_MID_X_DMA(xbuf + ((c + 1) & 1) * xbuf_bytes, min(c + 1, n_chunks - 1) << xc_log2, cur_rot, cur_ps)
             } else {
                 TUNA_MID_X_LOAD(min(c + 1, n_chunks - 1) << xc_log2, cur_rot << 5, cur_ps << 5)
+                TUNA_MID_S_LOAD(row0 - wm * 64, min(c + 1, n_chunks - 1) << xc_log2)
             }
             const unsigned char *xb = xbuf + (c & 1) * xbuf_bytes + xb_lane;
+            // BLK: this lane's four rows in the chunk's scale buffer
+            [[maybe_unused]] const unsigned char *sb_lane = sbuf + (c & 1) * sbuf_bytes + (size_t)(wm * 64 + i16 * 4) * 4;
             // (the first ring turn of a chunk is a copy of its own: there the x pieces just
             // requested are in flight behind the ring, and only straight-line code lets the
             // compiler count them into its waits instead of waiting them out)
@@ -396,6 +448,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
                     // the other buffer was last read in chunk c - 1, which ended with a barrier
                     __builtin_amdgcn_s_waitcnt(wait_vmcnt(U));  // exactly the last ring turn's refills are younger
                     TUNA_MID_X_STORE(xbuf + ((c + 1) & 1) * xbuf_bytes)
+                    TUNA_MID_S_STORE(sbuf + ((c + 1) & 1) * sbuf_bytes)
                 }
                 __syncthreads();
             }
@@ -513,6 +566,8 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     }
 #undef TUNA_MID_GROUP
 #undef TUNA_MID_X_LOAD
+#undef TUNA_MID_S_LOAD
+#undef TUNA_MID_S_STORE
 #undef TUNA_MID_X_STORE
 #undef TUNA_MID_X_DMA
 #undef TUNA_MID_TOP_DMA

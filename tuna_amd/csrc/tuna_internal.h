@@ -165,7 +165,11 @@ struct GemmPlan {
 hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream);
 // 17..128-token streaming twin of the general kernel (gemm_mid.hpp) for the launches it applies to.
 bool mid_applies(const GemmPlan &plan);
-bool mid_lds_applies(const GemmPlan &plan);  // ... with the packed weights staged through LDS
+bool mid_lds_applies(const GemmPlan &plan);
+// The streaming kernel's twins for scale blocks finer than a row (64 << blk_shift weights per scale): whether one takes
+// the planned launch (one token tile, unsplit, no stagger), and the launch.
+bool mid_blockwise_applies(const GemmPlan &plan, int blk_shift);
+hipError_t launch_gemm_mid_blockwise(const GemmPlan &plan, int blk_shift, int dev, int cus, hipStream_t stream);  // ... with the packed weights staged through LDS
 hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t stream);
 bool mid_describe(const GemmPlan &plan, char *buf, size_t len);
 // Name and template arguments of the kernel launch_gemm would start for `plan` on a device of `cus` CUs.
