@@ -1405,8 +1405,8 @@ TUNA_EXPORT int tuna_quantize_blockwise(const void *w, const void *code, void *q
 // Shapes on which the streaming kernel's scale-block twin beats the narrow-row and the batched kernel at up to 16
 // tokens: many rows (it does not split k) and 48 to 400 MB of packed weights.  Measured with a scale per 64 weights,
 // us, twin / narrow-row / batched: 62.2 / 77.4 / 74.6 on 57344 x 8192, 21.8 / 23.4 / 25.4 on 28672 x 4096,
-// 62.8 / 73.1 / 67.3 on 32768 x 14336, but 132 / 148 / 114 on 229376 x 4096 (whose per-row entry staggers the k walk
-// of its row tiles, which the twin does not).
+// 62.8 / 73.1 / 67.3 on 32768 x 14336, but 132 / 148 / 114 on 229376 x 4096 (whose per-row entry - 16 waves along the
+// rows, chunks of 2048 k - has more scales per thread and chunk than the twin stages).
 static bool mid_blockwise_wins(int m, int k)
 {
     const long long packed_bytes = (long long)m * k / 2;
@@ -1482,7 +1482,7 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
     // on 4096 x 14336, 22.1 / 18.3 on 2560 x 10240, 134 / 106 on 32768 x 14336 and 131 / 108 on 57344 x 8192.
     const long long packed_bytes = (long long)m * k / 2;
     // Up to 16 tokens, shapes whose per-row table entry is an unsplit launch of the streaming kernel (the large ones):
-    // that kernel's scale-block twin with the entry's workgroup shape, ring and x chunk (register ring, no stagger).
+    // that kernel's scale-block twin with the entry's workgroup shape, ring, x chunk and stagger (in whole x chunks; register ring).
     if (n <= 16 && (stream_mode == 3 || (stream_mode == 1 && mid_blockwise_wins(m, k)))) {
         tuna_gemm_config c;
         select_config(m, n, k, &c, nullptr);
@@ -1500,7 +1500,7 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
                 c.xcd_swizzle = 0;
             }
             c.lds_tile_rows = 0;
-            c.k_stagger = 0;
+            if (attempt == 1) c.k_stagger = 0;
             GemmPlan plan;
             const int shift = log2i(block_size) - 6;
             if (m % (64 * c.waves_m) != 0 || plan_gemm(m, n, k, c, TUNA_DECODE_GEMM, &plan) != TUNA_OK ||

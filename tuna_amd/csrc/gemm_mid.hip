@@ -204,13 +204,13 @@ static const MidBlkVariant kMidBlk[] = {
 static constexpr int kNumMidBlk = sizeof(kMidBlk) / sizeof(kMidBlk[0]);
 static OptInFlag g_mid_blk_attr_done[16][kNumMidBlk];
 
-// The BLK twin for a planned launch (an unsplit, unstaggered config of one token tile the streaming kernel takes, up
-// to four scales per thread and chunk), its x chunk and LDS size; null if there is none.
+// The BLK twin for a planned launch (an unsplit config of one token tile the streaming kernel takes, up to four - 1024
+// threads: two - scales per thread and chunk), its x chunk and LDS size; null if there is none.
 static const MidBlkVariant *mid_blk_variant(const GemmPlan &plan, int blk_shift, int *xc_out, size_t *lds_out)
 {
     const GemmArgs &a = plan.args;
     int xc = 0;
-    if (plan.token_tiles != 1 || a.split_k != 1 || a.k_stagger != 0 || plan.lds_weights || !mid_variant(plan, &xc)) return nullptr;
+    if (plan.token_tiles != 1 || a.split_k != 1 || plan.lds_weights || !mid_variant(plan, &xc)) return nullptr;
     if (a.n > 16 || a.k % (64 << blk_shift) != 0) return nullptr;
     const int pieces = 2 * xc;  // 16-byte x pieces per chunk (one token tile)
     if ((pieces + plan.threads - 1) / plan.threads > 4) return nullptr;
@@ -250,7 +250,7 @@ hipError_t launch_gemm_mid_blockwise(const GemmPlan &plan, int blk_shift, int de
     int xc_log2 = 0;
     while ((1 << xc_log2) < xc) ++xc_log2;
     const int n_wg = a.row_tiles < cus ? a.row_tiles : cus;  // one workgroup per CU, walking row tiles
-    const int packed = a.waves_m | a.epilogue << 5 | xc_log2 << 8 | a.wk_log2 << 13;
+    const int packed = a.waves_m | a.epilogue << 5 | xc_log2 << 8 | a.wk_log2 << 13 | a.k_stagger << 16;
     hipLaunchKernelGGL(v->fn, dim3((unsigned)n_wg, 1, 1), dim3(plan.threads), lds, stream, a.q, a.x, a.code, a.absmax, a.k, a.n, a.m,
                        packed, a.out, a.residual, a.row_tiles, n_wg, 0, nullptr, nullptr, 0, blk_shift);
     return hipGetLastError();

@@ -76,7 +76,8 @@ __device__ __forceinline__ void barrier_lds_only()
 // BLK: one scale per block of 64 << a_blk_shift weights of a row (absmax [m, k / block]) instead of one per row:
 // beside every x chunk the scales of the workgroup's rows for the chunk's blocks are staged in LDS (rounded to
 // fp16, twice in a dword, as [block of the chunk][row]; two buffers, switched with the x buffers), and a lane reads
-// its four rows' scales of a k-step's block with one 16-byte LDS read.  Register ring, no stagger, no split.
+// its four rows' scales of a k-step's block with one 16-byte LDS read.  Register ring, no split; the stagger of a
+// row tile's k walk is t * k_stagger whole x chunks.
 template <int U, int TT, int XB, int MAXT, int MINW, bool NT = true, bool LDSW = false, bool SPLIT = false, bool BLK = false>
 __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q, const void *a_x, const float *a_code,
                                                               const float *a_absmax, int a_k, int a_n, int a_m, int a_packed,
@@ -169,9 +170,12 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
     unsigned char *sbuf = xbuf + 2 * xbuf_bytes;                        // two scale buffers behind the x buffers
     float sv[BLK ? SB : 1];
     const int nblk = BLK ? a_k >> blk_log2 : 1;                         // scales per row
-#define TUNA_MID_S_LOAD(row0_wg, kbase)                                                          \
+    /* (kbase: the chunk's logical k; rot_k: the tile's stagger, whole chunks here, so a chunk never wraps inside) */ \
+#define TUNA_MID_S_LOAD(row0_wg, kbase, rot_k)                                                   \
     if constexpr (BLK) {                                                                       \
-        const float *sp_ = a_absmax + (size_t)(row0_wg) * (size_t)nblk + ((kbase) >> blk_log2); \
+        int kp_ = (kbase) + (rot_k);                                                           \
+        if (kp_ >= a_k) kp_ -= a_k;                                                            \
+        const float *sp_ = a_absmax + (size_t)(row0_wg) * (size_t)nblk + (kp_ >> blk_log2);    \
         _Pragma("unroll") for (int i = 0; i < SB; ++i)                                         \
         {                                                                                      \
             const int s_ = min(tid + i * nthreads, s_count - 1);                               \
@@ -260,12 +264,14 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
         ps = ((t) & ((1 << split_log2) - 1)) * n_steps;                                        \
         /* stagger: row tile t walks k starting rot steps in, wrapping around (gemm_kernel.hpp) */ \
         rot = (k_stagger && n_steps > 1) ? (int)(((unsigned)(t) * k_stagger) % (unsigned)n_steps) : 0; \
+        /* BLK: whole chunks, so that a chunk's scale blocks are contiguous */                 \
+        if constexpr (BLK) rot = (k_stagger && n_chunks > 1) ? (int)(((unsigned)(t) * k_stagger) % (unsigned)n_chunks) << (xc_log2 - 5) : 0; \
         lb = ((uint32_t)(row0_ >> 3) + (uint32_t)(i16 >> 1)) * kb_total * 32u + (uint32_t)(i16 & 1) * 16u + (uint32_t)g * 32u; \
         /* x and the scales first: vector loads return in order, and the tile's first barrier */ \
         /* waits for the x pieces only - the first ring turn stays in flight across it */        \
         if constexpr (!LDSW) TUNA_MID_X_LOAD(0, rot << 5, ps << 5)                             \
         if constexpr (BLK) {                                                                   \
-            TUNA_MID_S_LOAD(((t) >> split_log2) * (waves_m * 64), 0)                           \
+            TUNA_MID_S_LOAD(((t) >> split_log2) * (waves_m * 64), 0, rot << 5)                 \
         } else if constexpr (!LDSW) {                                                          \
             _Pragma("unroll") for (int j = 0; j < 4; ++j) sc32[j] = a_absmax[row0_ + i16 * 4 + j]; \
         }                                                                                      \
@@ -430,7 +436,7 @@ __global__ __launch_bounds__(MAXT, MINW) void gemm_mid_kernel(const uint8_t *a_q
                 TUNA_MID_X_DMA(xbuf + ((c + 1) & 1) * xbuf_bytes, min(c + 1, n_chunks - 1) << xc_log2, cur_rot, cur_ps)
             } else {
                 TUNA_MID_X_LOAD(min(c + 1, n_chunks - 1) << xc_log2, cur_rot << 5, cur_ps << 5)
-                TUNA_MID_S_LOAD(row0 - wm * 64, min(c + 1, n_chunks - 1) << xc_log2)
+                TUNA_MID_S_LOAD(row0 - wm * 64, min(c + 1, n_chunks - 1) << xc_log2, cur_rot << 5)
             }
             const unsigned char *xb = xbuf + (c & 1) * xbuf_bytes + xb_lane;
             // BLK: this lane's four rows in the chunk's scale buffer
