@@ -1404,8 +1404,8 @@ TUNA_EXPORT int tuna_quantize_blockwise(const void *w, const void *code, void *q
 
 // Shapes on which the streaming kernel's scale-block twin beats the narrow-row and the batched kernel at up to 16
 // tokens: many rows (it does not split k) and 48 to 400 MB of packed weights.  Measured with a scale per 64 weights,
-// us, twin / narrow-row / batched: 62.2 / 77.4 / 74.6 on 57344 x 8192, 21.8 / 23.4 / 25.4 on 28672 x 4096,
-// 62.8 / 73.1 / 67.3 on 32768 x 14336, but 132 / 148 / 114 on 229376 x 4096 (whose per-row entry - 16 waves along the
+// us, twin / narrow-row / batched: 62-64 / 77 / 68-69 on 57344 x 8192, 21.5-22.2 / 23.3 / 24.6 on 28672 x 4096,
+// 64-65 / 71 / 64 on 32768 x 14336, but 132 / 148 / 114 on 229376 x 4096 (whose per-row entry - 16 waves along the
 // rows, chunks of 2048 k - has more scales per thread and chunk than the twin stages).
 static bool mid_blockwise_wins(int m, int k)
 {
