@@ -1402,15 +1402,17 @@ TUNA_EXPORT int tuna_quantize_blockwise(const void *w, const void *code, void *q
     return quantize_impl(w, code, q, absmax, m, k, block_size, static_cast<hipStream_t>(stream));
 }
 
-// Shapes on which the streaming kernel's scale-block twin beats the narrow-row and the batched kernel at up to 16
-// tokens: many rows (it does not split k) and 48 to 400 MB of packed weights.  Measured with a scale per 64 weights,
-// us, twin / narrow-row / batched: 62-64 / 77 / 68-69 on 57344 x 8192, 21.5-22.2 / 23.3 / 24.6 on 28672 x 4096,
-// 64-65 / 71 / 64 on 32768 x 14336, but 132 / 148 / 114 on 229376 x 4096 (whose per-row entry - 16 waves along the
-// rows, chunks of 2048 k - has more scales per thread and chunk than the twin stages).
-static bool mid_blockwise_wins(int m, int k)
+// Shapes on which the streaming kernel's scale-block twin beats the narrow-row and the batched kernel at up to 32
+// tokens: many rows (it does not split k) and at least 48 MB of packed weights; up to 16 tokens less than 400 MB.
+// Measured with a scale per 64 weights, us, twin / narrow-row / batched.  16 tokens: 62-64 / 77 / 68-69 on
+// 57344 x 8192, 21.5-22.2 / 23.3 / 24.6 on 28672 x 4096, 64-65 / 71 / 64 on 32768 x 14336, but 132 / 148 / 114 on
+// 229376 x 4096 (whose per-row entry - 16 waves along the rows, chunks of 2048 k - has more scales per thread and
+// chunk than the twin stages).  32 tokens (two token tiles: one pass over the weights, where the batched kernel makes
+// two): 80 / 131 / 117, 30.7 / 31.5 / 40.6, 78 / 134 / 112 and 169 / 205 / 210.
+static bool mid_blockwise_wins(int m, int n, int k)
 {
     const long long packed_bytes = (long long)m * k / 2;
-    return m >= 16384 && packed_bytes >= (48ll << 20) && packed_bytes < (400ll << 20);
+    return m >= 16384 && packed_bytes >= (48ll << 20) && (n > 16 || packed_bytes < (400ll << 20));
 }
 
 TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n,
@@ -1481,12 +1483,13 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
     // 8192 x 8192, 30.9 / 38.7 on 28672 x 4096, 21.4 / 28.3 on 13824 x 5120, but 37.2 / 30.4 on 10240 x 8192, 29.6 / 22.7
     // on 4096 x 14336, 22.1 / 18.3 on 2560 x 10240, 134 / 106 on 32768 x 14336 and 131 / 108 on 57344 x 8192.
     const long long packed_bytes = (long long)m * k / 2;
-    // Up to 16 tokens, shapes whose per-row table entry is an unsplit launch of the streaming kernel (the large ones):
+    // Up to 32 tokens, shapes whose per-row table entry is an unsplit launch of the streaming kernel (the large ones):
     // that kernel's scale-block twin with the entry's workgroup shape, ring, x chunk and stagger (in whole x chunks; register ring).
-    if (n <= 16 && (stream_mode == 3 || (stream_mode == 1 && mid_blockwise_wins(m, k)))) {
+    if (n <= 32 && (stream_mode == 3 || (stream_mode == 1 && mid_blockwise_wins(m, n, k)))) {
         tuna_gemm_config c;
         select_config(m, n, k, &c, nullptr);
-        const bool entry_fits = c.lds_tile_rows <= 0 && c.rows_per_wave == 64 && c.token_tiles == 1 && c.split_k == 1 &&
+        const int tiles = n > 16 ? 2 : 1;  // token tiles: one pass over the weights
+        const bool entry_fits = c.lds_tile_rows <= 0 && c.rows_per_wave == 64 && c.token_tiles == tiles && c.split_k == 1 &&
                                 c.waves_m * c.waves_k >= 8 && (c.prefetch == 2 || c.prefetch == 4);
         for (int attempt = entry_fits ? 0 : 1; attempt < 2; ++attempt) {
             if (attempt == 1) {  // no such entry (or it does not fit the scale buffers): four waves along the rows, four along k
@@ -1496,7 +1499,7 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
                 c.split_k = 1;
                 c.prefetch = 2;
                 c.x_chunk = 512;
-                c.token_tiles = 1;
+                c.token_tiles = tiles;
                 c.xcd_swizzle = 0;
             }
             c.lds_tile_rows = 0;

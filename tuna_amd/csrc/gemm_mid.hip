@@ -190,40 +190,45 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
     return hipGetLastError();
 }
 
-// ---- scale blocks finer than a row: the BLK twins (one token tile, register ring) ---------------------------------
+// ---- scale blocks finer than a row: the BLK twins (one or two token tiles, register ring) -------------------------
 struct MidBlkVariant {
-    int u, maxt;
+    int u, tt, maxt;
     MidKernelFn fn;
 };
 static const MidBlkVariant kMidBlk[] = {
-    {2, 512, gemm_mid_kernel<2, 1, 4, 512, 2, true, false, false, true>},
-    {4, 512, gemm_mid_kernel<4, 1, 4, 512, 2, true, false, false, true>},
-    {2, 1024, gemm_mid_kernel<2, 1, 4, 1024, 4, true, false, false, true>},
-    {4, 1024, gemm_mid_kernel<4, 1, 4, 1024, 4, true, false, false, true>},
+    {2, 1, 512, gemm_mid_kernel<2, 1, 4, 512, 2, true, false, false, true>},
+    {4, 1, 512, gemm_mid_kernel<4, 1, 4, 512, 2, true, false, false, true>},
+    {2, 1, 1024, gemm_mid_kernel<2, 1, 4, 1024, 4, true, false, false, true>},
+    {4, 1, 1024, gemm_mid_kernel<4, 1, 4, 1024, 4, true, false, false, true>},
+    {2, 2, 512, gemm_mid_kernel<2, 2, 4, 512, 2, true, false, false, true>},
+    {4, 2, 512, gemm_mid_kernel<4, 2, 4, 512, 2, true, false, false, true>},
+    {2, 2, 1024, gemm_mid_kernel<2, 2, 4, 1024, 4, true, false, false, true>},
+    {4, 2, 1024, gemm_mid_kernel<4, 2, 4, 1024, 4, true, false, false, true>},
 };
 static constexpr int kNumMidBlk = sizeof(kMidBlk) / sizeof(kMidBlk[0]);
 static OptInFlag g_mid_blk_attr_done[16][kNumMidBlk];
 
-// The BLK twin for a planned launch (an unsplit config of one token tile the streaming kernel takes, up to four - 1024
+// The BLK twin for a planned launch (an unsplit config of one or two token tiles the streaming kernel takes, up to four - 1024
 // threads: two - scales per thread and chunk), its x chunk and LDS size; null if there is none.
 static const MidBlkVariant *mid_blk_variant(const GemmPlan &plan, int blk_shift, int *xc_out, size_t *lds_out)
 {
     const GemmArgs &a = plan.args;
     int xc = 0;
-    if (plan.token_tiles != 1 || a.split_k != 1 || plan.lds_weights || !mid_variant(plan, &xc)) return nullptr;
-    if (a.n > 16 || a.k % (64 << blk_shift) != 0) return nullptr;
-    const int pieces = 2 * xc;  // 16-byte x pieces per chunk (one token tile)
+    if ((plan.token_tiles != 1 && plan.token_tiles != 2) || a.split_k != 1 || plan.lds_weights || !mid_variant(plan, &xc))
+        return nullptr;
+    if (a.n > 16 * plan.token_tiles || a.k % (64 << blk_shift) != 0) return nullptr;  // (one pass over the weights)
+    const int pieces = plan.token_tiles * 2 * xc;  // 16-byte x pieces per chunk
     if ((pieces + plan.threads - 1) / plan.threads > 4) return nullptr;
     const int rows_wg = a.waves_m * 64;
     const int nbc = xc >> (6 + blk_shift) > 0 ? xc >> (6 + blk_shift) : 1;  // scale blocks per chunk
     if ((long long)rows_wg * nbc > (plan.threads > 512 ? 2LL : 4LL) * plan.threads) return nullptr;  // scales per thread and chunk
-    const size_t x_lds = 2 * (size_t)32 * (size_t)xc, s_lds = 2 * (size_t)nbc * (size_t)(rows_wg + 4) * 4;
+    const size_t x_lds = 2 * (size_t)plan.token_tiles * 32 * (size_t)xc, s_lds = 2 * (size_t)nbc * (size_t)(rows_wg + 4) * 4;
     const size_t red_lds = 2 * (size_t)(plan.threads / 64) * 1024;
     const size_t lds = (size_t)kLutBytes + (x_lds + s_lds > red_lds ? x_lds + s_lds : red_lds);
     if (lds > (size_t)kLdsLimit) return nullptr;
     const int maxt = plan.threads <= 512 ? 512 : 1024;
     for (int i = 0; i < kNumMidBlk; ++i)
-        if (kMidBlk[i].u == plan.prefetch && kMidBlk[i].maxt == maxt) {
+        if (kMidBlk[i].u == plan.prefetch && kMidBlk[i].tt == plan.token_tiles && kMidBlk[i].maxt == maxt) {
             *xc_out = xc;
             *lds_out = lds;
             return &kMidBlk[i];
