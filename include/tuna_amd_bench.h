@@ -100,10 +100,10 @@ int tuna_set_multi_weight_path(int through_lds);
  * many-token kernel's scale-block variants, and large launches whose shape allows (m a multiple of 64, k of 256 and of
  * the block; 17 to 32 tokens from 100 MB of packed weights, from 40 MB when k > 4096 and from 12 MB when k > 8192, 9 to 16 tokens from 100 MB or from 20 MB when k >= 12288,
  * 5 to 8 tokens from 100 MB, 1 to 4 tokens from 256 MB) through the scale-block variant of the batched streaming kernel
- * (a batch of one up to 16 tokens, the token chunks as a batch beyond), and launches of up to 32 tokens on shapes of at
- * least 16384 rows and 48 MB of packed weights (up to 16 tokens: less than 400 MB) through the streaming kernel's
- * scale-block twin; 2: the batched streaming kernel for every launch it can plan, whatever its size and token count;
- * 3: the streaming kernel's twin for every launch of up to 32 tokens it can plan; 0: always the narrow-row kernel's variants.  All decode fp16(code) * fp16(absmax of
+ * (a batch of one up to 16 tokens, the token chunks as a batch beyond), and, ahead of both, launches of up to 64 tokens
+ * on shapes of at least 16384 rows and 48 MB of packed weights (up to 16 tokens: less than 400 MB; from 33: at least
+ * 100 MB) through the streaming kernel's scale-block twin; 2: the batched streaming kernel for every launch it can plan,
+ * whatever its size and token count; 3: the streaming kernel's twin for every launch of up to 64 tokens it can plan; 0: always the narrow-row kernel's variants.  All decode fp16(code) * fp16(absmax of
  * the block); the sums differ in summation order only.  Returns the previous setting. */
 int tuna_set_blockwise_stream(int enabled);
 /* Diagnostic: tuna_matmul_blockwise calls so far in this process that ran the narrow-row kernel (kernel 0), launches of

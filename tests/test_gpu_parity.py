@@ -1848,10 +1848,11 @@ def test_blockwise_gemm_through_the_batched_streaming_kernel(m, n, k, bs):
 @pytest.mark.parametrize("m,n,k,bs", [(256, 16, 1024, 64), (512, 7, 2048, 64), (1024, 16, 4096, 128), (2048, 1, 8192, 64),
                                       (256 * 70, 16, 1024, 64), (768, 13, 5120, 64), (512, 16, 8192, 4096), (1024, 16, 2048, 1024),
                                       (4096, 16, 4096, 64), (16384, 16, 4096, 64), (28672, 16, 4096, 64),
-                                      (512, 32, 2048, 64), (1024, 23, 4096, 128), (256 * 70, 17, 1024, 64), (28672, 32, 4096, 64)])
+                                      (512, 32, 2048, 64), (1024, 23, 4096, 128), (256 * 70, 17, 1024, 64), (28672, 32, 4096, 64),
+                                      (512, 64, 2048, 64), (1024, 40, 4096, 128), (256 * 70, 33, 1024, 64), (28672, 64, 4096, 64)])
 def test_blockwise_gemm_through_the_streaming_kernel(m, n, k, bs):
-    """The scale-block twin of the streaming kernel (tuna_matmul_blockwise takes it for the largest shapes at up to 32
-    tokens, two token tiles from 17; the switch sends every launch it can plan there, with the per-row table's workgroup shape or four waves
+    """The scale-block twin of the streaming kernel (tuna_matmul_blockwise takes it for the largest shapes at up to 64
+    tokens, two token tiles from 17 and four from 33; the switch sends every launch it can plan there, with the per-row table's workgroup shape or four waves
     by four): oracle on a row sample, exact read-out of the decoded weights with random scales per block (blocks
     shorter and longer than an x chunk, workgroups that walk several row tiles), run-to-run identical."""
     import torch

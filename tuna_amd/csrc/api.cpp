@@ -1402,16 +1402,19 @@ TUNA_EXPORT int tuna_quantize_blockwise(const void *w, const void *code, void *q
     return quantize_impl(w, code, q, absmax, m, k, block_size, static_cast<hipStream_t>(stream));
 }
 
-// Shapes on which the streaming kernel's scale-block twin beats the narrow-row and the batched kernel at up to 32
-// tokens: many rows (it does not split k) and at least 48 MB of packed weights; up to 16 tokens less than 400 MB.
+// Shapes on which the streaming kernel's scale-block twin beats the narrow-row, the batched and the many-token kernel
+// at up to 64 tokens: many rows (it does not split k) and at least 48 MB of packed weights (up to 16 tokens: less than
+// 400 MB; from 33 tokens: at least 100 MB).
 // Measured with a scale per 64 weights, us, twin / narrow-row / batched.  16 tokens: 62-64 / 77 / 68-69 on
 // 57344 x 8192, 21.5-22.2 / 23.3 / 24.6 on 28672 x 4096, 64-65 / 71 / 64 on 32768 x 14336, but 132 / 148 / 114 on
 // 229376 x 4096 (whose per-row entry - 16 waves along the rows, chunks of 2048 k - has more scales per thread and
 // chunk than the twin stages).  32 tokens (two token tiles: one pass over the weights, where the batched kernel makes
-// two): 80 / 131 / 117, 30.7 / 31.5 / 40.6, 78 / 134 / 112 and 169 / 205 / 210.
+// two): 80 / 131 / 117, 30.7 / 31.5 / 40.6, 78 / 134 / 112 and 169 / 205 / 210.  64 tokens (four token tiles), twin /
+// many-token kernel: 103 / 130, 49.9 / 47.5, 111 / 125 and 182 / 252: from 100 MB there.
 static bool mid_blockwise_wins(int m, int n, int k)
 {
     const long long packed_bytes = (long long)m * k / 2;
+    if (n > 32) return m >= 16384 && packed_bytes >= (100ll << 20);
     return m >= 16384 && packed_bytes >= (48ll << 20) && (n > 16 || packed_bytes < (400ll << 20));
 }
 
@@ -1432,10 +1435,52 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
     if ((rc = check_ptr(q, "q", 16)) || (rc = check_ptr(x, "x", 16)) || (rc = check_ptr(code, "code", 4)) ||
         (rc = check_ptr(absmax, "absmax", 4)) || (rc = check_ptr(out, "out", 16)))
         return rc;
+    const int stream_mode = g_blockwise_stream.load(std::memory_order_relaxed);
+    // Up to 64 tokens, shapes whose per-row table entry is an unsplit launch of the streaming kernel (the large ones):
+    // that kernel's scale-block twin with the entry's workgroup shape, ring, x chunk and stagger (in whole x chunks; register ring).
+    if (n <= 64 && (stream_mode == 3 || (stream_mode == 1 && mid_blockwise_wins(m, n, k)))) {
+        tuna_gemm_config c;
+        select_config(m, n, k, &c, nullptr);
+        const int tiles = n > 32 ? 4 : n > 16 ? 2 : 1;  // token tiles: one pass over the weights
+        const bool entry_fits = c.lds_tile_rows <= 0 && c.rows_per_wave == 64 && c.token_tiles == tiles && c.split_k == 1 &&
+                                c.waves_m * c.waves_k >= 8 && (c.prefetch == 2 || c.prefetch == 4);
+        for (int attempt = entry_fits ? 0 : 1; attempt < 2; ++attempt) {
+            if (attempt == 1) {  // no such entry (or it does not fit the scale buffers): four waves along the rows, four along k
+                c.rows_per_wave = 64;
+                c.waves_m = m % 256 == 0 ? 4 : m % 128 == 0 ? 2 : 1;
+                c.waves_k = (tiles == 4 ? 8 : 16) / c.waves_m > 8 ? 8 : (tiles == 4 ? 8 : 16) / c.waves_m;  // (four token tiles: 512 threads)
+                c.split_k = 1;
+                c.prefetch = 2;
+                c.x_chunk = tiles == 4 ? 256 : 512;
+                c.token_tiles = tiles;
+                c.xcd_swizzle = 0;
+            }
+            c.lds_tile_rows = 0;
+            if (attempt == 1) c.k_stagger = 0;
+            GemmPlan plan;
+            const int shift = log2i(block_size) - 6;
+            if (m % (64 * c.waves_m) != 0 || plan_gemm(m, n, k, c, TUNA_DECODE_GEMM, &plan) != TUNA_OK ||
+                !mid_blockwise_applies(plan, shift))
+                continue;
+            int dev = 0, cus = 0;
+            hipError_t e = device_cus(&dev, &cus);
+            if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+            plan.args.q = static_cast<const uint8_t *>(q);
+            plan.args.x = x;
+            plan.args.code = static_cast<const float *>(code);
+            plan.args.absmax = static_cast<const float *>(absmax);
+            plan.args.out = out;
+            plan.args.epilogue = TUNA_EPILOGUE_NONE;
+            plan.args.residual = nullptr;
+            e = launch_gemm_mid_blockwise(plan, shift, dev, cus, static_cast<hipStream_t>(stream));
+            if (e != hipSuccess) return hip_fail(e, "streaming blockwise gemm launch");
+            g_blockwise_launches[3].fetch_add(1, std::memory_order_relaxed);
+            return TUNA_OK;
+        }
+    }
     // From 33 tokens: the many-token kernel's scale-block variants (the weights are decoded once per workgroup tile,
     // with the scale of the k-step's block) - the tile the per-row table has for the shape and token count if that is a
     // many-token entry, else 256 rows x 64 tokens up to 64 tokens, 128 x 128 up to 128 and 128 x 256 beyond.
-    const int stream_mode = g_blockwise_stream.load(std::memory_order_relaxed);
     if (n > 32 && stream_mode == 1) {
         tuna_gemm_config c;
         select_config(m, n, k, &c, nullptr);
@@ -1483,48 +1528,6 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
     // 8192 x 8192, 30.9 / 38.7 on 28672 x 4096, 21.4 / 28.3 on 13824 x 5120, but 37.2 / 30.4 on 10240 x 8192, 29.6 / 22.7
     // on 4096 x 14336, 22.1 / 18.3 on 2560 x 10240, 134 / 106 on 32768 x 14336 and 131 / 108 on 57344 x 8192.
     const long long packed_bytes = (long long)m * k / 2;
-    // Up to 32 tokens, shapes whose per-row table entry is an unsplit launch of the streaming kernel (the large ones):
-    // that kernel's scale-block twin with the entry's workgroup shape, ring, x chunk and stagger (in whole x chunks; register ring).
-    if (n <= 32 && (stream_mode == 3 || (stream_mode == 1 && mid_blockwise_wins(m, n, k)))) {
-        tuna_gemm_config c;
-        select_config(m, n, k, &c, nullptr);
-        const int tiles = n > 16 ? 2 : 1;  // token tiles: one pass over the weights
-        const bool entry_fits = c.lds_tile_rows <= 0 && c.rows_per_wave == 64 && c.token_tiles == tiles && c.split_k == 1 &&
-                                c.waves_m * c.waves_k >= 8 && (c.prefetch == 2 || c.prefetch == 4);
-        for (int attempt = entry_fits ? 0 : 1; attempt < 2; ++attempt) {
-            if (attempt == 1) {  // no such entry (or it does not fit the scale buffers): four waves along the rows, four along k
-                c.rows_per_wave = 64;
-                c.waves_m = m % 256 == 0 ? 4 : m % 128 == 0 ? 2 : 1;
-                c.waves_k = 16 / c.waves_m > 8 ? 8 : 16 / c.waves_m;
-                c.split_k = 1;
-                c.prefetch = 2;
-                c.x_chunk = 512;
-                c.token_tiles = tiles;
-                c.xcd_swizzle = 0;
-            }
-            c.lds_tile_rows = 0;
-            if (attempt == 1) c.k_stagger = 0;
-            GemmPlan plan;
-            const int shift = log2i(block_size) - 6;
-            if (m % (64 * c.waves_m) != 0 || plan_gemm(m, n, k, c, TUNA_DECODE_GEMM, &plan) != TUNA_OK ||
-                !mid_blockwise_applies(plan, shift))
-                continue;
-            int dev = 0, cus = 0;
-            hipError_t e = device_cus(&dev, &cus);
-            if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
-            plan.args.q = static_cast<const uint8_t *>(q);
-            plan.args.x = x;
-            plan.args.code = static_cast<const float *>(code);
-            plan.args.absmax = static_cast<const float *>(absmax);
-            plan.args.out = out;
-            plan.args.epilogue = TUNA_EPILOGUE_NONE;
-            plan.args.residual = nullptr;
-            e = launch_gemm_mid_blockwise(plan, shift, dev, cus, static_cast<hipStream_t>(stream));
-            if (e != hipSuccess) return hip_fail(e, "streaming blockwise gemm launch");
-            g_blockwise_launches[3].fetch_add(1, std::memory_order_relaxed);
-            return TUNA_OK;
-        }
-    }
     const bool stream_wins = n > 16  ? packed_bytes >= (100ll << 20) || (k > 8192 && packed_bytes >= (12ll << 20)) ||
                                            (k > 4096 && packed_bytes >= (40ll << 20))
                              : n > 4 ? packed_bytes >= (100ll << 20) || (n > 8 && k >= 12288 && packed_bytes >= (20ll << 20))

@@ -190,7 +190,7 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
     return hipGetLastError();
 }
 
-// ---- scale blocks finer than a row: the BLK twins (one or two token tiles, register ring) -------------------------
+// ---- scale blocks finer than a row: the BLK twins (one, two or four token tiles, register ring) -------------------------
 struct MidBlkVariant {
     int u, tt, maxt;
     MidKernelFn fn;
@@ -204,17 +204,20 @@ static const MidBlkVariant kMidBlk[] = {
     {4, 2, 512, gemm_mid_kernel<4, 2, 4, 512, 2, true, false, false, true>},
     {2, 2, 1024, gemm_mid_kernel<2, 2, 4, 1024, 4, true, false, false, true>},
     {4, 2, 1024, gemm_mid_kernel<4, 2, 4, 1024, 4, true, false, false, true>},
+    {2, 4, 512, gemm_mid_kernel<2, 4, 4, 512, 2, true, false, false, true>},
+    {4, 4, 512, gemm_mid_kernel<4, 4, 4, 512, 2, true, false, false, true>},
 };
 static constexpr int kNumMidBlk = sizeof(kMidBlk) / sizeof(kMidBlk[0]);
 static OptInFlag g_mid_blk_attr_done[16][kNumMidBlk];
 
-// The BLK twin for a planned launch (an unsplit config of one or two token tiles the streaming kernel takes, up to four - 1024
+// The BLK twin for a planned launch (an unsplit config of one, two or four token tiles the streaming kernel takes, up to four - 1024
 // threads: two - scales per thread and chunk), its x chunk and LDS size; null if there is none.
 static const MidBlkVariant *mid_blk_variant(const GemmPlan &plan, int blk_shift, int *xc_out, size_t *lds_out)
 {
     const GemmArgs &a = plan.args;
     int xc = 0;
-    if ((plan.token_tiles != 1 && plan.token_tiles != 2) || a.split_k != 1 || plan.lds_weights || !mid_variant(plan, &xc))
+    if ((plan.token_tiles != 1 && plan.token_tiles != 2 && plan.token_tiles != 4) || a.split_k != 1 || plan.lds_weights ||
+        !mid_variant(plan, &xc))
         return nullptr;
     if (a.n > 16 * plan.token_tiles || a.k % (64 << blk_shift) != 0) return nullptr;  // (one pass over the weights)
     const int pieces = plan.token_tiles * 2 * xc;  // 16-byte x pieces per chunk
