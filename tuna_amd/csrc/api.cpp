@@ -1444,8 +1444,11 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
         const int tiles = n > 32 ? 4 : n > 16 ? 2 : 1;  // token tiles: one pass over the weights
         const bool entry_fits = c.lds_tile_rows <= 0 && c.rows_per_wave == 64 && c.token_tiles == tiles && c.split_k == 1 &&
                                 c.waves_m * c.waves_k >= 8 && (c.prefetch == 2 || c.prefetch == 4);
-        for (int attempt = entry_fits ? 0 : 1; attempt < 2; ++attempt) {
-            if (attempt == 1) {  // no such entry (or it does not fit the scale buffers): four waves along the rows, four along k
+        // (the library's own routing takes the twin with such an entry only: up to 9 tokens the entries of these shapes
+        // are narrow-row ones, and there the narrow-row scale-block kernel is the faster one - 19.6 against 27.3 us on
+        // 28672 x 4096, 54.6 against 80 on 32768 x 14336 at one token)
+        for (int attempt = entry_fits ? 0 : 1; attempt < (stream_mode == 3 ? 2 : 1); ++attempt) {
+            if (attempt == 1) {  // the switch, without such an entry (or one that does not fit the scale buffers): four waves by four
                 c.rows_per_wave = 64;
                 c.waves_m = m % 256 == 0 ? 4 : m % 128 == 0 ? 2 : 1;
                 c.waves_k = (tiles == 4 ? 8 : 16) / c.waves_m > 8 ? 8 : (tiles == 4 ? 8 : 16) / c.waves_m;  // (four token tiles: 512 threads)
