@@ -370,14 +370,6 @@ static const BlockwiseVariant *choose_blockwise(int m, int k, int nblk, int cus,
     return tt > 1 ? choose_blockwise(m, k, nblk, cus, 1) : nullptr;  // (shapes only the 16-row, 4-wave tile of one token tile fits)
 }
 
-bool blockwise_describe(int m, int n, int k, char *buf, size_t len)
-{
-    const BlockwiseVariant *v = choose_blockwise(m, k, k / 64, kMaxCus, n > 16 ? 2 : 1);
-    if (!v) return false;
-    snprintf(buf, len, "gemm_narrow_kernel<LW=%d,WK=%d,U=%d,PERM=%d,TT=%d,BLK>", v->rows / 16, v->wk, v->u, n > 4 ? 1 : 0, v->tt);
-    return true;
-}
-
 hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, hipStream_t stream)
 {
     int dev = 0, cus = 0;

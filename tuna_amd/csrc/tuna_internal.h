@@ -190,9 +190,8 @@ struct NarrowArgs {
 bool narrow_variant_exists(int rows, int waves_k, int prefetch, int token_tiles);
 hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int prefetch, int token_tiles, hipStream_t stream);
 hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, hipStream_t stream);
-int set_blockwise_shape(int rows, int waves_k, int prefetch);
-int set_blockwise_scales_lds(int enabled);  // returns the previous setting  // 0 on success, -1: no such variant
-bool blockwise_describe(int m, int n, int k, char *buf, size_t len);
+int set_blockwise_shape(int rows, int waves_k, int prefetch);  // 0 on success, -1: no such variant
+int set_blockwise_scales_lds(int enabled);  // returns the previous setting
 int set_lean_kernels(int enabled);  // returns the previous setting
 int set_weight_path(int path);      // gemm_mid.hip; negative: query
 unsigned long long lean_launches();
