@@ -851,7 +851,7 @@ def test_many_token_kernel_decode_readout_is_bit_exact():
 # ----------------------------------------------------------------------------- stream capture / graph replay, several streams
 def test_graph_replay_matches_eager_for_split_k_and_many_token_configs():
     """The ops are stream-ordered and capturable once their workspace exists: a captured graph
-    of four GEMMs (fixed split-K, balanced split, many-token kernels with split-K) is replayed
+    of five GEMMs (fixed split-K, balanced split, many-token kernels with split-K, the streaming kernel's split twin) is replayed
     with new inputs written in place, with eager work and synchronisations in between, and
     every replay must give the bits of the eager call."""
     import torch
@@ -860,7 +860,10 @@ def test_graph_replay_matches_eager_for_split_k_and_many_token_configs():
 
     m, n, k = 1024, 144, 2048
     cfgs = [cfg(split_k=4, x_chunk=512), cfg(split_k=0, waves_m=1, waves_k=8, prefetch=2, x_chunk=512),
-            cfg(lds_tile_rows=128, token_tiles=8, split_k=2), cfg(lds_tile_rows=256, token_tiles=16, split_k=2)]
+            cfg(lds_tile_rows=128, token_tiles=8, split_k=2), cfg(lds_tile_rows=256, token_tiles=16, split_k=2),
+            # the streaming kernel's twin with k split across workgroups (two token tiles, five token chunks)
+            cfg(waves_m=2, waves_k=4, prefetch=2, x_chunk=256, token_tiles=2, split_k=4)]
+    assert "gemm_mid_kernel" in ops.describe_launch(m, n, k, cfgs[-1]) and "split_k=4" in ops.describe_launch(m, n, k, cfgs[-1])
     q, x, code, absmax = make_inputs_np(m, n, k, seed=31)
     dq, dx, dc, da = to_dev(q, x, code, absmax)
     outs = [torch.zeros((n, m), dtype=torch.float16, device="cuda") for _ in cfgs]
