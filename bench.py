@@ -8,14 +8,18 @@ out[16, 6144] = x[16, 4096] . W[6144, 4096]^T, benchmark configuration 1) on one
 of distinct, HBM-resident weight matrices, so that neither L2 nor the 256 MB Infinity Cache
 can serve re-reads.  W warm-up steps, then exactly K timed steps bracketed by HIP events on
 the launch stream (tuna_time_matmul, inside the C library, so that no Python overhead sits
-between launches).  One JSON line is printed:
+between launches).  The LAST line printed is one compact JSON object (under 2 KB, headline_line()):
 
   value        packed-weight bytes (m*k/2) per second, GB/s  - the roofline quantity
   ms_per_step  milliseconds per GEMM (x1000 = the metric's "us/GEMM")
   roofline     achieved / peak HBM bandwidth for the GEMM kernel (algorithmic bytes = m*k/2)
-  cpu_baseline the CPU oracle's dequantize-then-matmul on the same workload, host cores
-  shapes       the same measurement for every 16-token layer shape of the benchmark configurations
-  sweeps       Llama-70B 80-layer sweep (distinct weights per layer) and the token sweep
+  cpu_baseline the CPU oracle's dequantize-then-matmul on benchmark configuration 0, host cores
+  frac_hbm_by_shape   fraction of 8 TB/s for every 16-token layer shape of the benchmark configurations
+
+Everything else - the per-shape table with configs and kernels, the same shapes eight to a launch, the
+Llama-70B 80-layer sweep, the token sweep, the dequant / quantizer / blockwise timings and the yardsticks -
+goes into one "detail" JSON object that is printed on an earlier line and written to
+gpurun_out/bench_detail.json.
 """
 import argparse
 import json
@@ -639,7 +643,48 @@ def main():
     else:
         line["cpu_baseline"] = None
 
-    print(json.dumps(line))
+    detail_path = write_detail(line)
+    print(json.dumps({"detail": line}))
+    print(headline_line(line, detail_path))
+
+
+DETAIL_FILE = os.path.join("gpurun_out", "bench_detail.json")
+HEADLINE_KEYS = ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "us_per_gemm", "tflops",
+                 "higher_is_better", "scaling", "vs_baseline", "dtype", "data")
+ROOFLINE_KEYS = ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel", "algorithmic_bytes_per_launch",
+                 "avg_launch_us")
+CPU_KEYS = ("value", "unit", "cores", "kind", "sample", "us_per_gemm", "single_thread_us_per_gemm")
+
+
+def write_detail(detail):
+    """Writes the full result object beside the repository's other GPU-run outputs; -> the relative path, or None
+    where the directory cannot be written."""
+    try:
+        os.makedirs(os.path.join(ROOT, os.path.dirname(DETAIL_FILE)), exist_ok=True)
+        with open(os.path.join(ROOT, DETAIL_FILE), "w") as f:
+            json.dump(detail, f, indent=1)
+        return DETAIL_FILE
+    except OSError:
+        return None
+
+
+def headline_line(detail, detail_path=None):
+    """The last line bench.py prints: the headline measurement only, as compact JSON of well under 2 KB whatever the
+    detail object holds (the harness that runs the bench keeps the end of stdout and parses its last line)."""
+    line = {key: detail.get(key) for key in HEADLINE_KEYS}
+    cfg = detail.get("config") or {}
+    line["config"] = {"workload": str(cfg.get("workload", ""))[:300], "launch": cfg.get("launch"),
+                      "timed_launches": detail.get("steps"), "tile_config": cfg.get("tile_config")}
+    roof = detail.get("roofline") or {}
+    line["roofline"] = {key: roof.get(key) for key in ROOFLINE_KEYS}
+    cpu = detail.get("cpu_baseline")
+    line["cpu_baseline"] = None if cpu is None else {key: (str(cpu.get(key))[:200] if key == "sample" else cpu.get(key))
+                                                     for key in CPU_KEYS}
+    shapes = detail.get("shapes") or {}
+    if shapes:
+        line["frac_hbm_by_shape"] = {name: r.get("frac_hbm") for name, r in list(shapes.items())[:12]}
+    line["detail"] = detail_path
+    return json.dumps(line, separators=(",", ":"))
 
 
 if __name__ == "__main__":

@@ -20,7 +20,9 @@ extern "C" {
  * absmax_list (rotating over distinct weights defeats the L2 / MALL caches), and
  * returns the elapsed milliseconds of the timed launches measured with HIP events
  * recorded on `stream`.  use_graph != 0 captures one rotation into a HIP graph and
- * replays it.  This call synchronises the host with `stream`. */
+ * replays it iters / n_sets times, followed by one replay of a graph of the first
+ * iters % n_sets launches: the events bracket exactly `iters` launches either way.
+ * This call synchronises the host with `stream`. */
 int tuna_time_matmul(const void *const *q_list, const void *const *absmax_list, int n_sets,
                      const void *x, const void *code, void *out, int m, int n, int k,
                      const tuna_gemm_config *cfg, int decode_mode, int warmup, int iters,

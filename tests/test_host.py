@@ -519,3 +519,45 @@ def test_grouped_launch_gets_a_runnable_config_for_every_table_shape():
     assert c.waves_m >= 1 and 4096 % (64 * c.waves_m) == 0
     with pytest.raises(ops.TunaError):
         ops.select_config_grouped(4000, 8, 4, 14336)                   # not a multiple of 64 rows
+
+
+def test_bench_last_line_stays_compact_whatever_the_detail_holds():
+    """The harness that runs bench.py keeps the end of stdout and parses its last line: that line is the
+    headline only and stays far below 4 KB even when the detail object is hundreds of kilobytes."""
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench
+
+    shape_row = {"m": 6144, "n": 16, "k": 4096, "us_per_gemm": 7.0, "gbs": 1797.5, "frac_hbm": 0.2247,
+                 "kernel": "gemm_narrow_kernel<LW=2,WK=8,U=4,PERM=1,TT=1>", "config": {"rows_per_wave": 32} , "pad": "x" * 4000}
+    detail = {
+        "metric": bench.METRIC, "value": 1797.5, "unit": "GB/s", "n_gpus": 1, "steps": 20, "warmup": 5,
+        "ms_per_step": 0.007, "us_per_gemm": 7.0, "tflops": 115.0, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "benchmark config 1: Mistral-7B QKV projection, M=16 tokens, K=4096, N=6144; " + "y" * 5000,
+                   "tile_config": {"rows_per_wave": 32, "waves_m": 1, "waves_k": 8, "split_k": 1, "prefetch": 4, "x_chunk": 512,
+                                   "token_tiles": 1, "xcd_swizzle": 0, "k_stagger": 0, "lds_tile_rows": 0},
+                   "launch": "stream"},
+        "roofline": {"bound": "hbm", "achieved": 1797.5, "peak": 8000.0, "unit": "GB/s", "frac": 0.2247, "traffic": 13919232,
+                     "kernel": "tuna::gemm_narrow_kernel<LW=2,WK=8,U=4,PERM=1,TT=1>", "algorithmic_bytes_per_launch": 12582912,
+                     "avg_launch_us": 7.0, "extra": "z" * 3000},
+        "cpu_baseline": {"value": 3.3, "unit": "GB/s", "cores": 16, "kind": "port", "sample": "s" * 2000, "us_per_gemm": 2507.2,
+                         "us_decode": 1.0, "us_matmul": 2.0, "single_thread_us_per_gemm": 36553.9},
+        "shapes": {f"shape_{i}": dict(shape_row) for i in range(40)},
+        "sweeps": {"token_sweep": {str(t): {f"shape_{i}": dict(shape_row) for i in range(4)} for t in (1, 16, 64, 256, 1024, 4096)}},
+        "unit_rates": {f"unit_{i}": 1.0 for i in range(40)},
+    }
+    assert len(json.dumps(detail)) > 200_000
+    text = bench.headline_line(detail, "gpurun_out/bench_detail.json")
+    assert "\n" not in text and len(text) < 2048, len(text)
+    line = json.loads(text)
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "dtype", "data"):
+        assert line[key] == detail[key], key
+    assert line["config"]["workload"].startswith("benchmark config 1") and "model" not in line["config"]
+    assert set(line["roofline"]) == set(bench.ROOFLINE_KEYS) and line["roofline"]["frac"] == 0.2247
+    assert line["cpu_baseline"]["cores"] == 16 and line["cpu_baseline"]["kind"] == "port"
+    assert len(line["frac_hbm_by_shape"]) <= 12
+    # no CPU leg and no shape table (profiling runs): still one parseable line
+    bare = dict(detail, cpu_baseline=None)
+    del bare["shapes"]
+    assert json.loads(bench.headline_line(bare))["cpu_baseline"] is None

@@ -1218,7 +1218,8 @@ static int time_loop(F launch, int n_sets, int warmup, int iters, int use_graph,
         return hip_fail(e, "hipEventCreate");
     }
     hipGraph_t graph = nullptr;
-    hipGraphExec_t exec = nullptr;
+    hipGraphExec_t exec = nullptr, tail_exec = nullptr;
+    hipGraph_t tail_graph = nullptr;
     hipStream_t cap_stream = nullptr;
     rc = TUNA_OK;
     do {
@@ -1238,17 +1239,27 @@ static int time_loop(F launch, int n_sets, int warmup, int iters, int use_graph,
             if (rc) break;
             if (e != hipSuccess) { rc = hip_fail(e, "hipStreamEndCapture"); break; }
             if ((e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0)) != hipSuccess) { rc = hip_fail(e, "hipGraphInstantiate"); break; }
-            const int reps = (iters + n_sets - 1) / n_sets;
+            // exactly `iters` timed launches: `iters / n_sets` replays of the rotation and, when that leaves a
+            // remainder, one replay of a second graph that holds the first `iters % n_sets` launches of it
+            const int reps = iters / n_sets, rest = iters % n_sets;
+            if (rest > 0) {
+                if ((e = hipStreamBeginCapture(cap_stream, hipStreamCaptureModeThreadLocal)) != hipSuccess) { rc = hip_fail(e, "hipStreamBeginCapture"); break; }
+                for (int i = 0; i < rest && !rc; ++i) rc = launch(i, cap_stream);
+                e = hipStreamEndCapture(cap_stream, &tail_graph);
+                if (rc) break;
+                if (e != hipSuccess) { rc = hip_fail(e, "hipStreamEndCapture"); break; }
+                if ((e = hipGraphInstantiate(&tail_exec, tail_graph, nullptr, nullptr, 0)) != hipSuccess) { rc = hip_fail(e, "hipGraphInstantiate"); break; }
+                if ((e = hipGraphLaunch(tail_exec, cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipGraphLaunch"); break; }
+            }
             if ((e = hipGraphLaunch(exec, cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipGraphLaunch"); break; }
             if ((e = hipEventRecord(t0, cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipEventRecord"); break; }
             for (int r = 0; r < reps; ++r)
                 if ((e = hipGraphLaunch(exec, cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipGraphLaunch"); break; }
             if (rc) break;
+            if (rest > 0 && (e = hipGraphLaunch(tail_exec, cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipGraphLaunch"); break; }
             if ((e = hipEventRecord(t1, cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipEventRecord"); break; }
             if ((e = hipEventSynchronize(t1)) != hipSuccess) { rc = hip_fail(e, "hipEventSynchronize"); break; }
-            float ms = 0.f;
-            if ((e = hipEventElapsedTime(&ms, t0, t1)) != hipSuccess) { rc = hip_fail(e, "hipEventElapsedTime"); break; }
-            *elapsed_ms = ms * (float)iters / (float)(reps * n_sets);  // scaled to exactly `iters` launches
+            if ((e = hipEventElapsedTime(elapsed_ms, t0, t1)) != hipSuccess) { rc = hip_fail(e, "hipEventElapsedTime"); break; }
         } else {
             if ((e = hipEventRecord(t0, stream)) != hipSuccess) { rc = hip_fail(e, "hipEventRecord"); break; }
             for (int i = 0; i < iters && !rc; ++i) rc = launch((warmup + i) % n_sets, stream);
@@ -1260,6 +1271,8 @@ static int time_loop(F launch, int n_sets, int warmup, int iters, int use_graph,
     } while (0);
     if (exec) (void)hipGraphExecDestroy(exec);
     if (graph) (void)hipGraphDestroy(graph);
+    if (tail_exec) (void)hipGraphExecDestroy(tail_exec);
+    if (tail_graph) (void)hipGraphDestroy(tail_graph);
     if (cap_stream) {
         (void)hipStreamSynchronize(cap_stream);
         drop_workspace(cap_stream);
