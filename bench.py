@@ -439,7 +439,12 @@ def main():
 
     import torch
 
-    from tuna_amd import ops, synth
+    from tuna_amd import _lib, ops, synth
+
+    # The timing loops (HIP events around back-to-back launches, no Python in between) and the yardstick kernels
+    # live in the diagnostic build, libtuna_amd_bench.so: the product library's own object files plus those tools.
+    # Every GEMM this program times is launched through that library's tuna_matmul_ex / tuna_matmul_multi.
+    _lib.use_diagnostic_build()
 
     if not torch.cuda.is_available():
         print("bench.py needs a HIP device", file=sys.stderr)

@@ -247,6 +247,17 @@ int tuna_select_config_ex(int m, int n, int k, int decode_mode, tuna_gemm_config
  * of them with max_tokens.  Host only. */
 int tuna_select_config_grouped(int m_group, int n_active, int max_tokens, int k, int decode_mode,
                                tuna_gemm_config *cfg);
+/* The config the library derives for a shape when its table has no entry for it - also for shapes that have
+ * one: what the tuner seeds its search with, and what a table entry has to beat.  Host only. */
+int tuna_derive_config(int m, int n, int k, tuna_gemm_config *cfg);
+
+/* Name and template arguments of the kernel a GEMM launch would start (cfg NULL = the library's
+ * choice), e.g. "gemm_narrow_kernel<LW=2,WK=8,U=4,PERM=1,TT=1>": for logs, and for matching a timing
+ * with a profile.  Host only; with a device present the
+ * device's CU count decides between twins, otherwise 256 CUs are assumed. */
+int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config *cfg, int decode_mode,
+                         char *buf, size_t len);
+
 /* TUNA_OK if `cfg` can run shape (m, n, k); otherwise an error and tuna_last_error(). */
 int tuna_validate_config(int m, int n, int k, const tuna_gemm_config *cfg);
 /* Same for a decode mode (tuna_validate_config checks TUNA_DECODE_GEMM). */

@@ -1,10 +1,12 @@
 /*
- * tuna_amd - measurement and diagnostic entry points of libtuna_amd.so.
+ * tuna_amd - measurement and diagnostic entry points of libtuna_amd_bench.so, the diagnostic build.
  *
- * These are tools for bench.py, the tuner and the tests: timing loops with HIP events on the
- * launch stream, known-traffic yardstick kernels, and a switch between kernels that compute
- * identical results.  None of them replaces an interface of the reference; the product's C ABI
- * is tuna_amd.h.
+ * libtuna_amd_bench.so holds everything libtuna_amd.so holds (the same object files; it exports
+ * every entry point of tuna_amd.h too) plus the tools declared here for bench.py, the tuner and the
+ * tests: timing loops with HIP events on the launch stream, known-traffic yardstick kernels, and
+ * process-wide switches between kernels that compute identical results, with counters that tell which
+ * kernel ran.  The product library has none of these: its routing choices are constants.  None of
+ * them replaces an interface of the reference; the product's C ABI is tuna_amd.h.
  */
 #ifndef TUNA_AMD_BENCH_H
 #define TUNA_AMD_BENCH_H
@@ -70,17 +72,6 @@ int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int va
  * one launch; `sink`: 8 writable bytes. */
 int tuna_time_unit_rate(int unit, void *sink, int warmup, int iters, void *stream, float *elapsed_ms,
                         double *work_per_launch);
-
-/* The config the library derives for a shape when its table has no entry for it - also for shapes that have
- * one: what the tuner seeds its search with, and what a table entry has to beat.  Host only. */
-int tuna_derive_config(int m, int n, int k, tuna_gemm_config *cfg);
-
-/* Name and template arguments of the kernel a GEMM launch would start (cfg NULL = the library's
- * choice), e.g. "gemm_narrow_kernel<LW=2,WK=8,U=4,PERM=1,TT=1>": what the bench writes beside a
- * timing so that it can be matched with a profile.  Host only; with a device present the
- * device's CU count decides between twins, otherwise 256 CUs are assumed. */
-int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config *cfg, int decode_mode,
-                         char *buf, size_t len);
 
 /* Self-test of the quantizer's division: the kernel divides by a block's maximum with a refined
  * reciprocal and one fused correction instead of the general IEEE sequence; this runs that

@@ -26,3 +26,13 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture
+def diagnostic_build():
+    """Runs the test's ops in libtuna_amd_bench.so (the product's object files plus process-wide routing switches and
+    launch counters), so that tuna_set_* and tuna_*_launches apply to the calls the test makes.  Yields that library."""
+    from tuna_amd import _lib
+
+    with _lib.diagnostic_build() as L:
+        yield L

@@ -1043,6 +1043,7 @@ LEAN_CASES = [
 ]
 
 
+@pytest.mark.usefixtures("diagnostic_build")
 @pytest.mark.parametrize("ci", range(len(LEAN_CASES)))
 def test_lean_kernel_equals_general_kernel_bit_for_bit(ci):
     """Small aligned launches take a stripped-down kernel; it must give the bits of the general
@@ -1132,6 +1133,7 @@ MID_CASES = [
 ]
 
 
+@pytest.mark.usefixtures("diagnostic_build")
 @pytest.mark.parametrize("ci", range(len(MID_CASES)))
 def test_mid_token_kernel_equals_general_kernel_bit_for_bit(ci):
     """Dense launches with two, four or eight token tiles, unsplit or with k split into a power of two of
@@ -1194,6 +1196,7 @@ LDS_PATH_CASES = [
 ]
 
 
+@pytest.mark.usefixtures("diagnostic_build")
 @pytest.mark.gpu
 @pytest.mark.parametrize("ci", range(len(LDS_PATH_CASES)))
 def test_weights_staged_through_lds_equal_the_register_ring_bit_for_bit(ci):
@@ -1416,6 +1419,7 @@ def test_captured_graph_survives_growth_of_the_split_k_workspace():
     [(128, 16, 1024), (640, 3, 512), (384, 16, 2560)],                                             # 128-row tiles, short k, ragged shares
     [(8192, 16, 28672)],                                                                           # a batch of one
 ])
+@pytest.mark.usefixtures("diagnostic_build")
 def test_matmul_multi_with_weights_through_lds_gives_the_register_paths_bits(shapes):
     """The batched kernel's twin that stages packed weights and x through LDS (global -> LDS loads, x
     chunks of 512 k) adds the same products in the same order: equal bits, on batches that exercise
@@ -1476,6 +1480,7 @@ def _check_against_oracle(host, got_bits, m, n, k, seed, n_rows=256):
     return rel_err(f16_bits_to_f64(got_bits[:, rows]), ref)
 
 
+@pytest.mark.usefixtures("diagnostic_build")
 def test_matmul_multi_matches_the_oracle_and_separate_calls():
     """tuna_matmul_multi on a mixed batch: five problems that the batched persistent kernel takes
     in one launch (1..16 tokens, tuned and untuned shapes, k up to 14336), one it cannot take
@@ -1522,6 +1527,7 @@ def test_matmul_multi_matches_the_oracle_and_separate_calls():
     assert torch.equal(probs[0][4].view(torch.int16), want[0].view(torch.int16))
 
 
+@pytest.mark.usefixtures("diagnostic_build")
 @pytest.mark.parametrize("waves_m,prefetch", [(4, 2), (4, 4), (2, 2), (2, 4), (8, 2), (8, 4), (1, 2), (16, 2)])
 def test_matmul_multi_every_workgroup_shape_and_decode_readout(waves_m, prefetch):
     """The batched kernel with every workgroup shape it has (waves along rows x ring depth): oracle
@@ -1625,6 +1631,7 @@ def test_matmul_multi_in_a_captured_graph_replays_correctly():
     (4096, 1, 2048, dict(waves_m=8, waves_k=2, prefetch=4, x_chunk=256)),
     (3072, 16, 14336, dict(waves_m=1, waves_k=16, prefetch=2, x_chunk=1024)),
 ])
+@pytest.mark.usefixtures("diagnostic_build")
 def test_balanced_split_through_the_batched_kernel_equals_general_kernel_bit_for_bit(m, n, k, ckw):
     """A balanced split over 16-wave workgroups is run by the batched kernel as a batch of one.  It
     walks the segments gemm_kernel's balanced split walks, in the same order, and sums in the same
@@ -1750,6 +1757,7 @@ def test_blockwise_gemm_matches_oracle_and_reads_out_the_decode(m, n, k, bs):
     (768, 32, 8192, 64, None),           # two token tiles, the library's choice of rows
     (256, 32, 28672, 64, (64, 8, 4)),    # two token tiles, scales in memory (they do not fit in LDS)
 ])
+@pytest.mark.usefixtures("diagnostic_build")
 def test_blockwise_narrow_kernel_with_scales_in_lds_and_in_memory(m, n, k, bs, shape):
     """The narrow-row kernel's scale-block variants stage the workgroup's scales in LDS when they fit and read them
     from memory per ring slot when they do not (or when the switch says so): both orders of reading the same scales
@@ -1796,6 +1804,7 @@ def test_blockwise_narrow_kernel_with_scales_in_lds_and_in_memory(m, n, k, bs, s
         L.tuna_set_blockwise_stream(prev_stream)
 
 
+@pytest.mark.usefixtures("diagnostic_build")
 @pytest.mark.parametrize("m,n,k,bs", [(256, 16, 1280, 64), (128, 7, 1536, 64), (512, 16, 4096, 128), (1024, 1, 2048, 256),
                                       (256, 16, 2048, 512), (768, 13, 5120, 64), (4096, 16, 4096, 64), (8192, 16, 8192, 64),
                                       (512, 37, 2048, 256), (256, 100, 1024, 64), (256, 530, 512, 64)])
@@ -1848,6 +1857,7 @@ def test_blockwise_gemm_through_the_batched_streaming_kernel(m, n, k, bs):
         L.tuna_set_blockwise_stream(prev)
 
 
+@pytest.mark.usefixtures("diagnostic_build")
 @pytest.mark.parametrize("m,n,k,bs", [(256, 16, 1024, 64), (512, 7, 2048, 64), (1024, 16, 4096, 128), (2048, 1, 8192, 64),
                                       (256 * 70, 16, 1024, 64), (768, 13, 5120, 64), (512, 16, 8192, 4096), (1024, 16, 2048, 1024),
                                       (4096, 16, 4096, 64), (16384, 16, 4096, 64), (28672, 16, 4096, 64),
@@ -1898,6 +1908,7 @@ def test_blockwise_gemm_through_the_streaming_kernel(m, n, k, bs):
         L.tuna_set_blockwise_stream(prev)
 
 
+@pytest.mark.usefixtures("diagnostic_build")
 @pytest.mark.parametrize("m,n,k,bs", [(512, 64, 1024, 64), (528, 130, 2048, 128), (1024, 300, 4096, 64), (256, 1024, 512, 256),
                                       (4096, 33, 4096, 64), (272, 200, 1280, 64), (12288, 1000, 1024, 64)])
 def test_blockwise_gemm_with_many_tokens_through_the_many_token_kernel(m, n, k, bs):
@@ -1941,6 +1952,7 @@ def test_blockwise_gemm_with_many_tokens_through_the_many_token_kernel(m, n, k, 
     assert np.array_equal(out.cpu().numpy().view(np.uint16)[:nh], img[:, cols].T)
 
 
+@pytest.mark.usefixtures("diagnostic_build")
 def test_matmul_multi_blockwise_matches_the_oracle_and_separate_calls():
     """tuna_matmul_multi_blockwise: four problems with a scale per 64 weights in one launch of the batched kernel, one
     it cannot take (40 tokens) and one more behind it; every output against the oracle's float64 sums over the blockwise
@@ -2031,6 +2043,7 @@ def test_blockwise_entry_points_reject_what_they_cannot_run():
     torch.cuda.synchronize()
 
 
+@pytest.mark.usefixtures("diagnostic_build")
 def test_quantizer_division_is_the_ieee_division_for_every_quotient_it_can_form():
     """The quantizer divides by a block's maximum with a refined reciprocal and one fused correction.
     Every pair of fp16 values (w, a), a > 0 finite, |w| <= a - 1.0e9 pairs, all there are - gives

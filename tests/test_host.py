@@ -11,20 +11,50 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def test_library_loads_and_exports_every_declared_symbol():
+def _declared(header_name):
+    return set(re.findall(r"\b(tuna_[a-z0-9_]+)\s*\(", open(os.path.join(ROOT, "include", header_name)).read()))
+
+
+def _exported(path):
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", path], check=True, capture_output=True, text=True).stdout
+    return {line.split()[-1] for line in out.splitlines() if line.strip()}
+
+
+def test_product_library_exports_exactly_what_its_header_declares():
+    """libtuna_amd.so: every symbol include/tuna_amd.h declares and not one dynamic symbol more - no timing loops,
+    no yardstick kernels, no process-wide switches, no kernel launch stubs."""
     from tuna_amd import _lib
 
-    L = _lib.lib()
-    header = "".join(open(os.path.join(ROOT, "include", h)).read() for h in sorted(os.listdir(os.path.join(ROOT, "include")))
-                     if h.endswith(".h"))
-    declared = set(re.findall(r"\b(tuna_[a-z0-9_]+)\s*\(", header))
+    L = _lib._load("product")
+    declared = _declared("tuna_amd.h")
     assert declared, "no declarations parsed"
     assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
     for name in declared:
         assert hasattr(L, name), name
+    assert _exported(_lib.LIB_PATH) == declared, _exported(_lib.LIB_PATH) ^ declared
     assert L.tuna_version() == 100
     assert L.tuna_status_string(0) == b"ok"
     assert L.tuna_status_string(2) == b"unsupported shape or config"
+
+
+def test_diagnostic_build_exports_the_product_abi_plus_its_own_header():
+    from tuna_amd import _lib
+
+    L = _lib.bench_lib()
+    bench_only = _declared("tuna_amd_bench.h")
+    assert bench_only == set(_lib.BENCH_SIGNATURES), bench_only ^ set(_lib.BENCH_SIGNATURES)
+    assert not bench_only & _declared("tuna_amd.h")
+    for name in bench_only | set(_lib.SIGNATURES):
+        assert hasattr(L, name), name
+    assert _exported(_lib.BENCH_LIB_PATH) == bench_only | _declared("tuna_amd.h")
+    # the switches apply to ops while the diagnostic build is the active library, and only then
+    assert _lib.lib() is _lib._load("product")
+    with _lib.diagnostic_build() as D:
+        assert _lib.lib() is D is L
+        prev = D.tuna_set_lean_kernels(0)
+        assert D.tuna_set_lean_kernels(prev) == 0
+    assert _lib.lib() is _lib._load("product")
 
 
 def test_config_struct_matches_header():

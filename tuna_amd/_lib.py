@@ -1,15 +1,20 @@
-"""ctypes binding of tuna_amd/libtuna_amd.so (the C ABI declared in include/tuna_amd.h).
+"""ctypes binding of tuna_amd/libtuna_amd.so (the C ABI declared in include/tuna_amd.h) and of its
+diagnostic build tuna_amd/libtuna_amd_bench.so (include/tuna_amd_bench.h on top of the same ABI).
 
-The library is built in-tree by ``make -C tuna_amd/csrc`` (see build()).  There is no
-fallback implementation: if the shared object is missing or does not load, every op
-raises.
+Both are built in-tree by ``make -C tuna_amd/csrc`` (see build()) from the same object files; the
+diagnostic build adds timing loops, yardstick kernels and process-wide switches between kernels that
+compute identical results.  ``lib()`` is the library the ops call: the product library unless
+``diagnostic_build()`` is active (bench.py, the tuner, A/B tests).  There is no fallback
+implementation: if a shared object is missing or does not load, every op raises.
 """
+import contextlib
 import ctypes
 import os
 import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtuna_amd.so")
+BENCH_LIB_PATH = os.path.join(_HERE, "libtuna_amd_bench.so")
 CSRC = os.path.join(_HERE, "csrc")
 
 OK = 0
@@ -63,6 +68,7 @@ _cfgp = ctypes.POINTER(GemmConfig)
 _ip = ctypes.POINTER(ctypes.c_int)
 _fp = ctypes.POINTER(ctypes.c_float)
 _vpp = ctypes.POINTER(ctypes.c_void_p)
+# the product ABI (include/tuna_amd.h): every symbol libtuna_amd.so exports, and nothing else
 SIGNATURES = {
     "tuna_version": (_i, []),
     "tuna_status_string": (ctypes.c_char_p, [_i]),
@@ -84,7 +90,6 @@ SIGNATURES = {
     "tuna_select_config": (_i, [_i, _i, _i, _cfgp, _ip]),
     "tuna_select_config_ex": (_i, [_i, _i, _i, _i, _cfgp, _ip]),
     "tuna_derive_config": (_i, [_i, _i, _i, _cfgp]),
-    "tuna_set_blockwise_scales_lds": (_i, [_i]),
     "tuna_select_config_grouped": (_i, [_i, _i, _i, _i, _i, _cfgp]),
     "tuna_validate_config": (_i, [_i, _i, _i, _cfgp]),
     "tuna_validate_config_ex": (_i, [_i, _i, _i, _cfgp, _i]),
@@ -93,6 +98,12 @@ SIGNATURES = {
     "tuna_config_contributors": (_i, [_i, _i, _i, _cfgp, _i, _i, _ip, _ip, _ip]),
     "tuna_config_table_size": (_i, []),
     "tuna_config_table_entry": (_i, [_i, _ip, _ip, _ip, _ip, _cfgp]),
+    "tuna_describe_launch": (_i, [_i, _i, _i, _cfgp, _i, ctypes.c_char_p, _sz]),
+    "tuna_release_workspaces": (_i, []),
+}
+# what the diagnostic build exports on top of it (include/tuna_amd_bench.h)
+BENCH_SIGNATURES = {
+    "tuna_set_blockwise_scales_lds": (_i, [_i]),
     "tuna_time_matmul": (_i, [_vpp, _vpp, _i, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_matmul_multi": (_i, [ctypes.POINTER(GemmProblem), _i, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_matmul_grouped": (_i, [_vpp, _vpp, _i, _vp, _vp, _vp, _i, _i, _i, _ip, _cfgp, _i, _i, _i, _i, _vp, _fp]),
@@ -100,7 +111,6 @@ SIGNATURES = {
     "tuna_time_copy": (_i, [_vp, _vp, _sz, _i, _i, _vp, _fp]),
     "tuna_time_read": (_i, [_vp, _vp, _sz, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_unit_rate": (_i, [_i, _vp, _i, _i, _vp, _fp, ctypes.POINTER(ctypes.c_double)]),
-    "tuna_describe_launch": (_i, [_i, _i, _i, _cfgp, _i, ctypes.c_char_p, _sz]),
     "tuna_selftest_quantizer_division": (_i, [_vp, _vp]),
     "tuna_set_multi_shape": (_i, [_i, _i]),
     "tuna_set_multi_min_batch": (_i, [_i]),
@@ -112,7 +122,6 @@ SIGNATURES = {
     "tuna_set_weight_path": (_i, [_i]),
     "tuna_set_multi_weight_path": (_i, [_i]),
     "tuna_lean_launches": (ctypes.c_ulonglong, []),
-    "tuna_release_workspaces": (_i, []),
 }
 
 
@@ -126,16 +135,16 @@ def build(force: bool = True) -> str:
     return LIB_PATH
 
 
-_lib = None
+_libs = {}
+_active = "product"
 
 
-def lib():
-    """The loaded library; raises if it is not built (no fallback path exists)."""
-    global _lib
-    if _lib is None:
-        if not os.path.exists(LIB_PATH):
+def _load(which: str):
+    if which not in _libs:
+        path = LIB_PATH if which == "product" else BENCH_LIB_PATH
+        if not os.path.exists(path):
             raise RuntimeError(
-                f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+                f"{path} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
                 "or `make -C tuna_amd/csrc`; tuna_amd has no non-HIP fallback")
         # The HIP runtime must be the one PyTorch-ROCm already uses in this process (torch
         # bundles its own libamdhip64): load torch first so that this library binds to it.
@@ -143,13 +152,46 @@ def lib():
             import torch  # noqa: F401
         except ImportError:
             pass
-        L = ctypes.CDLL(LIB_PATH)
-        for name, (res, args) in SIGNATURES.items():
+        L = ctypes.CDLL(path)
+        sigs = dict(SIGNATURES)
+        if which != "product":
+            sigs.update(BENCH_SIGNATURES)
+        for name, (res, args) in sigs.items():
             fn = getattr(L, name)  # AttributeError if the library lacks a declared symbol
             fn.restype = res
             fn.argtypes = args
-        _lib = L
-    return _lib
+        _libs[which] = L
+    return _libs[which]
+
+
+def lib():
+    """The library the ops call: libtuna_amd.so, or the diagnostic build while diagnostic_build() is active.
+    Raises if it is not built (no fallback path exists)."""
+    return _load(_active)
+
+
+def bench_lib():
+    """libtuna_amd_bench.so: the product's object files plus timing loops, yardsticks and routing switches."""
+    return _load("bench")
+
+
+@contextlib.contextmanager
+def diagnostic_build():
+    """While active, every op of this package runs in libtuna_amd_bench.so, so that its process-wide switches
+    (tuna_set_*) and launch counters apply to the calls made.  Yields that library."""
+    global _active
+    prev, _active = _active, "bench"
+    try:
+        yield bench_lib()
+    finally:
+        _active = prev
+
+
+def use_diagnostic_build() -> None:
+    """For a whole process (bench.py, the tuner): route every op through libtuna_amd_bench.so from now on."""
+    global _active
+    _active = "bench"
+    bench_lib()
 
 
 class TunaError(RuntimeError):
@@ -158,8 +200,10 @@ class TunaError(RuntimeError):
         self.status = status
 
 
-def check(status: int) -> None:
+def check(status: int, L=None) -> None:
+    """Raises TunaError with the library's message unless `status` is OK (`L`: the library that returned it,
+    default the active one)."""
     if status != OK:
-        L = lib()
+        L = L or lib()
         msg = L.tuna_last_error().decode() or L.tuna_status_string(status).decode()
         raise TunaError(status, msg)

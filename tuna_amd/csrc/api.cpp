@@ -21,7 +21,7 @@ namespace tuna {
 
 static thread_local std::string g_error;
 
-static int fail(int code, const char *fmt, ...)
+int fail(int code, const char *fmt, ...)
 {
     char buf[512];
     va_list ap;
@@ -32,7 +32,7 @@ static int fail(int code, const char *fmt, ...)
     return code;
 }
 
-static int hip_fail(hipError_t e, const char *what)
+int hip_fail(hipError_t e, const char *what)
 {
     return fail(TUNA_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
@@ -737,7 +737,7 @@ static void free_workspace(Workspace &w)
     w = Workspace();
 }
 
-static void drop_workspace(hipStream_t stream)
+void drop_workspace(hipStream_t stream)
 {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return;
@@ -806,7 +806,7 @@ static int provide_workspace(bool use_static, hipStream_t stream, size_t ws_byte
     return TUNA_OK;
 }
 
-static int check_ptr(const void *p, const char *name, size_t align)
+int check_ptr(const void *p, const char *name, size_t align)
 {
     if (!p) return fail(TUNA_ERR_INVALID_ARG, "%s is null", name);
     if (reinterpret_cast<uintptr_t>(p) % align) return fail(TUNA_ERR_INVALID_ARG, "%s must be %zu-byte aligned", name, align);
@@ -818,12 +818,6 @@ static int check_ptr(const void *p, const char *name, size_t align)
 // batched persistent kernel can run (gemm_multi.hpp) are one launch each; anything else is
 // launched problem by problem on the same stream.
 // ---------------------------------------------------------------------------------------
-static std::atomic<int> g_multi_waves_m{0}, g_multi_prefetch{0};  // 0: the library's choice (diagnostic override)
-static std::atomic<unsigned long long> g_blockwise_launches[4];  // by kernel: narrow-row, batched streaming, many-token, streaming
-static std::atomic<int> g_blockwise_stream{1};  // tuna_matmul_blockwise takes the batched kernel's scale-block variant where it can
-static std::atomic<int> g_multi_lds{0};  // batches with a ring of 2 stage weights and x through LDS (tuna_set_multi_weight_path)
-static std::atomic<unsigned long long> g_multi_launches{0};
-static std::atomic<int> g_multi_min_batch{2};  // batches shorter than this are launched problem by problem
 
 struct MultiPlan {
     MultiArgs args;
@@ -839,8 +833,8 @@ static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, Mu
 {
     if (count < 1 || count > kMaxMultiProblems || cus < 1) return false;
     const bool blk = blk_shift >= 0;
-    if (!waves_m) waves_m = g_multi_waves_m.load(std::memory_order_relaxed);
-    if (!prefetch) prefetch = g_multi_prefetch.load(std::memory_order_relaxed);
+    if (!waves_m) waves_m = diag::multi_waves_m();
+    if (!prefetch) prefetch = diag::multi_prefetch();
     // (a ring of two: with every wait of the ring exact it streams as fast as a ring of four on the longest
     // batches and faster on the others - fewer bytes requested ahead at a segment switch)
     if (!prefetch) prefetch = 2;
@@ -910,7 +904,7 @@ static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, Mu
     a.blk_shift = blk ? blk_shift : 0;
     // variant -2: ring of 2 with weights and x staged through LDS (x chunks of 512 k: every wave needs a whole
     // number of ring turns per chunk, so at most 8 waves along k)
-    const bool lds = !blk && g_multi_lds.load(std::memory_order_relaxed) != 0 && prefetch == 2 && waves_k <= 8 && multi_variant_exists(-2);
+    const bool lds = !blk && diag::multi_lds() != 0 && prefetch == 2 && waves_k <= 8 && multi_variant_exists(-2);
     plan->prefetch = blk ? 10 + prefetch : lds ? -2 : prefetch;
     plan->ws_bytes = (size_t)n_wg * 2 * waves_m * 4096;
     plan->n_counters = (size_t)tiles;
@@ -919,12 +913,12 @@ static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, Mu
 
 // A dense launch the batched kernel (gemm_multi.hpp) takes as a batch of one: balanced split, 64 rows
 // per wave, 16 waves, one token tile, the GEMM's own decode, no fused epilogue.  (plan_multi checks
-// the shape's alignment.)  Off with the diagnostic switch that turns the other twins off.
+// the shape's alignment.)  A diagnostic build can turn it off together with the other twins (diag.h).
 static bool stream_applies(const tuna_gemm_config &c, int n, int decode, int epilogue)
 {
     return c.split_k == 0 && !c.lds_tile_rows && c.rows_per_wave == kRowsPerLoad && c.waves_m >= 1 && c.waves_m * c.waves_k == 16 &&
            c.token_tiles == 1 && n <= 16 && decode == TUNA_DECODE_GEMM && epilogue == TUNA_EPILOGUE_NONE &&
-           (c.prefetch == 2 || c.prefetch == 4) && set_lean_kernels(-1) != 0;
+           (c.prefetch == 2 || c.prefetch == 4) && diag::lean_kernels() != 0;
 }
 
 static int matmul_impl(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n, int k,
@@ -987,7 +981,7 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
             if ((rc = provide_workspace(static_ws, stream, mp.ws_bytes, mp.n_counters, &mp.args.ws, &mp.args.counters))) return rc;
             e = launch_gemm_multi(mp.args, mp.prefetch, dev, stream);
             if (e != hipSuccess) return hip_fail(e, "gemm launch");
-            g_multi_launches.fetch_add(1, std::memory_order_relaxed);
+            diag::count(diag::kMultiLaunches);
             return TUNA_OK;
         }
     }
@@ -1146,13 +1140,13 @@ static int matmul_multi_impl(const tuna_gemm_problem *problems, int count, hipSt
         // the longest run of problems from `first` that one launch can take
         MultiPlan plan;
         int take = count - first < kMaxMultiProblems ? count - first : kMaxMultiProblems;
-        const int min_batch = g_multi_min_batch.load(std::memory_order_relaxed);
+        const int min_batch = diag::multi_min_batch();
         while (take >= min_batch && !plan_multi(problems + first, take, cus, &plan)) --take;
         if (take >= min_batch) {
             if ((rc = provide_workspace(false, stream, plan.ws_bytes, plan.n_counters, &plan.args.ws, &plan.args.counters))) return rc;
             e = launch_gemm_multi(plan.args, plan.prefetch, dev, stream);
             if (e != hipSuccess) return hip_fail(e, "batched gemm launch");
-            g_multi_launches.fetch_add(1, std::memory_order_relaxed);
+            diag::count(diag::kMultiLaunches);
             first += take;
             continue;
         }
@@ -1204,92 +1198,12 @@ static int quantize_impl(const void *w, const void *code, void *q, void *absmax,
     return TUNA_OK;
 }
 
-// Times `iters` enqueues of `launch(i)` with HIP events on `stream`.
-template <typename F>
-static int time_loop(F launch, int n_sets, int warmup, int iters, int use_graph, hipStream_t stream, float *elapsed_ms)
-{
-    if (iters <= 0 || warmup < 0 || n_sets <= 0 || !elapsed_ms) return fail(TUNA_ERR_INVALID_ARG, "bad timing arguments");
-    int rc;
-    hipError_t e;
-    hipEvent_t t0 = nullptr, t1 = nullptr;
-    if ((e = hipEventCreate(&t0)) != hipSuccess) return hip_fail(e, "hipEventCreate");
-    if ((e = hipEventCreate(&t1)) != hipSuccess) {
-        (void)hipEventDestroy(t0);
-        return hip_fail(e, "hipEventCreate");
-    }
-    hipGraph_t graph = nullptr;
-    hipGraphExec_t exec = nullptr, tail_exec = nullptr;
-    hipGraph_t tail_graph = nullptr;
-    hipStream_t cap_stream = nullptr;
-    rc = TUNA_OK;
-    do {
-        for (int i = 0; i < warmup && !rc; ++i) rc = launch(i % n_sets, stream);
-        if (rc) break;
-        if (use_graph) {
-            // one rotation over the weight sets per graph launch; capture on a private
-            // stream so that the caller's stream (possibly the default one) is untouched
-            if ((e = hipStreamCreateWithFlags(&cap_stream, hipStreamNonBlocking)) != hipSuccess) { rc = hip_fail(e, "hipStreamCreate"); break; }
-            if ((e = hipStreamSynchronize(stream)) != hipSuccess) { rc = hip_fail(e, "hipStreamSynchronize"); break; }
-            for (int i = 0; i < n_sets && !rc; ++i) rc = launch(i, cap_stream);  // workspace for cap_stream grows here, before capture
-            if (rc) break;
-            if ((e = hipStreamSynchronize(cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipStreamSynchronize"); break; }
-            if ((e = hipStreamBeginCapture(cap_stream, hipStreamCaptureModeThreadLocal)) != hipSuccess) { rc = hip_fail(e, "hipStreamBeginCapture"); break; }
-            for (int i = 0; i < n_sets && !rc; ++i) rc = launch(i, cap_stream);
-            e = hipStreamEndCapture(cap_stream, &graph);
-            if (rc) break;
-            if (e != hipSuccess) { rc = hip_fail(e, "hipStreamEndCapture"); break; }
-            if ((e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0)) != hipSuccess) { rc = hip_fail(e, "hipGraphInstantiate"); break; }
-            // exactly `iters` timed launches: `iters / n_sets` replays of the rotation and, when that leaves a
-            // remainder, one replay of a second graph that holds the first `iters % n_sets` launches of it
-            const int reps = iters / n_sets, rest = iters % n_sets;
-            if (rest > 0) {
-                if ((e = hipStreamBeginCapture(cap_stream, hipStreamCaptureModeThreadLocal)) != hipSuccess) { rc = hip_fail(e, "hipStreamBeginCapture"); break; }
-                for (int i = 0; i < rest && !rc; ++i) rc = launch(i, cap_stream);
-                e = hipStreamEndCapture(cap_stream, &tail_graph);
-                if (rc) break;
-                if (e != hipSuccess) { rc = hip_fail(e, "hipStreamEndCapture"); break; }
-                if ((e = hipGraphInstantiate(&tail_exec, tail_graph, nullptr, nullptr, 0)) != hipSuccess) { rc = hip_fail(e, "hipGraphInstantiate"); break; }
-                if ((e = hipGraphLaunch(tail_exec, cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipGraphLaunch"); break; }
-            }
-            if ((e = hipGraphLaunch(exec, cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipGraphLaunch"); break; }
-            if ((e = hipEventRecord(t0, cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipEventRecord"); break; }
-            for (int r = 0; r < reps; ++r)
-                if ((e = hipGraphLaunch(exec, cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipGraphLaunch"); break; }
-            if (rc) break;
-            if (rest > 0 && (e = hipGraphLaunch(tail_exec, cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipGraphLaunch"); break; }
-            if ((e = hipEventRecord(t1, cap_stream)) != hipSuccess) { rc = hip_fail(e, "hipEventRecord"); break; }
-            if ((e = hipEventSynchronize(t1)) != hipSuccess) { rc = hip_fail(e, "hipEventSynchronize"); break; }
-            if ((e = hipEventElapsedTime(elapsed_ms, t0, t1)) != hipSuccess) { rc = hip_fail(e, "hipEventElapsedTime"); break; }
-        } else {
-            if ((e = hipEventRecord(t0, stream)) != hipSuccess) { rc = hip_fail(e, "hipEventRecord"); break; }
-            for (int i = 0; i < iters && !rc; ++i) rc = launch((warmup + i) % n_sets, stream);
-            if (rc) break;
-            if ((e = hipEventRecord(t1, stream)) != hipSuccess) { rc = hip_fail(e, "hipEventRecord"); break; }
-            if ((e = hipEventSynchronize(t1)) != hipSuccess) { rc = hip_fail(e, "hipEventSynchronize"); break; }
-            if ((e = hipEventElapsedTime(elapsed_ms, t0, t1)) != hipSuccess) { rc = hip_fail(e, "hipEventElapsedTime"); break; }
-        }
-    } while (0);
-    if (exec) (void)hipGraphExecDestroy(exec);
-    if (graph) (void)hipGraphDestroy(graph);
-    if (tail_exec) (void)hipGraphExecDestroy(tail_exec);
-    if (tail_graph) (void)hipGraphDestroy(tail_graph);
-    if (cap_stream) {
-        (void)hipStreamSynchronize(cap_stream);
-        drop_workspace(cap_stream);
-        (void)hipStreamDestroy(cap_stream);
-    }
-    (void)hipEventDestroy(t0);
-    (void)hipEventDestroy(t1);
-    return rc;
-}
-
 }  // namespace tuna
 
 using namespace tuna;
 
 extern "C" {
 
-#define TUNA_EXPORT __attribute__((visibility("default")))
 
 TUNA_EXPORT int tuna_version(void) { return TUNA_AMD_VERSION; }
 
@@ -1374,13 +1288,13 @@ TUNA_EXPORT int tuna_matmul_multi_blockwise(const tuna_gemm_problem *problems, i
     for (int first = 0; first < count;) {
         MultiPlan plan;
         int take = count - first < kMaxMultiProblems ? count - first : kMaxMultiProblems;
-        const int min_batch = g_multi_min_batch.load(std::memory_order_relaxed);
+        const int min_batch = diag::multi_min_batch();
         while (take >= min_batch && !plan_multi(problems + first, take, cus, &plan, 0, 0, shift)) --take;
         if (take >= min_batch) {
             if ((rc = provide_workspace(false, st, plan.ws_bytes, plan.n_counters, &plan.args.ws, &plan.args.counters))) return rc;
             e = launch_gemm_multi(plan.args, plan.prefetch, dev, st);
             if (e != hipSuccess) return hip_fail(e, "batched blockwise gemm launch");
-            g_multi_launches.fetch_add(1, std::memory_order_relaxed);
+            diag::count(diag::kMultiLaunches);
             first += take;
             continue;
         }
@@ -1448,7 +1362,7 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
     if ((rc = check_ptr(q, "q", 16)) || (rc = check_ptr(x, "x", 16)) || (rc = check_ptr(code, "code", 4)) ||
         (rc = check_ptr(absmax, "absmax", 4)) || (rc = check_ptr(out, "out", 16)))
         return rc;
-    const int stream_mode = g_blockwise_stream.load(std::memory_order_relaxed);
+    const int stream_mode = diag::blockwise_stream();
     // Up to 64 tokens, shapes whose per-row table entry is an unsplit launch of the streaming kernel (the large ones):
     // that kernel's scale-block twin with the entry's workgroup shape, ring, x chunk and stagger (in whole x chunks; register ring).
     if (n <= 64 && (stream_mode == 3 || (stream_mode == 1 && mid_blockwise_wins(m, n, k)))) {
@@ -1490,7 +1404,7 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
             plan.args.residual = nullptr;
             e = launch_gemm_mid_blockwise(plan, shift, dev, cus, static_cast<hipStream_t>(stream));
             if (e != hipSuccess) return hip_fail(e, "streaming blockwise gemm launch");
-            g_blockwise_launches[3].fetch_add(1, std::memory_order_relaxed);
+            diag::count(diag::kBlockwiseMid);
             return TUNA_OK;
         }
     }
@@ -1529,7 +1443,7 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
             if (tp.ws_bytes && (rc = provide_workspace(false, st, tp.ws_bytes, tp.n_counters, &tp.args.ws, &tp.args.counters))) return rc;
             hipError_t e = launch_gemm_tiled(tp.args, tp.tile_rows, tp.tile_tokens, false, st, true);
             if (e != hipSuccess) return hip_fail(e, "many-token blockwise gemm launch");
-            g_blockwise_launches[2].fetch_add(1, std::memory_order_relaxed);
+            diag::count(diag::kBlockwiseTiled);
             return TUNA_OK;
         }
     }
@@ -1582,13 +1496,13 @@ TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *
                 if ((rc = provide_workspace(false, st, plan.ws_bytes, plan.n_counters, &plan.args.ws, &plan.args.counters))) return rc;
                 e = launch_gemm_multi(plan.args, plan.prefetch, dev, st);
                 if (e != hipSuccess) return hip_fail(e, "blockwise gemm launch");
-                g_multi_launches.fetch_add(1, std::memory_order_relaxed);
-                g_blockwise_launches[1].fetch_add(1, std::memory_order_relaxed);
+                diag::count(diag::kMultiLaunches);
+                diag::count(diag::kBlockwiseMulti);
             }
             return TUNA_OK;
         }
     }
-    g_blockwise_launches[0].fetch_add(1, std::memory_order_relaxed);
+    diag::count(diag::kBlockwiseNarrow);
     NarrowArgs a;
     memset(&a, 0, sizeof(a));
     a.q = static_cast<const uint8_t *>(q);
@@ -1805,111 +1719,6 @@ TUNA_EXPORT int tuna_config_table_entry(int i, int *m, int *n_lo, int *n_hi, int
     return TUNA_OK;
 }
 
-TUNA_EXPORT int tuna_time_matmul(const void *const *q_list, const void *const *absmax_list, int n_sets, const void *x,
-                                 const void *code, void *out, int m, int n, int k, const tuna_gemm_config *cfg,
-                                 int decode_mode, int warmup, int iters, int use_graph, void *stream, float *elapsed_ms)
-{
-    if (!q_list || !absmax_list) return fail(TUNA_ERR_INVALID_ARG, "q_list / absmax_list is null");
-    auto launch = [&](int set, hipStream_t s) {
-        return matmul_impl(q_list[set], x, code, absmax_list[set], out, m, n, k, cfg, decode_mode, s);
-    };
-    return time_loop(launch, n_sets, warmup, iters, use_graph, static_cast<hipStream_t>(stream), elapsed_ms);
-}
-
-TUNA_EXPORT int tuna_time_matmul_multi(const tuna_gemm_problem *problems, int n_sets, int count, int warmup, int iters,
-                                       int use_graph, void *stream, float *elapsed_ms)
-{
-    if (!problems || count < 1) return fail(TUNA_ERR_INVALID_ARG, "problems is null or count < 1");
-    auto launch = [&](int set, hipStream_t s) { return matmul_multi_impl(problems + (size_t)set * count, count, s); };
-    return time_loop(launch, n_sets, warmup, iters, use_graph, static_cast<hipStream_t>(stream), elapsed_ms);
-}
-
-TUNA_EXPORT int tuna_time_matmul_grouped(const void *const *q_list, const void *const *absmax_list, int n_sets, const void *x,
-                                         const void *code, void *out, int m_group, int n_groups, int k,
-                                         const int32_t *token_offsets, const tuna_gemm_config *cfg, int decode_mode,
-                                         int warmup, int iters, int use_graph, void *stream, float *elapsed_ms)
-{
-    if (!q_list || !absmax_list) return fail(TUNA_ERR_INVALID_ARG, "q_list / absmax_list is null");
-    auto launch = [&](int set, hipStream_t s) {
-        return matmul_grouped_impl(q_list[set], x, code, absmax_list[set], out, m_group, n_groups, k, token_offsets, cfg,
-                                   decode_mode, s);
-    };
-    return time_loop(launch, n_sets, warmup, iters, use_graph, static_cast<hipStream_t>(stream), elapsed_ms);
-}
-
-TUNA_EXPORT int tuna_time_dequant(const void *const *q_list, const void *const *absmax_list, int n_sets, const void *code,
-                                  void *out, int m, int k, int warmup, int iters, void *stream, float *elapsed_ms)
-{
-    if (!q_list || !absmax_list) return fail(TUNA_ERR_INVALID_ARG, "q_list / absmax_list is null");
-    auto launch = [&](int set, hipStream_t s) {
-        return dequant_impl(q_list[set], absmax_list[set], code, out, m, k, k, TUNA_DECODE_DEQUANT, s);
-    };
-    return time_loop(launch, n_sets, warmup, iters, 0, static_cast<hipStream_t>(stream), elapsed_ms);
-}
-
-TUNA_EXPORT int tuna_time_copy(const void *src, void *dst, size_t bytes, int warmup, int iters, void *stream,
-                               float *elapsed_ms)
-{
-    int rc;
-    if ((rc = check_ptr(src, "src", 16)) || (rc = check_ptr(dst, "dst", 16))) return rc;
-    if (bytes == 0 || bytes % 16) return fail(TUNA_ERR_INVALID_ARG, "bytes must be a positive multiple of 16");
-    auto launch = [&](int, hipStream_t s) {
-        hipError_t e = launch_copy(src, dst, bytes, s);
-        return e == hipSuccess ? (int)TUNA_OK : hip_fail(e, "copy launch");
-    };
-    return time_loop(launch, 1, warmup, iters, 0, static_cast<hipStream_t>(stream), elapsed_ms);
-}
-
-TUNA_EXPORT int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int variant, int warmup, int iters,
-                               void *stream, float *elapsed_ms)
-{
-    int rc;
-    if ((rc = check_ptr(src, "src", 16)) || (rc = check_ptr(sink, "sink", 4))) return rc;
-    if (bytes == 0 || bytes % 16) return fail(TUNA_ERR_INVALID_ARG, "bytes must be a positive multiple of 16");
-    if (variant < 0 || variant > 5) return fail(TUNA_ERR_INVALID_ARG, "variant %d outside 0..5", variant);
-    auto launch = [&](int, hipStream_t s) {
-        hipError_t e = launch_read(src, sink, bytes, blocks, variant, s);
-        return e == hipSuccess ? (int)TUNA_OK : hip_fail(e, "read launch");
-    };
-    return time_loop(launch, 1, warmup, iters, 0, static_cast<hipStream_t>(stream), elapsed_ms);
-}
-
-TUNA_EXPORT int tuna_time_unit_rate(int unit, void *sink, int warmup, int iters, void *stream, float *elapsed_ms,
-                                    double *work_per_launch)
-{
-    int rc;
-    if ((rc = check_ptr(sink, "sink", 4))) return rc;
-    if (unit < 0 || unit > 16) return fail(TUNA_ERR_INVALID_ARG, "unit %d outside 0..16", unit);
-    if (!work_per_launch) return fail(TUNA_ERR_INVALID_ARG, "work_per_launch is null");
-    int dev = 0, cus = 0;
-    hipError_t e = device_cus(&dev, &cus);
-    if (e != hipSuccess) return hip_fail(e, "device query");
-    auto launch = [&](int, hipStream_t s) {
-        hipError_t e2 = launch_unit_rate(unit, cus, static_cast<uint32_t *>(sink), work_per_launch, s);
-        return e2 == hipSuccess ? (int)TUNA_OK : hip_fail(e2, "unit-rate launch");
-    };
-    return time_loop(launch, 1, warmup, iters, 0, static_cast<hipStream_t>(stream), elapsed_ms);
-}
-
-TUNA_EXPORT unsigned long long tuna_blockwise_launches(int kernel)
-{
-    return kernel >= 0 && kernel < 4 ? g_blockwise_launches[kernel].load(std::memory_order_relaxed) : 0ull;
-}
-
-TUNA_EXPORT int tuna_set_blockwise_stream(int enabled)
-{
-    return g_blockwise_stream.exchange(enabled < 0 ? 0 : enabled > 3 ? 3 : enabled, std::memory_order_relaxed);
-}
-
-TUNA_EXPORT int tuna_set_blockwise_scales_lds(int enabled) { return set_blockwise_scales_lds(enabled); }
-
-TUNA_EXPORT int tuna_set_blockwise_shape(int rows, int waves_k, int prefetch)
-{
-    if (set_blockwise_shape(rows, waves_k, prefetch))
-        return fail(TUNA_ERR_INVALID_ARG, "no blockwise GEMM variant with %d rows, %d waves, ring %d", rows, waves_k, prefetch);
-    return TUNA_OK;
-}
-
 TUNA_EXPORT int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config *cfg, int decode_mode, char *buf, size_t len)
 {
     if (!buf || len < 16) return fail(TUNA_ERR_INVALID_ARG, "buf is null or shorter than 16 bytes");
@@ -1950,36 +1759,6 @@ TUNA_EXPORT int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config
     describe_gemm_launch(plan, cus, buf, len);
     return TUNA_OK;
 }
-
-TUNA_EXPORT int tuna_selftest_quantizer_division(void *counts, void *stream)
-{
-    int rc = check_ptr(counts, "counts", 8);
-    if (rc) return rc;
-    hipError_t e = launch_division_selftest(static_cast<unsigned long long *>(counts), static_cast<hipStream_t>(stream));
-    if (e != hipSuccess) return hip_fail(e, "selftest launch");
-    return TUNA_OK;
-}
-
-TUNA_EXPORT int tuna_set_multi_shape(int waves_m, int prefetch)
-{
-    g_multi_waves_m.store(waves_m);
-    g_multi_prefetch.store(prefetch);
-    return TUNA_OK;
-}
-
-TUNA_EXPORT int tuna_set_multi_weight_path(int through_lds) { return g_multi_lds.exchange(through_lds ? 1 : 0); }
-
-TUNA_EXPORT int tuna_set_multi_min_batch(int count)
-{
-    return g_multi_min_batch.exchange(count < 1 ? 1 : count);
-}
-
-TUNA_EXPORT unsigned long long tuna_multi_launches(void) { return g_multi_launches.load(); }
-
-TUNA_EXPORT int tuna_set_lean_kernels(int enabled) { return tuna::set_lean_kernels(enabled ? 1 : 0); }
-TUNA_EXPORT int tuna_set_weight_path(int through_lds) { return tuna::set_weight_path(through_lds ? 1 : 0); }
-
-TUNA_EXPORT unsigned long long tuna_lean_launches(void) { return tuna::lean_launches(); }
 
 TUNA_EXPORT int tuna_release_workspaces(void)
 {

@@ -14,6 +14,7 @@
 //     fp32 multiply + round (TUNA_DECODE_DEQUANT, kernel.cu:3222-3228) or an fp16
 //     multiply (TUNA_DECODE_GEMM, kernel.cu:2178-2192).
 #include "tuna_internal.h"
+#include "quantize_div.hpp"
 
 #include <type_traits>
 
@@ -115,270 +116,6 @@ hipError_t launch_dequant(const uint8_t *q, const float *absmax, const float *co
     return hipGetLastError();
 }
 
-// Plain copy: the known-traffic yardstick for the HBM counters.
-__global__ __launch_bounds__(256) void copy_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst, size_t n16)
-{
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride)
-        __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
-}
-
-// Read-only stream: the ceiling a pure HBM reader reaches on this device.  UNROLL loads of 16
-// bytes in flight per lane (UNROLL * 4 KB per workgroup and step), blocks walk the buffer in
-// lockstep; NT selects nontemporal (streaming) or plain loads.
-template <int UNROLL, bool NT>
-__global__ __launch_bounds__(256) void read_kernel(const u32x4 *__restrict__ src, uint32_t *__restrict__ sink, size_t n16)
-{
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    u32x4 acc = u32x4{0u, 0u, 0u, 0u};
-    for (; i + (UNROLL - 1) * stride < n16; i += UNROLL * stride) {
-        u32x4 v[UNROLL];
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) v[u] = NT ? __builtin_nontemporal_load(src + i + u * stride) : src[i + u * stride];
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) acc ^= v[u];
-    }
-    for (; i < n16; i += stride) acc ^= NT ? __builtin_nontemporal_load(src + i) : src[i];
-    const uint32_t r = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
-    if (r == 0x9e3779b9u) sink[0] = r;  // practically never: keeps the loads alive
-}
-
-// variant: 0 nontemporal x8 (default), 1 plain x8, 2 nontemporal x16, 3 plain x16, 4 nontemporal x4, 5 plain x4
-hipError_t launch_read(const void *src, void *sink, size_t bytes, int blocks, int variant, hipStream_t stream)
-{
-    const size_t n16 = bytes / 16;
-    if (blocks <= 0) blocks = 256 * 8;
-    const u32x4 *s = reinterpret_cast<const u32x4 *>(src);
-    uint32_t *k = reinterpret_cast<uint32_t *>(sink);
-    const dim3 grid((unsigned)blocks), block(256);
-    switch (variant) {
-    case 0: hipLaunchKernelGGL((read_kernel<8, true>), grid, block, 0, stream, s, k, n16); break;
-    case 1: hipLaunchKernelGGL((read_kernel<8, false>), grid, block, 0, stream, s, k, n16); break;
-    case 2: hipLaunchKernelGGL((read_kernel<16, true>), grid, block, 0, stream, s, k, n16); break;
-    case 3: hipLaunchKernelGGL((read_kernel<16, false>), grid, block, 0, stream, s, k, n16); break;
-    case 4: hipLaunchKernelGGL((read_kernel<4, true>), grid, block, 0, stream, s, k, n16); break;
-    case 5: hipLaunchKernelGGL((read_kernel<4, false>), grid, block, 0, stream, s, k, n16); break;
-    default: return hipErrorInvalidValue;
-    }
-    return hipGetLastError();
-}
-
-// ---- unit rates: what the matrix cores and the LDS of this device deliver to the access patterns the
-// many-token kernel uses, measured the way the read kernel measures HBM --------------------------------
-typedef float rate_f32x16 __attribute__((ext_vector_type(16)));
-typedef float rate_f32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t rate_u32x2 __attribute__((ext_vector_type(2)));
-constexpr int kRateIters = 4096;
-
-// Independent MFMAs back to back, nothing else: NACC accumulators per wave, 4 waves per workgroup.  RANDOM: the
-// operands are four + four registers of pseudo-random fp16 values in (-1, 1) instead of one pair of small
-// regular numbers - what the matrix cores draw, and the clock they are then given, depends on the bits that toggle.
-template <bool M32, int NACC, bool RANDOM = false>
-__global__ __launch_bounds__(256) void mfma_rate_kernel(uint32_t *sink)
-{
-    constexpr int NOP = RANDOM ? 4 : 1;
-    f16x8 a[NOP], b[NOP];
-#pragma unroll
-    for (int o = 0; o < NOP; ++o)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            if constexpr (RANDOM) {
-                uint32_t h = (threadIdx.x * 8u + e + o * 4099u + blockIdx.x * 131071u) * 2654435761u;
-                h ^= h >> 15, h *= 2246822519u, h ^= h >> 13;
-                a[o][e] = (f16)((float)(int)(h & 0xffffu) * (1.0f / 32768.0f) - 1.0f);
-                b[o][e] = (f16)((float)(int)(h >> 16) * (1.0f / 32768.0f) - 1.0f);
-            } else {
-                a[o][e] = (f16)(0.001f * (float)threadIdx.x + (float)e);
-                b[o][e] = (f16)(0.5f * (float)e);
-            }
-        }
-    float s = 0.f;
-    if constexpr (M32) {
-        rate_f32x16 acc[NACC];
-#pragma unroll
-        for (int i = 0; i < NACC; ++i)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
-        for (int it = 0; it < kRateIters; ++it)
-#pragma unroll
-            for (int i = 0; i < NACC; ++i)
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[(i >> 2) % NOP], b[i % NOP], acc[i], 0, 0, 0);
-#pragma unroll
-        for (int i = 0; i < NACC; ++i)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) s += acc[i][e];
-    } else {
-        rate_f32x4 acc[NACC];
-#pragma unroll
-        for (int i = 0; i < NACC; ++i) acc[i] = rate_f32x4{0.f, 0.f, 0.f, 0.f};
-        for (int it = 0; it < kRateIters; ++it)
-#pragma unroll
-            for (int i = 0; i < NACC; ++i)
-                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[(i >> 2) % NOP], b[i % NOP], acc[i], 0, 0, 0);
-#pragma unroll
-        for (int i = 0; i < NACC; ++i) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
-    }
-    if (s == 12345.678f) sink[0] = 1u;  // practically never: keeps the chain alive
-}
-
-// LDS traffic of 8 (THREADS = 1024: 16) waves per CU, eight accesses per wave and iteration, addresses opaque to
-// the compiler.
-// MODE 0: 16-byte reads the way a wave reads an MFMA fragment from a tile of 128-byte rows (lane = row 0..15 x
-// k-group, slot ^ (row & 7)); 1: 4-byte reads the way the decode reads the byte-pair table ((byte << 8) | (lane
-// << 2), byte from a counter); 2: 16-byte writes the way the decoded weights are stored (4 rows x 8 k-blocks
-// per 32 lanes); 3: the same bytes as two 8-byte writes each; 4: 16-byte writes at consecutive addresses; 5 / 6:
-// the table reads of 1 with one copy of the table per 32 / 16 lanes and a pseudo-random byte per lane.
-template <int MODE, int THREADS = 512>
-__global__ __launch_bounds__(THREADS) void lds_rate_kernel(uint32_t *sink)
-{
-    extern __shared__ __align__(16) unsigned char smem[];
-    for (int i = threadIdx.x; i < 65536 / 4; i += THREADS) reinterpret_cast<uint32_t *>(smem)[i] = (uint32_t)i;
-    __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    uint32_t s = 0;
-    if constexpr (MODE == 0) {
-        const int row = lane & 15, g = lane >> 4;
-        const uint32_t base = (uint32_t)(row * 128 + ((g ^ (row & 7)) << 4) + wave * 4096);
-        for (int it = 0; it < kRateIters; ++it)
-#pragma unroll
-            for (int r = 0; r < 8; ++r) {
-                uint32_t off = (base + r * 2048 + (it & 1) * 32768) & 65535u;
-                asm volatile("" : "+v"(off));
-                const u32x4 v = *reinterpret_cast<const u32x4 *>(smem + off);
-                s += v[0] ^ v[1] ^ v[2] ^ v[3];
-            }
-    } else if constexpr (MODE == 1) {
-        for (int it = 0; it < kRateIters; ++it)
-#pragma unroll
-            for (int r = 0; r < 8; ++r) {
-                uint32_t off = ((uint32_t)((it * 8 + r + wave * 31) & 255) << 8) | ((uint32_t)lane << 2);
-                asm volatile("" : "+v"(off));
-                s += *reinterpret_cast<const uint32_t *>(smem + off);
-            }
-    } else if constexpr (MODE == 5 || MODE == 6) {
-        constexpr int REP = MODE == 5 ? 32 : 16;  // lanes that have a copy of the table of their own
-        for (int it = 0; it < kRateIters; ++it)
-#pragma unroll
-            for (int r = 0; r < 8; ++r) {
-                uint32_t off = ((uint32_t)(((it * 8 + r) * 37 + wave * 31 + lane * lane * 13 + (lane >> 3)) & 255) * (REP * 4)) | ((uint32_t)(lane % REP) << 2);
-                asm volatile("" : "+v"(off));
-                s += *reinterpret_cast<const uint32_t *>(smem + off);
-            }
-    } else if constexpr (MODE == 3) {
-        const int half = lane & 1, kb = (lane >> 1) & 7, mbl = lane >> 4;
-        rate_u32x2 v = {(uint32_t)threadIdx.x, 1u};
-        for (int it = 0; it < kRateIters; ++it) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = mbl * 8 + half * 4 + ((r >> 1) & 3);
-                uint32_t off = (uint32_t)(row * 128 + ((kb ^ (row & 7)) << 4) + (r & 1) * 8 + wave * 4096 + ((it + (r >> 3)) & 1) * 32768) & 65535u;
-                asm volatile("" : "+v"(off));
-                *reinterpret_cast<rate_u32x2 *>(smem + off) = v;
-            }
-            v[0] += 1u;
-        }
-        __syncthreads();
-        s = smem[threadIdx.x];
-    } else if constexpr (MODE == 4) {
-        u32x4 v = {(uint32_t)threadIdx.x, 1u, 2u, 3u};
-        for (int it = 0; it < kRateIters; ++it) {
-#pragma unroll
-            for (int r = 0; r < 8; ++r) {
-                uint32_t off = (uint32_t)(lane * 16 + r * 1024 + wave * 8192) & 65535u;
-                asm volatile("" : "+v"(off));
-                *reinterpret_cast<u32x4 *>(smem + off) = v;
-            }
-            v[0] += 1u;
-        }
-        __syncthreads();
-        s = smem[threadIdx.x];
-    } else {
-        const int half = lane & 1, kb = (lane >> 1) & 7, mbl = lane >> 4;
-        u32x4 v = {(uint32_t)threadIdx.x, 1u, 2u, 3u};
-        for (int it = 0; it < kRateIters; ++it) {
-#pragma unroll
-            for (int r = 0; r < 8; ++r) {
-                const int row = mbl * 8 + half * 4 + (r & 3);
-                uint32_t off = (uint32_t)(row * 128 + ((kb ^ (row & 7)) << 4) + wave * 4096 + ((it + (r >> 2)) & 1) * 32768) & 65535u;
-                asm volatile("" : "+v"(off));
-                *reinterpret_cast<u32x4 *>(smem + off) = v;
-            }
-            v[0] += 1u;
-        }
-        __syncthreads();
-        s = smem[threadIdx.x];
-    }
-    if (s == 0x9e3779b9u && sink[1] == 77u) sink[0] = s;  // practically never
-}
-
-// unit: 0 / 1 v_mfma_f32_16x16x32_f16 with one / two waves per SIMD (16 accumulators), 2 v_mfma_f32_32x32x16_f16
-// (one wave per SIMD, 4 accumulators); 3 LDS fragment reads, 4 LDS table reads, 5 LDS tile writes, 6 the tile
-// writes as 8-byte halves, 7 16-byte writes at consecutive addresses, 8 / 9 table reads with a copy of the table
-// per 32 / 16 lanes; 10 / 13 32x32x16 and 12 / 11 16x16x32 MFMAs on pseudo-random operands from one / two waves per
-// SIMD; 14 / 15 / 16: units 4 / 3 / 5 from 16 waves per compute unit.  *work = flops (0..2, 10..13) or bytes
-// (3..9, 14..16) of one launch on `cus` compute units.
-hipError_t launch_unit_rate(int unit, int cus, uint32_t *sink, double *work, hipStream_t stream)
-{
-    static OptInFlag attr[16][10];
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
-    switch (unit) {
-    case 0: hipLaunchKernelGGL((mfma_rate_kernel<false, 16>), dim3(cus), dim3(256), 0, stream, sink); *work = (double)cus * 4 * kRateIters * 16 * 16384.0; break;
-    case 1: hipLaunchKernelGGL((mfma_rate_kernel<false, 16>), dim3(2 * cus), dim3(256), 0, stream, sink); *work = (double)cus * 8 * kRateIters * 16 * 16384.0; break;
-    case 2: hipLaunchKernelGGL((mfma_rate_kernel<true, 4>), dim3(cus), dim3(256), 0, stream, sink); *work = (double)cus * 4 * kRateIters * 4 * 32768.0; break;
-    case 3:
-        if ((e = ensure_lds_opt_in(attr[dev][0], reinterpret_cast<const void *>(lds_rate_kernel<0>))) != hipSuccess) return e;
-        hipLaunchKernelGGL(lds_rate_kernel<0>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 16.0; break;
-    case 4:
-        if ((e = ensure_lds_opt_in(attr[dev][1], reinterpret_cast<const void *>(lds_rate_kernel<1>))) != hipSuccess) return e;
-        hipLaunchKernelGGL(lds_rate_kernel<1>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 4.0; break;
-    case 5:
-        if ((e = ensure_lds_opt_in(attr[dev][2], reinterpret_cast<const void *>(lds_rate_kernel<2>))) != hipSuccess) return e;
-        hipLaunchKernelGGL(lds_rate_kernel<2>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 16.0; break;
-    case 6:
-        if ((e = ensure_lds_opt_in(attr[dev][3], reinterpret_cast<const void *>(lds_rate_kernel<3>))) != hipSuccess) return e;
-        hipLaunchKernelGGL(lds_rate_kernel<3>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 16.0; break;
-    case 7:
-        if ((e = ensure_lds_opt_in(attr[dev][4], reinterpret_cast<const void *>(lds_rate_kernel<4>))) != hipSuccess) return e;
-        hipLaunchKernelGGL(lds_rate_kernel<4>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 16.0; break;
-    case 10: hipLaunchKernelGGL((mfma_rate_kernel<true, 16, true>), dim3(cus), dim3(256), 0, stream, sink); *work = (double)cus * 4 * kRateIters * 16 * 32768.0; break;
-    case 11: hipLaunchKernelGGL((mfma_rate_kernel<false, 16, true>), dim3(2 * cus), dim3(256), 0, stream, sink); *work = (double)cus * 8 * kRateIters * 16 * 16384.0; break;
-    case 12: hipLaunchKernelGGL((mfma_rate_kernel<false, 16, true>), dim3(cus), dim3(256), 0, stream, sink); *work = (double)cus * 4 * kRateIters * 16 * 16384.0; break;
-    case 13: hipLaunchKernelGGL((mfma_rate_kernel<true, 16, true>), dim3(2 * cus), dim3(256), 0, stream, sink); *work = (double)cus * 8 * kRateIters * 16 * 32768.0; break;
-    case 14:
-        if ((e = ensure_lds_opt_in(attr[dev][7], reinterpret_cast<const void *>(lds_rate_kernel<1, 1024>))) != hipSuccess) return e;
-        hipLaunchKernelGGL((lds_rate_kernel<1, 1024>), dim3(cus), dim3(1024), 65536, stream, sink); *work = (double)cus * 1024 * kRateIters * 8 * 4.0; break;
-    case 15:
-        if ((e = ensure_lds_opt_in(attr[dev][8], reinterpret_cast<const void *>(lds_rate_kernel<0, 1024>))) != hipSuccess) return e;
-        hipLaunchKernelGGL((lds_rate_kernel<0, 1024>), dim3(cus), dim3(1024), 65536, stream, sink); *work = (double)cus * 1024 * kRateIters * 8 * 16.0; break;
-    case 16:
-        if ((e = ensure_lds_opt_in(attr[dev][9], reinterpret_cast<const void *>(lds_rate_kernel<2, 1024>))) != hipSuccess) return e;
-        hipLaunchKernelGGL((lds_rate_kernel<2, 1024>), dim3(cus), dim3(1024), 65536, stream, sink); *work = (double)cus * 1024 * kRateIters * 8 * 16.0; break;
-    case 8:
-        if ((e = ensure_lds_opt_in(attr[dev][5], reinterpret_cast<const void *>(lds_rate_kernel<5>))) != hipSuccess) return e;
-        hipLaunchKernelGGL(lds_rate_kernel<5>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 4.0; break;
-    case 9:
-        if ((e = ensure_lds_opt_in(attr[dev][6], reinterpret_cast<const void *>(lds_rate_kernel<6>))) != hipSuccess) return e;
-        hipLaunchKernelGGL(lds_rate_kernel<6>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 4.0; break;
-    default: return hipErrorInvalidValue;
-    }
-    return hipGetLastError();
-}
-
-hipError_t launch_copy(const void *src, void *dst, size_t bytes, hipStream_t stream)
-{
-    const size_t n16 = bytes / 16;
-    size_t blocks = (n16 + 255) / 256;
-    if (blocks > 256 * 32) blocks = 256 * 32;
-    if (blocks == 0) blocks = 1;
-    hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
-                       reinterpret_cast<const u32x4 *>(src), reinterpret_cast<u32x4 *>(dst), n16);
-    return hipGetLastError();
-}
-
 // fp16 weights [m, k] -> packed 4-bit codes + absmax: the device form of the reference harness's
 // quantize_blockwise_dynamic_4bit (test.py:7-68).  Same arithmetic: absmax = max |w| over a block of
 // `bs` consecutive weights of a row as fp32 (bs == k: one scale per row, what the kernels of the
@@ -400,24 +137,6 @@ hipError_t launch_copy(const void *src, void *dst, size_t bytes, hipStream_t str
 // The division by the block maximum is a multiply by its refined reciprocal and one fused correction.  A thread's dword (one row, 8
 // consecutive k) is written through a 2 KB LDS tile so that the stores are 16 bytes per lane and
 // contiguous (the records of 64 block columns), not 4 bytes at a stride of 32.
-// fp32(w) / a, correctly rounded, for the quotients this kernel forms: w an fp16 value, a the
-// largest |fp16| of its block, so |w| <= a and both are normal binary32 numbers (or w is zero).
-// y is the reciprocal of a refined once from v_rcp_f32 (computed once per block); the quotient is one
-// multiply and one fused correction step.  No denormal-mode switches, no scaling: the ranges rule
-// out what the general division sequence guards against.  Equality with the IEEE division is
-// checked for every pair (w, a) of fp16 values with |w| <= a in tests/test_gpu_parity.py.
-__device__ __forceinline__ float refined_rcp(float a)
-{
-    const float y = __builtin_amdgcn_rcpf(a);
-    return __builtin_fmaf(__builtin_fmaf(-a, y, 1.0f), y, y);
-}
-
-__device__ __forceinline__ float div_by_block_max(float w, float a, float y)
-{
-    const float q = w * y;
-    return __builtin_fmaf(__builtin_fmaf(-q, a, w), y, q);
-}
-
 // Nearest entry of a sorted codebook: bnd[i] (i = 0..14) is the smallest binary32 value that the
 // argmin assigns to entry i + 1 rather than entry i, so the index is the number of boundaries <= nv:
 // a 4-step binary search, as a tree of selects over the 15 values (uniform, held in registers).
@@ -720,36 +439,6 @@ __global__ __launch_bounds__(512, NP == 16 ? 2 : 4) void quantize_kernel(const f
     if (tabled) run(std::integral_constant<int, 0>{});
     else if (fast) run(std::integral_constant<int, 1>{});
     else run(std::integral_constant<int, 2>{});
-}
-
-// Self-test of div_by_block_max: every pair of fp16 values (w, a) with a > 0 finite and |w| <= a,
-// against the IEEE division (zeros of either sign count as equal).  One workgroup per value of a;
-// counts[0] += pairs, counts[1] += mismatches.
-__global__ __launch_bounds__(256) void division_selftest_kernel(unsigned long long *counts)
-{
-    const uint16_t abits = (uint16_t)(blockIdx.x + 1);  // 0x0001 .. 0x7bff: every positive finite fp16
-    const float a = (float)__builtin_bit_cast(f16, abits);
-    const float y = refined_rcp(a);
-    unsigned long long n = 0, bad = 0;
-    for (uint32_t wb = threadIdx.x; wb < 65536u; wb += 256u) {
-        const uint16_t mag = (uint16_t)(wb & 0x7fffu);
-        if (mag > abits) continue;  // |w| > a, infinities, NaNs
-        const float w = (float)__builtin_bit_cast(f16, (uint16_t)wb);
-        const float got = div_by_block_max(w, a, y), want = __fdiv_rn(w, a);
-        ++n;
-        // (a zero quotient may come out with the other sign: -0 / a is -0, the correction step gives +0;
-        // every later use of the quotient is a comparison or a difference, where the two are one value)
-        const bool same = __builtin_bit_cast(uint32_t, got) == __builtin_bit_cast(uint32_t, want) || (got == 0.f && want == 0.f);
-        bad += same ? 0u : 1u;
-    }
-    atomicAdd(counts, n);
-    if (bad) atomicAdd(counts + 1, bad);
-}
-
-hipError_t launch_division_selftest(unsigned long long *counts, hipStream_t stream)
-{
-    hipLaunchKernelGGL(division_selftest_kernel, dim3(0x7bff), dim3(256), 0, stream, counts);
-    return hipGetLastError();
 }
 
 hipError_t launch_quantize(const void *w, const float *code, void *q, float *absmax, int m, int k, int bs, hipStream_t stream)

@@ -97,21 +97,11 @@ static size_t lean_lds_bytes(const GemmPlan &plan)
     return (size_t)kLutBytes + (x_bytes > red_bytes ? x_bytes : red_bytes) + 16;
 }
 
-static std::atomic<int> g_lean_enabled{1};
-static std::atomic<unsigned long long> g_lean_launches{0};
-
-unsigned long long lean_launches() { return g_lean_launches.load(); }
-
-int set_lean_kernels(int enabled)  // negative: query only
-{
-    return enabled < 0 ? g_lean_enabled.load() : g_lean_enabled.exchange(enabled ? 1 : 0);
-}
-
 // Launches the lean kernel computes exactly like the general one (conditions in gemm_lean.hpp).
 static const LeanVariant *lean_applies(const GemmPlan &plan, int cus)
 {
     const GemmArgs &a = plan.args;
-    if (!g_lean_enabled.load(std::memory_order_relaxed)) return nullptr;
+    if (!diag::lean_kernels()) return nullptr;
     if (a.group_rows || a.balanced || plan.rw != 1 || plan.token_tiles != 1 || plan.decode != TUNA_DECODE_GEMM) return nullptr;
     if (a.split_log2 < 0 || a.k_stagger != 0) return nullptr;
     if (plan.grid.x != (unsigned)a.tiles_total) return nullptr;
@@ -171,9 +161,9 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
     const Variant *v = find_variant(plan.rw, plan.prefetch, plan.token_tiles, plan.decode, plan.threads, plan.min_waves,
                                     plan.args.group_rows ? 1 : 0);
     // (deeper rings with four token tiles exist in the 17..128-token streaming kernel only)
-    if ((!v || plan.lds_weights || g_lean_enabled.load(std::memory_order_relaxed)) && mid_applies(plan)) {
+    if ((!v || plan.lds_weights || diag::lean_kernels()) && mid_applies(plan)) {
         e = launch_gemm_mid(plan, dev, cus, stream);
-        if (e == hipSuccess) g_lean_launches.fetch_add(1, std::memory_order_relaxed);
+        if (e == hipSuccess) diag::count(diag::kLeanLaunches);
         return e;
     }
     if (!v) return hipErrorInvalidConfiguration;
@@ -187,7 +177,7 @@ hipError_t launch_gemm(const GemmPlan &plan, hipStream_t stream)
                            a.k, a.n, a.steps_per_split, packed, a.m, a.out, a.residual, a.ws, a.counters,
                            a.row_tiles
         );
-        g_lean_launches.fetch_add(1, std::memory_order_relaxed);
+        diag::count(diag::kLeanLaunches);
         return hipGetLastError();
     }
     // a dense launch with a fixed split whose tiles all fit the device at once needs no tile
@@ -212,7 +202,7 @@ void describe_gemm_launch(const GemmPlan &plan, int cus, char *buf, size_t len)
     const unsigned slots = (unsigned)(cus * plan.wgs_per_cu);
     const Variant *v = find_variant(plan.rw, plan.prefetch, plan.token_tiles, plan.decode, plan.threads, plan.min_waves,
                                     plan.args.group_rows ? 1 : 0);
-    if ((!v || g_lean_enabled.load(std::memory_order_relaxed)) && mid_describe(plan, buf, len)) return;
+    if ((!v || diag::lean_kernels()) && mid_describe(plan, buf, len)) return;
     if (!v) {
         snprintf(buf, len, "none");
         return;
@@ -313,23 +303,13 @@ static const BlockwiseVariant kBlockwise[] = {
 #undef B
 #undef B2
 static constexpr int kNumBlockwise = sizeof(kBlockwise) / sizeof(kBlockwise[0]);
-static std::atomic<int> g_blockwise_shape[3];  // diagnostic override: rows, waves_k, ring depth (0: the library's choice)
-static std::atomic<int> g_blockwise_scales_lds{1};  // A/B switch: the workgroup's scales staged in LDS (1) or read from memory per step (0)
 
-int set_blockwise_scales_lds(int enabled) { return g_blockwise_scales_lds.exchange(enabled ? 1 : 0); }
-
-int set_blockwise_shape(int rows, int waves_k, int prefetch)
+bool blockwise_variant_exists(int rows, int waves_k, int prefetch)
 {
-    if (rows || waves_k || prefetch) {
-        bool found = false;
-        for (int i = 0; i < kNumBlockwise; ++i)
-            found |= kBlockwise[i].tt == 1 && kBlockwise[i].rows == rows && kBlockwise[i].wk == waves_k && kBlockwise[i].u == prefetch;
-        if (!found) return -1;
-    }
-    g_blockwise_shape[0].store(rows);
-    g_blockwise_shape[1].store(waves_k);
-    g_blockwise_shape[2].store(prefetch);
-    return 0;
+    bool found = false;
+    for (int i = 0; i < kNumBlockwise; ++i)
+        found |= kBlockwise[i].tt == 1 && kBlockwise[i].rows == rows && kBlockwise[i].wk == waves_k && kBlockwise[i].u == prefetch;
+    return found;
 }
 
 static bool blockwise_fits(const BlockwiseVariant &v, int m, int k) { return m % v.rows == 0 && k % (kStepK * v.wk * v.u) == 0; }
@@ -343,9 +323,9 @@ static size_t blockwise_scale_bytes(const BlockwiseVariant &v, int nblk) { retur
 // 144 to 256 wide workgroups beats two rounds of narrower ones, and scales read from memory cost 1.4 to 2x).
 static const BlockwiseVariant *choose_blockwise(int m, int k, int nblk, int cus, int tt)
 {
-    const int ov_rows = g_blockwise_shape[0].load();
+    const int ov_rows = diag::blockwise_shape(0);
     if (ov_rows) {
-        const int wk = g_blockwise_shape[1].load(), u = g_blockwise_shape[2].load();
+        const int wk = diag::blockwise_shape(1), u = diag::blockwise_shape(2);
         for (int t = tt; t >= 1; --t)  // (the two-tile twin of the named shape where one is built)
             for (int i = 0; i < kNumBlockwise; ++i)
                 if (kBlockwise[i].tt == t && kBlockwise[i].rows == ov_rows && kBlockwise[i].wk == wk && kBlockwise[i].u == u &&
@@ -388,7 +368,7 @@ hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, hipStrea
     const dim3 grid((unsigned)(args.m / v->rows), (unsigned)((args.n + 16 * v->tt - 1) / (16 * v->tt)), 1);
     // the workgroup's scales in LDS when they fit beside the table and the reduction planes
     const size_t scale_bytes = blockwise_scale_bytes(*v, nblk);
-    const int slds = g_blockwise_scales_lds.load(std::memory_order_relaxed) && lds + scale_bytes <= (size_t)kLdsLimit;
+    const int slds = diag::blockwise_scales_lds() && lds + scale_bytes <= (size_t)kLdsLimit;
     if (slds) lds += scale_bytes;
     hipLaunchKernelGGL(fn, grid, dim3(v->wk * 64), lds, stream, args.q, args.x, args.code, args.absmax, args.k, args.n,
                        args.k / kStepK / v->wk, args.m, args.out, TUNA_EPILOGUE_NONE, nullptr, blk_shift, nblk, slds);

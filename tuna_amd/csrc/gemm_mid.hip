@@ -48,15 +48,9 @@ static const MidVariant kMid[] = {
 #undef M10L
 static constexpr int kNumMid = sizeof(kMid) / sizeof(kMid[0]);
 
-// Diagnostic switch: 1 = launches that have an LDS-staged twin run it (tuna_set_weight_path).
-static std::atomic<int> g_weight_path{0};
-int set_weight_path(int path)
-{
-    return path < 0 ? g_weight_path.load(std::memory_order_relaxed) : g_weight_path.exchange(path ? 1 : 0, std::memory_order_relaxed);
-}
 static bool lds_path(const GemmPlan &plan)
 {
-    return (plan.lds_weights || g_weight_path.load(std::memory_order_relaxed) != 0) && (plan.threads == 512 || plan.threads == 1024) &&
+    return (plan.lds_weights || diag::weight_path() != 0) && (plan.threads == 512 || plan.threads == 1024) &&
            (plan.prefetch == 2 || plan.prefetch == 4);
 }
 

@@ -7,7 +7,9 @@
 #include <atomic>
 
 #include "../../include/tuna_amd.h"
-#include "../../include/tuna_amd_bench.h"
+#include "diag.h"
+
+#define TUNA_EXPORT __attribute__((visibility("default")))
 
 namespace tuna {
 
@@ -190,11 +192,7 @@ struct NarrowArgs {
 bool narrow_variant_exists(int rows, int waves_k, int prefetch, int token_tiles);
 hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int prefetch, int token_tiles, hipStream_t stream);
 hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, hipStream_t stream);
-int set_blockwise_shape(int rows, int waves_k, int prefetch);  // 0 on success, -1: no such variant
-int set_blockwise_scales_lds(int enabled);  // returns the previous setting
-int set_lean_kernels(int enabled);  // returns the previous setting
-int set_weight_path(int path);      // gemm_mid.hip; negative: query
-unsigned long long lean_launches();
+bool blockwise_variant_exists(int rows, int waves_k, int prefetch);  // a one-token-tile variant of the narrow-row blockwise kernel
 bool launch_is_lean(const GemmPlan &plan, int cus);  // the planned launch would take the lean kernel
 bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves, int grouped);
 
@@ -220,10 +218,13 @@ hipError_t launch_dequant(const uint8_t *q, const float *absmax, const float *co
                           int m, int k, int block_size, int decode, hipStream_t stream);
 hipError_t launch_quantize(const void *w, const float *code, void *q, float *absmax, int m, int k, int block_size,
                            hipStream_t stream);
-hipError_t launch_copy(const void *src, void *dst, size_t bytes, hipStream_t stream);
-hipError_t launch_division_selftest(unsigned long long *counts, hipStream_t stream);
-hipError_t launch_read(const void *src, void *sink, size_t bytes, int blocks, int variant, hipStream_t stream);
-hipError_t launch_unit_rate(int unit, int cus, uint32_t *sink, double *work, hipStream_t stream);
+
+// api.cpp: error reporting (the message tuna_last_error returns, per thread), argument checks and the per-stream
+// workspace, for the other host translation units
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+int hip_fail(hipError_t e, const char *what);
+int check_ptr(const void *p, const char *name, size_t align);
+void drop_workspace(hipStream_t stream);  // frees the split-K workspace of a stream that is about to be destroyed
 
 // config_table.cpp
 struct TableEntry {

@@ -335,12 +335,12 @@ def time_matmul(q_list, absmax_list, x, c, o, m, n, k, config=None, decode_mode=
     qp, _qk = _ptr_array(q_list)
     ap, _ak = _ptr_array(absmax_list)
     ms = ctypes.c_float(0)
-    L = _lib.lib()
+    L = _lib.bench_lib()
     with torch.cuda.device(x.device):
         rc = L.tuna_time_matmul(qp, ap, len(q_list), x.data_ptr(), c.data_ptr(), o.data_ptr(), int(m), int(n), int(k),
                                 ctypes.byref(config) if config is not None else None, int(decode_mode), int(warmup),
                                 int(iters), int(bool(use_graph)), _stream(x.device), ctypes.byref(ms))
-    _lib.check(rc)
+    _lib.check(rc, _lib.bench_lib())
     return ms.value
 
 
@@ -355,12 +355,12 @@ def time_matmul_grouped(q_list, absmax_list, x, c, o, m_group, n_groups, k, toke
     arr = (ctypes.c_int * (int(n_groups) + 1))(*[int(v) for v in token_offsets])
     ms = ctypes.c_float(0)
     with torch.cuda.device(x.device):
-        rc = _lib.lib().tuna_time_matmul_grouped(qp, ap, len(q_list), x.data_ptr(), c.data_ptr(), o.data_ptr(), int(m_group),
+        rc = _lib.bench_lib().tuna_time_matmul_grouped(qp, ap, len(q_list), x.data_ptr(), c.data_ptr(), o.data_ptr(), int(m_group),
                                                  int(n_groups), int(k), arr,
                                                  ctypes.byref(config) if config is not None else None, int(decode_mode),
                                                  int(warmup), int(iters), int(bool(use_graph)), _stream(x.device),
                                                  ctypes.byref(ms))
-    _lib.check(rc)
+    _lib.check(rc, _lib.bench_lib())
     return ms.value
 
 def time_matmul_multi(batches, warmup=10, iters=100, use_graph=False) -> float:
@@ -372,9 +372,9 @@ def time_matmul_multi(batches, warmup=10, iters=100, use_graph=False) -> float:
     dev = batches[0][0][0].device
     ms = ctypes.c_float(0)
     with torch.cuda.device(dev):
-        rc = _lib.lib().tuna_time_matmul_multi(arr, len(batches), count, int(warmup), int(iters), int(bool(use_graph)),
+        rc = _lib.bench_lib().tuna_time_matmul_multi(arr, len(batches), count, int(warmup), int(iters), int(bool(use_graph)),
                                                _stream(dev), ctypes.byref(ms))
-    _lib.check(rc)
+    _lib.check(rc, _lib.bench_lib())
     return ms.value
 
 
@@ -382,11 +382,11 @@ def time_dequant(q_list, absmax_list, c, o, m, k, warmup=5, iters=20) -> float:
     qp, _qk = _ptr_array(q_list)
     ap, _ak = _ptr_array(absmax_list)
     ms = ctypes.c_float(0)
-    L = _lib.lib()
+    L = _lib.bench_lib()
     with torch.cuda.device(o.device):
         rc = L.tuna_time_dequant(qp, ap, len(q_list), c.data_ptr(), o.data_ptr(), int(m), int(k), int(warmup),
                                  int(iters), _stream(o.device), ctypes.byref(ms))
-    _lib.check(rc)
+    _lib.check(rc, _lib.bench_lib())
     return ms.value
 
 
@@ -394,11 +394,11 @@ def time_copy(src, dst, warmup=5, iters=20) -> float:
     nbytes = src.numel() * src.element_size()
     assert dst.numel() * dst.element_size() >= nbytes
     ms = ctypes.c_float(0)
-    L = _lib.lib()
+    L = _lib.bench_lib()
     with torch.cuda.device(src.device):
         rc = L.tuna_time_copy(src.data_ptr(), dst.data_ptr(), nbytes, int(warmup), int(iters), _stream(src.device),
                               ctypes.byref(ms))
-    _lib.check(rc)
+    _lib.check(rc, _lib.bench_lib())
     return ms.value
 
 
@@ -407,11 +407,11 @@ def time_read(src, blocks=0, variant=0, warmup=5, iters=20) -> float:
     nbytes = src.numel() * src.element_size()
     sink = torch.zeros(4, dtype=torch.int32, device=src.device)
     ms = ctypes.c_float(0)
-    L = _lib.lib()
+    L = _lib.bench_lib()
     with torch.cuda.device(src.device):
         rc = L.tuna_time_read(src.data_ptr(), sink.data_ptr(), nbytes, int(blocks), int(variant), int(warmup), int(iters),
                               _stream(src.device), ctypes.byref(ms))
-    _lib.check(rc)
+    _lib.check(rc, _lib.bench_lib())
     return ms.value
 
 
@@ -422,9 +422,9 @@ def time_unit_rate(unit: int, device, warmup=2, iters=5):
     ms = ctypes.c_float(0)
     work = ctypes.c_double(0)
     with torch.cuda.device(device):
-        rc = _lib.lib().tuna_time_unit_rate(int(unit), sink.data_ptr(), int(warmup), int(iters), _stream(device),
+        rc = _lib.bench_lib().tuna_time_unit_rate(int(unit), sink.data_ptr(), int(warmup), int(iters), _stream(device),
                                             ctypes.byref(ms), ctypes.byref(work))
-    _lib.check(rc)
+    _lib.check(rc, _lib.bench_lib())
     return ms.value, work.value
 
 
@@ -437,17 +437,18 @@ def describe_launch(m: int, n: int, k: int, config: GemmConfig = None, decode_mo
 
 
 def set_lean_kernels(enabled: bool) -> bool:
-    """Diagnostic switch (tuna_set_lean_kernels): whether qualifying small launches use the
-    stripped-down kernel.  Results are bit-identical either way.  Returns the previous setting."""
-    return bool(_lib.lib().tuna_set_lean_kernels(int(bool(enabled))))
+    """Diagnostic switch (tuna_set_lean_kernels) of the diagnostic build: whether qualifying small launches use the
+    stripped-down kernel.  Results are bit-identical either way.  Returns the previous setting.  It applies to ops
+    called while _lib.diagnostic_build() is active; the product library has no such switch."""
+    return bool(_lib.bench_lib().tuna_set_lean_kernels(int(bool(enabled))))
 
 
 def set_weight_path(through_lds: bool) -> bool:
     """Diagnostic switch (tuna_set_weight_path): unsplit 16-wave launches of up to 16 tokens stage the
     packed weights through LDS instead of registers.  Bit-identical results.  Returns the previous setting."""
-    return bool(_lib.lib().tuna_set_weight_path(int(bool(through_lds))))
+    return bool(_lib.bench_lib().tuna_set_weight_path(int(bool(through_lds))))
 
 
 def lean_launches() -> int:
     """Diagnostic (tuna_lean_launches): GEMM launches of this process that took the stripped-down kernel."""
-    return int(_lib.lib().tuna_lean_launches())
+    return int(_lib.bench_lib().tuna_lean_launches())
