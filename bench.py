@@ -48,12 +48,17 @@ CACHE_BYTES = 256 << 20  # Infinity Cache; the rotation streams at least twice t
 # summaries under profiles/.  Keyed by shape AND by the kernel the profile was taken of: when the table or
 # the dispatcher picks another kernel for the shape, the entry no longer applies and `traffic` is null.
 MEASURED_TRAFFIC = {
-    # profiles/gemm_narrow_kernel_mistral_qkv_kernel_trace.md
-    ("mistral_qkv", "gemm_narrow_kernel<LW=2,WK=8,U=4,PERM=1,TT=1>"): (6700.5, 192.0),
-    # profiles/gemm_lean_kernel_llama70b_qkv_kernel_trace_and_counters.md
-    ("llama70b_qkv", "gemm_lean_kernel<WK=4,U=2,1024 threads> split_k=4"): (22857.5, 2886.2),
-    # profiles/gemm_mid_kernel_weights_through_lds_vs_registers.md
-    ("llama70b_gate_up", "gemm_mid_kernel<U=4,TT=1,XB=4,1024 threads,weights through LDS> x_chunk=512"): (116009.3, 1792.0),
+    # profiles/gemm_kernels_hbm_traffic_all_16_token_shapes.md
+    ("mistral_attn_out", "gemm_narrow_kernel<LW=1,WK=8,U=8,PERM=1,TT=1>"): (4666.0, 128.0),
+    ("mistral_qkv", "gemm_narrow_kernel<LW=2,WK=8,U=4,PERM=1,TT=1>"): (6707.1, 192.0),
+    ("mistral_gate_up", "gemm_mid_kernel<U=2,TT=1,XB=4,1024 threads,weights through LDS> x_chunk=512"): (29325.8, 896.0),
+    ("mistral_down", "gemm_lean_kernel<WK=4,U=2,512 threads> split_k=8"): (17215.1, 2185.0),
+    ("llama70b_qkv", "gemm_lean_kernel<WK=4,U=2,1024 threads> split_k=4"): (22859.5, 2886.2),
+    ("llama70b_attn_out", "gemm_lean_kernel<WK=4,U=8,512 threads> split_k=4"): (18547.0, 2314.0),
+    ("llama70b_gate_up", "gemm_mid_kernel<U=4,TT=1,XB=4,1024 threads,weights through LDS> x_chunk=512"): (116004.4, 1792.0),
+    ("llama70b_down", "gemm_multi_kernel<U=2> waves_m=4 waves_k=4"): (65442.8, 4361.0),
+    ("mixtral_gate_up_8e", "gemm_mid_kernel<U=4,TT=1,XB=4,1024 threads> x_chunk=1024"): (231760.9, 8960.0),
+    ("mixtral_down_8e", "gemm_mid_kernel<U=2,TT=1,XB=4,1024 threads,weights through LDS> x_chunk=512"): (116656.2, 1024.0),
 }
 
 
@@ -208,14 +213,46 @@ def copy_yardstick(ops, torch, dev, mib):
             "gbs_read_plus_write": round(2 * nb / (ms * 1e-4) / 1e9, 1)}
 
 
+def multi_stream(ops, synth, torch, dev, names=("mistral_attn_out", "mistral_qkv"), tokens=TOKENS, iters=1024):
+    """Independent GEMMs (rotating weights, one output buffer per stream) dealt round-robin to 1, 2 and 4 streams of
+    the default priority, and the empty kernel the same way: us per GEMM over all streams.  Beside the single-stream
+    headline, never instead of it: a decoder layer's GEMMs depend on each other and run on one stream."""
+    from tuna_amd.quantize import nf4_codebook
+
+    code = nf4_codebook(dev)
+    out = {"empty_kernel_us": {f"{ns}_{mode}": round(ops.time_empty_launches(dev, n_streams=ns, use_graph=mode == "graph", iters=2048) * 1000.0 / 2048, 3)
+                               for ns in (1, 2, 4) for mode in ("stream", "graph")}}
+    for nm in names:
+        m, k = synth.SHAPES[nm]
+        ns_sets = n_sets_for(m * k // 2, 2 << 30)
+        sets = [synth.make_weights_torch(m, k, 6000 + i, dev) for i in range(ns_sets)]
+        x = synth.make_x_torch(tokens, k, 5, dev)
+        row = {}
+        for ns in (1, 2, 4):
+            outs = [torch.empty((tokens, m), dtype=torch.float16, device=dev) for _ in range(ns)]
+            for mode in ("stream", "graph"):
+                args = ([s_[0] for s_ in sets], [s_[1] for s_ in sets], x, code, outs, m, tokens, k)
+                ops.time_matmul_streams(*args, warmup=50, iters=256, use_graph=mode == "graph")
+                ms = ops.time_matmul_streams(*args, warmup=50, iters=iters, use_graph=mode == "graph")
+                us = ms * 1000.0 / iters
+                row[f"{ns}_{mode}"] = {"us_per_gemm": round(us, 3), "frac_hbm": round(m * k / 2 / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+        out[nm] = row
+        del sets
+        torch.cuda.empty_cache()
+    return out
+
+
 def launch_floor(ops, torch, dev, headline_bytes):
-    tiny = torch.zeros(4096, dtype=torch.uint8, device=dev)
-    us_empty = ops.time_read(tiny, blocks=192, warmup=100, iters=1000) * 1000.0 / 1000
+    # a kernel that does nothing, 192 workgroups of 512 threads: replayed from a HIP graph (what the device needs
+    # per launch) and enqueued launch by launch (where the host's enqueue time can be the longer of the two)
+    us_empty = ops.time_empty_launches(dev, use_graph=True, iters=2000) * 1000.0 / 2000
+    us_empty_stream = ops.time_empty_launches(dev, use_graph=False, iters=2000) * 1000.0 / 2000
     sweep = read_sweep(ops, torch, dev)
     best = max(sweep, key=sweep.get)
     rate = sweep[best]
     return {
         "empty_launch_us": round(us_empty, 3),
+        "empty_launch_enqueued_one_by_one_us": round(us_empty_stream, 3),
         "read_kernel_gbs": rate,
         "read_kernel_best": best,
         "read_kernel_frac_of_peak": round(rate / HBM_PEAK_GBS, 4),
@@ -419,11 +456,12 @@ def main():
     ap.add_argument("--launch", choices=("both", "stream", "graph"), default="both")
     ap.add_argument("--settle", type=int, default=300,
                     help="untimed launches before the warm-up of the headline (a box that was idle ramps its clocks)")
-    ap.add_argument("--only", choices=("read", "dequant", "quantize", "multi", "mfma", "rates", "blockwise"), default=None,
+    ap.add_argument("--only", choices=("read", "dequant", "quantize", "multi", "mfma", "rates", "blockwise", "streams"), default=None,
                     help="profiling runs: launch only the read-kernel sweep / the dequant kernel / the quantizer / "
                          "the Llama-70B layer set through tuna_matmul_multi (16 layers) / the many-token kernel with "
                          "16x16x32 and with 32x32x16 MFMA tiles (Llama-70B gate+up and QKV, --tokens, default 1024) / the "
-                         "matrix-core and LDS yardstick kernels / the blockwise GEMM (a scale per 64 weights)")
+                         "matrix-core and LDS yardstick kernels / the blockwise GEMM (a scale per 64 weights) / the two "
+                         "smallest shapes dealt to 1, 2 and 4 streams")
     ap.add_argument("--weight-path", choices=("table", "registers", "lds"), default="table",
                     help="headline workload: the table's config as it is, or with the packed weights forced through "
                          "registers / staged through LDS (lds_tile_rows 0 / -1; A/B runs of the two weight paths)")
@@ -461,6 +499,8 @@ def main():
             res = {"quantize": time_quantize(ops, synth, torch, dev)}
         elif args.only == "rates":
             res = {"unit_rates": unit_rates(ops, dev)}
+        elif args.only == "streams":
+            res = {"headline_multi_stream": multi_stream(ops, synth, torch, dev, iters=256)}
         elif args.only == "blockwise":
             res = {"blockwise_gemm_block_64": time_blockwise(ops, synth, torch, dev)}
         elif args.only == "mfma":
@@ -525,6 +565,7 @@ def main():
     if not args.only_headline:
         line["launch_floor"] = launch_floor(ops, torch, dev, head["packed_bytes"])
         line["unit_rates"] = unit_rates(ops, dev)
+        line["headline_multi_stream"] = multi_stream(ops, synth, torch, dev)
 
     if args.copy_yardstick > 0:
         line["copy_yardstick"] = copy_yardstick(ops, torch, dev, args.copy_yardstick)

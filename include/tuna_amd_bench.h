@@ -29,6 +29,24 @@ int tuna_time_matmul(const void *const *q_list, const void *const *absmax_list, 
                      const void *x, const void *code, void *out, int m, int n, int k,
                      const tuna_gemm_config *cfg, int decode_mode, int warmup, int iters,
                      int use_graph, void *stream, float *elapsed_ms);
+/* The same GEMMs dealt round-robin to `n_streams` (1..16) streams of the default priority that the
+ * call creates and destroys: launch i goes to stream i mod n_streams, writes out_list[i mod n_streams]
+ * (n_streams distinct output buffers) and uses weight set i mod n_sets.  All streams start behind one
+ * event and the end event waits for all of them; the time is that of `iters` launches in all.
+ * use_graph != 0: up to 256 launches are recorded, with that fork and join, into one HIP graph of
+ * n_streams parallel branches and the graph is replayed, which takes the host's enqueue time out of
+ * the picture.  It answers one question: do independent GEMMs on different streams overlap on the
+ * device. */
+int tuna_time_matmul_streams(const void *const *q_list, const void *const *absmax_list, int n_sets,
+                             const void *x, const void *code, void *const *out_list, int n_streams,
+                             int m, int n, int k, const tuna_gemm_config *cfg, int decode_mode,
+                             int use_graph, int warmup, int iters, float *elapsed_ms);
+/* Launches of a kernel that does nothing (`blocks` workgroups of `threads` threads, one pointer
+ * argument), on one stream of the call's own - use_graph != 0: recorded into a HIP graph of 64 launches
+ * and replayed, which takes the host's enqueue time out of the cadence - or dealt to n_streams > 1
+ * streams as above: the time any launch costs on this device.  `sink`: 4 writable bytes. */
+int tuna_time_empty_launches(void *sink, int blocks, int threads, int n_streams, int use_graph,
+                             int warmup, int iters, float *elapsed_ms);
 /* Same protocol for tuna_matmul_multi: `problems` holds n_sets batches of `count` problems each,
  * iteration i is one call with batch (i mod n_sets); the time is that of `iters` calls. */
 int tuna_time_matmul_multi(const tuna_gemm_problem *problems, int n_sets, int count, int warmup,

@@ -105,6 +105,8 @@ SIGNATURES = {
 BENCH_SIGNATURES = {
     "tuna_set_blockwise_scales_lds": (_i, [_i]),
     "tuna_time_matmul": (_i, [_vpp, _vpp, _i, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _i, _i, _i, _vp, _fp]),
+    "tuna_time_matmul_streams": (_i, [_vpp, _vpp, _i, _vp, _vp, _vpp, _i, _i, _i, _i, _cfgp, _i, _i, _i, _i, _fp]),
+    "tuna_time_empty_launches": (_i, [_vp, _i, _i, _i, _i, _i, _i, _fp]),
     "tuna_time_matmul_multi": (_i, [ctypes.POINTER(GemmProblem), _i, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_matmul_grouped": (_i, [_vpp, _vpp, _i, _vp, _vp, _vp, _i, _i, _i, _ip, _cfgp, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_dequant": (_i, [_vpp, _vpp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _fp]),

@@ -87,6 +87,98 @@ static int time_loop(F launch, int n_sets, int warmup, int iters, int use_graph,
     return rc;
 }
 
+// Times `iters` enqueues of `launch(i, stream)` dealt round-robin to `n_streams` streams of the default priority that
+// this call creates: every stream waits for one start event, the end event waits for every stream.  What the time
+// shows is whether independent launches on different streams overlap on the device.
+template <typename F>
+static int time_loop_streams(F launch, int n_streams, int use_graph, int warmup, int iters, float *elapsed_ms)
+{
+    if (iters <= 0 || warmup < 0 || n_streams < 1 || n_streams > 16 || !elapsed_ms) return fail(TUNA_ERR_INVALID_ARG, "bad timing arguments");
+    hipStream_t streams[16] = {};
+    hipEvent_t joins[16] = {};
+    hipEvent_t t0 = nullptr, t1 = nullptr, fork = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipSuccess;
+    int rc = TUNA_OK, made = 0;
+    // fork: every stream waits for `ev`, recorded on stream 0; join: stream 0 waits for every other stream
+    auto fork_all = [&](hipEvent_t ev) {
+        if ((e = hipEventRecord(ev, streams[0])) != hipSuccess) return hip_fail(e, "hipEventRecord");
+        for (int j = 1; j < n_streams; ++j)
+            if ((e = hipStreamWaitEvent(streams[j], ev, 0)) != hipSuccess) return hip_fail(e, "hipStreamWaitEvent");
+        return (int)TUNA_OK;
+    };
+    auto join_all = [&]() {
+        for (int j = 1; j < n_streams; ++j) {
+            if ((e = hipEventRecord(joins[j], streams[j])) != hipSuccess) return hip_fail(e, "hipEventRecord");
+            if ((e = hipStreamWaitEvent(streams[0], joins[j], 0)) != hipSuccess) return hip_fail(e, "hipStreamWaitEvent");
+        }
+        return (int)TUNA_OK;
+    };
+    do {
+        if ((e = hipEventCreate(&t0)) != hipSuccess || (e = hipEventCreate(&t1)) != hipSuccess ||
+            (e = hipEventCreateWithFlags(&fork, hipEventDisableTiming)) != hipSuccess) { rc = hip_fail(e, "hipEventCreate"); break; }
+        for (; made < n_streams; ++made) {
+            if ((e = hipStreamCreateWithFlags(&streams[made], hipStreamNonBlocking)) != hipSuccess) { rc = hip_fail(e, "hipStreamCreate"); break; }
+            if ((e = hipEventCreateWithFlags(&joins[made], hipEventDisableTiming)) != hipSuccess) {
+                (void)hipStreamDestroy(streams[made]);
+                rc = hip_fail(e, "hipEventCreate");
+                break;
+            }
+        }
+        if (rc) break;
+        for (int i = 0; i < warmup * n_streams && !rc; ++i) rc = launch(i, i % n_streams, streams[i % n_streams]);
+        if (rc) break;
+        for (int j = 0; j < n_streams; ++j)
+            if ((e = hipStreamSynchronize(streams[j])) != hipSuccess) { rc = hip_fail(e, "hipStreamSynchronize"); break; }
+        if (rc) break;
+        if (use_graph) {
+            // one graph of up to 256 launches with n_streams parallel branches, replayed; the launches that do not fill
+            // a whole replay are left out of the timed count (the caller gets the time scaled to `iters`)
+            const int per_graph = iters < 256 ? iters : 256;
+            const int reps = iters / per_graph;
+            if ((e = hipStreamBeginCapture(streams[0], hipStreamCaptureModeThreadLocal)) != hipSuccess) { rc = hip_fail(e, "hipStreamBeginCapture"); break; }
+            rc = fork_all(fork);
+            for (int i = 0; i < per_graph && !rc; ++i) rc = launch(i, i % n_streams, streams[i % n_streams]);
+            if (!rc) rc = join_all();
+            e = hipStreamEndCapture(streams[0], &graph);
+            if (rc) break;
+            if (e != hipSuccess) { rc = hip_fail(e, "hipStreamEndCapture"); break; }
+            if ((e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0)) != hipSuccess) { rc = hip_fail(e, "hipGraphInstantiate"); break; }
+            if ((e = hipGraphLaunch(exec, streams[0])) != hipSuccess) { rc = hip_fail(e, "hipGraphLaunch"); break; }
+            if ((e = hipEventRecord(t0, streams[0])) != hipSuccess) { rc = hip_fail(e, "hipEventRecord"); break; }
+            for (int r = 0; r < reps; ++r)
+                if ((e = hipGraphLaunch(exec, streams[0])) != hipSuccess) { rc = hip_fail(e, "hipGraphLaunch"); break; }
+            if (rc) break;
+            if ((e = hipEventRecord(t1, streams[0])) != hipSuccess) { rc = hip_fail(e, "hipEventRecord"); break; }
+            if ((e = hipEventSynchronize(t1)) != hipSuccess) { rc = hip_fail(e, "hipEventSynchronize"); break; }
+            float ms = 0.f;
+            if ((e = hipEventElapsedTime(&ms, t0, t1)) != hipSuccess) { rc = hip_fail(e, "hipEventElapsedTime"); break; }
+            *elapsed_ms = ms * (float)iters / (float)(reps * per_graph);
+            break;
+        }
+        if ((rc = fork_all(t0))) break;
+        for (int i = 0; i < iters && !rc; ++i) rc = launch(i, i % n_streams, streams[i % n_streams]);
+        if (rc) break;
+        if ((rc = join_all())) break;
+        if ((e = hipEventRecord(t1, streams[0])) != hipSuccess) { rc = hip_fail(e, "hipEventRecord"); break; }
+        if ((e = hipEventSynchronize(t1)) != hipSuccess) { rc = hip_fail(e, "hipEventSynchronize"); break; }
+        if ((e = hipEventElapsedTime(elapsed_ms, t0, t1)) != hipSuccess) { rc = hip_fail(e, "hipEventElapsedTime"); break; }
+    } while (0);
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    for (int j = 0; j < made; ++j) {
+        (void)hipStreamSynchronize(streams[j]);
+        drop_workspace(streams[j]);
+        (void)hipStreamDestroy(streams[j]);
+        (void)hipEventDestroy(joins[j]);
+    }
+    if (t0) (void)hipEventDestroy(t0);
+    if (t1) (void)hipEventDestroy(t1);
+    if (fork) (void)hipEventDestroy(fork);
+    return rc;
+}
+
 }  // namespace tuna
 
 using namespace tuna;
@@ -102,6 +194,44 @@ TUNA_EXPORT int tuna_time_matmul(const void *const *q_list, const void *const *a
         return tuna_matmul_ex(q_list[set], x, code, absmax_list[set], out, m, n, k, cfg, decode_mode, s);
     };
     return time_loop(launch, n_sets, warmup, iters, use_graph, static_cast<hipStream_t>(stream), elapsed_ms);
+}
+
+TUNA_EXPORT int tuna_time_matmul_streams(const void *const *q_list, const void *const *absmax_list, int n_sets, const void *x,
+                                         const void *code, void *const *out_list, int n_streams, int m, int n, int k,
+                                         const tuna_gemm_config *cfg, int decode_mode, int use_graph, int warmup, int iters,
+                                         float *elapsed_ms)
+{
+    if (!q_list || !absmax_list || !out_list) return fail(TUNA_ERR_INVALID_ARG, "q_list / absmax_list / out_list is null");
+    if (n_sets <= 0) return fail(TUNA_ERR_INVALID_ARG, "n_sets must be positive");
+    auto launch = [&](int i, int lane, hipStream_t s) {
+        return tuna_matmul_ex(q_list[i % n_sets], x, code, absmax_list[i % n_sets], out_list[lane], m, n, k, cfg, decode_mode, s);
+    };
+    return time_loop_streams(launch, n_streams, use_graph, warmup, iters, elapsed_ms);
+}
+
+TUNA_EXPORT int tuna_time_empty_launches(void *sink, int blocks, int threads, int n_streams, int use_graph, int warmup, int iters,
+                                         float *elapsed_ms)
+{
+    int rc;
+    if ((rc = check_ptr(sink, "sink", 4))) return rc;
+    if (blocks < 1 || threads < 1 || threads > 1024) return fail(TUNA_ERR_INVALID_ARG, "bad launch shape");
+    if (n_streams > 1) {
+        auto launch = [&](int, int, hipStream_t s) {
+            hipError_t e = launch_empty(sink, blocks, threads, s);
+            return e == hipSuccess ? (int)TUNA_OK : hip_fail(e, "empty launch");
+        };
+        return time_loop_streams(launch, n_streams, use_graph, warmup, iters, elapsed_ms);
+    }
+    hipStream_t st = nullptr;
+    hipError_t e = hipStreamCreateWithFlags(&st, hipStreamNonBlocking);
+    if (e != hipSuccess) return hip_fail(e, "hipStreamCreate");
+    auto launch = [&](int, hipStream_t s) {
+        hipError_t e2 = launch_empty(sink, blocks, threads, s);
+        return e2 == hipSuccess ? (int)TUNA_OK : hip_fail(e2, "empty launch");
+    };
+    rc = time_loop(launch, 64, warmup, iters, use_graph, st, elapsed_ms);
+    (void)hipStreamDestroy(st);
+    return rc;
 }
 
 TUNA_EXPORT int tuna_time_matmul_multi(const tuna_gemm_problem *problems, int n_sets, int count, int warmup, int iters,

@@ -41,6 +41,19 @@ __global__ __launch_bounds__(256) void read_kernel(const u32x4 *__restrict__ src
     if (r == 0x9e3779b9u) sink[0] = r;  // practically never: keeps the loads alive
 }
 
+// A kernel that does nothing (one pointer argument, as every real kernel has at least one): what a launch costs by
+// itself.
+__global__ void empty_kernel(uint32_t *sink)
+{
+    if (sink == reinterpret_cast<uint32_t *>(1)) *sink = 0u;
+}
+
+hipError_t launch_empty(void *sink, int blocks, int threads, hipStream_t stream)
+{
+    hipLaunchKernelGGL(empty_kernel, dim3((unsigned)blocks), dim3((unsigned)threads), 0, stream, static_cast<uint32_t *>(sink));
+    return hipGetLastError();
+}
+
 // variant: 0 nontemporal x8 (default), 1 plain x8, 2 nontemporal x16, 3 plain x16, 4 nontemporal x4, 5 plain x4
 hipError_t launch_read(const void *src, void *sink, size_t bytes, int blocks, int variant, hipStream_t stream)
 {

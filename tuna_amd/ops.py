@@ -345,6 +345,36 @@ def time_matmul(q_list, absmax_list, x, c, o, m, n, k, config=None, decode_mode=
 
 
 
+def time_matmul_streams(q_list, absmax_list, x, c, outs, m, n, k, config=None, decode_mode=_lib.DECODE_GEMM, warmup=10,
+                        iters=100, use_graph=False) -> float:
+    """Milliseconds for `iters` GEMMs dealt round-robin to len(outs) streams (tuna_time_matmul_streams): launch i
+    writes outs[i % len(outs)] on stream i % len(outs).  Synchronises."""
+    assert len(q_list) == len(absmax_list) and len(q_list) > 0 and len(outs) > 0
+    qp, _qk = _ptr_array(q_list)
+    ap, _ak = _ptr_array(absmax_list)
+    op, _ok = _ptr_array(outs)
+    ms = ctypes.c_float(0)
+    L = _lib.bench_lib()
+    with torch.cuda.device(x.device):
+        rc = L.tuna_time_matmul_streams(qp, ap, len(q_list), x.data_ptr(), c.data_ptr(), op, len(outs), int(m), int(n), int(k),
+                                        ctypes.byref(config) if config is not None else None, int(decode_mode),
+                                        int(bool(use_graph)), int(warmup), int(iters), ctypes.byref(ms))
+    _lib.check(rc, L)
+    return ms.value
+
+
+def time_empty_launches(device, blocks=192, threads=512, n_streams=1, use_graph=False, warmup=100, iters=1000) -> float:
+    """Milliseconds for `iters` launches of a kernel that does nothing (tuna_time_empty_launches)."""
+    sink = torch.zeros(4, dtype=torch.int32, device=device)
+    ms = ctypes.c_float(0)
+    L = _lib.bench_lib()
+    with torch.cuda.device(device):
+        rc = L.tuna_time_empty_launches(sink.data_ptr(), int(blocks), int(threads), int(n_streams), int(bool(use_graph)),
+                                        int(warmup), int(iters), ctypes.byref(ms))
+    _lib.check(rc, L)
+    return ms.value
+
+
 def time_matmul_grouped(q_list, absmax_list, x, c, o, m_group, n_groups, k, token_offsets, config=None,
                         decode_mode=_lib.DECODE_GEMM, warmup=10, iters=100, use_graph=False) -> float:
     """Milliseconds for `iters` grouped GEMMs rotating over the weight sets
