@@ -242,6 +242,18 @@ def multi_stream(ops, synth, torch, dev, names=("mistral_attn_out", "mistral_qkv
     return out
 
 
+def handover_yardstick(ops, dev):
+    """One producer -> consumer step of a split-K hand-over between two workgroups, on one XCD and across XCDs, with the
+    kernels' device-coherent accesses (sc1 stores and loads) and with accesses that stay in the XCD's L2: nanoseconds
+    on an otherwise idle device, and whether the consumer read what the producer wrote."""
+    out = {}
+    for place, same in (("same_xcd", True), ("neighbouring_xcds", False)):
+        for label, st, ld, reuse in (("sc1_store_sc1_load", 1, 1, 1), ("plain_store_sc1_load", 0, 1, 1),
+                                     ("plain_store_plain_load", 0, 0, 1), ("plain_store_plain_load_fresh_lines", 0, 0, 0)):
+            out[f"{place}:{label}"] = ops.measure_handover(dev, same, st, ld, reuse)
+    return out
+
+
 def launch_floor(ops, torch, dev, headline_bytes):
     # a kernel that does nothing, 192 workgroups of 512 threads: replayed from a HIP graph (what the device needs
     # per launch) and enqueued launch by launch (where the host's enqueue time can be the longer of the two)
@@ -456,7 +468,7 @@ def main():
     ap.add_argument("--launch", choices=("both", "stream", "graph"), default="both")
     ap.add_argument("--settle", type=int, default=300,
                     help="untimed launches before the warm-up of the headline (a box that was idle ramps its clocks)")
-    ap.add_argument("--only", choices=("read", "dequant", "quantize", "multi", "mfma", "rates", "blockwise", "streams"), default=None,
+    ap.add_argument("--only", choices=("read", "dequant", "quantize", "multi", "mfma", "rates", "blockwise", "streams", "handover"), default=None,
                     help="profiling runs: launch only the read-kernel sweep / the dequant kernel / the quantizer / "
                          "the Llama-70B layer set through tuna_matmul_multi (16 layers) / the many-token kernel with "
                          "16x16x32 and with 32x32x16 MFMA tiles (Llama-70B gate+up and QKV, --tokens, default 1024) / the "
@@ -499,6 +511,8 @@ def main():
             res = {"quantize": time_quantize(ops, synth, torch, dev)}
         elif args.only == "rates":
             res = {"unit_rates": unit_rates(ops, dev)}
+        elif args.only == "handover":
+            res = {"handover_yardstick": handover_yardstick(ops, dev)}
         elif args.only == "streams":
             res = {"headline_multi_stream": multi_stream(ops, synth, torch, dev, iters=256)}
         elif args.only == "blockwise":
@@ -566,6 +580,7 @@ def main():
         line["launch_floor"] = launch_floor(ops, torch, dev, head["packed_bytes"])
         line["unit_rates"] = unit_rates(ops, dev)
         line["headline_multi_stream"] = multi_stream(ops, synth, torch, dev)
+        line["handover_yardstick"] = handover_yardstick(ops, dev)
 
     if args.copy_yardstick > 0:
         line["copy_yardstick"] = copy_yardstick(ops, torch, dev, args.copy_yardstick)

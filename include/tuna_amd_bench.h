@@ -47,6 +47,17 @@ int tuna_time_matmul_streams(const void *const *q_list, const void *const *absma
  * streams as above: the time any launch costs on this device.  `sink`: 4 writable bytes. */
 int tuna_time_empty_launches(void *sink, int blocks, int threads, int n_streams, int use_graph,
                              int warmup, int iters, float *elapsed_ms);
+/* Yardstick of the split-K hand-over: `pairs` (1..64) producer / consumer workgroup pairs, one workgroup per compute
+ * unit, partners on one XCD (same_xcd != 0: workgroups 8 apart in launch order) or on neighbouring XCDs, run `iters`
+ * rounds of: producer stores 1 KB and waits for the acknowledgement, bumps a flag with a returning device-scope atomic;
+ * consumer sees the flag, loads the 1 KB and checks it.  store_sc1 / load_sc1: the accesses carry the sc1 bit (what the
+ * kernels' hand-over uses: coherent across the eight L2s) or stay in the XCD's own L2; reuse != 0: the same 1 KB every
+ * round, so that a stale line in the consumer's caches shows as a mismatch.  out6 receives: nanoseconds per round for
+ * the acknowledged store, the atomic's round trip and the load; mismatching 16-byte pieces; rounds given up (every wait
+ * is bounded); pairs whose workgroups did share an XCD (read back from the hardware).  Allocates its own buffers and
+ * synchronises `stream`. */
+int tuna_measure_handover(int same_xcd, int store_sc1, int load_sc1, int reuse, int pairs, int iters,
+                          void *stream, double *out6);
 /* Same protocol for tuna_matmul_multi: `problems` holds n_sets batches of `count` problems each,
  * iteration i is one call with batch (i mod n_sets); the time is that of `iters` calls. */
 int tuna_time_matmul_multi(const tuna_gemm_problem *problems, int n_sets, int count, int warmup,

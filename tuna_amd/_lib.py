@@ -107,6 +107,7 @@ BENCH_SIGNATURES = {
     "tuna_time_matmul": (_i, [_vpp, _vpp, _i, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_matmul_streams": (_i, [_vpp, _vpp, _i, _vp, _vp, _vpp, _i, _i, _i, _i, _cfgp, _i, _i, _i, _i, _fp]),
     "tuna_time_empty_launches": (_i, [_vp, _i, _i, _i, _i, _i, _i, _fp]),
+    "tuna_measure_handover": (_i, [_i, _i, _i, _i, _i, _i, _vp, ctypes.POINTER(ctypes.c_double)]),
     "tuna_time_matmul_multi": (_i, [ctypes.POINTER(GemmProblem), _i, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_matmul_grouped": (_i, [_vpp, _vpp, _i, _vp, _vp, _vp, _i, _i, _i, _ip, _cfgp, _i, _i, _i, _i, _vp, _fp]),
     "tuna_time_dequant": (_i, [_vpp, _vpp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _fp]),

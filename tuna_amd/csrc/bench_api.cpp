@@ -234,6 +234,17 @@ TUNA_EXPORT int tuna_time_empty_launches(void *sink, int blocks, int threads, in
     return rc;
 }
 
+TUNA_EXPORT int tuna_measure_handover(int same_xcd, int store_sc1, int load_sc1, int reuse, int pairs, int iters, void *stream,
+                                      double *out6)
+{
+    if (!out6 || pairs < 1 || pairs > 64 || iters < 1 || iters > 4096) return fail(TUNA_ERR_INVALID_ARG, "bad hand-over yardstick arguments");
+    // workgroup L runs on XCD L mod 8 (what the yardstick reports back as the pairs that shared an XCD): partners 8
+    // apart share one, neighbours do not
+    const hipError_t e = run_handover_yardstick(same_xcd ? 8 : 1, pairs, store_sc1 != 0, load_sc1 != 0, reuse != 0, iters,
+                                                static_cast<hipStream_t>(stream), out6);
+    return e == hipSuccess ? (int)TUNA_OK : hip_fail(e, "hand-over yardstick");
+}
+
 TUNA_EXPORT int tuna_time_matmul_multi(const tuna_gemm_problem *problems, int n_sets, int count, int warmup, int iters,
                                        int use_graph, void *stream, float *elapsed_ms)
 {

@@ -54,6 +54,123 @@ hipError_t launch_empty(void *sink, int blocks, int threads, hipStream_t stream)
     return hipGetLastError();
 }
 
+// ---- hand-over yardstick: what one producer -> consumer step of a split-K hand-over costs between two workgroups --------
+// Workgroup pairs (producer b, consumer b + stride; one workgroup per compute unit): the producer stores 1 KB, waits for
+// the stores to be acknowledged, bumps a flag with a returning atomic; the consumer polls the flag, loads the 1 KB and
+// checks it, then acknowledges; `iters` rounds in lock step, every wait bounded.  store_sc1 / load_sc1: the accesses
+// carry the sc1 bit (coherent across the device's eight L2s: write-through stores, loads that do not hit in a
+// neighbouring compute unit's stale lines) or not (they stay in the XCD's own L2).  reuse: the same 1 KB every round
+// (a stale line in the consumer's caches then shows as a mismatch) or a fresh one.  Times in units of the 100 MHz
+// constant clock, summed over rounds.
+struct HandoverResult {
+    unsigned long long store_ack, atomic_rtt, load_lat, mismatches, timeouts, xcc_prod, xcc_cons;
+};
+
+__global__ __launch_bounds__(64) void handover_kernel(int stride, int npairs, int store_sc1, int load_sc1, int reuse, int iters,
+                                                      u32x4 *data, unsigned *flags, unsigned *acks, HandoverResult *res)
+{
+    extern __shared__ unsigned char occupy_the_cu[];
+    const int wg = blockIdx.x, lane = threadIdx.x;
+    // pairs tile the grid in groups of 2 * stride workgroups: the first `stride` produce, the next `stride` consume
+    const int grp = wg / (2 * stride), in = wg % (2 * stride);
+    const int p = grp * stride + (in % stride);
+    if (p >= npairs) return;
+    const bool producer = in < stride;
+    unsigned xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID, 0, 4)" : "=s"(xcc));
+    unsigned *flag = flags + p * 64, *ack = acks + p * 64;
+    unsigned long long t_st = 0, t_at = 0, t_ld = 0, mism = 0, tmo = 0;
+    for (int it = 1; it <= iters; ++it) {
+        u32x4 *d = data + ((size_t)p * (reuse ? 1 : iters) + (reuse ? 0 : it - 1)) * 64 + lane;
+        const unsigned want = (unsigned)it * 2654435761u + (unsigned)p;
+        if (producer) {
+            const u32x4 v = u32x4{want, want ^ 1u, want ^ 2u, want + (unsigned)lane};
+            const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();
+            if (store_sc1) asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" ::"v"(d), "v"(v) : "memory");
+            else asm volatile("global_store_dwordx4 %0, %1, off\n\ts_waitcnt vmcnt(0)" ::"v"(d), "v"(v) : "memory");
+            const unsigned long long t1 = __builtin_amdgcn_s_memrealtime();
+            if (lane == 0) (void)__hip_atomic_fetch_add(flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            const unsigned long long t2 = __builtin_amdgcn_s_memrealtime();
+            t_st += t1 - t0;
+            t_at += t2 - t1;
+            int spins = 0;
+            unsigned a = 0;
+            do {
+                a = lane == 0 ? __hip_atomic_load(ack, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+                a = __shfl(a, 0);
+            } while (a < (unsigned)it && ++spins < 1000000);
+            if (a < (unsigned)it) { ++tmo; break; }
+        } else {
+            int spins = 0;
+            unsigned f = 0;
+            do {
+                f = lane == 0 ? __hip_atomic_fetch_add(flag, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+                f = __shfl(f, 0);
+            } while (f < (unsigned)it && ++spins < 1000000);
+            if (f < (unsigned)it) { ++tmo; break; }
+            u32x4 v;
+            const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();
+            if (load_sc1) asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(d) : "memory");
+            else asm volatile("global_load_dwordx4 %0, %1, off\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(d) : "memory");
+            const unsigned long long t1 = __builtin_amdgcn_s_memrealtime();
+            t_ld += t1 - t0;
+            if (v[0] != want || v[1] != (want ^ 1u) || v[2] != (want ^ 2u) || v[3] != want + (unsigned)lane) ++mism;
+            if (lane == 0) __hip_atomic_store(ack, (unsigned)it, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    unsigned long long m_all = mism;
+    for (int o = 32; o; o >>= 1) m_all += __shfl_xor(m_all, o);
+    if (lane == 0) {
+        HandoverResult *r = res + p;
+        if (producer) { r->store_ack = t_st; r->atomic_rtt = t_at; r->xcc_prod = xcc; }
+        else { r->load_lat = t_ld; r->mismatches = m_all; r->xcc_cons = xcc; }
+        if (tmo) atomicAdd(&r->timeouts, tmo);
+    }
+}
+
+// out[0..5]: mean store-acknowledge, atomic round trip and load latency in nanoseconds per round, mismatching 16-byte
+// pieces, rounds given up, pairs whose two workgroups ran on one XCD.  Allocates and frees its own buffers; synchronises.
+hipError_t run_handover_yardstick(int stride, int npairs, int store_sc1, int load_sc1, int reuse, int iters, hipStream_t stream, double *out)
+{
+    const int groups = (npairs + stride - 1) / stride, grid = groups * 2 * stride;
+    u32x4 *data = nullptr;
+    unsigned *flags = nullptr, *acks = nullptr;
+    HandoverResult *res = nullptr;
+    const size_t data_bytes = (size_t)npairs * (reuse ? 1 : iters) * 1024;
+    hipError_t e;
+    if ((e = hipMalloc(&data, data_bytes)) != hipSuccess) return e;
+    if ((e = hipMalloc(&flags, (size_t)npairs * 256)) == hipSuccess && (e = hipMalloc(&acks, (size_t)npairs * 256)) == hipSuccess &&
+        (e = hipMalloc(&res, (size_t)npairs * sizeof(HandoverResult))) == hipSuccess &&
+        (e = hipMemsetAsync(data, 0, data_bytes, stream)) == hipSuccess && (e = hipMemsetAsync(flags, 0, (size_t)npairs * 256, stream)) == hipSuccess &&
+        (e = hipMemsetAsync(acks, 0, (size_t)npairs * 256, stream)) == hipSuccess &&
+        (e = hipMemsetAsync(res, 0, (size_t)npairs * sizeof(HandoverResult), stream)) == hipSuccess &&
+        (e = hipFuncSetAttribute(reinterpret_cast<const void *>(handover_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024)) == hipSuccess) {
+        // 100 KB of LDS per workgroup: one workgroup per compute unit, so that all pairs are resident together
+        hipLaunchKernelGGL(handover_kernel, dim3((unsigned)grid), dim3(64), 100 * 1024, stream, stride, npairs, store_sc1, load_sc1, reuse, iters,
+                           data, flags, acks, res);
+        e = hipGetLastError();
+        if (e == hipSuccess) e = hipStreamSynchronize(stream);
+        if (e == hipSuccess) {
+            HandoverResult *h = new HandoverResult[npairs];
+            e = hipMemcpy(h, res, (size_t)npairs * sizeof(HandoverResult), hipMemcpyDeviceToHost);
+            double st = 0, at = 0, ld = 0, mm = 0, to = 0, same = 0;
+            for (int i = 0; i < npairs; ++i) {
+                st += (double)h[i].store_ack; at += (double)h[i].atomic_rtt; ld += (double)h[i].load_lat;
+                mm += (double)h[i].mismatches; to += (double)h[i].timeouts; same += h[i].xcc_prod == h[i].xcc_cons ? 1.0 : 0.0;
+            }
+            const double den = (double)npairs * iters;
+            out[0] = st / den * 10.0; out[1] = at / den * 10.0; out[2] = ld / den * 10.0; out[3] = mm; out[4] = to; out[5] = same;
+            delete[] h;
+        }
+    }
+    (void)hipFree(data);
+    if (flags) (void)hipFree(flags);
+    if (acks) (void)hipFree(acks);
+    if (res) (void)hipFree(res);
+    return e;
+}
+
 // variant: 0 nontemporal x8 (default), 1 plain x8, 2 nontemporal x16, 3 plain x16, 4 nontemporal x4, 5 plain x4
 hipError_t launch_read(const void *src, void *sink, size_t bytes, int blocks, int variant, hipStream_t stream)
 {

@@ -375,6 +375,18 @@ def time_empty_launches(device, blocks=192, threads=512, n_streams=1, use_graph=
     return ms.value
 
 
+def measure_handover(device, same_xcd: bool, store_sc1: bool, load_sc1: bool, reuse: bool, pairs=16, iters=200) -> dict:
+    """The hand-over yardstick (tuna_measure_handover): latencies of one producer -> consumer step in nanoseconds."""
+    out = (ctypes.c_double * 6)()
+    L = _lib.bench_lib()
+    with torch.cuda.device(device):
+        rc = L.tuna_measure_handover(int(same_xcd), int(store_sc1), int(load_sc1), int(reuse), int(pairs), int(iters),
+                                     _stream(device), out)
+    _lib.check(rc, L)
+    return {"store_ack_ns": round(out[0], 1), "atomic_round_trip_ns": round(out[1], 1), "load_ns": round(out[2], 1),
+            "mismatches": int(out[3]), "timeouts": int(out[4]), "pairs_on_one_xcd": int(out[5]), "pairs": int(pairs)}
+
+
 def time_matmul_grouped(q_list, absmax_list, x, c, o, m_group, n_groups, k, token_offsets, config=None,
                         decode_mode=_lib.DECODE_GEMM, warmup=10, iters=100, use_graph=False) -> float:
     """Milliseconds for `iters` grouped GEMMs rotating over the weight sets
