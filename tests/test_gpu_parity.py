@@ -2084,3 +2084,31 @@ def test_quantizer_every_fp16_value_against_the_oracle():
         q_ref, a_ref = O.quantize(w, code, 8, 65536, block_size=bs)
         assert np.array_equal(a.cpu().numpy(), a_ref)
         assert np.array_equal(q.cpu().numpy(), q_ref), bs
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m,n,k", [(4096, 16, 4096), (6144, 16, 4096), (5120, 16, 5120), (4096, 1, 4096), (8192, 16, 8192),
+                                   (28672, 16, 4096), (8192, 16, 28672), (2560, 32, 2560)])
+def test_scales_that_are_only_float_aligned_run_through_the_dispatcher(m, n, k):
+    """absmax may be any float pointer (the reference's wrapper takes one): a view 4 bytes into a buffer, on shapes
+    whose library-chosen kernels read the scales two or four at a time (narrow-row, lean, LDS-staged and batched
+    launches), must run - the dispatcher takes a kernel that reads them one by one - and match the oracle."""
+    import torch
+
+    from tuna_amd import ops
+
+    print(f"float-aligned scales m={m} n={n} k={k}: aligned launch would be {ops.describe_launch(m, n, k, None)}", flush=True)
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=m + n + k)
+    dq, dx, dc = to_dev(q, x, code)
+    holder = torch.zeros(m + 8, dtype=torch.float32, device="cuda")
+    da = holder[1:m + 1]
+    da.copy_(torch.from_numpy(absmax))
+    assert da.data_ptr() % 16 == 4
+    out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+    ops.matmul(dx, dq, da, dc, out, m, n, k)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().view(np.uint16)
+    assert not np.isnan(f16_bits_to_f64(got)).any()
+    rows = np.sort(np.random.default_rng(k).choice(m, size=128, replace=False)).astype(np.int32)
+    ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1, rows=rows)
+    assert rel_err(f16_bits_to_f64(got[:, rows]), ref) <= REL_TOL

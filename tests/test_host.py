@@ -591,3 +591,29 @@ def test_bench_last_line_stays_compact_whatever_the_detail_holds():
     bare = dict(detail, cpu_baseline=None)
     del bare["shapes"]
     assert json.loads(bench.headline_line(bare))["cpu_baseline"] is None
+
+
+def test_library_chosen_configs_accept_scales_that_are_only_float_aligned():
+    """tuna_matmul(cfg = NULL) with an absmax pointer of the form 4 mod 16 on every shape of the table, at the token
+    counts its entries start at: never an argument error (the dispatcher moves off kernels that read the scales
+    two or four at a time).  Host only: fake pointers, so this runs where no device can take the launch."""
+    import torch
+
+    if torch.cuda.is_available():
+        pytest.skip("fake pointers: only where nothing can be launched")
+    from tuna_amd import _lib
+
+    L = _lib.lib()
+    m_, lo_, hi_, k_ = (ctypes.c_int() for _ in range(4))
+    cfg = _lib.GemmConfig()
+    seen = set()
+    for i in range(L.tuna_config_table_size()):
+        assert L.tuna_config_table_entry(i, ctypes.byref(m_), ctypes.byref(lo_), ctypes.byref(hi_), ctypes.byref(k_), ctypes.byref(cfg)) == 0
+        for n in {lo_.value, min(hi_.value, lo_.value + 3)}:
+            if n > 64 or (m_.value, n, k_.value) in seen:
+                continue
+            seen.add((m_.value, n, k_.value))
+            rc = L.tuna_matmul(0x10000, 0x20000, 0x30000, 0x40004, 0x50000, m_.value, n, k_.value, None)
+            assert rc != _lib.ERR_INVALID_ARG, (m_.value, n, k_.value, L.tuna_last_error())
+            assert rc in (_lib.ERR_HIP, _lib.ERR_NO_DEVICE, _lib.ERR_WORKSPACE), rc
+    assert len(seen) > 40

@@ -22,6 +22,54 @@ def _both(m, n, k, seed, config=None):
     return got.cpu().numpy().view(np.uint16), ref.cpu().numpy().view(np.uint16)
 
 
+def test_static_scratch_entry_point_allocates_no_device_memory_on_a_stream_without_a_workspace():
+    """What the entry point exists for: split-K launches through tuna_matmul_static on a stream the library has never
+    uses (it owns no workspace there: they are all released first) leave the device's free memory exactly where it was - the allocating entry
+    point would have taken 64 MB for that stream - and still give the bits of tuna_matmul_ex.  Runs before any other
+    call of this file touches the streams used here."""
+    import torch
+
+    from tuna_amd import _lib, ops
+
+    assert _lib.lib().tuna_init() == 0
+    m, n, k = 8192, 16, 8192
+    used, _hit = ops.select_config(m, n, k)
+    assert ops.config_footprint(m, n, k, used)[1] > 0          # the tuned entry splits k across workgroups
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=123)
+    dq, dx, dc, da = to_dev(q, x, code, absmax)
+    got = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+    ref = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+    small = torch.full((5, 1024), float("nan"), dtype=torch.float16, device="cuda")
+    q2, x2, code2, absmax2 = make_inputs_np(1024, 5, 2048, seed=124)
+    dq2, dx2, dc2, da2 = to_dev(q2, x2, code2, absmax2)
+    torch.cuda.synchronize()
+    # (torch hands out streams from a pool that earlier tests used too: drop every workspace the library holds)
+    assert _lib.lib().tuna_release_workspaces() == 0
+    warm, fresh = torch.cuda.Stream(), torch.cuda.Stream()
+    with torch.cuda.stream(warm):                              # (loads both kernels, finds the array's address)
+        ops.matmul_static(dx, dq, da, dc, got, m, n, k)
+        ops.matmul_static(dx2, dq2, da2, dc2, small, 1024, 5, 2048)
+    with torch.cuda.stream(fresh):                             # (the runtime sets a stream's queue up at its first launch)
+        got.fill_(float("nan"))
+        small.fill_(float("nan"))
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    with torch.cuda.stream(fresh):
+        ops.matmul_static(dx, dq, da, dc, got, m, n, k)
+        ops.matmul_static(dx2, dq2, da2, dc2, small, 1024, 5, 2048)     # a smaller launch over the first one's partial sums
+    fresh.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "tuna_matmul_static allocated device memory"
+    with torch.cuda.stream(fresh):
+        ops.matmul(dx, dq, da, dc, ref, m, n, k)                   # now the stream gets its workspace
+    fresh.synchronize()
+    assert torch.cuda.mem_get_info()[0] < free_before
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), ref.cpu().numpy().view(np.uint16))
+    ref2 = torch.full((5, 1024), float("nan"), dtype=torch.float16, device="cuda")
+    ops.matmul(dx2, dq2, da2, dc2, ref2, 1024, 5, 2048)
+    torch.cuda.synchronize()
+    assert np.array_equal(small.cpu().numpy().view(np.uint16), ref2.cpu().numpy().view(np.uint16))
+
+
 def test_static_scratch_entry_point_equals_the_allocating_one_on_two_calls_in_a_row():
     """Two split-K launches in a row through tuna_matmul_static, the second with a smaller input:
     both share the device's static array (partial sums of the first call are still in it, the

@@ -667,7 +667,9 @@ struct Workspace {
     std::vector<void *> retired;  // outgrown buffers, kept for graphs captured while they were current
 };
 
-constexpr size_t kWsFirstBytes = (size_t)64 << 20;
+// First allocation for a (device, stream) pair: what the launch asks for, but at least this much, so that a process
+// with many streams does not pay for the largest request of the table (48 MB) on each of them.
+constexpr size_t kWsFirstBytes = (size_t)8 << 20;
 constexpr size_t kWsFirstCounters = (size_t)64 << 10;
 
 static std::mutex g_ws_mutex;
@@ -709,15 +711,13 @@ static int get_workspace(hipStream_t stream, size_t ws_bytes, size_t n_counters,
             unsigned *fresh = nullptr;
             e = hipMalloc(reinterpret_cast<void **>(&fresh), want * sizeof(unsigned));
             if (e != hipSuccess) return fail(TUNA_ERR_WORKSPACE, "hipMalloc for the split-K counters: %s", hipGetErrorString(e));
-            e = hipMemset(fresh, 0, want * sizeof(unsigned));  // kernels leave them at zero afterwards
+            // zeroed on the launch stream (it is not capturing: checked above) and waited for there: a device-wide
+            // synchronisation would disturb other threads' streams and captures.  Kernels leave the counters at zero.
+            e = hipMemsetAsync(fresh, 0, want * sizeof(unsigned), stream);
+            if (e == hipSuccess) e = hipStreamSynchronize(stream);
             if (e != hipSuccess) {
                 (void)hipFree(fresh);
-                return hip_fail(e, "hipMemset(counters)");
-            }
-            e = hipDeviceSynchronize();
-            if (e != hipSuccess) {
-                (void)hipFree(fresh);
-                return hip_fail(e, "hipDeviceSynchronize");
+                return hip_fail(e, "clearing the split-K counters");
             }
             if (w.counters) w.retired.push_back(w.counters);
             w.counters = fresh;
@@ -951,6 +951,14 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
         hipError_t e = launch_gemm_tiled(tp.args, tp.tile_rows, tp.tile_tokens, tp.mfma32, stream);
         if (e != hipSuccess) return hip_fail(e, "many-token gemm launch");
         return TUNA_OK;
+    }
+    // The narrow-row kernel reads a lane's scales 2 or 4 rows at a time.  A caller that names such a config must align
+    // absmax for it; when the library picked the config itself it takes the streaming kernel's derived config for a
+    // pointer that is only float-aligned (every other kernel checks the alignment where it chooses its variant).
+    if (is_narrow(c) && !cfg) {
+        NarrowPlan probe;
+        if (plan_narrow(m, n, k, c, decode, &probe) == TUNA_OK && reinterpret_cast<uintptr_t>(absmax) % (probe.rows == 64 ? 16 : 8))
+            c = derive_streaming(m, n, k, decode);
     }
     if (is_narrow(c)) {
         NarrowPlan np;

@@ -104,6 +104,8 @@ bool mid_lds_applies(const GemmPlan &plan)
     int xc;
     const MidVariant *v = mid_variant(plan, &xc);
     if (!v || !v->fn_lds || !lds_path(plan)) return false;
+    // (the twin fetches a lane's four scales with one 16-byte global -> LDS load)
+    if ((reinterpret_cast<uintptr_t>(plan.args.absmax) & 15u) != 0) return false;
     // x pieces (one wave instruction per k-step and token tile) per wave and chunk: 1, 2 or 4
     const int pieces = (xc / 32) * plan.token_tiles, waves = plan.threads / 64;
     if (pieces % waves != 0 || (pieces / waves != 1 && pieces / waves != 2 && pieces / waves != 4)) return false;
@@ -147,7 +149,9 @@ hipError_t launch_gemm_mid(const GemmPlan &plan, int dev, int cus, hipStream_t s
     const bool staged = mid_lds_applies(plan);
     const size_t lds = (size_t)kLutBytes + (staged ? x_lds + (size_t)(plan.threads / 64) * plan.prefetch * 1024
                                                    : (x_lds > red_lds ? x_lds : red_lds));
-    if (plan.lds_weights && !staged) return hipErrorInvalidConfiguration;
+    // (a config that asks for the LDS-staged twin and cannot have it is an error, except for scales that are only
+    // float-aligned: the register twin computes the same bits from them)
+    if (plan.lds_weights && !staged && (reinterpret_cast<uintptr_t>(a.absmax) & 15u) == 0) return hipErrorInvalidConfiguration;
     dim3 grid = plan.grid;
     const int split_log2 = a.split_k > 1 ? a.split_log2 : 0;
     const int walk_tiles = a.row_tiles << split_log2;  // (row tile, part of k) pairs
