@@ -174,6 +174,16 @@ typedef struct tuna_gemm_problem {
  * of one call on `stream`; no problem may read what another one writes.  All problems are
  * checked before anything is enqueued.  No counterpart in the reference. */
 int tuna_matmul_multi(const tuna_gemm_problem *problems, int count, void *stream);
+/* tuna_matmul_multi with a fused epilogue per problem (those of tuna_matmul_fused): epilogues[i] is the
+ * TUNA_EPILOGUE_* of problem i and residuals[i] its residual (fp16 [n, m], 8-byte aligned, may be the problem's
+ * own output; ignored unless the epilogue is TUNA_EPILOGUE_RESIDUAL).  For TUNA_EPILOGUE_SILU_MUL the problem's
+ * weight rows are interleaved (2i: gate, 2i+1: up) and its out is fp16 [n, m/2].  Either array may be NULL
+ * (no epilogues / no residuals).  A decoder layer's projections launched together - SiLU-mul on the combined
+ * gate+up GEMM, the residual add on the out and down projections - cost one launch instead of four GEMMs and
+ * two element-wise kernels; as in tuna_matmul_multi no problem may read what another one writes.  No
+ * counterpart in the reference (README.md:25-27 counts a layer as four separate GEMMs). */
+int tuna_matmul_multi_fused(const tuna_gemm_problem *problems, const int32_t *epilogues,
+                            const void *const *residuals, int count, void *stream);
 /* The same for weights with one scale per block_size (64, 128, 256, ...) consecutive weights of a row: every
  * problem's absmax is fp32 [m, k / block_size] (the layout tuna_quantize_blockwise writes, the reference
  * quantizer's for block_size < k, test.py:7-17), 4-byte aligned.  Problems that do not qualify for the batched

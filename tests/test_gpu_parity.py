@@ -3,6 +3,8 @@
 Bit-exact for the decode (dequant op, and the GEMM's in-register decode read out through
 one-hot activations); GEMM outputs within REL_TOL of the oracle's float64 contraction.
 """
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -2112,3 +2114,84 @@ def test_scales_that_are_only_float_aligned_run_through_the_dispatcher(m, n, k):
     rows = np.sort(np.random.default_rng(k).choice(m, size=128, replace=False)).astype(np.int32)
     ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1, rows=rows)
     assert rel_err(f16_bits_to_f64(got[:, rows]), ref) <= REL_TOL
+
+
+@pytest.mark.gpu
+@pytest.mark.usefixtures("diagnostic_build")
+@pytest.mark.parametrize("n,dims", [(16, (1024, 512, 2816)), (5, (2048, 1024, 5632)), (16, (512, 256, 1408))])
+def test_a_layer_as_one_batched_launch_with_fused_epilogues(n, dims):
+    """The four projections of a decoder layer as ONE tuna_matmul_multi_fused call (independent inputs, as the entry
+    point requires): QKV plain, attention output + residual, the combined gate+up GEMM with SiLU-mul on interleaved
+    rows (output [n, m/2]), down + residual in place.  One launch of the batched kernel's fused-epilogue variant;
+    every output against the oracle's float64 sums pushed through the same formulas, and bit for bit against
+    tuna_matmul_fused's for the same problems where the two run the same sums (whole row tiles)."""
+    import torch
+
+    from tuna_amd import _lib, ops
+
+    hidden, kv, inter = dims
+    shapes = [(hidden + 2 * kv, hidden, _lib.EPILOGUE_NONE), (hidden, hidden, _lib.EPILOGUE_RESIDUAL),
+              (2 * inter, hidden, _lib.EPILOGUE_SILU_MUL), (hidden, inter, _lib.EPILOGUE_RESIDUAL)]
+    print(f"layer as one launch: tokens={n} shapes={[(m, k) for m, k, _ in shapes]}", flush=True)
+    rng = np.random.default_rng(n + hidden)
+    host, problems, eps, residuals, outs = [], [], [], [], []
+    code_dev = None
+    for i, (m, k, ep) in enumerate(shapes):
+        q, x, code, absmax = make_inputs_np(m, n, k, seed=400 + i + hidden)
+        res = (rng.standard_normal((n, m)) * 0.05).astype(np.float16)
+        dq, dx, dc, da, dres = to_dev(q, x, code, absmax, res)
+        code_dev = code_dev if code_dev is not None else dc          # one codebook pointer: one decode table per launch
+        om = m // 2 if ep == _lib.EPILOGUE_SILU_MUL else m
+        out = dres.clone() if i == 3 else torch.full((n, om), float("nan"), dtype=torch.float16, device="cuda")
+        host.append((q, x, code, absmax, res))
+        problems.append((dx, dq, da, code_dev, out, m, n, k))
+        eps.append(ep)
+        residuals.append(out if i == 3 else dres if ep == _lib.EPILOGUE_RESIDUAL else None)   # down: residual in place
+        outs.append(out)
+    L = _lib.lib()
+    before = L.tuna_multi_launches()
+    ops.matmul_multi(problems, epilogues=eps, residuals=residuals)
+    torch.cuda.synchronize()
+    assert L.tuna_multi_launches() == before + 1                       # all four in one launch
+    for i, ((m, k, ep), (q, x, code, absmax, res), out) in enumerate(zip(shapes, host, outs)):
+        ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1)
+        got = out.cpu().numpy().astype(np.float64)
+        assert not np.isnan(got).any(), i
+        if ep == _lib.EPILOGUE_RESIDUAL:
+            assert rel_err(got, ref + res.astype(np.float64)) <= REL_TOL, i
+        elif ep == _lib.EPILOGUE_SILU_MUL:
+            g, u = ref[:, 0::2], ref[:, 1::2]
+            assert rel_err(got, g / (1.0 + np.exp(-g)) * u, floor=REL_FLOOR_D2) <= REL_TOL, i
+        else:
+            assert rel_err(got, ref) <= REL_TOL, i
+    # without epilogues the same call writes the plain sums: the fused variant changes the stores only
+    plain = [torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda") for m, _, _ in shapes]
+    ops.matmul_multi([(p[0], p[1], p[2], p[3], o, p[5], p[6], p[7]) for p, o in zip(problems, plain)])
+    torch.cuda.synchronize()
+    assert torch.equal(plain[0].view(torch.int16), outs[0].view(torch.int16))
+
+
+@pytest.mark.gpu
+def test_batched_launch_with_epilogues_rejects_bad_arguments_and_falls_back_problem_by_problem():
+    """A residual epilogue without a residual is an argument error before anything is enqueued; a problem the batched
+    kernel cannot take (more than 16 tokens) runs through tuna_matmul_fused with its epilogue."""
+    import torch
+
+    from tuna_amd import _lib, ops
+
+    m, n, k = 512, 40, 1024
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=77)
+    res = (np.random.default_rng(5).standard_normal((n, m)) * 0.05).astype(np.float16)
+    dq, dx, dc, da, dres = to_dev(q, x, code, absmax, res)
+    out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError):
+        ops.matmul_multi([(dx, dq, da, dc, out, m, n, k)], epilogues=[_lib.EPILOGUE_RESIDUAL], residuals=[None])
+    arr = ops.problem_array([(dx, dq, da, dc, out, m, n, k)])
+    eps = (ctypes.c_int32 * 1)(_lib.EPILOGUE_RESIDUAL)
+    assert _lib.lib().tuna_matmul_multi_fused(arr, eps, None, 1, None) == _lib.ERR_INVALID_ARG
+    eps[0] = 7
+    assert _lib.lib().tuna_matmul_multi_fused(arr, eps, None, 1, None) == _lib.ERR_INVALID_ARG
+    ops.matmul_multi([(dx, dq, da, dc, out, m, n, k)], epilogues=[_lib.EPILOGUE_RESIDUAL], residuals=[dres])
+    torch.cuda.synchronize()
+    ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1) + res.astype(np.float64)
+    assert rel_err(out.cpu().numpy().astype(np.float64), ref) <= REL_TOL

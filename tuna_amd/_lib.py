@@ -79,6 +79,7 @@ SIGNATURES = {
     "tuna_matmul_static": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _vp]),
     "tuna_matmul_fused": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _cfgp, _i, _i, _vp, _vp]),
     "tuna_matmul_multi": (_i, [ctypes.POINTER(GemmProblem), _i, _vp]),
+    "tuna_matmul_multi_fused": (_i, [ctypes.POINTER(GemmProblem), ctypes.POINTER(ctypes.c_int32), _vpp, _i, _vp]),
     "tuna_matmul_multi_blockwise": (_i, [ctypes.POINTER(GemmProblem), _i, _i, _vp]),
     "tuna_matmul_grouped": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _ip, _cfgp, _i, _vp]),
     "tuna_dequant": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),

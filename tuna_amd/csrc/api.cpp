@@ -828,17 +828,21 @@ struct MultiPlan {
 // Whether problems[0..count) can run as one launch on a device of `cus` compute units; fills `plan`.
 // waves_m / prefetch: 0 = chosen here.
 // blk_shift >= 0: every problem's absmax is [m, k / (64 << blk_shift)], one scale per block of a row (the BLK variants).
+// epilogues / residuals: per problem, or null (the fused-epilogue variants run when any problem has one).
 static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, MultiPlan *plan, int waves_m = 0, int prefetch = 0,
-                       int blk_shift = -1)
+                       int blk_shift = -1, const int32_t *epilogues = nullptr, const void *const *residuals = nullptr)
 {
     if (count < 1 || count > kMaxMultiProblems || cus < 1) return false;
     const bool blk = blk_shift >= 0;
+    bool epi = false;
+    for (int i = 0; epilogues && i < count; ++i) epi = epi || epilogues[i] != TUNA_EPILOGUE_NONE;
+    if (epi && blk) return false;
     if (!waves_m) waves_m = diag::multi_waves_m();
     if (!prefetch) prefetch = diag::multi_prefetch();
     // (a ring of two: with every wait of the ring exact it streams as fast as a ring of four on the longest
     // batches and faster on the others - fewer bytes requested ahead at a segment switch)
     if (!prefetch) prefetch = 2;
-    if (!multi_variant_exists(blk ? 10 + prefetch : prefetch)) return false;
+    if (!multi_variant_exists(blk ? 10 + prefetch : epi ? 20 + prefetch : prefetch)) return false;
     if (!waves_m) {
         // 256-row tiles (4 x 4 waves) when every problem allows, else narrower tiles and more waves along k
         waves_m = 4;
@@ -877,6 +881,8 @@ static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, Mu
         mp.x = p.x;
         mp.absmax = static_cast<const float *>(p.absmax);
         mp.out = p.out;
+        mp.epilogue = epi ? epilogues[i] : TUNA_EPILOGUE_NONE;
+        mp.residual = (epi && residuals && epilogues[i] == TUNA_EPILOGUE_RESIDUAL) ? residuals[i] : nullptr;
         mp.m = p.m, mp.n = p.n, mp.k = p.k;
         mp.units_per_tile = p.k / (kStepK * unit_steps);
         a.unit_begin[i] = (int)units;
@@ -904,8 +910,8 @@ static bool plan_multi(const tuna_gemm_problem *problems, int count, int cus, Mu
     a.blk_shift = blk ? blk_shift : 0;
     // variant -2: ring of 2 with weights and x staged through LDS (x chunks of 512 k: every wave needs a whole
     // number of ring turns per chunk, so at most 8 waves along k)
-    const bool lds = !blk && diag::multi_lds() != 0 && prefetch == 2 && waves_k <= 8 && multi_variant_exists(-2);
-    plan->prefetch = blk ? 10 + prefetch : lds ? -2 : prefetch;
+    const bool lds = !blk && !epi && diag::multi_lds() != 0 && prefetch == 2 && waves_k <= 8 && multi_variant_exists(-2);
+    plan->prefetch = blk ? 10 + prefetch : epi ? 20 + prefetch : lds ? -2 : prefetch;
     plan->ws_bytes = (size_t)n_wg * 2 * waves_m * 4096;
     plan->n_counters = (size_t)tiles;
     return true;
@@ -1125,11 +1131,19 @@ static int matmul_grouped_impl(const void *q, const void *x, const void *code, c
 extern "C" int tuna_matmul_blockwise(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n,
                                      int k, int block_size, void *stream);
 
-static int matmul_multi_impl(const tuna_gemm_problem *problems, int count, hipStream_t stream)
+static int matmul_multi_impl(const tuna_gemm_problem *problems, int count, hipStream_t stream, const int32_t *epilogues = nullptr,
+                             const void *const *residuals = nullptr)
 {
     if (count < 0 || (count > 0 && !problems)) return fail(TUNA_ERR_INVALID_ARG, "problems is null or count=%d negative", count);
     if (count == 0) return TUNA_OK;
     int rc;
+    for (int i = 0; epilogues && i < count; ++i) {
+        const int ep = epilogues[i];
+        if (ep != TUNA_EPILOGUE_NONE && ep != TUNA_EPILOGUE_RESIDUAL && ep != TUNA_EPILOGUE_SILU_MUL)
+            return fail(TUNA_ERR_INVALID_ARG, "epilogues[%d]=%d is not a TUNA_EPILOGUE_* value", i, ep);
+        if (ep == TUNA_EPILOGUE_RESIDUAL && (!residuals || (rc = check_ptr(residuals[i], "residual", 8))))
+            return residuals ? rc : fail(TUNA_ERR_INVALID_ARG, "epilogues[%d] adds a residual but residuals is null", i);
+    }
     // every problem is checked before anything is enqueued: a bad one must not leave half a batch behind
     for (int i = 0; i < count; ++i) {
         const tuna_gemm_problem &p = problems[i];
@@ -1149,7 +1163,9 @@ static int matmul_multi_impl(const tuna_gemm_problem *problems, int count, hipSt
         MultiPlan plan;
         int take = count - first < kMaxMultiProblems ? count - first : kMaxMultiProblems;
         const int min_batch = diag::multi_min_batch();
-        while (take >= min_batch && !plan_multi(problems + first, take, cus, &plan)) --take;
+        while (take >= min_batch && !plan_multi(problems + first, take, cus, &plan, 0, 0, -1, epilogues ? epilogues + first : nullptr,
+                                                residuals ? residuals + first : nullptr))
+            --take;
         if (take >= min_batch) {
             if ((rc = provide_workspace(false, stream, plan.ws_bytes, plan.n_counters, &plan.args.ws, &plan.args.counters))) return rc;
             e = launch_gemm_multi(plan.args, plan.prefetch, dev, stream);
@@ -1159,7 +1175,10 @@ static int matmul_multi_impl(const tuna_gemm_problem *problems, int count, hipSt
             continue;
         }
         const tuna_gemm_problem &p = problems[first];
-        if ((rc = matmul_impl(p.q, p.x, p.code, p.absmax, p.out, p.m, p.n, p.k, nullptr, TUNA_DECODE_GEMM, stream))) return rc;
+        const int ep = epilogues ? epilogues[first] : TUNA_EPILOGUE_NONE;
+        if ((rc = matmul_impl(p.q, p.x, p.code, p.absmax, p.out, p.m, p.n, p.k, nullptr, TUNA_DECODE_GEMM, stream, ep,
+                              ep == TUNA_EPILOGUE_RESIDUAL ? residuals[first] : nullptr)))
+            return rc;
         ++first;
     }
     return TUNA_OK;
@@ -1265,6 +1284,12 @@ TUNA_EXPORT int tuna_matmul_fused(const void *q, const void *x, const void *code
 TUNA_EXPORT int tuna_matmul_multi(const tuna_gemm_problem *problems, int count, void *stream)
 {
     return matmul_multi_impl(problems, count, static_cast<hipStream_t>(stream));
+}
+
+TUNA_EXPORT int tuna_matmul_multi_fused(const tuna_gemm_problem *problems, const int32_t *epilogues, const void *const *residuals,
+                                        int count, void *stream)
+{
+    return matmul_multi_impl(problems, count, static_cast<hipStream_t>(stream), epilogues, residuals);
 }
 
 TUNA_EXPORT int tuna_matmul_multi_blockwise(const tuna_gemm_problem *problems, int count, int block_size, void *stream)

@@ -9,7 +9,8 @@ static const struct {
     int u;
     MultiKernelFn fn;
 } kMulti[] = {{2, gemm_multi_kernel<2>}, {4, gemm_multi_kernel<4>}, {-2, gemm_multi_kernel<2, true, true>},  // (-2: ring of 2, weights and x through LDS)
-              {12, gemm_multi_kernel<2, true, false, true>}, {14, gemm_multi_kernel<4, true, false, true>}};  // (10 + ring: a scale per block of a row)
+              {12, gemm_multi_kernel<2, true, false, true>}, {14, gemm_multi_kernel<4, true, false, true>},  // (10 + ring: a scale per block of a row)
+              {22, gemm_multi_kernel<2, true, false, false, true>}, {24, gemm_multi_kernel<4, true, false, false, true>}};  // (20 + ring: fused epilogues)
 static constexpr int kNumMulti = sizeof(kMulti) / sizeof(kMulti[0]);
 
 static OptInFlag g_multi_attr_done[16][kNumMulti];

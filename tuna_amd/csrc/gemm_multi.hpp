@@ -47,10 +47,11 @@ struct MultiProblem {
     const void *x;
     const float *absmax;
     void *out;
+    const void *residual;  // EPI variants: fp16 with the layout of out, added before the rounding (TUNA_EPILOGUE_RESIDUAL)
     int m, n, k;
     int units_per_tile;  // k / (32 * waves_k * U)
     int tile_begin;      // id of its first row tile (arrival counters)
-    int pad0, pad1, pad2;
+    int epilogue;        // EPI variants: TUNA_EPILOGUE_* of this problem's stores
 };
 
 struct MultiArgs {
@@ -71,7 +72,9 @@ struct MultiArgs {
     MultiProblem prob[kMaxMultiProblems];
 };
 
-template <int U, bool DEFER = true, bool LDSW = false, bool BLK = false>
+// EPI: the problems carry fused epilogues (epilogue.hpp): a segment remembers its problem and the two places that
+// store outputs look the problem's epilogue and residual up there (the other variants carry none of it).
+template <int U, bool DEFER = true, bool LDSW = false, bool BLK = false, bool EPI = false>
 __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
 {
     static_assert(!LDSW || U == 2, "LDS is full with a ring of two: table 64 KB, x 2 x 16 KB, rings 32 KB, reduction 32 KB");
@@ -128,6 +131,7 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         int tile_id;  // arrival counter
         int u0;       // first unit of the row tile in the batch's sequence
         int upt;      // units per row tile
+        int prob;     // EPI: index of the problem
     };
     int p_scan = a.first_problem[wg];  // problem of the last segment looked up (segments are looked up in order)
     auto seg_at = [&](int u) {
@@ -141,6 +145,7 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         s.out = reinterpret_cast<f16 *>(pr.out);
         s.m = pr.m, s.n = pr.n, s.k = pr.k;
         s.upt = pr.units_per_tile;
+        s.prob = EPI ? p_scan : 0;
         const int ul = u - unit_begin_p;
         const int row_tile = (int)((unsigned)ul / (unsigned)s.upt);
         const int u_in = ul - row_tile * s.upt;
@@ -296,13 +301,19 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
     // partial segments waiting for their hand-over, by slot (n_contrib == 0: none)
     struct Pending {
         f16 *out;
-        int m, n, row0, tile_id;
+        int m, n, row0, tile_id, prob;
         unsigned w_lo, n_contrib, first_slot;
     };
     Pending pend0 = {}, pend1 = {};
     // Last contributor of a row tile: every partial is in memory; add them in k order and store.
     auto finish = [&](const Pending &pd) {
         if (tid == 0) __hip_atomic_store(a.counters + pd.tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        int epi_ = TUNA_EPILOGUE_NONE;
+        const f16 *res_ = nullptr;
+        if constexpr (EPI) {
+            epi_ = a.prob[pd.prob].epilogue;
+            res_ = reinterpret_cast<const f16 *>(a.prob[pd.prob].residual);
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int f = ((i << wk_log2) + wk) * 64 + lane;
@@ -325,8 +336,8 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
             const int l = f >> 2, v = f & 3;
             const int tok = l & 15;
             if (tok < pd.n)
-                store_features4(pd.out, nullptr, TUNA_EPILOGUE_NONE, (size_t)tok, pd.m, pd.row0 + wm * 64 + (l >> 4) * 16 + v * 4, s4[0],
-                                s4[1], s4[2], s4[3]);
+                store_features4(pd.out, res_, epi_, (size_t)tok, pd.m, pd.row0 + wm * 64 + (l >> 4) * 16 + v * 4, s4[0], s4[1], s4[2],
+                                s4[3]);
         }
     };
 
@@ -474,6 +485,12 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
             sum_planes_any<2, 32>(wk_log2, redf, plane_floats, wm, wk, lane, o, 2 * h);
         }
         const bool partial = cur.part >= 0;
+        int epi_ = TUNA_EPILOGUE_NONE;
+        const f16 *res_ = nullptr;
+        if constexpr (EPI) {
+            epi_ = a.prob[cur.prob].epilogue;
+            res_ = reinterpret_cast<const f16 *>(a.prob[cur.prob].residual);
+        }
         float *mine = a.ws + ((size_t)wg * 2 + (size_t)(partial ? cur.part : 0)) * seg_floats + (size_t)wm * 1024;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -483,8 +500,8 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
                 const int l = f >> 2, v = f & 3;
                 const int tok = l & 15;
                 if (tok < cur.n)
-                    store_features4(cur.out, nullptr, TUNA_EPILOGUE_NONE, (size_t)tok, cur.m, cur.row0 + wm * 64 + (l >> 4) * 16 + v * 4,
-                                    o[i][0], o[i][1], o[i][2], o[i][3]);
+                    store_features4(cur.out, res_, epi_, (size_t)tok, cur.m, cur.row0 + wm * 64 + (l >> 4) * 16 + v * 4, o[i][0], o[i][1],
+                                    o[i][2], o[i][3]);
             } else {
                 store_partial(mine + (size_t)f * 4, f32x4{o[i][0], o[i][1], o[i][2], o[i][3]});
             }
@@ -492,7 +509,7 @@ __global__ __launch_bounds__(1024, 4) void gemm_multi_kernel(const MultiArgs a)
         if (partial) {
             Pending pd;
             pd.out = cur.out;
-            pd.m = cur.m, pd.n = cur.n, pd.row0 = cur.row0, pd.tile_id = cur.tile_id;
+            pd.m = cur.m, pd.n = cur.n, pd.row0 = cur.row0, pd.tile_id = cur.tile_id, pd.prob = cur.prob;
             const unsigned T = (unsigned)a.units_total, nw = (unsigned)a.n_wg;
             const unsigned u0 = (unsigned)cur.u0, u1 = u0 + (unsigned)cur.upt - 1u;
             pd.w_lo = ((u0 + 1u) * nw - 1u) / T;

@@ -110,9 +110,9 @@ def matmul_fused(x, q, s, c, o, m: int, n: int, k: int, epilogue: int, residual=
     _lib.check(rc)
 
 
-def problem_array(problems, block_size: int = None):
+def problem_array(problems, block_size: int = None, epilogues=None):
     """ctypes array of GemmProblem for matmul_multi / time_matmul_multi from (x, q, s, c, o, m, n, k) tuples
-    (block_size: s is [m, k / block_size])."""
+    (block_size: s is [m, k / block_size]; epilogues: per problem, EPILOGUE_SILU_MUL makes o [n, m/2])."""
     arr = (_lib.GemmProblem * len(problems))()
     for i, (x, q, s, c, o, m, n, k) in enumerate(problems):
         m, n, k = int(m), int(n), int(k)
@@ -120,23 +120,38 @@ def problem_array(problems, block_size: int = None):
         _require(q, "q", torch.uint8, m * k // 2)
         _require(s, "s", torch.float32, m if block_size is None else m * (k // int(block_size)))
         _require(c, "c", torch.float32, 16)
-        _require(o, "o", torch.float16, n * m)
+        _require(o, "o", torch.float16, n * m // 2 if epilogues is not None and epilogues[i] == _lib.EPILOGUE_SILU_MUL else n * m)
         arr[i] = _lib.GemmProblem(q.data_ptr(), x.data_ptr(), c.data_ptr(), s.data_ptr(), o.data_ptr(), m, n, k)
     return arr
 
 
-def matmul_multi(problems, block_size: int = None) -> None:
+def matmul_multi(problems, block_size: int = None, epilogues=None, residuals=None) -> None:
     """Several independent GEMMs in one call (tuna_matmul_multi): `problems` is a list of
     (x, q, s, c, o, m, n, k) tuples, each with the meaning of matmul's arguments.  With block_size every s is
-    [m, k / block_size], one scale per block of a row (tuna_matmul_multi_blockwise)."""
+    [m, k / block_size], one scale per block of a row (tuna_matmul_multi_blockwise).  With epilogues (one
+    EPILOGUE_* per problem) and residuals (a tensor or None per problem) the stores are fused as in matmul_fused
+    (tuna_matmul_multi_fused)."""
     if not problems:
         return
     if block_size is not None and (int(block_size) <= 0 or any(int(p[7]) % int(block_size) for p in problems)):
         raise ValueError(f"block_size={block_size} must divide every k")
-    arr = problem_array(problems, block_size)
+    if epilogues is not None and (block_size is not None or len(epilogues) != len(problems)):
+        raise ValueError("epilogues: one per problem, per-row scales only")
+    arr = problem_array(problems, block_size, epilogues)
     dev = problems[0][0].device
     with torch.cuda.device(dev):
-        if block_size is None:
+        if epilogues is not None:
+            eps = (ctypes.c_int32 * len(problems))(*[int(e) for e in epilogues])
+            res = (ctypes.c_void_p * len(problems))()
+            for i, (ep, (x, q, s, c, o, m, n, k)) in enumerate(zip(epilogues, problems)):
+                if ep == _lib.EPILOGUE_RESIDUAL:
+                    if residuals is None or residuals[i] is None:
+                        raise ValueError(f"problem {i}: EPILOGUE_RESIDUAL needs a residual tensor")
+                    _require(residuals[i], "residual", torch.float16, int(n) * int(m))
+                    res[i] = residuals[i].data_ptr()
+            rc = _lib.lib().tuna_matmul_multi_fused(arr, eps, ctypes.cast(res, ctypes.POINTER(ctypes.c_void_p)), len(problems),
+                                                    _stream(dev))
+        elif block_size is None:
             rc = _lib.lib().tuna_matmul_multi(arr, len(problems), _stream(dev))
         else:
             rc = _lib.lib().tuna_matmul_multi_blockwise(arr, len(problems), int(block_size), _stream(dev))
