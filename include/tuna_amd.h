@@ -243,6 +243,26 @@ int tuna_dequant_blockwise(const void *q, const void *absmax, const void *code, 
                            int block_size, int decode_mode, void *stream);
 int tuna_matmul_blockwise(const void *q, const void *x, const void *code, const void *absmax,
                           void *out, int m, int n, int k, int block_size, void *stream);
+/* tuna_matmul_blockwise with an explicit config (NULL: the library's choice, as tuna_matmul_blockwise).  The
+ * reference makes the scale block a field of every kernel config (deq_block_size, configs.cu:31); here a blockwise
+ * launch is described by the same tuna_gemm_config as a per-row one and what the config names decides the kernel:
+ * lds_tile_rows > 0 the many-token kernel (tile lds_tile_rows x 16 * token_tiles, k split split_k ways);
+ * rows_per_wave 16 / 32, or 64 with waves_m = 0, the narrow-row kernel (that many rows per workgroup, waves_k waves
+ * along k, ring `prefetch`, one or two token tiles); split_k == 0 the batched streaming kernel (waves_m x 16 / waves_m
+ * waves, ring `prefetch`); anything else the streaming kernel's scale-block twin (up to 64 tokens: unsplit row-tile
+ * walkers of waves_m x waves_k waves, ring, x chunk and stagger as named).  TUNA_ERR_UNSUPPORTED if the config cannot
+ * run the call. */
+int tuna_matmul_blockwise_ex(const void *q, const void *x, const void *code, const void *absmax,
+                             void *out, int m, int n, int k, int block_size,
+                             const tuna_gemm_config *cfg, void *stream);
+/* The config tuna_matmul_blockwise runs for (m, n, k, block_size): the tuned entry of the blockwise table, keyed by
+ * (m, token bucket, k, block_size), if there is one (*from_table = 1), else a config derived from the shape.  Host only. */
+int tuna_select_config_blockwise(int m, int n, int k, int block_size, tuna_gemm_config *cfg, int *from_table);
+/* TUNA_OK if `cfg` can run the blockwise GEMM (m, n, k, block_size).  Host only. */
+int tuna_validate_config_blockwise(int m, int n, int k, int block_size, const tuna_gemm_config *cfg);
+/* The blockwise table (generated from tuna_amd/configs/param_map_blockwise.json). */
+int tuna_blockwise_table_size(void);
+int tuna_blockwise_table_entry(int i, int *m, int *n_lo, int *n_hi, int *k, int *block_size, tuna_gemm_config *cfg);
 
 /* Shape -> config.  Replaces the if-chain of kernel.cu:3018-3156 over the constants of
  * configs.cu:56-3331 by a table lookup on (m, n-bucket, k) with a derived fallback.

@@ -58,6 +58,13 @@ int tuna_time_empty_launches(void *sink, int blocks, int threads, int n_streams,
  * synchronises `stream`. */
 int tuna_measure_handover(int same_xcd, int store_sc1, int load_sc1, int reuse, int pairs, int iters,
                           void *stream, double *out6);
+/* Same protocol for the blockwise GEMM with an explicit config, as tuna_matmul_blockwise_ex runs it: every absmax_list
+ * entry is fp32 [m, k / block_size]; cfg NULL = the library's choice.  What the tuner times the blockwise candidates
+ * with. */
+int tuna_time_matmul_blockwise(const void *const *q_list, const void *const *absmax_list, int n_sets,
+                               const void *x, const void *code, void *out, int m, int n, int k, int block_size,
+                               const tuna_gemm_config *cfg, int warmup, int iters, int use_graph,
+                               void *stream, float *elapsed_ms);
 /* Same protocol for tuna_matmul_multi: `problems` holds n_sets batches of `count` problems each,
  * iteration i is one call with batch (i mod n_sets); the time is that of `iters` calls. */
 int tuna_time_matmul_multi(const tuna_gemm_problem *problems, int n_sets, int count, int warmup,
@@ -118,16 +125,6 @@ int tuna_set_multi_shape(int waves_m, int prefetch);
  * (global -> LDS loads, as the LDS-staged twins of the streaming kernel do) instead of registers.
  * Bit-identical results; for A/B timing.  Returns the previous setting. */
 int tuna_set_multi_weight_path(int through_lds);
-/* Diagnostic switch, process-wide, default 1: tuna_matmul_blockwise runs launches of more than 32 tokens through the
- * many-token kernel's scale-block variants, and large launches whose shape allows (m a multiple of 64, k of 256 and of
- * the block; 17 to 32 tokens from 100 MB of packed weights, from 40 MB when k > 4096 and from 12 MB when k > 8192, 9 to 16 tokens from 100 MB or from 20 MB when k >= 12288,
- * 5 to 8 tokens from 100 MB, 1 to 4 tokens from 256 MB) through the scale-block variant of the batched streaming kernel
- * (a batch of one up to 16 tokens, the token chunks as a batch beyond), and, ahead of both, launches of up to 64 tokens
- * on shapes of at least 16384 rows and 48 MB of packed weights (up to 16 tokens: less than 400 MB; from 33: at least
- * 100 MB) through the streaming kernel's scale-block twin; 2: the batched streaming kernel for every launch it can plan,
- * whatever its size and token count; 3: the streaming kernel's twin for every launch of up to 64 tokens it can plan; 0: always the narrow-row kernel's variants.  All decode fp16(code) * fp16(absmax of
- * the block); the sums differ in summation order only.  Returns the previous setting. */
-int tuna_set_blockwise_stream(int enabled);
 /* Diagnostic: tuna_matmul_blockwise calls so far in this process that ran the narrow-row kernel (kernel 0), launches of
  * the batched streaming kernel (1), calls that ran the many-token kernel (2) and calls that ran the streaming kernel's
  * scale-block twin (3) on their behalf. */
@@ -137,10 +134,6 @@ unsigned long long tuna_blockwise_launches(int kernel);
  * Bit-identical results.  Returns the previous setting. */
 int tuna_set_blockwise_scales_lds(int enabled);
 
-/* Diagnostic override of the kernel variant tuna_matmul_blockwise runs: rows per workgroup (16, 32 or 64), waves along k
- * (4, 8 or 16) and ring depth (2 or 4); all zero = the library's choice.  TUNA_ERR_INVALID_ARG if no such variant is built;
- * a variant that does not fit a later call's shape makes that call fail with TUNA_ERR_UNSUPPORTED.  For A/B timing. */
-int tuna_set_blockwise_shape(int rows, int waves_k, int prefetch);
 /* Diagnostic: the shortest run of problems tuna_matmul_multi hands to the batched kernel
  * (default 2; 1 sends single problems through it as well).  Returns the previous value. */
 int tuna_set_multi_min_batch(int count);

@@ -1744,6 +1744,38 @@ def test_blockwise_gemm_matches_oracle_and_reads_out_the_decode(m, n, k, bs):
     assert np.array_equal(out.cpu().numpy().view(np.uint16), img[:, cols].T)
 
 
+def blockwise_cfg(family, m, n, k, bs, shape=None):
+    """An explicit config that sends a blockwise launch to one kernel family (the rule of tuna_matmul_blockwise_ex):
+    "narrow" with shape = (rows, waves along k, ring) or the first variant that fits, "batched" with the tallest row
+    tile the shape allows, "streaming" with four waves by four (eight waves for four token tiles)."""
+    from tuna_amd import ops
+
+    tiles = 4 if n > 32 else 2 if n > 16 else 1
+    cands = []
+    if family == "narrow":
+        shapes = [shape] if shape else [(64, 8, 4), (64, 8, 2), (32, 8, 4), (32, 8, 2), (16, 8, 4), (16, 4, 2)]
+        for rows, wk, u in shapes:
+            for tt in ((2, 1) if n > 16 else (1,)):
+                cands.append(cfg(rows_per_wave=rows, waves_m=0 if rows == 64 else 1, waves_k=wk, split_k=1, prefetch=u, x_chunk=512,
+                                 token_tiles=tt))
+    elif family == "batched":
+        for wm in (4, 2, 1):
+            cands.append(cfg(rows_per_wave=64, waves_m=wm, waves_k=16 // wm, split_k=0, prefetch=2, x_chunk=512, token_tiles=1))
+    elif family == "streaming":
+        wm = 4 if m % 256 == 0 else 2 if m % 128 == 0 else 1
+        wk = min(8, (8 if tiles == 4 else 16) // wm)
+        cands.append(cfg(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=1, prefetch=2, x_chunk=256 if tiles == 4 else 512,
+                         token_tiles=tiles))
+    for c in cands:
+        try:
+            ops.validate_config_blockwise(m, n, k, bs, c)
+            return c
+        except ops.TunaError:
+            continue
+    raise AssertionError(f"no {family} blockwise config for m={m} n={n} k={k} block={bs} shape={shape}")
+
+
+
 @pytest.mark.parametrize("m,n,k,bs,shape", [
     (256, 16, 28672, 64, None),          # 16-row tiles, 7168 scales per workgroup: two rounds of the prologue copy
     (1024, 16, 8192, 64, (64, 8, 4)),    # 64-row tiles, 8192 scales: two rounds
@@ -1773,12 +1805,11 @@ def test_blockwise_narrow_kernel_with_scales_in_lds_and_in_memory(m, n, k, bs, s
     absmax = rng.uniform(0.005, 0.02, size=(m, k // bs)).astype(np.float16).astype(np.float32)
     dq, dx, dc, da = to_dev(q, x, code, absmax)
     L = _lib.lib()
-    prev_stream = L.tuna_set_blockwise_stream(0)
     prev_lds = L.tuna_set_blockwise_scales_lds(1)
-    if shape:
-        assert L.tuna_set_blockwise_shape(*shape) == 0
+    c = blockwise_cfg("narrow", m, n, k, bs, shape)
+    before = L.tuna_blockwise_launches(0)
     try:
-        print(f"blockwise narrow rows m={m} n={n} k={k} block={bs} variant={shape}", flush=True)
+        print(f"blockwise narrow rows m={m} n={n} k={k} block={bs} variant={shape} cfg={c.to_dict()}", flush=True)
         cols = rng.choice(k, size=n, replace=False)
         xh = np.zeros((n, k), np.float16)
         xh[np.arange(n), cols] = 1.0
@@ -1788,12 +1819,13 @@ def test_blockwise_narrow_kernel_with_scales_in_lds_and_in_memory(m, n, k, bs, s
         for lds in (1, 0):
             L.tuna_set_blockwise_scales_lds(lds)
             out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
-            ops.matmul_blockwise(dx, dq, da, dc, out, m, n, k, bs)
+            ops.matmul_blockwise(dx, dq, da, dc, out, m, n, k, bs, config=c)
             torch.cuda.synchronize()
             got[lds] = out.cpu().numpy().view(np.uint16)
-            ops.matmul_blockwise(dxh, dq, da, dc, out, m, n, k, bs)
+            ops.matmul_blockwise(dxh, dq, da, dc, out, m, n, k, bs, config=c)
             torch.cuda.synchronize()
             assert np.array_equal(out.cpu().numpy().view(np.uint16), img[:, cols].T), lds
+        assert L.tuna_blockwise_launches(0) == before + 4          # the narrow-row kernel ran all four
         assert not np.isnan(got[1].view(np.float16)).any()
         assert np.array_equal(got[1], got[0])
         rows = np.sort(rng.choice(m, size=min(m, 128), replace=False)).astype(np.int32)
@@ -1801,9 +1833,7 @@ def test_blockwise_narrow_kernel_with_scales_in_lds_and_in_memory(m, n, k, bs, s
         e = rel_err(f16_bits_to_f64(got[1][:, rows]), ref)
         assert e <= REL_TOL, e
     finally:
-        L.tuna_set_blockwise_shape(0, 0, 0)
         L.tuna_set_blockwise_scales_lds(prev_lds)
-        L.tuna_set_blockwise_stream(prev_stream)
 
 
 @pytest.mark.usefixtures("diagnostic_build")
@@ -1811,8 +1841,8 @@ def test_blockwise_narrow_kernel_with_scales_in_lds_and_in_memory(m, n, k, bs, s
                                       (256, 16, 2048, 512), (768, 13, 5120, 64), (4096, 16, 4096, 64), (8192, 16, 8192, 64),
                                       (512, 37, 2048, 256), (256, 100, 1024, 64), (256, 530, 512, 64)])
 def test_blockwise_gemm_through_the_batched_streaming_kernel(m, n, k, bs):
-    """The scale-block variant of the batched streaming kernel (tuna_matmul_blockwise takes it from 20 MB of packed
-    weights; the switch sends every shape it can plan there): against the oracle's float64 sums over the blockwise D1
+    """The scale-block variant of the batched streaming kernel (tuna_matmul_blockwise takes it for large aligned shapes; here
+    an explicit config sends every shape there): against the oracle's float64 sums over the blockwise D1
     weights on a row sample, bit-exact through one-hot activations (every scale block of every sampled column read
     out), and run-to-run identical.  k ranges that are not whole x chunks, 128-row tiles, blocks longer than a chunk,
     shares that split row tiles (hand-over through the workspace); more than 16 tokens run as the token chunks of a
@@ -1827,11 +1857,11 @@ def test_blockwise_gemm_through_the_batched_streaming_kernel(m, n, k, bs):
     dq, dx, dc, da = to_dev(q, x, code, absmax)
     out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
     L = _lib.lib()
-    prev = L.tuna_set_blockwise_stream(2)
+    c = blockwise_cfg("batched", m, n, k, bs)
     launches = L.tuna_multi_launches()
-    try:
-        print(f"blockwise through the batched kernel m={m} n={n} k={k} block={bs}", flush=True)
-        ops.matmul_blockwise(dx, dq, da, dc, out, m, n, k, bs)
+    if True:
+        print(f"blockwise through the batched kernel m={m} n={n} k={k} block={bs} cfg={c.to_dict()}", flush=True)
+        ops.matmul_blockwise(dx, dq, da, dc, out, m, n, k, bs, config=c)
         torch.cuda.synchronize()
         got = out.cpu().numpy().view(np.uint16)
         assert L.tuna_multi_launches() == launches + -(-(-(-n // 16)) // 32)     # the batched kernel ran it
@@ -1841,7 +1871,7 @@ def test_blockwise_gemm_through_the_batched_streaming_kernel(m, n, k, bs):
         e = rel_err(f16_bits_to_f64(got[:, rows]), ref)
         assert e <= REL_TOL, e
         again = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
-        ops.matmul_blockwise(dx, dq, da, dc, again, m, n, k, bs)
+        ops.matmul_blockwise(dx, dq, da, dc, again, m, n, k, bs, config=c)
         torch.cuda.synchronize()
         assert np.array_equal(again.cpu().numpy().view(np.uint16), got)
         img = O.dequant(q, absmax, code, m, k, mode=O.D1, block_size=bs)
@@ -1852,11 +1882,9 @@ def test_blockwise_gemm_through_the_batched_streaming_kernel(m, n, k, bs):
             xh = np.zeros((n, k), np.float16)
             xh[np.arange(n), cols] = 1.0
             dxh, = to_dev(xh)
-            ops.matmul_blockwise(dxh, dq, da, dc, out, m, n, k, bs)
+            ops.matmul_blockwise(dxh, dq, da, dc, out, m, n, k, bs, config=c)
             torch.cuda.synchronize()
             assert np.array_equal(out.cpu().numpy().view(np.uint16), img[:, cols].T)
-    finally:
-        L.tuna_set_blockwise_stream(prev)
 
 
 @pytest.mark.usefixtures("diagnostic_build")
@@ -1867,8 +1895,8 @@ def test_blockwise_gemm_through_the_batched_streaming_kernel(m, n, k, bs):
                                       (512, 64, 2048, 64), (1024, 40, 4096, 128), (256 * 70, 33, 1024, 64), (28672, 64, 4096, 64)])
 def test_blockwise_gemm_through_the_streaming_kernel(m, n, k, bs):
     """The scale-block twin of the streaming kernel (tuna_matmul_blockwise takes it for the largest shapes at up to 64
-    tokens, two token tiles from 17 and four from 33; the switch sends every launch it can plan there, with the per-row table's workgroup shape or four waves
-    by four): oracle on a row sample, exact read-out of the decoded weights with random scales per block (blocks
+    tokens, two token tiles from 17 and four from 33; here every case goes there, with the library's own config where it names
+    this kernel, else four waves by four): oracle on a row sample, exact read-out of the decoded weights with random scales per block (blocks
     shorter and longer than an x chunk, workgroups that walk several row tiles), run-to-run identical."""
     import torch
 
@@ -1879,12 +1907,14 @@ def test_blockwise_gemm_through_the_streaming_kernel(m, n, k, bs):
     absmax = rng.uniform(0.005, 0.02, size=(m, k // bs)).astype(np.float16).astype(np.float32)
     dq, dx, dc, da = to_dev(q, x, code, absmax)
     L = _lib.lib()
-    prev = L.tuna_set_blockwise_stream(3)
+    c, hit = ops.select_config_blockwise(m, n, k, bs)
+    if ops.blockwise_family(c) != "streaming":      # (the library's own choice where that is this kernel already)
+        c = blockwise_cfg("streaming", m, n, k, bs)
     before = L.tuna_blockwise_launches(3)
-    try:
-        print(f"blockwise through the streaming kernel m={m} n={n} k={k} block={bs}", flush=True)
+    if True:
+        print(f"blockwise through the streaming kernel m={m} n={n} k={k} block={bs} cfg={c.to_dict()}", flush=True)
         out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
-        ops.matmul_blockwise(dx, dq, da, dc, out, m, n, k, bs)
+        ops.matmul_blockwise(dx, dq, da, dc, out, m, n, k, bs, config=c)
         torch.cuda.synchronize()
         assert L.tuna_blockwise_launches(3) == before + 1     # that kernel ran it
         got = out.cpu().numpy().view(np.uint16)
@@ -1894,7 +1924,7 @@ def test_blockwise_gemm_through_the_streaming_kernel(m, n, k, bs):
         e = rel_err(f16_bits_to_f64(got[:, rows]), ref)
         assert e <= REL_TOL, e
         again = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
-        ops.matmul_blockwise(dx, dq, da, dc, again, m, n, k, bs)
+        ops.matmul_blockwise(dx, dq, da, dc, again, m, n, k, bs, config=c)
         torch.cuda.synchronize()
         assert np.array_equal(again.cpu().numpy().view(np.uint16), got)
         img = O.dequant(q, absmax, code, m, k, mode=O.D1, block_size=bs)
@@ -1903,11 +1933,9 @@ def test_blockwise_gemm_through_the_streaming_kernel(m, n, k, bs):
             xh = np.zeros((n, k), np.float16)
             xh[np.arange(n), cols] = 1.0
             dxh, = to_dev(xh)
-            ops.matmul_blockwise(dxh, dq, da, dc, out, m, n, k, bs)
+            ops.matmul_blockwise(dxh, dq, da, dc, out, m, n, k, bs, config=c)
             torch.cuda.synchronize()
             assert np.array_equal(out.cpu().numpy().view(np.uint16), img[:, cols].T)
-    finally:
-        L.tuna_set_blockwise_stream(prev)
 
 
 @pytest.mark.usefixtures("diagnostic_build")

@@ -163,8 +163,27 @@ def test_generator_output_and_its_refusal_of_inconsistent_entries(tmp_path):
     # the checked-in table is what the generator produces from the checked-in json
     with open(os.path.join(ROOT, "tuna_amd", "configs", "param_map.json")) as f:
         real = json.load(f)
+    with open(os.path.join(ROOT, "tuna_amd", "configs", "param_map_blockwise.json")) as f:
+        real_blk = json.load(f)
     with open(os.path.join(ROOT, "tuna_amd", "csrc", "config_table.cpp")) as f:
-        assert f.read() == mc.generate(real)
+        assert f.read() == mc.generate(real) + mc.generate_blockwise(real_blk)
+    # blockwise entries: the config names the kernel family; inconsistent ones are refused with their key
+    blk = {"8192_16_8192_64": dict(rows_per_wave=64, waves_m=0, waves_k=8, split_k=1, prefetch=4, x_chunk=512, token_tiles=1, xcd_swizzle=0),
+           "57344_16_8192_64": dict(rows_per_wave=64, waves_m=4, waves_k=4, split_k=1, prefetch=4, x_chunk=512, token_tiles=1, xcd_swizzle=1,
+                                    k_stagger=5),
+           "8192_16_28672_128": dict(rows_per_wave=64, waves_m=4, waves_k=4, split_k=0, prefetch=2, x_chunk=512, token_tiles=1, xcd_swizzle=0),
+           "4096_64_4096_64": dict(rows_per_wave=64, waves_m=1, waves_k=1, split_k=2, prefetch=2, x_chunk=64, token_tiles=4, xcd_swizzle=0,
+                                   lds_tile_rows=256)}
+    text = mc.generate_blockwise(blk)
+    assert "{8192, 16, 31, 8192, 64, {64, 0, 8, 1, 4, 512, 1, 0, 0, 0}},  // 8192_16_8192_64: narrow" in text
+    assert "// 57344_16_8192_64: streaming" in text and "// 8192_16_28672_128: batched" in text and "// 4096_64_4096_64: many-token" in text
+    assert "kBlockwiseTableSize = 4" in text
+    for bad_key, bad in (("8192_16_8192_96", blk["8192_16_8192_64"]),                                   # not a power of two
+                         ("8192_16_8192_64", dict(blk["8192_16_8192_64"], waves_k=2)),                   # no such narrow variant
+                         ("4096_64_4096_64", dict(blk["4096_64_4096_64"], token_tiles=16)),              # the 256 x 256 tile has no scale blocks
+                         ("8192_128_8192_64", blk["57344_16_8192_64"])):                                # streaming twin: up to 64 tokens
+        with pytest.raises(ValueError, match=bad_key):
+            mc.generate_blockwise({bad_key: bad})
     # an entry like the reference's gemm_229376_4096_16 (thread count inconsistent with its warp grid) is refused
     pm["229376_16_4096"] = dict(pm["4096_16_4096"], waves_m=8, waves_k=8)
     with pytest.raises(ValueError, match="229376_16_4096"):

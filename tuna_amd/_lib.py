@@ -87,6 +87,11 @@ SIGNATURES = {
     "tuna_quantize_blockwise": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "tuna_dequant_blockwise": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "tuna_matmul_blockwise": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "tuna_matmul_blockwise_ex": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _cfgp, _vp]),
+    "tuna_select_config_blockwise": (_i, [_i, _i, _i, _i, _cfgp, _ip]),
+    "tuna_validate_config_blockwise": (_i, [_i, _i, _i, _i, _cfgp]),
+    "tuna_blockwise_table_size": (_i, []),
+    "tuna_blockwise_table_entry": (_i, [_i, _ip, _ip, _ip, _ip, _ip, _cfgp]),
     "tuna_dequant_ex": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "tuna_select_config": (_i, [_i, _i, _i, _cfgp, _ip]),
     "tuna_select_config_ex": (_i, [_i, _i, _i, _i, _cfgp, _ip]),
@@ -118,8 +123,7 @@ BENCH_SIGNATURES = {
     "tuna_selftest_quantizer_division": (_i, [_vp, _vp]),
     "tuna_set_multi_shape": (_i, [_i, _i]),
     "tuna_set_multi_min_batch": (_i, [_i]),
-    "tuna_set_blockwise_shape": (_i, [_i, _i, _i]),
-    "tuna_set_blockwise_stream": (_i, [_i]),
+    "tuna_time_matmul_blockwise": (_i, [_vpp, _vpp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _cfgp, _i, _i, _i, _vp, _fp]),
     "tuna_blockwise_launches": (ctypes.c_ulonglong, [_i]),
     "tuna_multi_launches": (ctypes.c_ulonglong, []),
     "tuna_set_lean_kernels": (_i, [_i]),

@@ -1362,190 +1362,325 @@ TUNA_EXPORT int tuna_quantize_blockwise(const void *w, const void *code, void *q
     return quantize_impl(w, code, q, absmax, m, k, block_size, static_cast<hipStream_t>(stream));
 }
 
-// Shapes on which the streaming kernel's scale-block twin beats the narrow-row, the batched and the many-token kernel
-// at up to 64 tokens: many rows (it does not split k) and at least 48 MB of packed weights (up to 16 tokens: less than
-// 400 MB; from 33 tokens: at least 100 MB).
-// Measured with a scale per 64 weights, us, twin / narrow-row / batched.  16 tokens: 62-64 / 77 / 68-69 on
-// 57344 x 8192, 21.5-22.2 / 23.3 / 24.6 on 28672 x 4096, 64-65 / 71 / 64 on 32768 x 14336, but 132 / 148 / 114 on
-// 229376 x 4096 (whose per-row entry - 16 waves along the rows, chunks of 2048 k - has more scales per thread and
-// chunk than the twin stages).  32 tokens (two token tiles: one pass over the weights, where the batched kernel makes
-// two): 80 / 131 / 117, 30.7 / 31.5 / 40.6, 78 / 134 / 112 and 169 / 205 / 210.  64 tokens (four token tiles), twin /
-// many-token kernel: 103 / 130, 49.9 / 47.5, 111 / 125 and 182 / 252: from 100 MB there.
-static bool mid_blockwise_wins(int m, int n, int k)
+// ---------------------------------------------------------------------------------------
+// GEMM with scale blocks finer than a row (absmax [m, k / block_size]).
+//
+// A launch is described by a tuna_gemm_config, like a per-row one, and what the config names decides the kernel:
+//   lds_tile_rows > 0                     the many-token kernel's scale-block variants: tile lds_tile_rows x 16 * token_tiles,
+//                                         k split split_k ways (16 x 16 x 32 MFMA tiles; no 256 x 256 tile)
+//   rows_per_wave 16 / 32, or 64 with     the narrow-row kernel's scale-block variants: that many rows per workgroup,
+//   waves_m = 0                           waves_k waves along k, ring `prefetch`, one or two token tiles per pass
+//   split_k == 0                          the batched streaming kernel as a batch of one (or of the token chunks):
+//                                         waves_m x 16 / waves_m waves, ring `prefetch`, balanced split
+//   anything else                         the streaming kernel's scale-block twin: unsplit row-tile walkers with the
+//                                         config's workgroup shape, ring, x chunk and stagger, 1 / 2 / 4 token tiles
+// A config comes from the caller (tuna_matmul_blockwise_ex), from the table of tuned entries keyed by (m, token bucket,
+// k, block_size) (config_table.cpp, written by the tuner), or from the rules of derive_blockwise below.
+// ---------------------------------------------------------------------------------------
+enum BlockwiseFamily { kBlkNarrow = 0, kBlkMulti = 1, kBlkTiled = 2, kBlkMid = 3 };
+
+static BlockwiseFamily blockwise_family(const tuna_gemm_config &c)
 {
+    if (c.lds_tile_rows > 0) return kBlkTiled;
+    if (is_narrow(c)) return kBlkNarrow;
+    if (c.split_k == 0) return kBlkMulti;
+    return kBlkMid;
+}
+
+struct BlockwiseCall {
+    const void *q, *x, *code, *absmax;
+    void *out;
+    int m, n, k, block_size;
+};
+
+// Runs `c` on the call (dry: checks only that it could, launches nothing, needs no device).
+static int run_blockwise(const BlockwiseCall &b, const tuna_gemm_config &c, hipStream_t st, bool dry)
+{
+    const int m = b.m, n = b.n, k = b.k, shift = log2i(b.block_size) - 6;
+    int rc, dev = 0, cus = kMaxCus;
+    hipError_t e = device_cus(&dev, &cus);
+    if (e != hipSuccess) {
+        if (!dry) return hip_fail(e, "hipGetDevice");
+        (void)hipGetLastError();
+        dev = 0, cus = kMaxCus;
+    }
+    switch (blockwise_family(c)) {
+    case kBlkNarrow: {
+        if (c.token_tiles != 1 && c.token_tiles != 2) return fail(TUNA_ERR_UNSUPPORTED, "narrow-row scale-block kernel: one or two token tiles");
+        if (!blockwise_narrow_runs(m, k, c.rows_per_wave, c.waves_k, c.prefetch, c.token_tiles))
+            return fail(TUNA_ERR_UNSUPPORTED, "no narrow-row scale-block variant with %d rows, %d waves, ring %d, %d token tiles fits m=%d k=%d",
+                        c.rows_per_wave, c.waves_k, c.prefetch, c.token_tiles, m, k);
+        if (dry) return TUNA_OK;
+        NarrowArgs a;
+        memset(&a, 0, sizeof(a));
+        a.q = static_cast<const uint8_t *>(b.q);
+        a.x = b.x;
+        a.code = static_cast<const float *>(b.code);
+        a.absmax = static_cast<const float *>(b.absmax);
+        a.out = b.out;
+        a.m = m, a.n = n, a.k = k;
+        e = launch_gemm_blockwise(a, shift, c.rows_per_wave, c.waves_k, c.prefetch, c.token_tiles, st);
+        if (e != hipSuccess) return hip_fail(e, "blockwise gemm launch");
+        diag::count(diag::kBlockwiseNarrow);
+        return TUNA_OK;
+    }
+    case kBlkMulti: {
+        // a batch of one for up to 16 tokens; the token chunks of 16 as the problems of a batch beyond that (every chunk
+        // streams the weights again, in one launch per 32 chunks)
+        const int chunks = (n + 15) / 16;
+        auto plan_batch = [&](int c0, MultiPlan *plan) {
+            const int cnt = chunks - c0 < kMaxMultiProblems ? chunks - c0 : kMaxMultiProblems;
+            tuna_gemm_problem probs[kMaxMultiProblems];
+            for (int ch = 0; ch < cnt; ++ch) {
+                const int t0 = (c0 + ch) * 16;
+                probs[ch] = {b.q, static_cast<const char *>(b.x) + (size_t)t0 * k * 2, b.code, b.absmax,
+                             static_cast<char *>(b.out) + (size_t)t0 * m * 2, m, n - t0 < 16 ? n - t0 : 16, k};
+            }
+            return plan_multi(probs, cnt, cus, plan, c.waves_m, c.prefetch, shift);
+        };
+        if (c.waves_m < 1 || c.waves_m * c.waves_k != 16) return fail(TUNA_ERR_UNSUPPORTED, "batched scale-block kernel: waves_m x waves_k must be 16 waves");
+        for (int c0 = 0; c0 < chunks; c0 += kMaxMultiProblems) {  // (nothing is enqueued unless every batch of chunks can run)
+            MultiPlan plan;
+            if (!plan_batch(c0, &plan)) return fail(TUNA_ERR_UNSUPPORTED, "the batched scale-block kernel cannot take m=%d n=%d k=%d with %d x %d waves, ring %d", m, n, k, c.waves_m, c.waves_k, c.prefetch);
+        }
+        if (dry) return TUNA_OK;
+        for (int c0 = 0; c0 < chunks; c0 += kMaxMultiProblems) {
+            MultiPlan plan;
+            if (!plan_batch(c0, &plan)) return fail(TUNA_ERR_UNSUPPORTED, "blockwise gemm: a batch of token chunks stopped planning");
+            if ((rc = provide_workspace(false, st, plan.ws_bytes, plan.n_counters, &plan.args.ws, &plan.args.counters))) return rc;
+            e = launch_gemm_multi(plan.args, plan.prefetch, dev, st);
+            if (e != hipSuccess) return hip_fail(e, "blockwise gemm launch");
+            diag::count(diag::kMultiLaunches);
+            diag::count(diag::kBlockwiseMulti);
+        }
+        return TUNA_OK;
+    }
+    case kBlkTiled: {
+        tuna_gemm_config t = c;
+        t.rows_per_wave = 64;  // (16 x 16 x 32 MFMA tiles: the scale-block variants exist for those)
+        // (the 256 x 256 tile has no scale-block variant: its threads have no registers left for eight more scales)
+        if (!tiled_variant_exists(t.lds_tile_rows, 16 * t.token_tiles, false) || (t.lds_tile_rows == 256 && t.token_tiles == 16))
+            return fail(TUNA_ERR_UNSUPPORTED, "no many-token scale-block variant with a %d x %d tile", t.lds_tile_rows, 16 * t.token_tiles);
+        TiledPlan tp;
+        if ((rc = plan_tiled(m, n, k, t, TUNA_DECODE_GEMM, &tp))) return rc;
+        if (dry) return TUNA_OK;
+        tp.args.q = static_cast<const uint8_t *>(b.q);
+        tp.args.x = b.x;
+        tp.args.code = static_cast<const float *>(b.code);
+        tp.args.absmax = static_cast<const float *>(b.absmax);
+        tp.args.out = b.out;
+        tp.args.epilogue = TUNA_EPILOGUE_NONE;
+        tp.args.residual = nullptr;
+        tp.args.blk_shift = shift;
+        if (tp.ws_bytes && (rc = provide_workspace(false, st, tp.ws_bytes, tp.n_counters, &tp.args.ws, &tp.args.counters))) return rc;
+        e = launch_gemm_tiled(tp.args, tp.tile_rows, tp.tile_tokens, false, st, true);
+        if (e != hipSuccess) return hip_fail(e, "many-token blockwise gemm launch");
+        diag::count(diag::kBlockwiseTiled);
+        return TUNA_OK;
+    }
+    case kBlkMid: {
+        tuna_gemm_config t = c;
+        t.lds_tile_rows = 0;  // (register ring: the twins have no LDS-staged form)
+        const int tiles = n > 32 ? 4 : n > 16 ? 2 : 1;  // token tiles: one pass over the weights
+        GemmPlan plan;
+        if (n > 64 || t.token_tiles != tiles || t.split_k != 1 || t.rows_per_wave != 64 || t.waves_m < 1 || m % (64 * t.waves_m) != 0)
+            return fail(TUNA_ERR_UNSUPPORTED, "streaming scale-block twin: up to 64 tokens in one pass (%d token tiles), unsplit, m=%d a multiple of 64 x waves_m", tiles, m);
+        if ((rc = plan_gemm(m, n, k, t, TUNA_DECODE_GEMM, &plan))) return rc;
+        if (!mid_blockwise_applies(plan, shift)) return fail(TUNA_ERR_UNSUPPORTED, "no streaming scale-block twin for this workgroup shape, ring and x chunk");
+        if (dry) return TUNA_OK;
+        plan.args.q = static_cast<const uint8_t *>(b.q);
+        plan.args.x = b.x;
+        plan.args.code = static_cast<const float *>(b.code);
+        plan.args.absmax = static_cast<const float *>(b.absmax);
+        plan.args.out = b.out;
+        plan.args.epilogue = TUNA_EPILOGUE_NONE;
+        plan.args.residual = nullptr;
+        e = launch_gemm_mid_blockwise(plan, shift, dev, cus, st);
+        if (e != hipSuccess) return hip_fail(e, "streaming blockwise gemm launch");
+        diag::count(diag::kBlockwiseMid);
+        return TUNA_OK;
+    }
+    }
+    return fail(TUNA_ERR_UNSUPPORTED, "unknown blockwise kernel family");
+}
+
+// The config for a shape that has no tuned entry, from what the tuner found on the benchmark shapes (a scale per 64
+// weights, us).  The streaming kernel's twin where the per-row table has an unsplit streaming entry for the shape and
+// it has many rows and at least 48 MB of packed weights (up to 16 tokens: less than 400 MB; from 33 tokens: at least
+// 100 MB) - twin / narrow-row / batched at 16 tokens: 62-64 / 77 / 68-69 on 57344 x 8192, 21.5-22.2 / 23.3 / 24.6 on
+// 28672 x 4096, 64-65 / 71 / 64 on 32768 x 14336, but 132 / 148 / 114 on 229376 x 4096; at 32 tokens 80 / 131 / 117,
+// 30.7 / 31.5 / 40.6, 78 / 134 / 112 and 169 / 205 / 210; at 64 tokens twin / many-token kernel 103 / 130, 49.9 / 47.5,
+// 111 / 125 and 182 / 252.  From 33 tokens otherwise the many-token kernel: the per-row entry's tile if it is one, else
+// 256 x 64 up to 64 tokens, 128 x 128 up to 128, 128 x 256 beyond, k split until the launch fills the device.  The
+// batched kernel for large aligned shapes - narrow / batched at 16 tokens: 8.7 / 15.5 on 6144 x 4096, 14.1 / 16.3 on
+// 8192 x 8192, 19.4 / 20.9 on 10240 x 8192, 22.4 / 24.2 on 28672 x 4096, but 18.5 / 16.5 on 4096 x 14336, 44 / 35 on
+// 8192 x 28672, 75 / 66 on 57344 x 8192; at one token the narrow kernel wins up to 57344 x 8192 (63 / 65) and loses on
+// 229376 x 4096 (117 / 102); at 32 tokens 11.9 / 16.9 on 6144 x 4096, 20.3 / 24.6 on 8192 x 8192, 30.9 / 38.7 on
+// 28672 x 4096, but 37.2 / 30.4 on 10240 x 8192, 29.6 / 22.7 on 4096 x 14336, 134 / 106 on 32768 x 14336.  Everything
+// else: the narrow-row kernel, the widest tile that gives nine workgroups per sixteen compute units.
+static int derive_blockwise(const BlockwiseCall &b, tuna_gemm_config *out)
+{
+    const int m = b.m, n = b.n, k = b.k, shift = log2i(b.block_size) - 6;
     const long long packed_bytes = (long long)m * k / 2;
-    if (n > 32) return m >= 16384 && packed_bytes >= (100ll << 20);
-    return m >= 16384 && packed_bytes >= (48ll << 20) && (n > 16 || packed_bytes < (400ll << 20));
+    int dev = 0, cus = kMaxCus;
+    if (device_cus(&dev, &cus) != hipSuccess) {
+        (void)hipGetLastError();
+        cus = kMaxCus;
+    }
+    tuna_gemm_config row;  // the per-row GEMM's config for the shape
+    select_config(m, n, k, &row, nullptr);
+    const bool mid_wins = n > 32 ? m >= 16384 && packed_bytes >= (100ll << 20)
+                                 : m >= 16384 && packed_bytes >= (48ll << 20) && (n > 16 || packed_bytes < (400ll << 20));
+    if (n <= 64 && mid_wins) {
+        const int tiles = n > 32 ? 4 : n > 16 ? 2 : 1;
+        tuna_gemm_config c = row;
+        c.lds_tile_rows = 0;
+        if (row.lds_tile_rows <= 0 && row.rows_per_wave == 64 && row.token_tiles == tiles && row.split_k == 1 && row.waves_m >= 1 &&
+            row.waves_m * row.waves_k >= 8 && (row.prefetch == 2 || row.prefetch == 4) && run_blockwise(b, c, nullptr, true) == TUNA_OK) {
+            *out = c;
+            return TUNA_OK;
+        }
+    }
+    if (n > 32) {
+        tuna_gemm_config c = row;
+        if (c.lds_tile_rows <= 0 || !tiled_variant_exists(c.lds_tile_rows, 16 * c.token_tiles, false) ||
+            (c.lds_tile_rows == 256 && c.token_tiles == 16)) {
+            c.lds_tile_rows = n > 64 ? 128 : 256;
+            c.token_tiles = n > 128 ? 16 : n > 64 ? 8 : 4;
+            c.waves_m = c.waves_k = 1, c.prefetch = 2, c.x_chunk = 64, c.xcd_swizzle = 0, c.k_stagger = 0;
+            // fewer tiles than compute units: split k until the launch fills them (at least eight k-steps per workgroup)
+            const long long tiles = (long long)ceil_div(m, c.lds_tile_rows) * ceil_div(n, 16 * c.token_tiles);
+            const int steps = ceil_div(k, 64);
+            long long split = tiles > 0 ? cus / tiles : 1;
+            if (split > steps / 8) split = steps / 8;
+            c.split_k = split < 1 ? 1 : (int)split;
+        }
+        c.rows_per_wave = 64;
+        if (run_blockwise(b, c, nullptr, true) == TUNA_OK) {
+            *out = c;
+            return TUNA_OK;
+        }
+    }
+    const bool stream_wins = n > 16  ? packed_bytes >= (100ll << 20) || (k > 8192 && packed_bytes >= (12ll << 20)) ||
+                                           (k > 4096 && packed_bytes >= (40ll << 20))
+                             : n > 4 ? packed_bytes >= (100ll << 20) || (n > 8 && k >= 12288 && packed_bytes >= (20ll << 20))
+                                     : packed_bytes >= (256ll << 20);
+    if (stream_wins) {
+        // the batched kernel's own choice of tile height (256 rows, 128 where those are fewer than workgroups), ring of
+        // two; then whatever height the row count allows
+        tuna_gemm_problem one = {b.q ? b.q : b.out, b.x, b.code, nullptr, b.out, m, n < 16 ? n : 16, k};
+        MultiPlan plan;
+        tuna_gemm_config c;
+        memset(&c, 0, sizeof(c));
+        c.rows_per_wave = 64, c.split_k = 0, c.x_chunk = 512, c.token_tiles = 1;
+        if (plan_multi(&one, 1, cus, &plan, 0, 0, shift)) {
+            c.waves_m = plan.args.waves_m, c.waves_k = 16 / c.waves_m, c.prefetch = plan.prefetch - 10;
+            if (run_blockwise(b, c, nullptr, true) == TUNA_OK) {
+                *out = c;
+                return TUNA_OK;
+            }
+        }
+        for (int wm = 4; wm >= 1; wm >>= 1) {
+            c.waves_m = wm, c.waves_k = 16 / wm, c.prefetch = 2;
+            if (run_blockwise(b, c, nullptr, true) == TUNA_OK) {
+                *out = c;
+                return TUNA_OK;
+            }
+        }
+    }
+    tuna_gemm_config c;
+    memset(&c, 0, sizeof(c));
+    int rows = 0, wk = 0, u = 0, tt = 0;
+    if (!derive_blockwise_narrow(m, k, shift, cus, n > 16 ? 2 : 1, &rows, &wk, &u, &tt))
+        return fail(TUNA_ERR_UNSUPPORTED, "no scale-block kernel takes m=%d n=%d k=%d block_size=%d", m, n, k, b.block_size);
+    c.rows_per_wave = rows, c.waves_m = rows == 64 ? 0 : 1, c.waves_k = wk, c.split_k = 1, c.prefetch = u, c.x_chunk = 512, c.token_tiles = tt;
+    *out = c;
+    return TUNA_OK;
+}
+
+// Tuned entry for (m, n, k, block_size) if the table has one that can run the call, else the derived config.
+static int select_blockwise(const BlockwiseCall &b, tuna_gemm_config *cfg, int *from_table)
+{
+    if (from_table) *from_table = 0;
+    for (int i = 0; i < kBlockwiseTableSize; ++i) {
+        const BlockwiseTableEntry &e = kBlockwiseTable[i];
+        if (e.m == b.m && e.k == b.k && e.block_size == b.block_size && b.n >= e.n_lo && b.n <= e.n_hi &&
+            run_blockwise(b, e.cfg, nullptr, true) == TUNA_OK) {
+            *cfg = e.cfg;
+            if (from_table) *from_table = 1;
+            return TUNA_OK;
+        }
+    }
+    return derive_blockwise(b, cfg);
+}
+
+static int check_blockwise_call(const BlockwiseCall &b, bool pointers)
+{
+    int rc;
+    if ((rc = check_shape(b.m, b.n, b.k))) return rc;
+    if (b.block_size < 64 || !is_pow2(b.block_size) || b.k % b.block_size || b.block_size >= b.k)
+        return fail(TUNA_ERR_UNSUPPORTED, "block_size=%d: the GEMM takes 64, 128, 256, ... (a power of two that divides k=%d) or k",
+                    b.block_size, b.k);
+    if (b.m % 16 || b.k % 256)
+        return fail(TUNA_ERR_UNSUPPORTED, "scale blocks need m a multiple of 16 and k of 256 (m=%d, k=%d)", b.m, b.k);
+    if ((unsigned long long)b.m * (unsigned long long)b.k / 2 >= (1ull << 32) || (unsigned long long)b.k * 32 >= (1ull << 32))
+        return fail(TUNA_ERR_UNSUPPORTED, "operands exceed the kernel's 32-bit offsets");
+    if ((b.n + 15) / 16 > 65535) return fail(TUNA_ERR_UNSUPPORTED, "n=%d needs more than 65535 token chunks", b.n);
+    if (pointers && ((rc = check_ptr(b.q, "q", 16)) || (rc = check_ptr(b.x, "x", 16)) || (rc = check_ptr(b.code, "code", 4)) ||
+                     (rc = check_ptr(b.absmax, "absmax", 4)) || (rc = check_ptr(b.out, "out", 16))))
+        return rc;
+    return TUNA_OK;
+}
+
+TUNA_EXPORT int tuna_matmul_blockwise_ex(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n,
+                                         int k, int block_size, const tuna_gemm_config *cfg, void *stream)
+{
+    if (block_size == k) return matmul_impl(q, x, code, absmax, out, m, n, k, cfg, TUNA_DECODE_GEMM, static_cast<hipStream_t>(stream));
+    const BlockwiseCall b = {q, x, code, absmax, out, m, n, k, block_size};
+    int rc;
+    if ((rc = check_blockwise_call(b, true))) return rc;
+    tuna_gemm_config c;
+    if (cfg) c = *cfg;
+    else if ((rc = select_blockwise(b, &c, nullptr))) return rc;
+    return run_blockwise(b, c, static_cast<hipStream_t>(stream), false);
 }
 
 TUNA_EXPORT int tuna_matmul_blockwise(const void *q, const void *x, const void *code, const void *absmax, void *out, int m, int n,
                                       int k, int block_size, void *stream)
 {
-    if (block_size == k) return matmul_impl(q, x, code, absmax, out, m, n, k, nullptr, TUNA_DECODE_GEMM, static_cast<hipStream_t>(stream));
+    return tuna_matmul_blockwise_ex(q, x, code, absmax, out, m, n, k, block_size, nullptr, stream);
+}
+
+TUNA_EXPORT int tuna_select_config_blockwise(int m, int n, int k, int block_size, tuna_gemm_config *cfg, int *from_table)
+{
+    if (!cfg) return fail(TUNA_ERR_INVALID_ARG, "cfg is null");
+    const BlockwiseCall b = {nullptr, nullptr, nullptr, nullptr, nullptr, m, n, k, block_size};
     int rc;
-    if ((rc = check_shape(m, n, k))) return rc;
-    if (block_size < 64 || !is_pow2(block_size) || k % block_size)
-        return fail(TUNA_ERR_UNSUPPORTED, "block_size=%d: the GEMM takes 64, 128, 256, ... (a power of two that divides k=%d) or k",
-                    block_size, k);
-    if (m % 16 || k % 256)
-        return fail(TUNA_ERR_UNSUPPORTED, "scale blocks need m a multiple of 16 and k of 256 (m=%d, k=%d)", m, k);
-    if ((unsigned long long)m * (unsigned long long)k / 2 >= (1ull << 32) || (unsigned long long)k * 32 >= (1ull << 32))
-        return fail(TUNA_ERR_UNSUPPORTED, "operands exceed the kernel's 32-bit offsets");
-    if ((n + 15) / 16 > 65535) return fail(TUNA_ERR_UNSUPPORTED, "n=%d needs more than 65535 token chunks", n);
-    if ((rc = check_ptr(q, "q", 16)) || (rc = check_ptr(x, "x", 16)) || (rc = check_ptr(code, "code", 4)) ||
-        (rc = check_ptr(absmax, "absmax", 4)) || (rc = check_ptr(out, "out", 16)))
-        return rc;
-    const int stream_mode = diag::blockwise_stream();
-    // Up to 64 tokens, shapes whose per-row table entry is an unsplit launch of the streaming kernel (the large ones):
-    // that kernel's scale-block twin with the entry's workgroup shape, ring, x chunk and stagger (in whole x chunks; register ring).
-    if (n <= 64 && (stream_mode == 3 || (stream_mode == 1 && mid_blockwise_wins(m, n, k)))) {
-        tuna_gemm_config c;
-        select_config(m, n, k, &c, nullptr);
-        const int tiles = n > 32 ? 4 : n > 16 ? 2 : 1;  // token tiles: one pass over the weights
-        const bool entry_fits = c.lds_tile_rows <= 0 && c.rows_per_wave == 64 && c.token_tiles == tiles && c.split_k == 1 &&
-                                c.waves_m * c.waves_k >= 8 && (c.prefetch == 2 || c.prefetch == 4);
-        // (the library's own routing takes the twin with such an entry only: up to 9 tokens the entries of these shapes
-        // are narrow-row ones, and there the narrow-row scale-block kernel is the faster one - 19.6 against 27.3 us on
-        // 28672 x 4096, 54.6 against 80 on 32768 x 14336 at one token)
-        for (int attempt = entry_fits ? 0 : 1; attempt < (stream_mode == 3 ? 2 : 1); ++attempt) {
-            if (attempt == 1) {  // the switch, without such an entry (or one that does not fit the scale buffers): four waves by four
-                c.rows_per_wave = 64;
-                c.waves_m = m % 256 == 0 ? 4 : m % 128 == 0 ? 2 : 1;
-                c.waves_k = (tiles == 4 ? 8 : 16) / c.waves_m > 8 ? 8 : (tiles == 4 ? 8 : 16) / c.waves_m;  // (four token tiles: 512 threads)
-                c.split_k = 1;
-                c.prefetch = 2;
-                c.x_chunk = tiles == 4 ? 256 : 512;
-                c.token_tiles = tiles;
-                c.xcd_swizzle = 0;
-            }
-            c.lds_tile_rows = 0;
-            if (attempt == 1) c.k_stagger = 0;
-            GemmPlan plan;
-            const int shift = log2i(block_size) - 6;
-            if (m % (64 * c.waves_m) != 0 || plan_gemm(m, n, k, c, TUNA_DECODE_GEMM, &plan) != TUNA_OK ||
-                !mid_blockwise_applies(plan, shift))
-                continue;
-            int dev = 0, cus = 0;
-            hipError_t e = device_cus(&dev, &cus);
-            if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
-            plan.args.q = static_cast<const uint8_t *>(q);
-            plan.args.x = x;
-            plan.args.code = static_cast<const float *>(code);
-            plan.args.absmax = static_cast<const float *>(absmax);
-            plan.args.out = out;
-            plan.args.epilogue = TUNA_EPILOGUE_NONE;
-            plan.args.residual = nullptr;
-            e = launch_gemm_mid_blockwise(plan, shift, dev, cus, static_cast<hipStream_t>(stream));
-            if (e != hipSuccess) return hip_fail(e, "streaming blockwise gemm launch");
-            diag::count(diag::kBlockwiseMid);
-            return TUNA_OK;
-        }
-    }
-    // From 33 tokens: the many-token kernel's scale-block variants (the weights are decoded once per workgroup tile,
-    // with the scale of the k-step's block) - the tile the per-row table has for the shape and token count if that is a
-    // many-token entry, else 256 rows x 64 tokens up to 64 tokens, 128 x 128 up to 128 and 128 x 256 beyond.
-    if (n > 32 && stream_mode == 1) {
-        tuna_gemm_config c;
-        select_config(m, n, k, &c, nullptr);
-        // (the 256 x 256 tile has no scale-block variant: its threads have no registers left for eight more scales)
-        if (c.lds_tile_rows <= 0 || !tiled_variant_exists(c.lds_tile_rows, 16 * c.token_tiles, false) ||
-            (c.lds_tile_rows == 256 && c.token_tiles == 16)) {
-            c.lds_tile_rows = n > 64 ? 128 : 256;
-            c.token_tiles = n > 128 ? 16 : n > 64 ? 8 : 4;
-            // fewer tiles than compute units: split k until the launch fills them (at least eight k-steps per workgroup)
-            int dev_ = 0, cus_ = kMaxCus;
-            (void)device_cus(&dev_, &cus_);
-            const long long tiles = (long long)ceil_div(m, c.lds_tile_rows) * ceil_div(n, 16 * c.token_tiles);
-            const int steps = ceil_div(k, 64);
-            long long split = tiles > 0 ? cus_ / tiles : 1;
-            if (split > steps / 8) split = steps / 8;
-            c.split_k = split < 1 ? 1 : (int)split;
-        }
-        c.rows_per_wave = 64;  // (16 x 16 x 32 MFMA tiles: the scale-block variants exist for those)
-        TiledPlan tp;
-        if (plan_tiled(m, n, k, c, TUNA_DECODE_GEMM, &tp) == TUNA_OK) {
-            hipStream_t st = static_cast<hipStream_t>(stream);
-            tp.args.q = static_cast<const uint8_t *>(q);
-            tp.args.x = x;
-            tp.args.code = static_cast<const float *>(code);
-            tp.args.absmax = static_cast<const float *>(absmax);
-            tp.args.out = out;
-            tp.args.epilogue = TUNA_EPILOGUE_NONE;
-            tp.args.residual = nullptr;
-            tp.args.blk_shift = log2i(block_size) - 6;
-            if (tp.ws_bytes && (rc = provide_workspace(false, st, tp.ws_bytes, tp.n_counters, &tp.args.ws, &tp.args.counters))) return rc;
-            hipError_t e = launch_gemm_tiled(tp.args, tp.tile_rows, tp.tile_tokens, false, st, true);
-            if (e != hipSuccess) return hip_fail(e, "many-token blockwise gemm launch");
-            diag::count(diag::kBlockwiseTiled);
-            return TUNA_OK;
-        }
-    }
-    // Large aligned shapes: the batched streaming kernel's scale-block variant, a batch of one for up to 16 tokens
-    // (balanced split over one workgroup per compute unit), the token chunks of 16 as the problems of a batch beyond
-    // that (every chunk streams the weights again, in one launch per 32 chunks).  Everything else: the narrow-row
-    // kernel's variants, whose single pass with the workgroup's scales in LDS is faster below these sizes.  Measured
-    // at 16 tokens, narrow against streaming: 8.7 / 15.5 us on 6144 x 4096, 14.1 / 16.3 on 8192 x 8192, 19.4 / 20.9 on
-    // 10240 x 8192, 22.4 / 24.2 on 28672 x 4096, but 18.5 / 16.5 on 4096 x 14336, 44 / 35 on 8192 x 28672 and 75 / 66 on
-    // 57344 x 8192; at one token the narrow kernel wins up to 57344 x 8192 (63 / 65) and loses on 229376 x 4096
-    // (117 / 102); at 32 tokens, with two token tiles per workgroup, 11.9 / 16.9 on 6144 x 4096, 20.3 / 24.6 on
-    // 8192 x 8192, 30.9 / 38.7 on 28672 x 4096, 21.4 / 28.3 on 13824 x 5120, but 37.2 / 30.4 on 10240 x 8192, 29.6 / 22.7
-    // on 4096 x 14336, 22.1 / 18.3 on 2560 x 10240, 134 / 106 on 32768 x 14336 and 131 / 108 on 57344 x 8192.
-    const long long packed_bytes = (long long)m * k / 2;
-    const bool stream_wins = n > 16  ? packed_bytes >= (100ll << 20) || (k > 8192 && packed_bytes >= (12ll << 20)) ||
-                                           (k > 4096 && packed_bytes >= (40ll << 20))
-                             : n > 4 ? packed_bytes >= (100ll << 20) || (n > 8 && k >= 12288 && packed_bytes >= (20ll << 20))
-                                     : packed_bytes >= (256ll << 20);
-    if (stream_mode == 2 || (stream_mode == 1 && stream_wins)) {
-        int dev = 0, cus = 0;
-        hipError_t e = device_cus(&dev, &cus);
-        if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
-        hipStream_t st = static_cast<hipStream_t>(stream);
-        const int shift = log2i(block_size) - 6;
-        const int chunks = (n + 15) / 16;
-        // batch `c0 / 32` of the token chunks as a list of problems, planned for this device
-        auto plan_batch = [&](int c0, MultiPlan *plan) {
-            const int cnt = chunks - c0 < kMaxMultiProblems ? chunks - c0 : kMaxMultiProblems;
-            tuna_gemm_problem probs[kMaxMultiProblems];
-            for (int c = 0; c < cnt; ++c) {
-                const int t0 = (c0 + c) * 16;
-                probs[c] = {q, static_cast<const char *>(x) + (size_t)t0 * k * 2, code, absmax,
-                            static_cast<char *>(out) + (size_t)t0 * m * 2, m, n - t0 < 16 ? n - t0 : 16, k};
-            }
-            // the batched kernel's own choice of tile height (256 rows, 128 where those are fewer than workgroups), ring of
-            // two; then whatever height the row count allows
-            bool ok = plan_multi(probs, cnt, cus, plan, 0, 0, shift);
-            for (int wm = 4; wm >= 1 && !ok; wm >>= 1) ok = plan_multi(probs, cnt, cus, plan, wm, 2, shift);
-            return ok;
-        };
-        bool planned_all = true;  // (nothing is enqueued unless every batch of chunks can run here)
-        for (int c0 = 0; c0 < chunks && planned_all; c0 += kMaxMultiProblems) {
-            MultiPlan plan;
-            planned_all = plan_batch(c0, &plan);
-        }
-        if (planned_all) {
-            for (int c0 = 0; c0 < chunks; c0 += kMaxMultiProblems) {
-                MultiPlan plan;
-                if (!plan_batch(c0, &plan)) return fail(TUNA_ERR_UNSUPPORTED, "blockwise gemm: a batch of token chunks stopped planning");
-                if ((rc = provide_workspace(false, st, plan.ws_bytes, plan.n_counters, &plan.args.ws, &plan.args.counters))) return rc;
-                e = launch_gemm_multi(plan.args, plan.prefetch, dev, st);
-                if (e != hipSuccess) return hip_fail(e, "blockwise gemm launch");
-                diag::count(diag::kMultiLaunches);
-                diag::count(diag::kBlockwiseMulti);
-            }
-            return TUNA_OK;
-        }
-    }
-    diag::count(diag::kBlockwiseNarrow);
-    NarrowArgs a;
-    memset(&a, 0, sizeof(a));
-    a.q = static_cast<const uint8_t *>(q);
-    a.x = x;
-    a.code = static_cast<const float *>(code);
-    a.absmax = static_cast<const float *>(absmax);
-    a.out = out;
-    a.m = m, a.n = n, a.k = k;
-    hipError_t e = launch_gemm_blockwise(a, log2i(block_size) - 6, static_cast<hipStream_t>(stream));
-    if (e != hipSuccess) return hip_fail(e, "blockwise gemm launch");
+    if ((rc = check_blockwise_call(b, false))) return rc;
+    return select_blockwise(b, cfg, from_table);
+}
+
+TUNA_EXPORT int tuna_validate_config_blockwise(int m, int n, int k, int block_size, const tuna_gemm_config *cfg)
+{
+    if (!cfg) return fail(TUNA_ERR_INVALID_ARG, "cfg is null");
+    const BlockwiseCall b = {nullptr, nullptr, nullptr, nullptr, nullptr, m, n, k, block_size};
+    int rc;
+    if ((rc = check_blockwise_call(b, false))) return rc;
+    return run_blockwise(b, *cfg, nullptr, true);
+}
+
+TUNA_EXPORT int tuna_blockwise_table_size(void) { return kBlockwiseTableSize; }
+
+TUNA_EXPORT int tuna_blockwise_table_entry(int i, int *m, int *n_lo, int *n_hi, int *k, int *block_size, tuna_gemm_config *cfg)
+{
+    if (i < 0 || i >= kBlockwiseTableSize) return fail(TUNA_ERR_INVALID_ARG, "table index %d out of range", i);
+    const BlockwiseTableEntry &e = kBlockwiseTable[i];
+    if (m) *m = e.m;
+    if (n_lo) *n_lo = e.n_lo;
+    if (n_hi) *n_hi = e.n_hi;
+    if (k) *k = e.k;
+    if (block_size) *block_size = e.block_size;
+    if (cfg) *cfg = e.cfg;
     return TUNA_OK;
 }
 

@@ -245,6 +245,18 @@ TUNA_EXPORT int tuna_measure_handover(int same_xcd, int store_sc1, int load_sc1,
     return e == hipSuccess ? (int)TUNA_OK : hip_fail(e, "hand-over yardstick");
 }
 
+TUNA_EXPORT int tuna_time_matmul_blockwise(const void *const *q_list, const void *const *absmax_list, int n_sets, const void *x,
+                                           const void *code, void *out, int m, int n, int k, int block_size,
+                                           const tuna_gemm_config *cfg, int warmup, int iters, int use_graph, void *stream,
+                                           float *elapsed_ms)
+{
+    if (!q_list || !absmax_list) return fail(TUNA_ERR_INVALID_ARG, "q_list / absmax_list is null");
+    auto launch = [&](int set, hipStream_t s) {
+        return tuna_matmul_blockwise_ex(q_list[set], x, code, absmax_list[set], out, m, n, k, block_size, cfg, s);
+    };
+    return time_loop(launch, n_sets, warmup, iters, use_graph, static_cast<hipStream_t>(stream), elapsed_ms);
+}
+
 TUNA_EXPORT int tuna_time_matmul_multi(const tuna_gemm_problem *problems, int n_sets, int count, int warmup, int iters,
                                        int use_graph, void *stream, float *elapsed_ms)
 {

@@ -17,9 +17,7 @@ int multi_waves_m();         // batched kernel: waves along the rows (0: the lib
 int multi_prefetch();        // batched kernel: ring depth (0: the library's choice)
 int multi_lds();             // 1: batches with a ring of two stage weights and x through LDS
 int multi_min_batch();       // batches shorter than this are launched problem by problem (2)
-int blockwise_stream();      // kernel family of tuna_matmul_blockwise (1: the library's rules)
 int blockwise_scales_lds();  // 1: the narrow-row blockwise kernel keeps a workgroup's scales in LDS
-int blockwise_shape(int i);  // forced variant of the narrow-row blockwise kernel: rows, waves along k, ring (0: none)
 
 enum Counter { kLeanLaunches, kMultiLaunches, kBlockwiseNarrow, kBlockwiseMulti, kBlockwiseTiled, kBlockwiseMid, kNumCounters };
 void count(Counter c);

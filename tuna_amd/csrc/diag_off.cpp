@@ -10,9 +10,7 @@ int multi_waves_m() { return 0; }
 int multi_prefetch() { return 0; }
 int multi_lds() { return 0; }
 int multi_min_batch() { return 2; }
-int blockwise_stream() { return 1; }
 int blockwise_scales_lds() { return 1; }
-int blockwise_shape(int) { return 0; }
 void count(Counter) {}
 
 }  // namespace diag

@@ -304,12 +304,12 @@ static const BlockwiseVariant kBlockwise[] = {
 #undef B2
 static constexpr int kNumBlockwise = sizeof(kBlockwise) / sizeof(kBlockwise[0]);
 
-bool blockwise_variant_exists(int rows, int waves_k, int prefetch)
+static const BlockwiseVariant *find_blockwise(int rows, int waves_k, int prefetch, int tt)
 {
-    bool found = false;
     for (int i = 0; i < kNumBlockwise; ++i)
-        found |= kBlockwise[i].tt == 1 && kBlockwise[i].rows == rows && kBlockwise[i].wk == waves_k && kBlockwise[i].u == prefetch;
-    return found;
+        if (kBlockwise[i].tt == tt && kBlockwise[i].rows == rows && kBlockwise[i].wk == waves_k && kBlockwise[i].u == prefetch)
+            return &kBlockwise[i];
+    return nullptr;
 }
 
 static bool blockwise_fits(const BlockwiseVariant &v, int m, int k) { return m % v.rows == 0 && k % (kStepK * v.wk * v.u) == 0; }
@@ -323,16 +323,6 @@ static size_t blockwise_scale_bytes(const BlockwiseVariant &v, int nblk) { retur
 // 144 to 256 wide workgroups beats two rounds of narrower ones, and scales read from memory cost 1.4 to 2x).
 static const BlockwiseVariant *choose_blockwise(int m, int k, int nblk, int cus, int tt)
 {
-    const int ov_rows = diag::blockwise_shape(0);
-    if (ov_rows) {
-        const int wk = diag::blockwise_shape(1), u = diag::blockwise_shape(2);
-        for (int t = tt; t >= 1; --t)  // (the two-tile twin of the named shape where one is built)
-            for (int i = 0; i < kNumBlockwise; ++i)
-                if (kBlockwise[i].tt == t && kBlockwise[i].rows == ov_rows && kBlockwise[i].wk == wk && kBlockwise[i].u == u &&
-                    blockwise_fits(kBlockwise[i], m, k))
-                    return &kBlockwise[i];
-        return nullptr;
-    }
     static const int pref[][3] = {{64, 8, 4}, {64, 8, 2}, {32, 8, 4}, {32, 8, 2}, {16, 8, 4}, {16, 4, 2}};
     for (int need_lds = 1; need_lds >= 0; --need_lds) {
         const BlockwiseVariant *fallback = nullptr;
@@ -350,15 +340,31 @@ static const BlockwiseVariant *choose_blockwise(int m, int k, int nblk, int cus,
     return tt > 1 ? choose_blockwise(m, k, nblk, cus, 1) : nullptr;  // (shapes only the 16-row, 4-wave tile of one token tile fits)
 }
 
-hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, hipStream_t stream)
+// The narrow-row scale-block variant the library derives for a shape (token_tiles 1 or 2: what one pass should cover).
+bool derive_blockwise_narrow(int m, int k, int blk_shift, int cus, int token_tiles, int *rows, int *waves_k, int *prefetch, int *tt)
+{
+    const BlockwiseVariant *v = choose_blockwise(m, k, k >> (6 + blk_shift), cus, token_tiles);
+    if (!v) return false;
+    *rows = v->rows, *waves_k = v->wk, *prefetch = v->u, *tt = v->tt;
+    return true;
+}
+
+// Whether the variant (rows per workgroup, waves along k, ring, token tiles) is built and fits the shape.
+bool blockwise_narrow_runs(int m, int k, int rows, int waves_k, int prefetch, int tt)
+{
+    const BlockwiseVariant *v = find_blockwise(rows, waves_k, prefetch, tt);
+    return v && blockwise_fits(*v, m, k);
+}
+
+hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, int rows, int waves_k, int prefetch, int tt, hipStream_t stream)
 {
     int dev = 0, cus = 0;
     hipError_t e = device_cus(&dev, &cus);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
     const int nblk = args.k >> (6 + blk_shift);
-    const BlockwiseVariant *v = choose_blockwise(args.m, args.k, nblk, cus, args.n > 16 ? 2 : 1);
-    if (!v) return hipErrorInvalidConfiguration;
+    const BlockwiseVariant *v = find_blockwise(rows, waves_k, prefetch, tt);
+    if (!v || !blockwise_fits(*v, args.m, args.k)) return hipErrorInvalidConfiguration;
     const int vi = (int)(v - kBlockwise);
     const int perm = args.n > 4;
     const NarrowKernelFn fn = perm ? v->fn_perm : v->fn;

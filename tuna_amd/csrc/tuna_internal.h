@@ -191,8 +191,11 @@ struct NarrowArgs {
 };
 bool narrow_variant_exists(int rows, int waves_k, int prefetch, int token_tiles);
 hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int prefetch, int token_tiles, hipStream_t stream);
-hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, hipStream_t stream);
-bool blockwise_variant_exists(int rows, int waves_k, int prefetch);  // a one-token-tile variant of the narrow-row blockwise kernel
+// the narrow-row kernel's scale-block variants (a scale per 64 << blk_shift weights of a row)
+hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, int rows, int waves_k, int prefetch, int token_tiles,
+                                 hipStream_t stream);
+bool derive_blockwise_narrow(int m, int k, int blk_shift, int cus, int token_tiles, int *rows, int *waves_k, int *prefetch, int *tt);
+bool blockwise_narrow_runs(int m, int k, int rows, int waves_k, int prefetch, int token_tiles);
 bool launch_is_lean(const GemmPlan &plan, int cus);  // the planned launch would take the lean kernel
 bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves, int grouped);
 
@@ -233,5 +236,12 @@ struct TableEntry {
 };
 extern const TableEntry kConfigTable[];
 extern const int kConfigTableSize;
+// tuned entries of the GEMM with scale blocks finer than a row: (m, token bucket, k, block_size) -> config
+struct BlockwiseTableEntry {
+    int m, n_lo, n_hi, k, block_size;
+    tuna_gemm_config cfg;
+};
+extern const BlockwiseTableEntry kBlockwiseTable[];
+extern const int kBlockwiseTableSize;
 
 }  // namespace tuna

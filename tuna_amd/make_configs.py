@@ -240,6 +240,88 @@ def lds_bytes(c: dict) -> int:
     return big if big <= LDS_LIMIT and (big == small or not two_wgs) else small
 
 
+# ---- the GEMM with scale blocks finer than a row: entries keyed "<m>_<n>_<k>_<block_size>" -------------------------
+# Narrow-row scale-block variants (rows per workgroup, waves along k, ring, token tiles); must match kBlockwise in
+# csrc/gemm_launch.hip
+BLOCKWISE_NARROW = ({(16, 4, 2, 1), (16, 8, 4, 1), (16, 16, 2, 1), (32, 8, 2, 1), (32, 8, 4, 1), (32, 16, 2, 1), (64, 4, 4, 1),
+                     (64, 8, 2, 1), (64, 8, 4, 1), (64, 16, 2, 1)}
+                    | {(16, 4, 2, 2), (16, 8, 4, 2), (32, 8, 2, 2), (32, 8, 4, 2), (64, 8, 2, 2), (64, 8, 4, 2)})
+# many-token tiles with a scale-block variant (16 x 16 x 32 MFMA; not the 256 x 256 tile)
+BLOCKWISE_TILED = {(64, 128), (64, 256), (128, 64), (128, 128), (128, 256), (256, 64), (256, 128)}
+BLOCKWISE_FAMILIES = ("narrow", "batched", "many-token", "streaming")
+
+
+def blockwise_family(c: dict) -> str:
+    """Which kernel a blockwise config names (mirrors blockwise_family in csrc/api.cpp)."""
+    if c.get("lds_tile_rows", 0) > 0:
+        return "many-token"
+    if is_narrow(c):
+        return "narrow"
+    if c["split_k"] == 0:
+        return "batched"
+    return "streaming"
+
+
+def validate_blockwise(m: int, n: int, k: int, bs: int, c: dict) -> None:
+    """Raise ValueError unless `c` is a runnable blockwise config for (m, n in bucket n, k, block size bs): the
+    structural checks of run_blockwise in csrc/api.cpp (the library's own validator, tuna_validate_config_blockwise,
+    is the full check and is run over the generated table by the tests)."""
+    if n not in N_BUCKETS:
+        raise ValueError(f"n={n} is not a token bucket key")
+    if bs < 64 or bs & (bs - 1) or k % bs or bs >= k or m % 16 or k % 256:
+        raise ValueError(f"block_size={bs}: a power of two >= 64 that divides k={k} (k a multiple of 256, m={m} of 16)")
+    fam = blockwise_family(c)
+    lo, _ = N_BUCKETS[n]
+    if fam == "narrow":
+        key = (c["rows_per_wave"], c["waves_k"], c["prefetch"], c["token_tiles"])
+        if key not in BLOCKWISE_NARROW:
+            raise ValueError(f"no narrow-row scale-block variant {key}")
+        if m % c["rows_per_wave"] or k % (STEP_K * c["waves_k"] * c["prefetch"]):
+            raise ValueError("narrow-row variant does not divide the shape")
+    elif fam == "batched":
+        if c["waves_m"] not in (1, 2, 4) or c["waves_m"] * c["waves_k"] != 16 or c["prefetch"] not in (2, 4):
+            raise ValueError("batched kernel: 1, 2 or 4 waves along the rows of 16, ring 2 or 4")
+        if m % (64 * c["waves_m"]) or k % (STEP_K * c["waves_k"] * c["prefetch"]) or k // bs < 2:
+            raise ValueError("batched kernel: row tile or ring turn does not divide the shape")
+    elif fam == "many-token":
+        if (c["lds_tile_rows"], 16 * c["token_tiles"]) not in BLOCKWISE_TILED or c["split_k"] < 1:
+            raise ValueError("no many-token scale-block variant with that tile")
+    else:
+        tiles = 4 if lo > 32 else 2 if lo > 16 else 1
+        if lo > 64 or c["token_tiles"] != tiles or c["split_k"] != 1 or c["rows_per_wave"] != 64 or c["waves_m"] < 1:
+            raise ValueError("streaming twin: up to 64 tokens in one pass, unsplit, 64 rows per wave")
+        if m % (64 * c["waves_m"]) or c["prefetch"] not in (2, 4) or c["waves_m"] * c["waves_k"] not in (8, 16):
+            raise ValueError("streaming twin: 8 or 16 waves, ring 2 or 4, whole row tiles")
+
+
+def generate_blockwise(param_map: dict) -> str:
+    rows = []
+    for key in sorted(param_map, key=lambda s: tuple(int(t) for t in s.split("_"))):
+        m, n, k, bs = (int(t) for t in key.split("_"))
+        c = param_map[key]
+        try:
+            validate_blockwise(m, n, k, bs, c)
+        except ValueError as e:
+            raise ValueError(f"blockwise param_map entry {key}: {e}") from None
+        lo, hi = N_BUCKETS[n]
+        vals = ", ".join(str(int(c.get(f, 0))) for f in FIELDS)
+        rows.append(f"    {{{m}, {lo}, {hi}, {k}, {bs}, {{{vals}}}}},  // {key}: {blockwise_family(c)}")
+    body = "\n".join(rows)
+    return f"""
+// Scale blocks finer than a row: (m, token bucket, k, block_size) -> config, searched by tuna_select_config_blockwise.
+// Generated from tuna_amd/configs/param_map_blockwise.json.  Entry: m, n_lo, n_hi, k, block_size, {{config}}
+namespace tuna {{
+
+const BlockwiseTableEntry kBlockwiseTable[] = {{
+{body}
+    {{0, 0, 0, 0, 0, {{0, 0, 0, 0, 0, 0, 0, 0, 0, 0}}}},  // sentinel (not counted)
+}};
+const int kBlockwiseTableSize = {len(rows)};
+
+}}  // namespace tuna
+"""
+
+
 def generate(param_map: dict) -> str:
     rows = []
     for key in sorted(param_map, key=lambda s: tuple(int(t) for t in s.split("_"))):
@@ -276,9 +358,16 @@ def main(argv):
     with open(src) as f:
         param_map = json.load(f)
     text = generate(param_map)
+    # the blockwise table sits beside the per-row one: <stem>_blockwise.json (absent: an empty table)
+    src_blk = os.path.splitext(src)[0] + "_blockwise.json"
+    blockwise = {}
+    if os.path.exists(src_blk):
+        with open(src_blk) as f:
+            blockwise = json.load(f)
+    text += generate_blockwise(blockwise)
     with open(dst, "w") as f:
         f.write(text)
-    print(f"{dst}: {len(param_map)} entries")
+    print(f"{dst}: {len(param_map)} entries, {len(blockwise)} blockwise entries")
 
 
 if __name__ == "__main__":

@@ -220,9 +220,9 @@ def dequant(q, absmax, codebook, o, m: int, k: int, decode_mode: int = _lib.DECO
     _lib.check(rc)
 
 
-def matmul_blockwise(x, q, s, c, o, m: int, n: int, k: int, block_size: int) -> None:
+def matmul_blockwise(x, q, s, c, o, m: int, n: int, k: int, block_size: int, config: GemmConfig = None) -> None:
     """matmul with one scale per block_size consecutive weights of a row: s fp32 [m, k/block_size]
-    (tuna_matmul_blockwise)."""
+    (tuna_matmul_blockwise_ex; config None = the library's choice: its blockwise table, else a derived config)."""
     m, n, k, bs = int(m), int(n), int(k), int(block_size)
     if bs <= 0 or k % bs:
         raise ValueError(f"block_size={bs} must divide k={k}")
@@ -232,9 +232,32 @@ def matmul_blockwise(x, q, s, c, o, m: int, n: int, k: int, block_size: int) -> 
     _require(c, "c", torch.float32, 16)
     _require(o, "o", torch.float16, n * m)
     with torch.cuda.device(x.device):
-        rc = _lib.lib().tuna_matmul_blockwise(q.data_ptr(), x.data_ptr(), c.data_ptr(), s.data_ptr(), o.data_ptr(), m, n, k, bs,
-                                              _stream(x.device))
+        rc = _lib.lib().tuna_matmul_blockwise_ex(q.data_ptr(), x.data_ptr(), c.data_ptr(), s.data_ptr(), o.data_ptr(), m, n, k, bs,
+                                                 ctypes.byref(config) if config is not None else None, _stream(x.device))
     _lib.check(rc)
+
+
+def select_config_blockwise(m: int, n: int, k: int, block_size: int):
+    """(config, from_table) tuna_matmul_blockwise runs for the shape (tuna_select_config_blockwise).  Host only."""
+    cfg = GemmConfig()
+    hit = ctypes.c_int(0)
+    _lib.check(_lib.lib().tuna_select_config_blockwise(int(m), int(n), int(k), int(block_size), ctypes.byref(cfg), ctypes.byref(hit)))
+    return cfg, bool(hit.value)
+
+
+def validate_config_blockwise(m: int, n: int, k: int, block_size: int, config: GemmConfig) -> None:
+    """Raises TunaError unless `config` can run the blockwise GEMM (tuna_validate_config_blockwise).  Host only."""
+    _lib.check(_lib.lib().tuna_validate_config_blockwise(int(m), int(n), int(k), int(block_size), ctypes.byref(config)))
+
+
+BLOCKWISE_FAMILIES = ("narrow", "batched", "many-token", "streaming")
+
+
+def blockwise_family(config: GemmConfig) -> str:
+    """The kernel a blockwise config names (the rule of tuna_matmul_blockwise_ex)."""
+    from .make_configs import blockwise_family as fam
+
+    return fam(config.to_dict())
 
 
 def quantize(w, codebook=None, block_size: int = None):
@@ -400,6 +423,22 @@ def measure_handover(device, same_xcd: bool, store_sc1: bool, load_sc1: bool, re
     _lib.check(rc, L)
     return {"store_ack_ns": round(out[0], 1), "atomic_round_trip_ns": round(out[1], 1), "load_ns": round(out[2], 1),
             "mismatches": int(out[3]), "timeouts": int(out[4]), "pairs_on_one_xcd": int(out[5]), "pairs": int(pairs)}
+
+
+def time_matmul_blockwise(q_list, absmax_list, x, c, o, m, n, k, block_size, config=None, warmup=10, iters=100,
+                          use_graph=False) -> float:
+    """Milliseconds for `iters` blockwise GEMMs rotating over the weight sets (tuna_time_matmul_blockwise)."""
+    assert len(q_list) == len(absmax_list) and len(q_list) > 0
+    qp, _qk = _ptr_array(q_list)
+    ap, _ak = _ptr_array(absmax_list)
+    ms = ctypes.c_float(0)
+    L = _lib.bench_lib()
+    with torch.cuda.device(x.device):
+        rc = L.tuna_time_matmul_blockwise(qp, ap, len(q_list), x.data_ptr(), c.data_ptr(), o.data_ptr(), int(m), int(n), int(k),
+                                          int(block_size), ctypes.byref(config) if config is not None else None, int(warmup),
+                                          int(iters), int(bool(use_graph)), _stream(x.device), ctypes.byref(ms))
+    _lib.check(rc, L)
+    return ms.value
 
 
 def time_matmul_grouped(q_list, absmax_list, x, c, o, m_group, n_groups, k, token_offsets, config=None,
