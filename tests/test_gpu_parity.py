@@ -2223,3 +2223,66 @@ def test_batched_launch_with_epilogues_rejects_bad_arguments_and_falls_back_prob
     torch.cuda.synchronize()
     ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1) + res.astype(np.float64)
     assert rel_err(out.cpu().numpy().astype(np.float64), ref) <= REL_TOL
+
+
+def _blockwise_table_entries():
+    import json
+    import os
+
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "tuna_amd", "configs", "param_map_blockwise.json")
+    with open(path) as f:
+        return sorted(json.load(f), key=lambda s: tuple(int(t) for t in s.split("_")))
+
+
+@pytest.mark.gpu
+@pytest.mark.usefixtures("diagnostic_build")
+@pytest.mark.parametrize("key", _blockwise_table_entries())
+def test_every_blockwise_table_entry_matches_the_oracle(key):
+    """Every tuned entry of the blockwise table at its real size, through the plain entry point (no config: the table
+    lookup is what is tested), at the lower edge of its token bucket and at a ragged count inside it: the kernel the
+    entry names runs, 64 random 8-row blocks match the oracle's float64 sums over the blockwise D1 weights, and one-hot
+    activations read the decoded weights of those rows out exactly (random scales per block)."""
+    import torch
+
+    from tuna_amd import _lib, make_configs, ops
+    from tuna_amd.quantize import nf4_codebook
+    from tuna_amd.synth import make_weights_torch, make_x_torch
+
+    m, n_key, k, bs = (int(t) for t in key.split("_"))
+    L = _lib.lib()
+    dev = torch.device("cuda")
+    q, _ = make_weights_torch(m, k, seed=m + k + bs, device=dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(bs + n_key)
+    absmax = (torch.rand((m, k // bs), dtype=torch.float32, device=dev, generator=gen) * 0.015 + 0.005).to(torch.float16).float()
+    code = nf4_codebook(dev)
+    rng = np.random.default_rng(m + n_key)
+    mbs = np.sort(rng.choice(m // 8, size=min(64, m // 8), replace=False))
+    rows = (mbs[:, None] * 8 + np.arange(8)[None, :]).ravel()
+    q_sub = q[torch.from_numpy(mbs).to(dev)].cpu().numpy()
+    a_sub = absmax.cpu().numpy()[rows]
+    code_np = code.cpu().numpy()
+    lo, hi = make_configs.N_BUCKETS[n_key]
+    for n in sorted({lo, min(hi, lo + max(1, lo // 2) + 1)}):
+        c, hit = ops.select_config_blockwise(m, n, k, bs)
+        fam = ops.blockwise_family(c)
+        print(f"blockwise table entry {key} at n={n}: {fam} {c.to_dict()} from_table={hit}", flush=True)
+        assert hit or n != lo          # (inside the bucket an entry that cannot make its one pass gives way to a derived config)
+        before = L.tuna_blockwise_launches(ops.BLOCKWISE_FAMILIES.index(fam))
+        x = make_x_torch(n, k, seed=n, device=dev)
+        out = torch.full((n, m), float("nan"), dtype=torch.float16, device=dev)
+        ops.matmul_blockwise(x, q, absmax, code, out, m, n, k, bs)
+        torch.cuda.synchronize()
+        assert L.tuna_blockwise_launches(ops.BLOCKWISE_FAMILIES.index(fam)) > before
+        assert not torch.isnan(out).any()
+        ref = O.gemm_f64(q_sub, x.cpu().numpy().view(np.uint16), code_np, a_sub, len(rows), n, k, mode=O.D1, block_size=bs)
+        e = rel_err(f16_bits_to_f64(out.cpu().numpy().view(np.uint16)[:, rows]), ref)
+        assert e <= REL_TOL, e
+        nh = min(n, k)
+        cols = rng.choice(k, size=nh, replace=False)
+        xh = torch.zeros((n, k), dtype=torch.float16, device=dev)
+        xh[torch.arange(nh, device=dev), torch.from_numpy(cols).to(dev)] = 1.0
+        ops.matmul_blockwise(xh, q, absmax, code, out, m, n, k, bs)
+        torch.cuda.synchronize()
+        img_sub = O.dequant(q_sub, a_sub, code_np, len(rows), k, mode=O.D1, block_size=bs)
+        assert np.array_equal(out.cpu().numpy().view(np.uint16)[:nh][:, rows], img_sub[:, cols].T)

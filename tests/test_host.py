@@ -636,3 +636,46 @@ def test_library_chosen_configs_accept_scales_that_are_only_float_aligned():
             assert rc != _lib.ERR_INVALID_ARG, (m_.value, n, k_.value, L.tuna_last_error())
             assert rc in (_lib.ERR_HIP, _lib.ERR_NO_DEVICE, _lib.ERR_WORKSPACE), rc
     assert len(seen) > 40
+
+
+def test_every_blockwise_table_entry_validates_and_derived_configs_are_runnable():
+    """The blockwise table: every entry of param_map_blockwise.json is in the library's table, passes the generator's
+    structural check and the library's own validator at the token count it was tuned at, and is what
+    tuna_select_config_blockwise returns there; shapes without an entry get a derived config that validates too."""
+    from tuna_amd import _lib, make_configs as mc, ops
+
+    with open(os.path.join(ROOT, "tuna_amd", "configs", "param_map_blockwise.json")) as f:
+        pm = json.load(f)
+    L = _lib.lib()
+    assert L.tuna_blockwise_table_size() == len(pm) > 0
+    seen = set()
+    m_, lo_, hi_, k_, bs_ = (ctypes.c_int() for _ in range(5))
+    cfg = _lib.GemmConfig()
+    for i in range(len(pm)):
+        assert L.tuna_blockwise_table_entry(i, ctypes.byref(m_), ctypes.byref(lo_), ctypes.byref(hi_), ctypes.byref(k_), ctypes.byref(bs_),
+                                            ctypes.byref(cfg)) == 0
+        n_key = [key for key, (lo, hi) in mc.N_BUCKETS.items() if lo == lo_.value][0]
+        key = f"{m_.value}_{n_key}_{k_.value}_{bs_.value}"
+        seen.add(key)
+        want = {f: int(pm[key].get(f, 0)) for f in mc.FIELDS}
+        assert cfg.to_dict() == want, key
+        mc.validate_blockwise(m_.value, n_key, k_.value, bs_.value, want)
+        ops.validate_config_blockwise(m_.value, lo_.value, k_.value, bs_.value, cfg)
+        for n in (lo_.value, hi_.value):
+            # (an entry that makes one pass over the weights with the token tiles of the bucket's lower edge cannot
+            # take the bucket's upper edge: the lookup then hands out a derived config, which must run as well)
+            got, hit = ops.select_config_blockwise(m_.value, n, k_.value, bs_.value)
+            ops.validate_config_blockwise(m_.value, n, k_.value, bs_.value, got)
+            assert (hit and got.to_dict() == want) or (not hit and n != lo_.value), (key, n)
+    assert seen == set(pm)
+    for (m, n, k, bs) in [(4096, 16, 4096, 64), (5120, 1, 5120, 128), (3072, 40, 9216, 64), (65536, 16, 4096, 256), (1024, 300, 2048, 64),
+                          (16, 1, 256, 64), (49152, 24, 6144, 64), (12288, 100, 4096, 128), (2048, 2000, 1024, 512)]:
+        got, hit = ops.select_config_blockwise(m, n, k, bs)
+        assert not hit and ops.blockwise_family(got) in ops.BLOCKWISE_FAMILIES
+        ops.validate_config_blockwise(m, n, k, bs, got)
+    # what cannot run is refused with a reason, not launched
+    bad = ops.GemmConfig.from_dict(dict(rows_per_wave=64, waves_m=4, waves_k=4, split_k=1, prefetch=2, x_chunk=512, token_tiles=1, xcd_swizzle=0))
+    with pytest.raises(ops.TunaError):
+        ops.validate_config_blockwise(4096, 100, 4096, 64, bad)          # the streaming twin: up to 64 tokens
+    with pytest.raises(ops.TunaError):
+        ops.validate_config_blockwise(4096, 16, 4096, 96, bad)           # not a power of two

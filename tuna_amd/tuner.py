@@ -347,6 +347,155 @@ def tune_shape(m, n, k, generations=6, population=24, seed=0, log=print, max_see
     return json.loads(final[0][1]), final[0][0]
 
 
+def blockwise_space(m: int, n_key: int, k: int, bs: int, row_entries=()):
+    """Every config of the GEMM with a scale per `bs` weights worth timing for the shape and token bucket: the
+    narrow-row variants, the batched kernel's workgroup shapes, the streaming kernel's scale-block twin (workgroup
+    shapes of the per-row table's entries for the shape, `row_entries`, and the plain 4 x 4 / 2 x 8 / 8 x 2 ones) and,
+    from 32 tokens, the many-token tiles with their k splits.  Small enough to time exhaustively."""
+    lo, _ = make_configs.N_BUCKETS[n_key]
+    out = []
+
+    def add(c):
+        c = dict(c)
+        c.setdefault("k_stagger", 0)
+        c.setdefault("lds_tile_rows", 0)
+        try:
+            make_configs.validate_blockwise(m, n_key, k, bs, c)
+        except ValueError:
+            return
+        out.append(c)
+
+    for rows, wk, u, tt in sorted(make_configs.BLOCKWISE_NARROW):
+        if tt == 2 and lo <= 16:
+            continue
+        add(dict(rows_per_wave=rows, waves_m=0 if rows == 64 else 1, waves_k=wk, split_k=1, prefetch=u, x_chunk=512, token_tiles=tt,
+                 xcd_swizzle=0))
+    for wm in (4, 2, 1):
+        for u in (2, 4):
+            add(dict(rows_per_wave=64, waves_m=wm, waves_k=16 // wm, split_k=0, prefetch=u, x_chunk=512, token_tiles=1, xcd_swizzle=0))
+    if lo <= 64:
+        tiles = 4 if lo > 32 else 2 if lo > 16 else 1
+        shapes = {(4, 4), (2, 8), (8, 2), (4, 2), (2, 4), (8, 1), (16, 1)}
+        shapes |= {(e["waves_m"], e["waves_k"]) for e in row_entries if e.get("rows_per_wave") == 64 and e.get("waves_m", 0) >= 1}
+        for wm, wk in sorted(shapes):
+            if wm * wk not in (8, 16) or (tiles == 4 and wm * wk != 8):
+                continue
+            for u in (2, 4):
+                for xc in (256, 512, 1024):
+                    for stg in (0, 1, 3):
+                        add(dict(rows_per_wave=64, waves_m=wm, waves_k=wk, split_k=1, prefetch=u, x_chunk=xc, token_tiles=tiles,
+                                 xcd_swizzle=1, k_stagger=stg))
+    if lo >= 32:
+        steps = -(-k // 64)
+        for rows, tokens in sorted(make_configs.BLOCKWISE_TILED):
+            if tokens > max(64, 2 * lo):
+                continue
+            tiles_n = -(-m // rows) * -(-lo // tokens)
+            for split in (1, 2, 3, 4, 6, 8, 12, 16):
+                if split > 1 and (steps // split < 4 or tiles_n * split > 4 * N_CU):
+                    continue
+                add(dict(rows_per_wave=64, waves_m=1, waves_k=1, split_k=split, prefetch=2, x_chunk=64, token_tiles=tokens // 16,
+                         xcd_swizzle=0, lds_tile_rows=rows))
+    uniq = {json.dumps(c, sort_keys=True): c for c in out}
+    return list(uniq.values())
+
+
+class BlockwiseEvaluator:
+    """Times blockwise configs for one shape on the GPU over rotating weight sets (tuna_time_matmul_blockwise)."""
+
+    def __init__(self, m, n, k, bs, iters=60, warmup=10):
+        import torch
+
+        from . import ops, synth
+        from .quantize import nf4_codebook
+
+        self.ops = ops
+        self.m, self.n, self.k, self.bs = m, n, k, bs
+        self.iters, self.warmup = iters, warmup
+        dev = torch.device("cuda")
+        n_sets = max(2, min(-(-(512 << 20) // (m * k // 2)), 32))
+        self.qs = [synth.make_weights_torch(m, k, 777 + i, dev)[0] for i in range(n_sets)]
+        self.scales = [torch.rand((m, k // bs), dtype=torch.float32, device=dev) * 0.015 + 0.005 for _ in range(n_sets)]
+        self.x = synth.make_x_torch(n, k, 1, dev)
+        self.code = nf4_codebook(dev)
+        self.out = torch.empty((n, m), dtype=torch.float16, device=dev)
+        self.cache = {}
+
+    def __call__(self, c) -> float:
+        key = "derived" if c is None else json.dumps(c, sort_keys=True)
+        if key not in self.cache:
+            cfg = None if c is None else self.ops.GemmConfig.from_dict(c)
+            try:
+                best = float("inf")
+                for _ in range(2):
+                    ms = self.ops.time_matmul_blockwise(self.qs, self.scales, self.x, self.code, self.out, self.m, self.n, self.k,
+                                                        self.bs, config=cfg, warmup=self.warmup, iters=self.iters, use_graph=True)
+                    best = min(best, ms * 1000.0 / self.iters)
+                self.cache[key] = best
+            except self.ops.TunaError:
+                self.cache[key] = float("inf")
+        return self.cache[key]
+
+
+def tune_blockwise(m, n, k, bs, row_entries=(), iters=60, log=print):
+    """Best blockwise config for the shape, its time, and the time of the config the library derives without a table
+    entry: the whole space is timed, the top five again with more launches."""
+    n_key = make_configs.bucket_of(n)
+    ev = BlockwiseEvaluator(m, n, k, bs, iters=iters, warmup=max(2, iters // 6))
+    t_derived = ev(None)
+    space = blockwise_space(m, n_key, k, bs, row_entries)
+    for c in space:
+        ev(c)
+    top = sorted((t, s) for s, t in ev.cache.items() if s != "derived")[:5]
+    ev2 = BlockwiseEvaluator.__new__(BlockwiseEvaluator)
+    ev2.__dict__.update(ev.__dict__)
+    ev2.cache, ev2.iters, ev2.warmup = {}, 4 * iters, max(2, iters // 2)
+    final = sorted((ev2(json.loads(s)), s) for _, s in top)
+    t_derived = min(t_derived, ev2(None))
+    log(f"  {len(space)} configs; best {final[0][0]:.2f} us ({make_configs.blockwise_family(json.loads(final[0][1]))}) {final[0][1]}; "
+        f"derived {t_derived:.2f} us")
+    return json.loads(final[0][1]), final[0][0], t_derived
+
+
+def main_blockwise(args, shapes, tokens):
+    """--block-size: tunes tuna_amd/configs/param_map_blockwise.json, keys "<m>_<n>_<k>_<block_size>".  An entry is
+    written only where the tuned config beats the derived one by the replace margin (the derived config needs no
+    table entry)."""
+    base = args.base if args.base.endswith("_blockwise.json") else os.path.splitext(args.base)[0] + "_blockwise.json"
+    param_map, row_map = {}, {}
+    if os.path.exists(base):
+        with open(base) as f:
+            param_map = json.load(f)
+    row_base = base.replace("_blockwise.json", ".json")
+    if os.path.exists(row_base):
+        with open(row_base) as f:
+            row_map = json.load(f)
+    out = args.out if args.out.endswith("_blockwise.json") else os.path.splitext(args.out)[0] + "_blockwise.json"
+    os.makedirs(os.path.dirname(os.path.abspath(out)), exist_ok=True)
+    for name, m, k in shapes:
+        for n in tokens:
+            for bs in args.block_size:
+                if k % bs or bs >= k:
+                    continue
+                t0 = time.time()
+                print(f"tuning blockwise {name} m={m} n={n} k={k} block={bs}", flush=True)
+                rows = [e for key_, e in row_map.items() if key_.split("_")[0] == str(m) and key_.split("_")[2] == str(k)]
+                best, us, t_derived = tune_blockwise(m, n, k, bs, rows, iters=args.iters, log=lambda s_: print(s_, flush=True))
+                key = f"{m}_{make_configs.bucket_of(n)}_{k}_{bs}"
+                margin = args.replace_margin if args.replace_margin > 0 else 1.0
+                if us < margin * t_derived:
+                    best = dict(best)
+                    best["us"] = round(us, 3)
+                    best["us_derived"] = round(t_derived, 3)
+                    param_map[key] = best
+                    print(f"  -> {key}: {us:.2f} us against {t_derived:.2f} derived ({time.time() - t0:.0f} s)", flush=True)
+                else:
+                    param_map.pop(key, None)
+                    print(f"  -> {key}: the derived config stays ({t_derived:.2f} us; best timed {us:.2f})", flush=True)
+                with open(out, "w") as f:
+                    json.dump(param_map, f, indent=1, sort_keys=True)
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--shapes", default="all", help="comma list of shape names or 'all' or 'MxK,...'")
@@ -363,6 +512,9 @@ def main(argv=None):
                     help="an entry of --base is replaced only if the new config takes less than this fraction of its "
                          "time, both timed on this box (0: always replace)")
     ap.add_argument("--eval", default=None, help="JSON config: just time it on the given shapes and exit")
+    ap.add_argument("--block-size", default=None,
+                    help="comma list of scale-block sizes (64, 128, ...): tune the blockwise GEMM's table "
+                         "(param_map_blockwise.json beside --base / --out) instead of the per-row one")
     args = ap.parse_args(argv)
 
     shapes = []
@@ -373,6 +525,10 @@ def main(argv=None):
             mm, kk = tok.lower().split("x")
             shapes.append((tok, int(mm), int(kk)))
     tokens = [int(t) for t in args.tokens.split(",")]
+
+    if args.block_size:
+        args.block_size = [int(t) for t in args.block_size.split(",")]
+        return main_blockwise(args, shapes, tokens)
 
     if args.eval:
         c0 = json.loads(args.eval)
