@@ -1761,6 +1761,11 @@ def blockwise_cfg(family, m, n, k, bs, shape=None):
     elif family == "batched":
         for wm in (4, 2, 1):
             cands.append(cfg(rows_per_wave=64, waves_m=wm, waves_k=16 // wm, split_k=0, prefetch=2, x_chunk=512, token_tiles=1))
+    elif family == "many-token":
+        rows, tok = (128, 16 if n > 128 else 8) if n > 64 else (256, 4)
+        tiles_n = -(-m // rows) * -(-n // (16 * tok))
+        split = max(1, min(256 // max(1, tiles_n), (k // 64) // 8))
+        cands.append(cfg(rows_per_wave=64, waves_m=1, waves_k=1, split_k=split, prefetch=2, x_chunk=64, token_tiles=tok, lds_tile_rows=rows))
     elif family == "streaming":
         wm = 4 if m % 256 == 0 else 2 if m % 128 == 0 else 1
         wk = min(8, (8 if tiles == 4 else 16) // wm)
@@ -1956,9 +1961,12 @@ def test_blockwise_gemm_with_many_tokens_through_the_many_token_kernel(m, n, k, 
     dq, dx, dc, da = to_dev(q, x, code, absmax)
     out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
     L = _lib.lib()
+    c, _hit = ops.select_config_blockwise(m, n, k, bs)
+    if ops.blockwise_family(c) != "many-token":     # (a tuned entry of another kernel family: the tile the derivation would take)
+        c = blockwise_cfg("many-token", m, n, k, bs)
     before = L.tuna_blockwise_launches(2)
-    print(f"blockwise through the many-token kernel m={m} n={n} k={k} block={bs}", flush=True)
-    ops.matmul_blockwise(dx, dq, da, dc, out, m, n, k, bs)
+    print(f"blockwise through the many-token kernel m={m} n={n} k={k} block={bs} cfg={c.to_dict()}", flush=True)
+    ops.matmul_blockwise(dx, dq, da, dc, out, m, n, k, bs, config=c)
     torch.cuda.synchronize()
     assert L.tuna_blockwise_launches(2) == before + 1
     got = out.cpu().numpy().view(np.uint16)
@@ -1968,7 +1976,7 @@ def test_blockwise_gemm_with_many_tokens_through_the_many_token_kernel(m, n, k, 
     e = rel_err(f16_bits_to_f64(got[:, rows]), ref)
     assert e <= REL_TOL, e
     again = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
-    ops.matmul_blockwise(dx, dq, da, dc, again, m, n, k, bs)
+    ops.matmul_blockwise(dx, dq, da, dc, again, m, n, k, bs, config=c)
     torch.cuda.synchronize()
     assert np.array_equal(again.cpu().numpy().view(np.uint16), got)
     nh = min(n, k)
@@ -1976,7 +1984,7 @@ def test_blockwise_gemm_with_many_tokens_through_the_many_token_kernel(m, n, k, 
     xh = np.zeros((n, k), np.float16)
     xh[np.arange(nh), cols] = 1.0
     dxh, = to_dev(xh)
-    ops.matmul_blockwise(dxh, dq, da, dc, out, m, n, k, bs)
+    ops.matmul_blockwise(dxh, dq, da, dc, out, m, n, k, bs, config=c)
     torch.cuda.synchronize()
     img = O.dequant(q, absmax, code, m, k, mode=O.D1, block_size=bs)
     assert np.array_equal(out.cpu().numpy().view(np.uint16)[:nh], img[:, cols].T)
