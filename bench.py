@@ -285,14 +285,20 @@ def unit_rates(ops, dev):
              "mfma_32x32x16_f16_random_operands_one_wave_per_simd_tflops", "mfma_16x16x32_f16_random_operands_two_waves_per_simd_tflops",
              "mfma_16x16x32_f16_random_operands_one_wave_per_simd_tflops", "mfma_32x32x16_f16_random_operands_two_waves_per_simd_tflops",
              "lds_table_reads_b32_16_waves_bytes_per_clk_per_cu", "lds_fragment_reads_b128_16_waves_bytes_per_clk_per_cu",
-             "lds_tile_writes_b128_16_waves_bytes_per_clk_per_cu"]
+             "lds_tile_writes_b128_16_waves_bytes_per_clk_per_cu",
+             "mixed_64_token_k_step_mfma_only_us", "mixed_64_token_k_step_lds_reads_only_us",
+             "mixed_64_token_k_step_both_in_every_wave_us", "mixed_64_token_k_step_four_mfma_waves_four_lds_waves_us",
+             "mixed_64_token_k_step_reads_between_the_mfmas_us"]
     out = {}
     for unit, nm in enumerate(names):
         best = 0.0
         for _ in range(3):
             ms, work = ops.time_unit_rate(unit, dev, warmup=1, iters=4)
             best = max(best, work * 4 / (ms * 1e-3))
-        out[nm] = round(best / 1e12, 1) if nm.startswith("mfma") else round(best / 256 / 2.4e9, 1)
+        if nm.startswith("mixed"):
+            out[nm] = round(work / best * 1e6, 1)  # microseconds per launch (1024 k-steps per wave, 8 waves per CU)
+        else:
+            out[nm] = round(best / 1e12, 1) if nm.startswith("mfma") else round(best / 256 / 2.4e9, 1)
     out["note"] = ("LDS rates per compute unit at the 2.4 GHz peak clock, 256 compute units, from 8 waves per compute unit unless the name "
                    "says 16 (reads are latency-bound at 8); the random-operand MFMA rates (operands "
                    "of pseudo-random fp16 values instead of one pair of small regular numbers) are what the matrix cores sustain "

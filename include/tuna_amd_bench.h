@@ -103,9 +103,15 @@ int tuna_time_read(const void *src, void *sink, size_t bytes, int blocks, int va
  * 12 / 11: v_mfma_f32_16x16x32_f16 from one / two waves per SIMD, 16 accumulators, with four + four operand
  * registers of pseudo-random fp16 values in (-1, 1) - the rate the matrix cores sustain on real data, which is
  * well below the rate on the regular operands of units 0..2; 14 / 15 / 16: units 4 / 3 / 5 with 16 waves per
- * compute unit (8 waves do not keep enough reads in flight to saturate the LDS).  One workgroup per compute unit
- * (two for units 1, 11, 13).  *work_per_launch receives the flops (0..2, 10..13) or LDS bytes (3..9, 14..16) of
- * one launch; `sink`: 8 writable bytes. */
+ * compute unit (8 waves do not keep enough reads in flight to saturate the LDS); 17..21: the k-step of a 64-token
+ * streaming launch without its memory side, eight waves per compute unit, per wave and iteration sixteen table reads
+ * + four fragment reads and sixteen 16x16x32 MFMAs on pseudo-random operands - 17 the MFMAs only, 18 the LDS reads
+ * only, 19 both in every wave (reads requested ahead of the MFMAs, used behind them), 20 four waves (one per SIMD)
+ * with the MFMAs of two and four with the reads of two, 21 both in every wave with the reads requested between the
+ * MFMAs and used an iteration later: whether 19..21 take the longer of 17 and 18 or their sum says whether a compute
+ * unit overlaps the two.  One
+ * workgroup per compute unit (two for units 1, 11, 13).  *work_per_launch receives the flops (0..2, 10..13, 17..21:
+ * the MFMAs' of 17, also for 18) or LDS bytes (3..9, 14..16) of one launch; `sink`: 8 writable bytes. */
 int tuna_time_unit_rate(int unit, void *sink, int warmup, int iters, void *stream, float *elapsed_ms,
                         double *work_per_launch);
 

@@ -320,7 +320,7 @@ TUNA_EXPORT int tuna_time_unit_rate(int unit, void *sink, int warmup, int iters,
 {
     int rc;
     if ((rc = check_ptr(sink, "sink", 4))) return rc;
-    if (unit < 0 || unit > 16) return fail(TUNA_ERR_INVALID_ARG, "unit %d outside 0..16", unit);
+    if (unit < 0 || unit > 21) return fail(TUNA_ERR_INVALID_ARG, "unit %d outside 0..21", unit);
     if (!work_per_launch) return fail(TUNA_ERR_INVALID_ARG, "work_per_launch is null");
     int dev = 0, cus = 0;
     hipError_t e = device_cus(&dev, &cus);

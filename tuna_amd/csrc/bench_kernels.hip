@@ -339,15 +339,134 @@ __global__ __launch_bounds__(THREADS) void lds_rate_kernel(uint32_t *sink)
     if (s == 0x9e3779b9u && sink[1] == 77u) sink[0] = s;  // practically never
 }
 
+// The k-step of a 64-token streaming launch without its memory side, eight waves per CU: per wave and iteration
+// sixteen table reads and four fragment reads from LDS and sixteen independent 16x16x32 MFMAs on pseudo-random
+// operands.  MODE 0: the MFMAs only; 1: the LDS reads only; 2: both in every wave, the reads requested ahead of the
+// MFMAs and used behind them; 3: waves 0-3 (one per SIMD) do the MFMAs of two waves, waves 4-7 the reads of two;
+// 4: both in every wave, one or two reads requested behind each MFMA and used two iterations later.
+// Whether 2 and 3 take the longer of 0 and 1 or their sum says whether a CU overlaps the two kinds of work.
+constexpr int kMixedIters = 1024;
+template <int MODE>
+__global__ __launch_bounds__(512) void mixed_rate_kernel(uint32_t *sink)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    for (int i = threadIdx.x; i < 65536 / 4; i += 512) reinterpret_cast<uint32_t *>(smem)[i] = (uint32_t)i;
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    f16x8 a[4], b[4];
+#pragma unroll
+    for (int o = 0; o < 4; ++o)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            uint32_t h = (threadIdx.x * 8u + e + o * 4099u + blockIdx.x * 131071u) * 2654435761u;
+            h ^= h >> 15, h *= 2246822519u, h ^= h >> 13;
+            a[o][e] = (f16)((float)(int)(h & 0xffffu) * (1.0f / 32768.0f) - 1.0f);
+            b[o][e] = (f16)((float)(int)(h >> 16) * (1.0f / 32768.0f) - 1.0f);
+        }
+    rate_f32x4 acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = rate_f32x4{0.f, 0.f, 0.f, 0.f};
+    uint32_t s = 0;
+    const bool do_mfma = MODE == 0 || MODE == 2 || (MODE == 3 && wave < 4);
+    const bool do_lds = MODE == 1 || MODE == 2 || (MODE == 3 && wave >= 4);
+    const int reps = MODE == 3 ? 2 : 1;
+    for (int it = 0; it < (MODE == 4 ? 0 : kMixedIters); ++it)
+        for (int rep = 0; rep < reps; ++rep) {
+            uint32_t t[16];
+            u32x4 f[4];
+            if (do_lds) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    uint32_t off = ((uint32_t)((it * 16 + r + wave * 31 + rep * 7) & 255) << 8) | ((uint32_t)lane << 2);
+                    asm volatile("" : "+v"(off));
+                    t[r] = *reinterpret_cast<const uint32_t *>(smem + off);
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    uint32_t off = (uint32_t)(lane * 16 + r * 1024 + wave * 4096 + ((it + rep) & 1) * 32768) & 65535u;
+                    asm volatile("" : "+v"(off));
+                    f[r] = *reinterpret_cast<const u32x4 *>(smem + off);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (do_mfma) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i >> 2], b[i & 3], acc[i], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (do_lds) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s += t[r];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) s += f[r][0] ^ f[r][1] ^ f[r][2] ^ f[r][3];
+            }
+        }
+    if constexpr (MODE == 4) {
+        // the reads of an iteration are requested between its MFMAs, one or two behind each, and used at the end of
+        // the next iteration (two register sets take turns: a copy would wait for the reads it copies)
+        uint32_t t[2][16];
+        u32x4 f[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) t[h][r] = 0u;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) f[h][r] = u32x4{0u, 0u, 0u, 0u};
+        }
+        for (int it = 0; it < kMixedIters; it += 2) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s += t[h][r];  // (requested an iteration ago... or two, for h = 0 of the first turn: zeros)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) s += f[h][r][0] ^ f[h][r][1] ^ f[h][r][2] ^ f[h][r][3];
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i >> 2], b[i & 3], acc[i], 0, 0, 0);
+                    uint32_t off = ((uint32_t)(((it + h) * 16 + i + wave * 31) & 255) << 8) | ((uint32_t)lane << 2);
+                    asm volatile("" : "+v"(off));
+                    t[h][i] = *reinterpret_cast<const uint32_t *>(smem + off);
+                    if (i < 4) {
+                        uint32_t off2 = (uint32_t)(lane * 16 + i * 1024 + wave * 4096 + h * 32768) & 65535u;
+                        asm volatile("" : "+v"(off2));
+                        f[h][i] = *reinterpret_cast<const u32x4 *>(smem + off2);
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // a table read and a fragment read
+                }
+#pragma unroll
+                for (int i = 4; i < 16; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s += t[h][r];
+    }
+    float fs = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) fs += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+    if ((s == 0x9e3779b9u && sink[1] == 77u) || fs == 12345.678f) sink[0] = s;  // practically never
+}
+
 // unit: 0 / 1 v_mfma_f32_16x16x32_f16 with one / two waves per SIMD (16 accumulators), 2 v_mfma_f32_32x32x16_f16
 // (one wave per SIMD, 4 accumulators); 3 LDS fragment reads, 4 LDS table reads, 5 LDS tile writes, 6 the tile
 // writes as 8-byte halves, 7 16-byte writes at consecutive addresses, 8 / 9 table reads with a copy of the table
 // per 32 / 16 lanes; 10 / 13 32x32x16 and 12 / 11 16x16x32 MFMAs on pseudo-random operands from one / two waves per
-// SIMD; 14 / 15 / 16: units 4 / 3 / 5 from 16 waves per compute unit.  *work = flops (0..2, 10..13) or bytes
-// (3..9, 14..16) of one launch on `cus` compute units.
+// SIMD; 14 / 15 / 16: units 4 / 3 / 5 from 16 waves per compute unit; 17..21: mixed_rate_kernel<0..4>.  *work = flops
+// (0..2, 10..13, 17..21: those of the MFMAs of modes 0, 2 and 3, also for mode 1, which has none - the four times
+// are what is compared) or bytes (3..9, 14..16) of one launch on `cus` compute units.
 hipError_t launch_unit_rate(int unit, int cus, uint32_t *sink, double *work, hipStream_t stream)
 {
-    static OptInFlag attr[16][10];
+    static OptInFlag attr[16][15];
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
@@ -384,6 +503,21 @@ hipError_t launch_unit_rate(int unit, int cus, uint32_t *sink, double *work, hip
     case 16:
         if ((e = ensure_lds_opt_in(attr[dev][9], reinterpret_cast<const void *>(lds_rate_kernel<2, 1024>))) != hipSuccess) return e;
         hipLaunchKernelGGL((lds_rate_kernel<2, 1024>), dim3(cus), dim3(1024), 65536, stream, sink); *work = (double)cus * 1024 * kRateIters * 8 * 16.0; break;
+    case 17:
+        if ((e = ensure_lds_opt_in(attr[dev][10], reinterpret_cast<const void *>(mixed_rate_kernel<0>))) != hipSuccess) return e;
+        hipLaunchKernelGGL(mixed_rate_kernel<0>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 8 * kMixedIters * 16 * 16384.0; break;
+    case 18:
+        if ((e = ensure_lds_opt_in(attr[dev][11], reinterpret_cast<const void *>(mixed_rate_kernel<1>))) != hipSuccess) return e;
+        hipLaunchKernelGGL(mixed_rate_kernel<1>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 8 * kMixedIters * 16 * 16384.0; break;
+    case 19:
+        if ((e = ensure_lds_opt_in(attr[dev][12], reinterpret_cast<const void *>(mixed_rate_kernel<2>))) != hipSuccess) return e;
+        hipLaunchKernelGGL(mixed_rate_kernel<2>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 8 * kMixedIters * 16 * 16384.0; break;
+    case 20:
+        if ((e = ensure_lds_opt_in(attr[dev][13], reinterpret_cast<const void *>(mixed_rate_kernel<3>))) != hipSuccess) return e;
+        hipLaunchKernelGGL(mixed_rate_kernel<3>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 8 * kMixedIters * 16 * 16384.0; break;
+    case 21:
+        if ((e = ensure_lds_opt_in(attr[dev][14], reinterpret_cast<const void *>(mixed_rate_kernel<4>))) != hipSuccess) return e;
+        hipLaunchKernelGGL(mixed_rate_kernel<4>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 8 * kMixedIters * 16 * 16384.0; break;
     case 8:
         if ((e = ensure_lds_opt_in(attr[dev][5], reinterpret_cast<const void *>(lds_rate_kernel<5>))) != hipSuccess) return e;
         hipLaunchKernelGGL(lds_rate_kernel<5>, dim3(cus), dim3(512), 65536, stream, sink); *work = (double)cus * 512 * kRateIters * 8 * 4.0; break;
