@@ -630,19 +630,23 @@ def main():
         sets = [synth.make_weights_torch(8 * gm, gk, 4000 + i, dev) for i in range(3)]
         moe = {}
         for label, counts in (("balanced_4_per_expert", [4] * 8), ("skewed", [9, 0, 6, 1, 0, 11, 5, 0]),
-                              ("two_experts", [16, 0, 0, 0, 16, 0, 0, 0])):
+                              ("two_experts", [16, 0, 0, 0, 16, 0, 0, 0]),
+                              ("prefill_256_per_expert", [256] * 8), ("prefill_skewed", [700, 3, 0, 90, 1024, 40, 0, 191])):
             offs = [0]
             for cnt in counts:
                 offs.append(offs[-1] + cnt)
             xg = synth.make_x_torch(offs[-1], gk, 7, dev)
             og = torch.empty((offs[-1], gm), dtype=torch.float16, device=dev)
+            big = max(counts) > 64  # (groups of more than 64 tokens run as dense GEMMs of their own: fewer, longer calls)
+            it = 12 if big else 100
             ms = ops.time_matmul_grouped([s_[0] for s_ in sets], [s_[1] for s_ in sets], xg, nf4_codebook(dev), og, gm, 8, gk,
-                                         offs, warmup=10, iters=100, use_graph=True)
-            us = ms * 10.0
+                                         offs, warmup=3 if big else 10, iters=it, use_graph=True)
+            us = ms * 1e3 / it
             active = sum(1 for cnt in counts if cnt)
             moe[label] = {"tokens_per_expert": counts, "us": round(us, 2), "active_experts": active,
                           "packed_bytes_read": active * gm * gk // 2,
-                          "gbs": round(active * gm * gk / 2 / (us * 1e-6) / 1e9, 1)}
+                          "gbs": round(active * gm * gk / 2 / (us * 1e-6) / 1e9, 1),
+                          "tflops": round(2.0 * offs[-1] * gm * gk / (us * 1e-6) / 1e12, 1)}
         del sets
         torch.cuda.empty_cache()
         line["mixtral_gate_up_routed"] = moe

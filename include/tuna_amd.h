@@ -199,7 +199,11 @@ int tuna_matmul_multi_blockwise(const tuna_gemm_problem *problems, int count, in
  *   out[t, r] = x[t, :] . decode(W_e)[r, :]   for t in group e.
  * Groups without tokens are skipped: their weights are not read.  m_group must be a multiple
  * of 64 (of the config's rows per workgroup if cfg is given; NULL = table lookup on
- * (n_groups*m_group, largest group, k)).  No counterpart in the reference, whose 8-expert
+ * (n_groups*m_group, largest group, k)).  With cfg NULL a group of more than 64 tokens (prefill
+ * sizes) runs as a dense GEMM of its own on the same stream - tuna_matmul on the group's slices
+ * of q, absmax, x and out, bit-identical to that call - and only the smaller groups share the
+ * grouped launch: the grouped kernel would stream such a group's weights once per 64 tokens, the
+ * many-token kernels decode them once per 128 to 256.  No counterpart in the reference, whose 8-expert
  * benchmark applies every expert to every token (README.md:16-18); this is the op a
  * router-driven Mixtral layer needs. */
 int tuna_matmul_grouped(const void *q, const void *x, const void *code, const void *absmax,

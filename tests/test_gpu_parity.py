@@ -719,6 +719,36 @@ def test_grouped_gemm_matches_per_expert_oracle(m_group, n_groups, k, counts, ck
     assert e <= REL_TOL, e
 
 
+@pytest.mark.parametrize("m_group,n_groups,k,counts", [
+    (256, 4, 1024, [65, 3, 0, 130]),        # two groups as dense GEMMs, one through the grouped kernel, one empty
+    (512, 3, 512, [200, 96, 257]),          # every group a dense GEMM (nothing left for the grouped kernel)
+    (256, 5, 2048, [64, 65, 1, 0, 300]),    # 64 tokens still fit one pass of the grouped kernel, 65 do not
+])
+def test_grouped_gemm_with_groups_of_many_tokens_matches_per_expert_oracle(m_group, n_groups, k, counts):
+    """Groups of more than 64 tokens run as dense GEMMs of their own (the library's config for their token count),
+    the others in one grouped launch: every row against the oracle, and the rows of a large group bit-identical to
+    the dense call on that group's slices."""
+    offsets = [0]
+    for c in counts:
+        offsets.append(offsets[-1] + c)
+    n_total = offsets[-1]
+    m = m_group * n_groups
+    print(f"grouped, many tokens: m_group={m_group} n_groups={n_groups} k={k} counts={counts}", flush=True)
+    q, x, code, absmax = make_inputs_np(m, n_total, k, seed=78)
+    got = _run_grouped(q, x, code, absmax, m_group, n_groups, k, offsets, None)
+    ref = _grouped_reference(q, x, code, absmax, m_group, n_groups, k, offsets)
+    assert not np.isnan(f16_bits_to_f64(got)).any()          # every output row was written
+    e = rel_err(f16_bits_to_f64(got), ref)
+    assert e <= REL_TOL, e
+    qb = q.reshape(n_groups, m_group // 8, k // 8, 32)
+    for g, c in enumerate(counts):
+        if c > 64:
+            lo, hi = offsets[g], offsets[g + 1]
+            dense = run_gemm(np.ascontiguousarray(qb[g]), np.ascontiguousarray(x[lo:hi]), code,
+                             np.ascontiguousarray(absmax[g * m_group:(g + 1) * m_group]), m_group, c, k)
+            assert np.array_equal(dense, got[lo:hi]), g
+
+
 def test_grouped_gemm_with_one_group_equals_dense_bits():
     """One group owning every token is the dense GEMM: identical bits."""
     m, n, k = 1024, 16, 2048

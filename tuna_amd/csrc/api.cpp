@@ -1086,11 +1086,44 @@ static int matmul_grouped_impl(const void *q, const void *x, const void *code, c
     if ((rc = check_ptr(q, "q", 16)) || (rc = check_ptr(x, "x", 16)) || (rc = check_ptr(code, "code", 4)) ||
         (rc = check_ptr(absmax, "absmax", 4)) || (rc = check_ptr(out, "out", 16)))
         return rc;
-    // Only groups with tokens are walked: the launch is planned for their rows alone.
+    // Groups with more tokens than one pass of the grouped kernel takes (64: it would stream their weights once per 64
+    // tokens) run as dense GEMMs of their own, each with the table's config for its token count - from 128 tokens a
+    // group that is the many-token kernel at two to three times the rate, and a launch per group is nothing beside
+    // hundreds of microseconds of matrix work.  (With an explicit config every group goes through the grouped kernel.)
+    constexpr int kGroupedPassTokens = 64;
+    const size_t group_q_bytes = (size_t)m_group * (size_t)k / 2;
+    if (!cfg) {
+        // (checked before anything is enqueued: a group that cannot run must not leave the others' rows written)
+        for (int e = 0; e < n_groups; ++e) {
+            const int cnt = offsets[e + 1] - offsets[e];
+            if (cnt <= kGroupedPassTokens) continue;
+            tuna_gemm_config dc;
+            select_config_for(m_group, cnt, k, decode, &dc, nullptr);
+            if ((rc = validate_for(m_group, cnt, k, dc, decode))) return rc;
+        }
+        for (int e = 0; e < n_groups; ++e) {
+            const int cnt = offsets[e + 1] - offsets[e];
+            if (cnt <= kGroupedPassTokens) continue;
+            // (x rows are k fp16 values and out rows m_group: both multiples of 16 bytes, so the slices stay aligned)
+            rc = matmul_impl(static_cast<const uint8_t *>(q) + (size_t)e * group_q_bytes,
+                             static_cast<const uint8_t *>(x) + (size_t)offsets[e] * (size_t)k * 2, code,
+                             static_cast<const float *>(absmax) + (size_t)e * (size_t)m_group,
+                             static_cast<uint8_t *>(out) + (size_t)offsets[e] * (size_t)m_group * 2, m_group, cnt, k, nullptr, decode,
+                             stream);
+            if (rc) return rc;
+        }
+    }
+    // Only the remaining groups with tokens are walked: the launch is planned for their rows alone.
     int n_active = 0;
     unsigned char act[kMaxGroups];
-    for (int e = 0; e < n_groups; ++e)
-        if (offsets[e + 1] > offsets[e]) act[n_active++] = (unsigned char)e;
+    max_tok = 0;
+    for (int e = 0; e < n_groups; ++e) {
+        const int cnt = offsets[e + 1] - offsets[e];
+        if (cnt <= 0 || (!cfg && cnt > kGroupedPassTokens)) continue;
+        act[n_active++] = (unsigned char)e;
+        if (cnt > max_tok) max_tok = cnt;
+    }
+    if (n_active == 0) return TUNA_OK;  // every group with tokens ran as a dense GEMM
     const int m_active = m_group * n_active;
     tuna_gemm_config c;
     GemmPlan plan;

@@ -165,7 +165,8 @@ def matmul_grouped(x, q, s, c, o, m_group: int, n_groups: int, k: int, token_off
 
     x fp16 [n_total, k], rows sorted by group; q uint8 [n_groups*m_group/8, k/8, 32] and s fp32
     [n_groups*m_group]: the groups' weights stacked along m; o fp16 [n_total, m_group];
-    token_offsets: n_groups+1 non-decreasing host ints.  Groups without tokens cost nothing.
+    token_offsets: n_groups+1 non-decreasing host ints.  Groups without tokens cost nothing; without a config a
+    group of more than 64 tokens runs as a dense GEMM of its own (same bits as `matmul` on its slices).
     """
     m_group, n_groups, k = int(m_group), int(n_groups), int(k)
     offs = [int(v) for v in token_offsets]
