@@ -18,8 +18,7 @@ between launches).  The LAST line printed is one compact JSON object (under 2 KB
 
 Everything else - the per-shape table with configs and kernels, the same shapes eight to a launch, the
 Llama-70B 80-layer sweep, the token sweep, the dequant / quantizer / blockwise timings and the yardsticks -
-goes into one "detail" JSON object that is printed on an earlier line and written to
-gpurun_out/bench_detail.json.
+goes into one "detail" JSON object that is printed on an earlier line and written to the file DETAIL_FILE names.
 """
 import argparse
 import json
