@@ -667,7 +667,7 @@ def test_errors_raise_instead_of_silent_noop():
 
 
 # ----------------------------------------------------------------------------- grouped GEMM (per-expert token lists)
-def _run_grouped(q, x, code, absmax, m_group, n_groups, k, offsets, config=None):
+def _run_grouped(q, x, code, absmax, m_group, n_groups, k, offsets, config=None, decode_mode=1):
     import torch
 
     from tuna_amd import ops
@@ -675,12 +675,12 @@ def _run_grouped(q, x, code, absmax, m_group, n_groups, k, offsets, config=None)
     dq, dx, dc, da = to_dev(q, x, code, absmax)
     n_total = offsets[-1]
     out = torch.full((max(n_total, 1), m_group), float("nan"), dtype=torch.float16, device="cuda")[:n_total]
-    ops.matmul_grouped(dx, dq, da, dc, out, m_group, n_groups, k, offsets, config=config)
+    ops.matmul_grouped(dx, dq, da, dc, out, m_group, n_groups, k, offsets, config=config, decode_mode=decode_mode)
     torch.cuda.synchronize()
     return out.cpu().numpy().view(np.uint16)
 
 
-def _grouped_reference(q, x, code, absmax, m_group, n_groups, k, offsets):
+def _grouped_reference(q, x, code, absmax, m_group, n_groups, k, offsets, mode=O.D1):
     """Per expert: the oracle's dense GEMM on that expert's packed rows and tokens."""
     n_total = offsets[-1]
     ref = np.zeros((n_total, m_group), dtype=np.float64)
@@ -689,7 +689,7 @@ def _grouped_reference(q, x, code, absmax, m_group, n_groups, k, offsets):
         lo, hi = offsets[e], offsets[e + 1]
         if hi > lo:
             ref[lo:hi] = O.gemm_f64(np.ascontiguousarray(qb[e]), np.ascontiguousarray(x[lo:hi]), code,
-                                    np.ascontiguousarray(absmax[e * m_group:(e + 1) * m_group]), m_group, hi - lo, k, mode=O.D1)
+                                    np.ascontiguousarray(absmax[e * m_group:(e + 1) * m_group]), m_group, hi - lo, k, mode=mode)
     return ref
 
 
@@ -747,6 +747,21 @@ def test_grouped_gemm_with_groups_of_many_tokens_matches_per_expert_oracle(m_gro
             dense = run_gemm(np.ascontiguousarray(qb[g]), np.ascontiguousarray(x[lo:hi]), code,
                              np.ascontiguousarray(absmax[g * m_group:(g + 1) * m_group]), m_group, c, k)
             assert np.array_equal(dense, got[lo:hi]), g
+
+
+def test_grouped_gemm_with_a_large_group_and_the_dequantizers_rounding():
+    """decode_mode D2 (fp32 multiply, then round) reaches the dense launches of the large groups too."""
+    m_group, n_groups, k, counts = 256, 3, 512, [7, 150, 0]
+    offsets = [0, 7, 157, 157]
+    q, x, code, absmax = make_inputs_np(m_group * n_groups, offsets[-1], k, seed=79)
+    got = _run_grouped(q, x, code, absmax, m_group, n_groups, k, offsets, None, decode_mode=O.D2)
+    ref = _grouped_reference(q, x, code, absmax, m_group, n_groups, k, offsets, mode=O.D2)
+    assert not np.isnan(f16_bits_to_f64(got)).any()
+    assert rel_err(f16_bits_to_f64(got), ref) <= REL_TOL
+    qb = q.reshape(n_groups, m_group // 8, k // 8, 32)
+    dense = run_gemm(np.ascontiguousarray(qb[1]), np.ascontiguousarray(x[7:157]), code, np.ascontiguousarray(absmax[256:512]),
+                     m_group, 150, k, decode_mode=O.D2)
+    assert np.array_equal(dense, got[7:157])
 
 
 def test_grouped_gemm_with_one_group_equals_dense_bits():
