@@ -702,6 +702,8 @@ def _grouped_reference(q, x, code, absmax, m_group, n_groups, k, offsets, mode=O
     (1024, 3, 512, [5, 5, 5], dict(waves_m=8, waves_k=1, prefetch=2, x_chunk=64)),            # register-store epilogue
     (256, 6, 2048, [1, 0, 2, 0, 0, 9], dict(split_k=0, waves_m=1, waves_k=4, prefetch=2, x_chunk=256)),  # balanced split
     (128, 64, 256, [i % 3 for i in range(64)], None),                      # 64 experts
+    (512, 4, 2048, [40, 64, 33, 7], None),                                 # 33..64 tokens: four token tiles, one pass
+    (1024, 3, 4096, [48, 0, 64], None),
 ])
 def test_grouped_gemm_matches_per_expert_oracle(m_group, n_groups, k, counts, ckw):
     offsets = [0]
