@@ -315,6 +315,10 @@ int tuna_config_contributors(int m, int n, int k, const tuna_gemm_config *cfg, i
 /* Enumerate the built-in table: entry i -> its shape key and config. */
 int tuna_config_table_size(void);
 int tuna_config_table_entry(int i, int *m, int *n_lo, int *n_hi, int *k, tuna_gemm_config *cfg);
+/* Entries are tuned at the lower edge n_lo of their token bucket; token counts from this value to n_hi get the next
+ * bucket's entry from tuna_select_config instead, where that entry can run them (n_hi + 1: none does; -1: bad
+ * index).  Written by the tuner, which times both entries inside the bucket. */
+int tuna_config_table_next_from(int i);
 
 /* Releases the library-owned split-K workspaces of the current device (synchronises
  * the device first).  Until then a workspace that a launch has used is never freed or moved -

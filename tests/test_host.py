@@ -71,20 +71,22 @@ def test_select_config_is_host_only_and_every_table_entry_validates():
     from tuna_amd import make_configs, ops
 
     table = ops.config_table()
+    next_from = ops.config_table_next_from()
     with open(os.path.join(ROOT, "tuna_amd", "configs", "param_map.json")) as f:
         pm = json.load(f)
-    assert len(table) == len(pm)
-    for m, lo, hi, k, cfg in table:
+    assert len(table) == len(pm) == len(next_from)
+    for (m, lo, hi, k, cfg), nf in zip(table, next_from):
         key = f"{m}_{make_configs.bucket_of(lo)}_{k}"
         assert key in pm
         assert cfg.to_dict() == {f: pm[key][f] for f in cfg.FIELDS}
-        for n in (lo, hi):
+        assert nf == make_configs.next_from_of(make_configs.bucket_of(lo), pm[key]) and lo < nf <= hi + 1
+        for n in sorted({lo, hi, min(nf, hi), max(nf - 1, lo)}):
             ops.validate_config(m, n, k, cfg)                      # the C side accepts it
             got, hit = ops.select_config(m, n, k)
             assert hit
-            # entries are tuned at their bucket's lower edge: a count inside one of the buckets
-            # 16.., 32.., 64.., 128.. takes the next bucket's entry (fewer passes over the weights), as do 10..15 tokens
-            nxt = pm.get(f"{m}_{hi + 1}_{k}") if (n > lo and (16 <= lo <= 128 or (lo == 1 and n >= 10))) else None
+            # entries are tuned at their bucket's lower edge: counts from the entry's next_from on take the next
+            # bucket's entry (fewer passes over the weights)
+            nxt = pm.get(f"{m}_{make_configs.bucket_of(hi + 1)}_{k}") if n >= nf and hi < 128000 else None
             if n >= 3072 and m < 24576 and k % 64 == 0:
                 # far into the open-ended last bucket (tuned at 2048 tokens): the 256 x 256 many-token tile
                 assert (got.lds_tile_rows, got.token_tiles, got.split_k, got.rows_per_wave) == (256, 16, 1, 64)
@@ -157,9 +159,16 @@ def test_generator_output_and_its_refusal_of_inconsistent_entries(tmp_path):
           "4096_1_4096": dict(rows_per_wave=64, waves_m=1, waves_k=8, split_k=4, prefetch=2, x_chunk=1024,
                               token_tiles=1, xcd_swizzle=0, k_stagger=3)}
     text = mc.generate(pm)
-    assert "{4096, 16, 31, 4096, {64, 1, 8, 4, 2, 1024, 1, 1, 0, 0}}" in text  # k_stagger, lds_tile_rows default to 0
-    assert "{4096, 1, 15, 4096, {64, 1, 8, 4, 2, 1024, 1, 0, 3, 0}}" in text
+    # (k_stagger, lds_tile_rows default to 0; next_from, the fifth value, to 17 in the bucket 16..31 and 10 in 1..15)
+    assert "{4096, 16, 31, 4096, 17, {64, 1, 8, 4, 2, 1024, 1, 1, 0, 0}}" in text
+    assert "{4096, 1, 15, 4096, 10, {64, 1, 8, 4, 2, 1024, 1, 0, 3, 0}}" in text
     assert "kConfigTableSize = 2" in text
+    # a tuned hand-over count is emitted as it is, one outside the bucket refused
+    assert "{4096, 16, 31, 4096, 25, {" in mc.generate({"4096_16_4096": dict(pm["4096_16_4096"], next_from=25)})
+    assert "{4096, 16, 31, 4096, 32, {" in mc.generate({"4096_16_4096": dict(pm["4096_16_4096"], next_from=32)})  # never
+    for bad in (16, 33, 0):
+        with pytest.raises(ValueError, match="next_from"):
+            mc.generate({"4096_16_4096": dict(pm["4096_16_4096"], next_from=bad)})
     # the checked-in table is what the generator produces from the checked-in json
     with open(os.path.join(ROOT, "tuna_amd", "configs", "param_map.json")) as f:
         real = json.load(f)

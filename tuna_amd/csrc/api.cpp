@@ -576,14 +576,13 @@ static bool config_runs(int m, int n, int k, const tuna_gemm_config &c)
     return plan_gemm(m, n, k, c, TUNA_DECODE_GEMM, &plan) == TUNA_OK;
 }
 
-// The table's buckets are the reference dispatcher's (kernel.cu:3022-3155) and every entry is
-// tuned at the lower edge of its bucket.  A token count inside one of the buckets 16..31, 32..63,
-// 64..127 or 128..255 takes two passes over the weights with that entry (it covers the lower
-// edge in one) but one pass with the entry of the next bucket, which is tuned for more tokens per
-// pass: measured on six of the benchmark shapes, 17..255 tokens, the next bucket's entry is 15-40 %
-// faster (8192 x 8192 at 20 tokens 23.8 -> 14.8 us, 57344 x 8192 at 24 tokens 81 -> 57 us,
-// 229376 x 4096 at 100 tokens 297 -> 237 us), so such a count takes it when it can run the shape.
-// Up to 9 tokens and from 256 tokens the containing bucket's entry stays (but see the last bucket below).
+// The table's buckets are the reference dispatcher's (kernel.cu:3022-3155) and every entry is tuned at the lower edge
+// of its bucket.  A token count inside a bucket often runs faster with the entry of the NEXT bucket, which is tuned for
+// more tokens per pass over the weights (8192 x 28672 at 17 tokens 79 -> 40 us, 8192 x 8192 at 20 tokens 23.8 -> 14.8,
+// 229376 x 4096 at 100 tokens 297 -> 237) - but not always (2560 x 2560 at 65..96 tokens: 6.7 us with its own entry,
+// 10.7 with the next).  Where the hand-over lies is therefore a field of the entry, next_from: the tuner times both
+// entries at several counts inside the bucket and writes the count from which the next one wins; entries without
+// a tuned value get make_configs.default_next_from.
 static int select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_table)
 {
     const TableEntry *own = nullptr;
@@ -591,10 +590,7 @@ static int select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_t
         const TableEntry &e = kConfigTable[i];
         if (e.m == m && e.k == k && n >= e.n_lo && n <= e.n_hi) own = &e;
     }
-    // The first bucket (1..15 tokens) is tuned at one token: from 10 tokens the 16-token entry is the better one too
-    // (ten benchmark shapes at 12 / 15 tokens: 3 % / 9 % less time in sum, 8192 x 28672 at 15 tokens 36.1 -> 28.9 us;
-    // at 8 tokens they are even, at 4 the one-token entry wins).
-    if (own && ((n > own->n_lo && own->n_lo >= 16 && own->n_lo <= 128) || (own->n_lo == 1 && n >= 10))) {
+    if (own && n >= own->next_from) {
         for (int i = 0; i < kConfigTableSize; ++i) {
             const TableEntry &e = kConfigTable[i];
             if (e.m == m && e.k == k && e.n_lo == own->n_hi + 1) {
@@ -1930,6 +1926,15 @@ TUNA_EXPORT int tuna_config_table_entry(int i, int *m, int *n_lo, int *n_hi, int
     if (k) *k = e.k;
     if (cfg) *cfg = e.cfg;
     return TUNA_OK;
+}
+
+TUNA_EXPORT int tuna_config_table_next_from(int i)
+{
+    if (i < 0 || i >= kConfigTableSize) {
+        fail(TUNA_ERR_INVALID_ARG, "table index %d out of range", i);
+        return -1;
+    }
+    return kConfigTable[i].next_from;
 }
 
 TUNA_EXPORT int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config *cfg, int decode_mode, char *buf, size_t len)

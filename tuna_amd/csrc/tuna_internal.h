@@ -232,6 +232,7 @@ void drop_workspace(hipStream_t stream);  // frees the split-K workspace of a st
 // config_table.cpp
 struct TableEntry {
     int m, n_lo, n_hi, k;
+    int next_from;  // token counts from here to n_hi take the next bucket's entry (n_hi + 1: none does)
     tuna_gemm_config cfg;
 };
 extern const TableEntry kConfigTable[];

@@ -322,6 +322,27 @@ const int kBlockwiseTableSize = {len(rows)};
 """
 
 
+def default_next_from(n_key: int) -> int:
+    """Where an entry without a tuned "next_from" hands over to the next bucket's entry: entries are tuned at the
+    lower edge of their bucket, and a count inside one of the buckets 16.., 32.., 64.., 128.. takes two passes over
+    the weights with such an entry but one with the next bucket's (from 10 tokens in the first bucket); the other
+    buckets keep their entry throughout (n_hi + 1: never)."""
+    lo, hi = N_BUCKETS[n_key]
+    if lo == 1:
+        return 10
+    return lo + 1 if 16 <= lo <= 128 else hi + 1
+
+
+def next_from_of(n_key: int, c: dict) -> int:
+    """The entry's "next_from" (the token count from which the lookup hands out the next bucket's entry instead;
+    written by the tuner, which times both entries inside the bucket), checked: n_lo < next_from <= n_hi + 1."""
+    lo, hi = N_BUCKETS[n_key]
+    nf = int(c.get("next_from", default_next_from(n_key)))
+    if not lo < nf <= hi + 1:
+        raise ValueError(f"next_from={nf} outside {lo + 1}..{hi + 1}")
+    return nf
+
+
 def generate(param_map: dict) -> str:
     rows = []
     for key in sorted(param_map, key=lambda s: tuple(int(t) for t in s.split("_"))):
@@ -329,22 +350,23 @@ def generate(param_map: dict) -> str:
         c = param_map[key]
         try:
             validate(m, n, k, c)
+            nf = next_from_of(n, c)
         except ValueError as e:
             raise ValueError(f"param_map entry {key}: {e}") from None
         lo, hi = N_BUCKETS[n]
         vals = ", ".join(str(int(c.get(f, 0))) for f in FIELDS)
-        rows.append(f"    {{{m}, {lo}, {hi}, {k}, {{{vals}}}}},  // {key}")
+        rows.append(f"    {{{m}, {lo}, {hi}, {k}, {nf}, {{{vals}}}}},  // {key}")
     body = "\n".join(rows)
     return f"""// GENERATED by tuna_amd/make_configs.py from tuna_amd/configs/param_map.json - do not edit.
 // Shape -> tile-config table, searched linearly by tuna_select_config.
-// Entry: m, n_lo, n_hi, k, {{{", ".join(FIELDS)}}}
+// Entry: m, n_lo, n_hi, k, next_from, {{{", ".join(FIELDS)}}}
 #include "tuna_internal.h"
 
 namespace tuna {{
 
 const TableEntry kConfigTable[] = {{
 {body}
-    {{0, 0, 0, 0, {{0, 0, 0, 0, 0, 0, 0, 0, 0, 0}}}},  // sentinel (not counted)
+    {{0, 0, 0, 0, 0, {{0, 0, 0, 0, 0, 0, 0, 0, 0, 0}}}},  // sentinel (not counted)
 }};
 const int kConfigTableSize = {len(rows)};
 

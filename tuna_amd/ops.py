@@ -361,6 +361,13 @@ def config_table():
     return out
 
 
+def config_table_next_from():
+    """Per entry of config_table(): the token count from which select_config hands out the next bucket's entry
+    (n_hi + 1: never)."""
+    L = _lib.lib()
+    return [L.tuna_config_table_next_from(i) for i in range(L.tuna_config_table_size())]
+
+
 def _ptr_array(tensors):
     arr = (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
     return ctypes.cast(arr, ctypes.POINTER(ctypes.c_void_p)), arr

@@ -496,6 +496,53 @@ def main_blockwise(args, shapes, tokens):
                     json.dump(param_map, f, indent=1, sort_keys=True)
 
 
+def next_from_samples(n_key: int):
+    """Token counts inside a bucket at which its entry is timed against the next bucket's."""
+    lo, hi = make_configs.N_BUCKETS[n_key]
+    if lo == 1:
+        return [2, 4, 6, 8, 10, 12, 15]
+    span = hi - lo
+    return sorted({lo + 1, lo + span // 4, lo + span // 2, lo + 3 * span // 4, hi})
+
+
+def tune_next_from(param_map, keys, iters=40, margin=0.98, log=print):
+    """Writes "next_from" into the entries `keys` of param_map: the smallest sampled token count from which the next
+    bucket's entry is faster than the entry itself (by the margin) at that count and at every larger sample of the
+    bucket; n_hi + 1 where it never is.  Entries of the last bucket, and entries whose shape has no entry in the next
+    bucket, are left alone."""
+    bucket_keys = sorted(make_configs.N_BUCKETS)
+    for key in keys:
+        m, nk, k = (int(t) for t in key.split("_"))
+        lo, hi = make_configs.N_BUCKETS[nk]
+        i = bucket_keys.index(nk)
+        nxt_key = f"{m}_{bucket_keys[i + 1]}_{k}" if i + 1 < len(bucket_keys) else None
+        if nxt_key is None or nxt_key not in param_map:
+            continue
+        own = {f: param_map[key].get(f, 0) for f in make_configs.FIELDS}
+        nxt = {f: param_map[nxt_key].get(f, 0) for f in make_configs.FIELDS}
+        if own == nxt:
+            param_map[key].pop("next_from", None)
+            continue
+        rows = []
+        for n in next_from_samples(nk):
+            ev = Evaluator(m, n, k, iters=max(10, iters // 4) if n >= 256 else iters, warmup=5)
+            t_own, t_nxt = ev(own), ev(nxt)
+            ev.cache.clear()
+            t_own, t_nxt = min(t_own, ev(own)), min(t_nxt, ev(nxt))
+            rows.append((n, t_own, t_nxt))
+            del ev
+        nf = hi + 1
+        for n, t_own, t_nxt in reversed(rows):
+            if t_nxt < margin * t_own:
+                nf = n
+            else:
+                break
+        if rows and nf == rows[0][0]:
+            nf = lo + 1
+        param_map[key]["next_from"] = int(nf)
+        log(f"{key}: next_from {nf}  " + "  ".join(f"n={n}: {a:.2f}/{b:.2f}" for n, a, b in rows))
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--shapes", default="all", help="comma list of shape names or 'all' or 'MxK,...'")
@@ -512,6 +559,10 @@ def main(argv=None):
                     help="an entry of --base is replaced only if the new config takes less than this fraction of its "
                          "time, both timed on this box (0: always replace)")
     ap.add_argument("--eval", default=None, help="JSON config: just time it on the given shapes and exit")
+    ap.add_argument("--next-from", action="store_true",
+                    help="instead of tuning configs: time every entry of --base for the given shapes (all token buckets) "
+                         "against the next bucket's entry at several counts inside its bucket and write the hand-over "
+                         "count (\"next_from\") into --out")
     ap.add_argument("--block-size", default=None,
                     help="comma list of scale-block sizes (64, 128, ...): tune the blockwise GEMM's table "
                          "(param_map_blockwise.json beside --base / --out) instead of the per-row one")
@@ -529,6 +580,18 @@ def main(argv=None):
     if args.block_size:
         args.block_size = [int(t) for t in args.block_size.split(",")]
         return main_blockwise(args, shapes, tokens)
+
+    if args.next_from:
+        with open(args.base) as f:
+            param_map = json.load(f)
+        os.makedirs(os.path.dirname(os.path.abspath(args.out)), exist_ok=True)
+        for name, m, k in shapes:
+            keys = sorted((key for key in param_map if key.split("_")[0] == str(m) and key.split("_")[2] == str(k)),
+                          key=lambda s_: int(s_.split("_")[1]))
+            tune_next_from(param_map, keys, iters=args.iters, log=lambda s_: print(s_, flush=True))
+            with open(args.out, "w") as f:
+                json.dump(param_map, f, indent=1, sort_keys=True)
+        return
 
     if args.eval:
         c0 = json.loads(args.eval)
