@@ -229,6 +229,42 @@ def test_tuner_repair_seeds_and_mutation_stay_valid():
                              token_tiles=1, xcd_swizzle=0), 4096, 16, 4096) is None
 
 
+def test_tuner_hand_over_count_from_timings(monkeypatch):
+    """tune_next_from with a stub in place of the GPU evaluator: the hand-over is the smallest sampled count from
+    which the next bucket's entry wins at every larger sample, the first count inside the bucket if it wins at all
+    of them, none (n_hi + 1) if it loses at the top; identical entries and last-bucket entries are left alone."""
+    from tuna_amd import make_configs as mc, tuner
+
+    own = dict(rows_per_wave=64, waves_m=1, waves_k=8, split_k=4, prefetch=2, x_chunk=1024, token_tiles=1, xcd_swizzle=1)
+    nxt = dict(own, token_tiles=2, x_chunk=512)
+    assert tuner.next_from_samples(64) == [65, 79, 95, 111, 127] and tuner.next_from_samples(1)[0] == 2
+    assert all(mc.N_BUCKETS[nk][0] < n <= mc.N_BUCKETS[nk][1] for nk in mc.N_BUCKETS if nk != 2048 for n in tuner.next_from_samples(nk))
+
+    def run(win_from):
+        class Stub:
+            def __init__(self, m, n, k, iters=0, warmup=0):
+                self.n, self.cache = n, {}
+
+            def __call__(self, c):
+                is_next = c["token_tiles"] == 2
+                return (9.0 if self.n >= win_from else 11.0) if is_next else 10.0
+
+        monkeypatch.setattr(tuner, "Evaluator", Stub)
+        pm = {"4096_64_4096": dict(own, us=1.0), "4096_128_4096": dict(nxt), "4096_2048_4096": dict(own)}
+        tuner.tune_next_from(pm, list(pm), log=lambda s_: None)
+        assert "next_from" not in pm["4096_2048_4096"] and "next_from" not in pm["4096_128_4096"]  # no next entry
+        mc.next_from_of(64, pm["4096_64_4096"])  # in range for the generator
+        return pm["4096_64_4096"]["next_from"]
+
+    assert run(0) == 65        # the next entry wins everywhere: from the first count inside the bucket
+    assert run(95) == 95       # wins from the third sample on
+    assert run(127) == 127
+    assert run(1000) == 128    # never: n_hi + 1
+    pm = {"4096_64_4096": dict(own, next_from=100), "4096_128_4096": dict(own)}
+    tuner.tune_next_from(pm, ["4096_64_4096"], log=lambda s_: None)
+    assert "next_from" not in pm["4096_64_4096"]  # the same config in both buckets: nothing to hand over
+
+
 def test_tuner_small_launch_config_spaces_are_valid_for_both_validators():
     """The exhaustively timed config spaces of the lean and the narrow-row kernel: every member
     passes the Python validator and the library's, narrow-row members report the footprint the
