@@ -678,9 +678,10 @@ def main():
             sweeps["llama70b_80_layers_multi"] = multi_layer_sweep(ops, synth, torch, dev, names, n, layers=80)
         except torch.OutOfMemoryError as e:  # pragma: no cover
             sweeps["llama70b_80_layers_multi"] = {"error": str(e)[:200]}
-        # token sweep on the Llama-70B layer set
+        # token sweep on the Llama-70B layer set: the lower edges of the token buckets (where the table's entries are
+        # tuned) and counts inside them (24, 100, 384: served by the entry their bucket's next_from points to)
         tok = {}
-        for nt in (1, 16, 64, 256, 1024, 4096):
+        for nt in (1, 16, 24, 64, 100, 256, 384, 1024, 4096):
             row = {}
             for nm in names:
                 sm, sk = synth.SHAPES[nm]
