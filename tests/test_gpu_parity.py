@@ -440,6 +440,55 @@ def test_token_sweep_llama70b_layer_set(name, n):
     assert e <= REL_TOL
 
 
+def _entries_for_keys_inside_buckets():
+    import json
+    import os
+
+    from tuna_amd import make_configs
+
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "tuna_amd", "configs", "param_map.json")
+    with open(path) as f:
+        return sorted(key for key in json.load(f) if int(key.split("_")[1]) in make_configs.SUB_KEYS)
+
+
+@pytest.mark.parametrize("key", _entries_for_keys_inside_buckets())
+def test_every_entry_for_the_upper_part_of_a_bucket_matches_the_oracle(key):
+    """Table entries whose key lies inside a token bucket (24, 48, 96, 192, 384: they cover the bucket from that count
+    up): the lookup hands out the entry at its lower edge, and the launch is checked against the oracle on a row
+    subset there, one token below (the bucket's own entry) and at the bucket's last count."""
+    import torch
+
+    from tuna_amd import make_configs, ops
+    from tuna_amd.quantize import nf4_codebook
+    from tuna_amd.synth import make_weights_torch, make_x_torch
+
+    m, n_key, k = (int(t) for t in key.split("_"))
+    dev = torch.device("cuda")
+    q, absmax = make_weights_torch(m, k, seed=n_key, device=dev)
+    code = nf4_codebook(dev)
+    rng = np.random.default_rng(m + n_key)
+    mbs = np.sort(rng.choice(m // 8, size=8, replace=False))
+    rows = (mbs[:, None] * 8 + np.arange(8)[None, :]).ravel()
+    q_sub = q[torch.from_numpy(mbs).to(dev)].cpu().numpy()
+    a_sub = absmax.cpu().numpy()[rows]
+    entry = [cfg for (m_, lo, hi, k_, cfg) in ops.config_table() if (m_, lo, k_) == (m, n_key, k)]
+    assert len(entry) == 1
+    for n in (n_key, n_key - 1, make_configs.N_BUCKETS[make_configs.SUB_KEYS[n_key]][1]):
+        used, hit = ops.select_config(m, n, k)
+        assert hit and (n != n_key or used.to_dict() == entry[0].to_dict())
+        print(f"entry {key} at n={n}: {ops.describe_launch(m, n, k, used)}", flush=True)
+        x = make_x_torch(n, k, seed=n, device=dev)
+        out = torch.full((n, m), float("nan"), dtype=torch.float16, device=dev)
+        ops.matmul(x, q, absmax, code, out, m, n, k)
+        torch.cuda.synchronize()
+        assert not torch.isnan(out).any()
+        ref = O.gemm_f64(q_sub, x.cpu().numpy().view(np.uint16), code.cpu().numpy(), a_sub, len(rows), n, k, mode=O.D1)
+        got = out[:, torch.from_numpy(rows).to(dev)].cpu().numpy().view(np.uint16)
+        e = rel_err(f16_bits_to_f64(got), ref)
+        print(f"  rel_err={e:.3e}", flush=True)
+        assert e <= REL_TOL
+
+
 @pytest.mark.parametrize("name,n", [("mistral_attn_out", 3072), ("mistral_down", 3100), ("llama70b_qkv", 4096)])
 def test_token_counts_far_into_the_last_bucket_take_the_256_x_256_tile(name, n):
     """The last bucket of the table is open-ended and tuned at 2048 tokens; from 3072 tokens a shape of fewer than

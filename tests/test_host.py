@@ -76,17 +76,22 @@ def test_select_config_is_host_only_and_every_table_entry_validates():
         pm = json.load(f)
     assert len(table) == len(pm) == len(next_from)
     for (m, lo, hi, k, cfg), nf in zip(table, next_from):
-        key = f"{m}_{make_configs.bucket_of(lo)}_{k}"
-        assert key in pm
+        # an entry's key is the lower edge of its range: a bucket key, or a key inside a bucket (which ends the
+        # range of the bucket's own entry one token earlier)
+        present = make_configs.keys_of_shape(pm, m, k)
+        n_key = make_configs.key_of(lo, present)
+        key = f"{m}_{n_key}_{k}"
+        assert key in pm and (lo, hi) == make_configs.key_range(n_key, present)
+        assert n_key == (lo if lo in make_configs.SUB_KEYS else make_configs.bucket_of(lo))
         assert cfg.to_dict() == {f: pm[key][f] for f in cfg.FIELDS}
-        assert nf == make_configs.next_from_of(make_configs.bucket_of(lo), pm[key]) and lo < nf <= hi + 1
+        assert nf == make_configs.next_from_of(n_key, pm[key], present) and lo < nf <= hi + 1
         for n in sorted({lo, hi, min(nf, hi), max(nf - 1, lo)}):
             ops.validate_config(m, n, k, cfg)                      # the C side accepts it
             got, hit = ops.select_config(m, n, k)
             assert hit
             # entries are tuned at their bucket's lower edge: counts from the entry's next_from on take the next
             # bucket's entry (fewer passes over the weights)
-            nxt = pm.get(f"{m}_{make_configs.bucket_of(hi + 1)}_{k}") if n >= nf and hi < 128000 else None
+            nxt = pm.get(f"{m}_{make_configs.key_of(hi + 1, present)}_{k}") if n >= nf and hi < 128000 else None
             if n >= 3072 and m < 24576 and k % 64 == 0:
                 # far into the open-ended last bucket (tuned at 2048 tokens): the 256 x 256 many-token tile
                 assert (got.lds_tile_rows, got.token_tiles, got.split_k, got.rows_per_wave) == (256, 16, 1, 64)
@@ -100,7 +105,7 @@ def test_select_config_is_host_only_and_every_table_entry_validates():
                     # the next entry (a different config) was passed over only because it cannot run n tokens
                     with pytest.raises(ops.TunaError):
                         ops.validate_config(m, n, k, ops.GemmConfig.from_dict({f: nxt[f] for f in cfg.FIELDS}))
-        make_configs.validate(m, make_configs.bucket_of(lo), k, cfg.to_dict())  # and the generator's twin
+        make_configs.validate(m, n_key, k, cfg.to_dict())  # and the generator's twin
         lds, ws = ops.config_footprint(m, lo, k, cfg)
         assert lds == make_configs.lds_bytes(cfg.to_dict()) and lds <= 160 * 1024
 
@@ -127,6 +132,14 @@ def test_token_buckets_follow_the_reference_dispatcher():
         assert mc.bucket_of(n) == want
     with pytest.raises(ValueError):
         mc.bucket_of(128001)
+    # keys inside a bucket (this table's own): m_<sub>_k covers sub .. the bucket's upper edge, and the bucket's entry
+    # then ends at sub - 1; shapes without such an entry keep the reference's ranges
+    assert mc.SUB_KEYS == {24: 16, 48: 32, 96: 64, 192: 128, 384: 256}
+    assert mc.key_range(256, [1, 16, 256, 512]) == (256, 511) and mc.key_range(256, [256, 384, 512]) == (256, 383)
+    assert mc.key_range(384, [256, 384, 512]) == (384, 511)
+    assert mc.key_of(383, [256, 384]) == 256 and mc.key_of(384, [256, 384]) == 384 and mc.key_of(400, [256]) == 256
+    assert mc.default_next_from(256, [256, 384]) == 384 and mc.default_next_from(384, [256, 384]) == 512
+    assert mc.default_next_from(64, [64]) == 65 and mc.default_next_from(64, [64, 96]) == 96
 
 
 def test_invalid_configs_are_rejected_by_both_validators():
@@ -169,6 +182,18 @@ def test_generator_output_and_its_refusal_of_inconsistent_entries(tmp_path):
     for bad in (16, 33, 0):
         with pytest.raises(ValueError, match="next_from"):
             mc.generate({"4096_16_4096": dict(pm["4096_16_4096"], next_from=bad)})
+    # a key inside a bucket: its entry takes the upper part of the bucket, the bucket's own entry the lower part; it
+    # needs the bucket's entry, and no other key is accepted
+    e16 = pm["4096_16_4096"]
+    text = mc.generate({"4096_16_4096": e16, "4096_24_4096": dict(e16, xcd_swizzle=0)})
+    assert "{4096, 16, 23, 4096, 24, {64, 1, 8, 4, 2, 1024, 1, 1," in text and "{4096, 24, 31, 4096, 32, {64, 1, 8, 4, 2, 1024, 1, 0," in text
+    assert "{4096, 16, 23, 4096, 20, {" in mc.generate({"4096_16_4096": dict(e16, next_from=20), "4096_24_4096": e16})
+    with pytest.raises(ValueError, match="next_from"):
+        mc.generate({"4096_16_4096": dict(e16, next_from=25), "4096_24_4096": e16})
+    with pytest.raises(ValueError, match="needs the bucket's own entry"):
+        mc.generate({"4096_24_4096": e16})
+    with pytest.raises(ValueError, match="not a bucket key"):
+        mc.generate({"4096_20_4096": e16})
     # the checked-in table is what the generator produces from the checked-in json
     with open(os.path.join(ROOT, "tuna_amd", "configs", "param_map.json")) as f:
         real = json.load(f)
@@ -237,7 +262,7 @@ def test_tuner_hand_over_count_from_timings(monkeypatch):
 
     own = dict(rows_per_wave=64, waves_m=1, waves_k=8, split_k=4, prefetch=2, x_chunk=1024, token_tiles=1, xcd_swizzle=1)
     nxt = dict(own, token_tiles=2, x_chunk=512)
-    assert tuner.next_from_samples(64) == [65, 79, 95, 111, 127] and tuner.next_from_samples(1)[0] == 2
+    assert tuner.next_from_samples(64) == [65, 79, 81, 95, 97, 111, 113, 127] and tuner.next_from_samples(1)[0] == 2
     assert all(mc.N_BUCKETS[nk][0] < n <= mc.N_BUCKETS[nk][1] for nk in mc.N_BUCKETS if nk != 2048 for n in tuner.next_from_samples(nk))
 
     def run(win_from):
@@ -263,6 +288,14 @@ def test_tuner_hand_over_count_from_timings(monkeypatch):
     pm = {"4096_64_4096": dict(own, next_from=100), "4096_128_4096": dict(own)}
     tuner.tune_next_from(pm, ["4096_64_4096"], log=lambda s_: None)
     assert "next_from" not in pm["4096_64_4096"]  # the same config in both buckets: nothing to hand over
+    # with an entry for the upper part of the bucket (key 96): the bucket's entry is sampled in 65..95 and hands over
+    # to that entry, which is sampled in 97..127 and hands over to the next bucket's
+    assert tuner.next_from_samples(64, [64, 96, 128]) == [65, 71, 79, 81, 87, 95]
+    assert tuner.next_from_samples(96, [64, 96, 128]) == [97, 103, 111, 113, 119, 127]
+    pm = {"4096_64_4096": dict(own), "4096_96_4096": dict(nxt), "4096_128_4096": dict(own)}
+    tuner.tune_next_from(pm, list(pm), log=lambda s_: None)   # (the stub of the last run: two token tiles always lose)
+    assert pm["4096_64_4096"]["next_from"] == 96 and pm["4096_96_4096"]["next_from"] == 97
+    mc.generate(pm)
 
 
 def test_tuner_small_launch_config_spaces_are_valid_for_both_validators():
@@ -320,7 +353,10 @@ def test_tuner_small_launch_config_spaces_are_valid_for_both_validators():
         big = tuner.mid_space(57344, n_key, 8192)
         assert big and all(mc.mid_applies(57344, 8192, c) for c in big)
         # 128 and 256 tokens: also passes of 32 and 64 tokens (they share the weights when they all fit the device)
-        assert {c["token_tiles"] for c in big} == ({8, 4, 2} if n_key <= 256 else {8})
+        assert {c["token_tiles"] for c in big} == ({8, 4, 2} if n_key <= 256 else {8, 4})
+    # 32 and 64 tokens: also chunks of fewer token tiles than the count needs, side by side
+    assert {c["token_tiles"] for c in tuner.mid_space(10240, 32, 8192)} == {2, 1}
+    assert {c["token_tiles"] for c in tuner.mid_space(10240, 64, 8192)} == {4, 2, 1}
     # packed weights staged through LDS (lds_tile_rows = -1): offered for 16-wave launches with one token tile, valid
     # for both validators exactly where the twin exists
     sp16 = tuner.mid_space(229376, 16, 4096)

@@ -35,6 +35,12 @@ N_BUCKETS = {
     2048: (1025, 128000),
 }
 
+# Optional keys inside a bucket (no counterpart in the reference's table): an entry m_<sub>_k covers the token
+# counts from <sub> to the upper edge of the bucket it sits in, and that bucket's own entry then ends at <sub> - 1.
+# An entry is tuned at the lower edge of its range, and the best launch at 1.5 times that count is often another
+# one (another number of token chunks side by side, another tile of the many-token kernel).
+SUB_KEYS = {24: 16, 48: 32, 96: 64, 192: 128, 384: 256}
+
 FIELDS = ("rows_per_wave", "waves_m", "waves_k", "split_k", "prefetch", "x_chunk",
           "token_tiles", "xcd_swizzle", "k_stagger", "lds_tile_rows")
 
@@ -86,6 +92,28 @@ def bucket_of(n: int):
     raise ValueError(f"n={n} outside every token bucket")
 
 
+def key_range(n_key: int, keys_present=()) -> tuple:
+    """The token counts [lo, hi] that the entry under key `n_key` covers when the entries of its (m, k) have the keys
+    `keys_present`: a bucket's range, cut short by a sub key inside it where there is one."""
+    if n_key in SUB_KEYS:
+        return n_key, N_BUCKETS[SUB_KEYS[n_key]][1]
+    lo, hi = N_BUCKETS[n_key]
+    subs = [s for s, parent in SUB_KEYS.items() if parent == n_key and s in keys_present]
+    return lo, (min(subs) - 1 if subs else hi)
+
+
+def key_of(n: int, keys_present=()) -> int:
+    """Token count -> the key of the entry that covers it, among the keys `keys_present` of one (m, k)."""
+    nk = bucket_of(n)
+    subs = [s for s, parent in SUB_KEYS.items() if parent == nk and s in keys_present and n >= s]
+    return max(subs) if subs else nk
+
+
+def keys_of_shape(param_map: dict, m: int, k: int) -> list:
+    """The token keys of the entries that `param_map` holds for (m, k), ascending."""
+    return sorted(int(key.split("_")[1]) for key in param_map if key.split("_")[0] == str(m) and key.split("_")[2] == str(k))
+
+
 def is_narrow(c: dict) -> bool:
     """The config selects the narrow-row kernel: rows_per_wave 16, 24 or 32, or 64 with waves_m 0."""
     return c.get("lds_tile_rows", 0) == 0 and (c["rows_per_wave"] in (16, 24, 32) or (c["rows_per_wave"] == 64 and c["waves_m"] == 0))
@@ -99,8 +127,8 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
         raise ValueError(f"missing fields {missing}")
     if m <= 0 or k <= 0 or m % 8 or k % 8:
         raise ValueError("m and k must be positive multiples of 8")
-    if n_key not in N_BUCKETS:
-        raise ValueError(f"n={n_key} is not a bucket key {sorted(N_BUCKETS)}")
+    if n_key not in N_BUCKETS and n_key not in SUB_KEYS:
+        raise ValueError(f"n={n_key} is not a bucket key {sorted(N_BUCKETS)} nor a key inside a bucket {sorted(SUB_KEYS)}")
     if c["lds_tile_rows"] not in (0, -1, 64, 128, 256):
         raise ValueError("lds_tile_rows must be 0, -1 (packed weights through LDS), 64, 128 or 256")
     if c["lds_tile_rows"] > 0:
@@ -322,22 +350,26 @@ const int kBlockwiseTableSize = {len(rows)};
 """
 
 
-def default_next_from(n_key: int) -> int:
+def default_next_from(n_key: int, keys_present=()) -> int:
     """Where an entry without a tuned "next_from" hands over to the next bucket's entry: entries are tuned at the
     lower edge of their bucket, and a count inside one of the buckets 16.., 32.., 64.., 128.. takes two passes over
     the weights with such an entry but one with the next bucket's (from 10 tokens in the first bucket); the other
-    buckets keep their entry throughout (n_hi + 1: never)."""
-    lo, hi = N_BUCKETS[n_key]
+    buckets keep their entry throughout (n_hi + 1: never)
+    (with keys inside buckets: `keys_present`, the keys of the entry's (m, k), gives the range; an entry whose range
+    a sub key starts or ends keeps its entry throughout)"""
+    lo, hi = key_range(n_key, keys_present)
+    if n_key in SUB_KEYS or hi != N_BUCKETS[n_key][1]:
+        return hi + 1
     if lo == 1:
         return 10
     return lo + 1 if 16 <= lo <= 128 else hi + 1
 
 
-def next_from_of(n_key: int, c: dict) -> int:
-    """The entry's "next_from" (the token count from which the lookup hands out the next bucket's entry instead;
-    written by the tuner, which times both entries inside the bucket), checked: n_lo < next_from <= n_hi + 1."""
-    lo, hi = N_BUCKETS[n_key]
-    nf = int(c.get("next_from", default_next_from(n_key)))
+def next_from_of(n_key: int, c: dict, keys_present=()) -> int:
+    """The entry's "next_from" (the token count from which the lookup hands out the next entry of its (m, k) instead;
+    written by the tuner, which times both entries inside the range), checked: n_lo < next_from <= n_hi + 1."""
+    lo, hi = key_range(n_key, keys_present)
+    nf = int(c.get("next_from", default_next_from(n_key, keys_present)))
     if not lo < nf <= hi + 1:
         raise ValueError(f"next_from={nf} outside {lo + 1}..{hi + 1}")
     return nf
@@ -348,12 +380,15 @@ def generate(param_map: dict) -> str:
     for key in sorted(param_map, key=lambda s: tuple(int(t) for t in s.split("_"))):
         m, n, k = (int(t) for t in key.split("_"))
         c = param_map[key]
+        present = keys_of_shape(param_map, m, k)
         try:
             validate(m, n, k, c)
-            nf = next_from_of(n, c)
+            if n in SUB_KEYS and SUB_KEYS[n] not in present:
+                raise ValueError(f"a key inside a bucket needs the bucket's own entry ({m}_{SUB_KEYS[n]}_{k})")
+            nf = next_from_of(n, c, present)
         except ValueError as e:
             raise ValueError(f"param_map entry {key}: {e}") from None
-        lo, hi = N_BUCKETS[n]
+        lo, hi = key_range(n, present)
         vals = ", ".join(str(int(c.get(f, 0))) for f in FIELDS)
         rows.append(f"    {{{m}, {lo}, {hi}, {k}, {nf}, {{{vals}}}}},  // {key}")
     body = "\n".join(rows)

@@ -137,7 +137,7 @@ def lean_space(m: int, n_key: int, k: int):
     token tile, no stagger, a power-of-two split, whole ring turns, all tiles resident at once.
     Small enough to time exhaustively."""
     lo, _ = make_configs.N_BUCKETS[n_key]
-    if lo > 32 or k % 32:
+    if lo > 64 or k % 32:
         return []
     steps = k // 32
     out = []
@@ -174,14 +174,15 @@ def mid_space(m: int, n_key: int, k: int):
     out = []
     # tuned at the bucket's lower edge; from 128 tokens on, passes of eight token tiles (on the
     # largest shapes they beat the many-token kernel at every token count)
-    # (128 and 256 tokens: also passes of 32 and 64 tokens, which run side by side and share the
-    # weights when they all fit the device - the mid-size shapes prefer them)
-    for tt in ((1,) if lo <= 16 else (2,) if lo <= 32 else (4,) if lo <= 64 else (8, 4, 2) if lo <= 256 else (8,)):
+    # (from 32 tokens on also chunks of fewer token tiles than the count needs: they run side by side and share
+    # the weights when they all fit the device, which fills it without a split of k and its hand-over - the
+    # mid-size shapes prefer them: 10240 x 8192 at 384 tokens 112 -> 82 us with six chunks of four token tiles)
+    for tt in ((1,) if lo <= 16 else (2, 1) if lo <= 32 else (4, 2, 1) if lo <= 64 else (8, 4, 2) if lo <= 256 else (8, 4)):
         for wm in range(1, 17):
             for wk in (1, 2, 4, 8):
                 if m % (64 * wm) or wm * wk > 16 or wm * wk < 4:
                     continue
-                if tt == 1 and (m // (64 * wm) < 100 or wm * wk < 8):
+                if tt == 1 and ((m // (64 * wm)) * -(-lo // 16) < 100 or wm * wk < 8):
                     continue        # one token tile: only launches that fill the device unsplit (others: lean, narrow-row)
                 for pf in (2, 4, 8):
                     for xc in (128, 256, 512, 1024, 2048):
@@ -305,7 +306,7 @@ def tune_shape(m, n, k, generations=6, population=24, seed=0, log=print, max_see
         return json.loads(scored[0][1]), scored[0][0]
     pool = seeds(m, n_key, k)
     rng.shuffle(pool)
-    pool = pool[:max_seed_evals] + lean_space(m, n_key, k) + mid_space(m, n_key, k) + derived
+    pool = pool[:max_seed_evals] + lean_space(m, n_key, k) + mid_space(m, n_key, k) + tiled_space(m, n_key, k) + derived
     # the winners of the other token buckets of this (m, k), where they are valid here: a config tuned
     # for 16 tokens also runs one token, and is sometimes what the bucket should have
     pool += [c for c in (repair(dict(e), m, n_key, k) for e in extra) if c is not None]
@@ -496,35 +497,41 @@ def main_blockwise(args, shapes, tokens):
                     json.dump(param_map, f, indent=1, sort_keys=True)
 
 
-def next_from_samples(n_key: int):
-    """Token counts inside a bucket at which its entry is timed against the next bucket's."""
-    lo, hi = make_configs.N_BUCKETS[n_key]
+def next_from_samples(n_key: int, keys_present=()):
+    """Token counts inside an entry's range at which the entry is timed against the next one of its shape."""
+    lo, hi = make_configs.key_range(n_key, keys_present)
     if lo == 1:
         return [2, 4, 6, 8, 10, 12, 15]
     span = hi - lo
-    return sorted({lo + 1, lo + span // 4, lo + span // 2, lo + 3 * span // 4, hi})
+    # the quarter points, and the first count past every multiple of 16 (32 in the wide ranges) tokens: a launch in
+    # chunks of token tiles gains a chunk there, which is where one entry overtakes the other
+    step = 16 if span <= 128 else 32
+    while span // step > 8:
+        step *= 2
+    edges = {v + 1 for v in range((lo // step + 1) * step, hi, step)}
+    return sorted({lo + 1, lo + span // 4, lo + span // 2, lo + 3 * span // 4, hi} | edges)
 
 
 def tune_next_from(param_map, keys, iters=40, margin=0.98, log=print):
     """Writes "next_from" into the entries `keys` of param_map: the smallest sampled token count from which the next
-    bucket's entry is faster than the entry itself (by the margin) at that count and at every larger sample of the
-    bucket; n_hi + 1 where it never is.  Entries of the last bucket, and entries whose shape has no entry in the next
-    bucket, are left alone."""
-    bucket_keys = sorted(make_configs.N_BUCKETS)
+    entry of the shape is faster than the entry itself (by the margin) at that count and at every larger sample of
+    the entry's range; n_hi + 1 where it never is.  The last entry of a shape, and an entry whose range is not
+    followed directly by another entry's, are left alone."""
     for key in keys:
         m, nk, k = (int(t) for t in key.split("_"))
-        lo, hi = make_configs.N_BUCKETS[nk]
-        i = bucket_keys.index(nk)
-        nxt_key = f"{m}_{bucket_keys[i + 1]}_{k}" if i + 1 < len(bucket_keys) else None
-        if nxt_key is None or nxt_key not in param_map:
+        present = make_configs.keys_of_shape(param_map, m, k)
+        lo, hi = make_configs.key_range(nk, present)
+        later = [p for p in present if p > nk]
+        if not later or make_configs.key_range(min(later), present)[0] != hi + 1:
             continue
+        nxt_key = f"{m}_{min(later)}_{k}"
         own = {f: param_map[key].get(f, 0) for f in make_configs.FIELDS}
         nxt = {f: param_map[nxt_key].get(f, 0) for f in make_configs.FIELDS}
         if own == nxt:
             param_map[key].pop("next_from", None)
             continue
         rows = []
-        for n in next_from_samples(nk):
+        for n in next_from_samples(nk, present):
             ev = Evaluator(m, n, k, iters=max(10, iters // 4) if n >= 256 else iters, warmup=5)
             t_own, t_nxt = ev(own), ev(nxt)
             ev.cache.clear()
@@ -559,6 +566,10 @@ def main(argv=None):
                     help="an entry of --base is replaced only if the new config takes less than this fraction of its "
                          "time, both timed on this box (0: always replace)")
     ap.add_argument("--eval", default=None, help="JSON config: just time it on the given shapes and exit")
+    ap.add_argument("--sub-keys", action="store_true",
+                    help="token counts that are keys inside a bucket (24, 48, 96, 192, 384) get an entry of their own "
+                         "for the upper part of the bucket, where it beats the lookup without it by --sub-key-margin")
+    ap.add_argument("--sub-key-margin", type=float, default=0.95)
     ap.add_argument("--next-from", action="store_true",
                     help="instead of tuning configs: time every entry of --base for the given shapes (all token buckets) "
                          "against the next bucket's entry at several counts inside its bucket and write the hand-over "
@@ -620,6 +631,22 @@ def main(argv=None):
                                   log=lambda s: print(s, flush=True), max_seed_evals=args.max_seed_evals,
                                   iters=args.iters, extra=others)
             key = f"{m}_{make_configs.bucket_of(n)}_{k}"
+            if args.sub_keys and n in make_configs.SUB_KEYS:
+                # an entry of its own for the upper part of the bucket: only where it beats what the lookup hands
+                # out at this count without it (the bucket's entry, or the next bucket's) by the margin
+                key = f"{m}_{n}_{k}"
+                if key not in param_map:
+                    from . import ops
+                    ev = Evaluator(m, n, k, iters=max(100, 2 * args.iters), warmup=15)
+                    c_sel = ops.select_config(m, n, k)[0].to_dict()
+                    t_old, t_new = ev(c_sel), ev(dict(best))
+                    ev.cache.clear()
+                    t_old, t_new = min(t_old, ev(c_sel)), min(t_new, ev(dict(best)))
+                    print(f"  lookup without the entry {t_old:.2f} us, new config {t_new:.2f} us on this box", flush=True)
+                    if not t_new < args.sub_key_margin * t_old:
+                        print(f"  -> {key}: no entry", flush=True)
+                        continue
+                    us = t_new
             old = param_map.get(key)
             if old is not None and args.replace_margin > 0:
                 # Boxes differ by several per cent, so a time recorded with the existing entry says
