@@ -95,7 +95,7 @@ typedef struct tuna_gemm_config {
                               (tiles of at least 32 tokens), any other value with 16 x 16 x 32
                               (the reference's counterpart: its MMA shapes, kernel.cu:411-465).
                               256 rows x 256 tokens is a kernel of its own (one wave per SIMD, a
-                              wave owns 128 x 128) and needs k to be a multiple of 64 */
+                              wave owns 128 x 128) */
 } tuna_gemm_config;
 
 int tuna_version(void);

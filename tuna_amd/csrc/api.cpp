@@ -222,8 +222,6 @@ static int plan_tiled(int m, int n, int k, const tuna_gemm_config &c, int decode
     if (!tiled_variant_exists(c.lds_tile_rows, tile_tokens, mfma32))
         return fail(TUNA_ERR_UNSUPPORTED, "no many-token kernel for a %d x %d tile (rows x tokens)%s", c.lds_tile_rows, tile_tokens,
                     mfma32 ? " with 32 x 32 MFMA tiles" : "");
-    if (c.lds_tile_rows == 256 && tile_tokens == 256 && k % 64 != 0)
-        return fail(TUNA_ERR_UNSUPPORTED, "the 256 x 256 many-token tile needs k a multiple of 64");
     const int steps = ceil_div(k, 64);
     if (c.split_k < 1 || c.split_k > steps)
         return fail(TUNA_ERR_UNSUPPORTED, "split_k=%d must be in 1..%d for the many-token kernel", c.split_k, steps);
@@ -525,7 +523,7 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         c.token_tiles = 4;
         if (config_runs(m, n, k, c)) return c;
     }
-    if (n >= 768 && k % 64 == 0) {
+    if (n >= 768) {
         // very many tokens: the 256 x 256 tile (one wave per SIMD) where it fills the device - from about 150
         // tiles, or from 90 with the k range split in two when k is 8192 or more (with k = 4096 the split loses:
         // 6144 x 4096 at 800 tokens 103 us against 63 of the 128-token tiles).  Measured on
@@ -605,7 +603,7 @@ static int select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_t
         // takes the 256 x 256 many-token tile whatever its entry says, when that tile fills the device: measured on
         // six benchmark shapes at 3072..8192 tokens it equals or beats every other entry there (4096 x 4096 at 8192
         // tokens 336 -> 255 us, 4096 x 14336 at 4096 tokens 469 -> 392 us, 10240 x 8192 at 8192 tokens 1582 -> 1200 us).
-        if (n >= 3072 && m < 24576 && k % 64 == 0 && !(cfg->lds_tile_rows == 256 && cfg->token_tiles == 16) &&
+        if (n >= 3072 && m < 24576 && !(cfg->lds_tile_rows == 256 && cfg->token_tiles == 16) &&
             (long long)ceil_div(m, 256) * ceil_div(n, 256) >= 150) {
             memset(cfg, 0, sizeof(*cfg));
             cfg->rows_per_wave = 64, cfg->waves_m = 1, cfg->waves_k = 1, cfg->prefetch = 2, cfg->x_chunk = 64;

@@ -24,7 +24,11 @@
 //     contiguous bytes of a block row's k-step; weights and activations come through buffer loads (descriptor in
 //     scalar registers, one 32-bit offset per lane, the k-step as a scalar offset): no 64-bit address
 //     arithmetic in the loop, which a single wave per SIMD would pay for in MFMA issue slots.
-// k must be a multiple of 64; the host checks.
+// KTAIL: k is any multiple of 8.  The last k-step is then partly beyond k: a thread whose 8-k slot of that step
+// lies beyond k loads the last slot inside k instead (no access leaves a row, whatever the descriptor's range
+// check covers), and the activations of those slots are stored as zeros, so the products vanish whatever the
+// weight slots hold (finite values: table entries times the row's own scale).  k a multiple of 64 runs the
+// variant without the selects.
 //
 // Decode and rounding are those of the other kernels (bit-identical to kernel.cu:2178-2192); the sums are the
 // same products in the same order as the variants of gemm_tiled.hip with the same MFMA shape.
@@ -39,7 +43,7 @@ constexpr int kWideBuf = (kWideRows + kWideTokens) * 128;
 
 typedef float wide_f32x16 __attribute__((ext_vector_type(16)));
 
-template <int NSETS, bool M32>
+template <int NSETS, bool M32, bool KTAIL>
 __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(const TiledArgs a)
 {
     static_assert(NSETS == 2 || NSETS == 4, "register sets of packed weights");
@@ -96,6 +100,11 @@ __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(const TiledA
         x_off[i] = ((uint32_t)(min(tok, a.n - 1) - tok_base) * (uint32_t)a.k + (uint32_t)(tid & 7) * 8u) * 2u;
     }
     unsigned char *x_dst = x_tile + (tid >> 3) * 128 + (((tid & 7) ^ ((tid >> 3) & 7)) << 4);  // piece i: + i * 4096
+    // KTAIL: the thread's slot of k-step s lies inside k while 64 s < x_k_left; in the last step a slot beyond k
+    // steps back to the last one inside (in bytes: 32 per slot of packed weights, 16 per slot of activations)
+    const int x_k_left = a.k - (tid & 7) * 8;
+    const int slots_back = KTAIL ? max(0, (tid & 7) - (((a.k >> 3) - 1) & 7)) : 0;
+    const uint32_t a_back = (uint32_t)slots_back * 32u, x_back = (uint32_t)slots_back * 16u;
 
     u32x4 wq[NSETS][2];
     u32x4 xr[XSETS][8];
@@ -109,11 +118,16 @@ __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(const TiledA
         (int)(uint32_t)min(x_rest, (size_t)0xffffffffu), 0x00020000);
 #define TUNA_WIDE_LOAD(set, s)                                                                  \
     {                                                                                          \
-        wq[set][0] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, (int)a_off, (s) * 256, 0);  \
-        wq[set][1] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, (int)a_off + 16, (s) * 256, 0); \
+        const uint32_t o_ = KTAIL && (s) == s_last ? a_off - a_back : a_off;                   \
+        wq[set][0] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, (int)o_, (s) * 256, 0);     \
+        wq[set][1] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, (int)o_ + 16, (s) * 256, 0); \
     }
 #define TUNA_WIDE_LOAD_X(set, s)                                                                \
-    _Pragma("unroll") for (int i = 0; i < 8; ++i) xr[set][i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)x_off[i], (s) * 128, 0);
+    {                                                                                          \
+        const uint32_t b_ = KTAIL && (s) == s_last ? x_back : 0u;                              \
+        _Pragma("unroll") for (int i = 0; i < 8; ++i)                                          \
+            xr[set][i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)(x_off[i] - b_), (s) * 128, 0); \
+    }
 
     const int s0 = blockIdx.z * a.steps_per_split;
     const int s1 = min(a.steps_total, s0 + a.steps_per_split);
@@ -211,7 +225,13 @@ __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(const TiledA
     }
     // ... and activation piece i into activation tile `buf`.
 #define TUNA_WIDE_XSTAGE(set, i, buf, s)                                                         \
-    *reinterpret_cast<u32x4 *>(x_dst + (buf) * BUF + (i) * 4096) = xr[set][i];
+    {                                                                                          \
+        u32x4 v_ = xr[set][i];                                                                 \
+        if constexpr (KTAIL) {                                                                 \
+            if ((s) * 64 >= x_k_left) v_ = u32x4{0u, 0u, 0u, 0u};                              \
+        }                                                                                      \
+        *reinterpret_cast<u32x4 *>(x_dst + (buf) * BUF + (i) * 4096) = v_;                     \
+    }
     // Iteration `it` (k-step `step`) of a tile: its tiles are complete in buffer it & 1, the fragments of its
     // first quarter in fr[0], the table reads of dwords 0..3 of step + 1 in lt.  Side work between the MFMAs:
     //   quarter 0: fragments of quarter 1; weights 0..3 of step + 1 scaled and stored into the other buffer, each
@@ -431,16 +451,18 @@ __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(const TiledA
 
 size_t wide_lds_bytes() { return (size_t)kWideLutBytes + 2 * (size_t)kWideBuf; }
 
-static OptInFlag g_wide_attr[16][2];
+static OptInFlag g_wide_attr[16][4];
 
 hipError_t launch_gemm_wide(const TiledArgs &args, bool mfma32, hipStream_t stream)
 {
-    const auto fn = mfma32 ? gemm_wide_kernel<2, true> : gemm_wide_kernel<2, false>;
+    const bool ktail = args.k % 64 != 0;
+    const auto fn = ktail ? (mfma32 ? gemm_wide_kernel<2, true, true> : gemm_wide_kernel<2, false, true>)
+                          : (mfma32 ? gemm_wide_kernel<2, true, false> : gemm_wide_kernel<2, false, false>);
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
-    if ((e = ensure_lds_opt_in(g_wide_attr[dev][mfma32], reinterpret_cast<const void *>(fn))) != hipSuccess) return e;
+    if ((e = ensure_lds_opt_in(g_wide_attr[dev][2 * ktail + mfma32], reinterpret_cast<const void *>(fn))) != hipSuccess) return e;
     TiledArgs a = args;
     a.row_tiles = ceil_div_i(args.m, kWideRows);
     a.tok_tiles = ceil_div_i(args.n, kWideTokens);

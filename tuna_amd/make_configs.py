@@ -75,7 +75,7 @@ NARROW_VARIANTS = (
     | {(24, 8, 2, 1), (24, 8, 4, 1), (24, 8, 8, 1), (24, 16, 2, 1), (24, 16, 4, 1)})
 
 # (rows, tokens) tiles of the many-token kernels; must match kTiled in csrc/gemm_tiled.hip, plus the 256 x 256 tile
-# of csrc/gemm_wide.hip (one wave per SIMD; k a multiple of 64)
+# of csrc/gemm_wide.hip (one wave per SIMD)
 TILED_VARIANTS = {(256, 256), (256, 128), (256, 64), (128, 256), (128, 128), (64, 256), (64, 128)}
 WIDE_LUT_BYTES = 256 * 32 * 4
 
@@ -139,8 +139,6 @@ def validate(m: int, n_key: int, k: int, c: dict) -> None:
             raise ValueError("the 64 x 128 tile has no 32 x 32 MFMA variant (one 16-token tile per wave)")
         if not 1 <= c["split_k"] <= -(-k // 64):
             raise ValueError("split_k of the many-token kernel must be in 1..ceil(k/64)")
-        if (c["lds_tile_rows"], 16 * c["token_tiles"]) == (256, 256) and k % 64:
-            raise ValueError("the 256 x 256 many-token tile needs k a multiple of 64")
         return
     if is_narrow(c):
         # narrow-row kernel: one workgroup per 16, 32 or 64 rows, all waves along k, no split
