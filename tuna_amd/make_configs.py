@@ -10,7 +10,9 @@ param_map.json values into a C++ template to produce configs.cu.  Differences:
   reference emits inconsistent entries such as gemm_229376_4096_16, whose
   warp_count_m * warp_count_n * 32 != tpb, param_map.json:4034-4069);
 * keys are "<m>_<n>_<k>" like the reference's (make_configs.py:111-115), n being the
-  lower edge of a token bucket; bucket edges follow kernel.cu:3022-3155.
+  lower edge of a token bucket; bucket edges follow kernel.cu:3022-3155.  In addition an entry may sit
+  under one of the keys of SUB_KEYS (1.5 times a bucket's lower edge): it covers the bucket from that token
+  count up, and the bucket's own entry the counts below.
 
 Usage:  python -m tuna_amd.make_configs [param_map.json] [config_table.cpp]
 """
