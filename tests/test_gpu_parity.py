@@ -489,9 +489,9 @@ def test_every_entry_for_the_upper_part_of_a_bucket_matches_the_oracle(key):
         assert e <= REL_TOL
 
 
-@pytest.mark.parametrize("name,n", [("mistral_attn_out", 3072), ("mistral_down", 3100), ("llama70b_qkv", 4096)])
+@pytest.mark.parametrize("name,n", [("mistral_attn_out", 3072), ("mistral_down", 3100), ("llama70b_qkv", 4096), ("llama70b_qkv", 2560)])
 def test_token_counts_far_into_the_last_bucket_take_the_256_x_256_tile(name, n):
-    """The last bucket of the table is open-ended and tuned at 2048 tokens; from 3072 tokens a shape of fewer than
+    """The last bucket of the table is open-ended and tuned at 2048 tokens; from 2560 tokens a shape of fewer than
     24576 rows runs the 256 x 256 many-token tile through the plain entry point.  Row-subset check against the oracle."""
     import torch
 
@@ -570,11 +570,15 @@ def test_derived_configs_for_untuned_shapes_up_to_16_tokens(m, k, n, kernel):
 @pytest.mark.parametrize("m,k,n,kernel", [(8192, 3072, 64, "gemm_narrow_kernel"), (5120, 5120, 20, "gemm_narrow_kernel"),
                                            (4096, 12288, 32, "gemm_lean_kernel"), (12288, 4096, 64, "weights through LDS"),
                                            (37888, 3584, 40, "weights through LDS"), (3072, 8192, 128, "weights through LDS"),
-                                           (5120, 5120, 200, "gemm_mid_kernel"), (12288, 4096, 300, "128 rows x 256 tokens"),
-                                           (3072, 8192, 512, "128 rows x 128 tokens")])
+                                           (5120, 5120, 200, "gemm_mid_kernel"), (12288, 4096, 300, "TT=4"),
+                                           (3072, 8192, 512, "TT=2"), (20480, 5120, 64, "TT=2"),
+                                           (18432, 6144, 256, "128 rows x 256 tokens"), (2048, 2048, 384, "TT=2"),
+                                           (20480, 5120, 384, "TT=8"), (16384, 8192, 640, "gemm_wide_kernel"),
+                                           (2560, 6912, 300, "gemm_mid_kernel"), (22016, 4096, 704, "128 rows x 256 tokens")])
 def test_derived_configs_for_untuned_shapes_from_17_to_512_tokens(m, k, n, kernel):
-    """The same for 17..512 tokens: narrow-row and lean workgroups with the token passes side by side in the grid,
-    the streaming kernel with 16, 32 or 64 tokens per pass, the many-token tiles."""
+    """The same for 17 tokens and more: narrow-row and lean workgroups with the token passes side by side in the grid,
+    the streaming kernel with 16, 32 or 64 tokens per pass, and from 256 tokens the tile that a cost model of the
+    grid picks (chunks of 32 ... 128 tokens of the streaming kernel side by side, or a many-token tile)."""
     _check_derived(m, k, n, kernel)
 
 
@@ -613,11 +617,11 @@ def _check_derived(m, k, n, kernel):
     assert e <= REL_TOL                                      # max relative error 1e-2
 
 
-@pytest.mark.parametrize("m,k,n,split", [(12288, 1024, 1000, 1), (5120, 8192, 1300, 2), (5120, 4096, 1300, None)])
+@pytest.mark.parametrize("m,k,n,split", [(12288, 1024, 1000, 1), (16384, 8192, 1000, 1), (5120, 8192, 1300, None), (5120, 4096, 1300, None)])
 def test_derived_config_for_an_untuned_shape_with_very_many_tokens(m, k, n, split):
-    """A shape outside the table with 768 tokens or more gets the 256 x 256 many-token tile when its tiles fill the
-    device (192 tiles; 120 tiles with the k range split in two; not with 120 tiles and k below 8192), through the plain
-    entry point; checked on a random subset of rows."""
+    """A shape outside the table with very many tokens gets the 256 x 256 many-token tile when its tiles fill the
+    device in one round (192 and 256 tiles), not when smaller tiles make a fuller round (120 tiles of 256 x 256
+    against 240 of 128 x 256), through the plain entry point; checked on a random subset of rows."""
     import torch
 
     from tuna_amd import ops

@@ -92,7 +92,7 @@ def test_select_config_is_host_only_and_every_table_entry_validates():
             # entries are tuned at their bucket's lower edge: counts from the entry's next_from on take the next
             # bucket's entry (fewer passes over the weights)
             nxt = pm.get(f"{m}_{make_configs.key_of(hi + 1, present)}_{k}") if n >= nf and hi < 128000 else None
-            if n >= 3072 and m < 24576:
+            if n >= 2560 and m < 24576:
                 # far into the open-ended last bucket (tuned at 2048 tokens): the 256 x 256 many-token tile
                 assert (got.lds_tile_rows, got.token_tiles, got.split_k, got.rows_per_wave) == (256, 16, 1, 64)
                 ops.validate_config(m, n, k, got)

@@ -423,8 +423,11 @@ static tuna_gemm_config derive_config(int m, int n, int k)
             memset(&c, 0, sizeof(c));
             c.rows_per_wave = 64, c.split_k = 1, c.token_tiles = n <= 16 ? 1 : 2, c.x_chunk = 512, c.xcd_swizzle = 1, c.k_stagger = 2;
             c.lds_tile_rows = -1;
+            // (4 x 4 also where the 128-row tiles of 2 x 8 times the passes would not fit the device at once:
+            // 20480 x 5120 at 64 tokens as 160 x 2 workgroups 41.5 us, as 80 x 2 31.7)
+            const bool second_round = n > 16 && (long long)(groups / 2) * ceil_div(n, 32) > kMaxCus;
             if (groups >= 576 && n > 32) c.waves_m = 4, c.waves_k = 2, c.prefetch = 2, c.token_tiles = 4, c.x_chunk = 256;
-            else if (groups >= 576) c.waves_m = 4, c.waves_k = 4, c.prefetch = (n <= 16 && k >= 3072) ? 4 : 2, c.x_chunk = n <= 16 ? 512 : 256;
+            else if (groups >= 576 || second_round) c.waves_m = 4, c.waves_k = 4, c.prefetch = (n <= 16 && k >= 3072) ? 4 : 2, c.x_chunk = n <= 16 ? 512 : 256;
             else c.waves_m = 2, c.waves_k = 8, c.prefetch = 2;
             if (config_runs(m, n, k, c)) return c;
         }
@@ -461,7 +464,7 @@ static tuna_gemm_config derive_config(int m, int n, int k)
     if (n > 64 && n <= 256 && k % 512 == 0) {
         // 65..256 tokens: the streaming kernel with the weights through LDS, 16 waves (8 with four token tiles), the
         // passes of 16, 32 or 64 tokens side by side in the grid (they share the weights through the L2), the tile
-        // height and the tokens per pass chosen so that row tiles x passes make one round of 150..300 workgroups -
+        // height and the tokens per pass chosen so that row tiles x passes make one round of 150..256 workgroups -
         // what the tuner finds on 3072 x 8192, 4096 x 12288, 5120 x 5120, 12288 x 4096 and 16384 x 8192 (128 tokens:
         // 22.8, 32.9, 21.1, 27.3, 53.2 us against 60.3, 49.8, 37.2, 33.2, 57.3 of the rules below, which split k for
         // the many-token kernel there).
@@ -470,7 +473,7 @@ static tuna_gemm_config derive_config(int m, int n, int k)
             const int tt = kTokWm[ci][0], wm = kTokWm[ci][1];
             if (m % (64 * wm) != 0) continue;
             const long long wgs = (long long)(m / (64 * wm)) * ceil_div(n, 16 * tt);
-            if (wgs < 150 || wgs > 300) continue;
+            if (wgs < 150 || wgs > kMaxCus) continue;  // (one round: 18432 x 6144 at 256 tokens as 288 workgroups 125 us, as 144 tiles of 128 x 256 89)
             for (int lds = -1; lds <= 0; ++lds) {
                 memset(&c, 0, sizeof(c));
                 c.rows_per_wave = 64, c.waves_m = wm, c.waves_k = (tt == 4 ? 8 : 16) / wm, c.prefetch = 2, c.split_k = 1;
@@ -522,6 +525,53 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         c.rows_per_wave = 64, c.waves_m = 2, c.waves_k = 4, c.split_k = 1, c.prefetch = 2, c.x_chunk = 256;
         c.token_tiles = 4;
         if (config_runs(m, n, k, c)) return c;
+    }
+    if (n >= 256 && m < 24576) {
+        // 256 tokens and more on shapes of fewer than 24576 rows: the tile whose grid costs least by a model read off
+        // the timings of 33 shapes outside the table (1024 x 8192 ... 23040 x 3072) at 256 ... 3000 tokens, each with
+        // up to thirty candidate launches.  A workgroup's time is its tile's rows x tokens (tokens beyond n included:
+        // a tile is computed whole) times a factor of the kernel - the 256 x 256 tile 0.85, the streaming kernel
+        // with eight token tiles on 512 rows 0.95, the 128 x 256 tile 1.00, eight token tiles on 256 rows 1.15,
+        // 256 x 128 1.20, 128 x 128 and four token tiles on 256 rows 1.45, two token tiles on 256 rows 1.78, four on
+        // 128 rows 1.95, two on 128 rows 2.0 - plus a fixed part that counts for short k (about 6 us), and grows by
+        // a seventh from 160 to 256 workgroups on the device (clock and memory are shared); a launch is as many
+        // rounds as its tiles need on 256 CUs, and a round that is not full takes nearly as long as a full one.
+        // What the rules below cost before this one: 12288 x 4096 at 288 tokens 68 us (128 x 256 tiles, half empty)
+        // against 46 (four token tiles, 240 workgroups), 20480 x 5120 at 384 tokens 153 against 91, 16384 x 8192 at
+        // 640 tokens 249 against 195 (256 x 256), 2048 x 2048 at 384 tokens 27 against 13.  Grids of fewer than 64
+        // workgroups are left to the rules below, which split k.
+        struct Cand { int rows, tokens, streaming; double factor; };
+        static const Cand kCand[10] = {{256, 256, 0, 0.85}, {512, 128, 1, 0.95}, {128, 256, 0, 1.00}, {256, 128, 1, 1.15}, {256, 128, 0, 1.20},
+                                       {128, 128, 0, 1.45}, {256, 64, 1, 1.45},  {256, 32, 1, 1.78},  {128, 64, 1, 1.95},  {128, 32, 1, 2.00}};
+        tuna_gemm_config best;
+        double best_cost = 0.0;
+        bool found = false;
+        for (const Cand &cd : kCand) {
+            if (cd.streaming && m % cd.rows != 0) continue;
+            const long long tiles = (long long)ceil_div(m, cd.rows) * ceil_div(n, cd.tokens);
+            if (tiles < 64) continue;
+            const long long full = tiles / kMaxCus, rest = tiles % kMaxCus;
+            const double rounds = 1.15 * (double)full + (rest ? 0.7 + 0.45 * (double)rest / kMaxCus : 0.0);
+            const double cost = rounds * ((double)cd.rows * cd.tokens * cd.factor + 1.2e7 / k);
+            if (found && cost >= best_cost) continue;
+            memset(&c, 0, sizeof(c));
+            c.rows_per_wave = 64, c.split_k = 1, c.prefetch = 2;
+            if (!cd.streaming) {
+                c.waves_m = 1, c.waves_k = 1, c.x_chunk = 64, c.token_tiles = cd.tokens / 16, c.lds_tile_rows = cd.rows;
+            } else {
+                c.token_tiles = cd.tokens / 16, c.waves_m = cd.rows / 64, c.waves_k = (c.token_tiles == 2 ? 16 : 8) / c.waves_m;
+                c.x_chunk = c.token_tiles == 8 ? 128 : c.token_tiles == 4 ? 256 : 512;
+                while (c.x_chunk > 64 && k % c.x_chunk != 0) c.x_chunk /= 2;
+                c.xcd_swizzle = 1, c.lds_tile_rows = cd.rows == 512 ? 0 : -1;
+            }
+            if (!config_runs(m, n, k, c)) {
+                if (c.lds_tile_rows != -1) continue;
+                c.lds_tile_rows = 0;  // (no twin with the weights through LDS for this k)
+                if (!config_runs(m, n, k, c)) continue;
+            }
+            best = c, best_cost = cost, found = true;
+        }
+        if (found) return best;
     }
     if (n >= 768) {
         // very many tokens: the 256 x 256 tile (one wave per SIMD) where it fills the device - from about 150
@@ -599,11 +649,12 @@ static int select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_t
     }
     if (own) {
         *cfg = own->cfg;
-        // The last bucket is open-ended and tuned at 2048 tokens.  From 3072 tokens a shape of fewer than 24576 rows
+        // The last bucket is open-ended and tuned at 2048 tokens.  From 2560 tokens a shape of fewer than 24576 rows
         // takes the 256 x 256 many-token tile whatever its entry says, when that tile fills the device: measured on
-        // six benchmark shapes at 3072..8192 tokens it equals or beats every other entry there (4096 x 4096 at 8192
-        // tokens 336 -> 255 us, 4096 x 14336 at 4096 tokens 469 -> 392 us, 10240 x 8192 at 8192 tokens 1582 -> 1200 us).
-        if (n >= 3072 && m < 24576 && !(cfg->lds_tile_rows == 256 && cfg->token_tiles == 16) &&
+        // six benchmark shapes at 2560..8192 tokens it equals or beats every other entry there (4096 x 4096 at 8192
+        // tokens 336 -> 255 us, 4096 x 14336 at 4096 tokens 469 -> 392 us, 10240 x 8192 at 8192 tokens 1582 -> 1200 us
+        // and at 2560 tokens 530 -> 420; at 2049..2304 tokens the entries hold: 10240 x 2560 133 us against 148).
+        if (n >= 2560 && m < 24576 && !(cfg->lds_tile_rows == 256 && cfg->token_tiles == 16) &&
             (long long)ceil_div(m, 256) * ceil_div(n, 256) >= 150) {
             memset(cfg, 0, sizeof(*cfg));
             cfg->rows_per_wave = 64, cfg->waves_m = 1, cfg->waves_k = 1, cfg->prefetch = 2, cfg->x_chunk = 64;
