@@ -657,7 +657,7 @@ def test_derived_config_for_an_untuned_shape_with_very_many_tokens(m, k, n, spli
 
 
 @pytest.mark.parametrize("m,k,n,tiles", [(66560, 1024, 50, 4), (66560, 1024, 100, 8), (66560, 1024, 300, 8),
-                                         (16384, 2048, 100, 4)])
+                                         (16384, 2048, 100, 2)])
 def test_derived_config_for_a_large_untuned_shape_with_many_tokens(m, k, n, tiles):
     """A shape outside the table with many rows and more than 32 tokens gets the streaming kernel
     with four or eight token tiles (one pass of 64 or 128 tokens, or three passes of 128 side by

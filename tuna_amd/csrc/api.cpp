@@ -461,7 +461,58 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         }
         if (best_wgs) return best;
     }
+    if (n > 64 && m < 24576) {
+        // 65 tokens and more on shapes of fewer than 24576 rows: the tile whose grid costs least by a model read off
+        // the timings of 36 shapes outside the table (1024 x 8192 ... 23040 x 3072) at 65 ... 3000 tokens, each with
+        // up to thirty candidate launches.  A workgroup's time is its tile's rows x tokens (tokens beyond n included:
+        // a tile is computed whole) times a factor of the kernel - the 256 x 256 tile 0.85, the streaming kernel
+        // with eight token tiles on 512 rows 0.95, the 128 x 256 tile 1.00, eight token tiles on 256 rows 1.15,
+        // 256 x 128 1.20, 128 x 128 and four token tiles on 256 rows 1.45, two token tiles on 256 rows 1.78, four on
+        // 128 rows 1.95, two on 128 rows 2.0, and up to 255 tokens one token tile on 256, 128 or 64 rows 2.6, 2.2, 4.0
+        // - plus a fixed part that counts for short k (about 6 us), and grows by
+        // a seventh from 160 to 256 workgroups on the device (clock and memory are shared); a launch is as many
+        // rounds as its tiles need on 256 CUs, and a round that is not full takes nearly as long as a full one.
+        // What the rules below cost before this one: 12288 x 4096 at 288 tokens 68 us (128 x 256 tiles, half empty)
+        // against 46 (four token tiles, 240 workgroups), 20480 x 5120 at 384 tokens 153 against 91, 16384 x 8192 at
+        // 640 tokens 249 against 195 (256 x 256), 2048 x 2048 at 384 tokens 27 against 13, 20480 x 5120 at 96 tokens
+        // 55 against 36, 1024 x 8192 at 160 tokens 89 against 29.  Grids of fewer than 32 workgroups (64 from 256
+        // tokens) are left to the rules below, which split k.
+        struct Cand { int rows, tokens, streaming; double factor; };
+        static const Cand kCand[13] = {{256, 256, 0, 0.85}, {512, 128, 1, 0.95}, {128, 256, 0, 1.00}, {256, 128, 1, 1.15}, {256, 128, 0, 1.20},
+                                       {128, 128, 0, 1.45}, {256, 64, 1, 1.45},  {256, 32, 1, 1.78},  {128, 64, 1, 1.95},  {128, 32, 1, 2.00},
+                                       {256, 16, 1, 2.60},  {128, 16, 1, 2.20},  {64, 16, 1, 4.00}};
+        tuna_gemm_config best;
+        double best_cost = 0.0;
+        bool found = false;
+        for (const Cand &cd : kCand) {
+            if ((cd.streaming && m % cd.rows != 0) || (cd.tokens == 16 && n >= 256)) continue;
+            const long long tiles = (long long)ceil_div(m, cd.rows) * ceil_div(n, cd.tokens);
+            if (tiles < (n >= 256 ? 64 : 32)) continue;
+            const long long full = tiles / kMaxCus, rest = tiles % kMaxCus;
+            const double rounds = 1.15 * (double)full + (rest ? 0.7 + 0.45 * (double)rest / kMaxCus : 0.0);
+            const double cost = rounds * ((double)cd.rows * cd.tokens * cd.factor + 1.2e7 / k);
+            if (found && cost >= best_cost) continue;
+            memset(&c, 0, sizeof(c));
+            c.rows_per_wave = 64, c.split_k = 1, c.prefetch = 2;
+            if (!cd.streaming) {
+                c.waves_m = 1, c.waves_k = 1, c.x_chunk = 64, c.token_tiles = cd.tokens / 16, c.lds_tile_rows = cd.rows;
+            } else {
+                c.token_tiles = cd.tokens / 16, c.waves_m = cd.rows / 64, c.waves_k = (c.token_tiles <= 2 ? 16 : 8) / c.waves_m;
+                c.x_chunk = c.token_tiles == 8 ? 128 : c.token_tiles == 4 ? 256 : 512;
+                while (c.x_chunk > 64 && k % c.x_chunk != 0) c.x_chunk /= 2;
+                c.xcd_swizzle = 1, c.lds_tile_rows = cd.rows == 512 ? 0 : -1;
+            }
+            if (!config_runs(m, n, k, c)) {
+                if (c.lds_tile_rows != -1) continue;
+                c.lds_tile_rows = 0;  // (no twin with the weights through LDS for this k)
+                if (!config_runs(m, n, k, c)) continue;
+            }
+            best = c, best_cost = cost, found = true;
+        }
+        if (found) return best;
+    }
     if (n > 64 && n <= 256 && k % 512 == 0) {
+        // (what the model above leaves: shapes of 24576 rows and more, and grids too small for it)
         // 65..256 tokens: the streaming kernel with the weights through LDS, 16 waves (8 with four token tiles), the
         // passes of 16, 32 or 64 tokens side by side in the grid (they share the weights through the L2), the tile
         // height and the tokens per pass chosen so that row tiles x passes make one round of 150..256 workgroups -
@@ -525,53 +576,6 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         c.rows_per_wave = 64, c.waves_m = 2, c.waves_k = 4, c.split_k = 1, c.prefetch = 2, c.x_chunk = 256;
         c.token_tiles = 4;
         if (config_runs(m, n, k, c)) return c;
-    }
-    if (n >= 256 && m < 24576) {
-        // 256 tokens and more on shapes of fewer than 24576 rows: the tile whose grid costs least by a model read off
-        // the timings of 33 shapes outside the table (1024 x 8192 ... 23040 x 3072) at 256 ... 3000 tokens, each with
-        // up to thirty candidate launches.  A workgroup's time is its tile's rows x tokens (tokens beyond n included:
-        // a tile is computed whole) times a factor of the kernel - the 256 x 256 tile 0.85, the streaming kernel
-        // with eight token tiles on 512 rows 0.95, the 128 x 256 tile 1.00, eight token tiles on 256 rows 1.15,
-        // 256 x 128 1.20, 128 x 128 and four token tiles on 256 rows 1.45, two token tiles on 256 rows 1.78, four on
-        // 128 rows 1.95, two on 128 rows 2.0 - plus a fixed part that counts for short k (about 6 us), and grows by
-        // a seventh from 160 to 256 workgroups on the device (clock and memory are shared); a launch is as many
-        // rounds as its tiles need on 256 CUs, and a round that is not full takes nearly as long as a full one.
-        // What the rules below cost before this one: 12288 x 4096 at 288 tokens 68 us (128 x 256 tiles, half empty)
-        // against 46 (four token tiles, 240 workgroups), 20480 x 5120 at 384 tokens 153 against 91, 16384 x 8192 at
-        // 640 tokens 249 against 195 (256 x 256), 2048 x 2048 at 384 tokens 27 against 13.  Grids of fewer than 64
-        // workgroups are left to the rules below, which split k.
-        struct Cand { int rows, tokens, streaming; double factor; };
-        static const Cand kCand[10] = {{256, 256, 0, 0.85}, {512, 128, 1, 0.95}, {128, 256, 0, 1.00}, {256, 128, 1, 1.15}, {256, 128, 0, 1.20},
-                                       {128, 128, 0, 1.45}, {256, 64, 1, 1.45},  {256, 32, 1, 1.78},  {128, 64, 1, 1.95},  {128, 32, 1, 2.00}};
-        tuna_gemm_config best;
-        double best_cost = 0.0;
-        bool found = false;
-        for (const Cand &cd : kCand) {
-            if (cd.streaming && m % cd.rows != 0) continue;
-            const long long tiles = (long long)ceil_div(m, cd.rows) * ceil_div(n, cd.tokens);
-            if (tiles < 64) continue;
-            const long long full = tiles / kMaxCus, rest = tiles % kMaxCus;
-            const double rounds = 1.15 * (double)full + (rest ? 0.7 + 0.45 * (double)rest / kMaxCus : 0.0);
-            const double cost = rounds * ((double)cd.rows * cd.tokens * cd.factor + 1.2e7 / k);
-            if (found && cost >= best_cost) continue;
-            memset(&c, 0, sizeof(c));
-            c.rows_per_wave = 64, c.split_k = 1, c.prefetch = 2;
-            if (!cd.streaming) {
-                c.waves_m = 1, c.waves_k = 1, c.x_chunk = 64, c.token_tiles = cd.tokens / 16, c.lds_tile_rows = cd.rows;
-            } else {
-                c.token_tiles = cd.tokens / 16, c.waves_m = cd.rows / 64, c.waves_k = (c.token_tiles == 2 ? 16 : 8) / c.waves_m;
-                c.x_chunk = c.token_tiles == 8 ? 128 : c.token_tiles == 4 ? 256 : 512;
-                while (c.x_chunk > 64 && k % c.x_chunk != 0) c.x_chunk /= 2;
-                c.xcd_swizzle = 1, c.lds_tile_rows = cd.rows == 512 ? 0 : -1;
-            }
-            if (!config_runs(m, n, k, c)) {
-                if (c.lds_tile_rows != -1) continue;
-                c.lds_tile_rows = 0;  // (no twin with the weights through LDS for this k)
-                if (!config_runs(m, n, k, c)) continue;
-            }
-            best = c, best_cost = cost, found = true;
-        }
-        if (found) return best;
     }
     if (n >= 768) {
         // very many tokens: the 256 x 256 tile (one wave per SIMD) where it fills the device - from about 150
