@@ -387,20 +387,30 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         // 32-row tiles: 20.9 us against 18.4).  17..64 tokens: the same with one or two token tiles per pass, the
         // passes side by side in the grid, so that rows x passes make the round (8192 x 3072 at 64 tokens as
         // 128 x 2 workgroups 11.4 us against 27.6; 64- and 32-row tiles only).
-        // (Second pass, shapes of up to 8 MB at up to 16 tokens that no tile height brings into that range: 96..600
+        // (Second pass, shapes of up to 8 MB that no tile height brings into that range: 96..600
         // workgroups - 2048 x 2048 as 128 workgroups of 16 rows 3.9 us against 9.0, 8960 x 1536 as 280 of 32 rows
-        // 6.0 against 7.9.)
+        // 6.0 against 7.9; at 17..64 tokens from 64 workgroups and with the short tiles up to k = 8192:
+        // 1280 x 5120 at 20 tokens as 80 x 2 of 16 rows 5.9 us against 16.7 of the general kernel.)
         static const int kRows[4] = {64, 32, 24, 16};
         static const int kRing[5][2] = {{8, 4}, {4, 8}, {8, 2}, {4, 4}, {4, 2}};  // waves along k, ring depth
-        for (int pass = 0; pass < (n <= 16 ? 2 : 1); ++pass) {
-            const int lo = pass ? 96 : 150, hi = pass ? 600 : 300;
+        for (int pass = 0; pass < 2; ++pass) {
+            const int lo = pass ? (n <= 16 ? 96 : 64) : 150, hi = pass ? 600 : 300;
             if (pass && (long long)m * k > (8ll << 21)) break;  // 8 MB of packed weights
-            for (int ri = 0; ri < (n <= 16 ? 4 : 2); ++ri) {
+            // (24- and 16-row tiles also at 17..64 tokens, for the shapes too small for a round of taller ones:
+            // 2048 x 2048 at 24 tokens as 128 x 2 workgroups of 16 rows 3.9 us against 6.1 of the lean kernel,
+            // 1536 x 1536 at 48 tokens as 64 x 3 of 24 rows 4.4 against 11.6 of the general kernel; an odd number
+            // of token tiles goes one tile per pass first where those passes fit the device at once, since passes of
+            // two would compute a tile of padding: 5120 x 5120 at 48 tokens 11.0 us against 16.0, 2560 x 5120 at 40
+            // tokens 7.5 against 12.0)
+            const int tt_first = n <= 16 ? 1 : 2;
+            for (int ri = 0; ri < 4; ++ri) {
                 const int r = kRows[ri];
-                if (m % r != 0 || (r < 32 && k > 4096) || (r < 64 && k > 8192)) continue;
-                for (int tt = n <= 16 ? 1 : 2; tt >= 1; --tt) {
+                if (m % r != 0 || (r < 32 && k > (pass && n > 16 ? 8192 : 4096)) || (r < 64 && k > 8192)) continue;
+                const int tt_step = (n > 32 && ceil_div(n, 16) % 2 == 1) ? 1 : -1;
+                for (int tt = tt_step > 0 ? 1 : tt_first; tt >= 1 && tt <= tt_first; tt += tt_step) {
                     const long long wgs = (long long)(m / r) * ceil_div(n, 16 * tt);
                     if (wgs < lo || wgs > hi) continue;
+                    if (tt_step > 0 && tt == 1 && wgs > kMaxCus) continue;  // (three passes only where they run at once)
                     if (!pass && n <= 16 && r == 64 && wgs > 260) continue;  // (two 64-row tiles on some CUs: the streaming twin below)
                     for (int gi = 0; gi < 5; ++gi) {
                         if (k % (32 * kRing[gi][0] * kRing[gi][1]) != 0 || (tt > 1 && kRing[gi][1] > 4)) continue;
