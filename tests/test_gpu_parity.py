@@ -489,10 +489,51 @@ def test_every_entry_for_the_upper_part_of_a_bucket_matches_the_oracle(key):
         assert e <= REL_TOL
 
 
+@pytest.mark.parametrize("name,n,kernel", [("mistral_qkv", 1200, "128 rows x 256 tokens"), ("llama70b_qkv", 1536, "gemm_wide_kernel"),
+                                           ("mistral_attn_out", 700, "TT=4"), ("llama70b_attn_out", 600, "128 rows x 256 tokens"),
+                                           ("mistral_down", 1000, "split_k=2")])
+def test_table_shapes_between_the_counts_their_upper_entries_are_tuned_at(name, n, kernel):
+    """Above 512 tokens the table's entries are tuned at 512, 1024 and 2048 tokens; at other counts a shape of fewer than
+    24576 rows runs what the derivation's cost model picks (its entry where that splits k: the last case), through the
+    plain entry point.  Row-subset check against the oracle."""
+    import torch
+
+    from tuna_amd import ops
+    from tuna_amd.quantize import nf4_codebook
+    from tuna_amd.synth import SHAPES, make_weights_torch, make_x_torch
+
+    m, k = SHAPES[name]
+    used, hit = ops.select_config(m, n, k)
+    desc = ops.describe_launch(m, n, k, None)
+    print(f"table shape {name} m={m} k={k} n={n}: {desc}", flush=True)
+    assert hit and kernel in desc
+    if "split_k=2" not in kernel:
+        assert used.to_dict() == ops.derive_config(m, n, k).to_dict()
+    dev = torch.device("cuda")
+    q, absmax = make_weights_torch(m, k, seed=n, device=dev)
+    x = make_x_torch(n, k, seed=n + 1, device=dev)
+    code = nf4_codebook(dev)
+    out = torch.full((n, m), float("nan"), dtype=torch.float16, device=dev)
+    ops.matmul(x, q, absmax, code, out, m, n, k)
+    torch.cuda.synchronize()
+    assert not torch.isnan(out).any()
+    rng = np.random.default_rng(n)
+    mbs = np.sort(rng.choice(m // 8, size=4, replace=False))
+    rows = (mbs[:, None] * 8 + np.arange(8)[None, :]).ravel()
+    q_sub = q[torch.from_numpy(mbs).to(dev)].cpu().numpy()
+    ref = O.gemm_f64(q_sub, x.cpu().numpy().view(np.uint16), code.cpu().numpy(), absmax.cpu().numpy()[rows],
+                     len(rows), n, k, mode=O.D1)
+    got = out[:, torch.from_numpy(rows).to(dev)].cpu().numpy().view(np.uint16)
+    e = rel_err(f16_bits_to_f64(got), ref)
+    print(f"  rel_err={e:.3e}", flush=True)
+    assert e <= REL_TOL
+
+
 @pytest.mark.parametrize("name,n", [("mistral_attn_out", 3072), ("mistral_down", 3100), ("llama70b_qkv", 4096), ("llama70b_qkv", 2560)])
 def test_token_counts_far_into_the_last_bucket_take_the_256_x_256_tile(name, n):
-    """The last bucket of the table is open-ended and tuned at 2048 tokens; from 2560 tokens a shape of fewer than
-    24576 rows runs the 256 x 256 many-token tile through the plain entry point.  Row-subset check against the oracle."""
+    """The last bucket of the table is open-ended and tuned at 2048 tokens; away from that count a shape of fewer than
+    24576 rows takes the pick of the derivation's cost model, which far into the bucket is the 256 x 256 many-token
+    tile, through the plain entry point.  Row-subset check against the oracle."""
     import torch
 
     from tuna_amd import ops

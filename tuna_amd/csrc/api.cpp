@@ -663,16 +663,17 @@ static int select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_t
     }
     if (own) {
         *cfg = own->cfg;
-        // The last bucket is open-ended and tuned at 2048 tokens.  From 2560 tokens a shape of fewer than 24576 rows
-        // takes the 256 x 256 many-token tile whatever its entry says, when that tile fills the device: measured on
-        // six benchmark shapes at 2560..8192 tokens it equals or beats every other entry there (4096 x 4096 at 8192
-        // tokens 336 -> 255 us, 4096 x 14336 at 4096 tokens 469 -> 392 us, 10240 x 8192 at 8192 tokens 1582 -> 1200 us
-        // and at 2560 tokens 530 -> 420; at 2049..2304 tokens the entries hold: 10240 x 2560 133 us against 148).
-        if (n >= 2560 && m < 24576 && !(cfg->lds_tile_rows == 256 && cfg->token_tiles == 16) &&
-            (long long)ceil_div(m, 256) * ceil_div(n, 256) >= 150) {
-            memset(cfg, 0, sizeof(*cfg));
-            cfg->rows_per_wave = 64, cfg->waves_m = 1, cfg->waves_k = 1, cfg->prefetch = 2, cfg->x_chunk = 64;
-            cfg->token_tiles = 16, cfg->lds_tile_rows = 256, cfg->split_k = 1;
+        // The entries of the three upper buckets are tuned at 512, 1024 and 2048 tokens, and between those counts
+        // the best grid changes with every token tile that n gains.  Shapes of fewer than 24576 rows therefore take
+        // the pick of the derivation's cost model there (the same tiles the tuner chooses among in these buckets):
+        // on the twelve such shapes of the table at 600 ... 2304 tokens the entries are 1.10 x the best of thirty
+        // timed launches on average (up to 1.56: 6144 x 4096 at 1200 tokens 106 us against 68; 10240 x 8192 at 1536
+        // tokens 289 against 217), the model's picks 1.02 x.  The entry stays where it was tuned - counts with as
+        // many 128-token tiles as its tuning count - and where it splits k (few rows with long k: the model has no
+        // split; 2560 x 10240 at 1000 tokens 84 us with its entry, 111 with the model's pick).
+        if (n > 512 && m < 24576 && own->cfg.split_k == 1) {
+            const int tuned = own->n_lo <= 512 ? 512 : own->n_lo <= 769 ? 1024 : 2048;
+            if (ceil_div(n, 128) != ceil_div(tuned, 128)) *cfg = derive_config(m, n, k);
         }
         if (from_table) *from_table = 1;
         return TUNA_OK;
