@@ -615,7 +615,7 @@ def test_derived_configs_for_untuned_shapes_up_to_16_tokens(m, k, n, kernel):
                                            (3072, 8192, 512, "TT=2"), (20480, 5120, 64, "TT=2"),
                                            (18432, 6144, 256, "128 rows x 256 tokens"), (2048, 2048, 384, "TT=2"),
                                            (20480, 5120, 384, "TT=8"), (16384, 8192, 640, "gemm_wide_kernel"),
-                                           (2560, 6912, 300, "gemm_mid_kernel"), (22016, 4096, 704, "128 rows x 256 tokens")])
+                                           (2560, 6912, 300, "128 rows x 128 tokens> split_k=3"), (4096, 11008, 100, "128 rows x 128 tokens> split_k=4"), (22016, 4096, 704, "128 rows x 256 tokens")])
 def test_derived_configs_for_untuned_shapes_from_17_to_512_tokens(m, k, n, kernel):
     """The same for 17 tokens and more: narrow-row and lean workgroups with the token passes side by side in the grid,
     the streaming kernel with 16, 32 or 64 tokens per pass, and from 256 tokens the tile that a cost model of the

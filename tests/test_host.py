@@ -102,9 +102,9 @@ def test_select_config_is_host_only_and_every_table_entry_validates():
                     pass      # (passed over only because it cannot run n tokens)
             # above 512 tokens the entries are tuned at 512, 1024 and 2048 tokens: away from those counts (another
             # number of 128-token tiles) a shape of fewer than 24576 rows takes the pick of the derivation's cost
-            # model - far into the open-ended last bucket the 256 x 256 tile - unless the entry splits k
+            # model - far into the open-ended last bucket the 256 x 256 tile
             tuned_at = 512 if eff_lo <= 512 else 1024 if eff_lo <= 769 else 2048
-            if n > 512 and m < 24576 and eff["split_k"] == 1 and -(-n // 128) != -(-tuned_at // 128):
+            if n > 512 and m < 24576 and -(-n // 128) != -(-tuned_at // 128):
                 assert got.to_dict() == ops.derive_config(m, n, k).to_dict()
                 if n >= 3000:
                     assert (got.lds_tile_rows, got.token_tiles, got.split_k, got.rows_per_wave) == (256, 16, 1, 64)

@@ -478,7 +478,7 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         // a tile is computed whole) times a factor of the kernel - the 256 x 256 tile 0.85, the streaming kernel
         // with eight token tiles on 512 rows 0.95, the 128 x 256 tile 1.00, eight token tiles on 256 rows 1.15,
         // 256 x 128 1.20, 128 x 128 and four token tiles on 256 rows 1.45, two token tiles on 256 rows 1.78, four on
-        // 128 rows 1.95, two on 128 rows 2.0, and up to 255 tokens one token tile on 256, 128 or 64 rows 2.6, 2.2, 4.0
+        // 128 rows 1.95, two on 128 rows 2.0, and up to 320 tokens one token tile on 256, 128 or 64 rows 2.6, 2.2, 4.0
         // - plus a fixed part that counts for short k (about 6 us), and grows by
         // a seventh from 160 to 256 workgroups on the device (clock and memory are shared); a launch is as many
         // rounds as its tiles need on 256 CUs, and a round that is not full takes nearly as long as a full one.
@@ -494,22 +494,35 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         tuna_gemm_config best;
         double best_cost = 0.0;
         bool found = false;
-        for (const Cand &cd : kCand) {
-            if ((cd.streaming && m % cd.rows != 0) || (cd.tokens == 16 && n >= 256)) continue;
-            const long long tiles = (long long)ceil_div(m, cd.rows) * ceil_div(n, cd.tokens);
-            if (tiles < (n >= 256 ? 64 : 32)) continue;
+        for (int ci = 0; ci < 13 * 4; ++ci) {
+            // (the 128- and 256-row tiles of the many-token kernel also with k split in 2, 3 or 4 while the grid
+            // stays within one round: a split workgroup does its share of the tile's time and the last one to
+            // arrive adds the partial tiles, which costs about 0.4 us per split and 1000 tile elements - what wins
+            // on few rows with long k: 2560 x 10240 at 1000 tokens 84 us as 80 tiles x 3 against 103 unsplit)
+            const Cand &cd = kCand[ci / 4];
+            const int split = ci % 4 + 1;
+            if ((cd.streaming && m % cd.rows != 0) || (cd.tokens == 16 && n > 320)) continue;
+            if (split > 1 && (cd.streaming || cd.rows * cd.tokens > 32768 || ceil_div(k, 64) / split < 8)) continue;
+            const long long tiles = (long long)ceil_div(m, cd.rows) * ceil_div(n, cd.tokens) * split;
+            if (tiles < (n >= 256 ? 64 : 32) || (split > 1 && tiles > kMaxCus)) continue;
             const long long full = tiles / kMaxCus, rest = tiles % kMaxCus;
             const double rounds = 1.15 * (double)full + (rest ? 0.7 + 0.45 * (double)rest / kMaxCus : 0.0);
-            const double cost = rounds * ((double)cd.rows * cd.tokens * cd.factor + 1.2e7 / k);
+            const double area = (double)cd.rows * cd.tokens;
+            double cost = rounds * (area * cd.factor / split + 1.2e7 / k) + (split > 1 ? 800.0 * area * split / k : 0.0);
             if (found && cost >= best_cost) continue;
             memset(&c, 0, sizeof(c));
-            c.rows_per_wave = 64, c.split_k = 1, c.prefetch = 2;
+            c.rows_per_wave = 64, c.split_k = split, c.prefetch = 2;
             if (!cd.streaming) {
                 c.waves_m = 1, c.waves_k = 1, c.x_chunk = 64, c.token_tiles = cd.tokens / 16, c.lds_tile_rows = cd.rows;
             } else {
                 c.token_tiles = cd.tokens / 16, c.waves_m = cd.rows / 64, c.waves_k = (c.token_tiles <= 2 ? 16 : 8) / c.waves_m;
                 c.x_chunk = c.token_tiles == 8 ? 128 : c.token_tiles == 4 ? 256 : 512;
+                // (a k that the chunk does not divide takes shorter chunks and loses the twin with the weights
+                // through LDS: the factors above were not measured on that launch - 4096 x 11008 at 72 tokens runs
+                // 62 us that way against 46 of 128 x 128 tiles with k split in 4 - so it is priced a third higher)
+                const int want_chunk = c.x_chunk;
                 while (c.x_chunk > 64 && k % c.x_chunk != 0) c.x_chunk /= 2;
+                if (c.x_chunk != want_chunk) cost *= 1.35;
                 c.xcd_swizzle = 1, c.lds_tile_rows = cd.rows == 512 ? 0 : -1;
             }
             if (!config_runs(m, n, k, c)) {
@@ -517,6 +530,7 @@ static tuna_gemm_config derive_config(int m, int n, int k)
                 c.lds_tile_rows = 0;  // (no twin with the weights through LDS for this k)
                 if (!config_runs(m, n, k, c)) continue;
             }
+            if (found && cost >= best_cost) continue;
             best = c, best_cost = cost, found = true;
         }
         if (found) return best;
@@ -668,10 +682,9 @@ static int select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_t
         // the pick of the derivation's cost model there (the same tiles the tuner chooses among in these buckets):
         // on the twelve such shapes of the table at 600 ... 2304 tokens the entries are 1.10 x the best of thirty
         // timed launches on average (up to 1.56: 6144 x 4096 at 1200 tokens 106 us against 68; 10240 x 8192 at 1536
-        // tokens 289 against 217), the model's picks 1.02 x.  The entry stays where it was tuned - counts with as
-        // many 128-token tiles as its tuning count - and where it splits k (few rows with long k: the model has no
-        // split; 2560 x 10240 at 1000 tokens 84 us with its entry, 111 with the model's pick).
-        if (n > 512 && m < 24576 && own->cfg.split_k == 1) {
+        // tokens 289 against 217), the model's picks 1.02 x.  The entry stays where it was tuned: counts with as
+        // many 128-token tiles as its tuning count.
+        if (n > 512 && m < 24576) {
             const int tuned = own->n_lo <= 512 ? 512 : own->n_lo <= 769 ? 1024 : 2048;
             if (ceil_div(n, 128) != ceil_div(tuned, 128)) *cfg = derive_config(m, n, k);
         }
