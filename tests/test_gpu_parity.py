@@ -494,8 +494,8 @@ def test_every_entry_for_the_upper_part_of_a_bucket_matches_the_oracle(key):
                                            ("mistral_down", 1000, "split_k=2")])
 def test_table_shapes_between_the_counts_their_upper_entries_are_tuned_at(name, n, kernel):
     """Above 512 tokens the table's entries are tuned at 512, 1024 and 2048 tokens; at other counts a shape of fewer than
-    24576 rows runs what the derivation's cost model picks (its entry where that splits k: the last case), through the
-    plain entry point.  Row-subset check against the oracle."""
+    24576 rows runs what the derivation's cost model picks (its entry at counts with as many 128-token tiles as the
+    tuning count: the last case), through the plain entry point.  Row-subset check against the oracle."""
     import torch
 
     from tuna_amd import ops
