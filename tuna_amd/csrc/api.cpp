@@ -471,8 +471,8 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         }
         if (best_wgs) return best;
     }
-    if (n > 64 && m < 24576) {
-        // 65 tokens and more on shapes of fewer than 24576 rows: the tile whose grid costs least by a model read off
+    if (n > 64) {
+        // 65 tokens and more: the tile whose grid costs least by a model read off
         // the timings of 36 shapes outside the table (1024 x 8192 ... 23040 x 3072) at 65 ... 3000 tokens, each with
         // up to thirty candidate launches.  A workgroup's time is its tile's rows x tokens (tokens beyond n included:
         // a tile is computed whole) times a factor of the kernel - the 256 x 256 tile 0.85, the streaming kernel
@@ -536,7 +536,7 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         if (found) return best;
     }
     if (n > 64 && n <= 256 && k % 512 == 0) {
-        // (what the model above leaves: shapes of 24576 rows and more, and grids too small for it)
+        // (what the model above leaves: grids too small for it)
         // 65..256 tokens: the streaming kernel with the weights through LDS, 16 waves (8 with four token tiles), the
         // passes of 16, 32 or 64 tokens side by side in the grid (they share the weights through the L2), the tile
         // height and the tokens per pass chosen so that row tiles x passes make one round of 150..256 workgroups -
@@ -557,6 +557,7 @@ static tuna_gemm_config derive_config(int m, int n, int k)
             }
         }
     }
+    // (The rules from here on serve what the model above leaves: grids too small for it, and launches it cannot run.)
     if (n >= 256 && m >= 24576 && m % 512 == 0 && k % 128 == 0) {
         // many rows, several passes of 128 tokens: the streaming kernel with eight token tiles
         // (64 rows per wave, no split), whose token chunks run side by side and share the
