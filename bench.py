@@ -679,9 +679,11 @@ def main():
         except torch.OutOfMemoryError as e:  # pragma: no cover
             sweeps["llama70b_80_layers_multi"] = {"error": str(e)[:200]}
         # token sweep on the Llama-70B layer set: the lower edges of the token buckets (where the table's entries are
-        # tuned) and counts inside them (24, 100, 384: served by the entry their bucket's next_from points to)
+        # tuned) and counts inside them (24, 100, 384: served by the entry their bucket's next_from points to, or an
+        # entry of their own; 1536: between two tuning counts, where shapes of fewer than 24576 rows take the pick
+        # of the derivation's cost model)
         tok = {}
-        for nt in (1, 16, 24, 64, 100, 256, 384, 1024, 4096):
+        for nt in (1, 16, 24, 64, 100, 256, 384, 1024, 1536, 4096):
             row = {}
             for nm in names:
                 sm, sk = synth.SHAPES[nm]
