@@ -127,6 +127,43 @@ def test_derived_config_is_valid_for_any_shape(shape):
     assert 0 < lds <= 160 * 1024
 
 
+def test_derived_and_looked_up_configs_are_valid_on_a_sweep_of_shapes_and_token_counts():
+    """The rules and the grid cost model behind tuna_select_config, on 4000 seeded shapes (every kind of m and k the
+    kernels treat differently: multiples of 8, 64, 256, 512) x token counts from 1 to 5000, and on every table shape x
+    150 token counts: each pick passes the library's own validator, fits the LDS, and is what a second call returns;
+    the blockwise derivation likewise where the shape admits scale blocks."""
+    import json
+
+    import numpy as np
+
+    from tuna_amd import ops
+
+    rng = np.random.default_rng(20241125)
+    cases = []
+    for _ in range(4000):
+        step = int(rng.choice([8, 64, 256, 512]))
+        m = int(rng.integers(1, 131072 // step)) * step if rng.random() < 0.3 else int(rng.integers(1, 24576 // step)) * step
+        ks = int(rng.choice([8, 64, 256, 512]))
+        k = int(rng.integers(1, 16384 // ks)) * ks
+        n = int(rng.choice([rng.integers(1, 17), rng.integers(17, 65), rng.integers(65, 256), rng.integers(256, 1025), rng.integers(1025, 5000)]))
+        if m * k // 2 < (1 << 32):
+            cases.append((m, n, k))
+    with open(os.path.join(ROOT, "tuna_amd", "configs", "param_map.json")) as f:
+        pairs = sorted({(int(key.split("_")[0]), int(key.split("_")[2])) for key in json.load(f)})
+    for (m, k) in pairs:
+        cases += [(m, int(n), k) for n in rng.integers(1, 4200, size=150)]
+    for (m, n, k) in cases:
+        cfg, hit = ops.select_config(m, n, k)
+        ops.validate_config(m, n, k, cfg)
+        lds, ws = ops.config_footprint(m, n, k, cfg)
+        assert 0 < lds <= 160 * 1024, (m, n, k, cfg.to_dict())
+        again, hit2 = ops.select_config(m, n, k)
+        assert again.to_dict() == cfg.to_dict() and hit2 == hit
+        if m % 16 == 0 and k % 256 == 0 and k > 64 and n % 7 == 0:
+            bcfg, _ = ops.select_config_blockwise(m, n, k, 64)
+            ops.validate_config_blockwise(m, n, k, 64, bcfg)
+
+
 def test_token_buckets_follow_the_reference_dispatcher():
     from tuna_amd import make_configs as mc
 
