@@ -494,21 +494,23 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         tuna_gemm_config best;
         double best_cost = 0.0;
         bool found = false;
-        for (int ci = 0; ci < 13 * 4; ++ci) {
-            // (the 128- and 256-row tiles of the many-token kernel also with k split in 2, 3 or 4 while the grid
-            // stays within one round: a split workgroup does its share of the tile's time and the last one to
-            // arrive adds the partial tiles, which costs about 0.4 us per split and 1000 tile elements - what wins
-            // on few rows with long k: 2560 x 10240 at 1000 tokens 84 us as 80 tiles x 3 against 103 unsplit)
-            const Cand &cd = kCand[ci / 4];
-            const int split = ci % 4 + 1;
+        static const int kSplit[6] = {1, 2, 3, 4, 6, 8};
+        for (int ci = 0; ci < 13 * 6; ++ci) {
+            // (the tiles of the many-token kernels also with k split in 2 ... 8 while the grid stays within one
+            // round: a split workgroup does its share of the tile's time and the last one to arrive adds the
+            // partial tiles, which costs about 0.3 us + 0.05 us per split and 1000 tile elements - what wins on
+            // few rows with long k: 4096 x 11008 at 128 tokens 30 us as 32 tiles x 8 against 67 of the best
+            // unsplit launch, 5120 x 13824 at 1000 tokens 154 us as 80 tiles of 256 x 256 x 3 against 200)
+            const Cand &cd = kCand[ci / 6];
+            const int split = kSplit[ci % 6];
             if ((cd.streaming && m % cd.rows != 0) || (cd.tokens == 16 && n > 320)) continue;
-            if (split > 1 && (cd.streaming || cd.rows * cd.tokens > 32768 || ceil_div(k, 64) / split < 8)) continue;
+            if (split > 1 && (cd.streaming || ceil_div(k, 64) / split < 8)) continue;
             const long long tiles = (long long)ceil_div(m, cd.rows) * ceil_div(n, cd.tokens) * split;
             if (tiles < (n >= 256 ? 64 : 32) || (split > 1 && tiles > kMaxCus)) continue;
             const long long full = tiles / kMaxCus, rest = tiles % kMaxCus;
             const double rounds = 1.15 * (double)full + (rest ? 0.7 + 0.45 * (double)rest / kMaxCus : 0.0);
             const double area = (double)cd.rows * cd.tokens;
-            double cost = rounds * (area * cd.factor / split + 1.2e7 / k) + (split > 1 ? 800.0 * area * split / k : 0.0);
+            double cost = rounds * (area * cd.factor / split + 1.2e7 / k) + (split > 1 ? (100.0 * split + 600.0) * area / k : 0.0);
             if (found && cost >= best_cost) continue;
             memset(&c, 0, sizeof(c));
             c.rows_per_wave = 64, c.split_k = split, c.prefetch = 2;

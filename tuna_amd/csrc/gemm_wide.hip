@@ -435,17 +435,45 @@ __global__ __launch_bounds__(kWideThreads, 1) void gemm_wide_kernel(const TiledA
     __syncthreads();
     if (*ticket != (unsigned)(a.split_k - 1)) return;
     if (tid == 0) __hip_atomic_store(a.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // (16-byte loads past this CU's and this XCD's caches - the writers sit on any XCD - two slots x two splits
+    // requested before the first is awaited, as in gemm_tiled.hip; a slot's sum adds its splits in ascending order)
     const f32x4 *src = ws4 + tile_id * a.split_k * kTileF4 + (size_t)wave * (64 * 64) + lane;
-#pragma unroll 4
-    for (int sl = 0; sl < 64; ++sl) {
-        const int row = slot_row(sl), tok = slot_tok(sl);
-        float s4[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int sp = 0; sp < a.split_k; ++sp) {
-            const float *p = reinterpret_cast<const float *>(src + (size_t)sp * kTileF4 + sl * 64);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) s4[j] += __hip_atomic_load(p + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int sl = 0; sl < 64; sl += 2) {
+        f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+        int sp = 0;
+        for (; sp + 1 < a.split_k; sp += 2) {
+            const f32x4 *p = src + (size_t)sp * kTileF4 + sl * 64;
+            f32x4 a0, a1, b0, b1;
+            asm volatile("global_load_dwordx4 %0, %4, off sc1\n\t"
+                         "global_load_dwordx4 %1, %5, off sc1\n\t"
+                         "global_load_dwordx4 %2, %6, off sc1\n\t"
+                         "global_load_dwordx4 %3, %7, off sc1\n\t"
+                         "s_waitcnt vmcnt(0)"
+                         : "=&v"(a0), "=&v"(a1), "=&v"(b0), "=&v"(b1)
+                         : "v"(p), "v"(p + 64), "v"(p + kTileF4), "v"(p + kTileF4 + 64)
+                         : "memory");
+            s0 += a0, s1 += a1;
+            s0 += b0, s1 += b1;
         }
-        if (tok < a.n && row + 4 <= a.m) store_features4(outp, resp, a.epilogue, (size_t)tok, a.m, row, s4[0], s4[1], s4[2], s4[3]);
+        if (sp < a.split_k) {
+            const f32x4 *p = src + (size_t)sp * kTileF4 + sl * 64;
+            f32x4 a0, a1;
+            asm volatile("global_load_dwordx4 %0, %2, off sc1\n\t"
+                         "global_load_dwordx4 %1, %3, off sc1\n\t"
+                         "s_waitcnt vmcnt(0)"
+                         : "=&v"(a0), "=&v"(a1)
+                         : "v"(p), "v"(p + 64)
+                         : "memory");
+            s0 += a0, s1 += a1;
+        }
+        {
+            const int row = slot_row(sl), tok = slot_tok(sl);
+            if (tok < a.n && row + 4 <= a.m) store_features4(outp, resp, a.epilogue, (size_t)tok, a.m, row, s0[0], s0[1], s0[2], s0[3]);
+        }
+        {
+            const int row = slot_row(sl + 1), tok = slot_tok(sl + 1);
+            if (tok < a.n && row + 4 <= a.m) store_features4(outp, resp, a.epilogue, (size_t)tok, a.m, row, s1[0], s1[1], s1[2], s1[3]);
+        }
     }
 }
 
