@@ -1664,14 +1664,14 @@ static int derive_blockwise(const BlockwiseCall &b, tuna_gemm_config *out)
     }
     if (n > 64) {
         // 65 tokens and more: the many-token tile and k split whose grid costs least by the model of derive_config,
-        // with the factors of the scale-block variants (128 x 256 tile 1.0, 256 x 128 1.2, 128 x 128 and 64 x 256 1.3,
-        // 256 x 64 1.6, 64 x 128 1.8; split in 2, 3, 4 or 6 while the grid stays near one round), read off fourteen
+        // with the factors of the scale-block variants (128 x 256 tile 1.0, 256 x 128, 128 x 128 and 64 x 256 1.2,
+        // 256 x 64 and 64 x 128 1.6; split in 2 ... 8 while the grid stays near one round), read off sixteen
         // shapes x ten counts from 72 to 2048 tokens with blocks of 64, each timed with every tile and split: the
-        // model's pick is within 7 % of the best on 139 of 140 cases (the rule below, which this one precedes: 1.23 x
+        // model's pick is within 7 % of the best on all 160 cases (the rule below, which this one precedes: 1.23 x
         // on average, up to 2.8 x where it split k by 8 or 10 - 4096 x 4096 at 200 tokens 74 us against 26).
         struct Tile { int rows, tokens; double factor; };
-        static const Tile kTiles[6] = {{128, 256, 1.0}, {256, 128, 1.2}, {128, 128, 1.3}, {64, 256, 1.3}, {256, 64, 1.6}, {64, 128, 1.8}};
-        static const int kSplits[5] = {1, 2, 3, 4, 6};
+        static const Tile kTiles[6] = {{128, 256, 1.0}, {256, 128, 1.2}, {128, 128, 1.2}, {64, 256, 1.2}, {256, 64, 1.6}, {64, 128, 1.6}};
+        static const int kSplits[6] = {1, 2, 3, 4, 6, 8};
         tuna_gemm_config best;
         double best_cost = 0.0;
         bool found = false;
@@ -1683,7 +1683,7 @@ static int derive_blockwise(const BlockwiseCall &b, tuna_gemm_config *out)
                 const long long full = tiles / kMaxCus, rest = tiles % kMaxCus;
                 const double rounds = 1.15 * (double)full + (rest ? 0.7 + 0.45 * (double)rest / kMaxCus : 0.0);
                 const double area = (double)t.rows * t.tokens;
-                const double cost = rounds * (area * t.factor / split + 0.6e7 / k) + (split > 1 ? 500.0 * area * split / k : 0.0);
+                const double cost = rounds * (area * t.factor / split + 0.6e7 / k) + (split > 1 ? (100.0 * split + 300.0) * area / k : 0.0);
                 if (found && cost >= best_cost) continue;
                 tuna_gemm_config c;
                 memset(&c, 0, sizeof(c));
