@@ -133,7 +133,8 @@ int tuna_init(void);
  * fixed array in device memory that is part of the loaded library (16 MB + 256 KB, held on
  * every GPU the library runs on until the process ends) and calls no allocating routine.  A
  * launch that needs more than TUNA_STATIC_WORKSPACE_BYTES of partial sums or more than 65536
- * counters fails with TUNA_ERR_WORKSPACE.  All calls on one GPU share that GPU's array: calls
+ * counters fails with TUNA_ERR_WORKSPACE (where the library picks the config - cfg NULL - and its
+ * pick splits k of a many-token tile further than that, it reduces the split until it fits).  All calls on one GPU share that GPU's array: calls
  * that may overlap (different streams) race; calls on one stream are ordered and safe.  The
  * kernels return the counters they used to zero, so nothing is cleared between calls.  Results
  * are those of tuna_matmul_ex, bit for bit. */

@@ -96,6 +96,35 @@ def test_static_scratch_entry_point_equals_the_allocating_one_on_two_calls_in_a_
     assert np.array_equal(got, ref)
 
 
+def test_static_scratch_entry_point_reduces_a_split_of_the_library_that_would_not_fit():
+    """Where the library picks the config itself and its pick splits k of a many-token tile into more partial tiles
+    than the static scratch holds, the entry point runs the same tile with the largest split that fits: the bits of
+    tuna_matmul_ex with that config."""
+    import torch
+
+    from tuna_amd import ops
+
+    m, n, k = 2560, 600, 6912
+    pick, hit = ops.select_config(m, n, k)
+    assert not hit and pick.lds_tile_rows > 0 and pick.split_k > 2
+    assert ops.config_footprint(m, n, k, pick)[1] > 16 << 20          # 60 tiles of 128 x 256 x 4 splits: 30 MB
+    fits = ops.GemmConfig.from_dict(pick.to_dict())
+    while ops.config_footprint(m, n, k, fits)[1] > 16 << 20:
+        fits.split_k -= 1
+    assert 1 < fits.split_k < pick.split_k
+    q, x, code, absmax = make_inputs_np(m, n, k, seed=5)
+    dq, dx, dc, da = to_dev(q, x, code, absmax)
+    got = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+    ref = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+    ops.matmul_static(dx, dq, da, dc, got, m, n, k)
+    ops.matmul(dx, dq, da, dc, ref, m, n, k, config=fits)
+    torch.cuda.synchronize()
+    assert not torch.isnan(got).any()
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), ref.cpu().numpy().view(np.uint16))
+    with pytest.raises(ops.TunaError):                                  # a config the caller names is taken as it is
+        ops.matmul_static(dx, dq, da, dc, got, m, n, k, config=pick)
+
+
 def test_static_scratch_entry_point_rejects_what_does_not_fit():
     import torch
 

@@ -1021,6 +1021,13 @@ static int matmul_impl(const void *q, const void *x, const void *code, const voi
     if (c.lds_tile_rows > 0) {
         TiledPlan tp;
         if ((rc = plan_tiled(m, n, k, c, decode, &tp))) return rc;
+        // the library's own pick may split k further than the static scratch has room for partial tiles (a split
+        // by 8 of 256 tiles of 128 x 256 needs 32 MB): the split is then reduced until it fits - slower, but the
+        // call that cannot allocate still runs; a config the caller names is taken as it is
+        while (static_ws && !cfg && c.split_k > 1 && (tp.ws_bytes > kStaticWsBytes || tp.n_counters > kStaticCounters)) {
+            c.split_k -= 1;
+            if ((rc = plan_tiled(m, n, k, c, decode, &tp))) return rc;
+        }
         tp.args.q = static_cast<const uint8_t *>(q);
         tp.args.x = x;
         tp.args.code = static_cast<const float *>(code);
