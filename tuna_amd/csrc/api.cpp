@@ -374,6 +374,52 @@ static tuna_gemm_config derive_streaming(int m, int n, int k, int decode)
 // workgroups along k to occupy the CUs.  Rings of 2 k-steps: those variants never spill.
 static bool config_runs(int m, int n, int k, const tuna_gemm_config &c);
 
+// One round of narrow-row workgroups for the shape, if some tile height and tokens per pass give one (the rule is
+// described where derive_config uses it).
+static bool narrow_round(int m, int n, int k, tuna_gemm_config *out)
+{
+    tuna_gemm_config c;
+    static const int kRows[4] = {64, 32, 24, 16};
+    static const int kRing[5][2] = {{8, 4}, {4, 8}, {8, 2}, {4, 4}, {4, 2}};  // waves along k, ring depth
+    for (int pass = 0; pass < 2; ++pass) {
+        // (65 tokens and more: three to eight passes side by side must run at once - 3072 x 8192 at 96 tokens as
+        // 48 x 6 workgroups 26.8 us, as 48 x 3 of two token tiles 20.8 - so the round is 128..256 workgroups there)
+        const int lo = n > 64 ? (pass ? 64 : 128) : pass ? (n <= 16 ? 96 : 64) : 150, hi = n > 64 ? kMaxCus : pass ? 600 : 300;
+        if (pass && (long long)m * k > (8ll << 21)) break;  // 8 MB of packed weights
+        // (24- and 16-row tiles also at 17..64 tokens, for the shapes too small for a round of taller ones:
+        // 2048 x 2048 at 24 tokens as 128 x 2 workgroups of 16 rows 3.9 us against 6.1 of the lean kernel,
+        // 1536 x 1536 at 48 tokens as 64 x 3 of 24 rows 4.4 against 11.6 of the general kernel; an odd number
+        // of token tiles goes one tile per pass first where those passes fit the device at once, since passes of
+        // two would compute a tile of padding: 5120 x 5120 at 48 tokens 11.0 us against 16.0, 2560 x 5120 at 40
+        // tokens 7.5 against 12.0)
+        const int tt_first = n <= 16 ? 1 : 2;
+        for (int ri = 0; ri < 4; ++ri) {
+            const int r = kRows[ri];
+            if (m % r != 0 || (r < 32 && k > (pass && n > 16 ? 8192 : 4096)) || (r < 64 && k > 8192)) continue;
+            const int tt_step = (n > 32 && ceil_div(n, 16) % 2 == 1) ? 1 : -1;
+            for (int tt = tt_step > 0 ? 1 : tt_first; tt >= 1 && tt <= tt_first; tt += tt_step) {
+                const long long wgs = (long long)(m / r) * ceil_div(n, 16 * tt);
+                if (wgs < lo || wgs > hi) continue;
+                if (tt_step > 0 && tt == 1 && wgs > kMaxCus) continue;  // (three passes only where they run at once)
+                if (!pass && n <= 16 && r == 64 && wgs > 260) continue;  // (two 64-row tiles on some CUs: the streaming twin below)
+                for (int gi = 0; gi < 5; ++gi) {
+                    if (k % (32 * kRing[gi][0] * kRing[gi][1]) != 0 || (tt > 1 && kRing[gi][1] > 4)) continue;
+                    if (n > 64 && kRing[gi][0] != 8) continue;  // (a k that only four waves divide: 4096 x 11008 at 72 tokens 38 us, a split many-token tile 28)
+                    memset(&c, 0, sizeof(c));
+                    c.rows_per_wave = r, c.waves_m = r == 64 ? 0 : 1, c.waves_k = kRing[gi][0], c.prefetch = kRing[gi][1];
+                    c.split_k = 1, c.token_tiles = tt, c.x_chunk = 32 * c.waves_k * c.prefetch;
+                    if (config_runs(m, n, k, c)) {
+                        *out = c;
+                        return true;
+                    }
+                }
+            }
+        }
+    }
+    return false;
+}
+
+
 static tuna_gemm_config derive_config(int m, int n, int k)
 {
     tuna_gemm_config c;
@@ -391,37 +437,7 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         // workgroups - 2048 x 2048 as 128 workgroups of 16 rows 3.9 us against 9.0, 8960 x 1536 as 280 of 32 rows
         // 6.0 against 7.9; at 17..64 tokens from 64 workgroups and with the short tiles up to k = 8192:
         // 1280 x 5120 at 20 tokens as 80 x 2 of 16 rows 5.9 us against 16.7 of the general kernel.)
-        static const int kRows[4] = {64, 32, 24, 16};
-        static const int kRing[5][2] = {{8, 4}, {4, 8}, {8, 2}, {4, 4}, {4, 2}};  // waves along k, ring depth
-        for (int pass = 0; pass < 2; ++pass) {
-            const int lo = pass ? (n <= 16 ? 96 : 64) : 150, hi = pass ? 600 : 300;
-            if (pass && (long long)m * k > (8ll << 21)) break;  // 8 MB of packed weights
-            // (24- and 16-row tiles also at 17..64 tokens, for the shapes too small for a round of taller ones:
-            // 2048 x 2048 at 24 tokens as 128 x 2 workgroups of 16 rows 3.9 us against 6.1 of the lean kernel,
-            // 1536 x 1536 at 48 tokens as 64 x 3 of 24 rows 4.4 against 11.6 of the general kernel; an odd number
-            // of token tiles goes one tile per pass first where those passes fit the device at once, since passes of
-            // two would compute a tile of padding: 5120 x 5120 at 48 tokens 11.0 us against 16.0, 2560 x 5120 at 40
-            // tokens 7.5 against 12.0)
-            const int tt_first = n <= 16 ? 1 : 2;
-            for (int ri = 0; ri < 4; ++ri) {
-                const int r = kRows[ri];
-                if (m % r != 0 || (r < 32 && k > (pass && n > 16 ? 8192 : 4096)) || (r < 64 && k > 8192)) continue;
-                const int tt_step = (n > 32 && ceil_div(n, 16) % 2 == 1) ? 1 : -1;
-                for (int tt = tt_step > 0 ? 1 : tt_first; tt >= 1 && tt <= tt_first; tt += tt_step) {
-                    const long long wgs = (long long)(m / r) * ceil_div(n, 16 * tt);
-                    if (wgs < lo || wgs > hi) continue;
-                    if (tt_step > 0 && tt == 1 && wgs > kMaxCus) continue;  // (three passes only where they run at once)
-                    if (!pass && n <= 16 && r == 64 && wgs > 260) continue;  // (two 64-row tiles on some CUs: the streaming twin below)
-                    for (int gi = 0; gi < 5; ++gi) {
-                        if (k % (32 * kRing[gi][0] * kRing[gi][1]) != 0 || (tt > 1 && kRing[gi][1] > 4)) continue;
-                        memset(&c, 0, sizeof(c));
-                        c.rows_per_wave = r, c.waves_m = r == 64 ? 0 : 1, c.waves_k = kRing[gi][0], c.prefetch = kRing[gi][1];
-                        c.split_k = 1, c.token_tiles = tt, c.x_chunk = 32 * c.waves_k * c.prefetch;
-                        if (config_runs(m, n, k, c)) return c;
-                    }
-                }
-            }
-        }
+        if (narrow_round(m, n, k, &c)) return c;
         // Many rows (from 330 groups of 64; from 170 at 17..64 tokens): the streaming kernel, unsplit, with the packed
         // weights staged through LDS, 16 waves as 2 x 8 (4 x 4 from 576 groups), chunks of 512 k, a staggered walk -
         // what the tuner finds from 22016 x 4096 to 49152 x 6144 (16 tokens: 14.3, 15.9, 19.3, 30.5 us against 18.1,
@@ -471,6 +487,11 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         }
         if (best_wgs) return best;
     }
+    // 65..127 tokens on small shapes: the narrow-row round of above with its passes of 16 or 32 tokens side by side,
+    // where one exists - what the tuner finds there (2048 x 2048 at 72 tokens 5.8 us against 9.2 of the model's pick
+    // below, 1536 x 6144 8.1 against 18.0, 3072 x 8192 14.2 against 22.5, 5120 x 5120 15.1 against 16.0); larger
+    // shapes have no such round and go on to the model.
+    if (n > 64 && n < 128 && narrow_round(m, n, k, &c)) return c;
     if (n > 64) {
         // 65 tokens and more: the tile whose grid costs least by a model read off
         // the timings of 36 shapes outside the table (1024 x 8192 ... 23040 x 3072) at 65 ... 3000 tokens, each with
