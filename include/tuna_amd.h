@@ -320,6 +320,11 @@ int tuna_config_table_entry(int i, int *m, int *n_lo, int *n_hi, int *k, tuna_ge
  * bucket's entry from tuna_select_config instead, where that entry can run them (n_hi + 1: none does; -1: bad
  * index).  Written by the tuner, which times both entries inside the bucket. */
 int tuna_config_table_next_from(int i);
+/* Token counts in [*from, *to), inside the entry's n_lo .. n_hi, get the derived config from tuna_select_config
+ * instead of the table's (0, 0: none do).  Written by the tuner, which times both at several counts inside the
+ * bucket: the derivation sizes its grid for n itself, an entry's grid was sized for n_lo.  No counterpart in the
+ * reference, whose buckets hand out one config each (kernel.cu:3022-3155). */
+int tuna_config_table_derived_range(int i, int *from, int *to);
 
 /* Releases the library-owned split-K workspaces of the current device (synchronises
  * the device first).  Until then a workspace that a launch has used is never freed or moved -

@@ -491,11 +491,13 @@ def test_every_entry_for_the_upper_part_of_a_bucket_matches_the_oracle(key):
 
 @pytest.mark.parametrize("name,n,kernel", [("mistral_qkv", 1200, "128 rows x 256 tokens"), ("llama70b_qkv", 1536, "gemm_wide_kernel"),
                                            ("mistral_attn_out", 700, "128 rows x 256 tokens> split_k=2"), ("llama70b_attn_out", 600, "128 rows x 256 tokens"),
-                                           ("mistral_down", 1000, "split_k=2")])
+                                           ("mistral_down", 1000, "split_k=2"),
+                                           ("mistral_qkv", 300, "TT=2"), ("mistral_qkv", 72, "TT=1"), ("llama70b_attn_out", 270, "gemm_")])
 def test_table_shapes_between_the_counts_their_upper_entries_are_tuned_at(name, n, kernel):
     """Above 512 tokens the table's entries are tuned at 512, 1024 and 2048 tokens; at other counts a shape of fewer than
     24576 rows runs what the derivation's cost model picks (its entry at counts with as many 128-token tiles as the
-    tuning count: the last case), through the plain entry point.  Row-subset check against the oracle."""
+    tuning count: mistral_down), through the plain entry point.  The last three cases lie in the stretch of a bucket
+    below 512 tokens where the tuner timed the derived config ahead of the entry.  Row-subset check against the oracle."""
     import torch
 
     from tuna_amd import ops
@@ -615,7 +617,7 @@ def test_derived_configs_for_untuned_shapes_up_to_16_tokens(m, k, n, kernel):
                                            (3072, 8192, 512, "128 rows x 256 tokens> split_k=4"), (20480, 5120, 64, "TT=2"),
                                            (18432, 6144, 256, "256 rows x 256 tokens> split_k=3"), (2048, 2048, 384, "TT=2"),
                                            (20480, 5120, 384, "TT=8"), (16384, 8192, 640, "gemm_wide_kernel"),
-                                           (2560, 6912, 300, "128 rows x 128 tokens> split_k=4"), (4096, 11008, 100, "128 rows x 128 tokens> split_k=8"), (5120, 13824, 1000, "256 rows x 256 tokens> split_k=3"), (22016, 4096, 704, "128 rows x 256 tokens")])
+                                           (2560, 6912, 300, "128 rows x 128 tokens> split_k=4"), (4096, 11008, 100, "64 rows x 128 tokens> split_k=4"), (5120, 13824, 1000, "256 rows x 256 tokens> split_k=3"), (22016, 4096, 704, "128 rows x 256 tokens")])
 def test_derived_configs_for_untuned_shapes_from_17_to_512_tokens(m, k, n, kernel):
     """The same for 17 tokens and more: narrow-row and lean workgroups with the token passes side by side in the grid,
     the streaming kernel with 16, 32 or 64 tokens per pass, and from 256 tokens the tile that a cost model of the

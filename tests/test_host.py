@@ -74,8 +74,10 @@ def test_select_config_is_host_only_and_every_table_entry_validates():
     next_from = ops.config_table_next_from()
     with open(os.path.join(ROOT, "tuna_amd", "configs", "param_map.json")) as f:
         pm = json.load(f)
-    assert len(table) == len(pm) == len(next_from)
-    for (m, lo, hi, k, cfg), nf in zip(table, next_from):
+    derived_ranges = ops.config_table_derived_ranges()
+    assert len(table) == len(pm) == len(next_from) == len(derived_ranges)
+    assert sum(r != (0, 0) for r in derived_ranges) >= 1
+    for (m, lo, hi, k, cfg), nf, (d_from, d_to) in zip(table, next_from, derived_ranges):
         # an entry's key is the lower edge of its range: a bucket key, or a key inside a bucket (which ends the
         # range of the bucket's own entry one token earlier)
         present = make_configs.keys_of_shape(pm, m, k)
@@ -85,7 +87,11 @@ def test_select_config_is_host_only_and_every_table_entry_validates():
         assert n_key == (lo if lo in make_configs.SUB_KEYS else make_configs.bucket_of(lo))
         assert cfg.to_dict() == {f: pm[key][f] for f in cfg.FIELDS}
         assert nf == make_configs.next_from_of(n_key, pm[key], present) and lo < nf <= hi + 1
-        for n in sorted({lo, hi, min(nf, hi), max(nf - 1, lo)}):
+        # the stretch of the range, if any, where the tuner timed the derived config ahead of the table's
+        assert (d_from, d_to) == make_configs.derived_range_of(n_key, pm[key], present)
+        assert (d_from, d_to) == (0, 0) or max(lo, 65) <= d_from < d_to <= hi + 1
+        inside = {d_from, d_to - 1, max(d_from - 1, lo), min(d_to, hi)} if d_to else set()
+        for n in sorted({lo, hi, min(nf, hi), max(nf - 1, lo)} | inside):
             ops.validate_config(m, n, k, cfg)                      # the C side accepts it
             got, hit = ops.select_config(m, n, k)
             assert hit
@@ -104,7 +110,7 @@ def test_select_config_is_host_only_and_every_table_entry_validates():
             # number of 128-token tiles) a shape of fewer than 24576 rows takes the pick of the derivation's cost
             # model - far into the open-ended last bucket the 256 x 256 tile
             tuned_at = 512 if eff_lo <= 512 else 1024 if eff_lo <= 769 else 2048
-            if n > 512 and m < 24576 and -(-n // 128) != -(-tuned_at // 128):
+            if (n > 512 and m < 24576 and -(-n // 128) != -(-tuned_at // 128)) or d_from <= n < d_to:
                 assert got.to_dict() == ops.derive_config(m, n, k).to_dict()
                 if n >= 3000:
                     assert (got.lds_tile_rows, got.token_tiles, got.split_k, got.rows_per_wave) == (256, 16, 1, 64)
@@ -235,6 +241,16 @@ def test_generator_output_and_its_refusal_of_inconsistent_entries(tmp_path):
         mc.generate({"4096_16_4096": dict(e16, next_from=25), "4096_24_4096": e16})
     with pytest.raises(ValueError, match="needs the bucket's own entry"):
         mc.generate({"4096_24_4096": e16})
+    # the stretch of token counts that takes the derived config follows the config in the row; it lies inside the
+    # entry's range, above 64 tokens, and its two fields come together
+    e64 = dict(e16, token_tiles=1)
+    assert "{4096, 64, 127, 4096, 65, {64, 1, 8, 4, 2, 1024, 1, 1, 0, 0}, 65, 81}," in mc.generate({"4096_64_4096": dict(e64, derived_from=65, derived_to=81)})
+    assert "0, 0}, 97, 128}," in mc.generate({"4096_64_4096": dict(e64, derived_from=97, derived_to=128)})
+    for bad in (dict(derived_from=64, derived_to=80), dict(derived_from=100, derived_to=129), dict(derived_from=90, derived_to=90), dict(derived_from=70)):
+        with pytest.raises(ValueError, match="derived"):
+            mc.generate({"4096_64_4096": dict(e64, **bad)})
+    with pytest.raises(ValueError, match="derived"):
+        mc.generate({"4096_16_4096": dict(e16, derived_from=20, derived_to=24)})
     with pytest.raises(ValueError, match="not a bucket key"):
         mc.generate({"4096_20_4096": e16})
     # the checked-in table is what the generator produces from the checked-in json
@@ -339,6 +355,42 @@ def test_tuner_hand_over_count_from_timings(monkeypatch):
     tuner.tune_next_from(pm, list(pm), log=lambda s_: None)   # (the stub of the last run: two token tiles always lose)
     assert pm["4096_64_4096"]["next_from"] == 96 and pm["4096_96_4096"]["next_from"] == 97
     mc.generate(pm)
+
+
+def test_tuner_derived_stretch_from_timings(monkeypatch):
+    """tune_derived_range with a stub in place of the GPU evaluator: the entry gets the longest run of sampled counts
+    at which the derived config is ahead of the table's by the margin, ending at the first sample that is not."""
+    from tuna_amd import make_configs as mc, ops, tuner
+
+    rows = [(65, 10, 8), (79, 10, 9.5), (81, 10, 8), (95, 10, 8), (97, 10, 9.2), (111, 10, 11), (127, 10, 9)]
+    assert tuner.derived_stretch(rows, 127, 0.93) == (81, 111)
+    assert tuner.derived_stretch(rows[:5], 127, 0.93) == (81, 128)        # a run up to the last sample: to the range's end
+    assert tuner.derived_stretch(rows, 127, 0.5) is None and tuner.derived_stretch([], 127, 0.93) is None
+
+    own = dict(rows_per_wave=64, waves_m=2, waves_k=8, split_k=1, prefetch=2, x_chunk=512, token_tiles=2, xcd_swizzle=1,
+               k_stagger=0, lds_tile_rows=-1)
+    wins_below = {"n": 0}
+
+    class Stub:
+        def __init__(self, m, n, k, **kw):
+            self.n, self.cache = n, {}
+
+        def __call__(self, cfg):   # the table's entries take 10 us; anything else 8 below the set count, 12 from it on
+            return 10.0 if cfg == own else (8.0 if self.n < wins_below["n"] else 12.0)
+
+    monkeypatch.setattr(tuner, "Evaluator", Stub)
+    pm = {"4096_64_4096": dict(own), "4096_128_4096": dict(own), "4096_32_4096": dict(own, token_tiles=1),
+          "4096_2048_4096": dict(own, token_tiles=8, x_chunk=128)}
+    wins_below["n"] = 96
+    tuner.tune_derived_range(pm, list(pm), log=lambda s_: None)
+    derived_differs = ops.derive_config(4096, 80, 4096).to_dict() != own
+    assert derived_differs
+    assert (pm["4096_64_4096"]["derived_from"], pm["4096_64_4096"]["derived_to"]) == (65, 97)
+    assert all("derived_from" not in pm[key_] for key_ in ("4096_128_4096", "4096_32_4096", "4096_2048_4096"))
+    assert mc.derived_range_of(64, pm["4096_64_4096"]) == (65, 97)          # in range for the generator
+    wins_below["n"] = 0
+    tuner.tune_derived_range(pm, list(pm), log=lambda s_: None)
+    assert "derived_from" not in pm["4096_64_4096"] and "derived_to" not in pm["4096_64_4096"]   # a stale range goes
 
 
 def test_tuner_small_launch_config_spaces_are_valid_for_both_validators():

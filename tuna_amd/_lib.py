@@ -105,6 +105,7 @@ SIGNATURES = {
     "tuna_config_table_size": (_i, []),
     "tuna_config_table_entry": (_i, [_i, _ip, _ip, _ip, _ip, _cfgp]),
     "tuna_config_table_next_from": (_i, [_i]),
+    "tuna_config_table_derived_range": (_i, [_i, _ip, _ip]),
     "tuna_describe_launch": (_i, [_i, _i, _i, _cfgp, _i, ctypes.c_char_p, _sz]),
     "tuna_release_workspaces": (_i, []),
 }

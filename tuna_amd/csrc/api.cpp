@@ -499,7 +499,8 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         // a tile is computed whole) times a factor of the kernel - the 256 x 256 tile 0.85, the streaming kernel
         // with eight token tiles on 512 rows 0.95, the 128 x 256 tile 1.00, eight token tiles on 256 rows 1.15,
         // 256 x 128 1.20, 128 x 128 and four token tiles on 256 rows 1.45, two token tiles on 256 rows 1.78, four on
-        // 128 rows 1.95, two on 128 rows 2.0, and up to 320 tokens one token tile on 256, 128 or 64 rows 2.6, 2.2, 4.0
+        // 128 rows 1.95, two on 128 rows 2.0, up to 320 tokens one token tile on 256, 128 or 64 rows 2.6, 2.2, 4.0, and
+        // the 64 x 128 tile 1.8 (what few rows with long k take, k split in 4 to 8; a 64 x 256 tile gains nothing)
         // - plus a fixed part that counts for short k (about 6 us), and grows by
         // a seventh from 160 to 256 workgroups on the device (clock and memory are shared); a launch is as many
         // rounds as its tiles need on 256 CUs, and a round that is not full takes nearly as long as a full one.
@@ -509,14 +510,14 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         // 55 against 36, 1024 x 8192 at 160 tokens 89 against 29.  Grids of fewer than 32 workgroups (64 from 256
         // tokens) are left to the rules below, which split k.
         struct Cand { int rows, tokens, streaming; double factor; };
-        static const Cand kCand[13] = {{256, 256, 0, 0.85}, {512, 128, 1, 0.95}, {128, 256, 0, 1.00}, {256, 128, 1, 1.15}, {256, 128, 0, 1.20},
+        static const Cand kCand[14] = {{256, 256, 0, 0.85}, {512, 128, 1, 0.95}, {128, 256, 0, 1.00}, {256, 128, 1, 1.15}, {256, 128, 0, 1.20},
                                        {128, 128, 0, 1.45}, {256, 64, 1, 1.45},  {256, 32, 1, 1.78},  {128, 64, 1, 1.95},  {128, 32, 1, 2.00},
-                                       {256, 16, 1, 2.60},  {128, 16, 1, 2.20},  {64, 16, 1, 4.00}};
+                                       {256, 16, 1, 2.60},  {128, 16, 1, 2.20},  {64, 16, 1, 4.00},   {64, 128, 0, 1.80}};
         tuna_gemm_config best;
         double best_cost = 0.0;
         bool found = false;
         static const int kSplit[6] = {1, 2, 3, 4, 6, 8};
-        for (int ci = 0; ci < 13 * 6; ++ci) {
+        for (int ci = 0; ci < 14 * 6; ++ci) {
             // (the tiles of the many-token kernels also with k split in 2 ... 8 while the grid stays within one
             // round: a split workgroup does its share of the tile's time and the last one to arrive adds the
             // partial tiles, which costs about 0.3 us + 0.05 us per split and 1000 tile elements - what wins on
@@ -690,6 +691,7 @@ static int select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_t
         const TableEntry &e = kConfigTable[i];
         if (e.m == m && e.k == k && n >= e.n_lo && n <= e.n_hi) own = &e;
     }
+    const TableEntry *bucket = own;
     if (own && n >= own->next_from) {
         for (int i = 0; i < kConfigTableSize; ++i) {
             const TableEntry &e = kConfigTable[i];
@@ -712,6 +714,12 @@ static int select_config(int m, int n, int k, tuna_gemm_config *cfg, int *from_t
             const int tuned = own->n_lo <= 512 ? 512 : own->n_lo <= 769 ? 1024 : 2048;
             if (ceil_div(n, 128) != ceil_div(tuned, 128)) *cfg = derive_config(m, n, k);
         }
+        // Inside a bucket too an entry can fall behind the derivation, which sizes its grid for n itself where the
+        // entry's was sized for the tuning count (6144 x 4096 at 288..300 tokens: 41 us with the entry tuned at 256
+        // tokens, 160 workgroups of 384 rows; 30 us derived, 240 of 256 rows) - and as often it does not (7680 x
+        // 2560 at 72 tokens: 11.9 us against 14.8).  So this too is measured: the tuner times both at the sampled
+        // counts of the bucket and writes the one stretch, if any, where the derived config wins into the entry.
+        if (n >= bucket->derived_from && n < bucket->derived_to) *cfg = derive_config(m, n, k);
         if (from_table) *from_table = 1;
         return TUNA_OK;
     }
@@ -2081,6 +2089,14 @@ TUNA_EXPORT int tuna_config_table_next_from(int i)
         return -1;
     }
     return kConfigTable[i].next_from;
+}
+
+TUNA_EXPORT int tuna_config_table_derived_range(int i, int *from, int *to)
+{
+    if (i < 0 || i >= kConfigTableSize) return fail(TUNA_ERR_INVALID_ARG, "table index %d out of range", i);
+    if (from) *from = kConfigTable[i].derived_from;
+    if (to) *to = kConfigTable[i].derived_to;
+    return TUNA_OK;
 }
 
 TUNA_EXPORT int tuna_describe_launch(int m, int n, int k, const tuna_gemm_config *cfg, int decode_mode, char *buf, size_t len)

@@ -234,6 +234,9 @@ struct TableEntry {
     int m, n_lo, n_hi, k;
     int next_from;  // token counts from here to n_hi take the next bucket's entry (n_hi + 1: none does)
     tuna_gemm_config cfg;
+    // token counts in [derived_from, derived_to), inside n_lo .. n_hi, take the derived config instead: the tuner
+    // timed it there at least a twentieth faster than what the table hands out (0, 0: nowhere)
+    int derived_from, derived_to;
 };
 extern const TableEntry kConfigTable[];
 extern const int kConfigTableSize;

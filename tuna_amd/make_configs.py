@@ -375,6 +375,23 @@ def next_from_of(n_key: int, c: dict, keys_present=()) -> int:
     return nf
 
 
+def derived_range_of(n_key: int, c: dict, keys_present=()):
+    """The entry's "derived_from" / "derived_to": the lookup hands out the derived config instead of the table's for
+    token counts in [derived_from, derived_to) (written by the tuner, which times both at the sampled counts of the
+    range; absent: (0, 0), nowhere).  Checked: both or neither, inside the entry's range, and above 64 tokens (below,
+    every count of a bucket has the same grid but for one chunk, and the entries are tuned for it)."""
+    if "derived_from" not in c and "derived_to" not in c:
+        return 0, 0
+    lo, hi = key_range(n_key, keys_present)
+    try:
+        a, b = int(c["derived_from"]), int(c["derived_to"])
+    except KeyError:
+        raise ValueError("derived_from and derived_to come together") from None
+    if not (max(lo, 65) <= a < b <= hi + 1):
+        raise ValueError(f"derived range {a}..{b} outside {max(lo, 65)}..{hi + 1}")
+    return a, b
+
+
 def generate(param_map: dict) -> str:
     rows = []
     for key in sorted(param_map, key=lambda s: tuple(int(t) for t in s.split("_"))):
@@ -386,15 +403,17 @@ def generate(param_map: dict) -> str:
             if n in SUB_KEYS and SUB_KEYS[n] not in present:
                 raise ValueError(f"a key inside a bucket needs the bucket's own entry ({m}_{SUB_KEYS[n]}_{k})")
             nf = next_from_of(n, c, present)
+            dr = derived_range_of(n, c, present)
         except ValueError as e:
             raise ValueError(f"param_map entry {key}: {e}") from None
         lo, hi = key_range(n, present)
         vals = ", ".join(str(int(c.get(f, 0))) for f in FIELDS)
-        rows.append(f"    {{{m}, {lo}, {hi}, {k}, {nf}, {{{vals}}}}},  // {key}")
+        tail = f", {dr[0]}, {dr[1]}" if dr != (0, 0) else ""
+        rows.append(f"    {{{m}, {lo}, {hi}, {k}, {nf}, {{{vals}}}{tail}}},  // {key}")
     body = "\n".join(rows)
     return f"""// GENERATED by tuna_amd/make_configs.py from tuna_amd/configs/param_map.json - do not edit.
 // Shape -> tile-config table, searched linearly by tuna_select_config.
-// Entry: m, n_lo, n_hi, k, next_from, {{{", ".join(FIELDS)}}}
+// Entry: m, n_lo, n_hi, k, next_from, {{{", ".join(FIELDS)}}}[, derived_from, derived_to]
 #include "tuna_internal.h"
 
 namespace tuna {{

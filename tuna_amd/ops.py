@@ -368,6 +368,18 @@ def config_table_next_from():
     return [L.tuna_config_table_next_from(i) for i in range(L.tuna_config_table_size())]
 
 
+def config_table_derived_ranges():
+    """Per entry of config_table(): (from, to) - select_config hands out the derived config for token counts in
+    [from, to) of the entry's range ((0, 0): for none)."""
+    L = _lib.lib()
+    out = []
+    for i in range(L.tuna_config_table_size()):
+        a, b = ctypes.c_int(), ctypes.c_int()
+        _lib.check(L.tuna_config_table_derived_range(i, ctypes.byref(a), ctypes.byref(b)))
+        out.append((a.value, b.value))
+    return out
+
+
 def _ptr_array(tensors):
     arr = (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
     return ctypes.cast(arr, ctypes.POINTER(ctypes.c_void_p)), arr

@@ -550,6 +550,74 @@ def tune_next_from(param_map, keys, iters=40, margin=0.98, log=print):
         log(f"{key}: next_from {nf}  " + "  ".join(f"n={n}: {a:.2f}/{b:.2f}" for n, a, b in rows))
 
 
+def derived_stretch(rows, hi, margin):
+    """rows: (token count, us with the table's config, us with the derived one) in ascending counts.  The longest run
+    of consecutive rows whose derived time is below margin x the table's, as (first count of the run, first count
+    after it - hi + 1 when the run reaches the last row); None without such a row."""
+    best, i = None, 0
+    while i < len(rows):
+        j = i
+        while j < len(rows) and rows[j][2] < margin * rows[j][1]:
+            j += 1
+        if j > i and (best is None or j - i > best[1] - best[0]):
+            best = (i, j)
+        i = max(j, i + 1)
+    if best is None:
+        return None
+    return int(rows[best[0]][0]), int(rows[best[1]][0]) if best[1] < len(rows) else hi + 1
+
+
+def tune_derived_range(param_map, keys, iters=40, margin=0.93, log=print):
+    """Writes "derived_from" / "derived_to" into the entries `keys` of param_map: the longest stretch of sampled token
+    counts of the entry's range (above 64 tokens) at which the library's derived config takes less than `margin` of
+    the time of what the table hands out there (the entry, or from its next_from on the next one) - from the first
+    such sample to the first sample after the stretch that does not.  Entries without such a stretch lose the
+    fields.  Shapes of fewer than 24576 rows are skipped above 512 tokens, where the lookup derives already, and every
+    shape's open-ended last bucket.  The
+    derived configs are the loaded library's: run this again after a change to its derivation rules."""
+    from . import ops
+    F = make_configs.FIELDS
+    for key in keys:
+        m, nk, k = (int(t) for t in key.split("_"))
+        present = make_configs.keys_of_shape(param_map, m, k)
+        lo, hi = make_configs.key_range(nk, present)
+        param_map[key].pop("derived_from", None)
+        param_map[key].pop("derived_to", None)
+        if hi <= 64 or hi >= 128000 or (lo >= 512 and m < 24576):
+            continue
+        own = {f: param_map[key].get(f, 0) for f in F}
+        nf = make_configs.next_from_of(nk, param_map[key], present)
+        later = [p for p in present if p > nk]
+        nxt = None
+        if later and make_configs.key_range(min(later), present)[0] == hi + 1:
+            nxt = {f: param_map[f"{m}_{min(later)}_{k}"].get(f, 0) for f in F}
+        samples = [n for n in next_from_samples(nk, present) if n > 64 and not (n > 512 and m < 24576)]
+        rows = []
+        for n in samples:
+            table = own
+            if nxt is not None and n >= nf:
+                try:
+                    ops.validate_config(m, n, k, ops.GemmConfig.from_dict(nxt))
+                    table = nxt
+                except ops.TunaError:
+                    pass
+            derived = ops.derive_config(m, n, k).to_dict()
+            if derived == table:
+                rows.append((n, 0.0, 0.0))
+                continue
+            ev = Evaluator(m, n, k, iters=max(10, iters // 4) if n >= 256 else iters, warmup=5)
+            t_tab, t_der = ev(table), ev(derived)
+            ev.cache.clear()
+            t_tab, t_der = min(t_tab, ev(table)), min(t_der, ev(derived))
+            rows.append((n, t_tab, t_der))
+            del ev
+        best = derived_stretch(rows, hi, margin)
+        if best is not None:
+            param_map[key]["derived_from"], param_map[key]["derived_to"] = best
+        log(f"{key}: derived " + (f"{best[0]}..{best[1] - 1}" if best else "nowhere")
+            + "  " + "  ".join(f"n={n}: {a:.2f}/{b:.2f}" for n, a, b in rows))
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--shapes", default="all", help="comma list of shape names or 'all' or 'MxK,...'")
@@ -574,6 +642,11 @@ def main(argv=None):
                     help="instead of tuning configs: time every entry of --base for the given shapes (all token buckets) "
                          "against the next bucket's entry at several counts inside its bucket and write the hand-over "
                          "count (\"next_from\") into --out")
+    ap.add_argument("--derived-range", action="store_true",
+                    help="instead of tuning configs: time what the table of --base hands out for the given shapes (all "
+                         "token buckets above 64 tokens) against the library's derived config at several counts inside "
+                         "each bucket and write the stretch where the derived one wins (\"derived_from\", "
+                         "\"derived_to\") into --out; run after --next-from")
     ap.add_argument("--block-size", default=None,
                     help="comma list of scale-block sizes (64, 128, ...): tune the blockwise GEMM's table "
                          "(param_map_blockwise.json beside --base / --out) instead of the per-row one")
@@ -592,14 +665,17 @@ def main(argv=None):
         args.block_size = [int(t) for t in args.block_size.split(",")]
         return main_blockwise(args, shapes, tokens)
 
-    if args.next_from:
+    if args.next_from or args.derived_range:
         with open(args.base) as f:
             param_map = json.load(f)
         os.makedirs(os.path.dirname(os.path.abspath(args.out)), exist_ok=True)
         for name, m, k in shapes:
             keys = sorted((key for key in param_map if key.split("_")[0] == str(m) and key.split("_")[2] == str(k)),
                           key=lambda s_: int(s_.split("_")[1]))
-            tune_next_from(param_map, keys, iters=args.iters, log=lambda s_: print(s_, flush=True))
+            if args.next_from:
+                tune_next_from(param_map, keys, iters=args.iters, log=lambda s_: print(s_, flush=True))
+            if args.derived_range:
+                tune_derived_range(param_map, keys, iters=args.iters, log=lambda s_: print(s_, flush=True))
             with open(args.out, "w") as f:
                 json.dump(param_map, f, indent=1, sort_keys=True)
         return
