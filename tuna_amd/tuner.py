@@ -13,6 +13,10 @@ Search: a seeded population of hand-derived configs, then generations of
 the GPU with HIP events over rotating, cache-defeating weight sets (tuna_time_matmul).
 
     python -m tuna_amd.tuner --tokens 16 --shapes all --generations 6 --out tuned/param_map.json
+
+Two more passes measure how the lookup treats token counts between the tuned ones: --next-from (from which count
+of a bucket the next bucket's entry is faster) and, with the table rebuilt into the library, --derived-range (the
+stretch of a bucket where the library's derived config is faster than the table's).
 """
 import argparse
 import json
