@@ -612,14 +612,14 @@ def test_derived_configs_for_untuned_shapes_up_to_16_tokens(m, k, n, kernel):
 
 @pytest.mark.parametrize("m,k,n,kernel", [(8192, 3072, 64, "gemm_narrow_kernel"), (5120, 5120, 20, "gemm_narrow_kernel"),
                                            (4096, 12288, 32, "gemm_lean_kernel"), (12288, 4096, 64, "weights through LDS"),
-                                           (37888, 3584, 40, "weights through LDS"), (3072, 8192, 128, "weights through LDS"),
+                                           (37888, 3584, 40, "weights through LDS"), (3072, 8192, 128, "gemm_narrow_kernel"), (1024, 8192, 256, "gemm_narrow_kernel<LW=4,WK=8,U=4,PERM=1,TT=1>"), (1536, 12288, 160, "gemm_narrow_kernel"), (1024, 4096, 512, "gemm_narrow_kernel<LW=4,WK=8,U=4,PERM=1,TT=2>"),
                                            (5120, 5120, 200, "128 rows x 128 tokens> split_k=3"), (12288, 4096, 300, "TT=4"),
                                            (3072, 8192, 512, "128 rows x 256 tokens> split_k=4"), (20480, 5120, 64, "TT=2"),
                                            (18432, 6144, 256, "256 rows x 256 tokens> split_k=3"), (2048, 2048, 384, "TT=2"),
                                            (20480, 5120, 384, "TT=8"), (16384, 8192, 640, "gemm_wide_kernel"),
                                            (2560, 6912, 300, "128 rows x 128 tokens> split_k=4"), (4096, 11008, 100, "64 rows x 128 tokens> split_k=4"), (5120, 13824, 1000, "256 rows x 256 tokens> split_k=3"), (22016, 4096, 704, "128 rows x 256 tokens")])
 def test_derived_configs_for_untuned_shapes_from_17_to_512_tokens(m, k, n, kernel):
-    """The same for 17 tokens and more: narrow-row and lean workgroups with the token passes side by side in the grid,
+    """The same for 17 tokens and more: narrow-row (up to 512 tokens on small shapes) and lean workgroups with the token passes side by side in the grid,
     the streaming kernel with 16, 32 or 64 tokens per pass, and from 256 tokens the tile that a cost model of the
     grid picks (chunks of 32 ... 128 tokens of the streaming kernel side by side, or a many-token tile)."""
     _check_derived(m, k, n, kernel)

@@ -396,7 +396,10 @@ static bool narrow_round(int m, int n, int k, tuna_gemm_config *out)
         for (int ri = 0; ri < 4; ++ri) {
             const int r = kRows[ri];
             if (m % r != 0 || (r < 32 && k > (pass && n > 16 ? 8192 : 4096)) || (r < 64 && k > 8192)) continue;
-            const int tt_step = (n > 32 && ceil_div(n, 16) % 2 == 1) ? 1 : -1;
+            // (65 tokens and more: one token tile per pass first wherever those passes fit the device at once, also for
+            // an even count of token tiles - 1024 x 8192 at 256 tokens as 16 x 16 workgroups 13.7 us, as 16 x 8 of two
+            // token tiles 19.8; 1024 x 4096 8.7 against 11.9)
+            const int tt_step = (n > 64 || (n > 32 && ceil_div(n, 16) % 2 == 1)) ? 1 : -1;
             for (int tt = tt_step > 0 ? 1 : tt_first; tt >= 1 && tt <= tt_first; tt += tt_step) {
                 const long long wgs = (long long)(m / r) * ceil_div(n, 16 * tt);
                 if (wgs < lo || wgs > hi) continue;
@@ -487,11 +490,13 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         }
         if (best_wgs) return best;
     }
-    // 65..127 tokens on small shapes: the narrow-row round of above with its passes of 16 or 32 tokens side by side,
+    // 65..512 tokens on small shapes: the narrow-row round of above with its passes of 16 or 32 tokens side by side,
     // where one exists - what the tuner finds there (2048 x 2048 at 72 tokens 5.8 us against 9.2 of the model's pick
-    // below, 1536 x 6144 8.1 against 18.0, 3072 x 8192 14.2 against 22.5, 5120 x 5120 15.1 against 16.0); larger
-    // shapes have no such round and go on to the model.
-    if (n > 64 && n < 128 && narrow_round(m, n, k, &c)) return c;
+    // below, 1536 x 6144 8.1 against 18.0, 3072 x 8192 14.2 against 22.5, 5120 x 5120 15.1 against 16.0; 1024 x 8192
+    // at 130..224 tokens 13.4 against 22.5, 1536 x 12288 at 160 tokens 19.1 against 31.9, 3072 x 8192 at 144 tokens
+    // 19.4 against 24.7, 1024 x 4096 at 512 tokens 12.4 against 16.2); larger shapes have no such round and go on to
+    // the model.
+    if (n > 64 && n <= 512 && narrow_round(m, n, k, &c)) return c;
     if (n > 64) {
         // 65 tokens and more: the tile whose grid costs least by a model read off
         // the timings of 36 shapes outside the table (1024 x 8192 ... 23040 x 3072) at 65 ... 3000 tokens, each with

@@ -571,7 +571,7 @@ def derived_stretch(rows, hi, margin):
     return int(rows[best[0]][0]), int(rows[best[1]][0]) if best[1] < len(rows) else hi + 1
 
 
-def tune_derived_range(param_map, keys, iters=40, margin=0.93, log=print):
+def tune_derived_range(param_map, keys, iters=40, margin=0.95, log=print):
     """Writes "derived_from" / "derived_to" into the entries `keys` of param_map: the longest stretch of sampled token
     counts of the entry's range (above 64 tokens) at which the library's derived config takes less than `margin` of
     the time of what the table hands out there (the entry, or from its next_from on the next one) - from the first
