@@ -476,7 +476,9 @@ def test_tuner_small_launch_config_spaces_are_valid_for_both_validators():
             mc.validate(229376, 16 if bad["token_tiles"] == 1 else 128, 4096, bad)
         with pytest.raises(ops.TunaError):
             ops.validate_config(229376, 16 if bad["token_tiles"] == 1 else 128, 4096, ops.GemmConfig.from_dict(bad))
-    assert tuner.narrow_space(4096, 128, 4096) == [] and tuner.lean_space(4096, 128, 4096) == []
+    # (narrow-row configs are offered up to the 512-token bucket - token passes side by side - and no further)
+    assert tuner.narrow_space(4096, 128, 4096) and tuner.narrow_space(4096, 512, 4096) and tuner.narrow_space(4096, 1024, 4096) == []
+    assert tuner.lean_space(4096, 128, 4096) == []
     assert tuner.lean_space(4096, 16, 4104) == []       # k not a multiple of 32: no lean launch
 
 

@@ -218,7 +218,7 @@ def narrow_space(m: int, n_key: int, k: int):
     """Every config of the narrow-row kernel (gemm_narrow.hpp: 16 or 32 rows per workgroup, all
     waves along k, no split) the shape admits.  Small enough to time exhaustively."""
     lo, hi = make_configs.N_BUCKETS[n_key]
-    if lo > 64:
+    if lo > 512:     # (up to 512 tokens: small shapes run one round of workgroups x token passes side by side)
         return []
     out = []
     for rows, wk, pf, tt in sorted(make_configs.NARROW_VARIANTS):
