@@ -194,6 +194,44 @@ def test_blockwise_gemm_through_the_dispatcher_on_random_shapes(m, n, k):
     assert np.array_equal(out.cpu().numpy().view(np.uint16)[:nh], img[:, cols].T)
 
 
+@pytest.mark.parametrize("m,n,k,bs", [(2048, 100, 2048, 64), (1024, 256, 4096, 64), (1536, 130, 6144, 128), (1024, 72, 8192, 64),
+                                      (3072, 130, 3072, 64), (1024, 500, 1024, 64)])
+def test_blockwise_gemm_on_small_shapes_from_65_to_512_tokens_runs_a_round_of_narrow_row_workgroups(m, n, k, bs):
+    """Small shapes at 65..512 tokens: the library's blockwise config is one round of narrow-row workgroups with the token
+    passes (one or two token tiles each) side by side; complete output, oracle on a row sample, exact read-out of the
+    decoded weights through one-hot activations."""
+    import torch
+
+    from tuna_amd import ops
+
+    c, hit = ops.select_config_blockwise(m, n, k, bs)
+    print(f"blockwise narrow round m={m} n={n} k={k} block={bs}: {c.to_dict()}", flush=True)
+    assert not hit and ops.blockwise_family(c) == "narrow" and c.token_tiles in (1, 2) and c.split_k == 1
+    assert 64 <= (m // c.rows_per_wave) * -(-n // (16 * c.token_tiles)) <= 256
+    rng = np.random.default_rng(m + n + k + bs)
+    q, x, code, _ = make_inputs_np(m, n, k, seed=m + 3 * n + k)
+    absmax = rng.uniform(0.005, 0.02, size=(m, k // bs)).astype(np.float16).astype(np.float32)
+    dq, dx, dc, da = to_dev(q, x, code, absmax)
+    out = torch.full((n, m), float("nan"), dtype=torch.float16, device="cuda")
+    ops.matmul_blockwise(dx, dq, da, dc, out, m, n, k, bs)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().view(np.uint16)
+    assert not np.isnan(got.view(np.float16)).any()
+    rows = np.sort(rng.choice(m, size=96, replace=False)).astype(np.int32)
+    ref = O.gemm_f64(q, x.view(np.uint16), code, absmax, m, n, k, mode=O.D1, rows=rows, block_size=bs)
+    e = rel_err(f16_bits_to_f64(got[:, rows]), ref)
+    assert e <= REL_TOL, e
+    nh = min(n, k)
+    cols = rng.choice(k, size=nh, replace=False)
+    xh = np.zeros((n, k), np.float16)
+    xh[np.arange(nh), cols] = 1.0
+    dxh, = to_dev(xh)
+    ops.matmul_blockwise(dxh, dq, da, dc, out, m, n, k, bs)
+    torch.cuda.synchronize()
+    img = O.dequant(q, absmax, code, m, k, mode=O.D1, block_size=bs)
+    assert np.array_equal(out.cpu().numpy().view(np.uint16)[:nh], img[:, cols].T)
+
+
 SMALL = [
     # m, n, k
     (8, 1, 8), (8, 16, 8), (64, 16, 64), (72, 3, 40), (136, 16, 1032), (256, 16, 128),

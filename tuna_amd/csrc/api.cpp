@@ -1703,6 +1703,35 @@ static int derive_blockwise(const BlockwiseCall &b, tuna_gemm_config *out)
             return TUNA_OK;
         }
     }
+    if (n > 64 && n <= 512) {
+        // 65..512 tokens on small shapes: one round of narrow-row workgroups with the token passes side by side, as in
+        // derive_config, where some tile height and tokens per pass give 128..256 of them (from 64 for shapes of up to
+        // 8 MB) and the workgroup's scales stay in LDS - 32-row tiles first, one token tile per pass first (blocks of
+        // 64, narrow round against the model's many-token tile below: 1024 x 4096 at 72..100 tokens 7.9 us against
+        // 14.2, 1536 x 6144 at 72 tokens 10.2 against 16.4, 2048 x 2048 at 100 tokens 7.3 against 12.2 and at 256
+        // tokens 10.6 against 13.4, 3072 x 3072 at 130 tokens 12.4 against 19.6, 3072 x 8192 at 72 tokens 17.8
+        // against 23.9; with the scales read from memory - 64-row tiles of two token tiles at k = 8192 - 42 us
+        // against 19..33).
+        static const int kTry[4][2] = {{32, 1}, {32, 2}, {64, 1}, {64, 2}};
+        static const int kRing[4][2] = {{8, 4}, {8, 2}, {4, 4}, {4, 2}};
+        for (const auto &t : kTry) {
+            const int r = t[0], tt = t[1];
+            if (m % r != 0 || (r < 64 && k > 8192)) continue;
+            const long long wgs = (long long)(m / r) * ceil_div(n, 16 * tt);
+            if (wgs > kMaxCus || wgs < (packed_bytes <= (8ll << 20) ? 64 : 128)) continue;
+            for (const auto &g : kRing) {
+                if (!blockwise_narrow_scales_in_lds(k, shift, r, g[0], g[1], tt)) continue;
+                tuna_gemm_config c;
+                memset(&c, 0, sizeof(c));
+                c.rows_per_wave = r, c.waves_m = r == 64 ? 0 : 1, c.waves_k = g[0], c.prefetch = g[1];
+                c.split_k = 1, c.token_tiles = tt, c.x_chunk = 512;
+                if (run_blockwise(b, c, nullptr, true) == TUNA_OK) {
+                    *out = c;
+                    return TUNA_OK;
+                }
+            }
+        }
+    }
     if (n > 64) {
         // 65 tokens and more: the many-token tile and k split whose grid costs least by the model of derive_config,
         // with the factors of the scale-block variants (128 x 256 tile 1.0, 256 x 128, 128 x 128 and 64 x 256 1.2,

@@ -195,6 +195,7 @@ hipError_t launch_gemm_narrow(const NarrowArgs &args, int rows, int waves_k, int
 hipError_t launch_gemm_blockwise(const NarrowArgs &args, int blk_shift, int rows, int waves_k, int prefetch, int token_tiles,
                                  hipStream_t stream);
 bool derive_blockwise_narrow(int m, int k, int blk_shift, int cus, int token_tiles, int *rows, int *waves_k, int *prefetch, int *tt);
+bool blockwise_narrow_scales_in_lds(int k, int blk_shift, int rows, int waves_k, int prefetch, int tt);
 bool blockwise_narrow_runs(int m, int k, int rows, int waves_k, int prefetch, int token_tiles);
 bool launch_is_lean(const GemmPlan &plan, int cus);  // the planned launch would take the lean kernel
 bool gemm_variant_exists(int rw, int prefetch, int token_tiles, int decode, int threads, int min_waves, int grouped);
