@@ -468,7 +468,7 @@ def main():
     ap.add_argument("--no-sweeps", action="store_true", help="skip the 80-layer and token sweeps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only-headline", action="store_true", help="headline workload only (profiling runs)")
-    ap.add_argument("--workload", default=HEADLINE, help="shape name timed as the headline (profiling runs)")
+    ap.add_argument("--workload", default=HEADLINE, help="shape name, or <rows>x<k>, timed as the headline (profiling runs)")
     ap.add_argument("--tokens", type=int, default=TOKENS, help="token count of the headline workload")
     ap.add_argument("--launch", choices=("both", "stream", "graph"), default="both")
     ap.add_argument("--settle", type=int, default=300,
@@ -532,7 +532,10 @@ def main():
         print(json.dumps(res))
         return
 
-    m, k = synth.SHAPES[args.workload]
+    if args.workload in synth.SHAPES:
+        m, k = synth.SHAPES[args.workload]
+    else:                                   # (profiling runs of a shape outside the benchmark set: "<rows>x<k>")
+        m, k = (int(t) for t in args.workload.lower().split("x"))
     n = args.tokens
     head_cfg = None
     if args.weight_path != "table":
