@@ -1703,22 +1703,28 @@ static int derive_blockwise(const BlockwiseCall &b, tuna_gemm_config *out)
             return TUNA_OK;
         }
     }
-    if (n > 64 && n <= 512) {
-        // 65..512 tokens on small shapes: one round of narrow-row workgroups with the token passes side by side, as in
-        // derive_config, where some tile height and tokens per pass give 128..256 of them (from 64 for shapes of up to
+    if (n > 32 && n <= 512) {
+        // 33..512 tokens on small shapes: one round of narrow-row workgroups with the token passes side by side, as in
+        // derive_config, where some tile height and tokens per pass give 128..256 of them (from 96 for shapes of up to
         // 8 MB) and the workgroup's scales stay in LDS - 32-row tiles first, one token tile per pass first (blocks of
         // 64, narrow round against the model's many-token tile below: 1024 x 4096 at 72..100 tokens 7.9 us against
         // 14.2, 1536 x 6144 at 72 tokens 10.2 against 16.4, 2048 x 2048 at 100 tokens 7.3 against 12.2 and at 256
         // tokens 10.6 against 13.4, 3072 x 3072 at 130 tokens 12.4 against 19.6, 3072 x 8192 at 72 tokens 17.8
         // against 23.9; with the scales read from memory - 64-row tiles of two token tiles at k = 8192 - 42 us
-        // against 19..33).
+        // against 19..33; at 33..64 tokens against the 256 x 64 tile with k split to fill the device, the rule below:
+        // 2048 x 2048 6.1..6.3 us against 18.0..18.8, 1024 x 8192 11.6..12.4 against 28.2..28.9, 2560 x 5120
+        // 9.6..13.9 against 25.6..26.4, 5120 x 5120 13.6..20.1 against 26.6..27.3, 8192 x 1024 8.5..9.2 against 17).
         static const int kTry[4][2] = {{32, 1}, {32, 2}, {64, 1}, {64, 2}};
         static const int kRing[4][2] = {{8, 4}, {8, 2}, {4, 4}, {4, 2}};
+        // (32-row tiles with k beyond 8192 only where no 64-row round exists: 2560 x 10240 at 36..48 tokens as 80 x 3
+        // workgroups of 32 rows 15.5..17.2 us, the model's many-token tile 22.8
+        // - up to 64 tokens: beyond, the passes lose to a split 64 x 128 tile, 1024 x 14336 at 100 tokens 26.8 against 23.7)
+        for (int long_k = 0; long_k < (n <= 64 ? 2 : 1); ++long_k)
         for (const auto &t : kTry) {
             const int r = t[0], tt = t[1];
-            if (m % r != 0 || (r < 64 && k > 8192)) continue;
+            if (m % r != 0 || (r < 64 && (k > 8192) != (long_k == 1)) || (r == 64 && long_k)) continue;
             const long long wgs = (long long)(m / r) * ceil_div(n, 16 * tt);
-            if (wgs > kMaxCus || wgs < (packed_bytes <= (8ll << 20) ? 64 : 128)) continue;
+            if (wgs > kMaxCus || wgs < (packed_bytes <= (8ll << 20) ? 96 : 128)) continue;  // (1024 x 14336 at 64 tokens as 64 workgroups: 28.2 us, a split 64 x 128 tile 23.3)
             for (const auto &g : kRing) {
                 if (!blockwise_narrow_scales_in_lds(k, shift, r, g[0], g[1], tt)) continue;
                 tuna_gemm_config c;
@@ -1732,8 +1738,8 @@ static int derive_blockwise(const BlockwiseCall &b, tuna_gemm_config *out)
             }
         }
     }
-    if (n > 64) {
-        // 65 tokens and more: the many-token tile and k split whose grid costs least by the model of derive_config,
+    if (n > 32) {
+        // 33 tokens and more: the many-token tile and k split whose grid costs least by the model of derive_config,
         // with the factors of the scale-block variants (128 x 256 tile 1.0, 256 x 128, 128 x 128 and 64 x 256 1.2,
         // 256 x 64 and 64 x 128 1.6; split in 2 ... 8 while the grid stays near one round), read off sixteen
         // shapes x ten counts from 72 to 2048 tokens with blocks of 64, each timed with every tile and split: the
@@ -1830,11 +1836,12 @@ static int select_blockwise(const BlockwiseCall &b, tuna_gemm_config *cfg, int *
     if (from_table) *from_table = 0;
     for (int i = 0; i < kBlockwiseTableSize; ++i) {
         const BlockwiseTableEntry &e = kBlockwiseTable[i];
-        // (from 65 tokens an entry holds at the count it was tuned at, its bucket's lower edge: further into the bucket
-        // the derivation's grid model knows the token tiles that n has gained - 8192 x 8192 at 100 tokens with blocks
-        // of 64 runs 68 us with the entry of the bucket 64..127 and 41 with the model's pick)
+        // (from 33 tokens an entry holds at the count it was tuned at, its bucket's lower edge: further into the bucket
+        // the derivation knows the token tiles that n has gained - 8192 x 8192 at 100 tokens with blocks of 64 runs
+        // 68 us with the entry of the bucket 64..127 and 41 with the model's pick, 8192 x 28672 at 56 tokens 115 us
+        // with the entry of the bucket 32..63 and 69 derived)
         if (e.m == b.m && e.k == b.k && e.block_size == b.block_size && b.n >= e.n_lo && b.n <= e.n_hi &&
-            (b.n <= 64 || b.n == e.n_lo) && run_blockwise(b, e.cfg, nullptr, true) == TUNA_OK) {
+            (b.n <= 32 || b.n == e.n_lo) && run_blockwise(b, e.cfg, nullptr, true) == TUNA_OK) {
             *cfg = e.cfg;
             if (from_table) *from_table = 1;
             return TUNA_OK;
