@@ -381,6 +381,40 @@ static bool narrow_round(int m, int n, int k, tuna_gemm_config *out)
     tuna_gemm_config c;
     static const int kRows[4] = {64, 32, 24, 16};
     static const int kRing[5][2] = {{8, 4}, {4, 8}, {8, 2}, {4, 4}, {4, 2}};  // waves along k, ring depth
+    // 17 tokens and more, first: passes of ONE token tile wherever some tile height puts 128..256 workgroups (from 64
+    // for shapes of up to 8 MB) on the device, the height that gives the most; else passes of two, likewise.  Against
+    // what the loops below pick (the tallest tile that fits their bounds, passes of two first for an even count of
+    // token tiles): 1024 x 8192 at 64 tokens as 64 x 4 workgroups of 16 rows 8.2 us against 12.8 (16 x 4 of 64 rows),
+    // 2048 x 8192 at 20 tokens 8.3 against 12.7, 1536 x 6144 at 40 tokens as 64 x 3 of 24 rows 7.9 against 10.5,
+    // 3072 x 8192 at 40 tokens as 48 x 3 of 64 rows 13.0 against 16.1 (96 x 2 of 32 rows, two token tiles).
+    if (n > 16) {
+        const bool small = (long long)m * k <= (8ll << 21);  // 8 MB of packed weights
+        for (int tt = 1; tt <= 2; ++tt) {
+            long long best_wgs = 0;
+            static const int kOrder[4] = {64, 32, 16, 24};  // (24-row tiles only where no other height fits: they run 2..7 % behind 32-row tiles of fewer workgroups)
+            for (int ri = 0; ri < 4; ++ri) {
+                const int r = kOrder[ri];
+                if (r == 24 && best_wgs) break;
+                if (m % r != 0 || (r < 32 && k > (small ? 8192 : 4096)) || (r < 64 && k > 8192)) continue;
+                const long long wgs = (long long)(m / r) * ceil_div(n, 16 * tt);
+                // (up to 32 tokens on larger shapes from 150 workgroups, as in the loops below: 128 workgroups of 64 rows
+                // lose to the lean kernel's split there - 4096 x 12288 at 17..32 tokens 19.8..20.9 us against 13.5..14.6)
+                // (likewise up to 64 tokens with k beyond 8192: 2048 x 12288 at 64 tokens as 32 x 4 workgroups 19.8 us, lean 13.3)
+                if (wgs < (small ? 64 : (n <= 32 || (n <= 64 && k > 8192)) ? 150 : 128) || wgs > kMaxCus || wgs <= best_wgs) continue;
+                for (int gi = 0; gi < 5; ++gi) {
+                    if (kRing[gi][0] != 8 || k % (32 * kRing[gi][0] * kRing[gi][1]) != 0 || (tt > 1 && kRing[gi][1] > 4)) continue;
+                    memset(&c, 0, sizeof(c));
+                    c.rows_per_wave = r, c.waves_m = r == 64 ? 0 : 1, c.waves_k = kRing[gi][0], c.prefetch = kRing[gi][1];
+                    c.split_k = 1, c.token_tiles = tt, c.x_chunk = 32 * c.waves_k * c.prefetch;
+                    if (config_runs(m, n, k, c)) {
+                        *out = c, best_wgs = wgs;
+                        break;
+                    }
+                }
+            }
+            if (best_wgs) return true;
+        }
+    }
     for (int pass = 0; pass < 2; ++pass) {
         // (65 tokens and more: three to eight passes side by side must run at once - 3072 x 8192 at 96 tokens as
         // 48 x 6 workgroups 26.8 us, as 48 x 3 of two token tiles 20.8 - so the round is 128..256 workgroups there)
@@ -465,12 +499,14 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         // divides that way: the few-row shapes the streaming derivation below gives the general kernel with an odd
         // split (4096 x 8192 and 3072 x 8192 at 16 tokens: 12.2 -> 8.4 us; 4096 x 12288 at 32 tokens 21.0 -> 14.4),
         // and mid-size shapes of many rows (20480 x 5120: 19.1 -> 17.5 us).  The most workgroups win, then the
-        // narrower row tile.
+        // narrower row tile.  Up to four passes (64 tokens): few rows with long k have no narrow-row round there
+        // either (2048 x 12288 at 33..48 tokens 30.1 -> 12.8 us, 1536 x 12288 at 56..64 tokens 33 -> 13,
+        // 1024 x 14336 at 33..48 tokens 26.6 -> 11.0).
         static const int kLeanShape[9][3] = {{1, 16, 2}, {1, 8, 4}, {1, 8, 2}, {2, 8, 2}, {2, 4, 4}, {2, 4, 2}, {4, 4, 4}, {4, 4, 2}, {4, 2, 4}};
         tuna_gemm_config best;
         long long best_wgs = 0;
         const int passes16 = ceil_div(n, 16);
-        for (int li = 0; li < 9 && passes16 <= 2; ++li) {
+        for (int li = 0; li < 9 && passes16 <= 4; ++li) {
             const int wm = kLeanShape[li][0], wk = kLeanShape[li][1], pf = kLeanShape[li][2];
             if (m % (64 * wm) != 0 || k % 32 != 0) continue;
             const int steps = k / 32;
