@@ -1739,10 +1739,17 @@ static int derive_blockwise(const BlockwiseCall &b, tuna_gemm_config *out)
             return TUNA_OK;
         }
     }
-    if (n > 32 && n <= 512) {
+    const bool stream_wins = n > 16  ? packed_bytes >= (100ll << 20) || (k > 8192 && packed_bytes >= (12ll << 20)) ||
+                                           (k > 4096 && packed_bytes >= (40ll << 20))
+                             : n > 4 ? packed_bytes >= (100ll << 20) || (n > 8 && k >= 12288 && packed_bytes >= (20ll << 20))
+                                     : packed_bytes >= (256ll << 20);
+    if ((n > 32 || (n > 16 && !stream_wins)) && n <= 512) {
+        // (17..32 tokens too, where the batched kernel's rule below does not claim the shape: passes of one token tile
+        // on more workgroups against one pass of two - 1024 x 8192 at 20 tokens 11.4 us against 13.0, 2560 x 5120 9.5
+        // against 10.6, 4096 x 4096 8.4 against 9.1)
         // 33..512 tokens on small shapes: one round of narrow-row workgroups with the token passes side by side, as in
-        // derive_config, where some tile height and tokens per pass give 128..256 of them (from 96 for shapes of up to
-        // 8 MB) and the workgroup's scales stay in LDS - 32-row tiles first, one token tile per pass first (blocks of
+        // derive_config, where some tile height and tokens per pass give 128..256 of them (32-row tiles from 64 for shapes
+        // of up to 8 MB) and the workgroup's scales stay in LDS - 32-row tiles first, one token tile per pass first (blocks of
         // 64, narrow round against the model's many-token tile below: 1024 x 4096 at 72..100 tokens 7.9 us against
         // 14.2, 1536 x 6144 at 72 tokens 10.2 against 16.4, 2048 x 2048 at 100 tokens 7.3 against 12.2 and at 256
         // tokens 10.6 against 13.4, 3072 x 3072 at 130 tokens 12.4 against 19.6, 3072 x 8192 at 72 tokens 17.8
@@ -1752,15 +1759,16 @@ static int derive_blockwise(const BlockwiseCall &b, tuna_gemm_config *out)
         // 9.6..13.9 against 25.6..26.4, 5120 x 5120 13.6..20.1 against 26.6..27.3, 8192 x 1024 8.5..9.2 against 17).
         static const int kTry[4][2] = {{32, 1}, {32, 2}, {64, 1}, {64, 2}};
         static const int kRing[4][2] = {{8, 4}, {8, 2}, {4, 4}, {4, 2}};
-        // (32-row tiles with k beyond 8192 only where no 64-row round exists: 2560 x 10240 at 36..48 tokens as 80 x 3
-        // workgroups of 32 rows 15.5..17.2 us, the model's many-token tile 22.8
-        // - up to 64 tokens: beyond, the passes lose to a split 64 x 128 tile, 1024 x 14336 at 100 tokens 26.8 against 23.7)
-        for (int long_k = 0; long_k < (n <= 64 ? 2 : 1); ++long_k)
+        // (32-row tiles whatever k, unlike the per-row kernel's round: 2560 x 10240 at 36..48 tokens as 80 x 3 workgroups
+        // of 32 rows 15.5..17.2 us, the model's many-token tile 22.8; 1024 x 14336 at 100 tokens as 32 x 7 18.7, as
+        // 16 x 7 of 64 rows 26.4)
         for (const auto &t : kTry) {
             const int r = t[0], tt = t[1];
-            if (m % r != 0 || (r < 64 && (k > 8192) != (long_k == 1)) || (r == 64 && long_k)) continue;
+            if (m % r != 0 || (r < 64 && tt > 1 && k > 8192)) continue;  // (two token tiles on 32 rows with long k: 1024 x 14336 at 200 tokens 31.2 us, a split 64 x 128 tile 24.4)
             const long long wgs = (long long)(m / r) * ceil_div(n, 16 * tt);
-            if (wgs > kMaxCus || wgs < (packed_bytes <= (8ll << 20) ? 96 : 128)) continue;  // (1024 x 14336 at 64 tokens as 64 workgroups: 28.2 us, a split 64 x 128 tile 23.3)
+            // (1024 x 14336 at 64 tokens as 64 workgroups of 64 rows: 28.2 us, a split 64 x 128 tile 23.3; 1024 x 8192 at
+            // 24 tokens as 64 workgroups of 32 rows: 11.4 us, one pass of two token tiles 14.1)
+            if (wgs > kMaxCus || wgs < (packed_bytes <= (8ll << 20) && r < 64 ? 64 : 128)) continue;
             for (const auto &g : kRing) {
                 if (!blockwise_narrow_scales_in_lds(k, shift, r, g[0], g[1], tt)) continue;
                 tuna_gemm_config c;
@@ -1829,10 +1837,6 @@ static int derive_blockwise(const BlockwiseCall &b, tuna_gemm_config *out)
             return TUNA_OK;
         }
     }
-    const bool stream_wins = n > 16  ? packed_bytes >= (100ll << 20) || (k > 8192 && packed_bytes >= (12ll << 20)) ||
-                                           (k > 4096 && packed_bytes >= (40ll << 20))
-                             : n > 4 ? packed_bytes >= (100ll << 20) || (n > 8 && k >= 12288 && packed_bytes >= (20ll << 20))
-                                     : packed_bytes >= (256ll << 20);
     if (stream_wins) {
         // the batched kernel's own choice of tile height (256 rows, 128 where those are fewer than workgroups), ring of
         // two; then whatever height the row count allows
