@@ -395,7 +395,11 @@ static bool narrow_round(int m, int n, int k, tuna_gemm_config *out)
             for (int ri = 0; ri < 4; ++ri) {
                 const int r = kOrder[ri];
                 if (r == 24 && best_wgs) break;
-                if (m % r != 0 || (r < 32 && k > (small ? 8192 : 4096)) || (r < 64 && k > 8192)) continue;
+                // (32-row tiles with k beyond 8192 from 65 tokens, one token tile per pass: below, the lean kernel's split
+                // is ahead - 1024 x 14336 at 100 tokens as 32 x 7 workgroups 15.1 us against 20.4 of 16 x 7 of 64 rows,
+                // at 40 tokens 15.1 against 11.1 of the lean kernel)
+                const bool long_k_ok = r == 32 && tt == 1 && n > 64;
+                if (m % r != 0 || (r < 32 && k > (small ? 8192 : 4096)) || (r < 64 && k > 8192 && !long_k_ok)) continue;
                 const long long wgs = (long long)(m / r) * ceil_div(n, 16 * tt);
                 // (up to 32 tokens on larger shapes from 150 workgroups, as in the loops below: 128 workgroups of 64 rows
                 // lose to the lean kernel's split there - 4096 x 12288 at 17..32 tokens 19.8..20.9 us against 13.5..14.6)
