@@ -643,7 +643,8 @@ def test_reference_table_2560_wide_shapes_every_bucket(m, k, n):
 @pytest.mark.parametrize("m,k,n,kernel", [(5120, 5120, 16, "gemm_narrow_kernel"), (2048, 2048, 3, "gemm_narrow_kernel"),
                                            (11008, 4096, 9, "gemm_narrow_kernel"), (3072, 8192, 16, "gemm_lean_kernel"),
                                            (20480, 5120, 1, "gemm_lean_kernel"), (22016, 4096, 16, "weights through LDS"),
-                                           (37888, 3584, 12, "weights through LDS"), (4096, 11008, 16, "gemm_kernel")])
+                                           (37888, 3584, 12, "weights through LDS"), (4096, 11008, 16, "gemm_kernel"),
+                                           (1024, 1024, 16, "gemm_narrow_kernel<LW=1"), (2560, 5120, 4, "gemm_narrow_kernel<LW=1"), (1024, 4096, 1, "gemm_narrow_kernel<LW=1")])
 def test_derived_configs_for_untuned_shapes_up_to_16_tokens(m, k, n, kernel):
     _check_derived(m, k, n, kernel)
 

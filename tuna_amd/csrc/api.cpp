@@ -422,7 +422,11 @@ static bool narrow_round(int m, int n, int k, tuna_gemm_config *out)
     for (int pass = 0; pass < 2; ++pass) {
         // (65 tokens and more: three to eight passes side by side must run at once - 3072 x 8192 at 96 tokens as
         // 48 x 6 workgroups 26.8 us, as 48 x 3 of two token tiles 20.8 - so the round is 128..256 workgroups there)
-        const int lo = n > 64 ? (pass ? 64 : 128) : pass ? (n <= 16 ? 96 : 64) : 150, hi = n > 64 ? kMaxCus : pass ? 600 : 300;
+        // (up to 16 tokens the second pass starts at 96 workgroups, at 64 with k below 8192, where the lean kernel is
+        // no alternative: 1024 x 1024 as 64 workgroups of 16 rows 2.8..3.2 us against 8.8 of the general kernel,
+        // 1024 x 4096 4.9..5.8 against 10.8, 2560 x 5120 as 80 of 32 rows 6.4..8.3 against 10.3; 2048 x 8192 as 64
+        // of 32 rows 10.7 against 8.0 of the lean kernel)
+        const int lo = n > 64 ? (pass ? 64 : 128) : pass ? (n <= 16 && k >= 8192 ? 96 : 64) : 150, hi = n > 64 ? kMaxCus : pass ? 600 : 300;
         if (pass && (long long)m * k > (8ll << 21)) break;  // 8 MB of packed weights
         // (24- and 16-row tiles also at 17..64 tokens, for the shapes too small for a round of taller ones:
         // 2048 x 2048 at 24 tokens as 128 x 2 workgroups of 16 rows 3.9 us against 6.1 of the lean kernel,
@@ -432,8 +436,10 @@ static bool narrow_round(int m, int n, int k, tuna_gemm_config *out)
         // tokens 7.5 against 12.0)
         const int tt_first = n <= 16 ? 1 : 2;
         for (int ri = 0; ri < 4; ++ri) {
-            const int r = kRows[ri];
-            if (m % r != 0 || (r < 32 && k > (pass && n > 16 ? 8192 : 4096)) || (r < 64 && k > 8192)) continue;
+            // (that second pass up to 16 tokens: the shortest tile first - 2048 x 2048 as 128 workgroups of 16 rows
+            // 3.5..3.9 us, as 64 of 32 rows 4.1..4.6; 2560 x 5120 as 160 of 16 rows 5.7..7.1, as 80 of 32 rows 6.4..8.3)
+            const int r = kRows[pass && n <= 16 ? 3 - ri : ri];
+            if (m % r != 0 || (r < 32 && k > (pass && (n > 16 || k < 8192) ? 8192 : 4096)) || (r < 64 && k > 8192)) continue;
             // (65 tokens and more: one token tile per pass first wherever those passes fit the device at once, also for
             // an even count of token tiles - 1024 x 8192 at 256 tokens as 16 x 16 workgroups 13.7 us, as 16 x 8 of two
             // token tiles 19.8; 1024 x 4096 8.7 against 11.9)
