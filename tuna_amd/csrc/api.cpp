@@ -451,7 +451,7 @@ static bool narrow_round(int m, int n, int k, tuna_gemm_config *out)
                 if (!pass && n <= 16 && r == 64 && wgs > 260) continue;  // (two 64-row tiles on some CUs: the streaming twin below)
                 for (int gi = 0; gi < 5; ++gi) {
                     if (k % (32 * kRing[gi][0] * kRing[gi][1]) != 0 || (tt > 1 && kRing[gi][1] > 4)) continue;
-                    if (n > 64 && kRing[gi][0] != 8) continue;  // (a k that only four waves divide: 4096 x 11008 at 72 tokens 38 us, a split many-token tile 28)
+                    if (n > 32 && kRing[gi][0] != 8) continue;  // (a k that only four waves divide: 4096 x 11008 at 64..72 tokens 37..38 us, a split many-token tile 28)
                     memset(&c, 0, sizeof(c));
                     c.rows_per_wave = r, c.waves_m = r == 64 ? 0 : 1, c.waves_k = kRing[gi][0], c.prefetch = kRing[gi][1];
                     c.split_k = 1, c.token_tiles = tt, c.x_chunk = 32 * c.waves_k * c.prefetch;
@@ -543,7 +543,10 @@ static tuna_gemm_config derive_config(int m, int n, int k)
     // 19.4 against 24.7, 1024 x 4096 at 512 tokens 12.4 against 16.2); larger shapes have no such round and go on to
     // the model.
     if (n > 64 && n <= 512 && narrow_round(m, n, k, &c)) return c;
-    if (n > 64) {
+    if (n > 32) {
+        // (from 33 tokens where the rules above found nothing - k that 512 does not divide, row counts between their
+        // bounds: the general kernel's two passes ran 1.1..2.0 x the model's pick on 57 such cases, 4096 x 11008 at
+        // 48 tokens 37.9 us against 27.6 of the 64 x 128 tile split in 4, 10240 x 6144 1.85 x)
         // 65 tokens and more: the tile whose grid costs least by a model read off
         // the timings of 36 shapes outside the table (1024 x 8192 ... 23040 x 3072) at 65 ... 3000 tokens, each with
         // up to thirty candidate launches.  A workgroup's time is its tile's rows x tokens (tokens beyond n included:
