@@ -451,7 +451,9 @@ static bool narrow_round(int m, int n, int k, tuna_gemm_config *out)
                 if (!pass && n <= 16 && r == 64 && wgs > 260) continue;  // (two 64-row tiles on some CUs: the streaming twin below)
                 for (int gi = 0; gi < 5; ++gi) {
                     if (k % (32 * kRing[gi][0] * kRing[gi][1]) != 0 || (tt > 1 && kRing[gi][1] > 4)) continue;
-                    if (n > 32 && kRing[gi][0] != 8) continue;  // (a k that only four waves divide: 4096 x 11008 at 64..72 tokens 37..38 us, a split many-token tile 28)
+                    // (a k that only four waves divide: 4096 x 11008 at 64..72 tokens 37..38 us, a split many-token tile 28;
+                    // 8192 x 11008 at 24 tokens 37.9 us, the general kernel 26.9; 8192 x 6912 25.0 against 19.7)
+                    if (n > 16 && kRing[gi][0] != 8) continue;
                     memset(&c, 0, sizeof(c));
                     c.rows_per_wave = r, c.waves_m = r == 64 ? 0 : 1, c.waves_k = kRing[gi][0], c.prefetch = kRing[gi][1];
                     c.split_k = 1, c.token_tiles = tt, c.x_chunk = 32 * c.waves_k * c.prefetch;
