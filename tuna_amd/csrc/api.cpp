@@ -389,7 +389,7 @@ static bool narrow_round(int m, int n, int k, tuna_gemm_config *out)
     // 3072 x 8192 at 40 tokens as 48 x 3 of 64 rows 13.0 against 16.1 (96 x 2 of 32 rows, two token tiles).
     if (n > 16) {
         const bool small = (long long)m * k <= (8ll << 21);  // 8 MB of packed weights
-        for (int tt = 1; tt <= 2; ++tt) {
+        for (int tt = 1; tt <= (k > 16384 ? 1 : 2); ++tt) {  // (two token tiles with k beyond 16384: 5120 x 27648 at 64 tokens 67 us, a split many-token tile 48)
             long long best_wgs = 0;
             static const int kOrder[4] = {64, 32, 16, 24};  // (24-row tiles only where no other height fits: they run 2..7 % behind 32-row tiles of fewer workgroups)
             for (int ri = 0; ri < 4; ++ri) {
@@ -446,7 +446,7 @@ static bool narrow_round(int m, int n, int k, tuna_gemm_config *out)
             const int tt_step = (n > 64 || (n > 32 && ceil_div(n, 16) % 2 == 1)) ? 1 : -1;
             for (int tt = tt_step > 0 ? 1 : tt_first; tt >= 1 && tt <= tt_first; tt += tt_step) {
                 const long long wgs = (long long)(m / r) * ceil_div(n, 16 * tt);
-                if (wgs < lo || wgs > hi) continue;
+                if (wgs < lo || wgs > hi || (tt > 1 && k > 16384)) continue;
                 if (tt_step > 0 && tt == 1 && wgs > kMaxCus) continue;  // (three passes only where they run at once)
                 if (!pass && n <= 16 && r == 64 && wgs > 260) continue;  // (two 64-row tiles on some CUs: the streaming twin below)
                 for (int gi = 0; gi < 5; ++gi) {
