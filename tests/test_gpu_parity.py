@@ -652,7 +652,7 @@ def test_derived_configs_for_untuned_shapes_up_to_16_tokens(m, k, n, kernel):
 @pytest.mark.parametrize("m,k,n,kernel", [(8192, 3072, 64, "gemm_narrow_kernel"), (5120, 5120, 20, "gemm_narrow_kernel"),
                                            (4096, 12288, 32, "gemm_lean_kernel"), (12288, 4096, 64, "weights through LDS"),
                                            (37888, 3584, 40, "weights through LDS"), (3072, 8192, 128, "gemm_narrow_kernel"), (1024, 8192, 64, "gemm_narrow_kernel<LW=1,WK=8,U=4,PERM=1,TT=1>"), (2048, 12288, 48, "gemm_lean_kernel"),
-                                           (1536, 6144, 40, "gemm_narrow_kernel<LW=2,WK=8,U=4,PERM=1,TT=1>"), (2048, 8192, 20, "gemm_narrow_kernel<LW=1"), (4096, 11008, 48, "64 rows x 128 tokens> split_k=4"), (1024, 8192, 256, "gemm_narrow_kernel<LW=4,WK=8,U=4,PERM=1,TT=1>"), (1536, 12288, 160, "gemm_narrow_kernel"), (1024, 4096, 512, "gemm_narrow_kernel<LW=4,WK=8,U=4,PERM=1,TT=2>"),
+                                           (1536, 6144, 40, "gemm_narrow_kernel<LW=2,WK=8,U=4,PERM=1,TT=1>"), (2048, 8192, 20, "gemm_narrow_kernel<LW=1"), (4096, 11008, 48, "64 rows x 128 tokens> split_k=4"), (6144, 24576, 48, "weights through LDS> x_chunk=256 split_k=4"), (1024, 8192, 256, "gemm_narrow_kernel<LW=4,WK=8,U=4,PERM=1,TT=1>"), (1536, 12288, 160, "gemm_narrow_kernel"), (1024, 4096, 512, "gemm_narrow_kernel<LW=4,WK=8,U=4,PERM=1,TT=2>"),
                                            (5120, 5120, 200, "128 rows x 128 tokens> split_k=3"), (12288, 4096, 300, "TT=4"),
                                            (3072, 8192, 512, "128 rows x 256 tokens> split_k=4"), (20480, 5120, 64, "TT=2"),
                                            (18432, 6144, 256, "256 rows x 256 tokens> split_k=3"), (2048, 2048, 384, "TT=2"),

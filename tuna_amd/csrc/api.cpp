@@ -545,6 +545,20 @@ static tuna_gemm_config derive_config(int m, int n, int k)
     // 19.4 against 24.7, 1024 x 4096 at 512 tokens 12.4 against 16.2); larger shapes have no such round and go on to
     // the model.
     if (n > 64 && n <= 512 && narrow_round(m, n, k, &c)) return c;
+    if (n > 32 && n <= 64 && k > 16384 && m % 128 == 0 && m <= 8192) {
+        // 33..64 tokens, k beyond 16384, where no narrow-row round exists: the streaming kernel with four token tiles,
+        // 128-row workgroups, the weights through LDS and k split in 4 or 8 across workgroups so that the grid fills
+        // one round - the table's entry for Llama-70B's down projection, and what the tuner finds on such shapes
+        // (5120 x 27648 at 64 tokens 52.5 us against 66.0 of the model's pick below, 6144 x 24576 48.5 against 60.5,
+        // 7168 x 18432 40.2 against 48.5, 8192 x 20480 44.1 against 53.7; 10240 x 17408, split in 2: 61.6 against 57.9)
+        for (int split = 8; split >= 4; split /= 2) {
+            if ((long long)(m / 128) * split > kMaxCus) continue;
+            memset(&c, 0, sizeof(c));
+            c.rows_per_wave = 64, c.waves_m = 2, c.waves_k = 4, c.split_k = split, c.prefetch = 2, c.x_chunk = 256;
+            c.token_tiles = 4, c.lds_tile_rows = -1;
+            if (config_runs(m, n, k, c)) return c;
+        }
+    }
     if (n > 32) {
         // (from 33 tokens where the rules above found nothing - k that 512 does not divide, row counts between their
         // bounds: the general kernel's two passes ran 1.1..2.0 x the model's pick on 57 such cases, 4096 x 11008 at
