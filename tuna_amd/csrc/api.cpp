@@ -486,7 +486,25 @@ static tuna_gemm_config derive_config(int m, int n, int k)
         // workgroups - 2048 x 2048 as 128 workgroups of 16 rows 3.9 us against 9.0, 8960 x 1536 as 280 of 32 rows
         // 6.0 against 7.9; at 17..64 tokens from 64 workgroups and with the short tiles up to k = 8192:
         // 1280 x 5120 at 20 tokens as 80 x 2 of 16 rows 5.9 us against 16.7 of the general kernel.)
-        if (narrow_round(m, n, k, &c)) return c;
+        if (narrow_round(m, n, k, &c)) {
+            // (33..64 tokens with k beyond 16384: the split streaming launch described further down instead, where it
+            // puts at least as many workgroups on the device as the round - 4096 x 24576 at 40 tokens 34.5 us against
+            // 38.5, 3072 x 32768 at 64 tokens 39.4 against 46.5; 5120 x 27648 at 40 tokens, 160 workgroups against the
+            // round's 240: 52.6 against 46.1)
+            if (n > 32 && k > 16384 && m % 128 == 0 && m <= 8192) {
+                const long long round_wgs = (long long)(m / c.rows_per_wave) * ceil_div(n, 16 * c.token_tiles);
+                for (int split = 8; split >= 4; split /= 2) {
+                    if ((long long)(m / 128) * split > kMaxCus) continue;
+                    if ((long long)(m / 128) * split < round_wgs) break;
+                    tuna_gemm_config s4;
+                    memset(&s4, 0, sizeof(s4));
+                    s4.rows_per_wave = 64, s4.waves_m = 2, s4.waves_k = 4, s4.split_k = split, s4.prefetch = 2, s4.x_chunk = 256;
+                    s4.token_tiles = 4, s4.lds_tile_rows = -1;
+                    if (config_runs(m, n, k, s4)) return s4;
+                }
+            }
+            return c;
+        }
         // Many rows (from 330 groups of 64; from 170 at 17..64 tokens): the streaming kernel, unsplit, with the packed
         // weights staged through LDS, 16 waves as 2 x 8 (4 x 4 from 576 groups), chunks of 512 k, a staggered walk -
         // what the tuner finds from 22016 x 4096 to 49152 x 6144 (16 tokens: 14.3, 15.9, 19.3, 30.5 us against 18.1,
